@@ -1,0 +1,455 @@
+"""Python-facing operators with the reference's names and positional signatures (the pybind `m.def` list of
+`fast_2d_gs/_C/src/**`), each a thin marshalling layer over one C-ABI entry point of libfsgs_hip.so.
+
+torch is used only to allocate device memory and to name the current stream. Argument checks mirror the reference's
+CHECK_INPUT / CHECK_SHAPE macros and raise RuntimeError like TORCH_CHECK does.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from .. import lib as L
+
+__all__ = [
+    'gs_2d_preprocess_forward', 'gs_2d_preprocess_backward', 'gs_2d_compute_transmat_forward',
+    'gs_2d_compute_trans_mat_backward', 'GS_prepare', 'GS_2D_render_forward', 'GS_2D_render_backward',
+    'SH_to_RGB_forward', 'SH_to_RGB_backward', 'sh_encode_forward', 'sh_encode_backward', 'freq_encode_forward',
+    'freq_encode_backward', 'cdist_top', 'cdist_top_backward', 'AdamMasksedUpdated', 'knn_topk', 'lbs_blend',
+]
+
+_TILE = 16
+
+
+def _lib():
+    return L.load()
+
+
+def _f32(what, **tensors):
+    L.require_cuda(what, **tensors)
+    for k, t in tensors.items():
+        if t is not None:
+            L.require_dtype(what, k, t, torch.float32)
+
+
+def _workspace(nbytes: int, device) -> Tensor:
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+# --------------------------------------------------------------------------------------------------------------------
+def gs_2d_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: bool, means3D: Tensor, scales: Tensor,
+                             rotations: Tensor, opacities: Tensor, shs: Tensor, sh_rest: Optional[Tensor],
+                             Tw2v: Tensor, Tv2c: Tensor, cam_pos: Tensor, trans_precomp: Optional[Tensor] = None,
+                             means2D: Optional[Tensor] = None, culling: Optional[Tensor] = None) -> List[Tensor]:
+    """gs_2d_preprocess.cu:331-421 -> [means2D, colors, trans_mat, normal_opacity, depths, radii, tiles_touched]."""
+    what = 'gs_2d_preprocess_forward'
+    _f32(what, means3D=means3D, scales=scales, rotations=rotations, opacities=opacities, shs=shs, Tw2v=Tw2v,
+         Tv2c=Tv2c, cam_pos=cam_pos)
+    if means3D.ndim != 2 or means3D.shape[-1] != 3:
+        raise RuntimeError('Error shape for means3D')
+    P = means3D.shape[0]
+    has_rest = sh_rest is not None and sh_rest.numel() > 0
+    M = 0
+    if has_rest:
+        _f32(what, sh_rest=sh_rest)
+        if not (sh_rest.ndim == 3 and sh_rest.shape[0] == P and sh_rest.shape[1] >= (1 + sh_degree) ** 2 - 1
+                and sh_rest.shape[2] == 3):
+            raise RuntimeError('Error shape for sh features')
+        M = sh_rest.shape[1]
+    elif sh_degree >= 0:
+        if not (shs.ndim == 3 and shs.shape[0] == P and shs.shape[1] >= (1 + sh_degree) ** 2 and shs.shape[2] == 3):
+            raise RuntimeError('Error shape for sh features')
+        M = shs.shape[1]
+    if means2D is not None:
+        _f32(what, means2D=means2D)
+        L.require_shape(what, 'means2D', means2D, P, 2)
+    if culling is not None:
+        L.require_cuda(what, culling=culling)
+        L.require_dtype(what, 'culling', culling, torch.bool)
+        L.require_shape(what, 'culling', culling, P)
+    if trans_precomp is not None:
+        _f32(what, trans_precomp=trans_precomp)
+    L.require_shape(what, 'scales', scales, P, 2)
+    L.require_shape(what, 'rotations', rotations, P, 4)
+    L.require_shape(what, 'opacities', opacities, P, 1)
+    L.require_shape(what, 'Tw2v', Tw2v, 4, 4)
+    L.require_shape(what, 'Tv2c', Tv2c, 4, 4)
+    L.require_shape(what, 'cam_pos', cam_pos, 3)
+    if sh_degree < 0:
+        L.require_shape(what, 'shs', shs, P, 3)
+
+    opt = dict(dtype=torch.float32, device=means3D.device)
+    colors = shs if sh_degree < 0 else torch.empty((P, 3), **opt)
+    trans_mat = trans_precomp if trans_precomp is not None else torch.empty((P, 3, 3), **opt)
+    preserve = means2D is not None
+    means2D_ = means2D if preserve else torch.empty((P, 2), **opt)
+    depths = torch.empty((P,), **opt)
+    radii = torch.empty((P,), dtype=torch.int32, device=means3D.device)
+    tiles_touched = torch.empty((P,), dtype=torch.int32, device=means3D.device)
+    normal_opacity = torch.empty((P, 4), **opt)
+    rc = _lib().fsgs_gs_2d_preprocess_forward(
+        P, W, H, sh_degree, M, L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(opacities), L.ptr(shs),
+        L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(cam_pos), L.ptr(trans_precomp),
+        L.ptr(culling), int(preserve), L.ptr(means2D_), None if sh_degree < 0 else L.ptr(colors),
+        None if trans_precomp is not None else L.ptr(trans_mat), L.ptr(normal_opacity), L.ptr(depths), L.ptr(radii),
+        L.ptr(tiles_touched), L.current_stream())
+    L.check(rc, what)
+    return [means2D_, colors, trans_mat, normal_opacity, depths, radii, tiles_touched]
+
+
+def gs_2d_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs, sh_rest,
+                              Tw2v, Tv2c, cam_pos, trans_mat, radii, colors, normal_opacity,
+                              grad_mean2D, grad_trans, grad_depth, grad_colors, grad_normals,
+                              grad_means3D, grad_scales, grad_rotations, grad_opacities, grad_shs, grad_sh_rest,
+                              grad_Tw2v=None, grad_campos=None) -> None:
+    """gs_2d_preprocess.cu:423-499: fills the caller's zeroed grad_* tensors in place and overwrites grad_mean2D."""
+    what = 'gs_2d_preprocess_backward'
+    _f32(what, grad_mean2D=grad_mean2D, grad_colors=grad_colors, grad_normals=grad_normals,
+         grad_means3D=grad_means3D, grad_trans=grad_trans, grad_scales=grad_scales, grad_rotations=grad_rotations,
+         grad_opacities=grad_opacities, grad_shs=grad_shs, grad_sh_rest=grad_sh_rest)
+    if grad_shs is not None and colors is None:
+        raise RuntimeError('shs and clamped must not be None when need grad_shs')
+    has_rest = sh_rest is not None and sh_rest.numel() > 0
+    P = means3D.shape[0]
+    M = sh_rest.shape[1] if has_rest else (shs.shape[1] if shs.ndim == 3 else 0)
+    L.require_shape(what, 'grad_means3D', grad_means3D, P, 3)
+    if grad_scales is None or grad_rotations is None:
+        raise RuntimeError(f'{what}: grad_scales and grad_rotations are required')
+    L.require_shape(what, 'grad_scales', grad_scales, P, 2)
+    L.require_shape(what, 'grad_rotations', grad_rotations, P, 4)
+    L.require_shape(what, 'grad_opacities', grad_opacities, P, 1)
+    rc = _lib().fsgs_gs_2d_preprocess_backward(
+        P, W, H, sh_degree, M, L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(shs),
+        L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(cam_pos), L.ptr(trans_mat),
+        L.ptr(radii), L.ptr(colors), L.ptr(grad_mean2D), L.ptr(grad_trans), L.ptr(grad_colors), L.ptr(grad_normals),
+        L.ptr(grad_means3D), L.ptr(grad_scales), L.ptr(grad_rotations), L.ptr(grad_opacities), L.ptr(grad_shs),
+        L.ptr(grad_sh_rest) if has_rest else None, L.current_stream())
+    L.check(rc, what)
+
+
+def gs_2d_compute_transmat_forward(W, H, means3D, scales, rotations, Tw2v, Tw2c) -> Tuple[Tensor, Tensor]:
+    """gs_2d_preprocess.cu:512-550 -> (trans_mat[P,3,3], normals[P,3])."""
+    what = 'gs_2d_compute_transmat_forward'
+    _f32(what, means3D=means3D, scales=scales, rotations=rotations, Tw2v=Tw2v, Tw2c=Tw2c)
+    P = means3D.shape[0]
+    L.require_shape(what, 'means3D', means3D, P, 3)
+    L.require_shape(what, 'scales', scales, P, 2)
+    L.require_shape(what, 'rotations', rotations, P, 4)
+    L.require_shape(what, 'Tw2v', Tw2v, 4, 4)
+    L.require_shape(what, 'Tw2c', Tw2c, 4, 4)
+    trans_mat = torch.empty((P, 3, 3), dtype=torch.float32, device=means3D.device)
+    normals = torch.empty((P, 3), dtype=torch.float32, device=means3D.device)
+    rc = _lib().fsgs_gs_2d_compute_transmat_forward(P, W, H, L.ptr(means3D), L.ptr(scales), L.ptr(rotations),
+                                                    L.ptr(Tw2v), L.ptr(Tw2c), L.ptr(trans_mat), L.ptr(normals),
+                                                    L.current_stream())
+    L.check(rc, what)
+    return trans_mat, normals
+
+
+def gs_2d_compute_trans_mat_backward(W, H, means3D, scales, rotations, Tw2v, Tw2c, grad_matrix,
+                                     grad_normals) -> List[Tensor]:
+    """gs_2d_preprocess.cu:564-599 -> [grad_means3D, grad_scales, grad_rotations]."""
+    what = 'gs_2d_compute_trans_mat_backward'
+    _f32(what, means3D=means3D, scales=scales, rotations=rotations, Tw2v=Tw2v, Tw2c=Tw2c, grad_matrix=grad_matrix,
+         grad_normals=grad_normals)
+    P = means3D.shape[0]
+    L.require_shape(what, 'grad_matrix', grad_matrix, P, 3, 3)
+    L.require_shape(what, 'grad_normals', grad_normals, P, 3)
+    g_means3D = torch.empty((P, 3), dtype=torch.float32, device=means3D.device)
+    g_scales = torch.empty((P, 2), dtype=torch.float32, device=means3D.device)
+    g_rot = torch.empty((P, 4), dtype=torch.float32, device=means3D.device)
+    rc = _lib().fsgs_gs_2d_compute_transmat_backward(P, W, H, L.ptr(means3D), L.ptr(scales), L.ptr(rotations),
+                                                     L.ptr(Tw2v), L.ptr(Tw2c), L.ptr(grad_matrix),
+                                                     L.ptr(grad_normals), L.ptr(g_means3D), L.ptr(g_scales),
+                                                     L.ptr(g_rot), L.current_stream())
+    L.check(rc, what)
+    return [g_means3D, g_scales, g_rot]
+
+
+# --------------------------------------------------------------------------------------------------------------------
+def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, tiles_touched: Tensor,
+               debug: bool = False, return_keys: bool = False) -> List[Tensor]:
+    """gaussian_prepare.cu:282-308 -> [ranges[T,2] int64, point_list[R] int32]."""
+    what = 'GS_prepare'
+    _f32(what, means2D=means2D, depths=depths)
+    L.require_cuda(what, radii=radii, tiles_touched=tiles_touched)
+    L.require_dtype(what, 'radii', radii, torch.int32)
+    L.require_dtype(what, 'tiles_touched', tiles_touched, torch.int32)
+    P = means2D.shape[0]
+    dev = means2D.device
+    lib = _lib()
+    stream = L.current_stream()
+    T = ((W + _TILE - 1) // _TILE) * ((H + _TILE - 1) // _TILE)
+    ranges = torch.empty((T, 2), dtype=torch.int64, device=dev)
+    offsets = torch.empty((max(P, 1),), dtype=torch.int64, device=dev)
+    ws1 = _workspace(lib.fsgs_gs_prepare_scan_workspace_bytes(P), dev)
+    R = ctypes.c_int64(0)
+    rc = lib.fsgs_gs_prepare_scan(P, L.ptr(tiles_touched), L.ptr(offsets), L.ptr(ws1), ws1.numel(),
+                                  ctypes.addressof(R), stream)
+    L.check(rc, what)
+    R = int(R.value)
+    point_list = torch.empty((R,), dtype=torch.int32, device=dev)
+    keys = torch.empty((R,), dtype=torch.int64, device=dev) if return_keys else None
+    ws2 = _workspace(lib.fsgs_gs_prepare_fill_workspace_bytes(R), dev)
+    rc = lib.fsgs_gs_prepare_fill(P, W, H, L.ptr(means2D), L.ptr(depths), L.ptr(radii), L.ptr(offsets), R,
+                                  L.ptr(ranges), L.ptr(point_list), L.ptr(keys), L.ptr(ws2), ws2.numel(), stream)
+    L.check(rc, what)
+    if debug:
+        torch.cuda.synchronize()
+    return [ranges, point_list, keys] if return_keys else [ranges, point_list]
+
+
+# --------------------------------------------------------------------------------------------------------------------
+def GS_2D_render_forward(width: int, height: int, means2D: Tensor, colors: Tensor, normal_opacity: Tensor,
+                         trans_mat: Tensor, point_list: Tensor, ranges: Tensor, near_n: float, far_n: float,
+                         only_image: bool, trans_mat_t2: Optional[Tensor] = None,
+                         accum_max_count: Optional[Tensor] = None, accum_weights_p: Optional[Tensor] = None,
+                         accum_weights_count: Optional[Tensor] = None):
+    """gs_2d_redner.cu:541-629 -> (colors[3,H,W], opacity[H,W], extras[9,H,W]|None, flow[H,W,2]|None, n_contrib)."""
+    what = 'GS_2D_render_forward'
+    _f32(what, colors=colors, trans_mat=trans_mat, means2D=means2D, normal_opacity=normal_opacity,
+         trans_mat_t2=trans_mat_t2, accum_weights_p=accum_weights_p)
+    if colors.ndim != 2:
+        raise RuntimeError(f'{what}: colors must have 2 dimensions')
+    P = colors.shape[0]
+    L.require_shape(what, 'trans_mat', trans_mat, P, 3, 3)
+    L.require_cuda(what, ranges=ranges, point_list=point_list, accum_max_count=accum_max_count,
+                   accum_weights_count=accum_weights_count)
+    L.require_dtype(what, 'ranges', ranges, torch.int64)
+    L.require_dtype(what, 'point_list', point_list, torch.int32)
+    for name, t, dt in (('accum_max_count', accum_max_count, torch.int32),
+                        ('accum_weights_count', accum_weights_count, torch.int32)):
+        if t is not None:
+            L.require_dtype(what, name, t, dt)
+            L.require_shape(what, name, t, P)
+    if accum_weights_p is not None:
+        L.require_shape(what, 'accum_weights_p', accum_weights_p, P)
+    if trans_mat_t2 is not None:
+        L.require_shape(what, 'trans_mat_t2', trans_mat_t2, P, 3, 3)
+    opt = dict(dtype=torch.float32, device=colors.device)
+    pixel_colors = torch.empty((3, height, width), **opt)
+    pixel_opacity = torch.empty((height, width), **opt)
+    n_contrib = torch.empty((2, height, width), dtype=torch.int32, device=colors.device)
+    pixel_extras = None if only_image else torch.empty((9, height, width), **opt)
+    pixel_flow = torch.empty((height, width, 2), **opt) if (not only_image and trans_mat_t2 is not None) else None
+    rc = _lib().fsgs_gs_2d_render_forward(
+        P, width, height, float(near_n), float(far_n), int(bool(only_image)), L.ptr(means2D), L.ptr(colors),
+        L.ptr(normal_opacity), L.ptr(trans_mat), L.ptr(point_list), L.ptr(ranges), L.ptr(trans_mat_t2),
+        L.ptr(accum_max_count), L.ptr(accum_weights_p), L.ptr(accum_weights_count), L.ptr(pixel_colors),
+        L.ptr(pixel_opacity), L.ptr(pixel_extras), L.ptr(pixel_flow), L.ptr(n_contrib), L.current_stream())
+    L.check(rc, what)
+    return pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib
+
+
+def GS_2D_render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat2, out_opacity, out_others, out_flows,
+                          dL_dout_color, dL_dout_opacity, dL_dothers, dL_dout_flows, ranges, point_list, n_contrib,
+                          near_n: float, far_n: float):
+    """gs_2d_redner.cu:631-717 -> (dL_dcolors[P,3], dL_dmeans2D[P,2], dL_dtrans_m[P,3,3], dL_dnorm_op[P,4])."""
+    what = 'GS_2D_render_backward'
+    L.require_cuda(what, dL_dout_color=dL_dout_color, dL_dout_opacity=dL_dout_opacity, dL_dothers=dL_dothers,
+                   dL_dout_flows=dL_dout_flows)
+    P = means2D.shape[0]
+    H, W = dL_dout_color.shape[1], dL_dout_color.shape[2]
+    opt = dict(dtype=torch.float32, device=out_opacity.device)
+    g_means2D = torch.zeros((P, 2), **opt)
+    g_norm_op = torch.zeros((P, 4), **opt)
+    g_colors = torch.zeros((P, 3), **opt)
+    g_trans = torch.zeros((P, 3, 3), **opt)
+    if P == 0:
+        return g_colors, g_means2D, g_trans, g_norm_op
+    c = lambda t: None if t is None else t.contiguous()
+    means2D, normal_opacity, colors, out_opacity = c(means2D), c(normal_opacity), c(colors), c(out_opacity)
+    dL_dout_color, dL_dout_opacity, dL_dothers, dL_dout_flows = (c(dL_dout_color), c(dL_dout_opacity),
+                                                                c(dL_dothers), c(dL_dout_flows))
+    ranges, point_list, n_contrib = c(ranges), c(point_list), c(n_contrib)
+    use_aux = out_others is not None and dL_dothers is not None
+    rc = _lib().fsgs_gs_2d_render_backward(
+        P, W, H, float(near_n), float(far_n), L.ptr(means2D), L.ptr(normal_opacity), L.ptr(colors), L.ptr(trans_mat),
+        L.ptr(trans_mat2), L.ptr(out_opacity), L.ptr(out_others) if use_aux else None,
+        L.ptr(out_flows) if dL_dout_flows is not None else None, L.ptr(dL_dout_color), L.ptr(dL_dout_opacity),
+        L.ptr(dL_dothers) if use_aux else None, L.ptr(dL_dout_flows), L.ptr(ranges), L.ptr(point_list),
+        L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_norm_op), L.current_stream())
+    L.check(rc, what)
+    return g_colors, g_means2D, g_trans, g_norm_op
+
+
+# --------------------------------------------------------------------------------------------------------------------
+def SH_to_RGB_forward(dir_or_pos: Tensor, campos: Optional[Tensor], sh_features: Tensor, degree: int,
+                      clamp: bool) -> Tensor:
+    """ops_3d/spherical_harmonics.cu:15-41 -> rgb[P,3]."""
+    what = 'SH_to_RGB_forward'
+    _f32(what, dir_or_pos=dir_or_pos, campos=campos, sh_features=sh_features)
+    if dir_or_pos.ndim != 2 or dir_or_pos.shape[-1] != 3:
+        raise RuntimeError('Error shape for dir_or_pos [P, 3]')
+    if campos is not None and not (campos.ndim == 1 and campos.numel() == 3):
+        raise RuntimeError('Error shape for campos')
+    P, F = dir_or_pos.shape[0], sh_features.shape[-2]
+    L.require_shape(what, 'sh_features', sh_features, P, F, 3)
+    if not (0 <= degree <= 7 and (1 << degree) <= F):
+        raise RuntimeError('degree error')
+    rgb = torch.empty((P, 3), dtype=torch.float32, device=dir_or_pos.device)
+    rc = _lib().fsgs_sh_to_rgb_forward(P, F, degree, int(bool(clamp)), L.ptr(dir_or_pos), L.ptr(campos),
+                                       L.ptr(sh_features), L.ptr(rgb), L.current_stream())
+    L.check(rc, what)
+    return rgb
+
+
+def SH_to_RGB_backward(degree: int, clamp: bool, dir_or_pos: Tensor, campos: Optional[Tensor], sh_features: Tensor,
+                       rgb: Tensor, grad_rgb: Tensor, grad_dir: Optional[Tensor], grad_campos: Optional[Tensor],
+                       grad_shs: Optional[Tensor]) -> None:
+    """ops_3d/spherical_harmonics.cu:68-102: fills grad_dir / grad_shs, accumulates into grad_campos."""
+    what = 'SH_to_RGB_backward'
+    _f32(what, grad_rgb=grad_rgb, rgb=rgb, grad_dir=grad_dir, grad_shs=grad_shs, grad_campos=grad_campos)
+    if grad_dir is not None and grad_dir.shape != dir_or_pos.shape:
+        raise RuntimeError('Error shape for grad_dir')
+    if grad_shs is not None and grad_shs.shape != sh_features.shape:
+        raise RuntimeError('Error shape for grad_shs')
+    if grad_campos is not None and grad_campos.shape != campos.shape:
+        raise RuntimeError('ERROR shape for grad_campos')
+    P, F = dir_or_pos.shape[0], sh_features.shape[-2]
+    rc = _lib().fsgs_sh_to_rgb_backward(P, F, degree, int(bool(clamp)), L.ptr(dir_or_pos.contiguous()),
+                                        L.ptr(campos), L.ptr(sh_features.contiguous()), L.ptr(rgb), L.ptr(grad_rgb),
+                                        L.ptr(grad_dir), L.ptr(grad_campos), L.ptr(grad_shs), L.current_stream())
+    L.check(rc, what)
+
+
+def sh_encode_forward(inputs: Tensor, outputs: Tensor, B: int, D: int, C: int) -> None:
+    """nerf/shencoder.cu:657-673: outputs[B,(C+1)^2] <- basis values of inputs[B,D][:, :3]."""
+    what = 'sh_encode_forward'
+    _f32(what, inputs=inputs, outputs=outputs)
+    rc = _lib().fsgs_sh_encode_forward(B, D, C, L.ptr(inputs), L.ptr(outputs), L.current_stream())
+    L.check(rc, what)
+
+
+def sh_encode_backward(grad: Tensor, inputs: Tensor, B: int, D: int, C: int, grad_inputs: Tensor) -> None:
+    """nerf/shencoder.cu:675-691."""
+    what = 'sh_encode_backward'
+    _f32(what, grad=grad, inputs=inputs, grad_inputs=grad_inputs)
+    rc = _lib().fsgs_sh_encode_backward(B, D, C, L.ptr(grad), L.ptr(inputs), L.ptr(grad_inputs), L.current_stream())
+    L.check(rc, what)
+
+
+def freq_encode_forward(inputs: Tensor, degree: int, include_inputs: bool, scale: float) -> Tensor:
+    """nerf/freqencoder.cu:63-81 -> outputs[..., D * (2 * degree + include_inputs)]."""
+    what = 'freq_encode_forward'
+    _f32(what, inputs=inputs)
+    Din = inputs.shape[-1]
+    Dout = Din * (degree * 2 + int(bool(include_inputs)))
+    B = inputs.numel() // Din
+    out = torch.empty((*inputs.shape[:-1], Dout), dtype=torch.float32, device=inputs.device)
+    rc = _lib().fsgs_freq_encode_forward(B, Din, degree, int(bool(include_inputs)), float(scale), L.ptr(inputs),
+                                         L.ptr(out), L.current_stream())
+    L.check(rc, what)
+    return out
+
+
+def freq_encode_backward(grad: Tensor, outputs: Tensor, degree: int, include_inputs: bool, scale: float) -> Tensor:
+    """nerf/freqencoder.cu:83-104 -> grad_inputs."""
+    what = 'freq_encode_backward'
+    _f32(what, grad=grad, outputs=outputs)
+    if grad.shape != outputs.shape:
+        raise RuntimeError(f'{what}: grad must have the shape of outputs')
+    Dout = outputs.shape[-1]
+    Din = Dout // (degree * 2 + int(bool(include_inputs)))
+    B = outputs.numel() // Dout
+    gin = torch.empty((*outputs.shape[:-1], Din), dtype=torch.float32, device=outputs.device)
+    rc = _lib().fsgs_freq_encode_backward(B, Din, degree, int(bool(include_inputs)), float(scale), L.ptr(grad),
+                                          L.ptr(outputs), L.ptr(gin), L.current_stream())
+    L.check(rc, what)
+    return gin
+
+
+# --------------------------------------------------------------------------------------------------------------------
+def cdist_top(x1: Tensor, x2: Tensor, largest: bool = False) -> List[Tensor]:
+    """other/cdist_top.cu:34-84 -> [distance[..., N] f32, index[..., N] int64]."""
+    what = 'cdist_top'
+    if x1.device != x2.device:
+        raise RuntimeError('x1 and x2 must be same device')
+    _f32(what, x1=x1, x2=x2)
+    N, M, D = x1.shape[-2], x2.shape[-2], x1.shape[-1]
+    B = x1.numel() // max(N * D, 1)
+    if x2.shape[-1] != D:
+        raise RuntimeError(f'The dimenstion of point must be {D}')
+    if x2.numel() != B * M * D:
+        raise RuntimeError('The shape[:-2] of x2 must be same with x1')
+    distance = torch.empty(x1.shape[:-1], dtype=torch.float32, device=x1.device)
+    index = torch.empty(x1.shape[:-1], dtype=torch.int64, device=x1.device)
+    rc = _lib().fsgs_cdist_top_forward(B, N, M, D, int(bool(largest)), L.ptr(x1), L.ptr(x2), L.ptr(distance),
+                                       L.ptr(index), L.current_stream())
+    L.check(rc, what)
+    return [distance, index]
+
+
+def cdist_top_backward(x1: Tensor, x2: Tensor, distance: Tensor, index: Tensor, grad_dist: Tensor) -> List[Tensor]:
+    """other/cdist_top.cu:107-154 -> [grad_x1, grad_x2]."""
+    what = 'cdist_top_backward'
+    _f32(what, x1=x1, x2=x2, distance=distance, grad_dist=grad_dist)
+    L.require_cuda(what, index=index)
+    N, D, M = x1.shape[-2], x1.shape[-1], x2.shape[-2]
+    B = x1.numel() // max(N * D, 1)
+    g1 = torch.zeros_like(x1)
+    g2 = torch.zeros_like(x2)
+    rc = _lib().fsgs_cdist_top_backward(B, N, M, D, L.ptr(x1), L.ptr(x2), L.ptr(distance), L.ptr(index),
+                                        L.ptr(grad_dist), L.ptr(g1), L.ptr(g2), L.current_stream())
+    L.check(rc, what)
+    return [g1, g2]
+
+
+def AdamMasksedUpdated(param: Tensor, param_grad: Tensor, exp_avg: Tensor, exp_avg_sq: Tensor, tiles_touched: Tensor,
+                       lr: float, b1: float, b2: float, eps: float, N: int, M: int) -> None:
+    """other/adam_masked_update.cu:30-35 (name kept as spelled there)."""
+    what = 'AdamMasksedUpdated'
+    _f32(what, param=param, exp_avg=exp_avg, exp_avg_sq=exp_avg_sq)
+    param_grad = param_grad.contiguous()
+    tiles_touched = tiles_touched.contiguous()
+    L.require_cuda(what, param_grad=param_grad, tiles_touched=tiles_touched)
+    L.require_dtype(what, 'tiles_touched', tiles_touched, torch.bool)
+    if param.numel() < N * M or tiles_touched.numel() < N:
+        raise RuntimeError(f'{what}: tensors are smaller than N x M = {N} x {M}')
+    rc = _lib().fsgs_adam_masked_update(int(N), int(M), L.ptr(tiles_touched), float(lr), float(b1), float(b2),
+                                        float(eps), L.ptr(param), L.ptr(param_grad), L.ptr(exp_avg),
+                                        L.ptr(exp_avg_sq), L.current_stream())
+    L.check(rc, what)
+
+
+# --------------------------------------------------------------------------------------------------------------------
+def knn_topk(x: Tensor, y: Tensor, K: int) -> Tuple[Tensor, Tensor]:
+    """K nearest rows of y[M,D] for each row of x[N,D] -> (dist2[N,K] ascending, index[N,K] int64).
+    Stands in for pytorch3d.ops.knn_points at fast_2d_gs/network.py:504 (squared distances, ties -> lower index)."""
+    what = 'knn_topk'
+    _f32(what, x=x, y=y)
+    N, D = x.shape
+    M = y.shape[0]
+    if y.shape[1] != D:
+        raise RuntimeError(f'{what}: feature dimensions differ')
+    dist2 = torch.empty((N, K), dtype=torch.float32, device=x.device)
+    index = torch.empty((N, K), dtype=torch.int64, device=x.device)
+    rc = _lib().fsgs_knn_topk(N, M, D, K, L.ptr(x), L.ptr(y), L.ptr(dist2), L.ptr(index), L.current_stream())
+    L.check(rc, what)
+    return dist2, index
+
+
+def lbs_blend(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_s: Optional[Tensor], dist2: Tensor,
+              index: Tensor, temperature: float = 1.0, centred: bool = False):
+    """LBS warp of fast_2d_gs/network.py:517,545-573 -> (d_xyz[N,3], d_rot[N,4], d_scale[N,S]|None, weights[N,K])."""
+    what = 'lbs_blend'
+    _f32(what, points=points, sp_points=sp_points, sp_t=sp_t, sp_r=sp_r, sp_s=sp_s, dist2=dist2)
+    L.require_cuda(what, index=index)
+    L.require_dtype(what, 'index', index, torch.int64)
+    N, K = dist2.shape
+    M = sp_points.shape[0]
+    S = 0 if sp_s is None else sp_s.shape[1]
+    opt = dict(dtype=torch.float32, device=points.device)
+    d_xyz, d_rot = torch.empty((N, 3), **opt), torch.empty((N, 4), **opt)
+    d_scale = torch.empty((N, S), **opt) if S else None
+    weights = torch.empty((N, K), **opt)
+    lib = _lib()
+    ws = _workspace(lib.fsgs_lbs_blend_workspace_bytes(M), points.device)
+    rc = lib.fsgs_lbs_blend(N, M, K, int(bool(centred)), float(temperature), L.ptr(points), L.ptr(sp_points),
+                            L.ptr(sp_t), L.ptr(sp_r), L.ptr(sp_s), S, L.ptr(dist2), L.ptr(index), L.ptr(weights),
+                            L.ptr(d_xyz), L.ptr(d_rot), L.ptr(d_scale), L.ptr(ws), ws.numel(), L.current_stream())
+    L.check(rc, what)
+    return d_xyz, d_rot, d_scale, weights

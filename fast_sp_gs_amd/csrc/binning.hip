@@ -1,0 +1,399 @@
+// Tile binning for gfx950: prefix sum of per-surfel tile counts, (tile | depth-bits) key duplication, a stable
+// least-significant-digit radix sort of 64-bit keys with 32-bit payloads, and per-tile range detection.
+//
+// Reference behaviour reproduced bit for bit: fast_2d_gs/_C/src/gaussian_splatting/gaussian_prepare.cu:32-83
+// (getHigherMsb, duplicateWithKeys), :192-220 (identifyTileRanges), :222-308 (prepare / GS_prepare, which uses
+// cub::DeviceScan::InclusiveSum and cub::DeviceRadixSort::SortPairs on bits [0, 32 + msb(T))).
+//
+// Wave64 design notes
+//  * scan: 2048 counts per 256-lane block, lane-local sums + wave prefix by cross-lane shifts + LDS across the 4 waves.
+//  * duplication: one lane per surfel for small rectangles; rectangles above 32 tiles are emitted cooperatively by the
+//    whole wavefront (64 coalesced keys per step) so one huge surfel cannot serialise a wave.
+//  * sort: 8-bit digits. Per pass: block histograms -> per-digit scan over blocks -> scatter. The scatter ranks keys
+//    with 64-bit ballot match masks (8 ballots per round, popcount of the mask below the lane), which is stable by
+//    construction: within a wave lower rounds and lower lanes come first, waves are ordered by an LDS prefix, blocks
+//    by the scanned histogram.
+#include "common.hpp"
+
+namespace fsgs {
+namespace {
+
+constexpr int kScanThreads = 256;
+constexpr int kScanItems   = 8;
+constexpr int kScanChunk   = kScanThreads * kScanItems;
+
+constexpr int kSortThreads = 256;
+constexpr int kSortWaves   = kSortThreads / kWave;
+constexpr int kSortItems   = 8;                          // keys per lane
+constexpr int kSortChunk   = kSortThreads * kSortItems;  // keys per block
+constexpr int kRadixBits   = 8;
+constexpr int kRadix       = 1 << kRadixBits;
+
+__device__ __forceinline__ unsigned long long lanemask_lt() {
+  const unsigned lane = __lane_id();
+  return lane == 0 ? 0ull : (~0ull >> (64 - lane));
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_inclusive_scan(T v) {
+  const int lane = __lane_id();
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const T o = __shfl_up(v, d, kWave);
+    if (lane >= d) v += o;
+  }
+  return v;
+}
+
+// Block-wide exclusive prefix of one value per thread (256 threads); also returns the block total.
+template <typename T>
+__device__ __forceinline__ T block_exclusive_scan(T v, T* s_wave /*[4]*/, T& total) {
+  const int lane = __lane_id(), wave = threadIdx.x / kWave;
+  const T inc = wave_inclusive_scan(v);
+  if (lane == kWave - 1) s_wave[wave] = inc;
+  __syncthreads();
+  T base = 0;
+  total  = 0;
+#pragma unroll
+  for (int w = 0; w < kScanThreads / kWave; ++w) {
+    const T s = s_wave[w];
+    if (w < wave) base += s;
+    total += s;
+  }
+  __syncthreads();
+  return base + inc - v;
+}
+
+// ---- inclusive scan of tiles_touched (int32) into int64 offsets ----------------------------------------------------
+__global__ void __launch_bounds__(kScanThreads) scan_block_sums_kernel(int P, const int32_t* __restrict__ in,
+                                                                       int64_t* __restrict__ block_sums) {
+  __shared__ int64_t s_wave[kScanThreads / kWave];
+  const int base = blockIdx.x * kScanChunk + threadIdx.x * kScanItems;
+  int64_t sum = 0;
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k)
+    if (base + k < P) sum += in[base + k];
+  int64_t total;
+  block_exclusive_scan<int64_t>(sum, s_wave, total);
+  if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+}
+
+__global__ void __launch_bounds__(kScanThreads) scan_spine_kernel(int n, int64_t* __restrict__ block_sums) {
+  __shared__ int64_t s_wave[kScanThreads / kWave];
+  int64_t carry = 0;
+  for (int start = 0; start < n; start += kScanThreads) {
+    const int i = start + threadIdx.x;
+    const int64_t v = i < n ? block_sums[i] : 0;
+    int64_t total;
+    const int64_t ex = block_exclusive_scan<int64_t>(v, s_wave, total);
+    if (i < n) block_sums[i] = carry + ex;
+    carry += total;
+  }
+}
+
+__global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(int P, const int32_t* __restrict__ in,
+                                                                  const int64_t* __restrict__ block_sums,
+                                                                  int64_t* __restrict__ out) {
+  __shared__ int64_t s_wave[kScanThreads / kWave];
+  const int base = blockIdx.x * kScanChunk + threadIdx.x * kScanItems;
+  int32_t v[kScanItems];
+  int64_t sum = 0;
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    v[k] = base + k < P ? in[base + k] : 0;
+    sum += v[k];
+  }
+  int64_t total;
+  int64_t run = block_sums[blockIdx.x] + block_exclusive_scan<int64_t>(sum, s_wave, total);
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    run += v[k];
+    if (base + k < P) out[base + k] = run;
+  }
+}
+
+// ---- key duplication ------------------------------------------------------------------------------------------------
+constexpr int kCoopThreshold = 32;
+
+__global__ void __launch_bounds__(256) duplicate_keys_kernel(int P, int gx, int gy, const float2* __restrict__ means2D,
+    const float* __restrict__ depths, const int32_t* __restrict__ radii, const int64_t* __restrict__ offsets,
+    uint64_t* __restrict__ keys, int32_t* __restrict__ vals) {
+  const int i    = blockIdx.x * blockDim.x + threadIdx.x;
+  const int lane = __lane_id();
+  int x0 = 0, y0 = 0, w = 0, h = 0;
+  int64_t off    = 0;
+  uint32_t dbits = 0;
+  if (i < P && radii[i] > 0) {
+    const float2 c   = means2D[i];
+    const TileRect r = tile_rect(c.x, c.y, radii[i], gx, gy);
+    x0 = r.x0, y0 = r.y0, w = r.x1 - r.x0, h = r.y1 - r.y0;
+    if (w < 0) w = 0;
+    if (h < 0) h = 0;
+    off   = i == 0 ? 0 : offsets[i - 1];
+    dbits = __float_as_uint(depths[i]);
+  }
+  const int count = w * h;
+  if (count > 0 && count <= kCoopThreshold) {
+    for (int y = 0; y < h; ++y)
+      for (int x = 0; x < w; ++x) {
+        keys[off] = ((uint64_t) (uint32_t) ((y0 + y) * gx + (x0 + x)) << 32) | dbits;
+        vals[off] = i;
+        ++off;
+      }
+  }
+  // Large rectangles: the wavefront walks them together, 64 keys per step in row-major tile order.
+  unsigned long long big = __ballot(count > kCoopThreshold);
+  while (big) {
+    const int src = __ffsll((long long) big) - 1;
+    big &= big - 1;
+    const int sx0 = __shfl(x0, src, kWave), sy0 = __shfl(y0, src, kWave), sw = __shfl(w, src, kWave);
+    const int scount = __shfl(count, src, kWave), sid = __shfl(i, src, kWave);
+    const uint32_t sbits = __shfl(dbits, src, kWave);
+    const int64_t soff   = ((int64_t) __shfl((int) (off >> 32), src, kWave) << 32) |
+                         (uint32_t) __shfl((int) (off & 0xffffffff), src, kWave);
+    for (int e = lane; e < scount; e += kWave) {
+      const int y = e / sw, x = e - y * sw;
+      keys[soff + e] = ((uint64_t) (uint32_t) ((sy0 + y) * gx + (sx0 + x)) << 32) | sbits;
+      vals[soff + e] = sid;
+    }
+  }
+}
+
+// ---- radix sort passes ----------------------------------------------------------------------------------------------
+// hist[digit * nblocks + block] = number of keys of `block` whose current digit is `digit`
+__global__ void __launch_bounds__(kSortThreads) sort_histogram_kernel(int64_t R, int shift, int nblocks,
+    const uint64_t* __restrict__ keys, uint32_t* __restrict__ hist) {
+  __shared__ uint32_t s_hist[kRadix];
+  s_hist[threadIdx.x] = 0;
+  __syncthreads();
+  const int64_t base = (int64_t) blockIdx.x * kSortChunk;
+#pragma unroll
+  for (int k = 0; k < kSortItems; ++k) {
+    const int64_t idx = base + k * kSortThreads + threadIdx.x;
+    if (idx < R) atomicAdd(&s_hist[(keys[idx] >> shift) & (kRadix - 1)], 1u);
+  }
+  __syncthreads();
+  hist[(size_t) threadIdx.x * nblocks + blockIdx.x] = s_hist[threadIdx.x];
+}
+
+// One block per digit: exclusive scan of that digit's row over blocks (in place) and the digit total.
+__global__ void __launch_bounds__(kScanThreads) sort_scan_rows_kernel(int nblocks, uint32_t* __restrict__ hist,
+                                                                      uint32_t* __restrict__ digit_totals) {
+  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  uint32_t* row  = hist + (size_t) blockIdx.x * nblocks;
+  uint32_t carry = 0;
+  for (int start = 0; start < nblocks; start += kScanThreads) {
+    const int i = start + threadIdx.x;
+    const uint32_t v = i < nblocks ? row[i] : 0;
+    uint32_t total;
+    const uint32_t ex = block_exclusive_scan<uint32_t>(v, s_wave, total);
+    if (i < nblocks) row[i] = carry + ex;
+    carry += total;
+  }
+  if (threadIdx.x == 0) digit_totals[blockIdx.x] = carry;
+}
+
+__global__ void __launch_bounds__(kSortThreads) sort_scatter_kernel(int64_t R, int shift, int nblocks,
+    const uint64_t* __restrict__ keys_in, const int32_t* __restrict__ vals_in, const uint32_t* __restrict__ hist,
+    const uint32_t* __restrict__ digit_totals, uint64_t* __restrict__ keys_out, int32_t* __restrict__ vals_out) {
+  __shared__ uint32_t s_cnt[kSortWaves][kRadix];  // per-wave running digit counts, then per-wave global bases
+  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  const int lane = __lane_id(), wave = threadIdx.x / kWave;
+#pragma unroll
+  for (int w = 0; w < kSortWaves; ++w) s_cnt[w][threadIdx.x] = 0;
+  // digit base = exclusive scan of digit totals (256 values, one per thread) + this block's offset inside the digit
+  uint32_t total_unused;
+  const uint32_t digit_base = block_exclusive_scan<uint32_t>(digit_totals[threadIdx.x], s_wave, total_unused) +
+                              hist[(size_t) threadIdx.x * nblocks + blockIdx.x];
+  // block_exclusive_scan ends with a barrier, so s_cnt is zeroed for everyone here.
+
+  const int64_t wave_base = (int64_t) blockIdx.x * kSortChunk + (int64_t) wave * (kSortItems * kWave);
+  uint64_t key[kSortItems];
+  int32_t val[kSortItems];
+  uint32_t pos[kSortItems];
+  const unsigned long long lt = lanemask_lt();
+#pragma unroll
+  for (int r = 0; r < kSortItems; ++r) {
+    const int64_t idx = wave_base + r * kWave + lane;
+    const bool valid  = idx < R;
+    key[r] = valid ? keys_in[idx] : 0;
+    val[r] = valid ? vals_in[idx] : 0;
+    const uint32_t d = (uint32_t) (key[r] >> shift) & (kRadix - 1);
+    unsigned long long peers = __ballot(valid);
+#pragma unroll
+    for (int b = 0; b < kRadixBits; ++b) {
+      const unsigned long long m = __ballot((d >> b) & 1u);
+      peers &= ((d >> b) & 1u) ? m : ~m;
+    }
+    const uint32_t rank  = __popcll(peers & lt);
+    const uint32_t count = __popcll(peers);
+    const int leader     = __ffsll((long long) peers) - 1;
+    uint32_t old = 0;
+    if (valid && lane == leader) {
+      old = s_cnt[wave][d];
+      s_cnt[wave][d] = old + count;
+    }
+    old    = __shfl(old, leader < 0 ? 0 : leader, kWave);
+    pos[r] = old + rank;
+  }
+  __syncthreads();
+  {  // turn per-wave counts into per-wave global bases for digit == threadIdx.x
+    uint32_t run = digit_base;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w) {
+      const uint32_t c = s_cnt[w][threadIdx.x];
+      s_cnt[w][threadIdx.x] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < kSortItems; ++r) {
+    const int64_t idx = wave_base + r * kWave + lane;
+    if (idx < R) {
+      const uint32_t d   = (uint32_t) (key[r] >> shift) & (kRadix - 1);
+      const uint32_t dst = s_cnt[wave][d] + pos[r];
+      keys_out[dst] = key[r];
+      vals_out[dst] = val[r];
+    }
+  }
+}
+
+// ---- ranges -----------------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) fill_zero_i64_kernel(int64_t n, int64_t* __restrict__ p) {
+  const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+__global__ void __launch_bounds__(256) tile_ranges_kernel(int64_t R, int num_tiles, const uint64_t* __restrict__ keys,
+                                                          int64_t* __restrict__ ranges) {
+  const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= R) return;
+  const uint32_t cur = (uint32_t) (keys[i] >> 32);
+  const bool cur_ok  = cur < (uint32_t) num_tiles;
+  if (i == 0) {
+    if (cur_ok) ranges[2 * (size_t) cur] = 0;
+  } else {
+    const uint32_t prev = (uint32_t) (keys[i - 1] >> 32);
+    if (cur != prev) {
+      if (prev < (uint32_t) num_tiles) ranges[2 * (size_t) prev + 1] = i;
+      if (cur_ok) ranges[2 * (size_t) cur] = i;
+    }
+  }
+  if (i == R - 1 && cur_ok) ranges[2 * (size_t) cur + 1] = R;
+}
+
+uint32_t higher_msb(uint32_t n) {  // number of bits needed for the tile id, as gaussian_prepare.cu:32-44 computes it
+  uint32_t msb = sizeof(n) * 4, step = msb;
+  while (step > 1) {
+    step /= 2;
+    if (n >> msb) msb += step;
+    else msb -= step;
+  }
+  if (n >> msb) msb++;
+  return msb;
+}
+
+struct SortLayout {
+  int nblocks;
+  size_t keys0, keys1, vals_alt, hist, totals, bytes;
+};
+
+SortLayout sort_layout(int64_t R) {
+  SortLayout L;
+  L.nblocks = div_up(R > 0 ? R : 1, kSortChunk);
+  size_t o  = 0;
+  L.keys0 = o, o = align_up(o + (size_t) R * 8, 256);
+  L.keys1 = o, o = align_up(o + (size_t) R * 8, 256);
+  L.vals_alt = o, o = align_up(o + (size_t) R * 4, 256);
+  L.hist = o, o = align_up(o + (size_t) kRadix * L.nblocks * 4, 256);
+  L.totals = o, o = align_up(o + (size_t) kRadix * 4, 256);
+  L.bytes = o;
+  return L;
+}
+
+}  // namespace
+}  // namespace fsgs
+
+using namespace fsgs;
+
+FSGS_API size_t fsgs_gs_prepare_scan_workspace_bytes(int P) {
+  return align_up((size_t) div_up(P > 0 ? P : 1, kScanChunk) * 8, 256);
+}
+
+FSGS_API int fsgs_gs_prepare_scan(int P, const int32_t* tiles_touched, int64_t* point_offsets, void* workspace,
+                                  size_t workspace_bytes, int64_t* num_rendered_host, void* stream) {
+  FSGS_REQUIRE(P >= 0 && num_rendered_host, "gs_prepare_scan: bad arguments");
+  *num_rendered_host = 0;
+  if (P == 0) return kOk;
+  FSGS_REQUIRE(tiles_touched && point_offsets && workspace, "gs_prepare_scan: null pointer");
+  if (workspace_bytes < fsgs_gs_prepare_scan_workspace_bytes(P))
+    return fail(kWorkspaceSmall, "gs_prepare_scan: workspace %zu < %zu bytes", workspace_bytes,
+                fsgs_gs_prepare_scan_workspace_bytes(P));
+  hipStream_t s     = (hipStream_t) stream;
+  const int nb      = div_up(P, kScanChunk);
+  int64_t* blk_sums = (int64_t*) workspace;
+  hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(kScanThreads), 0, s, P, tiles_touched, blk_sums);
+  hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanThreads), 0, s, nb, blk_sums);
+  hipLaunchKernelGGL(scan_apply_kernel, dim3(nb), dim3(kScanThreads), 0, s, P, tiles_touched, blk_sums,
+                     point_offsets);
+  if (int rc = check_launch("gs_prepare_scan")) return rc;
+  // The number of (surfel, tile) instances sizes the caller's output, so it has to reach the host here
+  // (the reference blocks in the same place, gaussian_prepare.cu:238-239).
+  FSGS_HIP(hipMemcpyAsync(num_rendered_host, point_offsets + (P - 1), sizeof(int64_t), hipMemcpyDeviceToHost, s));
+  FSGS_HIP(hipStreamSynchronize(s));
+  return kOk;
+}
+
+FSGS_API size_t fsgs_gs_prepare_fill_workspace_bytes(int64_t R) { return sort_layout(R).bytes; }
+
+FSGS_API int fsgs_gs_prepare_sort_bits(int W, int H) {
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  return 32 + (int) higher_msb((uint32_t) (gx * gy));
+}
+
+FSGS_API int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths,
+                                  const int32_t* radii, const int64_t* point_offsets, int64_t R, int64_t* ranges,
+                                  int32_t* point_list, int64_t* sorted_keys_out, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && R >= 0 && ranges, "gs_prepare_fill: bad arguments");
+  FSGS_REQUIRE(R < (int64_t) 0x7fffffff, "gs_prepare_fill: %lld instances exceed the 2^31-1 limit", (long long) R);
+  hipStream_t s = (hipStream_t) stream;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const int T  = gx * gy;
+  hipLaunchKernelGGL(fill_zero_i64_kernel, dim3(div_up(2 * (int64_t) T, 256)), dim3(256), 0, s, 2 * (int64_t) T,
+                     ranges);
+  if (R == 0 || P == 0) return check_launch("gs_prepare_fill(zero)");
+  FSGS_REQUIRE(means2D && depths && radii && point_offsets && point_list && workspace,
+               "gs_prepare_fill: null pointer");
+  const SortLayout L = sort_layout(R);
+  if (workspace_bytes < L.bytes)
+    return fail(kWorkspaceSmall, "gs_prepare_fill: workspace %zu < %zu bytes", workspace_bytes, L.bytes);
+  char* ws          = (char*) workspace;
+  uint64_t* kbuf[2] = {(uint64_t*) (ws + L.keys0), (uint64_t*) (ws + L.keys1)};
+  uint32_t* hist    = (uint32_t*) (ws + L.hist);
+  uint32_t* totals  = (uint32_t*) (ws + L.totals);
+  const int bits    = fsgs_gs_prepare_sort_bits(W, H);
+  const int passes  = (bits + kRadixBits - 1) / kRadixBits;
+  // ping-pong so that the last pass lands in point_list
+  int32_t* vbuf[2];
+  vbuf[passes & 1]       = point_list;
+  vbuf[(passes & 1) ^ 1] = (int32_t*) (ws + L.vals_alt);
+
+  hipLaunchKernelGGL(duplicate_keys_kernel, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, (const float2*) means2D,
+                     depths, radii, point_offsets, kbuf[0], vbuf[0]);
+  for (int p = 0; p < passes; ++p) {
+    const int shift = p * kRadixBits;
+    const int a = p & 1, b = a ^ 1;
+    hipLaunchKernelGGL(sort_histogram_kernel, dim3(L.nblocks), dim3(kSortThreads), 0, s, R, shift, L.nblocks, kbuf[a],
+                       hist);
+    hipLaunchKernelGGL(sort_scan_rows_kernel, dim3(kRadix), dim3(kScanThreads), 0, s, L.nblocks, hist, totals);
+    hipLaunchKernelGGL(sort_scatter_kernel, dim3(L.nblocks), dim3(kSortThreads), 0, s, R, shift, L.nblocks, kbuf[a],
+                       vbuf[a], hist, totals, kbuf[b], vbuf[b]);
+  }
+  const uint64_t* sorted = kbuf[passes & 1];
+  hipLaunchKernelGGL(tile_ranges_kernel, dim3(div_up(R, 256)), dim3(256), 0, s, R, T, sorted, ranges);
+  if (sorted_keys_out)
+    FSGS_HIP(hipMemcpyAsync(sorted_keys_out, sorted, (size_t) R * 8, hipMemcpyDeviceToDevice, s));
+  return check_launch("gs_prepare_fill");
+}

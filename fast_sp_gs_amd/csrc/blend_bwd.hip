@@ -1,0 +1,279 @@
+// Per-tile back-to-front backward pass of the 2D-Gaussian-surfel alpha blend for gfx950.
+//
+// Reference behaviour reproduced: fast_2d_gs/_C/src/gaussian_splatting/gs_2d_redner.cu:238-539 (kernel) and :631-717
+// (host entry GS_2D_render_backward). The transmittance is rebuilt by division T <- T / (1 - alpha) while walking the
+// tile's list backwards, gradient channels consumed are image, opacity, aux 0-5 (depth, normal, median depth,
+// distortion) and optional flow; the 0.99 alpha clamp is not masked in the gradient, as in the reference.
+//
+// Where the reference issues 18-21 global float atomics per (pixel, surfel) pair, this kernel
+//   1. sums each of the 18 per-surfel gradient components over the 64 pixels of a wavefront with DPP row shifts and
+//      row broadcasts (no LDS traffic), skipping surfels no pixel of the wavefront blends,
+//   2. adds the 4 wavefront partials of a tile into an LDS accumulator of the staged batch, and
+//   3. flushes one global atomic per surfel, component and tile when the batch retires.
+// Surfels behind the deepest contributor of the whole tile are never gathered.
+#include "blend.hpp"
+
+namespace fsgs {
+namespace {
+
+constexpr int kGradSlots = 18;  // colours 3 | means2D 2 | trans_mat 9 | normal 3 + opacity 1
+
+template <bool kAux, bool kFlow>
+__global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
+    int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    const int32_t* __restrict__ n_contrib, const float2* __restrict__ means2D,
+    const float4* __restrict__ normal_opacity, const float* __restrict__ colors, const float* __restrict__ trans_mat,
+    const float* __restrict__ trans_mat_t2, const float* __restrict__ out_opacity, const float* __restrict__ out_extras,
+    const float2* __restrict__ out_flow, const float* __restrict__ dL_dpix, const float* __restrict__ dL_dextras,
+    const float* __restrict__ dL_dopacity, const float2* __restrict__ dL_dflow, float* __restrict__ g_means2D,
+    float* __restrict__ g_normal_opacity, float* __restrict__ g_colors, float* __restrict__ g_trans) {
+  __shared__ SplatHot s_hot[kBatch];
+  __shared__ SplatCold s_cold[kBatch];
+  __shared__ float s_acc[kBatch][kGradSlots + 1];  // +1: odd stride keeps the flush conflict free
+  __shared__ float s_t2[kFlow ? kBatch * 9 : 1];
+  __shared__ int s_max_contrib;
+
+  const int gx = (W + kTile - 1) / kTile;
+  const int tile = blockIdx.x, tile_x = tile % gx, tile_y = tile / gx;
+  int px, py;
+  lane_pixel(tile_x, tile_y, px, py);
+  const bool inside = px < W && py < H;
+  const size_t HW   = (size_t) H * W;
+  const size_t pix  = (size_t) W * py + px;
+  const float pxf = (float) px, pyf = (float) py;
+  const int lane = threadIdx.x & 63;
+
+  const int64_t r0         = ranges[2 * (size_t) tile];
+  const int last_contrib   = inside ? n_contrib[pix] : 0;
+  const int median_contrib = (kAux && inside) ? n_contrib[pix + HW] : 0;
+
+  // deepest list position any pixel of the tile blended: nothing behind it needs to be gathered
+  if (threadIdx.x == 0) s_max_contrib = 0;
+  __syncthreads();
+  {
+    int m = last_contrib;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) m = max(m, __shfl_xor(m, d, kWave));
+    if (lane == 0) atomicMax(&s_max_contrib, m);
+  }
+#pragma unroll
+  for (int c = 0; c < kGradSlots + 1; ++c) s_acc[threadIdx.x][c] = 0.0f;
+  __syncthreads();
+  const int n_todo = s_max_contrib;  // positions [0, n_todo) of the tile's list, walked from n_todo-1 down to 0
+  const int rounds = (n_todo + kBatch - 1) / kBatch;
+
+  const float T_final = inside ? 1.0f - out_opacity[pix] : 0.0f;
+  float T = T_final;
+  float dLp0 = 0, dLp1 = 0, dLp2 = 0;
+  float dL_dreg = 0, dL_ddepth = 0, dL_daccum = 0, dLn0 = 0, dLn1 = 0, dLn2 = 0, dL_dmedian = 0;
+  float final_D = 0, final_D2 = 0, sum_w = 0;
+  if (inside) {
+    dLp0 = dL_dpix[pix], dLp1 = dL_dpix[pix + HW], dLp2 = dL_dpix[pix + 2 * HW];
+    if (kAux) {
+      dL_daccum  = dL_dopacity[pix];
+      dL_ddepth  = dL_dextras[pix + 0 * HW];
+      dLn0       = dL_dextras[pix + 1 * HW];
+      dLn1       = dL_dextras[pix + 2 * HW];
+      dLn2       = dL_dextras[pix + 3 * HW];
+      dL_dmedian = dL_dextras[pix + 4 * HW];
+      dL_dreg    = dL_dextras[pix + 5 * HW];
+      final_D    = out_extras[pix + 6 * HW];
+      final_D2   = out_extras[pix + 7 * HW];
+      sum_w      = out_extras[pix + 8 * HW];
+    }
+  }
+  const float final_A = 1.0f - T_final;
+  float dLf0 = 0, dLf1 = 0, dL_dsum_w = 0;
+  if (kFlow && inside) {
+    const float2 g = dL_dflow[pix], o = out_flow[pix];
+    dL_dsum_w = -(g.x * o.x + g.y * o.y) / (sum_w * sum_w);
+    dLf0 = g.x / sum_w, dLf1 = g.y / sum_w;
+  }
+
+  float acc_c0 = 0, acc_c1 = 0, acc_c2 = 0, last_c0 = 0, last_c1 = 0, last_c2 = 0;
+  float last_depth = 0, acc_depth = 0, acc_alpha = 0;
+  float last_n0 = 0, last_n1 = 0, last_n2 = 0, acc_n0 = 0, acc_n1 = 0, acc_n2 = 0;
+  float last_dL_dT = 0, last_alpha = 0, acc_w = 0;
+  float acc_f0 = 0, acc_f1 = 0, last_f0 = 0, last_f1 = 0;
+
+  Splat next;
+  float next_t2[9];
+  if ((int) threadIdx.x < n_todo) {
+    next = gather_splat(point_list[r0 + (n_todo - 1 - (int) threadIdx.x)], means2D, colors, normal_opacity, trans_mat);
+    if (kFlow)
+#pragma unroll
+      for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
+  }
+
+  for (int b = 0; b < rounds; ++b) {
+    const int n_here = min(kBatch, n_todo - b * kBatch);
+    if ((int) threadIdx.x < n_here) {
+      s_hot[threadIdx.x]  = next.hot;
+      s_cold[threadIdx.x] = next.cold;
+      if (kFlow)
+#pragma unroll
+        for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
+    }
+    __syncthreads();
+    const int nxt = (b + 1) * kBatch + (int) threadIdx.x;
+    if (nxt < n_todo) {
+      next = gather_splat(point_list[r0 + (n_todo - 1 - nxt)], means2D, colors, normal_opacity, trans_mat);
+      if (kFlow)
+#pragma unroll
+        for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
+    }
+
+    for (int j = 0; j < n_here; ++j) {
+      const int pos = n_todo - 1 - (b * kBatch + j);  // 0-based position in the tile's list
+      Hit h;
+      const bool hit = (pos < last_contrib) && intersect(s_hot[j], pxf, pyf, near_n, h);
+      if (__ballot(hit) == 0ull) continue;  // wave-uniform: nobody in this quadrant blends the surfel
+
+      float g[kGradSlots];
+#pragma unroll
+      for (int c = 0; c < kGradSlots; ++c) g[c] = 0.0f;
+      if (hit) {
+        const SplatHot& hot  = s_hot[j];
+        const SplatCold cold = s_cold[j];
+        T             = T / (1.0f - h.alpha);
+        const float w = h.alpha * T;
+        float dL_dalpha = 0.0f;
+        acc_c0 = last_alpha * last_c0 + (1.0f - last_alpha) * acc_c0, last_c0 = cold.r;
+        acc_c1 = last_alpha * last_c1 + (1.0f - last_alpha) * acc_c1, last_c1 = cold.g;
+        acc_c2 = last_alpha * last_c2 + (1.0f - last_alpha) * acc_c2, last_c2 = cold.b;
+        dL_dalpha += (cold.r - acc_c0) * dLp0 + (cold.g - acc_c1) * dLp1 + (cold.b - acc_c2) * dLp2;
+        g[0] = w * dLp0, g[1] = w * dLp1, g[2] = w * dLp2;
+
+        float dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f;
+        if (kAux) {
+          const float m_d    = far_n / (far_n - near_n) * (1.0f - near_n / h.depth);
+          const float dmd_dd = (far_n * near_n) / ((far_n - near_n) * h.depth * h.depth);
+          if (pos == median_contrib - 1) dL_dz += dL_dmedian;
+          const float dL_dweight = (final_D2 + m_d * m_d * final_A - 2.0f * m_d * final_D) * dL_dreg;
+          dL_dalpha += dL_dweight - last_dL_dT;
+          last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
+          const float dL_dmd = 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg;
+          dL_dz += dL_dmd * dmd_dd;
+          acc_depth  = last_alpha * last_depth + (1.0f - last_alpha) * acc_depth;
+          last_depth = h.depth;
+          dL_dalpha += (h.depth - acc_depth) * dL_ddepth;
+          acc_alpha = last_alpha * 1.0f + (1.0f - last_alpha) * acc_alpha;
+          dL_dalpha += (1.0f - acc_alpha) * dL_daccum;
+          acc_n0 = last_alpha * last_n0 + (1.0f - last_alpha) * acc_n0, last_n0 = cold.nx;
+          acc_n1 = last_alpha * last_n1 + (1.0f - last_alpha) * acc_n1, last_n1 = cold.ny;
+          acc_n2 = last_alpha * last_n2 + (1.0f - last_alpha) * acc_n2, last_n2 = cold.nz;
+          dL_dalpha += (cold.nx - acc_n0) * dLn0 + (cold.ny - acc_n1) * dLn1 + (cold.nz - acc_n2) * dLn2;
+          g[14] = w * dLn0, g[15] = w * dLn1, g[16] = w * dLn2;
+          dL_dz += w * dL_ddepth;
+          dsx = dL_dz * hot.m[6], dsy = dL_dz * hot.m[7];
+        }
+        if (kFlow) {
+          const float* Q = &s_t2[j * 9];
+          const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
+          const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
+          float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
+          w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
+          acc_f0 = last_alpha * last_f0 + (1.0f - last_alpha) * acc_f0;
+          acc_f1 = last_alpha * last_f1 + (1.0f - last_alpha) * acc_f1;
+          last_f0 = u2 / w2 - pxf, last_f1 = v2 / w2 - pyf;
+          dL_dalpha += (last_f0 - acc_f0) * dLf0 + (last_f1 - acc_f1) * dLf1;
+          const float gu = w / w2 * dLf0, gv = w / w2 * dLf1;
+          const float gw = -w / (w2 * w2) * (u2 * dLf0 + v2 * dLf1);
+          dsx += Q[0] * gu + Q[3] * gv + Q[6] * gw;
+          dsy += Q[1] * gu + Q[4] * gv + Q[7] * gw;
+        }
+        acc_w = last_alpha + (1.0f - last_alpha) * acc_w;
+        dL_dalpha += (1.0f - acc_w) * dL_dsum_w;
+        dL_dalpha *= T;
+        last_alpha = h.alpha;
+
+        const float dL_dG = hot.opacity * dL_dalpha;
+        if (h.rho3d <= h.rho2d) {
+          dsx += dL_dG * -h.G * h.sx;
+          dsy += dL_dG * -h.G * h.sy;
+          const float rz  = __builtin_amdgcn_rcpf(h.pz);
+          const float dpx = dsx * rz, dpy = dsy * rz;
+          const float dpz = -(dpx * h.sx + dpy * h.sy);
+          const float dkx = h.ly * dpz - h.lz * dpy, dky = h.lz * dpx - h.lx * dpz, dkz = h.lx * dpy - h.ly * dpx;
+          const float dlx = dpy * h.kz - dpz * h.ky, dly = dpz * h.kx - dpx * h.kz, dlz = dpx * h.ky - dpy * h.kx;
+          g[5] = -dkx, g[6] = -dky, g[7] = -dkz;
+          g[8] = -dlx, g[9] = -dly, g[10] = -dlz;
+          g[11] = pxf * dkx + pyf * dlx + dL_dz * h.sx;
+          g[12] = pxf * dky + pyf * dly + dL_dz * h.sy;
+          g[13] = pxf * dkz + pyf * dlz + dL_dz;
+        } else {
+          g[3]  = dL_dG * (-h.G * 2.0f * h.dx);
+          g[4]  = dL_dG * (-h.G * 2.0f * h.dy);
+          g[11] = dL_dz * h.sx;
+          g[12] = dL_dz * h.sy;
+          g[13] = dL_dz;
+        }
+        g[17] = h.G * dL_dalpha;
+      }
+#pragma unroll
+      for (int c = 0; c < kGradSlots; ++c) {
+        if (!kAux && c >= 14 && c <= 16) continue;
+        const float s = wave_sum_to_lane63(g[c]);
+        if (lane == 63) atomicAdd(&s_acc[j][c], s);
+      }
+    }
+    __syncthreads();
+    // flush the batch: one global atomic per surfel and component for this tile
+    if ((int) threadIdx.x < n_here) {
+      const int id = s_cold[threadIdx.x].id;
+      float* a     = s_acc[threadIdx.x];
+#pragma unroll
+      for (int c = 0; c < 3; ++c)
+        if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+        if (a[3 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[3 + c]);
+#pragma unroll
+      for (int c = 0; c < 9; ++c)
+        if (a[5 + c] != 0.0f) atomicAdd(&g_trans[9 * (size_t) id + c], a[5 + c]);
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (a[14 + c] != 0.0f) atomicAdd(&g_normal_opacity[4 * (size_t) id + c], a[14 + c]);
+#pragma unroll
+      for (int c = 0; c < kGradSlots; ++c) a[c] = 0.0f;
+    }
+    // No barrier needed here: a lane only touches its own record / accumulator row between this flush and the
+    // barrier that follows the next batch's LDS store.
+  }
+}
+
+}  // namespace
+}  // namespace fsgs
+
+using namespace fsgs;
+
+FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n, const float* means2D,
+    const float* normal_opacity, const float* colors, const float* trans_mat, const float* trans_mat_t2,
+    const float* out_opacity, const float* out_extras, const float* out_flow, const float* dL_dpix,
+    const float* dL_dopacity, const float* dL_dextras, const float* dL_dflow, const int64_t* ranges,
+    const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
+    float* g_normal_opacity, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_render_backward: bad sizes");
+  if (P == 0) return kOk;
+  FSGS_REQUIRE(means2D && normal_opacity && colors && trans_mat && out_opacity && dL_dpix && dL_dopacity && ranges &&
+                   n_contrib && g_colors && g_means2D && g_trans && g_normal_opacity,
+               "GS_2D_render_backward: null pointer");
+  const bool aux  = out_extras && dL_dextras;
+  const bool flow = dL_dflow != nullptr;
+  FSGS_REQUIRE(!flow || (trans_mat_t2 && out_flow && aux),
+               "GS_2D_render_backward: flow gradients need trans_mat_t2, out_flow and the auxiliary maps");
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const dim3 grid(gx * gy), block(kBlendThreads);
+  hipStream_t s = (hipStream_t) stream;
+#define FSGS_LAUNCH_BWD(AUX, FLOW)                                                                                   \
+  hipLaunchKernelGGL((blend_backward_kernel<AUX, FLOW>), grid, block, 0, s, W, H, (float) near_n, (float) far_n,     \
+                     ranges, point_list, n_contrib, (const float2*) means2D, (const float4*) normal_opacity, colors, \
+                     trans_mat, trans_mat_t2, out_opacity, out_extras, (const float2*) out_flow, dL_dpix,            \
+                     dL_dextras, dL_dopacity, (const float2*) dL_dflow, g_means2D, g_normal_opacity, g_colors,       \
+                     g_trans)
+  if (aux && flow) FSGS_LAUNCH_BWD(true, true);
+  else if (aux) FSGS_LAUNCH_BWD(true, false);
+  else FSGS_LAUNCH_BWD(false, false);
+#undef FSGS_LAUNCH_BWD
+  return check_launch("GS_2D_render_backward");
+}

@@ -1,0 +1,183 @@
+// Per-tile front-to-back alpha blend of 2D Gaussian surfels for gfx950.
+//
+// Reference behaviour reproduced: fast_2d_gs/_C/src/gaussian_splatting/gs_2d_redner.cu:28-236 (kernel) and :541-629
+// (host entry GS_2D_render_forward): colour, opacity, the 9 auxiliary maps (depth, normal xyz, median depth,
+// distortion, M1, M2, weight sum), optional flow, n_contrib = (last contributor, median contributor), and the optional
+// accum_max_count / accum_weights_p / accum_weights_count side outputs with their quirks (the arg-max flag is never
+// reset once set, :180-197).
+//
+// Layout: one 256-lane block per 16x16 tile; wavefront w owns an 8x8 pixel quadrant. Surfels of the tile's sorted
+// range are gathered 256 at a time (one per lane, colours included so the blend never goes back to HBM) into LDS as
+// 48-byte "hot" + 32-byte "cold" records; the next batch's gather is issued before the current batch is blended so its
+// HBM latency overlaps the arithmetic. All lanes of a wavefront read the same LDS record (broadcast, conflict free).
+#include "blend.hpp"
+
+namespace fsgs {
+namespace {
+
+template <bool kAux, bool kFlow, bool kAccum>
+__global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
+    int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    const float2* __restrict__ means2D, const float* __restrict__ colors, const float* __restrict__ trans_mat,
+    const float4* __restrict__ normal_opacity, const float* __restrict__ trans_mat_t2, int32_t* __restrict__ n_contrib,
+    float* __restrict__ out_color, float* __restrict__ out_opacity, float* __restrict__ out_extras,
+    float2* __restrict__ out_flow, int32_t* __restrict__ accum_max_count, float* __restrict__ accum_weights_p,
+    int32_t* __restrict__ accum_weights_count) {
+  __shared__ SplatHot s_hot[kBatch];
+  __shared__ SplatCold s_cold[kBatch];
+  __shared__ float s_t2[kFlow ? kBatch * 9 : 1];
+
+  const int gx = (W + kTile - 1) / kTile;
+  const int tile = blockIdx.x, tile_x = tile % gx, tile_y = tile / gx;
+  int px, py;
+  lane_pixel(tile_x, tile_y, px, py);
+  const bool inside = px < W && py < H;
+  const size_t HW   = (size_t) H * W;
+  const size_t pix  = (size_t) W * py + px;
+  const float pxf = (float) px, pyf = (float) py;
+
+  const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
+  const int n_todo = (int) (r1 - r0);
+  const int rounds = (n_todo + kBatch - 1) / kBatch;
+
+  bool done = !inside;
+  float T = 1.0f, C0 = 0, C1 = 0, C2 = 0;
+  float N0 = 0, N1 = 0, N2 = 0, D = 0, M1 = 0, M2 = 0, dist = 0, median = 0, wsum = 0, f0 = 0, f1 = 0;
+  int last = 0, median_c = -1, wmax_id = -1;
+  float wmax = 0;
+  bool flag  = false;
+
+  Splat next;
+  float next_t2[9];
+  if (threadIdx.x < n_todo) {
+    next = gather_splat(point_list[r0 + threadIdx.x], means2D, colors, normal_opacity, trans_mat);
+    if (kFlow)
+#pragma unroll
+      for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
+  }
+
+  for (int b = 0; b < rounds; ++b) {
+    // everyone has finished reading the previous batch; leave as soon as no pixel of the tile is still blending
+    if (__syncthreads_count(done) == kBlendThreads) break;
+    const int n_here = min(kBatch, n_todo - b * kBatch);
+    if ((int) threadIdx.x < n_here) {
+      s_hot[threadIdx.x]  = next.hot;
+      s_cold[threadIdx.x] = next.cold;
+      if (kFlow)
+#pragma unroll
+        for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
+    }
+    __syncthreads();
+    const int nxt = (b + 1) * kBatch + threadIdx.x;
+    if (nxt < n_todo) {
+      next = gather_splat(point_list[r0 + nxt], means2D, colors, normal_opacity, trans_mat);
+      if (kFlow)
+#pragma unroll
+        for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
+    }
+
+    for (int j = 0; !done && j < n_here; ++j) {
+      Hit h;
+      if (!intersect(s_hot[j], pxf, pyf, near_n, h)) continue;
+      const float test_T = T * (1.0f - h.alpha);
+      if (test_T < 0.0001f) {
+        done = true;
+        continue;
+      }
+      const float w        = h.alpha * T;
+      const SplatCold cold = s_cold[j];
+      const int contributor = b * kBatch + j + 1;
+      if (kAux) {
+        const float A = 1.0f - T;
+        const float m = far_n / (far_n - near_n) * (1.0f - near_n / h.depth);
+        dist += (m * m * A + M2 - 2.0f * m * M1) * w;
+        D += h.depth * w;
+        M1 += m * w;
+        M2 += m * m * w;
+        if (T > 0.5f) median = h.depth, median_c = contributor;
+        N0 += cold.nx * w, N1 += cold.ny * w, N2 += cold.nz * w;
+        if (kAccum) {
+          if (wmax < w) wmax = w, wmax_id = cold.id, flag = true;
+          if (accum_weights_p) atomicAdd(&accum_weights_p[cold.id], w);
+          if (accum_weights_count) atomicAdd(&accum_weights_count[cold.id], 1);
+        }
+        if (kFlow) {
+          const float* Q = &s_t2[j * 9];
+          const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
+          const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
+          float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
+          w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
+          f0 += (u2 / w2 - pxf) * w;
+          f1 += (v2 / w2 - pyf) * w;
+        }
+        wsum += w;
+      }
+      if (kAccum) {
+        if (flag && accum_max_count) atomicAdd(&accum_max_count[wmax_id], 1);
+      }
+      C0 += cold.r * w, C1 += cold.g * w, C2 += cold.b * w;
+      T    = test_T;
+      last = contributor;
+    }
+  }
+
+  if (inside) {
+    out_opacity[pix]      = 1.0f - T;
+    n_contrib[pix]        = last;
+    n_contrib[pix + HW]   = kAux ? median_c : 0;
+    out_color[pix]        = C0;
+    out_color[pix + HW]   = C1;
+    out_color[pix + 2 * HW] = C2;
+    if (kAux) {
+      out_extras[pix + 0 * HW] = D;
+      out_extras[pix + 1 * HW] = N0;
+      out_extras[pix + 2 * HW] = N1;
+      out_extras[pix + 3 * HW] = N2;
+      out_extras[pix + 4 * HW] = median;
+      out_extras[pix + 5 * HW] = dist;
+      out_extras[pix + 6 * HW] = M1;
+      out_extras[pix + 7 * HW] = M2;
+      out_extras[pix + 8 * HW] = wsum;
+      if (kFlow) {
+        const float ws = wsum == 0.0f ? 1e-7f : wsum;
+        out_flow[pix]  = make_float2(f0 / ws, f1 / ws);
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace fsgs
+
+using namespace fsgs;
+
+FSGS_API int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, double far_n, int only_image,
+    const float* means2D, const float* colors, const float* normal_opacity, const float* trans_mat,
+    const int32_t* point_list, const int64_t* ranges, const float* trans_mat_t2, int32_t* accum_max_count,
+    float* accum_weights_p, int32_t* accum_weights_count, float* out_color, float* out_opacity, float* out_extras,
+    float* out_flow, int32_t* n_contrib, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_render_forward: bad sizes");
+  FSGS_REQUIRE(ranges && out_color && out_opacity && n_contrib, "GS_2D_render_forward: null pointer");
+  FSGS_REQUIRE(P == 0 || (means2D && colors && normal_opacity && trans_mat),
+               "GS_2D_render_forward: null surfel tensor");
+  FSGS_REQUIRE(only_image || out_extras, "GS_2D_render_forward: out_extras is required unless only_image");
+  const bool aux   = !only_image;
+  const bool flow  = aux && trans_mat_t2 != nullptr;
+  const bool accum = aux && (accum_max_count || accum_weights_p || accum_weights_count);
+  FSGS_REQUIRE(!flow || out_flow, "GS_2D_render_forward: out_flow is required with trans_mat_t2");
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const dim3 grid(gx * gy), block(kBlendThreads);
+  hipStream_t s = (hipStream_t) stream;
+#define FSGS_LAUNCH_FWD(AUX, FLOW, ACC)                                                                              \
+  hipLaunchKernelGGL((blend_forward_kernel<AUX, FLOW, ACC>), grid, block, 0, s, W, H, (float) near_n, (float) far_n, \
+                     ranges, point_list, (const float2*) means2D, colors, trans_mat, (const float4*) normal_opacity, \
+                     trans_mat_t2, n_contrib, out_color, out_opacity, out_extras, (float2*) out_flow,                \
+                     accum_max_count, accum_weights_p, accum_weights_count)
+  if (!aux) FSGS_LAUNCH_FWD(false, false, false);
+  else if (flow && accum) FSGS_LAUNCH_FWD(true, true, true);
+  else if (flow) FSGS_LAUNCH_FWD(true, true, false);
+  else if (accum) FSGS_LAUNCH_FWD(true, false, true);
+  else FSGS_LAUNCH_FWD(true, false, false);
+#undef FSGS_LAUNCH_FWD
+  return check_launch("GS_2D_render_forward");
+}

@@ -1,0 +1,423 @@
+// 2D-Gaussian-surfel preprocess for gfx950: ray-splat transform, screen-space bound, tile rectangle, SH -> RGB,
+// and the matching backward. One lane per surfel; pure HBM streaming.
+//
+// Reference behaviour reproduced: fast_2d_gs/_C/src/gaussian_splatting/gs_2d_preprocess.cu:24-329.
+// The geometric part (transform, bound, radius, rectangle) is compiled with floating-point contraction off and in the
+// reference's operation order, so radii / tiles_touched / means2D / trans_mat / depths are reproducible bit for bit
+// against a plain IEEE evaluation of the same expressions.
+#include "common.hpp"
+#include "sh.hpp"
+
+namespace fsgs {
+namespace {
+
+#pragma clang fp contract(off)
+
+struct Mat4 {
+  float m[16];
+};
+
+__device__ __forceinline__ void mat4_mul(const float* A, const float* B, float* C) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      C[i * 4 + j] = A[i * 4 + 0] * B[0 * 4 + j] + A[i * 4 + 1] * B[1 * 4 + j] + A[i * 4 + 2] * B[2 * 4 + j] +
+                     A[i * 4 + 3] * B[3 * 4 + j];
+}
+
+__device__ __forceinline__ void ndc2pix(int W, int H, float* N) {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) N[i] = 0.0f;
+  N[0] = (float) (0.5 * W), N[3] = (float) (0.5 * (W - 1));
+  N[5] = (float) (0.5 * H), N[7] = (float) (0.5 * (H - 1));
+  N[11] = 1.0f, N[15] = 1.0f;
+}
+
+// Block-wide: Tw2c = Tv2c * Tw2v into shared memory (the reference does this product with a device matmul on the
+// host side, gs_2d_preprocess.cu:381).
+__device__ __forceinline__ void load_camera(const float* __restrict__ Tw2v, const float* __restrict__ Tv2c,
+                                            float* s_Tw2v, float* s_Tw2c) {
+  const int t = threadIdx.x;
+  if (t < 16) {
+    const int i = t >> 2, j = t & 3;
+    s_Tw2v[t] = Tw2v[t];
+    s_Tw2c[t] = Tv2c[i * 4 + 0] * Tw2v[0 * 4 + j] + Tv2c[i * 4 + 1] * Tw2v[1 * 4 + j] +
+                Tv2c[i * 4 + 2] * Tw2v[2 * 4 + j] + Tv2c[i * 4 + 3] * Tw2v[3 * 4 + j];
+  }
+  __syncthreads();
+}
+
+__device__ __forceinline__ void transmat(int W, int H, const float* p, float sx, float sy, const float4 q,
+                                         const float* Tw2c, const float* Tw2v, float* M, float* nrm) {
+  float L[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) L[i] = 0.0f;
+  const float x = q.x, y = q.y, z = q.z, w = q.w;
+  L[0]  = (1 - 2 * (y * y + z * z)) * sx;
+  L[1]  = 2 * (x * y - z * w) * sy;
+  L[2]  = p[0];
+  L[4]  = (2 * (x * y + z * w)) * sx;
+  L[5]  = (1 - 2 * (x * x + z * z)) * sy;
+  L[6]  = p[1];
+  L[8]  = (2 * (x * z - y * w)) * sx;
+  L[9]  = 2 * (x * w + y * z) * sy;
+  L[10] = p[2];
+  L[14] = 1.0f;
+  const float t0 = 2 * (y * w + x * z), t1 = 2 * (y * z - x * w), t2 = 1 - 2 * (x * x + y * y);
+  float N[16], A[16], B[16];
+  ndc2pix(W, H, N);
+  mat4_mul(Tw2c, L, A);
+  mat4_mul(N, A, B);
+#pragma unroll
+  for (int i = 0; i < 3; ++i)
+#pragma unroll
+    for (int j = 0; j < 3; ++j) M[i * 3 + j] = B[i * 4 + j];
+  nrm[0] = Tw2v[0] * t0 + Tw2v[1] * t1 + Tw2v[2] * t2;
+  nrm[1] = Tw2v[4] * t0 + Tw2v[5] * t1 + Tw2v[6] * t2;
+  nrm[2] = Tw2v[8] * t0 + Tw2v[9] * t1 + Tw2v[10] * t2;
+}
+
+__device__ __forceinline__ bool bound_3sigma(const float* M, float* c, float* ext) {
+  const float t0 = 9.0f, t1 = 9.0f, t2 = -1.0f;
+  const float d  = t0 * (M[6] * M[6]) + t1 * (M[7] * M[7]) + t2 * (M[8] * M[8]);
+  if (d == 0.0f) return false;
+  const float inv = 1 / d;
+  const float f0 = inv * t0, f1 = inv * t1, f2 = inv * t2;
+  const float px = f0 * (M[0] * M[6]) + f1 * (M[1] * M[7]) + f2 * (M[2] * M[8]);
+  const float py = f0 * (M[3] * M[6]) + f1 * (M[4] * M[7]) + f2 * (M[5] * M[8]);
+  const float hx = px * px - (f0 * (M[0] * M[0]) + f1 * (M[1] * M[1]) + f2 * (M[2] * M[2]));
+  const float hy = py * py - (f0 * (M[3] * M[3]) + f1 * (M[4] * M[4]) + f2 * (M[5] * M[5]));
+  c[0] = px, c[1] = py;
+  ext[0] = sqrtf(fmaxf(1e-4f, hx));
+  ext[1] = sqrtf(fmaxf(1e-4f, hy));
+  return true;
+}
+
+__global__ void __launch_bounds__(256) preprocess_forward_kernel(
+    int P, int W, int H, int sh_degree, int n_sh, const float* __restrict__ means3D, const float2* __restrict__ scales,
+    const float4* __restrict__ rotations, const float* __restrict__ opacities, const float* __restrict__ shs,
+    const float* __restrict__ sh_rest, const float* __restrict__ Tw2v_g, const float* __restrict__ Tv2c_g,
+    const float* __restrict__ campos, const float* __restrict__ trans_precomp, const uint8_t* __restrict__ culling,
+    int means2D_preserve, float2* __restrict__ means2D, float* __restrict__ colors, float* __restrict__ trans_mat,
+    float4* __restrict__ normal_opacity, float* __restrict__ depths, int32_t* __restrict__ radii,
+    int32_t* __restrict__ tiles_touched) {
+  __shared__ float s_Tw2v[16], s_Tw2c[16];
+  load_camera(Tw2v_g, Tv2c_g, s_Tw2v, s_Tw2c);
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= P) return;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+
+  bool ok = false;
+  float M[9], nrm[3] = {0, 0, 0}, c2[2] = {0, 0}, rgb[3] = {0, 0, 0}, depth = 0, radius = 0;
+  int area = 0;
+#pragma unroll
+  for (int k = 0; k < 9; ++k) M[k] = 0.0f;
+  const float p[3] = {means3D[3 * (size_t) i], means3D[3 * (size_t) i + 1], means3D[3 * (size_t) i + 2]};
+  do {
+    if (culling && culling[i]) break;
+    float Tw2v[16], Tw2c[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) Tw2v[k] = s_Tw2v[k], Tw2c[k] = s_Tw2c[k];
+    const float pv[3] = {Tw2v[0] * p[0] + Tw2v[1] * p[1] + Tw2v[2] * p[2] + Tw2v[3],
+                         Tw2v[4] * p[0] + Tw2v[5] * p[1] + Tw2v[6] * p[2] + Tw2v[7],
+                         Tw2v[8] * p[0] + Tw2v[9] * p[1] + Tw2v[10] * p[2] + Tw2v[11]};
+    if (pv[2] <= 0.2f) break;
+    if (trans_precomp == nullptr) {
+      const float2 s = scales[i];
+      transmat(W, H, p, s.x, s.y, rotations[i], Tw2c, Tw2v, M, nrm);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 9; ++k) M[k] = trans_precomp[9 * (size_t) i + k];
+      nrm[0] = 0.0f, nrm[1] = 0.0f, nrm[2] = 1.0f;
+    }
+    const float cosv = -(pv[0] * nrm[0] + pv[1] * nrm[1] + pv[2] * nrm[2]);
+    if (cosv == 0.0f) break;
+    const float mult = cosv > 0 ? 1.0f : -1.0f;
+    nrm[0] = mult * nrm[0], nrm[1] = mult * nrm[1], nrm[2] = mult * nrm[2];
+    float ext[2];
+    if (!bound_3sigma(M, c2, ext)) break;
+    radius = ceilf(fmaxf(fmaxf(ext[0], ext[1]), 3.0f * 0.707106f));
+    const TileRect r = tile_rect(c2[0], c2[1], f2i_sat(radius), gx, gy);
+    area = (r.y1 - r.y0) * (r.x1 - r.x0);
+    if (area == 0) break;
+    depth = pv[2];
+    ok    = true;
+  } while (false);
+
+  if (ok && sh_degree >= 0) {
+    float x, y, z, Y[16];
+    view_dir(p, campos, x, y, z);
+    sh_eval(sh_degree, x, y, z, Y);
+    const int n = sh_count(sh_degree);
+    const float* c0 = shs + (size_t) i * (sh_rest ? 1 : n_sh) * 3;
+    float r = c0[0] * Y[0], g = c0[1] * Y[0], b = c0[2] * Y[0];
+    const float* cr = sh_rest ? sh_rest + (size_t) i * n_sh * 3 - 3 : c0;
+    for (int l = 1; l < n; ++l) {
+      r += cr[3 * l] * Y[l], g += cr[3 * l + 1] * Y[l], b += cr[3 * l + 2] * Y[l];
+    }
+    rgb[0] = fmaxf(0.0f, r + 0.5f), rgb[1] = fmaxf(0.0f, g + 0.5f), rgb[2] = fmaxf(0.0f, b + 0.5f);
+  }
+
+  if (trans_precomp == nullptr) {
+#pragma unroll
+    for (int k = 0; k < 9; ++k) trans_mat[9 * (size_t) i + k] = ok ? M[k] : 0.0f;
+  }
+  if (sh_degree >= 0) {
+    colors[3 * (size_t) i] = rgb[0], colors[3 * (size_t) i + 1] = rgb[1], colors[3 * (size_t) i + 2] = rgb[2];
+  }
+  depths[i]        = depth;
+  radii[i]         = ok ? f2i_sat(radius) : 0;
+  tiles_touched[i] = ok ? area : 0;
+  if (ok || !means2D_preserve) means2D[i] = ok ? make_float2(c2[0], c2[1]) : make_float2(0.0f, 0.0f);
+  normal_opacity[i] = ok ? make_float4(nrm[0], nrm[1], nrm[2], opacities[i]) : make_float4(0, 0, 0, 0);
+}
+
+__device__ __forceinline__ void bound_backward(const float* M, float g2x, float g2y, float* gM) {
+  const float t[3] = {9.0f, 9.0f, -1.0f};
+  const float d    = t[0] * (M[6] * M[6]) + t[1] * (M[7] * M[7]) + t[2] * (M[8] * M[8]);
+  const float inv  = 1.0f / d;
+  float f[3], df[3];
+#pragma unroll
+  for (int a = 0; a < 3; ++a) f[a] = t[a] * inv;
+  float g0[3], g1[3], gr2[3];
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    g0[a]  = g2x * f[a] * M[6 + a];
+    g1[a]  = g2y * f[a] * M[6 + a];
+    gr2[a] = g2x * f[a] * M[a] + g2y * f[a] * M[3 + a];
+    df[a]  = g2x * M[a] * M[6 + a] + g2y * M[3 + a] * M[6 + a];
+  }
+  const float dd = (df[0] * f[0] + df[1] * f[1] + df[2] * f[2]) * -(1.0f / d);
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    gr2[a] += dd * (t[a] * M[6 + a] * 2.0f);
+    gM[a] += g0[a];
+    gM[3 + a] += g1[a];
+    gM[6 + a] += gr2[a];
+  }
+}
+
+__device__ __forceinline__ void transmat_backward(int W, int H, float sx, float sy, const float4 q, const float* Tw2c,
+                                                  const float* Tw2v, const float* gM, const float* gN, float* gp,
+                                                  float* gs, float* gq) {
+  float N[16], G[16], GL[16], dR[16];
+  ndc2pix(W, H, N);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) G[i] = 0.0f, GL[i] = 0.0f, dR[i] = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 3; ++i)
+#pragma unroll
+    for (int j = 0; j < 3; ++j) G[i * 4 + j] = gM[i * 3 + j];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) GL[i * 4 + j] += N[k * 4 + i] * G[k * 4 + j];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) dR[i * 4 + j] += Tw2c[k * 4 + i] * GL[k * 4 + j];
+  gp[0] = dR[2], gp[1] = dR[6], gp[2] = dR[10];
+  dR[2]  = gN[0] * Tw2v[0] + gN[1] * Tw2v[4] + gN[2] * Tw2v[8];
+  dR[6]  = gN[0] * Tw2v[1] + gN[1] * Tw2v[5] + gN[2] * Tw2v[9];
+  dR[10] = gN[0] * Tw2v[2] + gN[1] * Tw2v[6] + gN[2] * Tw2v[10];
+  const float x = q.x, y = q.y, z = q.z, w = q.w;
+  gs[0] = dR[0] * (1 - 2 * (y * y + z * z)) + dR[4] * (2 * (x * y + z * w)) + dR[8] * (2 * (x * z - y * w));
+  gs[1] = dR[1] * (2 * (x * y - z * w)) + dR[5] * (1 - 2 * (x * x + z * z)) + dR[9] * (2 * (x * w + y * z));
+  dR[0] *= sx, dR[1] *= sy, dR[4] *= sx, dR[5] *= sy, dR[8] *= sx, dR[9] *= sy;
+  gq[0] = 2 * (-2 * x * (dR[5] + dR[10]) + y * (dR[1] + dR[4]) + z * (dR[2] + dR[8]) + w * (dR[9] - dR[6]));
+  gq[1] = 2 * (x * (dR[1] + dR[4]) - 2 * y * (dR[0] + dR[10]) + z * (dR[6] + dR[9]) + w * (dR[2] - dR[8]));
+  gq[2] = 2 * (x * (dR[2] + dR[8]) + y * (dR[6] + dR[9]) - 2 * z * (dR[0] + dR[5]) + w * (dR[4] - dR[1]));
+  gq[3] = 2 * (x * (dR[9] - dR[6]) + y * (dR[2] - dR[8]) + z * (dR[4] - dR[1]));
+}
+
+__global__ void __launch_bounds__(256) preprocess_backward_kernel(
+    int P, int W, int H, int sh_degree, int n_sh, const float* __restrict__ means3D, const float2* __restrict__ scales,
+    const float4* __restrict__ rotations, const float* __restrict__ shs, const float* __restrict__ sh_rest,
+    const float* __restrict__ Tw2v_g, const float* __restrict__ Tv2c_g, const float* __restrict__ campos,
+    const float* __restrict__ trans_mat, const int32_t* __restrict__ radii, const float* __restrict__ colors,
+    float2* __restrict__ grad_mean2D, const float* __restrict__ grad_trans, const float* __restrict__ grad_colors,
+    const float4* __restrict__ grad_normal_opacity, float* __restrict__ g_means3D, float2* __restrict__ g_scales,
+    float4* __restrict__ g_rot, float* __restrict__ g_opac, float* __restrict__ g_shs,
+    float* __restrict__ g_sh_rest) {
+  __shared__ float s_Tw2v[16], s_Tw2c[16];
+  load_camera(Tw2v_g, Tv2c_g, s_Tw2v, s_Tw2c);
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= P || radii[i] <= 0) return;
+  float Tw2v[16], Tw2c[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) Tw2v[k] = s_Tw2v[k], Tw2c[k] = s_Tw2c[k];
+
+  const float4 gno = grad_normal_opacity[i];
+  g_opac[i]        = gno.w;
+  float gM[9], M[9], gM_in2, gM_in5;
+#pragma unroll
+  for (int k = 0; k < 9; ++k) gM[k] = grad_trans[9 * (size_t) i + k], M[k] = trans_mat[9 * (size_t) i + k];
+  gM_in2 = gM[2], gM_in5 = gM[5];
+  const float2 g2 = grad_mean2D[i];
+  bound_backward(M, g2.x, g2.y, gM);
+
+  const float4 q   = rotations[i];
+  const float p[3] = {means3D[3 * (size_t) i], means3D[3 * (size_t) i + 1], means3D[3 * (size_t) i + 2]};
+  const float t0 = 2 * (q.y * q.w + q.x * q.z), t1 = 2 * (q.y * q.z - q.x * q.w), t2 = 1 - 2 * (q.x * q.x + q.y * q.y);
+  const float nrm[3] = {Tw2v[0] * t0 + Tw2v[1] * t1 + Tw2v[2] * t2, Tw2v[4] * t0 + Tw2v[5] * t1 + Tw2v[6] * t2,
+                        Tw2v[8] * t0 + Tw2v[9] * t1 + Tw2v[10] * t2};
+  const float pv[3] = {Tw2v[0] * p[0] + Tw2v[1] * p[1] + Tw2v[2] * p[2] + Tw2v[3],
+                       Tw2v[4] * p[0] + Tw2v[5] * p[1] + Tw2v[6] * p[2] + Tw2v[7],
+                       Tw2v[8] * p[0] + Tw2v[9] * p[1] + Tw2v[10] * p[2] + Tw2v[11]};
+  const float cosv = -(pv[0] * nrm[0] + pv[1] * nrm[1] + pv[2] * nrm[2]);
+  const float mult = cosv > 0 ? 1.0f : -1.0f;
+  const float gN[3] = {mult * gno.x, mult * gno.y, mult * gno.z};
+  const float2 s = scales[i];
+  float gp[3], gs[2], gq[4];
+  transmat_backward(W, H, s.x, s.y, q, Tw2c, Tw2v, gM, gN, gp, gs, gq);
+
+  if (sh_degree >= 0) {
+    float x, y, z, Y[16], tl[16];
+    const float nn = view_dir(p, campos, x, y, z);
+    sh_eval(sh_degree, x, y, z, Y);
+    float g[3];
+#pragma unroll
+    for (int c = 0; c < 3; ++c) g[c] = grad_colors[3 * (size_t) i + c] * (float) (colors[3 * (size_t) i + c] > 0);
+    const int n  = sh_count(sh_degree);
+    const int m1 = sh_rest ? 1 : n_sh;
+    const float* c0 = shs + (size_t) i * m1 * 3;
+    const float* cr = sh_rest ? sh_rest + (size_t) i * n_sh * 3 - 3 : c0;
+    float* o0 = g_shs ? g_shs + (size_t) i * m1 * 3 : nullptr;
+    float* orr = g_sh_rest ? g_sh_rest + (size_t) i * n_sh * 3 - 3 : o0;
+    if (o0) o0[0] = g[0] * Y[0], o0[1] = g[1] * Y[0], o0[2] = g[2] * Y[0];
+    tl[0] = 0.0f;
+    for (int l = 1; l < n; ++l) {
+      tl[l] = g[0] * cr[3 * l] + g[1] * cr[3 * l + 1] + g[2] * cr[3 * l + 2];
+      if (o0) orr[3 * l] = g[0] * Y[l], orr[3 * l + 1] = g[1] * Y[l], orr[3 * l + 2] = g[2] * Y[l];
+    }
+    float dx = 0, dy = 0, dz = 0;
+    sh_grad_accumulate(sh_degree, x, y, z, tl, dx, dy, dz);
+    const float vx = p[0] - campos[0], vy = p[1] - campos[1], vz = p[2] - campos[2];
+    const float tt = -(vx * dx + vy * dy + vz * dz) * nn * nn * nn;
+    gp[0] = gp[0] + (dx * nn + tt * vx);
+    gp[1] = gp[1] + (dy * nn + tt * vy);
+    gp[2] = gp[2] + (dz * nn + tt * vz);
+  }
+  g_means3D[3 * (size_t) i] = gp[0], g_means3D[3 * (size_t) i + 1] = gp[1], g_means3D[3 * (size_t) i + 2] = gp[2];
+  g_scales[i] = make_float2(gs[0], gs[1]);
+  g_rot[i]    = make_float4(gq[0], gq[1], gq[2], gq[3]);
+  // densification proxy written over the incoming screen-space gradient (gs_2d_preprocess.cu:325-328)
+  const float depth = M[8];
+  grad_mean2D[i] = make_float2(gM_in2 * depth * 0.5f * (float) W, gM_in5 * depth * 0.5f * (float) H);
+}
+
+__global__ void __launch_bounds__(256) transmat_forward_kernel(int P, int W, int H, const float* __restrict__ means3D,
+    const float2* __restrict__ scales, const float4* __restrict__ rotations, const float* __restrict__ Tw2v_g,
+    const float* __restrict__ Tw2c_g, float* __restrict__ trans_mat, float* __restrict__ normals) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= P) return;
+  float Tw2v[16], Tw2c[16], M[9], nrm[3];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) Tw2v[k] = Tw2v_g[k], Tw2c[k] = Tw2c_g[k];
+  const float p[3] = {means3D[3 * (size_t) i], means3D[3 * (size_t) i + 1], means3D[3 * (size_t) i + 2]};
+  const float2 s = scales[i];
+  transmat(W, H, p, s.x, s.y, rotations[i], Tw2c, Tw2v, M, nrm);
+#pragma unroll
+  for (int k = 0; k < 9; ++k) trans_mat[9 * (size_t) i + k] = M[k];
+#pragma unroll
+  for (int k = 0; k < 3; ++k) normals[3 * (size_t) i + k] = nrm[k];
+}
+
+__global__ void __launch_bounds__(256) transmat_backward_kernel(int P, int W, int H, const float2* __restrict__ scales,
+    const float4* __restrict__ rotations, const float* __restrict__ Tw2v_g, const float* __restrict__ Tw2c_g,
+    const float* __restrict__ g_mat, const float* __restrict__ g_normals, float* __restrict__ g_means3D,
+    float2* __restrict__ g_scales, float4* __restrict__ g_rot) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= P) return;
+  float Tw2v[16], Tw2c[16], gM[9], gN[3], gp[3], gs[2], gq[4];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) Tw2v[k] = Tw2v_g[k], Tw2c[k] = Tw2c_g[k];
+#pragma unroll
+  for (int k = 0; k < 9; ++k) gM[k] = g_mat[9 * (size_t) i + k];
+#pragma unroll
+  for (int k = 0; k < 3; ++k) gN[k] = g_normals[3 * (size_t) i + k];
+  const float2 s = scales[i];
+  transmat_backward(W, H, s.x, s.y, rotations[i], Tw2c, Tw2v, gM, gN, gp, gs, gq);
+#pragma unroll
+  for (int k = 0; k < 3; ++k) g_means3D[3 * (size_t) i + k] = gp[k];
+  g_scales[i] = make_float2(gs[0], gs[1]);
+  g_rot[i]    = make_float4(gq[0], gq[1], gq[2], gq[3]);
+}
+
+}  // namespace
+}  // namespace fsgs
+
+using namespace fsgs;
+
+FSGS_API int fsgs_gs_2d_preprocess_forward(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
+    const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
+    const float* Tw2v, const float* Tv2c, const float* campos, const float* trans_precomp, const uint8_t* culling,
+    int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* normal_opacity, float* depths,
+    int32_t* radii, int32_t* tiles_touched, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "gs_2d_preprocess_forward: bad sizes P=%d W=%d H=%d", P, W, H);
+  FSGS_REQUIRE(sh_degree <= kMaxShDegree, "gs_2d_preprocess_forward: sh_degree %d > %d not supported", sh_degree,
+               kMaxShDegree);
+  if (sh_degree >= 0)
+    FSGS_REQUIRE(n_sh + (sh_rest ? 1 : 0) >= (sh_degree + 1) * (sh_degree + 1),
+                 "gs_2d_preprocess_forward: %d SH coefficients are too few for degree %d", n_sh, sh_degree);
+  FSGS_REQUIRE(means3D && scales && rotations && opacities && shs && Tw2v && Tv2c && campos && means2D &&
+                   normal_opacity && depths && radii && tiles_touched && (trans_mat || trans_precomp) &&
+                   (colors || sh_degree < 0),
+               "gs_2d_preprocess_forward: null pointer");
+  if (P == 0) return kOk;
+  hipLaunchKernelGGL(preprocess_forward_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H,
+                     sh_degree, n_sh, means3D, (const float2*) scales, (const float4*) rotations, opacities, shs,
+                     sh_rest, Tw2v, Tv2c, campos, trans_precomp, culling, means2D_preserve, (float2*) means2D, colors,
+                     trans_mat, (float4*) normal_opacity, depths, radii, tiles_touched);
+  return check_launch("gs_2d_preprocess_forward");
+}
+
+FSGS_API int fsgs_gs_2d_preprocess_backward(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
+    const float* scales, const float* rotations, const float* shs, const float* sh_rest, const float* Tw2v,
+    const float* Tv2c, const float* campos, const float* trans_mat, const int32_t* radii, const float* colors,
+    float* grad_mean2D, const float* grad_trans, const float* grad_colors, const float* grad_normal_opacity,
+    float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs, float* g_sh_rest, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "gs_2d_preprocess_backward: bad sizes");
+  FSGS_REQUIRE(sh_degree <= kMaxShDegree, "gs_2d_preprocess_backward: sh_degree %d > %d not supported", sh_degree,
+               kMaxShDegree);
+  FSGS_REQUIRE(means3D && scales && rotations && Tw2v && Tv2c && campos && trans_mat && radii && grad_mean2D &&
+                   grad_trans && grad_normal_opacity && g_means3D && g_scales && g_rot && g_opac,
+               "gs_2d_preprocess_backward: null pointer");
+  if (sh_degree >= 0)
+    FSGS_REQUIRE(shs && colors && grad_colors, "gs_2d_preprocess_backward: SH path needs shs, colors and grad_colors");
+  if (P == 0) return kOk;
+  hipLaunchKernelGGL(preprocess_backward_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H,
+                     sh_degree, n_sh, means3D, (const float2*) scales, (const float4*) rotations, shs, sh_rest, Tw2v,
+                     Tv2c, campos, trans_mat, radii, colors, (float2*) grad_mean2D, grad_trans, grad_colors,
+                     (const float4*) grad_normal_opacity, g_means3D, (float2*) g_scales, (float4*) g_rot, g_opac,
+                     g_shs, g_sh_rest);
+  return check_launch("gs_2d_preprocess_backward");
+}
+
+FSGS_API int fsgs_gs_2d_compute_transmat_forward(int P, int W, int H, const float* means3D, const float* scales,
+    const float* rotations, const float* Tw2v, const float* Tw2c, float* trans_mat, float* normals, void* stream) {
+  FSGS_REQUIRE(P >= 0 && means3D && scales && rotations && Tw2v && Tw2c && trans_mat && normals,
+               "gs_2d_compute_transmat_forward: bad arguments");
+  if (P == 0) return kOk;
+  hipLaunchKernelGGL(transmat_forward_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H,
+                     means3D, (const float2*) scales, (const float4*) rotations, Tw2v, Tw2c, trans_mat, normals);
+  return check_launch("gs_2d_compute_transmat_forward");
+}
+
+FSGS_API int fsgs_gs_2d_compute_transmat_backward(int P, int W, int H, const float* means3D, const float* scales,
+    const float* rotations, const float* Tw2v, const float* Tw2c, const float* g_mat, const float* g_normals,
+    float* g_means3D, float* g_scales, float* g_rot, void* stream) {
+  (void) means3D;
+  FSGS_REQUIRE(P >= 0 && scales && rotations && Tw2v && Tw2c && g_mat && g_normals && g_means3D && g_scales && g_rot,
+               "gs_2d_compute_transmat_backward: bad arguments");
+  if (P == 0) return kOk;
+  hipLaunchKernelGGL(transmat_backward_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H,
+                     (const float2*) scales, (const float4*) rotations, Tw2v, Tw2c, g_mat, g_normals, g_means3D,
+                     (float2*) g_scales, (float4*) g_rot);
+  return check_launch("gs_2d_compute_transmat_backward");
+}

@@ -1,0 +1,84 @@
+// Device-side real spherical harmonics (degree 0..3) in the reference's convention
+// (fast_2d_gs/_C/include/spherical_harmonic.h:40-79): l=1 is (-y, +z, -x), colours get +0.5 and a clamp at 0.
+// Values and Cartesian gradients are produced into register arrays so callers can fuse them with coefficient
+// loads of any layout.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace fsgs {
+
+constexpr int kMaxShDegree = 3;
+
+__device__ __forceinline__ int sh_count(int degree) { return (degree + 1) * (degree + 1); }
+
+// Y must hold 16 floats; entries beyond (degree+1)^2 are left untouched.
+__device__ __forceinline__ void sh_eval(int degree, float x, float y, float z, float* __restrict__ Y) {
+  Y[0] = 0.28209479177387814f;
+  if (degree < 1) return;
+  Y[1] = -0.48860251190291987f * y;
+  Y[2] = 0.48860251190291987f * z;
+  Y[3] = -0.48860251190291987f * x;
+  if (degree < 2) return;
+  const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
+  Y[4] = 1.0925484305920792f * xy;
+  Y[5] = -1.0925484305920792f * yz;
+  Y[6] = 0.94617469575755997f * zz - 0.31539156525251999f;
+  Y[7] = -1.0925484305920792f * xz;
+  Y[8] = 0.54627421529603959f * xx - 0.54627421529603959f * yy;
+  if (degree < 3) return;
+  Y[9]  = 0.59004358992664352f * y * (-3.0f * xx + yy);
+  Y[10] = 2.8906114426405538f * xy * z;
+  Y[11] = 0.45704579946446572f * y * (1.0f - 5.0f * zz);
+  Y[12] = 0.3731763325901154f * z * (5.0f * zz - 3.0f);
+  Y[13] = 0.45704579946446572f * x * (1.0f - 5.0f * zz);
+  Y[14] = 1.4453057213202769f * z * (xx - yy);
+  Y[15] = 0.59004358992664352f * x * (-xx + 3.0f * yy);
+}
+
+// Accumulates t_l * grad(Y_l) for l >= 1 into (dx, dy, dz); t[l] is the caller's per-basis scalar
+// (dot(grad_rgb, coeff_l) for SH->RGB, the upstream gradient for the bare encoder).
+__device__ __forceinline__ void sh_grad_accumulate(int degree, float x, float y, float z, const float* __restrict__ t,
+                                                   float& dx, float& dy, float& dz) {
+  if (degree < 1) return;
+  dy += t[1] * -0.48860251190291992f;
+  dz += t[2] * 0.48860251190291992f;
+  dx += t[3] * -0.48860251190291992f;
+  if (degree < 2) return;
+  const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
+  dx += t[4] * (1.0925484305920792f * y);
+  dy += t[4] * (1.0925484305920792f * x);
+  dy += t[5] * (-1.0925484305920792f * z);
+  dz += t[5] * (-1.0925484305920792f * y);
+  dz += t[6] * (1.8923493915151202f * z);
+  dx += t[7] * (-1.0925484305920792f * z);
+  dz += t[7] * (-1.0925484305920792f * x);
+  dx += t[8] * (1.0925484305920792f * x);
+  dy += t[8] * (-1.0925484305920792f * y);
+  if (degree < 3) return;
+  dx += t[9] * (-3.5402615395598609f * xy);
+  dy += t[9] * (-1.7701307697799304f * xx + 1.7701307697799304f * yy);
+  dx += t[10] * (2.8906114426405538f * yz);
+  dy += t[10] * (2.8906114426405538f * xz);
+  dz += t[10] * (2.8906114426405538f * xy);
+  dy += t[11] * (0.45704579946446572f - 2.2852289973223288f * zz);
+  dz += t[11] * (-4.5704579946446566f * yz);
+  dz += t[12] * (5.597644988851731f * zz - 1.1195289977703462f);
+  dx += t[13] * (0.45704579946446572f - 2.2852289973223288f * zz);
+  dz += t[13] * (-4.5704579946446566f * xz);
+  dx += t[14] * (2.8906114426405538f * xz);
+  dy += t[14] * (-2.8906114426405538f * yz);
+  dz += t[14] * (1.4453057213202769f * xx - 1.4453057213202769f * yy);
+  dx += t[15] * (-1.7701307697799304f * xx + 1.7701307697799304f * yy);
+  dy += t[15] * (3.5402615395598609f * xy);
+}
+
+// Unit view direction from the camera to p: (p - cam) * rsqrt(|p - cam|^2 + 1e-12) (spherical_harmonic.h:27-35).
+__device__ __forceinline__ float view_dir(const float* __restrict__ p, const float* __restrict__ cam, float& x,
+                                          float& y, float& z) {
+  x = p[0] - cam[0], y = p[1] - cam[1], z = p[2] - cam[2];
+  const float n = 1.0f / sqrtf(x * x + y * y + z * z + 1e-12f);
+  x *= n, y *= n, z *= n;
+  return n;
+}
+
+}  // namespace fsgs

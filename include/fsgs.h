@@ -1,0 +1,150 @@
+/*
+ * fsgs.h -- C ABI of libfsgs_hip.so, the MI355X (gfx950) implementation of the Fast-SP-GS `fast_2d_gs/_C` hot path.
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer to contiguous row-major fp32 / int32 / int64 / uint8 data unless it is named
+ *    *_host. NULL stands for an absent optional tensor (Python `None` at the reference's pybind boundary).
+ *  - `stream` is a hipStream_t (NULL = default stream). Calls enqueue work and return; the only blocking call is
+ *    fsgs_gs_prepare_scan, which has to hand the instance count to the host (the reference blocks in the same place).
+ *  - The library allocates nothing: outputs and workspaces come from the caller (the *_workspace_bytes functions size
+ *    them). Outputs need not be zero-initialised unless stated.
+ *  - Return value 0 = success; otherwise fsgs_last_error() describes the failure (thread local).
+ *  - `file:line` citations name the reference interface each entry point replaces (relative to the reference root).
+ */
+#ifndef FSGS_H
+#define FSGS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* fsgs_last_error(void);
+int fsgs_version(void);
+int fsgs_check_device(void);
+
+/* ---- 2DGS surfel preprocess ---------------------------------------------------------------------------------- */
+
+/* gs_2d_preprocess_forward -- fast_2d_gs/_C/src/gaussian_splatting/gs_2d_preprocess.cu:331-421 (kernel :158-246).
+ * means3D[P,3] scales[P,2] rotations[P,4](x,y,z,w, used un-normalised) opacities[P,1]; sh_degree >= 0: shs[P,n_sh,3]
+ * (or shs[P,1,3] + sh_rest[P,n_sh,3]); sh_degree < 0: colours are the caller's own tensor and `colors` is ignored.
+ * trans_precomp[P,3,3] replaces the computed transform (then trans_mat is not written). culling[P] != 0 rejects.
+ * Every output row is written (zeros for rejected surfels); rows of means2D belonging to rejected surfels are left
+ * untouched when means2D_preserve != 0 (the reference's caller-supplied means2D buffer). */
+int fsgs_gs_2d_preprocess_forward(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
+    const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
+    const float* Tw2v, const float* Tv2c, const float* campos, const float* trans_precomp, const uint8_t* culling,
+    int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* normal_opacity, float* depths,
+    int32_t* radii, int32_t* tiles_touched, void* stream);
+
+/* gs_2d_preprocess_backward -- gs_2d_preprocess.cu:423-499 (kernel :268-329). Gradients of visible surfels are
+ * ASSIGNED into g_* (the caller zero-fills them, as the reference's caller does); grad_mean2D[P,2] is read and then
+ * overwritten in place with the densification proxy. g_shs / g_sh_rest may be NULL. */
+int fsgs_gs_2d_preprocess_backward(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
+    const float* scales, const float* rotations, const float* shs, const float* sh_rest, const float* Tw2v,
+    const float* Tv2c, const float* campos, const float* trans_mat, const int32_t* radii, const float* colors,
+    float* grad_mean2D, const float* grad_trans, const float* grad_colors, const float* grad_normal_opacity,
+    float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs, float* g_sh_rest, void* stream);
+
+/* gs_2d_compute_transmat_forward / gs_2d_compute_trans_mat_backward -- gs_2d_preprocess.cu:512-550, :564-599. */
+int fsgs_gs_2d_compute_transmat_forward(int P, int W, int H, const float* means3D, const float* scales,
+    const float* rotations, const float* Tw2v, const float* Tw2c, float* trans_mat, float* normals, void* stream);
+int fsgs_gs_2d_compute_transmat_backward(int P, int W, int H, const float* means3D, const float* scales,
+    const float* rotations, const float* Tw2v, const float* Tw2c, const float* g_mat, const float* g_normals,
+    float* g_means3D, float* g_scales, float* g_rot, void* stream);
+
+/* ---- tile binning: GS_prepare -- fast_2d_gs/_C/src/gaussian_splatting/gaussian_prepare.cu:222-308 -------------- */
+
+/* Phase 1: inclusive scan of tiles_touched[P] into point_offsets[P] (int64) and the instance count R on the host
+ * (gaussian_prepare.cu:231-239). Blocks until R is known. */
+size_t fsgs_gs_prepare_scan_workspace_bytes(int P);
+int fsgs_gs_prepare_scan(int P, const int32_t* tiles_touched, int64_t* point_offsets, void* workspace,
+                         size_t workspace_bytes, int64_t* num_rendered_host, void* stream);
+
+/* Phase 2: key duplication, stable sort on bits [0, 32 + msb(T)), tile ranges (gaussian_prepare.cu:47-83, 254-277,
+ * 192-220). ranges[T,2] int64 (empty tile = (0,0)), point_list[R] int32. sorted_keys_out[R] (optional) receives the
+ * sorted 64-bit keys (tile << 32 | depth bits). */
+size_t fsgs_gs_prepare_fill_workspace_bytes(int64_t R);
+int fsgs_gs_prepare_sort_bits(int W, int H);
+int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
+                         const int64_t* point_offsets, int64_t R, int64_t* ranges, int32_t* point_list,
+                         int64_t* sorted_keys_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- per-tile alpha blend ------------------------------------------------------------------------------------- */
+
+/* GS_2D_render_forward -- fast_2d_gs/_C/src/gaussian_splatting/gs_2d_redner.cu:541-629 (kernel :28-236).
+ * out_color[3,H,W] out_opacity[H,W] n_contrib[2,H,W]; unless only_image: out_extras[9,H,W]; with trans_mat_t2:
+ * out_flow[H,W,2]. accum_* [P] are accumulated into (atomics), all other outputs are fully written. */
+int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, double far_n, int only_image,
+    const float* means2D, const float* colors, const float* normal_opacity, const float* trans_mat,
+    const int32_t* point_list, const int64_t* ranges, const float* trans_mat_t2, int32_t* accum_max_count,
+    float* accum_weights_p, int32_t* accum_weights_count, float* out_color, float* out_opacity, float* out_extras,
+    float* out_flow, int32_t* n_contrib, void* stream);
+
+/* GS_2D_render_backward -- gs_2d_redner.cu:631-717 (kernel :238-539). g_colors[P,3] g_means2D[P,2] g_trans[P,3,3]
+ * g_normal_opacity[P,4] MUST be zero-filled by the caller; gradients are accumulated into them. */
+int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n, const float* means2D,
+    const float* normal_opacity, const float* colors, const float* trans_mat, const float* trans_mat_t2,
+    const float* out_opacity, const float* out_extras, const float* out_flow, const float* dL_dpix,
+    const float* dL_dopacity, const float* dL_dextras, const float* dL_dflow, const int64_t* ranges,
+    const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
+    float* g_normal_opacity, void* stream);
+
+/* ---- spherical harmonics and encoders ------------------------------------------------------------------------- */
+
+/* SH_to_RGB_forward / SH_to_RGB_backward -- fast_2d_gs/_C/src/ops_3d/spherical_harmonics.cu:15-41, :68-102.
+ * grad_campos[3] is accumulated into; grad_dir[P,3] and grad_sh[P,F,3] are assigned (first (degree+1)^2 rows). */
+int fsgs_sh_to_rgb_forward(int P, int F, int degree, int clamp, const float* pos, const float* campos,
+                           const float* sh, float* rgb, void* stream);
+int fsgs_sh_to_rgb_backward(int P, int F, int degree, int clamp, const float* pos, const float* campos,
+    const float* sh, const float* rgb, const float* grad_rgb, float* grad_dir, float* grad_campos, float* grad_sh,
+    void* stream);
+
+/* sh_encode_forward / sh_encode_backward -- fast_2d_gs/_C/src/nerf/shencoder.cu:657-691. in[B,D>=3], out[B,(C+1)^2];
+ * the backward writes the first three components of every grad_in row. */
+int fsgs_sh_encode_forward(int B, int D, int C, const float* in, float* out, void* stream);
+int fsgs_sh_encode_backward(int B, int D, int C, const float* grad, const float* in, float* grad_in, void* stream);
+
+/* freq_encode_forward / freq_encode_backward -- fast_2d_gs/_C/src/nerf/freqencoder.cu:63-104.
+ * out[B, Din * (2 * degree + include_input)] laid out [x | sin 2^0 s x | cos 2^0 s x | sin 2^1 s x | ...]. */
+int fsgs_freq_encode_forward(int B, int Din, int degree, int include_input, double scale, const float* in,
+                             float* out, void* stream);
+int fsgs_freq_encode_backward(int B, int Din, int degree, int include_input, double scale, const float* grad,
+                              const float* outv, float* gin, void* stream);
+
+/* ---- nearest points, K-NN, LBS, optimiser ---------------------------------------------------------------------- */
+
+/* cdist_top / cdist_top_backward -- fast_2d_gs/_C/src/other/cdist_top.cu:34-84, :107-154. x[B,N,D] y[B,M,D] ->
+ * dist[B,N] (Euclidean), index[B,N] int64. Ties: smallest keeps the LAST equal minimum, largest the FIRST equal
+ * maximum. The backward assigns g1[B,N,D] and accumulates into caller-zeroed g2[B,M,D]. */
+int fsgs_cdist_top_forward(int B, int N, int M, int D, int largest, const float* x, const float* y, float* dist,
+                           int64_t* index, void* stream);
+int fsgs_cdist_top_backward(int B, int N, int M, int D, const float* p1, const float* p2, const float* dist,
+                            const int64_t* index, const float* gdist, float* g1, float* g2, void* stream);
+
+/* K nearest rows of y[M,D] for every row of x[N,D] (K <= 16): dist2[N,K] squared distances ascending, index[N,K]
+ * int64, ties -> lower index first; slots beyond M hold (-1, -1). Replaces the reference's call
+ * pytorch3d.ops.knn_points(points[None], sp_points[None], K=K) at fast_2d_gs/network.py:504. */
+int fsgs_knn_topk(int N, int M, int D, int K, const float* x, const float* y, float* dist2, int64_t* index,
+                  void* stream);
+
+/* LBS blend with weights softmax(-dist2 / temperature) -- fast_2d_gs/network.py:517 and :545-573 (warp with
+ * apply_rotate == 'add'): q_k = normalize(sp_r_k + (0,0,0,1)); centred: t_k += c_k - R(q_k) c_k;
+ * d_xyz = sum_k w_k (R(q_k) p + t_k) - p; d_rot = sum_k w_k sp_r_k; d_scale = sum_k w_k sp_s_k (S <= 4 columns). */
+size_t fsgs_lbs_blend_workspace_bytes(int M);
+int fsgs_lbs_blend(int N, int M, int K, int centred, double temperature, const float* points,
+    const float* sp_points, const float* sp_t, const float* sp_r, const float* sp_s, int S, const float* dist2,
+    const int64_t* index, float* weights_out, float* d_xyz, float* d_rot, float* d_scale, void* workspace,
+    size_t workspace_bytes, void* stream);
+
+/* AdamMasksedUpdated -- fast_2d_gs/_C/src/other/adam_masked_update.cu:30-35 (kernel :9-28). Rows of the [N,M]
+ * tensors whose mask byte is 0 are left untouched; eps is added to sqrt(v); lr carries the bias correction. */
+int fsgs_adam_masked_update(int64_t N, int64_t M, const uint8_t* mask, double lr, double b1, double b2, double eps,
+                            float* param, const float* grad, float* m, float* v, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FSGS_H */

@@ -1,0 +1,157 @@
+"""TEST INFRASTRUCTURE ONLY: ctypes loader and numpy-level wrappers of the CPU parity oracle (liboracle.so).
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this package; the product package
+never does. Every wrapper takes and returns numpy arrays (host memory).
+"""
+from __future__ import annotations
+
+import ctypes
+import re
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+HERE = Path(__file__).resolve().parent
+LIB_PATH = HERE / "_build" / "liboracle.so"
+
+_SCALARS = {"int": ctypes.c_int, "int32_t": ctypes.c_int32, "int64_t": ctypes.c_int64, "size_t": ctypes.c_size_t,
+            "double": ctypes.c_double, "float": ctypes.c_float, "uint32_t": ctypes.c_uint32}
+
+
+def build() -> Path:
+    proc = subprocess.run(["make", "-C", str(HERE), "-B"], capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("building the oracle failed:\n" + proc.stdout + proc.stderr)
+    return LIB_PATH
+
+
+def _parse(text: str):
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    out = {}
+    for m in re.finditer(r"([A-Za-z_]\w*)\s+(oracle_\w+)\s*\(([^)]*)\)\s*;", text):
+        ret, name, args = m.group(1), m.group(2), m.group(3).strip()
+        argtypes = []
+        if args not in ("", "void"):
+            for a in args.split(","):
+                argtypes.append(ctypes.c_void_p if "*" in a else _SCALARS[a.replace("const", "").split()[0]])
+        out[name] = (_SCALARS[ret], argtypes)
+    return out
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            build()
+        L = ctypes.CDLL(str(LIB_PATH))
+        for name, (restype, argtypes) in _parse((HERE / "oracle.h").read_text()).items():
+            for n in {name, name.replace("_f32", "_f64")}:
+                fn = getattr(L, n)
+                fn.restype, fn.argtypes = restype, argtypes
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    if a is None:
+        return None
+    assert isinstance(a, np.ndarray) and a.flags["C_CONTIGUOUS"], "oracle wants C-contiguous numpy arrays"
+    return a.ctypes.data
+
+
+def _suffix(dtype) -> str:
+    return {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64"}[np.dtype(dtype)]
+
+
+def call(name: str, *args):
+    """Calls oracle_<name> converting numpy arrays to addresses; raises on a non-zero status."""
+    fn = getattr(lib(), "oracle_" + name)
+    rc = fn(*[_p(a) if isinstance(a, np.ndarray) or a is None else a for a in args])
+    return rc
+
+
+def num_threads() -> int:
+    return int(lib().oracle_num_threads())
+
+
+# ---- numpy-level wrappers mirroring the operator signatures ------------------------------------------------------
+def preprocess_forward(W, H, sh_degree, means3D, scales, rotations, opacities, shs, sh_rest, Tw2v, Tv2c, campos,
+                       trans_precomp=None, means2D=None, culling=None):
+    dt = means3D.dtype
+    P = means3D.shape[0]
+    has_rest = sh_rest is not None and sh_rest.size > 0
+    n_sh = sh_rest.shape[1] if has_rest else (shs.shape[1] if sh_degree >= 0 else 0)
+    preserve = means2D is not None
+    m2 = means2D if preserve else np.zeros((P, 2), dt)
+    colors = shs if sh_degree < 0 else np.zeros((P, 3), dt)
+    tm = trans_precomp if trans_precomp is not None else np.zeros((P, 3, 3), dt)
+    no, dep = np.zeros((P, 4), dt), np.zeros((P,), dt)
+    radii, tt = np.zeros((P,), np.int32), np.zeros((P,), np.int32)
+    cul = None if culling is None else np.ascontiguousarray(culling.astype(np.uint8))
+    rc = call(f"gs_2d_preprocess_forward_{_suffix(dt)}", P, W, H, sh_degree, n_sh, means3D, scales, rotations,
+              opacities, shs, sh_rest if has_rest else None, Tw2v, Tv2c, campos, trans_precomp, cul, int(preserve), m2,
+              None if sh_degree < 0 else colors, None if trans_precomp is not None else tm, no, dep, radii, tt)
+    assert rc == 0
+    return m2, colors, tm, no, dep, radii, tt
+
+
+def preprocess_backward(W, H, sh_degree, means3D, scales, rotations, shs, sh_rest, Tw2v, Tv2c, campos, trans_mat,
+                        radii, colors, grad_mean2D, grad_trans, grad_colors, grad_normal_opacity):
+    """Returns (g_means3D, g_scales, g_rot, g_opac, g_shs, g_sh_rest, grad_mean2D_after)."""
+    dt = means3D.dtype
+    P = means3D.shape[0]
+    has_rest = sh_rest is not None and sh_rest.size > 0
+    n_sh = sh_rest.shape[1] if has_rest else (shs.shape[1] if sh_degree >= 0 else 0)
+    g3, gs, gr, go = np.zeros((P, 3), dt), np.zeros((P, 2), dt), np.zeros((P, 4), dt), np.zeros((P, 1), dt)
+    gsh = np.zeros_like(shs) if sh_degree >= 0 else None
+    gshr = np.zeros_like(sh_rest) if has_rest else None
+    gm2 = grad_mean2D.copy()
+    rc = call(f"gs_2d_preprocess_backward_{_suffix(dt)}", P, W, H, sh_degree, n_sh, means3D, scales, rotations, shs,
+              sh_rest if has_rest else None, Tw2v, Tv2c, campos, trans_mat, radii, colors, gm2, grad_trans,
+              grad_colors, grad_normal_opacity, g3, gs, gr, go, gsh, gshr)
+    assert rc == 0
+    return g3, gs, gr, go, gsh, gshr, gm2
+
+
+def prepare(W, H, means2D, depths, radii, tiles_touched, return_keys=False):
+    P = means2D.shape[0]
+    offsets = np.zeros((max(P, 1),), np.int64)
+    R = int(lib().oracle_gs_prepare_count(P, _p(np.ascontiguousarray(tiles_touched)), _p(offsets)))
+    T = ((W + 15) // 16) * ((H + 15) // 16)
+    ranges, pl = np.zeros((T, 2), np.int64), np.zeros((R,), np.int32)
+    keys = np.zeros((R,), np.int64) if return_keys else None
+    rc = call("gs_prepare_fill", P, W, H, means2D, depths, radii, offsets, R, ranges, pl, keys)
+    assert rc == 0
+    return (ranges, pl, keys) if return_keys else (ranges, pl)
+
+
+def render_forward(W, H, means2D, colors, normal_opacity, trans_mat, point_list, ranges, near, far, only_image,
+                   trans_mat_t2=None, accum_max_count=None, accum_weights_p=None, accum_weights_count=None):
+    dt = means2D.dtype
+    P = colors.shape[0]
+    oc, oo = np.zeros((3, H, W), dt), np.zeros((H, W), dt)
+    oe = None if only_image else np.zeros((9, H, W), dt)
+    of = np.zeros((H, W, 2), dt) if (not only_image and trans_mat_t2 is not None) else None
+    nc = np.zeros((2, H, W), np.int32)
+    rc = call(f"gs_2d_render_forward_{_suffix(dt)}", P, W, H, float(near), float(far), int(only_image), means2D,
+              colors, normal_opacity, trans_mat, point_list, ranges, trans_mat_t2, accum_max_count, accum_weights_p,
+              accum_weights_count, oc, oo, oe, of, nc)
+    assert rc == 0
+    return oc, oo, oe, of, nc
+
+
+def render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat_t2, out_opacity, out_extras, out_flow,
+                    dL_dpix, dL_dopacity, dL_dextras, dL_dflow, ranges, point_list, n_contrib, near, far):
+    dt = means2D.dtype
+    P = means2D.shape[0]
+    H, W = dL_dpix.shape[1:]
+    gc, gm, gt, gn = np.zeros((P, 3), dt), np.zeros((P, 2), dt), np.zeros((P, 3, 3), dt), np.zeros((P, 4), dt)
+    rc = call(f"gs_2d_render_backward_{_suffix(dt)}", P, W, H, float(near), float(far), means2D, normal_opacity,
+              colors, trans_mat, trans_mat_t2, out_opacity, out_extras, out_flow, dL_dpix, dL_dopacity, dL_dextras,
+              dL_dflow, ranges, point_list, n_contrib, gc, gm, gt, gn)
+    assert rc == 0
+    return gc, gm, gt, gn

@@ -1,0 +1,393 @@
+// TEST INFRASTRUCTURE ONLY (parity oracle + CPU baseline). Never linked, imported or called by the
+// product library.
+//
+// Scalar CPU restatement of the stand-alone operators on the hot path:
+//   SH_to_RGB fwd/bwd        fast_2d_gs/_C/src/ops_3d/spherical_harmonics.cu:6-66 (+ include/spherical_harmonic.h)
+//   sh_encode fwd/bwd        fast_2d_gs/_C/src/nerf/shencoder.cu:18-176, 178-655
+//   freq_encode fwd/bwd      fast_2d_gs/_C/src/nerf/freqencoder.cu:7-60
+//   cdist_top fwd/bwd        fast_2d_gs/_C/src/other/cdist_top.cu:3-154
+//   masked Adam              fast_2d_gs/_C/src/other/adam_masked_update.cu:9-28
+//   K-NN + LBS blend         fast_2d_gs/network.py:498-573 (host code; the K-NN itself is pytorch3d.ops.knn_points
+//                            and the rigid transforms are lietorch.SE3 -- both un-vendored third-party packages with
+//                            no pinned version; their published semantics are restated and the tie order
+//                            "lower index first" is this build's definition: PARITY UNPINNED at that boundary)
+//   deformation MLP          fast_2d_gs/network.py:1670-1776 (8 x Linear(256)+ReLU, input re-concatenated after
+//                            layer 4, three linear heads)
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <vector>
+
+#include "sh_basis.h"
+
+namespace oracle {
+
+template <typename T>
+static void sh_to_rgb_fwd(int P, int F, int degree, int clamp, const T* pos, const T* campos, const T* sh, T* rgb) {
+  const int n = (degree + 1) * (degree + 1);
+#pragma omp parallel for schedule(static)
+  for (int i = 0; i < P; ++i) {
+    T x = pos[3 * i], y = pos[3 * i + 1], z = pos[3 * i + 2];
+    if (campos) {
+      x = x - campos[0], y = y - campos[1], z = z - campos[2];
+      const T nn = T(1) / std::sqrt(x * x + y * y + z * z + T(1e-12));
+      x = x * nn, y = y * nn, z = z * nn;
+    }
+    T Y[16];
+    sh_basis(degree, x, y, z, Y);
+    const T* c = sh + (size_t) i * F * 3;
+    for (int ch = 0; ch < 3; ++ch) {
+      T r = c[ch] * Y[0];
+      for (int l = 1; l < n; ++l) r += c[l * 3 + ch] * Y[l];
+      r += T(0.5);
+      rgb[3 * i + ch] = clamp ? std::max(T(0), r) : r;
+    }
+  }
+}
+
+template <typename T>
+static void sh_to_rgb_bwd(int P, int F, int degree, int clamp, const T* pos, const T* campos, const T* sh,
+                          const T* rgb, const T* grad_rgb, T* grad_dir, T* grad_campos, T* grad_sh) {
+  const int n = (degree + 1) * (degree + 1);
+  T cam_acc[3] = {0, 0, 0};
+  for (int i = 0; i < P; ++i) {
+    T x = pos[3 * i], y = pos[3 * i + 1], z = pos[3 * i + 2], nn = 1;
+    if (campos) {
+      x = x - campos[0], y = y - campos[1], z = z - campos[2];
+      nn = T(1) / std::sqrt(x * x + y * y + z * z + T(1e-12));
+      x = x * nn, y = y * nn, z = z * nn;
+    }
+    T g[3] = {grad_rgb[3 * i], grad_rgb[3 * i + 1], grad_rgb[3 * i + 2]};
+    if (clamp)
+      for (int ch = 0; ch < 3; ++ch) g[ch] *= T(rgb[3 * i + ch] > 0);
+    T Y[16], dY[48];
+    sh_basis(degree, x, y, z, Y);
+    if (grad_sh) {
+      T* gs = grad_sh + (size_t) i * F * 3;
+      for (int l = 0; l < n; ++l)
+        for (int ch = 0; ch < 3; ++ch) gs[l * 3 + ch] = g[ch] * Y[l];
+    }
+    if (!grad_dir && !grad_campos) continue;
+    sh_basis_grad(degree, x, y, z, dY);
+    const T* c = sh + (size_t) i * F * 3;
+    T dx = 0, dy = 0, dz = 0;
+    for (int l = 1; l < n; ++l) {
+      const T t = g[0] * c[l * 3] + g[1] * c[l * 3 + 1] + g[2] * c[l * 3 + 2];
+      dx += t * dY[l * 3], dy += t * dY[l * 3 + 1], dz += t * dY[l * 3 + 2];
+    }
+    if (campos) {
+      const T vx = pos[3 * i] - campos[0], vy = pos[3 * i + 1] - campos[1], vz = pos[3 * i + 2] - campos[2];
+      const T t  = -(vx * dx + vy * dy + vz * dz) * nn * nn * nn;
+      dx = dx * nn + t * vx, dy = dy * nn + t * vy, dz = dz * nn + t * vz;
+    }
+    if (grad_dir) grad_dir[3 * i] = dx, grad_dir[3 * i + 1] = dy, grad_dir[3 * i + 2] = dz;
+    cam_acc[0] -= dx, cam_acc[1] -= dy, cam_acc[2] -= dz;
+  }
+  if (grad_campos)
+    for (int a = 0; a < 3; ++a) grad_campos[a] += cam_acc[a];
+}
+
+template <typename T>
+static void sh_encode_fwd(int B, int D, int C, const T* in, T* out) {
+  const int n = (C + 1) * (C + 1);
+#pragma omp parallel for schedule(static)
+  for (int b = 0; b < B; ++b) sh_basis(C, in[(size_t) b * D], in[(size_t) b * D + 1], in[(size_t) b * D + 2], out + (size_t) b * n);
+}
+
+template <typename T>
+static void sh_encode_bwd(int B, int D, int C, const T* grad, const T* in, T* grad_in) {
+  const int n = (C + 1) * (C + 1);
+#pragma omp parallel for schedule(static)
+  for (int b = 0; b < B; ++b) {
+    T dY[48];
+    sh_basis_grad(C, in[(size_t) b * D], in[(size_t) b * D + 1], in[(size_t) b * D + 2], dY);
+    T dx = 0, dy = 0, dz = 0;
+    for (int l = 0; l < n; ++l) {
+      const T g = grad[(size_t) b * n + l];
+      dx += g * dY[l * 3], dy += g * dY[l * 3 + 1], dz += g * dY[l * 3 + 2];
+    }
+    grad_in[(size_t) b * D] = dx, grad_in[(size_t) b * D + 1] = dy, grad_in[(size_t) b * D + 2] = dz;
+  }
+}
+
+template <typename T>
+static void freq_fwd(int B, int Din, int degree, int include_input, T scale, const T* in, T* out) {
+  const int Dout = Din * (2 * degree + (include_input ? 1 : 0));
+  for (int b = 0; b < B; ++b)
+    for (int c = 0; c < Din; ++c) {
+      T* o = out + (size_t) b * Dout + c;
+      T x  = in[(size_t) b * Din + c];
+      if (include_input) o[0] = x, o += Din;
+      x = x * scale;
+      for (int d = 0; d < degree; ++d) {
+        const T v = std::ldexp(x, d);
+        o[(2 * d + 0) * Din] = std::sin(v);
+        o[(2 * d + 1) * Din] = std::cos(v);
+      }
+    }
+}
+
+template <typename T>
+static void freq_bwd(int B, int Din, int degree, int include_input, T scale, const T* grad, const T* outv, T* gin) {
+  const int Dout = Din * (2 * degree + (include_input ? 1 : 0));
+  for (int b = 0; b < B; ++b)
+    for (int c = 0; c < Din; ++c) {
+      const T* g = grad + (size_t) b * Dout + c;
+      const T* o = outv + (size_t) b * Dout + c;
+      T gx = 0;
+      if (include_input) gx = g[0], g += Din, o += Din;
+      for (int f = 0; f < degree; ++f) {
+        gx += std::ldexp(T(1.0), f) * scale * (g[0] * o[Din] - g[Din] * o[0]);
+        g += 2 * Din, o += 2 * Din;
+      }
+      gin[(size_t) b * Din + c] = gx;
+    }
+}
+
+// cdist_top.cu:15-31. Tie rule: `m == 0 || (sum > top) == largest`.
+template <typename T>
+static void cdist_top_fwd(int B, int N, int M, int D, int largest, const T* x, const T* y, T* dist, int64_t* index) {
+#pragma omp parallel for schedule(static)
+  for (int64_t bn = 0; bn < (int64_t) B * N; ++bn) {
+    const int b = (int) (bn / N);
+    const T* xp = x + (size_t) bn * D;
+    const T* yb = y + (size_t) b * M * D;
+    T top = 0;
+    int topi = 0;
+    for (int m = 0; m < M; ++m) {
+      T sum = 0;
+      for (int d = 0; d < D; ++d) {
+        const T t = xp[d] - yb[(size_t) m * D + d];
+        sum += t * t;
+      }
+      if (m == 0 || (sum > top) == (bool) largest) top = sum, topi = m;
+    }
+    dist[bn]  = std::sqrt(top);
+    index[bn] = topi;
+  }
+}
+
+template <typename T>
+static void cdist_top_bwd(int B, int N, int M, int D, const T* p1, const T* p2, const T* dist, const int64_t* index,
+                          const T* gdist, T* g1, T* g2) {
+  for (int64_t i = 0; i < (int64_t) B * N; ++i) {
+    const int b  = (int) (i / N);
+    const int j2 = (int) index[i];
+    const T g    = gdist[i] / dist[i];
+    for (int d = 0; d < D; ++d) {
+      const T t = g * (p1[(size_t) i * D + d] - p2[((size_t) b * M + j2) * D + d]);
+      g1[(size_t) i * D + d] = t;
+      g2[((size_t) b * M + j2) * D + d] -= t;
+    }
+  }
+}
+
+// adam_masked_update.cu:16-27: eps is added to sqrt(v), lr already carries the bias correction.
+template <typename T>
+static void adam_masked(int64_t N, int64_t M, const uint8_t* mask, T lr, T b1, T b2, T eps, T* param, const T* grad,
+                        T* m, T* v) {
+  for (int64_t i = 0; i < N; ++i) {
+    if (!mask[i]) continue;
+    for (int64_t j = i * M; j < (i + 1) * M; ++j) {
+      const T g  = grad[j];
+      const T mm = b1 * m[j] + (T(1.0) - b1) * g;
+      const T vv = b2 * v[j] + (T(1.0) - b2) * g * g;
+      const T st = -lr * mm / (std::sqrt(vv) + eps);
+      param[j] += st;
+      m[j] = mm, v[j] = vv;
+    }
+  }
+}
+
+// K nearest rows of y for every row of x: squared distances ascending, ties -> lower index first.
+template <typename T>
+static void knn_topk(int N, int M, int D, int K, const T* x, const T* y, T* dist2, int64_t* index) {
+#pragma omp parallel for schedule(static)
+  for (int n = 0; n < N; ++n) {
+    std::vector<T> bd(K);
+    std::vector<int64_t> bi(K);
+    int cnt = 0;
+    for (int m = 0; m < M; ++m) {
+      T sum = 0;
+      for (int d = 0; d < D; ++d) {
+        const T t = x[(size_t) n * D + d] - y[(size_t) m * D + d];
+        sum += t * t;
+      }
+      if (cnt < K || sum < bd[cnt - 1]) {
+        int pos = cnt < K ? cnt : K - 1;
+        while (pos > 0 && bd[pos - 1] > sum) {
+          bd[pos] = bd[pos - 1], bi[pos] = bi[pos - 1];
+          --pos;
+        }
+        bd[pos] = sum, bi[pos] = m;
+        if (cnt < K) ++cnt;
+      }
+    }
+    for (int k = 0; k < K; ++k) {
+      dist2[(size_t) n * K + k] = k < cnt ? bd[k] : T(-1);
+      index[(size_t) n * K + k] = k < cnt ? bi[k] : -1;
+    }
+  }
+}
+
+// Rotation matrix of a unit quaternion (x, y, z, w): utils/ops_3d/quaternion.py:164-174.
+template <typename T>
+static inline void quat_R(const T* q, T* R) {
+  const T x = q[0], y = q[1], z = q[2], w = q[3];
+  R[0] = 1 - 2 * (y * y + z * z), R[1] = 2 * (x * y - z * w), R[2] = 2 * (y * w + x * z);
+  R[3] = 2 * (x * y + z * w), R[4] = 1 - 2 * (x * x + z * z), R[5] = 2 * (y * z - x * w);
+  R[6] = 2 * (x * z - y * w), R[7] = 2 * (x * w + y * z), R[8] = 1 - 2 * (x * x + y * y);
+}
+
+// LBS blend, network.py:517 (weights = softmax(-d2 / temperature)) and :545-573 (warp):
+// q_k = normalize(r_k + (0,0,0,1)); centred: t_k <- t_k + c_k + R(q_k)(-c_k);
+// d_xyz = sum_k w_k (R(q_k) p + t_k) - p ; d_rot = sum_k w_k r_k ; d_scale = sum_k w_k s_k.
+template <typename T>
+static void lbs_blend(int N, int M, int K, int centred, T temperature, const T* points, const T* sp_points,
+                      const T* sp_t, const T* sp_r, const T* sp_s, int S, const T* dist2, const int64_t* index,
+                      T* weights_out, T* d_xyz, T* d_rot, T* d_scale) {
+  (void) M;
+#pragma omp parallel for schedule(static)
+  for (int n = 0; n < N; ++n) {
+    std::vector<T> w(K);
+    T mx = -dist2[(size_t) n * K] / temperature;
+    for (int k = 1; k < K; ++k) mx = std::max(mx, -dist2[(size_t) n * K + k] / temperature);
+    T den = 0;
+    for (int k = 0; k < K; ++k) w[k] = std::exp(-dist2[(size_t) n * K + k] / temperature - mx), den += w[k];
+    for (int k = 0; k < K; ++k) w[k] = w[k] / den;
+    const T* p = points + 3 * (size_t) n;
+    T acc[3] = {0, 0, 0}, ar[4] = {0, 0, 0, 0};
+    std::vector<T> as(S, T(0));
+    for (int k = 0; k < K; ++k) {
+      const int64_t j = index[(size_t) n * K + k];
+      T q[4] = {sp_r[4 * j], sp_r[4 * j + 1], sp_r[4 * j + 2], sp_r[4 * j + 3] + T(1)};
+      const T nq = T(1) / std::max(std::sqrt(q[0] * q[0] + q[1] * q[1] + q[2] * q[2] + q[3] * q[3]), T(1e-12));
+      for (int a = 0; a < 4; ++a) q[a] *= nq;
+      T R[9];
+      quat_R(q, R);
+      T t[3] = {sp_t[3 * j], sp_t[3 * j + 1], sp_t[3 * j + 2]};
+      if (centred) {
+        const T* c = sp_points + 3 * j;
+        for (int a = 0; a < 3; ++a) t[a] = t[a] + c[a] - (R[a * 3] * c[0] + R[a * 3 + 1] * c[1] + R[a * 3 + 2] * c[2]);
+      }
+      for (int a = 0; a < 3; ++a) acc[a] += w[k] * (R[a * 3] * p[0] + R[a * 3 + 1] * p[1] + R[a * 3 + 2] * p[2] + t[a]);
+      for (int a = 0; a < 4; ++a) ar[a] += w[k] * sp_r[4 * j + a];
+      for (int a = 0; a < S; ++a) as[a] += w[k] * sp_s[(size_t) S * j + a];
+      if (weights_out) weights_out[(size_t) n * K + k] = w[k];
+    }
+    for (int a = 0; a < 3; ++a) d_xyz[3 * (size_t) n + a] = acc[a] - p[a];
+    for (int a = 0; a < 4; ++a) d_rot[4 * (size_t) n + a] = ar[a];
+    for (int a = 0; a < S; ++a) d_scale[(size_t) S * n + a] = as[a];
+  }
+}
+
+// Deformation MLP forward, network.py:1757-1776: h = in; for i in 0..L-1: h = relu(W_i h + b_i);
+// after layer index `skip` the input is re-concatenated in front: h = [in | h]. Heads are plain linears.
+// Weights are row-major [out, in] as torch.nn.Linear stores them.
+static void deform_mlp(int B, int Din, int Wd, int L, int skip, const float* in, const float* const* Ws,
+                       const float* const* bs, int n_heads, const int* head_dims, const float* const* hW,
+                       const float* const* hb, float* const* outs) {
+#pragma omp parallel for schedule(static)
+  for (int b = 0; b < B; ++b) {
+    std::vector<float> h(in + (size_t) b * Din, in + (size_t) (b + 1) * Din), nh;
+    for (int i = 0; i < L; ++i) {
+      const int din = (int) h.size();
+      nh.assign(Wd, 0.f);
+      for (int o = 0; o < Wd; ++o) {
+        float s = bs[i][o];
+        for (int k = 0; k < din; ++k) s += Ws[i][(size_t) o * din + k] * h[k];
+        nh[o] = s > 0.f ? s : 0.f;
+      }
+      if (i == skip) {
+        h.assign(in + (size_t) b * Din, in + (size_t) (b + 1) * Din);
+        h.insert(h.end(), nh.begin(), nh.end());
+      } else {
+        h = nh;
+      }
+    }
+    for (int hd = 0; hd < n_heads; ++hd)
+      for (int o = 0; o < head_dims[hd]; ++o) {
+        float s = hb[hd][o];
+        for (int k = 0; k < (int) h.size(); ++k) s += hW[hd][(size_t) o * h.size() + k] * h[k];
+        outs[hd][(size_t) b * head_dims[hd] + o] = s;
+      }
+  }
+}
+
+}  // namespace oracle
+
+using namespace oracle;
+#define ORACLE_API extern "C" __attribute__((visibility("default")))
+
+#define INSTANTIATE(SUF, T)                                                                                          \
+  ORACLE_API int oracle_sh_to_rgb_forward_##SUF(int P, int F, int degree, int clamp, const T* pos, const T* campos,  \
+                                                const T* sh, T* rgb) {                                               \
+    if (degree > kMaxShDegree) return 1;                                                                             \
+    sh_to_rgb_fwd<T>(P, F, degree, clamp, pos, campos, sh, rgb);                                                     \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_sh_to_rgb_backward_##SUF(int P, int F, int degree, int clamp, const T* pos,                  \
+      const T* campos, const T* sh, const T* rgb, const T* grad_rgb, T* grad_dir, T* grad_campos, T* grad_sh) {      \
+    if (degree > kMaxShDegree) return 1;                                                                             \
+    sh_to_rgb_bwd<T>(P, F, degree, clamp, pos, campos, sh, rgb, grad_rgb, grad_dir, grad_campos, grad_sh);           \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_sh_encode_forward_##SUF(int B, int D, int C, const T* in, T* out) {                          \
+    if (C > kMaxShDegree) return 1;                                                                                  \
+    sh_encode_fwd<T>(B, D, C, in, out);                                                                              \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_sh_encode_backward_##SUF(int B, int D, int C, const T* grad, const T* in, T* grad_in) {      \
+    if (C > kMaxShDegree) return 1;                                                                                  \
+    sh_encode_bwd<T>(B, D, C, grad, in, grad_in);                                                                    \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_freq_encode_forward_##SUF(int B, int Din, int degree, int include_input, double scale,       \
+                                                  const T* in, T* out) {                                             \
+    freq_fwd<T>(B, Din, degree, include_input, (T) scale, in, out);                                                  \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_freq_encode_backward_##SUF(int B, int Din, int degree, int include_input, double scale,      \
+                                                   const T* grad, const T* outv, T* gin) {                           \
+    freq_bwd<T>(B, Din, degree, include_input, (T) scale, grad, outv, gin);                                          \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_cdist_top_forward_##SUF(int B, int N, int M, int D, int largest, const T* x, const T* y,     \
+                                                T* dist, int64_t* index) {                                           \
+    cdist_top_fwd<T>(B, N, M, D, largest, x, y, dist, index);                                                        \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_cdist_top_backward_##SUF(int B, int N, int M, int D, const T* p1, const T* p2,               \
+      const T* dist, const int64_t* index, const T* gdist, T* g1, T* g2) {                                           \
+    cdist_top_bwd<T>(B, N, M, D, p1, p2, dist, index, gdist, g1, g2);                                                \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_adam_masked_update_##SUF(int64_t N, int64_t M, const uint8_t* mask, double lr, double b1,    \
+      double b2, double eps, T* param, const T* grad, T* m, T* v) {                                                  \
+    adam_masked<T>(N, M, mask, (T) lr, (T) b1, (T) b2, (T) eps, param, grad, m, v);                                  \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_knn_topk_##SUF(int N, int M, int D, int K, const T* x, const T* y, T* dist2,                 \
+                                       int64_t* index) {                                                             \
+    knn_topk<T>(N, M, D, K, x, y, dist2, index);                                                                     \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_lbs_blend_##SUF(int N, int M, int K, int centred, double temperature, const T* points,       \
+      const T* sp_points, const T* sp_t, const T* sp_r, const T* sp_s, int S, const T* dist2, const int64_t* index,  \
+      T* weights_out, T* d_xyz, T* d_rot, T* d_scale) {                                                              \
+    lbs_blend<T>(N, M, K, centred, (T) temperature, points, sp_points, sp_t, sp_r, sp_s, S, dist2, index,            \
+                 weights_out, d_xyz, d_rot, d_scale);                                                                \
+    return 0;                                                                                                        \
+  }
+
+INSTANTIATE(f32, float)
+INSTANTIATE(f64, double)
+
+ORACLE_API int oracle_deform_mlp_f32(int B, int Din, int Wd, int L, int skip, const float* in,
+                                     const float* const* Ws, const float* const* bs, int n_heads,
+                                     const int* head_dims, const float* const* hW, const float* const* hb,
+                                     float* const* outs) {
+  deform_mlp(B, Din, Wd, L, skip, in, Ws, bs, n_heads, head_dims, hW, hb, outs);
+  return 0;
+}

@@ -1,0 +1,57 @@
+/* TEST INFRASTRUCTURE ONLY. Prototypes of liboracle.so (the CPU parity oracle); host pointers everywhere.
+ * The *_f32 functions take float buffers, the *_f64 twins (same argument lists with double) exist for
+ * finite-difference checks and are bound by oracle/__init__.py by substituting the scalar type. */
+int oracle_gs_2d_preprocess_forward_f32(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
+    const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
+    const float* Tw2v, const float* Tv2c, const float* campos, const float* trans_precomp, const uint8_t* culling,
+    int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* normal_opacity, float* depths,
+    int32_t* radii, int32_t* tiles_touched);
+int oracle_gs_2d_preprocess_backward_f32(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
+    const float* scales, const float* rotations, const float* shs, const float* sh_rest, const float* Tw2v,
+    const float* Tv2c, const float* campos, const float* trans_mat, const int32_t* radii, const float* colors,
+    float* grad_mean2D, const float* grad_trans, const float* grad_colors, const float* grad_normal_opacity,
+    float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs, float* g_sh_rest);
+int oracle_gs_2d_compute_transmat_forward_f32(int P, int W, int H, const float* means3D, const float* scales,
+    const float* rotations, const float* Tw2v, const float* Tw2c, float* trans_mat, float* normals);
+int oracle_gs_2d_compute_transmat_backward_f32(int P, int W, int H, const float* means3D, const float* scales,
+    const float* rotations, const float* Tw2v, const float* Tw2c, const float* g_mat, const float* g_normals,
+    float* g_means3D, float* g_scales, float* g_rot);
+int oracle_gs_2d_render_forward_f32(int P, int W, int H, double near_n, double far_n, int only_image,
+    const float* means2D, const float* colors, const float* normal_opacity, const float* trans_mat,
+    const int32_t* point_list, const int64_t* ranges, const float* trans_mat_t2, int32_t* accum_max_count,
+    float* accum_weights_p, int32_t* accum_weights_count, float* out_color, float* out_opacity, float* out_extras,
+    float* out_flow, int32_t* n_contrib);
+int oracle_gs_2d_render_backward_f32(int P, int W, int H, double near_n, double far_n, const float* means2D,
+    const float* normal_opacity, const float* colors, const float* trans_mat, const float* trans_mat_t2,
+    const float* out_opacity, const float* out_extras, const float* out_flow, const float* dL_dpix,
+    const float* dL_dopacity, const float* dL_dextras, const float* dL_dflow, const int64_t* ranges,
+    const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
+    float* g_normal_opacity);
+int oracle_gs_2d_topk_weights_f32(int topk, int W, int H, double near_n, double far_n, const float* means2D,
+    const float* normal_opacity, const float* trans_mat, const int64_t* ranges, const int32_t* point_list,
+    int32_t* top_idx, float* top_w);
+int oracle_sh_to_rgb_forward_f32(int P, int F, int degree, int clamp, const float* pos, const float* campos,
+    const float* sh, float* rgb);
+int oracle_sh_to_rgb_backward_f32(int P, int F, int degree, int clamp, const float* pos, const float* campos,
+    const float* sh, const float* rgb, const float* grad_rgb, float* grad_dir, float* grad_campos, float* grad_sh);
+int oracle_sh_encode_forward_f32(int B, int D, int C, const float* in, float* out);
+int oracle_sh_encode_backward_f32(int B, int D, int C, const float* grad, const float* in, float* grad_in);
+int oracle_freq_encode_forward_f32(int B, int Din, int degree, int include_input, double scale, const float* in,
+    float* out);
+int oracle_freq_encode_backward_f32(int B, int Din, int degree, int include_input, double scale, const float* grad,
+    const float* outv, float* gin);
+int oracle_cdist_top_forward_f32(int B, int N, int M, int D, int largest, const float* x, const float* y, float* dist,
+    int64_t* index);
+int oracle_cdist_top_backward_f32(int B, int N, int M, int D, const float* p1, const float* p2, const float* dist,
+    const int64_t* index, const float* gdist, float* g1, float* g2);
+int oracle_adam_masked_update_f32(int64_t N, int64_t M, const uint8_t* mask, double lr, double b1, double b2,
+    double eps, float* param, const float* grad, float* m, float* v);
+int oracle_knn_topk_f32(int N, int M, int D, int K, const float* x, const float* y, float* dist2, int64_t* index);
+int oracle_lbs_blend_f32(int N, int M, int K, int centred, double temperature, const float* points,
+    const float* sp_points, const float* sp_t, const float* sp_r, const float* sp_s, int S, const float* dist2,
+    const int64_t* index, float* weights_out, float* d_xyz, float* d_rot, float* d_scale);
+int64_t oracle_gs_prepare_count(int P, const int32_t* tiles_touched, int64_t* offsets);
+int oracle_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
+    const int64_t* offsets, int64_t R, int64_t* ranges, int32_t* point_list, int64_t* keys_sorted_out);
+uint32_t oracle_higher_msb(uint32_t n);
+int oracle_num_threads(void);
