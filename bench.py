@@ -1,0 +1,173 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X: forward + backward frames/s of the 2DGS surfel renderer on the
+300k-surfel 800x800 synthetic scene (preprocess -> binning -> blend -> blend backward -> preprocess backward),
+with the roofline position of the dominant kernel and the CPU oracle timed beside it.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line. Only one GPU is supported: --gpus N with N > 1 exits with a message.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def algorithmic_bytes(stage: str, P: int, Pv: int, R: int, T: int, HW: int) -> int:
+    """Algorithmic HBM bytes of one launch of each stage at SH degree 3 (192 B of SH per surfel), 6 sort passes."""
+    S = 192
+    table = {
+        'gs_2d_preprocess_forward': P * (12 + 8 + 16 + 4 + S) + Pv * 76 + P * 8,
+        'gs_prepare_scan': P * 12,
+        'gs_prepare_fill': P * 24 + R * 12 + R * 12 * 2 * 6 + R * 8 + R * 8 + T * 16,
+        'gs_2d_render_forward': 76 * R + 16 * T + 60 * HW,
+        'gs_2d_render_backward': 76 * R + 16 * T + 60 * HW + 72 * (P + Pv),
+        'gs_2d_preprocess_backward': 4 * P + Pv * (352 + 240),
+    }
+    return int(table[stage])
+
+
+def cpu_baseline(scene, cam, budget_s: float = 20.0):
+    """The CPU oracle (scalar C++ restatement, OpenMP over pixels/surfels) on the same workload, whole frames until
+    about `budget_s` seconds are spent. A reported baseline, not a target."""
+    import oracle as O
+    n = lambda t: np.ascontiguousarray(t.cpu().numpy())
+    s = {k: n(getattr(scene, k)) for k in ('means3D', 'scales', 'rotations', 'opacities', 'shs')}
+    Tw2v, Tv2c, campos = n(cam.Tw2v), n(cam.Tv2c), n(cam.campos)
+    gi, ge, go = n(scene.extra['grad_image']), n(scene.extra['grad_extras']), n(scene.extra['grad_opacity'])
+    W, H = cam.W, cam.H
+    frames, t0 = 0, time.perf_counter()
+    while True:
+        m2, colors, tm, no, dep, radii, tt = O.preprocess_forward(W, H, 3, s['means3D'], s['scales'], s['rotations'],
+                                                                  s['opacities'], s['shs'], None, Tw2v, Tv2c, campos)
+        ranges, pl = O.prepare(W, H, m2, dep, radii, tt)
+        oc, oo, oe, _, nc = O.render_forward(W, H, m2, colors, no, tm, pl, ranges, cam.near, cam.far, False)
+        gc, gm, gt, gn = O.render_backward(m2, no, colors, tm, None, oo, oe, None, gi, go, ge, None, ranges, pl, nc,
+                                           cam.near, cam.far)
+        O.preprocess_backward(W, H, 3, s['means3D'], s['scales'], s['rotations'], s['shs'], None, Tw2v, Tv2c, campos,
+                              tm, radii, colors, gm, gt, gc, gn)
+        frames += 1
+        dt = time.perf_counter() - t0
+        if dt > budget_s or frames >= 8:
+            break
+    return {"value": frames / dt, "unit": "frames/s", "cores": O.num_threads(), "kind": "port",
+            "sample": f"{frames} full fwd+bwd frame(s) of the same 300k-surfel 800x800 workload ({dt:.1f} s), "
+                      f"host has {os.cpu_count()} logical cpus"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--surfels", type=int, default=300_000)
+    ap.add_argument("--size", type=int, default=800)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd._C import _ops, get_C_function
+    from fast_sp_gs_amd.renderer import render_step
+
+    dev = torch.device("cuda:0")
+    scene_h, cam_h = scenes.config2(P=args.surfels, size=args.size)
+    scene, cam = scene_h.to(dev), cam_h.to(dev)
+    gi = scene_h.extra['grad_image'].to(dev)
+    ge = scene_h.extra['grad_extras'].to(dev)
+    bg = torch.ones(3, 1, 1, device=dev)  # white background, composited on the host side as the reference does
+
+    def step():
+        # dL/dopacity of the white-background composite image = C + (1 - opacity) * bg
+        go = -(gi * bg).sum(0)
+        out = render_step(scene, cam, gi, ge, go)
+        out['composited'] = out['image'] + (1.0 - out['opacity']) * bg
+        return out
+
+    for _ in range(args.warmup):
+        out = step()
+    torch.cuda.synchronize()
+    _ops.STAGE_EVENTS = events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    _ops.STAGE_EVENTS = None
+
+    P = scene.P
+    Pv = int((out['radii'] > 0).sum())
+    R = int(out['point_list'].numel())
+    HW = cam.W * cam.H
+    T = ((cam.W + 15) // 16) * ((cam.H + 15) // 16)
+    stage_ms = {}
+    for name, a, b in events:
+        stage_ms.setdefault(name, []).append(a.elapsed_time(b))
+    stage_avg = {k: float(np.mean(v)) for k, v in stage_ms.items()}
+    dominant = max(stage_avg, key=stage_avg.get)
+    bytes_dom = algorithmic_bytes(dominant, P, Pv, R, T, HW)
+    achieved = bytes_dom / (stage_avg[dominant] * 1e-3) / 1e9
+    stages = {k: {"ms": round(v, 4),
+                  "algorithmic_GBps": round(algorithmic_bytes(k, P, Pv, R, T, HW) / (v * 1e-3) / 1e9, 1)}
+              for k, v in stage_avg.items()}
+
+    # top-k queries/s: 200k Gaussian centres against 512 control points, k = 4 (indices bit-exact, squared distances)
+    c1 = scenes.config1(n_dirs=8)
+    pts, ctrl = c1['points'].to(dev), c1['ctrl'].to(dev)
+    knn = get_C_function('knn_topk')
+    for _ in range(3):
+        knn(pts, ctrl, 4)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(20):
+        knn(pts, ctrl, 4)
+    e1.record()
+    torch.cuda.synchronize()
+    knn_ms = e0.elapsed_time(e1) / 20
+
+    result = {
+        "metric": "fwd+bwd frames/s, 300k surfels @800x800",
+        "value": args.steps / dt,
+        "unit": "frames/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"static 2DGS fwd+bwd: {P} surfels in the unit ball, {cam.W}x{cam.H}, FoV 40, radius 4, "
+                               "SH degree 3, white background, 16x16 tiles, key duplication + 64-bit radix sort + "
+                               "depth/normal outputs",
+                   "P": P, "P_visible": Pv, "R": R, "tiles": T},
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "algorithmic_bytes_per_launch": bytes_dom, "avg_launch_ms": stage_avg[dominant]},
+        "stages": stages,
+        "extra_metrics": {"knn_topk_queries_per_s": pts.shape[0] / (knn_ms * 1e-3),
+                          "knn_topk_workload": "200000 x 512, k=4, D=3"},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(scene_h, cam_h)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -23,6 +23,29 @@ __all__ = [
 
 _TILE = 16
 
+# When set to a list, every operator appends (name, start_event, end_event) recorded on the current stream tightly
+# around its C-ABI call (allocation and zero-fill of outputs stay outside), so callers can time the kernels themselves.
+STAGE_EVENTS = None
+
+
+class _timed:
+    __slots__ = ('name', 'start')
+
+    def __init__(self, name):
+        self.name = name
+
+    def __enter__(self):
+        if STAGE_EVENTS is not None:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+
+    def __exit__(self, *exc):
+        if STAGE_EVENTS is not None:
+            end = torch.cuda.Event(enable_timing=True)
+            end.record()
+            STAGE_EVENTS.append((self.name, self.start, end))
+        return False
+
 
 def _lib():
     return L.load()
@@ -90,12 +113,13 @@ def gs_2d_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: bool, me
     radii = torch.empty((P,), dtype=torch.int32, device=means3D.device)
     tiles_touched = torch.empty((P,), dtype=torch.int32, device=means3D.device)
     normal_opacity = torch.empty((P, 4), **opt)
-    rc = _lib().fsgs_gs_2d_preprocess_forward(
-        P, W, H, sh_degree, M, L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(opacities), L.ptr(shs),
-        L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(cam_pos), L.ptr(trans_precomp),
-        L.ptr(culling), int(preserve), L.ptr(means2D_), None if sh_degree < 0 else L.ptr(colors),
-        None if trans_precomp is not None else L.ptr(trans_mat), L.ptr(normal_opacity), L.ptr(depths), L.ptr(radii),
-        L.ptr(tiles_touched), L.current_stream())
+    with _timed('gs_2d_preprocess_forward'):
+        rc = _lib().fsgs_gs_2d_preprocess_forward(
+            P, W, H, sh_degree, M, L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(opacities), L.ptr(shs),
+            L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(cam_pos), L.ptr(trans_precomp),
+            L.ptr(culling), int(preserve), L.ptr(means2D_), None if sh_degree < 0 else L.ptr(colors),
+            None if trans_precomp is not None else L.ptr(trans_mat), L.ptr(normal_opacity), L.ptr(depths), L.ptr(radii),
+            L.ptr(tiles_touched), L.current_stream())
     L.check(rc, what)
     return [means2D_, colors, trans_mat, normal_opacity, depths, radii, tiles_touched]
 
@@ -121,12 +145,13 @@ def gs_2d_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotat
     L.require_shape(what, 'grad_scales', grad_scales, P, 2)
     L.require_shape(what, 'grad_rotations', grad_rotations, P, 4)
     L.require_shape(what, 'grad_opacities', grad_opacities, P, 1)
-    rc = _lib().fsgs_gs_2d_preprocess_backward(
-        P, W, H, sh_degree, M, L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(shs),
-        L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(cam_pos), L.ptr(trans_mat),
-        L.ptr(radii), L.ptr(colors), L.ptr(grad_mean2D), L.ptr(grad_trans), L.ptr(grad_colors), L.ptr(grad_normals),
-        L.ptr(grad_means3D), L.ptr(grad_scales), L.ptr(grad_rotations), L.ptr(grad_opacities), L.ptr(grad_shs),
-        L.ptr(grad_sh_rest) if has_rest else None, L.current_stream())
+    with _timed('gs_2d_preprocess_backward'):
+        rc = _lib().fsgs_gs_2d_preprocess_backward(
+            P, W, H, sh_degree, M, L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(shs),
+            L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(cam_pos), L.ptr(trans_mat),
+            L.ptr(radii), L.ptr(colors), L.ptr(grad_mean2D), L.ptr(grad_trans), L.ptr(grad_colors), L.ptr(grad_normals),
+            L.ptr(grad_means3D), L.ptr(grad_scales), L.ptr(grad_rotations), L.ptr(grad_opacities), L.ptr(grad_shs),
+            L.ptr(grad_sh_rest) if has_rest else None, L.current_stream())
     L.check(rc, what)
 
 
@@ -142,9 +167,10 @@ def gs_2d_compute_transmat_forward(W, H, means3D, scales, rotations, Tw2v, Tw2c)
     L.require_shape(what, 'Tw2c', Tw2c, 4, 4)
     trans_mat = torch.empty((P, 3, 3), dtype=torch.float32, device=means3D.device)
     normals = torch.empty((P, 3), dtype=torch.float32, device=means3D.device)
-    rc = _lib().fsgs_gs_2d_compute_transmat_forward(P, W, H, L.ptr(means3D), L.ptr(scales), L.ptr(rotations),
-                                                    L.ptr(Tw2v), L.ptr(Tw2c), L.ptr(trans_mat), L.ptr(normals),
-                                                    L.current_stream())
+    with _timed('gs_2d_compute_transmat_forward'):
+        rc = _lib().fsgs_gs_2d_compute_transmat_forward(P, W, H, L.ptr(means3D), L.ptr(scales), L.ptr(rotations),
+                                                        L.ptr(Tw2v), L.ptr(Tw2c), L.ptr(trans_mat), L.ptr(normals),
+                                                        L.current_stream())
     L.check(rc, what)
     return trans_mat, normals
 
@@ -161,10 +187,11 @@ def gs_2d_compute_trans_mat_backward(W, H, means3D, scales, rotations, Tw2v, Tw2
     g_means3D = torch.empty((P, 3), dtype=torch.float32, device=means3D.device)
     g_scales = torch.empty((P, 2), dtype=torch.float32, device=means3D.device)
     g_rot = torch.empty((P, 4), dtype=torch.float32, device=means3D.device)
-    rc = _lib().fsgs_gs_2d_compute_transmat_backward(P, W, H, L.ptr(means3D), L.ptr(scales), L.ptr(rotations),
-                                                     L.ptr(Tw2v), L.ptr(Tw2c), L.ptr(grad_matrix),
-                                                     L.ptr(grad_normals), L.ptr(g_means3D), L.ptr(g_scales),
-                                                     L.ptr(g_rot), L.current_stream())
+    with _timed('gs_2d_compute_transmat_backward'):
+        rc = _lib().fsgs_gs_2d_compute_transmat_backward(P, W, H, L.ptr(means3D), L.ptr(scales), L.ptr(rotations),
+                                                         L.ptr(Tw2v), L.ptr(Tw2c), L.ptr(grad_matrix),
+                                                         L.ptr(grad_normals), L.ptr(g_means3D), L.ptr(g_scales),
+                                                         L.ptr(g_rot), L.current_stream())
     L.check(rc, what)
     return [g_means3D, g_scales, g_rot]
 
@@ -187,15 +214,17 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
     offsets = torch.empty((max(P, 1),), dtype=torch.int64, device=dev)
     ws1 = _workspace(lib.fsgs_gs_prepare_scan_workspace_bytes(P), dev)
     R = ctypes.c_int64(0)
-    rc = lib.fsgs_gs_prepare_scan(P, L.ptr(tiles_touched), L.ptr(offsets), L.ptr(ws1), ws1.numel(),
-                                  ctypes.addressof(R), stream)
+    with _timed('gs_prepare_scan'):
+        rc = lib.fsgs_gs_prepare_scan(P, L.ptr(tiles_touched), L.ptr(offsets), L.ptr(ws1), ws1.numel(),
+                                      ctypes.addressof(R), stream)
     L.check(rc, what)
     R = int(R.value)
     point_list = torch.empty((R,), dtype=torch.int32, device=dev)
     keys = torch.empty((R,), dtype=torch.int64, device=dev) if return_keys else None
     ws2 = _workspace(lib.fsgs_gs_prepare_fill_workspace_bytes(R), dev)
-    rc = lib.fsgs_gs_prepare_fill(P, W, H, L.ptr(means2D), L.ptr(depths), L.ptr(radii), L.ptr(offsets), R,
-                                  L.ptr(ranges), L.ptr(point_list), L.ptr(keys), L.ptr(ws2), ws2.numel(), stream)
+    with _timed('gs_prepare_fill'):
+        rc = lib.fsgs_gs_prepare_fill(P, W, H, L.ptr(means2D), L.ptr(depths), L.ptr(radii), L.ptr(offsets), R,
+                                      L.ptr(ranges), L.ptr(point_list), L.ptr(keys), L.ptr(ws2), ws2.numel(), stream)
     L.check(rc, what)
     if debug:
         torch.cuda.synchronize()
@@ -235,11 +264,12 @@ def GS_2D_render_forward(width: int, height: int, means2D: Tensor, colors: Tenso
     n_contrib = torch.empty((2, height, width), dtype=torch.int32, device=colors.device)
     pixel_extras = None if only_image else torch.empty((9, height, width), **opt)
     pixel_flow = torch.empty((height, width, 2), **opt) if (not only_image and trans_mat_t2 is not None) else None
-    rc = _lib().fsgs_gs_2d_render_forward(
-        P, width, height, float(near_n), float(far_n), int(bool(only_image)), L.ptr(means2D), L.ptr(colors),
-        L.ptr(normal_opacity), L.ptr(trans_mat), L.ptr(point_list), L.ptr(ranges), L.ptr(trans_mat_t2),
-        L.ptr(accum_max_count), L.ptr(accum_weights_p), L.ptr(accum_weights_count), L.ptr(pixel_colors),
-        L.ptr(pixel_opacity), L.ptr(pixel_extras), L.ptr(pixel_flow), L.ptr(n_contrib), L.current_stream())
+    with _timed('gs_2d_render_forward'):
+        rc = _lib().fsgs_gs_2d_render_forward(
+            P, width, height, float(near_n), float(far_n), int(bool(only_image)), L.ptr(means2D), L.ptr(colors),
+            L.ptr(normal_opacity), L.ptr(trans_mat), L.ptr(point_list), L.ptr(ranges), L.ptr(trans_mat_t2),
+            L.ptr(accum_max_count), L.ptr(accum_weights_p), L.ptr(accum_weights_count), L.ptr(pixel_colors),
+            L.ptr(pixel_opacity), L.ptr(pixel_extras), L.ptr(pixel_flow), L.ptr(n_contrib), L.current_stream())
     L.check(rc, what)
     return pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib
 
@@ -266,12 +296,13 @@ def GS_2D_render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat2
                                                                 c(dL_dothers), c(dL_dout_flows))
     ranges, point_list, n_contrib = c(ranges), c(point_list), c(n_contrib)
     use_aux = out_others is not None and dL_dothers is not None
-    rc = _lib().fsgs_gs_2d_render_backward(
-        P, W, H, float(near_n), float(far_n), L.ptr(means2D), L.ptr(normal_opacity), L.ptr(colors), L.ptr(trans_mat),
-        L.ptr(trans_mat2), L.ptr(out_opacity), L.ptr(out_others) if use_aux else None,
-        L.ptr(out_flows) if dL_dout_flows is not None else None, L.ptr(dL_dout_color), L.ptr(dL_dout_opacity),
-        L.ptr(dL_dothers) if use_aux else None, L.ptr(dL_dout_flows), L.ptr(ranges), L.ptr(point_list),
-        L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_norm_op), L.current_stream())
+    with _timed('gs_2d_render_backward'):
+        rc = _lib().fsgs_gs_2d_render_backward(
+            P, W, H, float(near_n), float(far_n), L.ptr(means2D), L.ptr(normal_opacity), L.ptr(colors), L.ptr(trans_mat),
+            L.ptr(trans_mat2), L.ptr(out_opacity), L.ptr(out_others) if use_aux else None,
+            L.ptr(out_flows) if dL_dout_flows is not None else None, L.ptr(dL_dout_color), L.ptr(dL_dout_opacity),
+            L.ptr(dL_dothers) if use_aux else None, L.ptr(dL_dout_flows), L.ptr(ranges), L.ptr(point_list),
+            L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_norm_op), L.current_stream())
     L.check(rc, what)
     return g_colors, g_means2D, g_trans, g_norm_op
 
@@ -291,8 +322,9 @@ def SH_to_RGB_forward(dir_or_pos: Tensor, campos: Optional[Tensor], sh_features:
     if not (0 <= degree <= 7 and (1 << degree) <= F):
         raise RuntimeError('degree error')
     rgb = torch.empty((P, 3), dtype=torch.float32, device=dir_or_pos.device)
-    rc = _lib().fsgs_sh_to_rgb_forward(P, F, degree, int(bool(clamp)), L.ptr(dir_or_pos), L.ptr(campos),
-                                       L.ptr(sh_features), L.ptr(rgb), L.current_stream())
+    with _timed('sh_to_rgb_forward'):
+        rc = _lib().fsgs_sh_to_rgb_forward(P, F, degree, int(bool(clamp)), L.ptr(dir_or_pos), L.ptr(campos),
+                                           L.ptr(sh_features), L.ptr(rgb), L.current_stream())
     L.check(rc, what)
     return rgb
 
@@ -310,9 +342,10 @@ def SH_to_RGB_backward(degree: int, clamp: bool, dir_or_pos: Tensor, campos: Opt
     if grad_campos is not None and grad_campos.shape != campos.shape:
         raise RuntimeError('ERROR shape for grad_campos')
     P, F = dir_or_pos.shape[0], sh_features.shape[-2]
-    rc = _lib().fsgs_sh_to_rgb_backward(P, F, degree, int(bool(clamp)), L.ptr(dir_or_pos.contiguous()),
-                                        L.ptr(campos), L.ptr(sh_features.contiguous()), L.ptr(rgb), L.ptr(grad_rgb),
-                                        L.ptr(grad_dir), L.ptr(grad_campos), L.ptr(grad_shs), L.current_stream())
+    with _timed('sh_to_rgb_backward'):
+        rc = _lib().fsgs_sh_to_rgb_backward(P, F, degree, int(bool(clamp)), L.ptr(dir_or_pos.contiguous()),
+                                            L.ptr(campos), L.ptr(sh_features.contiguous()), L.ptr(rgb), L.ptr(grad_rgb),
+                                            L.ptr(grad_dir), L.ptr(grad_campos), L.ptr(grad_shs), L.current_stream())
     L.check(rc, what)
 
 
@@ -320,7 +353,8 @@ def sh_encode_forward(inputs: Tensor, outputs: Tensor, B: int, D: int, C: int) -
     """nerf/shencoder.cu:657-673: outputs[B,(C+1)^2] <- basis values of inputs[B,D][:, :3]."""
     what = 'sh_encode_forward'
     _f32(what, inputs=inputs, outputs=outputs)
-    rc = _lib().fsgs_sh_encode_forward(B, D, C, L.ptr(inputs), L.ptr(outputs), L.current_stream())
+    with _timed('sh_encode_forward'):
+        rc = _lib().fsgs_sh_encode_forward(B, D, C, L.ptr(inputs), L.ptr(outputs), L.current_stream())
     L.check(rc, what)
 
 
@@ -328,7 +362,8 @@ def sh_encode_backward(grad: Tensor, inputs: Tensor, B: int, D: int, C: int, gra
     """nerf/shencoder.cu:675-691."""
     what = 'sh_encode_backward'
     _f32(what, grad=grad, inputs=inputs, grad_inputs=grad_inputs)
-    rc = _lib().fsgs_sh_encode_backward(B, D, C, L.ptr(grad), L.ptr(inputs), L.ptr(grad_inputs), L.current_stream())
+    with _timed('sh_encode_backward'):
+        rc = _lib().fsgs_sh_encode_backward(B, D, C, L.ptr(grad), L.ptr(inputs), L.ptr(grad_inputs), L.current_stream())
     L.check(rc, what)
 
 
@@ -340,8 +375,9 @@ def freq_encode_forward(inputs: Tensor, degree: int, include_inputs: bool, scale
     Dout = Din * (degree * 2 + int(bool(include_inputs)))
     B = inputs.numel() // Din
     out = torch.empty((*inputs.shape[:-1], Dout), dtype=torch.float32, device=inputs.device)
-    rc = _lib().fsgs_freq_encode_forward(B, Din, degree, int(bool(include_inputs)), float(scale), L.ptr(inputs),
-                                         L.ptr(out), L.current_stream())
+    with _timed('freq_encode_forward'):
+        rc = _lib().fsgs_freq_encode_forward(B, Din, degree, int(bool(include_inputs)), float(scale), L.ptr(inputs),
+                                             L.ptr(out), L.current_stream())
     L.check(rc, what)
     return out
 
@@ -356,8 +392,9 @@ def freq_encode_backward(grad: Tensor, outputs: Tensor, degree: int, include_inp
     Din = Dout // (degree * 2 + int(bool(include_inputs)))
     B = outputs.numel() // Dout
     gin = torch.empty((*outputs.shape[:-1], Din), dtype=torch.float32, device=outputs.device)
-    rc = _lib().fsgs_freq_encode_backward(B, Din, degree, int(bool(include_inputs)), float(scale), L.ptr(grad),
-                                          L.ptr(outputs), L.ptr(gin), L.current_stream())
+    with _timed('freq_encode_backward'):
+        rc = _lib().fsgs_freq_encode_backward(B, Din, degree, int(bool(include_inputs)), float(scale), L.ptr(grad),
+                                              L.ptr(outputs), L.ptr(gin), L.current_stream())
     L.check(rc, what)
     return gin
 
@@ -377,8 +414,9 @@ def cdist_top(x1: Tensor, x2: Tensor, largest: bool = False) -> List[Tensor]:
         raise RuntimeError('The shape[:-2] of x2 must be same with x1')
     distance = torch.empty(x1.shape[:-1], dtype=torch.float32, device=x1.device)
     index = torch.empty(x1.shape[:-1], dtype=torch.int64, device=x1.device)
-    rc = _lib().fsgs_cdist_top_forward(B, N, M, D, int(bool(largest)), L.ptr(x1), L.ptr(x2), L.ptr(distance),
-                                       L.ptr(index), L.current_stream())
+    with _timed('cdist_top_forward'):
+        rc = _lib().fsgs_cdist_top_forward(B, N, M, D, int(bool(largest)), L.ptr(x1), L.ptr(x2), L.ptr(distance),
+                                           L.ptr(index), L.current_stream())
     L.check(rc, what)
     return [distance, index]
 
@@ -392,8 +430,9 @@ def cdist_top_backward(x1: Tensor, x2: Tensor, distance: Tensor, index: Tensor, 
     B = x1.numel() // max(N * D, 1)
     g1 = torch.zeros_like(x1)
     g2 = torch.zeros_like(x2)
-    rc = _lib().fsgs_cdist_top_backward(B, N, M, D, L.ptr(x1), L.ptr(x2), L.ptr(distance), L.ptr(index),
-                                        L.ptr(grad_dist), L.ptr(g1), L.ptr(g2), L.current_stream())
+    with _timed('cdist_top_backward'):
+        rc = _lib().fsgs_cdist_top_backward(B, N, M, D, L.ptr(x1), L.ptr(x2), L.ptr(distance), L.ptr(index),
+                                            L.ptr(grad_dist), L.ptr(g1), L.ptr(g2), L.current_stream())
     L.check(rc, what)
     return [g1, g2]
 
@@ -409,9 +448,10 @@ def AdamMasksedUpdated(param: Tensor, param_grad: Tensor, exp_avg: Tensor, exp_a
     L.require_dtype(what, 'tiles_touched', tiles_touched, torch.bool)
     if param.numel() < N * M or tiles_touched.numel() < N:
         raise RuntimeError(f'{what}: tensors are smaller than N x M = {N} x {M}')
-    rc = _lib().fsgs_adam_masked_update(int(N), int(M), L.ptr(tiles_touched), float(lr), float(b1), float(b2),
-                                        float(eps), L.ptr(param), L.ptr(param_grad), L.ptr(exp_avg),
-                                        L.ptr(exp_avg_sq), L.current_stream())
+    with _timed('adam_masked_update'):
+        rc = _lib().fsgs_adam_masked_update(int(N), int(M), L.ptr(tiles_touched), float(lr), float(b1), float(b2),
+                                            float(eps), L.ptr(param), L.ptr(param_grad), L.ptr(exp_avg),
+                                            L.ptr(exp_avg_sq), L.current_stream())
     L.check(rc, what)
 
 
@@ -427,7 +467,8 @@ def knn_topk(x: Tensor, y: Tensor, K: int) -> Tuple[Tensor, Tensor]:
         raise RuntimeError(f'{what}: feature dimensions differ')
     dist2 = torch.empty((N, K), dtype=torch.float32, device=x.device)
     index = torch.empty((N, K), dtype=torch.int64, device=x.device)
-    rc = _lib().fsgs_knn_topk(N, M, D, K, L.ptr(x), L.ptr(y), L.ptr(dist2), L.ptr(index), L.current_stream())
+    with _timed('knn_topk'):
+        rc = _lib().fsgs_knn_topk(N, M, D, K, L.ptr(x), L.ptr(y), L.ptr(dist2), L.ptr(index), L.current_stream())
     L.check(rc, what)
     return dist2, index
 
@@ -448,8 +489,9 @@ def lbs_blend(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_
     weights = torch.empty((N, K), **opt)
     lib = _lib()
     ws = _workspace(lib.fsgs_lbs_blend_workspace_bytes(M), points.device)
-    rc = lib.fsgs_lbs_blend(N, M, K, int(bool(centred)), float(temperature), L.ptr(points), L.ptr(sp_points),
-                            L.ptr(sp_t), L.ptr(sp_r), L.ptr(sp_s), S, L.ptr(dist2), L.ptr(index), L.ptr(weights),
-                            L.ptr(d_xyz), L.ptr(d_rot), L.ptr(d_scale), L.ptr(ws), ws.numel(), L.current_stream())
+    with _timed('lbs_blend'):
+        rc = lib.fsgs_lbs_blend(N, M, K, int(bool(centred)), float(temperature), L.ptr(points), L.ptr(sp_points),
+                                L.ptr(sp_t), L.ptr(sp_r), L.ptr(sp_s), S, L.ptr(dist2), L.ptr(index), L.ptr(weights),
+                                L.ptr(d_xyz), L.ptr(d_rot), L.ptr(d_scale), L.ptr(ws), ws.numel(), L.current_stream())
     L.check(rc, what)
     return d_xyz, d_rot, d_scale, weights

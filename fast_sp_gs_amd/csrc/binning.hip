@@ -115,7 +115,8 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(int P, const i
 // ---- key duplication ------------------------------------------------------------------------------------------------
 constexpr int kCoopThreshold = 32;
 
-__global__ void __launch_bounds__(256) duplicate_keys_kernel(int P, int gx, int gy, const float2* __restrict__ means2D,
+__global__ void __launch_bounds__(256) duplicate_keys_kernel(int P, int gx, int gy, int64_t R,
+    const float2* __restrict__ means2D,
     const float* __restrict__ depths, const int32_t* __restrict__ radii, const int64_t* __restrict__ offsets,
     uint64_t* __restrict__ keys, int32_t* __restrict__ vals) {
   const int i    = blockIdx.x * blockDim.x + threadIdx.x;
@@ -136,8 +137,10 @@ __global__ void __launch_bounds__(256) duplicate_keys_kernel(int P, int gx, int 
   if (count > 0 && count <= kCoopThreshold) {
     for (int y = 0; y < h; ++y)
       for (int x = 0; x < w; ++x) {
-        keys[off] = ((uint64_t) (uint32_t) ((y0 + y) * gx + (x0 + x)) << 32) | dbits;
-        vals[off] = i;
+        if (off < R) {  // offsets come from the caller's tiles_touched; never write past the buffers it sized
+          keys[off] = ((uint64_t) (uint32_t) ((y0 + y) * gx + (x0 + x)) << 32) | dbits;
+          vals[off] = i;
+        }
         ++off;
       }
   }
@@ -153,8 +156,10 @@ __global__ void __launch_bounds__(256) duplicate_keys_kernel(int P, int gx, int 
                          (uint32_t) __shfl((int) (off & 0xffffffff), src, kWave);
     for (int e = lane; e < scount; e += kWave) {
       const int y = e / sw, x = e - y * sw;
-      keys[soff + e] = ((uint64_t) (uint32_t) ((sy0 + y) * gx + (sx0 + x)) << 32) | sbits;
-      vals[soff + e] = sid;
+      if (soff + e < R) {
+        keys[soff + e] = ((uint64_t) (uint32_t) ((sy0 + y) * gx + (sx0 + x)) << 32) | sbits;
+        vals[soff + e] = sid;
+      }
     }
   }
 }
@@ -380,8 +385,8 @@ FSGS_API int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, con
   vbuf[passes & 1]       = point_list;
   vbuf[(passes & 1) ^ 1] = (int32_t*) (ws + L.vals_alt);
 
-  hipLaunchKernelGGL(duplicate_keys_kernel, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, (const float2*) means2D,
-                     depths, radii, point_offsets, kbuf[0], vbuf[0]);
+  hipLaunchKernelGGL(duplicate_keys_kernel, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
+                     (const float2*) means2D, depths, radii, point_offsets, kbuf[0], vbuf[0]);
   for (int p = 0; p < passes; ++p) {
     const int shift = p * kRadixBits;
     const int a = p & 1, b = a ^ 1;

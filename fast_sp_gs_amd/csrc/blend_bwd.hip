@@ -43,7 +43,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
   const float pxf = (float) px, pyf = (float) py;
   const int lane = threadIdx.x & 63;
 
-  const int64_t r0         = ranges[2 * (size_t) tile];
+  const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
   const int last_contrib   = inside ? n_contrib[pix] : 0;
   const int median_contrib = (kAux && inside) ? n_contrib[pix + HW] : 0;
 
@@ -59,7 +59,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
 #pragma unroll
   for (int c = 0; c < kGradSlots + 1; ++c) s_acc[threadIdx.x][c] = 0.0f;
   __syncthreads();
-  const int n_todo = s_max_contrib;  // positions [0, n_todo) of the tile's list, walked from n_todo-1 down to 0
+  const int n_todo = min(s_max_contrib, (int) (r1 - r0));  // positions [0, n_todo) of the tile's list, walked from n_todo-1 down to 0
   const int rounds = (n_todo + kBatch - 1) / kBatch;
 
   const float T_final = inside ? 1.0f - out_opacity[pix] : 0.0f;
