@@ -86,6 +86,49 @@ __device__ __forceinline__ bool intersect(const SplatHot& h, float pxf, float py
   return !(o.alpha < (1.0f / 255.0f));
 }
 
+// ---- conservative per-quadrant culling ------------------------------------------------------------------------------
+// A surfel can only be blended at a pixel if alpha = min(0.99, o * exp(-rho / 2)) >= 1/255, i.e. rho <= tau with
+// tau = 2 ln(255 o), where rho = min(rho3d, rho2d). The pixels with rho3d <= tau are the perspective image of the
+// ellipse u^2 + v^2 <= tau in the surfel's tangent plane; its exact screen-space bounding box follows from the same
+// homogeneous form the preprocess uses for its 3-sigma bound (gs_2d_preprocess.cu:125-156) with cutoff^2 = tau. The
+// pixels with rho2d <= tau are a disc of radius sqrt(tau / 2) around the screen-space centre. The union of both boxes,
+// padded by 1 pixel + 0.5 % of its extent against rounding, is tested against the four 8x8 quadrants of the tile; a
+// clear bit means no pixel of that quadrant can pass the reference's alpha test, so skipping it changes nothing.
+// Surfels whose tau-ellipse reaches the camera plane (no finite box) keep all bits set.
+__device__ __forceinline__ unsigned quadrant_mask(const SplatHot& h, int tile_px, int tile_py) {
+  const float oa = 255.0f * h.opacity;
+  if (!(oa >= 1.0f)) return 0u;  // alpha can never reach 1/255
+  const float tau = 2.0f * __logf(oa) * 1.0001f + 1e-3f;
+  float x0, x1, y0, y1;
+  const float r2 = sqrtf(0.5f * tau);
+  x0 = h.cx - r2, x1 = h.cx + r2, y0 = h.cy - r2, y1 = h.cy + r2;
+  const float* M = h.m;
+  const float d  = tau * (M[6] * M[6] + M[7] * M[7]) - M[8] * M[8];
+  bool finite_box = (M[8] > 0.0f) && (d < -1e-6f * M[8] * M[8]);
+  if (finite_box) {
+    const float inv = 1.0f / d;
+    const float f0 = tau * inv, f2 = -inv;
+    const float cx = f0 * (M[0] * M[6] + M[1] * M[7]) + f2 * (M[2] * M[8]);
+    const float cy = f0 * (M[3] * M[6] + M[4] * M[7]) + f2 * (M[5] * M[8]);
+    const float hx = cx * cx - (f0 * (M[0] * M[0] + M[1] * M[1]) + f2 * (M[2] * M[2]));
+    const float hy = cy * cy - (f0 * (M[3] * M[3] + M[4] * M[4]) + f2 * (M[5] * M[5]));
+    const float ex = sqrtf(fmaxf(hx, 0.0f)), ey = sqrtf(fmaxf(hy, 0.0f));
+    finite_box = (ex == ex) && (ey == ey) && (cx == cx) && (cy == cy);
+    x0 = fminf(x0, cx - ex), x1 = fmaxf(x1, cx + ex);
+    y0 = fminf(y0, cy - ey), y1 = fmaxf(y1, cy + ey);
+  }
+  if (!finite_box) return 0xfu;
+  const float padx = 1.0f + 0.005f * (x1 - x0), pady = 1.0f + 0.005f * (y1 - y0);
+  x0 -= padx, x1 += padx, y0 -= pady, y1 += pady;
+  unsigned m = 0u;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float qx = (float) (tile_px + (q & 1) * 8), qy = (float) (tile_py + (q >> 1) * 8);
+    if (x1 >= qx && x0 <= qx + 7.0f && y1 >= qy && y0 <= qy + 7.0f) m |= 1u << q;
+  }
+  return m;
+}
+
 // ---- wave64 reductions through DPP --------------------------------------------------------------------------------
 template <int kCtrl, int kRowMask, int kBankMask>
 __device__ __forceinline__ float dpp_shift_zero(float v) {

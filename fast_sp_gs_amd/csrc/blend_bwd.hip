@@ -32,6 +32,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
   __shared__ float s_acc[kBatch][kGradSlots + 1];  // +1: odd stride keeps the flush conflict free
   __shared__ float s_t2[kFlow ? kBatch * 9 : 1];
   __shared__ int s_max_contrib;
+  __shared__ unsigned char s_mask[kBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
 
   const int gx = (W + kTile - 1) / kTile;
   const int tile = blockIdx.x, tile_x = tile % gx, tile_y = tile / gx;
@@ -41,7 +42,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
   const size_t HW   = (size_t) H * W;
   const size_t pix  = (size_t) W * py + px;
   const float pxf = (float) px, pyf = (float) py;
-  const int lane = threadIdx.x & 63;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
   const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
   const int last_contrib   = inside ? n_contrib[pix] : 0;
@@ -50,12 +51,10 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
   // deepest list position any pixel of the tile blended: nothing behind it needs to be gathered
   if (threadIdx.x == 0) s_max_contrib = 0;
   __syncthreads();
-  {
-    int m = last_contrib;
+  int wave_max_contrib = last_contrib;  // deepest position blended by this wavefront's quadrant
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) m = max(m, __shfl_xor(m, d, kWave));
-    if (lane == 0) atomicMax(&s_max_contrib, m);
-  }
+  for (int d = 32; d >= 1; d >>= 1) wave_max_contrib = max(wave_max_contrib, __shfl_xor(wave_max_contrib, d, kWave));
+  if (lane == 0) atomicMax(&s_max_contrib, wave_max_contrib);
 #pragma unroll
   for (int c = 0; c < kGradSlots + 1; ++c) s_acc[threadIdx.x][c] = 0.0f;
   __syncthreads();
@@ -110,6 +109,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
     if ((int) threadIdx.x < n_here) {
       s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
+      s_mask[threadIdx.x] = (unsigned char) quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile);
       if (kFlow)
 #pragma unroll
         for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
@@ -123,7 +123,15 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
         for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
     }
 
-    for (int j = 0; j < n_here; ++j) {
+    // Work list of this wavefront for 64 staged surfels at a time: those that can reach its quadrant and are not
+    // behind its deepest contributor; consumed bit by bit with scalar instructions.
+    for (int chunk = 0; chunk < kBatch / kWave; ++chunk) {
+     const int jj = chunk * kWave + lane;
+     unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u) &&
+                                        (n_todo - 1 - (b * kBatch + jj)) < wave_max_contrib);
+     while (todo) {
+      const int j = chunk * kWave + __builtin_ctzll(todo);
+      todo &= todo - 1;
       const int pos = n_todo - 1 - (b * kBatch + j);  // 0-based position in the tile's list
       Hit h;
       const bool hit = (pos < last_contrib) && intersect(s_hot[j], pxf, pyf, near_n, h);
@@ -216,6 +224,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
         const float s = wave_sum_to_lane63(g[c]);
         if (lane == 63) atomicAdd(&s_acc[j][c], s);
       }
+     }
     }
     __syncthreads();
     // flush the batch: one global atomic per surfel and component for this tile

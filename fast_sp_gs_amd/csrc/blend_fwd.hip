@@ -26,6 +26,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   __shared__ SplatHot s_hot[kBatch];
   __shared__ SplatCold s_cold[kBatch];
   __shared__ float s_t2[kFlow ? kBatch * 9 : 1];
+  __shared__ unsigned char s_mask[kBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
 
   const int gx = (W + kTile - 1) / kTile;
   const int tile = blockIdx.x, tile_x = tile % gx, tile_y = tile / gx;
@@ -35,6 +36,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   const size_t HW   = (size_t) H * W;
   const size_t pix  = (size_t) W * py + px;
   const float pxf = (float) px, pyf = (float) py;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
   const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
   const int n_todo = (int) (r1 - r0);
@@ -63,6 +65,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
     if ((int) threadIdx.x < n_here) {
       s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
+      s_mask[threadIdx.x] = (unsigned char) quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile);
       if (kFlow)
 #pragma unroll
         for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
@@ -76,48 +79,58 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
         for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
     }
 
-    for (int j = 0; !done && j < n_here; ++j) {
-      Hit h;
-      if (!intersect(s_hot[j], pxf, pyf, near_n, h)) continue;
-      const float test_T = T * (1.0f - h.alpha);
-      if (test_T < 0.0001f) {
-        done = true;
-        continue;
-      }
-      const float w        = h.alpha * T;
-      const SplatCold cold = s_cold[j];
-      const int contributor = b * kBatch + j + 1;
-      if (kAux) {
-        const float A = 1.0f - T;
-        const float m = far_n / (far_n - near_n) * (1.0f - near_n / h.depth);
-        dist += (m * m * A + M2 - 2.0f * m * M1) * w;
-        D += h.depth * w;
-        M1 += m * w;
-        M2 += m * m * w;
-        if (T > 0.5f) median = h.depth, median_c = contributor;
-        N0 += cold.nx * w, N1 += cold.ny * w, N2 += cold.nz * w;
+    // Each wavefront walks only the surfels that can reach its quadrant: the ballot of the mask bit over 64 staged
+    // surfels is the (depth-ordered) work list, consumed bit by bit with scalar instructions.
+    for (int c = 0; c < kBatch / kWave; ++c) {
+      const int jj = c * kWave + lane;
+      unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u));
+      while (todo) {
+        if (__ballot(!done) == 0ull) break;  // every pixel of this quadrant is saturated
+        const int j = c * kWave + __builtin_ctzll(todo);
+        todo &= todo - 1;
+        if (done) continue;
+        Hit h;
+        if (!intersect(s_hot[j], pxf, pyf, near_n, h)) continue;
+        const float test_T = T * (1.0f - h.alpha);
+        if (test_T < 0.0001f) {
+          done = true;
+          continue;
+        }
+        const float w        = h.alpha * T;
+        const SplatCold cold = s_cold[j];
+        const int contributor = b * kBatch + j + 1;
+        if (kAux) {
+          const float A = 1.0f - T;
+          const float m = far_n / (far_n - near_n) * (1.0f - near_n / h.depth);
+          dist += (m * m * A + M2 - 2.0f * m * M1) * w;
+          D += h.depth * w;
+          M1 += m * w;
+          M2 += m * m * w;
+          if (T > 0.5f) median = h.depth, median_c = contributor;
+          N0 += cold.nx * w, N1 += cold.ny * w, N2 += cold.nz * w;
+          if (kAccum) {
+            if (wmax < w) wmax = w, wmax_id = cold.id, flag = true;
+            if (accum_weights_p) atomicAdd(&accum_weights_p[cold.id], w);
+            if (accum_weights_count) atomicAdd(&accum_weights_count[cold.id], 1);
+          }
+          if (kFlow) {
+            const float* Q = &s_t2[j * 9];
+            const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
+            const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
+            float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
+            w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
+            f0 += (u2 / w2 - pxf) * w;
+            f1 += (v2 / w2 - pyf) * w;
+          }
+          wsum += w;
+        }
         if (kAccum) {
-          if (wmax < w) wmax = w, wmax_id = cold.id, flag = true;
-          if (accum_weights_p) atomicAdd(&accum_weights_p[cold.id], w);
-          if (accum_weights_count) atomicAdd(&accum_weights_count[cold.id], 1);
+          if (flag && accum_max_count) atomicAdd(&accum_max_count[wmax_id], 1);
         }
-        if (kFlow) {
-          const float* Q = &s_t2[j * 9];
-          const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
-          const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
-          float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
-          w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
-          f0 += (u2 / w2 - pxf) * w;
-          f1 += (v2 / w2 - pyf) * w;
-        }
-        wsum += w;
+        C0 += cold.r * w, C1 += cold.g * w, C2 += cold.b * w;
+        T    = test_T;
+        last = contributor;
       }
-      if (kAccum) {
-        if (flag && accum_max_count) atomicAdd(&accum_max_count[wmax_id], 1);
-      }
-      C0 += cold.r * w, C1 += cold.g * w, C2 += cold.b * w;
-      T    = test_T;
-      last = contributor;
     }
   }
 
