@@ -147,4 +147,38 @@ __device__ __forceinline__ float wave_sum_to_lane63(float v) {
   return v;
 }
 
+// Sums 16 per-lane values over the 64 lanes at once ("transposed" butterfly): each step halves the number of live
+// registers while doubling the lanes a partial covers, so 16 wave-wide sums cost 15 merge steps (2 DPP adds + 1 select
+// each) plus two cross-row exchanges, instead of 16 x 6 dependent DPP adds. On return every lane holds the wave total of
+// v[lane & 15].
+__device__ __forceinline__ float wave_sum16_transposed(const float (&v)[16]) {
+  const int lane = __lane_id();
+  const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4, b3 = lane & 8;
+  float w[8], x[4], y[2];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float a = v[2 * i + 1] + dpp_shift_zero<0x111, 0xf, 0xf>(v[2 * i + 1]);  // row_shr:1, kept by odd lanes
+    const float b = v[2 * i] + dpp_shift_zero<0x101, 0xf, 0xf>(v[2 * i]);          // row_shl:1, kept by even lanes
+    w[i] = b0 ? a : b;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float a = w[2 * i + 1] + dpp_shift_zero<0x112, 0xf, 0xf>(w[2 * i + 1]);  // row_shr:2
+    const float b = w[2 * i] + dpp_shift_zero<0x102, 0xf, 0xf>(w[2 * i]);          // row_shl:2
+    x[i] = b1 ? a : b;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const float a = x[2 * i + 1] + dpp_shift_zero<0x114, 0xf, 0xf>(x[2 * i + 1]);  // row_shr:4
+    const float b = x[2 * i] + dpp_shift_zero<0x104, 0xf, 0xf>(x[2 * i]);          // row_shl:4
+    y[i] = b2 ? a : b;
+  }
+  const float a = y[1] + dpp_shift_zero<0x118, 0xf, 0xf>(y[1]);  // row_shr:8
+  const float b = y[0] + dpp_shift_zero<0x108, 0xf, 0xf>(y[0]);  // row_shl:8
+  float z = b3 ? a : b;                                          // lane l of every row: row total of v[l & 15]
+  z += __shfl_xor(z, 16, kWave);
+  z += __shfl_xor(z, 32, kWave);
+  return z;
+}
+
 }  // namespace fsgs

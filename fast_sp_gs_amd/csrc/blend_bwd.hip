@@ -16,7 +16,10 @@
 namespace fsgs {
 namespace {
 
-constexpr int kGradSlots = 18;  // colours 3 | means2D 2 | trans_mat 9 | normal 3 + opacity 1
+// Per-surfel gradient slots: 0-2 colours | 3-11 trans_mat | 12-14 normal | 15 opacity | 16-17 means2D.
+// The first 16 go through one transposed wave reduction; the means2D pair is only non-zero for pixels where the
+// screen-space low-pass filter wins (rho2d < rho3d) and is reduced separately when any lane took that branch.
+constexpr int kGradSlots = 18;
 
 template <bool kAux, bool kFlow>
 __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
@@ -81,7 +84,8 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
       sum_w      = out_extras[pix + 8 * HW];
     }
   }
-  const float final_A = 1.0f - T_final;
+  const float final_A   = 1.0f - T_final;
+  const float far_scale = far_n / (far_n - near_n);
   float dLf0 = 0, dLf1 = 0, dL_dsum_w = 0;
   if (kFlow && inside) {
     const float2 g = dL_dflow[pix], o = out_flow[pix];
@@ -137,13 +141,14 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
       const bool hit = (pos < last_contrib) && intersect(s_hot[j], pxf, pyf, near_n, h);
       if (__ballot(hit) == 0ull) continue;  // wave-uniform: nobody in this quadrant blends the surfel
 
-      float g[kGradSlots];
+      float g[16], g2x = 0.0f, g2y = 0.0f;
+      bool filtered = false;
 #pragma unroll
-      for (int c = 0; c < kGradSlots; ++c) g[c] = 0.0f;
+      for (int c = 0; c < 16; ++c) g[c] = 0.0f;
       if (hit) {
         const SplatHot& hot  = s_hot[j];
         const SplatCold cold = s_cold[j];
-        T             = T / (1.0f - h.alpha);
+        T             = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
         const float w = h.alpha * T;
         float dL_dalpha = 0.0f;
         acc_c0 = last_alpha * last_c0 + (1.0f - last_alpha) * acc_c0, last_c0 = cold.r;
@@ -154,8 +159,9 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
 
         float dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f;
         if (kAux) {
-          const float m_d    = far_n / (far_n - near_n) * (1.0f - near_n / h.depth);
-          const float dmd_dd = (far_n * near_n) / ((far_n - near_n) * h.depth * h.depth);
+          const float rd     = __builtin_amdgcn_rcpf(h.depth);
+          const float m_d    = far_scale * (1.0f - near_n * rd);
+          const float dmd_dd = far_scale * near_n * rd * rd;
           if (pos == median_contrib - 1) dL_dz += dL_dmedian;
           const float dL_dweight = (final_D2 + m_d * m_d * final_A - 2.0f * m_d * final_D) * dL_dreg;
           dL_dalpha += dL_dweight - last_dL_dT;
@@ -171,7 +177,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
           acc_n1 = last_alpha * last_n1 + (1.0f - last_alpha) * acc_n1, last_n1 = cold.ny;
           acc_n2 = last_alpha * last_n2 + (1.0f - last_alpha) * acc_n2, last_n2 = cold.nz;
           dL_dalpha += (cold.nx - acc_n0) * dLn0 + (cold.ny - acc_n1) * dLn1 + (cold.nz - acc_n2) * dLn2;
-          g[14] = w * dLn0, g[15] = w * dLn1, g[16] = w * dLn2;
+          g[12] = w * dLn0, g[13] = w * dLn1, g[14] = w * dLn2;
           dL_dz += w * dL_ddepth;
           dsx = dL_dz * hot.m[6], dsy = dL_dz * hot.m[7];
         }
@@ -204,25 +210,26 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
           const float dpz = -(dpx * h.sx + dpy * h.sy);
           const float dkx = h.ly * dpz - h.lz * dpy, dky = h.lz * dpx - h.lx * dpz, dkz = h.lx * dpy - h.ly * dpx;
           const float dlx = dpy * h.kz - dpz * h.ky, dly = dpz * h.kx - dpx * h.kz, dlz = dpx * h.ky - dpy * h.kx;
-          g[5] = -dkx, g[6] = -dky, g[7] = -dkz;
-          g[8] = -dlx, g[9] = -dly, g[10] = -dlz;
-          g[11] = pxf * dkx + pyf * dlx + dL_dz * h.sx;
-          g[12] = pxf * dky + pyf * dly + dL_dz * h.sy;
-          g[13] = pxf * dkz + pyf * dlz + dL_dz;
+          g[3] = -dkx, g[4] = -dky, g[5] = -dkz;
+          g[6] = -dlx, g[7] = -dly, g[8] = -dlz;
+          g[9]  = pxf * dkx + pyf * dlx + dL_dz * h.sx;
+          g[10] = pxf * dky + pyf * dly + dL_dz * h.sy;
+          g[11] = pxf * dkz + pyf * dlz + dL_dz;
         } else {
-          g[3]  = dL_dG * (-h.G * 2.0f * h.dx);
-          g[4]  = dL_dG * (-h.G * 2.0f * h.dy);
-          g[11] = dL_dz * h.sx;
-          g[12] = dL_dz * h.sy;
-          g[13] = dL_dz;
+          g2x   = dL_dG * (-h.G * 2.0f * h.dx);
+          g2y   = dL_dG * (-h.G * 2.0f * h.dy);
+          g[9]  = dL_dz * h.sx;
+          g[10] = dL_dz * h.sy;
+          g[11] = dL_dz;
+          filtered = true;
         }
-        g[17] = h.G * dL_dalpha;
+        g[15] = h.G * dL_dalpha;
       }
-#pragma unroll
-      for (int c = 0; c < kGradSlots; ++c) {
-        if (!kAux && c >= 14 && c <= 16) continue;
-        const float s = wave_sum_to_lane63(g[c]);
-        if (lane == 63) atomicAdd(&s_acc[j][c], s);
+      const float tot = wave_sum16_transposed(g);
+      if (lane < 16) atomicAdd(&s_acc[j][lane], tot);  // one LDS atomic instruction for all 16 components
+      if (__ballot(filtered) != 0ull) {
+        const float sx = wave_sum_to_lane63(g2x), sy = wave_sum_to_lane63(g2y);
+        if (lane == 63) atomicAdd(&s_acc[j][16], sx), atomicAdd(&s_acc[j][17], sy);
       }
      }
     }
@@ -235,14 +242,14 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
       for (int c = 0; c < 3; ++c)
         if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
-        if (a[3 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[3 + c]);
-#pragma unroll
       for (int c = 0; c < 9; ++c)
-        if (a[5 + c] != 0.0f) atomicAdd(&g_trans[9 * (size_t) id + c], a[5 + c]);
+        if (a[3 + c] != 0.0f) atomicAdd(&g_trans[9 * (size_t) id + c], a[3 + c]);
 #pragma unroll
       for (int c = 0; c < 4; ++c)
-        if (a[14 + c] != 0.0f) atomicAdd(&g_normal_opacity[4 * (size_t) id + c], a[14 + c]);
+        if (a[12 + c] != 0.0f) atomicAdd(&g_normal_opacity[4 * (size_t) id + c], a[12 + c]);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+        if (a[16 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[16 + c]);
 #pragma unroll
       for (int c = 0; c < kGradSlots; ++c) a[c] = 0.0f;
     }
