@@ -1,0 +1,118 @@
+"""Pins the oracle's spherical-harmonic code (oracle/sh_basis.h and its users) without the reference:
+orthonormality of the basis under sphere quadrature, the degree-0 closed form, the l=1 sign convention (-y, +z, -x),
+central finite differences for every derivative, and the clamp mask of SH -> RGB."""
+import numpy as np
+import pytest
+
+
+def _sphere_quadrature(n_theta=64, n_phi=128):
+    # Gauss-Legendre in cos(theta) x uniform in phi integrates polynomials up to high degree exactly
+    ct, wt = np.polynomial.legendre.leggauss(n_theta)
+    phi = (np.arange(n_phi) + 0.5) * (2 * np.pi / n_phi)
+    CT, PH = np.meshgrid(ct, phi, indexing="ij")
+    ST = np.sqrt(1 - CT ** 2)
+    dirs = np.stack([ST * np.cos(PH), ST * np.sin(PH), CT], -1).reshape(-1, 3)
+    w = (wt[:, None] * np.full((1, n_phi), 2 * np.pi / n_phi)).reshape(-1)
+    return np.ascontiguousarray(dirs), w
+
+
+def _encode(O, dirs, degree):
+    out = np.zeros((dirs.shape[0], (degree + 1) ** 2), dirs.dtype)
+    suffix = "f64" if dirs.dtype == np.float64 else "f32"
+    assert O.call(f"sh_encode_forward_{suffix}", dirs.shape[0], 3, degree, dirs, out) == 0
+    return out
+
+
+def test_basis_is_orthonormal(oracle_mod):
+    dirs, w = _sphere_quadrature()
+    Y = _encode(oracle_mod, dirs, 3)
+    gram = (Y * w[:, None]).T @ Y
+    assert np.abs(gram - np.eye(16)).max() < 1e-12
+
+
+def test_degree0_and_l1_signs(oracle_mod):
+    d = np.array([[0.3, -0.5, 0.81]], np.float64)
+    Y = _encode(oracle_mod, d, 1)[0]
+    c1 = np.sqrt(3 / (4 * np.pi))
+    assert abs(Y[0] - 0.5 / np.sqrt(np.pi)) < 1e-15
+    assert np.allclose(Y[1:4], [-c1 * d[0, 1], c1 * d[0, 2], -c1 * d[0, 0]], atol=1e-15)
+
+
+def test_float_matches_double(oracle_mod):
+    rng = np.random.default_rng(0)
+    d = rng.normal(size=(1000, 3))
+    d /= np.linalg.norm(d, axis=1, keepdims=True)
+    assert np.abs(_encode(oracle_mod, d.astype(np.float32), 3) - _encode(oracle_mod, d, 3)).max() < 2e-6
+
+
+@pytest.mark.parametrize("degree", [0, 1, 2, 3])
+def test_encoder_backward_is_the_gradient(oracle_mod, degree):
+    rng = np.random.default_rng(degree)
+    B, n = 50, (degree + 1) ** 2
+    x = np.ascontiguousarray(rng.normal(size=(B, 3)))
+    g = np.ascontiguousarray(rng.normal(size=(B, n)))
+    gin = np.zeros((B, 3))
+    assert oracle_mod.call("sh_encode_backward_f64", B, 3, degree, g, x, gin) == 0
+    eps = 1e-6
+    fd = np.zeros((B, 3))
+    for a in range(3):
+        xp, xm = x.copy(), x.copy()
+        xp[:, a] += eps
+        xm[:, a] -= eps
+        fd[:, a] = ((_encode(oracle_mod, xp, degree) - _encode(oracle_mod, xm, degree)) * g).sum(1) / (2 * eps)
+    assert np.abs(gin - fd).max() < 1e-7
+
+
+@pytest.mark.parametrize("use_campos", [False, True])
+def test_sh_to_rgb_forward_backward(oracle_mod, use_campos):
+    O = oracle_mod
+    rng = np.random.default_rng(7)
+    P, F, degree = 40, 16, 3
+    pos = np.ascontiguousarray(rng.normal(size=(P, 3)))
+    if not use_campos:
+        pos /= np.linalg.norm(pos, axis=1, keepdims=True)
+    cam = np.array([0.1, -0.2, 3.0]) if use_campos else None
+    sh = np.ascontiguousarray(rng.normal(size=(P, F, 3)) * 0.4)
+    grad = np.ascontiguousarray(rng.normal(size=(P, 3)))
+
+    def fwd(pos_, cam_, sh_, clamp=1):
+        rgb = np.zeros((P, 3))
+        assert O.call("sh_to_rgb_forward_f64", P, F, degree, clamp, pos_, cam_, sh_, rgb) == 0
+        return rgb
+
+    rgb = fwd(pos, cam, sh)
+    # forward = max(0, 0.5 + sum_l Y_l c_l) with the (optionally normalised) direction
+    d = pos - cam if use_campos else pos
+    if use_campos:
+        d = d / np.sqrt((d * d).sum(1, keepdims=True) + 1e-12)
+    Y = _encode(O, np.ascontiguousarray(d), degree)
+    assert np.abs(rgb - np.maximum(0, 0.5 + np.einsum("pl,plc->pc", Y, sh))).max() < 1e-12
+    assert (rgb == 0).any() and (rgb > 0).any()  # the clamp is exercised
+
+    g_dir, g_sh = np.zeros((P, 3)), np.zeros((P, F, 3))
+    g_cam = np.zeros(3) if use_campos else None
+    assert O.call("sh_to_rgb_backward_f64", P, F, degree, 1, pos, cam, sh, rgb, grad, g_dir, g_cam, g_sh) == 0
+    eps = 1e-6
+    loss = lambda pos_, cam_, sh_: (fwd(pos_, cam_, sh_) * grad).sum()
+    # coefficients
+    for (p, l, c) in [(0, 0, 0), (3, 5, 1), (7, 15, 2), (11, 9, 0)]:
+        shp, shm = sh.copy(), sh.copy()
+        shp[p, l, c] += eps
+        shm[p, l, c] -= eps
+        assert abs((loss(pos, cam, shp) - loss(pos, cam, shm)) / (2 * eps) - g_sh[p, l, c]) < 1e-7
+    # position / direction, and the camera position (sum over points, opposite sign)
+    cam_fd = np.zeros(3)
+    for a in range(3):
+        for p in range(0, P, 7):
+            pp, pm = pos.copy(), pos.copy()
+            pp[p, a] += eps
+            pm[p, a] -= eps
+            assert abs((loss(pp, cam, sh) - loss(pm, cam, sh)) / (2 * eps) - g_dir[p, a]) < 1e-6
+        if use_campos:
+            cp, cm = cam.copy(), cam.copy()
+            cp[a] += eps
+            cm[a] -= eps
+            cam_fd[a] = (loss(pos, cp, sh) - loss(pos, cm, sh)) / (2 * eps)
+    if use_campos:
+        assert np.abs(cam_fd - g_cam).max() < 1e-6
+        assert np.abs(g_cam + g_dir.sum(0)).max() < 1e-9
