@@ -1,0 +1,182 @@
+"""Pins the oracle's stand-alone operators (oracle/ops.cpp) against library routines and closed forms:
+cdist top-1 and its tie rules, K-NN, LBS, masked Adam vs torch.optim.Adam, the frequency encoder vs torch.sin/cos,
+the deformation MLP vs a torch.nn.functional.linear chain."""
+import numpy as np
+import pytest
+import torch
+
+
+def test_cdist_top_matches_torch_and_tie_rules(oracle_mod):
+    O = oracle_mod
+    rng = np.random.default_rng(0)
+    B, N, M, D = 2, 300, 40, 5
+    x = np.ascontiguousarray(rng.normal(size=(B, N, D)).astype(np.float32))
+    y = np.ascontiguousarray(rng.normal(size=(B, M, D)).astype(np.float32))
+    for largest in (0, 1):
+        dist, idx = np.zeros((B, N), np.float32), np.zeros((B, N), np.int64)
+        assert O.call("cdist_top_forward_f32", B, N, M, D, largest, x, y, dist, idx) == 0
+        full = torch.cdist(torch.from_numpy(x).double(), torch.from_numpy(y).double())
+        ref_v, ref_i = (full.max(-1) if largest else full.min(-1))
+        assert np.array_equal(idx, ref_i.numpy()) and np.abs(dist - ref_v.numpy()).max() < 1e-5
+    # ties: smallest keeps the LAST equal minimum, largest keeps the FIRST equal maximum (cdist_top.cu:24)
+    x1 = np.zeros((1, 1, 2), np.float32)
+    y1 = np.ascontiguousarray(np.array([[[1, 0], [0, 1], [-1, 0], [3, 0], [0, 3]]], np.float32))
+    dist, idx = np.zeros((1, 1), np.float32), np.zeros((1, 1), np.int64)
+    O.call("cdist_top_forward_f32", 1, 1, 5, 2, 0, x1, y1, dist, idx)
+    assert idx[0, 0] == 2 and dist[0, 0] == 1
+    O.call("cdist_top_forward_f32", 1, 1, 5, 2, 1, x1, y1, dist, idx)
+    assert idx[0, 0] == 3 and dist[0, 0] == 3
+
+
+def test_cdist_top_backward_matches_autograd(oracle_mod):
+    O = oracle_mod
+    rng = np.random.default_rng(1)
+    B, N, M, D = 2, 50, 20, 3
+    x = torch.from_numpy(rng.normal(size=(B, N, D))).requires_grad_()
+    y = torch.from_numpy(rng.normal(size=(B, M, D))).requires_grad_()
+    gd = torch.from_numpy(rng.normal(size=(B, N)))
+    v, i = torch.cdist(x, y).min(-1)
+    (v * gd).sum().backward()
+    g1, g2 = np.zeros((B, N, D)), np.zeros((B, M, D))
+    assert O.call("cdist_top_backward_f64", B, N, M, D, x.detach().numpy(), y.detach().numpy(), v.detach().numpy(),
+                  np.ascontiguousarray(i.numpy()), gd.numpy(), g1, g2) == 0
+    assert np.abs(g1 - x.grad.numpy()).max() < 1e-12 and np.abs(g2 - y.grad.numpy()).max() < 1e-12
+
+
+def test_knn_matches_sorting(oracle_mod):
+    O = oracle_mod
+    rng = np.random.default_rng(2)
+    N, M, D, K = 400, 64, 3, 4
+    x = np.ascontiguousarray(rng.uniform(-1, 1, size=(N, D)).astype(np.float32))
+    y = np.ascontiguousarray(rng.uniform(-1, 1, size=(M, D)).astype(np.float32))
+    y[10] = y[3]  # an exact duplicate: the lower index must come first
+    d2, idx = np.zeros((N, K), np.float32), np.zeros((N, K), np.int64)
+    assert O.call("knn_topk_f32", N, M, D, K, x, y, d2, idx) == 0
+    diff = x[:, None, :] - y[None]
+    full = ((diff[..., 0] * diff[..., 0] + diff[..., 1] * diff[..., 1]) + diff[..., 2] * diff[..., 2]).astype(np.float32)
+    order = np.argsort(full, axis=1, kind="stable")[:, :K]
+    assert np.array_equal(idx, order)
+    assert np.array_equal(d2, np.take_along_axis(full, order, 1))
+    assert (np.diff(d2, axis=1) >= 0).all()
+    # K larger than M: padded with -1
+    d2, idx = np.zeros((2, 5), np.float32), np.zeros((2, 5), np.int64)
+    O.call("knn_topk_f32", 2, 3, D, 5, x[:2].copy(), y[:3].copy(), d2, idx)
+    assert (idx[:, 3:] == -1).all() and (d2[:, 3:] == -1).all()
+
+
+def _lbs(O, points, ctrl, sp_t, sp_r, sp_s, d2, idx, temperature, centred):
+    N, K = d2.shape
+    S = sp_s.shape[1]
+    w, dx, dr, ds = np.zeros((N, K)), np.zeros((N, 3)), np.zeros((N, 4)), np.zeros((N, S))
+    assert O.call("lbs_blend_f64", N, ctrl.shape[0], K, int(centred), float(temperature), points, ctrl, sp_t, sp_r,
+                  sp_s, S, d2, idx, w, dx, dr, ds) == 0
+    return w, dx, dr, ds
+
+
+def test_lbs_closed_forms(oracle_mod):
+    O = oracle_mod
+    rng = np.random.default_rng(3)
+    N, M, K = 50, 8, 4
+    pts, ctrl = rng.normal(size=(N, 3)), rng.normal(size=(M, 3))
+    idx = np.ascontiguousarray(np.stack([rng.permutation(M)[:K] for _ in range(N)]).astype(np.int64))
+    d2 = np.ascontiguousarray(np.sort(rng.uniform(0, 0.05, size=(N, K)), 1))
+    zero3, zero4, s0 = np.zeros((M, 3)), np.zeros((M, 4)), np.zeros((M, 2))
+    # identity transforms (residual rotation 0 -> q = (0,0,0,1), t = 0) move nothing; weights are a softmax
+    w, dx, dr, ds = _lbs(O, pts, ctrl, zero3, zero4, s0, d2, idx, 0.01, False)
+    assert np.abs(dx).max() < 1e-14 and np.abs(dr).max() == 0
+    assert np.allclose(w, torch.softmax(torch.from_numpy(-d2 / 0.01), -1).numpy(), atol=1e-14)
+    # one control point everywhere with weight 1: a rigid motion p -> R p + t
+    ang, axis = 0.7, np.array([0.0, 0.6, 0.8])
+    q = np.concatenate([axis * np.sin(ang / 2), [np.cos(ang / 2)]])
+    from scipy.spatial.transform import Rotation
+    Rm = Rotation.from_quat(q).as_matrix()
+    t = np.array([0.1, -0.2, 0.3])
+    sp_r = np.tile(2.5 * q - np.array([0, 0, 0, 1.0]), (M, 1))  # normalize(r + (0,0,0,1)) == q
+    sp_t = np.tile(t, (M, 1))
+    w, dx, dr, ds = _lbs(O, pts, ctrl, sp_t, sp_r, s0 + 0.5, d2, idx, 0.01, False)
+    assert np.abs(dx - (pts @ Rm.T + t - pts)).max() < 1e-12
+    assert np.allclose(dr, sp_r[0]) and np.allclose(ds, 0.5)
+    # centred: rotation about the control point c: p -> R (p - c) + c + t
+    same = np.zeros((N, K), np.int64) + 5
+    w, dx, dr, ds = _lbs(O, pts, ctrl, sp_t, sp_r, s0, d2, same, 0.01, True)
+    assert np.abs(dx - ((pts - ctrl[5]) @ Rm.T + ctrl[5] + t - pts)).max() < 1e-12
+
+
+def test_masked_adam_matches_torch_adam(oracle_mod):
+    O = oracle_mod
+    rng = np.random.default_rng(4)
+    N, M = 64, 6
+    p0 = rng.normal(size=(N, M))
+    param = torch.nn.Parameter(torch.from_numpy(p0.copy()))
+    opt = torch.optim.Adam([param], lr=1.6e-4, betas=(0.9, 0.999), eps=1e-15)
+    p, m, v = p0.copy(), np.zeros((N, M)), np.zeros((N, M))
+    mask = np.ones(N, np.uint8)
+    for step in range(1, 4):
+        g = rng.normal(size=(N, M))
+        param.grad = torch.from_numpy(g.copy())
+        opt.step()
+        # SparseGaussianAdam folds the bias corrections into the learning rate (sparse_gaussian_adam.py:46)
+        lr = 1.6e-4 * (1 - 0.999 ** step) ** 0.5 / (1 - 0.9 ** step)
+        assert O.call("adam_masked_update_f64", N, M, mask, lr, 0.9, 0.999, 1e-15, p, np.ascontiguousarray(g), m, v) == 0
+        assert np.abs(p - param.detach().numpy()).max() < 1e-12
+    # masked rows are untouched, including their moments
+    mask[::2] = 0
+    before = (p.copy(), m.copy(), v.copy())
+    O.call("adam_masked_update_f64", N, M, mask, 1e-3, 0.9, 0.999, 1e-15, p, np.ascontiguousarray(rng.normal(size=(N, M))), m, v)
+    for a, b in zip(before, (p, m, v)):
+        assert np.array_equal(a[::2], b[::2]) and not np.array_equal(a[1::2], b[1::2])
+
+
+@pytest.mark.parametrize("include_input", [True, False])
+def test_freq_encoder(oracle_mod, include_input):
+    O = oracle_mod
+    rng = np.random.default_rng(5)
+    B, D, deg, scale = 37, 3, 10, 1.0
+    x = np.ascontiguousarray(rng.uniform(-1, 1, size=(B, D)))
+    Do = D * (2 * deg + int(include_input))
+    out = np.zeros((B, Do))
+    assert O.call("freq_encode_forward_f64", B, D, deg, int(include_input), scale, x, out) == 0
+    parts = [torch.from_numpy(x)] if include_input else []
+    for d in range(deg):
+        parts += [torch.sin(torch.from_numpy(x) * 2.0 ** d * scale), torch.cos(torch.from_numpy(x) * 2.0 ** d * scale)]
+    assert np.abs(out - torch.cat(parts, -1).numpy()).max() < 1e-9
+    g = np.ascontiguousarray(rng.normal(size=(B, Do)))
+    gin = np.zeros((B, D))
+    assert O.call("freq_encode_backward_f64", B, D, deg, int(include_input), scale, g, out, gin) == 0
+    xt = torch.from_numpy(x).requires_grad_()
+    parts = [xt] if include_input else []
+    for d in range(deg):
+        parts += [torch.sin(xt * 2.0 ** d * scale), torch.cos(xt * 2.0 ** d * scale)]
+    (torch.cat(parts, -1) * torch.from_numpy(g)).sum().backward()
+    assert np.abs(gin - xt.grad.numpy()).max() < 1e-8
+
+
+def test_deform_mlp_matches_torch(oracle_mod):
+    import ctypes
+    O = oracle_mod
+    torch.manual_seed(0)
+    B, Din, Wd, L, skip = 33, 84, 256, 8, 4
+    x = torch.randn(B, Din)
+    Ws, bs = [], []
+    for i in range(L):
+        din = Din if i == 0 else (Wd + Din if i == skip + 1 else Wd)
+        Ws.append(torch.randn(Wd, din) / din ** 0.5)
+        bs.append(torch.randn(Wd) * 0.1)
+    heads = [(torch.randn(3, Wd) * 0.1, torch.randn(3)), (torch.randn(4, Wd) * 0.1, torch.randn(4)),
+             (torch.randn(3, Wd) * 0.1, torch.randn(3))]
+    h = x
+    for i in range(L):  # network.py:1763-1767
+        h = torch.relu(torch.nn.functional.linear(h, Ws[i], bs[i]))
+        if i == skip:
+            h = torch.cat([x, h], -1)
+    ref = [torch.nn.functional.linear(h, w, b) for w, b in heads]
+    arr = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    outs = [torch.zeros(B, w.shape[0]) for w, _ in heads]
+    dims = (ctypes.c_int * 3)(3, 4, 3)
+    lib = O.lib()
+    lib.oracle_deform_mlp_f32.restype = ctypes.c_int
+    rc = lib.oracle_deform_mlp_f32(B, Din, Wd, L, skip, ctypes.c_void_p(x.data_ptr()), arr(Ws), arr(bs), 3, dims,
+                                   arr([w for w, _ in heads]), arr([b for _, b in heads]), arr(outs))
+    assert rc == 0
+    for o, r in zip(outs, ref):
+        assert (o - r).abs().max() < 1e-4
