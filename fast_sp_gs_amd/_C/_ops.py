@@ -19,6 +19,7 @@ __all__ = [
     'gs_2d_compute_trans_mat_backward', 'GS_prepare', 'GS_2D_render_forward', 'GS_2D_render_backward',
     'SH_to_RGB_forward', 'SH_to_RGB_backward', 'sh_encode_forward', 'sh_encode_backward', 'freq_encode_forward',
     'freq_encode_backward', 'cdist_top', 'cdist_top_backward', 'AdamMasksedUpdated', 'knn_topk', 'lbs_blend',
+    'gs_2d_topk_weights',
 ]
 
 _TILE = 16
@@ -305,6 +306,25 @@ def GS_2D_render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat2
             L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_norm_op), L.current_stream())
     L.check(rc, what)
     return g_colors, g_means2D, g_trans, g_norm_op
+
+
+def gs_2d_topk_weights(topk: int, W: int, H: int, near: float, far: float, means2D: Tensor, normal_opacity: Tensor,
+                       trans_mat: Tensor, ranges: Tensor, point_list: Tensor) -> Tuple[Tensor, Tensor]:
+    """gaussian_topk.cu:230-250 -> (top_indices[H,W,K] int32, top_weights[H,W,K])."""
+    what = 'gs_2d_topk_weights'
+    _f32(what, means2D=means2D, normal_opacity=normal_opacity, trans_mat=trans_mat)
+    L.require_cuda(what, ranges=ranges, point_list=point_list)
+    L.require_dtype(what, 'ranges', ranges, torch.int64)
+    L.require_dtype(what, 'point_list', point_list, torch.int32)
+    P = means2D.shape[0]
+    top_indices = torch.empty((H, W, topk), dtype=torch.int32, device=means2D.device)
+    top_weights = torch.empty((H, W, topk), dtype=torch.float32, device=means2D.device)
+    with _timed('gs_2d_topk_weights'):
+        rc = _lib().fsgs_gs_2d_topk_weights(topk, P, W, H, float(near), float(far), L.ptr(means2D),
+                                            L.ptr(normal_opacity), L.ptr(trans_mat), L.ptr(ranges), L.ptr(point_list),
+                                            L.ptr(top_indices), L.ptr(top_weights), L.current_stream())
+    L.check(rc, what)
+    return top_indices, top_weights
 
 
 # --------------------------------------------------------------------------------------------------------------------

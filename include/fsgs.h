@@ -92,6 +92,12 @@ int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n,
     const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
     float* g_normal_opacity, void* stream);
 
+/* gs_2d_topk_weights -- fast_2d_gs/_C/src/gaussian_splatting/gaussian_topk.cu:230-250 (kernel :95-210).
+ * top_indices[H,W,topk] int32 (-1 = empty), top_weights[H,W,topk] descending blend weights alpha*T; topk <= 16. */
+int fsgs_gs_2d_topk_weights(int topk, int P, int W, int H, double near_n, double far_n, const float* means2D,
+    const float* normal_opacity, const float* trans_mat, const int64_t* ranges, const int32_t* point_list,
+    int32_t* top_indices, float* top_weights, void* stream);
+
 /* ---- spherical harmonics and encoders ------------------------------------------------------------------------- */
 
 /* SH_to_RGB_forward / SH_to_RGB_backward -- fast_2d_gs/_C/src/ops_3d/spherical_harmonics.cu:15-41, :68-102.
