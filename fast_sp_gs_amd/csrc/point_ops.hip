@@ -19,6 +19,7 @@ namespace fsgs {
 namespace {
 
 // ---- SH -> RGB ----------------------------------------------------------------------------------------------------
+template <int kSh>
 __global__ void __launch_bounds__(256) sh_to_rgb_forward_kernel(int P, int F, int degree, int clamp,
     const float* __restrict__ pos, const float* __restrict__ campos, const float* __restrict__ sh,
     float* __restrict__ rgb) {
@@ -29,7 +30,7 @@ __global__ void __launch_bounds__(256) sh_to_rgb_forward_kernel(int P, int F, in
     const float p[3] = {x, y, z};
     view_dir(p, campos, x, y, z);
   }
-  float Y[16];
+  float Y[kSh];
   sh_eval(degree, x, y, z, Y);
   const int n    = sh_count(degree);
   const float* c = sh + (size_t) i * F * 3;
@@ -46,6 +47,7 @@ __device__ __forceinline__ float wave_sum_xor(float v) {
   return v;
 }
 
+template <int kSh>
 __global__ void __launch_bounds__(256) sh_to_rgb_backward_kernel(int P, int F, int degree, int clamp,
     const float* __restrict__ pos, const float* __restrict__ campos, const float* __restrict__ sh,
     const float* __restrict__ rgb, const float* __restrict__ grad_rgb, float* __restrict__ grad_dir,
@@ -63,7 +65,7 @@ __global__ void __launch_bounds__(256) sh_to_rgb_backward_kernel(int P, int F, i
       g[c] = grad_rgb[3 * (size_t) i + c];
       if (clamp) g[c] *= (float) (rgb[3 * (size_t) i + c] > 0);
     }
-    float Y[16], tl[16];
+    float Y[kSh], tl[kSh];
     sh_eval(degree, x, y, z, Y);
     const int n    = sh_count(degree);
     const float* c = sh + (size_t) i * F * 3;
@@ -96,11 +98,12 @@ __global__ void __launch_bounds__(256) sh_to_rgb_backward_kernel(int P, int F, i
 }
 
 // ---- bare SH encoder ------------------------------------------------------------------------------------------------
+template <int kSh>
 __global__ void __launch_bounds__(256) sh_encode_forward_kernel(int B, int D, int C, const float* __restrict__ in,
                                                                 float* __restrict__ out) {
   const int b = blockIdx.x * blockDim.x + threadIdx.x;
   if (b >= B) return;
-  float Y[16];
+  float Y[kSh];
   sh_eval(C, in[(size_t) b * D], in[(size_t) b * D + 1], in[(size_t) b * D + 2], Y);
   const int n = sh_count(C);
   float* o    = out + (size_t) b * n;
@@ -111,12 +114,13 @@ __global__ void __launch_bounds__(256) sh_encode_forward_kernel(int B, int D, in
   }
 }
 
+template <int kSh>
 __global__ void __launch_bounds__(256) sh_encode_backward_kernel(int B, int D, int C, const float* __restrict__ grad,
     const float* __restrict__ in, float* __restrict__ grad_in) {
   const int b = blockIdx.x * blockDim.x + threadIdx.x;
   if (b >= B) return;
   const int n = sh_count(C);
-  float t[16];
+  float t[kSh];
   const float* g = grad + (size_t) b * n;
   if ((n & 3) == 0) {
     for (int l = 0; l < n; l += 4) {
@@ -397,7 +401,8 @@ FSGS_API int fsgs_sh_to_rgb_forward(int P, int F, int degree, int clamp, const f
   FSGS_REQUIRE(0 <= degree && degree <= kMaxShDegree && (degree + 1) * (degree + 1) <= F,
                "SH_to_RGB_forward: degree %d unsupported or > features %d", degree, F);
   if (P == 0) return kOk;
-  hipLaunchKernelGGL(sh_to_rgb_forward_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, F, degree,
+  auto kernel = degree > 3 ? sh_to_rgb_forward_kernel<64> : sh_to_rgb_forward_kernel<16>;
+  hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, F, degree,
                      clamp, pos, campos, sh, rgb);
   return check_launch("SH_to_RGB_forward");
 }
@@ -410,7 +415,8 @@ FSGS_API int fsgs_sh_to_rgb_backward(int P, int F, int degree, int clamp, const 
                "SH_to_RGB_backward: degree %d unsupported or > features %d", degree, F);
   FSGS_REQUIRE(!grad_campos || campos, "SH_to_RGB_backward: grad_campos without campos");
   if (P == 0) return kOk;
-  hipLaunchKernelGGL(sh_to_rgb_backward_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, F, degree,
+  auto kernel = degree > 3 ? sh_to_rgb_backward_kernel<64> : sh_to_rgb_backward_kernel<16>;
+  hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, F, degree,
                      clamp, pos, campos, sh, rgb, grad_rgb, grad_dir, grad_campos, grad_sh);
   return check_launch("SH_to_RGB_backward");
 }
@@ -419,7 +425,8 @@ FSGS_API int fsgs_sh_encode_forward(int B, int D, int C, const float* in, float*
   FSGS_REQUIRE(B >= 0 && D >= 3 && in && out, "sh_encode_forward: bad arguments");
   FSGS_REQUIRE(0 <= C && C <= kMaxShDegree, "sh_encode_forward: degree %d not supported (max %d)", C, kMaxShDegree);
   if (B == 0) return kOk;
-  hipLaunchKernelGGL(sh_encode_forward_kernel, dim3(div_up(B, 256)), dim3(256), 0, (hipStream_t) stream, B, D, C, in,
+  auto kernel = C > 3 ? sh_encode_forward_kernel<64> : sh_encode_forward_kernel<16>;
+  hipLaunchKernelGGL(kernel, dim3(div_up(B, 256)), dim3(256), 0, (hipStream_t) stream, B, D, C, in,
                      out);
   return check_launch("sh_encode_forward");
 }
@@ -429,7 +436,8 @@ FSGS_API int fsgs_sh_encode_backward(int B, int D, int C, const float* grad, con
   FSGS_REQUIRE(B >= 0 && D >= 3 && grad && in && grad_in, "sh_encode_backward: bad arguments");
   FSGS_REQUIRE(0 <= C && C <= kMaxShDegree, "sh_encode_backward: degree %d not supported (max %d)", C, kMaxShDegree);
   if (B == 0) return kOk;
-  hipLaunchKernelGGL(sh_encode_backward_kernel, dim3(div_up(B, 256)), dim3(256), 0, (hipStream_t) stream, B, D, C,
+  auto kernel = C > 3 ? sh_encode_backward_kernel<64> : sh_encode_backward_kernel<16>;
+  hipLaunchKernelGGL(kernel, dim3(div_up(B, 256)), dim3(256), 0, (hipStream_t) stream, B, D, C,
                      grad, in, grad_in);
   return check_launch("sh_encode_backward");
 }

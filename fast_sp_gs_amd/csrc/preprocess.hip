@@ -94,6 +94,7 @@ __device__ __forceinline__ bool bound_3sigma(const float* M, float* c, float* ex
   return true;
 }
 
+template <int kSh>
 __global__ void __launch_bounds__(256) preprocess_forward_kernel(
     int P, int W, int H, int sh_degree, int n_sh, const float* __restrict__ means3D, const float2* __restrict__ scales,
     const float4* __restrict__ rotations, const float* __restrict__ opacities, const float* __restrict__ shs,
@@ -146,7 +147,7 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
   } while (false);
 
   if (ok && sh_degree >= 0) {
-    float x, y, z, Y[16];
+    float x, y, z, Y[kSh];
     view_dir(p, campos, x, y, z);
     sh_eval(sh_degree, x, y, z, Y);
     const int n = sh_count(sh_degree);
@@ -235,6 +236,7 @@ __device__ __forceinline__ void transmat_backward(int W, int H, float sx, float 
   gq[3] = 2 * (x * (dR[9] - dR[6]) + y * (dR[2] - dR[8]) + z * (dR[4] - dR[1]));
 }
 
+template <int kSh>
 __global__ void __launch_bounds__(256) preprocess_backward_kernel(
     int P, int W, int H, int sh_degree, int n_sh, const float* __restrict__ means3D, const float2* __restrict__ scales,
     const float4* __restrict__ rotations, const float* __restrict__ shs, const float* __restrict__ sh_rest,
@@ -277,7 +279,7 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
   transmat_backward(W, H, s.x, s.y, q, Tw2c, Tw2v, gM, gN, gp, gs, gq);
 
   if (sh_degree >= 0) {
-    float x, y, z, Y[16], tl[16];
+    float x, y, z, Y[kSh], tl[kSh];
     const float nn = view_dir(p, campos, x, y, z);
     sh_eval(sh_degree, x, y, z, Y);
     float g[3];
@@ -370,8 +372,8 @@ FSGS_API int fsgs_gs_2d_preprocess_forward(int P, int W, int H, int sh_degree, i
                    (colors || sh_degree < 0),
                "gs_2d_preprocess_forward: null pointer");
   if (P == 0) return kOk;
-  hipLaunchKernelGGL(preprocess_forward_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H,
-                     sh_degree, n_sh, means3D, (const float2*) scales, (const float4*) rotations, opacities, shs,
+  auto kernel = sh_degree > 3 ? preprocess_forward_kernel<64> : preprocess_forward_kernel<16>;
+  hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh, means3D, (const float2*) scales, (const float4*) rotations, opacities, shs,
                      sh_rest, Tw2v, Tv2c, campos, trans_precomp, culling, means2D_preserve, (float2*) means2D, colors,
                      trans_mat, (float4*) normal_opacity, depths, radii, tiles_touched);
   return check_launch("gs_2d_preprocess_forward");
@@ -391,8 +393,8 @@ FSGS_API int fsgs_gs_2d_preprocess_backward(int P, int W, int H, int sh_degree, 
   if (sh_degree >= 0)
     FSGS_REQUIRE(shs && colors && grad_colors, "gs_2d_preprocess_backward: SH path needs shs, colors and grad_colors");
   if (P == 0) return kOk;
-  hipLaunchKernelGGL(preprocess_backward_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H,
-                     sh_degree, n_sh, means3D, (const float2*) scales, (const float4*) rotations, shs, sh_rest, Tw2v,
+  auto kernel = sh_degree > 3 ? preprocess_backward_kernel<64> : preprocess_backward_kernel<16>;
+  hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh, means3D, (const float2*) scales, (const float4*) rotations, shs, sh_rest, Tw2v,
                      Tv2c, campos, trans_mat, radii, colors, (float2*) grad_mean2D, grad_trans, grad_colors,
                      (const float4*) grad_normal_opacity, g_means3D, (float2*) g_scales, (float4*) g_rot, g_opac,
                      g_shs, g_sh_rest);

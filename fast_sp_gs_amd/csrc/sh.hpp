@@ -1,18 +1,23 @@
-// Device-side real spherical harmonics (degree 0..3) in the reference's convention
-// (fast_2d_gs/_C/include/spherical_harmonic.h:40-79): l=1 is (-y, +z, -x), colours get +0.5 and a clamp at 0.
+// Device-side real spherical harmonics (degree 0..7) in the reference's convention
+// (fast_2d_gs/_C/include/spherical_harmonic.h:40-193): l=1 is (-y, +z, -x), colours get +0.5 and a clamp at 0.
 // Values and Cartesian gradients are produced into register arrays so callers can fuse them with coefficient
-// loads of any layout.
+// loads of any layout. Degree <= 3 is written out here; degree 4..7 comes from sh_generated.hpp (derived from the
+// closed form by gen_sh_tables.py). Kernels are instantiated for 16 coefficients (degree <= 3, the common case, small
+// register footprint) and for 64.
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include "sh_generated.hpp"
+
 namespace fsgs {
 
-constexpr int kMaxShDegree = 3;
+constexpr int kMaxShDegree = 7;
 
 __device__ __forceinline__ int sh_count(int degree) { return (degree + 1) * (degree + 1); }
 
-// Y must hold 16 floats; entries beyond (degree+1)^2 are left untouched.
-__device__ __forceinline__ void sh_eval(int degree, float x, float y, float z, float* __restrict__ Y) {
+// Entries beyond (degree+1)^2 are left untouched. kN = 16 serves degree <= 3, kN = 64 degree <= 7.
+template <int kN>
+__device__ __forceinline__ void sh_eval(int degree, float x, float y, float z, float (&Y)[kN]) {
   Y[0] = 0.28209479177387814f;
   if (degree < 1) return;
   Y[1] = -0.48860251190291987f * y;
@@ -33,11 +38,13 @@ __device__ __forceinline__ void sh_eval(int degree, float x, float y, float z, f
   Y[13] = 0.45704579946446572f * x * (1.0f - 5.0f * zz);
   Y[14] = 1.4453057213202769f * z * (xx - yy);
   Y[15] = 0.59004358992664352f * x * (-xx + 3.0f * yy);
+  if constexpr (kN > 16) sh_eval_high(degree, x, y, z, Y);
 }
 
 // Accumulates t_l * grad(Y_l) for l >= 1 into (dx, dy, dz); t[l] is the caller's per-basis scalar
 // (dot(grad_rgb, coeff_l) for SH->RGB, the upstream gradient for the bare encoder).
-__device__ __forceinline__ void sh_grad_accumulate(int degree, float x, float y, float z, const float* __restrict__ t,
+template <int kN>
+__device__ __forceinline__ void sh_grad_accumulate(int degree, float x, float y, float z, const float (&t)[kN],
                                                    float& dx, float& dy, float& dz) {
   if (degree < 1) return;
   dy += t[1] * -0.48860251190291992f;
@@ -70,6 +77,7 @@ __device__ __forceinline__ void sh_grad_accumulate(int degree, float x, float y,
   dz += t[14] * (1.4453057213202769f * xx - 1.4453057213202769f * yy);
   dx += t[15] * (-1.7701307697799304f * xx + 1.7701307697799304f * yy);
   dy += t[15] * (3.5402615395598609f * xy);
+  if constexpr (kN > 16) sh_grad_accumulate_high(degree, x, y, z, t, dx, dy, dz);
 }
 
 // Unit view direction from the camera to p: (p - cam) * rsqrt(|p - cam|^2 + 1e-12) (spherical_harmonic.h:27-35).

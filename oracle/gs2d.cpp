@@ -181,7 +181,7 @@ static inline void sh_to_rgb(int degree, const T* pos, const T* campos, const T*
     const T n = T(1) / std::sqrt(x * x + y * y + z * z + T(1e-12));
     x = x * n, y = y * n, z = z * n;
   }
-  T Y[16];
+  T Y[kMaxShCoeffs];
   sh_basis(degree, x, y, z, Y);
   const int n = (degree + 1) * (degree + 1);
   for (int c = 0; c < 3; ++c) {
@@ -208,7 +208,7 @@ static inline void sh_to_rgb_backward(int degree, const T* pos, const T* campos,
   if (clamp)
     for (int c = 0; c < 3; ++c) g[c] *= T(rgb[c] > 0);
   const int cnt = (degree + 1) * (degree + 1);
-  T Y[16], dY[48];
+  T Y[kMaxShCoeffs], dY[3 * kMaxShCoeffs];
   sh_basis(degree, x, y, z, Y);
   if (g_sh) {
     for (int c = 0; c < 3; ++c) g_sh[c] = g[c] * Y[0];

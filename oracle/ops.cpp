@@ -34,7 +34,7 @@ static void sh_to_rgb_fwd(int P, int F, int degree, int clamp, const T* pos, con
       const T nn = T(1) / std::sqrt(x * x + y * y + z * z + T(1e-12));
       x = x * nn, y = y * nn, z = z * nn;
     }
-    T Y[16];
+    T Y[kMaxShCoeffs];
     sh_basis(degree, x, y, z, Y);
     const T* c = sh + (size_t) i * F * 3;
     for (int ch = 0; ch < 3; ++ch) {
@@ -61,7 +61,7 @@ static void sh_to_rgb_bwd(int P, int F, int degree, int clamp, const T* pos, con
     T g[3] = {grad_rgb[3 * i], grad_rgb[3 * i + 1], grad_rgb[3 * i + 2]};
     if (clamp)
       for (int ch = 0; ch < 3; ++ch) g[ch] *= T(rgb[3 * i + ch] > 0);
-    T Y[16], dY[48];
+    T Y[kMaxShCoeffs], dY[3 * kMaxShCoeffs];
     sh_basis(degree, x, y, z, Y);
     if (grad_sh) {
       T* gs = grad_sh + (size_t) i * F * 3;
@@ -100,7 +100,7 @@ static void sh_encode_bwd(int B, int D, int C, const T* grad, const T* in, T* gr
   const int n = (C + 1) * (C + 1);
 #pragma omp parallel for schedule(static)
   for (int b = 0; b < B; ++b) {
-    T dY[48];
+    T dY[3 * kMaxShCoeffs];
     sh_basis_grad(C, in[(size_t) b * D], in[(size_t) b * D + 1], in[(size_t) b * D + 2], dY);
     T dx = 0, dy = 0, dz = 0;
     for (int l = 0; l < n; ++l) {

@@ -1,6 +1,6 @@
 // TEST INFRASTRUCTURE ONLY (parity oracle). Never linked, imported or called by the product library.
 //
-// Real spherical-harmonic basis, degree <= 3, in the sign/ordering convention of the reference
+// Real spherical-harmonic basis, degree <= 7 (degree <= 3 written out here, 4..7 generated), in the sign/ordering convention of the reference
 // (fast_2d_gs/_C/include/spherical_harmonic.h:40-79 for the basis, :387-460 for the derivative
 // polynomials; fast_2d_gs/_C/src/nerf/shencoder.cu:36-73 for the encoder form of the same basis).
 //
@@ -11,10 +11,12 @@
 // Pinned by tests/test_oracle_sh.py: orthonormality under sphere quadrature, degree-0 closed form,
 // the l=1 sign convention (-y, +z, -x), and central finite differences of Y for dY.
 #pragma once
+#include "sh_basis_generated.h"  // degree 4..7, generated from the closed form by gen_sh.py
 
 namespace oracle {
 
-constexpr int kMaxShDegree = 3;
+constexpr int kMaxShDegree = 7;
+constexpr int kMaxShCoeffs = 64;
 
 template <typename T>
 inline void sh_basis(int degree, T x, T y, T z, T* Y) {
@@ -38,6 +40,7 @@ inline void sh_basis(int degree, T x, T y, T z, T* Y) {
   Y[13] = T(0.45704579946446572) * x * (T(1.0) - T(5.0) * z2);
   Y[14] = T(1.4453057213202769) * z * (x2 - y2);
   Y[15] = T(0.59004358992664352) * x * (-x2 + T(3.0) * y2);
+  sh_basis_high(degree, x, y, z, Y);
 }
 
 // dY[l*3 + a] = d Y_l / d (x,y,z)_a, treating x,y,z as independent variables.
@@ -76,6 +79,7 @@ inline void sh_basis_grad(int degree, T x, T y, T z, T* dY) {
   dY[14 * 3 + 2] = T(1.4453057213202769) * x2 - T(1.4453057213202769) * y2;
   dY[15 * 3 + 0] = T(-1.7701307697799304) * x2 + T(1.7701307697799304) * y2;
   dY[15 * 3 + 1] = T(3.5402615395598609) * xy;
+  sh_basis_grad_high(degree, x, y, z, dY);
 }
 
 }  // namespace oracle

@@ -39,7 +39,8 @@ def test_sh_to_rgb_and_encoder(device, oracle_mod, c1):
         assert rel_err(npy(s.grad), gs) < 1e-5 and rel_err(npy(d.grad), gd) < 1e-4
         if cam is not None:
             assert rel_err(npy(c.grad), gc) < 1e-3
-    for degree in (0, 1, 2, 3):
+    grad_enc = torch.randn(P, 64, generator=g)
+    for degree in range(8):
         d = dirs.to(device).requires_grad_()
         enc = sh_encode(d, degree)
         n = (degree + 1) ** 2
@@ -47,7 +48,16 @@ def test_sh_to_rgb_and_encoder(device, oracle_mod, c1):
         ref, gref = np.zeros((P, n), np.float32), np.zeros((P, 3), np.float32)
         O.call("sh_encode_forward_f32", P, 3, degree, npy(dirs), ref)
         O.call("sh_encode_backward_f32", P, 3, degree, npy(grad_enc[:, :n].contiguous()), npy(dirs), gref)
-        assert abs_err(npy(enc), ref) < 1e-6 and abs_err(npy(d.grad), gref) < 1e-4
+        assert abs_err(npy(enc), ref) < 2e-6 * max(1, degree) and rel_err(npy(d.grad), gref) < 1e-5
+    # a degree above 3 through SH -> RGB (36 coefficients + one unused row)
+    hi = torch.randn(2000, 37, 3, generator=g) * 0.2
+    d, s = dirs[:2000].to(device).requires_grad_(), hi.to(device).requires_grad_()
+    rgb = SH_to_RGB(s, d, None, 5, True)
+    rgb.backward(grad_rgb[:2000].to(device))
+    ref, gd, gs = np.zeros((2000, 3), np.float32), np.zeros((2000, 3), np.float32), np.zeros((2000, 37, 3), np.float32)
+    O.call("sh_to_rgb_forward_f32", 2000, 37, 5, 1, npy(dirs[:2000]), None, npy(hi), ref)
+    O.call("sh_to_rgb_backward_f32", 2000, 37, 5, 1, npy(dirs[:2000]), None, npy(hi), ref, npy(grad_rgb[:2000]), gd, None, gs)
+    assert abs_err(npy(rgb), ref) < 5e-6 and rel_err(npy(s.grad), gs) < 1e-5 and rel_err(npy(d.grad), gd) < 1e-4
 
 
 def test_freq_encoder(device, oracle_mod):
