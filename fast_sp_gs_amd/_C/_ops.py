@@ -19,7 +19,7 @@ __all__ = [
     'gs_2d_compute_trans_mat_backward', 'GS_prepare', 'GS_2D_render_forward', 'GS_2D_render_backward',
     'SH_to_RGB_forward', 'SH_to_RGB_backward', 'sh_encode_forward', 'sh_encode_backward', 'freq_encode_forward',
     'freq_encode_backward', 'cdist_top', 'cdist_top_backward', 'AdamMasksedUpdated', 'knn_topk', 'lbs_blend',
-    'gs_2d_topk_weights',
+    'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward',
 ]
 
 _TILE = 16
@@ -515,3 +515,52 @@ def lbs_blend(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_
                                 L.ptr(d_xyz), L.ptr(d_rot), L.ptr(d_scale), L.ptr(ws), ws.numel(), L.current_stream())
     L.check(rc, what)
     return d_xyz, d_rot, d_scale, weights
+
+
+# --------------------------------------------------------------------------------------------------------------------
+def mlp_pack_weights(weights: List[Tensor], head_weights: Tensor, skip: int) -> Tensor:
+    """bf16 weight buffer of the fused deformation MLP: layer i as [256][round_up(K_i, 16)], then the stacked heads as
+    [32][256]. `weights` are torch.nn.Linear weights [256, K_i] in layer order (network.py:1723-1727)."""
+    what = 'mlp_pack_weights'
+    _f32(what, head_weights=head_weights, **{f'w{i}': w for i, w in enumerate(weights)})
+    Din, n_layers = weights[0].shape[1], len(weights)
+    lib = _lib()
+    total = lib.fsgs_mlp_packed_elems(Din, n_layers, skip)
+    packed = torch.empty((total,), dtype=torch.int16, device=weights[0].device)
+    off = 0
+    stream = L.current_stream()
+    for i, w in enumerate(weights):
+        K = w.shape[1]
+        K_pad = (K + 15) // 16 * 16
+        expect = Din if i == 0 else (Din + 256 if i == skip + 1 else 256)
+        if w.shape[0] != 256 or K != expect:
+            raise RuntimeError(f'{what}: layer {i} weight has shape {tuple(w.shape)}, expected (256, {expect})')
+        rc = lib.fsgs_pack_bf16(256, K, 256, K_pad, L.ptr(w), packed.data_ptr() + 2 * off, stream)
+        L.check(rc, what)
+        off += 256 * K_pad
+    n_out, Kh = head_weights.shape
+    if n_out > 32 or Kh != 256:
+        raise RuntimeError(f'{what}: stacked heads must be [<=32, 256], got {tuple(head_weights.shape)}')
+    rc = lib.fsgs_pack_bf16(n_out, Kh, 32, 256, L.ptr(head_weights), packed.data_ptr() + 2 * off, stream)
+    L.check(rc, what)
+    return packed
+
+
+def mlp_forward(inputs: Tensor, packed: Tensor, bias: Tensor, n_layers: int, skip: int, n_out: int) -> Tensor:
+    """Fused n_layers x (Linear(256)+ReLU) + heads forward on the matrix cores (bf16 in, fp32 accumulate);
+    network.py:1757-1776. inputs[B,Din] fp32, bias[n_layers*256 + n_out] fp32 -> out[B,n_out] fp32."""
+    what = 'mlp_forward'
+    _f32(what, inputs=inputs, bias=bias)
+    L.require_cuda(what, packed=packed)
+    B, Din = inputs.shape
+    if bias.numel() != n_layers * 256 + n_out:
+        raise RuntimeError(f'{what}: bias must have {n_layers * 256 + n_out} elements')
+    if packed.numel() != _lib().fsgs_mlp_packed_elems(Din, n_layers, skip):
+        raise RuntimeError(f'{what}: packed weight buffer has the wrong size')
+    out = torch.empty((B, n_out), dtype=torch.float32, device=inputs.device)
+    with _timed('mlp_forward'):
+        rc = _lib().fsgs_mlp_forward(B, Din, 256, n_layers, skip, n_out, L.ptr(inputs),
+                                     L.ptr(packed), L.ptr(bias),
+                                     L.ptr(out), L.current_stream())
+    L.check(rc, what)
+    return out

@@ -145,6 +145,17 @@ int fsgs_lbs_blend(int N, int M, int K, int centred, double temperature, const f
     const int64_t* index, float* weights_out, float* d_xyz, float* d_rot, float* d_scale, void* workspace,
     size_t workspace_bytes, void* stream);
 
+/* Deformation MLP forward (bf16 MFMA, fp32 accumulate) -- fast_2d_gs/network.py:1757-1776 (SC_GS_DeformNetwork.forward,
+ * fp32 there): n_layers x (Linear(256) + ReLU), input re-concatenated in front after layer `skip`, then n_out <= 32
+ * linear outputs (the three heads stacked). in[B,Din] fp32 (already frequency-encoded), Din <= 96, width must be 256.
+ * packed: bf16 weights from fsgs_pack_bf16, layer i as [256][round_up(K_i,16)] row-major (K_0 = Din, K_{skip+1} =
+ * Din + 256, else 256), then the heads as [32][256]; fsgs_mlp_packed_elems gives the total element count.
+ * bias[n_layers*256 + n_out] fp32. out[B,n_out] fp32. */
+int fsgs_pack_bf16(int rows, int K, int rows_pad, int K_pad, const float* src, uint16_t* dst, void* stream);
+size_t fsgs_mlp_packed_elems(int Din, int n_layers, int skip);
+int fsgs_mlp_forward(int B, int Din, int width, int n_layers, int skip, int n_out, const float* in,
+                     const uint16_t* packed, const float* bias, float* out, void* stream);
+
 /* AdamMasksedUpdated -- fast_2d_gs/_C/src/other/adam_masked_update.cu:30-35 (kernel :9-28). Rows of the [N,M]
  * tensors whose mask byte is 0 are left untouched; eps is added to sqrt(v); lr carries the bias correction. */
 int fsgs_adam_masked_update(int64_t N, int64_t M, const uint8_t* mask, double lr, double b1, double b2, double eps,
