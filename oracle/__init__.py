@@ -155,3 +155,87 @@ def render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat_t2, ou
               dL_dflow, ranges, point_list, n_contrib, gc, gm, gt, gn)
     assert rc == 0
     return gc, gm, gt, gn
+
+
+# ---- "fast" path ---------------------------------------------------------------------------------------------------
+def fast_preprocess_forward(W, H, sh_degree, means3D, scales, rotations, opacities, shs, sh_rest, Tw2v, Tv2s, campos,
+                            trans_precomp=None, means2D=None, culling=None):
+    """-> (means2D, colors, trans_mat, inverse_m, normal_opacity, depths, radii, tiles_touched)."""
+    dt = means3D.dtype
+    P = means3D.shape[0]
+    has_rest = sh_rest is not None and sh_rest.size > 0
+    n_sh = sh_rest.shape[1] if has_rest else (shs.shape[1] if sh_degree >= 0 else 0)
+    preserve = means2D is not None
+    m2 = means2D if preserve else np.zeros((P, 2), dt)
+    colors = shs if sh_degree < 0 else np.zeros((P, 3), dt)
+    tm = trans_precomp if trans_precomp is not None else np.zeros((P, 3, 3), dt)
+    im, no, dep = np.zeros((P, 3, 3), dt), np.zeros((P, 4), dt), np.zeros((P,), dt)
+    radii, tt = np.zeros((P,), np.int32), np.zeros((P,), np.int32)
+    cul = None if culling is None else np.ascontiguousarray(culling.astype(np.uint8))
+    rc = call(f"gs_2d_fast_preprocess_forward_{_suffix(dt)}", P, W, H, sh_degree, n_sh, means3D, scales, rotations,
+              opacities, shs, sh_rest if has_rest else None, Tw2v, Tv2s, campos, trans_precomp, cul, int(preserve), m2,
+              None if sh_degree < 0 else colors, tm, im, no, dep, radii, tt)
+    assert rc == 0
+    return m2, colors, tm, im, no, dep, radii, tt
+
+
+def fast_prepare(W, H, means2D, inverse_m, depths, opacities, radii, tiles_touched, return_keys=False):
+    P = means2D.shape[0]
+    offsets = np.zeros((max(P, 1),), np.int64)
+    R = int(lib().oracle_gs_prepare_count(P, _p(np.ascontiguousarray(tiles_touched)), _p(offsets)))
+    T = ((W + 15) // 16) * ((H + 15) // 16)
+    ranges, pl = np.zeros((T, 2), np.int64), np.zeros((R,), np.int32)
+    keys = np.zeros((R,), np.int64) if return_keys else None
+    rc = call("gs_fast_prepare_fill", P, W, H, means2D, inverse_m, depths, np.ascontiguousarray(opacities), radii,
+              offsets, R, ranges, pl, keys)
+    assert rc == 0
+    return (ranges, pl, keys) if return_keys else (ranges, pl)
+
+
+def fast_preprocess_backward(W, H, sh_degree, means3D, scales, rotations, shs, sh_rest, Tw2v, Tv2s, campos, trans_mat,
+                             radii, colors, grad_mean2D, grad_trans, grad_inv_m, grad_colors, grad_normal_opacity):
+    dt = means3D.dtype
+    P = means3D.shape[0]
+    has_rest = sh_rest is not None and sh_rest.size > 0
+    n_sh = sh_rest.shape[1] if has_rest else (shs.shape[1] if sh_degree >= 0 else 0)
+    g3, gs, gr, go = np.zeros((P, 3), dt), np.zeros((P, 2), dt), np.zeros((P, 4), dt), np.zeros((P, 1), dt)
+    gsh = np.zeros_like(shs) if sh_degree >= 0 else None
+    gshr = np.zeros_like(sh_rest) if has_rest else None
+    gm2 = grad_mean2D.copy()
+    rc = call(f"gs_2d_fast_preprocess_backward_{_suffix(dt)}", P, W, H, sh_degree, n_sh, means3D, scales, rotations,
+              shs, sh_rest if has_rest else None, Tw2v, Tv2s, campos, trans_mat, radii, colors, gm2, grad_trans,
+              grad_inv_m, grad_colors, grad_normal_opacity, g3, gs, gr, go, gsh, gshr)
+    assert rc == 0
+    return g3, gs, gr, go, gsh, gshr, gm2
+
+
+def fast_render_forward(W, H, near, far, only_image, means2D, colors, normal_opacity, trans_mat, inverse_m, point_list,
+                        ranges, bucket_offset=None):
+    dt = means2D.dtype
+    oc, oo = np.zeros((3, H, W), dt), np.zeros((H, W), dt)
+    oe = None if only_image else np.zeros((8, H, W), dt)
+    nc = np.zeros((2, H, W), np.int32)
+    snap = [None] * 5
+    if bucket_offset is not None and not only_image:
+        B = int(bucket_offset[-1])
+        T = ranges.shape[0]
+        snap = [np.zeros((T,), np.int32), np.zeros((B,), np.int32), np.zeros((B, 256), dt), np.zeros((B, 3, 256), dt),
+                np.zeros((B, 8, 256), dt)]
+    rc = call(f"gs_2d_fast_render_forward_{_suffix(dt)}", W, H, float(near), float(far), int(only_image), means2D,
+              colors, normal_opacity, trans_mat, inverse_m, point_list, ranges, bucket_offset, oc, oo, oe, nc, *snap)
+    assert rc == 0
+    return (oc, oo, oe, nc) + tuple(snap)
+
+
+def fast_render_backward(near, far, per_splat_form, means2D, normal_opacity, colors, trans_mat, inverse_m, out_opacity,
+                         out_extras, dL_dpix, dL_dopacity, dL_dextras, ranges, point_list, n_contrib):
+    dt = means2D.dtype
+    P = means2D.shape[0]
+    H, W = dL_dpix.shape[1:]
+    gc, gm, gt, gi, gn = (np.zeros((P, 3), dt), np.zeros((P, 2), dt), np.zeros((P, 3, 3), dt), np.zeros((P, 3, 3), dt),
+                          np.zeros((P, 4), dt))
+    rc = call(f"gs_2d_fast_render_backward_{_suffix(dt)}", P, W, H, float(near), float(far), int(per_splat_form),
+              means2D, normal_opacity, colors, trans_mat, inverse_m, out_opacity, out_extras, dL_dpix, dL_dopacity,
+              dL_dextras, ranges, point_list, n_contrib, gc, gm, gt, gi, gn)
+    assert rc == 0
+    return gc, gm, gt, gi, gn

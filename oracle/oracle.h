@@ -55,3 +55,34 @@ int oracle_gs_prepare_fill(int P, int W, int H, const float* means2D, const floa
     const int64_t* offsets, int64_t R, int64_t* ranges, int32_t* point_list, int64_t* keys_sorted_out);
 uint32_t oracle_higher_msb(uint32_t n);
 int oracle_num_threads(void);
+int oracle_gs_2d_fast_compute_transmat_forward_f32(int P, const float* means3D, const float* scales,
+    const float* rotations, const float* Tw2v, const float* Tv2s, float* trans_mat, float* normals);
+int oracle_gs_2d_fast_compute_transmat_backward_f32(int P, const float* means3D, const float* scales,
+    const float* rotations, const float* Tw2v, const float* Tv2s, const float* g_mat, const float* g_normals,
+    float* g_means3D, float* g_scales, float* g_rot);
+int oracle_gs_2d_fast_preprocess_forward_f32(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
+    const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
+    const float* Tw2v, const float* Tv2s, const float* campos, const float* trans_precomp, const uint8_t* culling,
+    int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* inverse_m, float* normal_opacity,
+    float* depths, int32_t* radii, int32_t* tiles_touched);
+int oracle_gs_2d_fast_preprocess_backward_f32(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
+    const float* scales, const float* rotations, const float* shs, const float* sh_rest, const float* Tw2v,
+    const float* Tv2s, const float* campos, const float* trans_mat, const int32_t* radii, const float* colors,
+    float* grad_mean2D, const float* grad_trans, const float* grad_inv_m, const float* grad_colors,
+    const float* grad_normal_opacity, float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs,
+    float* g_sh_rest);
+int oracle_gs_2d_fast_render_forward_f32(int W, int H, double near_n, double far_n, int only_image,
+    const float* means2D, const float* colors, const float* normal_opacity, const float* trans_mat,
+    const float* inverse_m, const int32_t* point_list, const int64_t* ranges, const int64_t* bucket_offset,
+    float* out_color, float* out_opacity, float* out_extras, int32_t* n_contrib, int32_t* max_contrib,
+    int32_t* bucket_to_tile, float* sampled_T, float* sampled_acc, float* sampled_aux);
+int oracle_gs_2d_fast_render_backward_f32(int P, int W, int H, double near_n, double far_n, int per_splat_form,
+    const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,
+    const float* inverse_m, const float* out_opacity, const float* out_extras, const float* dL_dpix,
+    const float* dL_dopacity, const float* dL_dextras, const int64_t* ranges, const int32_t* point_list,
+    const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans, float* g_inv,
+    float* g_normal_opacity);
+int oracle_gs_fast_prepare_fill(int P, int W, int H, const float* means2D, const float* inverse_m,
+    const float* depths, const float* opacities, const int32_t* radii, const int64_t* offsets, int64_t R,
+    int64_t* ranges, int32_t* point_list, int64_t* keys_sorted_out);
+int oracle_fast_corner_test_f64(const double* inverse_m, double opacity, int x, int y);
