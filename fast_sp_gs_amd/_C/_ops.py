@@ -19,7 +19,9 @@ __all__ = [
     'gs_2d_compute_trans_mat_backward', 'GS_prepare', 'GS_2D_render_forward', 'GS_2D_render_backward',
     'SH_to_RGB_forward', 'SH_to_RGB_backward', 'sh_encode_forward', 'sh_encode_backward', 'freq_encode_forward',
     'freq_encode_backward', 'cdist_top', 'cdist_top_backward', 'AdamMasksedUpdated', 'knn_topk', 'lbs_blend',
-    'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward',
+    'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'gs_2d_fast_preprocess_forward',
+    'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward', 'gs_2d_fast_compute_trans_mat_backward',
+    'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward',
 ]
 
 _TILE = 16
@@ -325,6 +327,275 @@ def gs_2d_topk_weights(topk: int, W: int, H: int, near: float, far: float, means
                                             L.ptr(top_indices), L.ptr(top_weights), L.current_stream())
     L.check(rc, what)
     return top_indices, top_weights
+
+
+# ---- "fast" surfel path ---------------------------------------------------------------------------------------------
+def gs_2d_fast_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: bool, means3D: Tensor, scales: Tensor,
+                                  rotations: Tensor, opacities: Tensor, shs: Tensor, sh_rest: Optional[Tensor],
+                                  Tw2v: Tensor, Tv2c: Tensor, Tv2s: Tensor, cam_pos: Tensor,
+                                  trans_precomp: Optional[Tensor] = None, means2D: Optional[Tensor] = None,
+                                  culling: Optional[Tensor] = None, debug: bool = False,
+                                  return_keys: bool = False) -> List[Tensor]:
+    """gs_2d_fast_preprocess.cu:611-782 -> [means2D, colors, trans_mat, inverse_m, normal_opacity, depths, radii,
+    ranges[T,2] int64, point_list[R] int32] (point_list keeps the -1 padding entries of culled tiles at its tail)."""
+    what = 'gs_2d_fast_preprocess_forward'
+    _f32(what, means3D=means3D, scales=scales, rotations=rotations, opacities=opacities, shs=shs, Tw2v=Tw2v,
+         Tv2c=Tv2c, Tv2s=Tv2s, cam_pos=cam_pos)
+    if means3D.ndim != 2 or means3D.shape[-1] != 3:
+        raise RuntimeError('Error shape for means3D')
+    P = means3D.shape[0]
+    has_rest = sh_rest is not None and sh_rest.numel() > 0
+    M = 0
+    if has_rest:
+        _f32(what, sh_rest=sh_rest)
+        if not (sh_rest.ndim == 3 and sh_rest.shape[0] == P and sh_rest.shape[1] >= (1 + sh_degree) ** 2 - 1
+                and sh_rest.shape[2] == 3):
+            raise RuntimeError('Error shape for sh features')
+        M = sh_rest.shape[1]
+    elif sh_degree >= 0:
+        if not (shs.ndim == 3 and shs.shape[0] == P and shs.shape[1] >= (1 + sh_degree) ** 2 and shs.shape[2] == 3):
+            raise RuntimeError('Error shape for sh features')
+        M = shs.shape[1]
+    if means2D is not None:
+        _f32(what, means2D=means2D)
+        L.require_shape(what, 'means2D', means2D, P, 2)
+    if culling is not None:
+        L.require_cuda(what, culling=culling)
+        L.require_dtype(what, 'culling', culling, torch.bool)
+        L.require_shape(what, 'culling', culling, P)
+    if trans_precomp is not None:
+        _f32(what, trans_precomp=trans_precomp)
+    L.require_shape(what, 'scales', scales, P, 2)
+    L.require_shape(what, 'rotations', rotations, P, 4)
+    L.require_shape(what, 'opacities', opacities, P, 1)
+    L.require_shape(what, 'Tw2v', Tw2v, 4, 4)
+    L.require_shape(what, 'Tv2c', Tv2c, 4, 4)
+    L.require_shape(what, 'Tv2s', Tv2s, 3, 3)
+    L.require_shape(what, 'cam_pos', cam_pos, 3)
+    if sh_degree < 0:
+        L.require_shape(what, 'shs', shs, P, 3)
+
+    dev = means3D.device
+    opt = dict(dtype=torch.float32, device=dev)
+    lib = _lib()
+    stream = L.current_stream()
+    colors = shs if sh_degree < 0 else torch.empty((P, 3), **opt)
+    trans_mat = trans_precomp if trans_precomp is not None else torch.empty((P, 3, 3), **opt)
+    inverse_m = torch.empty((P, 3, 3), **opt)
+    preserve = means2D is not None
+    means2D_ = means2D if preserve else torch.empty((P, 2), **opt)
+    depths = torch.empty((P,), **opt)
+    radii = torch.empty((P,), dtype=torch.int32, device=dev)
+    tiles_touched = torch.empty((P,), dtype=torch.int32, device=dev)
+    normal_opacity = torch.empty((P, 4), **opt)
+    with _timed('gs_2d_fast_preprocess_forward'):
+        rc = lib.fsgs_gs_2d_fast_preprocess_forward(
+            P, W, H, sh_degree, M, L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(opacities), L.ptr(shs),
+            L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2s), L.ptr(cam_pos), L.ptr(trans_precomp),
+            L.ptr(culling), int(preserve), L.ptr(means2D_), None if sh_degree < 0 else L.ptr(colors),
+            None if trans_precomp is not None else L.ptr(trans_mat), L.ptr(inverse_m), L.ptr(normal_opacity),
+            L.ptr(depths), L.ptr(radii), L.ptr(tiles_touched), stream)
+    L.check(rc, what)
+
+    T = ((W + _TILE - 1) // _TILE) * ((H + _TILE - 1) // _TILE)
+    ranges = torch.empty((T, 2), dtype=torch.int64, device=dev)
+    offsets = torch.empty((max(P, 1),), dtype=torch.int64, device=dev)
+    ws1 = _workspace(lib.fsgs_gs_prepare_scan_workspace_bytes(P), dev)
+    R = ctypes.c_int64(0)
+    with _timed('gs_prepare_scan'):
+        rc = lib.fsgs_gs_prepare_scan(P, L.ptr(tiles_touched), L.ptr(offsets), L.ptr(ws1), ws1.numel(),
+                                      ctypes.addressof(R), stream)
+    L.check(rc, what)
+    R = int(R.value)
+    point_list = torch.empty((R,), dtype=torch.int32, device=dev)
+    keys = torch.empty((R,), dtype=torch.int64, device=dev) if return_keys else None
+    ws2 = _workspace(lib.fsgs_gs_prepare_fill_workspace_bytes(R), dev)
+    with _timed('gs_2d_fast_prepare_fill'):
+        rc = lib.fsgs_gs_2d_fast_prepare_fill(P, W, H, L.ptr(means2D_), L.ptr(inverse_m), L.ptr(depths),
+                                              L.ptr(opacities), L.ptr(radii), L.ptr(offsets), R, L.ptr(ranges),
+                                              L.ptr(point_list), L.ptr(keys), L.ptr(ws2), ws2.numel(), stream)
+    L.check(rc, what)
+    if debug:
+        torch.cuda.synchronize()
+    out = [means2D_, colors, trans_mat, inverse_m, normal_opacity, depths, radii, ranges, point_list]
+    return out + [keys, tiles_touched] if return_keys else out
+
+
+def gs_2d_fast_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs, sh_rest,
+                                   Tw2v, Tv2s, cam_pos, trans_mat, radii, colors, normal_opacity,
+                                   grad_mean2D, grad_trans, grad_inv_m, grad_depth, grad_colors, grad_normals,
+                                   grad_means3D, grad_scales, grad_rotations, grad_opacities, grad_shs, grad_sh_rest,
+                                   grad_Tw2v=None, grad_campos=None) -> None:
+    """gs_2d_fast_preprocess.cu:784-858: fills the caller's zeroed grad_* tensors in place and overwrites grad_mean2D."""
+    what = 'gs_2d_fast_preprocess_backward'
+    _f32(what, grad_mean2D=grad_mean2D, grad_colors=grad_colors, grad_normals=grad_normals,
+         grad_means3D=grad_means3D, grad_trans=grad_trans, grad_inv_m=grad_inv_m, grad_scales=grad_scales,
+         grad_rotations=grad_rotations, grad_opacities=grad_opacities, grad_shs=grad_shs, grad_sh_rest=grad_sh_rest)
+    if grad_shs is not None and colors is None:
+        raise RuntimeError('shs and clamped must not be None when need grad_shs')
+    has_rest = sh_rest is not None and sh_rest.numel() > 0
+    P = means3D.shape[0]
+    M = sh_rest.shape[1] if has_rest else (shs.shape[1] if shs.ndim == 3 else 0)
+    L.require_shape(what, 'grad_means3D', grad_means3D, P, 3)
+    if grad_scales is None or grad_rotations is None:
+        raise RuntimeError(f'{what}: grad_scales and grad_rotations are required')
+    L.require_shape(what, 'grad_scales', grad_scales, P, 2)
+    L.require_shape(what, 'grad_rotations', grad_rotations, P, 4)
+    L.require_shape(what, 'grad_opacities', grad_opacities, P, 1)
+    L.require_shape(what, 'grad_inv_m', grad_inv_m, P, 3, 3)
+    with _timed('gs_2d_fast_preprocess_backward'):
+        rc = _lib().fsgs_gs_2d_fast_preprocess_backward(
+            P, W, H, sh_degree, M, L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(shs),
+            L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2s), L.ptr(cam_pos), L.ptr(trans_mat),
+            L.ptr(radii), L.ptr(colors), L.ptr(grad_mean2D), L.ptr(grad_trans), L.ptr(grad_inv_m), L.ptr(grad_colors),
+            L.ptr(grad_normals), L.ptr(grad_means3D), L.ptr(grad_scales), L.ptr(grad_rotations),
+            L.ptr(grad_opacities), L.ptr(grad_shs), L.ptr(grad_sh_rest) if has_rest else None, L.current_stream())
+    L.check(rc, what)
+
+
+def gs_2d_fast_compute_transmat_forward(means3D, scales, rotations, Tw2v, Tv2s) -> Tuple[Tensor, Tensor]:
+    """gs_2d_fast_preprocess.cu:871-909 -> (trans_mat[P,3,3], normals[P,3])."""
+    what = 'gs_2d_fast_compute_transmat_forward'
+    _f32(what, means3D=means3D, scales=scales, rotations=rotations, Tw2v=Tw2v, Tv2s=Tv2s)
+    P = means3D.shape[0]
+    L.require_shape(what, 'means3D', means3D, P, 3)
+    L.require_shape(what, 'scales', scales, P, 2)
+    L.require_shape(what, 'rotations', rotations, P, 4)
+    L.require_shape(what, 'Tw2v', Tw2v, 4, 4)
+    L.require_shape(what, 'Tv2s', Tv2s, 3, 3)
+    trans_mat = torch.empty((P, 3, 3), dtype=torch.float32, device=means3D.device)
+    normals = torch.empty((P, 3), dtype=torch.float32, device=means3D.device)
+    with _timed(what):
+        rc = _lib().fsgs_gs_2d_fast_compute_transmat_forward(P, L.ptr(means3D), L.ptr(scales), L.ptr(rotations),
+                                                             L.ptr(Tw2v), L.ptr(Tv2s), L.ptr(trans_mat),
+                                                             L.ptr(normals), L.current_stream())
+    L.check(rc, what)
+    return trans_mat, normals
+
+
+def gs_2d_fast_compute_trans_mat_backward(means3D, scales, rotations, Tw2v, Tv2s, grad_matrix,
+                                          grad_normals) -> List[Tensor]:
+    """gs_2d_fast_preprocess.cu:923-960 -> [grad_means3D, grad_scales, grad_rotations]."""
+    what = 'gs_2d_fast_compute_trans_mat_backward'
+    _f32(what, means3D=means3D, scales=scales, rotations=rotations, Tw2v=Tw2v, Tv2s=Tv2s, grad_matrix=grad_matrix,
+         grad_normals=grad_normals)
+    P = means3D.shape[0]
+    L.require_shape(what, 'grad_matrix', grad_matrix, P, 3, 3)
+    L.require_shape(what, 'grad_normals', grad_normals, P, 3)
+    g_means3D = torch.empty((P, 3), dtype=torch.float32, device=means3D.device)
+    g_scales = torch.empty((P, 2), dtype=torch.float32, device=means3D.device)
+    g_rot = torch.empty((P, 4), dtype=torch.float32, device=means3D.device)
+    with _timed(what):
+        rc = _lib().fsgs_gs_2d_fast_compute_transmat_backward(P, L.ptr(means3D), L.ptr(scales), L.ptr(rotations),
+                                                              L.ptr(Tw2v), L.ptr(Tv2s), L.ptr(grad_matrix),
+                                                              L.ptr(grad_normals), L.ptr(g_means3D), L.ptr(g_scales),
+                                                              L.ptr(g_rot), L.current_stream())
+    L.check(rc, what)
+    return [g_means3D, g_scales, g_rot]
+
+
+def GS_2D_fast_render_forward(width: int, height: int, near_n: float, far_n: float, only_image: bool,
+                              means2D: Tensor, colors: Tensor, normal_opacity: Tensor, trans_mat: Tensor,
+                              inverse_m: Tensor, point_list: Tensor, ranges: Tensor,
+                              trans_mat_t2: Optional[Tensor] = None, accum_max_count: Optional[Tensor] = None,
+                              accum_weights_p: Optional[Tensor] = None, accum_weights_count: Optional[Tensor] = None,
+                              per_tile_bucket_offset: Optional[Tensor] = None):
+    """gs_2d_fast_redner.cu:839-953 -> [colors[3,H,W], opacity[H,W], extras[8,H,W]|None, flow (always None), n_contrib]
+    plus [max_contrib, bucket_to_tile, sampled_T, sampled_acc, sampled_aux] when per_tile_bucket_offset is given."""
+    what = 'GS_2D_fast_render_forward'
+    if trans_mat_t2 is not None:
+        raise RuntimeError(f'{what}: optical flow (trans_mat_t2) is not supported on the fast path')
+    _f32(what, colors=colors, trans_mat=trans_mat, inverse_m=inverse_m, means2D=means2D,
+         normal_opacity=normal_opacity, accum_weights_p=accum_weights_p)
+    if colors.ndim != 2:
+        raise RuntimeError(f'{what}: colors must have 2 dimensions')
+    P = colors.shape[0]
+    L.require_shape(what, 'trans_mat', trans_mat, P, 3, 3)
+    L.require_shape(what, 'inverse_m', inverse_m, P, 3, 3)
+    L.require_cuda(what, ranges=ranges, point_list=point_list, accum_max_count=accum_max_count,
+                   accum_weights_count=accum_weights_count, per_tile_bucket_offset=per_tile_bucket_offset)
+    L.require_dtype(what, 'ranges', ranges, torch.int64)
+    L.require_dtype(what, 'point_list', point_list, torch.int32)
+    for name, t, dt in (('accum_max_count', accum_max_count, torch.int32),
+                        ('accum_weights_count', accum_weights_count, torch.int32)):
+        if t is not None:
+            L.require_dtype(what, name, t, dt)
+            L.require_shape(what, name, t, P)
+    if accum_weights_p is not None:
+        L.require_shape(what, 'accum_weights_p', accum_weights_p, P)
+    dev = colors.device
+    opt = dict(dtype=torch.float32, device=dev)
+    pixel_colors = torch.zeros((3, height, width), **opt)
+    pixel_opacity = torch.zeros((height, width), **opt)
+    n_contrib = torch.zeros((2, height, width), dtype=torch.int32, device=dev)
+    pixel_extras = None if only_image else torch.zeros((8, height, width), **opt)
+    outputs = [pixel_colors, pixel_opacity, pixel_extras, None, n_contrib]
+    max_contrib = bucket_to_tile = sampled_T = sampled_acc = sampled_aux = None
+    fast_bwd = per_tile_bucket_offset is not None
+    if fast_bwd:
+        L.require_dtype(what, 'per_tile_bucket_offset', per_tile_bucket_offset, torch.int64)
+        per_tile_bucket_offset = per_tile_bucket_offset.contiguous()
+        B = int(per_tile_bucket_offset.reshape(-1)[-1].item())
+        gy, gx = (height + _TILE - 1) // _TILE, (width + _TILE - 1) // _TILE
+        max_contrib = torch.zeros((gy, gx), dtype=torch.int32, device=dev)
+        nb = max(B, 1)  # keep the base pointers valid when no tile has any entry
+        bucket_to_tile = torch.empty((nb,), dtype=torch.int32, device=dev)
+        sampled_T = torch.empty((nb, _TILE * _TILE), **opt)
+        sampled_acc = torch.empty((nb, 3, _TILE * _TILE), **opt)
+        sampled_aux = torch.empty((nb, 8, _TILE * _TILE), **opt)
+        outputs += [max_contrib, bucket_to_tile[:B], sampled_T[:B], sampled_acc[:B], sampled_aux[:B]]
+    if P == 0:
+        return outputs
+    with _timed('gs_2d_fast_render_forward'):
+        rc = _lib().fsgs_gs_2d_fast_render_forward(
+            P, width, height, float(near_n), float(far_n), int(bool(only_image)), L.ptr(means2D.contiguous()),
+            L.ptr(colors.contiguous()), L.ptr(normal_opacity.contiguous()), L.ptr(trans_mat), L.ptr(inverse_m),
+            L.ptr(point_list.contiguous()), L.ptr(ranges.contiguous()), L.ptr(accum_max_count),
+            L.ptr(accum_weights_p), L.ptr(accum_weights_count),
+            L.ptr(per_tile_bucket_offset) if (fast_bwd and not only_image) else None, L.ptr(pixel_colors),
+            L.ptr(pixel_opacity), L.ptr(pixel_extras), L.ptr(n_contrib), L.ptr(max_contrib), L.ptr(bucket_to_tile),
+            L.ptr(sampled_T), L.ptr(sampled_acc), L.ptr(sampled_aux), L.current_stream())
+    L.check(rc, what)
+    return outputs
+
+
+def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inverse_m, trans_mat2, images, out_opacity,
+                               out_others, out_flows, dL_dout_color, dL_dout_opacity, dL_dothers, dL_dout_flow,
+                               ranges, point_list, n_contrib, near_n: float, far_n: float,
+                               per_tile_bucket_offset=None, bucket_to_tile=None, max_contrib=None, sampled_T=None,
+                               sampled_acc=None, sampled_aux=None):
+    """gs_2d_fast_redner.cu:955-1074 -> [dL_dcolors[P,3], dL_dmeans2D[P,2], dL_dtrans_m[P,3,3], dL_dinverse_m[P,3,3],
+    dL_dnorm_op[P,4]]. Passing per_tile_bucket_offset selects the per-splat channel set of the reference's second
+    kernel; the snapshot tensors themselves are not needed to evaluate it here."""
+    what = 'GS_2D_fast_render_backward'
+    if dL_dout_flow is not None:
+        raise RuntimeError(f'{what}: optical flow gradients are not supported on the fast path')
+    L.require_cuda(what, dL_dout_color=dL_dout_color, dL_dout_opacity=dL_dout_opacity, dL_dothers=dL_dothers)
+    P = means2D.shape[0]
+    H, W = dL_dout_color.shape[1], dL_dout_color.shape[2]
+    opt = dict(dtype=torch.float32, device=out_opacity.device)
+    g_means2D = torch.zeros((P, 2), **opt)
+    g_norm_op = torch.zeros((P, 4), **opt)
+    g_colors = torch.zeros((P, 3), **opt)
+    g_trans = torch.zeros((P, 3, 3), **opt)
+    g_inv = torch.zeros((P, 3, 3), **opt)
+    if P == 0:
+        return [g_colors, g_means2D, g_trans, g_inv, g_norm_op]
+    c = lambda t: None if t is None else t.contiguous()
+    means2D, normal_opacity, colors, out_opacity = c(means2D), c(normal_opacity), c(colors), c(out_opacity)
+    dL_dout_color, dL_dout_opacity, dL_dothers = c(dL_dout_color), c(dL_dout_opacity), c(dL_dothers)
+    ranges, point_list, n_contrib, out_others = c(ranges), c(point_list), c(n_contrib), c(out_others)
+    use_aux = out_others is not None and dL_dothers is not None
+    per_splat = per_tile_bucket_offset is not None
+    with _timed('gs_2d_fast_render_backward'):
+        rc = _lib().fsgs_gs_2d_fast_render_backward(
+            P, W, H, float(near_n), float(far_n), int(per_splat), L.ptr(means2D), L.ptr(normal_opacity), L.ptr(colors),
+            L.ptr(trans_mat), L.ptr(inverse_m), L.ptr(out_opacity), L.ptr(out_others) if use_aux else None,
+            L.ptr(dL_dout_color), L.ptr(dL_dout_opacity), L.ptr(dL_dothers) if use_aux else None, L.ptr(ranges),
+            L.ptr(point_list), L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_inv),
+            L.ptr(g_norm_op), L.current_stream())
+    L.check(rc, what)
+    return [g_colors, g_means2D, g_trans, g_inv, g_norm_op]
 
 
 # --------------------------------------------------------------------------------------------------------------------

@@ -13,7 +13,7 @@
 //    with 64-bit ballot match masks (8 ballots per round, popcount of the mask below the lane), which is stable by
 //    construction: within a wave lower rounds and lower lanes come first, waves are ordered by an LDS prefix, blocks
 //    by the scanned histogram.
-#include "common.hpp"
+#include "binning.hpp"
 
 namespace fsgs {
 namespace {
@@ -288,6 +288,8 @@ __global__ void __launch_bounds__(256) tile_ranges_kernel(int64_t R, int num_til
   if (i == R - 1 && cur_ok) ranges[2 * (size_t) cur + 1] = R;
 }
 
+}  // namespace
+
 uint32_t higher_msb(uint32_t n) {  // number of bits needed for the tile id, as gaussian_prepare.cu:32-44 computes it
   uint32_t msb = sizeof(n) * 4, step = msb;
   while (step > 1) {
@@ -317,7 +319,50 @@ SortLayout sort_layout(int64_t R) {
   return L;
 }
 
-}  // namespace
+
+// Stable LSD radix sort of (key, value) pairs on key bits [0, bits). `vals_in` holds the unsorted payload (it is one of
+// the two ping-pong buffers); on return the sorted payload is in `vals_out` and *sorted_keys points at the sorted keys
+// (inside the workspace). The caller picks vals_in so that the last pass lands in vals_out: see sort_vals_in().
+int radix_sort_pairs(int64_t R, int bits, void* workspace, int32_t* vals_out, const uint64_t** sorted_keys,
+                     hipStream_t s) {
+  const SortLayout L = sort_layout(R);
+  char* ws          = (char*) workspace;
+  uint64_t* kbuf[2] = {(uint64_t*) (ws + L.keys0), (uint64_t*) (ws + L.keys1)};
+  uint32_t* hist    = (uint32_t*) (ws + L.hist);
+  uint32_t* totals  = (uint32_t*) (ws + L.totals);
+  const int passes  = (bits + kRadixBits - 1) / kRadixBits;
+  int32_t* vbuf[2];
+  vbuf[passes & 1]       = vals_out;
+  vbuf[(passes & 1) ^ 1] = (int32_t*) (ws + L.vals_alt);
+  for (int p = 0; p < passes; ++p) {
+    const int shift = p * kRadixBits;
+    const int a = p & 1, b = a ^ 1;
+    hipLaunchKernelGGL(sort_histogram_kernel, dim3(L.nblocks), dim3(kSortThreads), 0, s, R, shift, L.nblocks, kbuf[a],
+                       hist);
+    hipLaunchKernelGGL(sort_scan_rows_kernel, dim3(kRadix), dim3(kScanThreads), 0, s, L.nblocks, hist, totals);
+    hipLaunchKernelGGL(sort_scatter_kernel, dim3(L.nblocks), dim3(kSortThreads), 0, s, R, shift, L.nblocks, kbuf[a],
+                       vbuf[a], hist, totals, kbuf[b], vbuf[b]);
+  }
+  *sorted_keys = kbuf[passes & 1];
+  return passes;
+}
+
+// Where the unsorted keys / payload must be written before radix_sort_pairs(R, bits, workspace, vals_out, ...).
+uint64_t* sort_keys_in(int64_t R, void* workspace) { return (uint64_t*) ((char*) workspace + sort_layout(R).keys0); }
+int32_t* sort_vals_in(int64_t R, int bits, void* workspace, int32_t* vals_out) {
+  const int passes = (bits + kRadixBits - 1) / kRadixBits;
+  return (passes & 1) ? (int32_t*) ((char*) workspace + sort_layout(R).vals_alt) : vals_out;
+}
+size_t sort_workspace_bytes(int64_t R) { return sort_layout(R).bytes; }
+
+void launch_zero_ranges(int num_tiles, int64_t* ranges, hipStream_t s) {
+  hipLaunchKernelGGL(fill_zero_i64_kernel, dim3(div_up(2 * (int64_t) num_tiles, 256)), dim3(256), 0, s,
+                     2 * (int64_t) num_tiles, ranges);
+}
+void launch_tile_ranges(int64_t R, int num_tiles, const uint64_t* sorted_keys, int64_t* ranges, hipStream_t s) {
+  hipLaunchKernelGGL(tile_ranges_kernel, dim3(div_up(R, 256)), dim3(256), 0, s, R, num_tiles, sorted_keys, ranges);
+}
+
 }  // namespace fsgs
 
 using namespace fsgs;
@@ -371,33 +416,16 @@ FSGS_API int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, con
   if (R == 0 || P == 0) return check_launch("gs_prepare_fill(zero)");
   FSGS_REQUIRE(means2D && depths && radii && point_offsets && point_list && workspace,
                "gs_prepare_fill: null pointer");
-  const SortLayout L = sort_layout(R);
-  if (workspace_bytes < L.bytes)
-    return fail(kWorkspaceSmall, "gs_prepare_fill: workspace %zu < %zu bytes", workspace_bytes, L.bytes);
-  char* ws          = (char*) workspace;
-  uint64_t* kbuf[2] = {(uint64_t*) (ws + L.keys0), (uint64_t*) (ws + L.keys1)};
-  uint32_t* hist    = (uint32_t*) (ws + L.hist);
-  uint32_t* totals  = (uint32_t*) (ws + L.totals);
-  const int bits    = fsgs_gs_prepare_sort_bits(W, H);
-  const int passes  = (bits + kRadixBits - 1) / kRadixBits;
-  // ping-pong so that the last pass lands in point_list
-  int32_t* vbuf[2];
-  vbuf[passes & 1]       = point_list;
-  vbuf[(passes & 1) ^ 1] = (int32_t*) (ws + L.vals_alt);
-
+  if (workspace_bytes < sort_workspace_bytes(R))
+    return fail(kWorkspaceSmall, "gs_prepare_fill: workspace %zu < %zu bytes", workspace_bytes,
+                sort_workspace_bytes(R));
+  const int bits = fsgs_gs_prepare_sort_bits(W, H);
   hipLaunchKernelGGL(duplicate_keys_kernel, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
-                     (const float2*) means2D, depths, radii, point_offsets, kbuf[0], vbuf[0]);
-  for (int p = 0; p < passes; ++p) {
-    const int shift = p * kRadixBits;
-    const int a = p & 1, b = a ^ 1;
-    hipLaunchKernelGGL(sort_histogram_kernel, dim3(L.nblocks), dim3(kSortThreads), 0, s, R, shift, L.nblocks, kbuf[a],
-                       hist);
-    hipLaunchKernelGGL(sort_scan_rows_kernel, dim3(kRadix), dim3(kScanThreads), 0, s, L.nblocks, hist, totals);
-    hipLaunchKernelGGL(sort_scatter_kernel, dim3(L.nblocks), dim3(kSortThreads), 0, s, R, shift, L.nblocks, kbuf[a],
-                       vbuf[a], hist, totals, kbuf[b], vbuf[b]);
-  }
-  const uint64_t* sorted = kbuf[passes & 1];
-  hipLaunchKernelGGL(tile_ranges_kernel, dim3(div_up(R, 256)), dim3(256), 0, s, R, T, sorted, ranges);
+                     (const float2*) means2D, depths, radii, point_offsets, sort_keys_in(R, workspace),
+                     sort_vals_in(R, bits, workspace, point_list));
+  const uint64_t* sorted = nullptr;
+  radix_sort_pairs(R, bits, workspace, point_list, &sorted, s);
+  launch_tile_ranges(R, T, sorted, ranges, s);
   if (sorted_keys_out)
     FSGS_HIP(hipMemcpyAsync(sorted_keys_out, sorted, (size_t) R * 8, hipMemcpyDeviceToDevice, s));
   return check_launch("gs_prepare_fill");

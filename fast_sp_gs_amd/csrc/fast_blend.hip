@@ -1,0 +1,552 @@
+// Per-tile alpha blend of the "fast" 2D-Gaussian-surfel path for gfx950: the ray-splat intersection is three dot
+// products with the adjugate of the transform (p = adj(M) (x, y, 1), s = p.xy / p.z) instead of a cross product of two
+// planes, 8 auxiliary maps, optional snapshots of the running state every 32 list entries, and two backward channel
+// sets.
+//
+// Reference behaviour reproduced: fast_2d_gs/_C/src/gaussian_splatting/gs_2d_fast_redner.cu:22-271 (forward),
+// :273-561 (backward, per-pixel form), :563-837 (backward, per-splat form), :839-1074 (host entries).
+// The per-splat form of the reference re-walks 32-entry buckets from the forward snapshots with one warp per bucket;
+// its result is the same derivative with a different set of live channels (no distortion gradient, M1/M2 maps as
+// plain weighted sums with the M1 depth term overwritten, :751-757). Here both forms run the same tile-per-block
+// back-to-front kernel and differ only in that channel set; the snapshots are still produced by the forward for callers
+// that consume them. Optical flow is not supported on this path.
+//
+// Layout as in the standard blend: one 256-lane block per tile, wavefront w owns an 8x8 quadrant, surfels staged 256 at
+// a time in LDS (64-byte hot record with the adjugate, 32-byte cold record), per-quadrant work lists from a
+// conservative bound, gradients reduced over the wavefront in registers before one LDS atomic per component.
+#include "blend.hpp"
+
+namespace fsgs {
+namespace {
+
+struct __attribute__((aligned(16))) FastHot {
+  float a[9];           // adjugate of the ray-splat transform
+  float tw0, tw1, tw2;  // third row of the transform (depth along the ray)
+  float cx, cy, opacity, pad;
+};
+
+struct FastSplat {
+  FastHot hot;
+  SplatCold cold;
+  float m[6];  // first two rows of the transform, only used for the quadrant bound while staging
+};
+
+__device__ __forceinline__ FastSplat gather_fast(int id, const float2* __restrict__ means2D,
+                                                 const float* __restrict__ colors,
+                                                 const float4* __restrict__ normal_opacity,
+                                                 const float* __restrict__ trans_mat,
+                                                 const float* __restrict__ inverse_m) {
+  FastSplat s;
+  const float* A = inverse_m + 9 * (size_t) id;
+  const float* M = trans_mat + 9 * (size_t) id;
+#pragma unroll
+  for (int k = 0; k < 9; ++k) s.hot.a[k] = A[k];
+#pragma unroll
+  for (int k = 0; k < 6; ++k) s.m[k] = M[k];
+  s.hot.tw0 = M[6], s.hot.tw1 = M[7], s.hot.tw2 = M[8];
+  const float2 c  = means2D[id];
+  const float4 no = normal_opacity[id];
+  s.hot.cx = c.x, s.hot.cy = c.y, s.hot.opacity = no.w, s.hot.pad = 0.0f;
+  s.cold.nx = no.x, s.cold.ny = no.y, s.cold.nz = no.z;
+  s.cold.r = colors[3 * (size_t) id], s.cold.g = colors[3 * (size_t) id + 1], s.cold.b = colors[3 * (size_t) id + 2];
+  s.cold.id = id, s.cold.pad = 0;
+  return s;
+}
+
+__device__ __forceinline__ unsigned fast_quadrant_mask(const FastSplat& s, int tile_px, int tile_py) {
+  SplatHot h;
+#pragma unroll
+  for (int k = 0; k < 6; ++k) h.m[k] = s.m[k];
+  h.m[6] = s.hot.tw0, h.m[7] = s.hot.tw1, h.m[8] = s.hot.tw2;
+  h.cx = s.hot.cx, h.cy = s.hot.cy, h.opacity = s.hot.opacity;
+  return quadrant_mask(h, tile_px, tile_py);
+}
+
+struct FastHit {
+  float pz, sx, sy, dx, dy, rho3d, rho2d, depth, G, alpha;
+};
+
+// gs_2d_fast_redner.cu:150-186. Returns false when the reference would `continue`.
+__device__ __forceinline__ bool fast_intersect(const FastHot& h, float pxf, float pyf, float near_n, FastHit& o) {
+  const float p0 = h.a[0] * pxf + h.a[1] * pyf + h.a[2];
+  const float p1 = h.a[3] * pxf + h.a[4] * pyf + h.a[5];
+  o.pz           = h.a[6] * pxf + h.a[7] * pyf + h.a[8];
+  if (o.pz == 0.0f) return false;
+  const float rz = __builtin_amdgcn_rcpf(o.pz);
+  o.sx = p0 * rz, o.sy = p1 * rz;
+  o.rho3d = o.sx * o.sx + o.sy * o.sy;
+  o.dx = h.cx - pxf, o.dy = h.cy - pyf;
+  o.rho2d = 2.0f * (o.dx * o.dx + o.dy * o.dy);
+  const float rho = fminf(o.rho3d, o.rho2d);
+  o.depth = (o.sx * h.tw0 + o.sy * h.tw1) + h.tw2;
+  if (o.depth < near_n) return false;
+  const float power = -0.5f * rho;
+  if (power > 0.0f) return false;
+  o.G     = __expf(power);
+  o.alpha = fminf(0.99f, h.opacity * o.G);
+  return !(o.alpha < (1.0f / 255.0f));
+}
+
+// Sums 8 per-lane values over the 64 lanes at once: three merge steps inside aligned groups of 8 lanes, one rotate by 8
+// inside the row of 16, two cross-row exchanges. On return every lane holds the wave total of v[lane & 7].
+__device__ __forceinline__ float wave_sum8_transposed(const float (&v)[8]) {
+  const int lane = __lane_id();
+  const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
+  float w[4], x[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float a = v[2 * i + 1] + dpp_shift_zero<0x111, 0xf, 0xf>(v[2 * i + 1]);  // row_shr:1
+    const float b = v[2 * i] + dpp_shift_zero<0x101, 0xf, 0xf>(v[2 * i]);          // row_shl:1
+    w[i] = b0 ? a : b;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const float a = w[2 * i + 1] + dpp_shift_zero<0x112, 0xf, 0xf>(w[2 * i + 1]);  // row_shr:2
+    const float b = w[2 * i] + dpp_shift_zero<0x102, 0xf, 0xf>(w[2 * i]);          // row_shl:2
+    x[i] = b1 ? a : b;
+  }
+  const float a = x[1] + dpp_shift_zero<0x114, 0xf, 0xf>(x[1]);  // row_shr:4
+  const float b = x[0] + dpp_shift_zero<0x104, 0xf, 0xf>(x[0]);  // row_shl:4
+  float z = b2 ? a : b;
+  z += dpp_shift_zero<0x128, 0xf, 0xf>(z);  // row_ror:8
+  z += __shfl_xor(z, 16, kWave);
+  z += __shfl_xor(z, 32, kWave);
+  return z;
+}
+
+template <bool kAux, bool kSnap, bool kAccum>
+__global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
+    int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    const float2* __restrict__ means2D, const float* __restrict__ colors, const float* __restrict__ trans_mat,
+    const float* __restrict__ inverse_m, const float4* __restrict__ normal_opacity,
+    const int64_t* __restrict__ bucket_offset, int32_t* __restrict__ n_contrib, float* __restrict__ out_color,
+    float* __restrict__ out_opacity, float* __restrict__ out_extras, int32_t* __restrict__ max_contrib,
+    int32_t* __restrict__ bucket_to_tile, float* __restrict__ sampled_T, float* __restrict__ sampled_acc,
+    float* __restrict__ sampled_aux, int32_t* __restrict__ accum_max_count, float* __restrict__ accum_weights_p,
+    int32_t* __restrict__ accum_weights_count) {
+  __shared__ FastHot s_hot[kBatch];
+  __shared__ SplatCold s_cold[kBatch];
+  __shared__ unsigned char s_mask[kBatch];
+  __shared__ int s_max_contrib;
+
+  const int gx = (W + kTile - 1) / kTile;
+  const int tile = blockIdx.x, tile_x = tile % gx, tile_y = tile / gx;
+  int px, py;
+  lane_pixel(tile_x, tile_y, px, py);
+  const bool inside = px < W && py < H;
+  const size_t HW   = (size_t) H * W;
+  const size_t pix  = (size_t) W * py + px;
+  const float pxf = (float) px, pyf = (float) py;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rank = (py - tile_y * kTile) * kTile + (px - tile_x * kTile);  // row-major position inside the tile
+
+  const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
+  const int n_todo = (int) (r1 - r0);
+  const int rounds = (n_todo + kBatch - 1) / kBatch;
+
+  int64_t bucket0 = 0;
+  if (kSnap) {
+    bucket0 = tile == 0 ? 0 : bucket_offset[tile - 1];
+    const int nb = (n_todo + 31) / 32;
+    for (int k = threadIdx.x; k < nb; k += kBlendThreads) bucket_to_tile[bucket0 + k] = tile;
+    if (threadIdx.x == 0) s_max_contrib = 0;
+  }
+
+  bool done = !inside;
+  float T = 1.0f, C0 = 0, C1 = 0, C2 = 0;
+  float N0 = 0, N1 = 0, N2 = 0, D = 0, M1 = 0, M2 = 0, dist = 0, median = 0;
+  int last = 0, median_c = -1, wmax_id = -1;
+  float wmax = 0;
+  bool flag  = false;
+
+  FastSplat next;
+  if ((int) threadIdx.x < n_todo)
+    next = gather_fast(point_list[r0 + threadIdx.x], means2D, colors, normal_opacity, trans_mat, inverse_m);
+
+  for (int b = 0; b < rounds; ++b) {
+    if (__syncthreads_count(done) == kBlendThreads) break;
+    const int n_here = min(kBatch, n_todo - b * kBatch);
+    if ((int) threadIdx.x < n_here) {
+      s_hot[threadIdx.x]  = next.hot;
+      s_cold[threadIdx.x] = next.cold;
+      s_mask[threadIdx.x] = (unsigned char) fast_quadrant_mask(next, tile_x * kTile, tile_y * kTile);
+    }
+    __syncthreads();
+    const int nxt = (b + 1) * kBatch + (int) threadIdx.x;
+    if (nxt < n_todo)
+      next = gather_fast(point_list[r0 + nxt], means2D, colors, normal_opacity, trans_mat, inverse_m);
+
+    for (int c = 0; c < kBatch / kWave; ++c) {
+      const int jj = c * kWave + lane;
+      const unsigned long long todo_all = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u));
+      for (int half = 0; half < (kSnap ? 2 : 1); ++half) {
+        unsigned long long todo = todo_all;
+        if (kSnap) {
+          const int base = c * kWave + half * 32;
+          if (base >= n_here) break;
+          if (!done) {
+            // state before list entry b * 256 + base, which starts a bucket of 32 (gs_2d_fast_redner.cu:126-147)
+            const size_t bk = (size_t) (bucket0 + (b * kBatch + base) / 32);
+            sampled_T[bk * 256 + rank]             = T;
+            sampled_acc[(bk * 3 + 0) * 256 + rank] = C0;
+            sampled_acc[(bk * 3 + 1) * 256 + rank] = C1;
+            sampled_acc[(bk * 3 + 2) * 256 + rank] = C2;
+            if (kAux) {
+              sampled_aux[(bk * 8 + 0) * 256 + rank] = D;
+              sampled_aux[(bk * 8 + 1) * 256 + rank] = N0;
+              sampled_aux[(bk * 8 + 2) * 256 + rank] = N1;
+              sampled_aux[(bk * 8 + 3) * 256 + rank] = N2;
+              sampled_aux[(bk * 8 + 5) * 256 + rank] = dist;
+              sampled_aux[(bk * 8 + 6) * 256 + rank] = M1;
+              sampled_aux[(bk * 8 + 7) * 256 + rank] = M2;
+            }
+          }
+          todo &= half ? 0xffffffff00000000ull : 0x00000000ffffffffull;
+        }
+        while (todo) {
+          if (__ballot(!done) == 0ull) break;
+          const int j = c * kWave + __builtin_ctzll(todo);
+          todo &= todo - 1;
+          if (done) continue;
+          FastHit h;
+          if (!fast_intersect(s_hot[j], pxf, pyf, near_n, h)) continue;
+          const float test_T = T * (1.0f - h.alpha);
+          if (test_T < 0.0001f) {
+            done = true;
+            continue;
+          }
+          const float w         = h.alpha * T;
+          const SplatCold cold  = s_cold[j];
+          const int contributor = b * kBatch + j + 1;
+          if (kAux) {
+            const float A = 1.0f - T;
+            const float m = far_n / (far_n - near_n) * (1.0f - near_n / h.depth);
+            dist += (m * m * A + M2 - 2.0f * m * M1) * w;
+            D += h.depth * w;
+            M1 += m * w;
+            M2 += m * m * w;
+            if (T > 0.5f) median = h.depth, median_c = contributor;
+            N0 += cold.nx * w, N1 += cold.ny * w, N2 += cold.nz * w;
+            if (kAccum) {
+              if (wmax < w) wmax = w, wmax_id = cold.id, flag = true;
+              if (accum_weights_p) atomicAdd(&accum_weights_p[cold.id], w);
+              if (accum_weights_count) atomicAdd(&accum_weights_count[cold.id], 1);
+            }
+          }
+          if (kAccum) {
+            if (flag && accum_max_count) atomicAdd(&accum_max_count[wmax_id], 1);
+          }
+          C0 += cold.r * w, C1 += cold.g * w, C2 += cold.b * w;
+          T    = test_T;
+          last = contributor;
+        }
+      }
+    }
+  }
+
+  if (inside) {
+    out_opacity[pix]        = 1.0f - T;
+    n_contrib[pix]          = last;
+    n_contrib[pix + HW]     = kAux ? median_c : 0;
+    out_color[pix]          = C0;
+    out_color[pix + HW]     = C1;
+    out_color[pix + 2 * HW] = C2;
+    if (kAux) {
+      out_extras[pix + 0 * HW] = D;
+      out_extras[pix + 1 * HW] = N0;
+      out_extras[pix + 2 * HW] = N1;
+      out_extras[pix + 3 * HW] = N2;
+      out_extras[pix + 4 * HW] = median;
+      out_extras[pix + 5 * HW] = dist;
+      out_extras[pix + 6 * HW] = M1;
+      out_extras[pix + 7 * HW] = M2;
+    }
+  }
+  if (kSnap) {
+    int wave_max = last;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) wave_max = max(wave_max, __shfl_xor(wave_max, d, kWave));
+    __syncthreads();  // s_max_contrib was cleared before the first barrier of the loop only if the loop ran
+    if (lane == 0) atomicMax(&s_max_contrib, wave_max);
+    __syncthreads();
+    if (threadIdx.x == 0) max_contrib[tile] = s_max_contrib;
+  }
+}
+
+// Per-surfel gradient slots: 0-2 colours | 3-11 adjugate | 12-14 normal | 15 opacity | 16-18 transform row 2 |
+// 19-20 means2D.
+constexpr int kFastGradSlots = 21;
+
+template <bool kAux, bool kPerSplat>
+__global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
+    int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    const int32_t* __restrict__ n_contrib, const float2* __restrict__ means2D,
+    const float4* __restrict__ normal_opacity, const float* __restrict__ colors, const float* __restrict__ trans_mat,
+    const float* __restrict__ inverse_m, const float* __restrict__ out_opacity, const float* __restrict__ out_extras,
+    const float* __restrict__ dL_dpix, const float* __restrict__ dL_dextras, const float* __restrict__ dL_dopacity,
+    float* __restrict__ g_means2D, float* __restrict__ g_normal_opacity, float* __restrict__ g_colors,
+    float* __restrict__ g_trans, float* __restrict__ g_inv) {
+  __shared__ FastHot s_hot[kBatch];
+  __shared__ SplatCold s_cold[kBatch];
+  __shared__ float s_acc[kBatch][kFastGradSlots];
+  __shared__ int s_max_contrib;
+  __shared__ unsigned char s_mask[kBatch];
+
+  const int gx = (W + kTile - 1) / kTile;
+  const int tile = blockIdx.x, tile_x = tile % gx, tile_y = tile / gx;
+  int px, py;
+  lane_pixel(tile_x, tile_y, px, py);
+  const bool inside = px < W && py < H;
+  const size_t HW   = (size_t) H * W;
+  const size_t pix  = (size_t) W * py + px;
+  const float pxf = (float) px, pyf = (float) py;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+  const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
+  const int last_contrib   = inside ? n_contrib[pix] : 0;
+  const int median_contrib = (kAux && inside) ? n_contrib[pix + HW] : 0;
+
+  if (threadIdx.x == 0) s_max_contrib = 0;
+  __syncthreads();
+  int wave_max_contrib = last_contrib;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) wave_max_contrib = max(wave_max_contrib, __shfl_xor(wave_max_contrib, d, kWave));
+  if (lane == 0) atomicMax(&s_max_contrib, wave_max_contrib);
+#pragma unroll
+  for (int c = 0; c < kFastGradSlots; ++c) s_acc[threadIdx.x][c] = 0.0f;
+  __syncthreads();
+  const int n_todo = min(s_max_contrib, (int) (r1 - r0));
+  const int rounds = (n_todo + kBatch - 1) / kBatch;
+
+  const float T_final = inside ? 1.0f - out_opacity[pix] : 0.0f;
+  float T = T_final;
+  float dLp0 = 0, dLp1 = 0, dLp2 = 0;
+  float dL_dreg = 0, dL_ddepth = 0, dL_daccum = 0, dLn0 = 0, dLn1 = 0, dLn2 = 0, dL_dmedian = 0, dL_dM1 = 0, dL_dM2 = 0;
+  float final_D = 0, final_D2 = 0;
+  if (inside) {
+    dLp0 = dL_dpix[pix], dLp1 = dL_dpix[pix + HW], dLp2 = dL_dpix[pix + 2 * HW];
+    if (kAux) {
+      dL_daccum  = dL_dopacity[pix];
+      dL_ddepth  = dL_dextras[pix + 0 * HW];
+      dLn0       = dL_dextras[pix + 1 * HW];
+      dLn1       = dL_dextras[pix + 2 * HW];
+      dLn2       = dL_dextras[pix + 3 * HW];
+      dL_dmedian = dL_dextras[pix + 4 * HW];
+      if (kPerSplat) dL_dM1 = dL_dextras[pix + 6 * HW], dL_dM2 = dL_dextras[pix + 7 * HW];
+      else dL_dreg = dL_dextras[pix + 5 * HW];
+      final_D  = out_extras[pix + 6 * HW];
+      final_D2 = out_extras[pix + 7 * HW];
+    } else if (kPerSplat) {
+      dL_daccum = dL_dopacity[pix];
+    }
+  }
+  const float final_A   = 1.0f - T_final;
+  const float far_scale = far_n / (far_n - near_n);
+
+  float acc_c0 = 0, acc_c1 = 0, acc_c2 = 0, last_c0 = 0, last_c1 = 0, last_c2 = 0;
+  float last_depth = 0, acc_depth = 0, acc_alpha = 0;
+  float last_n0 = 0, last_n1 = 0, last_n2 = 0, acc_n0 = 0, acc_n1 = 0, acc_n2 = 0;
+  float last_m = 0, acc_m = 0, last_m2 = 0, acc_m2 = 0;
+  float last_dL_dT = 0, last_alpha = 0;
+
+  FastSplat next;
+  if ((int) threadIdx.x < n_todo)
+    next = gather_fast(point_list[r0 + (n_todo - 1 - (int) threadIdx.x)], means2D, colors, normal_opacity, trans_mat,
+                       inverse_m);
+
+  for (int b = 0; b < rounds; ++b) {
+    const int n_here = min(kBatch, n_todo - b * kBatch);
+    if ((int) threadIdx.x < n_here) {
+      s_hot[threadIdx.x]  = next.hot;
+      s_cold[threadIdx.x] = next.cold;
+      s_mask[threadIdx.x] = (unsigned char) fast_quadrant_mask(next, tile_x * kTile, tile_y * kTile);
+    }
+    __syncthreads();
+    const int nxt = (b + 1) * kBatch + (int) threadIdx.x;
+    if (nxt < n_todo)
+      next = gather_fast(point_list[r0 + (n_todo - 1 - nxt)], means2D, colors, normal_opacity, trans_mat, inverse_m);
+
+    for (int chunk = 0; chunk < kBatch / kWave; ++chunk) {
+      const int jj = chunk * kWave + lane;
+      unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u) &&
+                                         (n_todo - 1 - (b * kBatch + jj)) < wave_max_contrib);
+      while (todo) {
+        const int j = chunk * kWave + __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const int pos = n_todo - 1 - (b * kBatch + j);
+        FastHit h;
+        const bool hit = (pos < last_contrib) && fast_intersect(s_hot[j], pxf, pyf, near_n, h);
+        if (__ballot(hit) == 0ull) continue;
+
+        float g[16], g8[8];
+        bool filtered = false;
+#pragma unroll
+        for (int c = 0; c < 16; ++c) g[c] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) g8[c] = 0.0f;
+        if (hit) {
+          const FastHot& hot   = s_hot[j];
+          const SplatCold cold = s_cold[j];
+          T             = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+          const float w = h.alpha * T;
+          float dL_dalpha = 0.0f;
+          acc_c0 = last_alpha * last_c0 + (1.0f - last_alpha) * acc_c0, last_c0 = cold.r;
+          acc_c1 = last_alpha * last_c1 + (1.0f - last_alpha) * acc_c1, last_c1 = cold.g;
+          acc_c2 = last_alpha * last_c2 + (1.0f - last_alpha) * acc_c2, last_c2 = cold.b;
+          dL_dalpha += (cold.r - acc_c0) * dLp0 + (cold.g - acc_c1) * dLp1 + (cold.b - acc_c2) * dLp2;
+          g[0] = w * dLp0, g[1] = w * dLp1, g[2] = w * dLp2;
+
+          float dL_dz = 0.0f;
+          if (kAux) {
+            const float rd     = __builtin_amdgcn_rcpf(h.depth);
+            const float m_d    = far_scale * (1.0f - near_n * rd);
+            const float dmd_dd = far_scale * near_n * rd * rd;
+            if (pos == median_contrib - 1) dL_dz += dL_dmedian;
+            if (!kPerSplat) {
+              const float dL_dweight = (final_D2 + m_d * m_d * final_A - 2.0f * m_d * final_D) * dL_dreg;
+              dL_dalpha += dL_dweight - last_dL_dT;
+              last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
+              dL_dz += 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg * dmd_dd;
+            } else {
+              acc_m  = last_alpha * last_m + (1.0f - last_alpha) * acc_m, last_m = m_d;
+              acc_m2 = last_alpha * last_m2 + (1.0f - last_alpha) * acc_m2, last_m2 = m_d * m_d;
+              dL_dalpha += (m_d - acc_m) * dL_dM1 + (m_d * m_d - acc_m2) * dL_dM2;
+              dL_dz += dmd_dd * (2.0f * m_d * w * dL_dM2);
+            }
+            acc_depth  = last_alpha * last_depth + (1.0f - last_alpha) * acc_depth;
+            last_depth = h.depth;
+            dL_dalpha += (h.depth - acc_depth) * dL_ddepth;
+            acc_n0 = last_alpha * last_n0 + (1.0f - last_alpha) * acc_n0, last_n0 = cold.nx;
+            acc_n1 = last_alpha * last_n1 + (1.0f - last_alpha) * acc_n1, last_n1 = cold.ny;
+            acc_n2 = last_alpha * last_n2 + (1.0f - last_alpha) * acc_n2, last_n2 = cold.nz;
+            dL_dalpha += (cold.nx - acc_n0) * dLn0 + (cold.ny - acc_n1) * dLn1 + (cold.nz - acc_n2) * dLn2;
+            g[12] = w * dLn0, g[13] = w * dLn1, g[14] = w * dLn2;
+            dL_dz += w * dL_ddepth;
+          }
+          if (kAux || kPerSplat) {
+            acc_alpha = last_alpha * 1.0f + (1.0f - last_alpha) * acc_alpha;
+            dL_dalpha += (1.0f - acc_alpha) * dL_daccum;
+          }
+          dL_dalpha *= T;
+          last_alpha = h.alpha;
+
+          const float dL_dG = hot.opacity * dL_dalpha;
+          if (h.rho3d <= h.rho2d) {
+            const float dsx = dL_dG * -h.G * h.sx + dL_dz * hot.tw0;
+            const float dsy = dL_dG * -h.G * h.sy + dL_dz * hot.tw1;
+            const float rz  = __builtin_amdgcn_rcpf(h.pz);
+            const float da = dsx * rz, db = dsy * rz;
+            const float dc = -(da * h.sx + db * h.sy);
+            g[3] = da * pxf, g[4] = da * pyf, g[5] = da;
+            g[6] = db * pxf, g[7] = db * pyf, g[8] = db;
+            g[9] = dc * pxf, g[10] = dc * pyf, g[11] = dc;
+          } else {
+            g8[3]    = dL_dG * (-h.G * 2.0f * h.dx);
+            g8[4]    = dL_dG * (-h.G * 2.0f * h.dy);
+            filtered = true;
+          }
+          g8[0] = dL_dz * h.sx, g8[1] = dL_dz * h.sy, g8[2] = dL_dz;
+          g[15] = h.G * dL_dalpha;
+        }
+        const float tot = wave_sum16_transposed(g);
+        if (lane < 16) atomicAdd(&s_acc[j][lane], tot);
+        if (kAux) {
+          const float tot8 = wave_sum8_transposed(g8);
+          if (lane < 5) atomicAdd(&s_acc[j][16 + lane], tot8);
+        } else if (__ballot(filtered) != 0ull) {
+          const float sx = wave_sum_to_lane63(g8[3]), sy = wave_sum_to_lane63(g8[4]);
+          if (lane == 63) atomicAdd(&s_acc[j][19], sx), atomicAdd(&s_acc[j][20], sy);
+        }
+      }
+    }
+    __syncthreads();
+    if ((int) threadIdx.x < n_here) {
+      const int id = s_cold[threadIdx.x].id;
+      float* a     = s_acc[threadIdx.x];
+#pragma unroll
+      for (int c = 0; c < 3; ++c)
+        if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
+#pragma unroll
+      for (int c = 0; c < 9; ++c)
+        if (a[3 + c] != 0.0f) atomicAdd(&g_inv[9 * (size_t) id + c], a[3 + c]);
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (a[12 + c] != 0.0f) atomicAdd(&g_normal_opacity[4 * (size_t) id + c], a[12 + c]);
+#pragma unroll
+      for (int c = 0; c < 3; ++c)
+        if (a[16 + c] != 0.0f) atomicAdd(&g_trans[9 * (size_t) id + 6 + c], a[16 + c]);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+        if (a[19 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[19 + c]);
+#pragma unroll
+      for (int c = 0; c < kFastGradSlots; ++c) a[c] = 0.0f;
+    }
+  }
+}
+
+}  // namespace
+}  // namespace fsgs
+
+using namespace fsgs;
+
+FSGS_API int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, double far_n, int only_image,
+    const float* means2D, const float* colors, const float* normal_opacity, const float* trans_mat,
+    const float* inverse_m, const int32_t* point_list, const int64_t* ranges, int32_t* accum_max_count,
+    float* accum_weights_p, int32_t* accum_weights_count, const int64_t* bucket_offset, float* out_color,
+    float* out_opacity, float* out_extras, int32_t* n_contrib, int32_t* max_contrib, int32_t* bucket_to_tile,
+    float* sampled_T, float* sampled_acc, float* sampled_aux, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_fast_render_forward: bad sizes");
+  FSGS_REQUIRE(ranges && out_color && out_opacity && n_contrib, "GS_2D_fast_render_forward: null pointer");
+  FSGS_REQUIRE(P == 0 || (means2D && colors && normal_opacity && trans_mat && inverse_m),
+               "GS_2D_fast_render_forward: null surfel tensor");
+  FSGS_REQUIRE(only_image || out_extras, "GS_2D_fast_render_forward: out_extras is required unless only_image");
+  const bool aux   = !only_image;
+  const bool snap  = aux && bucket_offset != nullptr;
+  const bool accum = aux && (accum_max_count || accum_weights_p || accum_weights_count);
+  FSGS_REQUIRE(!snap || (max_contrib && bucket_to_tile && sampled_T && sampled_acc && sampled_aux),
+               "GS_2D_fast_render_forward: snapshot outputs are required with per_tile_bucket_offset");
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const dim3 grid(gx * gy), block(kBlendThreads);
+  hipStream_t s = (hipStream_t) stream;
+#define FSGS_LAUNCH_FWD(AUX, SNAP, ACC)                                                                              \
+  hipLaunchKernelGGL((fast_blend_forward_kernel<AUX, SNAP, ACC>), grid, block, 0, s, W, H, (float) near_n,           \
+                     (float) far_n, ranges, point_list, (const float2*) means2D, colors, trans_mat, inverse_m,       \
+                     (const float4*) normal_opacity, bucket_offset, n_contrib, out_color, out_opacity, out_extras,   \
+                     max_contrib, bucket_to_tile, sampled_T, sampled_acc, sampled_aux, accum_max_count,              \
+                     accum_weights_p, accum_weights_count)
+  if (!aux) FSGS_LAUNCH_FWD(false, false, false);
+  else if (snap && accum) FSGS_LAUNCH_FWD(true, true, true);
+  else if (snap) FSGS_LAUNCH_FWD(true, true, false);
+  else if (accum) FSGS_LAUNCH_FWD(true, false, true);
+  else FSGS_LAUNCH_FWD(true, false, false);
+#undef FSGS_LAUNCH_FWD
+  return check_launch("GS_2D_fast_render_forward");
+}
+
+FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n, double far_n, int per_splat_form,
+    const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,
+    const float* inverse_m, const float* out_opacity, const float* out_extras, const float* dL_dpix,
+    const float* dL_dopacity, const float* dL_dextras, const int64_t* ranges, const int32_t* point_list,
+    const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans, float* g_inv,
+    float* g_normal_opacity, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_fast_render_backward: bad sizes");
+  if (P == 0) return kOk;
+  FSGS_REQUIRE(means2D && normal_opacity && colors && trans_mat && inverse_m && out_opacity && dL_dpix && dL_dopacity &&
+                   ranges && n_contrib && g_colors && g_means2D && g_trans && g_inv && g_normal_opacity,
+               "GS_2D_fast_render_backward: null pointer");
+  const bool aux = out_extras && dL_dextras;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const dim3 grid(gx * gy), block(kBlendThreads);
+  hipStream_t s = (hipStream_t) stream;
+#define FSGS_LAUNCH_BWD(AUX, SPLAT)                                                                                  \
+  hipLaunchKernelGGL((fast_blend_backward_kernel<AUX, SPLAT>), grid, block, 0, s, W, H, (float) near_n,              \
+                     (float) far_n, ranges, point_list, n_contrib, (const float2*) means2D,                          \
+                     (const float4*) normal_opacity, colors, trans_mat, inverse_m, out_opacity, out_extras, dL_dpix, \
+                     dL_dextras, dL_dopacity, g_means2D, g_normal_opacity, g_colors, g_trans, g_inv)
+  if (aux && per_splat_form) FSGS_LAUNCH_BWD(true, true);
+  else if (aux) FSGS_LAUNCH_BWD(true, false);
+  else if (per_splat_form) FSGS_LAUNCH_BWD(false, true);
+  else FSGS_LAUNCH_BWD(false, false);
+#undef FSGS_LAUNCH_BWD
+  return check_launch("GS_2D_fast_render_backward");
+}

@@ -7,6 +7,7 @@
 // against a plain IEEE evaluation of the same expressions.
 #include "common.hpp"
 #include "sh.hpp"
+#include "surfel_geom.hpp"
 
 namespace fsgs {
 namespace {
@@ -76,22 +77,6 @@ __device__ __forceinline__ void transmat(int W, int H, const float* p, float sx,
   nrm[0] = Tw2v[0] * t0 + Tw2v[1] * t1 + Tw2v[2] * t2;
   nrm[1] = Tw2v[4] * t0 + Tw2v[5] * t1 + Tw2v[6] * t2;
   nrm[2] = Tw2v[8] * t0 + Tw2v[9] * t1 + Tw2v[10] * t2;
-}
-
-__device__ __forceinline__ bool bound_3sigma(const float* M, float* c, float* ext) {
-  const float t0 = 9.0f, t1 = 9.0f, t2 = -1.0f;
-  const float d  = t0 * (M[6] * M[6]) + t1 * (M[7] * M[7]) + t2 * (M[8] * M[8]);
-  if (d == 0.0f) return false;
-  const float inv = 1 / d;
-  const float f0 = inv * t0, f1 = inv * t1, f2 = inv * t2;
-  const float px = f0 * (M[0] * M[6]) + f1 * (M[1] * M[7]) + f2 * (M[2] * M[8]);
-  const float py = f0 * (M[3] * M[6]) + f1 * (M[4] * M[7]) + f2 * (M[5] * M[8]);
-  const float hx = px * px - (f0 * (M[0] * M[0]) + f1 * (M[1] * M[1]) + f2 * (M[2] * M[2]));
-  const float hy = py * py - (f0 * (M[3] * M[3]) + f1 * (M[4] * M[4]) + f2 * (M[5] * M[5]));
-  c[0] = px, c[1] = py;
-  ext[0] = sqrtf(fmaxf(1e-4f, hx));
-  ext[1] = sqrtf(fmaxf(1e-4f, hy));
-  return true;
 }
 
 template <int kSh>
@@ -172,31 +157,6 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
   tiles_touched[i] = ok ? area : 0;
   if (ok || !means2D_preserve) means2D[i] = ok ? make_float2(c2[0], c2[1]) : make_float2(0.0f, 0.0f);
   normal_opacity[i] = ok ? make_float4(nrm[0], nrm[1], nrm[2], opacities[i]) : make_float4(0, 0, 0, 0);
-}
-
-__device__ __forceinline__ void bound_backward(const float* M, float g2x, float g2y, float* gM) {
-  const float t[3] = {9.0f, 9.0f, -1.0f};
-  const float d    = t[0] * (M[6] * M[6]) + t[1] * (M[7] * M[7]) + t[2] * (M[8] * M[8]);
-  const float inv  = 1.0f / d;
-  float f[3], df[3];
-#pragma unroll
-  for (int a = 0; a < 3; ++a) f[a] = t[a] * inv;
-  float g0[3], g1[3], gr2[3];
-#pragma unroll
-  for (int a = 0; a < 3; ++a) {
-    g0[a]  = g2x * f[a] * M[6 + a];
-    g1[a]  = g2y * f[a] * M[6 + a];
-    gr2[a] = g2x * f[a] * M[a] + g2y * f[a] * M[3 + a];
-    df[a]  = g2x * M[a] * M[6 + a] + g2y * M[3 + a] * M[6 + a];
-  }
-  const float dd = (df[0] * f[0] + df[1] * f[1] + df[2] * f[2]) * -(1.0f / d);
-#pragma unroll
-  for (int a = 0; a < 3; ++a) {
-    gr2[a] += dd * (t[a] * M[6 + a] * 2.0f);
-    gM[a] += g0[a];
-    gM[3 + a] += g1[a];
-    gM[6 + a] += gr2[a];
-  }
 }
 
 __device__ __forceinline__ void transmat_backward(int W, int H, float sx, float sy, const float4 q, const float* Tw2c,

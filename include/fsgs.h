@@ -92,6 +92,66 @@ int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n,
     const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
     float* g_normal_opacity, void* stream);
 
+/* ---- "fast" surfel path: transform through camera intrinsics Tv2s[3,3], adjugate-based intersection, fused
+ * corner-test binning. Flow outputs are not supported on this path. ---- */
+
+/* gs_2d_fast_preprocess_forward (per-surfel part) -- gs_2d_fast_preprocess.cu:160-262, host :611-709.
+ * Same outputs as fsgs_gs_2d_preprocess_forward plus inverse_m[P,3,3] (adjugate of trans_mat). Only the z translation
+ * of Tw2v enters the transform, as in the reference (:95). */
+int fsgs_gs_2d_fast_preprocess_forward(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
+    const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
+    const float* Tw2v, const float* Tv2s, const float* campos, const float* trans_precomp, const uint8_t* culling,
+    int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* inverse_m, float* normal_opacity,
+    float* depths, int32_t* radii, int32_t* tiles_touched, void* stream);
+
+/* Binning half of gs_2d_fast_preprocess_forward -- gs_2d_fast_preprocess.cu:264-327 (duplicateWithKeys with the
+ * per-tile corner test, x-major, unused slots padded with key = T << 32 / value = -1), :711-778 (sort on
+ * 32 + msb(T + 1) bits, ranges). The prefix scan is fsgs_gs_prepare_scan; workspace size is
+ * fsgs_gs_prepare_fill_workspace_bytes(R). point_list[R] keeps the -1 padding entries at its tail. */
+int fsgs_gs_2d_fast_prepare_sort_bits(int W, int H);
+int fsgs_gs_2d_fast_prepare_fill(int P, int W, int H, const float* means2D, const float* inverse_m,
+    const float* depths, const float* opacities, const int32_t* radii, const int64_t* point_offsets, int64_t R,
+    int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out, void* workspace, size_t workspace_bytes,
+    void* stream);
+
+/* gs_2d_fast_preprocess_backward -- gs_2d_fast_preprocess.cu:536-609, host :784-852. grad_mean2D is read, then
+ * overwritten with the densification proxy computed from the ACCUMULATED transform gradient (:606-608). */
+int fsgs_gs_2d_fast_preprocess_backward(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
+    const float* scales, const float* rotations, const float* shs, const float* sh_rest, const float* Tw2v,
+    const float* Tv2s, const float* campos, const float* trans_mat, const int32_t* radii, const float* colors,
+    float* grad_mean2D, const float* grad_trans, const float* grad_inv_m, const float* grad_colors,
+    const float* grad_normal_opacity, float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs,
+    float* g_sh_rest, void* stream);
+
+/* gs_2d_fast_compute_transmat_forward / gs_2d_fast_compute_trans_mat_backward -- gs_2d_fast_preprocess.cu:862-966
+ * (device functions :60-140). */
+int fsgs_gs_2d_fast_compute_transmat_forward(int P, const float* means3D, const float* scales,
+    const float* rotations, const float* Tw2v, const float* Tv2s, float* trans_mat, float* normals, void* stream);
+int fsgs_gs_2d_fast_compute_transmat_backward(int P, const float* means3D, const float* scales,
+    const float* rotations, const float* Tw2v, const float* Tv2s, const float* g_mat, const float* g_normals,
+    float* g_means3D, float* g_scales, float* g_rot, void* stream);
+
+/* GS_2D_fast_render_forward -- gs_2d_fast_redner.cu:839-953 (kernel :22-271). out_extras[8,H,W]. With
+ * bucket_offset[T] (inclusive cumsum of ceil(len/32) per tile) the kernel also writes max_contrib[T],
+ * bucket_to_tile[B], sampled_T[B,256], sampled_acc[B,3,256], sampled_aux[B,8,256] (state before every 32nd list
+ * entry, for pixels still blending; channel 4 of sampled_aux is never written, as in the reference). */
+int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, double far_n, int only_image,
+    const float* means2D, const float* colors, const float* normal_opacity, const float* trans_mat,
+    const float* inverse_m, const int32_t* point_list, const int64_t* ranges, int32_t* accum_max_count,
+    float* accum_weights_p, int32_t* accum_weights_count, const int64_t* bucket_offset, float* out_color,
+    float* out_opacity, float* out_extras, int32_t* n_contrib, int32_t* max_contrib, int32_t* bucket_to_tile,
+    float* sampled_T, float* sampled_acc, float* sampled_aux, void* stream);
+
+/* GS_2D_fast_render_backward -- gs_2d_fast_redner.cu:955-1074. per_splat_form = 0: kernel :273-561 (image, opacity,
+ * aux 0-5); per_splat_form = 1: the channel set of kernel :563-837 (image, opacity, aux 0-4 and 6-7, no distortion).
+ * All five gradient outputs MUST be zero-filled by the caller. */
+int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n, double far_n, int per_splat_form,
+    const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,
+    const float* inverse_m, const float* out_opacity, const float* out_extras, const float* dL_dpix,
+    const float* dL_dopacity, const float* dL_dextras, const int64_t* ranges, const int32_t* point_list,
+    const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans, float* g_inv,
+    float* g_normal_opacity, void* stream);
+
 /* gs_2d_topk_weights -- fast_2d_gs/_C/src/gaussian_splatting/gaussian_topk.cu:230-250 (kernel :95-210).
  * top_indices[H,W,topk] int32 (-1 = empty), top_weights[H,W,topk] descending blend weights alpha*T; topk <= 16. */
 int fsgs_gs_2d_topk_weights(int topk, int P, int W, int H, double near_n, double far_n, const float* means2D,

@@ -13,7 +13,8 @@
 //                                          term overwritten by the M2 one, :748-757)
 //
 // One documented deviation: the reference evaluates log2(opacity) in the corner test with PTX `lg2.approx.f32`
-// (gs_2d_fast_preprocess.cu:48-52, :282); the oracle and the GPU kernel both use the correctly rounded log2.
+// (gs_2d_fast_preprocess.cu:48-52, :282); the oracle and the GPU kernel both evaluate log2 in double precision and
+// round the result to the working type.
 //
 // Pinned by tests/test_oracle_fast.py: equivalence with the (independently pinned) standard path when the intrinsics
 // equal (ndc2pix * Tv2c)[:3,:3] and the camera has no x/y translation, brute-force corner tests in double precision,
@@ -163,7 +164,7 @@ template <typename T>
 struct CornerTest {
   T Wxx, Wyy, Wxy, Wx_, Wy_, W__;
   CornerTest(const T* IM, T opacity) {
-    const T d = -T(2) * T(0.69314718055f) * (T(7.9886846867721655) + std::log2(opacity));
+    const T d = -T(2) * T(0.69314718055f) * (T(7.9886846867721655) + T(std::log2((double) opacity)));
     Wxx = IM[0] * IM[0] + IM[3] * IM[3] + d * IM[6] * IM[6];
     Wyy = IM[1] * IM[1] + IM[4] * IM[4] + d * IM[7] * IM[7];
     W__ = IM[2] * IM[2] + IM[5] * IM[5] + d * IM[8] * IM[8];
