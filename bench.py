@@ -19,6 +19,38 @@ import numpy as np
 import torch
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+ROOT = os.path.dirname(os.path.abspath(__file__))
+# Hardware-counter summary of the dominant kernel (two rocprofv3 --pmc passes, calibrated against the copy probe).
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gs_2d_render_backward_300k_800x800.pmc_traffic.txt")
+
+
+def measured_traffic(kernel: str):
+    """HBM bytes per launch of `kernel` from the committed counter summary (a line `<kernel>.traffic_bytes = N`)."""
+    try:
+        with open(TRAFFIC_SUMMARY) as f:
+            for line in f:
+                if line.startswith(kernel + ".traffic_bytes"):
+                    return int(float(line.split("=")[1].split()[0]))
+    except OSError:
+        pass
+    return None
+
+
+def copy_probe_gbps(dev, nbytes: int = 1 << 30, reps: int = 10) -> float:
+    """Achievable HBM bandwidth: read + write bytes of a plain streaming copy kernel per second."""
+    from fast_sp_gs_amd import lib as L
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    lib, stream = L.load(), L.current_stream()
+    for _ in range(2):
+        L.check(lib.fsgs_copy_probe(L.ptr(src), L.ptr(dst), nbytes, stream), 'copy_probe')
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        lib.fsgs_copy_probe(L.ptr(src), L.ptr(dst), nbytes, stream)
+    e1.record()
+    torch.cuda.synchronize()
+    return 2.0 * nbytes * reps / (e0.elapsed_time(e1) * 1e-3) / 1e9
 
 
 def algorithmic_bytes(stage: str, P: int, Pv: int, R: int, T: int, HW: int) -> int:
@@ -140,6 +172,8 @@ def main():
     torch.cuda.synchronize()
     knn_ms = e0.elapsed_time(e1) / 20
 
+    copy_gbps = copy_probe_gbps(dev)
+
     result = {
         "metric": "fwd+bwd frames/s, 300k surfels @800x800",
         "value": args.steps / dt,
@@ -158,8 +192,9 @@ def main():
                                "depth/normal outputs",
                    "P": P, "P_visible": Pv, "R": R, "tiles": T},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
-                     "algorithmic_bytes_per_launch": bytes_dom, "avg_launch_ms": stage_avg[dominant]},
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(dominant),
+                     "algorithmic_bytes_per_launch": bytes_dom, "avg_launch_ms": stage_avg[dominant],
+                     "copy_kernel_GBps": round(copy_gbps, 1)},
         "stages": stages,
         "extra_metrics": {"knn_topk_queries_per_s": pts.shape[0] / (knn_ms * 1e-3),
                           "knn_topk_workload": "200000 x 512, k=4, D=3"},

@@ -18,7 +18,28 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+namespace {
+// Plain streaming copy, 16 bytes per lane and grid-stride: the yardstick for achievable HBM bandwidth and the known-size
+// kernel against which hardware byte counters are calibrated.
+__global__ void __launch_bounds__(256) copy_probe_kernel(const float4* __restrict__ src, float4* __restrict__ dst,
+                                                         size_t n) {
+  for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t) gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+}  // namespace
+
 }  // namespace fsgs
+
+FSGS_API int fsgs_copy_probe(const void* src, void* dst, size_t nbytes, void* stream) {
+  FSGS_REQUIRE(src && dst && nbytes % 16 == 0 && (((uintptr_t) src | (uintptr_t) dst) & 15) == 0,
+               "copy_probe: buffers must be 16-byte aligned and a multiple of 16 bytes long");
+  const size_t n = nbytes / 16;
+  if (n == 0) return fsgs::kOk;
+  const size_t blocks = (n + 255) / 256;
+  hipLaunchKernelGGL(fsgs::copy_probe_kernel, dim3((unsigned) (blocks < 16384 ? blocks : 16384)), dim3(256), 0,
+                     (hipStream_t) stream, (const float4*) src, (float4*) dst, n);
+  return fsgs::check_launch("copy_probe");
+}
 
 FSGS_API const char* fsgs_last_error() { return fsgs::last_error_buffer(); }
 

@@ -129,6 +129,62 @@ __device__ __forceinline__ unsigned quadrant_mask(const SplatHot& h, int tile_px
   return m;
 }
 
+// ---- longest-list-first tile schedule -------------------------------------------------------------------------------
+// Blocks are handed to the CUs in blockIdx order, and a tile's cost is proportional to the length of its list, so the
+// blend kernels map blockIdx -> tile through a table that lists tiles by descending list length (quarter-octave
+// buckets, arbitrary order inside a bucket). The long lists start first and the short ones fill the tail of the launch.
+// The table lives in a file-scope device array (one copy per translation unit that includes this header): calls that
+// overlap on different streams would race on it, so the blend entry points must be issued on one stream at a time.
+constexpr int kMaxOrderedTiles = 1 << 16;
+constexpr int kOrderBuckets    = 128;
+
+namespace {
+
+__device__ int g_tile_order[kMaxOrderedTiles];
+
+__device__ __forceinline__ int length_bucket(int64_t len64) {
+  const unsigned len = len64 > 0x7fffffff ? 0x7fffffffu : (unsigned) (len64 < 0 ? 0 : len64);
+  if (len == 0) return 0;
+  const int m    = 31 - __clz(len);
+  const int frac = m >= 2 ? (int) ((len >> (m - 2)) & 3u) : (int) ((len << (2 - m)) & 3u);
+  return 1 + m * 4 + frac;  // <= 124
+}
+
+__global__ void __launch_bounds__(1024) tile_order_kernel(int T, const int64_t* __restrict__ ranges) {
+  __shared__ int s_count[kOrderBuckets];
+  for (int b = threadIdx.x; b < kOrderBuckets; b += blockDim.x) s_count[b] = 0;
+  __syncthreads();
+  for (int t = threadIdx.x; t < T; t += blockDim.x)
+    atomicAdd(&s_count[length_bucket(ranges[2 * (size_t) t + 1] - ranges[2 * (size_t) t])], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {  // exclusive prefix from the longest bucket down
+    int run = 0;
+    for (int b = kOrderBuckets - 1; b >= 0; --b) {
+      const int c = s_count[b];
+      s_count[b]  = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < T; t += blockDim.x) {
+    const int pos     = atomicAdd(&s_count[length_bucket(ranges[2 * (size_t) t + 1] - ranges[2 * (size_t) t])], 1);
+    g_tile_order[pos] = t;
+  }
+}
+
+// Returns 1 when the table was built for this launch (T small enough), else 0 and blocks map to tiles directly.
+inline int launch_tile_order(int T, const int64_t* ranges, hipStream_t s) {
+  if (T > kMaxOrderedTiles) return 0;
+  hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, s, T, ranges);
+  return 1;
+}
+
+__device__ __forceinline__ int scheduled_tile(int ordered) {
+  return ordered ? g_tile_order[blockIdx.x] : (int) blockIdx.x;
+}
+
+}  // namespace
+
 // ---- wave64 reductions through DPP --------------------------------------------------------------------------------
 template <int kCtrl, int kRowMask, int kBankMask>
 __device__ __forceinline__ float dpp_shift_zero(float v) {

@@ -23,7 +23,7 @@ constexpr int kGradSlots = 18;
 
 template <bool kAux, bool kFlow>
 __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
-    int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const int32_t* __restrict__ n_contrib, const float2* __restrict__ means2D,
     const float4* __restrict__ normal_opacity, const float* __restrict__ colors, const float* __restrict__ trans_mat,
     const float* __restrict__ trans_mat_t2, const float* __restrict__ out_opacity, const float* __restrict__ out_extras,
@@ -38,7 +38,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
   __shared__ unsigned char s_mask[kBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
 
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = blockIdx.x, tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -281,8 +281,9 @@ FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, doub
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
+  const int ordered = launch_tile_order(gx * gy, ranges, s);
 #define FSGS_LAUNCH_BWD(AUX, FLOW)                                                                                   \
-  hipLaunchKernelGGL((blend_backward_kernel<AUX, FLOW>), grid, block, 0, s, W, H, (float) near_n, (float) far_n,     \
+  hipLaunchKernelGGL((blend_backward_kernel<AUX, FLOW>), grid, block, 0, s, ordered, W, H, (float) near_n, (float) far_n,     \
                      ranges, point_list, n_contrib, (const float2*) means2D, (const float4*) normal_opacity, colors, \
                      trans_mat, trans_mat_t2, out_opacity, out_extras, (const float2*) out_flow, dL_dpix,            \
                      dL_dextras, dL_dopacity, (const float2*) dL_dflow, g_means2D, g_normal_opacity, g_colors,       \

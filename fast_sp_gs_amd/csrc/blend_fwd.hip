@@ -17,7 +17,7 @@ namespace {
 
 template <bool kAux, bool kFlow, bool kAccum>
 __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
-    int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const float2* __restrict__ means2D, const float* __restrict__ colors, const float* __restrict__ trans_mat,
     const float4* __restrict__ normal_opacity, const float* __restrict__ trans_mat_t2, int32_t* __restrict__ n_contrib,
     float* __restrict__ out_color, float* __restrict__ out_opacity, float* __restrict__ out_extras,
@@ -29,7 +29,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   __shared__ unsigned char s_mask[kBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
 
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = blockIdx.x, tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -181,8 +181,9 @@ FSGS_API int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, doubl
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
+  const int ordered = launch_tile_order(gx * gy, ranges, s);
 #define FSGS_LAUNCH_FWD(AUX, FLOW, ACC)                                                                              \
-  hipLaunchKernelGGL((blend_forward_kernel<AUX, FLOW, ACC>), grid, block, 0, s, W, H, (float) near_n, (float) far_n, \
+  hipLaunchKernelGGL((blend_forward_kernel<AUX, FLOW, ACC>), grid, block, 0, s, ordered, W, H, (float) near_n, (float) far_n, \
                      ranges, point_list, (const float2*) means2D, colors, trans_mat, (const float4*) normal_opacity, \
                      trans_mat_t2, n_contrib, out_color, out_opacity, out_extras, (float2*) out_flow,                \
                      accum_max_count, accum_weights_p, accum_weights_count)

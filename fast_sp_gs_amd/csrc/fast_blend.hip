@@ -116,7 +116,7 @@ __device__ __forceinline__ float wave_sum8_transposed(const float (&v)[8]) {
 
 template <bool kAux, bool kSnap, bool kAccum>
 __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
-    int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const float2* __restrict__ means2D, const float* __restrict__ colors, const float* __restrict__ trans_mat,
     const float* __restrict__ inverse_m, const float4* __restrict__ normal_opacity,
     const int64_t* __restrict__ bucket_offset, int32_t* __restrict__ n_contrib, float* __restrict__ out_color,
@@ -130,7 +130,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
   __shared__ int s_max_contrib;
 
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = blockIdx.x, tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -279,7 +279,7 @@ constexpr int kFastGradSlots = 21;
 
 template <bool kAux, bool kPerSplat>
 __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
-    int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const int32_t* __restrict__ n_contrib, const float2* __restrict__ means2D,
     const float4* __restrict__ normal_opacity, const float* __restrict__ colors, const float* __restrict__ trans_mat,
     const float* __restrict__ inverse_m, const float* __restrict__ out_opacity, const float* __restrict__ out_extras,
@@ -293,7 +293,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
   __shared__ unsigned char s_mask[kBatch];
 
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = blockIdx.x, tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -508,8 +508,9 @@ FSGS_API int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, 
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
+  const int ordered = launch_tile_order(gx * gy, ranges, s);
 #define FSGS_LAUNCH_FWD(AUX, SNAP, ACC)                                                                              \
-  hipLaunchKernelGGL((fast_blend_forward_kernel<AUX, SNAP, ACC>), grid, block, 0, s, W, H, (float) near_n,           \
+  hipLaunchKernelGGL((fast_blend_forward_kernel<AUX, SNAP, ACC>), grid, block, 0, s, ordered, W, H, (float) near_n,           \
                      (float) far_n, ranges, point_list, (const float2*) means2D, colors, trans_mat, inverse_m,       \
                      (const float4*) normal_opacity, bucket_offset, n_contrib, out_color, out_opacity, out_extras,   \
                      max_contrib, bucket_to_tile, sampled_T, sampled_acc, sampled_aux, accum_max_count,              \
@@ -538,8 +539,9 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
+  const int ordered = launch_tile_order(gx * gy, ranges, s);
 #define FSGS_LAUNCH_BWD(AUX, SPLAT)                                                                                  \
-  hipLaunchKernelGGL((fast_blend_backward_kernel<AUX, SPLAT>), grid, block, 0, s, W, H, (float) near_n,              \
+  hipLaunchKernelGGL((fast_blend_backward_kernel<AUX, SPLAT>), grid, block, 0, s, ordered, W, H, (float) near_n,              \
                      (float) far_n, ranges, point_list, n_contrib, (const float2*) means2D,                          \
                      (const float4*) normal_opacity, colors, trans_mat, inverse_m, out_opacity, out_extras, dL_dpix, \
                      dL_dextras, dL_dopacity, g_means2D, g_normal_opacity, g_colors, g_trans, g_inv)

@@ -24,6 +24,9 @@ extern "C" {
 const char* fsgs_last_error(void);
 int fsgs_version(void);
 int fsgs_check_device(void);
+/* Measurement aid without a counterpart in the reference: copies nbytes (multiple of 16, 16-byte aligned) from src to
+ * dst with a plain streaming kernel; benchmarks use it as the achievable-bandwidth yardstick and counter calibration. */
+int fsgs_copy_probe(const void* src, void* dst, size_t nbytes, void* stream);
 
 /* ---- 2DGS surfel preprocess ---------------------------------------------------------------------------------- */
 
