@@ -287,10 +287,14 @@ def GS_2D_render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat2
     P = means2D.shape[0]
     H, W = dL_dout_color.shape[1], dL_dout_color.shape[2]
     opt = dict(dtype=torch.float32, device=out_opacity.device)
-    g_means2D = torch.zeros((P, 2), **opt)
-    g_norm_op = torch.zeros((P, 4), **opt)
-    g_colors = torch.zeros((P, 3), **opt)
-    g_trans = torch.zeros((P, 3, 3), **opt)
+    # one zero-fill for the four accumulated outputs; every segment starts on a 16-byte boundary
+    up = lambda n: (n + 3) // 4 * 4
+    o1, o2, o3 = up(4 * P), up(4 * P) + up(9 * P), up(4 * P) + up(9 * P) + up(3 * P)
+    flat = torch.zeros((o3 + 2 * P,), **opt)
+    g_norm_op = flat[:4 * P].view(P, 4)
+    g_trans = flat[o1:o1 + 9 * P].view(P, 3, 3)
+    g_colors = flat[o2:o2 + 3 * P].view(P, 3)
+    g_means2D = flat[o3:o3 + 2 * P].view(P, 2)
     if P == 0:
         return g_colors, g_means2D, g_trans, g_norm_op
     c = lambda t: None if t is None else t.contiguous()

@@ -203,6 +203,26 @@ __device__ __forceinline__ float wave_sum_to_lane63(float v) {
   return v;
 }
 
+// Adds the values held by the same lane position of the four 16-lane rows; every lane gets the total.
+// gfx950's row/half swaps do it in the VALU (no LDS round trip as with a bpermute): after swapping the odd rows of one
+// copy with the even rows of another, copy A holds rows (0,0,2,2) and copy B rows (1,1,3,3); the 32-lane swap does the
+// same for the halves. Written as inline assembly because the compiler's builtin for these instructions returns the
+// first result twice; the s_nop cover the VALU-write -> swap-read wait states the compiler would insert itself.
+__device__ __forceinline__ float cross_row_sum(float z) {
+#ifdef FSGS_NO_PERMLANE_SWAP
+  z += __shfl_xor(z, 16, kWave);
+  z += __shfl_xor(z, 32, kWave);
+  return z;
+#else
+  float a = z, b = z;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32_e32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  z = a + b;
+  a = z, b = z;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32_e32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+#endif
+}
+
 // Sums 16 per-lane values over the 64 lanes at once ("transposed" butterfly): each step halves the number of live
 // registers while doubling the lanes a partial covers, so 16 wave-wide sums cost 15 merge steps (2 DPP adds + 1 select
 // each) plus two cross-row exchanges, instead of 16 x 6 dependent DPP adds. On return every lane holds the wave total of
@@ -232,9 +252,7 @@ __device__ __forceinline__ float wave_sum16_transposed(const float (&v)[16]) {
   const float a = y[1] + dpp_shift_zero<0x118, 0xf, 0xf>(y[1]);  // row_shr:8
   const float b = y[0] + dpp_shift_zero<0x108, 0xf, 0xf>(y[0]);  // row_shl:8
   float z = b3 ? a : b;                                          // lane l of every row: row total of v[l & 15]
-  z += __shfl_xor(z, 16, kWave);
-  z += __shfl_xor(z, 32, kWave);
-  return z;
+  return cross_row_sum(z);
 }
 
 }  // namespace fsgs

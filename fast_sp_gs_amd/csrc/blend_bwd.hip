@@ -20,9 +20,17 @@ namespace {
 // The first 16 go through one transposed wave reduction; the means2D pair is only non-zero for pixels where the
 // screen-space low-pass filter wins (rho2d < rho3d) and is reduced separately when any lane took that branch.
 constexpr int kGradSlots = 18;
+#ifndef FSGS_BWD_BATCH
+#define FSGS_BWD_BATCH 64
+#endif
+#ifndef FSGS_BWD_WAVES
+#define FSGS_BWD_WAVES 4
+#endif
+constexpr int kBwdBatch = FSGS_BWD_BATCH;  // surfels staged per round (<= block size)
 
 template <bool kAux, bool kFlow>
-__global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
+__global__ void __launch_bounds__(kBlendThreads) __attribute__((amdgpu_waves_per_eu(FSGS_BWD_WAVES, FSGS_BWD_WAVES)))
+blend_backward_kernel(
     int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const int32_t* __restrict__ n_contrib, const float2* __restrict__ means2D,
     const float4* __restrict__ normal_opacity, const float* __restrict__ colors, const float* __restrict__ trans_mat,
@@ -30,12 +38,12 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
     const float2* __restrict__ out_flow, const float* __restrict__ dL_dpix, const float* __restrict__ dL_dextras,
     const float* __restrict__ dL_dopacity, const float2* __restrict__ dL_dflow, float* __restrict__ g_means2D,
     float* __restrict__ g_normal_opacity, float* __restrict__ g_colors, float* __restrict__ g_trans) {
-  __shared__ SplatHot s_hot[kBatch];
-  __shared__ SplatCold s_cold[kBatch];
-  __shared__ float s_acc[kBatch][kGradSlots + 1];  // +1: odd stride keeps the flush conflict free
-  __shared__ float s_t2[kFlow ? kBatch * 9 : 1];
+  __shared__ SplatHot s_hot[kBwdBatch];
+  __shared__ SplatCold s_cold[kBwdBatch];
+  __shared__ float s_acc[kBwdBatch][kGradSlots + 1];  // +1: odd stride keeps the flush conflict free
+  __shared__ float s_t2[kFlow ? kBwdBatch * 9 : 1];
   __shared__ int s_max_contrib;
-  __shared__ unsigned char s_mask[kBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
+  __shared__ unsigned char s_mask[kBwdBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
 
   const int gx = (W + kTile - 1) / kTile;
   const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
@@ -59,10 +67,11 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
   for (int d = 32; d >= 1; d >>= 1) wave_max_contrib = max(wave_max_contrib, __shfl_xor(wave_max_contrib, d, kWave));
   if (lane == 0) atomicMax(&s_max_contrib, wave_max_contrib);
 #pragma unroll
-  for (int c = 0; c < kGradSlots + 1; ++c) s_acc[threadIdx.x][c] = 0.0f;
+  for (int c = 0; c < kGradSlots + 1; ++c)
+    if ((int) threadIdx.x < kBwdBatch) s_acc[threadIdx.x][c] = 0.0f;
   __syncthreads();
   const int n_todo = min(s_max_contrib, (int) (r1 - r0));  // positions [0, n_todo) of the tile's list, walked from n_todo-1 down to 0
-  const int rounds = (n_todo + kBatch - 1) / kBatch;
+  const int rounds = (n_todo + kBwdBatch - 1) / kBwdBatch;
 
   const float T_final = inside ? 1.0f - out_opacity[pix] : 0.0f;
   float T = T_final;
@@ -93,15 +102,13 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
     dLf0 = g.x / sum_w, dLf1 = g.y / sum_w;
   }
 
-  float acc_c0 = 0, acc_c1 = 0, acc_c2 = 0, last_c0 = 0, last_c1 = 0, last_c2 = 0;
-  float last_depth = 0, acc_depth = 0, acc_alpha = 0;
-  float last_n0 = 0, last_n1 = 0, last_n2 = 0, acc_n0 = 0, acc_n1 = 0, acc_n2 = 0;
+  float acc_lin = 0, last_lin = 0;
   float last_dL_dT = 0, last_alpha = 0, acc_w = 0;
   float acc_f0 = 0, acc_f1 = 0, last_f0 = 0, last_f1 = 0;
 
   Splat next;
   float next_t2[9];
-  if ((int) threadIdx.x < n_todo) {
+  if ((int) threadIdx.x < min(n_todo, kBwdBatch)) {
     next = gather_splat(point_list[r0 + (n_todo - 1 - (int) threadIdx.x)], means2D, colors, normal_opacity, trans_mat);
     if (kFlow)
 #pragma unroll
@@ -109,7 +116,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
   }
 
   for (int b = 0; b < rounds; ++b) {
-    const int n_here = min(kBatch, n_todo - b * kBatch);
+    const int n_here = min(kBwdBatch, n_todo - b * kBwdBatch);
     if ((int) threadIdx.x < n_here) {
       s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
@@ -119,8 +126,8 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
         for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
     }
     __syncthreads();
-    const int nxt = (b + 1) * kBatch + (int) threadIdx.x;
-    if (nxt < n_todo) {
+    const int nxt = (b + 1) * kBwdBatch + (int) threadIdx.x;
+    if ((int) threadIdx.x < kBwdBatch && nxt < n_todo) {
       next = gather_splat(point_list[r0 + (n_todo - 1 - nxt)], means2D, colors, normal_opacity, trans_mat);
       if (kFlow)
 #pragma unroll
@@ -129,14 +136,14 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
 
     // Work list of this wavefront for 64 staged surfels at a time: those that can reach its quadrant and are not
     // behind its deepest contributor; consumed bit by bit with scalar instructions.
-    for (int chunk = 0; chunk < kBatch / kWave; ++chunk) {
+    for (int chunk = 0; chunk < kBwdBatch / kWave; ++chunk) {
      const int jj = chunk * kWave + lane;
      unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u) &&
-                                        (n_todo - 1 - (b * kBatch + jj)) < wave_max_contrib);
+                                        (n_todo - 1 - (b * kBwdBatch + jj)) < wave_max_contrib);
      while (todo) {
       const int j = chunk * kWave + __builtin_ctzll(todo);
       todo &= todo - 1;
-      const int pos = n_todo - 1 - (b * kBatch + j);  // 0-based position in the tile's list
+      const int pos = n_todo - 1 - (b * kBwdBatch + j);  // 0-based position in the tile's list
       Hit h;
       const bool hit = (pos < last_contrib) && intersect(s_hot[j], pxf, pyf, near_n, h);
       if (__ballot(hit) == 0ull) continue;  // wave-uniform: nobody in this quadrant blends the surfel
@@ -150,14 +157,13 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
         const SplatCold cold = s_cold[j];
         T             = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
         const float w = h.alpha * T;
-        float dL_dalpha = 0.0f;
-        acc_c0 = last_alpha * last_c0 + (1.0f - last_alpha) * acc_c0, last_c0 = cold.r;
-        acc_c1 = last_alpha * last_c1 + (1.0f - last_alpha) * acc_c1, last_c1 = cold.g;
-        acc_c2 = last_alpha * last_c2 + (1.0f - last_alpha) * acc_c2, last_c2 = cold.b;
-        dL_dalpha += (cold.r - acc_c0) * dLp0 + (cold.g - acc_c1) * dLp1 + (cold.b - acc_c2) * dLp2;
+        // All channels that enter the image linearly (colour, depth, opacity, normal) share one back-to-front
+        // recurrence: with c = <upstream gradient, channel values of this surfel>, the reference's per-channel
+        // accumulators acc_x = last_alpha * last_x + (1 - last_alpha) * acc_x contract to a single scalar.
+        float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
         g[0] = w * dLp0, g[1] = w * dLp1, g[2] = w * dLp2;
 
-        float dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f;
+        float dL_dalpha = 0.0f, dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f;
         if (kAux) {
           const float rd     = __builtin_amdgcn_rcpf(h.depth);
           const float m_d    = far_scale * (1.0f - near_n * rd);
@@ -168,19 +174,14 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
           last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
           const float dL_dmd = 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg;
           dL_dz += dL_dmd * dmd_dd;
-          acc_depth  = last_alpha * last_depth + (1.0f - last_alpha) * acc_depth;
-          last_depth = h.depth;
-          dL_dalpha += (h.depth - acc_depth) * dL_ddepth;
-          acc_alpha = last_alpha * 1.0f + (1.0f - last_alpha) * acc_alpha;
-          dL_dalpha += (1.0f - acc_alpha) * dL_daccum;
-          acc_n0 = last_alpha * last_n0 + (1.0f - last_alpha) * acc_n0, last_n0 = cold.nx;
-          acc_n1 = last_alpha * last_n1 + (1.0f - last_alpha) * acc_n1, last_n1 = cold.ny;
-          acc_n2 = last_alpha * last_n2 + (1.0f - last_alpha) * acc_n2, last_n2 = cold.nz;
-          dL_dalpha += (cold.nx - acc_n0) * dLn0 + (cold.ny - acc_n1) * dLn1 + (cold.nz - acc_n2) * dLn2;
+          c_lin += h.depth * dL_ddepth + dL_daccum + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
           g[12] = w * dLn0, g[13] = w * dLn1, g[14] = w * dLn2;
           dL_dz += w * dL_ddepth;
           dsx = dL_dz * hot.m[6], dsy = dL_dz * hot.m[7];
         }
+        acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
+        last_lin = c_lin;
+        dL_dalpha += c_lin - acc_lin;
         if (kFlow) {
           const float* Q = &s_t2[j * 9];
           const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
@@ -195,9 +196,9 @@ __global__ void __launch_bounds__(kBlendThreads) blend_backward_kernel(
           const float gw = -w / (w2 * w2) * (u2 * dLf0 + v2 * dLf1);
           dsx += Q[0] * gu + Q[3] * gv + Q[6] * gw;
           dsy += Q[1] * gu + Q[4] * gv + Q[7] * gw;
+          acc_w = last_alpha + (1.0f - last_alpha) * acc_w;
+          dL_dalpha += (1.0f - acc_w) * dL_dsum_w;
         }
-        acc_w = last_alpha + (1.0f - last_alpha) * acc_w;
-        dL_dalpha += (1.0f - acc_w) * dL_dsum_w;
         dL_dalpha *= T;
         last_alpha = h.alpha;
 

@@ -15,6 +15,11 @@
 namespace fsgs {
 namespace {
 
+#ifndef FSGS_FWD_BATCH
+#define FSGS_FWD_BATCH 128
+#endif
+constexpr int kFwdBatch = FSGS_FWD_BATCH;  // surfels staged per round (<= block size)
+
 template <bool kAux, bool kFlow, bool kAccum>
 __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
     int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
@@ -23,10 +28,10 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
     float* __restrict__ out_color, float* __restrict__ out_opacity, float* __restrict__ out_extras,
     float2* __restrict__ out_flow, int32_t* __restrict__ accum_max_count, float* __restrict__ accum_weights_p,
     int32_t* __restrict__ accum_weights_count) {
-  __shared__ SplatHot s_hot[kBatch];
-  __shared__ SplatCold s_cold[kBatch];
-  __shared__ float s_t2[kFlow ? kBatch * 9 : 1];
-  __shared__ unsigned char s_mask[kBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
+  __shared__ SplatHot s_hot[kFwdBatch];
+  __shared__ SplatCold s_cold[kFwdBatch];
+  __shared__ float s_t2[kFlow ? kFwdBatch * 9 : 1];
+  __shared__ unsigned char s_mask[kFwdBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
 
   const int gx = (W + kTile - 1) / kTile;
   const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
@@ -40,7 +45,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
 
   const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
   const int n_todo = (int) (r1 - r0);
-  const int rounds = (n_todo + kBatch - 1) / kBatch;
+  const int rounds = (n_todo + kFwdBatch - 1) / kFwdBatch;
 
   bool done = !inside;
   float T = 1.0f, C0 = 0, C1 = 0, C2 = 0;
@@ -51,7 +56,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
 
   Splat next;
   float next_t2[9];
-  if (threadIdx.x < n_todo) {
+  if ((int) threadIdx.x < min(n_todo, kFwdBatch)) {
     next = gather_splat(point_list[r0 + threadIdx.x], means2D, colors, normal_opacity, trans_mat);
     if (kFlow)
 #pragma unroll
@@ -61,7 +66,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   for (int b = 0; b < rounds; ++b) {
     // everyone has finished reading the previous batch; leave as soon as no pixel of the tile is still blending
     if (__syncthreads_count(done) == kBlendThreads) break;
-    const int n_here = min(kBatch, n_todo - b * kBatch);
+    const int n_here = min(kFwdBatch, n_todo - b * kFwdBatch);
     if ((int) threadIdx.x < n_here) {
       s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
@@ -71,8 +76,8 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
         for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
     }
     __syncthreads();
-    const int nxt = (b + 1) * kBatch + threadIdx.x;
-    if (nxt < n_todo) {
+    const int nxt = (b + 1) * kFwdBatch + threadIdx.x;
+    if ((int) threadIdx.x < kFwdBatch && nxt < n_todo) {
       next = gather_splat(point_list[r0 + nxt], means2D, colors, normal_opacity, trans_mat);
       if (kFlow)
 #pragma unroll
@@ -81,7 +86,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
 
     // Each wavefront walks only the surfels that can reach its quadrant: the ballot of the mask bit over 64 staged
     // surfels is the (depth-ordered) work list, consumed bit by bit with scalar instructions.
-    for (int c = 0; c < kBatch / kWave; ++c) {
+    for (int c = 0; c < kFwdBatch / kWave; ++c) {
       const int jj = c * kWave + lane;
       unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u));
       while (todo) {
@@ -98,7 +103,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
         }
         const float w        = h.alpha * T;
         const SplatCold cold = s_cold[j];
-        const int contributor = b * kBatch + j + 1;
+        const int contributor = b * kFwdBatch + j + 1;
         if (kAux) {
           const float A = 1.0f - T;
           const float m = far_n / (far_n - near_n) * (1.0f - near_n / h.depth);

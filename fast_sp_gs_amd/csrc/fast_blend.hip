@@ -109,9 +109,7 @@ __device__ __forceinline__ float wave_sum8_transposed(const float (&v)[8]) {
   const float b = x[0] + dpp_shift_zero<0x104, 0xf, 0xf>(x[0]);  // row_shl:4
   float z = b2 ? a : b;
   z += dpp_shift_zero<0x128, 0xf, 0xf>(z);  // row_ror:8
-  z += __shfl_xor(z, 16, kWave);
-  z += __shfl_xor(z, 32, kWave);
-  return z;
+  return cross_row_sum(z);
 }
 
 template <bool kAux, bool kSnap, bool kAccum>
@@ -343,10 +341,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
   const float final_A   = 1.0f - T_final;
   const float far_scale = far_n / (far_n - near_n);
 
-  float acc_c0 = 0, acc_c1 = 0, acc_c2 = 0, last_c0 = 0, last_c1 = 0, last_c2 = 0;
-  float last_depth = 0, acc_depth = 0, acc_alpha = 0;
-  float last_n0 = 0, last_n1 = 0, last_n2 = 0, acc_n0 = 0, acc_n1 = 0, acc_n2 = 0;
-  float last_m = 0, acc_m = 0, last_m2 = 0, acc_m2 = 0;
+  float acc_lin = 0, last_lin = 0;
   float last_dL_dT = 0, last_alpha = 0;
 
   FastSplat next;
@@ -389,14 +384,12 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
           const SplatCold cold = s_cold[j];
           T             = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
           const float w = h.alpha * T;
-          float dL_dalpha = 0.0f;
-          acc_c0 = last_alpha * last_c0 + (1.0f - last_alpha) * acc_c0, last_c0 = cold.r;
-          acc_c1 = last_alpha * last_c1 + (1.0f - last_alpha) * acc_c1, last_c1 = cold.g;
-          acc_c2 = last_alpha * last_c2 + (1.0f - last_alpha) * acc_c2, last_c2 = cold.b;
-          dL_dalpha += (cold.r - acc_c0) * dLp0 + (cold.g - acc_c1) * dLp1 + (cold.b - acc_c2) * dLp2;
+          // one back-to-front recurrence for every channel that enters the image linearly: c = <upstream gradient,
+          // channel values of this surfel> replaces the reference's per-channel accumulators
+          float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
           g[0] = w * dLp0, g[1] = w * dLp1, g[2] = w * dLp2;
 
-          float dL_dz = 0.0f;
+          float dL_dalpha = 0.0f, dL_dz = 0.0f;
           if (kAux) {
             const float rd     = __builtin_amdgcn_rcpf(h.depth);
             const float m_d    = far_scale * (1.0f - near_n * rd);
@@ -408,25 +401,17 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
               last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
               dL_dz += 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg * dmd_dd;
             } else {
-              acc_m  = last_alpha * last_m + (1.0f - last_alpha) * acc_m, last_m = m_d;
-              acc_m2 = last_alpha * last_m2 + (1.0f - last_alpha) * acc_m2, last_m2 = m_d * m_d;
-              dL_dalpha += (m_d - acc_m) * dL_dM1 + (m_d * m_d - acc_m2) * dL_dM2;
+              c_lin += m_d * dL_dM1 + (m_d * m_d) * dL_dM2;
               dL_dz += dmd_dd * (2.0f * m_d * w * dL_dM2);
             }
-            acc_depth  = last_alpha * last_depth + (1.0f - last_alpha) * acc_depth;
-            last_depth = h.depth;
-            dL_dalpha += (h.depth - acc_depth) * dL_ddepth;
-            acc_n0 = last_alpha * last_n0 + (1.0f - last_alpha) * acc_n0, last_n0 = cold.nx;
-            acc_n1 = last_alpha * last_n1 + (1.0f - last_alpha) * acc_n1, last_n1 = cold.ny;
-            acc_n2 = last_alpha * last_n2 + (1.0f - last_alpha) * acc_n2, last_n2 = cold.nz;
-            dL_dalpha += (cold.nx - acc_n0) * dLn0 + (cold.ny - acc_n1) * dLn1 + (cold.nz - acc_n2) * dLn2;
+            c_lin += h.depth * dL_ddepth + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
             g[12] = w * dLn0, g[13] = w * dLn1, g[14] = w * dLn2;
             dL_dz += w * dL_ddepth;
           }
-          if (kAux || kPerSplat) {
-            acc_alpha = last_alpha * 1.0f + (1.0f - last_alpha) * acc_alpha;
-            dL_dalpha += (1.0f - acc_alpha) * dL_daccum;
-          }
+          if (kAux || kPerSplat) c_lin += dL_daccum;
+          acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
+          last_lin = c_lin;
+          dL_dalpha += c_lin - acc_lin;
           dL_dalpha *= T;
           last_alpha = h.alpha;
 

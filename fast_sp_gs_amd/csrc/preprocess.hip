@@ -7,6 +7,7 @@
 // against a plain IEEE evaluation of the same expressions.
 #include "common.hpp"
 #include "sh.hpp"
+#include "sh_stage.hpp"
 #include "surfel_geom.hpp"
 
 namespace fsgs {
@@ -88,10 +89,13 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
     int means2D_preserve, float2* __restrict__ means2D, float* __restrict__ colors, float* __restrict__ trans_mat,
     float4* __restrict__ normal_opacity, float* __restrict__ depths, int32_t* __restrict__ radii,
     int32_t* __restrict__ tiles_touched) {
+  constexpr bool kStage = kSh == 16;  // degree <= 3: SH rows travel through LDS, read from HBM line by line
   __shared__ float s_Tw2v[16], s_Tw2c[16];
+  __shared__ float s_rows[kStage ? kShStageRows * kShStageStride : 1];
+  __shared__ unsigned char s_flag[kShStageRows];
   load_camera(Tw2v_g, Tv2c_g, s_Tw2v, s_Tw2c);
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= P) return;
+  const int i      = blockIdx.x * blockDim.x + threadIdx.x;
+  const bool valid = i < P;
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
 
   bool ok = false;
@@ -99,9 +103,10 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
   int area = 0;
 #pragma unroll
   for (int k = 0; k < 9; ++k) M[k] = 0.0f;
-  const float p[3] = {means3D[3 * (size_t) i], means3D[3 * (size_t) i + 1], means3D[3 * (size_t) i + 2]};
+  float p[3] = {0, 0, 0};
+  if (valid) p[0] = means3D[3 * (size_t) i], p[1] = means3D[3 * (size_t) i + 1], p[2] = means3D[3 * (size_t) i + 2];
   do {
-    if (culling && culling[i]) break;
+    if (!valid || (culling && culling[i])) break;
     float Tw2v[16], Tw2c[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) Tw2v[k] = s_Tw2v[k], Tw2c[k] = s_Tw2c[k];
@@ -131,19 +136,26 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
     ok    = true;
   } while (false);
 
-  if (ok && sh_degree >= 0) {
-    float x, y, z, Y[kSh];
-    view_dir(p, campos, x, y, z);
-    sh_eval(sh_degree, x, y, z, Y);
+  if (sh_degree >= 0) {
     const int n = sh_count(sh_degree);
-    const float* c0 = shs + (size_t) i * (sh_rest ? 1 : n_sh) * 3;
-    float r = c0[0] * Y[0], g = c0[1] * Y[0], b = c0[2] * Y[0];
-    const float* cr = sh_rest ? sh_rest + (size_t) i * n_sh * 3 - 3 : c0;
-    for (int l = 1; l < n; ++l) {
-      r += cr[3 * l] * Y[l], g += cr[3 * l + 1] * Y[l], b += cr[3 * l + 2] * Y[l];
+    if (kStage) {
+      s_flag[threadIdx.x] = ok;
+      __syncthreads();
+      stage_sh_rows(s_rows, s_flag, blockIdx.x * blockDim.x, P, n, n_sh, shs, sh_rest);
+      __syncthreads();
     }
-    rgb[0] = fmaxf(0.0f, r + 0.5f), rgb[1] = fmaxf(0.0f, g + 0.5f), rgb[2] = fmaxf(0.0f, b + 0.5f);
+    if (ok) {
+      float x, y, z, Y[kSh];
+      view_dir(p, campos, x, y, z);
+      sh_eval(sh_degree, x, y, z, Y);
+      const float* c0 = kStage ? &s_rows[threadIdx.x * kShStageStride] : shs + (size_t) i * (sh_rest ? 1 : n_sh) * 3;
+      const float* cr = kStage ? c0 : (sh_rest ? sh_rest + (size_t) i * n_sh * 3 - 3 : c0);
+      float r = c0[0] * Y[0], g = c0[1] * Y[0], b = c0[2] * Y[0];
+      for (int l = 1; l < n; ++l) r += cr[3 * l] * Y[l], g += cr[3 * l + 1] * Y[l], b += cr[3 * l + 2] * Y[l];
+      rgb[0] = fmaxf(0.0f, r + 0.5f), rgb[1] = fmaxf(0.0f, g + 0.5f), rgb[2] = fmaxf(0.0f, b + 0.5f);
+    }
   }
+  if (!valid) return;
 
   if (trans_precomp == nullptr) {
 #pragma unroll
@@ -206,71 +218,113 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
     const float4* __restrict__ grad_normal_opacity, float* __restrict__ g_means3D, float2* __restrict__ g_scales,
     float4* __restrict__ g_rot, float* __restrict__ g_opac, float* __restrict__ g_shs,
     float* __restrict__ g_sh_rest) {
+  constexpr bool kStage = kSh == 16;
   __shared__ float s_Tw2v[16], s_Tw2c[16];
+  __shared__ float s_rows[kStage ? kShStageRows * kShStageStride : 1];
+  __shared__ unsigned char s_flag[kShStageRows];
   load_camera(Tw2v_g, Tv2c_g, s_Tw2v, s_Tw2c);
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= P || radii[i] <= 0) return;
-  float Tw2v[16], Tw2c[16];
-#pragma unroll
-  for (int k = 0; k < 16; ++k) Tw2v[k] = s_Tw2v[k], Tw2c[k] = s_Tw2c[k];
-
-  const float4 gno = grad_normal_opacity[i];
-  g_opac[i]        = gno.w;
-  float gM[9], M[9], gM_in2, gM_in5;
-#pragma unroll
-  for (int k = 0; k < 9; ++k) gM[k] = grad_trans[9 * (size_t) i + k], M[k] = trans_mat[9 * (size_t) i + k];
-  gM_in2 = gM[2], gM_in5 = gM[5];
-  const float2 g2 = grad_mean2D[i];
-  bound_backward(M, g2.x, g2.y, gM);
-
-  const float4 q   = rotations[i];
-  const float p[3] = {means3D[3 * (size_t) i], means3D[3 * (size_t) i + 1], means3D[3 * (size_t) i + 2]};
-  const float t0 = 2 * (q.y * q.w + q.x * q.z), t1 = 2 * (q.y * q.z - q.x * q.w), t2 = 1 - 2 * (q.x * q.x + q.y * q.y);
-  const float nrm[3] = {Tw2v[0] * t0 + Tw2v[1] * t1 + Tw2v[2] * t2, Tw2v[4] * t0 + Tw2v[5] * t1 + Tw2v[6] * t2,
-                        Tw2v[8] * t0 + Tw2v[9] * t1 + Tw2v[10] * t2};
-  const float pv[3] = {Tw2v[0] * p[0] + Tw2v[1] * p[1] + Tw2v[2] * p[2] + Tw2v[3],
-                       Tw2v[4] * p[0] + Tw2v[5] * p[1] + Tw2v[6] * p[2] + Tw2v[7],
-                       Tw2v[8] * p[0] + Tw2v[9] * p[1] + Tw2v[10] * p[2] + Tw2v[11]};
-  const float cosv = -(pv[0] * nrm[0] + pv[1] * nrm[1] + pv[2] * nrm[2]);
-  const float mult = cosv > 0 ? 1.0f : -1.0f;
-  const float gN[3] = {mult * gno.x, mult * gno.y, mult * gno.z};
-  const float2 s = scales[i];
-  float gp[3], gs[2], gq[4];
-  transmat_backward(W, H, s.x, s.y, q, Tw2c, Tw2v, gM, gN, gp, gs, gq);
-
-  if (sh_degree >= 0) {
-    float x, y, z, Y[kSh], tl[kSh];
-    const float nn = view_dir(p, campos, x, y, z);
-    sh_eval(sh_degree, x, y, z, Y);
-    float g[3];
-#pragma unroll
-    for (int c = 0; c < 3; ++c) g[c] = grad_colors[3 * (size_t) i + c] * (float) (colors[3 * (size_t) i + c] > 0);
-    const int n  = sh_count(sh_degree);
-    const int m1 = sh_rest ? 1 : n_sh;
-    const float* c0 = shs + (size_t) i * m1 * 3;
-    const float* cr = sh_rest ? sh_rest + (size_t) i * n_sh * 3 - 3 : c0;
-    float* o0 = g_shs ? g_shs + (size_t) i * m1 * 3 : nullptr;
-    float* orr = g_sh_rest ? g_sh_rest + (size_t) i * n_sh * 3 - 3 : o0;
-    if (o0) o0[0] = g[0] * Y[0], o0[1] = g[1] * Y[0], o0[2] = g[2] * Y[0];
-    tl[0] = 0.0f;
-    for (int l = 1; l < n; ++l) {
-      tl[l] = g[0] * cr[3 * l] + g[1] * cr[3 * l + 1] + g[2] * cr[3 * l + 2];
-      if (o0) orr[3 * l] = g[0] * Y[l], orr[3 * l + 1] = g[1] * Y[l], orr[3 * l + 2] = g[2] * Y[l];
-    }
-    float dx = 0, dy = 0, dz = 0;
-    sh_grad_accumulate(sh_degree, x, y, z, tl, dx, dy, dz);
-    const float vx = p[0] - campos[0], vy = p[1] - campos[1], vz = p[2] - campos[2];
-    const float tt = -(vx * dx + vy * dy + vz * dz) * nn * nn * nn;
-    gp[0] = gp[0] + (dx * nn + tt * vx);
-    gp[1] = gp[1] + (dy * nn + tt * vy);
-    gp[2] = gp[2] + (dz * nn + tt * vz);
+  const int i      = blockIdx.x * blockDim.x + threadIdx.x;
+  const bool valid = i < P;
+  const bool vis   = valid && radii[i] > 0;
+  const int n      = sh_degree >= 0 ? sh_count(sh_degree) : 0;
+  const int m1     = sh_rest ? 1 : n_sh;
+  float* my_row    = &s_rows[kStage ? threadIdx.x * kShStageStride : 0];
+  if (kStage && sh_degree >= 0) {
+    s_flag[threadIdx.x] = vis;
+    __syncthreads();
+    stage_sh_rows(s_rows, s_flag, blockIdx.x * blockDim.x, P, n, n_sh, shs, sh_rest);
+    __syncthreads();
   }
-  g_means3D[3 * (size_t) i] = gp[0], g_means3D[3 * (size_t) i + 1] = gp[1], g_means3D[3 * (size_t) i + 2] = gp[2];
-  g_scales[i] = make_float2(gs[0], gs[1]);
-  g_rot[i]    = make_float4(gq[0], gq[1], gq[2], gq[3]);
-  // densification proxy written over the incoming screen-space gradient (gs_2d_preprocess.cu:325-328)
-  const float depth = M[8];
-  grad_mean2D[i] = make_float2(gM_in2 * depth * 0.5f * (float) W, gM_in5 * depth * 0.5f * (float) H);
+
+  if (vis) {
+    float Tw2v[16], Tw2c[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) Tw2v[k] = s_Tw2v[k], Tw2c[k] = s_Tw2c[k];
+
+    const float4 gno = grad_normal_opacity[i];
+    g_opac[i]        = gno.w;
+    float gM[9], M[9], gM_in2, gM_in5;
+#pragma unroll
+    for (int k = 0; k < 9; ++k) gM[k] = grad_trans[9 * (size_t) i + k], M[k] = trans_mat[9 * (size_t) i + k];
+    gM_in2 = gM[2], gM_in5 = gM[5];
+    const float2 g2 = grad_mean2D[i];
+    bound_backward(M, g2.x, g2.y, gM);
+
+    const float4 q   = rotations[i];
+    const float p[3] = {means3D[3 * (size_t) i], means3D[3 * (size_t) i + 1], means3D[3 * (size_t) i + 2]};
+    const float t0 = 2 * (q.y * q.w + q.x * q.z), t1 = 2 * (q.y * q.z - q.x * q.w),
+                t2 = 1 - 2 * (q.x * q.x + q.y * q.y);
+    const float nrm[3] = {Tw2v[0] * t0 + Tw2v[1] * t1 + Tw2v[2] * t2, Tw2v[4] * t0 + Tw2v[5] * t1 + Tw2v[6] * t2,
+                          Tw2v[8] * t0 + Tw2v[9] * t1 + Tw2v[10] * t2};
+    const float pv[3] = {Tw2v[0] * p[0] + Tw2v[1] * p[1] + Tw2v[2] * p[2] + Tw2v[3],
+                         Tw2v[4] * p[0] + Tw2v[5] * p[1] + Tw2v[6] * p[2] + Tw2v[7],
+                         Tw2v[8] * p[0] + Tw2v[9] * p[1] + Tw2v[10] * p[2] + Tw2v[11]};
+    const float cosv = -(pv[0] * nrm[0] + pv[1] * nrm[1] + pv[2] * nrm[2]);
+    const float mult = cosv > 0 ? 1.0f : -1.0f;
+    const float gN[3] = {mult * gno.x, mult * gno.y, mult * gno.z};
+    const float2 s = scales[i];
+    float gp[3], gs[2], gq[4];
+    transmat_backward(W, H, s.x, s.y, q, Tw2c, Tw2v, gM, gN, gp, gs, gq);
+
+    if (sh_degree >= 0) {
+      float x, y, z, Y[kSh], tl[kSh];
+      const float nn = view_dir(p, campos, x, y, z);
+      sh_eval(sh_degree, x, y, z, Y);
+      float g[3];
+#pragma unroll
+      for (int c = 0; c < 3; ++c) g[c] = grad_colors[3 * (size_t) i + c] * (float) (colors[3 * (size_t) i + c] > 0);
+      // coefficient rows are read from LDS when staged, and each gradient row is written over the coefficients it
+      // was computed from (a lane only ever touches its own row)
+      const float* c0 = kStage ? my_row : shs + (size_t) i * m1 * 3;
+      const float* cr = kStage ? my_row : (sh_rest ? sh_rest + (size_t) i * n_sh * 3 - 3 : c0);
+      float* o0  = kStage ? my_row : (g_shs ? g_shs + (size_t) i * m1 * 3 : nullptr);
+      float* orr = kStage ? my_row
+                          : (sh_rest ? (g_sh_rest ? g_sh_rest + (size_t) i * n_sh * 3 - 3 : nullptr) : o0);
+      if (o0) o0[0] = g[0] * Y[0], o0[1] = g[1] * Y[0], o0[2] = g[2] * Y[0];
+      tl[0] = 0.0f;
+      for (int l = 1; l < n; ++l) {
+        tl[l] = g[0] * cr[3 * l] + g[1] * cr[3 * l + 1] + g[2] * cr[3 * l + 2];
+        if (orr) orr[3 * l] = g[0] * Y[l], orr[3 * l + 1] = g[1] * Y[l], orr[3 * l + 2] = g[2] * Y[l];
+      }
+      if (!kStage && orr) {  // coefficients above the active degree
+        for (int l = n; l < (sh_rest ? n_sh + 1 : n_sh); ++l)
+          orr[3 * l] = 0.0f, orr[3 * l + 1] = 0.0f, orr[3 * l + 2] = 0.0f;
+      }
+      float dx = 0, dy = 0, dz = 0;
+      sh_grad_accumulate(sh_degree, x, y, z, tl, dx, dy, dz);
+      const float vx = p[0] - campos[0], vy = p[1] - campos[1], vz = p[2] - campos[2];
+      const float tt = -(vx * dx + vy * dy + vz * dz) * nn * nn * nn;
+      gp[0] = gp[0] + (dx * nn + tt * vx);
+      gp[1] = gp[1] + (dy * nn + tt * vy);
+      gp[2] = gp[2] + (dz * nn + tt * vz);
+    }
+    g_means3D[3 * (size_t) i] = gp[0], g_means3D[3 * (size_t) i + 1] = gp[1], g_means3D[3 * (size_t) i + 2] = gp[2];
+    g_scales[i] = make_float2(gs[0], gs[1]);
+    g_rot[i]    = make_float4(gq[0], gq[1], gq[2], gq[3]);
+    // densification proxy written over the incoming screen-space gradient (gs_2d_preprocess.cu:325-328)
+    const float depth = M[8];
+    grad_mean2D[i] = make_float2(gM_in2 * depth * 0.5f * (float) W, gM_in5 * depth * 0.5f * (float) H);
+  } else if (valid) {
+    // rows of surfels that were not rendered get explicit zeros, so the outputs need no initialisation
+    g_opac[i] = 0.0f;
+    g_means3D[3 * (size_t) i] = 0.0f, g_means3D[3 * (size_t) i + 1] = 0.0f, g_means3D[3 * (size_t) i + 2] = 0.0f;
+    g_scales[i] = make_float2(0.0f, 0.0f);
+    g_rot[i]    = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (sh_degree >= 0) {
+      if (kStage) {
+        for (int c = 0; c < n * 3; ++c) my_row[c] = 0.0f;
+      } else {
+        if (g_shs)
+          for (int c = 0; c < m1 * 3; ++c) g_shs[(size_t) i * m1 * 3 + c] = 0.0f;
+        if (g_sh_rest)
+          for (int c = 0; c < n_sh * 3; ++c) g_sh_rest[(size_t) i * n_sh * 3 + c] = 0.0f;
+      }
+    }
+  }
+  if (kStage && sh_degree >= 0 && (g_shs || g_sh_rest)) {
+    __syncthreads();
+    unstage_sh_grads(s_rows, blockIdx.x * blockDim.x, P, n, n_sh, sh_rest != nullptr, g_shs, g_sh_rest);
+  }
 }
 
 __global__ void __launch_bounds__(256) transmat_forward_kernel(int P, int W, int H, const float* __restrict__ means3D,

@@ -1,0 +1,80 @@
+// Block-cooperative movement of per-surfel SH rows between HBM and LDS for the one-lane-per-surfel preprocess kernels.
+// A lane that walks its own 192-byte row touches one 128-byte line per instruction and relies on the caches to keep 96
+// lines per wavefront alive between touches; moving the block's rows with consecutive lanes on consecutive addresses
+// reads (writes) every line once. Used when the active degree is <= 3 (at most 16 coefficients, 48 floats per row).
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace fsgs {
+
+constexpr int kShStageRows   = 256;  // surfels per block
+constexpr int kShStageFloats = 48;   // 16 coefficients x rgb
+constexpr int kShStageStride = 49;   // odd stride: a lane reading its own row hits a different bank than its neighbours
+
+// e / d for 0 <= e < 2^20 and 1 <= d <= 256 without an integer division: (e + 0.5) / d is at least 0.5 / d away from any
+// integer, far more than the rounding error of the float product.
+__device__ __forceinline__ int small_div(int e, float inv_d) { return (int) (((float) e + 0.5f) * inv_d); }
+
+// Copies the first n coefficients (n * 3 floats) of every flagged row of the block into LDS. Row r of the block is
+// surfel block_base + r. With sh_rest the DC coefficient comes from shs[P,1,3] and the others from sh_rest[P,n_sh,3].
+__device__ __forceinline__ void stage_sh_rows(float* __restrict__ s_rows, const unsigned char* __restrict__ s_flag,
+                                              int block_base, int P, int n, int n_sh, const float* __restrict__ shs,
+                                              const float* __restrict__ sh_rest) {
+  const int per_row = n * 3;
+  const int rows    = min(kShStageRows, P - block_base);
+  if (sh_rest == nullptr) {
+    const size_t stride = (size_t) n_sh * 3;
+    const float inv     = 1.0f / (float) per_row;
+    for (int e = threadIdx.x; e < rows * per_row; e += blockDim.x) {
+      const int r = small_div(e, inv), c = e - r * per_row;
+      if (s_flag[r]) s_rows[r * kShStageStride + c] = shs[(size_t) (block_base + r) * stride + c];
+    }
+  } else {
+    for (int e = threadIdx.x; e < rows * 3; e += blockDim.x) {
+      const int r = e / 3, c = e - r * 3;
+      if (s_flag[r]) s_rows[r * kShStageStride + c] = shs[(size_t) (block_base + r) * 3 + c];
+    }
+    const int rest    = per_row - 3;
+    const size_t stride = (size_t) n_sh * 3;
+    const float inv     = 1.0f / (float) max(rest, 1);
+    for (int e = threadIdx.x; e < rows * rest; e += blockDim.x) {
+      const int r = small_div(e, inv), c = e - r * rest;
+      if (s_flag[r]) s_rows[r * kShStageStride + 3 + c] = sh_rest[(size_t) (block_base + r) * stride + c];
+    }
+  }
+}
+
+// Writes the block's staged gradient rows (n * 3 floats each, zeros where the owning lane stored zeros) to
+// g_shs / g_sh_rest and zero-fills the coefficients above the active degree, so the caller's tensors need no
+// initialisation. With the split layout (has_rest) either output may be absent.
+__device__ __forceinline__ void unstage_sh_grads(const float* __restrict__ s_rows, int block_base, int P, int n,
+                                                 int n_sh, bool has_rest, float* __restrict__ g_shs,
+                                                 float* __restrict__ g_sh_rest) {
+  const int rows = min(kShStageRows, P - block_base);
+  if (!has_rest) {
+    if (g_shs == nullptr) return;
+    const int per_row = n_sh * 3, live = n * 3;
+    const float inv   = 1.0f / (float) per_row;
+    for (int e = threadIdx.x; e < rows * per_row; e += blockDim.x) {
+      const int r = small_div(e, inv), c = e - r * per_row;
+      g_shs[(size_t) (block_base + r) * per_row + c] = c < live ? s_rows[r * kShStageStride + c] : 0.0f;
+    }
+    return;
+  }
+  if (g_shs != nullptr) {
+    for (int e = threadIdx.x; e < rows * 3; e += blockDim.x) {
+      const int r = e / 3, c = e - r * 3;
+      g_shs[(size_t) (block_base + r) * 3 + c] = s_rows[r * kShStageStride + c];
+    }
+  }
+  if (g_sh_rest != nullptr) {
+    const int per_row = n_sh * 3, live = n * 3 - 3;
+    const float inv   = 1.0f / (float) max(per_row, 1);
+    for (int e = threadIdx.x; e < rows * per_row; e += blockDim.x) {
+      const int r = small_div(e, inv), c = e - r * per_row;
+      g_sh_rest[(size_t) (block_base + r) * per_row + c] = c < live ? s_rows[r * kShStageStride + 3 + c] : 0.0f;
+    }
+  }
+}
+
+}  // namespace fsgs

@@ -97,11 +97,14 @@ class _GS_2D_Render(torch.autograd.Function):
         grad_colors, grad_means2D, grad_trans, grad_normal_opacity = _GS_2D_Render._render_backward(
             means2D, normal_opacity, colors, trans_mat, transe_mat_t2, pixel_opacity, pixel_extras, pixel_flow,
             grad_images, grad_opacity, grad_others, grad_flows, tile_range, point_list, n_contrib, near_n, far_n)
+        # the preprocess backward writes every row of its outputs (zeros for surfels that were not rendered), so they
+        # are allocated uninitialised; pre-computed colours (sh_degree < 0) receive no gradient, as in the reference
+        new = torch.empty_like
         grad_inputs = [
-            torch.zeros_like(means3D), torch.zeros_like(scales), torch.zeros_like(rotations),
-            torch.zeros_like(opacities),
-            torch.zeros_like(shs_or_colors) if ctx.needs_input_grad[4] else None,
-            torch.zeros_like(shs_rest) if shs_rest is not None and ctx.needs_input_grad[5] else None,
+            new(means3D), new(scales), new(rotations), new(opacities),
+            (new(shs_or_colors) if sh_degree >= 0 else torch.zeros_like(shs_or_colors))
+            if ctx.needs_input_grad[4] else None,
+            new(shs_rest) if shs_rest is not None and ctx.needs_input_grad[5] else None,
             None, None, None, None, None, None, None, None, None, None, grad_means2D, None, None, None, None, None,
         ]
         _GS_2D_Render._preprocess_backward(
@@ -172,8 +175,8 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
         grad_opacity = torch.zeros((H, W), dtype=torch.float32, device=dev)
     gc, gm2, gt, gno = f('GS_2D_render_backward')(m2, no, colors, tm, None, oo, oe, None, grad_image, grad_opacity,
                                                   grad_extras, None, ranges, point_list, nc, cam.near, cam.far)
-    g_means3D, g_scales = torch.zeros_like(scene.means3D), torch.zeros_like(scene.scales)
-    g_rot, g_opac, g_shs = torch.zeros_like(scene.rotations), torch.zeros_like(scene.opacities), torch.zeros_like(scene.shs)
+    g_means3D, g_scales = torch.empty_like(scene.means3D), torch.empty_like(scene.scales)
+    g_rot, g_opac, g_shs = torch.empty_like(scene.rotations), torch.empty_like(scene.opacities), torch.empty_like(scene.shs)
     f('gs_2d_preprocess_backward')(W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations,
                                    scene.opacities, scene.shs, None, cam.Tw2v, cam.Tv2c, cam.campos, tm, radii, colors,
                                    no, gm2, gt, None, gc, gno, g_means3D, g_scales, g_rot, g_opac, g_shs, None)

@@ -42,9 +42,11 @@ int fsgs_gs_2d_preprocess_forward(int P, int W, int H, int sh_degree, int n_sh, 
     int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* normal_opacity, float* depths,
     int32_t* radii, int32_t* tiles_touched, void* stream);
 
-/* gs_2d_preprocess_backward -- gs_2d_preprocess.cu:423-499 (kernel :268-329). Gradients of visible surfels are
- * ASSIGNED into g_* (the caller zero-fills them, as the reference's caller does); grad_mean2D[P,2] is read and then
- * overwritten in place with the densification proxy. g_shs / g_sh_rest may be NULL. */
+/* gs_2d_preprocess_backward -- gs_2d_preprocess.cu:423-499 (kernel :268-329). Every row of g_* is ASSIGNED: the
+ * gradient for surfels with radii > 0, zeros for the others and for SH coefficients above the active degree (the
+ * reference relies on its caller's zero-fill for those), so the outputs need no initialisation. grad_mean2D[P,2] is
+ * read and then overwritten in place with the densification proxy (rows with radii <= 0 are left as they are).
+ * g_shs / g_sh_rest may be NULL. */
 int fsgs_gs_2d_preprocess_backward(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
     const float* scales, const float* rotations, const float* shs, const float* sh_rest, const float* Tw2v,
     const float* Tv2c, const float* campos, const float* trans_mat, const int32_t* radii, const float* colors,
