@@ -18,6 +18,9 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+static bool g_culling_enabled = true;
+bool culling_enabled() { return g_culling_enabled; }
+
 namespace {
 // Plain streaming copy, 16 bytes per lane and grid-stride: the yardstick for achievable HBM bandwidth and the known-size
 // kernel against which hardware byte counters are calibrated.
@@ -39,6 +42,11 @@ FSGS_API int fsgs_copy_probe(const void* src, void* dst, size_t nbytes, void* st
   hipLaunchKernelGGL(fsgs::copy_probe_kernel, dim3((unsigned) (blocks < 16384 ? blocks : 16384)), dim3(256), 0,
                      (hipStream_t) stream, (const float4*) src, (float4*) dst, n);
   return fsgs::check_launch("copy_probe");
+}
+
+FSGS_API int fsgs_debug_set_culling(int enabled) {
+  fsgs::g_culling_enabled = enabled != 0;
+  return fsgs::kOk;
 }
 
 FSGS_API const char* fsgs_last_error() { return fsgs::last_error_buffer(); }

@@ -5,6 +5,10 @@
 
 namespace fsgs {
 
+// Launch flags of the blend kernels (see launch_tile_order).
+constexpr int kFlagOrdered = 1, kFlagNoCull = 2;
+bool culling_enabled();  // host-side switch, on by default
+
 constexpr int kBlendThreads = 256;  // one 16x16 tile per block = 4 wavefronts, each owning an 8x8 pixel quadrant
 constexpr int kBatch        = 256;  // surfels staged in LDS per round
 
@@ -92,34 +96,45 @@ __device__ __forceinline__ bool intersect(const SplatHot& h, float pxf, float py
 // ellipse u^2 + v^2 <= tau in the surfel's tangent plane; its exact screen-space bounding box follows from the same
 // homogeneous form the preprocess uses for its 3-sigma bound (gs_2d_preprocess.cu:125-156) with cutoff^2 = tau. The
 // pixels with rho2d <= tau are a disc of radius sqrt(tau / 2) around the screen-space centre. The union of both boxes,
-// padded by 1 pixel + 0.5 % of its extent against rounding, is tested against the four 8x8 quadrants of the tile; a
+// padded by 1/8 pixel + 0.5 % of its extent against rounding, is tested against the four 8x8 quadrants of the tile; a
 // clear bit means no pixel of that quadrant can pass the reference's alpha test, so skipping it changes nothing.
 // Surfels whose tau-ellipse reaches the camera plane (no finite box) keep all bits set.
-__device__ __forceinline__ unsigned quadrant_mask(const SplatHot& h, int tile_px, int tile_py) {
+#ifndef FSGS_CULL_PAD
+#define FSGS_CULL_PAD 0.125f
+#endif
+constexpr float kCullPad = FSGS_CULL_PAD;  // pixels added around the footprint box against rounding
+
+__device__ __forceinline__ unsigned quadrant_mask(const SplatHot& h, int tile_px, int tile_py, int flags) {
+  if (flags & kFlagNoCull) return 0xfu;
   const float oa = 255.0f * h.opacity;
   if (!(oa >= 1.0f)) return 0u;  // alpha can never reach 1/255
   const float tau = 2.0f * __logf(oa) * 1.0001f + 1e-3f;
+  // Work in coordinates relative to the screen-space centre: the box centre and half extents are differences of
+  // squares (c^2 - ...), which cancel catastrophically at pixel coordinates in the thousands but not near the origin.
+  const float ox = h.cx, oy = h.cy;
   float x0, x1, y0, y1;
   const float r2 = sqrtf(0.5f * tau);
-  x0 = h.cx - r2, x1 = h.cx + r2, y0 = h.cy - r2, y1 = h.cy + r2;
+  x0 = -r2, x1 = r2, y0 = -r2, y1 = r2;
   const float* M = h.m;
+  const float u0 = M[0] - ox * M[6], u1 = M[1] - ox * M[7], u2 = M[2] - ox * M[8];
+  const float v0 = M[3] - oy * M[6], v1 = M[4] - oy * M[7], v2 = M[5] - oy * M[8];
   const float d  = tau * (M[6] * M[6] + M[7] * M[7]) - M[8] * M[8];
   bool finite_box = (M[8] > 0.0f) && (d < -1e-6f * M[8] * M[8]);
   if (finite_box) {
     const float inv = 1.0f / d;
     const float f0 = tau * inv, f2 = -inv;
-    const float cx = f0 * (M[0] * M[6] + M[1] * M[7]) + f2 * (M[2] * M[8]);
-    const float cy = f0 * (M[3] * M[6] + M[4] * M[7]) + f2 * (M[5] * M[8]);
-    const float hx = cx * cx - (f0 * (M[0] * M[0] + M[1] * M[1]) + f2 * (M[2] * M[2]));
-    const float hy = cy * cy - (f0 * (M[3] * M[3] + M[4] * M[4]) + f2 * (M[5] * M[5]));
+    const float cx = f0 * (u0 * M[6] + u1 * M[7]) + f2 * (u2 * M[8]);
+    const float cy = f0 * (v0 * M[6] + v1 * M[7]) + f2 * (v2 * M[8]);
+    const float hx = cx * cx - (f0 * (u0 * u0 + u1 * u1) + f2 * (u2 * u2));
+    const float hy = cy * cy - (f0 * (v0 * v0 + v1 * v1) + f2 * (v2 * v2));
     const float ex = sqrtf(fmaxf(hx, 0.0f)), ey = sqrtf(fmaxf(hy, 0.0f));
     finite_box = (ex == ex) && (ey == ey) && (cx == cx) && (cy == cy);
     x0 = fminf(x0, cx - ex), x1 = fmaxf(x1, cx + ex);
     y0 = fminf(y0, cy - ey), y1 = fmaxf(y1, cy + ey);
   }
   if (!finite_box) return 0xfu;
-  const float padx = 1.0f + 0.005f * (x1 - x0), pady = 1.0f + 0.005f * (y1 - y0);
-  x0 -= padx, x1 += padx, y0 -= pady, y1 += pady;
+  const float padx = kCullPad + 0.005f * (x1 - x0), pady = kCullPad + 0.005f * (y1 - y0);
+  x0 += ox - padx, x1 += ox + padx, y0 += oy - pady, y1 += oy + pady;
   unsigned m = 0u;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
@@ -172,15 +187,17 @@ __global__ void __launch_bounds__(1024) tile_order_kernel(int T, const int64_t* 
   }
 }
 
-// Returns 1 when the table was built for this launch (T small enough), else 0 and blocks map to tiles directly.
+// Launch flags of the blend kernels: bit 0 = the tile table was built for this launch (T small enough; otherwise blocks
+// map to tiles directly), bit 1 = per-quadrant culling switched off (verification aid, see fsgs_debug_set_culling).
 inline int launch_tile_order(int T, const int64_t* ranges, hipStream_t s) {
-  if (T > kMaxOrderedTiles) return 0;
+  int flags = culling_enabled() ? 0 : kFlagNoCull;
+  if (T > kMaxOrderedTiles) return flags;
   hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, s, T, ranges);
-  return 1;
+  return flags | kFlagOrdered;
 }
 
-__device__ __forceinline__ int scheduled_tile(int ordered) {
-  return ordered ? g_tile_order[blockIdx.x] : (int) blockIdx.x;
+__device__ __forceinline__ int scheduled_tile(int flags) {
+  return (flags & kFlagOrdered) ? g_tile_order[blockIdx.x] : (int) blockIdx.x;
 }
 
 }  // namespace

@@ -120,7 +120,7 @@ blend_backward_kernel(
     if ((int) threadIdx.x < n_here) {
       s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
-      s_mask[threadIdx.x] = (unsigned char) quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile);
+      s_mask[threadIdx.x] = (unsigned char) quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile, ordered);
       if (kFlow)
 #pragma unroll
         for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];

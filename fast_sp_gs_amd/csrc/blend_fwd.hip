@@ -48,6 +48,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   const int rounds = (n_todo + kFwdBatch - 1) / kFwdBatch;
 
   bool done = !inside;
+  const float far_scale = far_n / (far_n - near_n);
   float T = 1.0f, C0 = 0, C1 = 0, C2 = 0;
   float N0 = 0, N1 = 0, N2 = 0, D = 0, M1 = 0, M2 = 0, dist = 0, median = 0, wsum = 0, f0 = 0, f1 = 0;
   int last = 0, median_c = -1, wmax_id = -1;
@@ -70,7 +71,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
     if ((int) threadIdx.x < n_here) {
       s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
-      s_mask[threadIdx.x] = (unsigned char) quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile);
+      s_mask[threadIdx.x] = (unsigned char) quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile, ordered);
       if (kFlow)
 #pragma unroll
         for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
@@ -106,7 +107,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
         const int contributor = b * kFwdBatch + j + 1;
         if (kAux) {
           const float A = 1.0f - T;
-          const float m = far_n / (far_n - near_n) * (1.0f - near_n / h.depth);
+          const float m = far_scale * (1.0f - near_n * __builtin_amdgcn_rcpf(h.depth));
           dist += (m * m * A + M2 - 2.0f * m * M1) * w;
           D += h.depth * w;
           M1 += m * w;

@@ -55,7 +55,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_topk_kernel(
       h.cx = c.x, h.cy = c.y, h.opacity = normal_opacity[id].w;
       s_hot[threadIdx.x]  = h;
       s_id[threadIdx.x]   = id;
-      s_mask[threadIdx.x] = (unsigned char) quadrant_mask(h, tile_x * kTile, tile_y * kTile);
+      s_mask[threadIdx.x] = (unsigned char) quadrant_mask(h, tile_x * kTile, tile_y * kTile, ordered);
     }
     __syncthreads();
     for (int c = 0; c < kBatch / kWave; ++c) {

@@ -53,13 +53,13 @@ __device__ __forceinline__ FastSplat gather_fast(int id, const float2* __restric
   return s;
 }
 
-__device__ __forceinline__ unsigned fast_quadrant_mask(const FastSplat& s, int tile_px, int tile_py) {
+__device__ __forceinline__ unsigned fast_quadrant_mask(const FastSplat& s, int tile_px, int tile_py, int flags) {
   SplatHot h;
 #pragma unroll
   for (int k = 0; k < 6; ++k) h.m[k] = s.m[k];
   h.m[6] = s.hot.tw0, h.m[7] = s.hot.tw1, h.m[8] = s.hot.tw2;
   h.cx = s.hot.cx, h.cy = s.hot.cy, h.opacity = s.hot.opacity;
-  return quadrant_mask(h, tile_px, tile_py);
+  return quadrant_mask(h, tile_px, tile_py, flags);
 }
 
 struct FastHit {
@@ -151,6 +151,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
   }
 
   bool done = !inside;
+  const float far_scale = far_n / (far_n - near_n);
   float T = 1.0f, C0 = 0, C1 = 0, C2 = 0;
   float N0 = 0, N1 = 0, N2 = 0, D = 0, M1 = 0, M2 = 0, dist = 0, median = 0;
   int last = 0, median_c = -1, wmax_id = -1;
@@ -167,7 +168,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
     if ((int) threadIdx.x < n_here) {
       s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
-      s_mask[threadIdx.x] = (unsigned char) fast_quadrant_mask(next, tile_x * kTile, tile_y * kTile);
+      s_mask[threadIdx.x] = (unsigned char) fast_quadrant_mask(next, tile_x * kTile, tile_y * kTile, ordered);
     }
     __syncthreads();
     const int nxt = (b + 1) * kBatch + (int) threadIdx.x;
@@ -218,7 +219,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
           const int contributor = b * kBatch + j + 1;
           if (kAux) {
             const float A = 1.0f - T;
-            const float m = far_n / (far_n - near_n) * (1.0f - near_n / h.depth);
+            const float m = far_scale * (1.0f - near_n * __builtin_amdgcn_rcpf(h.depth));
             dist += (m * m * A + M2 - 2.0f * m * M1) * w;
             D += h.depth * w;
             M1 += m * w;
@@ -354,7 +355,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
     if ((int) threadIdx.x < n_here) {
       s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
-      s_mask[threadIdx.x] = (unsigned char) fast_quadrant_mask(next, tile_x * kTile, tile_y * kTile);
+      s_mask[threadIdx.x] = (unsigned char) fast_quadrant_mask(next, tile_x * kTile, tile_y * kTile, ordered);
     }
     __syncthreads();
     const int nxt = (b + 1) * kBatch + (int) threadIdx.x;
