@@ -201,8 +201,9 @@ def gs_2d_compute_trans_mat_backward(W, H, means3D, scales, rotations, Tw2v, Tw2
 
 # --------------------------------------------------------------------------------------------------------------------
 def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, tiles_touched: Tensor,
-               debug: bool = False, return_keys: bool = False) -> List[Tensor]:
-    """gaussian_prepare.cu:282-308 -> [ranges[T,2] int64, point_list[R] int32]."""
+               debug: bool = False, return_keys: bool = False, return_offsets: bool = False) -> List[Tensor]:
+    """gaussian_prepare.cu:282-308 -> [ranges[T,2] int64, point_list[R] int32] (+ sorted keys, + the prefix scan of
+    tiles_touched, which GS_2D_render_backward can use to sum gradients without atomics)."""
     what = 'GS_prepare'
     _f32(what, means2D=means2D, depths=depths)
     L.require_cuda(what, radii=radii, tiles_touched=tiles_touched)
@@ -231,7 +232,12 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
     L.check(rc, what)
     if debug:
         torch.cuda.synchronize()
-    return [ranges, point_list, keys] if return_keys else [ranges, point_list]
+    out = [ranges, point_list]
+    if return_keys:
+        out.append(keys)
+    if return_offsets:
+        out.append(offsets)
+    return out
 
 
 # --------------------------------------------------------------------------------------------------------------------
@@ -279,18 +285,26 @@ def GS_2D_render_forward(width: int, height: int, means2D: Tensor, colors: Tenso
 
 def GS_2D_render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat2, out_opacity, out_others, out_flows,
                           dL_dout_color, dL_dout_opacity, dL_dothers, dL_dout_flows, ranges, point_list, n_contrib,
-                          near_n: float, far_n: float):
-    """gs_2d_redner.cu:631-717 -> (dL_dcolors[P,3], dL_dmeans2D[P,2], dL_dtrans_m[P,3,3], dL_dnorm_op[P,4])."""
+                          near_n: float, far_n: float, point_offsets: Optional[Tensor] = None,
+                          radii: Optional[Tensor] = None):
+    """gs_2d_redner.cu:631-717 -> (dL_dcolors[P,3], dL_dmeans2D[P,2], dL_dtrans_m[P,3,3], dL_dnorm_op[P,4]).
+    With `point_offsets` (GS_prepare(..., return_offsets=True)) and `radii` the per-surfel sums are taken in a fixed
+    order from per-instance records instead of with atomics."""
     what = 'GS_2D_render_backward'
     L.require_cuda(what, dL_dout_color=dL_dout_color, dL_dout_opacity=dL_dout_opacity, dL_dothers=dL_dothers,
-                   dL_dout_flows=dL_dout_flows)
+                   dL_dout_flows=dL_dout_flows, point_offsets=point_offsets, radii=radii)
     P = means2D.shape[0]
     H, W = dL_dout_color.shape[1], dL_dout_color.shape[2]
+    R = int(point_list.numel())
     opt = dict(dtype=torch.float32, device=out_opacity.device)
-    # one zero-fill for the four accumulated outputs; every segment starts on a 16-byte boundary
+    ordered = point_offsets is not None and P > 0
+    if ordered and radii is None:
+        raise RuntimeError(f'{what}: radii is required together with point_offsets')
+    # the four outputs share one allocation; every segment starts on a 16-byte boundary. The atomic path accumulates
+    # into them (one zero-fill), the ordered path writes every row itself.
     up = lambda n: (n + 3) // 4 * 4
     o1, o2, o3 = up(4 * P), up(4 * P) + up(9 * P), up(4 * P) + up(9 * P) + up(3 * P)
-    flat = torch.zeros((o3 + 2 * P,), **opt)
+    flat = (torch.empty if ordered else torch.zeros)((o3 + 2 * P,), **opt)
     g_norm_op = flat[:4 * P].view(P, 4)
     g_trans = flat[o1:o1 + 9 * P].view(P, 3, 3)
     g_colors = flat[o2:o2 + 3 * P].view(P, 3)
@@ -303,13 +317,21 @@ def GS_2D_render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat2
                                                                 c(dL_dothers), c(dL_dout_flows))
     ranges, point_list, n_contrib = c(ranges), c(point_list), c(n_contrib)
     use_aux = out_others is not None and dL_dothers is not None
+    lib = _lib()
+    ws = None
+    if ordered:
+        L.require_dtype(what, 'point_offsets', point_offsets, torch.int64)
+        L.require_dtype(what, 'radii', radii, torch.int32)
+        ws = _workspace(lib.fsgs_gs_2d_render_backward_workspace_bytes(R), out_opacity.device)
     with _timed('gs_2d_render_backward'):
-        rc = _lib().fsgs_gs_2d_render_backward(
+        rc = lib.fsgs_gs_2d_render_backward(
             P, W, H, float(near_n), float(far_n), L.ptr(means2D), L.ptr(normal_opacity), L.ptr(colors), L.ptr(trans_mat),
             L.ptr(trans_mat2), L.ptr(out_opacity), L.ptr(out_others) if use_aux else None,
             L.ptr(out_flows) if dL_dout_flows is not None else None, L.ptr(dL_dout_color), L.ptr(dL_dout_opacity),
             L.ptr(dL_dothers) if use_aux else None, L.ptr(dL_dout_flows), L.ptr(ranges), L.ptr(point_list),
-            L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_norm_op), L.current_stream())
+            L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_norm_op), R,
+            L.ptr(point_offsets) if ordered else None, L.ptr(radii) if ordered else None, L.ptr(ws),
+            ws.numel() if ws is not None else 0, L.current_stream())
     L.check(rc, what)
     return g_colors, g_means2D, g_trans, g_norm_op
 

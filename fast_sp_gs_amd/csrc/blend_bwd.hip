@@ -11,6 +11,8 @@
 //   2. adds the 4 wavefront partials of a tile into an LDS accumulator of the staged batch, and
 //   3. flushes one global atomic per surfel, component and tile when the batch retires.
 // Surfels behind the deepest contributor of the whole tile are never gathered.
+#include <algorithm>
+
 #include "blend.hpp"
 
 namespace fsgs {
@@ -28,7 +30,7 @@ constexpr int kGradSlots = 18;
 #endif
 constexpr int kBwdBatch = FSGS_BWD_BATCH;  // surfels staged per round (<= block size)
 
-template <bool kAux, bool kFlow>
+template <bool kAux, bool kFlow, bool kSlots>
 __global__ void __launch_bounds__(kBlendThreads) __attribute__((amdgpu_waves_per_eu(FSGS_BWD_WAVES, FSGS_BWD_WAVES)))
 blend_backward_kernel(
     int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
@@ -37,15 +39,17 @@ blend_backward_kernel(
     const float* __restrict__ trans_mat_t2, const float* __restrict__ out_opacity, const float* __restrict__ out_extras,
     const float2* __restrict__ out_flow, const float* __restrict__ dL_dpix, const float* __restrict__ dL_dextras,
     const float* __restrict__ dL_dopacity, const float2* __restrict__ dL_dflow, float* __restrict__ g_means2D,
-    float* __restrict__ g_normal_opacity, float* __restrict__ g_colors, float* __restrict__ g_trans) {
+    float* __restrict__ g_normal_opacity, float* __restrict__ g_colors, float* __restrict__ g_trans,
+    const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii, float* __restrict__ slot_grads) {
   __shared__ SplatHot s_hot[kBwdBatch];
   __shared__ SplatCold s_cold[kBwdBatch];
   __shared__ float s_acc[kBwdBatch][kGradSlots + 1];  // +1: odd stride keeps the flush conflict free
+  __shared__ int s_slot[kSlots ? kBwdBatch : 1];      // where this (surfel, tile) instance sits in surfel order
   __shared__ float s_t2[kFlow ? kBwdBatch * 9 : 1];
   __shared__ int s_max_contrib;
   __shared__ unsigned char s_mask[kBwdBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
 
-  const int gx = (W + kTile - 1) / kTile;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
@@ -108,11 +112,17 @@ blend_backward_kernel(
 
   Splat next;
   float next_t2[9];
+  int next_radius = 0;
+  int64_t next_off = 0;
   if ((int) threadIdx.x < min(n_todo, kBwdBatch)) {
     next = gather_splat(point_list[r0 + (n_todo - 1 - (int) threadIdx.x)], means2D, colors, normal_opacity, trans_mat);
     if (kFlow)
 #pragma unroll
       for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
+    if (kSlots) {
+      next_radius = radii[next.cold.id];
+      next_off    = next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1];
+    }
   }
 
   for (int b = 0; b < rounds; ++b) {
@@ -124,6 +134,12 @@ blend_backward_kernel(
       if (kFlow)
 #pragma unroll
         for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
+      if (kSlots) {
+        // position of this instance in the surfel-ordered key list: the binning emits a surfel's tiles row-major
+        // over its rectangle, starting at the surfel's prefix-scan offset (gaussian_prepare.cu:47-83)
+        const TileRect r = tile_rect(next.hot.cx, next.hot.cy, next_radius, gx, gy);
+        s_slot[threadIdx.x] = (int) (next_off + (int64_t) (tile_y - r.y0) * (r.x1 - r.x0) + (tile_x - r.x0));
+      }
     }
     __syncthreads();
     const int nxt = (b + 1) * kBwdBatch + (int) threadIdx.x;
@@ -132,6 +148,10 @@ blend_backward_kernel(
       if (kFlow)
 #pragma unroll
         for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
+      if (kSlots) {
+        next_radius = radii[next.cold.id];
+        next_off    = next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1];
+      }
     }
 
     // Work list of this wavefront for 64 staged surfels at a time: those that can reach its quadrant and are not
@@ -235,22 +255,36 @@ blend_backward_kernel(
      }
     }
     __syncthreads();
-    // flush the batch: one global atomic per surfel and component for this tile
+    // flush the batch
     if ((int) threadIdx.x < n_here) {
-      const int id = s_cold[threadIdx.x].id;
-      float* a     = s_acc[threadIdx.x];
+      float* a = s_acc[threadIdx.x];
+      if (kSlots) {
+        // one 72-byte record per (surfel, tile) instance at the instance's position in surfel order; the per-surfel
+        // sums are taken afterwards by slot_reduce_kernel. Records nobody contributed to stay at their zero fill.
+        bool any = false;
 #pragma unroll
-      for (int c = 0; c < 3; ++c)
-        if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
+        for (int c = 0; c < kGradSlots; ++c) any |= a[c] != 0.0f;
+        if (any) {
+          float2* dst = (float2*) (slot_grads + (size_t) s_slot[threadIdx.x] * kGradSlots);
 #pragma unroll
-      for (int c = 0; c < 9; ++c)
-        if (a[3 + c] != 0.0f) atomicAdd(&g_trans[9 * (size_t) id + c], a[3 + c]);
+          for (int c = 0; c < kGradSlots / 2; ++c) dst[c] = make_float2(a[2 * c], a[2 * c + 1]);
+        }
+      } else {
+        // one global atomic per surfel and component for this tile
+        const int id = s_cold[threadIdx.x].id;
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        if (a[12 + c] != 0.0f) atomicAdd(&g_normal_opacity[4 * (size_t) id + c], a[12 + c]);
+        for (int c = 0; c < 3; ++c)
+          if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
-        if (a[16 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[16 + c]);
+        for (int c = 0; c < 9; ++c)
+          if (a[3 + c] != 0.0f) atomicAdd(&g_trans[9 * (size_t) id + c], a[3 + c]);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (a[12 + c] != 0.0f) atomicAdd(&g_normal_opacity[4 * (size_t) id + c], a[12 + c]);
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+          if (a[16 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[16 + c]);
+      }
 #pragma unroll
       for (int c = 0; c < kGradSlots; ++c) a[c] = 0.0f;
     }
@@ -259,17 +293,62 @@ blend_backward_kernel(
   }
 }
 
+// Zero fill of the per-instance gradient records (float4 stores).
+__global__ void __launch_bounds__(256) slot_fill_kernel(size_t n4, float4* __restrict__ p) {
+  for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t) gridDim.x * blockDim.x)
+    p[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+}
+
+// Per-surfel sums of the instance records. Nine lanes per surfel, each owning one float2 of the 18-float record, so
+// the lanes of a surfel read 72 contiguous bytes per step and neighbouring surfels continue where the previous one
+// ends. Every row of the four outputs is written (zeros for surfels without instances): no initialisation, no atomics,
+// and the sum order is fixed.
+__global__ void __launch_bounds__(256) slot_reduce_kernel(int P, const int64_t* __restrict__ point_offsets,
+    const int32_t* __restrict__ radii, const float* __restrict__ slot_grads, float* __restrict__ g_colors,
+    float* __restrict__ g_means2D, float* __restrict__ g_trans, float* __restrict__ g_normal_opacity) {
+  constexpr int kPerWave = 7, kLanes = 9;  // 63 of 64 lanes busy
+  const int lane = threadIdx.x & 63;
+  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int sub = lane / kLanes, k = lane - sub * kLanes;
+  const int i   = wave * kPerWave + sub;
+  if (sub >= kPerWave || i >= P) return;
+  float2 acc = make_float2(0.0f, 0.0f);
+  if (radii[i] > 0) {
+    const int64_t e0 = i == 0 ? 0 : point_offsets[i - 1], e1 = point_offsets[i];
+    const float2* src = (const float2*) slot_grads + k;
+    for (int64_t e = e0; e < e1; ++e) {
+      const float2 v = src[(size_t) e * kLanes];
+      acc.x += v.x, acc.y += v.y;
+    }
+  }
+  // record layout: 0-2 colours | 3-11 trans_mat | 12-14 normal | 15 opacity | 16-17 means2D
+  const float vals[2] = {acc.x, acc.y};
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int c = 2 * k + h;
+    if (c < 3) g_colors[3 * (size_t) i + c] = vals[h];
+    else if (c < 12) g_trans[9 * (size_t) i + (c - 3)] = vals[h];
+    else if (c < 16) g_normal_opacity[4 * (size_t) i + (c - 12)] = vals[h];
+    else g_means2D[2 * (size_t) i + (c - 16)] = vals[h];
+  }
+}
+
 }  // namespace
 }  // namespace fsgs
 
 using namespace fsgs;
+
+FSGS_API size_t fsgs_gs_2d_render_backward_workspace_bytes(int64_t R) {
+  return align_up((size_t) (R > 0 ? R : 0) * kGradSlots * 4 + 16, 256);
+}
 
 FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n, const float* means2D,
     const float* normal_opacity, const float* colors, const float* trans_mat, const float* trans_mat_t2,
     const float* out_opacity, const float* out_extras, const float* out_flow, const float* dL_dpix,
     const float* dL_dopacity, const float* dL_dextras, const float* dL_dflow, const int64_t* ranges,
     const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
-    float* g_normal_opacity, void* stream) {
+    float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
+    size_t workspace_bytes, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_render_backward: bad sizes");
   if (P == 0) return kOk;
   FSGS_REQUIRE(means2D && normal_opacity && colors && trans_mat && out_opacity && dL_dpix && dL_dopacity && ranges &&
@@ -279,19 +358,43 @@ FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, doub
   const bool flow = dL_dflow != nullptr;
   FSGS_REQUIRE(!flow || (trans_mat_t2 && out_flow && aux),
                "GS_2D_render_backward: flow gradients need trans_mat_t2, out_flow and the auxiliary maps");
+  const bool slots = point_offsets != nullptr;
+  if (slots) {
+    FSGS_REQUIRE(radii && workspace && R >= 0 && R < (int64_t) 0x7fffffff,
+                 "GS_2D_render_backward: the ordered-sum path needs radii, a workspace and the instance count R");
+    if (workspace_bytes < fsgs_gs_2d_render_backward_workspace_bytes(R))
+      return fail(kWorkspaceSmall, "GS_2D_render_backward: workspace %zu < %zu bytes", workspace_bytes,
+                  fsgs_gs_2d_render_backward_workspace_bytes(R));
+  }
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
+  float* slot_grads = slots ? (float*) workspace : nullptr;
+  if (slots) {
+    const size_t n4 = ((size_t) R * kGradSlots + 3) / 4;
+    if (n4 > 0)
+      hipLaunchKernelGGL(slot_fill_kernel, dim3((unsigned) std::min<size_t>((n4 + 255) / 256, 8192)), dim3(256), 0, s,
+                         n4, (float4*) slot_grads);
+  }
   const int ordered = launch_tile_order(gx * gy, ranges, s);
-#define FSGS_LAUNCH_BWD(AUX, FLOW)                                                                                   \
-  hipLaunchKernelGGL((blend_backward_kernel<AUX, FLOW>), grid, block, 0, s, ordered, W, H, (float) near_n, (float) far_n,     \
-                     ranges, point_list, n_contrib, (const float2*) means2D, (const float4*) normal_opacity, colors, \
-                     trans_mat, trans_mat_t2, out_opacity, out_extras, (const float2*) out_flow, dL_dpix,            \
-                     dL_dextras, dL_dopacity, (const float2*) dL_dflow, g_means2D, g_normal_opacity, g_colors,       \
-                     g_trans)
-  if (aux && flow) FSGS_LAUNCH_BWD(true, true);
-  else if (aux) FSGS_LAUNCH_BWD(true, false);
-  else FSGS_LAUNCH_BWD(false, false);
+#define FSGS_LAUNCH_BWD(AUX, FLOW, SLOTS)                                                                            \
+  hipLaunchKernelGGL((blend_backward_kernel<AUX, FLOW, SLOTS>), grid, block, 0, s, ordered, W, H, (float) near_n,    \
+                     (float) far_n, ranges, point_list, n_contrib, (const float2*) means2D,                          \
+                     (const float4*) normal_opacity, colors, trans_mat, trans_mat_t2, out_opacity, out_extras,       \
+                     (const float2*) out_flow, dL_dpix, dL_dextras, dL_dopacity, (const float2*) dL_dflow,           \
+                     g_means2D, g_normal_opacity, g_colors, g_trans, point_offsets, radii, slot_grads)
+  if (slots) {
+    if (aux && flow) FSGS_LAUNCH_BWD(true, true, true);
+    else if (aux) FSGS_LAUNCH_BWD(true, false, true);
+    else FSGS_LAUNCH_BWD(false, false, true);
+    const int waves = div_up(P, 7);
+    hipLaunchKernelGGL(slot_reduce_kernel, dim3(div_up((int64_t) waves * 64, 256)), dim3(256), 0, s, P, point_offsets,
+                       radii, slot_grads, g_colors, g_means2D, g_trans, g_normal_opacity);
+  } else {
+    if (aux && flow) FSGS_LAUNCH_BWD(true, true, false);
+    else if (aux) FSGS_LAUNCH_BWD(true, false, false);
+    else FSGS_LAUNCH_BWD(false, false, false);
+  }
 #undef FSGS_LAUNCH_BWD
   return check_launch("GS_2D_render_backward");
 }

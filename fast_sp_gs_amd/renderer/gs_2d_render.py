@@ -69,14 +69,15 @@ class _GS_2D_Render(torch.autograd.Function):
         means2D, colors, trans_mat, normal_opacity, depths, radii, tiles_touched = _GS_2D_Render._preprocess_forward(
             W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c,
             campos, trans_precomp, means2D, culling)
-        tile_range, point_list = GS_prepare(W, H, means2D, depths, radii, tiles_touched, False)
+        tile_range, point_list, point_offsets = GS_prepare(W, H, means2D, depths, radii, tiles_touched, False,
+                                                           return_offsets=True)
         pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib = _GS_2D_Render._render_forward(
             W, H, means2D, colors, normal_opacity, trans_mat, point_list, tile_range, near_n, far_n, only_image,
             transe_mat_t2, accum_max_count, accum_weights_p, accum_weights_count)
         ctx._info = (W, H, sh_degree, is_opengl, near_n, far_n)
         ctx.save_for_backward(means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, campos,
                               means2D, trans_mat, transe_mat_t2, radii, colors, normal_opacity, tile_range,
-                              point_list, pixel_extras, pixel_opacity, pixel_flow, n_contrib)
+                              point_list, pixel_extras, pixel_opacity, pixel_flow, n_contrib, point_offsets)
         buffer = RasterizeBuffer(int(W), int(H), means3D.shape[0], point_list.shape[0], near_n, far_n, tile_range,
                                  point_list, n_contrib, means2D, normal_opacity, trans_mat)
         ctx.mark_non_differentiable(n_contrib, radii)
@@ -87,7 +88,7 @@ class _GS_2D_Render(torch.autograd.Function):
     def backward(ctx, *grad_outputs):
         (means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, campos, means2D, trans_mat,
          transe_mat_t2, radii, colors, normal_opacity, tile_range, point_list, pixel_extras, pixel_opacity, pixel_flow,
-         n_contrib) = ctx.saved_tensors
+         n_contrib, point_offsets) = ctx.saved_tensors
         W, H, sh_degree, is_opengl, near_n, far_n = ctx._info
         grad_images, grad_opacity, grad_others, grad_flows = grad_outputs[:4]
         if grad_images is None:
@@ -96,7 +97,8 @@ class _GS_2D_Render(torch.autograd.Function):
             grad_opacity = torch.zeros((H, W), dtype=torch.float32, device=means3D.device)
         grad_colors, grad_means2D, grad_trans, grad_normal_opacity = _GS_2D_Render._render_backward(
             means2D, normal_opacity, colors, trans_mat, transe_mat_t2, pixel_opacity, pixel_extras, pixel_flow,
-            grad_images, grad_opacity, grad_others, grad_flows, tile_range, point_list, n_contrib, near_n, far_n)
+            grad_images, grad_opacity, grad_others, grad_flows, tile_range, point_list, n_contrib, near_n, far_n,
+            point_offsets, radii)
         # the preprocess backward writes every row of its outputs (zeros for surfels that were not rendered), so they
         # are allocated uninitialised; pre-computed colours (sh_degree < 0) receive no gradient, as in the reference
         new = torch.empty_like
@@ -156,7 +158,8 @@ def GS_2D_topk_weights(topk: int, buffer: RasterizeBuffer) -> Tuple[Tensor, Tens
               buffer.trans_mat, buffer.tile_ranges, buffer.point_list)
 
 
-def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad_opacity: Tensor = None):
+def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad_opacity: Tensor = None,
+                ordered_sums: bool = True):
     """One forward + backward pass of the hot path on raw operators (no autograd graph): preprocess -> binning ->
     blend -> blend backward -> preprocess backward, in the order `_GS_2D_Render` runs them. Returns a dict with every
     intermediate so callers (benchmark, parity tests) can inspect or time the stages."""
@@ -166,7 +169,7 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
     m2, colors, tm, no, depths, radii, tt = f('gs_2d_preprocess_forward')(
         W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs, None,
         cam.Tw2v, cam.Tv2c, cam.campos, None, None, None)
-    ranges, point_list = f('GS_prepare')(W, H, m2, depths, radii, tt, False)
+    ranges, point_list, offsets = f('GS_prepare')(W, H, m2, depths, radii, tt, False, return_offsets=True)
     oc, oo, oe, of, nc = f('GS_2D_render_forward')(W, H, m2, colors, no, tm, point_list, ranges, cam.near, cam.far,
                                                    False, None, None, None, None)
     if grad_extras is None:
@@ -174,7 +177,8 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
     if grad_opacity is None:
         grad_opacity = torch.zeros((H, W), dtype=torch.float32, device=dev)
     gc, gm2, gt, gno = f('GS_2D_render_backward')(m2, no, colors, tm, None, oo, oe, None, grad_image, grad_opacity,
-                                                  grad_extras, None, ranges, point_list, nc, cam.near, cam.far)
+                                                  grad_extras, None, ranges, point_list, nc, cam.near, cam.far,
+                                                  offsets if ordered_sums else None, radii)
     g_means3D, g_scales = torch.empty_like(scene.means3D), torch.empty_like(scene.scales)
     g_rot, g_opac, g_shs = torch.empty_like(scene.rotations), torch.empty_like(scene.opacities), torch.empty_like(scene.shs)
     f('gs_2d_preprocess_backward')(W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations,

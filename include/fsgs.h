@@ -92,14 +92,23 @@ int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, double far_n, 
     float* accum_weights_p, int32_t* accum_weights_count, float* out_color, float* out_opacity, float* out_extras,
     float* out_flow, int32_t* n_contrib, void* stream);
 
-/* GS_2D_render_backward -- gs_2d_redner.cu:631-717 (kernel :238-539). g_colors[P,3] g_means2D[P,2] g_trans[P,3,3]
- * g_normal_opacity[P,4] MUST be zero-filled by the caller; gradients are accumulated into them. */
+/* GS_2D_render_backward -- gs_2d_redner.cu:631-717 (kernel :238-539). Two ways of summing a surfel's gradient over the
+ * tiles it touches:
+ *  - point_offsets == NULL: device-scope float atomics, as the reference does; g_colors[P,3] g_means2D[P,2]
+ *    g_trans[P,3,3] g_normal_opacity[P,4] MUST be zero-filled by the caller.
+ *  - point_offsets[P] (the prefix scan fsgs_gs_prepare_scan produced for this point_list) with radii[P], R and a workspace
+ *    of fsgs_gs_2d_render_backward_workspace_bytes(R): every (surfel, tile) instance writes one record at its position
+ *    in surfel order and a second kernel sums each surfel's records in a fixed order. No atomics to HBM, the four outputs
+ *    are fully written (no initialisation needed). Requires the point_list of fsgs_gs_prepare_fill for these means2D /
+ *    radii (the position of an instance is recomputed from the surfel's tile rectangle). */
+size_t fsgs_gs_2d_render_backward_workspace_bytes(int64_t R);
 int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n, const float* means2D,
     const float* normal_opacity, const float* colors, const float* trans_mat, const float* trans_mat_t2,
     const float* out_opacity, const float* out_extras, const float* out_flow, const float* dL_dpix,
     const float* dL_dopacity, const float* dL_dextras, const float* dL_dflow, const int64_t* ranges,
     const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
-    float* g_normal_opacity, void* stream);
+    float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
+    size_t workspace_bytes, void* stream);
 
 /* ---- "fast" surfel path: transform through camera intrinsics Tv2s[3,3], adjugate-based intersection, fused
  * corner-test binning. Flow outputs are not supported on this path. ---- */

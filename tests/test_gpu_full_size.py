@@ -4,7 +4,8 @@
     of the reordered atomic sums;
   * binning invariants: sorted masked keys, ranges partition [0, R) in tile order, every entry carries its tile's id;
   * the blend weights accumulated per surfel sum to the opacity image;
-  * the backward is linear in the upstream gradients;
+  * the backward is linear in the upstream gradients, and its two ways of summing a surfel's gradient over tiles
+    (per-instance records summed in order / device-scope atomics) agree;
   * K-NN at 3M x 2048, k = 8: distances ascending, equal to the distance recomputed from the returned index, and no
     closer control point exists for a sample of queries (brute force with torch).
 Sizes: 300 000 surfels at 800x800, 3 000 000 surfels at 1352x1014 (one view), 400 000 surfels at 3840x2160.
@@ -21,9 +22,9 @@ def _culling(enabled):
     lib.check(lib.load().fsgs_debug_set_culling(int(enabled)), 'debug_set_culling')
 
 
-def _render(scene, cam, gi, ge, go):
+def _render(scene, cam, gi, ge, go, ordered_sums=True):
     from fast_sp_gs_amd.renderer import render_step
-    out = render_step(scene, cam, gi, ge, go)
+    out = render_step(scene, cam, gi, ge, go, ordered_sums=ordered_sums)
     torch.cuda.synchronize()
     return out
 
@@ -85,6 +86,12 @@ def test_render_path_properties(config, device):
     for k in ('g_colors', 'g_trans', 'g_normal_opacity', 'g_means3D', 'g_scales', 'g_rot', 'g_opac', 'g_shs'):
         ref = b[k].abs().max().clamp_min(1e-30)
         assert float((a[k] - b[k]).abs().max() / ref) < 2e-5, k
+
+    # per-surfel sums through per-instance records (default) == device-scope atomics
+    d = _render(scene, cam, gi, ge, go, ordered_sums=False)
+    for k in ('g_colors', 'g_trans', 'g_normal_opacity', 'g_means2D', 'g_means3D', 'g_scales', 'g_rot', 'g_opac', 'g_shs'):
+        ref = a[k].abs().max().clamp_min(1e-30)
+        assert float((a[k] - d[k]).abs().max() / ref) < 2e-5, k
 
     # accumulated blend weights == opacity image (both are the sum of alpha * T over blended pairs)
     acc = torch.zeros(scene.P, device=device)
