@@ -63,6 +63,7 @@ def algorithmic_bytes(stage: str, P: int, Pv: int, R: int, T: int, HW: int) -> i
         'gs_2d_render_forward': 76 * R + 16 * T + 60 * HW,
         'gs_2d_render_backward': 76 * R + 16 * T + 60 * HW + 72 * (P + Pv),
         'gs_2d_preprocess_backward': 4 * P + Pv * (352 + 240),
+        'gs_2d_pack_records': P * (72 + 12 + 80),  # optional packed per-surfel records: read 4 tensors, write 80 B
     }
     return int(table[stage])
 

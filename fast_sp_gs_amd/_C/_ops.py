@@ -19,7 +19,7 @@ __all__ = [
     'gs_2d_compute_trans_mat_backward', 'GS_prepare', 'GS_2D_render_forward', 'GS_2D_render_backward',
     'SH_to_RGB_forward', 'SH_to_RGB_backward', 'sh_encode_forward', 'sh_encode_backward', 'freq_encode_forward',
     'freq_encode_backward', 'cdist_top', 'cdist_top_backward', 'AdamMasksedUpdated', 'knn_topk', 'lbs_blend',
-    'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'gs_2d_fast_preprocess_forward',
+    'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'gs_2d_pack_records', 'gs_2d_fast_preprocess_forward',
     'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward', 'gs_2d_fast_compute_trans_mat_backward',
     'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward',
 ]
@@ -245,8 +245,9 @@ def GS_2D_render_forward(width: int, height: int, means2D: Tensor, colors: Tenso
                          trans_mat: Tensor, point_list: Tensor, ranges: Tensor, near_n: float, far_n: float,
                          only_image: bool, trans_mat_t2: Optional[Tensor] = None,
                          accum_max_count: Optional[Tensor] = None, accum_weights_p: Optional[Tensor] = None,
-                         accum_weights_count: Optional[Tensor] = None):
-    """gs_2d_redner.cu:541-629 -> (colors[3,H,W], opacity[H,W], extras[9,H,W]|None, flow[H,W,2]|None, n_contrib)."""
+                         accum_weights_count: Optional[Tensor] = None, records: Optional[Tensor] = None):
+    """gs_2d_redner.cu:541-629 -> (colors[3,H,W], opacity[H,W], extras[9,H,W]|None, flow[H,W,2]|None, n_contrib).
+    `records` (gs_2d_pack_records) is an optional packed copy of the per-surfel inputs."""
     what = 'GS_2D_render_forward'
     _f32(what, colors=colors, trans_mat=trans_mat, means2D=means2D, normal_opacity=normal_opacity,
          trans_mat_t2=trans_mat_t2, accum_weights_p=accum_weights_p)
@@ -278,15 +279,40 @@ def GS_2D_render_forward(width: int, height: int, means2D: Tensor, colors: Tenso
             P, width, height, float(near_n), float(far_n), int(bool(only_image)), L.ptr(means2D), L.ptr(colors),
             L.ptr(normal_opacity), L.ptr(trans_mat), L.ptr(point_list), L.ptr(ranges), L.ptr(trans_mat_t2),
             L.ptr(accum_max_count), L.ptr(accum_weights_p), L.ptr(accum_weights_count), L.ptr(pixel_colors),
-            L.ptr(pixel_opacity), L.ptr(pixel_extras), L.ptr(pixel_flow), L.ptr(n_contrib), L.current_stream())
+            L.ptr(pixel_opacity), L.ptr(pixel_extras), L.ptr(pixel_flow), L.ptr(n_contrib), L.ptr(records),
+            L.current_stream())
     L.check(rc, what)
     return pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib
+
+
+def gs_2d_pack_records(means2D: Tensor, colors: Tensor, normal_opacity: Tensor, trans_mat: Tensor,
+                       radii: Optional[Tensor] = None, point_offsets: Optional[Tensor] = None) -> Tensor:
+    """-> records[P,20]: one 80-byte record per surfel with everything the blend kernels gather (no reference
+    counterpart; optional input of GS_2D_render_forward / GS_2D_render_backward)."""
+    what = 'gs_2d_pack_records'
+    _f32(what, means2D=means2D, colors=colors, normal_opacity=normal_opacity, trans_mat=trans_mat)
+    L.require_cuda(what, radii=radii, point_offsets=point_offsets)
+    P = means2D.shape[0]
+    L.require_shape(what, 'colors', colors, P, 3)
+    L.require_shape(what, 'normal_opacity', normal_opacity, P, 4)
+    L.require_shape(what, 'trans_mat', trans_mat, P, 3, 3)
+    if radii is not None:
+        L.require_dtype(what, 'radii', radii, torch.int32)
+    if point_offsets is not None:
+        L.require_dtype(what, 'point_offsets', point_offsets, torch.int64)
+    records = torch.empty((P, 20), dtype=torch.float32, device=means2D.device)
+    with _timed(what):
+        rc = _lib().fsgs_gs_2d_pack_records(P, L.ptr(means2D.contiguous()), L.ptr(colors.contiguous()),
+                                            L.ptr(normal_opacity.contiguous()), L.ptr(trans_mat.contiguous()),
+                                            L.ptr(radii), L.ptr(point_offsets), L.ptr(records), L.current_stream())
+    L.check(rc, what)
+    return records
 
 
 def GS_2D_render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat2, out_opacity, out_others, out_flows,
                           dL_dout_color, dL_dout_opacity, dL_dothers, dL_dout_flows, ranges, point_list, n_contrib,
                           near_n: float, far_n: float, point_offsets: Optional[Tensor] = None,
-                          radii: Optional[Tensor] = None):
+                          radii: Optional[Tensor] = None, records: Optional[Tensor] = None):
     """gs_2d_redner.cu:631-717 -> (dL_dcolors[P,3], dL_dmeans2D[P,2], dL_dtrans_m[P,3,3], dL_dnorm_op[P,4]).
     With `point_offsets` (GS_prepare(..., return_offsets=True)) and `radii` the per-surfel sums are taken in a fixed
     order from per-instance records instead of with atomics."""
@@ -331,7 +357,7 @@ def GS_2D_render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat2
             L.ptr(dL_dothers) if use_aux else None, L.ptr(dL_dout_flows), L.ptr(ranges), L.ptr(point_list),
             L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_norm_op), R,
             L.ptr(point_offsets) if ordered else None, L.ptr(radii) if ordered else None, L.ptr(ws),
-            ws.numel() if ws is not None else 0, L.current_stream())
+            ws.numel() if ws is not None else 0, L.ptr(records), L.current_stream())
     L.check(rc, what)
     return g_colors, g_means2D, g_trans, g_norm_op
 

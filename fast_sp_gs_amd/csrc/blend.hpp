@@ -31,11 +31,35 @@ struct Splat {
   SplatCold cold;
 };
 
+// Optional packed copy of everything the blend kernels gather per surfel: one 80-byte, 16-byte-aligned record
+// (five float4) instead of four tensors, i.e. one or two 128-byte lines per list entry instead of four to six.
+//   q0 = M0 M1 M2 M3 | q1 = M4 M5 M6 M7 | q2 = M8 cx cy opacity | q3 = nx ny nz r | q4 = g b radius(int) offset(int)
+// radius / offset (prefix scan of tiles_touched before this surfel) are only meaningful when the packer was given them.
+constexpr int kRecordFloats = 20;
+
+struct SplatExtra {
+  int radius;
+  int64_t offset;
+};
+
 __device__ __forceinline__ Splat gather_splat(int id, const float2* __restrict__ means2D,
                                               const float* __restrict__ colors,
                                               const float4* __restrict__ normal_opacity,
-                                              const float* __restrict__ trans_mat) {
+                                              const float* __restrict__ trans_mat,
+                                              const float4* __restrict__ records, SplatExtra* extra = nullptr) {
   Splat s;
+  if (records != nullptr) {
+    const float4* r = records + 5 * (size_t) id;
+    const float4 q0 = r[0], q1 = r[1], q2 = r[2], q3 = r[3], q4 = r[4];
+    s.hot.m[0] = q0.x, s.hot.m[1] = q0.y, s.hot.m[2] = q0.z, s.hot.m[3] = q0.w;
+    s.hot.m[4] = q1.x, s.hot.m[5] = q1.y, s.hot.m[6] = q1.z, s.hot.m[7] = q1.w;
+    s.hot.m[8] = q2.x, s.hot.cx = q2.y, s.hot.cy = q2.z, s.hot.opacity = q2.w;
+    s.cold.nx = q3.x, s.cold.ny = q3.y, s.cold.nz = q3.z, s.cold.r = q3.w;
+    s.cold.g = q4.x, s.cold.b = q4.y;
+    s.cold.id = id, s.cold.pad = 0;
+    if (extra) extra->radius = __float_as_int(q4.z), extra->offset = __float_as_int(q4.w);
+    return s;
+  }
   const float* M = trans_mat + 9 * (size_t) id;
 #pragma unroll
   for (int k = 0; k < 9; ++k) s.hot.m[k] = M[k];
@@ -144,14 +168,18 @@ __device__ __forceinline__ unsigned quadrant_mask(const SplatHot& h, int tile_px
   return m;
 }
 
-// ---- longest-list-first tile schedule -------------------------------------------------------------------------------
-// Blocks are handed to the CUs in blockIdx order, and a tile's cost is proportional to the length of its list, so the
-// blend kernels map blockIdx -> tile through a table that lists tiles by descending list length (quarter-octave
-// buckets, arbitrary order inside a bucket). The long lists start first and the short ones fill the tail of the launch.
+// ---- tile schedule: longest lists first, neighbouring tiles on the same XCD -----------------------------------------
+// Blocks are handed out in blockIdx order, consecutive blocks go to consecutive XCDs (8 of them, each with its own L2),
+// and a tile's cost is proportional to the length of its list. The blend kernels therefore map blockIdx -> tile through
+// a table built per launch: small square groups of tiles are dealt to 8 regions, region r owns the table positions p with
+// p % 8 == r (as long as it has tiles left), and inside a region tiles are listed by descending list length
+// (quarter-octave buckets, arbitrary order inside a bucket). Long lists start first and short ones fill the tail of the launch; a surfel
+// that overlaps several neighbouring tiles is gathered by blocks that share an L2.
 // The table lives in a file-scope device array (one copy per translation unit that includes this header): calls that
 // overlap on different streams would race on it, so the blend entry points must be issued on one stream at a time.
 constexpr int kMaxOrderedTiles = 1 << 16;
 constexpr int kOrderBuckets    = 128;
+constexpr int kOrderRegions    = 8;
 
 namespace {
 
@@ -165,34 +193,54 @@ __device__ __forceinline__ int length_bucket(int64_t len64) {
   return 1 + m * 4 + frac;  // <= 124
 }
 
-__global__ void __launch_bounds__(1024) tile_order_kernel(int T, const int64_t* __restrict__ ranges) {
-  __shared__ int s_count[kOrderBuckets];
-  for (int b = threadIdx.x; b < kOrderBuckets; b += blockDim.x) s_count[b] = 0;
+#ifndef FSGS_TILE_GROUP
+#define FSGS_TILE_GROUP 2
+#endif
+// Groups of FSGS_TILE_GROUP x FSGS_TILE_GROUP tiles are dealt to the 8 regions in a skewed pattern, so every region is a
+// fine-grained sample of the whole image (equal load whatever the scene's layout) while direct neighbours mostly share
+// a region.
+__device__ __forceinline__ int tile_region(int t, int gx, int gy) {
+  const int tx = t % gx, ty = t / gx;
+  (void) gy;
+  return ((tx / FSGS_TILE_GROUP) + 3 * (ty / FSGS_TILE_GROUP)) & (kOrderRegions - 1);
+}
+
+__global__ void __launch_bounds__(1024) tile_order_kernel(int gx, int gy, const int64_t* __restrict__ ranges) {
+  __shared__ int s_count[kOrderRegions][kOrderBuckets];
+  __shared__ int s_total[kOrderRegions];
+  const int T = gx * gy;
+  for (int b = threadIdx.x; b < kOrderRegions * kOrderBuckets; b += blockDim.x) (&s_count[0][0])[b] = 0;
   __syncthreads();
   for (int t = threadIdx.x; t < T; t += blockDim.x)
-    atomicAdd(&s_count[length_bucket(ranges[2 * (size_t) t + 1] - ranges[2 * (size_t) t])], 1);
+    atomicAdd(&s_count[tile_region(t, gx, gy)][length_bucket(ranges[2 * (size_t) t + 1] - ranges[2 * (size_t) t])], 1);
   __syncthreads();
-  if (threadIdx.x == 0) {  // exclusive prefix from the longest bucket down
+  if (threadIdx.x < kOrderRegions) {  // exclusive prefix from the longest bucket down, per region
     int run = 0;
     for (int b = kOrderBuckets - 1; b >= 0; --b) {
-      const int c = s_count[b];
-      s_count[b]  = run;
+      const int c = s_count[threadIdx.x][b];
+      s_count[threadIdx.x][b] = run;
       run += c;
     }
+    s_total[threadIdx.x] = run;
   }
   __syncthreads();
   for (int t = threadIdx.x; t < T; t += blockDim.x) {
-    const int pos     = atomicAdd(&s_count[length_bucket(ranges[2 * (size_t) t + 1] - ranges[2 * (size_t) t])], 1);
+    const int r = tile_region(t, gx, gy);
+    const int k = atomicAdd(&s_count[r][length_bucket(ranges[2 * (size_t) t + 1] - ranges[2 * (size_t) t])], 1);
+    // position of the k-th tile of region r when the regions are dealt round-robin, skipping exhausted ones
+    int pos = 0;
+#pragma unroll
+    for (int q = 0; q < kOrderRegions; ++q) pos += min(s_total[q], k) + ((q < r && s_total[q] > k) ? 1 : 0);
     g_tile_order[pos] = t;
   }
 }
 
 // Launch flags of the blend kernels: bit 0 = the tile table was built for this launch (T small enough; otherwise blocks
 // map to tiles directly), bit 1 = per-quadrant culling switched off (verification aid, see fsgs_debug_set_culling).
-inline int launch_tile_order(int T, const int64_t* ranges, hipStream_t s) {
+inline int launch_tile_order(int gx, int gy, const int64_t* ranges, hipStream_t s) {
   int flags = culling_enabled() ? 0 : kFlagNoCull;
-  if (T > kMaxOrderedTiles) return flags;
-  hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, s, T, ranges);
+  if ((int64_t) gx * gy > kMaxOrderedTiles) return flags;
+  hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, s, gx, gy, ranges);
   return flags | kFlagOrdered;
 }
 

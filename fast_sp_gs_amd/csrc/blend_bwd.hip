@@ -40,7 +40,8 @@ blend_backward_kernel(
     const float2* __restrict__ out_flow, const float* __restrict__ dL_dpix, const float* __restrict__ dL_dextras,
     const float* __restrict__ dL_dopacity, const float2* __restrict__ dL_dflow, float* __restrict__ g_means2D,
     float* __restrict__ g_normal_opacity, float* __restrict__ g_colors, float* __restrict__ g_trans,
-    const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii, float* __restrict__ slot_grads) {
+    const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii, float* __restrict__ slot_grads,
+    const float4* __restrict__ records) {
   __shared__ SplatHot s_hot[kBwdBatch];
   __shared__ SplatCold s_cold[kBwdBatch];
   __shared__ float s_acc[kBwdBatch][kGradSlots + 1];  // +1: odd stride keeps the flush conflict free
@@ -115,13 +116,18 @@ blend_backward_kernel(
   int next_radius = 0;
   int64_t next_off = 0;
   if ((int) threadIdx.x < min(n_todo, kBwdBatch)) {
-    next = gather_splat(point_list[r0 + (n_todo - 1 - (int) threadIdx.x)], means2D, colors, normal_opacity, trans_mat);
+    SplatExtra ex;
+    next = gather_splat(point_list[r0 + (n_todo - 1 - (int) threadIdx.x)], means2D, colors, normal_opacity, trans_mat,
+                        records, &ex);
     if (kFlow)
 #pragma unroll
       for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
     if (kSlots) {
-      next_radius = radii[next.cold.id];
-      next_off    = next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1];
+      if (records) next_radius = ex.radius, next_off = ex.offset;
+      else {
+        next_radius = radii[next.cold.id];
+        next_off    = next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1];
+      }
     }
   }
 
@@ -144,13 +150,18 @@ blend_backward_kernel(
     __syncthreads();
     const int nxt = (b + 1) * kBwdBatch + (int) threadIdx.x;
     if ((int) threadIdx.x < kBwdBatch && nxt < n_todo) {
-      next = gather_splat(point_list[r0 + (n_todo - 1 - nxt)], means2D, colors, normal_opacity, trans_mat);
+      SplatExtra ex;
+      next = gather_splat(point_list[r0 + (n_todo - 1 - nxt)], means2D, colors, normal_opacity, trans_mat, records,
+                          &ex);
       if (kFlow)
 #pragma unroll
         for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
       if (kSlots) {
-        next_radius = radii[next.cold.id];
-        next_off    = next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1];
+        if (records) next_radius = ex.radius, next_off = ex.offset;
+        else {
+          next_radius = radii[next.cold.id];
+          next_off    = next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1];
+        }
       }
     }
 
@@ -348,7 +359,7 @@ FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, doub
     const float* dL_dopacity, const float* dL_dextras, const float* dL_dflow, const int64_t* ranges,
     const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
     float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
-    size_t workspace_bytes, void* stream) {
+    size_t workspace_bytes, const float* records, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_render_backward: bad sizes");
   if (P == 0) return kOk;
   FSGS_REQUIRE(means2D && normal_opacity && colors && trans_mat && out_opacity && dL_dpix && dL_dopacity && ranges &&
@@ -358,6 +369,7 @@ FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, doub
   const bool flow = dL_dflow != nullptr;
   FSGS_REQUIRE(!flow || (trans_mat_t2 && out_flow && aux),
                "GS_2D_render_backward: flow gradients need trans_mat_t2, out_flow and the auxiliary maps");
+  FSGS_REQUIRE(((uintptr_t) records & 15) == 0, "GS_2D_render_backward: records must be 16-byte aligned");
   const bool slots = point_offsets != nullptr;
   if (slots) {
     FSGS_REQUIRE(radii && workspace && R >= 0 && R < (int64_t) 0x7fffffff,
@@ -376,13 +388,14 @@ FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, doub
       hipLaunchKernelGGL(slot_fill_kernel, dim3((unsigned) std::min<size_t>((n4 + 255) / 256, 8192)), dim3(256), 0, s,
                          n4, (float4*) slot_grads);
   }
-  const int ordered = launch_tile_order(gx * gy, ranges, s);
+  const int ordered = launch_tile_order(gx, gy, ranges, s);
 #define FSGS_LAUNCH_BWD(AUX, FLOW, SLOTS)                                                                            \
   hipLaunchKernelGGL((blend_backward_kernel<AUX, FLOW, SLOTS>), grid, block, 0, s, ordered, W, H, (float) near_n,    \
                      (float) far_n, ranges, point_list, n_contrib, (const float2*) means2D,                          \
                      (const float4*) normal_opacity, colors, trans_mat, trans_mat_t2, out_opacity, out_extras,       \
                      (const float2*) out_flow, dL_dpix, dL_dextras, dL_dopacity, (const float2*) dL_dflow,           \
-                     g_means2D, g_normal_opacity, g_colors, g_trans, point_offsets, radii, slot_grads)
+                     g_means2D, g_normal_opacity, g_colors, g_trans, point_offsets, radii, slot_grads,               \
+                     (const float4*) records)
   if (slots) {
     if (aux && flow) FSGS_LAUNCH_BWD(true, true, true);
     else if (aux) FSGS_LAUNCH_BWD(true, false, true);

@@ -24,7 +24,8 @@ template <bool kAux, bool kFlow, bool kAccum>
 __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
     int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const float2* __restrict__ means2D, const float* __restrict__ colors, const float* __restrict__ trans_mat,
-    const float4* __restrict__ normal_opacity, const float* __restrict__ trans_mat_t2, int32_t* __restrict__ n_contrib,
+    const float4* __restrict__ normal_opacity, const float4* __restrict__ records,
+    const float* __restrict__ trans_mat_t2, int32_t* __restrict__ n_contrib,
     float* __restrict__ out_color, float* __restrict__ out_opacity, float* __restrict__ out_extras,
     float2* __restrict__ out_flow, int32_t* __restrict__ accum_max_count, float* __restrict__ accum_weights_p,
     int32_t* __restrict__ accum_weights_count) {
@@ -58,7 +59,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   Splat next;
   float next_t2[9];
   if ((int) threadIdx.x < min(n_todo, kFwdBatch)) {
-    next = gather_splat(point_list[r0 + threadIdx.x], means2D, colors, normal_opacity, trans_mat);
+    next = gather_splat(point_list[r0 + threadIdx.x], means2D, colors, normal_opacity, trans_mat, records);
     if (kFlow)
 #pragma unroll
       for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
@@ -79,7 +80,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
     __syncthreads();
     const int nxt = (b + 1) * kFwdBatch + threadIdx.x;
     if ((int) threadIdx.x < kFwdBatch && nxt < n_todo) {
-      next = gather_splat(point_list[r0 + nxt], means2D, colors, normal_opacity, trans_mat);
+      next = gather_splat(point_list[r0 + nxt], means2D, colors, normal_opacity, trans_mat, records);
       if (kFlow)
 #pragma unroll
         for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
@@ -165,20 +166,52 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   }
 }
 
+__global__ void __launch_bounds__(256) pack_records_kernel(int P, const float2* __restrict__ means2D,
+    const float* __restrict__ colors, const float4* __restrict__ normal_opacity, const float* __restrict__ trans_mat,
+    const int32_t* __restrict__ radii, const int64_t* __restrict__ point_offsets, float4* __restrict__ records) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= P) return;
+  const float* M  = trans_mat + 9 * (size_t) i;
+  const float2 c  = means2D[i];
+  const float4 no = normal_opacity[i];
+  const float* rgb = colors + 3 * (size_t) i;
+  const int radius  = radii ? radii[i] : 0;
+  const int offset  = point_offsets ? (i == 0 ? 0 : (int) point_offsets[i - 1]) : 0;
+  float4* r = records + 5 * (size_t) i;
+  r[0] = make_float4(M[0], M[1], M[2], M[3]);
+  r[1] = make_float4(M[4], M[5], M[6], M[7]);
+  r[2] = make_float4(M[8], c.x, c.y, no.w);
+  r[3] = make_float4(no.x, no.y, no.z, rgb[0]);
+  r[4] = make_float4(rgb[1], rgb[2], __int_as_float(radius), __int_as_float(offset));
+}
+
 }  // namespace
 }  // namespace fsgs
 
 using namespace fsgs;
 
+FSGS_API int fsgs_gs_2d_pack_records(int P, const float* means2D, const float* colors, const float* normal_opacity,
+    const float* trans_mat, const int32_t* radii, const int64_t* point_offsets, float* records, void* stream) {
+  FSGS_REQUIRE(P >= 0, "gs_2d_pack_records: bad size");
+  if (P == 0) return kOk;
+  FSGS_REQUIRE(means2D && colors && normal_opacity && trans_mat && records && ((uintptr_t) records & 15) == 0,
+               "gs_2d_pack_records: null or misaligned pointer");
+  hipLaunchKernelGGL(pack_records_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P,
+                     (const float2*) means2D, colors, (const float4*) normal_opacity, trans_mat, radii, point_offsets,
+                     (float4*) records);
+  return check_launch("gs_2d_pack_records");
+}
+
 FSGS_API int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, double far_n, int only_image,
     const float* means2D, const float* colors, const float* normal_opacity, const float* trans_mat,
     const int32_t* point_list, const int64_t* ranges, const float* trans_mat_t2, int32_t* accum_max_count,
     float* accum_weights_p, int32_t* accum_weights_count, float* out_color, float* out_opacity, float* out_extras,
-    float* out_flow, int32_t* n_contrib, void* stream) {
+    float* out_flow, int32_t* n_contrib, const float* records, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_render_forward: bad sizes");
   FSGS_REQUIRE(ranges && out_color && out_opacity && n_contrib, "GS_2D_render_forward: null pointer");
-  FSGS_REQUIRE(P == 0 || (means2D && colors && normal_opacity && trans_mat),
+  FSGS_REQUIRE(P == 0 || records || (means2D && colors && normal_opacity && trans_mat),
                "GS_2D_render_forward: null surfel tensor");
+  FSGS_REQUIRE(((uintptr_t) records & 15) == 0, "GS_2D_render_forward: records must be 16-byte aligned");
   FSGS_REQUIRE(only_image || out_extras, "GS_2D_render_forward: out_extras is required unless only_image");
   const bool aux   = !only_image;
   const bool flow  = aux && trans_mat_t2 != nullptr;
@@ -187,11 +220,11 @@ FSGS_API int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, doubl
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
-  const int ordered = launch_tile_order(gx * gy, ranges, s);
+  const int ordered = launch_tile_order(gx, gy, ranges, s);
 #define FSGS_LAUNCH_FWD(AUX, FLOW, ACC)                                                                              \
   hipLaunchKernelGGL((blend_forward_kernel<AUX, FLOW, ACC>), grid, block, 0, s, ordered, W, H, (float) near_n, (float) far_n, \
                      ranges, point_list, (const float2*) means2D, colors, trans_mat, (const float4*) normal_opacity, \
-                     trans_mat_t2, n_contrib, out_color, out_opacity, out_extras, (float2*) out_flow,                \
+                     (const float4*) records, trans_mat_t2, n_contrib, out_color, out_opacity, out_extras, (float2*) out_flow,                \
                      accum_max_count, accum_weights_p, accum_weights_count)
   if (!aux) FSGS_LAUNCH_FWD(false, false, false);
   else if (flow && accum) FSGS_LAUNCH_FWD(true, true, true);

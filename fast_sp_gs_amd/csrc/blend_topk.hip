@@ -129,7 +129,7 @@ FSGS_API int fsgs_gs_2d_topk_weights(int topk, int P, int W, int H, double near_
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
-  const int ordered = launch_tile_order(gx * gy, ranges, s);
+  const int ordered = launch_tile_order(gx, gy, ranges, s);
 #define FSGS_TOPK(KK)                                                                                            \
   hipLaunchKernelGGL((blend_topk_kernel<KK>), grid, block, 0, s, ordered, W, H, topk, (float) near_n, ranges, point_list, \
                      (const float2*) means2D, trans_mat, (const float4*) normal_opacity, top_indices, top_weights)

@@ -494,7 +494,7 @@ FSGS_API int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, 
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
-  const int ordered = launch_tile_order(gx * gy, ranges, s);
+  const int ordered = launch_tile_order(gx, gy, ranges, s);
 #define FSGS_LAUNCH_FWD(AUX, SNAP, ACC)                                                                              \
   hipLaunchKernelGGL((fast_blend_forward_kernel<AUX, SNAP, ACC>), grid, block, 0, s, ordered, W, H, (float) near_n,           \
                      (float) far_n, ranges, point_list, (const float2*) means2D, colors, trans_mat, inverse_m,       \
@@ -525,7 +525,7 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
-  const int ordered = launch_tile_order(gx * gy, ranges, s);
+  const int ordered = launch_tile_order(gx, gy, ranges, s);
 #define FSGS_LAUNCH_BWD(AUX, SPLAT)                                                                                  \
   hipLaunchKernelGGL((fast_blend_backward_kernel<AUX, SPLAT>), grid, block, 0, s, ordered, W, H, (float) near_n,              \
                      (float) far_n, ranges, point_list, n_contrib, (const float2*) means2D,                          \

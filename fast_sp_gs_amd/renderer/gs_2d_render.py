@@ -60,6 +60,7 @@ class _GS_2D_Render(torch.autograd.Function):
     _preprocess_backward = get_C_function('gs_2d_preprocess_backward')
     _render_forward = get_C_function('GS_2D_render_forward')
     _render_backward = get_C_function('GS_2D_render_backward')
+    _pack_records = get_C_function('gs_2d_pack_records')
 
     @staticmethod
     def forward(ctx, means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, campos, size,
@@ -71,13 +72,14 @@ class _GS_2D_Render(torch.autograd.Function):
             campos, trans_precomp, means2D, culling)
         tile_range, point_list, point_offsets = GS_prepare(W, H, means2D, depths, radii, tiles_touched, False,
                                                            return_offsets=True)
+        records = _GS_2D_Render._pack_records(means2D, colors, normal_opacity, trans_mat, radii, point_offsets)
         pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib = _GS_2D_Render._render_forward(
             W, H, means2D, colors, normal_opacity, trans_mat, point_list, tile_range, near_n, far_n, only_image,
-            transe_mat_t2, accum_max_count, accum_weights_p, accum_weights_count)
+            transe_mat_t2, accum_max_count, accum_weights_p, accum_weights_count, records)
         ctx._info = (W, H, sh_degree, is_opengl, near_n, far_n)
         ctx.save_for_backward(means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, campos,
                               means2D, trans_mat, transe_mat_t2, radii, colors, normal_opacity, tile_range,
-                              point_list, pixel_extras, pixel_opacity, pixel_flow, n_contrib, point_offsets)
+                              point_list, pixel_extras, pixel_opacity, pixel_flow, n_contrib, point_offsets, records)
         buffer = RasterizeBuffer(int(W), int(H), means3D.shape[0], point_list.shape[0], near_n, far_n, tile_range,
                                  point_list, n_contrib, means2D, normal_opacity, trans_mat)
         ctx.mark_non_differentiable(n_contrib, radii)
@@ -88,7 +90,7 @@ class _GS_2D_Render(torch.autograd.Function):
     def backward(ctx, *grad_outputs):
         (means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, campos, means2D, trans_mat,
          transe_mat_t2, radii, colors, normal_opacity, tile_range, point_list, pixel_extras, pixel_opacity, pixel_flow,
-         n_contrib, point_offsets) = ctx.saved_tensors
+         n_contrib, point_offsets, records) = ctx.saved_tensors
         W, H, sh_degree, is_opengl, near_n, far_n = ctx._info
         grad_images, grad_opacity, grad_others, grad_flows = grad_outputs[:4]
         if grad_images is None:
@@ -98,7 +100,7 @@ class _GS_2D_Render(torch.autograd.Function):
         grad_colors, grad_means2D, grad_trans, grad_normal_opacity = _GS_2D_Render._render_backward(
             means2D, normal_opacity, colors, trans_mat, transe_mat_t2, pixel_opacity, pixel_extras, pixel_flow,
             grad_images, grad_opacity, grad_others, grad_flows, tile_range, point_list, n_contrib, near_n, far_n,
-            point_offsets, radii)
+            point_offsets, radii, records)
         # the preprocess backward writes every row of its outputs (zeros for surfels that were not rendered), so they
         # are allocated uninitialised; pre-computed colours (sh_degree < 0) receive no gradient, as in the reference
         new = torch.empty_like
@@ -159,7 +161,7 @@ def GS_2D_topk_weights(topk: int, buffer: RasterizeBuffer) -> Tuple[Tensor, Tens
 
 
 def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad_opacity: Tensor = None,
-                ordered_sums: bool = True):
+                ordered_sums: bool = True, packed: bool = True):
     """One forward + backward pass of the hot path on raw operators (no autograd graph): preprocess -> binning ->
     blend -> blend backward -> preprocess backward, in the order `_GS_2D_Render` runs them. Returns a dict with every
     intermediate so callers (benchmark, parity tests) can inspect or time the stages."""
@@ -170,15 +172,16 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
         W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs, None,
         cam.Tw2v, cam.Tv2c, cam.campos, None, None, None)
     ranges, point_list, offsets = f('GS_prepare')(W, H, m2, depths, radii, tt, False, return_offsets=True)
+    rec = f('gs_2d_pack_records')(m2, colors, no, tm, radii, offsets) if packed else None
     oc, oo, oe, of, nc = f('GS_2D_render_forward')(W, H, m2, colors, no, tm, point_list, ranges, cam.near, cam.far,
-                                                   False, None, None, None, None)
+                                                   False, None, None, None, None, rec)
     if grad_extras is None:
         grad_extras = torch.zeros((9, H, W), dtype=torch.float32, device=dev)
     if grad_opacity is None:
         grad_opacity = torch.zeros((H, W), dtype=torch.float32, device=dev)
     gc, gm2, gt, gno = f('GS_2D_render_backward')(m2, no, colors, tm, None, oo, oe, None, grad_image, grad_opacity,
                                                   grad_extras, None, ranges, point_list, nc, cam.near, cam.far,
-                                                  offsets if ordered_sums else None, radii)
+                                                  offsets if ordered_sums else None, radii, rec)
     g_means3D, g_scales = torch.empty_like(scene.means3D), torch.empty_like(scene.scales)
     g_rot, g_opac, g_shs = torch.empty_like(scene.rotations), torch.empty_like(scene.opacities), torch.empty_like(scene.shs)
     f('gs_2d_preprocess_backward')(W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations,

@@ -83,6 +83,14 @@ int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, const float*
 
 /* ---- per-tile alpha blend ------------------------------------------------------------------------------------- */
 
+/* Optional accelerator without a counterpart in the reference: packs what the blend kernels gather per surfel
+ * (trans_mat, means2D, opacity, normal, colour, and -- when given -- radius and prefix-scan offset) into one 80-byte
+ * record, records[P,20] floats, 16-byte aligned. Passing `records` to fsgs_gs_2d_render_forward / _backward makes them
+ * read one record per list entry instead of four tensors; results are identical. Pass radii and point_offsets here if
+ * the backward is going to use its ordered-sum path. */
+int fsgs_gs_2d_pack_records(int P, const float* means2D, const float* colors, const float* normal_opacity,
+    const float* trans_mat, const int32_t* radii, const int64_t* point_offsets, float* records, void* stream);
+
 /* GS_2D_render_forward -- fast_2d_gs/_C/src/gaussian_splatting/gs_2d_redner.cu:541-629 (kernel :28-236).
  * out_color[3,H,W] out_opacity[H,W] n_contrib[2,H,W]; unless only_image: out_extras[9,H,W]; with trans_mat_t2:
  * out_flow[H,W,2]. accum_* [P] are accumulated into (atomics), all other outputs are fully written. */
@@ -90,7 +98,7 @@ int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, double far_n, 
     const float* means2D, const float* colors, const float* normal_opacity, const float* trans_mat,
     const int32_t* point_list, const int64_t* ranges, const float* trans_mat_t2, int32_t* accum_max_count,
     float* accum_weights_p, int32_t* accum_weights_count, float* out_color, float* out_opacity, float* out_extras,
-    float* out_flow, int32_t* n_contrib, void* stream);
+    float* out_flow, int32_t* n_contrib, const float* records, void* stream);
 
 /* GS_2D_render_backward -- gs_2d_redner.cu:631-717 (kernel :238-539). Two ways of summing a surfel's gradient over the
  * tiles it touches:
@@ -108,7 +116,7 @@ int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n,
     const float* dL_dopacity, const float* dL_dextras, const float* dL_dflow, const int64_t* ranges,
     const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
     float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
-    size_t workspace_bytes, void* stream);
+    size_t workspace_bytes, const float* records, void* stream);
 
 /* ---- "fast" surfel path: transform through camera intrinsics Tv2s[3,3], adjugate-based intersection, fused
  * corner-test binning. Flow outputs are not supported on this path. ---- */

@@ -22,9 +22,9 @@ def _culling(enabled):
     lib.check(lib.load().fsgs_debug_set_culling(int(enabled)), 'debug_set_culling')
 
 
-def _render(scene, cam, gi, ge, go, ordered_sums=True):
+def _render(scene, cam, gi, ge, go, ordered_sums=True, packed=True):
     from fast_sp_gs_amd.renderer import render_step
-    out = render_step(scene, cam, gi, ge, go, ordered_sums=ordered_sums)
+    out = render_step(scene, cam, gi, ge, go, ordered_sums=ordered_sums, packed=packed)
     torch.cuda.synchronize()
     return out
 
@@ -88,7 +88,10 @@ def test_render_path_properties(config, device):
         assert float((a[k] - b[k]).abs().max() / ref) < 2e-5, k
 
     # per-surfel sums through per-instance records (default) == device-scope atomics
-    d = _render(scene, cam, gi, ge, go, ordered_sums=False)
+    # ... and gathering from the packed per-surfel records (default) == gathering from the four tensors
+    d = _render(scene, cam, gi, ge, go, ordered_sums=False, packed=False)
+    for k in ('image', 'opacity', 'extras', 'n_contrib'):
+        assert torch.equal(a[k], d[k]), f"{k} depends on the packed records"
     for k in ('g_colors', 'g_trans', 'g_normal_opacity', 'g_means2D', 'g_means3D', 'g_scales', 'g_rot', 'g_opac', 'g_shs'):
         ref = a[k].abs().max().clamp_min(1e-30)
         assert float((a[k] - d[k]).abs().max() / ref) < 2e-5, k
