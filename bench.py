@@ -96,12 +96,91 @@ def cpu_baseline(scene, cam, budget_s: float = 20.0):
                       f"host has {os.cpu_count()} logical cpus"}
 
 
+def _ssim(img1, img2):
+    """Plain PyTorch SSIM (11x11 Gaussian window, sigma 1.5, C1 = 0.01^2, C2 = 0.03^2), the reference's fallback form
+    (losses/ssim.py:49-67); the fused SSIM kernel is not part of this build."""
+    import torch.nn.functional as F
+    k = torch.arange(11, dtype=torch.float32, device=img1.device) - 5
+    g = torch.exp(-k * k / (2 * 1.5 ** 2))
+    g = (g / g.sum())
+    w = (g[:, None] * g[None, :]).expand(3, 1, 11, 11).contiguous()
+    a, b = img1[None], img2[None]
+    mu1, mu2 = F.conv2d(a, w, padding=5, groups=3), F.conv2d(b, w, padding=5, groups=3)
+    s11 = F.conv2d(a * a, w, padding=5, groups=3) - mu1 * mu1
+    s22 = F.conv2d(b * b, w, padding=5, groups=3) - mu2 * mu2
+    s12 = F.conv2d(a * b, w, padding=5, groups=3) - mu1 * mu2
+    c1, c2 = 0.01 ** 2, 0.03 ** 2
+    return (((2 * mu1 * mu2 + c1) * (2 * s12 + c2)) / ((mu1 * mu1 + mu2 * mu2 + c1) * (s11 + s22 + c2))).mean()
+
+
+def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
+    """Config 3 (dynamic scene, 200k surfels, 512 control points): bf16 MFMA deformation MLP on the control points ->
+    K-NN (k = 4) -> LBS -> render forward -> 0.8 L1 + 0.2 (1 - SSIM) (PyTorch) -> render backward -> masked Adam on the
+    surfel parameters. The deformation branch is forward-only in this build (no MLP / LBS gradients)."""
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd.deform import DeformNetwork, superpoint_deform
+    from fast_sp_gs_amd.renderer import GS_2D_render
+    from fast_sp_gs_amd.sparse_gaussian_adam import SparseGaussianAdam
+    scene_h, cam_h = scenes.config2(P=200_000, size=800, seed=2)
+    scene, cam = scene_h.to(dev), cam_h.to(dev)
+    g = torch.Generator().manual_seed(2)
+    ctrl = (torch.rand(512, 3, generator=g) * 2 - 1).to(dev)
+    target = torch.rand(3, cam.H, cam.W, generator=g).to(dev)
+    net = DeformNetwork().to(dev)
+    net.pack()
+    names = ('means3D', 'scales', 'rotations', 'opacities', 'shs')
+    params = [getattr(scene, k).clone().requires_grad_(True) for k in names]
+    opt = SparseGaussianAdam([{'params': [p_], 'name': k} for p_, k in zip(params, names)], lr=1.6e-4, eps=1e-15)
+    bg = torch.ones(3, 1, 1, device=dev)
+
+    def step(i):
+        t = torch.full((1,), (i % 17) / 17.0, device=dev)
+        c_xyz, c_rot, c_scale, _ = net(ctrl, t)
+        d_xyz, d_rot, d_scale, _, _ = superpoint_deform(params[0].detach(), ctrl, c_xyz.contiguous(),
+                                                        c_rot.contiguous(), c_scale[:, :2].contiguous(), K=4,
+                                                        temperature=0.01)
+        out = GS_2D_render(params[0] + d_xyz, params[1] + d_scale, params[2] + d_rot, params[3], (cam.W, cam.H),
+                           cam.Tw2v, cam.Tv2c, campos=cam.campos, near=cam.near, far=cam.far, sh_degree=3,
+                           sh_features=params[4])
+        image = out['images'] + (1.0 - out['opacity']) * bg
+        loss = 0.8 * (image - target).abs().mean() + 0.2 * (1.0 - _ssim(image, target))
+        loss.backward()
+        opt.set_before_step(out['radii'] > 0, params[0].shape[0])
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i)
+    torch.cuda.synchronize()
+    return steps / (time.perf_counter() - t0)
+
+
+def fast_path_rate(dev, scene, cam, gi, steps: int = 20, warmup: int = 3):
+    """The "fast" variant (adjugate intersection, fused corner-test binning) on the benchmark scene, forward + backward."""
+    from fast_sp_gs_amd.renderer import fast_render_step
+    ge = torch.zeros(8, cam.H, cam.W, device=dev)
+    go = -gi.sum(0)
+    for _ in range(warmup):
+        fast_render_step(scene, cam, gi, ge, go)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fast_render_step(scene, cam, gi, ge, go)
+    torch.cuda.synchronize()
+    return steps / (time.perf_counter() - t0)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the fast-path and dynamic-step side measurements")
     ap.add_argument("--surfels", type=int, default=300_000)
     ap.add_argument("--size", type=int, default=800)
     args = ap.parse_args()
@@ -174,6 +253,14 @@ def main():
     knn_ms = e0.elapsed_time(e1) / 20
 
     copy_gbps = copy_probe_gbps(dev)
+    extra = {"knn_topk_queries_per_s": pts.shape[0] / (knn_ms * 1e-3), "knn_topk_workload": "200000 x 512, k=4, D=3"}
+    if not args.no_extras:
+        extra["fast_path_frames_per_s"] = fast_path_rate(dev, scene, cam, gi)
+        extra["fast_path_workload"] = "same scene through GS_2D_fast_* (corner-test binning keeps fewer instances)"
+        extra["dynamic_step_frames_per_s"] = dynamic_step_rate(dev)
+        extra["dynamic_step_workload"] = ("200000 surfels, 512 control points, bf16 MFMA MLP + K-NN(4) + LBS -> render "
+                                          "800x800 -> 0.8 L1 + 0.2 D-SSIM (PyTorch) -> backward -> masked Adam; "
+                                          "deformation branch forward-only")
 
     result = {
         "metric": "fwd+bwd frames/s, 300k surfels @800x800",
@@ -197,8 +284,7 @@ def main():
                      "algorithmic_bytes_per_launch": bytes_dom, "avg_launch_ms": stage_avg[dominant],
                      "copy_kernel_GBps": round(copy_gbps, 1)},
         "stages": stages,
-        "extra_metrics": {"knn_topk_queries_per_s": pts.shape[0] / (knn_ms * 1e-3),
-                          "knn_topk_workload": "200000 x 512, k=4, D=3"},
+        "extra_metrics": extra,
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(scene_h, cam_h)
