@@ -13,6 +13,8 @@
 //    with 64-bit ballot match masks (8 ballots per round, popcount of the mask below the lane), which is stable by
 //    construction: within a wave lower rounds and lower lanes come first, waves are ordered by an LDS prefix, blocks
 //    by the scanned histogram.
+#include <algorithm>
+
 #include "binning.hpp"
 
 namespace fsgs {
@@ -160,6 +162,327 @@ __global__ void __launch_bounds__(256) duplicate_keys_kernel(int P, int gx, int 
         keys[soff + e] = ((uint64_t) (uint32_t) ((sy0 + y) * gx + (sx0 + x)) << 32) | sbits;
         vals[soff + e] = sid;
       }
+    }
+  }
+}
+
+// ---- binning by tile buckets -----------------------------------------------------------------------------------------
+// The reference sorts all (tile << 32 | depth bits) keys with one device-wide radix sort (6 passes of 8 bits for 2500
+// tiles). The same final order -- tiles ascending, inside a tile depth bits ascending, equal depths by surfel index,
+// which is what the stable radix sort leaves from the emission order -- is produced here in four steps that touch the
+// instances twice instead of twelve times:
+//   1. count the instances of every tile (64-bit atomics straight into ranges[t].y),
+//   2. exclusive scan over the tiles: ranges[t] = (start, start),
+//   3. scatter (depth bits << 32 | surfel) into the tile's segment at a position drawn from ranges[t].y, which thereby
+//      ends at the segment's end,
+//   4. one block per tile sorts its segment (unique 64-bit keys, so the arbitrary order of step 3 does not matter):
+//      bitonic network in LDS for segments up to 16384 entries, in global memory beyond that.
+// Empty tiles get (0, 0) as the reference's zero-initialised ranges have.
+
+// Visits every (surfel, tile) pair; kScatter = false counts, true scatters.
+template <bool kScatter>
+__global__ void __launch_bounds__(256) tile_emit_kernel(int P, int gx, int gy, int64_t R,
+    const float2* __restrict__ means2D, const float* __restrict__ depths, const int32_t* __restrict__ radii,
+    unsigned long long* __restrict__ ranges, uint64_t* __restrict__ entries) {
+  const int i    = blockIdx.x * blockDim.x + threadIdx.x;
+  const int lane = __lane_id();
+  int x0 = 0, y0 = 0, w = 0, h = 0;
+  uint32_t dbits = 0;
+  if (i < P && radii[i] > 0) {
+    const float2 c   = means2D[i];
+    const TileRect r = tile_rect(c.x, c.y, radii[i], gx, gy);
+    x0 = r.x0, y0 = r.y0, w = max(r.x1 - r.x0, 0), h = max(r.y1 - r.y0, 0);
+    if (kScatter) dbits = __float_as_uint(depths[i]);
+  }
+  auto visit = [&](int tile, uint32_t bits, int id) {
+    unsigned long long* slot = ranges + 2 * (size_t) tile + 1;
+    if (kScatter) {
+      const unsigned long long pos = atomicAdd(slot, 1ull);
+      if ((int64_t) pos < R) entries[pos] = ((uint64_t) bits << 32) | (uint32_t) id;
+    } else {
+      atomicAdd(slot, 1ull);
+    }
+  };
+  const int count = w * h;
+  if (count > 0 && count <= kCoopThreshold) {
+    for (int y = 0; y < h; ++y)
+      for (int x = 0; x < w; ++x) visit((y0 + y) * gx + (x0 + x), dbits, i);
+  }
+  unsigned long long big = __ballot(count > kCoopThreshold);
+  while (big) {
+    const int src = __ffsll((long long) big) - 1;
+    big &= big - 1;
+    const int sx0 = __shfl(x0, src, kWave), sy0 = __shfl(y0, src, kWave), sw = __shfl(w, src, kWave);
+    const int scount = __shfl(count, src, kWave), sid = __shfl(i, src, kWave);
+    const uint32_t sbits = __shfl(dbits, src, kWave);
+    for (int e = lane; e < scount; e += kWave) {
+      const int y = e / sw, x = e - y * sw;
+      visit((sy0 + y) * gx + (sx0 + x), sbits, sid);
+    }
+  }
+}
+
+// Same traversal with the same-address traffic taken off the fabric: a block of 1024 lanes walks a few thousand
+// surfels, counts their instances per tile in LDS, and touches each global tile counter once. (Device-scope atomics on
+// one address are served one after the other at fabric latency; the busiest tile of a frame would otherwise receive a
+// thousand of them.) kScatter = true additionally reserves a contiguous run per (block, tile) and walks the surfels a
+// second time to place the entries. Needs T <= kMaxLdsTiles.
+constexpr int kMaxLdsTiles = 16384;
+#ifndef FSGS_EMIT_PER_BLOCK
+#define FSGS_EMIT_PER_BLOCK 2048
+#endif
+
+template <typename Visit>
+__device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, const float2* __restrict__ means2D,
+                                                  const int32_t* __restrict__ radii, Visit visit) {
+  const int lane = __lane_id();
+  int x0 = 0, y0 = 0, w = 0, h = 0;
+  if (i < P && radii[i] > 0) {
+    const float2 c   = means2D[i];
+    const TileRect r = tile_rect(c.x, c.y, radii[i], gx, gy);
+    x0 = r.x0, y0 = r.y0, w = max(r.x1 - r.x0, 0), h = max(r.y1 - r.y0, 0);
+  }
+  const int count = w * h;
+  if (count > 0 && count <= kCoopThreshold) {
+    for (int y = 0; y < h; ++y)
+      for (int x = 0; x < w; ++x) visit((y0 + y) * gx + (x0 + x), i);
+  }
+  unsigned long long big = __ballot(count > kCoopThreshold);
+  while (big) {
+    const int src = __ffsll((long long) big) - 1;
+    big &= big - 1;
+    const int sx0 = __shfl(x0, src, kWave), sy0 = __shfl(y0, src, kWave), sw = __shfl(w, src, kWave);
+    const int scount = __shfl(count, src, kWave), sid = __shfl(i, src, kWave);
+    for (int e = lane; e < scount; e += kWave) {
+      const int y = e / sw, x = e - y * sw;
+      visit((sy0 + y) * gx + (sx0 + x), sid);
+    }
+  }
+}
+
+template <bool kScatter>
+__global__ void __launch_bounds__(1024) tile_emit_lds_kernel(int P, int per_block, int gx, int gy, int64_t R,
+    const float2* __restrict__ means2D, const float* __restrict__ depths, const int32_t* __restrict__ radii,
+    unsigned long long* __restrict__ ranges, uint64_t* __restrict__ entries) {
+  __shared__ unsigned s_count[kMaxLdsTiles];  // instances of this block per tile, then the block's cursor per tile
+  const int T = gx * gy;
+  for (int t = threadIdx.x; t < T; t += blockDim.x) s_count[t] = 0u;
+  __syncthreads();
+  const int first = blockIdx.x * per_block, last = min(P, first + per_block);
+  // whole wavefronts stay in the loop together: the traversal uses ballots and shuffles
+  const int rounds = (last - first + (int) blockDim.x - 1) / (int) blockDim.x;
+  for (int r = 0; r < rounds; ++r) {
+    const int i = first + r * blockDim.x + threadIdx.x;
+    for_each_instance(i < last ? i : P, P, gx, gy, means2D, radii, [&](int tile, int) { atomicAdd(&s_count[tile], 1u); });
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < T; t += blockDim.x) {
+    const unsigned c = s_count[t];
+    if (c == 0u) continue;
+    if (kScatter) s_count[t] = (unsigned) atomicAdd(ranges + 2 * (size_t) t + 1, (unsigned long long) c);
+    else atomicAdd(ranges + 2 * (size_t) t + 1, (unsigned long long) c);
+  }
+  if (!kScatter) return;
+  __syncthreads();
+  for (int r = 0; r < rounds; ++r) {
+    const int i = first + r * blockDim.x + threadIdx.x;
+    for_each_instance(i < last ? i : P, P, gx, gy, means2D, radii, [&](int tile, int id) {
+      const unsigned pos = atomicAdd(&s_count[tile], 1u);
+      if ((int64_t) pos < R) entries[pos] = ((uint64_t) __float_as_uint(depths[id]) << 32) | (uint32_t) id;
+    });
+  }
+}
+
+// One block: exclusive scan of the per-tile counts, 4 tiles per lane and step.
+__global__ void __launch_bounds__(1024) tile_scan_kernel(int T, unsigned long long* __restrict__ ranges,
+                                                         int* __restrict__ large_count) {
+  __shared__ unsigned long long s_wave[16];
+  const int lane = __lane_id(), wave = threadIdx.x / kWave;
+  unsigned long long carry = 0;
+  for (int start = 0; start < T; start += 4096) {
+    const int t0 = start + threadIdx.x * 4;
+    unsigned long long c[4], sum = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) c[k] = t0 + k < T ? ranges[2 * (size_t) (t0 + k) + 1] : 0ull, sum += c[k];
+    const unsigned long long inc = wave_inclusive_scan(sum);
+    if (lane == kWave - 1) s_wave[wave] = inc;
+    __syncthreads();
+    unsigned long long base = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const unsigned long long v = s_wave[w];
+      if (w < wave) base += v;
+      total += v;
+    }
+    __syncthreads();
+    unsigned long long run = carry + base + inc - sum;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (t0 + k < T) ranges[2 * (size_t) (t0 + k)] = run, ranges[2 * (size_t) (t0 + k) + 1] = run;
+      run += c[k];
+    }
+    carry += total;
+  }
+  if (threadIdx.x == 0) *large_count = 0;
+}
+
+__device__ __forceinline__ void tile_sort_output(int tile, int64_t start, int n, const uint64_t* sorted_local,
+                                                 int32_t* __restrict__ point_list, int64_t* __restrict__ keys_out) {
+  for (int k = threadIdx.x; k < n; k += blockDim.x) {
+    const uint64_t e = sorted_local[k];
+    point_list[start + k] = (int32_t) (uint32_t) e;
+    if (keys_out) keys_out[start + k] = (int64_t) (((uint64_t) (uint32_t) tile << 32) | (e >> 32));
+  }
+}
+
+// Bitonic sorting network for any length n (all compare-exchanges ascending: the first step of every merge pairs an
+// element with its mirror image inside the block, the following steps are plain half-cleaners). Pairs whose upper
+// element lies beyond n are skipped, which is the same as padding with +infinity. `sync` separates the steps.
+template <typename Index, typename Sync>
+__device__ __forceinline__ void bitonic_sort(uint64_t* e, Index n, int threads, Sync sync) {
+  Index m = 2;
+  while (m < n) m <<= 1;
+  int log_half = 0;
+  for (Index size = 2; size <= m; size <<= 1, ++log_half) {
+    const Index half = size >> 1;
+    for (Index k = threadIdx.x; k < (m >> 1); k += threads) {
+      const Index blk = k >> log_half, off = k & (half - 1);
+      const Index lo = blk * size + off, hi = blk * size + size - 1 - off;
+      if (hi < n) {
+        const uint64_t a = e[lo], b = e[hi];
+        if (a > b) e[lo] = b, e[hi] = a;
+      }
+    }
+    sync();
+    for (Index stride = half >> 1; stride > 0; stride >>= 1) {
+      for (Index k = threadIdx.x; k < (m >> 1); k += threads) {
+        const Index lo = ((k & ~(stride - 1)) << 1) | (k & (stride - 1));  // index with the `stride` bit clear
+        const Index hi = lo | stride;
+        if (hi < n) {
+          const uint64_t a = e[lo], b = e[hi];
+          if (a > b) e[lo] = b, e[hi] = a;
+        }
+      }
+      sync();
+    }
+  }
+}
+
+// The same network for a segment held in LDS, two network steps per barrier: a lane loads four elements that are closed
+// under two consecutive steps (mirror + first half-cleaner, or two half-cleaners), exchanges them in registers and
+// stores them back. Elements beyond n read as +infinity and are never stored.
+__device__ __forceinline__ void cx(uint64_t& a, uint64_t& b) {
+  const uint64_t lo = a < b ? a : b, hi = a < b ? b : a;
+  a = lo, b = hi;
+}
+
+__device__ __forceinline__ void bitonic_sort_lds(uint64_t* e, int n, int threads) {
+  int m = 2;
+  while (m < n) m <<= 1;
+  auto ld = [&](int i) { return i < n ? e[i] : ~0ull; };
+  auto st = [&](int i, uint64_t v) { if (i < n) e[i] = v; };
+  auto single = [&](int size, int log_half, int stride) {  // stride == 0: the mirror step of `size`
+    for (int k = threadIdx.x; k < (m >> 1); k += threads) {
+      int lo, hi;
+      if (stride == 0) {
+        const int blk = k >> log_half, off = k & ((size >> 1) - 1);
+        lo = blk * size + off, hi = blk * size + size - 1 - off;
+      } else {
+        lo = ((k & ~(stride - 1)) << 1) | (k & (stride - 1)), hi = lo | stride;
+      }
+      if (hi < n) {
+        uint64_t a = e[lo], b = e[hi];
+        if (a > b) e[lo] = b, e[hi] = a;
+      }
+    }
+    __syncthreads();
+  };
+  int log_half = 0;
+  for (int size = 2; size <= m; size <<= 1, ++log_half) {
+    if (size == 2) {
+      single(2, 0, 0);
+      continue;
+    }
+    const int quarter = size >> 2;
+    for (int q = threadIdx.x; q < (m >> 2); q += threads) {  // mirror step + half-cleaner of stride size / 4
+      const int blk = q >> (log_half - 1), off = q & (quarter - 1);
+      const int base = blk * size;
+      const int ia = base + off, ib = ia + quarter, ja = base + size - 1 - off, jb = ja - quarter;
+      uint64_t a = ld(ia), b = ld(ib), bm = ld(jb), am = ld(ja);
+      cx(a, am), cx(b, bm);
+      cx(a, b), cx(bm, am);
+      st(ia, a), st(ib, b), st(jb, bm), st(ja, am);
+    }
+    __syncthreads();
+    int stride = quarter >> 1;
+    for (; stride >= 2; stride >>= 2) {  // half-cleaners of strides `stride` and `stride / 2`
+      const int lo_s = stride >> 1;
+      for (int q = threadIdx.x; q < (m >> 2); q += threads) {
+        const int base = ((q & ~(lo_s - 1)) << 2) | (q & (lo_s - 1));
+        const int i0 = base, i1 = base | lo_s, i2 = base | stride, i3 = base | stride | lo_s;
+        uint64_t v0 = ld(i0), v1 = ld(i1), v2 = ld(i2), v3 = ld(i3);
+        cx(v0, v2), cx(v1, v3);
+        cx(v0, v1), cx(v2, v3);
+        st(i0, v0), st(i1, v1), st(i2, v2), st(i3, v3);
+      }
+      __syncthreads();
+    }
+    if (stride == 1) single(size, log_half, 1);
+  }
+}
+
+constexpr int kSmallSegment = 2048;   // entries sorted by a 256-lane block in 16 KB of LDS
+constexpr int kLargeSegment = 16384;  // entries sorted by a 1024-lane block in 128 KB of LDS
+
+// One block per tile: segments up to kSmallSegment entries are sorted in LDS, longer ones are queued for
+// tile_sort_large_kernel; empty tiles get the (0, 0) range the reference's zero-initialised output has.
+__global__ void __launch_bounds__(256) tile_sort_small_kernel(int64_t* __restrict__ ranges,
+    const uint64_t* __restrict__ entries, int32_t* __restrict__ point_list, int64_t* __restrict__ keys_out,
+    int* __restrict__ large_count, int* __restrict__ large_list) {
+  __shared__ uint64_t s_e[kSmallSegment];
+  const int tile = blockIdx.x;
+  const int64_t start = ranges[2 * (size_t) tile];
+  const int64_t len   = ranges[2 * (size_t) tile + 1] - start;
+  if (len == 0) {
+    if (threadIdx.x == 0) ranges[2 * (size_t) tile] = 0, ranges[2 * (size_t) tile + 1] = 0;
+    return;
+  }
+  if (len > kSmallSegment) {
+    if (threadIdx.x == 0) large_list[atomicAdd(large_count, 1)] = tile;
+    return;
+  }
+  const int n = (int) len;
+  for (int k = threadIdx.x; k < n; k += 256) s_e[k] = entries[start + k];
+  __syncthreads();
+  bitonic_sort_lds(s_e, n, 256);
+  tile_sort_output(tile, start, n, s_e, point_list, keys_out);
+}
+
+// A few blocks walk the queue of long segments: up to kLargeSegment entries in LDS, beyond that the same network on the
+// global array (slow, but such a segment means tens of thousands of surfels over one 16x16 tile).
+__global__ void __launch_bounds__(1024) tile_sort_large_kernel(const int64_t* __restrict__ ranges,
+    uint64_t* __restrict__ entries, int32_t* __restrict__ point_list, int64_t* __restrict__ keys_out,
+    const int* __restrict__ large_count, const int* __restrict__ large_list) {
+  __shared__ uint64_t s_e[kLargeSegment];
+  const int n_large = *large_count;
+  for (int q = blockIdx.x; q < n_large; q += gridDim.x) {
+    const int tile = large_list[q];
+    const int64_t start = ranges[2 * (size_t) tile];
+    const int64_t len   = ranges[2 * (size_t) tile + 1] - start;
+    if (len <= kLargeSegment) {
+      const int n = (int) len;
+      for (int k = threadIdx.x; k < n; k += 1024) s_e[k] = entries[start + k];
+      __syncthreads();
+      bitonic_sort_lds(s_e, n, 1024);
+      tile_sort_output(tile, start, n, s_e, point_list, keys_out);
+      __syncthreads();
+    } else {
+      uint64_t* e = entries + start;
+      bitonic_sort<int64_t>(e, len, 1024, [] {
+        __threadfence_block();
+        __syncthreads();
+      });
+      tile_sort_output(tile, start, (int) len, e, point_list, keys_out);
     }
   }
 }
@@ -419,14 +742,33 @@ FSGS_API int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, con
   if (workspace_bytes < sort_workspace_bytes(R))
     return fail(kWorkspaceSmall, "gs_prepare_fill: workspace %zu < %zu bytes", workspace_bytes,
                 sort_workspace_bytes(R));
-  const int bits = fsgs_gs_prepare_sort_bits(W, H);
-  hipLaunchKernelGGL(duplicate_keys_kernel, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
-                     (const float2*) means2D, depths, radii, point_offsets, sort_keys_in(R, workspace),
-                     sort_vals_in(R, bits, workspace, point_list));
-  const uint64_t* sorted = nullptr;
-  radix_sort_pairs(R, bits, workspace, point_list, &sorted, s);
-  launch_tile_ranges(R, T, sorted, ranges, s);
-  if (sorted_keys_out)
-    FSGS_HIP(hipMemcpyAsync(sorted_keys_out, sorted, (size_t) R * 8, hipMemcpyDeviceToDevice, s));
+  // ranges was zeroed above; it doubles as the per-tile counter / cursor array of the bucket sort
+  unsigned long long* rng = (unsigned long long*) ranges;
+  uint64_t* entries       = sort_keys_in(R, workspace);
+  // the LDS-aggregated traversal needs one LDS counter per tile; larger tile grids count straight in global memory
+  const bool lds_path = T <= kMaxLdsTiles;
+  const int per_block = std::max(FSGS_EMIT_PER_BLOCK, div_up(P, 256));
+  const dim3 lgrid(div_up(P, per_block)), lblock(1024);
+  const dim3 pgrid(div_up(P, 256)), pblock(256);
+  if (lds_path)
+    hipLaunchKernelGGL(tile_emit_lds_kernel<false>, lgrid, lblock, 0, s, P, per_block, gx, gy, R,
+                       (const float2*) means2D, depths, radii, rng, entries);
+  else
+    hipLaunchKernelGGL(tile_emit_kernel<false>, pgrid, pblock, 0, s, P, gx, gy, R, (const float2*) means2D, depths,
+                       radii, rng, entries);
+  // queue of long segments: at most R / kSmallSegment tiles, kept behind the entries in the workspace
+  int* large_count = (int*) ((char*) workspace + sort_layout(R).keys1);
+  int* large_list  = large_count + 1;
+  hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, large_count);
+  if (lds_path)
+    hipLaunchKernelGGL(tile_emit_lds_kernel<true>, lgrid, lblock, 0, s, P, per_block, gx, gy, R,
+                       (const float2*) means2D, depths, radii, rng, entries);
+  else
+    hipLaunchKernelGGL(tile_emit_kernel<true>, pgrid, pblock, 0, s, P, gx, gy, R, (const float2*) means2D, depths,
+                       radii, rng, entries);
+  hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
+                     large_count, large_list);
+  hipLaunchKernelGGL(tile_sort_large_kernel, dim3(64), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,
+                     large_count, large_list);
   return check_launch("gs_prepare_fill");
 }

@@ -1,0 +1,58 @@
+"""Bit-exact parity of the tile binning (ranges, point list, sorted keys) with the oracle's stable sort, on the GPU's own
+preprocess outputs, for every segment-length class of the per-tile sort: short segments (<= 2048 entries, LDS, one
+block per tile), long ones (<= 16384, LDS, queued) and very long ones (sorted in global memory), a tile grid too large for the
+LDS counters, plus equal depths
+(ties must come out in surfel order) and empty tiles."""
+import numpy as np
+import pytest
+import torch
+
+from util import npy
+
+pytestmark = pytest.mark.gpu
+
+CASES = {
+    # name: (P, W, H, scale multiplier, duplicate depths)
+    "short_segments": (20_000, 320, 200, 1.0, False),
+    "long_segments_lds": (9_000, 32, 32, 1.0, False),       # 4 tiles, ~9000 entries each
+    "very_long_segments": (40_000, 32, 16, 1.0, False),     # 2 tiles, > 16384 entries each
+    "equal_depths": (6_000, 64, 48, 2.0, True),
+    "many_tiles": (5_000, 2100, 2100, 20.0, False),         # > 16384 tiles: counters in global memory
+}
+
+
+@pytest.mark.parametrize("name", list(CASES))
+def test_binning_bit_exact(name, device, oracle_mod):
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd._C import get_C_function
+    O = oracle_mod
+    P, W, H, mul, dup = CASES[name]
+    scene, _ = scenes.config0(P=P, size=max(W, H), seed=21)
+    scene.scales = scene.scales * mul
+    if W <= 32:  # squeeze everything into the few tiles of a tiny image
+        scene.means3D = scene.means3D * 0.05
+    if dup:      # a plane parallel to the image plane: thousands of identical depths
+        scene.means3D[:, 2] = 0.25
+    cam = scenes.pinhole(W, H, 50.0, torch.tensor([0., 0., 4.]))
+    d = lambda t: t.to(device).contiguous()
+    print(f"[binning {name}] P={P} {W}x{H}", flush=True)
+    m2, colors, tm, no, dep, radii, tt = get_C_function('gs_2d_preprocess_forward')(
+        W, H, 3, False, d(scene.means3D), d(scene.scales), d(scene.rotations), d(scene.opacities), d(scene.shs), None,
+        d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), None, None, None)
+    ranges, pl, keys, offsets = get_C_function('GS_prepare')(W, H, m2, dep, radii, tt, False, return_keys=True,
+                                                           return_offsets=True)
+    torch.cuda.synchronize()
+    r_ranges, r_pl, r_keys = O.prepare(W, H, npy(m2), npy(dep), npy(radii), npy(tt), return_keys=True)
+    lens = r_ranges[:, 1] - r_ranges[:, 0]
+    print(f"[binning {name}] R={r_pl.size} longest segment {int(lens.max())} empty tiles {int((lens == 0).sum())}",
+          flush=True)
+    if name == "long_segments_lds":
+        assert 2048 < lens.max() <= 16384
+    if name == "very_long_segments":
+        assert lens.max() > 16384
+    if dup:
+        assert np.unique(npy(dep)[npy(radii) > 0]).size < (npy(radii) > 0).sum()
+    assert np.array_equal(npy(ranges), r_ranges)
+    assert np.array_equal(npy(pl), r_pl)
+    assert np.array_equal(npy(keys), r_keys)
+    assert np.array_equal(npy(offsets)[:P], np.cumsum(npy(tt).astype(np.int64)))
