@@ -1,5 +1,5 @@
-// Tile binning for gfx950: prefix sum of per-surfel tile counts, (tile | depth-bits) key duplication, a stable
-// least-significant-digit radix sort of 64-bit keys with 32-bit payloads, and per-tile range detection.
+// Tile binning for gfx950: prefix sum of per-surfel tile counts, then the (tile, depth) ordering of all (surfel, tile)
+// instances and the per-tile ranges.
 //
 // Reference behaviour reproduced bit for bit: fast_2d_gs/_C/src/gaussian_splatting/gaussian_prepare.cu:32-83
 // (getHigherMsb, duplicateWithKeys), :192-220 (identifyTileRanges), :222-308 (prepare / GS_prepare, which uses
@@ -7,12 +7,14 @@
 //
 // Wave64 design notes
 //  * scan: 2048 counts per 256-lane block, lane-local sums + wave prefix by cross-lane shifts + LDS across the 4 waves.
-//  * duplication: one lane per surfel for small rectangles; rectangles above 32 tiles are emitted cooperatively by the
-//    whole wavefront (64 coalesced keys per step) so one huge surfel cannot serialise a wave.
-//  * sort: 8-bit digits. Per pass: block histograms -> per-digit scan over blocks -> scatter. The scatter ranks keys
-//    with 64-bit ballot match masks (8 ballots per round, popcount of the mask below the lane), which is stable by
-//    construction: within a wave lower rounds and lower lanes come first, waves are ordered by an LDS prefix, blocks
-//    by the scanned histogram.
+//  * standard path: bucket the instances by tile (count -> scan -> scatter) and sort every tile's segment on its own
+//    (see "binning by tile buckets" below); rectangles above 32 tiles are walked cooperatively by the whole wavefront
+//    so one huge surfel cannot serialise a wave.
+//  * device-wide radix sort (used by the fused corner-test binning of the fast path, whose padding entries and sort width
+//    follow the reference): 8-bit digits. Per pass: block histograms -> per-digit scan over blocks -> scatter. The
+//    scatter ranks keys with 64-bit ballot match masks (8 ballots per round, popcount of the mask below the lane),
+//    which is stable by construction: within a wave lower rounds and lower lanes come first, waves are ordered by an
+//    LDS prefix, blocks by the scanned histogram.
 #include <algorithm>
 
 #include "binning.hpp"
@@ -114,57 +116,7 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(int P, const i
   }
 }
 
-// ---- key duplication ------------------------------------------------------------------------------------------------
-constexpr int kCoopThreshold = 32;
-
-__global__ void __launch_bounds__(256) duplicate_keys_kernel(int P, int gx, int gy, int64_t R,
-    const float2* __restrict__ means2D,
-    const float* __restrict__ depths, const int32_t* __restrict__ radii, const int64_t* __restrict__ offsets,
-    uint64_t* __restrict__ keys, int32_t* __restrict__ vals) {
-  const int i    = blockIdx.x * blockDim.x + threadIdx.x;
-  const int lane = __lane_id();
-  int x0 = 0, y0 = 0, w = 0, h = 0;
-  int64_t off    = 0;
-  uint32_t dbits = 0;
-  if (i < P && radii[i] > 0) {
-    const float2 c   = means2D[i];
-    const TileRect r = tile_rect(c.x, c.y, radii[i], gx, gy);
-    x0 = r.x0, y0 = r.y0, w = r.x1 - r.x0, h = r.y1 - r.y0;
-    if (w < 0) w = 0;
-    if (h < 0) h = 0;
-    off   = i == 0 ? 0 : offsets[i - 1];
-    dbits = __float_as_uint(depths[i]);
-  }
-  const int count = w * h;
-  if (count > 0 && count <= kCoopThreshold) {
-    for (int y = 0; y < h; ++y)
-      for (int x = 0; x < w; ++x) {
-        if (off < R) {  // offsets come from the caller's tiles_touched; never write past the buffers it sized
-          keys[off] = ((uint64_t) (uint32_t) ((y0 + y) * gx + (x0 + x)) << 32) | dbits;
-          vals[off] = i;
-        }
-        ++off;
-      }
-  }
-  // Large rectangles: the wavefront walks them together, 64 keys per step in row-major tile order.
-  unsigned long long big = __ballot(count > kCoopThreshold);
-  while (big) {
-    const int src = __ffsll((long long) big) - 1;
-    big &= big - 1;
-    const int sx0 = __shfl(x0, src, kWave), sy0 = __shfl(y0, src, kWave), sw = __shfl(w, src, kWave);
-    const int scount = __shfl(count, src, kWave), sid = __shfl(i, src, kWave);
-    const uint32_t sbits = __shfl(dbits, src, kWave);
-    const int64_t soff   = ((int64_t) __shfl((int) (off >> 32), src, kWave) << 32) |
-                         (uint32_t) __shfl((int) (off & 0xffffffff), src, kWave);
-    for (int e = lane; e < scount; e += kWave) {
-      const int y = e / sw, x = e - y * sw;
-      if (soff + e < R) {
-        keys[soff + e] = ((uint64_t) (uint32_t) ((sy0 + y) * gx + (sx0 + x)) << 32) | sbits;
-        vals[soff + e] = sid;
-      }
-    }
-  }
-}
+constexpr int kCoopThreshold = 32;  // rectangles with more tiles are walked by the whole wavefront
 
 // ---- binning by tile buckets -----------------------------------------------------------------------------------------
 // The reference sorts all (tile << 32 | depth bits) keys with one device-wide radix sort (6 passes of 8 bits for 2500
