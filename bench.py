@@ -96,31 +96,15 @@ def cpu_baseline(scene, cam, budget_s: float = 20.0):
                       f"host has {os.cpu_count()} logical cpus"}
 
 
-def _ssim(img1, img2):
-    """Plain PyTorch SSIM (11x11 Gaussian window, sigma 1.5, C1 = 0.01^2, C2 = 0.03^2), the reference's fallback form
-    (losses/ssim.py:49-67); the fused SSIM kernel is not part of this build."""
-    import torch.nn.functional as F
-    k = torch.arange(11, dtype=torch.float32, device=img1.device) - 5
-    g = torch.exp(-k * k / (2 * 1.5 ** 2))
-    g = (g / g.sum())
-    w = (g[:, None] * g[None, :]).expand(3, 1, 11, 11).contiguous()
-    a, b = img1[None], img2[None]
-    mu1, mu2 = F.conv2d(a, w, padding=5, groups=3), F.conv2d(b, w, padding=5, groups=3)
-    s11 = F.conv2d(a * a, w, padding=5, groups=3) - mu1 * mu1
-    s22 = F.conv2d(b * b, w, padding=5, groups=3) - mu2 * mu2
-    s12 = F.conv2d(a * b, w, padding=5, groups=3) - mu1 * mu2
-    c1, c2 = 0.01 ** 2, 0.03 ** 2
-    return (((2 * mu1 * mu2 + c1) * (2 * s12 + c2)) / ((mu1 * mu1 + mu2 * mu2 + c1) * (s11 + s22 + c2))).mean()
-
-
 def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
     """Config 3 (dynamic scene, 200k surfels, 512 control points): bf16 MFMA deformation MLP on the control points ->
-    K-NN (k = 4) -> LBS -> render forward -> 0.8 L1 + 0.2 (1 - SSIM) (PyTorch) -> render backward -> masked Adam on the
-    surfel parameters. The deformation branch is forward-only in this build (no MLP / LBS gradients)."""
+    K-NN (k = 4) -> LBS -> render forward -> 0.8 L1 + 0.2 (1 - SSIM) (fused SSIM kernel) -> render backward -> masked Adam
+    on the surfel parameters. The deformation branch is forward-only in this build (no MLP / LBS gradients)."""
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd.deform import DeformNetwork, superpoint_deform
     from fast_sp_gs_amd.renderer import GS_2D_render
     from fast_sp_gs_amd.sparse_gaussian_adam import SparseGaussianAdam
+    from fast_sp_gs_amd.ssim import ssim
     scene_h, cam_h = scenes.config2(P=200_000, size=800, seed=2)
     scene, cam = scene_h.to(dev), cam_h.to(dev)
     g = torch.Generator().manual_seed(2)
@@ -143,7 +127,7 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
                            cam.Tw2v, cam.Tv2c, campos=cam.campos, near=cam.near, far=cam.far, sh_degree=3,
                            sh_features=params[4])
         image = out['images'] + (1.0 - out['opacity']) * bg
-        loss = 0.8 * (image - target).abs().mean() + 0.2 * (1.0 - _ssim(image, target))
+        loss = 0.8 * (image - target).abs().mean() + 0.2 * (1.0 - ssim(image, target).mean())
         loss.backward()
         opt.set_before_step(out['radii'] > 0, params[0].shape[0])
         opt.step()
@@ -157,6 +141,33 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
         step(i)
     torch.cuda.synchronize()
     return steps / (time.perf_counter() - t0)
+
+
+def ssim_rate(dev, reps: int = 20):
+    """Fused SSIM forward (with the partial-derivative maps) + backward on one 3 x 800 x 800 image pair."""
+    from fast_sp_gs_amd._C import get_C_function
+    fwd, bwd = get_C_function('fusedssim'), get_C_function('fusedssim_backward')
+    g = torch.Generator().manual_seed(3)
+    a, b, gm = (torch.rand(1, 3, 800, 800, generator=g).to(dev) for _ in range(3))
+    for _ in range(3):
+        m, d1, d2, d3 = fwd(1e-4, 9e-4, a, b, True)
+        bwd(1e-4, 9e-4, a, b, gm, d1, d2, d3)
+    torch.cuda.synchronize()
+    e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    e[0].record()
+    for _ in range(reps):
+        m, d1, d2, d3 = fwd(1e-4, 9e-4, a, b, True)
+    e[1].record()
+    for _ in range(reps):
+        bwd(1e-4, 9e-4, a, b, gm, d1, d2, d3)
+    e[2].record()
+    torch.cuda.synchronize()
+    n = a.numel() * 4
+    f_ms, b_ms = e[0].elapsed_time(e[1]) / reps, e[1].elapsed_time(e[2]) / reps
+    return {"fusedssim_forward_ms": f_ms, "fusedssim_backward_ms": b_ms,
+            "fusedssim_forward_GBps": 6 * n / (f_ms * 1e-3) / 1e9,   # 2 images in, map + 3 partial maps out
+            "fusedssim_backward_GBps": 7 * n / (b_ms * 1e-3) / 1e9,  # 2 images + dL/dmap + 3 maps in, gradient out
+            "fusedssim_workload": "1 x 3 x 800 x 800, train = true (times include output allocation)"}
 
 
 def fast_path_rate(dev, scene, cam, gi, steps: int = 20, warmup: int = 3):
@@ -255,11 +266,12 @@ def main():
     copy_gbps = copy_probe_gbps(dev)
     extra = {"knn_topk_queries_per_s": pts.shape[0] / (knn_ms * 1e-3), "knn_topk_workload": "200000 x 512, k=4, D=3"}
     if not args.no_extras:
+        extra.update(ssim_rate(dev))
         extra["fast_path_frames_per_s"] = fast_path_rate(dev, scene, cam, gi)
         extra["fast_path_workload"] = "same scene through GS_2D_fast_* (corner-test binning keeps fewer instances)"
         extra["dynamic_step_frames_per_s"] = dynamic_step_rate(dev)
         extra["dynamic_step_workload"] = ("200000 surfels, 512 control points, bf16 MFMA MLP + K-NN(4) + LBS -> render "
-                                          "800x800 -> 0.8 L1 + 0.2 D-SSIM (PyTorch) -> backward -> masked Adam; "
+                                          "800x800 -> 0.8 L1 + 0.2 D-SSIM (fused kernel) -> backward -> masked Adam; "
                                           "deformation branch forward-only")
 
     result = {

@@ -21,7 +21,7 @@ __all__ = [
     'freq_encode_backward', 'cdist_top', 'cdist_top_backward', 'AdamMasksedUpdated', 'knn_topk', 'lbs_blend',
     'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'gs_2d_pack_records', 'gs_2d_fast_preprocess_forward',
     'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward', 'gs_2d_fast_compute_trans_mat_backward',
-    'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward',
+    'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward', 'fusedssim', 'fusedssim_backward',
 ]
 
 _TILE = 16
@@ -887,3 +887,47 @@ def mlp_forward(inputs: Tensor, packed: Tensor, bias: Tensor, n_layers: int, ski
                                      L.ptr(out), L.current_stream())
     L.check(rc, what)
     return out
+
+
+# --------------------------------------------------------------------------------------------------------------------
+def fusedssim(C1: float, C2: float, img1: Tensor, img2: Tensor, train: bool):
+    """structural_similarity.cu:340-363 -> (ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12), all [B,CH,H,W]; the three
+    partial-derivative maps are empty tensors when `train` is false."""
+    what = 'fusedssim'
+    _f32(what, img1=img1, img2=img2)
+    if img1.ndim != 4 or img1.shape != img2.shape:
+        raise RuntimeError(f'{what}: img1 and img2 must be [B,CH,H,W] tensors of the same shape')
+    img1, img2 = img1.contiguous(), img2.contiguous()
+    B, CH, H, W = img1.shape
+    ssim_map = torch.empty_like(img1)
+    if train:
+        d1, d2, d3 = torch.empty_like(img1), torch.empty_like(img1), torch.empty_like(img1)
+    else:
+        d1 = d2 = d3 = None
+    with _timed(what):
+        rc = _lib().fsgs_fusedssim_forward(B, CH, H, W, float(C1), float(C2), L.ptr(img1), L.ptr(img2),
+                                           L.ptr(ssim_map), L.ptr(d1), L.ptr(d2), L.ptr(d3), L.current_stream())
+    L.check(rc, what)
+    if not train:
+        d1, d2, d3 = (torch.empty(0) for _ in range(3))
+    return ssim_map, d1, d2, d3
+
+
+def fusedssim_backward(C1: float, C2: float, img1: Tensor, img2: Tensor, dL_dmap: Tensor, dm_dmu1: Tensor,
+                       dm_dsigma1_sq: Tensor, dm_dsigma12: Tensor) -> Tensor:
+    """structural_similarity.cu:365-380 -> dL_dimg1[B,CH,H,W]."""
+    what = 'fusedssim_backward'
+    _f32(what, img1=img1, img2=img2, dL_dmap=dL_dmap, dm_dmu1=dm_dmu1, dm_dsigma1_sq=dm_dsigma1_sq,
+         dm_dsigma12=dm_dsigma12)
+    img1, img2, dL_dmap = img1.contiguous(), img2.contiguous(), dL_dmap.contiguous()
+    B, CH, H, W = img1.shape
+    for name, t in (('img2', img2), ('dL_dmap', dL_dmap), ('dm_dmu1', dm_dmu1), ('dm_dsigma1_sq', dm_dsigma1_sq),
+                    ('dm_dsigma12', dm_dsigma12)):
+        L.require_shape(what, name, t, B, CH, H, W)
+    grad = torch.empty_like(img1)
+    with _timed(what):
+        rc = _lib().fsgs_fusedssim_backward(B, CH, H, W, L.ptr(img1), L.ptr(img2), L.ptr(dL_dmap),
+                                            L.ptr(dm_dmu1.contiguous()), L.ptr(dm_dsigma1_sq.contiguous()),
+                                            L.ptr(dm_dsigma12.contiguous()), L.ptr(grad), L.current_stream())
+    L.check(rc, what)
+    return grad

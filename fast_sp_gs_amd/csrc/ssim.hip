@@ -1,0 +1,180 @@
+// Fused SSIM map and its backward for gfx950.
+//
+// Reference behaviour reproduced: fast_2d_gs/_C/src/other/structural_similarity.cu:187-277 (forward kernel), :279-338
+// (backward kernel), :340-380 (host entries): separable 11-tap Gaussian (sigma 1.5, the literal weights of :11-21), zero
+// padding, per channel; the forward also returns dm/dmu1, dm/dsigma1^2, dm/dsigma12 for the backward.
+//
+// Where the reference convolves one quantity at a time through a shared scratchpad (five passes and ~25 barriers per
+// channel), each block here loads the 42x42 halo of both images once, forms all five moments (I1, I1^2, I2, I2^2, I1 I2)
+// in one horizontal pass into LDS and finishes them in one vertical pass: two barriers per channel. A block is 256 lanes
+// (4 wavefronts) for a 32x32 output tile, every lane owning one column of 4 output rows.
+#include "common.hpp"
+
+namespace fsgs {
+namespace {
+
+constexpr int kSsimTile = 32;
+constexpr int kSsimHalo = kSsimTile + 10;  // 42
+constexpr int kSsimThreads = 256;
+
+__constant__ float kGauss[11] = {0.001028380123898387f, 0.0075987582094967365f, 0.036000773310661316f,
+                                 0.10936068743467331f,  0.21300552785396576f,   0.26601171493530273f,
+                                 0.21300552785396576f,  0.10936068743467331f,   0.036000773310661316f,
+                                 0.0075987582094967365f, 0.001028380123898387f};
+
+__device__ __forceinline__ float pixel_or_zero(const float* __restrict__ plane, int y, int x, int H, int W) {
+  return (x >= 0 && y >= 0 && x < W && y < H) ? plane[(size_t) y * W + x] : 0.0f;
+}
+
+template <bool kTrain>
+__global__ void __launch_bounds__(kSsimThreads) ssim_forward_kernel(int H, int W, int CH, float C1, float C2,
+    const float* __restrict__ img1, const float* __restrict__ img2, float* __restrict__ ssim_map,
+    float* __restrict__ dm_dmu1, float* __restrict__ dm_dsigma1_sq, float* __restrict__ dm_dsigma12) {
+  __shared__ float s_a[kSsimHalo][kSsimHalo + 1];
+  __shared__ float s_b[kSsimHalo][kSsimHalo + 1];
+  __shared__ float s_h[5][kSsimHalo][kSsimTile + 1];  // horizontally filtered moments
+  const int x0 = blockIdx.x * kSsimTile, y0 = blockIdx.y * kSsimTile;
+  const size_t plane = (size_t) H * W;
+  float g[11];
+#pragma unroll
+  for (int k = 0; k < 11; ++k) g[k] = kGauss[k];
+
+  for (int c = 0; c < CH; ++c) {
+    const float* p1 = img1 + ((size_t) blockIdx.z * CH + c) * plane;
+    const float* p2 = img2 + ((size_t) blockIdx.z * CH + c) * plane;
+    for (int e = threadIdx.x; e < kSsimHalo * kSsimHalo; e += kSsimThreads) {
+      const int ly = e / kSsimHalo, lx = e - ly * kSsimHalo;
+      s_a[ly][lx] = pixel_or_zero(p1, y0 + ly - 5, x0 + lx - 5, H, W);
+      s_b[ly][lx] = pixel_or_zero(p2, y0 + ly - 5, x0 + lx - 5, H, W);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < kSsimHalo * kSsimTile; e += kSsimThreads) {
+      const int ly = e / kSsimTile, lx = e - ly * kSsimTile;
+      float m1 = 0, m11 = 0, m2 = 0, m22 = 0, m12 = 0;
+#pragma unroll
+      for (int k = 0; k < 11; ++k) {
+        const float a = s_a[ly][lx + k], b = s_b[ly][lx + k];
+        m1 += g[k] * a, m11 += g[k] * (a * a), m2 += g[k] * b, m22 += g[k] * (b * b), m12 += g[k] * (a * b);
+      }
+      s_h[0][ly][lx] = m1, s_h[1][ly][lx] = m11, s_h[2][ly][lx] = m2, s_h[3][ly][lx] = m22, s_h[4][ly][lx] = m12;
+    }
+    __syncthreads();
+    const int lx = threadIdx.x & 31;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int ly = (threadIdx.x >> 5) * 4 + r;
+      float mu1 = 0, e11 = 0, mu2 = 0, e22 = 0, e12 = 0;
+#pragma unroll
+      for (int k = 0; k < 11; ++k) {
+        mu1 += g[k] * s_h[0][ly + k][lx], e11 += g[k] * s_h[1][ly + k][lx], mu2 += g[k] * s_h[2][ly + k][lx];
+        e22 += g[k] * s_h[3][ly + k][lx], e12 += g[k] * s_h[4][ly + k][lx];
+      }
+      const int px = x0 + lx, py = y0 + ly;
+      if (px < W && py < H) {
+        const float sigma1_sq = e11 - mu1 * mu1, sigma2_sq = e22 - mu2 * mu2, sigma12 = e12 - mu1 * mu2;
+        const float mu1_sq = mu1 * mu1, mu2_sq = mu2 * mu2, mu1_mu2 = mu1 * mu2;
+        const float C = 2.0f * mu1_mu2 + C1, D = 2.0f * sigma12 + C2;
+        const float A = mu1_sq + mu2_sq + C1, B = sigma1_sq + sigma2_sq + C2;
+        const size_t idx = ((size_t) blockIdx.z * CH + c) * plane + (size_t) py * W + px;
+        ssim_map[idx] = (C * D) / (A * B);
+        if (kTrain) {
+          dm_dmu1[idx] = (mu2 * 2.0f * D) / (A * B) - (mu2 * 2.0f * C) / (A * B) - (mu1 * 2.0f * C * D) / (A * A * B) +
+                         (mu1 * 2.0f * C * D) / (A * B * B);
+          dm_dsigma1_sq[idx] = (-C * D) / (A * B * B);
+          dm_dsigma12[idx]   = (2.0f * C) / (A * B);
+        }
+      }
+    }
+    __syncthreads();  // the next channel overwrites the halo and the filtered moments
+  }
+}
+
+__global__ void __launch_bounds__(kSsimThreads) ssim_backward_kernel(int H, int W, int CH,
+    const float* __restrict__ img1, const float* __restrict__ img2, const float* __restrict__ dL_dmap,
+    const float* __restrict__ dm_dmu1, const float* __restrict__ dm_dsigma1_sq, const float* __restrict__ dm_dsigma12,
+    float* __restrict__ dL_dimg1) {
+  __shared__ float s_p[3][kSsimHalo][kSsimHalo + 1];  // dL/dmap times each of the three partials
+  __shared__ float s_h[3][kSsimHalo][kSsimTile + 1];
+  const int x0 = blockIdx.x * kSsimTile, y0 = blockIdx.y * kSsimTile;
+  const size_t plane = (size_t) H * W;
+  float g[11];
+#pragma unroll
+  for (int k = 0; k < 11; ++k) g[k] = kGauss[k];
+
+  for (int c = 0; c < CH; ++c) {
+    const size_t off = ((size_t) blockIdx.z * CH + c) * plane;
+    for (int e = threadIdx.x; e < kSsimHalo * kSsimHalo; e += kSsimThreads) {
+      const int ly = e / kSsimHalo, lx = e - ly * kSsimHalo;
+      const int y = y0 + ly - 5, x = x0 + lx - 5;
+      const float gmap = pixel_or_zero(dL_dmap + off, y, x, H, W);
+      s_p[0][ly][lx] = pixel_or_zero(dm_dmu1 + off, y, x, H, W) * gmap;
+      s_p[1][ly][lx] = pixel_or_zero(dm_dsigma1_sq + off, y, x, H, W) * gmap;
+      s_p[2][ly][lx] = pixel_or_zero(dm_dsigma12 + off, y, x, H, W) * gmap;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < kSsimHalo * kSsimTile; e += kSsimThreads) {
+      const int ly = e / kSsimTile, lx = e - ly * kSsimTile;
+      float a0 = 0, a1 = 0, a2 = 0;
+#pragma unroll
+      for (int k = 0; k < 11; ++k)
+        a0 += g[k] * s_p[0][ly][lx + k], a1 += g[k] * s_p[1][ly][lx + k], a2 += g[k] * s_p[2][ly][lx + k];
+      s_h[0][ly][lx] = a0, s_h[1][ly][lx] = a1, s_h[2][ly][lx] = a2;
+    }
+    __syncthreads();
+    const int lx = threadIdx.x & 31;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int ly = (threadIdx.x >> 5) * 4 + r;
+      float a0 = 0, a1 = 0, a2 = 0;
+#pragma unroll
+      for (int k = 0; k < 11; ++k)
+        a0 += g[k] * s_h[0][ly + k][lx], a1 += g[k] * s_h[1][ly + k][lx], a2 += g[k] * s_h[2][ly + k][lx];
+      const int px = x0 + lx, py = y0 + ly;
+      if (px < W && py < H) {
+        const size_t idx = off + (size_t) py * W + px;
+        float grad = a0;
+        grad += img1[idx] * 2.0f * a1;
+        grad += img2[idx] * a2;
+        dL_dimg1[idx] = grad;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+}  // namespace
+}  // namespace fsgs
+
+using namespace fsgs;
+
+FSGS_API int fsgs_fusedssim_forward(int B, int CH, int H, int W, double C1, double C2, const float* img1,
+    const float* img2, float* ssim_map, float* dm_dmu1, float* dm_dsigma1_sq, float* dm_dsigma12, void* stream) {
+  FSGS_REQUIRE(B >= 0 && CH >= 0 && H >= 0 && W >= 0, "fusedssim: bad sizes");
+  if ((size_t) B * CH * H * W == 0) return kOk;
+  FSGS_REQUIRE(img1 && img2 && ssim_map, "fusedssim: null pointer");
+  const bool train = dm_dmu1 != nullptr;
+  FSGS_REQUIRE(!train || (dm_dsigma1_sq && dm_dsigma12), "fusedssim: the three partial-derivative maps go together");
+  FSGS_REQUIRE(B <= 65535, "fusedssim: batch %d exceeds the grid limit", B);
+  const dim3 grid(div_up(W, kSsimTile), div_up(H, kSsimTile), B), block(kSsimThreads);
+  if (train)
+    hipLaunchKernelGGL(ssim_forward_kernel<true>, grid, block, 0, (hipStream_t) stream, H, W, CH, (float) C1,
+                       (float) C2, img1, img2, ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12);
+  else
+    hipLaunchKernelGGL(ssim_forward_kernel<false>, grid, block, 0, (hipStream_t) stream, H, W, CH, (float) C1,
+                       (float) C2, img1, img2, ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12);
+  return check_launch("fusedssim");
+}
+
+FSGS_API int fsgs_fusedssim_backward(int B, int CH, int H, int W, const float* img1, const float* img2,
+    const float* dL_dmap, const float* dm_dmu1, const float* dm_dsigma1_sq, const float* dm_dsigma12,
+    float* dL_dimg1, void* stream) {
+  FSGS_REQUIRE(B >= 0 && CH >= 0 && H >= 0 && W >= 0, "fusedssim_backward: bad sizes");
+  if ((size_t) B * CH * H * W == 0) return kOk;
+  FSGS_REQUIRE(img1 && img2 && dL_dmap && dm_dmu1 && dm_dsigma1_sq && dm_dsigma12 && dL_dimg1,
+               "fusedssim_backward: null pointer");
+  FSGS_REQUIRE(B <= 65535, "fusedssim_backward: batch %d exceeds the grid limit", B);
+  const dim3 grid(div_up(W, kSsimTile), div_up(H, kSsimTile), B), block(kSsimThreads);
+  hipLaunchKernelGGL(ssim_backward_kernel, grid, block, 0, (hipStream_t) stream, H, W, CH, img1, img2, dL_dmap,
+                     dm_dmu1, dm_dsigma1_sq, dm_dsigma12, dL_dimg1);
+  return check_launch("fusedssim_backward");
+}

@@ -231,6 +231,18 @@ int fsgs_lbs_blend(int N, int M, int K, int centred, double temperature, const f
     const int64_t* index, float* weights_out, float* d_xyz, float* d_rot, float* d_scale, void* workspace,
     size_t workspace_bytes, void* stream);
 
+/* ---- fused SSIM ------------------------------------------------------------------------------------------------ */
+
+/* fusedssim -- fast_2d_gs/_C/src/other/structural_similarity.cu:340-363 (kernel :187-277). img1, img2, ssim_map and
+ * the three optional partial-derivative maps are [B,CH,H,W]; pass the three maps as NULL for train = false. Every
+ * output element is written. */
+int fsgs_fusedssim_forward(int B, int CH, int H, int W, double C1, double C2, const float* img1, const float* img2,
+    float* ssim_map, float* dm_dmu1, float* dm_dsigma1_sq, float* dm_dsigma12, void* stream);
+
+/* fusedssim_backward -- structural_similarity.cu:365-380 (kernel :279-338) -> dL_dimg1[B,CH,H,W], fully written. */
+int fsgs_fusedssim_backward(int B, int CH, int H, int W, const float* img1, const float* img2, const float* dL_dmap,
+    const float* dm_dmu1, const float* dm_dsigma1_sq, const float* dm_dsigma12, float* dL_dimg1, void* stream);
+
 /* Deformation MLP forward (bf16 MFMA, fp32 accumulate) -- fast_2d_gs/network.py:1757-1776 (SC_GS_DeformNetwork.forward,
  * fp32 there): n_layers x (Linear(256) + ReLU), input re-concatenated in front after layer `skip`, then n_out <= 32
  * linear outputs (the three heads stacked). in[B,Din] fp32 (already frequency-encoded), Din <= 96, width must be 256.

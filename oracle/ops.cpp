@@ -11,6 +11,7 @@
 //                            and the rigid transforms are lietorch.SE3 -- both un-vendored third-party packages with
 //                            no pinned version; their published semantics are restated and the tie order
 //                            "lower index first" is this build's definition: PARITY UNPINNED at that boundary)
+//   fused SSIM fwd/bwd       fast_2d_gs/_C/src/other/structural_similarity.cu:11-21, 187-338
 //   deformation MLP          fast_2d_gs/network.py:1670-1776 (8 x Linear(256)+ReLU, input re-concatenated after
 //                            layer 4, three linear heads)
 #include <algorithm>
@@ -315,6 +316,82 @@ static void deform_mlp(int B, int Din, int Wd, int L, int skip, const float* in,
   }
 }
 
+// ---- fused SSIM (structural_similarity.cu:11-21 weights, :187-277 forward, :279-338 backward) ----------------------
+// The weights are the reference's float literals; in the double instantiation they are those floats widened.
+static const float kSsimGauss[11] = {0.001028380123898387f, 0.0075987582094967365f, 0.036000773310661316f,
+                                     0.10936068743467331f,  0.21300552785396576f,   0.26601171493530273f,
+                                     0.21300552785396576f,  0.10936068743467331f,   0.036000773310661316f,
+                                     0.0075987582094967365f, 0.001028380123898387f};
+
+// Separable 11-tap filter of one zero-padded plane, x first then y, taps accumulated from 0 to 10 as the reference does.
+template <typename T, typename F>
+static void ssim_filter(int H, int W, F value, std::vector<T>& out) {
+  std::vector<T> tmp((size_t) H * W);
+  for (int y = 0; y < H; ++y)
+    for (int x = 0; x < W; ++x) {
+      T v = 0;
+      for (int k = 0; k < 11; ++k) {
+        const int xx = x + k - 5;
+        v += (T) kSsimGauss[k] * ((xx >= 0 && xx < W) ? value(y, xx) : T(0));
+      }
+      tmp[(size_t) y * W + x] = v;
+    }
+  out.assign((size_t) H * W, T(0));
+  for (int y = 0; y < H; ++y)
+    for (int x = 0; x < W; ++x) {
+      T v = 0;
+      for (int k = 0; k < 11; ++k) {
+        const int yy = y + k - 5;
+        v += (T) kSsimGauss[k] * ((yy >= 0 && yy < H) ? tmp[(size_t) yy * W + x] : T(0));
+      }
+      out[(size_t) y * W + x] = v;
+    }
+}
+
+template <typename T>
+static void fusedssim_forward(int B, int CH, int H, int W, T C1, T C2, const T* img1, const T* img2, T* map, T* dmu1,
+                              T* dsig1, T* dsig12) {
+  const size_t plane = (size_t) H * W;
+#pragma omp parallel for schedule(dynamic, 1)
+  for (int bc = 0; bc < B * CH; ++bc) {
+    const T* a = img1 + bc * plane;
+    const T* b = img2 + bc * plane;
+    std::vector<T> mu1, e11, mu2, e22, e12;
+    ssim_filter<T>(H, W, [&](int y, int x) { return a[(size_t) y * W + x]; }, mu1);
+    ssim_filter<T>(H, W, [&](int y, int x) { return a[(size_t) y * W + x] * a[(size_t) y * W + x]; }, e11);
+    ssim_filter<T>(H, W, [&](int y, int x) { return b[(size_t) y * W + x]; }, mu2);
+    ssim_filter<T>(H, W, [&](int y, int x) { return b[(size_t) y * W + x] * b[(size_t) y * W + x]; }, e22);
+    ssim_filter<T>(H, W, [&](int y, int x) { return a[(size_t) y * W + x] * b[(size_t) y * W + x]; }, e12);
+    for (size_t i = 0; i < plane; ++i) {
+      const T m1 = mu1[i], m2 = mu2[i];
+      const T s1 = e11[i] - m1 * m1, s2 = e22[i] - m2 * m2, s12 = e12[i] - m1 * m2;
+      const T C = T(2) * m1 * m2 + C1, D = T(2) * s12 + C2, A = m1 * m1 + m2 * m2 + C1, Bq = s1 + s2 + C2;
+      map[bc * plane + i] = (C * D) / (A * Bq);
+      if (dmu1) {
+        dmu1[bc * plane + i] = (m2 * T(2) * D) / (A * Bq) - (m2 * T(2) * C) / (A * Bq) -
+                               (m1 * T(2) * C * D) / (A * A * Bq) + (m1 * T(2) * C * D) / (A * Bq * Bq);
+        dsig1[bc * plane + i]  = (-C * D) / (A * Bq * Bq);
+        dsig12[bc * plane + i] = (T(2) * C) / (A * Bq);
+      }
+    }
+  }
+}
+
+template <typename T>
+static void fusedssim_backward(int B, int CH, int H, int W, const T* img1, const T* img2, const T* dL_dmap,
+                               const T* dmu1, const T* dsig1, const T* dsig12, T* dL_dimg1) {
+  const size_t plane = (size_t) H * W;
+#pragma omp parallel for schedule(dynamic, 1)
+  for (int bc = 0; bc < B * CH; ++bc) {
+    const size_t o = bc * plane;
+    std::vector<T> c0, c1, c2;
+    ssim_filter<T>(H, W, [&](int y, int x) { return dmu1[o + (size_t) y * W + x] * dL_dmap[o + (size_t) y * W + x]; }, c0);
+    ssim_filter<T>(H, W, [&](int y, int x) { return dsig1[o + (size_t) y * W + x] * dL_dmap[o + (size_t) y * W + x]; }, c1);
+    ssim_filter<T>(H, W, [&](int y, int x) { return dsig12[o + (size_t) y * W + x] * dL_dmap[o + (size_t) y * W + x]; }, c2);
+    for (size_t i = 0; i < plane; ++i) dL_dimg1[o + i] = c0[i] + img1[o + i] * T(2) * c1[i] + img2[o + i] * c2[i];
+  }
+}
+
 }  // namespace oracle
 
 using namespace oracle;
@@ -383,6 +460,20 @@ using namespace oracle;
 
 INSTANTIATE(f32, float)
 INSTANTIATE(f64, double)
+
+#define INSTANTIATE_SSIM(SUF, T)                                                                                     \
+  ORACLE_API int oracle_fusedssim_forward_##SUF(int B, int CH, int H, int W, double C1, double C2, const T* img1,    \
+      const T* img2, T* ssim_map, T* dm_dmu1, T* dm_dsigma1_sq, T* dm_dsigma12) {                                    \
+    fusedssim_forward<T>(B, CH, H, W, (T) C1, (T) C2, img1, img2, ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12);    \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_fusedssim_backward_##SUF(int B, int CH, int H, int W, const T* img1, const T* img2,          \
+      const T* dL_dmap, const T* dm_dmu1, const T* dm_dsigma1_sq, const T* dm_dsigma12, T* dL_dimg1) {               \
+    fusedssim_backward<T>(B, CH, H, W, img1, img2, dL_dmap, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, dL_dimg1);          \
+    return 0;                                                                                                        \
+  }
+INSTANTIATE_SSIM(f32, float)
+INSTANTIATE_SSIM(f64, double)
 
 ORACLE_API int oracle_deform_mlp_f32(int B, int Din, int Wd, int L, int skip, const float* in,
                                      const float* const* Ws, const float* const* bs, int n_heads,

@@ -40,6 +40,10 @@ int oracle_freq_encode_forward_f32(int B, int Din, int degree, int include_input
     float* out);
 int oracle_freq_encode_backward_f32(int B, int Din, int degree, int include_input, double scale, const float* grad,
     const float* outv, float* gin);
+int oracle_fusedssim_forward_f32(int B, int CH, int H, int W, double C1, double C2, const float* img1,
+    const float* img2, float* ssim_map, float* dm_dmu1, float* dm_dsigma1_sq, float* dm_dsigma12);
+int oracle_fusedssim_backward_f32(int B, int CH, int H, int W, const float* img1, const float* img2,
+    const float* dL_dmap, const float* dm_dmu1, const float* dm_dsigma1_sq, const float* dm_dsigma12, float* dL_dimg1);
 int oracle_cdist_top_forward_f32(int B, int N, int M, int D, int largest, const float* x, const float* y, float* dist,
     int64_t* index);
 int oracle_cdist_top_backward_f32(int B, int N, int M, int D, const float* p1, const float* p2, const float* dist,

@@ -180,3 +180,44 @@ def test_deform_mlp_matches_torch(oracle_mod):
     assert rc == 0
     for o, r in zip(outs, ref):
         assert (o - r).abs().max() < 1e-4
+
+
+def test_fusedssim_matches_conv2d_and_autograd(oracle_mod):
+    """The oracle's fused SSIM against the textbook form the reference keeps as its fallback (losses/ssim.py:49-67):
+    grouped conv2d with the normalised 11x11 Gaussian window (sigma 1.5, built here from its definition), zero padding;
+    the backward against autograd of that form. Sizes are not multiples of the 32-pixel blocks."""
+    import math
+    import torch.nn.functional as F
+    O = oracle_mod
+    B, CH, H, W = 2, 3, 45, 70
+    g = torch.Generator().manual_seed(0)
+    img1 = torch.rand(B, CH, H, W, generator=g, dtype=torch.float64, requires_grad=True)
+    img2 = torch.rand(B, CH, H, W, generator=g, dtype=torch.float64)
+    gmap = torch.randn(B, CH, H, W, generator=g, dtype=torch.float64)
+    w1 = torch.tensor([math.exp(-(x - 5) ** 2 / (2 * 1.5 ** 2)) for x in range(11)], dtype=torch.float64)
+    w1 = w1 / w1.sum()
+    win = (w1[:, None] * w1[None, :]).expand(CH, 1, 11, 11).contiguous()
+    C1, C2 = 0.01 ** 2, 0.03 ** 2
+    conv = lambda t: F.conv2d(t, win, padding=5, groups=CH)
+    mu1, mu2 = conv(img1), conv(img2)
+    s1, s2, s12 = conv(img1 * img1) - mu1 * mu1, conv(img2 * img2) - mu2 * mu2, conv(img1 * img2) - mu1 * mu2
+    ref = ((2 * mu1 * mu2 + C1) * (2 * s12 + C2)) / ((mu1 * mu1 + mu2 * mu2 + C1) * (s1 + s2 + C2))
+    (ref * gmap).sum().backward()
+
+    a, b = img1.detach().numpy().copy(), img2.numpy().copy()
+    out, d1, d2, d3 = (np.zeros_like(a) for _ in range(4))
+    assert O.call("fusedssim_forward_f64", B, CH, H, W, C1, C2, a, b, out, d1, d2, d3) == 0
+    # the kernel's weights are float literals: they differ from the exact Gaussian by float rounding
+    assert np.abs(out - ref.detach().numpy()).max() < 1e-6
+    grad = np.zeros_like(a)
+    assert O.call("fusedssim_backward_f64", B, CH, H, W, a, b, gmap.numpy().copy(), d1, d2, d3, grad) == 0
+    gref = img1.grad.numpy()
+    assert np.abs(grad - gref).max() < 1e-5 * np.abs(gref).max()
+    # without the partial-derivative maps only the SSIM map is produced
+    out2 = np.zeros_like(a)
+    assert O.call("fusedssim_forward_f64", B, CH, H, W, C1, C2, a, b, out2, None, None, None) == 0
+    assert np.array_equal(out, out2)
+    # identical images: SSIM is exactly 1 wherever the window is defined
+    same = np.zeros_like(a)
+    assert O.call("fusedssim_forward_f64", B, CH, H, W, C1, C2, a, a, same, None, None, None) == 0
+    assert np.abs(same - 1.0).max() < 1e-12
