@@ -288,7 +288,7 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": f"static 2DGS fwd+bwd: {P} surfels in the unit ball, {cam.W}x{cam.H}, FoV 40, radius 4, "
-                               "SH degree 3, white background, 16x16 tiles, key duplication + 64-bit radix sort + "
+                               "SH degree 3, white background, 16x16 tiles, per-tile binning of (tile, depth) keys + "
                                "depth/normal outputs",
                    "P": P, "P_visible": Pv, "R": R, "tiles": T},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",

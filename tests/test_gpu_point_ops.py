@@ -163,7 +163,7 @@ def test_sparse_adam(device, oracle_mod):
 
 
 def test_full_size_properties(device):
-    """BASELINE-size runs checked through size-independent properties (no oracle at this size)."""
+    """Full benchmark-size runs checked through size-independent properties (no oracle at this size)."""
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd._C import get_C_function
     c = scenes.config1(n_dirs=1_000_000, n_points=200_000, n_ctrl=512)
