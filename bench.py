@@ -99,7 +99,8 @@ def cpu_baseline(scene, cam, budget_s: float = 20.0):
 def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
     """Config 3 (dynamic scene, 200k surfels, 512 control points): bf16 MFMA deformation MLP on the control points ->
     K-NN (k = 4) -> LBS -> render forward -> 0.8 L1 + 0.2 (1 - SSIM) (fused SSIM kernel) -> render backward -> masked Adam
-    on the surfel parameters. The deformation branch is forward-only in this build (no MLP / LBS gradients)."""
+    on the surfel parameters + Adam on the MLP weights and the control points (gradients reach them through the LBS and
+    K-NN backward kernels and the MLP's fp32 GEMM backward)."""
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd.deform import DeformNetwork, superpoint_deform
     from fast_sp_gs_amd.renderer import GS_2D_render
@@ -108,10 +109,12 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
     scene_h, cam_h = scenes.config2(P=200_000, size=800, seed=2)
     scene, cam = scene_h.to(dev), cam_h.to(dev)
     g = torch.Generator().manual_seed(2)
-    ctrl = (torch.rand(512, 3, generator=g) * 2 - 1).to(dev)
+    ctrl = (torch.rand(512, 3, generator=g) * 2 - 1).to(dev).requires_grad_(True)
     target = torch.rand(3, cam.H, cam.W, generator=g).to(dev)
     net = DeformNetwork().to(dev)
-    net.pack()
+    # a tiny rate keeps the random-target synthetic scene from drifting (Adam's steps are |lr| whatever the gradient, and
+    # the scale residuals are added after the activation, network.py:643), so every timed step sees the same workload
+    net_opt = torch.optim.Adam(list(net.parameters()) + [ctrl], lr=1e-7)
     names = ('means3D', 'scales', 'rotations', 'opacities', 'shs')
     params = [getattr(scene, k).clone().requires_grad_(True) for k in names]
     opt = SparseGaussianAdam([{'params': [p_], 'name': k} for p_, k in zip(params, names)], lr=1.6e-4, eps=1e-15)
@@ -119,11 +122,12 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
 
     def step(i):
         t = torch.full((1,), (i % 17) / 17.0, device=dev)
-        c_xyz, c_rot, c_scale, _ = net(ctrl, t)
+        c_xyz, c_rot, c_scale, _ = net(ctrl.detach(), t)
         d_xyz, d_rot, d_scale, _, _ = superpoint_deform(params[0].detach(), ctrl, c_xyz.contiguous(),
                                                         c_rot.contiguous(), c_scale[:, :2].contiguous(), K=4,
                                                         temperature=0.01)
-        out = GS_2D_render(params[0] + d_xyz, params[1] + d_scale, params[2] + d_rot, params[3], (cam.W, cam.H),
+        out = GS_2D_render(params[0] + d_xyz, params[1] + d_scale, torch.nn.functional.normalize(params[2] + d_rot, dim=-1),
+                           params[3], (cam.W, cam.H),
                            cam.Tw2v, cam.Tv2c, campos=cam.campos, near=cam.near, far=cam.far, sh_degree=3,
                            sh_features=params[4])
         image = out['images'] + (1.0 - out['opacity']) * bg
@@ -132,6 +136,8 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
         opt.set_before_step(out['radii'] > 0, params[0].shape[0])
         opt.step()
         opt.zero_grad(set_to_none=True)
+        net_opt.step()
+        net_opt.zero_grad(set_to_none=True)
 
     for i in range(warmup):
         step(i)

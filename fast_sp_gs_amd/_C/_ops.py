@@ -19,6 +19,7 @@ __all__ = [
     'gs_2d_compute_trans_mat_backward', 'GS_prepare', 'GS_2D_render_forward', 'GS_2D_render_backward',
     'SH_to_RGB_forward', 'SH_to_RGB_backward', 'sh_encode_forward', 'sh_encode_backward', 'freq_encode_forward',
     'freq_encode_backward', 'cdist_top', 'cdist_top_backward', 'AdamMasksedUpdated', 'knn_topk', 'lbs_blend',
+    'knn_topk_backward', 'lbs_blend_backward',
     'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'gs_2d_pack_records', 'gs_2d_fast_preprocess_forward',
     'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward', 'gs_2d_fast_compute_trans_mat_backward',
     'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward', 'fusedssim', 'fusedssim_backward',
@@ -838,6 +839,63 @@ def lbs_blend(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_
                                 L.ptr(d_xyz), L.ptr(d_rot), L.ptr(d_scale), L.ptr(ws), ws.numel(), L.current_stream())
     L.check(rc, what)
     return d_xyz, d_rot, d_scale, weights
+
+
+def lbs_blend_backward(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_s: Optional[Tensor],
+                       dist2: Tensor, index: Tensor, grad_xyz: Tensor, grad_rot: Tensor, grad_scale: Optional[Tensor],
+                       temperature: float = 1.0, centred: bool = False, need_points: bool = True):
+    """Gradients of `lbs_blend` (what autograd gives for fast_2d_gs/network.py:517,545-573) ->
+    (g_points[N,3]|None, g_dist2[N,K], g_sp_points[M,3], g_sp_t[M,3], g_sp_r[M,4], g_sp_s[M,S]|None)."""
+    what = 'lbs_blend_backward'
+    _f32(what, points=points, sp_points=sp_points, sp_t=sp_t, sp_r=sp_r, sp_s=sp_s, dist2=dist2, grad_xyz=grad_xyz,
+         grad_rot=grad_rot, grad_scale=grad_scale)
+    L.require_cuda(what, index=index)
+    L.require_dtype(what, 'index', index, torch.int64)
+    N, K = dist2.shape
+    M = sp_points.shape[0]
+    S = 0 if sp_s is None else sp_s.shape[1]
+    if S and grad_scale is None:
+        raise RuntimeError(f'{what}: grad_scale is required when sp_s is given')
+    if tuple(grad_xyz.shape) != (N, 3) or tuple(grad_rot.shape) != (N, 4) or tuple(index.shape) != (N, K) or \
+            (S and tuple(grad_scale.shape) != (N, S)):
+        raise RuntimeError(f'{what}: gradient / index shapes do not match dist2 {tuple(dist2.shape)}')
+    opt = dict(dtype=torch.float32, device=points.device)
+    g_points = torch.empty((N, 3), **opt) if need_points else None
+    g_dist2 = torch.empty((N, K), **opt)
+    g_sp_points, g_sp_t, g_sp_r = torch.empty((M, 3), **opt), torch.empty((M, 3), **opt), torch.empty((M, 4), **opt)
+    g_sp_s = torch.empty((M, S), **opt) if S else None
+    lib = _lib()
+    ws = _workspace(lib.fsgs_lbs_blend_backward_workspace_bytes(N, M, S), points.device)
+    with _timed('lbs_blend_backward'):
+        rc = lib.fsgs_lbs_blend_backward(
+            N, M, K, int(bool(centred)), float(temperature), L.ptr(points), L.ptr(sp_points), L.ptr(sp_t), L.ptr(sp_r),
+            L.ptr(sp_s), S, L.ptr(dist2), L.ptr(index), L.ptr(grad_xyz), L.ptr(grad_rot), L.ptr(grad_scale),
+            L.ptr(g_points), L.ptr(g_dist2), L.ptr(g_sp_points), L.ptr(g_sp_t), L.ptr(g_sp_r), L.ptr(g_sp_s),
+            L.ptr(ws), ws.numel(), L.current_stream())
+    L.check(rc, what)
+    return g_points, g_dist2, g_sp_points, g_sp_t, g_sp_r, g_sp_s
+
+
+def knn_topk_backward(x: Tensor, y: Tensor, index: Tensor, grad_dist2: Tensor, need_x: bool = True):
+    """Gradients of `knn_topk`'s squared distances -> (g_x[N,D]|None, g_y[M,D])."""
+    what = 'knn_topk_backward'
+    _f32(what, x=x, y=y, grad_dist2=grad_dist2)
+    L.require_cuda(what, index=index)
+    L.require_dtype(what, 'index', index, torch.int64)
+    N, D = x.shape
+    M = y.shape[0]
+    K = index.shape[1]
+    if y.shape[1] != D or tuple(index.shape) != (N, K) or tuple(grad_dist2.shape) != (N, K):
+        raise RuntimeError(f'{what}: shapes do not match')
+    g_x = torch.empty_like(x) if need_x else None
+    g_y = torch.empty_like(y)
+    lib = _lib()
+    ws = _workspace(lib.fsgs_knn_topk_backward_workspace_bytes(N, M, D), x.device)
+    with _timed('knn_topk_backward'):
+        rc = lib.fsgs_knn_topk_backward(N, M, D, K, L.ptr(x), L.ptr(y), L.ptr(index), L.ptr(grad_dist2), L.ptr(g_x),
+                                        L.ptr(g_y), L.ptr(ws), ws.numel(), L.current_stream())
+    L.check(rc, what)
+    return g_x, g_y
 
 
 # --------------------------------------------------------------------------------------------------------------------

@@ -324,24 +324,32 @@ __global__ void __launch_bounds__(256) lbs_prepare_kernel(int M, int centred, co
   for (int k = 0; k < 3; ++k) xf[12 * j + 9 + k] = t[k];
 }
 
-__global__ void __launch_bounds__(256) lbs_blend_kernel(int N, int K, int S, float temperature,
+__global__ void __launch_bounds__(256) lbs_blend_kernel(int N, int M, int K, int S, float temperature,
     const float* __restrict__ points, const float* __restrict__ xf, const float* __restrict__ sp_r,
     const float* __restrict__ sp_s, const float* __restrict__ dist2, const int64_t* __restrict__ index,
     float* __restrict__ weights_out, float* __restrict__ d_xyz, float* __restrict__ d_rot,
     float* __restrict__ d_scale) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= N) return;
-  const float* d2 = dist2 + (size_t) n * K;
-  float mx = -d2[0] / temperature;
-  for (int k = 1; k < K; ++k) mx = fmaxf(mx, -d2[k] / temperature);
+  const float* d2   = dist2 + (size_t) n * K;
+  const int64_t* id = index + (size_t) n * K;
+  // slots without a neighbour (index -1 when K > M) take no part in the softmax
+  float mx = -__builtin_inff();
+  for (int k = 0; k < K; ++k)
+    if (id[k] >= 0 && id[k] < M) mx = fmaxf(mx, -d2[k] / temperature);
   float den = 0.0f;
-  for (int k = 0; k < K; ++k) den += expf(-d2[k] / temperature - mx);
+  for (int k = 0; k < K; ++k)
+    if (id[k] >= 0 && id[k] < M) den += expf(-d2[k] / temperature - mx);
   const float p[3] = {points[3 * (size_t) n], points[3 * (size_t) n + 1], points[3 * (size_t) n + 2]};
   float acc[3] = {0, 0, 0}, ar[4] = {0, 0, 0, 0}, as[4] = {0, 0, 0, 0};
   for (int k = 0; k < K; ++k) {
-    const float w   = expf(-d2[k] / temperature - mx) / den;
-    const int64_t j = index[(size_t) n * K + k];
-    const float* X  = xf + 12 * j;
+    const int64_t j = id[k];
+    if (j < 0 || j >= M) {
+      if (weights_out) weights_out[(size_t) n * K + k] = 0.0f;
+      continue;
+    }
+    const float w  = expf(-d2[k] / temperature - mx) / den;
+    const float* X = xf + 12 * j;
 #pragma unroll
     for (int a = 0; a < 3; ++a) acc[a] += w * (X[a * 3] * p[0] + X[a * 3 + 1] * p[1] + X[a * 3 + 2] * p[2] + X[9 + a]);
 #pragma unroll
@@ -520,7 +528,7 @@ FSGS_API int fsgs_lbs_blend(int N, int M, int K, int centred, double temperature
   hipStream_t s = (hipStream_t) stream;
   float* xf     = (float*) workspace;
   hipLaunchKernelGGL(lbs_prepare_kernel, dim3(div_up(M, 256)), dim3(256), 0, s, M, centred, sp_points, sp_t, sp_r, xf);
-  hipLaunchKernelGGL(lbs_blend_kernel, dim3(div_up(N, 256)), dim3(256), 0, s, N, K, S, (float) temperature, points, xf,
+  hipLaunchKernelGGL(lbs_blend_kernel, dim3(div_up(N, 256)), dim3(256), 0, s, N, M, K, S, (float) temperature, points, xf,
                      sp_r, sp_s, dist2, index, weights_out, d_xyz, d_rot, d_scale);
   return check_launch("lbs_blend");
 }

@@ -1,6 +1,8 @@
 """Host side of the superpoint deformation branch: frequency encoders + fused MFMA MLP, K-NN of Gaussians to control
-points, and LBS skinning -- the forward path of the reference's `SC_GS_DeformNetwork` (fast_2d_gs/network.py:1670-1776)
-and `calc_LBS_weight` / `warp` (network.py:498-573) on the HIP operators."""
+points, and LBS skinning -- the reference's `SC_GS_DeformNetwork` (fast_2d_gs/network.py:1670-1776) and
+`calc_LBS_weight` / `warp` (network.py:498-573) on the HIP operators, differentiable like the reference's torch code:
+K-NN distances and the LBS blend have HIP backward kernels; the MLP's backward re-runs its layers as fp32 library
+GEMMs (the bf16 MFMA kernel keeps no activations)."""
 from __future__ import annotations
 
 import math
@@ -56,10 +58,25 @@ class DeformNetwork(nn.Module):
         t_emb = self.pos_enc_t(t.view(-1, 1)).expand(x.shape[0], self.pos_enc_t.output_dim)
         return torch.cat([self.pos_enc_p(x), t_emb], dim=-1).contiguous()
 
-    @torch.no_grad()
+    def _mlp_parameters(self) -> List[Tensor]:
+        layers = list(self.linear) + [self.gaussian_warp, self.gaussian_rotation, self.gaussian_scaling]
+        return [p for l in layers for p in (l.weight, l.bias)]
+
     def forward(self, x: Tensor, t: Tensor):
-        packed, bias = self._packed if self._packed is not None else self.pack()
-        out = get_C_function('mlp_forward')(self.encode(x, t), packed, bias, self.D, self.skip, 10)
+        """bf16 MFMA forward. With gradients enabled the weights are re-packed when they changed since the last call
+        and the output carries a backward (see `_DeformMlp`); under `torch.no_grad()` the cached pack is used."""
+        params = self._mlp_parameters()
+        x_enc = self.encode(x, t)
+        track = torch.is_grad_enabled() and (x_enc.requires_grad or any(p.requires_grad for p in params))
+        versions = tuple(p._version for p in params)
+        if self._packed is None or (track and getattr(self, '_packed_versions', None) != versions):
+            self.pack()
+            self._packed_versions = versions
+        packed, bias = self._packed
+        if track:
+            out = _DeformMlp.apply(x_enc, packed, bias, self.D, self.skip, *params)
+        else:
+            out = get_C_function('mlp_forward')(x_enc.detach(), packed, bias, self.D, self.skip, 10)
         d_xyz, rotation, scaling = out[:, 0:3], out[:, 3:7], out[:, 7:10]
         return d_xyz, rotation, scaling, None
 
@@ -74,13 +91,88 @@ class DeformNetwork(nn.Module):
         return self.gaussian_warp(h), self.gaussian_rotation(h), self.gaussian_scaling(h), None
 
 
-@torch.no_grad()
+def _mlp_fp32(x0: Tensor, params: List[Tensor], D: int, skip: int) -> Tensor:
+    """The network of `DeformNetwork` as plain fp32 linears on explicit parameter tensors (weight, bias per layer, then
+    the three heads) -> [B, 10]."""
+    h = x0
+    for i in range(D):
+        h = torch.relu(torch.nn.functional.linear(h, params[2 * i], params[2 * i + 1]))
+        if i == skip:
+            h = torch.cat([x0, h], -1)
+    heads = [torch.nn.functional.linear(h, params[2 * (D + k)], params[2 * (D + k) + 1]) for k in range(3)]
+    return torch.cat(heads, -1)
+
+
+class _DeformMlp(torch.autograd.Function):
+    """Forward: the fused bf16 MFMA kernel. Backward: the same layers re-run in fp32 with torch's GEMMs under autograd
+    (activations are recomputed, none are saved by the forward), which yields the gradients of the fp32 network the
+    reference trains (network.py:1757-1776) at the current weights."""
+
+    @staticmethod
+    def forward(ctx, x_enc, packed, bias, D, skip, *params):
+        ctx.save_for_backward(x_enc, *params)
+        ctx.D, ctx.skip = D, skip
+        return get_C_function('mlp_forward')(x_enc, packed, bias, D, skip, 10)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x_enc, *params = ctx.saved_tensors
+        need = [ctx.needs_input_grad[0]] + list(ctx.needs_input_grad[5:])
+        with torch.enable_grad():
+            x = x_enc.detach().requires_grad_(need[0])
+            ps = [p.detach().requires_grad_(n) for p, n in zip(params, need[1:])]
+            out = _mlp_fp32(x, ps, ctx.D, ctx.skip)
+            wanted = [t for t, n in zip([x] + ps, need) if n]
+            got = iter(torch.autograd.grad(out, wanted, grad_out.contiguous(), allow_unused=True))
+        grads = [next(got) if n else None for n in need]
+        return (grads[0], None, None, None, None, *grads[1:])
+
+
+class _KnnTopk(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, y, K):
+        d2, idx = get_C_function('knn_topk')(x, y, K)
+        ctx.save_for_backward(x, y, idx)
+        ctx.mark_non_differentiable(idx)
+        return d2, idx
+
+    @staticmethod
+    def backward(ctx, g_d2, _):
+        x, y, idx = ctx.saved_tensors
+        g_x, g_y = get_C_function('knn_topk_backward')(x, y, idx, g_d2.contiguous(), ctx.needs_input_grad[0])
+        return g_x, (g_y if ctx.needs_input_grad[1] else None), None
+
+
+class _LbsBlend(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, points, sp_points, sp_t, sp_r, sp_s, d2, idx, temperature, centred):
+        d_xyz, d_rot, d_scale, w = get_C_function('lbs_blend')(points, sp_points, sp_t, sp_r, sp_s, d2, idx,
+                                                               temperature, centred)
+        ctx.save_for_backward(points, sp_points, sp_t, sp_r, sp_s, d2, idx)
+        ctx.temperature, ctx.centred = temperature, centred
+        ctx.mark_non_differentiable(w)
+        return d_xyz, d_rot, d_scale, w
+
+    @staticmethod
+    def backward(ctx, g_xyz, g_rot, g_scale, _):
+        points, sp_points, sp_t, sp_r, sp_s, d2, idx = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        g_points, g_d2, g_c, g_t, g_r, g_s = get_C_function('lbs_blend_backward')(
+            points, sp_points, sp_t, sp_r, sp_s, d2, idx, g_xyz.contiguous(), g_rot.contiguous(),
+            None if sp_s is None else g_scale.contiguous(), ctx.temperature, ctx.centred, need[0])
+        pick = lambda g, n: g if n else None
+        return (g_points, pick(g_c, need[1]), pick(g_t, need[2]), pick(g_r, need[3]), pick(g_s, need[4]),
+                pick(g_d2, need[5]), None, None, None)
+
+
 def superpoint_deform(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_s: Tensor, K: int = 4,
                       temperature: float = 1.0, centred: bool = False):
     """K-NN of Gaussians to control points, `softmax(-d^2 / temperature)` weights (LBS_method='dist', network.py:517) and
-    the LBS warp (network.py:545-573). Returns (d_xyz, d_rot, d_scale, weights, indices)."""
-    d2, idx = get_C_function('knn_topk')(points, sp_points, K)
-    d_xyz, d_rot, d_scale, w = get_C_function('lbs_blend')(points, sp_points, sp_t.contiguous(), sp_r.contiguous(),
-                                                           None if sp_s is None else sp_s.contiguous(), d2, idx,
-                                                           temperature, centred)
+    the LBS warp (network.py:545-573). Returns (d_xyz, d_rot, d_scale, weights, indices). Differentiable with respect to
+    points, sp_points (through the distances and, when centred, the pivot), sp_t, sp_r and sp_s; the returned weights
+    are detached. The reference detaches `points` before this stage (network.py:577)."""
+    d2, idx = _KnnTopk.apply(points.contiguous(), sp_points.contiguous(), K)
+    d_xyz, d_rot, d_scale, w = _LbsBlend.apply(points.contiguous(), sp_points.contiguous(), sp_t.contiguous(),
+                                               sp_r.contiguous(), None if sp_s is None else sp_s.contiguous(), d2, idx,
+                                               temperature, centred)
     return d_xyz, d_rot, d_scale, w, idx

@@ -231,6 +231,26 @@ int fsgs_lbs_blend(int N, int M, int K, int centred, double temperature, const f
     const int64_t* index, float* weights_out, float* d_xyz, float* d_rot, float* d_scale, void* workspace,
     size_t workspace_bytes, void* stream);
 
+/* Backward of fsgs_lbs_blend. The reference has no kernel for it: torch autograd differentiates
+ * fast_2d_gs/network.py:517 and :545-573 op by op. Inputs as in the forward plus g_xyz[N,3], g_rot[N,4], g_scale[N,S].
+ * Every output element is written: g_points[N,3] (optional), g_dist2[N,K], g_sp_points[M,3] (optional; zero unless
+ * centred), g_sp_t[M,3], g_sp_r[M,4], g_sp_s[M,S]. Per-control-point sums use LDS float atomics inside a block and a
+ * fixed order across blocks while M * (16 + S) <= 36864, device-scope float atomics beyond; either way the last bits
+ * of the per-control-point outputs can differ between runs. */
+size_t fsgs_lbs_blend_backward_workspace_bytes(int N, int M, int S);
+int fsgs_lbs_blend_backward(int N, int M, int K, int centred, double temperature, const float* points,
+    const float* sp_points, const float* sp_t, const float* sp_r, const float* sp_s, int S, const float* dist2,
+    const int64_t* index, const float* g_xyz, const float* g_rot, const float* g_scale, float* g_points,
+    float* g_dist2, float* g_sp_points, float* g_sp_t, float* g_sp_r, float* g_sp_s, void* workspace,
+    size_t workspace_bytes, void* stream);
+
+/* Backward of fsgs_knn_topk's squared distances (what autograd through pytorch3d.ops.knn_points gives at
+ * fast_2d_gs/network.py:504): g_x[N,D] (optional) = sum_k 2 g_dist2[n,k] (x_n - y_index), g_y[M,D] = minus the same
+ * summed over the queries that selected the row. Slots with index -1 are skipped. Both outputs fully written. */
+size_t fsgs_knn_topk_backward_workspace_bytes(int N, int M, int D);
+int fsgs_knn_topk_backward(int N, int M, int D, int K, const float* x, const float* y, const int64_t* index,
+    const float* g_dist2, float* g_x, float* g_y, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- fused SSIM ------------------------------------------------------------------------------------------------ */
 
 /* fusedssim -- fast_2d_gs/_C/src/other/structural_similarity.cu:340-363 (kernel :187-277). img1, img2, ssim_map and

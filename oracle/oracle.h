@@ -54,6 +54,12 @@ int oracle_knn_topk_f32(int N, int M, int D, int K, const float* x, const float*
 int oracle_lbs_blend_f32(int N, int M, int K, int centred, double temperature, const float* points,
     const float* sp_points, const float* sp_t, const float* sp_r, const float* sp_s, int S, const float* dist2,
     const int64_t* index, float* weights_out, float* d_xyz, float* d_rot, float* d_scale);
+int oracle_lbs_blend_backward_f32(int N, int M, int K, int centred, double temperature, const float* points,
+    const float* sp_points, const float* sp_t, const float* sp_r, const float* sp_s, int S, const float* dist2,
+    const int64_t* index, const float* g_xyz, const float* g_rot, const float* g_scale, float* g_points,
+    float* g_dist2, float* g_sp_points, float* g_sp_t, float* g_sp_r, float* g_sp_s);
+int oracle_knn_topk_backward_f32(int N, int M, int D, int K, const float* x, const float* y, const int64_t* index,
+    const float* g_dist2, float* g_x, float* g_y);
 int64_t oracle_gs_prepare_count(int P, const int32_t* tiles_touched, int64_t* offsets);
 int oracle_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
     const int64_t* offsets, int64_t R, int64_t* ranges, int32_t* point_list, int64_t* keys_sorted_out);

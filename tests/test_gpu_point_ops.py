@@ -133,6 +133,111 @@ def test_knn_and_lbs(device, oracle_mod, c1):
         assert abs_err(npy(dr), rr) < 1e-5 and abs_err(npy(ds), rs) < 1e-6
 
 
+def _lbs_backward_case(O, device, pts, ctrl, sp_t, sp_r, sp_s, K, tau, centred, seed):
+    from fast_sp_gs_amd._C import get_C_function
+    N, M = pts.shape[0], ctrl.shape[0]
+    S = 0 if sp_s is None else sp_s.shape[1]
+    g = torch.Generator().manual_seed(seed)
+    gx, gr = torch.randn(N, 3, generator=g), torch.randn(N, 4, generator=g)
+    gs = torch.randn(N, S, generator=g) if S else None
+    d = lambda t: None if t is None else t.to(device).contiguous()
+    d2, idx = get_C_function('knn_topk')(d(pts), d(ctrl), K)
+    print(f"[lbs backward] N={N} M={M} K={K} S={S} centred={centred}", flush=True)
+    out = get_C_function('lbs_blend_backward')(d(pts), d(ctrl), d(sp_t), d(sp_r), d(sp_s), d2, idx, d(gx), d(gr),
+                                               d(gs), tau, centred)
+    torch.cuda.synchronize()
+    z = lambda *shape: np.zeros(shape, np.float32)
+    ref = [z(N, 3), z(N, K), z(M, 3), z(M, 3), z(M, 4), z(M, max(S, 1))]
+    O.call("lbs_blend_backward_f32", N, M, K, int(centred), tau, npy(pts), npy(ctrl), npy(sp_t), npy(sp_r),
+           None if sp_s is None else npy(sp_s), S, npy(d2), npy(idx), npy(gx), npy(gr), None if gs is None else npy(gs),
+           *ref)
+    names = ('points', 'dist2', 'sp_points', 'sp_t', 'sp_r', 'sp_s')
+    for name, a, b in zip(names, out, ref):
+        if a is None:
+            continue
+        # sums of thousands of fp32 terms in a different association than the oracle's running sum
+        assert rel_err(npy(a), b) < 2e-4, (name, rel_err(npy(a), b))
+    # the squared-distance gradient continues into both point sets
+    gd = out[1]
+    g_x, g_y = get_C_function('knn_topk_backward')(d(pts), d(ctrl), idx, gd)
+    torch.cuda.synchronize()
+    rx, ry = z(N, 3), z(M, 3)
+    O.call("knn_topk_backward_f32", N, M, 3, K, npy(pts), npy(ctrl), npy(idx), npy(gd), rx, ry)
+    assert rel_err(npy(g_x), rx) < 1e-5 and rel_err(npy(g_y), ry) < 2e-4
+
+
+def test_lbs_and_knn_backward(device, oracle_mod, c1):
+    O = oracle_mod
+    pts, ctrl = c1['points'][:30011], c1['ctrl']
+    for centred in (False, True):
+        _lbs_backward_case(O, device, pts, ctrl, c1['sp_t'], c1['sp_r'], c1['sp_s'], 4, 0.01, centred, seed=21)
+    g = torch.Generator().manual_seed(22)
+    # no scale residuals, K = 8, fewer points than one block
+    small_ctrl = torch.rand(40, 3, generator=g) * 2 - 1
+    _lbs_backward_case(O, device, pts[:100], small_ctrl, 0.1 * torch.randn(40, 3, generator=g),
+                       0.2 * torch.randn(40, 4, generator=g), None, 8, 0.05, True, seed=23)
+    # more neighbours asked for than control points exist: the padded slots (index -1) carry nothing
+    tiny_ctrl = torch.rand(3, 3, generator=g) * 2 - 1
+    _lbs_backward_case(O, device, pts[:500], tiny_ctrl, 0.1 * torch.randn(3, 3, generator=g),
+                       0.2 * torch.randn(3, 4, generator=g), 0.1 * torch.randn(3, 2, generator=g), 5, 0.05, False,
+                       seed=24)
+    # a control set whose table exceeds LDS takes the atomic path
+    big_ctrl = torch.rand(2500, 3, generator=g) * 2 - 1
+    _lbs_backward_case(O, device, pts[:20000], big_ctrl, 0.1 * torch.randn(2500, 3, generator=g),
+                       0.2 * torch.randn(2500, 4, generator=g), 0.1 * torch.randn(2500, 2, generator=g), 4, 0.01, True,
+                       seed=25)
+
+
+def test_deform_branch_autograd(device):
+    """superpoint_deform and the MLP are differentiable end to end: gradients through the HIP backward kernels equal
+    torch autograd of the same formulas written with torch ops on the device."""
+    from fast_sp_gs_amd.deform import DeformNetwork, superpoint_deform
+    g = torch.Generator().manual_seed(31)
+    N, M, K, tau = 5000, 64, 4, 0.02
+    pts = (torch.rand(N, 3, generator=g) * 2 - 1).to(device)
+    ctrl = (torch.rand(M, 3, generator=g) * 2 - 1).to(device).requires_grad_()
+    net = DeformNetwork().to(device)
+    for head in (net.gaussian_warp, net.gaussian_rotation, net.gaussian_scaling):
+        torch.nn.init.normal_(head.weight, std=0.05)  # the default 1e-5 would make every gradient vanish
+    t = torch.full((1,), 0.3, device=device)
+    gx, gr, gs = (torch.randn(N, c, generator=g).to(device) for c in (3, 4, 2))
+
+    def loss_of(d_xyz, d_rot, d_scale):
+        return (d_xyz * gx).sum() + (d_rot * gr).sum() + (d_scale * gs).sum()
+
+    c_xyz, c_rot, c_scale, _ = net(ctrl.detach(), t)
+    assert c_xyz.requires_grad
+    d_xyz, d_rot, d_scale, w, idx = superpoint_deform(pts, ctrl, c_xyz, c_rot, c_scale[:, :2], K=K, temperature=tau,
+                                                      centred=True)
+    params = list(net.parameters())
+    grads = torch.autograd.grad(loss_of(d_xyz, d_rot, d_scale), [ctrl] + params, allow_unused=True)
+
+    # the same computation with torch ops (fp32 network, explicit softmax / rotation / blend)
+    r_xyz, r_rot, r_scale, _ = net.forward_fp32(ctrl.detach(), t)
+    diff = pts[:, None, :] - ctrl[idx]
+    wt = torch.softmax(-(diff * diff).sum(-1) / tau, -1)
+    q = r_rot + torch.tensor([0, 0, 0, 1.0], device=device)
+    q = q / q.norm(dim=-1, keepdim=True)
+    x, y, z, s = q.unbind(-1)
+    R = torch.stack([1 - 2 * (y * y + z * z), 2 * (x * y - z * s), 2 * (y * s + x * z),
+                     2 * (x * y + z * s), 1 - 2 * (x * x + z * z), 2 * (y * z - x * s),
+                     2 * (x * z - y * s), 2 * (x * s + y * z), 1 - 2 * (x * x + y * y)], -1).view(M, 3, 3)
+    tt = r_xyz + ctrl - torch.einsum('mab,mb->ma', R, ctrl)
+    moved = torch.einsum('nkab,nb->nka', R[idx], pts) + tt[idx]
+    e_xyz = (wt[..., None] * moved).sum(1) - pts
+    e_rot = (wt[..., None] * r_rot[idx]).sum(1)
+    e_scale = (wt[..., None] * r_scale[:, :2][idx]).sum(1)
+    assert float((e_xyz - d_xyz).abs().max()) < 2e-2 * float(e_xyz.abs().max())  # bf16 forward
+    ref = torch.autograd.grad(loss_of(e_xyz, e_rot, e_scale), [ctrl] + params, allow_unused=True)
+    for name, a, b in zip(['sp_points'] + [n for n, _ in net.named_parameters()], grads, ref):
+        assert (a is None) == (b is None), name
+        if a is None:
+            continue
+        scale = float(b.abs().max())
+        # the HIP forward runs the layers in bf16, so the values the chain rule is evaluated at differ by ~1e-2 rel
+        assert float((a - b).abs().max()) <= 5e-2 * scale + 1e-12, (name, float((a - b).abs().max()), scale)
+
+
 def test_sparse_adam(device, oracle_mod):
     O = oracle_mod
     from fast_sp_gs_amd.sparse_gaussian_adam import SparseGaussianAdam

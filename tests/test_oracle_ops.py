@@ -102,6 +102,61 @@ def test_lbs_closed_forms(oracle_mod):
     assert np.abs(dx - ((pts - ctrl[5]) @ Rm.T + ctrl[5] + t - pts)).max() < 1e-12
 
 
+def test_lbs_and_knn_backward_match_autograd(oracle_mod):
+    """The oracle's hand-derived LBS / K-NN gradients against torch autograd (fp64) of the forward written a different
+    way: rotation through Rodrigues' form R = (w^2 - v.v) I + 2 v v^T + 2 w [v]x of the normalised quaternion, weights
+    through torch.softmax, distances through explicit differences."""
+    O = oracle_mod
+    g = torch.Generator().manual_seed(12)
+    N, M, K, S, tau = 70, 9, 4, 2, 0.05
+    for centred in (False, True):
+        pts = torch.randn(N, 3, generator=g, dtype=torch.float64, requires_grad=True)
+        ctrl = torch.randn(M, 3, generator=g, dtype=torch.float64, requires_grad=True)
+        sp_t = (0.2 * torch.randn(M, 3, generator=g, dtype=torch.float64)).requires_grad_()
+        sp_r = (0.4 * torch.randn(M, 4, generator=g, dtype=torch.float64)).requires_grad_()
+        sp_s = (0.1 * torch.randn(M, S, generator=g, dtype=torch.float64)).requires_grad_()
+        with torch.no_grad():
+            idx = torch.cdist(pts, ctrl).topk(K, largest=False).indices.contiguous()
+        diff = pts[:, None, :] - ctrl[idx]
+        d2 = (diff * diff).sum(-1)
+        d2_leaf = d2.detach().clone().requires_grad_()
+        w = torch.softmax(-d2_leaf / tau, -1)
+        q = sp_r + torch.tensor([0, 0, 0, 1.0], dtype=torch.float64)
+        q = q / q.norm(dim=-1, keepdim=True)
+        v, s = q[:, :3], q[:, 3:]
+        zero = torch.zeros(M, dtype=torch.float64)
+        skew = torch.stack([zero, -v[:, 2], v[:, 1], v[:, 2], zero, -v[:, 0], -v[:, 1], v[:, 0], zero], -1).view(M, 3, 3)
+        eye = torch.eye(3, dtype=torch.float64)
+        R = (s * s - (v * v).sum(-1, keepdim=True))[..., None] * eye + 2 * v[:, :, None] * v[:, None, :] + \
+            2 * s[..., None] * skew
+        t = sp_t + ctrl - torch.einsum('mab,mb->ma', R, ctrl) if centred else sp_t
+        moved = torch.einsum('nkab,nb->nka', R[idx], pts) + t[idx]
+        d_xyz = (w[..., None] * moved).sum(1) - pts
+        d_rot = (w[..., None] * sp_r[idx]).sum(1)
+        d_scale = (w[..., None] * sp_s[idx]).sum(1)
+        gx, gr, gs = (torch.randn(*t_.shape, generator=g, dtype=torch.float64) for t_ in (d_xyz, d_rot, d_scale))
+        loss = (d_xyz * gx).sum() + (d_rot * gr).sum() + (d_scale * gs).sum()
+        a_pts, a_d2, a_ctrl, a_t, a_r, a_s = torch.autograd.grad(loss, [pts, d2_leaf, ctrl, sp_t, sp_r, sp_s],
+                                                                  allow_unused=True)
+        n = lambda x: np.ascontiguousarray(x.detach().numpy())
+        o_pts, o_d2, o_ctrl = np.zeros((N, 3)), np.zeros((N, K)), np.zeros((M, 3))
+        o_t, o_r, o_s = np.zeros((M, 3)), np.zeros((M, 4)), np.zeros((M, S))
+        assert O.call("lbs_blend_backward_f64", N, M, K, int(centred), tau, n(pts), n(ctrl), n(sp_t), n(sp_r), n(sp_s),
+                      S, n(d2), n(idx), n(gx), n(gr), n(gs), o_pts, o_d2, o_ctrl, o_t, o_r, o_s) == 0
+        a_ctrl = torch.zeros(M, 3, dtype=torch.float64) if a_ctrl is None else a_ctrl
+        for name, a, o in (("points", a_pts, o_pts), ("dist2", a_d2, o_d2), ("sp_points", a_ctrl, o_ctrl),
+                           ("sp_t", a_t, o_t), ("sp_r", a_r, o_r), ("sp_s", a_s, o_s)):
+            scale = max(float(a.abs().max()), 1e-30)
+            assert np.abs(n(a) - o).max() < 1e-11 * max(scale, 1.0), (centred, name)
+        assert centred or not o_ctrl.any()
+        # K-NN distances: gradient of sum(g * d2) w.r.t. both point sets
+        gd = torch.randn(N, K, generator=g, dtype=torch.float64)
+        k_x, k_y = torch.autograd.grad((d2 * gd).sum(), [pts, ctrl])
+        o_x, o_y = np.zeros((N, 3)), np.zeros((M, 3))
+        assert O.call("knn_topk_backward_f64", N, M, 3, K, n(pts), n(ctrl), n(idx), n(gd), o_x, o_y) == 0
+        assert np.abs(n(k_x) - o_x).max() < 1e-12 and np.abs(n(k_y) - o_y).max() < 1e-12
+
+
 def test_masked_adam_matches_torch_adam(oracle_mod):
     O = oracle_mod
     rng = np.random.default_rng(4)
