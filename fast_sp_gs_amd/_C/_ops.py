@@ -20,7 +20,7 @@ __all__ = [
     'SH_to_RGB_forward', 'SH_to_RGB_backward', 'sh_encode_forward', 'sh_encode_backward', 'freq_encode_forward',
     'freq_encode_backward', 'cdist_top', 'cdist_top_backward', 'AdamMasksedUpdated', 'knn_topk', 'lbs_blend',
     'knn_topk_backward', 'lbs_blend_backward',
-    'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'gs_2d_pack_records', 'gs_2d_fast_preprocess_forward',
+    'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'mlp_pack_transposed', 'mlp_backward', 'gs_2d_pack_records', 'gs_2d_fast_preprocess_forward',
     'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward', 'gs_2d_fast_compute_trans_mat_backward',
     'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward', 'fusedssim', 'fusedssim_backward',
 ]
@@ -900,8 +900,9 @@ def knn_topk_backward(x: Tensor, y: Tensor, index: Tensor, grad_dist2: Tensor, n
 
 # --------------------------------------------------------------------------------------------------------------------
 def mlp_pack_weights(weights: List[Tensor], head_weights: Tensor, skip: int) -> Tensor:
-    """bf16 weight buffer of the fused deformation MLP: layer i as [256][round_up(K_i, 16)], then the stacked heads as
-    [32][256]. `weights` are torch.nn.Linear weights [256, K_i] in layer order (network.py:1723-1727)."""
+    """bf16 weight buffer of the fused deformation MLP: layer i as a [256][round_up(K_i, 16)] matrix, then the stacked
+    heads as [32][256], each in the tile order the matrix cores read (see fsgs_pack_bf16). `weights` are torch.nn.Linear
+    weights [256, K_i] in layer order (network.py:1723-1727)."""
     what = 'mlp_pack_weights'
     _f32(what, head_weights=head_weights, **{f'w{i}': w for i, w in enumerate(weights)})
     Din, n_layers = weights[0].shape[1], len(weights)
@@ -927,9 +928,11 @@ def mlp_pack_weights(weights: List[Tensor], head_weights: Tensor, skip: int) -> 
     return packed
 
 
-def mlp_forward(inputs: Tensor, packed: Tensor, bias: Tensor, n_layers: int, skip: int, n_out: int) -> Tensor:
+def mlp_forward(inputs: Tensor, packed: Tensor, bias: Tensor, n_layers: int, skip: int, n_out: int,
+                save: bool = False):
     """Fused n_layers x (Linear(256)+ReLU) + heads forward on the matrix cores (bf16 in, fp32 accumulate);
-    network.py:1757-1776. inputs[B,Din] fp32, bias[n_layers*256 + n_out] fp32 -> out[B,n_out] fp32."""
+    network.py:1757-1776. inputs[B,Din] fp32, bias[n_layers*256 + n_out] fp32 -> out[B,n_out] fp32; with `save` also
+    the [n_layers,B,256] bf16 (stored as int16) post-ReLU states that `mlp_backward` needs -> (out, saved)."""
     what = 'mlp_forward'
     _f32(what, inputs=inputs, bias=bias)
     L.require_cuda(what, packed=packed)
@@ -939,12 +942,55 @@ def mlp_forward(inputs: Tensor, packed: Tensor, bias: Tensor, n_layers: int, ski
     if packed.numel() != _lib().fsgs_mlp_packed_elems(Din, n_layers, skip):
         raise RuntimeError(f'{what}: packed weight buffer has the wrong size')
     out = torch.empty((B, n_out), dtype=torch.float32, device=inputs.device)
+    saved = torch.empty((n_layers, B, 256), dtype=torch.int16, device=inputs.device) if save else None
     with _timed('mlp_forward'):
         rc = _lib().fsgs_mlp_forward(B, Din, 256, n_layers, skip, n_out, L.ptr(inputs),
                                      L.ptr(packed), L.ptr(bias),
-                                     L.ptr(out), L.current_stream())
+                                     L.ptr(out), L.ptr(saved), L.current_stream())
     L.check(rc, what)
-    return out
+    return (out, saved) if save else out
+
+
+def mlp_pack_transposed(weights: List[Tensor]) -> Tensor:
+    """bf16 copy, transposed to [256 in][256 out], of the last 256 input columns of every layer's weight except the
+    first: what `mlp_backward` multiplies dZ with. -> int16 [n_layers-1, 256, 256]."""
+    what = 'mlp_pack_transposed'
+    _f32(what, **{f'w{i}': w for i, w in enumerate(weights)})
+    n = len(weights) - 1
+    packed_t = torch.empty((max(n, 1), 256, 256), dtype=torch.int16, device=weights[0].device)
+    if n > 0:
+        src = torch.stack([w[:, -256:].t() for w in weights[1:]]).contiguous()
+        rc = _lib().fsgs_pack_bf16(n * 256, 256, n * 256, 256, L.ptr(src), L.ptr(packed_t), L.current_stream())
+        L.check(rc, what)
+    return packed_t
+
+
+def mlp_backward(inputs: Tensor, packed_t: Tensor, head_weights: Tensor, saved: Tensor, grad_out: Tensor,
+                 n_layers: int, skip: int) -> Tuple[Tensor, Tensor]:
+    """Weight and bias gradients of `mlp_forward` (autograd through nn.Linear / relu in the reference,
+    network.py:1757-1776) -> (g_w flat: layers' [256,K_l] back to back then heads [n_out,256]; g_b[n_layers*256+n_out])."""
+    what = 'mlp_backward'
+    _f32(what, inputs=inputs, head_weights=head_weights, grad_out=grad_out)
+    L.require_cuda(what, packed_t=packed_t, saved=saved)
+    B, Din = inputs.shape
+    n_out = head_weights.shape[0]
+    if tuple(saved.shape) != (n_layers, B, 256) or saved.dtype != torch.int16:
+        raise RuntimeError(f'{what}: saved must be the int16 [{n_layers},{B},256] tensor mlp_forward(save=True) returned')
+    if tuple(grad_out.shape) != (B, n_out) or head_weights.shape[1] != 256:
+        raise RuntimeError(f'{what}: grad_out / head_weights shapes do not match')
+    if packed_t.numel() < max(n_layers - 1, 1) * 65536:
+        raise RuntimeError(f'{what}: packed_t is too small for {n_layers} layers')
+    n_w = 256 * Din + (n_layers - 1) * 65536 + 256 * Din + n_out * 256
+    g = torch.empty((n_w + n_layers * 256 + n_out,), dtype=torch.float32, device=inputs.device)
+    g_w, g_b = g[:n_w], g[n_w:]
+    lib = _lib()
+    ws = _workspace(lib.fsgs_mlp_backward_workspace_bytes(B, n_layers), inputs.device)
+    with _timed('mlp_backward'):
+        rc = lib.fsgs_mlp_backward(B, Din, 256, n_layers, skip, n_out, L.ptr(inputs), L.ptr(packed_t),
+                                   L.ptr(head_weights), L.ptr(saved), L.ptr(grad_out), L.ptr(g_w), L.ptr(g_b),
+                                   L.ptr(ws), ws.numel(), L.current_stream())
+    L.check(rc, what)
+    return g_w, g_b
 
 
 # --------------------------------------------------------------------------------------------------------------------

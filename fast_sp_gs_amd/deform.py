@@ -1,8 +1,7 @@
 """Host side of the superpoint deformation branch: frequency encoders + fused MFMA MLP, K-NN of Gaussians to control
 points, and LBS skinning -- the reference's `SC_GS_DeformNetwork` (fast_2d_gs/network.py:1670-1776) and
 `calc_LBS_weight` / `warp` (network.py:498-573) on the HIP operators, differentiable like the reference's torch code:
-K-NN distances and the LBS blend have HIP backward kernels; the MLP's backward re-runs its layers as fp32 library
-GEMMs (the bf16 MFMA kernel keeps no activations)."""
+K-NN distances, the LBS blend and the MLP (bf16 MFMA, fp32 accumulation) all have HIP backward kernels."""
 from __future__ import annotations
 
 import math
@@ -52,6 +51,8 @@ class DeformNetwork(nn.Module):
         packed = get_C_function('mlp_pack_weights')(weights, heads_w.detach().contiguous(), self.skip)
         bias = torch.cat([l.bias.detach() for l in self.linear] + [heads_b.detach()]).contiguous()
         self._packed = (packed, bias)
+        self._packed_t = None  # transposed copy for the backward, made on demand
+        self._heads_w = heads_w.detach().contiguous()
         return self._packed
 
     def encode(self, x: Tensor, t: Tensor) -> Tensor:
@@ -74,7 +75,9 @@ class DeformNetwork(nn.Module):
             self._packed_versions = versions
         packed, bias = self._packed
         if track:
-            out = _DeformMlp.apply(x_enc, packed, bias, self.D, self.skip, *params)
+            if self._packed_t is None:
+                self._packed_t = get_C_function('mlp_pack_transposed')([l.weight.detach() for l in self.linear])
+            out = _DeformMlp.apply(x_enc, packed, bias, self._packed_t, self._heads_w, self.D, self.skip, *params)
         else:
             out = get_C_function('mlp_forward')(x_enc.detach(), packed, bias, self.D, self.skip, 10)
         d_xyz, rotation, scaling = out[:, 0:3], out[:, 3:7], out[:, 7:10]
@@ -91,41 +94,35 @@ class DeformNetwork(nn.Module):
         return self.gaussian_warp(h), self.gaussian_rotation(h), self.gaussian_scaling(h), None
 
 
-def _mlp_fp32(x0: Tensor, params: List[Tensor], D: int, skip: int) -> Tensor:
-    """The network of `DeformNetwork` as plain fp32 linears on explicit parameter tensors (weight, bias per layer, then
-    the three heads) -> [B, 10]."""
-    h = x0
-    for i in range(D):
-        h = torch.relu(torch.nn.functional.linear(h, params[2 * i], params[2 * i + 1]))
-        if i == skip:
-            h = torch.cat([x0, h], -1)
-    heads = [torch.nn.functional.linear(h, params[2 * (D + k)], params[2 * (D + k) + 1]) for k in range(3)]
-    return torch.cat(heads, -1)
-
-
 class _DeformMlp(torch.autograd.Function):
-    """Forward: the fused bf16 MFMA kernel. Backward: the same layers re-run in fp32 with torch's GEMMs under autograd
-    (activations are recomputed, none are saved by the forward), which yields the gradients of the fp32 network the
-    reference trains (network.py:1757-1776) at the current weights."""
+    """Forward: the fused bf16 MFMA kernel, which also stores every layer's post-ReLU state. Backward: the chain and
+    weight-gradient MFMA kernels; gradients come back in one flat buffer and are handed out as views in parameter
+    order (weight, bias per layer, then the warp / rotation / scaling heads). The encoded input gets no gradient (the
+    reference feeds detached control points, network.py:586)."""
 
     @staticmethod
-    def forward(ctx, x_enc, packed, bias, D, skip, *params):
-        ctx.save_for_backward(x_enc, *params)
+    def forward(ctx, x_enc, packed, bias, packed_t, heads_w, D, skip, *params):
+        out, saved = get_C_function('mlp_forward')(x_enc, packed, bias, D, skip, 10, True)
+        ctx.save_for_backward(x_enc, packed_t, heads_w, saved)
         ctx.D, ctx.skip = D, skip
-        return get_C_function('mlp_forward')(x_enc, packed, bias, D, skip, 10)
+        return out
 
     @staticmethod
     def backward(ctx, grad_out):
-        x_enc, *params = ctx.saved_tensors
-        need = [ctx.needs_input_grad[0]] + list(ctx.needs_input_grad[5:])
-        with torch.enable_grad():
-            x = x_enc.detach().requires_grad_(need[0])
-            ps = [p.detach().requires_grad_(n) for p, n in zip(params, need[1:])]
-            out = _mlp_fp32(x, ps, ctx.D, ctx.skip)
-            wanted = [t for t, n in zip([x] + ps, need) if n]
-            got = iter(torch.autograd.grad(out, wanted, grad_out.contiguous(), allow_unused=True))
-        grads = [next(got) if n else None for n in need]
-        return (grads[0], None, None, None, None, *grads[1:])
+        x_enc, packed_t, heads_w, saved = ctx.saved_tensors
+        D, skip, Din = ctx.D, ctx.skip, x_enc.shape[1]
+        g_w, g_b = get_C_function('mlp_backward')(x_enc, packed_t, heads_w, saved, grad_out.contiguous(), D, skip)
+        grads, off = [], 0
+        for i in range(D):
+            K = Din if i == 0 else (Din + 256 if i == skip + 1 else 256)
+            grads += [g_w[off:off + 256 * K].view(256, K), g_b[256 * i:256 * (i + 1)]]
+            off += 256 * K
+        lo = 0
+        for n in (3, 4, 3):  # gaussian_warp, gaussian_rotation, gaussian_scaling rows of the stacked heads
+            grads += [g_w[off + 256 * lo:off + 256 * (lo + n)].view(n, 256), g_b[256 * D + lo:256 * D + lo + n]]
+            lo += n
+        need = ctx.needs_input_grad[7:]
+        return (None,) * 7 + tuple(g if n else None for g, n in zip(grads, need))
 
 
 class _KnnTopk(torch.autograd.Function):

@@ -266,13 +266,30 @@ int fsgs_fusedssim_backward(int B, int CH, int H, int W, const float* img1, cons
 /* Deformation MLP forward (bf16 MFMA, fp32 accumulate) -- fast_2d_gs/network.py:1757-1776 (SC_GS_DeformNetwork.forward,
  * fp32 there): n_layers x (Linear(256) + ReLU), input re-concatenated in front after layer `skip`, then n_out <= 32
  * linear outputs (the three heads stacked). in[B,Din] fp32 (already frequency-encoded), Din <= 96, width must be 256.
- * packed: bf16 weights from fsgs_pack_bf16, layer i as [256][round_up(K_i,16)] row-major (K_0 = Din, K_{skip+1} =
+ * packed: bf16 weights from fsgs_pack_bf16, layer i as a [256][round_up(K_i,16)] matrix (K_0 = Din, K_{skip+1} =
  * Din + 256, else 256), then the heads as [32][256]; fsgs_mlp_packed_elems gives the total element count.
- * bias[n_layers*256 + n_out] fp32. out[B,n_out] fp32. */
+ * fsgs_pack_bf16 converts a row-major fp32 [rows][K] matrix to bf16, zero-padded to [rows_pad][K_pad] (multiples of 32
+ * and 16), in the order the matrix cores read it: 32-row x 16-column tiles, tile (r / 32, k / 16) at
+ * ((r / 32) * (K_pad / 16) + k / 16) * 512 elements, element (r, k) inside it at (r % 32 + 32 * ((k % 16) / 8)) * 8 +
+ * k % 8.
+ * bias[n_layers*256 + n_out] fp32. out[B,n_out] fp32. saved: NULL, or [n_layers][B][256] bf16 that receives every
+ * layer's post-ReLU hidden state for fsgs_mlp_backward. */
 int fsgs_pack_bf16(int rows, int K, int rows_pad, int K_pad, const float* src, uint16_t* dst, void* stream);
 size_t fsgs_mlp_packed_elems(int Din, int n_layers, int skip);
 int fsgs_mlp_forward(int B, int Din, int width, int n_layers, int skip, int n_out, const float* in,
-                     const uint16_t* packed, const float* bias, float* out, void* stream);
+                     const uint16_t* packed, const float* bias, float* out, uint16_t* saved, void* stream);
+
+/* Backward of fsgs_mlp_forward with respect to the weights and biases (torch autograd in the reference:
+ * fast_2d_gs/network.py:1757-1776 is plain nn.Linear / relu). `saved` is the [n_layers][B][256] bf16 post-ReLU state the
+ * forward wrote when given a non-NULL `saved`; packed_t holds, for layers 1 .. n_layers-1, the last 256 input columns
+ * of the weight transposed to [256 in][256 out] bf16 (fsgs_pack_bf16 of the transposed slice); heads_w[n_out][256] and
+ * g_out[B][n_out] are fp32. Outputs, fully written: g_w = the layers' [256][K_l] gradients back to back (unpadded,
+ * K_0 = Din, K_{skip+1} = Din + 256, else 256) followed by the heads' [n_out][256]; g_b[n_layers*256 + n_out].
+ * Operands are bf16, accumulation fp32. No gradient is produced for `in`. */
+size_t fsgs_mlp_backward_workspace_bytes(int B, int n_layers);
+int fsgs_mlp_backward(int B, int Din, int width, int n_layers, int skip, int n_out, const float* in,
+    const uint16_t* packed_t, const float* heads_w, const uint16_t* saved, const float* g_out, float* g_w, float* g_b,
+    void* workspace, size_t workspace_bytes, void* stream);
 
 /* AdamMasksedUpdated -- fast_2d_gs/_C/src/other/adam_masked_update.cu:30-35 (kernel :9-28). Rows of the [N,M]
  * tensors whose mask byte is 0 are left untouched; eps is added to sqrt(v); lr carries the bias correction. */
