@@ -277,8 +277,9 @@ def main():
         extra["fast_path_workload"] = "same scene through GS_2D_fast_* (corner-test binning keeps fewer instances)"
         extra["dynamic_step_frames_per_s"] = dynamic_step_rate(dev)
         extra["dynamic_step_workload"] = ("200000 surfels, 512 control points, bf16 MFMA MLP + K-NN(4) + LBS -> render "
-                                          "800x800 -> 0.8 L1 + 0.2 D-SSIM (fused kernel) -> backward -> masked Adam; "
-                                          "deformation branch forward-only")
+                                          "800x800 -> 0.8 L1 + 0.2 D-SSIM (fused kernel) -> backward through LBS / K-NN / MLP "
+                                          "(HIP kernels) -> masked Adam on the surfels + Adam on the MLP and control "
+                                          "points")
 
     result = {
         "metric": "fwd+bwd frames/s, 300k surfels @800x800",
