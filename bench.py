@@ -64,6 +64,10 @@ def algorithmic_bytes(stage: str, P: int, Pv: int, R: int, T: int, HW: int) -> i
         'gs_2d_render_backward': 76 * R + 16 * T + 60 * HW + 72 * (P + Pv),
         'gs_2d_preprocess_backward': 4 * P + Pv * (352 + 240),
         'gs_2d_pack_records': P * (72 + 12 + 80),  # optional packed per-surfel records: read 4 tensors, write 80 B
+        # fused per-pixel epilogue: reads extras 0-4, opacity, image (9 planes), writes 11; the backward reads 2 depth
+        # planes, opacity and 9 gradient planes, writes dL/dextras (9) and dL/dopacity (1)
+        'gs_2d_epilogue_forward': HW * 4 * (9 + 11),
+        'gs_2d_epilogue_backward': HW * 4 * (12 + 10),
     }
     return int(table[stage])
 
@@ -75,7 +79,7 @@ def cpu_baseline(scene, cam, budget_s: float = 20.0):
     n = lambda t: np.ascontiguousarray(t.cpu().numpy())
     s = {k: n(getattr(scene, k)) for k in ('means3D', 'scales', 'rotations', 'opacities', 'shs')}
     Tw2v, Tv2c, campos = n(cam.Tw2v), n(cam.Tv2c), n(cam.campos)
-    gi, ge, go = n(scene.extra['grad_image']), n(scene.extra['grad_extras']), n(scene.extra['grad_opacity'])
+    gi, ge = n(scene.extra['grad_image']), n(scene.extra['grad_extras'])
     W, H = cam.W, cam.H
     frames, t0 = 0, time.perf_counter()
     while True:
@@ -83,7 +87,16 @@ def cpu_baseline(scene, cam, budget_s: float = 20.0):
                                                                   s['opacities'], s['shs'], None, Tw2v, Tv2c, campos)
         ranges, pl = O.prepare(W, H, m2, dep, radii, tt)
         oc, oo, oe, _, nc = O.render_forward(W, H, m2, colors, no, tm, pl, ranges, cam.near, cam.far, False)
-        gc, gm, gt, gn = O.render_backward(m2, no, colors, tm, None, oo, oe, None, gi, go, ge, None, ranges, pl, nc,
+        # the per-pixel epilogue between the two blend passes, as in the GPU step
+        z = lambda *shape: np.zeros(shape, np.float32)
+        bg = np.ones(3, np.float32)
+        O.call("gs_2d_epilogue_forward_f32", W, H, 1.0, Tw2v, Tv2c, oe, oo, oc, bg, z(3, H, W), z(1, H, W), z(1, H, W),
+               z(3, H, W), z(3, H, W))
+        ge2, go = z(9, H, W), z(H, W)
+        O.call("gs_2d_epilogue_backward_f32", W, H, 1.0, Tw2v, Tv2c, oe, oo, bg, np.ascontiguousarray(ge[1:4]),
+               np.ascontiguousarray(ge[4:5]), np.ascontiguousarray(ge[0:1]), None, np.ascontiguousarray(ge[5:6]), gi,
+               ge2, go)
+        gc, gm, gt, gn = O.render_backward(m2, no, colors, tm, None, oo, oe, None, gi, go, ge2, None, ranges, pl, nc,
                                            cam.near, cam.far)
         O.preprocess_backward(W, H, 3, s['means3D'], s['scales'], s['rotations'], s['shs'], None, Tw2v, Tv2c, campos,
                               tm, radii, colors, gm, gt, gc, gn)
@@ -118,7 +131,7 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
     names = ('means3D', 'scales', 'rotations', 'opacities', 'shs')
     params = [getattr(scene, k).clone().requires_grad_(True) for k in names]
     opt = SparseGaussianAdam([{'params': [p_], 'name': k} for p_, k in zip(params, names)], lr=1.6e-4, eps=1e-15)
-    bg = torch.ones(3, 1, 1, device=dev)
+    bg = torch.ones(3, device=dev)
 
     def step(i):
         t = torch.full((1,), (i % 17) / 17.0, device=dev)
@@ -129,8 +142,8 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
         out = GS_2D_render(params[0] + d_xyz, params[1] + d_scale, torch.nn.functional.normalize(params[2] + d_rot, dim=-1),
                            params[3], (cam.W, cam.H),
                            cam.Tw2v, cam.Tv2c, campos=cam.campos, near=cam.near, far=cam.far, sh_degree=3,
-                           sh_features=params[4])
-        image = out['images'] + (1.0 - out['opacity']) * bg
+                           sh_features=params[4], background=bg)
+        image = out['images']
         loss = 0.8 * (image - target).abs().mean() + 0.2 * (1.0 - ssim(image, target).mean())
         loss.backward()
         opt.set_before_step(out['radii'] > 0, params[0].shape[0])
@@ -218,14 +231,13 @@ def main():
     scene, cam = scene_h.to(dev), cam_h.to(dev)
     gi = scene_h.extra['grad_image'].to(dev)
     ge = scene_h.extra['grad_extras'].to(dev)
-    bg = torch.ones(3, 1, 1, device=dev)  # white background, composited on the host side as the reference does
+    bg = torch.ones(3, device=dev)  # white background
 
     def step():
-        # dL/dopacity of the white-background composite image = C + (1 - opacity) * bg
-        go = -(gi * bg).sum(0)
-        out = render_step(scene, cam, gi, ge, go)
-        out['composited'] = out['image'] + (1.0 - out['opacity']) * bg
-        return out
+        # the fused per-pixel epilogue runs between the two blend passes, as in training: composite on the background,
+        # normals to world space, surf_depth, pseudo surface normal; its backward supplies dL/dextras and the
+        # composite's dL/dopacity = -sum_c dL/dimage_c * bg_c to the blend backward
+        return render_step(scene, cam, gi, ge, None, background=bg)
 
     for _ in range(args.warmup):
         out = step()
@@ -295,8 +307,9 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": f"static 2DGS fwd+bwd: {P} surfels in the unit ball, {cam.W}x{cam.H}, FoV 40, radius 4, "
-                               "SH degree 3, white background, 16x16 tiles, per-tile binning of (tile, depth) keys + "
-                               "depth/normal outputs",
+                               "SH degree 3, white background, 16x16 tiles, per-tile binning of (tile, depth) keys, "
+                               "depth/normal outputs, fused per-pixel epilogue (composite, world normals, surf depth / "
+                               "normal) and its backward between the two blend passes",
                    "P": P, "P_visible": Pv, "R": R, "tiles": T},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(dominant),

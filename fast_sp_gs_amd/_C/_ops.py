@@ -23,6 +23,7 @@ __all__ = [
     'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'mlp_pack_transposed', 'mlp_backward', 'gs_2d_pack_records', 'gs_2d_fast_preprocess_forward',
     'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward', 'gs_2d_fast_compute_trans_mat_backward',
     'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward', 'fusedssim', 'fusedssim_backward',
+    'gs_2d_epilogue_forward', 'gs_2d_epilogue_backward',
 ]
 
 _TILE = 16
@@ -1035,3 +1036,60 @@ def fusedssim_backward(C1: float, C2: float, img1: Tensor, img2: Tensor, dL_dmap
                                             L.ptr(dm_dsigma12.contiguous()), L.ptr(grad), L.current_stream())
     L.check(rc, what)
     return grad
+
+
+# --------------------------------------------------------------------------------------------------------------------
+def gs_2d_epilogue_forward(W: int, H: int, depth_ratio: float, Tw2v: Tensor, Tv2c: Tensor, extras: Tensor,
+                           opacity: Tensor, images: Optional[Tensor] = None, background: Optional[Tensor] = None):
+    """The per-pixel tail of GS_2D_render (renderer/gs_2d_render.py:608-617, helpers :439-470) and, with `images` and
+    `background[3]`, the composite of network.py:725-726, in one kernel ->
+    (normals[3,H,W], depths[1,H,W], surf_depth[1,H,W], surf_normal[3,H,W], composited[3,H,W]|None)."""
+    what = 'gs_2d_epilogue_forward'
+    _f32(what, Tw2v=Tw2v, Tv2c=Tv2c, extras=extras, opacity=opacity, images=images, background=background)
+    if tuple(extras.shape) != (9, H, W) or opacity.numel() != H * W or Tw2v.numel() != 16 or Tv2c.numel() != 16:
+        raise RuntimeError(f'{what}: extras must be [9,{H},{W}], opacity [{H},{W}], the matrices 4x4')
+    if (images is None) != (background is None):
+        raise RuntimeError(f'{what}: images and background go together')
+    if images is not None and (tuple(images.shape) != (3, H, W) or background.numel() != 3):
+        raise RuntimeError(f'{what}: images must be [3,{H},{W}] and background [3]')
+    opt = dict(dtype=torch.float32, device=extras.device)
+    normals, surf_normal = torch.empty((3, H, W), **opt), torch.empty((3, H, W), **opt)
+    depths, surf_depth = torch.empty((1, H, W), **opt), torch.empty((1, H, W), **opt)
+    comp = torch.empty((3, H, W), **opt) if images is not None else None
+    with _timed('gs_2d_epilogue_forward'):
+        rc = _lib().fsgs_gs_2d_epilogue_forward(W, H, float(depth_ratio), L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(extras),
+                                                L.ptr(opacity), L.ptr(images), L.ptr(background), L.ptr(normals),
+                                                L.ptr(depths), L.ptr(surf_depth), L.ptr(surf_normal), L.ptr(comp),
+                                                L.current_stream())
+    L.check(rc, what)
+    return normals, depths, surf_depth, surf_normal, comp
+
+
+def gs_2d_epilogue_backward(W: int, H: int, depth_ratio: float, Tw2v: Tensor, Tv2c: Tensor, extras: Tensor,
+                            opacity: Tensor, background: Optional[Tensor], g_normals: Optional[Tensor],
+                            g_depths: Optional[Tensor], g_surf_depth: Optional[Tensor], g_surf_normal: Optional[Tensor],
+                            g_distortion: Optional[Tensor], g_composited: Optional[Tensor]):
+    """Backward of `gs_2d_epilogue_forward` -> (g_extras[9,H,W], g_opacity[H,W]|None). The gradient of `images` is
+    g_composited itself; the opacity only receives the composite's term (it is detached in surf_normal)."""
+    what = 'gs_2d_epilogue_backward'
+    grads = dict(g_normals=g_normals, g_depths=g_depths, g_surf_depth=g_surf_depth, g_surf_normal=g_surf_normal,
+                 g_distortion=g_distortion, g_composited=g_composited)
+    _f32(what, Tw2v=Tw2v, Tv2c=Tv2c, extras=extras, opacity=opacity, background=background, **grads)
+    if tuple(extras.shape) != (9, H, W) or opacity.numel() != H * W:
+        raise RuntimeError(f'{what}: extras must be [9,{H},{W}] and opacity [{H},{W}]')
+    for k, (t, c) in dict(g_normals=(g_normals, 3), g_depths=(g_depths, 1), g_surf_depth=(g_surf_depth, 1),
+                          g_surf_normal=(g_surf_normal, 3), g_distortion=(g_distortion, 1),
+                          g_composited=(g_composited, 3)).items():
+        if t is not None and t.numel() != c * H * W:
+            raise RuntimeError(f'{what}: {k} must have {c} x {H} x {W} elements')
+    if g_composited is not None and background is None:
+        raise RuntimeError(f'{what}: g_composited needs the background')
+    g_extras = torch.empty_like(extras)
+    g_opacity = torch.empty((H, W), dtype=torch.float32, device=extras.device) if g_composited is not None else None
+    with _timed('gs_2d_epilogue_backward'):
+        rc = _lib().fsgs_gs_2d_epilogue_backward(
+            W, H, float(depth_ratio), L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(extras), L.ptr(opacity), L.ptr(background),
+            L.ptr(g_normals), L.ptr(g_depths), L.ptr(g_surf_depth), L.ptr(g_surf_normal), L.ptr(g_distortion),
+            L.ptr(g_composited), L.ptr(g_extras), L.ptr(g_opacity), L.current_stream())
+    L.check(rc, what)
+    return g_extras, g_opacity

@@ -119,13 +119,44 @@ class _GS_2D_Render(torch.autograd.Function):
         return tuple(grad_inputs)
 
 
+class _GS_2D_Epilogue(torch.autograd.Function):
+    """normals to world space, nan_to_num of the depth maps, surf_depth, depth_to_normal * opacity.detach() and the
+    optional background composite (gs_2d_render.py:608-617, network.py:725-726) through the fused kernels."""
+    _forward = get_C_function('gs_2d_epilogue_forward')
+    _backward = get_C_function('gs_2d_epilogue_backward')
+
+    @staticmethod
+    def forward(ctx, extras, opacity, images, background, Tw2v, Tv2c, depth_ratio, W, H):
+        extras, opacity = extras.contiguous(), opacity.contiguous()
+        bg = None if background is None else background.detach().reshape(3).contiguous()
+        normals, depths, surf_depth, surf_normal, comp = _GS_2D_Epilogue._forward(
+            W, H, depth_ratio, Tw2v, Tv2c, extras, opacity, None if images is None else images.contiguous(), bg)
+        ctx.save_for_backward(extras, opacity, Tw2v, Tv2c, bg)
+        ctx._info = (W, H, depth_ratio)
+        ctx.set_materialize_grads(False)
+        return normals, depths, surf_depth, surf_normal, comp
+
+    @staticmethod
+    def backward(ctx, g_normals, g_depths, g_surf_depth, g_surf_normal, g_comp):
+        extras, opacity, Tw2v, Tv2c, bg = ctx.saved_tensors
+        W, H, depth_ratio = ctx._info
+        c = lambda t: None if t is None else t.contiguous()
+        g_extras, g_opacity = _GS_2D_Epilogue._backward(W, H, depth_ratio, Tw2v, Tv2c, extras, opacity, bg,
+                                                        c(g_normals), c(g_depths), c(g_surf_depth), c(g_surf_normal),
+                                                        None, c(g_comp))
+        return g_extras, g_opacity, g_comp, None, None, None, None, None, None
+
+
 def GS_2D_render(points: Tensor, scales: Tensor, rotations: Tensor, opacity: Tensor,
                  size: Union[Tuple[int, int], Tensor], Tw2v: Tensor, Tv2c: Tensor, campos: Tensor = None,
                  focals: Tensor = None, FoV: Tensor = None, is_opengl=False, near=0.2, far=100, sh_degree=0,
                  colors: Tensor = None, sh_features: Tensor = None, sh_features_rest: Tensor = None, depth_ratio=1.,
                  culling: Tensor = None, trans_mat_t2: Tensor = None, accum_max_count: Tensor = None,
-                 accum_weights_p: Tensor = None, accum_weights_count: Tensor = None, **kwargs):
-    """Same inputs, outputs and dict keys as the reference's GS_2D_render (gs_2d_render.py:550-633)."""
+                 accum_weights_p: Tensor = None, accum_weights_count: Tensor = None, background: Tensor = None,
+                 **kwargs):
+    """Same inputs, outputs and dict keys as the reference's GS_2D_render (gs_2d_render.py:550-633). The per-pixel tail
+    (:608-617) runs as one fused kernel each way. `background` ([3], optional, not in the reference's signature) also
+    folds the caller's composite `images + (1 - opacity) * background` (network.py:725-726) into that kernel."""
     means2D = points.new_zeros(points.shape[0], 2, requires_grad=True)
     W, H = size
     if campos is None:
@@ -135,13 +166,24 @@ def GS_2D_render(points: Tensor, scales: Tensor, rotations: Tensor, opacity: Ten
         Tw2v.contiguous(), Tv2c.contiguous(), campos.contiguous(), size, sh_degree if colors is None else -1,
         is_opengl, near, far, False, None, means2D, trans_mat_t2, culling, accum_max_count, accum_weights_p,
         accum_weights_count)
-    depths, normals, median_depths, distortion, _ = out_extras.split([1, 3, 1, 1, 3], dim=0)
-    normals = (normals.permute(1, 2, 0) @ Tw2v[:3, :3]).permute(2, 0, 1)
-    median_depths = torch.nan_to_num(median_depths, 0, 0)
-    depths = torch.nan_to_num(depths, 0, 0)
-    surf_depth = depths * (1 - depth_ratio) + depth_ratio * median_depths
-    surf_normal = depth_to_normal(Tw2v, Tv2c, (W, H), surf_depth).permute(2, 0, 1)
-    surf_normal = surf_normal * opacities.detach()
+    distortion = out_extras[5:6]
+    if Tw2v.requires_grad or Tv2c.requires_grad:
+        # camera optimisation: the fused epilogue produces no camera gradients, take the reference's torch ops
+        if background is not None:
+            images = images + (1.0 - opacities) * background.view(3, 1, 1)
+        depths, normals, median_depths, _, _ = out_extras.split([1, 3, 1, 1, 3], dim=0)
+        normals = (normals.permute(1, 2, 0) @ Tw2v[:3, :3]).permute(2, 0, 1)
+        median_depths = torch.nan_to_num(median_depths, 0, 0)
+        depths = torch.nan_to_num(depths, 0, 0)
+        surf_depth = depths * (1 - depth_ratio) + depth_ratio * median_depths
+        surf_normal = depth_to_normal(Tw2v, Tv2c, (W, H), surf_depth).permute(2, 0, 1)
+        surf_normal = surf_normal * opacities.detach()
+    else:
+        normals, median_depths, surf_depth, surf_normal, composited = _GS_2D_Epilogue.apply(
+            out_extras, opacities, images if background is not None else None, background, Tw2v.contiguous(),
+            Tv2c.contiguous(), float(depth_ratio), W, H)
+        if background is not None:
+            images = composited
     outputs = {
         'images': images, 'depths': median_depths, 'normals': normals, 'opacity': opacities,
         'distortion': distortion, 'surf_depth': surf_depth, 'surf_normal': surf_normal, 'radii': radii,
@@ -161,10 +203,16 @@ def GS_2D_topk_weights(topk: int, buffer: RasterizeBuffer) -> Tuple[Tensor, Tens
 
 
 def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad_opacity: Tensor = None,
-                ordered_sums: bool = True, packed: bool = True):
+                ordered_sums: bool = True, packed: bool = True, background: Tensor = None, depth_ratio: float = 1.0):
     """One forward + backward pass of the hot path on raw operators (no autograd graph): preprocess -> binning ->
     blend -> blend backward -> preprocess backward, in the order `_GS_2D_Render` runs them. Returns a dict with every
-    intermediate so callers (benchmark, parity tests) can inspect or time the stages."""
+    intermediate so callers (benchmark, parity tests) can inspect or time the stages.
+
+    With `background` ([3]) the per-pixel epilogue of `GS_2D_render` runs between the two blend passes as it does in
+    training: forward -> normals / depths / surf_depth / surf_normal / composited image; then `grad_image` is the
+    gradient of the COMPOSITED image and the first six channels of `grad_extras` are read as the gradients of
+    (surf_depth, normals x 3, depths, distortion); the epilogue backward turns them into the blend's dL/dextras and
+    the composite's dL/dopacity (added to `grad_opacity`)."""
     f = get_C_function
     W, H = cam.W, cam.H
     dev = scene.means3D.device
@@ -175,6 +223,19 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
     rec = f('gs_2d_pack_records')(m2, colors, no, tm, radii, offsets) if packed else None
     oc, oo, oe, of, nc = f('GS_2D_render_forward')(W, H, m2, colors, no, tm, point_list, ranges, cam.near, cam.far,
                                                    False, None, None, None, None, rec)
+    epilogue = {}
+    if background is not None:
+        normals, med, surf_depth, surf_normal, comp = f('gs_2d_epilogue_forward')(
+            W, H, depth_ratio, cam.Tw2v, cam.Tv2c, oe, oo, oc, background)
+        ge = grad_extras
+        g_ex, g_op = f('gs_2d_epilogue_backward')(
+            W, H, depth_ratio, cam.Tw2v, cam.Tv2c, oe, oo, background,
+            None if ge is None else ge[1:4], None if ge is None else ge[4:5], None if ge is None else ge[0:1],
+            None, None if ge is None else ge[5:6], grad_image)
+        grad_extras = g_ex
+        grad_opacity = g_op if grad_opacity is None else grad_opacity + g_op
+        epilogue = dict(normals=normals, median_depths=med, surf_depth=surf_depth, surf_normal=surf_normal,
+                        composited=comp)
     if grad_extras is None:
         grad_extras = torch.zeros((9, H, W), dtype=torch.float32, device=dev)
     if grad_opacity is None:
@@ -190,4 +251,4 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
     return dict(means2D=m2, colors=colors, trans_mat=tm, normal_opacity=no, depths=depths, radii=radii,
                 tiles_touched=tt, ranges=ranges, point_list=point_list, image=oc, opacity=oo, extras=oe,
                 n_contrib=nc, g_colors=gc, g_means2D=gm2, g_trans=gt, g_normal_opacity=gno, g_means3D=g_means3D,
-                g_scales=g_scales, g_rot=g_rot, g_opac=g_opac, g_shs=g_shs)
+                g_scales=g_scales, g_rot=g_rot, g_opac=g_opac, g_shs=g_shs, **epilogue)

@@ -251,6 +251,28 @@ size_t fsgs_knn_topk_backward_workspace_bytes(int N, int M, int D);
 int fsgs_knn_topk_backward(int N, int M, int D, int K, const float* x, const float* y, const int64_t* index,
     const float* g_dist2, float* g_x, float* g_y, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- render epilogue -------------------------------------------------------------------------------------------- */
+
+/* Everything fast_2d_gs/renderer/gs_2d_render.py:608-617 does per pixel after the blend, in one kernel: normals[3,H,W] =
+ * extras[1:4] as row vectors times Tw2v[:3,:3]; depths[H,W] = nan_to_num(extras[4], 0, 0); surf_depth[H,W] =
+ * nan_to_num(extras[0], 0, 0) * (1 - depth_ratio) + depth_ratio * depths; surf_normal[3,H,W] = depth_to_normal
+ * (gs_2d_render.py:439-470: normalised cross product of the central differences of the back-projected surf_depth, zero
+ * on the one-pixel border) times opacity; and, when composited is not NULL, composited[3,H,W] = images + (1 - opacity)
+ * * background[3] (fast_2d_gs/network.py:725-726). Tw2v[4,4] must be affine (last row 0 0 0 1), Tv2c[4,4] is the
+ * projection; both are read on the device. Every output element is written. */
+int fsgs_gs_2d_epilogue_forward(int W, int H, double depth_ratio, const float* Tw2v, const float* Tv2c,
+    const float* extras, const float* opacity, const float* images, const float* background, float* normals,
+    float* depths, float* surf_depth, float* surf_normal, float* composited, void* stream);
+
+/* Backward of the above (torch autograd in the reference). Any of the six upstream gradients may be NULL (= zero).
+ * g_extras[9,H,W] is fully written (channels 6-8 zero); the opacity is treated as detached in surf_normal, as the
+ * reference does, so g_opacity[H,W] (optional) only receives the composite's -sum_c g_composited[c] * background[c];
+ * the gradient of `images` is g_composited itself. No gradient is produced for the camera matrices. */
+int fsgs_gs_2d_epilogue_backward(int W, int H, double depth_ratio, const float* Tw2v, const float* Tv2c,
+    const float* extras, const float* opacity, const float* background, const float* g_normals, const float* g_depths,
+    const float* g_surf_depth, const float* g_surf_normal, const float* g_distortion, const float* g_composited,
+    float* g_extras, float* g_opacity, void* stream);
+
 /* ---- fused SSIM ------------------------------------------------------------------------------------------------ */
 
 /* fusedssim -- fast_2d_gs/_C/src/other/structural_similarity.cu:340-363 (kernel :187-277). img1, img2, ssim_map and

@@ -402,6 +402,156 @@ static void knn_topk_backward(int N, int M, int D, int K, const T* x, const T* y
   }
 }
 
+// ---- render epilogue -------------------------------------------------------------------------------------------------
+// renderer/gs_2d_render.py:608-617 with depths_to_points / depth_to_normal (:439-470) and the background composite of
+// network.py:725-726, and the backward torch autograd derives from them. Tw2v is taken as affine (last row 0 0 0 1), so
+// c2w = [R^-1 | -R^-1 t]; intrins = (ndc2pix Tv2c)[:3,:3], which is what the reference's
+// ((c2w^T (Tv2c Tw2v)^T) ndc2pix^T)[:3,:3]^T reduces to.
+template <typename T>
+static void inv3(const T* a, T* inv) {
+  const T c00 = a[4] * a[8] - a[5] * a[7], c01 = a[5] * a[6] - a[3] * a[8], c02 = a[3] * a[7] - a[4] * a[6];
+  const T r = T(1) / (a[0] * c00 + a[1] * c01 + a[2] * c02);
+  inv[0] = c00 * r, inv[1] = (a[2] * a[7] - a[1] * a[8]) * r, inv[2] = (a[1] * a[5] - a[2] * a[4]) * r;
+  inv[3] = c01 * r, inv[4] = (a[0] * a[8] - a[2] * a[6]) * r, inv[5] = (a[2] * a[3] - a[0] * a[5]) * r;
+  inv[6] = c02 * r, inv[7] = (a[1] * a[6] - a[0] * a[7]) * r, inv[8] = (a[0] * a[4] - a[1] * a[3]) * r;
+}
+
+template <typename T>
+struct EpilogueCamera {
+  T m[9], o[3];
+  EpilogueCamera(int W, int H, const T* Tw2v, const T* Tv2c) {
+    const T R[9] = {Tw2v[0], Tw2v[1], Tw2v[2], Tw2v[4], Tw2v[5], Tw2v[6], Tw2v[8], Tw2v[9], Tw2v[10]};
+    T Ri[9], K[9], Ki[9];
+    inv3(R, Ri);
+    for (int a = 0; a < 3; ++a) o[a] = -(Ri[a * 3] * Tw2v[3] + Ri[a * 3 + 1] * Tw2v[7] + Ri[a * 3 + 2] * Tw2v[11]);
+    const T hw = T(0.5) * W, hh = T(0.5) * H;
+    for (int c = 0; c < 3; ++c) {
+      K[c]     = hw * Tv2c[c] + hw * Tv2c[12 + c];
+      K[3 + c] = hh * Tv2c[4 + c] + hh * Tv2c[12 + c];
+      K[6 + c] = Tv2c[12 + c];
+    }
+    inv3(K, Ki);
+    for (int a = 0; a < 3; ++a)
+      for (int b = 0; b < 3; ++b) m[a * 3 + b] = Ri[a * 3] * Ki[b] + Ri[a * 3 + 1] * Ki[3 + b] + Ri[a * 3 + 2] * Ki[6 + b];
+  }
+  void ray(int x, int y, T* d) const {
+    for (int a = 0; a < 3; ++a) d[a] = m[a * 3] * x + m[a * 3 + 1] * y + m[a * 3 + 2];
+  }
+};
+
+template <typename T>
+static inline T nan_to_zero(T v) {  // torch.nan_to_num(v, 0, 0)
+  if (v != v || v == std::numeric_limits<T>::infinity()) return 0;
+  return v == -std::numeric_limits<T>::infinity() ? std::numeric_limits<T>::lowest() : v;
+}
+
+template <typename T>
+static void epilogue_forward(int W, int H, T ratio, const T* Tw2v, const T* Tv2c, const T* extras, const T* opacity,
+                             const T* images, const T* background, T* normals, T* depths, T* surf_depth,
+                             T* surf_normal, T* composited) {
+  const size_t HW = (size_t) H * W;
+  const EpilogueCamera<T> cam(W, H, Tw2v, Tv2c);
+  std::vector<T> pts(HW * 3);
+  for (int y = 0; y < H; ++y)
+    for (int x = 0; x < W; ++x) {
+      const size_t p = (size_t) y * W + x;
+      for (int j = 0; j < 3; ++j)
+        normals[j * HW + p] = extras[HW + p] * Tw2v[j] + extras[2 * HW + p] * Tw2v[4 + j] + extras[3 * HW + p] * Tw2v[8 + j];
+      depths[p]     = nan_to_zero(extras[4 * HW + p]);
+      surf_depth[p] = nan_to_zero(extras[p]) * (1 - ratio) + ratio * depths[p];
+      T d[3];
+      cam.ray(x, y, d);
+      for (int a = 0; a < 3; ++a) pts[3 * p + a] = surf_depth[p] * d[a] + cam.o[a];
+      if (composited)
+        for (int c = 0; c < 3; ++c) composited[c * HW + p] = images[c * HW + p] + (1 - opacity[p]) * background[c];
+    }
+  for (int y = 0; y < H; ++y)
+    for (int x = 0; x < W; ++x) {
+      const size_t p = (size_t) y * W + x;
+      T n[3] = {0, 0, 0};
+      if (x >= 1 && y >= 1 && x <= W - 2 && y <= H - 2) {
+        T a[3], b[3];
+        for (int k = 0; k < 3; ++k) {
+          a[k] = pts[3 * (p + W) + k] - pts[3 * (p - W) + k];
+          b[k] = pts[3 * (p + 1) + k] - pts[3 * (p - 1) + k];
+        }
+        const T c[3] = {a[1] * b[2] - a[2] * b[1], a[2] * b[0] - a[0] * b[2], a[0] * b[1] - a[1] * b[0]};
+        const T len  = std::max(std::sqrt(c[0] * c[0] + c[1] * c[1] + c[2] * c[2]), T(1e-12));
+        for (int k = 0; k < 3; ++k) n[k] = c[k] / len * opacity[p];
+      }
+      for (int k = 0; k < 3; ++k) surf_normal[k * HW + p] = n[k];
+    }
+}
+
+template <typename T>
+static void epilogue_backward(int W, int H, T ratio, const T* Tw2v, const T* Tv2c, const T* extras, const T* opacity,
+                              const T* background, const T* g_normals, const T* g_depths, const T* g_surf_depth,
+                              const T* g_surf_normal, const T* g_distortion, const T* g_composited, T* g_extras,
+                              T* g_opacity) {
+  const size_t HW = (size_t) H * W;
+  const EpilogueCamera<T> cam(W, H, Tw2v, Tv2c);
+  std::vector<T> pts(HW * 3), gpts(HW * 3, T(0));
+  for (int y = 0; y < H; ++y)
+    for (int x = 0; x < W; ++x) {
+      const size_t p = (size_t) y * W + x;
+      const T sd = nan_to_zero(extras[p]) * (1 - ratio) + ratio * nan_to_zero(extras[4 * HW + p]);
+      T d[3];
+      cam.ray(x, y, d);
+      for (int a = 0; a < 3; ++a) pts[3 * p + a] = sd * d[a] + cam.o[a];
+    }
+  if (g_surf_normal)
+    for (int y = 1; y <= H - 2; ++y)
+      for (int x = 1; x <= W - 2; ++x) {
+        const size_t p = (size_t) y * W + x;
+        T a[3], b[3], gn[3], gc[3];
+        for (int k = 0; k < 3; ++k) {
+          a[k]  = pts[3 * (p + W) + k] - pts[3 * (p - W) + k];
+          b[k]  = pts[3 * (p + 1) + k] - pts[3 * (p - 1) + k];
+          gn[k] = g_surf_normal[k * HW + p] * opacity[p];
+        }
+        const T c[3] = {a[1] * b[2] - a[2] * b[1], a[2] * b[0] - a[0] * b[2], a[0] * b[1] - a[1] * b[0]};
+        const T len  = std::sqrt(c[0] * c[0] + c[1] * c[1] + c[2] * c[2]);
+        if (len > T(1e-12)) {
+          const T n[3] = {c[0] / len, c[1] / len, c[2] / len};
+          const T t    = n[0] * gn[0] + n[1] * gn[1] + n[2] * gn[2];
+          for (int k = 0; k < 3; ++k) gc[k] = (gn[k] - n[k] * t) / len;
+        } else {
+          for (int k = 0; k < 3; ++k) gc[k] = gn[k] / T(1e-12);
+        }
+        const T ga[3] = {b[1] * gc[2] - b[2] * gc[1], b[2] * gc[0] - b[0] * gc[2], b[0] * gc[1] - b[1] * gc[0]};
+        const T gb[3] = {gc[1] * a[2] - gc[2] * a[1], gc[2] * a[0] - gc[0] * a[2], gc[0] * a[1] - gc[1] * a[0]};
+        for (int k = 0; k < 3; ++k) {
+          gpts[3 * (p + W) + k] += ga[k], gpts[3 * (p - W) + k] -= ga[k];
+          gpts[3 * (p + 1) + k] += gb[k], gpts[3 * (p - 1) + k] -= gb[k];
+        }
+      }
+  for (int y = 0; y < H; ++y)
+    for (int x = 0; x < W; ++x) {
+      const size_t p = (size_t) y * W + x;
+      T d[3];
+      cam.ray(x, y, d);
+      T g_sd = g_surf_depth ? g_surf_depth[p] : T(0);
+      for (int a = 0; a < 3; ++a) g_sd += gpts[3 * p + a] * d[a];
+      const bool fin_d = std::isfinite(extras[p]), fin_m = std::isfinite(extras[4 * HW + p]);
+      g_extras[p]          = fin_d ? (1 - ratio) * g_sd : T(0);
+      g_extras[4 * HW + p] = fin_m ? ratio * g_sd + (g_depths ? g_depths[p] : T(0)) : T(0);
+      for (int i = 0; i < 3; ++i) {
+        T g = 0;
+        if (g_normals)
+          for (int j = 0; j < 3; ++j) g += g_normals[j * HW + p] * Tw2v[4 * i + j];
+        g_extras[(1 + i) * HW + p] = g;
+      }
+      g_extras[5 * HW + p] = g_distortion ? g_distortion[p] : T(0);
+      for (int c = 6; c < 9; ++c) g_extras[c * HW + p] = 0;
+      if (g_opacity) {
+        T s = 0;
+        if (g_composited)
+          for (int c = 0; c < 3; ++c) s += g_composited[c * HW + p] * background[c];
+        g_opacity[p] = -s;
+      }
+    }
+}
+
 // Deformation MLP forward, network.py:1757-1776: h = in; for i in 0..L-1: h = relu(W_i h + b_i);
 // after layer index `skip` the input is re-concatenated in front: h = [in | h]. Heads are plain linears.
 // Weights are row-major [out, in] as torch.nn.Linear stores them.
@@ -614,3 +764,23 @@ ORACLE_API int oracle_deform_mlp_f32(int B, int Din, int Wd, int L, int skip, co
   deform_mlp(B, Din, Wd, L, skip, in, Ws, bs, n_heads, head_dims, hW, hb, outs);
   return 0;
 }
+
+#define INSTANTIATE_EPILOGUE(SUF, T)                                                                                 \
+  ORACLE_API int oracle_gs_2d_epilogue_forward_##SUF(int W, int H, double ratio, const T* Tw2v, const T* Tv2c,       \
+      const T* extras, const T* opacity, const T* images, const T* background, T* normals, T* depths,                \
+      T* surf_depth, T* surf_normal, T* composited) {                                                                \
+    epilogue_forward<T>(W, H, (T) ratio, Tw2v, Tv2c, extras, opacity, images, background, normals, depths,           \
+                        surf_depth, surf_normal, composited);                                                        \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_gs_2d_epilogue_backward_##SUF(int W, int H, double ratio, const T* Tw2v, const T* Tv2c,      \
+      const T* extras, const T* opacity, const T* background, const T* g_normals, const T* g_depths,                 \
+      const T* g_surf_depth, const T* g_surf_normal, const T* g_distortion, const T* g_composited, T* g_extras,      \
+      T* g_opacity) {                                                                                                \
+    epilogue_backward<T>(W, H, (T) ratio, Tw2v, Tv2c, extras, opacity, background, g_normals, g_depths,              \
+                         g_surf_depth, g_surf_normal, g_distortion, g_composited, g_extras, g_opacity);              \
+    return 0;                                                                                                        \
+  }
+
+INSTANTIATE_EPILOGUE(f32, float)
+INSTANTIATE_EPILOGUE(f64, double)

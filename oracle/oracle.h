@@ -60,6 +60,13 @@ int oracle_lbs_blend_backward_f32(int N, int M, int K, int centred, double tempe
     float* g_dist2, float* g_sp_points, float* g_sp_t, float* g_sp_r, float* g_sp_s);
 int oracle_knn_topk_backward_f32(int N, int M, int D, int K, const float* x, const float* y, const int64_t* index,
     const float* g_dist2, float* g_x, float* g_y);
+int oracle_gs_2d_epilogue_forward_f32(int W, int H, double ratio, const float* Tw2v, const float* Tv2c,
+    const float* extras, const float* opacity, const float* images, const float* background, float* normals,
+    float* depths, float* surf_depth, float* surf_normal, float* composited);
+int oracle_gs_2d_epilogue_backward_f32(int W, int H, double ratio, const float* Tw2v, const float* Tv2c,
+    const float* extras, const float* opacity, const float* background, const float* g_normals, const float* g_depths,
+    const float* g_surf_depth, const float* g_surf_normal, const float* g_distortion, const float* g_composited,
+    float* g_extras, float* g_opacity);
 int64_t oracle_gs_prepare_count(int P, const int32_t* tiles_touched, int64_t* offsets);
 int oracle_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
     const int64_t* offsets, int64_t R, int64_t* ranges, int32_t* point_list, int64_t* keys_sorted_out);
