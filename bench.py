@@ -10,6 +10,7 @@ Prints ONE JSON line. Only one GPU is supported: --gpus N with N > 1 exits with 
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -155,11 +156,33 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()  # as in the main measurement: no cyclic-collector stalls inside the timed region
     t0 = time.perf_counter()
     for i in range(steps):
         step(i)
     torch.cuda.synchronize()
-    return steps / (time.perf_counter() - t0)
+    dt = time.perf_counter() - t0
+    gc.enable()
+    return steps / dt
+
+
+def simple_knn_ms(dev, scene):
+    """simple_knn (mean squared 3-NN distance, used to initialise the surfel scales) on the benchmark scene's 300k
+    centres and on 3M uniform points."""
+    from fast_sp_gs_amd._C import get_C_function
+    fn = get_C_function('simple_knn')
+    out = {}
+    big = torch.rand(3_000_000, 3, generator=torch.Generator().manual_seed(5)).to(dev)
+    for name, pts in (("simple_knn_300k_ms", scene.means3D.contiguous()), ("simple_knn_3m_ms", big)):
+        fn(pts)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(3):
+            fn(pts)
+        torch.cuda.synchronize()
+        out[name] = (time.perf_counter() - t0) / 3 * 1e3
+    return out
 
 
 def ssim_rate(dev, reps: int = 20):
@@ -197,11 +220,15 @@ def fast_path_rate(dev, scene, cam, gi, steps: int = 20, warmup: int = 3):
     for _ in range(warmup):
         fast_render_step(scene, cam, gi, ge, go)
     torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()
     t0 = time.perf_counter()
     for _ in range(steps):
         fast_render_step(scene, cam, gi, ge, go)
     torch.cuda.synchronize()
-    return steps / (time.perf_counter() - t0)
+    dt = time.perf_counter() - t0
+    gc.enable()
+    return steps / dt
 
 
 def main():
@@ -239,9 +266,19 @@ def main():
         # composite's dL/dopacity = -sum_c dL/dimage_c * bg_c to the blend backward
         return render_step(scene, cam, gi, ge, None, background=bg)
 
+    # The per-stage events of the timed steps are created and recorded once here, outside the timed region: the runtime
+    # grows its event pool in bursts that stall the host for tens of milliseconds.
+    _ops.EVENT_POOL[:] = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps * 2 * 12)]
+    for e in _ops.EVENT_POOL:
+        e.record()
+    torch.cuda.synchronize()
     for _ in range(args.warmup):
         out = step()
     torch.cuda.synchronize()
+    # Python's cyclic collector is kept out of the timed region (a full collection with torch loaded stalls the host
+    # for ~35 ms, 28 steps' worth; nothing in a step creates reference cycles): collect now, switch it back on after.
+    gc.collect()
+    gc.disable()
     _ops.STAGE_EVENTS = events = []
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -249,6 +286,7 @@ def main():
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     _ops.STAGE_EVENTS = None
+    gc.enable()
 
     P = scene.P
     Pv = int((out['radii'] > 0).sum())
@@ -285,6 +323,7 @@ def main():
     extra = {"knn_topk_queries_per_s": pts.shape[0] / (knn_ms * 1e-3), "knn_topk_workload": "200000 x 512, k=4, D=3"}
     if not args.no_extras:
         extra.update(ssim_rate(dev))
+        extra.update(simple_knn_ms(dev, scene))
         extra["fast_path_frames_per_s"] = fast_path_rate(dev, scene, cam, gi)
         extra["fast_path_workload"] = "same scene through GS_2D_fast_* (corner-test binning keeps fewer instances)"
         extra["dynamic_step_frames_per_s"] = dynamic_step_rate(dev)

@@ -23,7 +23,7 @@ __all__ = [
     'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'mlp_pack_transposed', 'mlp_backward', 'gs_2d_pack_records', 'gs_2d_fast_preprocess_forward',
     'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward', 'gs_2d_fast_compute_trans_mat_backward',
     'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward', 'fusedssim', 'fusedssim_backward',
-    'gs_2d_epilogue_forward', 'gs_2d_epilogue_backward',
+    'gs_2d_epilogue_forward', 'gs_2d_epilogue_backward', 'simple_knn',
 ]
 
 _TILE = 16
@@ -31,6 +31,13 @@ _TILE = 16
 # When set to a list, every operator appends (name, start_event, end_event) recorded on the current stream tightly
 # around its C-ABI call (allocation and zero-fill of outputs stay outside), so callers can time the kernels themselves.
 STAGE_EVENTS = None
+# Events to use for that (already created and recorded once by the caller): creating timing events is not free -- the
+# runtime grows its event pool in bursts of tens of milliseconds -- so a caller that times a region fills this first.
+EVENT_POOL: list = []
+
+
+def _event():
+    return EVENT_POOL.pop() if EVENT_POOL else torch.cuda.Event(enable_timing=True)
 
 
 class _timed:
@@ -41,12 +48,12 @@ class _timed:
 
     def __enter__(self):
         if STAGE_EVENTS is not None:
-            self.start = torch.cuda.Event(enable_timing=True)
+            self.start = _event()
             self.start.record()
 
     def __exit__(self, *exc):
         if STAGE_EVENTS is not None:
-            end = torch.cuda.Event(enable_timing=True)
+            end = _event()
             end.record()
             STAGE_EVENTS.append((self.name, self.start, end))
         return False
@@ -1093,3 +1100,23 @@ def gs_2d_epilogue_backward(W: int, H: int, depth_ratio: float, Tw2v: Tensor, Tv
             L.ptr(g_composited), L.ptr(g_extras), L.ptr(g_opacity), L.current_stream())
     L.check(rc, what)
     return g_extras, g_opacity
+
+
+# --------------------------------------------------------------------------------------------------------------------
+def simple_knn(points: Tensor) -> Tensor:
+    """other/knn.cu:180-205: mean squared distance of every point to its three nearest neighbours -> [P]."""
+    what = 'simple_knn'
+    if not isinstance(points, Tensor) or not points.is_cuda:
+        raise RuntimeError(f'{what}: points must be a CUDA tensor')
+    L.require_dtype(what, 'points', points, torch.float32)
+    if points.ndim != 2 or points.shape[-1] != 3:
+        raise RuntimeError(f'{what}: Error shape for points')
+    points = points.contiguous()
+    P = points.shape[0]
+    means = torch.empty((P,), dtype=torch.float32, device=points.device)
+    lib = _lib()
+    ws = _workspace(lib.fsgs_simple_knn_workspace_bytes(P), points.device)
+    with _timed('simple_knn'):
+        rc = lib.fsgs_simple_knn(P, L.ptr(points), L.ptr(means), L.ptr(ws), ws.numel(), L.current_stream())
+    L.check(rc, what)
+    return means

@@ -273,6 +273,14 @@ int fsgs_gs_2d_epilogue_backward(int W, int H, double depth_ratio, const float* 
     const float* g_surf_depth, const float* g_surf_normal, const float* g_distortion, const float* g_composited,
     float* g_extras, float* g_opacity, void* stream);
 
+/* simple_knn -- fast_2d_gs/_C/src/other/knn.cu:180-205 (kernels :57-178). points[P,3] -> mean_dist2[P]: the mean of
+ * the three smallest squared distances from each point to the other points (exact search; with fewer than four
+ * points the missing distances stay FLT_MAX, so the mean is FLT_MAX / 3 or overflows to inf as it does in the
+ * reference). Every output element is written. */
+size_t fsgs_simple_knn_workspace_bytes(int P);
+int fsgs_simple_knn(int P, const float* points, float* mean_dist2, void* workspace, size_t workspace_bytes,
+                    void* stream);
+
 /* ---- fused SSIM ------------------------------------------------------------------------------------------------ */
 
 /* fusedssim -- fast_2d_gs/_C/src/other/structural_similarity.cu:340-363 (kernel :187-277). img1, img2, ssim_map and

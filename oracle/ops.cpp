@@ -552,6 +552,27 @@ static void epilogue_backward(int W, int H, T ratio, const T* Tw2v, const T* Tv2
     }
 }
 
+// simple_knn, other/knn.cu:111-160: mean of the three smallest squared distances dx*dx + dy*dy + dz*dz to the other
+// points (index != own), missing entries FLT_MAX. The reference's Morton ordering and boxes only prune an exact
+// search, so a plain all-pairs scan gives the same three distances; they are kept with the reference's insertion rule.
+template <typename T>
+static void simple_knn(int P, const T* points, T* mean_dist2) {
+  const T big = std::numeric_limits<T>::max();
+#pragma omp parallel for schedule(static)
+  for (int i = 0; i < P; ++i) {
+    T best[3] = {big, big, big};
+    for (int j = 0; j < P; ++j) {
+      if (j == i) continue;
+      const T dx = points[3 * (size_t) j] - points[3 * (size_t) i], dy = points[3 * (size_t) j + 1] - points[3 * (size_t) i + 1],
+              dz = points[3 * (size_t) j + 2] - points[3 * (size_t) i + 2];
+      T dist = dx * dx + dy * dy + dz * dz;
+      for (int k = 0; k < 3; ++k)
+        if (best[k] > dist) std::swap(best[k], dist);
+    }
+    mean_dist2[i] = (best[0] + best[1] + best[2]) / T(3);
+  }
+}
+
 // Deformation MLP forward, network.py:1757-1776: h = in; for i in 0..L-1: h = relu(W_i h + b_i);
 // after layer index `skip` the input is re-concatenated in front: h = [in | h]. Heads are plain linears.
 // Weights are row-major [out, in] as torch.nn.Linear stores them.
@@ -784,3 +805,12 @@ ORACLE_API int oracle_deform_mlp_f32(int B, int Din, int Wd, int L, int skip, co
 
 INSTANTIATE_EPILOGUE(f32, float)
 INSTANTIATE_EPILOGUE(f64, double)
+
+ORACLE_API int oracle_simple_knn_f32(int P, const float* points, float* mean_dist2) {
+  simple_knn<float>(P, points, mean_dist2);
+  return 0;
+}
+ORACLE_API int oracle_simple_knn_f64(int P, const double* points, double* mean_dist2) {
+  simple_knn<double>(P, points, mean_dist2);
+  return 0;
+}

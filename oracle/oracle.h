@@ -67,6 +67,7 @@ int oracle_gs_2d_epilogue_backward_f32(int W, int H, double ratio, const float* 
     const float* extras, const float* opacity, const float* background, const float* g_normals, const float* g_depths,
     const float* g_surf_depth, const float* g_surf_normal, const float* g_distortion, const float* g_composited,
     float* g_extras, float* g_opacity);
+int oracle_simple_knn_f32(int P, const float* points, float* mean_dist2);
 int64_t oracle_gs_prepare_count(int P, const int32_t* tiles_touched, int64_t* offsets);
 int oracle_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
     const int64_t* offsets, int64_t R, int64_t* ranges, int32_t* point_list, int64_t* keys_sorted_out);

@@ -406,3 +406,47 @@ def test_deform_mlp_mfma(device, oracle_mod):
         ref = torch.cat(outs, -1)
         # remaining difference: activations are re-rounded to bf16 between layers on the GPU only
         assert float((got - ref).abs().max() / ref.abs().max()) < 1e-2
+
+
+@pytest.mark.parametrize("P,kind", [(20000, "ball"), (5000, "clusters"), (777, "plane"), (3, "ball"), (2, "ball"),
+                                    (1, "ball"), (4097, "same")])
+def test_simple_knn(P, kind, device, oracle_mod):
+    """Mean squared 3-NN distance: bit-exact against the all-pairs oracle (the search is exact and both sides add the
+    squares in the same order with contraction off) on clouds that stress the pruning: clusters far apart, a flat
+    cloud (degenerate bounding box), duplicates, fewer points than neighbours."""
+    from fast_sp_gs_amd._C import get_C_function
+    O = oracle_mod
+    g = torch.Generator().manual_seed(60 + P)
+    if kind == "ball":
+        pts = torch.randn(P, 3, generator=g)
+    elif kind == "clusters":
+        centres = torch.randn(7, 3, generator=g) * 50.0
+        pts = centres[torch.randint(0, 7, (P,), generator=g)] + 0.01 * torch.randn(P, 3, generator=g)
+    elif kind == "plane":
+        pts = torch.cat([torch.rand(P, 2, generator=g), torch.full((P, 1), 0.25)], 1)
+    else:
+        pts = torch.ones(P, 3) * 0.5  # every point identical: all distances 0, the curve order is all ties
+    pts = pts.contiguous()
+    print(f"[simple_knn] P={P} {kind}", flush=True)
+    got = get_C_function('simple_knn')(pts.to(device))
+    torch.cuda.synchronize()
+    ref = np.zeros(P, np.float32)
+    with np.errstate(over='ignore'):
+        O.call("simple_knn_f32", P, npy(pts), ref)
+    assert np.array_equal(npy(got), ref)
+
+
+def test_simple_knn_full_size(device):
+    """3 M points: every result equals the 3-NN mean recomputed by brute force for a sample of queries."""
+    from fast_sp_gs_amd._C import get_C_function
+    g = torch.Generator().manual_seed(71)
+    P = 3_000_000
+    pts = (torch.rand(P, 3, generator=g) * 2 - 1).to(device)
+    print(f"[simple_knn] P={P}", flush=True)
+    got = get_C_function('simple_knn')(pts)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(got).all()) and float(got.min()) >= 0
+    sample = torch.randint(0, P, (256,), generator=g).to(device)
+    d2 = ((pts[sample][:, None, :] - pts[None, :, :]) ** 2).sum(-1)  # [256, P]
+    best = d2.topk(4, dim=1, largest=False).values[:, 1:]            # drop the point itself (distance 0)
+    assert float((best.mean(1) - got[sample]).abs().max()) <= 1e-6 * float(best.max())

@@ -222,6 +222,28 @@ def test_epilogue_matches_reference_formulation(oracle_mod):
     assert torch.equal(a_im, grads[5])                # and the image gradient is the composite's, unchanged
 
 
+def test_simple_knn_matches_kdtree(oracle_mod):
+    """Exact 3-NN mean squared distance against scipy's k-d tree (k = 4 with the point itself first)."""
+    O = oracle_mod
+    from scipy.spatial import cKDTree
+    rng = np.random.default_rng(17)
+    pts = rng.normal(size=(3000, 3))
+    pts[10] = pts[11]            # a duplicate pair: distance 0 counts
+    out = np.zeros(3000)
+    assert O.call("simple_knn_f64", 3000, pts, out) == 0
+    d, _ = cKDTree(pts).query(pts, k=4)
+    assert np.abs(out - (d[:, 1:] ** 2).mean(1)).max() < 1e-12
+    assert out[10] < out.mean() and out[10] == out[11]
+    # fewer than four points: missing neighbours stay at the largest float, as in the reference (FLT_MAX / 3 with one
+    # missing, overflow to inf with two)
+    few = np.ascontiguousarray(pts[:3].astype(np.float32))
+    o32 = np.zeros(3, np.float32)
+    assert O.call("simple_knn_f32", 3, few, o32) == 0
+    assert np.allclose(o32, np.finfo(np.float32).max / 3, rtol=1e-6)
+    assert O.call("simple_knn_f32", 2, few[:2].copy(), o32) == 0
+    assert np.isinf(o32[:2]).all()
+
+
 def test_masked_adam_matches_torch_adam(oracle_mod):
     O = oracle_mod
     rng = np.random.default_rng(4)
