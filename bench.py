@@ -185,6 +185,56 @@ def simple_knn_ms(dev, scene):
     return out
 
 
+def reference_note_blend_ms(dev, reps: int = 100):
+    """The only timing the reference records for this path (developer note at
+    fast_2d_gs/renderer/gs_2d_fast_render.py:1288-1292, GPU not stated): the two standard blend kernels alone on
+    102 400 surfels with means ~ N(0,1), scales ~ U[0,1], opacity ~ U[0,1], 128 x 128 pixels, focal 500, camera at
+    (0,0,4), auxiliary maps and optical flow on (_gen_random_data :883-910, test_rasterize_fast :1185-1287), 100
+    iterations after a warm-up. Same workload, same two operators, same arguments here."""
+    import math
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd._C import get_C_function as f
+    g = torch.Generator().manual_seed(1234)
+    P, W, H = 102_400, 128, 128
+    means3D = torch.randn(P, 3, generator=g).to(dev)
+    scales = torch.rand(P, 2, generator=g).to(dev)
+    rot = torch.nn.functional.normalize(torch.randn(P, 4, generator=g), dim=-1).to(dev)
+    opac = torch.rand(P, 1, generator=g).to(dev)
+    shs = torch.randn(P, 1, 3, generator=g).to(dev)
+    cam = scenes.pinhole(W, H, math.degrees(2 * math.atan(W / 2 / 500.0)), torch.tensor([0.0, 0.0, 4.0])).to(dev)
+    m2, colors, tm, no, depths, radii, tt = f('gs_2d_preprocess_forward')(
+        W, H, 0, False, means3D, scales, rot, opac, shs, None, cam.Tw2v, cam.Tv2c, cam.campos, None, None, None)
+    ranges, point_list = f('GS_prepare')(W, H, m2, depths, radii, tt, False)
+    Tw2c = (cam.Tv2c @ cam.Tw2v).contiguous()
+    t2 = f('gs_2d_compute_transmat_forward')(W, H, (means3D + 0.1 * torch.randn(P, 3, generator=g).to(dev)).contiguous(),
+                                             scales, rot, cam.Tw2v, Tw2c)[0]
+    t2 = (t2 * (radii[:, None, None] > 0)).contiguous()
+    fwd, bwd = f('GS_2D_render_forward'), f('GS_2D_render_backward')
+    run_f = lambda: fwd(W, H, m2, colors, no, tm, point_list, ranges, 0.2, 100.0, False, t2, None, None, None)
+    oc, oo, oe, of, nc = run_f()
+    gi, go = torch.randn(3, H, W, generator=g).to(dev), torch.randn(H, W, generator=g).to(dev)
+    ge = torch.randn(9, H, W, generator=g).to(dev)
+    ge[5:] = 0
+    gf = torch.randn(H, W, 2, generator=g).to(dev)
+    run_b = lambda: bwd(m2, no, colors, tm, t2, oo, oe, of, gi, go, ge, gf, ranges, point_list, nc, 0.2, 100.0)
+    run_b()
+    torch.cuda.synchronize()
+    e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    e[0].record()
+    for _ in range(reps):
+        run_f()
+    e[1].record()
+    for _ in range(reps):
+        run_b()
+    e[2].record()
+    torch.cuda.synchronize()
+    return {"reference_note_blend_forward_ms": e[0].elapsed_time(e[1]) / reps,
+            "reference_note_blend_backward_ms": e[1].elapsed_time(e[2]) / reps,
+            "reference_note_workload": f"102400 surfels N(0,1), scales U[0,1], 128x128, focal 500, aux + flow, "
+                                       f"R = {int(point_list.numel())}; the reference's own note for its CUDA kernels on "
+                                       f"an unnamed GPU: forward 0.092-0.100 ms, backward 0.678-0.718 ms"}
+
+
 def ssim_rate(dev, reps: int = 20):
     """Fused SSIM forward (with the partial-derivative maps) + backward on one 3 x 800 x 800 image pair."""
     from fast_sp_gs_amd._C import get_C_function
@@ -324,6 +374,7 @@ def main():
     if not args.no_extras:
         extra.update(ssim_rate(dev))
         extra.update(simple_knn_ms(dev, scene))
+        extra.update(reference_note_blend_ms(dev))
         extra["fast_path_frames_per_s"] = fast_path_rate(dev, scene, cam, gi)
         extra["fast_path_workload"] = "same scene through GS_2D_fast_* (corner-test binning keeps fewer instances)"
         extra["dynamic_step_frames_per_s"] = dynamic_step_rate(dev)
