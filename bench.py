@@ -23,6 +23,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 ROOT = os.path.dirname(os.path.abspath(__file__))
 # Hardware-counter summary of the dominant kernel (two rocprofv3 --pmc passes, calibrated against the copy probe).
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gs_2d_render_backward_300k_800x800.pmc_traffic.txt")
+SQ_SUMMARY = os.path.join(ROOT, "profiles", "blend_kernels_300k_800x800_and_deform_mlp.pmc_sq.txt")
 
 
 def measured_traffic(kernel: str):
@@ -32,6 +33,19 @@ def measured_traffic(kernel: str):
             for line in f:
                 if line.startswith(kernel + ".traffic_bytes"):
                     return int(float(line.split("=")[1].split()[0]))
+    except OSError:
+        pass
+    return None
+
+
+def measured_valu_issue(kernel: str):
+    """Share of the chip's vector-ALU issue slots the operator's blend kernel filled, from the committed counter summary
+    (a line `<kernel>.valu_issue_frac = x`)."""
+    try:
+        with open(SQ_SUMMARY) as f:
+            for line in f:
+                if line.startswith(kernel + ".valu_issue_frac"):
+                    return float(line.split("=")[1].split()[0])
     except OSError:
         pass
     return None
@@ -403,7 +417,7 @@ def main():
                    "P": P, "P_visible": Pv, "R": R, "tiles": T},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(dominant),
-                     "algorithmic_bytes_per_launch": bytes_dom, "avg_launch_ms": stage_avg[dominant],
+                     "algorithmic_bytes_per_launch": bytes_dom, "valu_issue_frac": measured_valu_issue(dominant), "avg_launch_ms": stage_avg[dominant],
                      "copy_kernel_GBps": round(copy_gbps, 1)},
         "stages": stages,
         "extra_metrics": extra,
