@@ -249,6 +249,48 @@ def reference_note_blend_ms(dev, reps: int = 100):
                                        f"an unnamed GPU: forward 0.092-0.100 ms, backward 0.678-0.718 ms"}
 
 
+def gs3d_path_rate(dev, scene, cam, gi, steps: int = 30, warmup: int = 5):
+    """The 3D-Gaussian (EWA) path on the benchmark scene with a third scale per Gaussian: preprocess -> binning ->
+    conic blend -> blend backward -> preprocess backward through the raw operators."""
+    from fast_sp_gs_amd._C import get_C_function as f
+    g = torch.Generator().manual_seed(11)
+    scales = torch.cat([scene.scales.cpu(), scene.scales[:, :1].cpu() * (0.5 + torch.rand(scene.P, 1, generator=g))],
+                       1).to(dev).contiguous()
+    W, H = cam.W, cam.H
+    tan_fov = (W / 2 / float(cam.Tv2s[0, 0]), H / 2 / float(cam.Tv2s[1, 1]))
+    go = -gi.sum(0)  # white-background composite
+    R = [0]
+
+    def step():
+        m2, dep, col, rad, tt, c3, co = f('gs_preprocess_forward')(
+            W, H, 3, False, scene.means3D, scales, scene.rotations, scene.opacities, scene.shs, None, cam.Tw2v,
+            cam.Tv2c, cam.campos, tan_fov, None, None, None, None)
+        ranges, pl = f('GS_prepare')(W, H, m2, dep, rad, tt, False)
+        oc, oo, _, nc = f('gaussian_rasterize_forward')(W, H, m2, co, col, None, pl, ranges)
+        g_col, _, g_m2, g_co = f('gaussian_rasterize_backward')(m2, co, col, None, oo, gi, go, None, ranges, pl, nc)
+        g3, gs, gq = torch.empty_like(scene.means3D), torch.empty_like(scales), torch.empty_like(scene.rotations)
+        gop, gsh = torch.empty_like(scene.opacities), torch.empty_like(scene.shs)
+        f('gs_preprocess_backward')(W, H, 3, False, scene.means3D, scales, scene.rotations, scene.opacities, scene.shs,
+                                    None, cam.Tw2v, cam.Tv2c, cam.campos, tan_fov, c3, None, rad, col, g_m2, None, g_col,
+                                    g_co, g3, gs, gq, gop, gsh, None, None)
+        R[0] = pl.numel()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    gc.enable()
+    return {"gs3d_path_frames_per_s": steps / dt,
+            "gs3d_path_workload": f"same 300k centres as 3D Gaussians (third scale added), 800x800, SH degree 3, "
+                                  f"R = {R[0]}: gs_preprocess fwd/bwd + GS_prepare + gaussian_rasterize fwd/bwd"}
+
+
 def ssim_rate(dev, reps: int = 20):
     """Fused SSIM forward (with the partial-derivative maps) + backward on one 3 x 800 x 800 image pair."""
     from fast_sp_gs_amd._C import get_C_function
@@ -389,6 +431,7 @@ def main():
         extra.update(ssim_rate(dev))
         extra.update(simple_knn_ms(dev, scene))
         extra.update(reference_note_blend_ms(dev))
+        extra.update(gs3d_path_rate(dev, scene, cam, gi))
         extra["fast_path_frames_per_s"] = fast_path_rate(dev, scene, cam, gi)
         extra["fast_path_workload"] = "same scene through GS_2D_fast_* (corner-test binning keeps fewer instances)"
         extra["dynamic_step_frames_per_s"] = dynamic_step_rate(dev)

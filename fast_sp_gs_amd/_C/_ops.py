@@ -23,7 +23,8 @@ __all__ = [
     'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'mlp_pack_transposed', 'mlp_backward', 'gs_2d_pack_records', 'gs_2d_fast_preprocess_forward',
     'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward', 'gs_2d_fast_compute_trans_mat_backward',
     'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward', 'fusedssim', 'fusedssim_backward',
-    'gs_2d_epilogue_forward', 'gs_2d_epilogue_backward', 'simple_knn',
+    'gs_2d_epilogue_forward', 'gs_2d_epilogue_backward', 'simple_knn', 'gs_preprocess_forward',
+    'gs_preprocess_backward', 'gaussian_rasterize_forward', 'gaussian_rasterize_backward',
 ]
 
 _TILE = 16
@@ -1132,3 +1133,186 @@ def simple_knn(points: Tensor) -> Tensor:
         rc = lib.fsgs_simple_knn(P, L.ptr(points), L.ptr(means), L.ptr(ws), ws.numel(), L.current_stream())
     L.check(rc, what)
     return means
+
+
+# ---- 3D-Gaussian (EWA) path ------------------------------------------------------------------------------------------
+def _tan_fov(tanFoV) -> Tuple[float, float]:
+    if isinstance(tanFoV, Tensor):
+        if tanFoV.numel() != 2:
+            raise RuntimeError('tanFoV must have 2 elements')
+        v = tanFoV.detach().cpu().tolist()  # the reference reads it with .item() too (gaussian_preprocess.cu:424-425)
+        return float(v[0]), float(v[1])
+    return float(tanFoV[0]), float(tanFoV[1])
+
+
+def gs_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: bool, means3D: Tensor, scales: Tensor,
+                          rotations: Tensor, opacities: Tensor, shs: Tensor, sh_rest: Optional[Tensor], Tw2v: Tensor,
+                          Tv2c: Tensor, cam_pos: Tensor, tanFoV, cov3D_precomp: Optional[Tensor] = None,
+                          cov2D_precomp: Optional[Tensor] = None, means2D: Optional[Tensor] = None,
+                          culling: Optional[Tensor] = None) -> List[Tensor]:
+    """gaussian_preprocess.cu:372-466 -> [means2D, depths, colors, radii, tiles_touched, cov3Ds, conic_opacity]."""
+    what = 'gs_preprocess_forward'
+    if cov3D_precomp is not None or cov2D_precomp is not None:
+        raise RuntimeError(f'{what}: pre-computed covariances are not supported by this library')
+    _f32(what, means3D=means3D, scales=scales, rotations=rotations, opacities=opacities, shs=shs, Tw2v=Tw2v,
+         Tv2c=Tv2c, cam_pos=cam_pos)
+    if means3D.ndim != 2 or means3D.shape[-1] != 3:
+        raise RuntimeError('Error shape for means3D')
+    P = means3D.shape[0]
+    has_rest = sh_rest is not None and sh_rest.numel() > 0
+    M = 0
+    if has_rest:
+        _f32(what, sh_rest=sh_rest)
+        if not (sh_rest.ndim == 3 and sh_rest.shape[0] == P and sh_rest.shape[1] >= (1 + sh_degree) ** 2 - 1
+                and sh_rest.shape[2] == 3):
+            raise RuntimeError('Error shape for sh features')
+        M = sh_rest.shape[1]
+    elif sh_degree >= 0:
+        if not (shs.ndim == 3 and shs.shape[0] == P and shs.shape[1] >= (1 + sh_degree) ** 2 and shs.shape[2] == 3):
+            raise RuntimeError('Error shape for sh features')
+        M = shs.shape[1]
+    if means2D is not None:
+        _f32(what, means2D=means2D)
+        L.require_shape(what, 'means2D', means2D, P, 2)
+    if culling is not None:
+        L.require_cuda(what, culling=culling)
+        L.require_dtype(what, 'culling', culling, torch.bool)
+        L.require_shape(what, 'culling', culling, P)
+    L.require_shape(what, 'scales', scales, P, 3)
+    L.require_shape(what, 'rotations', rotations, P, 4)
+    L.require_shape(what, 'opacities', opacities, P, 1)
+    L.require_shape(what, 'Tw2v', Tw2v, 4, 4)
+    L.require_shape(what, 'Tv2c', Tv2c, 4, 4)
+    L.require_shape(what, 'cam_pos', cam_pos, 3)
+    if sh_degree < 0:
+        L.require_shape(what, 'shs', shs, P, 3)
+    tx, ty = _tan_fov(tanFoV)
+    opt = dict(dtype=torch.float32, device=means3D.device)
+    colors = shs if sh_degree < 0 else torch.empty((P, 3), **opt)
+    preserve = means2D is not None
+    means2D_ = means2D if preserve else torch.empty((P, 2), **opt)
+    depths, cov3Ds, conic_opacity = torch.empty((P,), **opt), torch.empty((P, 6), **opt), torch.empty((P, 4), **opt)
+    radii = torch.empty((P,), dtype=torch.int32, device=means3D.device)
+    tiles_touched = torch.empty((P,), dtype=torch.int32, device=means3D.device)
+    with _timed('gs_preprocess_forward'):
+        rc = _lib().fsgs_gs_preprocess_forward(
+            P, W, H, sh_degree, M, int(bool(is_opengl)), L.ptr(means3D), L.ptr(scales), L.ptr(rotations),
+            L.ptr(opacities), L.ptr(shs), L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c),
+            L.ptr(cam_pos), tx, ty, L.ptr(culling), int(preserve), L.ptr(means2D_), L.ptr(depths),
+            None if sh_degree < 0 else L.ptr(colors), L.ptr(radii), L.ptr(tiles_touched), L.ptr(cov3Ds),
+            L.ptr(conic_opacity), L.current_stream())
+    L.check(rc, what)
+    return [means2D_, depths, colors, radii, tiles_touched, cov3Ds, conic_opacity]
+
+
+def gs_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs, sh_rest, Tw2v,
+                           Tv2c, cam_pos, tanFoV, cov3Ds, cov2Ds, radii, colors, grad_mean2D, grad_depth, grad_colors,
+                           grad_conic, grad_means3D, grad_scales, grad_rotations, grad_opacities, grad_shs,
+                           grad_sh_rest, grad_cov=None, grad_Tw2v=None, grad_campos=None) -> None:
+    """gaussian_preprocess.cu:567-636: fills the caller's grad_* tensors in place (every row is assigned) and rewrites
+    grad_mean2D as the reference does. grad_depth is ignored there too."""
+    what = 'gs_preprocess_backward'
+    if cov2Ds is not None:
+        raise RuntimeError(f'{what}: pre-computed 2D covariances are not supported by this library')
+    if grad_Tw2v is not None or grad_campos is not None:
+        raise RuntimeError(f'{what}: camera gradients are not supported by this library')
+    _f32(what, grad_mean2D=grad_mean2D, grad_colors=grad_colors, grad_conic=grad_conic, grad_means3D=grad_means3D,
+         grad_scales=grad_scales, grad_rotations=grad_rotations, grad_opacities=grad_opacities, grad_shs=grad_shs,
+         grad_sh_rest=grad_sh_rest, grad_cov=grad_cov, cov3Ds=cov3Ds)
+    has_rest = sh_rest is not None and sh_rest.numel() > 0
+    P = means3D.shape[0]
+    M = sh_rest.shape[1] if has_rest else (shs.shape[1] if shs.ndim == 3 else 0)
+    L.require_shape(what, 'grad_means3D', grad_means3D, P, 3)
+    L.require_shape(what, 'grad_conic', grad_conic, P, 4)
+    L.require_shape(what, 'grad_opacities', grad_opacities, P, 1)
+    if sh_degree >= 0 and grad_colors is None:
+        raise RuntimeError(f'{what}: grad_colors is required with SH colours')
+    tx, ty = _tan_fov(tanFoV)
+    with _timed('gs_preprocess_backward'):
+        rc = _lib().fsgs_gs_preprocess_backward(
+            P, W, H, sh_degree, M, int(bool(is_opengl)), L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(shs),
+            L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(cam_pos), tx, ty, L.ptr(radii),
+            L.ptr(colors), L.ptr(cov3Ds), L.ptr(grad_mean2D), L.ptr(grad_colors), L.ptr(grad_conic),
+            L.ptr(grad_means3D), L.ptr(grad_scales), L.ptr(grad_rotations), L.ptr(grad_opacities), L.ptr(grad_shs),
+            L.ptr(grad_sh_rest) if has_rest else None, L.ptr(grad_cov), L.current_stream())
+    L.check(rc, what)
+
+
+def gaussian_rasterize_forward(width: int, height: int, means2D: Tensor, conic_opacity: Tensor, colors: Tensor,
+                               extras: Optional[Tensor], point_list: Tensor, ranges: Tensor,
+                               accum_max_count: Optional[Tensor] = None, accum_weights_p: Optional[Tensor] = None,
+                               accum_weights_count: Optional[Tensor] = None,
+                               per_tile_bucket_offset: Optional[Tensor] = None):
+    """gaussian_render.cu:212-293 -> [pixel_colors[3,H,W], pixel_opacity[H,W], pixel_extras[E,H,W]|None,
+    n_contrib[H,W]]. The bucket snapshots for the per-Gaussian backward (per_tile_bucket_offset) are not built."""
+    what = 'gaussian_rasterize_forward'
+    if per_tile_bucket_offset is not None:
+        raise RuntimeError(f'{what}: the per-Gaussian (bucketed) backward is not supported by this library')
+    _f32(what, means2D=means2D, conic_opacity=conic_opacity, colors=colors, extras=extras,
+         accum_weights_p=accum_weights_p)
+    L.require_cuda(what, point_list=point_list, ranges=ranges, accum_max_count=accum_max_count,
+                   accum_weights_count=accum_weights_count)
+    if colors.ndim != 2:
+        raise RuntimeError(f'{what}: colors must be [P,3]')
+    P = colors.shape[0]
+    E = 0
+    if extras is not None:
+        if extras.ndim != 2 or extras.shape[0] != P:
+            raise RuntimeError(f'{what}: extras must be [P,E]')
+        E = extras.shape[1]
+        if E > 4:
+            raise RuntimeError('Only support NUM_EXTRA=0,1,2,3,4')
+    L.require_shape(what, 'colors', colors, P, 3)
+    L.require_dtype(what, 'point_list', point_list, torch.int32)
+    L.require_dtype(what, 'ranges', ranges, torch.int64)
+    for name, t, dt in (('accum_max_count', accum_max_count, torch.int32),
+                        ('accum_weights_count', accum_weights_count, torch.int32)):
+        if t is not None:
+            L.require_dtype(what, name, t, dt)
+            L.require_shape(what, name, t, P)
+    if accum_weights_p is not None:
+        L.require_shape(what, 'accum_weights_p', accum_weights_p, P)
+    opt = dict(dtype=torch.float32, device=colors.device)
+    pixel_colors, pixel_opacity = torch.empty((3, height, width), **opt), torch.empty((height, width), **opt)
+    pixel_extras = torch.empty((E, height, width), **opt) if extras is not None else None
+    n_contrib = torch.empty((height, width), dtype=torch.int32, device=colors.device)
+    with _timed('gaussian_rasterize_forward'):
+        rc = _lib().fsgs_gaussian_rasterize_forward(
+            P, width, height, E, L.ptr(means2D), L.ptr(conic_opacity), L.ptr(colors), L.ptr(extras) if E else None,
+            L.ptr(point_list), L.ptr(ranges), L.ptr(accum_max_count), L.ptr(accum_weights_p),
+            L.ptr(accum_weights_count), L.ptr(pixel_colors), L.ptr(pixel_opacity),
+            L.ptr(pixel_extras) if E else None, L.ptr(n_contrib), L.current_stream())
+    L.check(rc, what)
+    return [pixel_colors, pixel_opacity, pixel_extras, n_contrib]
+
+
+def gaussian_rasterize_backward(means2D: Tensor, conic_opacity: Tensor, colors: Tensor, extras: Optional[Tensor],
+                                out_opacity: Tensor, dL_dout_color: Tensor, dL_dout_opacity: Tensor,
+                                dL_dout_extra: Optional[Tensor], ranges: Tensor, point_list: Tensor,
+                                n_contrib: Tensor):
+    """gaussian_render.cu:486-536 -> (dL_dcolors[P,3], dL_dextras[P,E]|None, dL_dmeans2D[P,2], dL_dconic_opacity[P,4])."""
+    what = 'gaussian_rasterize_backward'
+    L.require_cuda(what, dL_dout_color=dL_dout_color, dL_dout_opacity=dL_dout_opacity, dL_dout_extra=dL_dout_extra)
+    P = means2D.shape[0]
+    H, W = dL_dout_color.shape[1], dL_dout_color.shape[2]
+    E = extras.shape[-1] if (dL_dout_extra is not None and extras is not None) else 0
+    if E > 4:
+        raise RuntimeError('Only support NUM_EXTRA=0,1,2,3,4')
+    opt = dict(dtype=torch.float32, device=out_opacity.device)
+    grads = torch.zeros((P, 9 + E), **opt)  # one zero fill: means2D 2 | conic_opacity 4 | colours 3 | extras E
+    g_flat = grads.view(-1)
+    dL_dmeans2D = g_flat[:2 * P].view(P, 2)
+    dL_dconic_o = g_flat[2 * P:6 * P].view(P, 4)
+    dL_dcolors = g_flat[6 * P:9 * P].view(P, 3)
+    dL_dextras = g_flat[9 * P:].view(P, E) if E else None
+    if P == 0:
+        return dL_dcolors, dL_dextras, dL_dmeans2D, dL_dconic_o
+    c = lambda t: None if t is None else t.contiguous()
+    args = [c(means2D), c(conic_opacity), c(colors), c(extras) if E else None, c(out_opacity), c(n_contrib),
+            c(dL_dout_color), c(dL_dout_extra) if E else None, c(dL_dout_opacity), c(point_list), c(ranges)]
+    with _timed('gaussian_rasterize_backward'):
+        rc = _lib().fsgs_gaussian_rasterize_backward(
+            P, W, H, E, *[L.ptr(a) for a in args], L.ptr(dL_dmeans2D), L.ptr(dL_dconic_o), L.ptr(dL_dcolors),
+            L.ptr(dL_dextras), L.current_stream())
+    L.check(rc, what)
+    return dL_dcolors, dL_dextras, dL_dmeans2D, dL_dconic_o

@@ -1,0 +1,363 @@
+// Per-tile alpha blend of 3D Gaussians (conic footprint) and its backward, for gfx950.
+//
+// Reference behaviour reproduced: fast_2d_gs/_C/src/gaussian_splatting/gaussian_render.cu:20-173 (forward kernel; host
+// gaussian_rasterize_forward :212-293) and :296-444 (backward kernel; host gaussian_rasterize_backward :486-536):
+// alpha = min(0.99, o * exp(-0.5 (a dx^2 + c dy^2) - b dx dy)) with d = mean - pixel, skipped when the exponent is
+// positive or alpha < 1/255, front-to-back blending until T * (1 - alpha) < 1e-4; 3 colour channels plus up to 4 extra
+// per-Gaussian feature channels; optional accum_max_count / accum_weights_p / accum_weights_count. The backward walks
+// each tile's list back to front, rebuilding T by division, with the reference's accumulators
+// (sum of c * alpha * T behind the current Gaussian) and without masking the 0.99 clamp.
+//
+// Same skeleton as the surfel blend: one block = one 16x16 tile = 4 wavefronts x 8x8 quadrant, a batch of Gaussians
+// staged in LDS with the next batch's gather in flight, a conservative per-quadrant footprint test (bounding box of the
+// alpha >= 1/255 ellipse) whose ballot is the wavefront's work list, longest lists scheduled first. Where the
+// reference issues 9 + E global float atomics per (pixel, Gaussian) pair, the backward sums the 9 + E gradient
+// components over the 64 pixels of a wavefront with one transposed DPP butterfly, adds the four wavefronts' partials
+// with one 16-lane LDS atomic, and flushes one global atomic per Gaussian, component and tile.
+#include "blend.hpp"
+
+namespace fsgs {
+namespace {
+
+constexpr int kG3Batch = 128;   // Gaussians staged per round
+constexpr int kMaxExtra = 4;    // the reference dispatches E = 0..4 (gaussian_render.cu:455-481)
+
+struct __attribute__((aligned(16))) G3Hot {
+  float x, y;       // screen-space mean
+  float a, b, c;    // conic
+  float opacity;
+  int id;
+  unsigned mask;    // 8x8 quadrants of the tile the alpha >= 1/255 ellipse can reach
+};
+
+struct G3Entry {
+  G3Hot hot;
+  float feat[3 + kMaxExtra];
+};
+
+template <int E>
+__device__ __forceinline__ G3Entry gather_gaussian(int id, const float2* __restrict__ means2D,
+    const float4* __restrict__ conic_opacity, const float* __restrict__ colors, const float* __restrict__ extras) {
+  G3Entry g;
+  const float2 m = means2D[id];
+  const float4 co = conic_opacity[id];
+  g.hot.x = m.x, g.hot.y = m.y, g.hot.a = co.x, g.hot.b = co.y, g.hot.c = co.z, g.hot.opacity = co.w;
+  g.hot.id = id, g.hot.mask = 0xfu;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) g.feat[k] = colors[3 * (size_t) id + k];
+#pragma unroll
+  for (int k = 0; k < E; ++k) g.feat[3 + k] = extras[(size_t) E * id + k];
+  return g;
+}
+
+// alpha >= 1/255 needs 0.5 d^T Q d <= tau = ln(255 o) with Q = [[a, b], [b, c]]: for a positive definite Q that is an
+// ellipse with half extents sqrt(2 tau c / det), sqrt(2 tau a / det). Anything else (o < 1/255: never; Q not positive
+// definite: unbounded) is decided without a box.
+__device__ __forceinline__ unsigned conic_quadrant_mask(const G3Hot& h, int tile_px, int tile_py, int flags) {
+  if (flags & kFlagNoCull) return 0xfu;
+  const float oa = 255.0f * h.opacity;
+  if (!(oa >= 1.0f)) return 0u;
+  const float det = h.a * h.c - h.b * h.b;
+  if (!(det > 0.0f) || !(h.a > 0.0f)) return 0xfu;
+  const float tau2 = 2.0f * (__logf(oa) * 1.0001f + 1e-3f);
+  const float ex = sqrtf(tau2 * h.c / det), ey = sqrtf(tau2 * h.a / det);
+  if (!(ex == ex) || !(ey == ey)) return 0xfu;
+  const float padx = kCullPad + 0.01f * ex, pady = kCullPad + 0.01f * ey;
+  const float x0 = h.x - ex - padx, x1 = h.x + ex + padx, y0 = h.y - ey - pady, y1 = h.y + ey + pady;
+  unsigned m = 0u;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float qx = (float) (tile_px + (q & 1) * 8), qy = (float) (tile_py + (q >> 1) * 8);
+    if (x1 >= qx && x0 <= qx + 7.0f && y1 >= qy && y0 <= qy + 7.0f) m |= 1u << q;
+  }
+  return m;
+}
+
+struct G3Hit {
+  float dx, dy, G, alpha;
+};
+
+__device__ __forceinline__ bool conic_alpha(const G3Hot& h, float pxf, float pyf, G3Hit& o) {
+  o.dx = h.x - pxf, o.dy = h.y - pyf;
+  const float power = -0.5f * (h.a * o.dx * o.dx + h.c * o.dy * o.dy) - h.b * o.dx * o.dy;
+  if (power > 0.0f) return false;
+  o.G     = __expf(power);
+  o.alpha = fminf(0.99f, h.opacity * o.G);
+  return !(o.alpha < (1.0f / 255.0f));
+}
+
+template <int E, bool kAccum>
+__global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, int W, int H,
+    const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
+    const float4* __restrict__ conic_opacity, const float* __restrict__ colors, const float* __restrict__ extras,
+    float* __restrict__ out_color, float* __restrict__ out_opacity, float* __restrict__ out_extras,
+    int32_t* __restrict__ n_contrib, int32_t* __restrict__ accum_max_count, float* __restrict__ accum_weights_p,
+    int32_t* __restrict__ accum_weights_count) {
+  __shared__ G3Hot s_hot[kG3Batch];
+  __shared__ float s_feat[kG3Batch][3 + kMaxExtra + 1];  // odd stride
+  const int gx = (W + kTile - 1) / kTile;
+  const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
+  int px, py;
+  lane_pixel(tile_x, tile_y, px, py);
+  const bool inside = px < W && py < H;
+  const size_t HW = (size_t) H * W, pix = (size_t) W * py + px;
+  const float pxf = (float) px, pyf = (float) py;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
+  const int n_todo = (int) (r1 - r0);
+  const int rounds = (n_todo + kG3Batch - 1) / kG3Batch;
+
+  bool done = !inside;
+  float T = 1.0f, C[3 + (E > 0 ? E : 1)];
+#pragma unroll
+  for (int k = 0; k < 3 + E; ++k) C[k] = 0.0f;
+  int last = 0, wmax_id = -1;
+  float wmax = 0.0f;
+  bool flag = false;
+
+  G3Entry next;
+  if ((int) threadIdx.x < min(n_todo, kG3Batch))
+    next = gather_gaussian<E>(point_list[r0 + threadIdx.x], means2D, conic_opacity, colors, extras);
+  for (int b = 0; b < rounds; ++b) {
+    if (__syncthreads_count(done) == kBlendThreads) break;
+    const int n_here = min(kG3Batch, n_todo - b * kG3Batch);
+    if ((int) threadIdx.x < n_here) {
+      next.hot.mask = conic_quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile, flags);
+      s_hot[threadIdx.x] = next.hot;
+#pragma unroll
+      for (int k = 0; k < 3 + E; ++k) s_feat[threadIdx.x][k] = next.feat[k];
+    }
+    __syncthreads();
+    const int nxt = (b + 1) * kG3Batch + (int) threadIdx.x;
+    if ((int) threadIdx.x < kG3Batch && nxt < n_todo)
+      next = gather_gaussian<E>(point_list[r0 + nxt], means2D, conic_opacity, colors, extras);
+    for (int c = 0; c < kG3Batch / kWave; ++c) {
+      const int jj = c * kWave + lane;
+      unsigned long long todo = __ballot(jj < n_here && ((s_hot[jj < kG3Batch ? jj : 0].mask >> wave) & 1u));
+      while (todo) {
+        if (__ballot(!done) == 0ull) break;
+        const int j = c * kWave + __builtin_ctzll(todo);
+        todo &= todo - 1;
+        if (done) continue;
+        G3Hit h;
+        if (!conic_alpha(s_hot[j], pxf, pyf, h)) continue;
+        const float test_T = T * (1.0f - h.alpha);
+        if (test_T < 0.0001f) {
+          done = true;
+          continue;
+        }
+        const float w = h.alpha * T;
+#pragma unroll
+        for (int k = 0; k < 3 + E; ++k) C[k] += s_feat[j][k] * w;
+        if (kAccum) {
+          const int id = s_hot[j].id;
+          if (wmax < w) wmax = w, wmax_id = id, flag = true;
+          if (accum_weights_p) atomicAdd(&accum_weights_p[id], w);
+          if (accum_weights_count) atomicAdd(&accum_weights_count[id], 1);
+        }
+        T    = test_T;
+        last = b * kG3Batch + j + 1;
+      }
+    }
+  }
+  if (kAccum && flag && accum_max_count) atomicAdd(&accum_max_count[wmax_id], 1);
+  if (inside) {
+    out_opacity[pix] = 1.0f - T;
+    n_contrib[pix]   = last;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) out_color[k * HW + pix] = C[k];
+#pragma unroll
+    for (int k = 0; k < E; ++k) out_extras[k * HW + pix] = C[3 + k];
+  }
+}
+
+// gradient slots of one Gaussian: 0-2 colour | 3-6 extras | 7-8 mean2D | 9-11 conic | 12 opacity | 13-15 unused
+template <int E>
+__global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags, int W, int H,
+    const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
+    const float4* __restrict__ conic_opacity, const float* __restrict__ colors, const float* __restrict__ extras,
+    const float* __restrict__ out_opacity, const int32_t* __restrict__ n_contrib, const float* __restrict__ dL_dpix,
+    const float* __restrict__ dL_dout_extras, const float* __restrict__ dL_dout_opacity,
+    float* __restrict__ g_means2D, float* __restrict__ g_conic_opacity, float* __restrict__ g_colors,
+    float* __restrict__ g_extras) {
+  constexpr int kB = 64;
+  __shared__ G3Hot s_hot[kB];
+  __shared__ float s_feat[kB][3 + kMaxExtra + 1];
+  __shared__ float s_acc[kB][17];
+  __shared__ int s_max_contrib;
+  const int gx = (W + kTile - 1) / kTile;
+  const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
+  int px, py;
+  lane_pixel(tile_x, tile_y, px, py);
+  const bool inside = px < W && py < H;
+  const size_t HW = (size_t) H * W, pix = (size_t) W * py + px;
+  const float pxf = (float) px, pyf = (float) py;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
+  const int last_contrib = inside ? n_contrib[pix] : 0;
+
+  if (threadIdx.x == 0) s_max_contrib = 0;
+  __syncthreads();
+  int wave_max = last_contrib;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) wave_max = max(wave_max, __shfl_xor(wave_max, d, kWave));
+  if (lane == 0) atomicMax(&s_max_contrib, wave_max);
+  if ((int) threadIdx.x < kB)
+#pragma unroll
+    for (int c = 0; c < 17; ++c) s_acc[threadIdx.x][c] = 0.0f;
+  __syncthreads();
+  const int n_todo = min(s_max_contrib, (int) (r1 - r0));
+  const int rounds = (n_todo + kB - 1) / kB;
+
+  const float T_final = inside ? 1.0f - out_opacity[pix] : 0.0f;
+  float T = T_final;
+  const float dL_dT = inside ? -dL_dout_opacity[pix] : 0.0f;
+  float g_out[3 + (E > 0 ? E : 1)], accum[3 + (E > 0 ? E : 1)];
+#pragma unroll
+  for (int k = 0; k < 3 + E; ++k) {
+    accum[k] = 0.0f;
+    g_out[k] = !inside ? 0.0f : (k < 3 ? dL_dpix[k * HW + pix] : dL_dout_extras[(k - 3) * HW + pix]);
+  }
+
+  G3Entry next;
+  if ((int) threadIdx.x < min(n_todo, kB))
+    next = gather_gaussian<E>(point_list[r0 + (n_todo - 1 - (int) threadIdx.x)], means2D, conic_opacity, colors, extras);
+  for (int b = 0; b < rounds; ++b) {
+    const int n_here = min(kB, n_todo - b * kB);
+    if ((int) threadIdx.x < n_here) {
+      next.hot.mask = conic_quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile, flags);
+      s_hot[threadIdx.x] = next.hot;
+#pragma unroll
+      for (int k = 0; k < 3 + E; ++k) s_feat[threadIdx.x][k] = next.feat[k];
+    }
+    __syncthreads();
+    const int nxt = (b + 1) * kB + (int) threadIdx.x;
+    if ((int) threadIdx.x < kB && nxt < n_todo)
+      next = gather_gaussian<E>(point_list[r0 + (n_todo - 1 - nxt)], means2D, conic_opacity, colors, extras);
+
+    unsigned long long todo = __ballot(lane < n_here && ((s_hot[lane].mask >> wave) & 1u) &&
+                                       (n_todo - 1 - (b * kB + lane)) < wave_max);
+    while (todo) {
+      const int j = __builtin_ctzll(todo);
+      todo &= todo - 1;
+      const int pos = n_todo - 1 - (b * kB + j);  // 0-based position in the tile's list
+      G3Hit h;
+      const bool hit = (pos < last_contrib) && conic_alpha(s_hot[j], pxf, pyf, h);
+      if (__ballot(hit) == 0ull) continue;
+      float g[16];
+#pragma unroll
+      for (int c = 0; c < 16; ++c) g[c] = 0.0f;
+      if (hit) {
+        const G3Hot& hot = s_hot[j];
+        T = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+        const float dch = h.alpha * T;
+        float dL_dalpha = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 3 + E; ++k) {
+          const float v = s_feat[j][k];
+          dL_dalpha += (v * T * (1.0f - h.alpha) - accum[k]) * g_out[k];
+          accum[k] += v * dch;
+          g[k < 3 ? k : 3 + (k - 3)] = dch * g_out[k];
+        }
+        dL_dalpha = (dL_dalpha - T_final * dL_dT) * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+        const float dL_dG = -hot.opacity * h.G * dL_dalpha;
+        g[7]  = dL_dG * (hot.a * h.dx + hot.b * h.dy);
+        g[8]  = dL_dG * (hot.c * h.dy + hot.b * h.dx);
+        g[9]  = 0.5f * h.dx * h.dx * dL_dG;
+        g[10] = h.dx * h.dy * dL_dG;
+        g[11] = 0.5f * h.dy * h.dy * dL_dG;
+        g[12] = h.G * dL_dalpha;
+      }
+      const float tot = wave_sum16_transposed(g);
+      if (lane < 16) atomicAdd(&s_acc[j][lane], tot);
+    }
+    __syncthreads();
+    if ((int) threadIdx.x < n_here) {
+      float* a = s_acc[threadIdx.x];
+      const int id = s_hot[threadIdx.x].id;
+#pragma unroll
+      for (int c = 0; c < 3; ++c)
+        if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
+#pragma unroll
+      for (int c = 0; c < E; ++c)
+        if (a[3 + c] != 0.0f) atomicAdd(&g_extras[(size_t) E * id + c], a[3 + c]);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+        if (a[7 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[7 + c]);
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (a[9 + c] != 0.0f) atomicAdd(&g_conic_opacity[4 * (size_t) id + c], a[9 + c]);
+#pragma unroll
+      for (int c = 0; c < 16; ++c) a[c] = 0.0f;
+    }
+    // a lane only touches its own accumulator row and staged entry between this flush and the barrier that follows
+    // the next batch's LDS store
+  }
+}
+
+}  // namespace
+}  // namespace fsgs
+
+using namespace fsgs;
+
+FSGS_API int fsgs_gaussian_rasterize_forward(int P, int W, int H, int E, const float* means2D,
+    const float* conic_opacity, const float* colors, const float* extras, const int32_t* point_list,
+    const int64_t* ranges, int32_t* accum_max_count, float* accum_weights_p, int32_t* accum_weights_count,
+    float* out_color, float* out_opacity, float* out_extras, int32_t* n_contrib, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "gaussian_rasterize_forward: bad sizes");
+  FSGS_REQUIRE(E >= 0 && E <= kMaxExtra, "gaussian_rasterize_forward: only 0..%d extra channels are supported", kMaxExtra);
+  FSGS_REQUIRE(ranges && out_color && out_opacity && n_contrib && (E == 0 || (extras && out_extras)),
+               "gaussian_rasterize_forward: null pointer");
+  FSGS_REQUIRE(P == 0 || (means2D && conic_opacity && colors), "gaussian_rasterize_forward: null pointer");
+  hipStream_t s = (hipStream_t) stream;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const int flags = launch_tile_order(gx, gy, ranges, s);
+  const dim3 grid(gx * gy), block(kBlendThreads);
+  const bool accum = accum_max_count || accum_weights_p || accum_weights_count;
+#define FSGS_G3_FWD(EE, ACC)                                                                                        \
+  hipLaunchKernelGGL((gs3d_forward_kernel<EE, ACC>), grid, block, 0, s, flags, W, H, ranges, point_list,           \
+                     (const float2*) means2D, (const float4*) conic_opacity, colors, extras, out_color,             \
+                     out_opacity, out_extras, n_contrib, accum_max_count, accum_weights_p, accum_weights_count)
+#define FSGS_G3_FWD_E(EE) \
+  if (accum) FSGS_G3_FWD(EE, true); else FSGS_G3_FWD(EE, false)
+  switch (E) {
+    case 0: FSGS_G3_FWD_E(0); break;
+    case 1: FSGS_G3_FWD_E(1); break;
+    case 2: FSGS_G3_FWD_E(2); break;
+    case 3: FSGS_G3_FWD_E(3); break;
+    default: FSGS_G3_FWD_E(4); break;
+  }
+#undef FSGS_G3_FWD_E
+#undef FSGS_G3_FWD
+  return check_launch("gaussian_rasterize_forward");
+}
+
+FSGS_API int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const float* means2D,
+    const float* conic_opacity, const float* colors, const float* extras, const float* out_opacity,
+    const int32_t* n_contrib, const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity,
+    const int32_t* point_list, const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors,
+    float* g_extras, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "gaussian_rasterize_backward: bad sizes");
+  FSGS_REQUIRE(E >= 0 && E <= kMaxExtra, "gaussian_rasterize_backward: only 0..%d extra channels are supported", kMaxExtra);
+  if (P == 0) return kOk;
+  FSGS_REQUIRE(means2D && conic_opacity && colors && out_opacity && n_contrib && dL_dpix && dL_dout_opacity && ranges &&
+                   g_means2D && g_conic_opacity && g_colors && (E == 0 || (extras && dL_dout_extras && g_extras)),
+               "gaussian_rasterize_backward: null pointer");
+  hipStream_t s = (hipStream_t) stream;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const int flags = launch_tile_order(gx, gy, ranges, s);
+  const dim3 grid(gx * gy), block(kBlendThreads);
+#define FSGS_G3_BWD(EE)                                                                                             \
+  hipLaunchKernelGGL((gs3d_backward_kernel<EE>), grid, block, 0, s, flags, W, H, ranges, point_list,               \
+                     (const float2*) means2D, (const float4*) conic_opacity, colors, extras, out_opacity, n_contrib, \
+                     dL_dpix, dL_dout_extras, dL_dout_opacity, g_means2D, g_conic_opacity, g_colors, g_extras)
+  switch (E) {
+    case 0: FSGS_G3_BWD(0); break;
+    case 1: FSGS_G3_BWD(1); break;
+    case 2: FSGS_G3_BWD(2); break;
+    case 3: FSGS_G3_BWD(3); break;
+    default: FSGS_G3_BWD(4); break;
+  }
+#undef FSGS_G3_BWD
+  return check_launch("gaussian_rasterize_backward");
+}

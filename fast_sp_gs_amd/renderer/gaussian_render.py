@@ -1,0 +1,184 @@
+"""Host side of the 3D-Gaussian (EWA) render path on the HIP operators: the autograd wiring and entry points of the
+reference's fast_2d_gs/renderer/gaussian_render.py (`_preprocess` :495-566, `preprocess` :569-, `GS_prepare` :742-772,
+`_GS_render` :775-800, `GS_render` :840-, `RasterizeGaussians` :226-274, `render` :277-359) for covariances computed
+from scales + rotations. Extra feature channels beyond the first group of <= 4 (`render_extra`), pre-computed
+covariances and camera gradients are not part of this build and raise."""
+from __future__ import annotations
+
+from typing import NamedTuple, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from fast_sp_gs_amd._C import get_C_function
+from fast_sp_gs_amd.renderer.gs_2d_render import GS_prepare
+
+__all__ = ['RasterizeBuffer3D', 'preprocess', 'GS_render', 'RasterizeGaussians', 'render']
+
+
+class RasterizeBuffer3D(NamedTuple):
+    """gaussian_render.py:37-51"""
+    W: int
+    H: int
+    P: int
+    R: int
+    tile_ranges: Tensor
+    point_list: Tensor
+    n_contribed: Tensor
+    conic_opacity: Tensor
+    means2D: Tensor
+    opacity: Tensor
+
+
+class _preprocess(torch.autograd.Function):
+    _forward = get_C_function('gs_preprocess_forward')
+    _backward = get_C_function('gs_preprocess_backward')
+
+    @staticmethod
+    def forward(ctx, means3D, scales, rotations, opacities, sh_or_colors, sh_rest, Tw2v, Tv2c, campos, tanFoV, W, H,
+                sh_degree, is_opengl, cov3D, cov2D, means2D, culling):
+        if cov3D is not None or cov2D is not None:
+            raise RuntimeError('pre-computed covariances are not supported by this library')
+        tan = (float(tanFoV[0]), float(tanFoV[1]))
+        ctx._args = (W, H, sh_degree, is_opengl, tan)
+        means2D, depths, colors, radii, tiles_touched, cov3D, conic_opacity = _preprocess._forward(
+            W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, sh_or_colors, sh_rest, Tw2v, Tv2c,
+            campos, tan, None, None, means2D, culling)
+        ctx.save_for_backward(means3D, scales, rotations, opacities, sh_or_colors, sh_rest, Tw2v, Tv2c, campos, cov3D,
+                              radii, colors)
+        ctx.mark_non_differentiable(radii, tiles_touched)
+        return means2D, depths, colors, radii, tiles_touched, conic_opacity
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, g_means2D, g_depths, g_colors, _g_radii, _g_tiles, g_conic):
+        means3D, scales, rotations, opacities, sh_or_colors, sh_rest, Tw2v, Tv2c, campos, cov3D, radii, colors = \
+            ctx.saved_tensors
+        W, H, sh_degree, is_opengl, tan = ctx._args
+        if ctx.needs_input_grad[6] or ctx.needs_input_grad[8]:
+            raise RuntimeError('camera gradients are not supported by this library')
+        P = means3D.shape[0]
+        zeros = lambda *shape: torch.zeros(shape, dtype=torch.float32, device=means3D.device)
+        g_means2D = zeros(P, 2) if g_means2D is None else g_means2D.contiguous().clone()
+        g_conic = zeros(P, 4) if g_conic is None else g_conic.contiguous()
+        g_colors = zeros(P, 3) if g_colors is None else g_colors.contiguous()
+        # every row of these is assigned by the kernel
+        grad_means3D, grad_opacities = torch.empty_like(means3D), torch.empty_like(opacities)
+        grad_scales = torch.empty_like(scales) if ctx.needs_input_grad[1] else None
+        grad_rotations = torch.empty_like(rotations) if ctx.needs_input_grad[2] else None
+        grad_shs = torch.empty_like(sh_or_colors) if sh_degree >= 0 and ctx.needs_input_grad[4] else None
+        grad_sh_rest = torch.empty_like(sh_rest) if (sh_degree >= 0 and sh_rest is not None and
+                                                     ctx.needs_input_grad[5]) else None
+        _preprocess._backward(W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, sh_or_colors, sh_rest,
+                              Tw2v, Tv2c, campos, tan, cov3D, None, radii, colors, g_means2D, None, g_colors, g_conic,
+                              grad_means3D, grad_scales, grad_rotations, grad_opacities, grad_shs, grad_sh_rest, None,
+                              None, None)
+        grad_inputs = [grad_means3D, grad_scales, grad_rotations, grad_opacities, grad_shs, grad_sh_rest] + [None] * 12
+        if sh_degree < 0:
+            grad_inputs[4] = g_colors if ctx.needs_input_grad[4] else None  # pre-computed colours pass through
+        # the dummy screen-space leaf receives the (rewritten) screen-space gradient: it is what densification reads
+        grad_inputs[-2] = g_means2D if ctx.needs_input_grad[-2] else None
+        return tuple(grad_inputs)
+
+
+def preprocess(means3D: Tensor, scales: Tensor, rotations: Tensor, opacities: Tensor, sh_or_colors: Tensor,
+               sh_rest: Optional[Tensor], Tw2v: Tensor, Tv2c: Tensor, campos: Tensor, tanFoV: Tensor, W: int, H: int,
+               sh_degree=0, is_opengl=True, cov3D: Tensor = None, cov2D: Tensor = None, means2D: Tensor = None,
+               culling: Tensor = None):
+    """-> (means2D, depths, colors, radii, tiles_touched, conic_opacity); gaussian_render.py:569-626."""
+    return _preprocess.apply(means3D, scales, rotations, opacities, sh_or_colors, sh_rest, Tw2v, Tv2c, campos, tanFoV,
+                             W, H, sh_degree, is_opengl, cov3D, cov2D, means2D, culling)
+
+
+class _GS_render(torch.autograd.Function):
+    _forward = get_C_function('gaussian_rasterize_forward')
+    _backward = get_C_function('gaussian_rasterize_backward')
+
+    @staticmethod
+    def forward(ctx, W, H, mean2D, colors, conic_opacity, tile_range, point_list, extras, accum_max_count,
+                accum_weights_p, accum_weights_count):
+        images, out_opacity, out_extras, n_contrib = _GS_render._forward(
+            W, H, mean2D, conic_opacity, colors, extras, point_list, tile_range, accum_max_count, accum_weights_p,
+            accum_weights_count, None)
+        ctx.save_for_backward(mean2D, colors, conic_opacity, extras, tile_range, point_list, out_opacity, n_contrib)
+        ctx.mark_non_differentiable(n_contrib)
+        return images, out_opacity, out_extras, n_contrib
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_images, grad_alpha, grad_out_extra, _):
+        mean2D, colors, conic_opacity, extras, tile_range, point_list, out_opacity, n_contrib = ctx.saved_tensors
+        zeros_like = lambda t: torch.zeros_like(t)
+        grad_images = zeros_like(out_opacity).expand(3, -1, -1).contiguous() if grad_images is None else grad_images
+        grad_alpha = zeros_like(out_opacity) if grad_alpha is None else grad_alpha
+        if extras is not None and grad_out_extra is None:
+            grad_out_extra = torch.zeros((extras.shape[1],) + tuple(out_opacity.shape), dtype=torch.float32,
+                                         device=out_opacity.device)
+        grad_colors, grad_extra, grad_means2D, grad_conic_opacity = _GS_render._backward(
+            mean2D, conic_opacity, colors, extras, out_opacity, grad_images.contiguous(), grad_alpha.contiguous(),
+            None if grad_out_extra is None else grad_out_extra.contiguous(), tile_range, point_list, n_contrib)
+        return None, None, grad_means2D, grad_colors, grad_conic_opacity, None, None, grad_extra, None, None, None
+
+
+def GS_render(W: int, H: int, mean2D: Tensor, colors: Tensor, conic_opacity: Tensor, tile_range: Tensor,
+              point_list: Tensor, extra: Tensor = None, accum_max_count=None, accum_weights_p=None,
+              accum_weights_count=None):
+    """-> (images[3,H,W], opacity[H,W], extras[E,H,W]|None, n_contrib[H,W]); gaussian_render.py:839-845."""
+    return _GS_render.apply(W, H, mean2D, colors, conic_opacity, tile_range, point_list, extra, accum_max_count,
+                            accum_weights_p, accum_weights_count)
+
+
+def RasterizeGaussians(means3D: Tensor, means2D: Optional[Tensor], colors: Tensor, sh_rest: Optional[Tensor],
+                       opacities: Tensor, scales: Optional[Tensor], rotations: Optional[Tensor],
+                       cov3Ds_precomp: Optional[Tensor], cov2Ds_precomp: Optional[Tensor], extras: Optional[Tensor],
+                       image_size: Tuple[int, int], sh_degree: int, Tw2v: Tensor, Tv2c: Tensor, cam_pos: Tensor,
+                       tanFoV: Tensor, is_opengl: bool, culling: Optional[Tensor], accum_max_count: Optional[Tensor],
+                       accum_weights_p: Optional[Tensor], accum_weights_count: Optional[Tensor], *other_extras: Tensor):
+    """gaussian_render.py:226-274: preprocess -> binning -> blend."""
+    if other_extras:
+        raise RuntimeError('RasterizeGaussians: additional extra groups (render_extra) are not supported by this library')
+    W, H = image_size
+    means2D, depths, colors, radii, tiles_touched, conic_opacity = preprocess(
+        means3D, scales, rotations, opacities, colors, sh_rest, Tw2v, Tv2c, cam_pos, tanFoV, W, H, sh_degree,
+        is_opengl, cov3Ds_precomp, cov2Ds_precomp, means2D, culling)
+    tile_ranges, point_list = GS_prepare(W, H, means2D.detach(), depths.detach(), radii, tiles_touched, False)
+    out_pixels, out_opacities, out_extras, n_contrib = GS_render(
+        W, H, means2D, colors, conic_opacity, tile_ranges, point_list, extras, accum_max_count, accum_weights_p,
+        accum_weights_count)
+    buffer = RasterizeBuffer3D(W, H, len(opacities), point_list.shape[0], tile_ranges, point_list, n_contrib,
+                               conic_opacity, means2D, out_opacities)
+    return out_pixels, out_opacities, out_extras, radii, buffer
+
+
+def render(Tw2v: Tensor, Tv2c: Tensor, size: Tuple[int, int], points: Tensor, opacity: Tensor, scales: Tensor = None,
+           rotations: Tensor = None, campos: Tensor = None, FoV: Tensor = None, focals: Tensor = None,
+           cov3Ds: Tensor = None, cov2Ds: Tensor = None, sh_features: Tensor = None, sh_features_rest: Tensor = None,
+           colors: Tensor = None, sh_degree=0, is_opengl=False, culling: Tensor = None,
+           accum_max_count: Tensor = None, accum_weights_p: Tensor = None, accum_weights_count: Tensor = None,
+           **kwargs):
+    """Same inputs, outputs and dict keys as the reference's `render` (gaussian_render.py:277-359)."""
+    means2D = torch.zeros_like(points[:, :2]).contiguous().requires_grad_()
+    if campos is None:
+        campos = Tw2v.inverse()[:3, 3].contiguous()
+    if FoV is None:
+        tanFoV = 0.5 * torch.as_tensor(size, device=Tw2v.device) / focals
+    else:
+        tanFoV = torch.tan(torch.as_tensor(FoV) * 0.5)
+    extras, extra_key = None, None
+    for k, v in list(kwargs.items()):
+        if isinstance(v, Tensor) and v.shape[-1] <= 4:
+            extras, extra_key = v, k
+            kwargs.pop(k)
+            break
+    c = lambda t: None if t is None else t.contiguous()
+    image, out_opacity, out_extra, radii, buffer = RasterizeGaussians(
+        points.contiguous(), means2D, c(sh_features) if colors is None else colors.contiguous(), c(sh_features_rest),
+        opacity.contiguous(), c(scales), c(rotations), c(cov3Ds), c(cov2Ds), c(extras), size,
+        sh_degree if colors is None else -1, Tw2v.view(4, 4).contiguous(), Tv2c.view(4, 4).contiguous(),
+        campos.view(3).contiguous(), tanFoV.view(2), is_opengl, culling, accum_max_count, accum_weights_p,
+        accum_weights_count, *[v for v in kwargs.values() if isinstance(v, Tensor)])
+    out = {'images': image, 'opacity': out_opacity, 'viewspace_points': means2D, 'visibility_filter': radii > 0,
+           'radii': radii, 'buffer': buffer}
+    if extra_key is not None:
+        out[extra_key] = out_extra
+    return out

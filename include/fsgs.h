@@ -251,6 +251,47 @@ size_t fsgs_knn_topk_backward_workspace_bytes(int N, int M, int D);
 int fsgs_knn_topk_backward(int N, int M, int D, int K, const float* x, const float* y, const int64_t* index,
     const float* g_dist2, float* g_x, float* g_y, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- 3D-Gaussian (EWA) path ------------------------------------------------------------------------------------ */
+
+/* gs_preprocess_forward -- fast_2d_gs/_C/src/gaussian_splatting/gaussian_preprocess.cu:372-466 (kernel :44-128):
+ * scales[P,3], rotations[P,4] (x,y,z,w, used as given), opacities[P,1], shs[P,n_sh,3] (or shs[P,1,3] + sh_rest, or
+ * colours[P,3] with sh_degree < 0), Tw2v, Tv2c [4,4], campos[3], tan(FoV/2) per axis -> means2D[P,2] (pixel - 0.5
+ * convention unless is_opengl), depths[P], colors[P,3], radii[P], tiles_touched[P], cov3Ds[P,6], conic_opacity[P,4].
+ * Covariances always come from scales + rotations (the reference's cov3D_precomp / cov2D_precomp inputs are not
+ * implemented). Every row of every output is written; means2D_preserve keeps the caller's means2D rows of Gaussians
+ * that are not rendered. culling: optional P bytes, non-zero = skip. */
+int fsgs_gs_preprocess_forward(int P, int W, int H, int sh_degree, int n_sh, int is_opengl, const float* means3D,
+    const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
+    const float* Tw2v, const float* Tv2c, const float* campos, double tan_fovx, double tan_fovy,
+    const uint8_t* culling, int means2D_preserve, float* means2D, float* depths, float* colors, int32_t* radii,
+    int32_t* tiles_touched, float* cov3Ds, float* conic_opacity, void* stream);
+
+/* gs_preprocess_backward -- gaussian_preprocess.cu:567-636 (kernel :246-372, with gaussian_compute_cov2D.cu:64-186 and
+ * gaussian_compute_cov3D.cu:76-118). grad_mean2D[P,2] is rewritten in place as (0.5 W g.x, +-0.5 H g.y) as in the
+ * reference; grad_conic[P,4] carries dL/dconic and dL/dopacity. All gradient rows are assigned (zeros for Gaussians
+ * that were not rendered). g_scales, g_rot, g_shs, g_sh_rest, g_cov3D are optional. No camera gradients. */
+int fsgs_gs_preprocess_backward(int P, int W, int H, int sh_degree, int n_sh, int is_opengl, const float* means3D,
+    const float* scales, const float* rotations, const float* shs, const float* sh_rest, const float* Tw2v,
+    const float* Tv2c, const float* campos, double tan_fovx, double tan_fovy, const int32_t* radii,
+    const float* colors, const float* cov3Ds, float* grad_mean2D, const float* grad_colors, const float* grad_conic,
+    float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs, float* g_sh_rest, float* g_cov3D,
+    void* stream);
+
+/* gaussian_rasterize_forward -- gaussian_render.cu:212-293 (kernel :20-173) without the bucket snapshots of the
+ * per-Gaussian backward. colors[P,3], extras[P,E] (E <= 4, optional) -> out_color[3,H,W], out_opacity[H,W],
+ * out_extras[E,H,W], n_contrib[H,W]; every output element is written. accum_* as in the surfel forward. */
+int fsgs_gaussian_rasterize_forward(int P, int W, int H, int E, const float* means2D, const float* conic_opacity,
+    const float* colors, const float* extras, const int32_t* point_list, const int64_t* ranges,
+    int32_t* accum_max_count, float* accum_weights_p, int32_t* accum_weights_count, float* out_color,
+    float* out_opacity, float* out_extras, int32_t* n_contrib, void* stream);
+
+/* gaussian_rasterize_backward -- gaussian_render.cu:486-536 (kernel :296-444). Accumulates into caller-zeroed
+ * g_means2D[P,2], g_conic_opacity[P,4], g_colors[P,3], g_extras[P,E]. */
+int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const float* means2D, const float* conic_opacity,
+    const float* colors, const float* extras, const float* out_opacity, const int32_t* n_contrib,
+    const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
+    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, void* stream);
+
 /* ---- render epilogue -------------------------------------------------------------------------------------------- */
 
 /* Everything fast_2d_gs/renderer/gs_2d_render.py:608-617 does per pixel after the blend, in one kernel: normals[3,H,W] =

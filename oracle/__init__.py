@@ -239,3 +239,66 @@ def fast_render_backward(near, far, per_splat_form, means2D, normal_opacity, col
               dL_dextras, ranges, point_list, n_contrib, gc, gm, gt, gi, gn)
     assert rc == 0
     return gc, gm, gt, gi, gn
+
+
+# ---- 3D-Gaussian (EWA) path ------------------------------------------------------------------------------------------
+def gs3d_preprocess_forward(W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs, sh_rest, Tw2v,
+                            Tv2c, campos, tan_fov, culling=None, means2D=None):
+    dt = means3D.dtype
+    P = means3D.shape[0]
+    n_sh = 0 if sh_degree < 0 else (sh_rest.shape[1] if sh_rest is not None else shs.shape[1])
+    m2 = np.zeros((P, 2), dt) if means2D is None else means2D
+    depths, cov3D, conic = np.zeros((P,), dt), np.zeros((P, 6), dt), np.zeros((P, 4), dt)
+    colors = np.zeros((P, 3), dt) if sh_degree >= 0 else shs
+    radii, tt = np.zeros((P,), np.int32), np.zeros((P,), np.int32)
+    cull = None if culling is None else np.ascontiguousarray(culling.astype(np.uint8))
+    rc = call(f"gs3d_preprocess_forward_{_suffix(dt)}", P, W, H, sh_degree, n_sh, int(is_opengl), means3D, scales,
+              rotations, opacities, shs, sh_rest, Tw2v, Tv2c, campos, float(tan_fov[0]), float(tan_fov[1]), cull, m2,
+              depths, colors, radii, tt, cov3D, conic)
+    assert rc == 0
+    return m2, depths, colors, radii, tt, cov3D, conic
+
+
+def gs3d_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotations, shs, sh_rest, Tw2v, Tv2c, campos,
+                             tan_fov, radii, colors, cov3D, grad_mean2D, grad_colors, grad_conic):
+    """-> (g_means3D, g_scales, g_rot, g_opac, g_shs, g_sh_rest, g_cov3D, grad_mean2D rewritten)"""
+    dt = means3D.dtype
+    P = means3D.shape[0]
+    n_sh = 0 if sh_degree < 0 else (sh_rest.shape[1] if sh_rest is not None else shs.shape[1])
+    g3, gs, gq, go = np.zeros((P, 3), dt), np.zeros((P, 3), dt), np.zeros((P, 4), dt), np.zeros((P, 1), dt)
+    gsh = np.zeros_like(shs) if sh_degree >= 0 else None
+    grest = np.zeros_like(sh_rest) if (sh_degree >= 0 and sh_rest is not None) else None
+    gcov = np.zeros((P, 6), dt)
+    gm2 = np.ascontiguousarray(grad_mean2D.copy())
+    rc = call(f"gs3d_preprocess_backward_{_suffix(dt)}", P, W, H, sh_degree, n_sh, int(is_opengl), means3D, scales,
+              rotations, shs, sh_rest, Tw2v, Tv2c, campos, float(tan_fov[0]), float(tan_fov[1]), radii, colors, cov3D,
+              gm2, grad_colors, grad_conic, g3, gs, gq, go, gsh, grest, gcov)
+    assert rc == 0
+    return g3, gs, gq, go, gsh, grest, gcov, gm2
+
+
+def gs3d_render_forward(W, H, means2D, conic_opacity, colors, extras, point_list, ranges, accum_max_count=None,
+                        accum_weights_p=None, accum_weights_count=None):
+    dt = means2D.dtype
+    E = 0 if extras is None else extras.shape[1]
+    oc, oo = np.zeros((3, H, W), dt), np.zeros((H, W), dt)
+    oe = np.zeros((E, H, W), dt) if E else None
+    nc = np.zeros((H, W), np.int32)
+    rc = call(f"gs3d_render_forward_{_suffix(dt)}", W, H, E, means2D, conic_opacity, colors, extras, point_list, ranges,
+              oc, oo, oe, nc, accum_max_count, accum_weights_p, accum_weights_count)
+    assert rc == 0
+    return oc, oo, oe, nc
+
+
+def gs3d_render_backward(W, H, means2D, conic_opacity, colors, extras, out_opacity, n_contrib, dL_dpix, dL_dextras,
+                         dL_dopacity, point_list, ranges):
+    """-> (g_colors, g_extras, g_means2D, g_conic_opacity)"""
+    dt = means2D.dtype
+    P = means2D.shape[0]
+    E = 0 if extras is None else extras.shape[1]
+    gm, gc, gcol = np.zeros((P, 2), dt), np.zeros((P, 4), dt), np.zeros((P, 3), dt)
+    gex = np.zeros((P, E), dt) if E else None
+    rc = call(f"gs3d_render_backward_{_suffix(dt)}", W, H, E, means2D, conic_opacity, colors, extras, out_opacity,
+              n_contrib, dL_dpix, dL_dextras, dL_dopacity, point_list, ranges, gm, gc, gcol, gex)
+    assert rc == 0
+    return gcol, gex, gm, gc

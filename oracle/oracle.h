@@ -68,6 +68,24 @@ int oracle_gs_2d_epilogue_backward_f32(int W, int H, double ratio, const float* 
     const float* g_surf_depth, const float* g_surf_normal, const float* g_distortion, const float* g_composited,
     float* g_extras, float* g_opacity);
 int oracle_simple_knn_f32(int P, const float* points, float* mean_dist2);
+int oracle_gs3d_preprocess_forward_f32(int P, int W, int H, int sh_degree, int n_sh, int is_opengl,
+    const float* means3D, const float* scales, const float* rotations, const float* opacities, const float* shs,
+    const float* sh_rest, const float* Tw2v, const float* Tv2c, const float* campos, double tanx, double tany,
+    const uint8_t* culling, float* means2D, float* depths, float* colors, int32_t* radii, int32_t* tiles_touched,
+    float* cov3Ds, float* conic_opacity);
+int oracle_gs3d_preprocess_backward_f32(int P, int W, int H, int sh_degree, int n_sh, int is_opengl,
+    const float* means3D, const float* scales, const float* rotations, const float* shs, const float* sh_rest,
+    const float* Tw2v, const float* Tv2c, const float* campos, double tanx, double tany, const int32_t* radii,
+    const float* colors, const float* cov3Ds, float* grad_mean2D, const float* grad_colors, const float* grad_conic,
+    float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs, float* g_sh_rest, float* g_cov3D);
+int oracle_gs3d_render_forward_f32(int W, int H, int E, const float* means2D, const float* conic_opacity,
+    const float* colors, const float* extras, const int32_t* point_list, const int64_t* ranges, float* out_color,
+    float* out_opacity, float* out_extras, int32_t* n_contrib, int32_t* accum_max_count, float* accum_weights_p,
+    int32_t* accum_weights_count);
+int oracle_gs3d_render_backward_f32(int W, int H, int E, const float* means2D, const float* conic_opacity,
+    const float* colors, const float* extras, const float* out_opacity, const int32_t* n_contrib,
+    const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
+    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras);
 int64_t oracle_gs_prepare_count(int P, const int32_t* tiles_touched, int64_t* offsets);
 int oracle_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
     const int64_t* offsets, int64_t R, int64_t* ranges, int32_t* point_list, int64_t* keys_sorted_out);

@@ -1,0 +1,169 @@
+"""GPU parity of the 3D-Gaussian (EWA) path against the oracle, through the operators: preprocess forward (bit-exact
+geometry) / backward, rasterise forward / backward with 0..4 extra channels and the accumulators, and the autograd entry
+point `gaussian_render.render` end to end. Tolerances as for the surfel path: images 1e-4 abs, gradients 1e-3 of the
+largest entry; contraction is off in the geometry, on in the blend kernels."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from util import abs_err, npy, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _scene(P, W, H, seed, device):
+    from fast_sp_gs_amd import scenes
+    scene, _ = scenes.config0(P=P, size=max(W, H), seed=seed)
+    cam = scenes.pinhole(W, H, 50.0, torch.tensor([0.3, -0.2, 4.0]))
+    g = torch.Generator().manual_seed(seed + 100)
+    scales = torch.cat([scene.scales * 3, scene.scales[:, :1] * (0.5 + 3.5 * torch.rand(P, 1, generator=g))], 1).contiguous()
+    scene.means3D[::9, 2] += 9.0  # some behind the camera
+    tan_fov = (W / 2 / float(cam.Tv2s[0, 0]), H / 2 / float(cam.Tv2s[1, 1]))
+    return scene, scales, cam, tan_fov
+
+
+@pytest.mark.parametrize("name,deg,P,W,H", [("deg3", 3, 5001, 200, 120), ("deg0", 0, 3000, 97, 65),
+                                            ("colors", -1, 2000, 64, 64), ("deg4", 4, 1500, 80, 48)])
+def test_gs3d_preprocess(name, deg, P, W, H, device):
+    from fast_sp_gs_amd._C import get_C_function
+    scene, scales, cam, tan_fov = _scene(P, W, H, 21, device)
+    g = torch.Generator().manual_seed(5)
+    n_rows = {3: 16, 0: 1, 4: 25}.get(deg, 0)
+    shs = torch.rand(P, 3, generator=g) if deg < 0 else (torch.randn(P, n_rows, 3, generator=g) * 0.3)
+    culling = torch.rand(P, generator=g) < 0.1
+    d = lambda t: None if t is None else t.to(device).contiguous()
+    print(f"[gs3d preprocess {name}] P={P} {W}x{H}", flush=True)
+    out = get_C_function('gs_preprocess_forward')(
+        W, H, deg, False, d(scene.means3D), d(scales), d(scene.rotations), d(scene.opacities), d(shs), None,
+        d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), tan_fov, None, None, None, d(culling))
+    torch.cuda.synchronize()
+    m2, dep, col, rad, tt, c3, co = [npy(t) for t in out]
+    ref = O.gs3d_preprocess_forward(W, H, deg, False, npy(scene.means3D), npy(scales), npy(scene.rotations),
+                                    npy(scene.opacities), npy(shs), None, npy(cam.Tw2v), npy(cam.Tv2c),
+                                    npy(cam.campos), tan_fov, culling=npy(culling))
+    r_m2, r_dep, r_col, r_rad, r_tt, r_c3, r_co = ref
+    assert 0 < (rad > 0).sum() < P
+    assert np.array_equal(rad, r_rad) and np.array_equal(tt, r_tt)
+    assert np.array_equal(m2, r_m2) and np.array_equal(dep, r_dep) and np.array_equal(co, r_co)
+    assert np.array_equal(c3, r_c3)
+    assert abs_err(col, r_col) < 2e-6
+
+    gm2, gcol, gco = torch.randn(P, 2, generator=g), torch.randn(P, 3, generator=g), torch.randn(P, 4, generator=g)
+    nan = lambda *shape: torch.full(shape, float('nan'), device=device)
+    g3, gs, gq, gop, gcov = nan(P, 3), nan(P, 3), nan(P, 4), nan(P, 1), nan(P, 6)
+    gsh = None if deg < 0 else nan(*shs.shape)
+    gm2_d = d(gm2)
+    get_C_function('gs_preprocess_backward')(
+        W, H, deg, False, d(scene.means3D), d(scales), d(scene.rotations), d(scene.opacities), d(shs), None,
+        d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), tan_fov, out[5], None, out[3], out[2], gm2_d, None, d(gcol), d(gco),
+        g3, gs, gq, gop, gsh, None, gcov)
+    torch.cuda.synchronize()
+    r3, rs, rq, rop, rsh, _, rcov, rm2 = O.gs3d_preprocess_backward(
+        W, H, deg, False, npy(scene.means3D), npy(scales), npy(scene.rotations), npy(shs), None, npy(cam.Tw2v),
+        npy(cam.Tv2c), npy(cam.campos), tan_fov, rad, col, c3, npy(gm2), npy(gcol), npy(gco))
+    vis = rad > 0
+    pairs = dict(means3D=(g3, r3), scales=(gs, rs), rot=(gq, rq), opac=(gop, rop), cov3D=(gcov, rcov))
+    if gsh is not None:
+        pairs['shs'] = (gsh, rsh)
+    for k, (a, b) in pairs.items():
+        a = npy(a)
+        assert np.isfinite(a).all(), f"{k}: rows left unwritten"
+        assert rel_err(a, b) < 1e-5, (k, rel_err(a, b))
+        assert not a[~vis].any(), k
+    assert np.array_equal(npy(gm2_d)[vis], rm2[vis]) and np.array_equal(npy(gm2_d)[~vis], npy(gm2)[~vis])
+
+
+def _binned(P, W, H, seed, device):
+    from fast_sp_gs_amd._C import get_C_function
+    scene, scales, cam, tan_fov = _scene(P, W, H, seed, device)
+    d = lambda t: None if t is None else t.to(device).contiguous()
+    out = get_C_function('gs_preprocess_forward')(
+        W, H, 3, False, d(scene.means3D), d(scales), d(scene.rotations), d(scene.opacities), d(scene.shs), None,
+        d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), tan_fov, None, None, None, None)
+    m2, dep, col, rad, tt, c3, co = out
+    ranges, pl = get_C_function('GS_prepare')(W, H, m2, dep, rad, tt, False)
+    return m2, col, co, ranges, pl
+
+
+@pytest.mark.parametrize("P,W,H,E", [(4000, 160, 96, 0), (4000, 131, 77, 2), (20000, 128, 128, 4), (3, 40, 40, 1)])
+def test_gs3d_rasterize(P, W, H, E, device):
+    from fast_sp_gs_amd._C import get_C_function
+    m2, col, co, ranges, pl = _binned(P, W, H, 31 + E, device)
+    g = torch.Generator().manual_seed(9)
+    ex = torch.randn(P, E, generator=g).to(device) if E else None
+    acc_max = torch.zeros(P, dtype=torch.int32, device=device)
+    acc_w, acc_n = torch.zeros(P, device=device), torch.zeros(P, dtype=torch.int32, device=device)
+    print(f"[gs3d rasterize] P={P} {W}x{H} E={E} R={pl.numel()}", flush=True)
+    oc, oo, oe, nc = get_C_function('gaussian_rasterize_forward')(W, H, m2, co, col, ex, pl, ranges, acc_max, acc_w,
+                                                                  acc_n)
+    torch.cuda.synchronize()
+    n = lambda t: None if t is None else npy(t)
+    r_max, r_w, r_n = np.zeros(P, np.int32), np.zeros(P, np.float32), np.zeros(P, np.int32)
+    r_oc, r_oo, r_oe, r_nc = O.gs3d_render_forward(W, H, n(m2), n(co), n(col), n(ex), n(pl), n(ranges), r_max, r_w, r_n)
+    assert abs_err(n(oc), r_oc) < 1e-4 and abs_err(n(oo), r_oo) < 1e-4
+    if E:
+        assert abs_err(n(oe), r_oe) < 1e-4 * max(1.0, float(np.abs(r_oe).max()))
+    flips = int((n(nc) != r_nc).sum())
+    assert flips <= max(2, int(1e-4 * W * H)), flips  # pairs within rounding of the 1/255 or 1e-4 thresholds
+    assert abs(float(acc_w.sum()) - float(r_w.sum())) < 1e-3 * max(1.0, float(r_w.sum()))
+    assert abs(int(acc_n.sum()) - int(r_n.sum())) <= 4 and abs(int(acc_max.sum()) - int(r_max.sum())) <= 2
+    # the plain variant (no accumulators) gives the same image
+    oc2, oo2, _, nc2 = get_C_function('gaussian_rasterize_forward')(W, H, m2, co, col, ex, pl, ranges)
+    assert torch.equal(oc, oc2) and torch.equal(oo, oo2) and torch.equal(nc, nc2)
+
+    gi, go = torch.randn(3, H, W, generator=g).to(device), torch.randn(H, W, generator=g).to(device)
+    ge = torch.randn(E, H, W, generator=g).to(device) if E else None
+    g_col, g_ex, g_m2, g_co = get_C_function('gaussian_rasterize_backward')(m2, co, col, ex, oo, gi, go, ge, ranges,
+                                                                            pl, nc)
+    torch.cuda.synchronize()
+    # the oracle backward from the GPU's own forward state, so threshold flips of the forward do not enter
+    r_col, r_ex, r_m2, r_co = O.gs3d_render_backward(W, H, n(m2), n(co), n(col), n(ex), n(oo), n(nc), n(gi), n(ge),
+                                                     n(go), n(pl), n(ranges))
+    assert rel_err(n(g_col), r_col) < 1e-3 and rel_err(n(g_m2), r_m2) < 1e-3 and rel_err(n(g_co), r_co) < 1e-3
+    if E:
+        assert rel_err(n(g_ex), r_ex) < 1e-3
+    else:
+        assert g_ex is None
+
+
+def test_gs3d_render_autograd_and_empty(device):
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd.renderer import gaussian_render as GR
+    P, W, H = 3000, 112, 80
+    scene, scales, cam, tan_fov = _scene(P, W, H, 41, device)
+    d = lambda t: t.to(device).contiguous()
+    params = [d(t).requires_grad_(True) for t in (scene.means3D, scales, scene.rotations, scene.opacities, scene.shs)]
+    feat = d(torch.randn(P, 2, generator=torch.Generator().manual_seed(2))).requires_grad_(True)
+    focals = torch.tensor([float(cam.Tv2s[0, 0]), float(cam.Tv2s[1, 1])], device=device)
+    out = GR.render(d(cam.Tw2v), d(cam.Tv2c), (W, H), params[0], params[3], scales=params[1], rotations=params[2],
+                    campos=d(cam.campos), focals=focals, sh_features=params[4], sh_degree=3, feat=feat)
+    assert set(out) >= {'images', 'opacity', 'viewspace_points', 'visibility_filter', 'radii', 'buffer', 'feat'}
+    g = torch.Generator().manual_seed(3)
+    gi, go, gf = (torch.randn(*out[k].shape, generator=g).to(device) for k in ('images', 'opacity', 'feat'))
+    ((out['images'] * gi).sum() + (out['opacity'] * go).sum() + (out['feat'] * gf).sum()).backward()
+    torch.cuda.synchronize()
+    # the same chain on the oracle
+    n = lambda t: npy(t.detach())
+    m2, dep, col, rad, tt, c3, co = O.gs3d_preprocess_forward(W, H, 3, False, n(params[0]), n(params[1]), n(params[2]),
+                                                              n(params[3]), n(params[4]), None, npy(cam.Tw2v),
+                                                              npy(cam.Tv2c), npy(cam.campos), tan_fov)
+    ranges, pl = O.prepare(W, H, m2, dep, rad, tt)
+    oc, oo, oe, nc = O.gs3d_render_forward(W, H, m2, co, col, n(feat), pl, ranges)
+    assert abs_err(n(out['images']), oc) < 1e-4 and abs_err(n(out['feat']), oe) < 1e-4 * max(1, np.abs(oe).max())
+    assert np.array_equal(n(out['radii']), rad)
+    g_col, g_ex, g_m2, g_co = O.gs3d_render_backward(W, H, m2, co, col, n(feat), oo, nc, npy(gi), npy(gf), npy(go), pl,
+                                                     ranges)
+    r3, rs, rq, rop, rsh, _, _, rm2 = O.gs3d_preprocess_backward(W, H, 3, False, n(params[0]), n(params[1]),
+                                                                 n(params[2]), n(params[4]), None, npy(cam.Tw2v),
+                                                                 npy(cam.Tv2c), npy(cam.campos), tan_fov, rad, col, c3,
+                                                                 g_m2, g_col, g_co)
+    for name, p_, r in zip(('means3D', 'scales', 'rotations', 'opacities', 'shs'), params, (r3, rs, rq, rop, rsh)):
+        assert rel_err(n(p_.grad), r) < 1e-3, (name, rel_err(n(p_.grad), r))
+    assert rel_err(n(feat.grad), g_ex) < 1e-3
+    assert rel_err(n(out['viewspace_points'].grad), rm2) < 1e-3  # what densification reads
+    # empty scene
+    z = lambda *s: torch.zeros(s, device=device)
+    out = GR.render(d(cam.Tw2v), d(cam.Tv2c), (W, H), z(0, 3), z(0, 1), scales=z(0, 3), rotations=z(0, 4),
+                    campos=d(cam.campos), focals=focals, sh_features=z(0, 16, 3), sh_degree=3)
+    assert out['images'].shape == (3, H, W) and not out['images'].any() and not out['opacity'].any()

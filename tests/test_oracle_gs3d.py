@@ -1,0 +1,198 @@
+"""Pins the oracle's 3D-Gaussian (EWA) path (oracle/gs3d.cpp) without the reference: textbook forms in numpy for the
+covariances, the conic, the projection and the compositing, and central finite differences in fp64 for both backward
+passes. CPU only."""
+import numpy as np
+import pytest
+import torch
+from scipy.spatial.transform import Rotation
+
+import oracle as O
+from fast_sp_gs_amd import scenes
+
+
+def _scene(P=400, size=96, seed=0):
+    scene, cam = scenes.config0(P=P, size=size, seed=seed)
+    n = lambda t: np.ascontiguousarray(t.double().numpy())
+    g = np.random.default_rng(seed + 1)
+    s = dict(means3D=n(scene.means3D), rotations=n(scene.rotations), opacities=n(scene.opacities), shs=n(scene.shs),
+             scales=np.ascontiguousarray(np.concatenate([n(scene.scales) * 3, n(scene.scales[:, :1]) * g.uniform(0.5, 4, (P, 1))], 1)),
+             Tw2v=n(cam.Tw2v), Tv2c=n(cam.Tv2c), campos=n(cam.campos))
+    s['rotations'] = np.ascontiguousarray(s['rotations'] / np.linalg.norm(s['rotations'], axis=1, keepdims=True))
+    tan_fov = (cam.W / 2 / float(cam.Tv2s[0, 0]), cam.H / 2 / float(cam.Tv2s[1, 1]))
+    return s, cam, tan_fov
+
+
+def _forward(s, cam, tan_fov, **over):
+    a = {**s, **over}
+    return O.gs3d_preprocess_forward(cam.W, cam.H, 3, False, a['means3D'], a['scales'], a['rotations'], a['opacities'],
+                                     a['shs'], None, a['Tw2v'], a['Tv2c'], a['campos'], tan_fov)
+
+
+def test_preprocess_forward_textbook_forms():
+    s, cam, tan_fov = _scene()
+    W, H = cam.W, cam.H
+    m2, dep, col, rad, tt, c3, co = _forward(s, cam, tan_fov)
+    vis = rad > 0
+    assert vis.sum() > 300
+    fx, fy = 0.5 * W / tan_fov[0], 0.5 * H / tan_fov[1]
+    for i in np.flatnonzero(vis)[:60]:
+        R = Rotation.from_quat(s['rotations'][i]).as_matrix()  # the scene's quaternions are unit (x, y, z, w)
+        S = np.diag(s['scales'][i] ** 2)
+        Sigma = R @ S @ R.T
+        assert np.allclose([Sigma[0, 0], Sigma[0, 1], Sigma[0, 2], Sigma[1, 1], Sigma[1, 2], Sigma[2, 2]], c3[i], rtol=1e-10, atol=1e-16)
+        t = s['Tw2v'][:3, :3] @ s['means3D'][i] + s['Tw2v'][:3, 3]
+        assert t[2] > 0.2 and abs(t[0]) < 1.3 * tan_fov[0] * t[2]  # inside the clamp, so J is the plain Jacobian
+        J = np.array([[fx / t[2], 0, -fx * t[0] / t[2] ** 2], [0, fy / t[2], -fy * t[1] / t[2] ** 2]])
+        Wm = s['Tw2v'][:3, :3]
+        cov = J @ Wm @ Sigma @ Wm.T @ J.T + 0.3 * np.eye(2)
+        conic = np.linalg.inv(cov)
+        assert np.allclose([conic[0, 0], conic[0, 1], conic[1, 1]], co[i, :3], rtol=1e-9)
+        assert co[i, 3] == s['opacities'][i, 0] and dep[i] == pytest.approx(t[2], rel=1e-12)
+        clip = s['Tv2c'] @ np.append(t, 1.0)
+        ndc = clip[:2] / clip[3]
+        assert np.allclose(m2[i], [(ndc[0] + 1) * 0.5 * W - 0.5, (ndc[1] + 1) * 0.5 * H - 0.5], atol=1e-5)
+        lam = np.linalg.eigvalsh(cov).max()
+        assert rad[i] in (int(np.ceil(3 * np.sqrt(lam))), int(np.ceil(3 * np.sqrt(lam))) + 1)  # the 0.1 floor under the root
+        x0, x1 = np.clip([int((m2[i, 0] - rad[i]) / 16), int((m2[i, 0] + rad[i] + 15) / 16)], 0, (W + 15) // 16)
+        y0, y1 = np.clip([int((m2[i, 1] - rad[i]) / 16), int((m2[i, 1] + rad[i] + 15) / 16)], 0, (H + 15) // 16)
+        assert tt[i] == (x1 - x0) * (y1 - y0)
+    # rejected rows stay zero; a culling mask rejects
+    behind = dict(means3D=s['means3D'] + np.array([0, 0, 50.0]))
+    out = _forward(s, cam, tan_fov, **behind)
+    assert not out[3].any() and not out[0].any() and not out[6].any()
+    cull = np.zeros(len(rad), bool)
+    cull[::2] = True
+    out = O.gs3d_preprocess_forward(W, H, 3, False, s['means3D'], s['scales'], s['rotations'], s['opacities'], s['shs'],
+                                    None, s['Tw2v'], s['Tv2c'], s['campos'], tan_fov, culling=cull)
+    assert not out[3][::2].any() and np.array_equal(out[3][1::2], rad[1::2])
+
+
+def _composite_numpy(W, H, m2, co, col, ex, pl, ranges):
+    img, opa = np.zeros((3, H, W)), np.zeros((H, W))
+    ext = np.zeros((ex.shape[1], H, W))
+    gx = (W + 15) // 16
+    for py in range(H):
+        for px in range(W):
+            r0, r1 = ranges[(py // 16) * gx + px // 16]
+            ids = pl[r0:r1]
+            d = m2[ids] - np.array([px, py], float)
+            power = -0.5 * (co[ids, 0] * d[:, 0] ** 2 + co[ids, 2] * d[:, 1] ** 2) - co[ids, 1] * d[:, 0] * d[:, 1]
+            alpha = np.minimum(0.99, co[ids, 3] * np.exp(power))
+            alpha[(power > 0) | (alpha < 1 / 255)] = 0
+            T = 1.0
+            for k in range(len(ids)):
+                if alpha[k] == 0:
+                    continue
+                if T * (1 - alpha[k]) < 1e-4:
+                    break
+                img[:, py, px] += col[ids[k]] * alpha[k] * T
+                ext[:, py, px] += ex[ids[k]] * alpha[k] * T
+                T *= 1 - alpha[k]
+            opa[py, px] = 1 - T
+    return img, opa, ext
+
+
+def test_render_forward_closed_form_and_compositor():
+    # one Gaussian: image = alpha * colour with alpha = min(0.99, o * exp(-0.5 d^T Q d))
+    W = H = 32
+    m2 = np.array([[13.3, 17.8]])
+    co = np.array([[0.08, 0.02, 0.05, 0.8]])
+    col, ex = np.array([[0.2, 0.5, 0.9]]), np.array([[2.0, -1.0]])
+    ranges = np.zeros((4, 2), np.int64)
+    ranges[:, 1] = 1  # every tile lists the Gaussian
+    pl = np.zeros(1, np.int32)
+    oc, oo, oe, nc = O.gs3d_render_forward(W, H, m2, co, col, ex, pl, ranges)
+    yy, xx = np.mgrid[0:H, 0:W].astype(float)
+    dx, dy = m2[0, 0] - xx, m2[0, 1] - yy
+    alpha = np.minimum(0.99, 0.8 * np.exp(-0.5 * (0.08 * dx * dx + 0.05 * dy * dy) - 0.02 * dx * dy))
+    alpha[alpha < 1 / 255] = 0
+    assert np.abs(oo - alpha).max() < 1e-14 and np.abs(oc - alpha[None] * col[0][:, None, None]).max() < 1e-14
+    assert np.abs(oe - alpha[None] * ex[0][:, None, None]).max() < 1e-14
+    assert np.array_equal(nc, (alpha > 0).astype(np.int32))
+    # a scene: independent per-pixel numpy compositor
+    s, cam, tan_fov = _scene(P=600, size=64, seed=3)
+    m2, dep, col, rad, tt, c3, co = _forward(s, cam, tan_fov)
+    ex = np.random.default_rng(1).normal(size=(len(rad), 2))
+    ranges, pl = O.prepare(cam.W, cam.H, m2.astype(np.float32), dep.astype(np.float32), rad, tt)
+    acc_w, acc_n, acc_max = np.zeros(len(rad)), np.zeros(len(rad), np.int32), np.zeros(len(rad), np.int32)
+    oc, oo, oe, nc = O.gs3d_render_forward(cam.W, cam.H, m2, co, col, ex, pl, ranges, acc_max, acc_w, acc_n)
+    img, opa, ext = _composite_numpy(cam.W, cam.H, m2, co, col, ex, pl, ranges)
+    assert np.abs(oc - img).max() < 1e-12 and np.abs(oo - opa).max() < 1e-12 and np.abs(oe - ext).max() < 1e-12
+    assert oo.max() > 0.5 and abs(acc_w.sum() - oo.sum()) < 1e-9  # blend weights sum to the opacity image
+    assert acc_max.sum() == int((oo > 0).sum()) and acc_n.sum() >= acc_max.sum()
+
+
+def test_render_backward_finite_differences():
+    s, cam, tan_fov = _scene(P=150, size=48, seed=5)
+    W, H = cam.W, cam.H
+    m2, dep, col, rad, tt, c3, co = _forward(s, cam, tan_fov)
+    P = len(rad)
+    rng = np.random.default_rng(2)
+    ex = rng.normal(size=(P, 3))
+    ranges, pl = O.prepare(W, H, m2.astype(np.float32), dep.astype(np.float32), rad, tt)
+    gi, go, ge = rng.normal(size=(3, H, W)), rng.normal(size=(H, W)), rng.normal(size=(3, H, W))
+
+    def loss(m2_, co_, col_, ex_):
+        oc, oo, oe, _ = O.gs3d_render_forward(W, H, m2_, co_, col_, ex_, pl, ranges)
+        return (oc * gi).sum() + (oo * go).sum() + (oe * ge).sum()
+
+    oc, oo, oe, nc = O.gs3d_render_forward(W, H, m2, co, col, ex, pl, ranges)
+    g_col, g_ex, g_m2, g_co = O.gs3d_render_backward(W, H, m2, co, col, ex, oo, nc, gi, ge, go, pl, ranges)
+    vis = np.flatnonzero(rad > 0)
+    h = 1e-6
+    checked = 0
+    for i in vis[rng.permutation(len(vis))[:25]]:
+        for name, arr, grad, cols in (("means2D", m2, g_m2, 2), ("conic_opacity", co, g_co, 4), ("colors", col, g_col, 3),
+                                      ("extras", ex, g_ex, 3)):
+            for c in range(cols):
+                a, b = arr.copy(), arr.copy()
+                a[i, c] += h
+                b[i, c] -= h
+                args = {"means2D": (m2, co, col, ex), }
+                if name == "means2D":
+                    fd = (loss(a, co, col, ex) - loss(b, co, col, ex)) / (2 * h)
+                elif name == "conic_opacity":
+                    fd = (loss(m2, a, col, ex) - loss(m2, b, col, ex)) / (2 * h)
+                elif name == "colors":
+                    fd = (loss(m2, co, a, ex) - loss(m2, co, b, ex)) / (2 * h)
+                else:
+                    fd = (loss(m2, co, col, a) - loss(m2, co, col, b)) / (2 * h)
+                scale = max(abs(fd), np.abs(grad).max() * 1e-3, 1e-6)
+                # thresholds (alpha = 1/255, T = 1e-4, the 0.99 clamp) make the image piecewise smooth: a step that
+                # crosses one shows up as a large mismatch; those are rare and skipped by the count below
+                if abs(fd - grad[i, c]) <= 2e-4 * scale:
+                    checked += 1
+    assert checked >= 0.97 * 25 * 12
+
+
+def test_preprocess_backward_finite_differences():
+    s, cam, tan_fov = _scene(P=60, size=64, seed=7)
+    W, H = cam.W, cam.H
+    m2, dep, col, rad, tt, c3, co = _forward(s, cam, tan_fov)
+    P = len(rad)
+    rng = np.random.default_rng(4)
+    g_m2, g_col, g_co = rng.normal(size=(P, 2)), rng.normal(size=(P, 3)), rng.normal(size=(P, 4))
+
+    def loss(**over):
+        o = _forward(s, cam, tan_fov, **over)
+        return (o[0] * g_m2).sum() + (o[2] * g_col).sum() + (o[6] * g_co).sum()
+
+    g3, gs, gq, gop, gsh, _, gcov, gm2_out = O.gs3d_preprocess_backward(
+        W, H, 3, False, s['means3D'], s['scales'], s['rotations'], s['shs'], None, s['Tw2v'], s['Tv2c'], s['campos'],
+        tan_fov, rad, col, c3, g_m2, g_col, g_co)
+    assert np.allclose(gm2_out[rad > 0], g_m2[rad > 0] * np.array([0.5 * W, 0.5 * H]))
+    assert np.array_equal(gop[rad > 0, 0], g_co[rad > 0, 3])
+    h = 1e-6
+    vis = np.flatnonzero(rad > 0)
+    for name, grad in (("means3D", g3), ("scales", gs), ("rotations", gq), ("shs", gsh)):
+        base = s[name]
+        worst = 0.0
+        for i in vis[:12]:
+            idxs = [(c,) for c in range(base.shape[1])] if base.ndim == 2 else [(k, c) for k in (0, 3, 9, 15) for c in range(3)]
+            for ix in idxs:
+                a, b = base.copy(), base.copy()
+                a[(i,) + ix] += h
+                b[(i,) + ix] -= h
+                fd = (loss(**{name: a}) - loss(**{name: b})) / (2 * h)
+                worst = max(worst, abs(fd - grad[(i,) + ix]) / max(np.abs(grad[vis[:12]]).max(), 1e-9))
+        assert worst < 2e-5, (name, worst)
