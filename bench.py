@@ -291,6 +291,110 @@ def gs3d_path_rate(dev, scene, cam, gi, steps: int = 30, warmup: int = 5):
                                   f"R = {R[0]}: gs_preprocess fwd/bwd + GS_prepare + gaussian_rasterize fwd/bwd"}
 
 
+def density_control_ms(dev, scene, reps: int = 5):
+    """Densify (clone + split) and prune of the 300k-point set with populated Adam moments: the table-driven kernels
+    against the same operations done the reference's way (boolean indexing / cat / repeat per tensor and per moment,
+    gaussian_splatting.py:497-636) with torch on the same GPU."""
+    from fast_sp_gs_amd.adaptive_control import GaussianPoints
+    from fast_sp_gs_amd._C import get_C_function as f
+    P = scene.P
+    g = torch.Generator().manual_seed(5)
+    acc = (torch.rand(P, 1, generator=g) * 4e-4).to(dev)
+    den = torch.randint(1, 3, (P, 1), generator=g).float().to(dev)
+    radii = (torch.rand(P, generator=g) * 30).to(dev)
+
+    def fresh():
+        m = GaussianPoints(scene.means3D, scene.shs[:, :1].contiguous(), scene.shs[:, 1:].contiguous(),
+                           torch.log(scene.scales), scene.rotations, torch.logit(scene.opacities.clamp(1e-4, 1 - 1e-4)))
+        opt = torch.optim.Adam(m.param_groups(1e-3), eps=1e-15)
+        for grp in opt.param_groups:
+            grp['params'][0].grad = torch.zeros_like(grp['params'][0])
+        opt.step()
+        m.xyz_gradient_accum, m.denom, m.max_radii2D = acc.clone(), den.clone(), radii.clone()
+        return m, opt
+
+    def ours(m, opt):
+        m.densify(opt, 2e-4, 4.0, 0.01)
+        m.max_radii2D = radii[:1].expand(m._xyz.shape[0]).contiguous()
+        m.prune(opt, 0.05, 4.0, 20.0, 0.1)
+
+    def reference_way(m, opt):  # the reference's sequence with torch indexing, one tensor and one moment at a time
+        names = m.param_names_map
+
+        def change(tensors, op):
+            for grp in opt.param_groups:
+                old = grp['params'][0]
+                t = tensors[grp['name']] if isinstance(tensors, dict) else tensors
+                new = torch.nn.Parameter(torch.cat([old, t]) if op == 'concat' else old[t])
+                st = opt.state.pop(old)
+                for k in ('exp_avg', 'exp_avg_sq'):
+                    st[k] = torch.cat([st[k], torch.zeros_like(t)]) if op == 'concat' else st[k][t]
+                grp['params'][0] = new
+                opt.state[new] = st
+                setattr(m, [a for a, n in names.items() if n == grp['name']][0], new)
+            m.training_setup() if op == 'concat' else None
+
+        grads = m.xyz_gradient_accum / m.denom
+        grads[grads.isnan()] = 0.0
+        sel = (torch.norm(grads, dim=-1) >= 2e-4) & (torch.amax(m.get_scaling, dim=1) <= 0.04)
+        change({n: getattr(m, a)[sel] for a, n in names.items()}, 'concat')
+        Pn = m._xyz.shape[0]
+        padded = torch.zeros(Pn, device=dev)
+        padded[:grads.shape[0]] = grads.squeeze()
+        sel = (padded >= 2e-4) & (torch.amax(m.get_scaling, dim=1) > 0.04)
+        stds = m.get_scaling[sel].repeat(2, 1)
+        stds = torch.cat([stds, 0 * torch.ones_like(stds[:, :1])], dim=-1)
+        samples = torch.normal(mean=torch.zeros_like(stds), std=stds)
+        q = torch.nn.functional.normalize(m._rotation[sel], dim=-1)
+        x, y, z, w = q.unbind(-1)
+        R = torch.stack([1 - 2 * y * y - 2 * z * z, 2 * x * y - 2 * w * z, 2 * w * y + 2 * x * z,
+                         2 * x * y + 2 * w * z, 1 - 2 * x * x - 2 * z * z, 2 * y * z - 2 * w * x,
+                         2 * x * z - 2 * w * y, 2 * w * x + 2 * y * z, 1 - 2 * x * x - 2 * y * y], -1).reshape(-1, 3, 3)
+        new = {n: getattr(m, a)[sel].repeat(2, *[1] * (getattr(m, a).ndim - 1)) for a, n in names.items()}
+        new['xyz'] = torch.bmm(R.repeat(2, 1, 1), samples[..., None]).squeeze(-1) + m._xyz[sel].repeat(2, 1)
+        new['scaling'] = torch.log(m.get_scaling[sel].repeat(2, 1) / 1.6)
+        change(new, 'concat')
+        change(~torch.cat((sel, sel.new_zeros(2 * sel.sum()))), 'prune')
+        m.max_radii2D = radii[:1].expand(m._xyz.shape[0]).contiguous()
+        mask = (m.get_opacity < 0.05).squeeze() | (m.max_radii2D > 20.0) | (m.get_scaling.amax(dim=1) > 0.4)
+        change(~mask, 'prune')
+
+    out = {}
+    with torch.no_grad():
+        for name, fn in (("density_control_ms", ours), ("density_control_torch_indexing_ms", reference_way)):
+            times = []
+            for _ in range(reps + 1):
+                m, opt = fresh()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                fn(m, opt)
+                torch.cuda.synchronize()
+                times.append((time.perf_counter() - t0) * 1e3)
+            out[name] = min(times[1:])
+            out[name.replace("_ms", "_points_after")] = int(m._xyz.shape[0])
+        # the gather alone: all 6 parameters + 12 moments of a prune that keeps 90 %
+        m, opt = fresh()
+        tensors = [grp['params'][0] for grp in opt.param_groups]
+        tensors += [opt.state[t][k] for t in tensors for k in ('exp_avg', 'exp_avg_sq')]
+        rows = f('select_indices')(torch.rand(P, device=dev) < 0.9)
+        for _ in range(3):
+            f('gather_rows')(tensors, rows)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            f('gather_rows')(tensors, rows)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / 10
+        nbytes = 2 * rows.numel() * sum(t[0].numel() * 4 for t in tensors) + 4 * rows.numel()
+    out["gather_rows_ms"] = ms
+    out["gather_rows_GBps"] = nbytes / (ms * 1e-3) / 1e9
+    out["density_control_workload"] = (f"{P} surfels with Adam moments (177 floats per point): densify (clone + split, "
+                                       "N = 2) then prune; gather_rows = 18 tensors, 90 % of the rows kept, allocation "
+                                       "of the outputs included")
+    return out
+
+
 def ssim_rate(dev, reps: int = 20):
     """Fused SSIM forward (with the partial-derivative maps) + backward on one 3 x 800 x 800 image pair."""
     from fast_sp_gs_amd._C import get_C_function
@@ -432,6 +536,7 @@ def main():
         extra.update(simple_knn_ms(dev, scene))
         extra.update(reference_note_blend_ms(dev))
         extra.update(gs3d_path_rate(dev, scene, cam, gi))
+        extra.update(density_control_ms(dev, scene))
         extra["fast_path_frames_per_s"] = fast_path_rate(dev, scene, cam, gi)
         extra["fast_path_workload"] = "same scene through GS_2D_fast_* (corner-test binning keeps fewer instances)"
         extra["dynamic_step_frames_per_s"] = dynamic_step_rate(dev)

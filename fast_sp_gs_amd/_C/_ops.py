@@ -7,7 +7,7 @@ CHECK_INPUT / CHECK_SHAPE macros and raise RuntimeError like TORCH_CHECK does.
 from __future__ import annotations
 
 import ctypes
-from typing import List, Optional, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 from torch import Tensor
@@ -24,7 +24,8 @@ __all__ = [
     'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward', 'gs_2d_fast_compute_trans_mat_backward',
     'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward', 'fusedssim', 'fusedssim_backward',
     'gs_2d_epilogue_forward', 'gs_2d_epilogue_backward', 'simple_knn', 'gs_preprocess_forward',
-    'gs_preprocess_backward', 'gaussian_rasterize_forward', 'gaussian_rasterize_backward',
+    'gs_preprocess_backward', 'gaussian_rasterize_forward', 'gaussian_rasterize_backward', 'select_indices',
+    'gather_rows', 'densify_masks', 'prune_mask', 'split_children', 'densification_stats',
 ]
 
 _TILE = 16
@@ -1133,6 +1134,184 @@ def simple_knn(points: Tensor) -> Tensor:
         rc = lib.fsgs_simple_knn(P, L.ptr(points), L.ptr(means), L.ptr(ws), ws.numel(), L.current_stream())
     L.check(rc, what)
     return means
+
+
+# ---- adaptive density control as stream compaction ---------------------------------------------------------------------
+def _as_bytes(what: str, name: str, mask: Tensor) -> Tensor:
+    if not isinstance(mask, Tensor) or not mask.is_cuda:
+        raise RuntimeError(f'{what}: {name} must be a CUDA tensor')
+    if mask.dtype not in (torch.bool, torch.uint8):
+        raise RuntimeError(f'{what}: {name} must be a bool or uint8 tensor')
+    mask = mask.contiguous()
+    return mask.view(torch.uint8) if mask.dtype == torch.bool else mask
+
+
+def select_indices(mask: Tensor, invert: bool = False) -> Tensor:
+    """Ascending positions of the set (or, with invert, the clear) entries of a 1-D mask, int32 -- the index form of the
+    reference's `tensor[mask]` / `tensor[~mask]` (gaussian_splatting.py:526-527, :558)."""
+    what = 'select_indices'
+    m = _as_bytes(what, 'mask', mask)
+    if m.ndim != 1:
+        raise RuntimeError(f'{what}: mask must be one-dimensional')
+    P, dev = m.shape[0], m.device
+    indices = torch.empty((max(P, 1),), dtype=torch.int32, device=dev)
+    lib = _lib()
+    ws = _workspace(lib.fsgs_select_indices_workspace_bytes(P), dev)
+    count = _pinned_count()
+    with _timed('select_indices'):
+        rc = lib.fsgs_select_indices(P, L.ptr(m), int(bool(invert)), L.ptr(indices), L.ptr(ws), ws.numel(),
+                                     count.data_ptr(), L.current_stream())
+    L.check(rc, what)
+    return indices[:ctypes.c_int64.from_address(count.data_ptr()).value]
+
+
+def gather_rows(tensors: Sequence[Tensor], source_row: Tensor) -> List[Tensor]:
+    """For every tensor t: out[r] = t[source_row[r]], or a row of zeros where source_row[r] < 0 -- `old[mask]`, `torch.cat`
+    with copies of selected rows and the zero Adam moments of new points (gaussian_splatting.py:524-551) for all per-point
+    tensors in one launch per 24 tensors."""
+    what = 'gather_rows'
+    if not isinstance(source_row, Tensor) or not source_row.is_cuda or source_row.dtype != torch.int32 or \
+            source_row.ndim != 1:
+        raise RuntimeError(f'{what}: source_row must be a one-dimensional int32 CUDA tensor')
+    source_row = source_row.contiguous()
+    n_rows, dev = source_row.shape[0], source_row.device
+    srcs, outs = [], []
+    for i, t in enumerate(tensors):
+        if not isinstance(t, Tensor) or not t.is_cuda or t.ndim < 1:
+            raise RuntimeError(f'{what}: tensor {i} must be a CUDA tensor with a leading point dimension')
+        t = t.detach().contiguous()
+        srcs.append(t)
+        outs.append(torch.empty((n_rows,) + tuple(t.shape[1:]), dtype=t.dtype, device=dev))
+    lib = _lib()
+    step = lib.fsgs_gather_rows_max_tensors()
+    stream = L.current_stream()
+    for lo in range(0, len(srcs), step):
+        # tensors without bytes (no rows in, none out, or an empty trailing shape) have nothing to move
+        part = [(a, b) for a, b in zip(srcs[lo:lo + step], outs[lo:lo + step]) if b.numel() > 0]
+        if not part:
+            continue
+        for a, _ in part:
+            if a.shape[0] == 0:
+                raise RuntimeError(f'{what}: cannot gather rows from an empty tensor')
+        n = len(part)
+        src_arr = (ctypes.c_void_p * n)(*[a.data_ptr() for a, _ in part])
+        dst_arr = (ctypes.c_void_p * n)(*[b.data_ptr() for _, b in part])
+        row_arr = (ctypes.c_int64 * n)(*[b[0].numel() * b.element_size() for _, b in part])
+        with _timed('gather_rows'):
+            rc = lib.fsgs_gather_rows(n, ctypes.addressof(src_arr), ctypes.addressof(dst_arr),
+                                      ctypes.addressof(row_arr), n_rows, L.ptr(source_row), stream)
+        L.check(rc, what)
+    return outs
+
+
+def _point_scalars(what: str, name: str, t: Tensor, P: int) -> Tensor:
+    L.require_cuda(what, **{name: t})
+    L.require_dtype(what, name, t, torch.float32)
+    if t.numel() != P:
+        raise RuntimeError(f'{what}: {name} must have {P} elements')
+    return t
+
+
+def densify_masks(grad_accum: Tensor, denom: Tensor, scaling: Tensor, grad_threshold: float,
+                  scale_threshold: float) -> Tuple[Tensor, Tensor]:
+    """Clone and split selections of gaussian_splatting.py:623-626, :612-615, :585-589 from the accumulated screen-space
+    gradient statistics and the ACTIVATED scales [P,S] -> two bool masks [P]."""
+    what = 'densify_masks'
+    L.require_cuda(what, scaling=scaling)
+    L.require_dtype(what, 'scaling', scaling, torch.float32)
+    if scaling.ndim != 2 or not 1 <= scaling.shape[1] <= 3:
+        raise RuntimeError(f'{what}: Error shape for scaling')
+    P, S = scaling.shape
+    _point_scalars(what, 'grad_accum', grad_accum, P)
+    _point_scalars(what, 'denom', denom, P)
+    clone = torch.empty((P,), dtype=torch.bool, device=scaling.device)
+    split = torch.empty((P,), dtype=torch.bool, device=scaling.device)
+    with _timed('densify_masks'):
+        rc = _lib().fsgs_densify_masks(P, S, L.ptr(grad_accum), L.ptr(denom), L.ptr(scaling), float(grad_threshold),
+                                       float(scale_threshold), L.ptr(clone), L.ptr(split), L.current_stream())
+    L.check(rc, what)
+    return clone, split
+
+
+def prune_mask(opacity: Tensor, max_radii2D: Optional[Tensor], scaling: Optional[Tensor], min_opacity: float,
+               max_screen_size: Optional[float], world_threshold: float = 0.0) -> Tensor:
+    """Prune selection of gaussian_splatting.py:630-635 from ACTIVATED opacities [P,1] and scales [P,S] -> bool [P]. A
+    false `max_screen_size` (None or 0) keeps only the opacity test, as the reference's `if max_screen_size:` does."""
+    what = 'prune_mask'
+    L.require_cuda(what, opacity=opacity, max_radii2D=max_radii2D, scaling=scaling)
+    L.require_dtype(what, 'opacity', opacity, torch.float32)
+    P = opacity.numel()
+    use_size = bool(max_screen_size)
+    S = 1
+    if use_size:
+        if max_radii2D is None or scaling is None:
+            raise RuntimeError(f'{what}: max_radii2D and scaling are needed with max_screen_size')
+        _point_scalars(what, 'max_radii2D', max_radii2D, P)
+        L.require_dtype(what, 'scaling', scaling, torch.float32)
+        if scaling.ndim != 2 or scaling.shape[0] != P or not 1 <= scaling.shape[1] <= 3:
+            raise RuntimeError(f'{what}: Error shape for scaling')
+        S = scaling.shape[1]
+    mask = torch.empty((P,), dtype=torch.bool, device=opacity.device)
+    with _timed('prune_mask'):
+        rc = _lib().fsgs_prune_mask(P, S, L.ptr(opacity), L.ptr(max_radii2D) if use_size else None,
+                                    L.ptr(scaling) if use_size else None, float(min_opacity), int(use_size),
+                                    float(max_screen_size or 0.0), float(world_threshold), L.ptr(mask),
+                                    L.current_stream())
+    L.check(rc, what)
+    return mask
+
+
+def split_children(selected: Tensor, N: int, xyz: Tensor, scaling: Tensor, rotations: Tensor,
+                   noise: Tensor) -> Tuple[Tensor, Tensor]:
+    """Positions and raw (log) scales of the N children of every selected point (gaussian_splatting.py:591-597,
+    network.py:1170-1183): `R(q) (noise * scale) + xyz` and `log(scale / (0.8 N))`, children ordered as
+    `x[selected].repeat(N, 1)`. scaling [P,S] is ACTIVATED, noise [N * len(selected), 3] standard normal."""
+    what = 'split_children'
+    L.require_cuda(what, selected=selected, xyz=xyz, scaling=scaling, rotations=rotations, noise=noise)
+    L.require_dtype(what, 'selected', selected, torch.int32)
+    for name, t in (('xyz', xyz), ('scaling', scaling), ('rotations', rotations), ('noise', noise)):
+        L.require_dtype(what, name, t, torch.float32)
+    P = xyz.shape[0]
+    if scaling.ndim != 2 or scaling.shape[0] != P or scaling.shape[1] not in (2, 3):
+        raise RuntimeError(f'{what}: Error shape for scaling')
+    S, n_sel = scaling.shape[1], selected.numel()
+    L.require_shape(what, 'xyz', xyz, P, 3)
+    L.require_shape(what, 'rotations', rotations, P, 4)
+    L.require_shape(what, 'noise', noise, n_sel * N, 3)
+    out_xyz = torch.empty((n_sel * N, 3), dtype=torch.float32, device=xyz.device)
+    out_scaling = torch.empty((n_sel * N, S), dtype=torch.float32, device=xyz.device)
+    with _timed('split_children'):
+        rc = _lib().fsgs_split_children(P, n_sel, int(N), S, L.ptr(selected), L.ptr(xyz), L.ptr(scaling),
+                                        L.ptr(rotations), L.ptr(noise), L.ptr(out_xyz), L.ptr(out_scaling),
+                                        L.current_stream())
+    L.check(rc, what)
+    return out_xyz, out_scaling
+
+
+def densification_stats(radii: Tensor, grad: Tensor, max_radii2D: Tensor, grad_accum: Tensor, denom: Tensor,
+                        factor: Optional[Tensor] = None) -> Tensor:
+    """Per-step statistics of network.py:1276-1282 (+ gaussian_splatting.py:486-495): for points with radii > 0 updates
+    max_radii2D, grad_accum (+= |grad[:, :2]|, times factor if given) and denom IN PLACE; returns `radii > 0` (bool)."""
+    what = 'densification_stats'
+    L.require_cuda(what, radii=radii, grad=grad, max_radii2D=max_radii2D, grad_accum=grad_accum, denom=denom,
+                   factor=factor)
+    L.require_dtype(what, 'radii', radii, torch.int32)
+    L.require_dtype(what, 'grad', grad, torch.float32)
+    P = radii.numel()
+    if grad.ndim != 2 or grad.shape[0] != P or grad.shape[1] < 2:
+        raise RuntimeError(f'{what}: Error shape for grad')
+    _point_scalars(what, 'max_radii2D', max_radii2D, P)
+    _point_scalars(what, 'grad_accum', grad_accum, P)
+    _point_scalars(what, 'denom', denom, P)
+    if factor is not None:
+        _point_scalars(what, 'factor', factor, P)
+    visible = torch.empty((P,), dtype=torch.bool, device=radii.device)
+    with _timed('densification_stats'):
+        rc = _lib().fsgs_densification_stats(P, grad.shape[1], L.ptr(radii), L.ptr(grad), L.ptr(factor),
+                                             L.ptr(max_radii2D), L.ptr(grad_accum), L.ptr(denom), L.ptr(visible),
+                                             L.current_stream())
+    L.check(rc, what)
+    return visible
 
 
 # ---- 3D-Gaussian (EWA) path ------------------------------------------------------------------------------------------

@@ -9,7 +9,7 @@ PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libfsgs_hip.so"
 SOURCES = ["api.hip", "preprocess.hip", "binning.hip", "blend_fwd.hip", "blend_bwd.hip", "blend_topk.hip", "fast_preprocess.hip",
-           "fast_blend.hip", "point_ops.hip", "lbs_bwd.hip", "ssim.hip", "epilogue.hip", "simple_knn.hip", "gs3d_preprocess.hip", "gs3d_blend.hip", "mlp.hip"]
+           "fast_blend.hip", "point_ops.hip", "lbs_bwd.hip", "ssim.hip", "epilogue.hip", "simple_knn.hip", "compaction.hip", "gs3d_preprocess.hip", "gs3d_blend.hip", "mlp.hip"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
     # packed-FP32 instructions are kept out of the generated code on purpose

@@ -362,6 +362,53 @@ int fsgs_mlp_backward(int B, int Din, int width, int n_layers, int skip, int n_o
     const uint16_t* packed_t, const float* heads_w, const uint16_t* saved, const float* g_out, float* g_w, float* g_b,
     void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- adaptive density control as stream compaction ------------------------------------------------------------- */
+/* The reference changes the point set with torch indexing on the host side, one tensor and one Adam moment at a time
+ * (fast_2d_gs/gaussian_splatting.py:497-637, fast_2d_gs/network.py:1156-1215, :1276-1282). Here a mask becomes an
+ * ascending index list and every structural change is one table source_row[new_row] applied to all tensors at once. */
+
+/* `mask[mask_or_keep]` -> indices: the ascending positions of the non-zero (invert = 0) or zero (invert = 1) bytes of
+ * mask[P], i.e. torch.nonzero(mask) / torch.nonzero(~mask) (gaussian_splatting.py:526-527, :558). indices needs room
+ * for P entries. Blocks until the count is on the host (torch's boolean indexing blocks in the same place). */
+size_t fsgs_select_indices_workspace_bytes(int P);
+int fsgs_select_indices(int P, const uint8_t* mask, int invert, int32_t* indices, void* workspace,
+                        size_t workspace_bytes, int64_t* count_host, void* stream);
+
+/* dst_t[r] = source_row[r] >= 0 ? src_t[source_row[r]] : zeros, for r < n_rows and every tensor t < n_tensors in one
+ * launch (gaussian_splatting.py:524-551: `old[mask]`, `torch.cat`, the zero moments of new points). The three *_host
+ * arrays are HOST arrays of n_tensors device pointers / row sizes in bytes; rows are contiguous. A tensor's source and
+ * destination must not overlap. At most fsgs_gather_rows_max_tensors() tensors per call. */
+int fsgs_gather_rows_max_tensors(void);
+int fsgs_gather_rows(int n_tensors, const void* const* src_host, void* const* dst_host, const int64_t* row_bytes_host,
+                     int64_t n_rows, const int32_t* source_row, void* stream);
+
+/* densify_and_clone / densify_and_split selection -- gaussian_splatting.py:623-626, :612-615, :585-589. g = grad_accum /
+ * denom with NaN -> 0; clone = |g| >= grad_threshold and max(scaling) <= scale_threshold; split = g >= grad_threshold
+ * and max(scaling) > scale_threshold. scaling[P,S] holds ACTIVATED scales. Masks are bytes (0 / 1). */
+int fsgs_densify_masks(int P, int S, const float* grad_accum, const float* denom, const float* scaling,
+                       float grad_threshold, float scale_threshold, uint8_t* clone_mask, uint8_t* split_mask,
+                       void* stream);
+
+/* prune selection -- gaussian_splatting.py:630-635: opacity < min_opacity, and with use_size also max_radii2D >
+ * max_screen_size or max(scaling) > world_threshold. opacity[P] and scaling[P,S] are ACTIVATED values. */
+int fsgs_prune_mask(int P, int S, const float* opacity, const float* max_radii2D, const float* scaling,
+                    float min_opacity, int use_size, float max_screen_size, float world_threshold, uint8_t* mask,
+                    void* stream);
+
+/* Children of a split -- gaussian_splatting.py:591-597, network.py:1170-1183. Child j < N * n_selected has parent
+ * p = selected[j % n_selected]: out_xyz[j] = R(normalize(rotations[p])) * (noise[j] * scaling[p]) + xyz[p] (a surfel,
+ * S = 2, has a zero third axis) and out_scaling[j] = log(scaling[p] / (0.8 N)). noise[N * n_selected, 3] are standard
+ * normal samples drawn by the caller; scaling holds ACTIVATED scales, out_scaling raw (log) ones. */
+int fsgs_split_children(int P, int n_selected, int N, int S, const int32_t* selected, const float* xyz,
+                        const float* scaling, const float* rotations, const float* noise, float* out_xyz,
+                        float* out_scaling, void* stream);
+
+/* Per-step statistics -- network.py:1276-1282 with gaussian_splatting.py:486-495 / network.py:1152-1154. For points
+ * with radii > 0: max_radii2D = max(max_radii2D, radii); grad_accum += |grad[:, :2]| (* factor if given); denom += 1.
+ * grad has grad_stride floats per row; visible[P] (optional) receives radii > 0 as bytes. */
+int fsgs_densification_stats(int P, int grad_stride, const int32_t* radii, const float* grad, const float* factor,
+                             float* max_radii2D, float* grad_accum, float* denom, uint8_t* visible, void* stream);
+
 /* AdamMasksedUpdated -- fast_2d_gs/_C/src/other/adam_masked_update.cu:30-35 (kernel :9-28). Rows of the [N,M]
  * tensors whose mask byte is 0 are left untouched; eps is added to sqrt(v); lr carries the bias correction. */
 int fsgs_adam_masked_update(int64_t N, int64_t M, const uint8_t* mask, double lr, double b1, double b2, double eps,
