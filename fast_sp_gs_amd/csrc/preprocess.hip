@@ -80,7 +80,8 @@ __device__ __forceinline__ void transmat(int W, int H, const float* p, float sx,
   nrm[2] = Tw2v[8] * t0 + Tw2v[9] * t1 + Tw2v[10] * t2;
 }
 
-template <int kSh>
+// kWave: complete degree-3 rows in one 16-byte aligned [P,16,3] tensor, moved by each wavefront on its own.
+template <int kSh, bool kWave>
 __global__ void __launch_bounds__(256) preprocess_forward_kernel(
     int P, int W, int H, int sh_degree, int n_sh, const float* __restrict__ means3D, const float2* __restrict__ scales,
     const float4* __restrict__ rotations, const float* __restrict__ opacities, const float* __restrict__ shs,
@@ -105,6 +106,17 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
   for (int k = 0; k < 9; ++k) M[k] = 0.0f;
   float p[3] = {0, 0, 0};
   if (valid) p[0] = means3D[3 * (size_t) i], p[1] = means3D[3 * (size_t) i + 1], p[2] = means3D[3 * (size_t) i + 2];
+  const int wave_base = blockIdx.x * blockDim.x + (threadIdx.x & ~63);
+  float* s_wave_rows  = &s_rows[kWave ? (threadIdx.x & ~63) * kShStageStride : 0];
+  ShWaveRows sh_regs;
+  unsigned long long wanted = 0;
+  if (kWave) {
+    // the two cheapest rejections decide which rows are fetched; the fetch is then in flight during the geometry
+    bool maybe = valid && !(culling && culling[i]);
+    maybe = maybe && !((s_Tw2v[8] * p[0] + s_Tw2v[9] * p[1] + s_Tw2v[10] * p[2] + s_Tw2v[11]) <= 0.2f);
+    wanted = __ballot(maybe);
+    if (wanted) wave_fetch_sh_rows(sh_regs, wanted, wave_base, (const float4*) shs);
+  }
   do {
     if (!valid || (culling && culling[i])) break;
     float Tw2v[16], Tw2c[16];
@@ -138,7 +150,10 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
 
   if (sh_degree >= 0) {
     const int n = sh_count(sh_degree);
-    if (kStage) {
+    if (kWave) {
+      if (wanted) wave_rows_to_lds(sh_regs, s_wave_rows);
+      wave_lds_sync();
+    } else if (kStage) {
       s_flag[threadIdx.x] = ok;
       __syncthreads();
       stage_sh_rows(s_rows, s_flag, blockIdx.x * blockDim.x, P, n, n_sh, shs, sh_rest);
@@ -208,7 +223,7 @@ __device__ __forceinline__ void transmat_backward(int W, int H, float sx, float 
   gq[3] = 2 * (x * (dR[9] - dR[6]) + y * (dR[2] - dR[8]) + z * (dR[4] - dR[1]));
 }
 
-template <int kSh>
+template <int kSh, bool kWave>
 __global__ void __launch_bounds__(256) preprocess_backward_kernel(
     int P, int W, int H, int sh_degree, int n_sh, const float* __restrict__ means3D, const float2* __restrict__ scales,
     const float4* __restrict__ rotations, const float* __restrict__ shs, const float* __restrict__ sh_rest,
@@ -229,7 +244,33 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
   const int n      = sh_degree >= 0 ? sh_count(sh_degree) : 0;
   const int m1     = sh_rest ? 1 : n_sh;
   float* my_row    = &s_rows[kStage ? threadIdx.x * kShStageStride : 0];
-  if (kStage && sh_degree >= 0) {
+  const int wave_base = blockIdx.x * blockDim.x + (threadIdx.x & ~63);
+  float* s_wave_rows  = &s_rows[kWave ? (threadIdx.x & ~63) * kShStageStride : 0];
+  const unsigned long long wanted = kWave ? __ballot(vis) : 0ull;
+  if (kWave) {
+    if (wanted == 0ull) {  // nothing of this wavefront was rendered: its gradient rows are zeros
+      if (wave_base < P) {
+#pragma unroll
+        for (int k = 0; k < kShWavePieces; ++k) {
+          int r, c4;
+          wave_piece(k, r, c4);
+          if (wave_base + r < P)
+            ((float4*) g_shs)[(size_t) (wave_base + r) * kShWavePieces + c4] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+      }
+      if (valid) {
+        g_opac[i] = 0.0f;
+        g_means3D[3 * (size_t) i] = 0.0f, g_means3D[3 * (size_t) i + 1] = 0.0f, g_means3D[3 * (size_t) i + 2] = 0.0f;
+        g_scales[i] = make_float2(0.0f, 0.0f);
+        g_rot[i]    = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      }
+      return;
+    }
+    ShWaveRows sh_regs;
+    wave_fetch_sh_rows(sh_regs, wanted, wave_base, (const float4*) shs);
+    wave_rows_to_lds(sh_regs, s_wave_rows);
+    wave_lds_sync();
+  } else if (kStage && sh_degree >= 0) {
     s_flag[threadIdx.x] = vis;
     __syncthreads();
     stage_sh_rows(s_rows, s_flag, blockIdx.x * blockDim.x, P, n, n_sh, shs, sh_rest);
@@ -321,7 +362,10 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
       }
     }
   }
-  if (kStage && sh_degree >= 0 && (g_shs || g_sh_rest)) {
+  if (kWave) {
+    wave_lds_sync();
+    wave_rows_to_global(s_wave_rows, wave_base, P, (float4*) g_shs);
+  } else if (kStage && sh_degree >= 0 && (g_shs || g_sh_rest)) {
     __syncthreads();
     unstage_sh_grads(s_rows, blockIdx.x * blockDim.x, P, n, n_sh, sh_rest != nullptr, g_shs, g_sh_rest);
   }
@@ -386,7 +430,9 @@ FSGS_API int fsgs_gs_2d_preprocess_forward(int P, int W, int H, int sh_degree, i
                    (colors || sh_degree < 0),
                "gs_2d_preprocess_forward: null pointer");
   if (P == 0) return kOk;
-  auto kernel = sh_degree > 3 ? preprocess_forward_kernel<64> : preprocess_forward_kernel<16>;
+  const bool wave_rows = sh_degree == 3 && n_sh == 16 && !sh_rest && (uintptr_t) shs % 16 == 0;
+  auto kernel = sh_degree > 3 ? preprocess_forward_kernel<64, false>
+                              : (wave_rows ? preprocess_forward_kernel<16, true> : preprocess_forward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh, means3D, (const float2*) scales, (const float4*) rotations, opacities, shs,
                      sh_rest, Tw2v, Tv2c, campos, trans_precomp, culling, means2D_preserve, (float2*) means2D, colors,
                      trans_mat, (float4*) normal_opacity, depths, radii, tiles_touched);
@@ -407,7 +453,10 @@ FSGS_API int fsgs_gs_2d_preprocess_backward(int P, int W, int H, int sh_degree, 
   if (sh_degree >= 0)
     FSGS_REQUIRE(shs && colors && grad_colors, "gs_2d_preprocess_backward: SH path needs shs, colors and grad_colors");
   if (P == 0) return kOk;
-  auto kernel = sh_degree > 3 ? preprocess_backward_kernel<64> : preprocess_backward_kernel<16>;
+  const bool wave_rows = sh_degree == 3 && n_sh == 16 && !sh_rest && g_shs && (uintptr_t) shs % 16 == 0 &&
+                         (uintptr_t) g_shs % 16 == 0;
+  auto kernel = sh_degree > 3 ? preprocess_backward_kernel<64, false>
+                              : (wave_rows ? preprocess_backward_kernel<16, true> : preprocess_backward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh, means3D, (const float2*) scales, (const float4*) rotations, shs, sh_rest, Tw2v,
                      Tv2c, campos, trans_mat, radii, colors, (float2*) grad_mean2D, grad_trans, grad_colors,
                      (const float4*) grad_normal_opacity, g_means3D, (float2*) g_scales, (float4*) g_rot, g_opac,

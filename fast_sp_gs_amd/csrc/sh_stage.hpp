@@ -77,4 +77,68 @@ __device__ __forceinline__ void unstage_sh_grads(const float* __restrict__ s_row
   }
 }
 
+// ---- wavefront-private variant for complete degree-3 rows -----------------------------------------------------------
+// With all 16 coefficients in one [P,16,3] tensor a row is twelve 16-byte pieces. A wavefront then moves its own 64 rows
+// by itself: piece e = k * 64 + lane (k < 12) of the wavefront's 768 pieces belongs to row e / 12, so every load or store
+// instruction covers 1 KB of consecutive addresses, the loads can be issued before the data is needed (they are held in
+// registers while the lane does its geometry) and no block-wide barrier is involved.
+constexpr int kShWavePieces = 12;
+
+struct ShWaveRows {
+  float4 v[kShWavePieces];
+};
+
+__device__ __forceinline__ void wave_piece(int k, int& r, int& c4) {
+  const int e = k * 64 + (int) __lane_id();
+  r  = (e * 5462) >> 16;  // e / 12 for 0 <= e < 768
+  c4 = e - r * 12;
+}
+
+// `flags` has bit r set for the rows that are needed (all of them existing rows); the others re-read the first needed
+// row's line instead of branching. flags must not be 0.
+__device__ __forceinline__ void wave_fetch_sh_rows(ShWaveRows& regs, unsigned long long flags, int wave_base,
+                                                   const float4* __restrict__ shs4) {
+  const int first = __builtin_ctzll(flags);
+#pragma unroll
+  for (int k = 0; k < kShWavePieces; ++k) {
+    int r, c4;
+    wave_piece(k, r, c4);
+    const bool on   = (flags >> r) & 1ull;
+    const size_t at = (size_t) (wave_base + (on ? r : first)) * kShWavePieces + (on ? c4 : 0);
+    regs.v[k]       = shs4[at];
+  }
+}
+
+__device__ __forceinline__ void wave_rows_to_lds(const ShWaveRows& regs, float* __restrict__ s_wave_rows) {
+#pragma unroll
+  for (int k = 0; k < kShWavePieces; ++k) {
+    int r, c4;
+    wave_piece(k, r, c4);
+    float* d = s_wave_rows + r * kShStageStride + 4 * c4;
+    d[0] = regs.v[k].x, d[1] = regs.v[k].y, d[2] = regs.v[k].z, d[3] = regs.v[k].w;
+  }
+}
+
+// Orders a wavefront's LDS writes before its later LDS reads of other lanes' data (no instruction is generated: a
+// wavefront's LDS operations complete in order; this only stops the compiler from moving them across).
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Writes the wavefront's 64 staged rows (every existing row) to g4[P,12].
+__device__ __forceinline__ void wave_rows_to_global(const float* __restrict__ s_wave_rows, int wave_base, int P,
+                                                    float4* __restrict__ g4) {
+#pragma unroll
+  for (int k = 0; k < kShWavePieces; ++k) {
+    int r, c4;
+    wave_piece(k, r, c4);
+    if (wave_base + r < P) {
+      const float* s = s_wave_rows + r * kShStageStride + 4 * c4;
+      g4[(size_t) (wave_base + r) * kShWavePieces + c4] = make_float4(s[0], s[1], s[2], s[3]);
+    }
+  }
+}
+
 }  // namespace fsgs
