@@ -311,55 +311,43 @@ __global__ void __launch_bounds__(256) slot_fill_kernel(size_t n4, float4* __res
 }
 
 // Per-surfel sums of the instance records. Nine lanes per surfel, each owning one float2 of the 18-float record, so
-// the lanes of a surfel read 72 contiguous bytes per step and neighbouring surfels continue where the previous one
-// ends. Every row of the four outputs is written (zeros for surfels without instances): no initialisation, no atomics,
-// and the sum order is fixed.
+// the lanes of a surfel read 72 contiguous bytes per record and neighbouring surfels continue where the previous one
+// ends. A surfel's records are fetched eight at a time (past its last record the last one is read again and not added),
+// so most surfels need one round trip to memory; the sum itself runs in instance order. Every row of the four outputs
+// is written (zeros for surfels without instances): no initialisation, no atomics, and the sum order is fixed.
 __global__ void __launch_bounds__(256) slot_reduce_kernel(int P, const int64_t* __restrict__ point_offsets,
     const float* __restrict__ slot_grads, float* __restrict__ g_colors, float* __restrict__ g_means2D,
     float* __restrict__ g_trans, float* __restrict__ g_normal_opacity) {
   constexpr int kPerWave = 7, kLanes = 9;  // 63 of 64 lanes busy
-  constexpr int kUnroll  = 4;              // surfels per lane group: their loads are in flight together
+  constexpr int kDepth   = 8;              // records of one surfel in flight together
   const int lane = threadIdx.x & 63;
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
   const int sub = lane / kLanes, k = lane - sub * kLanes;
-  if (sub >= kPerWave) return;
+  const int i = wave * kPerWave + sub;
+  if (sub >= kPerWave || i >= P) return;
   // A surfel without instances (not rendered) has equal scan offsets, so the visibility need not be read.
-  int64_t e0[kUnroll], e1[kUnroll];
-#pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    const int i = (wave * kUnroll + u) * kPerWave + sub;
-    e0[u] = (i > 0 && i < P) ? point_offsets[i - 1] : 0;
-    e1[u] = i < P ? point_offsets[i] : 0;
-    if (i >= P) e0[u] = e1[u] = 0;
-  }
+  const int64_t e0 = i > 0 ? point_offsets[i - 1] : 0, e1 = point_offsets[i];
   const float2* src = (const float2*) slot_grads + k;
-  float2 acc[kUnroll];
+  float2 acc = make_float2(0.0f, 0.0f);
+  for (int64_t base = e0; base < e1; base += kDepth) {
+    float2 v[kDepth];
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) acc[u] = make_float2(0.0f, 0.0f);
-  // first instance of every surfel together (most surfels have one to four), then the rest in order
+    for (int j = 0; j < kDepth; ++j) v[j] = src[(size_t) (base + j < e1 ? base + j : e1 - 1) * kLanes];
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u)
-    if (e0[u] < e1[u]) acc[u] = src[(size_t) e0[u] * kLanes];
-#pragma unroll
-  for (int u = 0; u < kUnroll; ++u)
-    for (int64_t e = e0[u] + 1; e < e1[u]; ++e) {
-      const float2 v = src[(size_t) e * kLanes];
-      acc[u].x += v.x, acc[u].y += v.y;
+    for (int j = 0; j < kDepth; ++j) {
+      const bool on = base + j < e1;
+      acc.x += on ? v[j].x : 0.0f, acc.y += on ? v[j].y : 0.0f;
     }
+  }
   // record layout: 0-2 colours | 3-11 trans_mat | 12-14 normal | 15 opacity | 16-17 means2D
+  const float vals[2] = {acc.x, acc.y};
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    const int i = (wave * kUnroll + u) * kPerWave + sub;
-    if (i >= P) continue;
-    const float vals[2] = {acc[u].x, acc[u].y};
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int c = 2 * k + h;
-      if (c < 3) g_colors[3 * (size_t) i + c] = vals[h];
-      else if (c < 12) g_trans[9 * (size_t) i + (c - 3)] = vals[h];
-      else if (c < 16) g_normal_opacity[4 * (size_t) i + (c - 12)] = vals[h];
-      else g_means2D[2 * (size_t) i + (c - 16)] = vals[h];
-    }
+  for (int h = 0; h < 2; ++h) {
+    const int c = 2 * k + h;
+    if (c < 3) g_colors[3 * (size_t) i + c] = vals[h];
+    else if (c < 12) g_trans[9 * (size_t) i + (c - 3)] = vals[h];
+    else if (c < 16) g_normal_opacity[4 * (size_t) i + (c - 12)] = vals[h];
+    else g_means2D[2 * (size_t) i + (c - 16)] = vals[h];
   }
 }
 
@@ -419,7 +407,7 @@ FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, doub
     if (aux && flow) FSGS_LAUNCH_BWD(true, true, true);
     else if (aux) FSGS_LAUNCH_BWD(true, false, true);
     else FSGS_LAUNCH_BWD(false, false, true);
-    const int waves = div_up(P, 7 * 4);  // kPerWave * kUnroll surfels per wavefront
+    const int waves = div_up(P, 7);  // kPerWave surfels per wavefront
     hipLaunchKernelGGL(slot_reduce_kernel, dim3(div_up((int64_t) waves * 64, 256)), dim3(256), 0, s, P, point_offsets,
                        slot_grads, g_colors, g_means2D, g_trans, g_normal_opacity);
   } else {
