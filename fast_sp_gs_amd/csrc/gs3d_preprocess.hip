@@ -219,7 +219,8 @@ __device__ __forceinline__ bool screen_geometry(int W, int H, int gx, int gy, bo
   return true;
 }
 
-template <int kSh>
+// kWave: complete degree-3 rows in one 16-byte aligned [P,16,3] tensor, moved by each wavefront on its own.
+template <int kSh, bool kWave>
 __global__ void __launch_bounds__(256) gs3d_preprocess_forward_kernel(int P, int W, int H, int sh_degree, int n_sh,
     int is_opengl, const float* __restrict__ means3D, const float* __restrict__ scales,
     const float4* __restrict__ rotations, const float* __restrict__ opacities, const float* __restrict__ shs,
@@ -243,6 +244,14 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_forward_kernel(int P, int
   float p[3] = {0, 0, 0}, c3[6] = {0, 0, 0, 0, 0, 0}, rgb[3] = {0, 0, 0};
   Screen sc = {};
   if (valid) p[0] = means3D[3 * (size_t) i], p[1] = means3D[3 * (size_t) i + 1], p[2] = means3D[3 * (size_t) i + 2];
+  const int wave_base = blockIdx.x * blockDim.x + (threadIdx.x & ~63);
+  float* s_wave_rows  = &s_rows[kWave ? (threadIdx.x & ~63) * kShStageStride : 0];
+  ShWaveRows sh_regs;
+  unsigned long long wanted = 0;
+  if (kWave) {  // the fetch of the rows is in flight during the geometry
+    wanted = __ballot(valid && !(culling && culling[i]));
+    if (wanted) wave_fetch_sh_rows(sh_regs, wanted, wave_base, (const float4*) shs);
+  }
   do {
     if (!valid || (culling && culling[i])) break;
     float Tw2v[16], Tv2c[16];
@@ -258,7 +267,10 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_forward_kernel(int P, int
 
   if (sh_degree >= 0) {
     const int n = sh_count(sh_degree);
-    if (kStage) {
+    if (kWave) {
+      if (wanted) wave_rows_to_lds(sh_regs, s_wave_rows);
+      wave_lds_sync();
+    } else if (kStage) {
       s_flag[threadIdx.x] = ok;
       __syncthreads();
       stage_sh_rows(s_rows, s_flag, blockIdx.x * blockDim.x, P, n, n_sh, shs, sh_rest);
@@ -288,7 +300,7 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_forward_kernel(int P, int
   conic_opacity[i] = ok ? make_float4(sc.conic[0], sc.conic[1], sc.conic[2], opacities[i]) : make_float4(0, 0, 0, 0);
 }
 
-template <int kSh>
+template <int kSh, bool kWave>
 __global__ void __launch_bounds__(256) gs3d_preprocess_backward_kernel(int P, int W, int H, int sh_degree, int n_sh,
     int is_opengl, const float* __restrict__ means3D, const float* __restrict__ scales,
     const float4* __restrict__ rotations, const float* __restrict__ shs, const float* __restrict__ sh_rest,
@@ -311,7 +323,17 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_backward_kernel(int P, in
   const int m1     = sh_rest ? 1 : n_sh;
   float* my_row    = &s_rows[kStage ? threadIdx.x * kShStageStride : 0];
   const float fx = 0.5f * (float) W / tanx, fy = 0.5f * (float) H / tany;
-  if (kStage && sh_degree >= 0) {
+  const int wave_base = blockIdx.x * blockDim.x + (threadIdx.x & ~63);
+  float* s_wave_rows  = &s_rows[kWave ? (threadIdx.x & ~63) * kShStageStride : 0];
+  if (kWave) {
+    const unsigned long long wanted = __ballot(vis);
+    if (wanted) {
+      ShWaveRows sh_regs;
+      wave_fetch_sh_rows(sh_regs, wanted, wave_base, (const float4*) shs);
+      wave_rows_to_lds(sh_regs, s_wave_rows);
+    }
+    wave_lds_sync();
+  } else if (kStage && sh_degree >= 0) {
     s_flag[threadIdx.x] = vis;
     __syncthreads();
     stage_sh_rows(s_rows, s_flag, blockIdx.x * blockDim.x, P, n, n_sh, shs, sh_rest);
@@ -406,7 +428,10 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_backward_kernel(int P, in
       }
     }
   }
-  if (kStage && sh_degree >= 0 && (g_shs || g_sh_rest)) {
+  if (kWave) {
+    wave_lds_sync();
+    wave_rows_to_global(s_wave_rows, wave_base, P, (float4*) g_shs);
+  } else if (kStage && sh_degree >= 0 && (g_shs || g_sh_rest)) {
     __syncthreads();
     unstage_sh_grads(s_rows, blockIdx.x * blockDim.x, P, n, n_sh, sh_rest != nullptr, g_shs, g_sh_rest);
   }
@@ -432,7 +457,10 @@ FSGS_API int fsgs_gs_preprocess_forward(int P, int W, int H, int sh_degree, int 
   FSGS_REQUIRE(means3D && scales && rotations && opacities && shs && Tw2v && Tv2c && campos && means2D && depths &&
                    radii && tiles_touched && cov3Ds && conic_opacity && (colors || sh_degree < 0),
                "gs_preprocess_forward: null pointer");
-  auto kernel = sh_degree > 3 ? gs3d_preprocess_forward_kernel<64> : gs3d_preprocess_forward_kernel<16>;
+  const bool wave_rows = sh_degree == 3 && n_sh == 16 && !sh_rest && (uintptr_t) shs % 16 == 0;
+  auto kernel = sh_degree > 3 ? gs3d_preprocess_forward_kernel<64, false>
+                              : (wave_rows ? gs3d_preprocess_forward_kernel<16, true>
+                                           : gs3d_preprocess_forward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh,
                      is_opengl, means3D, scales, (const float4*) rotations, opacities, shs, sh_rest, Tw2v, Tv2c,
                      campos, (float) tan_fovx, (float) tan_fovy, culling, means2D_preserve, (float2*) means2D, depths,
@@ -455,7 +483,11 @@ FSGS_API int fsgs_gs_preprocess_backward(int P, int W, int H, int sh_degree, int
                "gs_preprocess_backward: null pointer");
   if (sh_degree >= 0)
     FSGS_REQUIRE(shs && colors && grad_colors, "gs_preprocess_backward: SH path needs shs, colors and grad_colors");
-  auto kernel = sh_degree > 3 ? gs3d_preprocess_backward_kernel<64> : gs3d_preprocess_backward_kernel<16>;
+  const bool wave_rows = sh_degree == 3 && n_sh == 16 && !sh_rest && g_shs && (uintptr_t) shs % 16 == 0 &&
+                         (uintptr_t) g_shs % 16 == 0;
+  auto kernel = sh_degree > 3 ? gs3d_preprocess_backward_kernel<64, false>
+                              : (wave_rows ? gs3d_preprocess_backward_kernel<16, true>
+                                           : gs3d_preprocess_backward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh,
                      is_opengl, means3D, scales, (const float4*) rotations, shs, sh_rest, Tw2v, Tv2c, campos,
                      (float) tan_fovx, (float) tan_fovy, radii, colors, cov3Ds, (float2*) grad_mean2D, grad_colors,
