@@ -12,6 +12,7 @@
 // counts, keys, ranges and point lists are reproducible bit for bit against a plain IEEE evaluation.
 #include "binning.hpp"
 #include "sh.hpp"
+#include "sh_stage.hpp"
 #include "surfel_geom.hpp"
 
 FSGS_API int fsgs_gs_prepare_scan(int P, const int32_t* tiles_touched, int64_t* point_offsets, void* workspace,
@@ -95,7 +96,8 @@ __device__ __forceinline__ void fast_transmat_backward(float sx, float sy, const
   gq[3] = 2 * (x * (dR[7] - dR[5]) + y * (dR[2] - dR[6]) + z * (dR[3] - dR[1]));
 }
 
-template <int kSh>
+// kWave: complete degree-3 rows in one 16-byte aligned [P,16,3] tensor, moved by each wavefront on its own (sh_stage.hpp).
+template <int kSh, bool kWave>
 __global__ void __launch_bounds__(256) fast_preprocess_forward_kernel(
     int P, int W, int H, int sh_degree, int n_sh, const float* __restrict__ means3D, const float2* __restrict__ scales,
     const float4* __restrict__ rotations, const float* __restrict__ opacities, const float* __restrict__ shs,
@@ -104,8 +106,11 @@ __global__ void __launch_bounds__(256) fast_preprocess_forward_kernel(
     int means2D_preserve, float2* __restrict__ means2D, float* __restrict__ colors, float* __restrict__ trans_mat,
     float* __restrict__ inverse_m, float4* __restrict__ normal_opacity, float* __restrict__ depths,
     int32_t* __restrict__ radii, int32_t* __restrict__ tiles_touched) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= P) return;
+  __shared__ float s_rows[kWave ? kShStageRows * kShStageStride : 1];
+  const int i0     = blockIdx.x * blockDim.x + threadIdx.x;
+  const bool valid = i0 < P;
+  if (!kWave && !valid) return;
+  const int i = valid ? i0 : P - 1;  // lanes past the end stay for the wavefront's row movement and write nothing
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   float Tw2v[16], Tv2s[9];
 #pragma unroll
@@ -119,8 +124,19 @@ __global__ void __launch_bounds__(256) fast_preprocess_forward_kernel(
 #pragma unroll
   for (int k = 0; k < 9; ++k) M[k] = 0.0f;
   const float p[3] = {means3D[3 * (size_t) i], means3D[3 * (size_t) i + 1], means3D[3 * (size_t) i + 2]};
+  const int wave_base = blockIdx.x * blockDim.x + (threadIdx.x & ~63);
+  float* s_wave_rows  = &s_rows[kWave ? (threadIdx.x & ~63) * kShStageStride : 0];
+  ShWaveRows sh_regs;
+  unsigned long long wanted = 0;
+  if (kWave) {
+    // the two cheapest rejections decide which rows are fetched; the fetch is then in flight during the geometry
+    bool maybe = valid && !(culling && culling[i]);
+    maybe = maybe && !((Tw2v[8] * p[0] + Tw2v[9] * p[1] + Tw2v[10] * p[2] + Tw2v[11]) <= 0.2f);
+    wanted = __ballot(maybe);
+    if (wanted) wave_fetch_sh_rows(sh_regs, wanted, wave_base, (const float4*) shs);
+  }
   do {
-    if (culling && culling[i]) break;
+    if (!valid || (culling && culling[i])) break;
     const float pv[3] = {Tw2v[0] * p[0] + Tw2v[1] * p[1] + Tw2v[2] * p[2] + Tw2v[3],
                          Tw2v[4] * p[0] + Tw2v[5] * p[1] + Tw2v[6] * p[2] + Tw2v[7],
                          Tw2v[8] * p[0] + Tw2v[9] * p[1] + Tw2v[10] * p[2] + Tw2v[11]};
@@ -147,17 +163,22 @@ __global__ void __launch_bounds__(256) fast_preprocess_forward_kernel(
     ok    = true;
   } while (false);
 
+  if (kWave) {
+    if (wanted) wave_rows_to_lds(sh_regs, s_wave_rows);
+    wave_lds_sync();
+  }
   if (ok && sh_degree >= 0) {
     float x, y, z, Y[kSh];
     view_dir(p, campos, x, y, z);
     sh_eval(sh_degree, x, y, z, Y);
     const int n = sh_count(sh_degree);
-    const float* c0 = shs + (size_t) i * (sh_rest ? 1 : n_sh) * 3;
+    const float* c0 = kWave ? &s_rows[threadIdx.x * kShStageStride] : shs + (size_t) i * (sh_rest ? 1 : n_sh) * 3;
     float r = c0[0] * Y[0], g = c0[1] * Y[0], b = c0[2] * Y[0];
-    const float* cr = sh_rest ? sh_rest + (size_t) i * n_sh * 3 - 3 : c0;
+    const float* cr = kWave ? c0 : (sh_rest ? sh_rest + (size_t) i * n_sh * 3 - 3 : c0);
     for (int l = 1; l < n; ++l) r += cr[3 * l] * Y[l], g += cr[3 * l + 1] * Y[l], b += cr[3 * l + 2] * Y[l];
     rgb[0] = fmaxf(0.0f, r + 0.5f), rgb[1] = fmaxf(0.0f, g + 0.5f), rgb[2] = fmaxf(0.0f, b + 0.5f);
   }
+  if (!valid) return;
   float adj[9];
 #pragma unroll
   for (int k = 0; k < 9; ++k) adj[k] = 0.0f;
@@ -281,7 +302,7 @@ __global__ void __launch_bounds__(256) fast_duplicate_keys_kernel(int P, int gx,
   }
 }
 
-template <int kSh>
+template <int kSh, bool kWave>
 __global__ void __launch_bounds__(256) fast_preprocess_backward_kernel(
     int P, int W, int H, int sh_degree, int n_sh, const float* __restrict__ means3D, const float2* __restrict__ scales,
     const float4* __restrict__ rotations, const float* __restrict__ shs, const float* __restrict__ sh_rest,
@@ -291,8 +312,27 @@ __global__ void __launch_bounds__(256) fast_preprocess_backward_kernel(
     const float* __restrict__ grad_colors, const float4* __restrict__ grad_normal_opacity,
     float* __restrict__ g_means3D, float2* __restrict__ g_scales, float4* __restrict__ g_rot,
     float* __restrict__ g_opac, float* __restrict__ g_shs, float* __restrict__ g_sh_rest) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= P || radii[i] <= 0) return;
+  __shared__ float s_rows[kWave ? kShStageRows * kShStageStride : 1];
+  const int i    = blockIdx.x * blockDim.x + threadIdx.x;
+  const bool vis = i < P && radii[i] > 0;
+  const int wave_base = blockIdx.x * blockDim.x + (threadIdx.x & ~63);
+  float* s_wave_rows  = &s_rows[kWave ? (threadIdx.x & ~63) * kShStageStride : 0];
+  float* my_row       = &s_rows[kWave ? threadIdx.x * kShStageStride : 0];
+  if (kWave) {
+    const unsigned long long wanted = __ballot(vis);
+    if (wanted == 0ull) return;  // rows nobody rendered keep the caller's zeros
+    ShWaveRows sh_regs;
+    wave_fetch_sh_rows(sh_regs, wanted, wave_base, (const float4*) shs);
+    wave_rows_to_lds(sh_regs, s_wave_rows);
+    wave_lds_sync();
+    if (!vis) {
+#pragma unroll
+      for (int c = 0; c < kShStageFloats; ++c) my_row[c] = 0.0f;
+    }
+  } else if (!vis) {
+    return;
+  }
+  if (vis) {
   float Tw2v[16], Tv2s[9];
 #pragma unroll
   for (int k = 0; k < 16; ++k) Tw2v[k] = Tw2v_g[k];
@@ -344,10 +384,11 @@ __global__ void __launch_bounds__(256) fast_preprocess_backward_kernel(
     for (int c = 0; c < 3; ++c) g[c] = grad_colors[3 * (size_t) i + c] * (float) (colors[3 * (size_t) i + c] > 0);
     const int n  = sh_count(sh_degree);
     const int m1 = sh_rest ? 1 : n_sh;
-    const float* c0 = shs + (size_t) i * m1 * 3;
-    const float* cr = sh_rest ? sh_rest + (size_t) i * n_sh * 3 - 3 : c0;
-    float* o0  = g_shs ? g_shs + (size_t) i * m1 * 3 : nullptr;
-    float* orr = g_sh_rest ? g_sh_rest + (size_t) i * n_sh * 3 - 3 : o0;
+    // with kWave the coefficients are read from the lane's staged row and the gradient row is written over them
+    const float* c0 = kWave ? my_row : shs + (size_t) i * m1 * 3;
+    const float* cr = kWave ? my_row : (sh_rest ? sh_rest + (size_t) i * n_sh * 3 - 3 : c0);
+    float* o0  = kWave ? my_row : (g_shs ? g_shs + (size_t) i * m1 * 3 : nullptr);
+    float* orr = kWave ? my_row : (g_sh_rest ? g_sh_rest + (size_t) i * n_sh * 3 - 3 : o0);
     if (o0) o0[0] = g[0] * Y[0], o0[1] = g[1] * Y[0], o0[2] = g[2] * Y[0];
     tl[0] = 0.0f;
     for (int l = 1; l < n; ++l) {
@@ -368,6 +409,11 @@ __global__ void __launch_bounds__(256) fast_preprocess_backward_kernel(
   // densification proxy from the ACCUMULATED transform gradient (gs_2d_fast_preprocess.cu:606-608)
   const float depth = m[8];
   grad_mean2D[i] = make_float2(gT[2] * depth * 0.5f * (float) W, gT[5] * depth * 0.5f * (float) H);
+  }
+  if (kWave) {
+    wave_lds_sync();
+    wave_rows_to_global(s_wave_rows, wave_base, P, (float4*) g_shs);
+  }
 }
 
 __global__ void __launch_bounds__(256) fast_transmat_forward_kernel(int P, const float* __restrict__ means3D,
@@ -430,7 +476,10 @@ FSGS_API int fsgs_gs_2d_fast_preprocess_forward(int P, int W, int H, int sh_degr
                    (colors || sh_degree < 0),
                "gs_2d_fast_preprocess_forward: null pointer");
   if (P == 0) return kOk;
-  auto kernel = sh_degree > 3 ? fast_preprocess_forward_kernel<64> : fast_preprocess_forward_kernel<16>;
+  const bool wave_rows = sh_degree == 3 && n_sh == 16 && !sh_rest && (uintptr_t) shs % 16 == 0;
+  auto kernel = sh_degree > 3 ? fast_preprocess_forward_kernel<64, false>
+                              : (wave_rows ? fast_preprocess_forward_kernel<16, true>
+                                           : fast_preprocess_forward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh,
                      means3D, (const float2*) scales, (const float4*) rotations, opacities, shs, sh_rest, Tw2v, Tv2s,
                      campos, trans_precomp, culling, means2D_preserve, (float2*) means2D, colors, trans_mat, inverse_m,
@@ -486,7 +535,11 @@ FSGS_API int fsgs_gs_2d_fast_preprocess_backward(int P, int W, int H, int sh_deg
   if (sh_degree >= 0)
     FSGS_REQUIRE(shs && colors && grad_colors, "gs_2d_fast_preprocess_backward: SH path needs shs, colors, grad_colors");
   if (P == 0) return kOk;
-  auto kernel = sh_degree > 3 ? fast_preprocess_backward_kernel<64> : fast_preprocess_backward_kernel<16>;
+  const bool wave_rows = sh_degree == 3 && n_sh == 16 && !sh_rest && g_shs && (uintptr_t) shs % 16 == 0 &&
+                         (uintptr_t) g_shs % 16 == 0;
+  auto kernel = sh_degree > 3 ? fast_preprocess_backward_kernel<64, false>
+                              : (wave_rows ? fast_preprocess_backward_kernel<16, true>
+                                           : fast_preprocess_backward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh,
                      means3D, (const float2*) scales, (const float4*) rotations, shs, sh_rest, Tw2v, Tv2s, campos,
                      trans_mat, radii, colors, (float2*) grad_mean2D, grad_trans, grad_inv_m, grad_colors,
