@@ -278,10 +278,17 @@ __global__ void __launch_bounds__(1024) tile_scan_kernel(int T, unsigned long lo
   if (threadIdx.x == 0) *large_count = 0;
 }
 
+// Where element i of a segment sits in LDS. With kPad one slot in five stays empty: the rounds of the sorting network
+// whose lanes each own four consecutive elements, or four elements 4 apart, then spread a wavefront's 8-byte accesses
+// over all banks instead of piling them sixteen deep on a quarter of them.
+template <bool kPad>
+__device__ __forceinline__ int lds_slot(int i) { return kPad ? i + (i >> 2) : i; }
+
+template <bool kPad>
 __device__ __forceinline__ void tile_sort_output(int tile, int64_t start, int n, const uint64_t* sorted_local,
                                                  int32_t* __restrict__ point_list, int64_t* __restrict__ keys_out) {
   for (int k = threadIdx.x; k < n; k += blockDim.x) {
-    const uint64_t e = sorted_local[k];
+    const uint64_t e = sorted_local[lds_slot<kPad>(k)];
     point_list[start + k] = (int32_t) (uint32_t) e;
     if (keys_out) keys_out[start + k] = (int64_t) (((uint64_t) (uint32_t) tile << 32) | (e >> 32));
   }
@@ -322,37 +329,76 @@ __device__ __forceinline__ void bitonic_sort(uint64_t* e, Index n, int threads, 
 
 // The same network for a segment held in LDS, two network steps per barrier: a lane loads four elements that are closed
 // under two consecutive steps (mirror + first half-cleaner, or two half-cleaners), exchanges them in registers and
-// stores them back. Elements beyond n read as +infinity and are never stored.
+// stores them back.
 __device__ __forceinline__ void cx(uint64_t& a, uint64_t& b) {
   const uint64_t lo = a < b ? a : b, hi = a < b ? b : a;
   a = lo, b = hi;
 }
 
-__device__ __forceinline__ void bitonic_sort_lds(uint64_t* e, int n, int threads) {
+// A lane's four elements of a round lie inside an aligned span of the array (the merge size for a mirror round, twice
+// the larger stride for a pair of half-cleaners), and with quads dealt to lanes in order a wavefront's 64 quads of one
+// loop iteration cover one aligned 256-element chunk. Rounds whose span fits such a chunk therefore exchange data only
+// between lanes of the same wavefront, which needs no block-wide barrier (a wavefront's LDS operations complete in
+// order): of the 33 rounds that sort 2048 entries only 7 end in a barrier.
+constexpr int kWaveSpan = 4 * kWave;
+
+__device__ __forceinline__ void end_round(int span, int next_span) {
+  if (span <= kWaveSpan && next_span <= kWaveSpan) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  } else {
+    __syncthreads();
+  }
+}
+
+// Power of two that a segment of n entries is padded to (with +infinity keys) before bitonic_sort_lds.
+__device__ __forceinline__ int padded_length(int n) {
   int m = 2;
   while (m < n) m <<= 1;
-  auto ld = [&](int i) { return i < n ? e[i] : ~0ull; };
-  auto st = [&](int i, uint64_t v) { if (i < n) e[i] = v; };
+  return m;
+}
+
+// Sorts m = 2^k >= 2 entries; every one of the m slots holds a key (the caller pads with ~0), so no access is
+// conditional: bounds checks around the loads and stores made the compiler serialise them, one LDS round trip each.
+template <bool kPad>
+__device__ __forceinline__ void bitonic_sort_lds(uint64_t* e, int m, int threads) {
+  auto ld = [&](int i) { return e[lds_slot<kPad>(i)]; };
+  auto st = [&](int i, uint64_t v) { e[lds_slot<kPad>(i)] = v; };
+  // one network step on pairs (two pairs per lane and iteration, so that the quads-in-order property above holds)
   auto single = [&](int size, int log_half, int stride) {  // stride == 0: the mirror step of `size`
-    for (int k = threadIdx.x; k < (m >> 1); k += threads) {
-      int lo, hi;
-      if (stride == 0) {
-        const int blk = k >> log_half, off = k & ((size >> 1) - 1);
-        lo = blk * size + off, hi = blk * size + size - 1 - off;
-      } else {
-        lo = ((k & ~(stride - 1)) << 1) | (k & (stride - 1)), hi = lo | stride;
-      }
-      if (hi < n) {
-        uint64_t a = e[lo], b = e[hi];
-        if (a > b) e[lo] = b, e[hi] = a;
+    for (int q = threadIdx.x; q < (m >> 2); q += threads) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int k = 2 * q + h;
+        int lo, hi;
+        if (stride == 0) {
+          const int blk = k >> log_half, off = k & ((size >> 1) - 1);
+          lo = blk * size + off, hi = blk * size + size - 1 - off;
+        } else {
+          lo = ((k & ~(stride - 1)) << 1) | (k & (stride - 1)), hi = lo | stride;
+        }
+        uint64_t a = ld(lo), b = ld(hi);
+        cx(a, b);
+        st(lo, a), st(hi, b);
       }
     }
-    __syncthreads();
   };
   int log_half = 0;
   for (int size = 2; size <= m; size <<= 1, ++log_half) {
+    const int next_size_span = size < m ? 2 * size : 0;
     if (size == 2) {
+      if (m == 2) {
+        if (threadIdx.x == 0) {
+          uint64_t a = ld(0), b = ld(1);
+          cx(a, b);
+          st(0, a), st(1, b);
+        }
+        __syncthreads();
+        return;
+      }
       single(2, 0, 0);
+      end_round(2, next_size_span);
       continue;
     }
     const int quarter = size >> 2;
@@ -365,8 +411,8 @@ __device__ __forceinline__ void bitonic_sort_lds(uint64_t* e, int n, int threads
       cx(a, b), cx(bm, am);
       st(ia, a), st(ib, b), st(jb, bm), st(ja, am);
     }
-    __syncthreads();
     int stride = quarter >> 1;
+    end_round(size, stride >= 2 ? 2 * stride : (stride == 1 ? 2 : next_size_span));
     for (; stride >= 2; stride >>= 2) {  // half-cleaners of strides `stride` and `stride / 2`
       const int lo_s = stride >> 1;
       for (int q = threadIdx.x; q < (m >> 2); q += threads) {
@@ -377,10 +423,15 @@ __device__ __forceinline__ void bitonic_sort_lds(uint64_t* e, int n, int threads
         cx(v0, v1), cx(v2, v3);
         st(i0, v0), st(i1, v1), st(i2, v2), st(i3, v3);
       }
-      __syncthreads();
+      const int next = stride >> 2;
+      end_round(2 * stride, next >= 2 ? 2 * next : (next == 1 ? 2 : next_size_span));
     }
-    if (stride == 1) single(size, log_half, 1);
+    if (stride == 1) {
+      single(size, log_half, 1);
+      end_round(2, next_size_span);
+    }
   }
+  __syncthreads();
 }
 
 constexpr int kSmallSegment = 2048;   // entries sorted by a 256-lane block in 16 KB of LDS
@@ -391,7 +442,7 @@ constexpr int kLargeSegment = 16384;  // entries sorted by a 1024-lane block in 
 __global__ void __launch_bounds__(256) tile_sort_small_kernel(int64_t* __restrict__ ranges,
     const uint64_t* __restrict__ entries, int32_t* __restrict__ point_list, int64_t* __restrict__ keys_out,
     int* __restrict__ large_count, int* __restrict__ large_list) {
-  __shared__ uint64_t s_e[kSmallSegment];
+  __shared__ uint64_t s_e[kSmallSegment + kSmallSegment / 4];
   const int tile = blockIdx.x;
   const int64_t start = ranges[2 * (size_t) tile];
   const int64_t len   = ranges[2 * (size_t) tile + 1] - start;
@@ -404,10 +455,11 @@ __global__ void __launch_bounds__(256) tile_sort_small_kernel(int64_t* __restric
     return;
   }
   const int n = (int) len;
-  for (int k = threadIdx.x; k < n; k += 256) s_e[k] = entries[start + k];
+  const int m = padded_length(n);
+  for (int k = threadIdx.x; k < m; k += 256) s_e[lds_slot<true>(k)] = k < n ? entries[start + k] : ~0ull;
   __syncthreads();
-  bitonic_sort_lds(s_e, n, 256);
-  tile_sort_output(tile, start, n, s_e, point_list, keys_out);
+  bitonic_sort_lds<true>(s_e, m, 256);
+  tile_sort_output<true>(tile, start, n, s_e, point_list, keys_out);
 }
 
 // A few blocks walk the queue of long segments: up to kLargeSegment entries in LDS, beyond that the same network on the
@@ -423,10 +475,11 @@ __global__ void __launch_bounds__(1024) tile_sort_large_kernel(const int64_t* __
     const int64_t len   = ranges[2 * (size_t) tile + 1] - start;
     if (len <= kLargeSegment) {
       const int n = (int) len;
-      for (int k = threadIdx.x; k < n; k += 1024) s_e[k] = entries[start + k];
+      const int m = padded_length(n);
+      for (int k = threadIdx.x; k < m; k += 1024) s_e[k] = k < n ? entries[start + k] : ~0ull;
       __syncthreads();
-      bitonic_sort_lds(s_e, n, 1024);
-      tile_sort_output(tile, start, n, s_e, point_list, keys_out);
+      bitonic_sort_lds<false>(s_e, m, 1024);
+      tile_sort_output<false>(tile, start, n, s_e, point_list, keys_out);
       __syncthreads();
     } else {
       uint64_t* e = entries + start;
@@ -434,7 +487,7 @@ __global__ void __launch_bounds__(1024) tile_sort_large_kernel(const int64_t* __
         __threadfence_block();
         __syncthreads();
       });
-      tile_sort_output(tile, start, (int) len, e, point_list, keys_out);
+      tile_sort_output<false>(tile, start, (int) len, e, point_list, keys_out);
     }
   }
 }
