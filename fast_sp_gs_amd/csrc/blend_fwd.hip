@@ -91,20 +91,27 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
     for (int c = 0; c < kFwdBatch / kWave; ++c) {
       const int jj = c * kWave + lane;
       unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u));
+      if (todo == 0ull) continue;
+      // A wavefront walks its list alone, so the LDS round trip for a surfel's record would be paid once per entry on
+      // the tile's critical path: the record of the NEXT entry is requested before the current one is evaluated.
+      SplatHot hot_next = s_hot[c * kWave + __builtin_ctzll(todo)];
       while (todo) {
         if (__ballot(!done) == 0ull) break;  // every pixel of this quadrant is saturated
         const int j = c * kWave + __builtin_ctzll(todo);
         todo &= todo - 1;
+        const SplatHot hot = hot_next;
+        hot_next           = s_hot[c * kWave + (todo ? __builtin_ctzll(todo) : 0)];
+        const SplatCold cold = s_cold[j];  // needed only if a pixel blends the surfel, but then without waiting
+        __builtin_amdgcn_sched_barrier(0);
         if (done) continue;
         Hit h;
-        if (!intersect(s_hot[j], pxf, pyf, near_n, h)) continue;
+        if (!intersect(hot, pxf, pyf, near_n, h)) continue;
         const float test_T = T * (1.0f - h.alpha);
         if (test_T < 0.0001f) {
           done = true;
           continue;
         }
         const float w        = h.alpha * T;
-        const SplatCold cold = s_cold[j];
         const int contributor = b * kFwdBatch + j + 1;
         if (kAux) {
           const float A = 1.0f - T;
