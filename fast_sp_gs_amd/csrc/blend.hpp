@@ -114,6 +114,30 @@ __device__ __forceinline__ bool intersect(const SplatHot& h, float pxf, float py
   return !(o.alpha < (1.0f / 255.0f));
 }
 
+// The same test without early exits: every lane runs the whole sequence and the rejections are combined at the end, so
+// the caller gets one predicate instead of nested divergent regions. Contraction is switched off and every fused
+// multiply-add is written out, so that each inlined copy of this function rounds alike (a kernel that instantiates it
+// twice must not depend on which copy evaluated a surfel).
+__device__ __forceinline__ bool intersect_flat(const SplatHot& h, float pxf, float pyf, float near_n, Hit& o) {
+#pragma clang fp contract(off)
+  o.kx = fmaf(pxf, h.m[6], -h.m[0]), o.ky = fmaf(pxf, h.m[7], -h.m[1]), o.kz = fmaf(pxf, h.m[8], -h.m[2]);
+  o.lx = fmaf(pyf, h.m[6], -h.m[3]), o.ly = fmaf(pyf, h.m[7], -h.m[4]), o.lz = fmaf(pyf, h.m[8], -h.m[5]);
+  const float px_ = fmaf(o.ky, o.lz, -(o.kz * o.ly));
+  const float py_ = fmaf(o.kz, o.lx, -(o.kx * o.lz));
+  o.pz            = fmaf(o.kx, o.ly, -(o.ky * o.lx));
+  const float rz = __builtin_amdgcn_rcpf(o.pz);
+  o.sx = px_ * rz, o.sy = py_ * rz;
+  o.rho3d = fmaf(o.sx, o.sx, o.sy * o.sy);
+  o.dx = h.cx - pxf, o.dy = h.cy - pyf;
+  o.rho2d = 2.0f * fmaf(o.dx, o.dx, o.dy * o.dy);
+  const float rho = fminf(o.rho3d, o.rho2d);
+  o.depth = fmaf(o.sx, h.m[6], o.sy * h.m[7]) + h.m[8];
+  const float power = -0.5f * rho;
+  o.G     = __expf(power);
+  o.alpha = fminf(0.99f, h.opacity * o.G);
+  return (o.pz != 0.0f) & !(o.depth < near_n) & !(power > 0.0f) & !(o.alpha < (1.0f / 255.0f));
+}
+
 // ---- conservative per-quadrant culling ------------------------------------------------------------------------------
 // A surfel can only be blended at a pixel if alpha = min(0.99, o * exp(-rho / 2)) >= 1/255, i.e. rho <= tau with
 // tau = 2 ln(255 o), where rho = min(rho3d, rho2d). The pixels with rho3d <= tau are the perspective image of the

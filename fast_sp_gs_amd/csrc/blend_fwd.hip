@@ -92,58 +92,80 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
       const int jj = c * kWave + lane;
       unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u));
       if (todo == 0ull) continue;
-      // A wavefront walks its list alone, so the LDS round trip for a surfel's record would be paid once per entry on
-      // the tile's critical path: the record of the NEXT entry is requested before the current one is evaluated.
-      SplatHot hot_next = s_hot[c * kWave + __builtin_ctzll(todo)];
-      while (todo) {
-        if (__ballot(!done) == 0ull) break;  // every pixel of this quadrant is saturated
+      // One list entry: `hot` was requested an entry earlier. A wavefront walks its list alone, so everything that
+      // waits -- the LDS round trip for a surfel's record, chains of nested divergent branches -- is paid once per
+      // entry on the tile's critical path (the launch lasts as long as its longest tile). Hence: the NEXT entry's record
+      // is requested before the current one is evaluated, into alternating registers; the intersection runs without
+      // early exits and yields one predicate; the blend is one divergent region.
+      auto blend_entry = [&](const SplatHot& hot, const SplatCold& cold, int j) {
+#pragma clang fp contract(off)  // two copies of this body exist (alternating registers): both must round alike
+        Hit h;
+        const bool hit = intersect_flat(hot, pxf, pyf, near_n, h) && !done;
+        if (__ballot(hit) == 0ull) return;
+        const float test_T = T * (1.0f - h.alpha);
+        const bool sat     = hit && test_T < 0.0001f;
+        done               = done || sat;
+        if (hit && !sat) {
+          const float w         = h.alpha * T;
+          const int contributor = b * kFwdBatch + j + 1;
+          if (kAux) {
+            const float A  = 1.0f - T;
+            const float m  = far_scale * fmaf(-near_n, __builtin_amdgcn_rcpf(h.depth), 1.0f);
+            const float mm = m * m;
+            dist = fmaf(fmaf(-2.0f * m, M1, fmaf(mm, A, M2)), w, dist);
+            D    = fmaf(h.depth, w, D);
+            M1   = fmaf(m, w, M1);
+            M2   = fmaf(mm, w, M2);
+            if (T > 0.5f) median = h.depth, median_c = contributor;
+            N0 = fmaf(cold.nx, w, N0), N1 = fmaf(cold.ny, w, N1), N2 = fmaf(cold.nz, w, N2);
+            if (kAccum) {
+              if (wmax < w) wmax = w, wmax_id = cold.id, flag = true;
+              if (accum_weights_p) atomicAdd(&accum_weights_p[cold.id], w);
+              if (accum_weights_count) atomicAdd(&accum_weights_count[cold.id], 1);
+            }
+            if (kFlow) {
+              const float* Q = &s_t2[j * 9];
+              const float u2 = fmaf(Q[0], h.sx, fmaf(Q[1], h.sy, Q[2]));
+              const float v2 = fmaf(Q[3], h.sx, fmaf(Q[4], h.sy, Q[5]));
+              float w2       = fmaf(Q[6], h.sx, fmaf(Q[7], h.sy, Q[8]));
+              w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
+              f0 = fmaf(u2 / w2 - pxf, w, f0);
+              f1 = fmaf(v2 / w2 - pyf, w, f1);
+            }
+            wsum += w;
+          }
+          if (kAccum) {
+            if (flag && accum_max_count) atomicAdd(&accum_max_count[wmax_id], 1);
+          }
+          C0 = fmaf(cold.r, w, C0), C1 = fmaf(cold.g, w, C1), C2 = fmaf(cold.b, w, C2);
+          T    = test_T;
+          last = contributor;
+        }
+      };
+      auto pop = [&]() {
         const int j = c * kWave + __builtin_ctzll(todo);
         todo &= todo - 1;
-        const SplatHot hot = hot_next;
-        hot_next           = s_hot[c * kWave + (todo ? __builtin_ctzll(todo) : 0)];
-        const SplatCold cold = s_cold[j];  // needed only if a pixel blends the surfel, but then without waiting
-        __builtin_amdgcn_sched_barrier(0);
-        if (done) continue;
-        Hit h;
-        if (!intersect(hot, pxf, pyf, near_n, h)) continue;
-        const float test_T = T * (1.0f - h.alpha);
-        if (test_T < 0.0001f) {
-          done = true;
-          continue;
+        return j;
+      };
+      auto peek = [&]() { return c * kWave + (todo ? __builtin_ctzll(todo) : 0); };
+      SplatHot hot_a = s_hot[peek()], hot_b;
+      while (todo) {
+        if (__ballot(!done) == 0ull) break;  // every pixel of this quadrant is saturated
+        {
+          const int j = pop();
+          hot_b       = s_hot[peek()];
+          const SplatCold cold = s_cold[j];  // read only if a pixel blends the surfel, but then without waiting
+          __builtin_amdgcn_sched_barrier(0);
+          blend_entry(hot_a, cold, j);
         }
-        const float w        = h.alpha * T;
-        const int contributor = b * kFwdBatch + j + 1;
-        if (kAux) {
-          const float A = 1.0f - T;
-          const float m = far_scale * (1.0f - near_n * __builtin_amdgcn_rcpf(h.depth));
-          dist += (m * m * A + M2 - 2.0f * m * M1) * w;
-          D += h.depth * w;
-          M1 += m * w;
-          M2 += m * m * w;
-          if (T > 0.5f) median = h.depth, median_c = contributor;
-          N0 += cold.nx * w, N1 += cold.ny * w, N2 += cold.nz * w;
-          if (kAccum) {
-            if (wmax < w) wmax = w, wmax_id = cold.id, flag = true;
-            if (accum_weights_p) atomicAdd(&accum_weights_p[cold.id], w);
-            if (accum_weights_count) atomicAdd(&accum_weights_count[cold.id], 1);
-          }
-          if (kFlow) {
-            const float* Q = &s_t2[j * 9];
-            const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
-            const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
-            float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
-            w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
-            f0 += (u2 / w2 - pxf) * w;
-            f1 += (v2 / w2 - pyf) * w;
-          }
-          wsum += w;
+        if (todo == 0ull || __ballot(!done) == 0ull) break;
+        {
+          const int j = pop();
+          hot_a       = s_hot[peek()];
+          const SplatCold cold = s_cold[j];
+          __builtin_amdgcn_sched_barrier(0);
+          blend_entry(hot_b, cold, j);
         }
-        if (kAccum) {
-          if (flag && accum_max_count) atomicAdd(&accum_max_count[wmax_id], 1);
-        }
-        C0 += cold.r * w, C1 += cold.g * w, C2 += cold.b * w;
-        T    = test_T;
-        last = contributor;
       }
     }
   }
