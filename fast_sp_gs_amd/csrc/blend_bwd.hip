@@ -176,7 +176,7 @@ blend_backward_kernel(
       todo &= todo - 1;
       const int pos = n_todo - 1 - (b * kBwdBatch + j);  // 0-based position in the tile's list
       Hit h;
-      const bool hit = (pos < last_contrib) && intersect(s_hot[j], pxf, pyf, near_n, h);
+      const bool hit = intersect_flat(s_hot[j], pxf, pyf, near_n, h) && (pos < last_contrib);
       if (__ballot(hit) == 0ull) continue;  // wave-uniform: nobody in this quadrant blends the surfel
 
       float g[16], g2x = 0.0f, g2y = 0.0f;
