@@ -171,21 +171,17 @@ blend_backward_kernel(
      const int jj = chunk * kWave + lane;
      unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u) &&
                                         (n_todo - 1 - (b * kBwdBatch + jj)) < wave_max_contrib);
-     while (todo) {
-      const int j = chunk * kWave + __builtin_ctzll(todo);
-      todo &= todo - 1;
+     auto backward_entry = [&](const SplatHot& hot, const SplatCold& cold, int j) {
       const int pos = n_todo - 1 - (b * kBwdBatch + j);  // 0-based position in the tile's list
       Hit h;
-      const bool hit = intersect_flat(s_hot[j], pxf, pyf, near_n, h) && (pos < last_contrib);
-      if (__ballot(hit) == 0ull) continue;  // wave-uniform: nobody in this quadrant blends the surfel
+      const bool hit = intersect_flat(hot, pxf, pyf, near_n, h) && (pos < last_contrib);
+      if (__ballot(hit) == 0ull) return;  // wave-uniform: nobody in this quadrant blends the surfel
 
       float g[16], g2x = 0.0f, g2y = 0.0f;
       bool filtered = false;
 #pragma unroll
       for (int c = 0; c < 16; ++c) g[c] = 0.0f;
       if (hit) {
-        const SplatHot& hot  = s_hot[j];
-        const SplatCold cold = s_cold[j];
         T             = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
         const float w = h.alpha * T;
         // All channels that enter the image linearly (colour, depth, opacity, normal) share one back-to-front
@@ -263,6 +259,33 @@ blend_backward_kernel(
         const float sx = wave_sum_to_lane63(g2x), sy = wave_sum_to_lane63(g2y);
         if (lane == 63) atomicAdd(&s_acc[j][16], sx), atomicAdd(&s_acc[j][17], sy);
       }
+     };
+     // The record of the next entry is requested before the current one is evaluated (alternating registers): a
+     // wavefront walks its list alone, so an exposed LDS round trip per entry sits on the tile's critical path.
+     if (todo == 0ull) continue;
+     auto pop = [&]() {
+       const int j = chunk * kWave + __builtin_ctzll(todo);
+       todo &= todo - 1;
+       return j;
+     };
+     auto peek = [&]() { return chunk * kWave + (todo ? __builtin_ctzll(todo) : 0); };
+     SplatHot hot_a = s_hot[peek()], hot_b;
+     while (todo) {
+       {
+         const int j = pop();
+         hot_b       = s_hot[peek()];
+         const SplatCold cold = s_cold[j];
+         __builtin_amdgcn_sched_barrier(0);
+         backward_entry(hot_a, cold, j);
+       }
+       if (todo == 0ull) break;
+       {
+         const int j = pop();
+         hot_a       = s_hot[peek()];
+         const SplatCold cold = s_cold[j];
+         __builtin_amdgcn_sched_barrier(0);
+         backward_entry(hot_b, cold, j);
+       }
      }
     }
     __syncthreads();
