@@ -86,6 +86,17 @@ __device__ __forceinline__ bool conic_alpha(const G3Hot& h, float pxf, float pyf
   return !(o.alpha < (1.0f / 255.0f));
 }
 
+// The same without an early exit and with every fused multiply-add written out (contraction off): a kernel that inlines
+// it twice gets the same rounding from both copies.
+__device__ __forceinline__ bool conic_alpha_flat(const G3Hot& h, float pxf, float pyf, G3Hit& o) {
+#pragma clang fp contract(off)
+  o.dx = h.x - pxf, o.dy = h.y - pyf;
+  const float power = fmaf(-0.5f, fmaf(h.a * o.dx, o.dx, h.c * o.dy * o.dy), -(h.b * o.dx * o.dy));
+  o.G     = __expf(power);
+  o.alpha = fminf(0.99f, h.opacity * o.G);
+  return !(power > 0.0f) & !(o.alpha < (1.0f / 255.0f));
+}
+
 template <int E, bool kAccum>
 __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, int W, int H,
     const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
@@ -134,29 +145,54 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
     for (int c = 0; c < kG3Batch / kWave; ++c) {
       const int jj = c * kWave + lane;
       unsigned long long todo = __ballot(jj < n_here && ((s_hot[jj < kG3Batch ? jj : 0].mask >> wave) & 1u));
-      while (todo) {
-        if (__ballot(!done) == 0ull) break;
+      if (todo == 0ull) continue;
+      // One list entry. A wavefront walks its list alone and the launch lasts as long as its longest tile, so the next
+      // entry's record is requested before the current one is evaluated (alternating registers) and the blend is one
+      // divergent region behind one predicate.
+      auto blend_entry = [&](const G3Hot& hot, int j) {
+#pragma clang fp contract(off)  // two copies of this body exist: both must round alike
+        G3Hit h;
+        const bool hit = conic_alpha_flat(hot, pxf, pyf, h) && !done;
+        if (__ballot(hit) == 0ull) return;
+        const float test_T = T * (1.0f - h.alpha);
+        const bool sat     = hit && test_T < 0.0001f;
+        done               = done || sat;
+        if (hit && !sat) {
+          const float w = h.alpha * T;
+#pragma unroll
+          for (int k = 0; k < 3 + E; ++k) C[k] = fmaf(s_feat[j][k], w, C[k]);
+          if (kAccum) {
+            const int id = hot.id;
+            if (wmax < w) wmax = w, wmax_id = id, flag = true;
+            if (accum_weights_p) atomicAdd(&accum_weights_p[id], w);
+            if (accum_weights_count) atomicAdd(&accum_weights_count[id], 1);
+          }
+          T    = test_T;
+          last = b * kG3Batch + j + 1;
+        }
+      };
+      auto pop = [&]() {
         const int j = c * kWave + __builtin_ctzll(todo);
         todo &= todo - 1;
-        if (done) continue;
-        G3Hit h;
-        if (!conic_alpha(s_hot[j], pxf, pyf, h)) continue;
-        const float test_T = T * (1.0f - h.alpha);
-        if (test_T < 0.0001f) {
-          done = true;
-          continue;
+        return j;
+      };
+      auto peek = [&]() { return c * kWave + (todo ? __builtin_ctzll(todo) : 0); };
+      G3Hot hot_a = s_hot[peek()], hot_b;
+      while (todo) {
+        if (__ballot(!done) == 0ull) break;
+        {
+          const int j = pop();
+          hot_b       = s_hot[peek()];
+          __builtin_amdgcn_sched_barrier(0);
+          blend_entry(hot_a, j);
         }
-        const float w = h.alpha * T;
-#pragma unroll
-        for (int k = 0; k < 3 + E; ++k) C[k] += s_feat[j][k] * w;
-        if (kAccum) {
-          const int id = s_hot[j].id;
-          if (wmax < w) wmax = w, wmax_id = id, flag = true;
-          if (accum_weights_p) atomicAdd(&accum_weights_p[id], w);
-          if (accum_weights_count) atomicAdd(&accum_weights_count[id], 1);
+        if (todo == 0ull || __ballot(!done) == 0ull) break;
+        {
+          const int j = pop();
+          hot_a       = s_hot[peek()];
+          __builtin_amdgcn_sched_barrier(0);
+          blend_entry(hot_b, j);
         }
-        T    = test_T;
-        last = b * kG3Batch + j + 1;
       }
     }
   }
@@ -242,7 +278,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
       todo &= todo - 1;
       const int pos = n_todo - 1 - (b * kB + j);  // 0-based position in the tile's list
       G3Hit h;
-      const bool hit = (pos < last_contrib) && conic_alpha(s_hot[j], pxf, pyf, h);
+      const bool hit = conic_alpha_flat(s_hot[j], pxf, pyf, h) && (pos < last_contrib);
       if (__ballot(hit) == 0ull) continue;
       float g[16];
 #pragma unroll
