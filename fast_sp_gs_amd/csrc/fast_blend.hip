@@ -67,11 +67,13 @@ struct FastHit {
 };
 
 // gs_2d_fast_redner.cu:150-186. Returns false when the reference would `continue`.
-__device__ __forceinline__ bool fast_intersect(const FastHot& h, float pxf, float pyf, float near_n, FastHit& o) {
+// Written without early exits: every lane runs the whole sequence and the rejections (behind the camera plane, nearer
+// than `near`, positive exponent, alpha < 1/255) are combined into one predicate at the end, so the callers have one
+// divergent region instead of a nest of them on their per-entry critical path.
+__device__ __forceinline__ bool fast_intersect_flat(const FastHot& h, float pxf, float pyf, float near_n, FastHit& o) {
   const float p0 = h.a[0] * pxf + h.a[1] * pyf + h.a[2];
   const float p1 = h.a[3] * pxf + h.a[4] * pyf + h.a[5];
   o.pz           = h.a[6] * pxf + h.a[7] * pyf + h.a[8];
-  if (o.pz == 0.0f) return false;
   const float rz = __builtin_amdgcn_rcpf(o.pz);
   o.sx = p0 * rz, o.sy = p1 * rz;
   o.rho3d = o.sx * o.sx + o.sy * o.sy;
@@ -79,12 +81,10 @@ __device__ __forceinline__ bool fast_intersect(const FastHot& h, float pxf, floa
   o.rho2d = 2.0f * (o.dx * o.dx + o.dy * o.dy);
   const float rho = fminf(o.rho3d, o.rho2d);
   o.depth = (o.sx * h.tw0 + o.sy * h.tw1) + h.tw2;
-  if (o.depth < near_n) return false;
   const float power = -0.5f * rho;
-  if (power > 0.0f) return false;
   o.G     = __expf(power);
   o.alpha = fminf(0.99f, h.opacity * o.G);
-  return !(o.alpha < (1.0f / 255.0f));
+  return (o.pz != 0.0f) & !(o.depth < near_n) & !(power > 0.0f) & !(o.alpha < (1.0f / 255.0f));
 }
 
 // Sums 8 per-lane values over the 64 lanes at once: three merge steps inside aligned groups of 8 lanes, one rotate by 8
@@ -206,14 +206,13 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
           if (__ballot(!done) == 0ull) break;
           const int j = c * kWave + __builtin_ctzll(todo);
           todo &= todo - 1;
-          if (done) continue;
           FastHit h;
-          if (!fast_intersect(s_hot[j], pxf, pyf, near_n, h)) continue;
+          const bool hit = fast_intersect_flat(s_hot[j], pxf, pyf, near_n, h) && !done;
+          if (__ballot(hit) == 0ull) continue;
           const float test_T = T * (1.0f - h.alpha);
-          if (test_T < 0.0001f) {
-            done = true;
-            continue;
-          }
+          const bool sat     = hit && test_T < 0.0001f;
+          done               = done || sat;
+          if (!hit || sat) continue;
           const float w         = h.alpha * T;
           const SplatCold cold  = s_cold[j];
           const int contributor = b * kBatch + j + 1;
@@ -371,7 +370,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
         todo &= todo - 1;
         const int pos = n_todo - 1 - (b * kBatch + j);
         FastHit h;
-        const bool hit = (pos < last_contrib) && fast_intersect(s_hot[j], pxf, pyf, near_n, h);
+        const bool hit = fast_intersect_flat(s_hot[j], pxf, pyf, near_n, h) && (pos < last_contrib);
         if (__ballot(hit) == 0ull) continue;
 
         float g[16], g8[8];

@@ -77,17 +77,9 @@ struct G3Hit {
   float dx, dy, G, alpha;
 };
 
-__device__ __forceinline__ bool conic_alpha(const G3Hot& h, float pxf, float pyf, G3Hit& o) {
-  o.dx = h.x - pxf, o.dy = h.y - pyf;
-  const float power = -0.5f * (h.a * o.dx * o.dx + h.c * o.dy * o.dy) - h.b * o.dx * o.dy;
-  if (power > 0.0f) return false;
-  o.G     = __expf(power);
-  o.alpha = fminf(0.99f, h.opacity * o.G);
-  return !(o.alpha < (1.0f / 255.0f));
-}
-
-// The same without an early exit and with every fused multiply-add written out (contraction off): a kernel that inlines
-// it twice gets the same rounding from both copies.
+// Alpha of one Gaussian at one pixel (gaussian_render.cu:118-130); false where the reference would `continue`. No early
+// exit, and every fused multiply-add is written out with contraction off: a kernel that inlines this twice gets the
+// same rounding from both copies.
 __device__ __forceinline__ bool conic_alpha_flat(const G3Hot& h, float pxf, float pyf, G3Hit& o) {
 #pragma clang fp contract(off)
   o.dx = h.x - pxf, o.dy = h.y - pyf;
