@@ -395,6 +395,51 @@ def density_control_ms(dev, scene, reps: int = 5):
     return out
 
 
+def large_scene_ms(dev, views: int = 4, reps: int = 3):
+    """BASELINE config 4: 3M surfels, a batch of 4 views at 1352x1014 rendered forward + backward one after the other,
+    and the K-NN of the 3M centres against 2048 control points with k = 8."""
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd._C import get_C_function
+    from fast_sp_gs_amd.renderer import render_step
+    scene_h, cams = scenes.config4()
+    scene = scene_h.to(dev)
+    bg = torch.ones(3, device=dev)
+    g = torch.Generator().manual_seed(9)
+    cams = [c.to(dev) for c in cams[:views]]
+    gi = torch.randn(3, cams[0].H, cams[0].W, generator=g).to(dev)
+    ge = torch.cat([torch.randn(6, cams[0].H, cams[0].W, generator=g), torch.zeros(3, cams[0].H, cams[0].W)]).to(dev)
+
+    def batch():
+        for cam in cams:
+            out = render_step(scene, cam, gi, ge, None, background=bg)
+        return out
+
+    out = batch()
+    torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        batch()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / reps
+    gc.enable()
+    knn = get_C_function('knn_topk')
+    ctrl = (torch.randn(2048, 3, generator=g) * 2).to(dev)
+    knn(scene.means3D, ctrl, 8)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(3):
+        knn(scene.means3D, ctrl, 8)
+    torch.cuda.synchronize()
+    knn_ms = (time.perf_counter() - t0) / 3 * 1e3
+    return {"large_scene_batch_ms": dt * 1e3, "large_scene_views_per_s": views / dt,
+            "large_scene_knn_ms": knn_ms, "large_scene_knn_queries_per_s": scene.P / (knn_ms * 1e-3),
+            "large_scene_workload": f"{scene.P} surfels, {views} views {cams[0].W}x{cams[0].H} forward + backward in "
+                                    f"sequence (R = {out['point_list'].numel()} instances in the last view); K-NN "
+                                    f"{scene.P} x 2048, k = 8"}
+
+
 def ssim_rate(dev, reps: int = 20):
     """Fused SSIM forward (with the partial-derivative maps) + backward on one 3 x 800 x 800 image pair."""
     from fast_sp_gs_amd._C import get_C_function
@@ -537,6 +582,7 @@ def main():
         extra.update(reference_note_blend_ms(dev))
         extra.update(gs3d_path_rate(dev, scene, cam, gi))
         extra.update(density_control_ms(dev, scene))
+        extra.update(large_scene_ms(dev))
         extra["fast_path_frames_per_s"] = fast_path_rate(dev, scene, cam, gi)
         extra["fast_path_workload"] = "same scene through GS_2D_fast_* (corner-test binning keeps fewer instances)"
         extra["dynamic_step_frames_per_s"] = dynamic_step_rate(dev)
