@@ -33,6 +33,9 @@ _TILE = 16
 # When set to a list, every operator appends (name, start_event, end_event) recorded on the current stream tightly
 # around its C-ABI call (allocation and zero-fill of outputs stay outside), so callers can time the kernels themselves.
 STAGE_EVENTS = None
+# Optional set of operator names: when set, only these are timed. An event is a packet of its own in the device queue
+# and costs a few microseconds between two kernels, so a caller that times a whole region brackets only what it needs.
+STAGE_FILTER = None
 # Events to use for that (already created and recorded once by the caller): creating timing events is not free -- the
 # runtime grows its event pool in bursts of tens of milliseconds -- so a caller that times a region fills this first.
 EVENT_POOL: list = []
@@ -49,12 +52,13 @@ class _timed:
         self.name = name
 
     def __enter__(self):
-        if STAGE_EVENTS is not None:
+        self.start = None
+        if STAGE_EVENTS is not None and (STAGE_FILTER is None or self.name in STAGE_FILTER):
             self.start = _event()
             self.start.record()
 
     def __exit__(self, *exc):
-        if STAGE_EVENTS is not None:
+        if self.start is not None and STAGE_EVENTS is not None:
             end = _event()
             end.record()
             STAGE_EVENTS.append((self.name, self.start, end))
@@ -224,9 +228,11 @@ def gs_2d_compute_trans_mat_backward(W, H, means3D, scales, rotations, Tw2v, Tw2
 
 # --------------------------------------------------------------------------------------------------------------------
 def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, tiles_touched: Tensor,
-               debug: bool = False, return_keys: bool = False, return_offsets: bool = False) -> List[Tensor]:
+               debug: bool = False, return_keys: bool = False, return_offsets: bool = False,
+               overlap=None) -> List[Tensor]:
     """gaussian_prepare.cu:282-308 -> [ranges[T,2] int64, point_list[R] int32] (+ sorted keys, + the prefix scan of
-    tiles_touched, which GS_2D_render_backward can use to sum gradients without atomics)."""
+    tiles_touched, which GS_2D_render_backward can use to sum gradients without atomics). `overlap(offsets)`, if given,
+    is called once the scan is queued and before the host waits for the instance count; its result is appended."""
     what = 'GS_prepare'
     _f32(what, means2D=means2D, depths=depths)
     L.require_cuda(what, radii=radii, tiles_touched=tiles_touched)
@@ -240,18 +246,28 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
     ranges = torch.empty((T, 2), dtype=torch.int64, device=dev)
     offsets = torch.empty((max(P, 1),), dtype=torch.int64, device=dev)
     ws1 = _workspace(lib.fsgs_gs_prepare_scan_workspace_bytes(P), dev)
+    large_count = torch.empty((1,), dtype=torch.int32, device=dev)
     count = _pinned_count()
+    # The host has to learn the instance count before it can size point_list. Everything that does not depend on it is
+    # queued behind the count's copy first -- the per-tile counting, and whatever the caller hands in as `overlap` -- so
+    # the device works while the host waits for the copy and allocates.
     with _timed('gs_prepare_scan'):
-        rc = lib.fsgs_gs_prepare_scan(P, L.ptr(tiles_touched), L.ptr(offsets), L.ptr(ws1), ws1.numel(),
-                                      count.data_ptr(), stream)
+        rc = lib.fsgs_gs_prepare_scan_begin(P, L.ptr(tiles_touched), L.ptr(offsets), L.ptr(ws1), ws1.numel(),
+                                            count.data_ptr(), stream)
     L.check(rc, what)
+    with _timed('gs_prepare_fill'):  # first of the operator's two parts: callers that time stages add them up
+        rc = lib.fsgs_gs_prepare_count(P, W, H, L.ptr(means2D), L.ptr(radii), L.ptr(ranges), L.ptr(large_count), stream)
+    L.check(rc, what)
+    overlapped = overlap(offsets) if overlap is not None else None
+    L.check(lib.fsgs_gs_prepare_scan_end(), what)
     R = ctypes.c_int64.from_address(count.data_ptr()).value
     point_list = torch.empty((R,), dtype=torch.int32, device=dev)
     keys = torch.empty((R,), dtype=torch.int64, device=dev) if return_keys else None
     ws2 = _workspace(lib.fsgs_gs_prepare_fill_workspace_bytes(R), dev)
     with _timed('gs_prepare_fill'):
-        rc = lib.fsgs_gs_prepare_fill(P, W, H, L.ptr(means2D), L.ptr(depths), L.ptr(radii), L.ptr(offsets), R,
-                                      L.ptr(ranges), L.ptr(point_list), L.ptr(keys), L.ptr(ws2), ws2.numel(), stream)
+        rc = lib.fsgs_gs_prepare_fill_counted(P, W, H, L.ptr(means2D), L.ptr(depths), L.ptr(radii), R, L.ptr(ranges),
+                                              L.ptr(point_list), L.ptr(keys), L.ptr(large_count), L.ptr(ws2),
+                                              ws2.numel(), stream)
     L.check(rc, what)
     if debug:
         torch.cuda.synchronize()
@@ -260,6 +276,8 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
         out.append(keys)
     if return_offsets:
         out.append(offsets)
+    if overlap is not None:
+        out.append(overlapped)
     return out
 
 

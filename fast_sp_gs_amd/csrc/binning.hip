@@ -699,28 +699,62 @@ FSGS_API size_t fsgs_gs_prepare_scan_workspace_bytes(int P) {
   return align_up((size_t) div_up(P > 0 ? P : 1, kScanChunk) * 8, 256);
 }
 
-FSGS_API int fsgs_gs_prepare_scan(int P, const int32_t* tiles_touched, int64_t* point_offsets, void* workspace,
-                                  size_t workspace_bytes, int64_t* num_rendered_host, void* stream) {
+namespace {
+// One event per host thread marks "the instance count has been copied": waiting on it instead of on the stream lets the
+// caller queue work that does not depend on the count behind the copy.
+hipEvent_t count_event() {
+  static thread_local hipEvent_t ev = nullptr;
+  if (!ev && hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) ev = nullptr;
+  return ev;
+}
+thread_local bool t_count_pending = false;  // a scan_begin of this thread has queued a copy nobody has waited for
+}  // namespace
+
+FSGS_API int fsgs_gs_prepare_scan_begin(int P, const int32_t* tiles_touched, int64_t* point_offsets, void* workspace,
+                                        size_t workspace_bytes, int64_t* num_rendered_host, void* stream) {
   FSGS_REQUIRE(P >= 0 && num_rendered_host, "gs_prepare_scan: bad arguments");
   *num_rendered_host = 0;
-  if (P == 0) return kOk;
-  FSGS_REQUIRE(tiles_touched && point_offsets && workspace, "gs_prepare_scan: null pointer");
-  if (workspace_bytes < fsgs_gs_prepare_scan_workspace_bytes(P))
-    return fail(kWorkspaceSmall, "gs_prepare_scan: workspace %zu < %zu bytes", workspace_bytes,
-                fsgs_gs_prepare_scan_workspace_bytes(P));
-  hipStream_t s     = (hipStream_t) stream;
-  const int nb      = div_up(P, kScanChunk);
-  int64_t* blk_sums = (int64_t*) workspace;
-  hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(kScanThreads), 0, s, P, tiles_touched, blk_sums);
-  hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanThreads), 0, s, nb, blk_sums);
-  hipLaunchKernelGGL(scan_apply_kernel, dim3(nb), dim3(kScanThreads), 0, s, P, tiles_touched, blk_sums,
-                     point_offsets);
-  if (int rc = check_launch("gs_prepare_scan")) return rc;
-  // The number of (surfel, tile) instances sizes the caller's output, so it has to reach the host here
-  // (the reference blocks in the same place, gaussian_prepare.cu:238-239).
-  FSGS_HIP(hipMemcpyAsync(num_rendered_host, point_offsets + (P - 1), sizeof(int64_t), hipMemcpyDeviceToHost, s));
-  FSGS_HIP(hipStreamSynchronize(s));
+  t_count_pending    = false;
+  if (P == 0) return kOk;  // nothing is queued, nothing to wait for
+  hipStream_t s = (hipStream_t) stream;
+  hipEvent_t ev = count_event();
+  FSGS_REQUIRE(ev != nullptr, "gs_prepare_scan: cannot create an event");
+  {
+    FSGS_REQUIRE(tiles_touched && point_offsets && workspace, "gs_prepare_scan: null pointer");
+    if (workspace_bytes < fsgs_gs_prepare_scan_workspace_bytes(P))
+      return fail(kWorkspaceSmall, "gs_prepare_scan: workspace %zu < %zu bytes", workspace_bytes,
+                  fsgs_gs_prepare_scan_workspace_bytes(P));
+    const int nb      = div_up(P, kScanChunk);
+    int64_t* blk_sums = (int64_t*) workspace;
+    hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(kScanThreads), 0, s, P, tiles_touched, blk_sums);
+    hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanThreads), 0, s, nb, blk_sums);
+    hipLaunchKernelGGL(scan_apply_kernel, dim3(nb), dim3(kScanThreads), 0, s, P, tiles_touched, blk_sums,
+                       point_offsets);
+    if (int rc = check_launch("gs_prepare_scan")) return rc;
+    // The number of (surfel, tile) instances sizes the caller's output, so it has to reach the host
+    // (the reference blocks for it, gaussian_prepare.cu:238-239).
+    FSGS_HIP(hipMemcpyAsync(num_rendered_host, point_offsets + (P - 1), sizeof(int64_t), hipMemcpyDeviceToHost, s));
+  }
+  FSGS_HIP(hipEventRecord(ev, s));
+  t_count_pending = true;
   return kOk;
+}
+
+FSGS_API int fsgs_gs_prepare_scan_end(void) {
+  if (!t_count_pending) return kOk;
+  t_count_pending = false;
+  hipEvent_t ev   = count_event();
+  FSGS_REQUIRE(ev != nullptr, "gs_prepare_scan: cannot create an event");
+  FSGS_HIP(hipEventSynchronize(ev));
+  return kOk;
+}
+
+FSGS_API int fsgs_gs_prepare_scan(int P, const int32_t* tiles_touched, int64_t* point_offsets, void* workspace,
+                                  size_t workspace_bytes, int64_t* num_rendered_host, void* stream) {
+  if (int rc = fsgs_gs_prepare_scan_begin(P, tiles_touched, point_offsets, workspace, workspace_bytes,
+                                          num_rendered_host, stream))
+    return rc;
+  return fsgs_gs_prepare_scan_end();
 }
 
 FSGS_API size_t fsgs_gs_prepare_fill_workspace_bytes(int64_t R) { return sort_layout(R).bytes; }
@@ -730,6 +764,80 @@ FSGS_API int fsgs_gs_prepare_sort_bits(int W, int H) {
   return 32 + (int) higher_msb((uint32_t) (gx * gy));
 }
 
+namespace {
+// First part of the bucket binning, independent of the instance count: zero the ranges, count the instances of every
+// tile into ranges[t].y, scan them to ranges[t] = (start, start); *large_count is reset.
+int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, int64_t* ranges, int* large_count,
+               hipStream_t s) {
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const int T  = gx * gy;
+  hipLaunchKernelGGL(fill_zero_i64_kernel, dim3(div_up(2 * (int64_t) T, 256)), dim3(256), 0, s, 2 * (int64_t) T,
+                     ranges);
+  unsigned long long* rng = (unsigned long long*) ranges;
+  if (P > 0) {
+    // the LDS-aggregated traversal needs one LDS counter per tile; larger tile grids count straight in global memory
+    const bool lds_path = T <= kMaxLdsTiles;
+    const int per_block = std::max(FSGS_EMIT_PER_BLOCK, div_up(P, 256));
+    if (lds_path)
+      hipLaunchKernelGGL(tile_emit_lds_kernel<false>, dim3(div_up(P, per_block)), dim3(1024), 0, s, P, per_block, gx, gy,
+                         (int64_t) 0, (const float2*) means2D, (const float*) nullptr, radii, rng, (uint64_t*) nullptr);
+    else
+      hipLaunchKernelGGL(tile_emit_kernel<false>, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, (int64_t) 0,
+                         (const float2*) means2D, (const float*) nullptr, radii, rng, (uint64_t*) nullptr);
+  }
+  hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, large_count);
+  return check_launch("gs_prepare_count");
+}
+
+// Second part: scatter (depth bits << 32 | surfel) into the tile segments and sort every segment.
+int fill_sort(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii, int64_t R,
+              int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out, void* workspace, int* large_count,
+              hipStream_t s) {
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const int T  = gx * gy;
+  unsigned long long* rng = (unsigned long long*) ranges;
+  uint64_t* entries       = sort_keys_in(R, workspace);
+  const bool lds_path = T <= kMaxLdsTiles;
+  const int per_block = std::max(FSGS_EMIT_PER_BLOCK, div_up(P, 256));
+  // queue of long segments: at most R / kSmallSegment tiles, kept behind the entries in the workspace (its first
+  // word is where fsgs_gs_prepare_fill keeps the queue's counter)
+  int* large_list = (int*) ((char*) workspace + sort_layout(R).keys1) + 1;
+  if (lds_path)
+    hipLaunchKernelGGL(tile_emit_lds_kernel<true>, dim3(div_up(P, per_block)), dim3(1024), 0, s, P, per_block, gx, gy, R,
+                       (const float2*) means2D, depths, radii, rng, entries);
+  else
+    hipLaunchKernelGGL(tile_emit_kernel<true>, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
+                       (const float2*) means2D, depths, radii, rng, entries);
+  hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
+                     large_count, large_list);
+  hipLaunchKernelGGL(tile_sort_large_kernel, dim3(64), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,
+                     large_count, large_list);
+  return check_launch("gs_prepare_fill");
+}
+}  // namespace
+
+FSGS_API int fsgs_gs_prepare_count(int P, int W, int H, const float* means2D, const int32_t* radii, int64_t* ranges,
+                                   int32_t* large_count, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && ranges && large_count, "gs_prepare_count: bad arguments");
+  FSGS_REQUIRE(P == 0 || (means2D && radii), "gs_prepare_count: null pointer");
+  return fill_count(P, W, H, means2D, radii, ranges, large_count, (hipStream_t) stream);
+}
+
+FSGS_API int fsgs_gs_prepare_fill_counted(int P, int W, int H, const float* means2D, const float* depths,
+                                          const int32_t* radii, int64_t R, int64_t* ranges, int32_t* point_list,
+                                          int64_t* sorted_keys_out, int32_t* large_count, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && R >= 0 && ranges && large_count, "gs_prepare_fill: bad arguments");
+  FSGS_REQUIRE(R < (int64_t) 0x7fffffff, "gs_prepare_fill: %lld instances exceed the 2^31-1 limit", (long long) R);
+  if (R == 0 || P == 0) return kOk;  // the counting part left every range at (0, 0)
+  FSGS_REQUIRE(means2D && depths && radii && point_list && workspace, "gs_prepare_fill: null pointer");
+  if (workspace_bytes < sort_workspace_bytes(R))
+    return fail(kWorkspaceSmall, "gs_prepare_fill: workspace %zu < %zu bytes", workspace_bytes,
+                sort_workspace_bytes(R));
+  return fill_sort(P, W, H, means2D, depths, radii, R, ranges, point_list, sorted_keys_out, workspace, large_count,
+                   (hipStream_t) stream);
+}
+
 FSGS_API int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths,
                                   const int32_t* radii, const int64_t* point_offsets, int64_t R, int64_t* ranges,
                                   int32_t* point_list, int64_t* sorted_keys_out, void* workspace,
@@ -737,43 +845,19 @@ FSGS_API int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, con
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && R >= 0 && ranges, "gs_prepare_fill: bad arguments");
   FSGS_REQUIRE(R < (int64_t) 0x7fffffff, "gs_prepare_fill: %lld instances exceed the 2^31-1 limit", (long long) R);
   hipStream_t s = (hipStream_t) stream;
-  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
-  const int T  = gx * gy;
-  hipLaunchKernelGGL(fill_zero_i64_kernel, dim3(div_up(2 * (int64_t) T, 256)), dim3(256), 0, s, 2 * (int64_t) T,
-                     ranges);
-  if (R == 0 || P == 0) return check_launch("gs_prepare_fill(zero)");
+  if (R == 0 || P == 0) {
+    const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+    hipLaunchKernelGGL(fill_zero_i64_kernel, dim3(div_up(2 * (int64_t) gx * gy, 256)), dim3(256), 0, s,
+                       2 * (int64_t) gx * gy, ranges);
+    return check_launch("gs_prepare_fill(zero)");
+  }
   FSGS_REQUIRE(means2D && depths && radii && point_offsets && point_list && workspace,
                "gs_prepare_fill: null pointer");
   if (workspace_bytes < sort_workspace_bytes(R))
     return fail(kWorkspaceSmall, "gs_prepare_fill: workspace %zu < %zu bytes", workspace_bytes,
                 sort_workspace_bytes(R));
-  // ranges was zeroed above; it doubles as the per-tile counter / cursor array of the bucket sort
-  unsigned long long* rng = (unsigned long long*) ranges;
-  uint64_t* entries       = sort_keys_in(R, workspace);
-  // the LDS-aggregated traversal needs one LDS counter per tile; larger tile grids count straight in global memory
-  const bool lds_path = T <= kMaxLdsTiles;
-  const int per_block = std::max(FSGS_EMIT_PER_BLOCK, div_up(P, 256));
-  const dim3 lgrid(div_up(P, per_block)), lblock(1024);
-  const dim3 pgrid(div_up(P, 256)), pblock(256);
-  if (lds_path)
-    hipLaunchKernelGGL(tile_emit_lds_kernel<false>, lgrid, lblock, 0, s, P, per_block, gx, gy, R,
-                       (const float2*) means2D, depths, radii, rng, entries);
-  else
-    hipLaunchKernelGGL(tile_emit_kernel<false>, pgrid, pblock, 0, s, P, gx, gy, R, (const float2*) means2D, depths,
-                       radii, rng, entries);
-  // queue of long segments: at most R / kSmallSegment tiles, kept behind the entries in the workspace
+  // the counter of long segments sits in front of their list, behind the entries in the workspace
   int* large_count = (int*) ((char*) workspace + sort_layout(R).keys1);
-  int* large_list  = large_count + 1;
-  hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, large_count);
-  if (lds_path)
-    hipLaunchKernelGGL(tile_emit_lds_kernel<true>, lgrid, lblock, 0, s, P, per_block, gx, gy, R,
-                       (const float2*) means2D, depths, radii, rng, entries);
-  else
-    hipLaunchKernelGGL(tile_emit_kernel<true>, pgrid, pblock, 0, s, P, gx, gy, R, (const float2*) means2D, depths,
-                       radii, rng, entries);
-  hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
-                     large_count, large_list);
-  hipLaunchKernelGGL(tile_sort_large_kernel, dim3(64), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,
-                     large_count, large_list);
-  return check_launch("gs_prepare_fill");
+  if (int rc = fill_count(P, W, H, means2D, radii, ranges, large_count, s)) return rc;
+  return fill_sort(P, W, H, means2D, depths, radii, R, ranges, point_list, sorted_keys_out, workspace, large_count, s);
 }

@@ -70,9 +70,10 @@ class _GS_2D_Render(torch.autograd.Function):
         means2D, colors, trans_mat, normal_opacity, depths, radii, tiles_touched = _GS_2D_Render._preprocess_forward(
             W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c,
             campos, trans_precomp, means2D, culling)
-        tile_range, point_list, point_offsets = GS_prepare(W, H, means2D, depths, radii, tiles_touched, False,
-                                                           return_offsets=True)
-        records = _GS_2D_Render._pack_records(means2D, colors, normal_opacity, trans_mat, radii, point_offsets)
+        # the packed records need the scan but not the instance count: they are built while the host waits for it
+        tile_range, point_list, point_offsets, records = GS_prepare(
+            W, H, means2D, depths, radii, tiles_touched, False, return_offsets=True,
+            overlap=lambda off: _GS_2D_Render._pack_records(means2D, colors, normal_opacity, trans_mat, radii, off))
         pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib = _GS_2D_Render._render_forward(
             W, H, means2D, colors, normal_opacity, trans_mat, point_list, tile_range, near_n, far_n, only_image,
             transe_mat_t2, accum_max_count, accum_weights_p, accum_weights_count, records)
@@ -219,8 +220,10 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
     m2, colors, tm, no, depths, radii, tt = f('gs_2d_preprocess_forward')(
         W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs, None,
         cam.Tw2v, cam.Tv2c, cam.campos, None, None, None)
-    ranges, point_list, offsets = f('GS_prepare')(W, H, m2, depths, radii, tt, False, return_offsets=True)
-    rec = f('gs_2d_pack_records')(m2, colors, no, tm, radii, offsets) if packed else None
+    # the packed records need the scan but not the instance count: they are built while the host waits for it
+    ranges, point_list, offsets, rec = f('GS_prepare')(
+        W, H, m2, depths, radii, tt, False, return_offsets=True,
+        overlap=lambda off: f('gs_2d_pack_records')(m2, colors, no, tm, radii, off) if packed else None)
     oc, oo, oe, of, nc = f('GS_2D_render_forward')(W, H, m2, colors, no, tm, point_list, ranges, cam.near, cam.far,
                                                    False, None, None, None, None, rec)
     epilogue = {}

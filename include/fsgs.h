@@ -81,6 +81,23 @@ int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, const float*
                          const int64_t* point_offsets, int64_t R, int64_t* ranges, int32_t* point_list,
                          int64_t* sorted_keys_out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same two phases cut where the host has to wait, for callers that want the device to stay busy meanwhile (no
+ * counterpart in the reference, which blocks inside GS_prepare). fsgs_gs_prepare_scan_begin queues the scan and the
+ * copy of the instance count into *num_rendered_host (page-locked memory, or the copy is not asynchronous) and
+ * returns; fsgs_gs_prepare_scan_end blocks the calling host thread until that copy has landed (one scan in flight per
+ * host thread). Work queued on the stream in between runs while the host waits and allocates: fsgs_gs_prepare_count is
+ * the part of the fill that does not need the count (zeroes ranges[T,2], counts the instances per tile, scans them,
+ * resets *large_count, a device int32 the caller keeps until the fill has run); fsgs_gs_prepare_fill_counted is the rest
+ * (scatter + per-tile sort). scan_begin + scan_end == fsgs_gs_prepare_scan, count + fill_counted == fsgs_gs_prepare_fill. */
+int fsgs_gs_prepare_scan_begin(int P, const int32_t* tiles_touched, int64_t* point_offsets, void* workspace,
+                               size_t workspace_bytes, int64_t* num_rendered_host, void* stream);
+int fsgs_gs_prepare_scan_end(void);
+int fsgs_gs_prepare_count(int P, int W, int H, const float* means2D, const int32_t* radii, int64_t* ranges,
+                          int32_t* large_count, void* stream);
+int fsgs_gs_prepare_fill_counted(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
+                                 int64_t R, int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out,
+                                 int32_t* large_count, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- per-tile alpha blend ------------------------------------------------------------------------------------- */
 
 /* Optional accelerator without a counterpart in the reference: packs what the blend kernels gather per surfel
