@@ -56,3 +56,41 @@ def test_binning_bit_exact(name, device, oracle_mod):
     assert np.array_equal(npy(pl), r_pl)
     assert np.array_equal(npy(keys), r_keys)
     assert np.array_equal(npy(offsets)[:P], np.cumsum(npy(tt).astype(np.int64)))
+
+
+def test_blocking_entry_points_match_the_operator(device):
+    """`GS_prepare` runs the binning cut where the host waits (scan_begin / count / scan_end / fill_counted); the blocking
+    pair fsgs_gs_prepare_scan + fsgs_gs_prepare_fill, called straight through the C ABI, must give the same lists, and
+    the `overlap` hook must see the finished scan."""
+    import ctypes
+    from fast_sp_gs_amd import lib as L, scenes
+    from fast_sp_gs_amd._C import get_C_function
+    P, W, H = 20_000, 320, 200
+    scene, _ = scenes.config0(P=P, size=W, seed=5)
+    cam = scenes.pinhole(W, H, 50.0, torch.tensor([0., 0., 4.]))
+    d = lambda t: t.to(device).contiguous()
+    print(f"[binning blocking entries] P={P} {W}x{H}", flush=True)
+    m2, colors, tm, no, dep, radii, tt = get_C_function('gs_2d_preprocess_forward')(
+        W, H, 3, False, d(scene.means3D), d(scene.scales), d(scene.rotations), d(scene.opacities), d(scene.shs), None,
+        d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), None, None, None)
+    seen = {}
+    ranges, pl, offsets, hooked = get_C_function('GS_prepare')(
+        W, H, m2, dep, radii, tt, False, return_offsets=True, overlap=lambda off: seen.setdefault('sum', off[P - 1].clone()))
+    torch.cuda.synchronize()
+    assert int(hooked) == int(tt.sum()) == pl.numel()
+
+    lib = L.load()
+    T = ((W + 15) // 16) * ((H + 15) // 16)
+    stream = L.current_stream()
+    off2 = torch.empty(P, dtype=torch.int64, device=device)
+    ws1 = torch.empty(lib.fsgs_gs_prepare_scan_workspace_bytes(P), dtype=torch.uint8, device=device)
+    R = ctypes.c_int64(-1)
+    L.check(lib.fsgs_gs_prepare_scan(P, L.ptr(tt), L.ptr(off2), L.ptr(ws1), ws1.numel(), ctypes.addressof(R), stream), 'scan')
+    assert R.value == pl.numel() and torch.equal(off2, offsets[:P])
+    ranges2 = torch.empty((T, 2), dtype=torch.int64, device=device)
+    pl2 = torch.empty(R.value, dtype=torch.int32, device=device)
+    ws2 = torch.empty(lib.fsgs_gs_prepare_fill_workspace_bytes(R.value), dtype=torch.uint8, device=device)
+    L.check(lib.fsgs_gs_prepare_fill(P, W, H, L.ptr(m2), L.ptr(dep), L.ptr(radii), L.ptr(off2), R.value, L.ptr(ranges2),
+                                     L.ptr(pl2), None, L.ptr(ws2), ws2.numel(), stream), 'fill')
+    torch.cuda.synchronize()
+    assert torch.equal(ranges2, ranges) and torch.equal(pl2, pl)
