@@ -26,6 +26,7 @@ __all__ = [
     'gs_2d_epilogue_forward', 'gs_2d_epilogue_backward', 'simple_knn', 'gs_preprocess_forward',
     'gs_preprocess_backward', 'gaussian_rasterize_forward', 'gaussian_rasterize_backward', 'select_indices',
     'gather_rows', 'densify_masks', 'prune_mask', 'split_children', 'densification_stats',
+    'gs_compute_cov3D_forward', 'gs_compute_cov3D_backward', 'gs_compute_cov2D_forward', 'gs_compute_cov2D_backward',
 ]
 
 _TILE = 16
@@ -1340,6 +1341,76 @@ def _tan_fov(tanFoV) -> Tuple[float, float]:
         v = tanFoV.detach().cpu().tolist()  # the reference reads it with .item() too (gaussian_preprocess.cu:424-425)
         return float(v[0]), float(v[1])
     return float(tanFoV[0]), float(tanFoV[1])
+
+
+def gs_compute_cov3D_forward(q: Tensor, s: Tensor) -> Tensor:
+    """gaussian_compute_cov3D.cu:122-137: q[..., 4] (x, y, z, w), s[..., 3] -> cov3D[..., 6]."""
+    what = 'gs_compute_cov3D_forward'
+    _f32(what, q=q, s=s)
+    if s.shape[-1] != 3 or tuple(q.shape) != tuple(s.shape[:-1]) + (4,):
+        raise RuntimeError(f'{what}: q.shape[:-1] == s.shape[:-1]')
+    N = s.numel() // 3
+    cov3D = torch.empty(tuple(s.shape[:-1]) + (6,), dtype=torch.float32, device=s.device)
+    with _timed(what):
+        rc = _lib().fsgs_gs_compute_cov3D_forward(N, L.ptr(q), L.ptr(s), L.ptr(cov3D), L.current_stream())
+    L.check(rc, what)
+    return cov3D
+
+
+def gs_compute_cov3D_backward(q: Tensor, s: Tensor, dL_dCov3D: Tensor) -> List[Tensor]:
+    """gaussian_compute_cov3D.cu:151-161 -> [dq, ds]."""
+    what = 'gs_compute_cov3D_backward'
+    dL_dCov3D = dL_dCov3D.contiguous()
+    _f32(what, q=q, s=s, dL_dCov3D=dL_dCov3D)
+    N = s.numel() // 3
+    if dL_dCov3D.numel() != 6 * N or q.numel() != 4 * N:
+        raise RuntimeError(f'{what}: Error shape')
+    dq, ds = torch.empty_like(q), torch.empty_like(s)
+    with _timed(what):
+        rc = _lib().fsgs_gs_compute_cov3D_backward(N, L.ptr(q), L.ptr(s), L.ptr(dL_dCov3D), L.ptr(dq), L.ptr(ds),
+                                                   L.current_stream())
+    L.check(rc, what)
+    return [dq, ds]
+
+
+def gs_compute_cov2D_forward(cov3D: Tensor, mean: Tensor, viewmatrix: Tensor, focal_x: float, focal_y: float,
+                             tan_fovx: float, tan_fovy: float) -> Tensor:
+    """gaussian_compute_cov2D.cu:199-210: cov3D[N,6], mean[N,3], row-major Tw2v[4,4] -> cov2D[N,3]."""
+    what = 'gs_compute_cov2D_forward'
+    _f32(what, cov3D=cov3D, mean=mean, viewmatrix=viewmatrix)
+    N = mean.numel() // 3
+    if cov3D.numel() != 6 * N or viewmatrix.numel() != 16:
+        raise RuntimeError(f'{what}: Error shape')
+    cov2D = torch.empty_like(mean)
+    with _timed(what):
+        rc = _lib().fsgs_gs_compute_cov2D_forward(N, L.ptr(cov3D), L.ptr(mean), L.ptr(viewmatrix), float(focal_x),
+                                                  float(focal_y), float(tan_fovx), float(tan_fovy), L.ptr(cov2D),
+                                                  L.current_stream())
+    L.check(rc, what)
+    return cov2D
+
+
+def gs_compute_cov2D_backward(cov3D: Tensor, mean: Tensor, viewmatrix: Tensor, focal_x: float, focal_y: float,
+                              tan_fovx: float, tan_fovy: float, grad_cov2D: Tensor,
+                              grad_vm: Optional[Tensor] = None) -> List[Tensor]:
+    """gaussian_compute_cov2D.cu:229-248 -> [grad_cov3D, grad_mean]. The optional accumulation into a view-matrix
+    gradient is not supported."""
+    what = 'gs_compute_cov2D_backward'
+    if grad_vm is not None:
+        raise RuntimeError(f'{what}: the gradient to the view matrix is not supported')
+    grad_cov2D = grad_cov2D.contiguous()
+    _f32(what, cov3D=cov3D, mean=mean, viewmatrix=viewmatrix, grad_cov2D=grad_cov2D)
+    N = mean.numel() // 3
+    if cov3D.numel() != 6 * N or viewmatrix.numel() != 16 or grad_cov2D.numel() != 3 * N:
+        raise RuntimeError(f'{what}: Error shape')
+    g_cov3D, g_mean = torch.empty_like(cov3D), torch.empty_like(mean)
+    with _timed(what):
+        rc = _lib().fsgs_gs_compute_cov2D_backward(N, L.ptr(cov3D), L.ptr(mean), L.ptr(viewmatrix), float(focal_x),
+                                                   float(focal_y), float(tan_fovx), float(tan_fovy),
+                                                   L.ptr(grad_cov2D), L.ptr(g_cov3D), L.ptr(g_mean),
+                                                   L.current_stream())
+    L.check(rc, what)
+    return [g_cov3D, g_mean]
 
 
 def gs_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: bool, means3D: Tensor, scales: Tensor,

@@ -125,23 +125,11 @@ __device__ __forceinline__ void cov2d_product(const float* M, const float* c, fl
   out[0] = cov[0], out[1] = cov[1], out[2] = cov[3];
 }
 
-// dL/dconic -> dL/dcov3D (6) and dL/dmean (3); false when the covariance determinant is exactly zero.
-__device__ __forceinline__ bool cov2d_backward(const float* mean, const float* c3, float fx, float fy, float tanx,
-                                               float tany, const float* V, const float* g_conic, float* g_cov3D,
-                                               float* g_mean) {
+// dL/dcov2D = (da, db, dc) (b is the one stored off-diagonal entry) -> dL/dcov3D (6) and dL/dmean (3).
+__device__ __forceinline__ void cov2d_backward_cov(const Cov2DTerms& k, const float* c3, float fx, float fy,
+                                                   const float* V, float da, float db, float dc, float* g_cov3D,
+                                                   float* g_mean) {
 #pragma clang fp contract(off)
-  Cov2DTerms k;
-  cov2d_terms(mean, fx, fy, tanx, tany, V, k);
-  float cov[3];
-  cov2d_product(k.M, c3, cov);
-  const float a = cov[0] + 0.3f, b = cov[1], c = cov[2] + 0.3f;
-  const float denom = a * c - b * b;
-  if (denom == 0.0f) return false;
-  const float denom2inv = 1.0f / ((denom * denom) + 0.0000001f);
-  const float tt = c * g_conic[0] - b * g_conic[1] + a * g_conic[2];
-  const float da = denom2inv * (-c * tt + denom * g_conic[2]);
-  const float dc = denom2inv * (-a * tt + denom * g_conic[0]);
-  const float db = denom2inv * (2.0f * b * tt - denom * g_conic[1]);
   const float* M = k.M;
   g_cov3D[0] = (M[0] * M[0] * da + M[0] * M[3] * db + M[3] * M[3] * dc);
   g_cov3D[3] = (M[1] * M[1] * da + M[1] * M[4] * db + M[4] * M[4] * dc);
@@ -168,6 +156,26 @@ __device__ __forceinline__ bool cov2d_backward(const float* mean, const float* c
       -fx * tz2 * dJ00 - fy * tz2 * dJ11 + (2 * fx * k.t[0]) * tz3 * dJ02 + (2 * fy * k.t[1]) * tz3 * dJ12;
 #pragma unroll
   for (int a2 = 0; a2 < 3; ++a2) g_mean[a2] = V[a2] * dtx + V[4 + a2] * dty + V[8 + a2] * dtz;
+}
+
+// dL/dconic -> dL/dcov3D (6) and dL/dmean (3); false when the covariance determinant is exactly zero.
+__device__ __forceinline__ bool cov2d_backward(const float* mean, const float* c3, float fx, float fy, float tanx,
+                                               float tany, const float* V, const float* g_conic, float* g_cov3D,
+                                               float* g_mean) {
+#pragma clang fp contract(off)
+  Cov2DTerms k;
+  cov2d_terms(mean, fx, fy, tanx, tany, V, k);
+  float cov[3];
+  cov2d_product(k.M, c3, cov);
+  const float a = cov[0] + 0.3f, b = cov[1], c = cov[2] + 0.3f;
+  const float denom = a * c - b * b;
+  if (denom == 0.0f) return false;
+  const float denom2inv = 1.0f / ((denom * denom) + 0.0000001f);
+  const float tt = c * g_conic[0] - b * g_conic[1] + a * g_conic[2];
+  const float da = denom2inv * (-c * tt + denom * g_conic[2]);
+  const float dc = denom2inv * (-a * tt + denom * g_conic[0]);
+  const float db = denom2inv * (2.0f * b * tt - denom * g_conic[1]);
+  cov2d_backward_cov(k, c3, fx, fy, V, da, db, dc, g_cov3D, g_mean);
   return true;
 }
 
@@ -437,10 +445,114 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_backward_kernel(int P, in
   }
 }
 
+// ---- the covariance steps as operators of their own --------------------------------------------------------------
+__global__ void __launch_bounds__(256) cov3d_forward_kernel(int N, const float4* __restrict__ q,
+                                                            const float* __restrict__ s, float* __restrict__ cov3D) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= N) return;
+  const float sc[3] = {s[3 * (size_t) i], s[3 * (size_t) i + 1], s[3 * (size_t) i + 2]};
+  float c[6];
+  cov3d_forward(sc, q[i], c);
+#pragma unroll
+  for (int k = 0; k < 6; ++k) cov3D[6 * (size_t) i + k] = c[k];
+}
+
+__global__ void __launch_bounds__(256) cov3d_backward_kernel(int N, const float4* __restrict__ q,
+    const float* __restrict__ s, const float* __restrict__ g, float4* __restrict__ gq, float* __restrict__ gs) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= N) return;
+  const float sc[3] = {s[3 * (size_t) i], s[3 * (size_t) i + 1], s[3 * (size_t) i + 2]};
+  float gc[6], os[3], oq[4];
+#pragma unroll
+  for (int k = 0; k < 6; ++k) gc[k] = g[6 * (size_t) i + k];
+  cov3d_backward(sc, q[i], gc, os, oq);
+  gq[i] = make_float4(oq[0], oq[1], oq[2], oq[3]);
+#pragma unroll
+  for (int k = 0; k < 3; ++k) gs[3 * (size_t) i + k] = os[k];
+}
+
+__global__ void __launch_bounds__(256) cov2d_forward_kernel(int N, const float* __restrict__ cov3D,
+    const float* __restrict__ mean, const float* __restrict__ Tw2v, float fx, float fy, float tanx, float tany,
+    float* __restrict__ cov2D) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= N) return;
+  float V[16], c3[6], o[3];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) V[k] = Tw2v[k];
+#pragma unroll
+  for (int k = 0; k < 6; ++k) c3[k] = cov3D[6 * (size_t) i + k];
+  const float p[3] = {mean[3 * (size_t) i], mean[3 * (size_t) i + 1], mean[3 * (size_t) i + 2]};
+  Cov2DTerms t;
+  cov2d_terms(p, fx, fy, tanx, tany, V, t);
+  cov2d_product(t.M, c3, o);
+  cov2D[3 * (size_t) i] = o[0] + 0.3f, cov2D[3 * (size_t) i + 1] = o[1], cov2D[3 * (size_t) i + 2] = o[2] + 0.3f;
+}
+
+__global__ void __launch_bounds__(256) cov2d_backward_kernel(int N, const float* __restrict__ cov3D,
+    const float* __restrict__ mean, const float* __restrict__ Tw2v, float fx, float fy, float tanx, float tany,
+    const float* __restrict__ g, float* __restrict__ g_cov3D, float* __restrict__ g_mean) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= N) return;
+  float V[16], c3[6], gc[6], gm[3];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) V[k] = Tw2v[k];
+#pragma unroll
+  for (int k = 0; k < 6; ++k) c3[k] = cov3D[6 * (size_t) i + k];
+  const float p[3] = {mean[3 * (size_t) i], mean[3 * (size_t) i + 1], mean[3 * (size_t) i + 2]};
+  Cov2DTerms t;
+  cov2d_terms(p, fx, fy, tanx, tany, V, t);
+  cov2d_backward_cov(t, c3, fx, fy, V, g[3 * (size_t) i], g[3 * (size_t) i + 1], g[3 * (size_t) i + 2], gc, gm);
+#pragma unroll
+  for (int k = 0; k < 6; ++k) g_cov3D[6 * (size_t) i + k] = gc[k];
+#pragma unroll
+  for (int k = 0; k < 3; ++k) g_mean[3 * (size_t) i + k] = gm[k];
+}
+
 }  // namespace
 }  // namespace fsgs
 
 using namespace fsgs;
+
+FSGS_API int fsgs_gs_compute_cov3D_forward(int N, const float* q, const float* s, float* cov3D, void* stream) {
+  FSGS_REQUIRE(N >= 0, "gs_compute_cov3D_forward: bad size");
+  if (N == 0) return kOk;
+  FSGS_REQUIRE(q && s && cov3D, "gs_compute_cov3D_forward: null pointer");
+  hipLaunchKernelGGL(cov3d_forward_kernel, dim3(div_up(N, 256)), dim3(256), 0, (hipStream_t) stream, N,
+                     (const float4*) q, s, cov3D);
+  return check_launch("gs_compute_cov3D_forward");
+}
+
+FSGS_API int fsgs_gs_compute_cov3D_backward(int N, const float* q, const float* s, const float* g_cov3D, float* g_q,
+                                            float* g_s, void* stream) {
+  FSGS_REQUIRE(N >= 0, "gs_compute_cov3D_backward: bad size");
+  if (N == 0) return kOk;
+  FSGS_REQUIRE(q && s && g_cov3D && g_q && g_s, "gs_compute_cov3D_backward: null pointer");
+  hipLaunchKernelGGL(cov3d_backward_kernel, dim3(div_up(N, 256)), dim3(256), 0, (hipStream_t) stream, N,
+                     (const float4*) q, s, g_cov3D, (float4*) g_q, g_s);
+  return check_launch("gs_compute_cov3D_backward");
+}
+
+FSGS_API int fsgs_gs_compute_cov2D_forward(int N, const float* cov3D, const float* mean, const float* Tw2v,
+    double focal_x, double focal_y, double tan_fovx, double tan_fovy, float* cov2D, void* stream) {
+  FSGS_REQUIRE(N >= 0, "gs_compute_cov2D_forward: bad size");
+  if (N == 0) return kOk;
+  FSGS_REQUIRE(cov3D && mean && Tw2v && cov2D, "gs_compute_cov2D_forward: null pointer");
+  hipLaunchKernelGGL(cov2d_forward_kernel, dim3(div_up(N, 256)), dim3(256), 0, (hipStream_t) stream, N, cov3D, mean,
+                     Tw2v, (float) focal_x, (float) focal_y, (float) tan_fovx, (float) tan_fovy, cov2D);
+  return check_launch("gs_compute_cov2D_forward");
+}
+
+FSGS_API int fsgs_gs_compute_cov2D_backward(int N, const float* cov3D, const float* mean, const float* Tw2v,
+    double focal_x, double focal_y, double tan_fovx, double tan_fovy, const float* g_cov2D, float* g_cov3D,
+    float* g_mean, void* stream) {
+  FSGS_REQUIRE(N >= 0, "gs_compute_cov2D_backward: bad size");
+  if (N == 0) return kOk;
+  FSGS_REQUIRE(cov3D && mean && Tw2v && g_cov2D && g_cov3D && g_mean, "gs_compute_cov2D_backward: null pointer");
+  hipLaunchKernelGGL(cov2d_backward_kernel, dim3(div_up(N, 256)), dim3(256), 0, (hipStream_t) stream, N, cov3D, mean,
+                     Tw2v, (float) focal_x, (float) focal_y, (float) tan_fovx, (float) tan_fovy, g_cov2D, g_cov3D,
+                     g_mean);
+  return check_launch("gs_compute_cov2D_backward");
+}
 
 FSGS_API int fsgs_gs_preprocess_forward(int P, int W, int H, int sh_degree, int n_sh, int is_opengl,
     const float* means3D, const float* scales, const float* rotations, const float* opacities, const float* shs,

@@ -13,7 +13,8 @@ from torch import Tensor
 from fast_sp_gs_amd._C import get_C_function
 from fast_sp_gs_amd.renderer.gs_2d_render import GS_prepare
 
-__all__ = ['RasterizeBuffer3D', 'preprocess', 'GS_render', 'RasterizeGaussians', 'render']
+__all__ = ['RasterizeBuffer3D', 'preprocess', 'GS_render', 'RasterizeGaussians', 'render', 'compute_cov3D',
+           'compute_cov2D']
 
 
 class RasterizeBuffer3D(NamedTuple):
@@ -28,6 +29,55 @@ class RasterizeBuffer3D(NamedTuple):
     conic_opacity: Tensor
     means2D: Tensor
     opacity: Tensor
+
+
+class _compute_cov3D(torch.autograd.Function):
+    """renderer/gaussian_render.py:370-387 of the reference."""
+
+    @staticmethod
+    def forward(ctx, scaling, rotation):
+        scaling, rotation = scaling.contiguous(), rotation.contiguous()
+        ctx.save_for_backward(rotation, scaling)
+        return get_C_function('gs_compute_cov3D_forward')(rotation, scaling)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_cov3D):
+        rotation, scaling = ctx.saved_tensors
+        grad_rotation, grad_scaling = get_C_function('gs_compute_cov3D_backward')(rotation, scaling, grad_cov3D)
+        return grad_scaling, grad_rotation
+
+
+def compute_cov3D(scaling: Tensor, rotation: Tensor) -> Tensor:
+    """Upper triangle [N,6] of R(q) diag(s^2) R(q)^T (reference: renderer/gaussian_render.py:420-424)."""
+    return _compute_cov3D.apply(scaling, rotation)
+
+
+class _compute_cov2D(torch.autograd.Function):
+    """renderer/gaussian_render.py:427-447 of the reference; the view matrix gets no gradient here."""
+
+    @staticmethod
+    def forward(ctx, means, cov3D, Tw2v, fx, fy, tx, ty):
+        means, cov3D, Tw2v = means.contiguous(), cov3D.contiguous(), Tw2v.contiguous()
+        ctx.focal_fov = (fx, fy, tx, ty)
+        ctx.save_for_backward(cov3D, means, Tw2v)
+        return get_C_function('gs_compute_cov2D_forward')(cov3D, means, Tw2v, fx, fy, tx, ty)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_cov2D):
+        cov3D, means, Tw2v = ctx.saved_tensors
+        if ctx.needs_input_grad[2]:
+            raise RuntimeError('compute_cov2D: the gradient to the view matrix is not supported')
+        grad_cov3D, grad_mean = get_C_function('gs_compute_cov2D_backward')(cov3D, means, Tw2v, *ctx.focal_fov,
+                                                                           grad_cov2D)
+        return grad_mean, grad_cov3D, None, None, None, None, None
+
+
+def compute_cov2D(means: Tensor, cov3D: Tensor, Tw2v: Tensor, focal_x: float, focal_y: float, tan_fovx: float,
+                  tan_fovy: float) -> Tensor:
+    """(a, b, c) [N,3] of J W cov3D W^T J^T + 0.3 I (reference: renderer/gaussian_render.py:450-493)."""
+    return _compute_cov2D.apply(means, cov3D, Tw2v, focal_x, focal_y, tan_fovx, tan_fovy)
 
 
 class _preprocess(torch.autograd.Function):

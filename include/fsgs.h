@@ -294,6 +294,22 @@ int fsgs_gs_preprocess_backward(int P, int W, int H, int sh_degree, int n_sh, in
     float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs, float* g_sh_rest, float* g_cov3D,
     void* stream);
 
+/* gs_compute_cov3D_forward / gs_compute_cov3D_backward -- fast_2d_gs/_C/src/gaussian_splatting/
+ * gaussian_compute_cov3D.cu:122-161: cov3D[N,6] = upper triangle of R(q) diag(s^2) R(q)^T for q[N,4] (x, y, z, w, used as
+ * given, not normalised) and s[N,3]; the backward writes g_q[N,4] and g_s[N,3] in full. */
+int fsgs_gs_compute_cov3D_forward(int N, const float* q, const float* s, float* cov3D, void* stream);
+int fsgs_gs_compute_cov3D_backward(int N, const float* q, const float* s, const float* g_cov3D, float* g_q, float* g_s,
+                                   void* stream);
+
+/* gs_compute_cov2D_forward / gs_compute_cov2D_backward -- gaussian_compute_cov2D.cu:186-248: cov2D[N,3] = (a, b, c) of
+ * J W cov3D W^T J^T + 0.3 I with the view-space mean clamped to 1.3 x the field of view (W = rotation block of the
+ * row-major Tw2v[4,4]); the backward takes dL/dcov2D[N,3] and writes g_cov3D[N,6] and g_mean[N,3] in full. The
+ * reference's optional gradient to the view matrix is not produced. */
+int fsgs_gs_compute_cov2D_forward(int N, const float* cov3D, const float* mean, const float* Tw2v, double focal_x,
+    double focal_y, double tan_fovx, double tan_fovy, float* cov2D, void* stream);
+int fsgs_gs_compute_cov2D_backward(int N, const float* cov3D, const float* mean, const float* Tw2v, double focal_x,
+    double focal_y, double tan_fovx, double tan_fovy, const float* g_cov2D, float* g_cov3D, float* g_mean, void* stream);
+
 /* gaussian_rasterize_forward -- gaussian_render.cu:212-293 (kernel :20-173) without the bucket snapshots of the
  * per-Gaussian backward. colors[P,3], extras[P,E] (E <= 4, optional) -> out_color[3,H,W], out_opacity[H,W],
  * out_extras[E,H,W], n_contrib[H,W]; every output element is written. accum_* as in the surfel forward. */

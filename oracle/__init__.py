@@ -277,6 +277,40 @@ def gs3d_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotati
     return g3, gs, gq, go, gsh, grest, gcov, gm2
 
 
+def gs3d_compute_cov3D(q, s):
+    """gs_compute_cov3D_forward(q, s) -> cov3D [N,6] (gaussian_compute_cov3D.cu:122-137)."""
+    N = s.shape[0]
+    out = np.zeros((N, 6), s.dtype)
+    assert call(f"gs3d_compute_cov3D_{_suffix(s.dtype)}", N, q, s, out) == 0
+    return out
+
+
+def gs3d_compute_cov3D_backward(q, s, g):
+    """gs_compute_cov3D_backward(q, s, dL_dcov3D) -> (dq, ds) (gaussian_compute_cov3D.cu:151-161)."""
+    N = s.shape[0]
+    gq, gs = np.zeros((N, 4), s.dtype), np.zeros((N, 3), s.dtype)
+    assert call(f"gs3d_compute_cov3D_backward_{_suffix(s.dtype)}", N, q, s, g, gq, gs) == 0
+    return gq, gs
+
+
+def gs3d_compute_cov2D(cov3D, mean, Tw2v, fx, fy, tanx, tany):
+    """gs_compute_cov2D_forward -> cov2D [N,3] with the 0.3 low-pass term (gaussian_compute_cov2D.cu:199-210)."""
+    N = mean.shape[0]
+    out = np.zeros((N, 3), mean.dtype)
+    assert call(f"gs3d_compute_cov2D_{_suffix(mean.dtype)}", N, cov3D, mean, Tw2v, float(fx), float(fy), float(tanx),
+                float(tany), out) == 0
+    return out
+
+
+def gs3d_compute_cov2D_backward(cov3D, mean, Tw2v, fx, fy, tanx, tany, g):
+    """gs_compute_cov2D_backward -> (grad_cov3D, grad_mean), no view-matrix gradient (gaussian_compute_cov2D.cu:229-248)."""
+    N = mean.shape[0]
+    gc, gm = np.zeros((N, 6), mean.dtype), np.zeros((N, 3), mean.dtype)
+    assert call(f"gs3d_compute_cov2D_backward_{_suffix(mean.dtype)}", N, cov3D, mean, Tw2v, float(fx), float(fy),
+                float(tanx), float(tany), g, gc, gm) == 0
+    return gc, gm
+
+
 def gs3d_render_forward(W, H, means2D, conic_opacity, colors, extras, point_list, ranges, accum_max_count=None,
                         accum_weights_p=None, accum_weights_count=None):
     dt = means2D.dtype

@@ -125,23 +125,11 @@ inline void cov2d_product(const T* M, const T* c, T* out) {
   out[0] = cov[0], out[1] = cov[1], out[2] = cov[3];
 }
 
-// gaussian_compute_cov2D.cu:64-186 with dL_dconic given (dL_dcov2D absent), no view-matrix gradient.
-// Returns false when the determinant is exactly zero (the reference returns without writing).
+// gaussian_compute_cov2D.cu:96-186: from dL/dcov2D = (da, db, dc) (b is the one stored off-diagonal entry) to dL/dcov3D
+// and dL/dmean, no view-matrix gradient.
 template <typename T>
-inline bool cov2d_backward(const T* mean, const T* c3, T fx, T fy, T tanx, T tany, const T* V, const T* g_conic,
-                           T* g_cov3D, T* g_mean) {
-  Cov2DTerms<T> k;
-  cov2d_terms(mean, fx, fy, tanx, tany, V, k);
-  T cov[3];
-  cov2d_product(k.M, c3, cov);
-  const T a = cov[0] + T(0.3), b = cov[1], c = cov[2] + T(0.3);
-  const T denom = a * c - b * b;
-  if (denom == 0) return false;
-  const T denom2inv = T(1.) / ((denom * denom) + T(0.0000001));
-  const T tt = c * g_conic[0] - b * g_conic[1] + a * g_conic[2];
-  const T da = denom2inv * (-c * tt + denom * g_conic[2]);
-  const T dc = denom2inv * (-a * tt + denom * g_conic[0]);
-  const T db = denom2inv * (T(2) * b * tt - denom * g_conic[1]);
+inline void cov2d_backward_cov(const Cov2DTerms<T>& k, const T* c3, T fx, T fy, const T* V, T da, T db, T dc,
+                               T* g_cov3D, T* g_mean) {
   const T* M = k.M;
   if (g_cov3D) {
     g_cov3D[0] = (M[0] * M[0] * da + M[0] * M[3] * db + M[3] * M[3] * dc);
@@ -168,7 +156,63 @@ inline bool cov2d_backward(const T* mean, const T* c3, T fx, T fy, T tanx, T tan
   const T dty = k.y_mul * -fy * tz2 * dJ12;
   const T dtz = -fx * tz2 * dJ00 - fy * tz2 * dJ11 + (2 * fx * k.t[0]) * tz3 * dJ02 + (2 * fy * k.t[1]) * tz3 * dJ12;
   for (int a2 = 0; a2 < 3; ++a2) g_mean[a2] = V[a2] * dtx + V[4 + a2] * dty + V[8 + a2] * dtz;
+}
+
+// gaussian_compute_cov2D.cu:64-95 in front of the above: dL_dconic given (dL_dcov2D absent).
+// Returns false when the determinant is exactly zero (the reference returns without writing).
+template <typename T>
+inline bool cov2d_backward(const T* mean, const T* c3, T fx, T fy, T tanx, T tany, const T* V, const T* g_conic,
+                           T* g_cov3D, T* g_mean) {
+  Cov2DTerms<T> k;
+  cov2d_terms(mean, fx, fy, tanx, tany, V, k);
+  T cov[3];
+  cov2d_product(k.M, c3, cov);
+  const T a = cov[0] + T(0.3), b = cov[1], c = cov[2] + T(0.3);
+  const T denom = a * c - b * b;
+  if (denom == 0) return false;
+  const T denom2inv = T(1.) / ((denom * denom) + T(0.0000001));
+  const T tt = c * g_conic[0] - b * g_conic[1] + a * g_conic[2];
+  const T da = denom2inv * (-c * tt + denom * g_conic[2]);
+  const T dc = denom2inv * (-a * tt + denom * g_conic[0]);
+  const T db = denom2inv * (T(2) * b * tt - denom * g_conic[1]);
+  cov2d_backward_cov(k, c3, fx, fy, V, da, db, dc, g_cov3D, g_mean);
   return true;
+}
+
+// gs_compute_cov3D_forward / _backward (gaussian_compute_cov3D.cu:122-161) and gs_compute_cov2D_forward / _backward
+// (gaussian_compute_cov2D.cu:186-248, without the view-matrix gradient) as stand-alone operators.
+template <typename T>
+void compute_cov3D(int N, const T* q, const T* s, T* cov3D) {
+#pragma omp parallel for
+  for (int i = 0; i < N; ++i) cov3d_forward(s + 3 * (size_t) i, q + 4 * (size_t) i, cov3D + 6 * (size_t) i);
+}
+template <typename T>
+void compute_cov3D_backward(int N, const T* q, const T* s, const T* g, T* gq, T* gs) {
+#pragma omp parallel for
+  for (int i = 0; i < N; ++i)
+    cov3d_backward(s + 3 * (size_t) i, q + 4 * (size_t) i, g + 6 * (size_t) i, gs + 3 * (size_t) i, gq + 4 * (size_t) i);
+}
+template <typename T>
+void compute_cov2D(int N, const T* cov3D, const T* mean, const T* V, T fx, T fy, T tanx, T tany, T* cov2D) {
+#pragma omp parallel for
+  for (int i = 0; i < N; ++i) {
+    Cov2DTerms<T> k;
+    cov2d_terms(mean + 3 * (size_t) i, fx, fy, tanx, tany, V, k);
+    T* o = cov2D + 3 * (size_t) i;
+    cov2d_product(k.M, cov3D + 6 * (size_t) i, o);
+    o[0] += T(0.3), o[2] += T(0.3);
+  }
+}
+template <typename T>
+void compute_cov2D_backward(int N, const T* cov3D, const T* mean, const T* V, T fx, T fy, T tanx, T tany, const T* g,
+                            T* g_cov3D, T* g_mean) {
+#pragma omp parallel for
+  for (int i = 0; i < N; ++i) {
+    Cov2DTerms<T> k;
+    cov2d_terms(mean + 3 * (size_t) i, fx, fy, tanx, tany, V, k);
+    cov2d_backward_cov(k, cov3D + 6 * (size_t) i, fx, fy, V, g[3 * (size_t) i], g[3 * (size_t) i + 1],
+                       g[3 * (size_t) i + 2], g_cov3D + 6 * (size_t) i, g_mean + 3 * (size_t) i);
+  }
 }
 
 // gaussian_preprocess.cu:44-128 (preprocess_forward_kernel) + host :372-466. Outputs are expected zero-filled, except
@@ -411,6 +455,24 @@ using namespace oracle;
     render_backward<T>(W, H, E, means2D, conic_opacity, colors, extras, out_opacity, n_contrib, dL_dpix,             \
                        dL_dout_extras, dL_dout_opacity, point_list, ranges, g_means2D, g_conic_opacity, g_colors,    \
                        g_extras);                                                                                    \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_gs3d_compute_cov3D_##SUF(int N, const T* q, const T* s, T* cov3D) {                          \
+    compute_cov3D<T>(N, q, s, cov3D);                                                                                \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_gs3d_compute_cov3D_backward_##SUF(int N, const T* q, const T* s, const T* g, T* gq, T* gs) { \
+    compute_cov3D_backward<T>(N, q, s, g, gq, gs);                                                                   \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_gs3d_compute_cov2D_##SUF(int N, const T* cov3D, const T* mean, const T* Tw2v, double fx,     \
+      double fy, double tanx, double tany, T* cov2D) {                                                               \
+    compute_cov2D<T>(N, cov3D, mean, Tw2v, (T) fx, (T) fy, (T) tanx, (T) tany, cov2D);                               \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_gs3d_compute_cov2D_backward_##SUF(int N, const T* cov3D, const T* mean, const T* Tw2v,       \
+      double fx, double fy, double tanx, double tany, const T* g, T* g_cov3D, T* g_mean) {                           \
+    compute_cov2D_backward<T>(N, cov3D, mean, Tw2v, (T) fx, (T) fy, (T) tanx, (T) tany, g, g_cov3D, g_mean);         \
     return 0;                                                                                                        \
   }
 

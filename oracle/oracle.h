@@ -86,6 +86,12 @@ int oracle_gs3d_render_backward_f32(int W, int H, int E, const float* means2D, c
     const float* colors, const float* extras, const float* out_opacity, const int32_t* n_contrib,
     const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
     const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras);
+int oracle_gs3d_compute_cov3D_f32(int N, const float* q, const float* s, float* cov3D);
+int oracle_gs3d_compute_cov3D_backward_f32(int N, const float* q, const float* s, const float* g, float* gq, float* gs);
+int oracle_gs3d_compute_cov2D_f32(int N, const float* cov3D, const float* mean, const float* Tw2v, double fx, double fy,
+    double tanx, double tany, float* cov2D);
+int oracle_gs3d_compute_cov2D_backward_f32(int N, const float* cov3D, const float* mean, const float* Tw2v, double fx,
+    double fy, double tanx, double tany, const float* g, float* g_cov3D, float* g_mean);
 int64_t oracle_gs_prepare_count(int P, const int32_t* tiles_touched, int64_t* offsets);
 int oracle_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
     const int64_t* offsets, int64_t R, int64_t* ranges, int32_t* point_list, int64_t* keys_sorted_out);

@@ -167,3 +167,46 @@ def test_gs3d_render_autograd_and_empty(device):
     out = GR.render(d(cam.Tw2v), d(cam.Tv2c), (W, H), z(0, 3), z(0, 1), scales=z(0, 3), rotations=z(0, 4),
                     campos=d(cam.campos), focals=focals, sh_features=z(0, 16, 3), sh_degree=3)
     assert out['images'].shape == (3, H, W) and not out['images'].any() and not out['opacity'].any()
+
+
+def test_covariance_operators(device):
+    """gs_compute_cov3D_* / gs_compute_cov2D_* against the oracle (geometry evaluated with contraction off: forward
+    values bit for bit, gradients to 1e-5 of the largest entry), and the autograd wrappers end to end."""
+    from fast_sp_gs_amd._C import get_C_function as f
+    from fast_sp_gs_amd.renderer.gaussian_render import compute_cov2D, compute_cov3D
+    g = torch.Generator().manual_seed(4)
+    N = 70001
+    q = torch.randn(N, 4, generator=g)
+    s = torch.rand(N, 3, generator=g) * 0.3 + 0.01
+    gc = torch.randn(N, 6, generator=g)
+    print(f"[gs3d covariance operators] N={N}", flush=True)
+    d = lambda t: t.to(device).contiguous()
+    cov3D = f('gs_compute_cov3D_forward')(d(q), d(s))
+    want = O.gs3d_compute_cov3D(npy(q), npy(s))
+    assert np.array_equal(npy(cov3D), want)
+    dq, ds = f('gs_compute_cov3D_backward')(d(q), d(s), d(gc))
+    wq, ws = O.gs3d_compute_cov3D_backward(npy(q), npy(s), npy(gc))
+    assert rel_err(npy(dq), wq) < 1e-5 and rel_err(npy(ds), ws) < 1e-5
+
+    Tw2v = torch.eye(4)
+    Tw2v[:3, :3] = torch.tensor([[0.92, 0.0, 0.39], [0.1, 0.99, -0.05], [-0.39, 0.05, 0.92]])
+    Tw2v[:3, 3] = torch.tensor([0.2, -0.1, 4.0])
+    means = torch.randn(N, 3, generator=g) * torch.tensor([2.0, 2.0, 0.5])
+    fx, fy, tx, ty = 500.0, 480.0, 0.4, 0.35
+    g2 = torch.randn(N, 3, generator=g)
+    cov2D = f('gs_compute_cov2D_forward')(cov3D, d(means), d(Tw2v), fx, fy, tx, ty)
+    want2 = O.gs3d_compute_cov2D(want, npy(means), npy(Tw2v), fx, fy, tx, ty)
+    assert np.array_equal(npy(cov2D), want2)
+    g_cov3D, g_mean = f('gs_compute_cov2D_backward')(cov3D, d(means), d(Tw2v), fx, fy, tx, ty, d(g2))
+    w3, wm = O.gs3d_compute_cov2D_backward(want, npy(means), npy(Tw2v), fx, fy, tx, ty, npy(g2))
+    assert rel_err(npy(g_cov3D), w3) < 1e-5 and rel_err(npy(g_mean), wm) < 1e-5
+    with pytest.raises(RuntimeError):
+        f('gs_compute_cov2D_backward')(cov3D, d(means), d(Tw2v), fx, fy, tx, ty, d(g2), torch.zeros(4, 4, device=device))
+
+    # autograd wrappers: scaling / rotation / means receive the chained gradients
+    sa, qa, ma = d(s).requires_grad_(True), d(q).requires_grad_(True), d(means).requires_grad_(True)
+    out = compute_cov2D(ma, compute_cov3D(sa, qa), d(Tw2v), fx, fy, tx, ty)
+    out.backward(d(g2))
+    c3g, wm2 = O.gs3d_compute_cov2D_backward(want, npy(means), npy(Tw2v), fx, fy, tx, ty, npy(g2))
+    wq2, ws2 = O.gs3d_compute_cov3D_backward(npy(q), npy(s), c3g)
+    assert rel_err(npy(ma.grad), wm2) < 1e-5 and rel_err(npy(qa.grad), wq2) < 1e-4 and rel_err(npy(sa.grad), ws2) < 1e-4

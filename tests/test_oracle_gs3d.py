@@ -196,3 +196,76 @@ def test_preprocess_backward_finite_differences():
                 fd = (loss(**{name: a}) - loss(**{name: b})) / (2 * h)
                 worst = max(worst, abs(fd - grad[(i,) + ix]) / max(np.abs(grad[vis[:12]]).max(), 1e-9))
         assert worst < 2e-5, (name, worst)
+
+
+def _ref_cov3D(scaling, rotation):
+    """The reference's own torch formulation, renderer/gaussian_render.py:389-424 (build_rotation without normalising,
+    L = R S, L L^T, upper triangle), in the dtype of its arguments."""
+    x, y, z, r = rotation.unbind(-1)
+    R = torch.stack([1 - 2 * (y * y + z * z), 2 * (x * y - r * z), 2 * (x * z + r * y),
+                     2 * (x * y + r * z), 1 - 2 * (x * x + z * z), 2 * (y * z - r * x),
+                     2 * (x * z - r * y), 2 * (y * z + r * x), 1 - 2 * (x * x + y * y)], -1).view(-1, 3, 3)
+    Lm = R @ torch.diag_embed(scaling)
+    C = Lm @ Lm.transpose(1, 2)
+    return torch.stack([C[:, 0, 0], C[:, 0, 1], C[:, 0, 2], C[:, 1, 1], C[:, 1, 2], C[:, 2, 2]], -1)
+
+
+def _ref_cov2D(means, cov3D, Tw2v, fx, fy, tx, ty):
+    """renderer/gaussian_render.py:450-493 of the reference, line by line."""
+    P = means.shape[0]
+    R = Tw2v[:3, :3]
+    p = torch.einsum('pi,ji->pj', means, R) + Tw2v[:3, 3]
+    x, y, z = p.unbind(-1)
+    limit_x, limit_y = z.detach() * 1.3 * tx, z.detach() * 1.3 * ty
+    x = torch.minimum(torch.maximum(x, -limit_x), limit_x)
+    y = torch.minimum(torch.maximum(y, -limit_y), limit_y)
+    v0 = torch.zeros_like(z)
+    J = torch.stack([fx / z, v0, -(fx * x) / (z * z), v0, fy / z, -(fy * y) / (z * z)], -1).view(P, 2, 3)
+    T = J @ R
+    V = torch.stack([cov3D[:, 0], cov3D[:, 1], cov3D[:, 2], cov3D[:, 1], cov3D[:, 3], cov3D[:, 4],
+                     cov3D[:, 2], cov3D[:, 4], cov3D[:, 5]], -1).view(-1, 3, 3)
+    V_ = T @ V @ T.transpose(-1, -2)
+    return torch.stack([V_[:, 0, 0] + 0.3, V_[:, 0, 1], V_[:, 1, 1] + 0.3], -1)
+
+
+def test_covariance_operators_match_the_reference_formulation():
+    """gs_compute_cov3D_* / gs_compute_cov2D_*: the oracle in fp64 against the reference's torch fallbacks and their
+    autograd, with points inside and outside the 1.3 x field-of-view clamp."""
+    import torch
+    g = torch.Generator().manual_seed(3)
+    N = 300
+    q = torch.randn(N, 4, generator=g, dtype=torch.float64)            # not normalised on purpose
+    s = torch.rand(N, 3, generator=g, dtype=torch.float64) * 0.3 + 0.01
+    gc = torch.randn(N, 6, generator=g, dtype=torch.float64)
+    qa, sa = q.clone().requires_grad_(True), s.clone().requires_grad_(True)
+    want = _ref_cov3D(sa, qa)
+    want.backward(gc)
+    got = O.gs3d_compute_cov3D(q.numpy(), s.numpy())
+    np.testing.assert_allclose(got, want.detach().numpy(), rtol=1e-12, atol=1e-14)
+    gq, gs = O.gs3d_compute_cov3D_backward(q.numpy(), s.numpy(), gc.numpy())
+    np.testing.assert_allclose(gq, qa.grad.numpy(), rtol=1e-11, atol=1e-13)
+    np.testing.assert_allclose(gs, sa.grad.numpy(), rtol=1e-11, atol=1e-13)
+
+    Tw2v = torch.eye(4, dtype=torch.float64)
+    ang = 0.4
+    Tw2v[:3, :3] = torch.tensor([[np.cos(ang), 0, np.sin(ang)], [0.1, 0.99, -0.05], [-np.sin(ang), 0.05, np.cos(ang)]])
+    Tw2v[:3, 3] = torch.tensor([0.2, -0.1, 4.0])
+    means = torch.randn(N, 3, generator=g, dtype=torch.float64) * torch.tensor([3.0, 3.0, 0.8])  # many beyond the clamp
+    cov3D = want.detach()
+    fx, fy, tx, ty = 500.0, 480.0, 0.4, 0.35
+    pv = means @ Tw2v[:3, :3].T + Tw2v[:3, 3]
+    keep = pv[:, 2] > 0.5  # in front of the camera, as every Gaussian that reaches this step is
+    means, cov3D, pv, N = means[keep], cov3D[keep], pv[keep], int(keep.sum())
+    assert N > 200
+    outside = (pv[:, 0].abs() > 1.3 * tx * pv[:, 2]) | (pv[:, 1].abs() > 1.3 * ty * pv[:, 2])
+    assert outside.any() and (~outside).any()
+    ma, ca = means.clone().requires_grad_(True), cov3D.clone().requires_grad_(True)
+    want2 = _ref_cov2D(ma, ca, Tw2v, fx, fy, tx, ty)
+    g2 = torch.randn(N, 3, generator=g, dtype=torch.float64)
+    want2.backward(g2)
+    got2 = O.gs3d_compute_cov2D(cov3D.numpy(), means.numpy(), Tw2v.numpy(), fx, fy, tx, ty)
+    np.testing.assert_allclose(got2, want2.detach().numpy(), rtol=1e-11, atol=1e-12)
+    g_cov3D, g_mean = O.gs3d_compute_cov2D_backward(cov3D.numpy(), means.numpy(), Tw2v.numpy(), fx, fy, tx, ty,
+                                                    g2.numpy())
+    np.testing.assert_allclose(g_cov3D, ca.grad.numpy(), rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(g_mean, ma.grad.numpy(), rtol=1e-9, atol=1e-9 * float(ma.grad.abs().max()))
