@@ -27,6 +27,7 @@ __all__ = [
     'gs_preprocess_backward', 'gaussian_rasterize_forward', 'gaussian_rasterize_backward', 'select_indices',
     'gather_rows', 'densify_masks', 'prune_mask', 'split_children', 'densification_stats',
     'gs_compute_cov3D_forward', 'gs_compute_cov3D_backward', 'gs_compute_cov2D_forward', 'gs_compute_cov2D_backward',
+    'gaussian_topk_weights',
 ]
 
 _TILE = 16
@@ -1341,6 +1342,24 @@ def _tan_fov(tanFoV) -> Tuple[float, float]:
         v = tanFoV.detach().cpu().tolist()  # the reference reads it with .item() too (gaussian_preprocess.cu:424-425)
         return float(v[0]), float(v[1])
     return float(tanFoV[0]), float(tanFoV[1])
+
+
+def gaussian_topk_weights(topk: int, W: int, H: int, P: int, R: int, means2D: Tensor, conic_opacity: Tensor,
+                          ranges: Tensor, point_list: Tensor) -> Tuple[Tensor, Tensor]:
+    """gaussian_topk.cu:212-228 -> (top_indices[H,W,K] int32, top_weights[H,W,K])."""
+    what = 'gaussian_topk_weights'
+    _f32(what, means2D=means2D, conic_opacity=conic_opacity)
+    L.require_cuda(what, ranges=ranges, point_list=point_list)
+    L.require_dtype(what, 'ranges', ranges, torch.int64)
+    L.require_dtype(what, 'point_list', point_list, torch.int32)
+    top_indices = torch.empty((H, W, topk), dtype=torch.int32, device=means2D.device)
+    top_weights = torch.empty((H, W, topk), dtype=torch.float32, device=means2D.device)
+    with _timed(what):
+        rc = _lib().fsgs_gaussian_topk_weights(topk, means2D.shape[0], W, H, L.ptr(means2D), L.ptr(conic_opacity),
+                                               L.ptr(ranges), L.ptr(point_list), L.ptr(top_indices),
+                                               L.ptr(top_weights), L.current_stream())
+    L.check(rc, what)
+    return top_indices, top_weights
 
 
 def gs_compute_cov3D_forward(q: Tensor, s: Tensor) -> Tensor:

@@ -199,6 +199,84 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
   }
 }
 
+// Per-pixel top-k blend weights (gaussian_topk.cu:12-93): the forward traversal with the k slots in registers instead of
+// the reference's read-modify-write of global memory per contributing pair. `w >= slot` takes a slot (a later Gaussian
+// wins ties); indices start at -1, weights at 0.
+template <int kK>
+__global__ void __launch_bounds__(kBlendThreads) gs3d_topk_kernel(int flags, int W, int H, int topk,
+    const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
+    const float4* __restrict__ conic_opacity, int32_t* __restrict__ top_indices, float* __restrict__ top_weights) {
+  __shared__ G3Hot s_hot[kG3Batch];
+  const int gx = (W + kTile - 1) / kTile;
+  const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
+  int px, py;
+  lane_pixel(tile_x, tile_y, px, py);
+  const bool inside = px < W && py < H;
+  const size_t pix  = (size_t) W * py + px;
+  const float pxf = (float) px, pyf = (float) py;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
+  const int n_todo = (int) (r1 - r0);
+  const int rounds = (n_todo + kG3Batch - 1) / kG3Batch;
+  bool done = !inside;
+  float T = 1.0f, tw[kK];
+  int ti[kK];
+#pragma unroll
+  for (int k = 0; k < kK; ++k) tw[k] = 0.0f, ti[k] = -1;
+  for (int b = 0; b < rounds; ++b) {
+    if (__syncthreads_count(done) == kBlendThreads) break;
+    const int n_here = min(kG3Batch, n_todo - b * kG3Batch);
+    if ((int) threadIdx.x < n_here) {
+      const int id    = point_list[r0 + b * kG3Batch + threadIdx.x];
+      const float2 c  = means2D[id];
+      const float4 co = conic_opacity[id];
+      G3Hot h;
+      h.x = c.x, h.y = c.y, h.a = co.x, h.b = co.y, h.c = co.z, h.opacity = co.w, h.id = id;
+      h.mask = conic_quadrant_mask(h, tile_x * kTile, tile_y * kTile, flags);
+      s_hot[threadIdx.x] = h;
+    }
+    __syncthreads();
+    for (int c = 0; c < kG3Batch / kWave; ++c) {
+      const int jj = c * kWave + lane;
+      unsigned long long todo = __ballot(jj < n_here && ((s_hot[jj < kG3Batch ? jj : 0].mask >> wave) & 1u));
+      while (todo) {
+        if (__ballot(!done) == 0ull) break;
+        const int j = c * kWave + __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const G3Hot hot = s_hot[j];
+        G3Hit h;
+        const bool hit = conic_alpha_flat(hot, pxf, pyf, h) && !done;
+        if (__ballot(hit) == 0ull) continue;
+        const float test_T = T * (1.0f - h.alpha);
+        const bool sat     = hit && test_T < 0.0001f;
+        done               = done || sat;
+        if (hit && !sat) {
+          float w = h.alpha * T;
+          int idx = hot.id;
+#pragma unroll
+          for (int k = 0; k < kK; ++k) {
+            if (k < topk && w >= tw[k]) {
+              const float ow = tw[k];
+              const int oi   = ti[k];
+              tw[k] = w, ti[k] = idx;
+              w = ow, idx = oi;
+            }
+          }
+          T = test_T;
+        }
+      }
+    }
+  }
+  if (inside) {
+#pragma unroll
+    for (int k = 0; k < kK; ++k)
+      if (k < topk) {
+        top_weights[pix * topk + k] = tw[k];
+        top_indices[pix * topk + k] = ti[k];
+      }
+  }
+}
+
 // gradient slots of one Gaussian: 0-2 colour | 3-6 extras | 7-8 mean2D | 9-11 conic | 12 opacity | 13-15 unused
 template <int E>
 __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags, int W, int H,
@@ -388,4 +466,25 @@ FSGS_API int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const 
   }
 #undef FSGS_G3_BWD
   return check_launch("gaussian_rasterize_backward");
+}
+
+FSGS_API int fsgs_gaussian_topk_weights(int topk, int P, int W, int H, const float* means2D,
+    const float* conic_opacity, const int64_t* ranges, const int32_t* point_list, int32_t* top_indices,
+    float* top_weights, void* stream) {
+  FSGS_REQUIRE(topk > 0 && W > 0 && H > 0 && P >= 0 && ranges && top_indices && top_weights,
+               "gaussian_topk_weights: bad arguments");
+  FSGS_REQUIRE(topk <= 16, "gaussian_topk_weights: topk=%d exceeds the supported maximum of 16", topk);
+  FSGS_REQUIRE(P == 0 || (means2D && conic_opacity && point_list), "gaussian_topk_weights: null pointer");
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const dim3 grid(gx * gy), block(kBlendThreads);
+  hipStream_t s   = (hipStream_t) stream;
+  const int flags = launch_tile_order(gx, gy, ranges, s);
+#define FSGS_TOPK3(KK)                                                                                          \
+  hipLaunchKernelGGL((gs3d_topk_kernel<KK>), grid, block, 0, s, flags, W, H, topk, ranges, point_list,          \
+                     (const float2*) means2D, (const float4*) conic_opacity, top_indices, top_weights)
+  if (topk <= 4) FSGS_TOPK3(4);
+  else if (topk <= 8) FSGS_TOPK3(8);
+  else FSGS_TOPK3(16);
+#undef FSGS_TOPK3
+  return check_launch("gaussian_topk_weights");
 }

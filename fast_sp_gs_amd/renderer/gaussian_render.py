@@ -14,7 +14,7 @@ from fast_sp_gs_amd._C import get_C_function
 from fast_sp_gs_amd.renderer.gs_2d_render import GS_prepare
 
 __all__ = ['RasterizeBuffer3D', 'preprocess', 'GS_render', 'RasterizeGaussians', 'render', 'compute_cov3D',
-           'compute_cov2D']
+           'compute_cov2D', 'topk_weights']
 
 
 class RasterizeBuffer3D(NamedTuple):
@@ -29,6 +29,12 @@ class RasterizeBuffer3D(NamedTuple):
     conic_opacity: Tensor
     means2D: Tensor
     opacity: Tensor
+
+
+def topk_weights(topk: int, buffer: RasterizeBuffer3D) -> Tuple[Tensor, Tensor]:
+    """Per-pixel top-k Gaussian indices and blend weights of a rendered view (reference: gaussian_render.py:362-367)."""
+    return get_C_function('gaussian_topk_weights')(topk, buffer.W, buffer.H, buffer.P, buffer.R, buffer.means2D,
+                                                   buffer.conic_opacity, buffer.tile_ranges, buffer.point_list)
 
 
 class _compute_cov3D(torch.autograd.Function):

@@ -294,6 +294,12 @@ int fsgs_gs_preprocess_backward(int P, int W, int H, int sh_degree, int n_sh, in
     float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs, float* g_sh_rest, float* g_cov3D,
     void* stream);
 
+/* gaussian_topk_weights -- fast_2d_gs/_C/src/gaussian_splatting/gaussian_topk.cu:212-228 (kernel :12-93): per pixel
+ * the topk (<= 16) largest blend weights of the 3D-Gaussian rasteriser and their Gaussian ids, descending;
+ * top_indices[H,W,topk] int32 (-1 = empty slot), top_weights[H,W,topk], both fully written. */
+int fsgs_gaussian_topk_weights(int topk, int P, int W, int H, const float* means2D, const float* conic_opacity,
+    const int64_t* ranges, const int32_t* point_list, int32_t* top_indices, float* top_weights, void* stream);
+
 /* gs_compute_cov3D_forward / gs_compute_cov3D_backward -- fast_2d_gs/_C/src/gaussian_splatting/
  * gaussian_compute_cov3D.cu:122-161: cov3D[N,6] = upper triangle of R(q) diag(s^2) R(q)^T for q[N,4] (x, y, z, w, used as
  * given, not normalised) and s[N,3]; the backward writes g_q[N,4] and g_s[N,3] in full. */

@@ -277,6 +277,15 @@ def gs3d_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotati
     return g3, gs, gq, go, gsh, grest, gcov, gm2
 
 
+def gs3d_topk_weights(topk, W, H, means2D, conic_opacity, ranges, point_list):
+    """gaussian_topk_weights -> (top_indices[H,W,K] int32, top_weights[H,W,K]) (gaussian_topk.cu:212-228)."""
+    ti = np.zeros((H, W, topk), np.int32)
+    tw = np.zeros((H, W, topk), means2D.dtype)
+    assert call(f"gs3d_topk_weights_{_suffix(means2D.dtype)}", topk, W, H, means2D, conic_opacity, ranges, point_list,
+                ti, tw) == 0
+    return ti, tw
+
+
 def gs3d_compute_cov3D(q, s):
     """gs_compute_cov3D_forward(q, s) -> cov3D [N,6] (gaussian_compute_cov3D.cu:122-137)."""
     N = s.shape[0]

@@ -179,6 +179,41 @@ inline bool cov2d_backward(const T* mean, const T* c3, T fx, T fy, T tanx, T tan
   return true;
 }
 
+// gaussian_topk_weights -- gaussian_topk.cu:12-93 (kernel) and :212-228: per pixel the k largest blend weights
+// w = alpha * T of the front-to-back traversal with their Gaussian ids; `w >= slot` takes a slot, so a later Gaussian
+// wins ties; indices start at -1, weights at 0.
+template <typename T>
+void topk_weights(int topk, int W, int H, const T* means2D, const T* conic_opacity, const int64_t* ranges,
+                  const int32_t* point_list, int32_t* top_idx, T* top_w) {
+  const int gx = (W + 15) / 16;
+#pragma omp parallel for schedule(dynamic, 4)
+  for (int py = 0; py < H; ++py)
+    for (int px = 0; px < W; ++px) {
+      const size_t pix = (size_t) py * W + px;
+      int32_t* ti = top_idx + pix * topk;
+      T* tw       = top_w + pix * topk;
+      for (int k = 0; k < topk; ++k) ti[k] = -1, tw[k] = 0;
+      const int tile = (py / 16) * gx + px / 16;
+      T t = 1;
+      for (int64_t e = ranges[2 * tile]; e < ranges[2 * tile + 1]; ++e) {
+        const int id = point_list[e];
+        const T dx = means2D[2 * (size_t) id] - (T) px, dy = means2D[2 * (size_t) id + 1] - (T) py;
+        const T* co = conic_opacity + 4 * (size_t) id;
+        const T power = T(-0.5) * (co[0] * dx * dx + co[2] * dy * dy) - co[1] * dx * dy;
+        if (power > 0) continue;
+        const T alpha = std::min(T(0.99), co[3] * std::exp(power));
+        if (alpha < T(1) / T(255)) continue;
+        const T test_T = t * (1 - alpha);
+        if (test_T < T(0.0001)) break;
+        T w = alpha * t;
+        int idx = id;
+        for (int k = 0; k < topk; ++k)
+          if (w >= tw[k]) std::swap(w, tw[k]), std::swap(idx, ti[k]);
+        t = test_T;
+      }
+    }
+}
+
 // gs_compute_cov3D_forward / _backward (gaussian_compute_cov3D.cu:122-161) and gs_compute_cov2D_forward / _backward
 // (gaussian_compute_cov2D.cu:186-248, without the view-matrix gradient) as stand-alone operators.
 template <typename T>
@@ -455,6 +490,11 @@ using namespace oracle;
     render_backward<T>(W, H, E, means2D, conic_opacity, colors, extras, out_opacity, n_contrib, dL_dpix,             \
                        dL_dout_extras, dL_dout_opacity, point_list, ranges, g_means2D, g_conic_opacity, g_colors,    \
                        g_extras);                                                                                    \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_gs3d_topk_weights_##SUF(int topk, int W, int H, const T* means2D, const T* conic_opacity,    \
+      const int64_t* ranges, const int32_t* point_list, int32_t* top_idx, T* top_w) {                                \
+    topk_weights<T>(topk, W, H, means2D, conic_opacity, ranges, point_list, top_idx, top_w);                         \
     return 0;                                                                                                        \
   }                                                                                                                  \
   ORACLE_API int oracle_gs3d_compute_cov3D_##SUF(int N, const T* q, const T* s, T* cov3D) {                          \

@@ -127,6 +127,24 @@ def test_gs3d_rasterize(P, W, H, E, device):
         assert g_ex is None
 
 
+@pytest.mark.parametrize("K", [1, 4, 7, 16])
+def test_gs3d_topk_weights(K, device):
+    from fast_sp_gs_amd._C import get_C_function
+    P, W, H = 6000, 150, 90
+    m2, col, co, ranges, pl = _binned(P, W, H, 41, device)
+    print(f"[gs3d topk] K={K} P={P} {W}x{H} R={pl.numel()}", flush=True)
+    ti, tw = get_C_function('gaussian_topk_weights')(K, W, H, P, pl.numel(), m2, co, ranges, pl)
+    torch.cuda.synchronize()
+    r_ti, r_tw = O.gs3d_topk_weights(K, W, H, npy(m2), npy(co), npy(ranges), npy(pl))
+    assert abs_err(npy(tw), r_tw) < 1e-5
+    # the same Gaussians in the same slots, except where two weights are equal to rounding or a pair sits on a threshold
+    differ = (npy(ti) != r_ti).any(-1)
+    assert int(differ.sum()) <= max(2, int(2e-3 * W * H)), int(differ.sum())
+    assert (np.diff(npy(tw), axis=-1) <= 0).all() and ((npy(ti) == -1) == (npy(tw) == 0)).all()
+    with pytest.raises(RuntimeError):
+        get_C_function('gaussian_topk_weights')(17, W, H, P, pl.numel(), m2, co, ranges, pl)
+
+
 def test_gs3d_render_autograd_and_empty(device):
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd.renderer import gaussian_render as GR

@@ -122,6 +122,41 @@ def test_render_forward_closed_form_and_compositor():
     assert acc_max.sum() == int((oo > 0).sum()) and acc_n.sum() >= acc_max.sum()
 
 
+def test_topk_weights_are_the_largest_blend_weights():
+    """gaussian_topk_weights against an independent per-pixel pass: collect every contributing (w, id) front to back,
+    sort by weight (a later Gaussian first among equals), keep k."""
+    s, cam, tan_fov = _scene(P=500, size=48, seed=5)
+    m2, dep, col, rad, tt, c3, co = _forward(s, cam, tan_fov)
+    ranges, pl = O.prepare(cam.W, cam.H, m2.astype(np.float32), dep.astype(np.float32), rad, tt)
+    K, W, H = 3, cam.W, cam.H
+    ti, tw = O.gs3d_topk_weights(K, W, H, m2, co, ranges, pl)
+    assert (np.diff(tw, axis=-1) <= 0).all() and ((ti == -1) == (tw == 0)).all()
+    gx, crowded = (W + 15) // 16, 0
+    for y in range(H):
+        for x in range(W):
+            r0, r1 = ranges[(y // 16) * gx + x // 16]
+            T, ws = 1.0, []
+            for order, e in enumerate(range(r0, r1)):
+                i = pl[e]
+                dx, dy = m2[i, 0] - x, m2[i, 1] - y
+                power = -0.5 * (co[i, 0] * dx * dx + co[i, 2] * dy * dy) - co[i, 1] * dx * dy
+                if power > 0:
+                    continue
+                a = min(0.99, co[i, 3] * np.exp(power))
+                if a < 1 / 255:
+                    continue
+                if T * (1 - a) < 1e-4:
+                    break
+                ws.append((a * T, order, i))
+                T *= 1 - a
+            ws.sort(key=lambda t: (-t[0], -t[1]))
+            top = [(w, i) for w, _, i in ws[:K]] + [(0.0, -1)] * (K - len(ws[:K]))
+            assert np.allclose(tw[y, x], [t[0] for t in top], atol=1e-13)
+            assert list(ti[y, x]) == [t[1] for t in top]
+            crowded += len(ws) > K
+    assert crowded > 20
+
+
 def test_render_backward_finite_differences():
     s, cam, tan_fov = _scene(P=150, size=48, seed=5)
     W, H = cam.W, cam.H
