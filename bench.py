@@ -278,6 +278,7 @@ def gs3d_path_rate(dev, scene, cam, gi, steps: int = 30, warmup: int = 5):
                                     None, cam.Tw2v, cam.Tv2c, cam.campos, tan_fov, c3, None, rad, col, g_m2, None, g_col,
                                     g_co, g3, gs, gq, gop, gsh, None, None)
         R[0] = pl.numel()
+        return m2, co, ranges, pl, nc, oo
 
     for _ in range(warmup):
         step()
@@ -286,13 +287,35 @@ def gs3d_path_rate(dev, scene, cam, gi, steps: int = 30, warmup: int = 5):
     gc.disable()
     t0 = time.perf_counter()
     for _ in range(steps):
-        step()
+        state = step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     gc.enable()
+
+    # a 16-channel feature table blended with the finished view's weights, and its backward
+    m2, co, ranges, pl, nc, oo = state
+    feat = torch.randn(scene.P, 16, generator=g).to(dev)
+    g_out = torch.randn(H, W, 16, generator=g).to(dev)
+    g_feat, g_m2, g_co = torch.zeros_like(feat), torch.zeros_like(m2), torch.zeros_like(co)
+    x_f = lambda: f('gaussian_rasterize_extra_forward')(W, H, feat, m2, co, ranges, pl, nc)
+    x_b = lambda: f('gaussian_rasterize_extra_backward')(W, H, feat, oo, g_out, m2, co, ranges, pl, nc, g_feat, g_m2,
+                                                         g_co)
+    x_f(), x_b()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    ev[0].record()
+    for _ in range(10):
+        x_f()
+    ev[1].record()
+    for _ in range(10):
+        x_b()
+    ev[2].record()
+    torch.cuda.synchronize()
     return {"gs3d_path_frames_per_s": steps / dt,
             "gs3d_path_workload": f"same 300k centres as 3D Gaussians (third scale added), 800x800, SH degree 3, "
-                                  f"R = {R[0]}: gs_preprocess fwd/bwd + GS_prepare + gaussian_rasterize fwd/bwd"}
+                                  f"R = {R[0]}: gs_preprocess fwd/bwd + GS_prepare + gaussian_rasterize fwd/bwd",
+            "gs3d_extra16_forward_ms": ev[0].elapsed_time(ev[1]) / 10,
+            "gs3d_extra16_backward_ms": ev[1].elapsed_time(ev[2]) / 10,
+            "gs3d_extra16_workload": "gaussian_rasterize_extra_forward / _backward, a [300000,16] table on that view"}
 
 
 def density_control_ms(dev, scene, reps: int = 5):

@@ -27,7 +27,8 @@ __all__ = [
     'gs_preprocess_backward', 'gaussian_rasterize_forward', 'gaussian_rasterize_backward', 'select_indices',
     'gather_rows', 'densify_masks', 'prune_mask', 'split_children', 'densification_stats',
     'gs_compute_cov3D_forward', 'gs_compute_cov3D_backward', 'gs_compute_cov2D_forward', 'gs_compute_cov2D_backward',
-    'gaussian_topk_weights',
+    'gaussian_topk_weights', 'gaussian_rasterize_extra_forward', 'gaussian_rasterize_extra_backward',
+    'gaussian_rasterize_extra_backward_v2',
 ]
 
 _TILE = 16
@@ -1360,6 +1361,71 @@ def gaussian_topk_weights(topk: int, W: int, H: int, P: int, R: int, means2D: Te
                                                L.ptr(top_weights), L.current_stream())
     L.check(rc, what)
     return top_indices, top_weights
+
+
+def gaussian_rasterize_extra_forward(W: int, H: int, extras: Tensor, means2D: Tensor, conic_opacity: Tensor,
+                                     ranges: Tensor, point_list: Tensor, n_contrib: Tensor) -> Tensor:
+    """gaussian_rasterizer_extra.cu:317-339: extras[P,E] -> pixel_extras[H,W,E] with the blend weights of the main pass."""
+    what = 'gaussian_rasterize_extra_forward'
+    extras = extras.contiguous()  # as the reference's host function does
+    _f32(what, extras=extras, means2D=means2D, conic_opacity=conic_opacity)
+    L.require_cuda(what, ranges=ranges, point_list=point_list, n_contrib=n_contrib)
+    L.require_dtype(what, 'ranges', ranges, torch.int64)
+    L.require_dtype(what, 'point_list', point_list, torch.int32)
+    L.require_dtype(what, 'n_contrib', n_contrib, torch.int32)
+    if extras.ndim != 2:
+        raise RuntimeError(f'{what}: Error shape for extras')
+    P, E = extras.shape
+    if means2D.shape[0] != P or conic_opacity.shape[0] != P or n_contrib.numel() != W * H:
+        raise RuntimeError(f'{what}: extras, means2D, conic_opacity share P and n_contrib is [H,W]')
+    out = torch.empty((H, W, E), dtype=torch.float32, device=extras.device)
+    if E == 0:
+        return out
+    with _timed(what):
+        rc = _lib().fsgs_gaussian_rasterize_extra_forward(
+            P, W, H, E, L.ptr(extras), L.ptr(means2D), L.ptr(conic_opacity), L.ptr(ranges),
+            L.ptr(point_list), L.ptr(n_contrib), L.ptr(out), L.current_stream())
+    L.check(rc, what)
+    return out
+
+
+def gaussian_rasterize_extra_backward(W: int, H: int, extras: Tensor, out_opacity: Tensor, grad_out: Tensor,
+                                      means2D: Tensor, conic_opacity: Tensor, ranges: Tensor, point_list: Tensor,
+                                      n_contrib: Tensor, grad_extra: Optional[Tensor], grad_means2D: Optional[Tensor],
+                                      grad_conic: Optional[Tensor]) -> None:
+    """gaussian_rasterizer_extra.cu:341-365: adds into the gradient tensors that are given."""
+    what = 'gaussian_rasterize_extra_backward'
+    extras, grad_out = extras.contiguous(), grad_out.contiguous()  # as the reference's host function does
+    _f32(what, extras=extras, out_opacity=out_opacity, grad_out=grad_out, means2D=means2D,
+         conic_opacity=conic_opacity, grad_extra=grad_extra, grad_means2D=grad_means2D, grad_conic=grad_conic)
+    L.require_cuda(what, ranges=ranges, point_list=point_list, n_contrib=n_contrib)
+    L.require_dtype(what, 'ranges', ranges, torch.int64)
+    L.require_dtype(what, 'point_list', point_list, torch.int32)
+    L.require_dtype(what, 'n_contrib', n_contrib, torch.int32)
+    P, E = extras.shape
+    if grad_out.numel() != W * H * E or out_opacity.numel() != W * H or n_contrib.numel() != W * H:
+        raise RuntimeError(f'{what}: grad_out is [H,W,E], out_opacity and n_contrib are [H,W]')
+    for name, g, like in (('grad_extra', grad_extra, extras), ('grad_means2D', grad_means2D, means2D),
+                          ('grad_conic', grad_conic, conic_opacity)):
+        if g is not None and (tuple(g.shape) != tuple(like.shape) or not g.is_contiguous()):
+            raise RuntimeError(f'{what}: {name} must be contiguous and shaped like its input')
+    if E == 0:
+        return
+    with _timed(what):
+        rc = _lib().fsgs_gaussian_rasterize_extra_backward(
+            P, W, H, E, L.ptr(extras), L.ptr(out_opacity), L.ptr(grad_out), L.ptr(means2D),
+            L.ptr(conic_opacity), L.ptr(ranges), L.ptr(point_list), L.ptr(n_contrib), L.ptr(grad_extra),
+            L.ptr(grad_means2D), L.ptr(grad_conic), L.current_stream())
+    L.check(rc, what)
+
+
+def gaussian_rasterize_extra_backward_v2(W, H, extras, out_opacity, grad_out, means2D, conic_opacity, ranges,
+                                         point_list, n_contrib, grad_extra, grad_means2D, grad_conic) -> None:
+    """gaussian_rasterizer_extra.cu:367-391: the variant that assumes all three gradient tensors are given."""
+    if grad_extra is None or grad_means2D is None or grad_conic is None:
+        raise RuntimeError('gaussian_rasterize_extra_backward_v2: all three gradient tensors are required')
+    gaussian_rasterize_extra_backward(W, H, extras, out_opacity, grad_out, means2D, conic_opacity, ranges, point_list,
+                                      n_contrib, grad_extra, grad_means2D, grad_conic)
 
 
 def gs_compute_cov3D_forward(q: Tensor, s: Tensor) -> Tensor:

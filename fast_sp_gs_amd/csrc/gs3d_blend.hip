@@ -401,6 +401,227 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
   }
 }
 
+// Largest n_contrib of the tile's 256 pixels: no pixel looks past that list position.
+__device__ __forceinline__ int block_max_contrib(int last_contrib, int* s_max) {
+  if (threadIdx.x == 0) *s_max = 0;
+  __syncthreads();
+  int wave_max = last_contrib;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) wave_max = max(wave_max, __shfl_xor(wave_max, d, kWave));
+  if ((threadIdx.x & 63) == 0) atomicMax(s_max, wave_max);
+  __syncthreads();
+  return *s_max;
+}
+
+// Feature channels [e0, e0 + kC) of an arbitrary-width per-Gaussian table blended with the weights of the main forward
+// pass (gaussian_rasterizer_extra.cu:12-101): the traversal stops at the pixel's n_contrib. blockIdx.y selects the group
+// of channels, so groups run side by side where the reference walks the list once per group in sequence. Output is
+// pixel-major [H, W, E].
+template <int kC>
+__global__ void __launch_bounds__(kBlendThreads) gs3d_extra_forward_kernel(int flags, int W, int H, int E,
+    const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
+    const float4* __restrict__ conic_opacity, const int32_t* __restrict__ n_contrib, const float* __restrict__ extras,
+    float* __restrict__ out) {
+  constexpr int kHalf = kC / 2;  // two threads gather one Gaussian's channels
+  __shared__ G3Hot s_hot[kG3Batch];
+  __shared__ float s_feat[kG3Batch][kC + 1];
+  __shared__ int s_max_contrib;
+  const int gx = (W + kTile - 1) / kTile;
+  const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
+  int px, py;
+  lane_pixel(tile_x, tile_y, px, py);
+  const bool inside = px < W && py < H;
+  const size_t pix  = (size_t) W * py + px;
+  const float pxf = (float) px, pyf = (float) py;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int e0 = blockIdx.y * kC, n_ch = min(kC, E - e0);
+  const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
+  const int last_contrib = inside ? n_contrib[pix] : 0;
+  const int n_todo = min(block_max_contrib(last_contrib, &s_max_contrib), (int) (r1 - r0));
+  const int rounds = (n_todo + kG3Batch - 1) / kG3Batch;
+  const int slot = threadIdx.x & (kG3Batch - 1), half = threadIdx.x / kG3Batch;
+
+  bool done = last_contrib == 0;
+  float T = 1.0f, C[kC];
+#pragma unroll
+  for (int k = 0; k < kC; ++k) C[k] = 0.0f;
+
+  for (int b = 0; b < rounds; ++b) {
+    if (__syncthreads_count(done) == kBlendThreads) break;
+    const int n_here = min(kG3Batch, n_todo - b * kG3Batch);
+    if (slot < n_here) {
+      const int id = point_list[r0 + b * kG3Batch + slot];
+      if (half == 0) {
+        const float2 c  = means2D[id];
+        const float4 co = conic_opacity[id];
+        G3Hot h;
+        h.x = c.x, h.y = c.y, h.a = co.x, h.b = co.y, h.c = co.z, h.opacity = co.w, h.id = id;
+        h.mask = conic_quadrant_mask(h, tile_x * kTile, tile_y * kTile, flags);
+        s_hot[slot] = h;
+      }
+#pragma unroll
+      for (int k = half * kHalf; k < half * kHalf + kHalf; ++k)
+        s_feat[slot][k] = k < n_ch ? extras[(size_t) E * id + e0 + k] : 0.0f;
+    }
+    __syncthreads();
+    for (int c = 0; c < kG3Batch / kWave; ++c) {
+      const int jj = c * kWave + lane;
+      unsigned long long todo = __ballot(jj < n_here && ((s_hot[jj < kG3Batch ? jj : 0].mask >> wave) & 1u));
+      while (todo) {
+        if (__ballot(!done) == 0ull) break;
+        const int j = c * kWave + __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const int pos = b * kG3Batch + j;  // 0-based position in the tile's list
+        done = done || pos >= last_contrib;
+        G3Hit h;
+        const bool hit = conic_alpha_flat(s_hot[j], pxf, pyf, h) && !done;
+        if (__ballot(hit) == 0ull) continue;
+        const float test_T = T * (1.0f - h.alpha);
+        const bool sat     = hit && test_T < 0.0001f;
+        done               = done || sat;
+        if (hit && !sat) {
+          const float w = h.alpha * T;
+#pragma unroll
+          for (int k = 0; k < kC; ++k) C[k] = fmaf(s_feat[j][k], w, C[k]);
+          T = test_T;
+        }
+      }
+    }
+  }
+  if (inside) {
+    float* o = out + pix * E + e0;
+    if ((E & 3) == 0) {
+#pragma unroll
+      for (int k = 0; k < kC; k += 4)
+        if (k < n_ch) *reinterpret_cast<float4*>(o + k) = make_float4(C[k], C[k + 1], C[k + 2], C[k + 3]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < kC; ++k)
+        if (k < n_ch) o[k] = C[k];
+    }
+  }
+}
+
+// Backward of the feature-channel blend (gaussian_rasterizer_extra.cu:103-209), 8 channels per block: back to front from
+// T_final = 1 - out_opacity without the background and opacity terms of the main backward. Each block adds its group's
+// share of the mean / conic / opacity gradients, as each of the reference's sequential groups does.
+// gradient slots of one Gaussian: 0-7 channels | 8-9 mean2D | 10-12 conic | 13 opacity | 14-15 unused
+__global__ void __launch_bounds__(kBlendThreads) gs3d_extra_backward_kernel(int flags, int W, int H, int E,
+    const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
+    const float4* __restrict__ conic_opacity, const float* __restrict__ out_opacity,
+    const int32_t* __restrict__ n_contrib, const float* __restrict__ extras, const float* __restrict__ dL_dout,
+    float* __restrict__ g_means2D, float* __restrict__ g_conic_opacity, float* __restrict__ g_extras) {
+  constexpr int kB = 64, kC = 8, kPart = kC / 4;  // four threads gather one Gaussian's channels
+  __shared__ G3Hot s_hot[kB];
+  __shared__ float s_feat[kB][kC + 1];
+  __shared__ float s_acc[kB][17];
+  __shared__ int s_max_contrib;
+  const int gx = (W + kTile - 1) / kTile;
+  const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
+  int px, py;
+  lane_pixel(tile_x, tile_y, px, py);
+  const bool inside = px < W && py < H;
+  const size_t pix  = (size_t) W * py + px;
+  const float pxf = (float) px, pyf = (float) py;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int e0 = blockIdx.y * kC, n_ch = min(kC, E - e0);
+  const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
+  const int last_contrib = inside ? n_contrib[pix] : 0;
+  if ((int) threadIdx.x < kB)
+#pragma unroll
+    for (int c = 0; c < 17; ++c) s_acc[threadIdx.x][c] = 0.0f;
+  const int n_todo = min(block_max_contrib(last_contrib, &s_max_contrib), (int) (r1 - r0));
+  const int rounds = (n_todo + kB - 1) / kB;
+  int wave_max = last_contrib;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) wave_max = max(wave_max, __shfl_xor(wave_max, d, kWave));
+
+  float T = inside ? 1.0f - out_opacity[pix] : 0.0f;
+  float g_out[kC], accum[kC];
+#pragma unroll
+  for (int k = 0; k < kC; ++k) {
+    accum[k] = 0.0f;
+    g_out[k] = (inside && k < n_ch) ? dL_dout[pix * E + e0 + k] : 0.0f;
+  }
+  const int slot = threadIdx.x & (kB - 1), part = threadIdx.x / kB;
+
+  for (int b = 0; b < rounds; ++b) {
+    const int n_here = min(kB, n_todo - b * kB);
+    if (slot < n_here) {
+      const int id = point_list[r0 + (n_todo - 1 - (b * kB + slot))];
+      if (part == 0) {
+        const float2 c  = means2D[id];
+        const float4 co = conic_opacity[id];
+        G3Hot h;
+        h.x = c.x, h.y = c.y, h.a = co.x, h.b = co.y, h.c = co.z, h.opacity = co.w, h.id = id;
+        h.mask = conic_quadrant_mask(h, tile_x * kTile, tile_y * kTile, flags);
+        s_hot[slot] = h;
+      }
+#pragma unroll
+      for (int k = part * kPart; k < part * kPart + kPart; ++k)
+        s_feat[slot][k] = k < n_ch ? extras[(size_t) E * id + e0 + k] : 0.0f;
+    }
+    __syncthreads();
+    unsigned long long todo = __ballot(lane < n_here && ((s_hot[lane].mask >> wave) & 1u) &&
+                                       (n_todo - 1 - (b * kB + lane)) < wave_max);
+    while (todo) {
+      const int j = __builtin_ctzll(todo);
+      todo &= todo - 1;
+      const int pos = n_todo - 1 - (b * kB + j);  // 0-based position in the tile's list
+      G3Hit h;
+      const bool hit = conic_alpha_flat(s_hot[j], pxf, pyf, h) && (pos < last_contrib);
+      if (__ballot(hit) == 0ull) continue;
+      float g[16];
+#pragma unroll
+      for (int c = 0; c < 16; ++c) g[c] = 0.0f;
+      if (hit) {
+        const G3Hot& hot = s_hot[j];
+        T = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+        const float dch = h.alpha * T;
+        float dL_dalpha = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kC; ++k) {
+          const float v = s_feat[j][k];
+          dL_dalpha += (v * T * (1.0f - h.alpha) - accum[k]) * g_out[k];
+          accum[k] += v * dch;
+          g[k] = dch * g_out[k];
+        }
+        dL_dalpha = dL_dalpha * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+        const float dL_dG = -hot.opacity * h.G * dL_dalpha;
+        g[8]  = dL_dG * (hot.a * h.dx + hot.b * h.dy);
+        g[9]  = dL_dG * (hot.c * h.dy + hot.b * h.dx);
+        g[10] = 0.5f * h.dx * h.dx * dL_dG;
+        g[11] = h.dx * h.dy * dL_dG;
+        g[12] = 0.5f * h.dy * h.dy * dL_dG;
+        g[13] = h.G * dL_dalpha;
+      }
+      const float tot = wave_sum16_transposed(g);
+      if (lane < 16) atomicAdd(&s_acc[j][lane], tot);
+    }
+    __syncthreads();
+    if ((int) threadIdx.x < n_here) {
+      float* a = s_acc[threadIdx.x];
+      const int id = s_hot[threadIdx.x].id;
+      if (g_extras)
+#pragma unroll
+        for (int c = 0; c < kC; ++c)
+          if (c < n_ch && a[c] != 0.0f) atomicAdd(&g_extras[(size_t) E * id + e0 + c], a[c]);
+      if (g_means2D)
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+          if (a[8 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[8 + c]);
+      if (g_conic_opacity)
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (a[10 + c] != 0.0f) atomicAdd(&g_conic_opacity[4 * (size_t) id + c], a[10 + c]);
+#pragma unroll
+      for (int c = 0; c < 16; ++c) a[c] = 0.0f;
+    }
+    // between this flush and the barrier after the next batch's LDS store a lane touches its own accumulator row and
+    // its own s_hot entry only; s_feat was last read before the barrier above
+  }
+}
+
 }  // namespace
 }  // namespace fsgs
 
@@ -487,4 +708,44 @@ FSGS_API int fsgs_gaussian_topk_weights(int topk, int P, int W, int H, const flo
   else FSGS_TOPK3(16);
 #undef FSGS_TOPK3
   return check_launch("gaussian_topk_weights");
+}
+
+FSGS_API int fsgs_gaussian_rasterize_extra_forward(int P, int W, int H, int E, const float* extras,
+    const float* means2D, const float* conic_opacity, const int64_t* ranges, const int32_t* point_list,
+    const int32_t* n_contrib, float* out_pixels, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && E > 0, "gaussian_rasterize_extra_forward: bad sizes");
+  FSGS_REQUIRE(ranges && n_contrib && out_pixels, "gaussian_rasterize_extra_forward: null pointer");
+  FSGS_REQUIRE(P == 0 || (extras && means2D && conic_opacity && point_list),
+               "gaussian_rasterize_extra_forward: null pointer");
+  FSGS_REQUIRE((E & 3) != 0 || (reinterpret_cast<uintptr_t>(out_pixels) & 15) == 0,
+               "gaussian_rasterize_extra_forward: out_pixels must be 16-byte aligned");
+  hipStream_t s = (hipStream_t) stream;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const int flags = launch_tile_order(gx, gy, ranges, s);
+  const dim3 block(kBlendThreads);
+#define FSGS_G3_EXTRA(CC)                                                                                          \
+  hipLaunchKernelGGL((gs3d_extra_forward_kernel<CC>), dim3(gx * gy, (E + CC - 1) / CC), block, 0, s, flags, W, H,  \
+                     E, ranges, point_list, (const float2*) means2D, (const float4*) conic_opacity, n_contrib,     \
+                     extras, out_pixels)
+  if (E <= 8) FSGS_G3_EXTRA(8);
+  else FSGS_G3_EXTRA(16);
+#undef FSGS_G3_EXTRA
+  return check_launch("gaussian_rasterize_extra_forward");
+}
+
+FSGS_API int fsgs_gaussian_rasterize_extra_backward(int P, int W, int H, int E, const float* extras,
+    const float* out_opacity, const float* grad_out, const float* means2D, const float* conic_opacity,
+    const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib, float* grad_extras,
+    float* grad_means2D, float* grad_conic_opacity, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && E > 0, "gaussian_rasterize_extra_backward: bad sizes");
+  if (P == 0 || (!grad_extras && !grad_means2D && !grad_conic_opacity)) return kOk;
+  FSGS_REQUIRE(extras && out_opacity && grad_out && means2D && conic_opacity && ranges && point_list && n_contrib,
+               "gaussian_rasterize_extra_backward: null pointer");
+  hipStream_t s = (hipStream_t) stream;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const int flags = launch_tile_order(gx, gy, ranges, s);
+  hipLaunchKernelGGL(gs3d_extra_backward_kernel, dim3(gx * gy, (E + 7) / 8), dim3(kBlendThreads), 0, s, flags, W, H, E,
+                     ranges, point_list, (const float2*) means2D, (const float4*) conic_opacity, out_opacity,
+                     n_contrib, extras, grad_out, grad_means2D, grad_conic_opacity, grad_extras);
+  return check_launch("gaussian_rasterize_extra_backward");
 }

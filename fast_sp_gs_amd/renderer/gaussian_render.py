@@ -1,8 +1,8 @@
 """Host side of the 3D-Gaussian (EWA) render path on the HIP operators: the autograd wiring and entry points of the
 reference's fast_2d_gs/renderer/gaussian_render.py (`_preprocess` :495-566, `preprocess` :569-, `GS_prepare` :742-772,
 `_GS_render` :775-800, `GS_render` :840-, `RasterizeGaussians` :226-274, `render` :277-359) for covariances computed
-from scales + rotations. Extra feature channels beyond the first group of <= 4 (`render_extra`), pre-computed
-covariances and camera gradients are not part of this build and raise."""
+from scales + rotations, and `_render_extra` / `render_extra` :925-962 for further feature tables of any width.
+Pre-computed covariances and camera gradients are not part of this build and raise."""
 from __future__ import annotations
 
 from typing import NamedTuple, Optional, Tuple
@@ -14,7 +14,7 @@ from fast_sp_gs_amd._C import get_C_function
 from fast_sp_gs_amd.renderer.gs_2d_render import GS_prepare
 
 __all__ = ['RasterizeBuffer3D', 'preprocess', 'GS_render', 'RasterizeGaussians', 'render', 'compute_cov3D',
-           'compute_cov2D', 'topk_weights']
+           'compute_cov2D', 'topk_weights', 'render_extra']
 
 
 class RasterizeBuffer3D(NamedTuple):
@@ -35,6 +35,42 @@ def topk_weights(topk: int, buffer: RasterizeBuffer3D) -> Tuple[Tensor, Tensor]:
     """Per-pixel top-k Gaussian indices and blend weights of a rendered view (reference: gaussian_render.py:362-367)."""
     return get_C_function('gaussian_topk_weights')(topk, buffer.W, buffer.H, buffer.P, buffer.R, buffer.means2D,
                                                    buffer.conic_opacity, buffer.tile_ranges, buffer.point_list)
+
+
+class _render_extra(torch.autograd.Function):
+    """renderer/gaussian_render.py:925-949 of the reference."""
+
+    @staticmethod
+    def forward(ctx, W, H, extras, means2D, conic_opacity, ranges, point_list, n_contrib, out_opacity):
+        extras = extras.contiguous()
+        out_pixels = get_C_function('gaussian_rasterize_extra_forward')(W, H, extras, means2D, conic_opacity, ranges,
+                                                                        point_list, n_contrib)
+        ctx.save_for_backward(out_opacity, extras, means2D, conic_opacity, ranges, point_list, n_contrib)
+        return out_pixels
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_out):
+        out_opacity, extras, means2D, conic_opacity, ranges, point_list, n_contrib = ctx.saved_tensors
+        H, W = out_opacity.shape
+        grad_extra = torch.zeros_like(extras) if ctx.needs_input_grad[2] else None
+        grad_means2D = torch.zeros_like(means2D) if ctx.needs_input_grad[3] else None
+        grad_conic = torch.zeros_like(conic_opacity) if ctx.needs_input_grad[4] else None
+        get_C_function('gaussian_rasterize_extra_backward')(
+            W, H, extras, out_opacity, grad_out, means2D, conic_opacity, ranges, point_list, n_contrib, grad_extra,
+            grad_means2D, grad_conic)
+        return None, None, grad_extra, grad_means2D, grad_conic, None, None, None, None
+
+
+def render_extra(buffer: RasterizeBuffer3D, *args: Tensor, detach=False):
+    """Blends further per-Gaussian tables [P,E] with a rendered view's weights -> [H,W,E] each (reference:
+    gaussian_render.py:952-962); `detach` keeps the gradient away from the geometry."""
+    means2D, conic_opacity = buffer.means2D, buffer.conic_opacity
+    if detach:
+        means2D, conic_opacity = means2D.detach(), conic_opacity.detach()
+    outputs = [_render_extra.apply(buffer.W, buffer.H, x, means2D, conic_opacity, buffer.tile_ranges, buffer.point_list,
+                                   buffer.n_contribed, buffer.opacity) for x in args]
+    return outputs[0] if len(args) == 1 else outputs
 
 
 class _compute_cov3D(torch.autograd.Function):
@@ -191,8 +227,6 @@ def RasterizeGaussians(means3D: Tensor, means2D: Optional[Tensor], colors: Tenso
                        tanFoV: Tensor, is_opengl: bool, culling: Optional[Tensor], accum_max_count: Optional[Tensor],
                        accum_weights_p: Optional[Tensor], accum_weights_count: Optional[Tensor], *other_extras: Tensor):
     """gaussian_render.py:226-274: preprocess -> binning -> blend."""
-    if other_extras:
-        raise RuntimeError('RasterizeGaussians: additional extra groups (render_extra) are not supported by this library')
     W, H = image_size
     means2D, depths, colors, radii, tiles_touched, conic_opacity = preprocess(
         means3D, scales, rotations, opacities, colors, sh_rest, Tw2v, Tv2c, cam_pos, tanFoV, W, H, sh_degree,
@@ -203,7 +237,9 @@ def RasterizeGaussians(means3D: Tensor, means2D: Optional[Tensor], colors: Tenso
         accum_weights_count)
     buffer = RasterizeBuffer3D(W, H, len(opacities), point_list.shape[0], tile_ranges, point_list, n_contrib,
                                conic_opacity, means2D, out_opacities)
-    return out_pixels, out_opacities, out_extras, radii, buffer
+    out_other_extras = [_render_extra.apply(W, H, extras_, means2D, conic_opacity, tile_ranges, point_list, n_contrib,
+                                            out_opacities) for extras_ in other_extras]
+    return (out_pixels, out_opacities, out_extras, radii, buffer, *out_other_extras)
 
 
 def render(Tw2v: Tensor, Tv2c: Tensor, size: Tuple[int, int], points: Tensor, opacity: Tensor, scales: Tensor = None,
@@ -227,14 +263,16 @@ def render(Tw2v: Tensor, Tv2c: Tensor, size: Tuple[int, int], points: Tensor, op
             kwargs.pop(k)
             break
     c = lambda t: None if t is None else t.contiguous()
-    image, out_opacity, out_extra, radii, buffer = RasterizeGaussians(
+    others = {k: v for k, v in kwargs.items() if isinstance(v, Tensor)}
+    image, out_opacity, out_extra, radii, buffer, *out_others = RasterizeGaussians(
         points.contiguous(), means2D, c(sh_features) if colors is None else colors.contiguous(), c(sh_features_rest),
         opacity.contiguous(), c(scales), c(rotations), c(cov3Ds), c(cov2Ds), c(extras), size,
         sh_degree if colors is None else -1, Tw2v.view(4, 4).contiguous(), Tv2c.view(4, 4).contiguous(),
         campos.view(3).contiguous(), tanFoV.view(2), is_opengl, culling, accum_max_count, accum_weights_p,
-        accum_weights_count, *[v for v in kwargs.values() if isinstance(v, Tensor)])
+        accum_weights_count, *others.values())
     out = {'images': image, 'opacity': out_opacity, 'viewspace_points': means2D, 'visibility_filter': radii > 0,
            'radii': radii, 'buffer': buffer}
+    out.update(zip(others.keys(), out_others))  # each [H,W,E], pixel-major as in the reference
     if extra_key is not None:
         out[extra_key] = out_extra
     return out

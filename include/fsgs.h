@@ -300,6 +300,21 @@ int fsgs_gs_preprocess_backward(int P, int W, int H, int sh_degree, int n_sh, in
 int fsgs_gaussian_topk_weights(int topk, int P, int W, int H, const float* means2D, const float* conic_opacity,
     const int64_t* ranges, const int32_t* point_list, int32_t* top_indices, float* top_weights, void* stream);
 
+/* gaussian_rasterize_extra_forward / gaussian_rasterize_extra_backward -- fast_2d_gs/_C/src/gaussian_splatting/
+ * gaussian_rasterizer_extra.cu:317-339 and :341-365 (kernels :12-101, :103-209; bound by
+ * renderer/gaussian_render.py:925-949): any number E >= 1 of per-Gaussian feature channels extras[P,E] blended with the
+ * weights of a finished gaussian_rasterize_forward, whose n_contrib[H,W] bounds each pixel's traversal and whose
+ * out_opacity[H,W] seeds the backward. out_pixels[H,W,E] is pixel-major and fully written (16-byte aligned when E is a
+ * multiple of 4). The backward takes grad_out[H,W,E] and ADDS into whichever of grad_extras[P,E], grad_means2D[P,2],
+ * grad_conic_opacity[P,4] is non-null (the reference's optional tensors); with all three null it does nothing. */
+int fsgs_gaussian_rasterize_extra_forward(int P, int W, int H, int E, const float* extras, const float* means2D,
+    const float* conic_opacity, const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib,
+    float* out_pixels, void* stream);
+int fsgs_gaussian_rasterize_extra_backward(int P, int W, int H, int E, const float* extras, const float* out_opacity,
+    const float* grad_out, const float* means2D, const float* conic_opacity, const int64_t* ranges,
+    const int32_t* point_list, const int32_t* n_contrib, float* grad_extras, float* grad_means2D,
+    float* grad_conic_opacity, void* stream);
+
 /* gs_compute_cov3D_forward / gs_compute_cov3D_backward -- fast_2d_gs/_C/src/gaussian_splatting/
  * gaussian_compute_cov3D.cu:122-161: cov3D[N,6] = upper triangle of R(q) diag(s^2) R(q)^T for q[N,4] (x, y, z, w, used as
  * given, not normalised) and s[N,3]; the backward writes g_q[N,4] and g_s[N,3] in full. */

@@ -277,6 +277,29 @@ def gs3d_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotati
     return g3, gs, gq, go, gsh, grest, gcov, gm2
 
 
+def gs3d_extra_forward(W, H, extras, means2D, conic_opacity, ranges, point_list, n_contrib):
+    """gaussian_rasterize_extra_forward -> pixel_extras [H,W,E] (gaussian_rasterizer_extra.cu:317-339)."""
+    E = extras.shape[1]
+    out = np.zeros((H, W, E), extras.dtype)
+    assert call(f"gs3d_extra_forward_{_suffix(extras.dtype)}", W, H, E, extras, means2D, conic_opacity, ranges,
+                point_list, n_contrib, out) == 0
+    return out
+
+
+def gs3d_extra_backward(W, H, extras, out_opacity, grad_out, means2D, conic_opacity, ranges, point_list, n_contrib,
+                        want=(True, True, True)):
+    """gaussian_rasterize_extra_backward -> (g_extras, g_means2D, g_conic_opacity), None where not wanted
+    (gaussian_rasterizer_extra.cu:341-365)."""
+    P, E = extras.shape
+    dt = extras.dtype
+    ge = np.zeros((P, E), dt) if want[0] else None
+    gm = np.zeros((P, 2), dt) if want[1] else None
+    gc = np.zeros((P, 4), dt) if want[2] else None
+    assert call(f"gs3d_extra_backward_{_suffix(dt)}", W, H, E, extras, out_opacity, np.ascontiguousarray(grad_out),
+                means2D, conic_opacity, ranges, point_list, n_contrib, ge, gm, gc) == 0
+    return ge, gm, gc
+
+
 def gs3d_topk_weights(topk, W, H, means2D, conic_opacity, ranges, point_list):
     """gaussian_topk_weights -> (top_indices[H,W,K] int32, top_weights[H,W,K]) (gaussian_topk.cu:212-228)."""
     ti = np.zeros((H, W, topk), np.int32)

@@ -4,6 +4,7 @@
 //   3D covariance forward/backward  gaussian_compute_cov3D.cu:18-36, :76-118
 //   2D covariance forward/backward  gaussian_compute_cov2D.cu:18-62, :64-186
 //   rasterise forward / backward    gaussian_render.cu:20-173, :296-444
+//   feature-channel blend fwd/bwd   gaussian_rasterizer_extra.cu:12-101, :103-209
 // Scope: covariances from scales + rotations (no pre-computed cov3D / cov2D), no camera gradients.
 //
 // Pinned by tests/test_oracle_gs3d.py: cov3D = R S^2 R^T and cov2D = J W cov3D W^T J^T + 0.3 I with numpy, the conic as
@@ -450,6 +451,96 @@ void render_backward(int W, int H, int E, const T* means2D, const T* conic_opaci
     }
 }
 
+// gaussian_rasterize_extra_forward -- gaussian_rasterizer_extra.cu:12-101 (kernel), :317-339 (host): any number of
+// per-Gaussian feature channels blended with the weights of the main forward pass, whose n_contrib bounds the
+// traversal; output pixel-major [H, W, E]. The reference walks the list once per group of 16 channels; the weights do not
+// depend on the group, so one walk is the same computation.
+template <typename T>
+void extra_forward(int W, int H, int E, const T* extras, const T* means2D, const T* conic_opacity,
+                   const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib, T* out) {
+  const int gx = (W + kTile - 1) / kTile;
+  for (int py = 0; py < H; ++py)
+    for (int px = 0; px < W; ++px) {
+      const int tile = (py / kTile) * gx + px / kTile;
+      const size_t pix = (size_t) py * W + px;
+      const int last = n_contrib[pix];
+      std::vector<T> acc(E, T(0));
+      T t = 1;
+      int contributor = 0;
+      for (int64_t e = ranges[2 * tile]; e < ranges[2 * tile + 1]; ++e) {
+        if (++contributor > last) break;
+        const int id = point_list[e];
+        const T dx = means2D[2 * (size_t) id] - T(px), dy = means2D[2 * (size_t) id + 1] - T(py);
+        const T* co = conic_opacity + 4 * (size_t) id;
+        const T power = T(-0.5) * (co[0] * dx * dx + co[2] * dy * dy) - co[1] * dx * dy;
+        if (power > T(0.0)) continue;
+        const T alpha = std::min(T(0.99), co[3] * std::exp(power));
+        if (alpha < T(1.0 / 255.0)) continue;
+        const T test_T = t * (1 - alpha);
+        if (test_T < T(0.0001)) break;
+        for (int c = 0; c < E; ++c) acc[c] += extras[(size_t) E * id + c] * alpha * t;
+        t = test_T;
+      }
+      for (int c = 0; c < E; ++c) out[pix * E + c] = acc[c];
+    }
+}
+
+// gaussian_rasterize_extra_backward -- gaussian_rasterizer_extra.cu:103-209 (kernel), :341-365 (host): back to front
+// from T_final = 1 - out_opacity, entries behind n_contrib skipped, no background and no opacity term. Each of the three
+// gradients is optional and accumulated into. The reference adds the mean / conic / opacity gradient once per group of
+// 16 channels; the sum over groups is the single sum over all channels taken here.
+template <typename T>
+void extra_backward(int W, int H, int E, const T* extras, const T* out_opacity, const T* grad_out, const T* means2D,
+                    const T* conic_opacity, const int64_t* ranges, const int32_t* point_list,
+                    const int32_t* n_contrib, T* g_extras, T* g_means2D, T* g_conic_opacity) {
+  const int gx = (W + kTile - 1) / kTile;
+  for (int py = 0; py < H; ++py)
+    for (int px = 0; px < W; ++px) {
+      const int tile = (py / kTile) * gx + px / kTile;
+      const int64_t r0 = ranges[2 * tile], r1 = ranges[2 * tile + 1];
+      const size_t pix = (size_t) py * W + px;
+      T t = T(1.0) - out_opacity[pix];
+      const int last = n_contrib[pix];
+      std::vector<T> accum(E, T(0));
+      const T* g = grad_out + pix * E;
+      int contributor = (int) (r1 - r0);
+      for (int64_t e = r1 - 1; e >= r0; --e) {
+        --contributor;
+        if (contributor >= last) continue;
+        const int id = point_list[e];
+        const T dx = means2D[2 * (size_t) id] - T(px), dy = means2D[2 * (size_t) id + 1] - T(py);
+        const T* co = conic_opacity + 4 * (size_t) id;
+        const T power = T(-0.5) * (co[0] * dx * dx + co[2] * dy * dy) - co[1] * dx * dy;
+        if (power > T(0.0)) continue;
+        const T G = std::exp(power);
+        const T alpha = std::min(T(0.99), co[3] * G);
+        if (alpha < T(1.0 / 255.0)) continue;
+        t = t / (T(1.0) - alpha);
+        const T dch = alpha * t;
+        T dL_dalpha = 0;
+        for (int c = 0; c < E; ++c) {
+          const T v = extras[(size_t) E * id + c];
+          dL_dalpha += (v * t * (T(1.0) - alpha) - accum[c]) * g[c];
+          accum[c] += v * dch;
+          if (g_extras) g_extras[(size_t) E * id + c] += dch * g[c];
+        }
+        dL_dalpha = dL_dalpha / (T(1.0) - alpha);
+        const T dL_dG = -co[3] * G * dL_dalpha;
+        if (g_means2D) {
+          g_means2D[2 * (size_t) id] += dL_dG * (co[0] * dx + co[1] * dy);
+          g_means2D[2 * (size_t) id + 1] += dL_dG * (co[2] * dy + co[1] * dx);
+        }
+        if (g_conic_opacity) {
+          T* gc = g_conic_opacity + 4 * (size_t) id;
+          gc[0] += T(0.5) * dx * dx * dL_dG;
+          gc[1] += T(1.0) * dx * dy * dL_dG;
+          gc[2] += T(0.5) * dy * dy * dL_dG;
+          gc[3] += G * dL_dalpha;
+        }
+      }
+    }
+}
+
 }  // namespace
 }  // namespace oracle
 
@@ -490,6 +581,18 @@ using namespace oracle;
     render_backward<T>(W, H, E, means2D, conic_opacity, colors, extras, out_opacity, n_contrib, dL_dpix,             \
                        dL_dout_extras, dL_dout_opacity, point_list, ranges, g_means2D, g_conic_opacity, g_colors,    \
                        g_extras);                                                                                    \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_gs3d_extra_forward_##SUF(int W, int H, int E, const T* extras, const T* means2D,             \
+      const T* conic_opacity, const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib, T* out) {  \
+    extra_forward<T>(W, H, E, extras, means2D, conic_opacity, ranges, point_list, n_contrib, out);                   \
+    return 0;                                                                                                        \
+  }                                                                                                                  \
+  ORACLE_API int oracle_gs3d_extra_backward_##SUF(int W, int H, int E, const T* extras, const T* out_opacity,        \
+      const T* grad_out, const T* means2D, const T* conic_opacity, const int64_t* ranges, const int32_t* point_list, \
+      const int32_t* n_contrib, T* g_extras, T* g_means2D, T* g_conic_opacity) {                                     \
+    extra_backward<T>(W, H, E, extras, out_opacity, grad_out, means2D, conic_opacity, ranges, point_list, n_contrib, \
+                      g_extras, g_means2D, g_conic_opacity);                                                         \
     return 0;                                                                                                        \
   }                                                                                                                  \
   ORACLE_API int oracle_gs3d_topk_weights_##SUF(int topk, int W, int H, const T* means2D, const T* conic_opacity,    \

@@ -86,6 +86,11 @@ int oracle_gs3d_render_backward_f32(int W, int H, int E, const float* means2D, c
     const float* colors, const float* extras, const float* out_opacity, const int32_t* n_contrib,
     const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
     const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras);
+int oracle_gs3d_extra_forward_f32(int W, int H, int E, const float* extras, const float* means2D,
+    const float* conic_opacity, const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib, float* out);
+int oracle_gs3d_extra_backward_f32(int W, int H, int E, const float* extras, const float* out_opacity,
+    const float* grad_out, const float* means2D, const float* conic_opacity, const int64_t* ranges,
+    const int32_t* point_list, const int32_t* n_contrib, float* g_extras, float* g_means2D, float* g_conic_opacity);
 int oracle_gs3d_topk_weights_f32(int topk, int W, int H, const float* means2D, const float* conic_opacity,
     const int64_t* ranges, const int32_t* point_list, int32_t* top_idx, float* top_w);
 int oracle_gs3d_compute_cov3D_f32(int N, const float* q, const float* s, float* cov3D);

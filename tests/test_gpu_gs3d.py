@@ -187,6 +187,97 @@ def test_gs3d_render_autograd_and_empty(device):
     assert out['images'].shape == (3, H, W) and not out['images'].any() and not out['opacity'].any()
 
 
+@pytest.mark.parametrize("P,W,H,E", [(6000, 150, 90, 16), (4000, 131, 77, 5), (20000, 128, 128, 37), (3, 40, 40, 1)])
+def test_gs3d_rasterize_extra(P, W, H, E, device):
+    """gaussian_rasterize_extra_forward / backward: any number of channels on the weights of a finished forward pass;
+    the oracle runs from the GPU's own n_contrib / opacity, so threshold flips of the main pass do not enter."""
+    from fast_sp_gs_amd._C import get_C_function
+    m2, col, co, ranges, pl = _binned(P, W, H, 51 + E, device)
+    g = torch.Generator().manual_seed(10)
+    ex = torch.randn(P, E, generator=g).to(device)
+    print(f"[gs3d extra] P={P} {W}x{H} E={E} R={pl.numel()}", flush=True)
+    oc, oo, _, nc = get_C_function('gaussian_rasterize_forward')(W, H, m2, co, col, None, pl, ranges)
+    out = get_C_function('gaussian_rasterize_extra_forward')(W, H, ex, m2, co, ranges, pl, nc)
+    torch.cuda.synchronize()
+    n = npy
+    r_out = O.gs3d_extra_forward(W, H, n(ex), n(m2), n(co), n(ranges), n(pl), n(nc))
+    assert out.shape == (H, W, E) and abs_err(n(out), r_out) < 1e-4 * max(1.0, float(np.abs(r_out).max()))
+    # a shortened n_contrib cuts every pixel's traversal at that list position
+    cut = (nc // 2).contiguous()
+    out_cut = get_C_function('gaussian_rasterize_extra_forward')(W, H, ex, m2, co, ranges, pl, cut)
+    r_cut = O.gs3d_extra_forward(W, H, n(ex), n(m2), n(co), n(ranges), n(pl), n(cut))
+    assert abs_err(n(out_cut), r_cut) < 1e-4 * max(1.0, float(np.abs(r_cut).max()))
+
+    go = torch.randn(H, W, E, generator=g).to(device)
+    bwd = get_C_function('gaussian_rasterize_extra_backward')
+    ge, gm, gc = torch.zeros_like(ex), torch.zeros_like(m2), torch.zeros_like(co)
+    bwd(W, H, ex, oo, go, m2, co, ranges, pl, nc, ge, gm, gc)
+    torch.cuda.synchronize()
+    r_ge, r_gm, r_gc = O.gs3d_extra_backward(W, H, n(ex), n(oo), n(go), n(m2), n(co), n(ranges), n(pl), n(nc))
+    assert rel_err(n(ge), r_ge) < 1e-3 and rel_err(n(gm), r_gm) < 1e-3 and rel_err(n(gc), r_gc) < 1e-3
+    # optional outputs: only what is given is touched, and it is added to
+    ge2 = torch.ones_like(ex)
+    bwd(W, H, ex, oo, go, m2, co, ranges, pl, nc, ge2, None, None)
+    assert rel_err(n(ge2) - 1.0, r_ge) < 1e-3
+    gm2, gc2 = torch.zeros_like(m2), torch.zeros_like(co)
+    get_C_function('gaussian_rasterize_extra_backward_v2')(W, H, ex, oo, go, m2, co, ranges, pl, nc,
+                                                           torch.zeros_like(ex), gm2, gc2)
+    assert rel_err(n(gm2), r_gm) < 1e-3 and rel_err(n(gc2), r_gc) < 1e-3
+    bwd(W, H, ex, oo, go, m2, co, ranges, pl, nc, None, None, None)
+    with pytest.raises(RuntimeError):
+        get_C_function('gaussian_rasterize_extra_backward_v2')(W, H, ex, oo, go, m2, co, ranges, pl, nc, ge, None, gc)
+    with pytest.raises(RuntimeError):
+        get_C_function('gaussian_rasterize_extra_forward')(W, H, ex[None], m2, co, ranges, pl, nc)
+
+
+def test_gs3d_render_extra_autograd(device):
+    """`render(..., wide=[P,E > 4])` and `render_extra(buffer, ...)`: the autograd wiring of the further feature tables,
+    against the oracle chain; with detach=True the geometry gets no gradient from them."""
+    from fast_sp_gs_amd.renderer import gaussian_render as GR
+    P, W, H, E = 3000, 112, 80, 12
+    scene, scales, cam, tan_fov = _scene(P, W, H, 43, device)
+    d = lambda t: t.to(device).contiguous()
+    params = [d(t).requires_grad_(True) for t in (scene.means3D, scales, scene.rotations, scene.opacities, scene.shs)]
+    gen = torch.Generator().manual_seed(5)
+    wide = d(torch.randn(P, E, generator=gen)).requires_grad_(True)
+    focals = torch.tensor([float(cam.Tv2s[0, 0]), float(cam.Tv2s[1, 1])], device=device)
+    out = GR.render(d(cam.Tw2v), d(cam.Tv2c), (W, H), params[0], params[3], scales=params[1], rotations=params[2],
+                    campos=d(cam.campos), focals=focals, sh_features=params[4], sh_degree=3, wide=wide)
+    assert out['wide'].shape == (H, W, E)
+    gw = torch.randn(H, W, E, generator=gen).to(device)
+    (out['wide'] * gw).sum().backward()
+    torch.cuda.synchronize()
+    n = lambda t: npy(t.detach())
+    m2, dep, col, rad, tt, c3, co = O.gs3d_preprocess_forward(W, H, 3, False, n(params[0]), n(params[1]), n(params[2]),
+                                                              n(params[3]), n(params[4]), None, npy(cam.Tw2v),
+                                                              npy(cam.Tv2c), npy(cam.campos), tan_fov)
+    ranges, pl = O.prepare(W, H, m2, dep, rad, tt)
+    oc, oo, _, nc = O.gs3d_render_forward(W, H, m2, co, col, None, pl, ranges)
+    r_out = O.gs3d_extra_forward(W, H, n(wide), m2, co, ranges, pl, nc)
+    assert abs_err(n(out['wide']), r_out) < 1e-4 * max(1.0, float(np.abs(r_out).max()))
+    r_ge, r_gm, r_gc = O.gs3d_extra_backward(W, H, n(wide), oo, npy(gw), m2, co, ranges, pl, nc)
+    z3 = np.zeros((P, 3), np.float32)
+    r3, rs, rq, rop, rsh, _, _, rm2 = O.gs3d_preprocess_backward(W, H, 3, False, n(params[0]), n(params[1]),
+                                                                 n(params[2]), n(params[4]), None, npy(cam.Tw2v),
+                                                                 npy(cam.Tv2c), npy(cam.campos), tan_fov, rad, col, c3,
+                                                                 r_gm, z3, r_gc)
+    assert rel_err(n(wide.grad), r_ge) < 1e-3
+    for name, p_, r in zip(('means3D', 'scales', 'rotations', 'opacities'), params, (r3, rs, rq, rop)):
+        assert rel_err(n(p_.grad), r) < 1e-3, (name, rel_err(n(p_.grad), r))
+    # render_extra on the buffer, detached from the geometry
+    for p_ in params:
+        p_.grad = None
+    wide.grad = None
+    out2 = GR.render(d(cam.Tw2v), d(cam.Tv2c), (W, H), params[0], params[3], scales=params[1], rotations=params[2],
+                     campos=d(cam.campos), focals=focals, sh_features=params[4], sh_degree=3)
+    a, b = GR.render_extra(out2['buffer'], wide, wide[:, :3] * 2.0, detach=True)
+    assert torch.equal(a, out['wide']) and b.shape == (H, W, 3)
+    assert abs_err(n(b), 2.0 * r_out[..., :3]) < 2e-4 * max(1.0, float(np.abs(r_out).max()))
+    ((a * gw).sum() + b.sum()).backward()
+    assert all(p_.grad is None or not p_.grad.any() for p_ in params[:4])
+    assert rel_err(n(wide.grad)[:, 3:], r_ge[:, 3:]) < 1e-3 and wide.grad[:, :3].ne(0).any()
+
+
 def test_covariance_operators(device):
     """gs_compute_cov3D_* / gs_compute_cov2D_* against the oracle (geometry evaluated with contraction off: forward
     values bit for bit, gradients to 1e-5 of the largest entry), and the autograd wrappers end to end."""

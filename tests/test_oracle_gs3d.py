@@ -304,3 +304,73 @@ def test_covariance_operators_match_the_reference_formulation():
                                                     g2.numpy())
     np.testing.assert_allclose(g_cov3D, ca.grad.numpy(), rtol=1e-10, atol=1e-11)
     np.testing.assert_allclose(g_mean, ma.grad.numpy(), rtol=1e-9, atol=1e-9 * float(ma.grad.abs().max()))
+
+
+def test_extra_channels_forward_and_backward():
+    """gaussian_rasterize_extra_*: 20 channels (two of the reference's groups of 16). Forward against the independent
+    numpy compositor and, with a shortened n_contrib, against a per-pixel pass cut at that list position; backward
+    against the finite-difference-pinned main backward fed zero colour / opacity gradients, and against central
+    differences of the extra forward itself."""
+    s, cam, tan_fov = _scene(P=300, size=48, seed=9)
+    W, H = cam.W, cam.H
+    m2, dep, col, rad, tt, c3, co = _forward(s, cam, tan_fov)
+    P, E = len(rad), 20
+    rng = np.random.default_rng(4)
+    ex = rng.normal(size=(P, E))
+    ranges, pl = O.prepare(W, H, m2.astype(np.float32), dep.astype(np.float32), rad, tt)
+    oc, oo, _, nc = O.gs3d_render_forward(W, H, m2, co, col, np.ascontiguousarray(ex[:, :1]), pl, ranges)
+    out = O.gs3d_extra_forward(W, H, ex, m2, co, ranges, pl, nc)
+    assert out.shape == (H, W, E)
+    _, _, ext = _composite_numpy(W, H, m2, co, col, ex, pl, ranges)
+    assert np.abs(out - ext.transpose(1, 2, 0)).max() < 1e-12 and np.abs(out).max() > 0.5
+
+    cut = nc // 2  # stop each pixel half way down its list
+    out_cut = O.gs3d_extra_forward(W, H, ex, m2, co, ranges, pl, cut)
+    gx, shortened = (W + 15) // 16, 0
+    for y in range(0, H, 3):
+        for x in range(0, W, 3):
+            r0, _ = ranges[(y // 16) * gx + x // 16]
+            T, acc = 1.0, np.zeros(E)
+            for e in range(r0, r0 + cut[y, x]):
+                i = pl[e]
+                dx, dy = m2[i, 0] - x, m2[i, 1] - y
+                power = -0.5 * (co[i, 0] * dx * dx + co[i, 2] * dy * dy) - co[i, 1] * dx * dy
+                a = min(0.99, co[i, 3] * np.exp(power))
+                if power > 0 or a < 1 / 255:
+                    continue
+                acc += ex[i] * a * T
+                T *= 1 - a
+            assert np.abs(out_cut[y, x] - acc).max() < 1e-12
+            shortened += np.abs(out_cut[y, x] - out[y, x]).max() > 1e-6
+    assert shortened > 20
+
+    g = rng.normal(size=(H, W, E))
+    ge, gm, gc = O.gs3d_extra_backward(W, H, ex, oo, g, m2, co, ranges, pl, nc)
+    z3, z1 = np.zeros((3, H, W)), np.zeros((H, W))
+    r_col, r_ex, r_m2, r_co = O.gs3d_render_backward(W, H, m2, co, col, ex, oo, nc, z3,
+                                                     np.ascontiguousarray(g.transpose(2, 0, 1)), z1, pl, ranges)
+    for mine, ref in ((ge, r_ex), (gm, r_m2), (gc, r_co)):
+        assert np.abs(mine - ref).max() <= 1e-12 * max(1.0, np.abs(ref).max()) and np.abs(ref).max() > 1e-3
+    assert np.abs(r_col).max() == 0
+    only_e = O.gs3d_extra_backward(W, H, ex, oo, g, m2, co, ranges, pl, nc, want=(True, False, False))
+    assert np.array_equal(only_e[0], ge) and only_e[1] is None and only_e[2] is None
+    only_g = O.gs3d_extra_backward(W, H, ex, oo, g, m2, co, ranges, pl, nc, want=(False, True, True))
+    assert only_g[0] is None and np.array_equal(only_g[1], gm) and np.array_equal(only_g[2], gc)
+
+    def loss(m2_, co_, ex_):
+        return (O.gs3d_extra_forward(W, H, ex_, m2_, co_, ranges, pl, nc) * g).sum()
+
+    h, ok, n = 1e-6, 0, 0
+    vis = np.flatnonzero(rad > 0)
+    for i in vis[rng.permutation(len(vis))[:12]]:
+        for which, arr, grad, cols in ((0, m2, gm, (0, 1)), (1, co, gc, (0, 1, 2, 3)), (2, ex, ge, (0, 7, 19))):
+            for c in cols:
+                a, b = arr.copy(), arr.copy()
+                a[i, c] += h
+                b[i, c] -= h
+                args_a, args_b = [m2, co, ex], [m2, co, ex]
+                args_a[which], args_b[which] = a, b
+                fd = (loss(*args_a) - loss(*args_b)) / (2 * h)
+                n += 1
+                ok += abs(fd - grad[i, c]) <= 2e-4 * max(abs(fd), np.abs(grad).max() * 1e-3, 1e-6)
+    assert ok >= 0.97 * n  # a step that crosses the alpha = 1/255 threshold is the rare miss
