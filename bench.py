@@ -146,7 +146,7 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
     net = DeformNetwork().to(dev)
     # a tiny rate keeps the random-target synthetic scene from drifting (Adam's steps are |lr| whatever the gradient, and
     # the scale residuals are added after the activation, network.py:643), so every timed step sees the same workload
-    net_opt = torch.optim.Adam(list(net.parameters()) + [ctrl], lr=1e-7)
+    net_opt = torch.optim.Adam(list(net.parameters()) + [ctrl], lr=1e-7, fused=True)
     names = ('means3D', 'scales', 'rotations', 'opacities', 'shs')
     params = [getattr(scene, k).clone().requires_grad_(True) for k in names]
     opt = SparseGaussianAdam([{'params': [p_], 'name': k} for p_, k in zip(params, names)], lr=1.6e-4, eps=1e-15)

@@ -28,7 +28,7 @@ __all__ = [
     'gather_rows', 'densify_masks', 'prune_mask', 'split_children', 'densification_stats',
     'gs_compute_cov3D_forward', 'gs_compute_cov3D_backward', 'gs_compute_cov2D_forward', 'gs_compute_cov2D_backward',
     'gaussian_topk_weights', 'gaussian_rasterize_extra_forward', 'gaussian_rasterize_extra_backward',
-    'gaussian_rasterize_extra_backward_v2',
+    'gaussian_rasterize_extra_backward_v2', 'AdamMasksedUpdatedMulti', 'mlp_pack_all',
 ]
 
 _TILE = 16
@@ -842,6 +842,44 @@ def AdamMasksedUpdated(param: Tensor, param_grad: Tensor, exp_avg: Tensor, exp_a
     L.check(rc, what)
 
 
+def AdamMasksedUpdatedMulti(params: List[Tensor], grads: List[Tensor], exp_avgs: List[Tensor],
+                            exp_avg_sqs: List[Tensor], tiles_touched: Tensor, lrs: List[float], b1: float, b2: float,
+                            epss: List[float], N: int) -> None:
+    """`AdamMasksedUpdated` for all parameter tensors [N, ...] of a point set in one launch (the loop of
+    sparse_gaussian_adam.py:20-45); bit-identical to the calls one by one."""
+    what = 'AdamMasksedUpdatedMulti'
+    lib = _lib()
+    n = len(params)
+    if not (len(grads) == len(exp_avgs) == len(exp_avg_sqs) == len(lrs) == len(epss) == n):
+        raise RuntimeError(f'{what}: one gradient, two moments, a rate and an eps per parameter tensor')
+    if n > lib.fsgs_adam_masked_update_max_tensors():
+        raise RuntimeError(f'{what}: at most {lib.fsgs_adam_masked_update_max_tensors()} tensors per call')
+    tiles_touched = tiles_touched.contiguous()
+    L.require_cuda(what, tiles_touched=tiles_touched)
+    L.require_dtype(what, 'tiles_touched', tiles_touched, torch.bool)
+    grads = [g.contiguous() for g in grads]
+    Ms = []
+    for i, (p_, g, m, v) in enumerate(zip(params, grads, exp_avgs, exp_avg_sqs)):
+        _f32(what, **{f'param{i}': p_, f'grad{i}': g, f'exp_avg{i}': m, f'exp_avg_sq{i}': v})
+        if N <= 0 or p_.numel() % N or not (g.numel() == m.numel() == v.numel() == p_.numel()):
+            raise RuntimeError(f'{what}: tensor {i} is not [N, M] with N = {N}, or its gradient / moments differ in size')
+        Ms.append(p_.numel() // N)
+    if n == 0 or N == 0:
+        return
+    if tiles_touched.numel() < N:
+        raise RuntimeError(f'{what}: the mask has fewer than N = {N} entries')
+    ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])
+    a_p, a_g, a_m, a_v = ptrs(params), ptrs(grads), ptrs(exp_avgs), ptrs(exp_avg_sqs)
+    a_M = (ctypes.c_int64 * n)(*Ms)
+    a_lr, a_eps = (ctypes.c_double * n)(*map(float, lrs)), (ctypes.c_double * n)(*map(float, epss))
+    with _timed('adam_masked_update'):
+        rc = lib.fsgs_adam_masked_update_multi(n, int(N), ctypes.addressof(a_M), L.ptr(tiles_touched),
+                                               ctypes.addressof(a_lr), float(b1), float(b2), ctypes.addressof(a_eps),
+                                               ctypes.addressof(a_p), ctypes.addressof(a_g), ctypes.addressof(a_m),
+                                               ctypes.addressof(a_v), L.current_stream())
+    L.check(rc, what)
+
+
 # --------------------------------------------------------------------------------------------------------------------
 def knn_topk(x: Tensor, y: Tensor, K: int) -> Tuple[Tensor, Tensor]:
     """K nearest rows of y[M,D] for each row of x[N,D] -> (dist2[N,K] ascending, index[N,K] int64).
@@ -969,6 +1007,44 @@ def mlp_pack_weights(weights: List[Tensor], head_weights: Tensor, skip: int) -> 
     rc = lib.fsgs_pack_bf16(n_out, Kh, 32, 256, L.ptr(head_weights), packed.data_ptr() + 2 * off, stream)
     L.check(rc, what)
     return packed
+
+
+def mlp_pack_all(weights: List[Tensor], biases: List[Tensor], head_weights: List[Tensor], head_biases: List[Tensor],
+                 skip: int, transposed: bool = True):
+    """`mlp_pack_weights` + `mlp_pack_transposed` + the bias and head concatenations in one launch
+    -> (packed, packed_t | None, bias[n_layers*256 + n_out], heads_w[n_out, 256])."""
+    what = 'mlp_pack_all'
+    named = {f'w{i}': w for i, w in enumerate(weights)}
+    named.update({f'b{i}': b for i, b in enumerate(biases)})
+    named.update({f'hw{i}': w for i, w in enumerate(head_weights)})
+    named.update({f'hb{i}': b for i, b in enumerate(head_biases)})
+    _f32(what, **named)
+    Din, n_layers, n_heads = weights[0].shape[1], len(weights), len(head_weights)
+    if len(biases) != n_layers or len(head_biases) != n_heads:
+        raise RuntimeError(f'{what}: one bias per weight')
+    for i, (w, b) in enumerate(zip(weights, biases)):
+        expect = Din if i == 0 else (Din + 256 if i == skip + 1 else 256)
+        if tuple(w.shape) != (256, expect) or b.numel() != 256:
+            raise RuntimeError(f'{what}: layer {i} has weight {tuple(w.shape)} / bias {tuple(b.shape)}, expected '
+                               f'(256, {expect}) / (256,)')
+    rows = [w.shape[0] for w in head_weights]
+    if sum(rows) > 32 or any(w.shape[1] != 256 for w in head_weights) or \
+            any(b.numel() != r for b, r in zip(head_biases, rows)):
+        raise RuntimeError(f'{what}: the heads must be [rows, 256] with at most 32 rows together')
+    lib, dev = _lib(), weights[0].device
+    packed = torch.empty((lib.fsgs_mlp_packed_elems(Din, n_layers, skip),), dtype=torch.int16, device=dev)
+    packed_t = torch.empty((max(n_layers - 1, 1), 256, 256), dtype=torch.int16, device=dev) if transposed else None
+    bias = torch.empty((n_layers * 256 + sum(rows),), dtype=torch.float32, device=dev)
+    heads_w = torch.empty((sum(rows), 256), dtype=torch.float32, device=dev)
+    arr = lambda ts: (ctypes.c_void_p * max(len(ts), 1))(*[t.data_ptr() for t in ts])
+    a_w, a_b, a_hw, a_hb = arr(weights), arr(biases), arr(head_weights), arr(head_biases)
+    a_rows = (ctypes.c_int * max(n_heads, 1))(*rows)
+    rc = lib.fsgs_mlp_pack_all(Din, n_layers, skip, ctypes.addressof(a_w), ctypes.addressof(a_b), n_heads,
+                               ctypes.addressof(a_hw), ctypes.addressof(a_hb), ctypes.addressof(a_rows), L.ptr(packed),
+                               L.ptr(packed_t) if n_layers > 1 else None, L.ptr(bias), L.ptr(heads_w),
+                               L.current_stream())
+    L.check(rc, what)
+    return packed, packed_t, bias, heads_w
 
 
 def mlp_forward(inputs: Tensor, packed: Tensor, bias: Tensor, n_layers: int, skip: int, n_out: int,

@@ -23,6 +23,8 @@
 //     the batch for the bias gradient. No atomics: every output element has one writer.
 // Gradients with respect to the (frequency-encoded) input are not produced; the reference detaches it
 // (network.py:586).
+#include <algorithm>
+
 #include "common.hpp"
 
 namespace fsgs {
@@ -59,6 +61,36 @@ __global__ void __launch_bounds__(256) pack_bf16_kernel(int rows, int K, int row
   if (i >= rows_pad * K_pad) return;
   const int r = i / K_pad, k = i - r * K_pad;
   dst[frag_index(r, k, K_pad)] = (r < rows && k < K) ? f32_to_bf16(src[(size_t) r * K + k]) : (uint16_t) 0;
+}
+
+// Every per-step re-pack of the network in one launch: blockIdx.y selects a job of the table passed by value.
+struct PackJob {
+  const float* src;
+  void* dst;
+  int rows, K;            // extent of the source that exists: rows x K values
+  int rows_cover, K_pad;  // fragment rows this job writes (zeros past `rows`), padded row length of the fragment matrix
+  int dst_row0;           // first fragment row
+  int src_ld, col0;       // leading dimension and first column of the source
+  int kind;               // 0 fragment pack | 1 fragment pack of the transpose | 2 plain float copy of `rows` values
+};
+constexpr int kMaxPackJobs = 40;
+struct PackTable {
+  PackJob job[kMaxPackJobs];
+};
+
+__global__ void __launch_bounds__(256) pack_jobs_kernel(PackTable table) {
+  const PackJob& j = table.job[blockIdx.y];
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j.kind == 2) {
+    if (i < j.rows) ((float*) j.dst)[i] = j.src[i];
+    return;
+  }
+  if (i >= j.rows_cover * j.K_pad) return;
+  const int r = i / j.K_pad, k = i - r * j.K_pad;
+  float v = 0.0f;
+  if (r < j.rows && k < j.K)
+    v = j.kind == 0 ? j.src[(size_t) r * j.src_ld + j.col0 + k] : j.src[(size_t) k * j.src_ld + j.col0 + r];
+  ((uint16_t*) j.dst)[frag_index(j.dst_row0 + r, k, j.K_pad)] = f32_to_bf16(v);
 }
 
 // D layout of the 32x32 accumulator: register r of lane l holds row 8 * (r / 4) + 4 * (l / 32) + (r % 4), column l % 32.
@@ -385,6 +417,55 @@ FSGS_API int fsgs_pack_bf16(int rows, int K, int rows_pad, int K_pad, const floa
   hipLaunchKernelGGL(pack_bf16_kernel, dim3(div_up((int64_t) rows_pad * K_pad, 256)), dim3(256), 0,
                      (hipStream_t) stream, rows, K, rows_pad, K_pad, src, dst);
   return check_launch("pack_bf16");
+}
+
+// All buffers the fused network reads, refreshed from the fp32 parameters in one launch: `packed` (what
+// fsgs_mlp_forward reads: the layers' fragment matrices, then the heads stacked into one [32][256] matrix), `packed_t`
+// (optional; what fsgs_mlp_backward reads: [n_layers - 1][256 in][256 out] fragments of the last 256 input columns of
+// layers 1..), `bias_out` (layer biases then head biases) and `heads_w_out` (the heads' fp32 rows stacked).
+FSGS_API int fsgs_mlp_pack_all(int Din, int n_layers, int skip, const float* const* weights,
+    const float* const* biases, int n_heads, const float* const* head_weights, const float* const* head_biases,
+    const int* head_rows, uint16_t* packed, uint16_t* packed_t, float* bias_out, float* heads_w_out, void* stream) {
+  FSGS_REQUIRE(Din > 0 && n_layers >= 1 && skip < n_layers - 1 && weights && biases && packed && bias_out,
+               "mlp_pack_all: bad arguments");
+  FSGS_REQUIRE(n_heads >= 0 && (n_heads == 0 || (head_weights && head_biases && head_rows && heads_w_out)),
+               "mlp_pack_all: bad head arguments");
+  FSGS_REQUIRE(2 * n_layers + 3 * n_heads + (packed_t ? n_layers - 1 : 0) <= kMaxPackJobs,
+               "mlp_pack_all: too many layers / heads for one launch (%d jobs at most)", kMaxPackJobs);
+  PackTable table{};
+  int n = 0, most = 0;
+  auto add = [&](const PackJob& j) {
+    most = std::max(most, j.kind == 2 ? j.rows : j.rows_cover * j.K_pad);
+    table.job[n++] = j;
+  };
+  size_t off = 0;
+  int K = Din;
+  for (int l = 0; l < n_layers; ++l) {
+    FSGS_REQUIRE(weights[l] && biases[l], "mlp_pack_all: null layer tensor");
+    const int K_pad = (K + 15) & ~15;
+    add({weights[l], packed + off, kMlpWidth, K, kMlpWidth, K_pad, 0, K, 0, 0});
+    add({biases[l], bias_out + (size_t) l * kMlpWidth, kMlpWidth, 0, 0, 0, 0, 0, 0, 2});
+    if (packed_t && l > 0)
+      add({weights[l], packed_t + (size_t) (l - 1) * kMlpWidth * kMlpWidth, kMlpWidth, kMlpWidth, kMlpWidth,
+           kMlpWidth, 0, K, K - kMlpWidth, 1});
+    off += (size_t) kMlpWidth * K_pad;
+    K = (l == skip) ? Din + kMlpWidth : kMlpWidth;
+  }
+  FSGS_REQUIRE(K == kMlpWidth, "mlp_pack_all: the heads must follow a %d-wide layer", kMlpWidth);
+  int row0 = 0;
+  for (int h = 0; h < n_heads; ++h) {
+    FSGS_REQUIRE(head_weights[h] && head_biases[h] && head_rows[h] > 0, "mlp_pack_all: bad head tensor");
+    const bool last = h == n_heads - 1;
+    FSGS_REQUIRE(row0 + head_rows[h] <= 32, "mlp_pack_all: the heads have more than 32 rows together");
+    add({head_weights[h], packed + off, head_rows[h], kMlpWidth, last ? 32 - row0 : head_rows[h], kMlpWidth, row0,
+         kMlpWidth, 0, 0});
+    add({head_biases[h], bias_out + (size_t) n_layers * kMlpWidth + row0, head_rows[h], 0, 0, 0, 0, 0, 0, 2});
+    add({head_weights[h], heads_w_out + (size_t) row0 * kMlpWidth, head_rows[h] * kMlpWidth, 0, 0, 0, 0, 0, 0, 2});
+    row0 += head_rows[h];
+  }
+  if (n_heads == 0) add({weights[0], packed + off, 0, kMlpWidth, 32, kMlpWidth, 0, kMlpWidth, 0, 0});  // zero head block
+  hipLaunchKernelGGL(pack_jobs_kernel, dim3(div_up(most, 256), n), dim3(256), 0, (hipStream_t) stream, table);
+  return check_launch("mlp_pack_all");
 }
 
 // Number of bf16 elements of the packed weight buffer: per layer [256][K_pad_i], then the heads as [32][K_pad_last].

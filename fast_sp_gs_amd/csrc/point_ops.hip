@@ -12,6 +12,8 @@
 // All of these are HBM-streaming or small brute-force searches: one lane per point, control points staged in LDS and
 // read as wave-wide broadcasts, distances accumulated in the reference's order with contraction off so that indices
 // are reproducible bit for bit.
+#include <algorithm>
+
 #include "common.hpp"
 #include "sh.hpp"
 
@@ -398,10 +400,87 @@ __global__ void __launch_bounds__(256) adam_masked_kernel(int64_t total, int64_t
   }
 }
 
+// The same update for every parameter tensor of a point set in one launch (blockIdx.y = tensor): the reference steps
+// its parameter groups one kernel at a time (sparse_gaussian_adam.py:20-45), each a few microseconds of work behind a
+// launch. Table passed by value; same arithmetic as adam_masked_kernel, element for element.
+constexpr int kMaxAdamTensors = 12;
+struct AdamTable {
+  float* param[kMaxAdamTensors];
+  const float* grad[kMaxAdamTensors];
+  float* m[kMaxAdamTensors];
+  float* v[kMaxAdamTensors];
+  int64_t M[kMaxAdamTensors];
+  float lr[kMaxAdamTensors], eps[kMaxAdamTensors];
+  int vec4[kMaxAdamTensors];
+};
+
+template <int kVec>
+__device__ __forceinline__ void adam_masked_body(int64_t e, float lr, float b1, float b2, float eps,
+    float* __restrict__ param, const float* __restrict__ grad, float* __restrict__ m, float* __restrict__ v) {
+#pragma clang fp contract(off)
+  float g[kVec], mm[kVec], vv[kVec], pp[kVec];
+  if (kVec == 4) {
+    *(float4*) g  = *(const float4*) (grad + e);
+    *(float4*) mm = *(const float4*) (m + e);
+    *(float4*) vv = *(const float4*) (v + e);
+    *(float4*) pp = *(const float4*) (param + e);
+  } else {
+    g[0] = grad[e], mm[0] = m[e], vv[0] = v[e], pp[0] = param[e];
+  }
+#pragma unroll
+  for (int k = 0; k < kVec; ++k) {
+    mm[k] = b1 * mm[k] + (1.0f - b1) * g[k];
+    vv[k] = b2 * vv[k] + (1.0f - b2) * g[k] * g[k];
+    pp[k] += -lr * mm[k] / (sqrtf(vv[k]) + eps);
+  }
+  if (kVec == 4) {
+    *(float4*) (param + e) = *(float4*) pp;
+    *(float4*) (m + e)     = *(float4*) mm;
+    *(float4*) (v + e)     = *(float4*) vv;
+  } else {
+    param[e] = pp[0], m[e] = mm[0], v[e] = vv[0];
+  }
+}
+
+__global__ void __launch_bounds__(256) adam_masked_multi_kernel(AdamTable t, int64_t N, float b1, float b2,
+                                                                const uint8_t* __restrict__ mask) {
+  const int q      = blockIdx.y;
+  const int64_t M  = t.M[q], total = N * M;
+  const int vec    = t.vec4[q] ? 4 : 1;
+  const int64_t e  = ((int64_t) blockIdx.x * blockDim.x + threadIdx.x) * vec;
+  if (e >= total || !mask[e / M]) return;
+  if (vec == 4) adam_masked_body<4>(e, t.lr[q], b1, b2, t.eps[q], t.param[q], t.grad[q], t.m[q], t.v[q]);
+  else adam_masked_body<1>(e, t.lr[q], b1, b2, t.eps[q], t.param[q], t.grad[q], t.m[q], t.v[q]);
+}
+
 }  // namespace
 }  // namespace fsgs
 
 using namespace fsgs;
+
+FSGS_API int fsgs_adam_masked_update_max_tensors(void) { return kMaxAdamTensors; }
+
+FSGS_API int fsgs_adam_masked_update_multi(int n_tensors, int64_t N, const int64_t* M, const uint8_t* mask,
+    const double* lr, double b1, double b2, const double* eps, float* const* param, const float* const* grad,
+    float* const* m, float* const* v, void* stream) {
+  FSGS_REQUIRE(n_tensors >= 0 && n_tensors <= kMaxAdamTensors && N >= 0,
+               "AdamMasksedUpdated (multi): bad arguments (at most %d tensors)", kMaxAdamTensors);
+  if (n_tensors == 0 || N == 0) return kOk;
+  FSGS_REQUIRE(M && mask && lr && eps && param && grad && m && v, "AdamMasksedUpdated (multi): null pointer");
+  AdamTable t{};
+  int64_t most = 0;
+  for (int q = 0; q < n_tensors; ++q) {
+    FSGS_REQUIRE(M[q] > 0 && param[q] && grad[q] && m[q] && v[q], "AdamMasksedUpdated (multi): bad tensor %d", q);
+    t.param[q] = param[q], t.grad[q] = grad[q], t.m[q] = m[q], t.v[q] = v[q], t.M[q] = M[q];
+    t.lr[q] = (float) lr[q], t.eps[q] = (float) eps[q];
+    t.vec4[q] = (M[q] % 4 == 0) &&
+                (((uintptr_t) param[q] | (uintptr_t) grad[q] | (uintptr_t) m[q] | (uintptr_t) v[q]) % 16 == 0);
+    most = std::max<int64_t>(most, t.vec4[q] ? N * M[q] / 4 : N * M[q]);
+  }
+  hipLaunchKernelGGL(adam_masked_multi_kernel, dim3((unsigned) div_up(most, (int64_t) 256), n_tensors), dim3(256), 0,
+                     (hipStream_t) stream, t, N, (float) b1, (float) b2, mask);
+  return check_launch("AdamMasksedUpdated");
+}
 
 FSGS_API int fsgs_sh_to_rgb_forward(int P, int F, int degree, int clamp, const float* pos, const float* campos,
                                     const float* sh, float* rgb, void* stream) {

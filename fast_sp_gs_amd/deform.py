@@ -43,16 +43,16 @@ class DeformNetwork(nn.Module):
             nn.init.zeros_(head.bias)
         self._packed = None
 
-    def pack(self):
-        """Refresh the bf16 weight buffer (call after every optimiser step on these parameters)."""
-        heads_w = torch.cat([self.gaussian_warp.weight, self.gaussian_rotation.weight, self.gaussian_scaling.weight], 0)
-        heads_b = torch.cat([self.gaussian_warp.bias, self.gaussian_rotation.bias, self.gaussian_scaling.bias], 0)
-        weights = [l.weight.detach().contiguous() for l in self.linear]
-        packed = get_C_function('mlp_pack_weights')(weights, heads_w.detach().contiguous(), self.skip)
-        bias = torch.cat([l.bias.detach() for l in self.linear] + [heads_b.detach()]).contiguous()
+    def pack(self, transposed: bool = True):
+        """Refresh the bf16 weight buffers, the bias vector and the stacked head rows from the parameters in one launch
+        (call after every optimiser step on these parameters). `transposed` also makes the copy the backward reads."""
+        heads = (self.gaussian_warp, self.gaussian_rotation, self.gaussian_scaling)
+        packed, packed_t, bias, heads_w = get_C_function('mlp_pack_all')(
+            [l.weight.detach() for l in self.linear], [l.bias.detach() for l in self.linear],
+            [h.weight.detach() for h in heads], [h.bias.detach() for h in heads], self.skip, transposed)
         self._packed = (packed, bias)
-        self._packed_t = None  # transposed copy for the backward, made on demand
-        self._heads_w = heads_w.detach().contiguous()
+        self._packed_t = packed_t
+        self._heads_w = heads_w
         return self._packed
 
     def encode(self, x: Tensor, t: Tensor) -> Tensor:
@@ -70,13 +70,12 @@ class DeformNetwork(nn.Module):
         x_enc = self.encode(x, t)
         track = torch.is_grad_enabled() and (x_enc.requires_grad or any(p.requires_grad for p in params))
         versions = tuple(p._version for p in params)
-        if self._packed is None or (track and getattr(self, '_packed_versions', None) != versions):
-            self.pack()
+        if self._packed is None or (track and (getattr(self, '_packed_versions', None) != versions or
+                                               self._packed_t is None)):
+            self.pack(transposed=track)
             self._packed_versions = versions
         packed, bias = self._packed
         if track:
-            if self._packed_t is None:
-                self._packed_t = get_C_function('mlp_pack_transposed')([l.weight.detach() for l in self.linear])
             out = _DeformMlp.apply(x_enc, packed, bias, self._packed_t, self._heads_w, self.D, self.skip, *params)
         else:
             out = get_C_function('mlp_forward')(x_enc.detach(), packed, bias, self.D, self.skip, 10)

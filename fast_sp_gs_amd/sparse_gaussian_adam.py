@@ -10,6 +10,8 @@ __all__ = ['SparseGaussianAdam']
 
 class SparseGaussianAdam(torch.optim.Adam):
     _update_C = staticmethod(get_C_function('AdamMasksedUpdated'))
+    _update_multi_C = staticmethod(get_C_function('AdamMasksedUpdatedMulti'))
+    _MAX = 12  # tensors per launch (fsgs_adam_masked_update_max_tensors)
 
     def __init__(self, params, lr, eps):
         super().__init__(params=params, lr=lr, eps=eps)
@@ -18,6 +20,9 @@ class SparseGaussianAdam(torch.optim.Adam):
 
     @torch.no_grad()
     def step(self):
+        """The reference's loop over parameter groups (sparse_gaussian_adam.py:20-45), with the groups' kernels folded
+        into one launch per `_MAX` tensors; the arithmetic per element is the single-tensor kernel's."""
+        params, grads, ms, vs, lrs, epss = [], [], [], [], [], []
         for group in self.param_groups:
             lr = group["lr"]
             eps = group["eps"]
@@ -30,13 +35,15 @@ class SparseGaussianAdam(torch.optim.Adam):
                 state['step'] = torch.tensor(0.0, dtype=torch.float32)
                 state['exp_avg'] = torch.zeros_like(param, memory_format=torch.preserve_format)
                 state['exp_avg_sq'] = torch.zeros_like(param, memory_format=torch.preserve_format)
-            exp_avg, exp_avg_sq = state["exp_avg"], state["exp_avg_sq"]
             state['step'] += 1
             step = float(state['step'])
-            M = param.numel() // self.N
+            params.append(param), grads.append(param.grad), ms.append(state["exp_avg"]), vs.append(state["exp_avg_sq"])
             # bias corrections folded into the learning rate: lr * sqrt(1 - b2^t) / (1 - b1^t)
-            self._update_C(param, param.grad, exp_avg, exp_avg_sq, self.visibility,
-                           lr * (1 - 0.999 ** step) ** 0.5 / (1 - 0.9 ** step), 0.9, 0.999, eps, self.N, M)
+            lrs.append(lr * (1 - 0.999 ** step) ** 0.5 / (1 - 0.9 ** step))
+            epss.append(eps)
+        for i in range(0, len(params), self._MAX):
+            j = slice(i, i + self._MAX)
+            self._update_multi_C(params[j], grads[j], ms[j], vs[j], self.visibility, lrs[j], 0.9, 0.999, epss[j], self.N)
 
     def set_before_step(self, visibility, N):
         self.visibility, self.N = visibility, N

@@ -401,6 +401,15 @@ int fsgs_fusedssim_backward(int B, int CH, int H, int W, const float* img1, cons
  * layer's post-ReLU hidden state for fsgs_mlp_backward. */
 int fsgs_pack_bf16(int rows, int K, int rows_pad, int K_pad, const float* src, uint16_t* dst, void* stream);
 size_t fsgs_mlp_packed_elems(int Din, int n_layers, int skip);
+/* Every buffer fsgs_mlp_forward / fsgs_mlp_backward read, refreshed from the fp32 torch.nn.Linear parameters in one
+ * launch (the reference has no such step: its network runs on the fp32 parameters, network.py:1757-1776). Host arrays
+ * of device pointers: weights[n_layers] ([256][K_l] row-major), biases[n_layers] ([256]), head_weights[n_heads]
+ * ([head_rows[h]][256]), head_biases[n_heads]; the heads' rows are stacked in the order given (<= 32 rows together).
+ * Outputs: packed (fsgs_mlp_packed_elems elements), packed_t (NULL, or (n_layers-1)*65536 elements), bias_out
+ * [n_layers*256 + sum(head_rows)], heads_w_out [sum(head_rows)][256] fp32. */
+int fsgs_mlp_pack_all(int Din, int n_layers, int skip, const float* const* weights, const float* const* biases,
+    int n_heads, const float* const* head_weights, const float* const* head_biases, const int* head_rows,
+    uint16_t* packed, uint16_t* packed_t, float* bias_out, float* heads_w_out, void* stream);
 int fsgs_mlp_forward(int B, int Din, int width, int n_layers, int skip, int n_out, const float* in,
                      const uint16_t* packed, const float* bias, float* out, uint16_t* saved, void* stream);
 
@@ -467,6 +476,13 @@ int fsgs_densification_stats(int P, int grad_stride, const int32_t* radii, const
  * tensors whose mask byte is 0 are left untouched; eps is added to sqrt(v); lr carries the bias correction. */
 int fsgs_adam_masked_update(int64_t N, int64_t M, const uint8_t* mask, double lr, double b1, double b2, double eps,
                             float* param, const float* grad, float* m, float* v, void* stream);
+/* The same update for up to fsgs_adam_masked_update_max_tensors() tensors [N, M[q]] of one point set in one launch
+ * (the loop over parameter groups of fast_2d_gs/sparse_gaussian_adam.py:20-45, one kernel each there). M, lr, eps,
+ * param, grad, m, v are host arrays with one entry per tensor; results equal the single-tensor calls bit for bit. */
+int fsgs_adam_masked_update_max_tensors(void);
+int fsgs_adam_masked_update_multi(int n_tensors, int64_t N, const int64_t* M, const uint8_t* mask, const double* lr,
+    double b1, double b2, const double* eps, float* const* param, const float* const* grad, float* const* m,
+    float* const* v, void* stream);
 
 #ifdef __cplusplus
 }

@@ -345,6 +345,65 @@ def test_sparse_adam(device, oracle_mod):
         assert np.array_equal(npy(opt.state[p]['exp_avg']), r)
 
 
+def test_multi_tensor_entry_points_match_the_single_ones(device):
+    """`AdamMasksedUpdatedMulti` against `AdamMasksedUpdated` tensor by tensor (own rate and eps each, more tensors than
+    one launch takes through the optimiser class), and `mlp_pack_all` against the separate packing operators plus
+    torch.cat: bit for bit."""
+    from fast_sp_gs_amd._C import get_C_function
+    from fast_sp_gs_amd.deform import DeformNetwork
+    from fast_sp_gs_amd.sparse_gaussian_adam import SparseGaussianAdam
+    g = torch.Generator().manual_seed(17)
+    N = 3001
+    shapes = [(N, 3), (N, 16, 3), (N, 1), (N, 2), (N, 4), (N, 5), (N, 8)]
+    mk = lambda: [torch.randn(s, generator=g).to(device) for s in shapes]
+    p1, gr, m1 = mk(), mk(), mk()
+    v1 = [t.abs() for t in mk()]
+    p2, m2, v2 = [t.clone() for t in p1], [t.clone() for t in m1], [t.clone() for t in v1]
+    vis = (torch.rand(N, generator=g) < 0.5).to(device)
+    lrs = [1e-3 * (k + 1) for k in range(len(shapes))]
+    epss = [1e-15 * 10 ** k for k in range(len(shapes))]
+    get_C_function('AdamMasksedUpdatedMulti')(p1, gr, m1, v1, vis, lrs, 0.9, 0.999, epss, N)
+    for k, s_ in enumerate(shapes):
+        get_C_function('AdamMasksedUpdated')(p2[k], gr[k], m2[k], v2[k], vis, lrs[k], 0.9, 0.999, epss[k], N,
+                                             p2[k].numel() // N)
+    for a, b in zip(p1 + m1 + v1, p2 + m2 + v2):
+        assert torch.equal(a, b)
+    assert not torch.equal(p1[1][vis], mk()[1][vis])  # something moved
+    # 14 groups: two launches inside the optimiser
+    params = [torch.nn.Parameter(torch.randn(N, 1 + k % 4, generator=g).to(device)) for k in range(14)]
+    before = [p_.detach().clone() for p_ in params]
+    opt = SparseGaussianAdam([{'params': [p_], 'lr': 1e-3 * (k + 1)} for k, p_ in enumerate(params)], lr=1e-3, eps=1e-15)
+    for p_ in params:
+        p_.grad = torch.randn(p_.shape, generator=g).to(device)
+    opt.set_before_step(vis, N)
+    opt.step()
+    for k, (p_, b) in enumerate(zip(params, before)):
+        assert torch.equal(p_[~vis], b[~vis]) and not torch.equal(p_[vis], b[vis]), k
+        # first step of Adam: |update| = lr * sqrt(1 - b2) / (1 - b1) * (1 - b1) |g| / (sqrt((1 - b2) g^2) + eps) = lr
+        assert float(((p_ - b)[vis].abs() - 1e-3 * (k + 1)).abs().max()) < 1e-3 * (k + 1) * 1e-3
+    with pytest.raises(RuntimeError):
+        get_C_function('AdamMasksedUpdatedMulti')(p1, gr[:-1], m1, v1, vis, lrs, 0.9, 0.999, epss, N)
+
+    net = DeformNetwork().to(device)
+    with torch.no_grad():
+        for p_ in net.parameters():
+            p_.add_(0.05 * torch.randn(p_.shape, generator=g).to(device))
+    heads = (net.gaussian_warp, net.gaussian_rotation, net.gaussian_scaling)
+    weights = [l.weight.detach() for l in net.linear]
+    packed, packed_t, bias, heads_w = get_C_function('mlp_pack_all')(
+        weights, [l.bias.detach() for l in net.linear], [h.weight.detach() for h in heads],
+        [h.bias.detach() for h in heads], net.skip)
+    hw = torch.cat([h.weight.detach() for h in heads], 0).contiguous()
+    assert torch.equal(packed, get_C_function('mlp_pack_weights')(weights, hw, net.skip))
+    assert torch.equal(packed_t, get_C_function('mlp_pack_transposed')(weights))
+    assert torch.equal(bias, torch.cat([l.bias.detach() for l in net.linear] + [h.bias.detach() for h in heads]))
+    assert torch.equal(heads_w, hw)
+    only = get_C_function('mlp_pack_all')(weights, [l.bias.detach() for l in net.linear],
+                                          [h.weight.detach() for h in heads], [h.bias.detach() for h in heads],
+                                          net.skip, False)
+    assert only[1] is None and torch.equal(only[0], packed)
+
+
 def test_full_size_properties(device):
     """Full benchmark-size runs checked through size-independent properties (no oracle at this size)."""
     from fast_sp_gs_amd import scenes
