@@ -137,7 +137,7 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
     from fast_sp_gs_amd.deform import DeformNetwork, superpoint_deform
     from fast_sp_gs_amd.renderer import GS_2D_render
     from fast_sp_gs_amd.sparse_gaussian_adam import SparseGaussianAdam
-    from fast_sp_gs_amd.ssim import ssim
+    from fast_sp_gs_amd.ssim import l1_dssim_loss
     scene_h, cam_h = scenes.config2(P=200_000, size=800, seed=2)
     scene, cam = scene_h.to(dev), cam_h.to(dev)
     g = torch.Generator().manual_seed(2)
@@ -163,7 +163,7 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
                            cam.Tw2v, cam.Tv2c, campos=cam.campos, near=cam.near, far=cam.far, sh_degree=3,
                            sh_features=params[4], background=bg)
         image = out['images']
-        loss = 0.8 * (image - target).abs().mean() + 0.2 * (1.0 - ssim(image, target).mean())
+        loss = l1_dssim_loss(image, target, 0.2)  # 0.8 * L1 + 0.2 * (1 - mean SSIM), fused
         loss.backward()
         opt.set_before_step(out['radii'] > 0, params[0].shape[0])
         opt.step()

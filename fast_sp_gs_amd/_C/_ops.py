@@ -29,6 +29,7 @@ __all__ = [
     'gs_compute_cov3D_forward', 'gs_compute_cov3D_backward', 'gs_compute_cov2D_forward', 'gs_compute_cov2D_backward',
     'gaussian_topk_weights', 'gaussian_rasterize_extra_forward', 'gaussian_rasterize_extra_backward',
     'gaussian_rasterize_extra_backward_v2', 'AdamMasksedUpdatedMulti', 'mlp_pack_all',
+    'image_loss_forward', 'image_loss_backward',
 ]
 
 _TILE = 16
@@ -1152,6 +1153,49 @@ def fusedssim_backward(C1: float, C2: float, img1: Tensor, img2: Tensor, dL_dmap
         rc = _lib().fsgs_fusedssim_backward(B, CH, H, W, L.ptr(img1), L.ptr(img2), L.ptr(dL_dmap),
                                             L.ptr(dm_dmu1.contiguous()), L.ptr(dm_dsigma1_sq.contiguous()),
                                             L.ptr(dm_dsigma12.contiguous()), L.ptr(grad), L.current_stream())
+    L.check(rc, what)
+    return grad
+
+
+def image_loss_forward(C1: float, C2: float, lambda_dssim: float, img: Tensor, target: Tensor, train: bool):
+    """(1 - lambda) * L1 + lambda * (1 - mean SSIM) of [B,CH,H,W] images without image-sized intermediates
+    (gaussian_splatting.py:321 with losses/ssim.py:24-47) -> (loss[3] = (loss, L1 mean, SSIM mean), dm_dmu1,
+    dm_dsigma1_sq, dm_dsigma12); the three maps are None when `train` is false."""
+    what = 'image_loss_forward'
+    _f32(what, img=img, target=target)
+    if img.ndim != 4 or img.shape != target.shape or img.numel() == 0:
+        raise RuntimeError(f'{what}: img and target must be non-empty [B,CH,H,W] tensors of the same shape')
+    B, CH, H, W = img.shape
+    lib = _lib()
+    loss = torch.empty((3,), dtype=torch.float32, device=img.device)
+    d1, d2, d3 = (torch.empty_like(img) for _ in range(3)) if train else (None, None, None)
+    nbytes = lib.fsgs_image_loss_workspace_bytes(B, H, W)
+    ws = _workspace(nbytes, img.device)
+    with _timed(what):
+        rc = lib.fsgs_image_loss_forward(B, CH, H, W, float(C1), float(C2), float(lambda_dssim), L.ptr(img),
+                                         L.ptr(target), L.ptr(loss), L.ptr(d1), L.ptr(d2), L.ptr(d3), L.ptr(ws), nbytes,
+                                         L.current_stream())
+    L.check(rc, what)
+    return loss, d1, d2, d3
+
+
+def image_loss_backward(lambda_dssim: float, img: Tensor, target: Tensor, grad_loss: Tensor, dm_dmu1: Tensor,
+                        dm_dsigma1_sq: Tensor, dm_dsigma12: Tensor) -> Tensor:
+    """Gradient of `image_loss_forward`'s loss[0] with respect to img; grad_loss is the one-element upstream gradient."""
+    what = 'image_loss_backward'
+    _f32(what, img=img, target=target, grad_loss=grad_loss, dm_dmu1=dm_dmu1, dm_dsigma1_sq=dm_dsigma1_sq,
+         dm_dsigma12=dm_dsigma12)
+    B, CH, H, W = img.shape
+    for name, t in (('target', target), ('dm_dmu1', dm_dmu1), ('dm_dsigma1_sq', dm_dsigma1_sq),
+                    ('dm_dsigma12', dm_dsigma12)):
+        L.require_shape(what, name, t, B, CH, H, W)
+    if grad_loss.numel() != 1:
+        raise RuntimeError(f'{what}: grad_loss must have one element')
+    grad = torch.empty_like(img)
+    with _timed(what):
+        rc = _lib().fsgs_image_loss_backward(B, CH, H, W, float(lambda_dssim), L.ptr(img), L.ptr(target),
+                                             L.ptr(grad_loss), L.ptr(dm_dmu1), L.ptr(dm_dsigma1_sq),
+                                             L.ptr(dm_dsigma12), L.ptr(grad), L.current_stream())
     L.check(rc, what)
     return grad
 

@@ -26,10 +26,11 @@ __device__ __forceinline__ float pixel_or_zero(const float* __restrict__ plane, 
   return (x >= 0 && y >= 0 && x < W && y < H) ? plane[(size_t) y * W + x] : 0.0f;
 }
 
-template <bool kTrain>
+template <bool kTrain, bool kLoss>
 __global__ void __launch_bounds__(kSsimThreads) ssim_forward_kernel(int H, int W, int CH, float C1, float C2,
     const float* __restrict__ img1, const float* __restrict__ img2, float* __restrict__ ssim_map,
-    float* __restrict__ dm_dmu1, float* __restrict__ dm_dsigma1_sq, float* __restrict__ dm_dsigma12) {
+    float* __restrict__ dm_dmu1, float* __restrict__ dm_dsigma1_sq, float* __restrict__ dm_dsigma12,
+    float* __restrict__ partials) {
   __shared__ float s_a[kSsimHalo][kSsimHalo + 1];
   __shared__ float s_b[kSsimHalo][kSsimHalo + 1];
   __shared__ float s_h[5][kSsimHalo][kSsimTile + 1];  // horizontally filtered moments
@@ -38,6 +39,7 @@ __global__ void __launch_bounds__(kSsimThreads) ssim_forward_kernel(int H, int W
   float g[11];
 #pragma unroll
   for (int k = 0; k < 11; ++k) g[k] = kGauss[k];
+  float sum_ssim = 0.0f, sum_l1 = 0.0f;  // kLoss: this lane's share of the two image sums
 
   for (int c = 0; c < CH; ++c) {
     const float* p1 = img1 + ((size_t) blockIdx.z * CH + c) * plane;
@@ -76,7 +78,12 @@ __global__ void __launch_bounds__(kSsimThreads) ssim_forward_kernel(int H, int W
         const float C = 2.0f * mu1_mu2 + C1, D = 2.0f * sigma12 + C2;
         const float A = mu1_sq + mu2_sq + C1, B = sigma1_sq + sigma2_sq + C2;
         const size_t idx = ((size_t) blockIdx.z * CH + c) * plane + (size_t) py * W + px;
-        ssim_map[idx] = (C * D) / (A * B);
+        if (kLoss) {
+          sum_ssim += (C * D) / (A * B);
+          sum_l1 += fabsf(s_a[ly + 5][lx + 5] - s_b[ly + 5][lx + 5]);
+        } else {
+          ssim_map[idx] = (C * D) / (A * B);
+        }
         if (kTrain) {
           dm_dmu1[idx] = (mu2 * 2.0f * D) / (A * B) - (mu2 * 2.0f * C) / (A * B) - (mu1 * 2.0f * C * D) / (A * A * B) +
                          (mu1 * 2.0f * C * D) / (A * B * B);
@@ -87,12 +94,50 @@ __global__ void __launch_bounds__(kSsimThreads) ssim_forward_kernel(int H, int W
     }
     __syncthreads();  // the next channel overwrites the halo and the filtered moments
   }
+  if (kLoss) {
+    // block sums in a fixed order: lanes by xor butterfly, then the four wavefronts in turn
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) sum_ssim += __shfl_xor(sum_ssim, d, 64), sum_l1 += __shfl_xor(sum_l1, d, 64);
+    float* s_red = &s_h[0][0][0];
+    if ((threadIdx.x & 63) == 0) s_red[2 * (threadIdx.x >> 6)] = sum_ssim, s_red[2 * (threadIdx.x >> 6) + 1] = sum_l1;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const size_t blk = ((size_t) blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+      float a = 0.0f, b = 0.0f;
+      for (int w = 0; w < kSsimThreads / 64; ++w) a += s_red[2 * w], b += s_red[2 * w + 1];
+      partials[2 * blk] = a, partials[2 * blk + 1] = b;
+    }
+  }
 }
 
+// loss_out[0] = (1 - lambda) * mean|img - target| + lambda * (1 - mean SSIM); [1] = the L1 mean, [2] = the SSIM mean.
+// One block; the per-block partial sums are added in a fixed order.
+__global__ void __launch_bounds__(256) image_loss_finish_kernel(int n_blocks, const float* __restrict__ partials,
+                                                                float inv_n, float lambda, float* __restrict__ loss_out) {
+  __shared__ float s_red[2][256];
+  float a = 0.0f, b = 0.0f;
+  for (int i = threadIdx.x; i < n_blocks; i += 256) a += partials[2 * i], b += partials[2 * i + 1];
+  s_red[0][threadIdx.x] = a, s_red[1][threadIdx.x] = b;
+  __syncthreads();
+  for (int d = 128; d >= 1; d >>= 1) {
+    if ((int) threadIdx.x < d)
+      s_red[0][threadIdx.x] += s_red[0][threadIdx.x + d], s_red[1][threadIdx.x] += s_red[1][threadIdx.x + d];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const float ssim_mean = s_red[0][0] * inv_n, l1_mean = s_red[1][0] * inv_n;
+    loss_out[0] = (1.0f - lambda) * l1_mean + lambda * (1.0f - ssim_mean);
+    loss_out[1] = l1_mean, loss_out[2] = ssim_mean;
+  }
+}
+
+// kLoss: the gradient of the fused image loss. dL/dmap is the same number at every pixel, -lambda / n times the
+// upstream gradient of the scalar loss (read from device memory), and (1 - lambda) / n * sign(img1 - img2) is added.
+template <bool kLoss>
 __global__ void __launch_bounds__(kSsimThreads) ssim_backward_kernel(int H, int W, int CH,
     const float* __restrict__ img1, const float* __restrict__ img2, const float* __restrict__ dL_dmap,
     const float* __restrict__ dm_dmu1, const float* __restrict__ dm_dsigma1_sq, const float* __restrict__ dm_dsigma12,
-    float* __restrict__ dL_dimg1) {
+    float* __restrict__ dL_dimg1, float map_scale, float l1_scale) {
   __shared__ float s_p[3][kSsimHalo][kSsimHalo + 1];  // dL/dmap times each of the three partials
   __shared__ float s_h[3][kSsimHalo][kSsimTile + 1];
   const int x0 = blockIdx.x * kSsimTile, y0 = blockIdx.y * kSsimTile;
@@ -106,7 +151,8 @@ __global__ void __launch_bounds__(kSsimThreads) ssim_backward_kernel(int H, int 
     for (int e = threadIdx.x; e < kSsimHalo * kSsimHalo; e += kSsimThreads) {
       const int ly = e / kSsimHalo, lx = e - ly * kSsimHalo;
       const int y = y0 + ly - 5, x = x0 + lx - 5;
-      const float gmap = pixel_or_zero(dL_dmap + off, y, x, H, W);
+      const float gmap = kLoss ? ((y >= 0 && y < H && x >= 0 && x < W) ? map_scale * dL_dmap[0] : 0.0f)
+                               : pixel_or_zero(dL_dmap + off, y, x, H, W);
       s_p[0][ly][lx] = pixel_or_zero(dm_dmu1 + off, y, x, H, W) * gmap;
       s_p[1][ly][lx] = pixel_or_zero(dm_dsigma1_sq + off, y, x, H, W) * gmap;
       s_p[2][ly][lx] = pixel_or_zero(dm_dsigma12 + off, y, x, H, W) * gmap;
@@ -135,6 +181,10 @@ __global__ void __launch_bounds__(kSsimThreads) ssim_backward_kernel(int H, int 
         float grad = a0;
         grad += img1[idx] * 2.0f * a1;
         grad += img2[idx] * a2;
+        if (kLoss) {
+          const float d = img1[idx] - img2[idx];
+          grad += l1_scale * dL_dmap[0] * (d > 0.0f ? 1.0f : (d < 0.0f ? -1.0f : 0.0f));
+        }
         dL_dimg1[idx] = grad;
       }
     }
@@ -157,11 +207,11 @@ FSGS_API int fsgs_fusedssim_forward(int B, int CH, int H, int W, double C1, doub
   FSGS_REQUIRE(B <= 65535, "fusedssim: batch %d exceeds the grid limit", B);
   const dim3 grid(div_up(W, kSsimTile), div_up(H, kSsimTile), B), block(kSsimThreads);
   if (train)
-    hipLaunchKernelGGL(ssim_forward_kernel<true>, grid, block, 0, (hipStream_t) stream, H, W, CH, (float) C1,
-                       (float) C2, img1, img2, ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12);
+    hipLaunchKernelGGL((ssim_forward_kernel<true, false>), grid, block, 0, (hipStream_t) stream, H, W, CH, (float) C1,
+                       (float) C2, img1, img2, ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, nullptr);
   else
-    hipLaunchKernelGGL(ssim_forward_kernel<false>, grid, block, 0, (hipStream_t) stream, H, W, CH, (float) C1,
-                       (float) C2, img1, img2, ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12);
+    hipLaunchKernelGGL((ssim_forward_kernel<false, false>), grid, block, 0, (hipStream_t) stream, H, W, CH, (float) C1,
+                       (float) C2, img1, img2, ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, nullptr);
   return check_launch("fusedssim");
 }
 
@@ -174,7 +224,51 @@ FSGS_API int fsgs_fusedssim_backward(int B, int CH, int H, int W, const float* i
                "fusedssim_backward: null pointer");
   FSGS_REQUIRE(B <= 65535, "fusedssim_backward: batch %d exceeds the grid limit", B);
   const dim3 grid(div_up(W, kSsimTile), div_up(H, kSsimTile), B), block(kSsimThreads);
-  hipLaunchKernelGGL(ssim_backward_kernel, grid, block, 0, (hipStream_t) stream, H, W, CH, img1, img2, dL_dmap,
-                     dm_dmu1, dm_dsigma1_sq, dm_dsigma12, dL_dimg1);
+  hipLaunchKernelGGL(ssim_backward_kernel<false>, grid, block, 0, (hipStream_t) stream, H, W, CH, img1, img2, dL_dmap,
+                     dm_dmu1, dm_dsigma1_sq, dm_dsigma12, dL_dimg1, 0.0f, 0.0f);
   return check_launch("fusedssim_backward");
+}
+
+FSGS_API size_t fsgs_image_loss_workspace_bytes(int B, int H, int W) {
+  if (B <= 0 || H <= 0 || W <= 0) return 256;
+  return align_up((size_t) B * div_up(W, kSsimTile) * div_up(H, kSsimTile) * 2 * sizeof(float), 256);
+}
+
+FSGS_API int fsgs_image_loss_forward(int B, int CH, int H, int W, double C1, double C2, double lambda_dssim,
+    const float* img, const float* target, float* loss_out, float* dm_dmu1, float* dm_dsigma1_sq,
+    float* dm_dsigma12, void* workspace, size_t workspace_bytes, void* stream) {
+  FSGS_REQUIRE(B > 0 && CH > 0 && H > 0 && W > 0 && B <= 65535, "image_loss: bad sizes");
+  FSGS_REQUIRE(img && target && loss_out && workspace, "image_loss: null pointer");
+  const bool train = dm_dmu1 != nullptr;
+  FSGS_REQUIRE(!train || (dm_dsigma1_sq && dm_dsigma12), "image_loss: the three partial-derivative maps go together");
+  if (workspace_bytes < fsgs_image_loss_workspace_bytes(B, H, W))
+    return fail(kWorkspaceSmall, "image_loss: workspace %zu < %zu bytes", workspace_bytes,
+                fsgs_image_loss_workspace_bytes(B, H, W));
+  const dim3 grid(div_up(W, kSsimTile), div_up(H, kSsimTile), B), block(kSsimThreads);
+  hipStream_t s = (hipStream_t) stream;
+  float* partials = (float*) workspace;
+  if (train)
+    hipLaunchKernelGGL((ssim_forward_kernel<true, true>), grid, block, 0, s, H, W, CH, (float) C1, (float) C2, img,
+                       target, nullptr, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, partials);
+  else
+    hipLaunchKernelGGL((ssim_forward_kernel<false, true>), grid, block, 0, s, H, W, CH, (float) C1, (float) C2, img,
+                       target, nullptr, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, partials);
+  const double n = (double) B * CH * H * W;
+  hipLaunchKernelGGL(image_loss_finish_kernel, dim3(1), dim3(256), 0, s, (int) (grid.x * grid.y * grid.z), partials,
+                     (float) (1.0 / n), (float) lambda_dssim, loss_out);
+  return check_launch("image_loss");
+}
+
+FSGS_API int fsgs_image_loss_backward(int B, int CH, int H, int W, double lambda_dssim, const float* img,
+    const float* target, const float* grad_loss, const float* dm_dmu1, const float* dm_dsigma1_sq,
+    const float* dm_dsigma12, float* dL_dimg, void* stream) {
+  FSGS_REQUIRE(B > 0 && CH > 0 && H > 0 && W > 0 && B <= 65535, "image_loss_backward: bad sizes");
+  FSGS_REQUIRE(img && target && grad_loss && dm_dmu1 && dm_dsigma1_sq && dm_dsigma12 && dL_dimg,
+               "image_loss_backward: null pointer");
+  const dim3 grid(div_up(W, kSsimTile), div_up(H, kSsimTile), B), block(kSsimThreads);
+  const double n = (double) B * CH * H * W;
+  hipLaunchKernelGGL(ssim_backward_kernel<true>, grid, block, 0, (hipStream_t) stream, H, W, CH, img, target,
+                     grad_loss, dm_dmu1, dm_dsigma1_sq, dm_dsigma12, dL_dimg, (float) (-lambda_dssim / n),
+                     (float) ((1.0 - lambda_dssim) / n));
+  return check_launch("image_loss_backward");
 }

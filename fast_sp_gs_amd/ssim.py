@@ -5,7 +5,7 @@ from torch import Tensor, nn
 
 from fast_sp_gs_amd._C import get_C_function
 
-__all__ = ['FusedSSIM', 'ssim', 'SSIM_Loss']
+__all__ = ['FusedSSIM', 'ssim', 'SSIM_Loss', 'l1_dssim_loss']
 
 
 class FusedSSIM(torch.autograd.Function):
@@ -35,6 +35,42 @@ def ssim(img1: Tensor, img2: Tensor) -> Tensor:
     if img1.ndim == 3:
         return FusedSSIM.apply(img1[None], img2[None], None)[0]
     return FusedSSIM.apply(img1, img2, None)
+
+
+class _L1DssimLoss(torch.autograd.Function):
+    """(1 - lambda) * L1 + lambda * (1 - mean SSIM) on the fused kernels: the block sums are taken inside the SSIM
+    kernel and the L1 term's sign is added inside its backward, so nothing image-sized is written but the gradient."""
+
+    @staticmethod
+    def forward(ctx, img, target, lambda_dssim):
+        img, target = img.contiguous(), target.contiguous()
+        loss, d1, d2, d3 = get_C_function('image_loss_forward')(FusedSSIM.C1, FusedSSIM.C2, lambda_dssim, img, target,
+                                                                ctx.needs_input_grad[0])
+        assert not ctx.needs_input_grad[1]
+        ctx.lambda_dssim = lambda_dssim
+        if ctx.needs_input_grad[0]:
+            ctx.save_for_backward(img, target, d1, d2, d3)
+        terms = loss[1:]
+        ctx.mark_non_differentiable(terms)
+        return loss[0], terms
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_loss, _):
+        img, target, d1, d2, d3 = ctx.saved_tensors
+        grad = get_C_function('image_loss_backward')(ctx.lambda_dssim, img, target, grad_loss.reshape(1).contiguous(),
+                                                     d1, d2, d3)
+        return grad, None, None
+
+
+def l1_dssim_loss(img: Tensor, target: Tensor, lambda_dssim: float = 0.2, return_terms: bool = False):
+    """The photometric loss of a training step, (1 - lambda) * mean|img - target| + lambda * (1 - mean SSIM), as one
+    scalar (reference: the 'rgb' and 'ssim' terms summed at fast_2d_gs/gaussian_splatting.py:321 with their weights).
+    [CH,H,W] or [B,CH,H,W]; differentiable in img. With `return_terms` also (L1 mean, SSIM mean), detached."""
+    if img.ndim == 3:
+        img, target = img[None], target[None]
+    loss, terms = _L1DssimLoss.apply(img, target, float(lambda_dssim))
+    return (loss, terms.detach()) if return_terms else loss
 
 
 class SSIM_Loss(nn.Module):

@@ -388,6 +388,21 @@ int fsgs_fusedssim_forward(int B, int CH, int H, int W, double C1, double C2, co
 int fsgs_fusedssim_backward(int B, int CH, int H, int W, const float* img1, const float* img2, const float* dL_dmap,
     const float* dm_dmu1, const float* dm_dsigma1_sq, const float* dm_dsigma12, float* dL_dimg1, void* stream);
 
+/* The photometric loss of a training step in two launches forward and one backward, with no image-sized intermediate:
+ * loss = (1 - lambda) * mean|img - target| + lambda * (1 - mean SSIM(img, target)) -- the 'rgb' + 'ssim' terms of
+ * fast_2d_gs/gaussian_splatting.py:321 / network.py:1027 with losses/ssim.py:24-47, which the reference evaluates as an
+ * L1 in torch, the fusedssim map, two means and their autograd. img, target [B,CH,H,W]. loss_out[3] = (loss, L1 mean,
+ * SSIM mean). dm_* are NULL (no gradient wanted) or the three [B,CH,H,W] maps the backward reads. The workspace holds
+ * two partial sums per 32x32 block, added in a fixed order. The backward reads the upstream gradient of the scalar loss
+ * from device memory (grad_loss[0]) and writes dL_dimg[B,CH,H,W] in full. */
+size_t fsgs_image_loss_workspace_bytes(int B, int H, int W);
+int fsgs_image_loss_forward(int B, int CH, int H, int W, double C1, double C2, double lambda_dssim, const float* img,
+    const float* target, float* loss_out, float* dm_dmu1, float* dm_dsigma1_sq, float* dm_dsigma12, void* workspace,
+    size_t workspace_bytes, void* stream);
+int fsgs_image_loss_backward(int B, int CH, int H, int W, double lambda_dssim, const float* img, const float* target,
+    const float* grad_loss, const float* dm_dmu1, const float* dm_dsigma1_sq, const float* dm_dsigma12, float* dL_dimg,
+    void* stream);
+
 /* Deformation MLP forward (bf16 MFMA, fp32 accumulate) -- fast_2d_gs/network.py:1757-1776 (SC_GS_DeformNetwork.forward,
  * fp32 there): n_layers x (Linear(256) + ReLU), input re-concatenated in front after layer `skip`, then n_out <= 32
  * linear outputs (the three heads stacked). in[B,Din] fp32 (already frequency-encoded), Din <= 96, width must be 256.

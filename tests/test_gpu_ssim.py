@@ -60,3 +60,45 @@ def test_ssim_autograd_and_loss(device):
     fd = (f(img1.detach() + eps * d) - f(img1.detach() - eps * d)) / (2 * eps)
     an = float((img1.grad * d).sum())
     assert abs(fd - an) < 2e-2 * max(abs(an), 1e-6) + 1e-6
+
+
+@pytest.mark.parametrize("shape,lam", [((1, 3, 800, 800), 0.2), ((2, 3, 45, 70), 0.35), ((1, 1, 7, 5), 1.0),
+                                       ((3, 2, 32, 64), 0.0)])
+def test_fused_image_loss(shape, lam, device, oracle_mod):
+    """(1 - lambda) L1 + lambda (1 - mean SSIM) in the fused kernels against the CPU oracle's SSIM map and partials with
+    the L1 term, the means and the chain rule taken in float64 numpy, and against the composition of the separate
+    operators through torch autograd."""
+    from fast_sp_gs_amd.ssim import l1_dssim_loss, ssim
+    O = oracle_mod
+    B, CH, H, W = shape
+    g = torch.Generator().manual_seed(3)
+    img1, img2 = torch.rand(*shape, generator=g), torch.rand(*shape, generator=g)
+    img2[..., : W // 2] = img1[..., : W // 2] * 0.9
+    img2[..., 0, :] = img1[..., 0, :]  # a row of equal pixels: the L1 term's gradient is exactly zero there
+    x = img1.to(device).requires_grad_(True)
+    print(f"[image loss] {shape} lambda={lam}", flush=True)
+    loss, terms = l1_dssim_loss(x, img2.to(device), lam, return_terms=True)
+    (3.0 * loss).backward()
+    torch.cuda.synchronize()
+    a, b = npy(img1), npy(img2)
+    rm, r1, r2, r3 = (np.zeros_like(a) for _ in range(4))
+    assert O.call("fusedssim_forward_f32", B, CH, H, W, 0.01 ** 2, 0.03 ** 2, a, b, rm, r1, r2, r3) == 0
+    n = a.size
+    l1, sm = np.abs(a.astype(np.float64) - b).mean(), rm.astype(np.float64).mean()
+    want = (1 - lam) * l1 + lam * (1 - sm)
+    assert abs(float(loss) - want) < 2e-6 * max(1.0, abs(want))
+    assert abs(float(terms[0]) - l1) < 2e-6 and abs(float(terms[1]) - sm) < 2e-6
+    rg = np.zeros_like(a)
+    gmap = np.full_like(a, -3.0 * lam / n)
+    assert O.call("fusedssim_backward_f32", B, CH, H, W, a, b, gmap, r1, r2, r3, rg) == 0
+    rg = rg.astype(np.float64) + 3.0 * (1 - lam) / n * np.sign(a.astype(np.float64) - b)
+    assert rel_err(npy(x.grad), rg.astype(np.float32)) < 1e-4
+    # the separate operators through autograd
+    y = img1.to(device).requires_grad_(True)
+    t = img2.to(device)
+    ref = (1 - lam) * (y - t).abs().mean() + lam * (1.0 - ssim(y, t).mean())
+    (3.0 * ref).backward()
+    assert abs(float(loss) - float(ref)) < 2e-6 * max(1.0, abs(float(ref)))
+    assert rel_err(npy(x.grad), npy(y.grad)) < 1e-5
+    # no gradient wanted: the same number
+    assert float(l1_dssim_loss(img1.to(device), t, lam)) == float(loss)
