@@ -134,7 +134,7 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
     on the surfel parameters + Adam on the MLP weights and the control points (gradients reach them through the LBS and
     K-NN backward kernels and the MLP's fp32 GEMM backward)."""
     from fast_sp_gs_amd import scenes
-    from fast_sp_gs_amd.deform import DeformNetwork, superpoint_deform
+    from fast_sp_gs_amd.deform import DeformNetwork, deform_apply, superpoint_deform
     from fast_sp_gs_amd.renderer import GS_2D_render
     from fast_sp_gs_amd.sparse_gaussian_adam import SparseGaussianAdam
     from fast_sp_gs_amd.ssim import l1_dssim_loss
@@ -158,8 +158,8 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
         d_xyz, d_rot, d_scale, _, _ = superpoint_deform(params[0].detach(), ctrl, c_xyz.contiguous(),
                                                         c_rot.contiguous(), c_scale[:, :2].contiguous(), K=4,
                                                         temperature=0.01)
-        out = GS_2D_render(params[0] + d_xyz, params[1] + d_scale, torch.nn.functional.normalize(params[2] + d_rot, dim=-1),
-                           params[3], (cam.W, cam.H),
+        xyz, scales, rot = deform_apply(params[0], d_xyz, params[1], d_scale, params[2], d_rot)
+        out = GS_2D_render(xyz, scales, rot, params[3], (cam.W, cam.H),
                            cam.Tw2v, cam.Tv2c, campos=cam.campos, near=cam.near, far=cam.far, sh_degree=3,
                            sh_features=params[4], background=bg)
         image = out['images']

@@ -29,7 +29,7 @@ __all__ = [
     'gs_compute_cov3D_forward', 'gs_compute_cov3D_backward', 'gs_compute_cov2D_forward', 'gs_compute_cov2D_backward',
     'gaussian_topk_weights', 'gaussian_rasterize_extra_forward', 'gaussian_rasterize_extra_backward',
     'gaussian_rasterize_extra_backward_v2', 'AdamMasksedUpdatedMulti', 'mlp_pack_all',
-    'image_loss_forward', 'image_loss_backward',
+    'image_loss_forward', 'image_loss_backward', 'deform_apply_forward', 'deform_apply_backward',
 ]
 
 _TILE = 16
@@ -841,6 +841,45 @@ def AdamMasksedUpdated(param: Tensor, param_grad: Tensor, exp_avg: Tensor, exp_a
                                             float(eps), L.ptr(param), L.ptr(param_grad), L.ptr(exp_avg),
                                             L.ptr(exp_avg_sq), L.current_stream())
     L.check(rc, what)
+
+
+def deform_apply_forward(points: Tensor, d_xyz: Tensor, scales: Tensor, d_scale: Tensor, rotations: Tensor,
+                         d_rotation: Tensor, log_scales: bool):
+    """network.py:630, :643, :645 in one kernel -> (points + d_xyz, act(scales) + d_scale, normalize(rot + d_rot))."""
+    what = 'deform_apply_forward'
+    _f32(what, points=points, d_xyz=d_xyz, scales=scales, d_scale=d_scale, rotations=rotations, d_rotation=d_rotation)
+    N, S = scales.shape
+    for name, t, c in (('points', points, 3), ('d_xyz', d_xyz, 3), ('d_scale', d_scale, S), ('rotations', rotations, 4),
+                       ('d_rotation', d_rotation, 4)):
+        L.require_shape(what, name, t, N, c)
+    out_p, out_s, out_r = torch.empty_like(points), torch.empty_like(scales), torch.empty_like(rotations)
+    with _timed(what):
+        rc = _lib().fsgs_deform_apply_forward(N, S, int(bool(log_scales)), L.ptr(points), L.ptr(d_xyz), L.ptr(scales),
+                                              L.ptr(d_scale), L.ptr(rotations), L.ptr(d_rotation), L.ptr(out_p),
+                                              L.ptr(out_s), L.ptr(out_r), L.current_stream())
+    L.check(rc, what)
+    return out_p, out_s, out_r
+
+
+def deform_apply_backward(scales: Tensor, rotations: Tensor, d_rotation: Tensor, grad_scales: Optional[Tensor],
+                          grad_rot: Tensor, log_scales: bool):
+    """-> (g_scales | None, g_rot): the two gradients of `deform_apply_forward` that are not its upstream gradients
+    themselves (g_scales only for logarithmic scales)."""
+    what = 'deform_apply_backward'
+    _f32(what, scales=scales, rotations=rotations, d_rotation=d_rotation, grad_scales=grad_scales, grad_rot=grad_rot)
+    N, S = scales.shape
+    L.require_shape(what, 'grad_rot', grad_rot, N, 4)
+    g_rot = torch.empty_like(rotations)
+    g_scales = None
+    if log_scales:
+        L.require_shape(what, 'grad_scales', grad_scales, N, S)
+        g_scales = torch.empty_like(scales)
+    with _timed(what):
+        rc = _lib().fsgs_deform_apply_backward(N, S, int(bool(log_scales)), L.ptr(scales), L.ptr(rotations),
+                                               L.ptr(d_rotation), L.ptr(grad_scales), L.ptr(grad_rot), L.ptr(g_scales),
+                                               L.ptr(g_rot), L.current_stream())
+    L.check(rc, what)
+    return g_scales, g_rot
 
 
 def AdamMasksedUpdatedMulti(params: List[Tensor], grads: List[Tensor], exp_avgs: List[Tensor],

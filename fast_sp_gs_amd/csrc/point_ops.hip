@@ -400,6 +400,61 @@ __global__ void __launch_bounds__(256) adam_masked_kernel(int64_t total, int64_t
   }
 }
 
+// ---- deformed parameters --------------------------------------------------------------------------------------------
+// network.py:630, :643, :645: points + d_xyz, scaling_activation(scales) + d_scale (exp when the scales are stored as
+// logarithms), normalize(rotations + d_rotation) with torch.nn.functional.normalize's 1e-12 floor on the norm. One lane
+// per point; the reference runs these as separate torch operators with their autograd nodes.
+template <int S>
+__global__ void __launch_bounds__(256) deform_apply_forward_kernel(int N, int log_scales,
+    const float* __restrict__ points, const float* __restrict__ d_xyz, const float* __restrict__ scales,
+    const float* __restrict__ d_scale, const float* __restrict__ rot, const float* __restrict__ d_rot,
+    float* __restrict__ out_points, float* __restrict__ out_scales, float* __restrict__ out_rot) {
+#pragma clang fp contract(off)
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N) return;
+#pragma unroll
+  for (int c = 0; c < 3; ++c) out_points[3 * (size_t) i + c] = points[3 * (size_t) i + c] + d_xyz[3 * (size_t) i + c];
+#pragma unroll
+  for (int c = 0; c < S; ++c) {
+    const float v = scales[S * (size_t) i + c];
+    out_scales[S * (size_t) i + c] = (log_scales ? expf(v) : v) + d_scale[S * (size_t) i + c];
+  }
+  const float4 a = ((const float4*) rot)[i], b = ((const float4*) d_rot)[i];
+  const float x = a.x + b.x, y = a.y + b.y, z = a.z + b.z, w = a.w + b.w;
+  const float inv = 1.0f / fmaxf(sqrtf(x * x + y * y + z * z + w * w), 1e-12f);
+  ((float4*) out_rot)[i] = make_float4(x * inv, y * inv, z * inv, w * inv);
+}
+
+// Gradients that are not the upstream gradient itself: through the normalisation to rotations / d_rotation (the same
+// tensor for both) and, for logarithmic scales, g * exp(scale). points, d_xyz and d_scale receive their output's
+// gradient unchanged, so nothing is computed for them.
+template <int S>
+__global__ void __launch_bounds__(256) deform_apply_backward_kernel(int N, int log_scales,
+    const float* __restrict__ scales, const float* __restrict__ rot, const float* __restrict__ d_rot,
+    const float* __restrict__ g_out_scales, const float* __restrict__ g_out_rot, float* __restrict__ g_scales,
+    float* __restrict__ g_rot) {
+#pragma clang fp contract(off)
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N) return;
+  if (log_scales)
+#pragma unroll
+    for (int c = 0; c < S; ++c)
+      g_scales[S * (size_t) i + c] = g_out_scales[S * (size_t) i + c] * expf(scales[S * (size_t) i + c]);
+  const float4 a = ((const float4*) rot)[i], b = ((const float4*) d_rot)[i], g = ((const float4*) g_out_rot)[i];
+  const float x = a.x + b.x, y = a.y + b.y, z = a.z + b.z, w = a.w + b.w;
+  const float n = sqrtf(x * x + y * y + z * z + w * w);
+  float4 o;
+  if (n > 1e-12f) {
+    const float inv = 1.0f / n;
+    const float qx = x * inv, qy = y * inv, qz = z * inv, qw = w * inv;
+    const float dot = qx * g.x + qy * g.y + qz * g.z + qw * g.w;
+    o = make_float4((g.x - qx * dot) * inv, (g.y - qy * dot) * inv, (g.z - qz * dot) * inv, (g.w - qw * dot) * inv);
+  } else {
+    o = make_float4(g.x * 1e12f, g.y * 1e12f, g.z * 1e12f, g.w * 1e12f);
+  }
+  ((float4*) g_rot)[i] = o;
+}
+
 // The same update for every parameter tensor of a point set in one launch (blockIdx.y = tensor): the reference steps
 // its parameter groups one kernel at a time (sparse_gaussian_adam.py:20-45), each a few microseconds of work behind a
 // launch. Table passed by value; same arithmetic as adam_masked_kernel, element for element.
@@ -457,6 +512,36 @@ __global__ void __launch_bounds__(256) adam_masked_multi_kernel(AdamTable t, int
 }  // namespace fsgs
 
 using namespace fsgs;
+
+FSGS_API int fsgs_deform_apply_forward(int N, int S, int log_scales, const float* points, const float* d_xyz,
+    const float* scales, const float* d_scale, const float* rot, const float* d_rot, float* out_points,
+    float* out_scales, float* out_rot, void* stream) {
+  FSGS_REQUIRE(N >= 0 && (S == 2 || S == 3), "deform_apply: N >= 0 and 2 or 3 scales per point");
+  if (N == 0) return kOk;
+  FSGS_REQUIRE(points && d_xyz && scales && d_scale && rot && d_rot && out_points && out_scales && out_rot,
+               "deform_apply: null pointer");
+  FSGS_REQUIRE((((uintptr_t) rot | (uintptr_t) d_rot | (uintptr_t) out_rot) & 15) == 0,
+               "deform_apply: rotations must be 16-byte aligned");
+  auto kernel = S == 2 ? deform_apply_forward_kernel<2> : deform_apply_forward_kernel<3>;
+  hipLaunchKernelGGL(kernel, dim3(div_up(N, 256)), dim3(256), 0, (hipStream_t) stream, N, log_scales, points, d_xyz,
+                     scales, d_scale, rot, d_rot, out_points, out_scales, out_rot);
+  return check_launch("deform_apply");
+}
+
+FSGS_API int fsgs_deform_apply_backward(int N, int S, int log_scales, const float* scales, const float* rot,
+    const float* d_rot, const float* g_out_scales, const float* g_out_rot, float* g_scales, float* g_rot,
+    void* stream) {
+  FSGS_REQUIRE(N >= 0 && (S == 2 || S == 3), "deform_apply_backward: N >= 0 and 2 or 3 scales per point");
+  if (N == 0) return kOk;
+  FSGS_REQUIRE(rot && d_rot && g_out_rot && g_rot && (!log_scales || (scales && g_out_scales && g_scales)),
+               "deform_apply_backward: null pointer");
+  FSGS_REQUIRE((((uintptr_t) rot | (uintptr_t) d_rot | (uintptr_t) g_out_rot | (uintptr_t) g_rot) & 15) == 0,
+               "deform_apply_backward: rotations must be 16-byte aligned");
+  auto kernel = S == 2 ? deform_apply_backward_kernel<2> : deform_apply_backward_kernel<3>;
+  hipLaunchKernelGGL(kernel, dim3(div_up(N, 256)), dim3(256), 0, (hipStream_t) stream, N, log_scales, scales, rot,
+                     d_rot, g_out_scales, g_out_rot, g_scales, g_rot);
+  return check_launch("deform_apply_backward");
+}
 
 FSGS_API int fsgs_adam_masked_update_max_tensors(void) { return kMaxAdamTensors; }
 

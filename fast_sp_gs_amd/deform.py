@@ -13,7 +13,7 @@ from torch import Tensor, nn
 from fast_sp_gs_amd._C import get_C_function
 from fast_sp_gs_amd.ops import FreqEncoder
 
-__all__ = ['DeformNetwork', 'superpoint_deform']
+__all__ = ['DeformNetwork', 'superpoint_deform', 'deform_apply']
 
 
 class DeformNetwork(nn.Module):
@@ -172,3 +172,39 @@ def superpoint_deform(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Ten
                                                sp_r.contiguous(), None if sp_s is None else sp_s.contiguous(), d2, idx,
                                                temperature, centred)
     return d_xyz, d_rot, d_scale, w, idx
+
+
+class _DeformApply(torch.autograd.Function):
+    """points + d_xyz, act(scales) + d_scale, normalize(rotations + d_rotation) (network.py:630, :643, :645) as one
+    kernel forward and one backward; sums hand their upstream gradient to both addends unchanged."""
+
+    @staticmethod
+    def forward(ctx, points, d_xyz, scales, d_scale, rotations, d_rotation, log_scales):
+        args = [t.contiguous() for t in (points, d_xyz, scales, d_scale, rotations, d_rotation)]
+        out = get_C_function('deform_apply_forward')(*args, log_scales)
+        ctx.save_for_backward(args[2], args[4], args[5])
+        ctx.log_scales = log_scales
+        return out
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, g_points, g_scales, g_rot):
+        scales, rotations, d_rotation = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        gs = g_r = None
+        if need[4] or need[5] or (ctx.log_scales and need[2]):
+            gs, g_r = get_C_function('deform_apply_backward')(
+                scales, rotations, d_rotation, g_scales.contiguous() if ctx.log_scales else None, g_rot.contiguous(),
+                ctx.log_scales)
+        if not ctx.log_scales:
+            gs = g_scales
+        pick = lambda g, k: g if need[k] else None
+        return pick(g_points, 0), pick(g_points, 1), pick(gs, 2), pick(g_scales, 3), pick(g_r, 4), pick(g_r, 5), None
+
+
+def deform_apply(points: Tensor, d_xyz: Tensor, scales: Tensor, d_scale: Tensor, rotations: Tensor, d_rotation: Tensor,
+                 log_scales: bool = False):
+    """The deformed parameters handed to the renderer (reference: fast_2d_gs/network.py:630, :643, :645 with
+    apply_rotate == 'add'): (points + d_xyz, scales + d_scale, normalize(rotations + d_rotation)); with `log_scales`
+    the scales are stored as logarithms and exp is applied first (gaussian_splatting.py:142)."""
+    return _DeformApply.apply(points, d_xyz, scales, d_scale, rotations, d_rotation, bool(log_scales))

@@ -487,6 +487,17 @@ int fsgs_split_children(int P, int n_selected, int N, int S, const int32_t* sele
 int fsgs_densification_stats(int P, int grad_stride, const int32_t* radii, const float* grad, const float* factor,
                              float* max_radii2D, float* grad_accum, float* denom, uint8_t* visible, void* stream);
 
+/* The deformed parameters of a dynamic step -- fast_2d_gs/network.py:630, :643, :645 (torch operators there):
+ * out_points = points + d_xyz, out_scales = (log_scales ? exp(scales) : scales) + d_scale with S = 2 or 3 scales per
+ * point, out_rot = normalize(rot + d_rot) with a 1e-12 floor on the norm. The backward computes only what differs from
+ * the upstream gradient: g_rot[N,4] (shared by rot and d_rot) and, when log_scales, g_scales[N,S] = g_out_scales *
+ * exp(scales); points, d_xyz and d_scale take their output's gradient as it is. */
+int fsgs_deform_apply_forward(int N, int S, int log_scales, const float* points, const float* d_xyz,
+    const float* scales, const float* d_scale, const float* rot, const float* d_rot, float* out_points,
+    float* out_scales, float* out_rot, void* stream);
+int fsgs_deform_apply_backward(int N, int S, int log_scales, const float* scales, const float* rot, const float* d_rot,
+    const float* g_out_scales, const float* g_out_rot, float* g_scales, float* g_rot, void* stream);
+
 /* AdamMasksedUpdated -- fast_2d_gs/_C/src/other/adam_masked_update.cu:30-35 (kernel :9-28). Rows of the [N,M]
  * tensors whose mask byte is 0 are left untouched; eps is added to sqrt(v); lr carries the bias correction. */
 int fsgs_adam_masked_update(int64_t N, int64_t M, const uint8_t* mask, double lr, double b1, double b2, double eps,

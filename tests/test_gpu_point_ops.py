@@ -404,6 +404,38 @@ def test_multi_tensor_entry_points_match_the_single_ones(device):
     assert only[1] is None and torch.equal(only[0], packed)
 
 
+@pytest.mark.parametrize("S,log_scales", [(2, False), (3, True), (2, True)])
+def test_deform_apply_matches_the_torch_operators(S, log_scales, device):
+    """points + d_xyz, act(scales) + d_scale, normalize(rot + d_rot) (network.py:630, :643, :645) in one kernel each way
+    against the torch operators the reference runs, forward and through autograd; one rotation row sums to zero."""
+    from fast_sp_gs_amd.deform import deform_apply
+    g = torch.Generator().manual_seed(23)
+    N = 7001
+    mk = lambda *s_: torch.randn(*s_, generator=g).to(device)
+    base = [mk(N, 3), mk(N, 3) * 0.1, mk(N, S) * 0.5, mk(N, S) * 0.1, mk(N, 4), mk(N, 4) * 0.1]
+    base[5][7] = -base[4][7]  # rot + d_rot == 0 there: normalize's floor on the norm decides
+    a = [t.clone().requires_grad_(True) for t in base]
+    b = [t.clone().requires_grad_(True) for t in base]
+    out = deform_apply(*a, log_scales=log_scales)
+    ref = (b[0] + b[1], (torch.exp(b[2]) if log_scales else b[2]) + b[3],
+           torch.nn.functional.normalize(b[4] + b[5], dim=-1))
+    for o, r in zip(out, ref):
+        assert o.shape == r.shape and float((o - r).abs().max()) <= 2e-6 * max(1.0, float(r.abs().max()))
+    assert not out[2][7].any()
+    go = [mk(*o.shape) for o in out]
+    go[2][7] *= 1e-9  # keeps g / 1e-12 finite in float32
+    sum((o * g_).sum() for o, g_ in zip(out, go)).backward()
+    sum((r * g_).sum() for r, g_ in zip(ref, go)).backward()
+    for k, (x, y) in enumerate(zip(a, b)):
+        assert rel_err(npy(x.grad), npy(y.grad)) < 1e-5, k
+    # only the deltas need gradients (parameters detached)
+    c = [t.clone().requires_grad_(k % 2 == 1) for k, t in enumerate(base)]
+    out2 = deform_apply(*c, log_scales=log_scales)
+    sum((o * g_).sum() for o, g_ in zip(out2, go)).backward()
+    assert all((t.grad is None) == (k % 2 == 0) for k, t in enumerate(c))
+    assert torch.equal(c[5].grad, a[5].grad) and torch.equal(c[1].grad, a[1].grad)
+
+
 def test_full_size_properties(device):
     """Full benchmark-size runs checked through size-independent properties (no oracle at this size)."""
     from fast_sp_gs_amd import scenes
