@@ -44,7 +44,10 @@ blend_backward_kernel(
     const float4* __restrict__ records) {
   __shared__ SplatHot s_hot[kBwdBatch];
   __shared__ SplatCold s_cold[kBwdBatch];
-  __shared__ float s_acc[kBwdBatch][kGradSlots + 1];  // +1: odd stride keeps the flush conflict free
+  // Each wavefront's sums over its 64 pixels, one row per staged surfel, written once per entry with a plain store (a
+  // wavefront meets an entry once per batch); the flush adds the four rows in wavefront order, so a tile's sums do not
+  // depend on timing. +1: the odd stride keeps the flush free of bank conflicts.
+  __shared__ float s_part[4][kBwdBatch][kGradSlots + 1];
   __shared__ int s_slot[kSlots ? kBwdBatch : 1];      // where this (surfel, tile) instance sits in surfel order
   __shared__ float s_t2[kFlow ? kBwdBatch * 9 : 1];
   __shared__ int s_max_contrib;
@@ -71,9 +74,7 @@ blend_backward_kernel(
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) wave_max_contrib = max(wave_max_contrib, __shfl_xor(wave_max_contrib, d, kWave));
   if (lane == 0) atomicMax(&s_max_contrib, wave_max_contrib);
-#pragma unroll
-  for (int c = 0; c < kGradSlots + 1; ++c)
-    if ((int) threadIdx.x < kBwdBatch) s_acc[threadIdx.x][c] = 0.0f;
+  for (int e = threadIdx.x; e < 4 * kBwdBatch * (kGradSlots + 1); e += kBlendThreads) (&s_part[0][0][0])[e] = 0.0f;
   __syncthreads();
   const int n_todo = min(s_max_contrib, (int) (r1 - r0));  // positions [0, n_todo) of the tile's list, walked from n_todo-1 down to 0
   const int rounds = (n_todo + kBwdBatch - 1) / kBwdBatch;
@@ -254,10 +255,10 @@ blend_backward_kernel(
         g[15] = h.G * dL_dalpha;
       }
       const float tot = wave_sum16_transposed(g);
-      if (lane < 16) atomicAdd(&s_acc[j][lane], tot);  // one LDS atomic instruction for all 16 components
+      if (lane < 16) s_part[wave][j][lane] = tot;  // a wavefront meets an entry once per batch: a plain store
       if (__ballot(filtered) != 0ull) {
         const float sx = wave_sum_to_lane63(g2x), sy = wave_sum_to_lane63(g2y);
-        if (lane == 63) atomicAdd(&s_acc[j][16], sx), atomicAdd(&s_acc[j][17], sy);
+        if (lane == 63) s_part[wave][j][16] = sx, s_part[wave][j][17] = sy;
       }
      };
      // The record of the next entry is requested before the current one is evaluated (alternating registers): a
@@ -291,7 +292,14 @@ blend_backward_kernel(
     __syncthreads();
     // flush the batch
     if ((int) threadIdx.x < n_here) {
-      float* a = s_acc[threadIdx.x];
+      float a[kGradSlots];
+#pragma unroll
+      for (int c = 0; c < kGradSlots; ++c) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum += s_part[w][threadIdx.x][c], s_part[w][threadIdx.x][c] = 0.0f;
+        a[c] = sum;
+      }
       if (kSlots) {
         // one 72-byte record per (surfel, tile) instance at the instance's position in surfel order; the per-surfel
         // sums are taken afterwards by slot_reduce_kernel. Records nobody contributed to stay at their zero fill.
@@ -319,10 +327,8 @@ blend_backward_kernel(
         for (int c = 0; c < 2; ++c)
           if (a[16 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[16 + c]);
       }
-#pragma unroll
-      for (int c = 0; c < kGradSlots; ++c) a[c] = 0.0f;
     }
-    // No barrier needed here: a lane only touches its own record / accumulator row between this flush and the
+    // No barrier needed here: a lane only touches its own record / its own rows of s_part between this flush and the
     // barrier that follows the next batch's LDS store.
   }
 }

@@ -12,8 +12,9 @@
 // staged in LDS with the next batch's gather in flight, a conservative per-quadrant footprint test (bounding box of the
 // alpha >= 1/255 ellipse) whose ballot is the wavefront's work list, longest lists scheduled first. Where the
 // reference issues 9 + E global float atomics per (pixel, Gaussian) pair, the backward sums the 9 + E gradient
-// components over the 64 pixels of a wavefront with one transposed DPP butterfly, adds the four wavefronts' partials
-// with one 16-lane LDS atomic, and flushes one global atomic per Gaussian, component and tile.
+// components over the 64 pixels of a wavefront with one transposed DPP butterfly, stores each wavefront's partial in
+// its own LDS row (LDS float atomics cost about three cycles per lane here), adds the four rows in wavefront order and
+// flushes one global atomic per Gaussian, component and tile.
 #include "blend.hpp"
 
 namespace fsgs {
@@ -289,7 +290,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
   constexpr int kB = 64;
   __shared__ G3Hot s_hot[kB];
   __shared__ float s_feat[kB][3 + kMaxExtra + 1];
-  __shared__ float s_acc[kB][17];
+  __shared__ float s_part[4][kB][17];  // each wavefront's sums per staged Gaussian: plain stores, added in wavefront order
   __shared__ int s_max_contrib;
   const int gx = (W + kTile - 1) / kTile;
   const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
@@ -308,9 +309,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) wave_max = max(wave_max, __shfl_xor(wave_max, d, kWave));
   if (lane == 0) atomicMax(&s_max_contrib, wave_max);
-  if ((int) threadIdx.x < kB)
-#pragma unroll
-    for (int c = 0; c < 17; ++c) s_acc[threadIdx.x][c] = 0.0f;
+  for (int e = threadIdx.x; e < 4 * kB * 17; e += kBlendThreads) (&s_part[0][0][0])[e] = 0.0f;
   __syncthreads();
   const int n_todo = min(s_max_contrib, (int) (r1 - r0));
   const int rounds = (n_todo + kB - 1) / kB;
@@ -375,11 +374,18 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
         g[12] = h.G * dL_dalpha;
       }
       const float tot = wave_sum16_transposed(g);
-      if (lane < 16) atomicAdd(&s_acc[j][lane], tot);
+      if (lane < 16) s_part[wave][j][lane] = tot;  // a wavefront meets an entry once per batch
     }
     __syncthreads();
     if ((int) threadIdx.x < n_here) {
-      float* a = s_acc[threadIdx.x];
+      float a[16];
+#pragma unroll
+      for (int c = 0; c < 16; ++c) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum += s_part[w][threadIdx.x][c], s_part[w][threadIdx.x][c] = 0.0f;
+        a[c] = sum;
+      }
       const int id = s_hot[threadIdx.x].id;
 #pragma unroll
       for (int c = 0; c < 3; ++c)
@@ -393,10 +399,8 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
 #pragma unroll
       for (int c = 0; c < 4; ++c)
         if (a[9 + c] != 0.0f) atomicAdd(&g_conic_opacity[4 * (size_t) id + c], a[9 + c]);
-#pragma unroll
-      for (int c = 0; c < 16; ++c) a[c] = 0.0f;
     }
-    // a lane only touches its own accumulator row and staged entry between this flush and the barrier that follows
+    // a lane only touches its own rows of s_part and its staged entry between this flush and the barrier that follows
     // the next batch's LDS store
   }
 }
@@ -514,7 +518,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_extra_backward_kernel(int 
   constexpr int kB = 64, kC = 8, kPart = kC / 4;  // four threads gather one Gaussian's channels
   __shared__ G3Hot s_hot[kB];
   __shared__ float s_feat[kB][kC + 1];
-  __shared__ float s_acc[kB][17];
+  __shared__ float s_part[4][kB][17];  // each wavefront's sums per staged Gaussian: plain stores, added in wavefront order
   __shared__ int s_max_contrib;
   const int gx = (W + kTile - 1) / kTile;
   const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
@@ -527,9 +531,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_extra_backward_kernel(int 
   const int e0 = blockIdx.y * kC, n_ch = min(kC, E - e0);
   const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
   const int last_contrib = inside ? n_contrib[pix] : 0;
-  if ((int) threadIdx.x < kB)
-#pragma unroll
-    for (int c = 0; c < 17; ++c) s_acc[threadIdx.x][c] = 0.0f;
+  for (int e = threadIdx.x; e < 4 * kB * 17; e += kBlendThreads) (&s_part[0][0][0])[e] = 0.0f;
   const int n_todo = min(block_max_contrib(last_contrib, &s_max_contrib), (int) (r1 - r0));
   const int rounds = (n_todo + kB - 1) / kB;
   int wave_max = last_contrib;
@@ -596,11 +598,18 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_extra_backward_kernel(int 
         g[13] = h.G * dL_dalpha;
       }
       const float tot = wave_sum16_transposed(g);
-      if (lane < 16) atomicAdd(&s_acc[j][lane], tot);
+      if (lane < 16) s_part[wave][j][lane] = tot;  // a wavefront meets an entry once per batch
     }
     __syncthreads();
     if ((int) threadIdx.x < n_here) {
-      float* a = s_acc[threadIdx.x];
+      float a[16];
+#pragma unroll
+      for (int c = 0; c < 16; ++c) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum += s_part[w][threadIdx.x][c], s_part[w][threadIdx.x][c] = 0.0f;
+        a[c] = sum;
+      }
       const int id = s_hot[threadIdx.x].id;
       if (g_extras)
 #pragma unroll
@@ -614,10 +623,8 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_extra_backward_kernel(int 
 #pragma unroll
         for (int c = 0; c < 4; ++c)
           if (a[10 + c] != 0.0f) atomicAdd(&g_conic_opacity[4 * (size_t) id + c], a[10 + c]);
-#pragma unroll
-      for (int c = 0; c < 16; ++c) a[c] = 0.0f;
     }
-    // between this flush and the barrier after the next batch's LDS store a lane touches its own accumulator row and
+    // between this flush and the barrier after the next batch's LDS store a lane touches its own rows of s_part and
     // its own s_hot entry only; s_feat was last read before the barrier above
   }
 }

@@ -19,7 +19,7 @@ namespace {
 
 constexpr int kTableFloats  = 36864;  // 144 KB of LDS for the per-block table
 constexpr int kMaxAccBlocks = 256;    // partial tables per launch
-constexpr int kAccThreads   = 256;
+constexpr int kAccThreads   = 1024;  // 16 wavefronts share one LDS table: the loop is bound by gather latency, not by the atomics
 
 __global__ void __launch_bounds__(256) zero_floats_kernel(size_t n, float* __restrict__ p) {
   for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t) gridDim.x * blockDim.x)
@@ -58,16 +58,30 @@ __global__ void __launch_bounds__(256) lbs_backward_prepare_kernel(int M, int ce
 
 // Table row of control point j: [0,9) dL/dR, [9,12) dL/dt_eff, [12,16) direct rotation-residual gradient,
 // [16,16+S) scale-residual gradient.
-template <bool kLds>
+// kMode 0: atomics into a zeroed accumulator in global memory. 1: block-private table in LDS, stored as one partial.
+// 2: as 1 with a smaller table, and the control points' transforms and residuals staged in LDS as well: the loop's 18
+// gathers per neighbour are scattered 4-byte reads, which cost a cache-line lookup per lane in the texture path and a
+// bank access in LDS.
+constexpr int kStageTable  = 12288;  // table floats in mode 2 (48 KB)
+constexpr int kStageFloats = 16384;  // staged control-point floats in mode 2 (64 KB)
+template <int kMode>
 __global__ void __launch_bounds__(kAccThreads) lbs_backward_accumulate_kernel(int N, int M, int K, int S,
     float temperature, const float* __restrict__ points, const float* __restrict__ xf,
     const float* __restrict__ sp_r, const float* __restrict__ sp_s, const float* __restrict__ dist2,
     const int64_t* __restrict__ index, const float* __restrict__ g_xyz, const float* __restrict__ g_rot,
     const float* __restrict__ g_scale, float* __restrict__ g_points, float* __restrict__ g_dist2,
-    float* __restrict__ out /* kLds: partial[gridDim.x][M*F]; else accumulator[M*F], zeroed */) {
-  __shared__ float s_tab[kLds ? kTableFloats : 1];
+    float* __restrict__ out /* kMode > 0: partial[gridDim.x][M*F]; else accumulator[M*F], zeroed */) {
+  constexpr bool kLds = kMode > 0, kStage = kMode == 2;
+  __shared__ float s_tab[kStage ? kStageTable : (kLds ? kTableFloats : 1)];
+  __shared__ float s_ctrl[kStage ? kStageFloats : 1];
   const int F = 16 + S, cells = M * F;
   float* tab = kLds ? s_tab : out;
+  if (kStage) {  // [M][kXf] transforms, [M][4] rotation residuals, [M][S] scale residuals
+    for (int e = threadIdx.x; e < M * kXf; e += kAccThreads) s_ctrl[e] = xf[e];
+    for (int e = threadIdx.x; e < M * 4; e += kAccThreads) s_ctrl[M * kXf + e] = sp_r[e];
+    for (int e = threadIdx.x; e < M * S; e += kAccThreads) s_ctrl[M * (kXf + 4) + e] = sp_s[e];
+    xf = s_ctrl, sp_r = s_ctrl + M * kXf, sp_s = s_ctrl + M * (kXf + 4);
+  }
   if (kLds) {
     for (int e = threadIdx.x; e < cells; e += kAccThreads) s_tab[e] = 0.0f;
     __syncthreads();
@@ -281,13 +295,15 @@ FSGS_API int fsgs_lbs_blend_backward(int N, int M, int K, int centred, double te
                        acc);
   if (N > 0) {
     if (plan.lds) {
-      hipLaunchKernelGGL(lbs_backward_accumulate_kernel<true>, dim3(plan.blocks), dim3(kAccThreads), 0, s, N, M, K, S,
+      const bool stage = cells <= kStageTable && (int64_t) M * (kXf + 4 + S) <= kStageFloats;
+      auto kernel = stage ? lbs_backward_accumulate_kernel<2> : lbs_backward_accumulate_kernel<1>;
+      hipLaunchKernelGGL(kernel, dim3(plan.blocks), dim3(kAccThreads), 0, s, N, M, K, S,
                          (float) temperature, points, xf, sp_r, sp_s, dist2, index, g_xyz, g_rot, g_scale, g_points,
                          g_dist2, partial);
       hipLaunchKernelGGL(partial_sum_kernel, dim3(div_up(cells, kWave)), dim3(512), 0, s, cells, plan.blocks, partial,
                          acc);
     } else {
-      hipLaunchKernelGGL(lbs_backward_accumulate_kernel<false>, dim3(plan.blocks), dim3(kAccThreads), 0, s, N, M, K, S,
+      hipLaunchKernelGGL(lbs_backward_accumulate_kernel<0>, dim3(plan.blocks), dim3(kAccThreads), 0, s, N, M, K, S,
                          (float) temperature, points, xf, sp_r, sp_s, dist2, index, g_xyz, g_rot, g_scale, g_points,
                          g_dist2, acc);
     }
