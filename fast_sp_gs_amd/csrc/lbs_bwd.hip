@@ -59,11 +59,7 @@ __global__ void __launch_bounds__(256) lbs_backward_prepare_kernel(int M, int ce
 // Table row of control point j: [0,9) dL/dR, [9,12) dL/dt_eff, [12,16) direct rotation-residual gradient,
 // [16,16+S) scale-residual gradient.
 // kMode 0: atomics into a zeroed accumulator in global memory. 1: block-private table in LDS, stored as one partial.
-// 2: as 1 with a smaller table, and the control points' transforms and residuals staged in LDS as well: the loop's 18
-// gathers per neighbour are scattered 4-byte reads, which cost a cache-line lookup per lane in the texture path and a
-// bank access in LDS.
-constexpr int kStageTable  = 12288;  // table floats in mode 2 (48 KB)
-constexpr int kStageFloats = 16384;  // staged control-point floats in mode 2 (64 KB)
+constexpr int kStageTable = 12288;  // table floats of the binned variant below (48 KB)
 template <int kMode>
 __global__ void __launch_bounds__(kAccThreads) lbs_backward_accumulate_kernel(int N, int M, int K, int S,
     float temperature, const float* __restrict__ points, const float* __restrict__ xf,
@@ -71,17 +67,10 @@ __global__ void __launch_bounds__(kAccThreads) lbs_backward_accumulate_kernel(in
     const int64_t* __restrict__ index, const float* __restrict__ g_xyz, const float* __restrict__ g_rot,
     const float* __restrict__ g_scale, float* __restrict__ g_points, float* __restrict__ g_dist2,
     float* __restrict__ out /* kMode > 0: partial[gridDim.x][M*F]; else accumulator[M*F], zeroed */) {
-  constexpr bool kLds = kMode > 0, kStage = kMode == 2;
-  __shared__ float s_tab[kStage ? kStageTable : (kLds ? kTableFloats : 1)];
-  __shared__ float s_ctrl[kStage ? kStageFloats : 1];
+  constexpr bool kLds = kMode > 0;
+  __shared__ float s_tab[kLds ? kTableFloats : 1];
   const int F = 16 + S, cells = M * F;
   float* tab = kLds ? s_tab : out;
-  if (kStage) {  // [M][kXf] transforms, [M][4] rotation residuals, [M][S] scale residuals
-    for (int e = threadIdx.x; e < M * kXf; e += kAccThreads) s_ctrl[e] = xf[e];
-    for (int e = threadIdx.x; e < M * 4; e += kAccThreads) s_ctrl[M * kXf + e] = sp_r[e];
-    for (int e = threadIdx.x; e < M * S; e += kAccThreads) s_ctrl[M * (kXf + 4) + e] = sp_s[e];
-    xf = s_ctrl, sp_r = s_ctrl + M * kXf, sp_s = s_ctrl + M * (kXf + 4);
-  }
   if (kLds) {
     for (int e = threadIdx.x; e < cells; e += kAccThreads) s_tab[e] = 0.0f;
     __syncthreads();
@@ -144,6 +133,134 @@ __global__ void __launch_bounds__(kAccThreads) lbs_backward_accumulate_kernel(in
     float* mine = out + (size_t) blockIdx.x * cells;
     for (int e = threadIdx.x; e < cells; e += kAccThreads) mine[e] = s_tab[e];
   }
+}
+
+// The same sums without float atomics, for tables of up to kStageTable cells and K <= kBinK neighbours: LDS float
+// atomics retire about one lane every three cycles on this chip, and the 18 per neighbour above are what the kernel's
+// time is made of. A block takes 1024 points at a time. Every lane does its point's own outputs and counts its
+// neighbours per control point (integer LDS atomics), the counts are scanned, every (point, neighbour) pair is placed
+// in its control point's bin (weight and the lane that owns the point), and then each table cell is summed by one lane
+// over its control point's bin from the points' gradients parked in LDS. Partial tables go out as in mode 1.
+constexpr int kBinK = 4;
+constexpr int kBinFeat = 14;  // g[3] p[3] g_rot[4] g_scale[<= 4] per point
+__global__ void __launch_bounds__(kAccThreads) lbs_backward_binned_kernel(int N, int M, int K, int S,
+    float temperature, const float* __restrict__ points, const float* __restrict__ xf,
+    const float* __restrict__ sp_r, const float* __restrict__ sp_s, const float* __restrict__ dist2,
+    const int64_t* __restrict__ index, const float* __restrict__ g_xyz, const float* __restrict__ g_rot,
+    const float* __restrict__ g_scale, float* __restrict__ g_points, float* __restrict__ g_dist2,
+    float* __restrict__ out /* partial[gridDim.x][M*F] */) {
+  __shared__ float s_tab[kStageTable];
+  __shared__ float s_feat[kAccThreads][kBinFeat + 1];
+  __shared__ float s_pw[kAccThreads * kBinK];
+  __shared__ unsigned short s_pp[kAccThreads * kBinK];
+  __shared__ int s_count[kAccThreads], s_off[kAccThreads + 1], s_cursor[kAccThreads], s_wsum[kAccThreads / kWave];
+  const int F = 16 + S, cells = M * F;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int e = tid; e < cells; e += kAccThreads) s_tab[e] = 0.0f;
+  const float inv_t = 1.0f / temperature;
+  for (int n0 = blockIdx.x * kAccThreads; n0 < N; n0 += gridDim.x * kAccThreads) {
+    const int n = n0 + tid;
+    const bool live = n < N;
+    s_count[tid] = 0;
+    __syncthreads();
+    float mx = -__builtin_inff(), inv_den = 0.0f;
+    if (live) {
+      const float* d2   = dist2 + (size_t) n * K;
+      const int64_t* id = index + (size_t) n * K;
+      for (int k = 0; k < K; ++k)
+        if (id[k] >= 0 && id[k] < M) mx = fmaxf(mx, -d2[k] * inv_t);
+      float den = 0.0f;
+      for (int k = 0; k < K; ++k)
+        if (id[k] >= 0 && id[k] < M) den += expf(-d2[k] * inv_t - mx);
+      inv_den = den > 0.0f ? 1.0f / den : 0.0f;
+      const float p[3]  = {points[3 * (size_t) n], points[3 * (size_t) n + 1], points[3 * (size_t) n + 2]};
+      const float g[3]  = {g_xyz[3 * (size_t) n], g_xyz[3 * (size_t) n + 1], g_xyz[3 * (size_t) n + 2]};
+      const float gr[4] = {g_rot[4 * (size_t) n], g_rot[4 * (size_t) n + 1], g_rot[4 * (size_t) n + 2],
+                           g_rot[4 * (size_t) n + 3]};
+      float gs[4] = {0, 0, 0, 0};
+      for (int a = 0; a < S; ++a) gs[a] = g_scale[(size_t) S * n + a];
+      float* ft = s_feat[tid];
+#pragma unroll
+      for (int a = 0; a < 3; ++a) ft[a] = g[a], ft[3 + a] = p[a];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) ft[6 + a] = gr[a], ft[10 + a] = gs[a];
+      float gp[3] = {-g[0], -g[1], -g[2]}, dot = 0.0f;
+      for (int k = 0; k < K; ++k) {
+        const int64_t j = id[k];
+        if (j < 0 || j >= M) {
+          g_dist2[(size_t) n * K + k] = 0.0f;
+          continue;
+        }
+        atomicAdd(&s_count[j], 1);
+        const float w  = expf(-d2[k] * inv_t - mx) * inv_den;
+        const float* X = xf + (size_t) kXf * j;
+        float v = 0.0f;
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+          v += g[a] * (X[a * 3] * p[0] + X[a * 3 + 1] * p[1] + X[a * 3 + 2] * p[2] + X[9 + a]);
+          gp[a] += w * (X[a] * g[0] + X[3 + a] * g[1] + X[6 + a] * g[2]);
+        }
+#pragma unroll
+        for (int a = 0; a < 4; ++a) v += gr[a] * sp_r[4 * j + a];
+        for (int a = 0; a < S; ++a) v += gs[a] * sp_s[(size_t) S * j + a];
+        g_dist2[(size_t) n * K + k] = v;  // parked until the weighted mean is known
+        dot += w * v;
+      }
+      for (int k = 0; k < K; ++k) {
+        const int64_t j = id[k];
+        if (j < 0 || j >= M) continue;
+        const float w = expf(-d2[k] * inv_t - mx) * inv_den;
+        g_dist2[(size_t) n * K + k] = -(w * (g_dist2[(size_t) n * K + k] - dot)) * inv_t;
+      }
+      if (g_points) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) g_points[3 * (size_t) n + a] = gp[a];
+      }
+    }
+    __syncthreads();
+    // exclusive scan of the counts (M <= 1024: one control point per lane)
+    const int cnt = tid < M ? s_count[tid] : 0;
+    int incl = cnt;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int t = __shfl_up(incl, d, kWave);
+      if (lane >= d) incl += t;
+    }
+    if (lane == kWave - 1) s_wsum[wave] = incl;
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < wave; ++w) base += s_wsum[w];
+    s_off[tid] = s_cursor[tid] = base + incl - cnt;
+    if (tid == kAccThreads - 1) s_off[kAccThreads] = base + incl;
+    __syncthreads();
+    if (live) {
+      const float* d2   = dist2 + (size_t) n * K;
+      const int64_t* id = index + (size_t) n * K;
+      for (int k = 0; k < K; ++k) {
+        const int64_t j = id[k];
+        if (j < 0 || j >= M) continue;
+        const int pos = atomicAdd(&s_cursor[j], 1);
+        s_pw[pos] = expf(-d2[k] * inv_t - mx) * inv_den;
+        s_pp[pos] = (unsigned short) tid;
+      }
+    }
+    __syncthreads();
+    // table row of control point j: [0,9) w g[a] p[b], [9,12) w g[a], [12,16) w g_rot[a], [16,16+S) w g_scale[a]
+    for (int cell = tid; cell < cells; cell += kAccThreads) {
+      const int j = cell / F, c = cell - j * F;
+      const int fa = c < 9 ? c / 3 : (c < 12 ? c - 9 : c - 6), fb = c < 9 ? 3 + (c - 3 * (c / 3)) : -1;
+      float sum = 0.0f;
+      for (int q = s_off[j]; q < s_off[j + 1]; ++q) {
+        const float* ft = s_feat[s_pp[q]];
+        const float f   = fb >= 0 ? ft[fa] * ft[fb] : ft[fa];
+        sum += s_pw[q] * f;
+      }
+      s_tab[cell] += sum;
+    }
+    __syncthreads();
+  }
+  float* mine = out + (size_t) blockIdx.x * cells;
+  for (int e = tid; e < cells; e += kAccThreads) mine[e] = s_tab[e];
 }
 
 // g_x[n] = sum_k 2 g_k (x_n - y_idx) written directly; -that accumulated into row idx of the table [M][D].
@@ -295,8 +412,8 @@ FSGS_API int fsgs_lbs_blend_backward(int N, int M, int K, int centred, double te
                        acc);
   if (N > 0) {
     if (plan.lds) {
-      const bool stage = cells <= kStageTable && (int64_t) M * (kXf + 4 + S) <= kStageFloats;
-      auto kernel = stage ? lbs_backward_accumulate_kernel<2> : lbs_backward_accumulate_kernel<1>;
+      const bool binned = cells <= kStageTable && M <= kAccThreads && K <= kBinK;
+      auto kernel = binned ? lbs_backward_binned_kernel : lbs_backward_accumulate_kernel<1>;
       hipLaunchKernelGGL(kernel, dim3(plan.blocks), dim3(kAccThreads), 0, s, N, M, K, S,
                          (float) temperature, points, xf, sp_r, sp_s, dist2, index, g_xyz, g_rot, g_scale, g_points,
                          g_dist2, partial);
