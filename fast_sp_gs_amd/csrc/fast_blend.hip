@@ -284,11 +284,14 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
     const float* __restrict__ dL_dpix, const float* __restrict__ dL_dextras, const float* __restrict__ dL_dopacity,
     float* __restrict__ g_means2D, float* __restrict__ g_normal_opacity, float* __restrict__ g_colors,
     float* __restrict__ g_trans, float* __restrict__ g_inv) {
-  __shared__ FastHot s_hot[kBatch];
-  __shared__ SplatCold s_cold[kBatch];
-  __shared__ float s_acc[kBatch][kFastGradSlots];
+  constexpr int kB = 64;  // surfels staged per round
+  __shared__ FastHot s_hot[kB];
+  __shared__ SplatCold s_cold[kB];
+  // each wavefront's sums per staged surfel, written once per entry with a plain store and added in wavefront order at
+  // the flush (LDS float atomics cost about three cycles per lane)
+  __shared__ float s_part[4][kB][kFastGradSlots];
   __shared__ int s_max_contrib;
-  __shared__ unsigned char s_mask[kBatch];
+  __shared__ unsigned char s_mask[kB];
 
   const int gx = (W + kTile - 1) / kTile;
   const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
@@ -310,11 +313,10 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) wave_max_contrib = max(wave_max_contrib, __shfl_xor(wave_max_contrib, d, kWave));
   if (lane == 0) atomicMax(&s_max_contrib, wave_max_contrib);
-#pragma unroll
-  for (int c = 0; c < kFastGradSlots; ++c) s_acc[threadIdx.x][c] = 0.0f;
+  for (int e = threadIdx.x; e < 4 * kB * kFastGradSlots; e += kBlendThreads) (&s_part[0][0][0])[e] = 0.0f;
   __syncthreads();
   const int n_todo = min(s_max_contrib, (int) (r1 - r0));
-  const int rounds = (n_todo + kBatch - 1) / kBatch;
+  const int rounds = (n_todo + kB - 1) / kB;
 
   const float T_final = inside ? 1.0f - out_opacity[pix] : 0.0f;
   float T = T_final;
@@ -345,30 +347,30 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
   float last_dL_dT = 0, last_alpha = 0;
 
   FastSplat next;
-  if ((int) threadIdx.x < n_todo)
+  if ((int) threadIdx.x < min(n_todo, kB))
     next = gather_fast(point_list[r0 + (n_todo - 1 - (int) threadIdx.x)], means2D, colors, normal_opacity, trans_mat,
                        inverse_m);
 
   for (int b = 0; b < rounds; ++b) {
-    const int n_here = min(kBatch, n_todo - b * kBatch);
+    const int n_here = min(kB, n_todo - b * kB);
     if ((int) threadIdx.x < n_here) {
       s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
       s_mask[threadIdx.x] = (unsigned char) fast_quadrant_mask(next, tile_x * kTile, tile_y * kTile, ordered);
     }
     __syncthreads();
-    const int nxt = (b + 1) * kBatch + (int) threadIdx.x;
-    if (nxt < n_todo)
+    const int nxt = (b + 1) * kB + (int) threadIdx.x;
+    if ((int) threadIdx.x < kB && nxt < n_todo)
       next = gather_fast(point_list[r0 + (n_todo - 1 - nxt)], means2D, colors, normal_opacity, trans_mat, inverse_m);
 
-    for (int chunk = 0; chunk < kBatch / kWave; ++chunk) {
+    for (int chunk = 0; chunk < kB / kWave; ++chunk) {
       const int jj = chunk * kWave + lane;
       unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u) &&
-                                         (n_todo - 1 - (b * kBatch + jj)) < wave_max_contrib);
+                                         (n_todo - 1 - (b * kB + jj)) < wave_max_contrib);
       while (todo) {
         const int j = chunk * kWave + __builtin_ctzll(todo);
         todo &= todo - 1;
-        const int pos = n_todo - 1 - (b * kBatch + j);
+        const int pos = n_todo - 1 - (b * kB + j);
         FastHit h;
         const bool hit = fast_intersect_flat(s_hot[j], pxf, pyf, near_n, h) && (pos < last_contrib);
         if (__ballot(hit) == 0ull) continue;
@@ -434,20 +436,27 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
           g[15] = h.G * dL_dalpha;
         }
         const float tot = wave_sum16_transposed(g);
-        if (lane < 16) atomicAdd(&s_acc[j][lane], tot);
+        if (lane < 16) s_part[wave][j][lane] = tot;
         if (kAux) {
           const float tot8 = wave_sum8_transposed(g8);
-          if (lane < 5) atomicAdd(&s_acc[j][16 + lane], tot8);
+          if (lane < 5) s_part[wave][j][16 + lane] = tot8;
         } else if (__ballot(filtered) != 0ull) {
           const float sx = wave_sum_to_lane63(g8[3]), sy = wave_sum_to_lane63(g8[4]);
-          if (lane == 63) atomicAdd(&s_acc[j][19], sx), atomicAdd(&s_acc[j][20], sy);
+          if (lane == 63) s_part[wave][j][19] = sx, s_part[wave][j][20] = sy;
         }
       }
     }
     __syncthreads();
     if ((int) threadIdx.x < n_here) {
       const int id = s_cold[threadIdx.x].id;
-      float* a     = s_acc[threadIdx.x];
+      float a[kFastGradSlots];
+#pragma unroll
+      for (int c = 0; c < kFastGradSlots; ++c) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum += s_part[w][threadIdx.x][c], s_part[w][threadIdx.x][c] = 0.0f;
+        a[c] = sum;
+      }
 #pragma unroll
       for (int c = 0; c < 3; ++c)
         if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
@@ -463,8 +472,6 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
 #pragma unroll
       for (int c = 0; c < 2; ++c)
         if (a[19 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[19 + c]);
-#pragma unroll
-      for (int c = 0; c < kFastGradSlots; ++c) a[c] = 0.0f;
     }
   }
 }
