@@ -239,12 +239,17 @@ __global__ void __launch_bounds__(256) cdist_top_backward_kernel(int B, int N, i
 }
 
 // ---- K nearest control points ---------------------------------------------------------------------------------------------
-// Squared distances ascending, ties -> lower index first. One lane per query, candidates broadcast from LDS.
+// Squared distances ascending, ties -> lower index first. One lane per query, candidates broadcast from LDS eight at a
+// time: the eight distances are formed first (their LDS reads are issued together instead of one exposed round trip per
+// candidate), then each is offered to the sorted list. The list update is a clamp per slot for the distances
+// (new[k] = med3(old[k-1], d, old[k]), the list being sorted) and two selects per slot for the indices, decided by the
+// strict comparisons against the old list, so an equal distance never displaces an earlier (lower) index.
+constexpr int kKnnUnroll = 8;
 template <int kD, int kK>
 __global__ void __launch_bounds__(256) knn_topk_kernel(int N, int M, int D, int K, const float* __restrict__ x,
     const float* __restrict__ y, float* __restrict__ dist2, int64_t* __restrict__ index) {
 #pragma clang fp contract(off)
-  __shared__ float s_y[kD > 0 ? kCtrlChunk * kD : 1];
+  __shared__ __attribute__((aligned(16))) float s_y[kD > 0 ? (kCtrlChunk + kKnnUnroll) * kD : 1];
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   const float* xp = x + (size_t) (n < N ? n : 0) * D;
   float xr[kD > 0 ? kD : 1];
@@ -255,38 +260,51 @@ __global__ void __launch_bounds__(256) knn_topk_kernel(int N, int M, int D, int 
   int bi[kK];
 #pragma unroll
   for (int k = 0; k < kK; ++k) bd[k] = __builtin_inff(), bi[k] = -1;
+  auto offer = [&](float cd, int ci) {
+    if (cd < bd[kK - 1]) {
+      bool lt[kK];
+#pragma unroll
+      for (int k = 0; k < kK; ++k) lt[k] = cd < bd[k];
+#pragma unroll
+      for (int k = kK - 1; k >= 1; --k) {
+        bd[k] = __builtin_amdgcn_fmed3f(bd[k - 1], cd, bd[k]);
+        bi[k] = lt[k - 1] ? bi[k - 1] : (lt[k] ? ci : bi[k]);
+      }
+      bd[0] = fminf(bd[0], cd);
+      bi[0] = lt[0] ? ci : bi[0];
+    }
+  };
   for (int m0 = 0; m0 < M; m0 += kCtrlChunk) {
     const int mc = min(kCtrlChunk, M - m0);
     if (kD > 0) {
       __syncthreads();
-      for (int k = threadIdx.x; k < mc * kD; k += blockDim.x) s_y[k] = y[(size_t) m0 * kD + k];
+      const int padded = (mc + kKnnUnroll - 1) / kKnnUnroll * kKnnUnroll;  // candidates past the end sit at infinity
+      for (int k = threadIdx.x; k < padded * kD; k += blockDim.x)
+        s_y[k] = k < mc * kD ? y[(size_t) m0 * kD + k] : __builtin_inff();
       __syncthreads();
-    }
-    for (int m = 0; m < mc; ++m) {
-      float sum = 0.0f;
-      if (kD > 0) {
+      for (int m = 0; m < mc; m += kKnnUnroll) {
+        float cand[kKnnUnroll];
 #pragma unroll
-        for (int d = 0; d < kD; ++d) {
-          const float t = xr[d] - s_y[m * kD + d];
-          sum += t * t;
+        for (int u = 0; u < kKnnUnroll; ++u) {
+          float sum = 0.0f;
+#pragma unroll
+          for (int d = 0; d < kD; ++d) {
+            const float t = xr[d] - s_y[(m + u) * kD + d];
+            sum += t * t;
+          }
+          cand[u] = sum;
         }
-      } else {
+#pragma unroll
+        for (int u = 0; u < kKnnUnroll; ++u) offer(cand[u], m0 + m + u);
+      }
+    } else {
+      for (int m = 0; m < mc; ++m) {
+        float sum = 0.0f;
         for (int d = 0; d < D; ++d) {
           const float t = xp[d] - y[(size_t) (m0 + m) * D + d];
           sum += t * t;
         }
-      }
-      if (sum < bd[kK - 1]) {  // strict: an equal distance never displaces an earlier (lower) index
-        float cd = sum;
-        int ci   = m0 + m;
-#pragma unroll
-        for (int k = 0; k < kK; ++k) {
-          const bool sw = cd < bd[k];
-          const float td = bd[k];
-          const int ti   = bi[k];
-          bd[k] = sw ? cd : td, bi[k] = sw ? ci : ti;
-          cd = sw ? td : cd, ci = sw ? ti : ci;
-        }
+        offer(sum, m0 + m);
       }
     }
   }
