@@ -44,6 +44,15 @@ inline int check_launch(const char* what) {
 
 inline int div_up(int64_t a, int64_t b) { return (int) ((a + b - 1) / b); }
 
+// Block barrier that orders LDS traffic only. __syncthreads() also waits for every global load and store the
+// wavefront has in flight (s_waitcnt vmcnt(0)), which puts the latency of loads issued ahead of time, and of stores
+// nobody in the block reads back, on the critical path of each round; this one waits for LDS alone.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 // float -> int with saturation and NaN -> 0 (what v_cvt_i32_f32 does; spelled out so the result does not depend on

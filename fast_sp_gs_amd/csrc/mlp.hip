@@ -38,6 +38,10 @@ constexpr int kMlpRows    = 32;                       // rows per block
 constexpr int kMlpMaxIn   = 96;                       // padded input width limit
 constexpr int kMlpStride  = kMlpWidth + kMlpMaxIn + 8;  // LDS row stride in bf16 (+8 keeps 16-byte rows off one bank)
 constexpr int kMlpThreads = 256;
+// Forward and backward chain: eight wavefronts per block, one 32 x 32 output tile each. The batch is small (16 blocks at
+// B = 512) and the nine layers depend on each other, so a layer's time is the latency of its weight fragments: with one
+// tile per wavefront a whole layer's 16 fragments fit in registers and are requested together.
+constexpr int kChainThreads = 512;
 
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest even
   uint32_t u = __float_as_uint(f);
@@ -97,7 +101,7 @@ __global__ void __launch_bounds__(256) pack_jobs_kernel(PackTable table) {
 __device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
 
 template <bool kSave>
-__global__ void __launch_bounds__(kMlpThreads) mlp_forward_kernel(int B, int Din, int n_layers, int skip, int n_out,
+__global__ void __launch_bounds__(kChainThreads) mlp_forward_kernel(int B, int Din, int n_layers, int skip, int n_out,
     const float* __restrict__ in, const uint16_t* __restrict__ packed, const float* __restrict__ bias,
     float* __restrict__ out, uint16_t* __restrict__ saved) {
   __shared__ __attribute__((aligned(16))) uint16_t s_act[2][kMlpRows][kMlpStride];
@@ -107,7 +111,7 @@ __global__ void __launch_bounds__(kMlpThreads) mlp_forward_kernel(int B, int Din
   const int Din_pad = (Din + 15) & ~15;
 
   // stage the (bf16) input rows, zero padded
-  for (int e = threadIdx.x; e < kMlpRows * Din_pad; e += kMlpThreads) {
+  for (int e = threadIdx.x; e < kMlpRows * Din_pad; e += kChainThreads) {
     const int r = e / Din_pad, k = e - r * Din_pad;
     const float v = (row0 + r < B && k < Din) ? in[(size_t) (row0 + r) * Din + k] : 0.0f;
     const uint16_t h = f32_to_bf16(v);
@@ -120,49 +124,63 @@ __global__ void __launch_bounds__(kMlpThreads) mlp_forward_kernel(int B, int Din
   int K = Din, K_pad = Din_pad;
   const uint16_t* W = packed;
   const float* bl   = bias;
+  // Fragment u (k-step u, clamped to the layer's last step) of row tile `wave` of a layer whose weights start at Wl;
+  // consecutive k-steps are 512 elements apart.
+  auto fragment = [&](const uint16_t* Wl, int K_pad_l, int u) {
+    const int steps = K_pad_l >> 4;
+    return *(const bf16x8*) (Wl + ((size_t) wave * steps + min(u, steps - 1)) * 512 + lane * 8);
+  };
+  // The weights do not depend on the activations: the first sixteen fragments of the NEXT layer are requested at the
+  // start of each layer and arrive while this layer's products, epilogue and barrier run.
+  bf16x8 ahead[16];
+#pragma unroll
+  for (int u = 0; u < 16; ++u) ahead[u] = fragment(W, K_pad, u);
   for (int layer = 0; layer < n_layers; ++layer) {
-    floatx16 acc[2];
+    floatx16 acc;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
     const int arow = lane & 31, kofs = 8 * (lane >> 5);
-    // row tiles 2 * wave and 2 * wave + 1 of this layer; consecutive k-steps are 512 elements apart, which is what
-    // advancing k0 by 16 does to a pointer that steps 32 elements per unit of k0
-    const uint16_t* wrow0 = W + (size_t) (2 * wave) * (K_pad >> 4) * 512 + lane * 8;
-    const uint16_t* wrow1 = wrow0 + (size_t) (K_pad >> 4) * 512;
-    int k0 = 0;
-    for (; k0 + 64 <= K_pad; k0 += 64) {  // four k-steps per trip: eight weight reads in flight
-      bf16x8 b0[4], b1[4];
+    const uint16_t* wrow = W + (size_t) wave * (K_pad >> 4) * 512 + lane * 8;
+    bf16x8 b[16];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        b0[u] = *(const bf16x8*) (wrow0 + (k0 + 16 * u) * 32);
-        b1[u] = *(const bf16x8*) (wrow1 + (k0 + 16 * u) * 32);
+    for (int u = 0; u < 16; ++u) b[u] = ahead[u];
+    if (layer + 1 < n_layers) {
+      const int K_after = (((layer == skip) ? Din + kMlpWidth : kMlpWidth) + 15) & ~15;
+#pragma unroll
+      for (int u = 0; u < 16; ++u) ahead[u] = fragment(W + (size_t) kMlpWidth * K_pad, K_after, u);
+    }
+    const int first = min(K_pad >> 4, 16);
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      if (u < first) {
+        const bf16x8 a = *(const bf16x8*) &s_act[cur][arow][16 * u + kofs];
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[u], acc, 0, 0, 0);
       }
+    int k0 = 16 * first;
+    for (; k0 + 64 <= K_pad; k0 += 64) {
+      bf16x8 b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) b[u] = *(const bf16x8*) (wrow + (k0 + 16 * u) * 32);
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const bf16x8 a = *(const bf16x8*) &s_act[cur][arow][k0 + 16 * u + kofs];
-        acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0[u], acc[0], 0, 0, 0);
-        acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1[u], acc[1], 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[u], acc, 0, 0, 0);
       }
     }
     for (; k0 < K_pad; k0 += 16) {
-      const bf16x8 a  = *(const bf16x8*) &s_act[cur][arow][k0 + kofs];
-      const bf16x8 b0 = *(const bf16x8*) (wrow0 + k0 * 32);
-      const bf16x8 b1 = *(const bf16x8*) (wrow1 + k0 * 32);
-      acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0, acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1, acc[1], 0, 0, 0);
+      const bf16x8 a = *(const bf16x8*) &s_act[cur][arow][k0 + kofs];
+      const bf16x8 b = *(const bf16x8*) (wrow + k0 * 32);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
     }
     // bias + ReLU -> bf16 into the other buffer; after the skip layer the input goes in front of the hidden state
     const int nxt = cur ^ 1;
     const int col_shift = (layer == skip) ? Din : 0;
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int col = wave * 64 + t * 32 + (lane & 31);
+    {
+      const int col  = wave * 32 + (lane & 31);
       const float bv = bl[col];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float v    = fmaxf(acc[t][r] + bv, 0.0f);
+        const float v    = fmaxf(acc[r] + bv, 0.0f);
         const uint16_t h = f32_to_bf16(v);
         const int row    = acc_row(r, lane);
         s_act[nxt][row][col_shift + col] = h;
@@ -172,17 +190,17 @@ __global__ void __launch_bounds__(kMlpThreads) mlp_forward_kernel(int B, int Din
     int K_next = kMlpWidth;
     if (layer == skip) {
       K_next = Din + kMlpWidth;
-      for (int e = threadIdx.x; e < kMlpRows * Din; e += kMlpThreads) {
+      for (int e = threadIdx.x; e < kMlpRows * Din; e += kChainThreads) {
         const int r = e / Din, k = e - r * Din;
         s_act[nxt][r][k] = s_in[r][k];
       }
     }
     const int K_next_pad = (K_next + 15) & ~15;
-    for (int e = threadIdx.x; e < kMlpRows * (K_next_pad - K_next); e += kMlpThreads) {
+    for (int e = threadIdx.x; e < kMlpRows * (K_next_pad - K_next); e += kChainThreads) {
       const int r = e / (K_next_pad - K_next), k = e - r * (K_next_pad - K_next);
       s_act[nxt][r][K_next + k] = 0;
     }
-    __syncthreads();
+    lds_barrier();
     W += (size_t) kMlpWidth * K_pad;
     bl += kMlpWidth;
     K = K_next, K_pad = K_next_pad;
@@ -219,7 +237,7 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_floa
 
 // dZ[l] for every layer, back to front. packed_t holds, for l = 1 .. n_layers-1, the hidden part of W_l transposed:
 // [256 inputs][256 outputs] bf16.
-__global__ void __launch_bounds__(kMlpThreads) mlp_backward_chain_kernel(int B, int n_layers, int n_out,
+__global__ void __launch_bounds__(kChainThreads) mlp_backward_chain_kernel(int B, int n_layers, int n_out,
     const float* __restrict__ heads_w /*[n_out][256] fp32*/, const uint16_t* __restrict__ packed_t,
     const uint16_t* __restrict__ saved, const float* __restrict__ g_out, uint16_t* __restrict__ dz) {
   __shared__ __attribute__((aligned(16))) uint16_t s_dz[kMlpRows][kMlpWidth + 8];
@@ -228,11 +246,12 @@ __global__ void __launch_bounds__(kMlpThreads) mlp_backward_chain_kernel(int B, 
   const int row0 = blockIdx.x * kMlpRows;
   {
     // dZ of the last layer: (g_out . W_heads) where the stored state is non-zero. Lane t owns column t of all 32 rows.
-    for (int e = threadIdx.x; e < kMlpRows * 32; e += kMlpThreads) {
+    for (int e = threadIdx.x; e < kMlpRows * 32; e += kChainThreads) {
       const int r = e >> 5, k = e & 31;
       s_g[r][k] = (row0 + r < B && k < n_out) ? g_out[(size_t) (row0 + r) * n_out + k] : 0.0f;
     }
     __syncthreads();
+    if (threadIdx.x < kMlpWidth) {
     const int c = threadIdx.x;
     const size_t top = (size_t) (n_layers - 1) * B;
     uint16_t keep[kMlpRows];  // read at clamped rows, unconditionally, so the loads overlap the products below
@@ -253,49 +272,54 @@ __global__ void __launch_bounds__(kMlpThreads) mlp_backward_chain_kernel(int B, 
       if (live) dz[(top + row0 + r) * kMlpWidth + c] = h;
       s_dz[r][c] = h;
     }
+    }
   }
+  // all sixteen weight fragments of a wavefront's tile are requested together, one layer ahead (they do not depend on
+  // dZ), and the stored states that mask a layer's result are fetched while the matrix cores run
+  auto fragment = [&](int layer, int u) {
+    return *(const bf16x8*) (packed_t + ((size_t) ((layer - 1) * 8 + wave) * (kMlpWidth / 16) + u) * 512 + lane * 8);
+  };
+  bf16x8 ahead[16];
+  if (n_layers >= 2)
+#pragma unroll
+    for (int u = 0; u < 16; ++u) ahead[u] = fragment(n_layers - 1, u);
   __syncthreads();
   for (int layer = n_layers - 1; layer >= 1; --layer) {
-    floatx16 acc[2];
+    floatx16 acc;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
     const int arow = lane & 31, kofs = 8 * (lane >> 5);
-    const uint16_t* wrow0 = packed_t + (size_t) ((layer - 1) * 8 + 2 * wave) * (kMlpWidth / 16) * 512 + lane * 8;
-    const uint16_t* wrow1 = wrow0 + (size_t) (kMlpWidth / 16) * 512;
-    // the stored states that mask this layer's result are fetched while the matrix cores run
+    bf16x8 b[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) b[u] = ahead[u];
+    if (layer >= 2)
+#pragma unroll
+      for (int u = 0; u < 16; ++u) ahead[u] = fragment(layer - 1, u);
     const size_t base = (size_t) (layer - 1) * B;
-    uint16_t keep[2][16];
+    uint16_t keep[16];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        // rows past the batch reuse the last row's mask: their results stay in LDS and are never stored
-        const int row = min(row0 + acc_row(r, lane), B - 1);
-        keep[t][r] = saved[(base + row) * kMlpWidth + wave * 64 + t * 32 + (lane & 31)];
-      }
-#pragma unroll 8
-    for (int k0 = 0; k0 < kMlpWidth; k0 += 16) {
-      const bf16x8 a  = *(const bf16x8*) &s_dz[arow][k0 + kofs];
-      const bf16x8 b0 = *(const bf16x8*) (wrow0 + k0 * 32);
-      const bf16x8 b1 = *(const bf16x8*) (wrow1 + k0 * 32);
-      acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0, acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1, acc[1], 0, 0, 0);
+    for (int r = 0; r < 16; ++r) {
+      // rows past the batch reuse the last row's mask: their results stay in LDS and are never stored
+      const int row = min(row0 + acc_row(r, lane), B - 1);
+      keep[r] = saved[(base + row) * kMlpWidth + wave * 32 + (lane & 31)];
     }
-    __syncthreads();  // every wavefront has read dZ[layer] before it is overwritten
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int col = wave * 64 + t * 32 + (lane & 31);
+    for (int u = 0; u < 16; ++u) {
+      const bf16x8 a = *(const bf16x8*) &s_dz[arow][16 * u + kofs];
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[u], acc, 0, 0, 0);
+    }
+    lds_barrier();  // every wavefront has read dZ[layer] before it is overwritten
+    {
+      const int col = wave * 32 + (lane & 31);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row    = acc_row(r, lane);
-        const uint16_t h = keep[t][r] != 0 ? f32_to_bf16(acc[t][r]) : (uint16_t) 0;
+        const uint16_t h = keep[r] != 0 ? f32_to_bf16(acc[r]) : (uint16_t) 0;
         if (row0 + row < B) dz[(base + row0 + row) * kMlpWidth + col] = h;
         s_dz[row][col] = h;
       }
     }
-    __syncthreads();
+    lds_barrier();
   }
 }
 
@@ -489,7 +513,7 @@ FSGS_API int fsgs_mlp_forward(int B, int Din, int width, int n_layers, int skip,
                "mlp_forward: bad layer structure (layers %d, skip %d, outputs %d)", n_layers, skip, n_out);
   if (B == 0) return kOk;
   auto kernel = saved ? mlp_forward_kernel<true> : mlp_forward_kernel<false>;
-  hipLaunchKernelGGL(kernel, dim3(div_up(B, kMlpRows)), dim3(kMlpThreads), 0, (hipStream_t) stream, B, Din, n_layers,
+  hipLaunchKernelGGL(kernel, dim3(div_up(B, kMlpRows)), dim3(kChainThreads), 0, (hipStream_t) stream, B, Din, n_layers,
                      skip, n_out, in, packed, bias, out, saved);
   return check_launch("mlp_forward");
 }
@@ -515,7 +539,7 @@ FSGS_API int fsgs_mlp_backward(int B, int Din, int width, int n_layers, int skip
   uint16_t* dz  = (uint16_t*) workspace;
   // with an empty batch the weight kernel's chunk loop does not run and it writes zeros
   if (B > 0)
-    hipLaunchKernelGGL(mlp_backward_chain_kernel, dim3(div_up(B, kMlpRows)), dim3(kMlpThreads), 0, s, B, n_layers,
+    hipLaunchKernelGGL(mlp_backward_chain_kernel, dim3(div_up(B, kMlpRows)), dim3(kChainThreads), 0, s, B, n_layers,
                        n_out, heads_w, packed_t, saved, g_out, dz);
   int tiles = 0, K = Din;
   for (int l = 0; l <= n_layers; ++l) {
