@@ -28,7 +28,8 @@ constexpr int kGradSlots = 18;
 #ifndef FSGS_BWD_WAVES
 #define FSGS_BWD_WAVES 4
 #endif
-constexpr int kBwdBatch = FSGS_BWD_BATCH;  // surfels staged per round (<= block size)
+constexpr int kBwdBatch = FSGS_BWD_BATCH;  // surfels staged per round
+static_assert(kBwdBatch <= kWave, "one wavefront stages a batch and another flushes it");
 
 template <bool kAux, bool kFlow, bool kSlots>
 __global__ void __launch_bounds__(kBlendThreads) __attribute__((amdgpu_waves_per_eu(FSGS_BWD_WAVES, FSGS_BWD_WAVES)))
@@ -48,7 +49,9 @@ blend_backward_kernel(
   // wavefront meets an entry once per batch); the flush adds the four rows in wavefront order, so a tile's sums do not
   // depend on timing. +1: the odd stride keeps the flush free of bank conflicts.
   __shared__ float s_part[4][kBwdBatch][kGradSlots + 1];
-  __shared__ int s_slot[kSlots ? kBwdBatch : 1];      // where this (surfel, tile) instance sits in surfel order
+  // Where a staged (surfel, tile) instance's sums go: its position in surfel order (kSlots) or the surfel's id. Two
+  // copies by batch parity: wavefront 1 stages batch b + 1 while wavefront 0 still flushes batch b.
+  __shared__ int s_slot[2][kBwdBatch];
   __shared__ float s_t2[kFlow ? kBwdBatch * 9 : 1];
   __shared__ int s_max_contrib;
   __shared__ unsigned char s_mask[kBwdBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
@@ -116,9 +119,12 @@ blend_backward_kernel(
   float next_t2[9];
   int next_radius = 0;
   int64_t next_off = 0;
-  if ((int) threadIdx.x < min(n_todo, kBwdBatch)) {
+  // Gathering and staging are wavefront 1's job, the flush of a finished batch wavefront 0's: both sit between the same
+  // two barriers, where the other wavefronts wait, and so run side by side instead of one after the other.
+  const int st = (int) threadIdx.x - kWave;  // staging slot of this lane (wavefront 1: 0 .. 63)
+  if (st >= 0 && st < min(n_todo, kBwdBatch)) {
     SplatExtra ex;
-    next = gather_splat(point_list[r0 + (n_todo - 1 - (int) threadIdx.x)], means2D, colors, normal_opacity, trans_mat,
+    next = gather_splat(point_list[r0 + (n_todo - 1 - st)], means2D, colors, normal_opacity, trans_mat,
                         records, &ex);
     if (kFlow)
 #pragma unroll
@@ -134,23 +140,25 @@ blend_backward_kernel(
 
   for (int b = 0; b < rounds; ++b) {
     const int n_here = min(kBwdBatch, n_todo - b * kBwdBatch);
-    if ((int) threadIdx.x < n_here) {
-      s_hot[threadIdx.x]  = next.hot;
-      s_cold[threadIdx.x] = next.cold;
-      s_mask[threadIdx.x] = (unsigned char) quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile, ordered);
+    if (st >= 0 && st < n_here) {
+      s_hot[st]  = next.hot;
+      s_cold[st] = next.cold;
+      s_mask[st] = (unsigned char) quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile, ordered);
       if (kFlow)
 #pragma unroll
-        for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
+        for (int k = 0; k < 9; ++k) s_t2[st * 9 + k] = next_t2[k];
       if (kSlots) {
         // position of this instance in the surfel-ordered key list: the binning emits a surfel's tiles row-major
         // over its rectangle, starting at the surfel's prefix-scan offset (gaussian_prepare.cu:47-83)
         const TileRect r = tile_rect(next.hot.cx, next.hot.cy, next_radius, gx, gy);
-        s_slot[threadIdx.x] = (int) (next_off + (int64_t) (tile_y - r.y0) * (r.x1 - r.x0) + (tile_x - r.x0));
+        s_slot[b & 1][st] = (int) (next_off + (int64_t) (tile_y - r.y0) * (r.x1 - r.x0) + (tile_x - r.x0));
+      } else {
+        s_slot[b & 1][st] = next.cold.id;
       }
     }
     __syncthreads();
-    const int nxt = (b + 1) * kBwdBatch + (int) threadIdx.x;
-    if ((int) threadIdx.x < kBwdBatch && nxt < n_todo) {
+    const int nxt = (b + 1) * kBwdBatch + st;
+    if (st >= 0 && st < kBwdBatch && nxt < n_todo) {
       SplatExtra ex;
       next = gather_splat(point_list[r0 + (n_todo - 1 - nxt)], means2D, colors, normal_opacity, trans_mat, records,
                           &ex);
@@ -290,7 +298,7 @@ blend_backward_kernel(
      }
     }
     __syncthreads();
-    // flush the batch
+    // flush the batch (wavefront 0: lane = staged surfel), adding the four wavefronts' rows in wavefront order
     if ((int) threadIdx.x < n_here) {
       float a[kGradSlots];
 #pragma unroll
@@ -307,13 +315,13 @@ blend_backward_kernel(
 #pragma unroll
         for (int c = 0; c < kGradSlots; ++c) any |= a[c] != 0.0f;
         if (any) {
-          float2* dst = (float2*) (slot_grads + (size_t) s_slot[threadIdx.x] * kGradSlots);
+          float2* dst = (float2*) (slot_grads + (size_t) s_slot[b & 1][threadIdx.x] * kGradSlots);
 #pragma unroll
           for (int c = 0; c < kGradSlots / 2; ++c) dst[c] = make_float2(a[2 * c], a[2 * c + 1]);
         }
       } else {
         // one global atomic per surfel and component for this tile
-        const int id = s_cold[threadIdx.x].id;
+        const int id = s_slot[b & 1][threadIdx.x];
 #pragma unroll
         for (int c = 0; c < 3; ++c)
           if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
@@ -328,8 +336,9 @@ blend_backward_kernel(
           if (a[16 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[16 + c]);
       }
     }
-    // No barrier needed here: a lane only touches its own record / its own rows of s_part between this flush and the
-    // barrier that follows the next batch's LDS store.
+    // No barrier needed here: between this flush and the barrier that follows the next batch's LDS store, wavefront 0
+    // touches its lanes' rows of s_part and this batch's copy of s_slot, wavefront 1 the staging arrays and the other
+    // copy of s_slot.
   }
 }
 
