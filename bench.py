@@ -494,6 +494,27 @@ def ssim_rate(dev, reps: int = 20):
             "fusedssim_workload": "1 x 3 x 800 x 800, train = true (times include output allocation)"}
 
 
+def topk_weights_ms(dev, scene, cam, reps: int = 20):
+    """Per-pixel top-k blend weights (k = 4) of the benchmark view: `gs_2d_topk_weights` on the binned scene."""
+    from fast_sp_gs_amd._C import get_C_function as f
+    W, H = cam.W, cam.H
+    m2, colors, tm, no, depths, radii, tt = f('gs_2d_preprocess_forward')(
+        W, H, 3, False, scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs, None, cam.Tw2v,
+        cam.Tv2c, cam.campos, None, None, None)
+    ranges, point_list = f('GS_prepare')(W, H, m2, depths, radii, tt, False)
+    run = lambda: f('gs_2d_topk_weights')(4, W, H, cam.near, cam.far, m2, no, tm, ranges, point_list)
+    run()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    return {"gs_2d_topk_weights_ms": ms, "gs_2d_topk_weights_pixels_per_s": W * H / (ms * 1e-3),
+            "gs_2d_topk_weights_workload": f"k = 4 on the 300k-surfel 800x800 view, R = {int(point_list.numel())}"}
+
+
 def fast_path_rate(dev, scene, cam, gi, steps: int = 20, warmup: int = 3):
     """The "fast" variant (adjugate intersection, fused corner-test binning) on the benchmark scene, forward + backward."""
     from fast_sp_gs_amd.renderer import fast_render_step
@@ -623,6 +644,7 @@ def main():
         extra.update(ssim_rate(dev))
         extra.update(simple_knn_ms(dev, scene))
         extra.update(reference_note_blend_ms(dev))
+        extra.update(topk_weights_ms(dev, scene, cam))
         extra.update(gs3d_path_rate(dev, scene, cam, gi))
         extra.update(density_control_ms(dev, scene))
         extra.update(large_scene_ms(dev))

@@ -252,17 +252,22 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_topk_kernel(int flags, int
         const bool sat     = hit && test_T < 0.0001f;
         done               = done || sat;
         if (hit && !sat) {
-          float w = h.alpha * T;
-          int idx = hot.id;
+          // sorted insertion: a slot's new weight is the offered one clamped between the slot and the slot above, its
+          // id follows the comparisons against the old list
+          const float w = h.alpha * T;
+          const int idx = hot.id;
+          bool ge[kK];
 #pragma unroll
-          for (int k = 0; k < kK; ++k) {
-            if (k < topk && w >= tw[k]) {
-              const float ow = tw[k];
-              const int oi   = ti[k];
-              tw[k] = w, ti[k] = idx;
-              w = ow, idx = oi;
+          for (int k = 0; k < kK; ++k) ge[k] = k < topk && w >= tw[k];
+#pragma unroll
+          for (int k = kK - 1; k >= 1; --k) {
+            if (k < topk) {
+              tw[k] = __builtin_amdgcn_fmed3f(tw[k - 1], w, tw[k]);
+              ti[k] = ge[k - 1] ? ti[k - 1] : (ge[k] ? idx : ti[k]);
             }
           }
+          tw[0] = fmaxf(tw[0], w);
+          ti[0] = ge[0] ? idx : ti[0];
           T = test_T;
         }
       }
