@@ -810,7 +810,7 @@ int fill_sort(int P, int W, int H, const float* means2D, const float* depths, co
                        (const float2*) means2D, depths, radii, rng, entries);
   hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
                      large_count, large_list);
-  hipLaunchKernelGGL(tile_sort_large_kernel, dim3(64), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,
+  hipLaunchKernelGGL(tile_sort_large_kernel, dim3(256), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,
                      large_count, large_list);
   return check_launch("gs_prepare_fill");
 }
