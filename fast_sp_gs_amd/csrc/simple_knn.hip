@@ -18,7 +18,7 @@
 namespace fsgs {
 namespace {
 
-constexpr int kBox = 256;  // points per box == queries per block
+constexpr int kBox = 64;  // points per box == queries per block (one wavefront)
 
 struct Bounds {
   float lo[3], hi[3];
@@ -145,15 +145,31 @@ __device__ __forceinline__ void update_best3(const float* ref, const float4 pt, 
     }
 }
 
-__global__ void __launch_bounds__(kBox) mean_dist_kernel(int P, int num_boxes, const float4* __restrict__ sorted,
-                                                         const Bounds* __restrict__ boxes, float* __restrict__ out) {
-  __shared__ float4 s_pts[kBox];
-  __shared__ int s_list[kBox];
-  __shared__ int s_count;
-  __shared__ float s_bound[kBox / kWave];
+// Bounds of every run of 64 boxes (one wavefront per group): the first level of the candidate search.
+__global__ void __launch_bounds__(kWave) group_boxes_kernel(int num_boxes, const Bounds* __restrict__ boxes,
+                                                            Bounds* __restrict__ groups) {
+  const int b = blockIdx.x * kWave + threadIdx.x;
+  const Bounds mine = boxes[b < num_boxes ? b : num_boxes - 1];
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    float lo = mine.lo[a], hi = mine.hi[a];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) lo = fminf(lo, __shfl_xor(lo, d, kWave)), hi = fmaxf(hi, __shfl_xor(hi, d, kWave));
+    if (threadIdx.x == 0) groups[blockIdx.x].lo[a] = lo, groups[blockIdx.x].hi[a] = hi;
+  }
+}
+
+// One wavefront = one box = 64 consecutive points of the curve, on its own: its pruning bound is the widest any of its
+// 64 queries still has, its bounding box is tested against 64 candidates per ballot (one per lane) on two levels
+// (groups of 64 boxes, then the boxes of a surviving group), and a surviving box's points are read with
+// wavefront-uniform addresses, i.e. as scalar loads feeding the vector ALU directly: no LDS, no barriers. Boxes of 64
+// points prune far better than longer runs of the curve, whose bounds overlap widely.
+__global__ void __launch_bounds__(kBox) mean_dist_kernel(int P, int num_boxes, int num_groups,
+    const float4* __restrict__ sorted, const Bounds* __restrict__ boxes, const Bounds* __restrict__ groups,
+    float* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
   const int idx  = blockIdx.x * kBox + threadIdx.x;
   const bool live = idx < P;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float p[3] = {0.0f, 0.0f, 0.0f};
   int id = 0;
   if (live) {
@@ -167,42 +183,48 @@ __global__ void __launch_bounds__(kBox) mean_dist_kernel(int P, int num_boxes, c
       if (i != idx) update_best3(p, sorted[i], best);
   const float reject = best[2];
   best[0] = best[1] = best[2] = FLT_MAX;
-  const Bounds mine = boxes[blockIdx.x];
+  // bounds of this wavefront's points
+  Bounds mine;
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    float lo = live ? p[a] : FLT_MAX, hi = live ? p[a] : -FLT_MAX;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) lo = fminf(lo, __shfl_xor(lo, d, kWave)), hi = fmaxf(hi, __shfl_xor(hi, d, kWave));
+    mine.lo[a] = lo, mine.hi[a] = hi;
+  }
+  if (__ballot(live) == 0ull) return;
 
-  for (int b0 = 0; b0 < num_boxes; b0 += kBox) {
-    // the widest bound any query of the block still has
+  // the widest bound any query of the wavefront still has
+  auto wave_bound = [&]() {
     float bound = live ? fminf(reject, best[2]) : 0.0f;
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) bound = fmaxf(bound, __shfl_xor(bound, d, kWave));
-    if (lane == 0) s_bound[wave] = bound;
-    if (threadIdx.x == 0) s_count = 0;
-    __syncthreads();
-    bound = s_bound[0];
-#pragma unroll
-    for (int w = 1; w < kBox / kWave; ++w) bound = fmaxf(bound, s_bound[w]);
-    // one lane per candidate box: keep those the block's bounding box can still reach
-    const int b = b0 + (int) threadIdx.x;
-    const bool keep = b < num_boxes && box_box_dist2(mine, boxes[b]) <= bound;
-    const unsigned long long m = __ballot(keep);
-    int base = 0;
-    if (lane == 0 && m) base = atomicAdd(&s_count, __popcll(m));
-    base = __shfl(base, 0, kWave);
-    if (keep) s_list[base + __popcll(m & ((1ull << lane) - 1ull))] = b;
-    __syncthreads();
-    const int n_list = s_count;
-    for (int k = 0; k < n_list; ++k) {
-      const int cb    = s_list[k];
-      const int first = cb * kBox, count = min(kBox, P - first);
-      __syncthreads();  // the previous box's points have been consumed
-      if ((int) threadIdx.x < count) s_pts[threadIdx.x] = sorted[first + threadIdx.x];
-      __syncthreads();
-      if (!live) continue;
-      const float dist = box_point_dist2(boxes[cb], p);
-      if (dist > reject || dist > best[2]) continue;  // knn.cu:149
-      for (int i = 0; i < count; ++i)
-        if (first + i != idx) update_best3(p, s_pts[i], best);
+    return bound;
+  };
+  // two levels, 64 candidates per ballot: groups of 64 boxes, then the boxes of a group that can still matter
+  for (int g0 = 0; g0 < num_groups; g0 += kWave) {
+    const int g = g0 + lane;
+    unsigned long long mg =
+        __ballot(g < num_groups && box_box_dist2(mine, groups[g < num_groups ? g : 0]) <= wave_bound());
+    while (mg) {
+      const int b0 = (g0 + __builtin_ctzll(mg)) * kWave;  // the same group for every lane
+      mg &= mg - 1;
+      const int b = b0 + lane;
+      unsigned long long m =
+          __ballot(b < num_boxes && box_box_dist2(mine, boxes[b < num_boxes ? b : 0]) <= wave_bound());
+      while (m) {
+        const int cb = b0 + __builtin_ctzll(m);  // the same box for every lane
+        m &= m - 1;
+        const float dist = box_point_dist2(boxes[cb], p);
+        const bool take  = live && !(dist > reject || dist > best[2]);  // knn.cu:149
+        if (__ballot(take) == 0ull) continue;
+        const int first = cb * kBox, count = min(kBox, P - first);
+        if (take) {
+          for (int i = 0; i < count; ++i)
+            if (first + i != idx) update_best3(p, sorted[first + i], best);
+        }
+      }
     }
-    __syncthreads();  // s_list / s_count are rewritten by the next step
   }
   if (live) {
 #pragma clang fp contract(off)
@@ -211,20 +233,22 @@ __global__ void __launch_bounds__(kBox) mean_dist_kernel(int P, int num_boxes, c
 }
 
 struct KnnLayout {
-  size_t sort, order, sorted, boxes, partial, bbox, bytes;
-  int num_boxes, bbox_blocks;
+  size_t sort, order, sorted, boxes, groups, partial, bbox, bytes;
+  int num_boxes, num_groups, bbox_blocks;
 };
 
 KnnLayout knn_layout(int P) {
   KnnLayout L;
   const int n     = P > 0 ? P : 1;
   L.num_boxes   = div_up(n, kBox);
+  L.num_groups  = div_up(L.num_boxes, kWave);
   L.bbox_blocks = std::min(div_up(n, 256), 512);
   size_t o = 0;
   L.sort = o, o = align_up(o + sort_workspace_bytes(n), 256);
   L.order = o, o = align_up(o + (size_t) n * 4, 256);
   L.sorted = o, o = align_up(o + (size_t) n * 16, 256);
   L.boxes = o, o = align_up(o + (size_t) L.num_boxes * sizeof(Bounds), 256);
+  L.groups = o, o = align_up(o + (size_t) L.num_groups * sizeof(Bounds), 256);
   L.partial = o, o = align_up(o + (size_t) L.bbox_blocks * 6 * 4, 256);
   L.bbox = o, o = align_up(o + 6 * 4, 256);
   L.bytes = o;
@@ -262,6 +286,9 @@ FSGS_API int fsgs_simple_knn(int P, const float* points, float* mean_dist2, void
   const uint64_t* sorted_keys = nullptr;
   radix_sort_pairs(P, bits, sort_ws, order, &sorted_keys, s);
   hipLaunchKernelGGL(gather_boxes_kernel, dim3(L.num_boxes), dim3(kBox), 0, s, P, points, order, sorted, boxes);
-  hipLaunchKernelGGL(mean_dist_kernel, dim3(L.num_boxes), dim3(kBox), 0, s, P, L.num_boxes, sorted, boxes, mean_dist2);
+  Bounds* groups = (Bounds*) (ws + L.groups);
+  hipLaunchKernelGGL(group_boxes_kernel, dim3(L.num_groups), dim3(kWave), 0, s, L.num_boxes, boxes, groups);
+  hipLaunchKernelGGL(mean_dist_kernel, dim3(L.num_boxes), dim3(kBox), 0, s, P, L.num_boxes, L.num_groups, sorted, boxes,
+                     groups, mean_dist2);
   return check_launch("simple_knn");
 }
