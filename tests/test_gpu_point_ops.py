@@ -181,6 +181,13 @@ def test_lbs_and_knn_backward(device, oracle_mod, c1):
     _lbs_backward_case(O, device, pts[:500], tiny_ctrl, 0.1 * torch.randn(3, 3, generator=g),
                        0.2 * torch.randn(3, 4, generator=g), 0.1 * torch.randn(3, 2, generator=g), 5, 0.05, False,
                        seed=24)
+    # K = 4 with a padded slot (3 control points), through the binned variant
+    _lbs_backward_case(O, device, pts[:700], tiny_ctrl, 0.1 * torch.randn(3, 3, generator=g),
+                       0.2 * torch.randn(3, 4, generator=g), 0.1 * torch.randn(3, 2, generator=g), 4, 0.05, True,
+                       seed=26)
+    # more points than one pass of the launch covers: every block bins several chunks into its table
+    many = torch.rand(280_001, 3, generator=g) * 2 - 1
+    _lbs_backward_case(O, device, many, ctrl, c1['sp_t'], c1['sp_r'], c1['sp_s'], 4, 0.01, False, seed=27)
     # a control set whose table exceeds LDS takes the atomic path
     big_ctrl = torch.rand(2500, 3, generator=g) * 2 - 1
     _lbs_backward_case(O, device, pts[:20000], big_ctrl, 0.1 * torch.randn(2500, 3, generator=g),
