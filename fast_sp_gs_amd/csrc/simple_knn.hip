@@ -194,7 +194,8 @@ __global__ void __launch_bounds__(kBox) mean_dist_kernel(int P, int num_boxes, i
   }
   if (__ballot(live) == 0ull) return;
 
-  // the widest bound any query of the wavefront still has
+  // the widest bound any query of the wavefront still has; its lane exchanges need all 64 lanes, so it is evaluated on
+  // its own line, never on the right of a short-circuit inside a ballot
   auto wave_bound = [&]() {
     float bound = live ? fminf(reject, best[2]) : 0.0f;
 #pragma unroll
@@ -204,14 +205,16 @@ __global__ void __launch_bounds__(kBox) mean_dist_kernel(int P, int num_boxes, i
   // two levels, 64 candidates per ballot: groups of 64 boxes, then the boxes of a group that can still matter
   for (int g0 = 0; g0 < num_groups; g0 += kWave) {
     const int g = g0 + lane;
+    const float group_bound = wave_bound();
     unsigned long long mg =
-        __ballot(g < num_groups && box_box_dist2(mine, groups[g < num_groups ? g : 0]) <= wave_bound());
+        __ballot(g < num_groups && box_box_dist2(mine, groups[g < num_groups ? g : 0]) <= group_bound);
     while (mg) {
       const int b0 = (g0 + __builtin_ctzll(mg)) * kWave;  // the same group for every lane
       mg &= mg - 1;
       const int b = b0 + lane;
+      const float box_bound = wave_bound();
       unsigned long long m =
-          __ballot(b < num_boxes && box_box_dist2(mine, boxes[b < num_boxes ? b : 0]) <= wave_bound());
+          __ballot(b < num_boxes && box_box_dist2(mine, boxes[b < num_boxes ? b : 0]) <= box_bound);
       while (m) {
         const int cb = b0 + __builtin_ctzll(m);  // the same box for every lane
         m &= m - 1;

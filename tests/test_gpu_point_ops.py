@@ -507,11 +507,12 @@ def test_deform_mlp_mfma(device, oracle_mod):
 
 
 @pytest.mark.parametrize("P,kind", [(20000, "ball"), (5000, "clusters"), (777, "plane"), (3, "ball"), (2, "ball"),
-                                    (1, "ball"), (4097, "same")])
+                                    (1, "ball"), (4097, "same"), (5000, "halo"), (7000, "halo"), (20001, "halo")])
 def test_simple_knn(P, kind, device, oracle_mod):
     """Mean squared 3-NN distance: bit-exact against the all-pairs oracle (the search is exact and both sides add the
     squares in the same order with contraction off) on clouds that stress the pruning: clusters far apart, a flat
-    cloud (degenerate bounding box), duplicates, fewer points than neighbours."""
+    cloud (degenerate bounding box), duplicates, fewer points than neighbours, and a tight cluster inside a sparse halo
+    (a wavefront whose queries have very different pruning bounds: the widest of all 64 has to be used)."""
     from fast_sp_gs_amd._C import get_C_function
     O = oracle_mod
     g = torch.Generator().manual_seed(60 + P)
@@ -522,6 +523,9 @@ def test_simple_knn(P, kind, device, oracle_mod):
         pts = centres[torch.randint(0, 7, (P,), generator=g)] + 0.01 * torch.randn(P, 3, generator=g)
     elif kind == "plane":
         pts = torch.cat([torch.rand(P, 2, generator=g), torch.full((P, 1), 0.25)], 1)
+    elif kind == "halo":
+        dense = 0.002 * torch.randn(P - P // 8, 3, generator=g)
+        pts = torch.cat([dense, torch.rand(P // 8, 3, generator=g) * 4 - 2])[torch.randperm(P, generator=g)]
     else:
         pts = torch.ones(P, 3) * 0.5  # every point identical: all distances 0, the curve order is all ties
     pts = pts.contiguous()
@@ -548,3 +552,24 @@ def test_simple_knn_full_size(device):
     d2 = ((pts[sample][:, None, :] - pts[None, :, :]) ** 2).sum(-1)  # [256, P]
     best = d2.topk(4, dim=1, largest=False).values[:, 1:]            # drop the point itself (distance 0)
     assert float((best.mean(1) - got[sample]).abs().max()) <= 1e-6 * float(best.max())
+
+
+def test_simple_knn_mixed_density_large(device):
+    """More points than one round of 64 x 64 boxes covers (so the group level runs a partial last round), most of them in
+    a tight cluster, the rest a sparse halo: the halo points' results against brute force."""
+    from fast_sp_gs_amd._C import get_C_function
+    g = torch.Generator().manual_seed(72)
+    P, n_halo = 300_001, 3_000
+    pts = torch.cat([0.002 * torch.randn(P - n_halo, 3, generator=g), torch.rand(n_halo, 3, generator=g) * 4 - 2])
+    perm = torch.randperm(P, generator=g)
+    pts = pts[perm].contiguous().to(device)
+    halo = torch.nonzero(perm >= P - n_halo).flatten()[:1024].to(device)
+    sample = torch.cat([halo, torch.randint(0, P, (256,), generator=g).to(device)])
+    print(f"[simple_knn] mixed density P={P}", flush=True)
+    got = get_C_function('simple_knn')(pts)
+    torch.cuda.synchronize()
+    for part in sample.split(256):
+        d2 = ((pts[part][:, None, :] - pts[None, :, :]) ** 2).sum(-1)
+        best = d2.topk(4, dim=1, largest=False).values[:, 1:]
+        want = best.mean(1)
+        assert float(((want - got[part]).abs() / want.clamp_min(1e-30)).max()) <= 1e-5
