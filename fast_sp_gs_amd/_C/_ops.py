@@ -73,6 +73,20 @@ def _lib():
     return L.load()
 
 
+def _cuda_f32(what, **tensors):
+    """CHECK_CUDA only (common.hpp:25-27): device fp32 tensors of any stride; returns them made contiguous, which is what
+    the reference's hosts that call `.contiguous()` themselves do (structural_similarity.cu:341-357)."""
+    out = []
+    for k, t in tensors.items():
+        if not isinstance(t, torch.Tensor):
+            raise RuntimeError(f"{what}: {k} must be a Tensor")
+        if not t.is_cuda:
+            raise RuntimeError(f"{what}: {k} must be a CUDA tensor")
+        L.require_dtype(what, k, t, torch.float32)
+        out.append(t.contiguous())
+    return out
+
+
 def _f32(what, **tensors):
     L.require_cuda(what, **tensors)
     for k, t in tensors.items():
@@ -1157,10 +1171,9 @@ def fusedssim(C1: float, C2: float, img1: Tensor, img2: Tensor, train: bool):
     """structural_similarity.cu:340-363 -> (ssim_map, dm_dmu1, dm_dsigma1_sq, dm_dsigma12), all [B,CH,H,W]; the three
     partial-derivative maps are empty tensors when `train` is false."""
     what = 'fusedssim'
-    _f32(what, img1=img1, img2=img2)
+    img1, img2 = _cuda_f32(what, img1=img1, img2=img2)
     if img1.ndim != 4 or img1.shape != img2.shape:
         raise RuntimeError(f'{what}: img1 and img2 must be [B,CH,H,W] tensors of the same shape')
-    img1, img2 = img1.contiguous(), img2.contiguous()
     B, CH, H, W = img1.shape
     ssim_map = torch.empty_like(img1)
     if train:
@@ -1180,9 +1193,9 @@ def fusedssim_backward(C1: float, C2: float, img1: Tensor, img2: Tensor, dL_dmap
                        dm_dsigma1_sq: Tensor, dm_dsigma12: Tensor) -> Tensor:
     """structural_similarity.cu:365-380 -> dL_dimg1[B,CH,H,W]."""
     what = 'fusedssim_backward'
-    _f32(what, img1=img1, img2=img2, dL_dmap=dL_dmap, dm_dmu1=dm_dmu1, dm_dsigma1_sq=dm_dsigma1_sq,
-         dm_dsigma12=dm_dsigma12)
-    img1, img2, dL_dmap = img1.contiguous(), img2.contiguous(), dL_dmap.contiguous()
+    img1, img2, dL_dmap, dm_dmu1, dm_dsigma1_sq, dm_dsigma12 = _cuda_f32(
+        what, img1=img1, img2=img2, dL_dmap=dL_dmap, dm_dmu1=dm_dmu1, dm_dsigma1_sq=dm_dsigma1_sq,
+        dm_dsigma12=dm_dsigma12)
     B, CH, H, W = img1.shape
     for name, t in (('img2', img2), ('dL_dmap', dL_dmap), ('dm_dmu1', dm_dmu1), ('dm_dsigma1_sq', dm_dsigma1_sq),
                     ('dm_dsigma12', dm_dsigma12)):
@@ -1190,8 +1203,8 @@ def fusedssim_backward(C1: float, C2: float, img1: Tensor, img2: Tensor, dL_dmap
     grad = torch.empty_like(img1)
     with _timed(what):
         rc = _lib().fsgs_fusedssim_backward(B, CH, H, W, L.ptr(img1), L.ptr(img2), L.ptr(dL_dmap),
-                                            L.ptr(dm_dmu1.contiguous()), L.ptr(dm_dsigma1_sq.contiguous()),
-                                            L.ptr(dm_dsigma12.contiguous()), L.ptr(grad), L.current_stream())
+                                            L.ptr(dm_dmu1), L.ptr(dm_dsigma1_sq), L.ptr(dm_dsigma12), L.ptr(grad),
+                                            L.current_stream())
     L.check(rc, what)
     return grad
 

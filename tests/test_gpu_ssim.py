@@ -62,6 +62,28 @@ def test_ssim_autograd_and_loss(device):
     assert abs(fd - an) < 2e-2 * max(abs(an), 1e-6) + 1e-6
 
 
+def test_ssim_loss_channel_last_and_sliced_inputs(device):
+    """The reference's loss call hands SSIM_Loss [H,W,3] renders and `targets['images'][..., :3]` of an RGBA batch
+    (gaussian_splatting.py:295-297, 317-321): permuted / sliced views, not contiguous. The operator accepts any strides
+    (structural_similarity.cu:341-357 checks the device only), forward and backward."""
+    from fast_sp_gs_amd.ssim import SSIM_Loss
+    g = torch.Generator().manual_seed(4)
+    hwc = torch.rand(2, 40, 56, 3, generator=g).to(device).requires_grad_(True)
+    rgba = torch.rand(2, 40, 56, 4, generator=g).to(device)
+    target = rgba[..., :3]
+    assert not target.is_contiguous()
+    loss = SSIM_Loss()(hwc, target)
+    loss.backward()
+    chw = hwc.detach().permute(0, 3, 1, 2).contiguous().requires_grad_(True)
+    ref = SSIM_Loss()(chw, target.permute(0, 3, 1, 2).contiguous())
+    ref.backward()
+    assert float(loss) == float(ref)
+    assert hwc.grad.shape == hwc.shape and torch.equal(hwc.grad.permute(0, 3, 1, 2), chw.grad)
+    # one [H,W,3] image
+    one = SSIM_Loss()(hwc.detach()[0], target[0])
+    assert abs(float(one) - float(SSIM_Loss()(chw.detach()[:1], target[:1].permute(0, 3, 1, 2).contiguous()))) < 1e-7
+
+
 @pytest.mark.parametrize("shape,lam", [((1, 3, 800, 800), 0.2), ((2, 3, 45, 70), 0.35), ((1, 1, 7, 5), 1.0),
                                        ((3, 2, 32, 64), 0.0)])
 def test_fused_image_loss(shape, lam, device, oracle_mod):
