@@ -10,6 +10,8 @@
 // (4 wavefronts) for a 32x32 output tile, every lane owning one column of 4 output rows.
 #include "common.hpp"
 
+#include <atomic>
+
 namespace fsgs {
 namespace {
 
@@ -257,6 +259,45 @@ FSGS_API int fsgs_image_loss_forward(int B, int CH, int H, int W, double C1, dou
   hipLaunchKernelGGL(image_loss_finish_kernel, dim3(1), dim3(256), 0, s, (int) (grid.x * grid.y * grid.z), partials,
                      (float) (1.0 / n), (float) lambda_dssim, loss_out);
   return check_launch("image_loss");
+}
+
+// ---- the same forward for callers that cannot allocate ----------------------------------------------------------------
+// The per-block partial sums live in a file-scope device array instead of a caller workspace. Every GPU the library
+// runs on holds its own copy of the array at its own address until the process ends; the address is looked up once per
+// device and only that pointer is handed to kernels (the array's name is a host-side stand-in, not a device address).
+constexpr int kStaticLossMaxBlocks = 65536;  // 32x32-pixel blocks, e.g. one 8192x8192 image or 40 images of 1280x1280
+static __device__ __align__(256) float scratch[2 * kStaticLossMaxBlocks];  // 512 KiB
+constexpr int kMaxDevices = 64;
+static std::atomic<float*> g_scratch_ptr[kMaxDevices];
+
+static int static_scratch(float** out) {
+  int dev = -1;
+  FSGS_HIP(hipGetDevice(&dev));
+  FSGS_REQUIRE(dev >= 0 && dev < kMaxDevices, "image_loss_static: device ordinal %d out of range", dev);
+  float* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    FSGS_HIP(hipGetSymbolAddress((void**) &p, HIP_SYMBOL(scratch)));
+    FSGS_REQUIRE(p != nullptr, "image_loss_static: no device address for the scratch array");
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return kOk;
+}
+
+FSGS_API int fsgs_image_loss_static_max_blocks(void) { return kStaticLossMaxBlocks; }
+
+FSGS_API int fsgs_image_loss_forward_static(int B, int CH, int H, int W, double C1, double C2, double lambda_dssim,
+    const float* img, const float* target, float* loss_out, float* dm_dmu1, float* dm_dsigma1_sq,
+    float* dm_dsigma12, void* stream) {
+  FSGS_REQUIRE(B > 0 && CH > 0 && H > 0 && W > 0 && B <= 65535, "image_loss_static: bad sizes");
+  const int64_t blocks = (int64_t) B * div_up(W, kSsimTile) * div_up(H, kSsimTile);
+  if (blocks > kStaticLossMaxBlocks)
+    return fail(kUnsupported, "image_loss_static: %lld blocks of 32x32 pixels exceed the built-in scratch of %d blocks; "
+                "use fsgs_image_loss_forward with a workspace", (long long) blocks, kStaticLossMaxBlocks);
+  float* partials = nullptr;
+  if (int rc = static_scratch(&partials)) return rc;
+  return fsgs_image_loss_forward(B, CH, H, W, C1, C2, lambda_dssim, img, target, loss_out, dm_dmu1, dm_dsigma1_sq,
+                                 dm_dsigma12, partials, (size_t) 2 * kStaticLossMaxBlocks * sizeof(float), stream);
 }
 
 FSGS_API int fsgs_image_loss_backward(int B, int CH, int H, int W, double lambda_dssim, const float* img,

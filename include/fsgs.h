@@ -403,6 +403,18 @@ int fsgs_image_loss_backward(int B, int CH, int H, int W, double lambda_dssim, c
     const float* grad_loss, const float* dm_dmu1, const float* dm_dsigma1_sq, const float* dm_dsigma12, float* dL_dimg,
     void* stream);
 
+/* fsgs_image_loss_forward for callers that cannot allocate device memory or carry a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Same inputs,
+ * outputs and results as fsgs_image_loss_forward; the per-block partial sums go into a device array built into the
+ * library (512 KiB per GPU, held until the process ends) instead of a workspace, so the call allocates nothing. Limit:
+ * B * ceil(W / 32) * ceil(H / 32) <= fsgs_image_loss_static_max_blocks() (65536: one 8192 x 8192 image); larger inputs
+ * are rejected with an error. All calls on one GPU share that array: calls that overlap on one GPU (two streams, two
+ * host threads) race; calls on one stream are ordered. Nothing in the array has to be cleared between calls. */
+int fsgs_image_loss_static_max_blocks(void);
+int fsgs_image_loss_forward_static(int B, int CH, int H, int W, double C1, double C2, double lambda_dssim,
+    const float* img, const float* target, float* loss_out, float* dm_dmu1, float* dm_dsigma1_sq, float* dm_dsigma12,
+    void* stream);
+
 /* Deformation MLP forward (bf16 MFMA, fp32 accumulate) -- fast_2d_gs/network.py:1757-1776 (SC_GS_DeformNetwork.forward,
  * fp32 there): n_layers x (Linear(256) + ReLU), input re-concatenated in front after layer `skip`, then n_out <= 32
  * linear outputs (the three heads stacked). in[B,Din] fp32 (already frequency-encoded), Din <= 96, width must be 256.

@@ -1,0 +1,51 @@
+"""The allocation-free variant of the fused image loss (fsgs_image_loss_forward_static) against the workspace variant,
+called through the C ABI: two calls in a row, the second on a smaller input, results bit-identical; inputs beyond the
+built-in scratch are rejected."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _call(lib, L, static, img, target, lam, train, ws=None):
+    B, CH, H, W = img.shape
+    loss = torch.full((3,), float('nan'), device=img.device)
+    d = [torch.full_like(img, float('nan')) for _ in range(3)] if train else [None] * 3
+    args = (B, CH, H, W, 0.01 ** 2, 0.03 ** 2, lam, L.ptr(img), L.ptr(target), L.ptr(loss), L.ptr(d[0]), L.ptr(d[1]),
+            L.ptr(d[2]))
+    if static:
+        rc = lib.fsgs_image_loss_forward_static(*args, L.current_stream())
+    else:
+        rc = lib.fsgs_image_loss_forward(*args, L.ptr(ws), ws.numel(), L.current_stream())
+    L.check(rc, 'image_loss')
+    return loss, d
+
+
+def test_image_loss_static_matches_workspace_variant(device):
+    from fast_sp_gs_amd import lib as L
+    lib = L.load()
+    g = torch.Generator().manual_seed(11)
+    for shape, lam, train in [((2, 3, 200, 333), 0.2, True), ((1, 3, 45, 70), 0.35, True), ((1, 1, 7, 5), 1.0, False)]:
+        print(f"[no-alloc image loss] {shape}", flush=True)
+        img, target = torch.rand(*shape, generator=g).to(device), torch.rand(*shape, generator=g).to(device)
+        ws = torch.empty(lib.fsgs_image_loss_workspace_bytes(shape[0], shape[2], shape[3]), dtype=torch.uint8,
+                         device=device)
+        want, dw = _call(lib, L, False, img, target, lam, train, ws)
+        got, dg = _call(lib, L, True, img, target, lam, train)
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(want).all()) and torch.equal(got, want)
+        for a, b in zip(dg, dw):
+            assert (a is None and b is None) or torch.equal(a, b)
+
+
+def test_image_loss_static_rejects_oversize(device):
+    from fast_sp_gs_amd import lib as L
+    lib = L.load()
+    cap = lib.fsgs_image_loss_static_max_blocks()
+    assert cap == 65536
+    tiny = torch.zeros(1, 1, 4, 4, device=device)
+    loss = torch.zeros(3, device=device)
+    # sizes only: (cap + 1) blocks of 32x32 pixels in one row of blocks; the pointers are never followed
+    rc = lib.fsgs_image_loss_forward_static(1, 1, 32, 32 * (cap + 1), 1e-4, 9e-4, 0.2, L.ptr(tiny), L.ptr(tiny),
+                                            L.ptr(loss), None, None, None, L.current_stream())
+    assert rc != 0 and b'exceed' in lib.fsgs_last_error()
