@@ -143,7 +143,7 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
     g = torch.Generator().manual_seed(2)
     ctrl = (torch.rand(512, 3, generator=g) * 2 - 1).to(dev).requires_grad_(True)
     target = torch.rand(3, cam.H, cam.W, generator=g).to(dev)
-    net = DeformNetwork().to(dev)
+    net = DeformNetwork(local_frame=True).to(dev)  # the fourth head gives each control point its rotation (6-DoF warp)
     # a tiny rate keeps the random-target synthetic scene from drifting (Adam's steps are |lr| whatever the gradient, and
     # the scale residuals are added after the activation, network.py:643), so every timed step sees the same workload
     net_opt = torch.optim.Adam(list(net.parameters()) + [ctrl], lr=1e-7, fused=True)
@@ -154,10 +154,10 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
 
     def step(i):
         t = torch.full((1,), (i % 17) / 17.0, device=dev)
-        c_xyz, c_rot, c_scale, _ = net(ctrl.detach(), t)
-        d_xyz, d_rot, d_scale, _, _ = superpoint_deform(params[0].detach(), ctrl, c_xyz.contiguous(),
-                                                        c_rot.contiguous(), c_scale[:, :2].contiguous(), K=4,
-                                                        temperature=0.01)
+        c_xyz, c_rot, c_scale, c_local = net(ctrl.detach(), t)
+        d_xyz, d_rot, d_scale, _, _ = superpoint_deform(params[0].detach(), ctrl, c_xyz, c_rot, c_scale[:, :2],
+                                                        sp_rot=c_local, K=4, temperature=0.01, warp_method='LBS',
+                                                        LBS_method='dist')
         xyz, scales, rot = deform_apply(params[0], d_xyz, params[1], d_scale, params[2], d_rot)
         out = GS_2D_render(xyz, scales, rot, params[3], (cam.W, cam.H),
                            cam.Tw2v, cam.Tv2c, campos=cam.campos, near=cam.near, far=cam.far, sh_degree=3,

@@ -952,16 +952,49 @@ def knn_topk(x: Tensor, y: Tensor, K: int) -> Tuple[Tensor, Tensor]:
     return dist2, index
 
 
-def lbs_blend(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_s: Optional[Tensor], dist2: Tensor,
-              index: Tensor, temperature: float = 1.0, centred: bool = False):
-    """LBS warp of fast_2d_gs/network.py:517,545-573 -> (d_xyz[N,3], d_rot[N,4], d_scale[N,S]|None, weights[N,K])."""
+_LBS_WARP = {None: 0, 'none': 0, 'LBS': 1, 'LBS_c': 2}
+_LBS_WEIGHT = {'dist': 0, 'kernel': 1, 'weighted_kernel': 1, 'W': 2, 'logits': 2, 'given': 3}
+
+
+def _lbs_modes(what, warp_method, weight_method, sp_rot, sp_log_radius, sp_weight_logit):
+    if weight_method not in _LBS_WEIGHT:
+        raise RuntimeError(f'{what}: unknown weight method {weight_method!r} (one of {sorted(_LBS_WEIGHT)})')
+    if sp_rot is None:
+        warp = 0  # warp() without a local rotation blends the translations only, whatever the method (network.py:563-564)
+    else:
+        if warp_method not in ('LBS', 'LBS_c'):
+            raise RuntimeError(f'{what}: warp method must be LBS or LBS_c when sp_rot is given, got {warp_method!r}')
+        warp = _LBS_WARP[warp_method]
+    weight = _LBS_WEIGHT[weight_method]
+    if weight == 1 and sp_log_radius is None:
+        raise RuntimeError(f'{what}: the kernel weights need sp_log_radius')
+    if weight_method == 'weighted_kernel' and sp_weight_logit is None:
+        raise RuntimeError(f'{what}: weighted_kernel needs sp_weight_logit')
+    return warp, weight
+
+
+def lbs_blend(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_s: Optional[Tensor], pair_in: Tensor,
+              index: Tensor, temperature: float = 1.0, warp_method: Optional[str] = None,
+              sp_rot: Optional[Tensor] = None, weight_method: str = 'dist', sp_log_radius: Optional[Tensor] = None,
+              sp_weight_logit: Optional[Tensor] = None):
+    """Neighbour weights and warp of fast_2d_gs/network.py:507-517, 545-573 ->
+    (d_xyz[N,3], d_rot[N,4], d_scale[N,S]|None, weights[N,K]). `pair_in`[N,K]: squared distances ('dist', 'kernel',
+    'weighted_kernel'), gathered logits ('W') or finished weights ('given'). Without `sp_rot` the translations alone are
+    blended; with it `warp_method` is 'LBS' or 'LBS_c'."""
     what = 'lbs_blend'
-    _f32(what, points=points, sp_points=sp_points, sp_t=sp_t, sp_r=sp_r, sp_s=sp_s, dist2=dist2)
+    _f32(what, points=points, sp_points=sp_points, sp_t=sp_t, sp_r=sp_r, sp_s=sp_s, pair_in=pair_in, sp_rot=sp_rot,
+         sp_log_radius=sp_log_radius, sp_weight_logit=sp_weight_logit)
     L.require_cuda(what, index=index)
     L.require_dtype(what, 'index', index, torch.int64)
-    N, K = dist2.shape
+    warp, weight = _lbs_modes(what, warp_method, weight_method, sp_rot, sp_log_radius, sp_weight_logit)
+    N, K = pair_in.shape
     M = sp_points.shape[0]
     S = 0 if sp_s is None else sp_s.shape[1]
+    L.require_shape(what, 'index', index, N, K)
+    L.require_shape(what, 'sp_t', sp_t, M, 3)
+    L.require_shape(what, 'sp_r', sp_r, M, 4)
+    if sp_rot is not None:
+        L.require_shape(what, 'sp_rot', sp_rot, M, 4)
     opt = dict(dtype=torch.float32, device=points.device)
     d_xyz, d_rot = torch.empty((N, 3), **opt), torch.empty((N, 4), **opt)
     d_scale = torch.empty((N, S), **opt) if S else None
@@ -969,46 +1002,59 @@ def lbs_blend(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_
     lib = _lib()
     ws = _workspace(lib.fsgs_lbs_blend_workspace_bytes(M), points.device)
     with _timed('lbs_blend'):
-        rc = lib.fsgs_lbs_blend(N, M, K, int(bool(centred)), float(temperature), L.ptr(points), L.ptr(sp_points),
-                                L.ptr(sp_t), L.ptr(sp_r), L.ptr(sp_s), S, L.ptr(dist2), L.ptr(index), L.ptr(weights),
-                                L.ptr(d_xyz), L.ptr(d_rot), L.ptr(d_scale), L.ptr(ws), ws.numel(), L.current_stream())
+        rc = lib.fsgs_lbs_blend(N, M, K, warp, weight, float(temperature), L.ptr(points), L.ptr(sp_points),
+                                L.ptr(sp_t), L.ptr(sp_rot), L.ptr(sp_r), L.ptr(sp_s), S, L.ptr(pair_in), L.ptr(index),
+                                L.ptr(sp_log_radius) if weight == 1 else None,
+                                L.ptr(sp_weight_logit) if weight == 1 else None, L.ptr(weights), L.ptr(d_xyz),
+                                L.ptr(d_rot), L.ptr(d_scale), L.ptr(ws), ws.numel(), L.current_stream())
     L.check(rc, what)
     return d_xyz, d_rot, d_scale, weights
 
 
 def lbs_blend_backward(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_s: Optional[Tensor],
-                       dist2: Tensor, index: Tensor, grad_xyz: Tensor, grad_rot: Tensor, grad_scale: Optional[Tensor],
-                       temperature: float = 1.0, centred: bool = False, need_points: bool = True):
-    """Gradients of `lbs_blend` (what autograd gives for fast_2d_gs/network.py:517,545-573) ->
-    (g_points[N,3]|None, g_dist2[N,K], g_sp_points[M,3], g_sp_t[M,3], g_sp_r[M,4], g_sp_s[M,S]|None)."""
+                       pair_in: Tensor, index: Tensor, grad_xyz: Tensor, grad_rot: Tensor,
+                       grad_scale: Optional[Tensor], temperature: float = 1.0, warp_method: Optional[str] = None,
+                       sp_rot: Optional[Tensor] = None, weight_method: str = 'dist',
+                       sp_log_radius: Optional[Tensor] = None, sp_weight_logit: Optional[Tensor] = None,
+                       need_points: bool = True):
+    """Gradients of `lbs_blend` (what autograd gives for fast_2d_gs/network.py:507-517, 545-573) -> dict with g_points
+    [N,3]|None, g_pair[N,K] (gradient of `pair_in`), g_sp_points[M,3], g_sp_t[M,3], g_sp_rot[M,4]|None, g_sp_r[M,4],
+    g_sp_s[M,S]|None, g_log_radius[M]|None, g_weight_logit[M]|None."""
     what = 'lbs_blend_backward'
-    _f32(what, points=points, sp_points=sp_points, sp_t=sp_t, sp_r=sp_r, sp_s=sp_s, dist2=dist2, grad_xyz=grad_xyz,
-         grad_rot=grad_rot, grad_scale=grad_scale)
+    _f32(what, points=points, sp_points=sp_points, sp_t=sp_t, sp_r=sp_r, sp_s=sp_s, pair_in=pair_in, grad_xyz=grad_xyz,
+         grad_rot=grad_rot, grad_scale=grad_scale, sp_rot=sp_rot, sp_log_radius=sp_log_radius,
+         sp_weight_logit=sp_weight_logit)
     L.require_cuda(what, index=index)
     L.require_dtype(what, 'index', index, torch.int64)
-    N, K = dist2.shape
+    warp, weight = _lbs_modes(what, warp_method, weight_method, sp_rot, sp_log_radius, sp_weight_logit)
+    N, K = pair_in.shape
     M = sp_points.shape[0]
     S = 0 if sp_s is None else sp_s.shape[1]
     if S and grad_scale is None:
         raise RuntimeError(f'{what}: grad_scale is required when sp_s is given')
     if tuple(grad_xyz.shape) != (N, 3) or tuple(grad_rot.shape) != (N, 4) or tuple(index.shape) != (N, K) or \
             (S and tuple(grad_scale.shape) != (N, S)):
-        raise RuntimeError(f'{what}: gradient / index shapes do not match dist2 {tuple(dist2.shape)}')
+        raise RuntimeError(f'{what}: gradient / index shapes do not match pair_in {tuple(pair_in.shape)}')
     opt = dict(dtype=torch.float32, device=points.device)
     g_points = torch.empty((N, 3), **opt) if need_points else None
-    g_dist2 = torch.empty((N, K), **opt)
+    g_pair = torch.empty((N, K), **opt)
     g_sp_points, g_sp_t, g_sp_r = torch.empty((M, 3), **opt), torch.empty((M, 3), **opt), torch.empty((M, 4), **opt)
+    g_sp_rot = torch.empty((M, 4), **opt) if warp else None
     g_sp_s = torch.empty((M, S), **opt) if S else None
+    g_rad = torch.empty((M,), **opt) if weight == 1 else None
+    g_wl = torch.empty((M,), **opt) if weight == 1 and sp_weight_logit is not None else None
     lib = _lib()
     ws = _workspace(lib.fsgs_lbs_blend_backward_workspace_bytes(N, M, S), points.device)
     with _timed('lbs_blend_backward'):
         rc = lib.fsgs_lbs_blend_backward(
-            N, M, K, int(bool(centred)), float(temperature), L.ptr(points), L.ptr(sp_points), L.ptr(sp_t), L.ptr(sp_r),
-            L.ptr(sp_s), S, L.ptr(dist2), L.ptr(index), L.ptr(grad_xyz), L.ptr(grad_rot), L.ptr(grad_scale),
-            L.ptr(g_points), L.ptr(g_dist2), L.ptr(g_sp_points), L.ptr(g_sp_t), L.ptr(g_sp_r), L.ptr(g_sp_s),
-            L.ptr(ws), ws.numel(), L.current_stream())
+            N, M, K, warp, weight, float(temperature), L.ptr(points), L.ptr(sp_points), L.ptr(sp_t), L.ptr(sp_rot),
+            L.ptr(sp_r), L.ptr(sp_s), S, L.ptr(pair_in), L.ptr(index), L.ptr(sp_log_radius) if weight == 1 else None,
+            L.ptr(sp_weight_logit) if weight == 1 else None, L.ptr(grad_xyz), L.ptr(grad_rot), L.ptr(grad_scale),
+            L.ptr(g_points), L.ptr(g_pair), L.ptr(g_sp_points), L.ptr(g_sp_t), L.ptr(g_sp_rot), L.ptr(g_sp_r),
+            L.ptr(g_sp_s), L.ptr(g_rad), L.ptr(g_wl), L.ptr(ws), ws.numel(), L.current_stream())
     L.check(rc, what)
-    return g_points, g_dist2, g_sp_points, g_sp_t, g_sp_r, g_sp_s
+    return dict(g_points=g_points, g_pair=g_pair, g_sp_points=g_sp_points, g_sp_t=g_sp_t, g_sp_rot=g_sp_rot,
+                g_sp_r=g_sp_r, g_sp_s=g_sp_s, g_log_radius=g_rad, g_weight_logit=g_wl)
 
 
 def knn_topk_backward(x: Tensor, y: Tensor, index: Tensor, grad_dist2: Tensor, need_x: bool = True):
@@ -1139,9 +1185,11 @@ def mlp_pack_transposed(weights: List[Tensor]) -> Tensor:
 
 
 def mlp_backward(inputs: Tensor, packed_t: Tensor, head_weights: Tensor, saved: Tensor, grad_out: Tensor,
-                 n_layers: int, skip: int) -> Tuple[Tensor, Tensor]:
+                 n_layers: int, skip: int, return_dz: bool = False):
     """Weight and bias gradients of `mlp_forward` (autograd through nn.Linear / relu in the reference,
-    network.py:1757-1776) -> (g_w flat: layers' [256,K_l] back to back then heads [n_out,256]; g_b[n_layers*256+n_out])."""
+    network.py:1757-1776) -> (g_w flat: layers' [256,K_l] back to back then heads [n_out,256]; g_b[n_layers*256+n_out]).
+    With `return_dz` also dZ[n_layers,B,256] (bf16): the gradient of every layer's pre-activation, from which a caller
+    forms the gradient of the network's input (dZ_0 W_0 + dZ_{skip+1} W_{skip+1}[:, :Din])."""
     what = 'mlp_backward'
     _f32(what, inputs=inputs, head_weights=head_weights, grad_out=grad_out)
     L.require_cuda(what, packed_t=packed_t, saved=saved)
@@ -1163,6 +1211,8 @@ def mlp_backward(inputs: Tensor, packed_t: Tensor, head_weights: Tensor, saved: 
                                    L.ptr(head_weights), L.ptr(saved), L.ptr(grad_out), L.ptr(g_w), L.ptr(g_b),
                                    L.ptr(ws), ws.numel(), L.current_stream())
     L.check(rc, what)
+    if return_dz:
+        return g_w, g_b, ws[:n_layers * B * 256 * 2].view(torch.bfloat16).view(n_layers, B, 256)
     return g_w, g_b
 
 

@@ -15,6 +15,7 @@
 #include <algorithm>
 
 #include "common.hpp"
+#include "lbs.hpp"
 #include "sh.hpp"
 
 namespace fsgs {
@@ -318,67 +319,44 @@ __global__ void __launch_bounds__(256) knn_topk_kernel(int N, int M, int D, int 
   }
 }
 
-// ---- LBS skinning -------------------------------------------------------------------------------------------------------
-// Per control point (one lane each): unit quaternion of r + (0,0,0,1), its rotation matrix, and the translation
-// (re-centred about the control point when `centred`). 12 floats per control point.
-__global__ void __launch_bounds__(256) lbs_prepare_kernel(int M, int centred, const float* __restrict__ sp_points,
-    const float* __restrict__ sp_t, const float* __restrict__ sp_r, float* __restrict__ xf /*[M,12]*/) {
-  const int j = blockIdx.x * blockDim.x + threadIdx.x;
-  if (j >= M) return;
-  float q[4] = {sp_r[4 * j], sp_r[4 * j + 1], sp_r[4 * j + 2], sp_r[4 * j + 3] + 1.0f};
-  const float nq = 1.0f / fmaxf(sqrtf(q[0] * q[0] + q[1] * q[1] + q[2] * q[2] + q[3] * q[3]), 1e-12f);
-  const float x = q[0] * nq, y = q[1] * nq, z = q[2] * nq, w = q[3] * nq;
-  float R[9];
-  R[0] = 1 - 2 * (y * y + z * z), R[1] = 2 * (x * y - z * w), R[2] = 2 * (y * w + x * z);
-  R[3] = 2 * (x * y + z * w), R[4] = 1 - 2 * (x * x + z * z), R[5] = 2 * (y * z - x * w);
-  R[6] = 2 * (x * z - y * w), R[7] = 2 * (x * w + y * z), R[8] = 1 - 2 * (x * x + y * y);
-  float t[3] = {sp_t[3 * j], sp_t[3 * j + 1], sp_t[3 * j + 2]};
-  if (centred) {
-    const float* c = sp_points + 3 * j;
-#pragma unroll
-    for (int a = 0; a < 3; ++a) t[a] = t[a] + c[a] - (R[a * 3] * c[0] + R[a * 3 + 1] * c[1] + R[a * 3 + 2] * c[2]);
-  }
-#pragma unroll
-  for (int k = 0; k < 9; ++k) xf[12 * j + k] = R[k];
-#pragma unroll
-  for (int k = 0; k < 3; ++k) xf[12 * j + 9 + k] = t[k];
-}
-
-__global__ void __launch_bounds__(256) lbs_blend_kernel(int N, int M, int K, int S, float temperature,
-    const float* __restrict__ points, const float* __restrict__ xf, const float* __restrict__ sp_r,
-    const float* __restrict__ sp_s, const float* __restrict__ dist2, const int64_t* __restrict__ index,
+// ---- LBS skinning (per-control-point table and weights: lbs.hpp) -----------------------------------------------------
+template <int kMaxK>
+__global__ void __launch_bounds__(256) lbs_blend_kernel(int N, int M, int K, int S, int warp_mode, int weight_mode,
+    float temperature, const float* __restrict__ points, const float* __restrict__ xf, const float* __restrict__ sp_r,
+    const float* __restrict__ sp_s, const float* __restrict__ pair_in, const int64_t* __restrict__ index,
     float* __restrict__ weights_out, float* __restrict__ d_xyz, float* __restrict__ d_rot,
     float* __restrict__ d_scale) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= N) return;
-  const float* d2   = dist2 + (size_t) n * K;
   const int64_t* id = index + (size_t) n * K;
-  // slots without a neighbour (index -1 when K > M) take no part in the softmax
-  float mx = -__builtin_inff();
-  for (int k = 0; k < K; ++k)
-    if (id[k] >= 0 && id[k] < M) mx = fmaxf(mx, -d2[k] / temperature);
-  float den = 0.0f;
-  for (int k = 0; k < K; ++k)
-    if (id[k] >= 0 && id[k] < M) den += expf(-d2[k] / temperature - mx);
+  float u[kMaxK], inv_den;
+  lbs_weights<kMaxK>(weight_mode, K, M, 1.0f / temperature, pair_in + (size_t) n * K, id, xf, u, inv_den);
   const float p[3] = {points[3 * (size_t) n], points[3 * (size_t) n + 1], points[3 * (size_t) n + 2]};
   float acc[3] = {0, 0, 0}, ar[4] = {0, 0, 0, 0}, as[4] = {0, 0, 0, 0};
-  for (int k = 0; k < K; ++k) {
+#pragma unroll
+  for (int k = 0; k < kMaxK; ++k) {
+    if (k >= K) break;
     const int64_t j = id[k];
     if (j < 0 || j >= M) {
       if (weights_out) weights_out[(size_t) n * K + k] = 0.0f;
       continue;
     }
-    const float w  = expf(-d2[k] / temperature - mx) / den;
-    const float* X = xf + 12 * j;
+    const float w  = u[k] * inv_den;
+    const float* X = xf + (size_t) kXf * j;
+    if (warp_mode != 0) {
 #pragma unroll
-    for (int a = 0; a < 3; ++a) acc[a] += w * (X[a * 3] * p[0] + X[a * 3 + 1] * p[1] + X[a * 3 + 2] * p[2] + X[9 + a]);
+      for (int a = 0; a < 3; ++a) acc[a] += w * (X[a * 3] * p[0] + X[a * 3 + 1] * p[1] + X[a * 3 + 2] * p[2] + X[9 + a]);
+    } else {
+#pragma unroll
+      for (int a = 0; a < 3; ++a) acc[a] += w * X[9 + a];
+    }
 #pragma unroll
     for (int a = 0; a < 4; ++a) ar[a] += w * sp_r[4 * j + a];
     for (int a = 0; a < S; ++a) as[a] += w * sp_s[(size_t) S * j + a];
     if (weights_out) weights_out[(size_t) n * K + k] = w;
   }
 #pragma unroll
-  for (int a = 0; a < 3; ++a) d_xyz[3 * (size_t) n + a] = acc[a] - p[a];
+  for (int a = 0; a < 3; ++a) d_xyz[3 * (size_t) n + a] = warp_mode != 0 ? acc[a] - p[a] : acc[a];
 #pragma unroll
   for (int a = 0; a < 4; ++a) d_rot[4 * (size_t) n + a] = ar[a];
   for (int a = 0; a < S; ++a) d_scale[(size_t) S * n + a] = as[a];
@@ -694,24 +672,32 @@ FSGS_API int fsgs_knn_topk(int N, int M, int D, int K, const float* x, const flo
   return check_launch("knn_topk");
 }
 
-FSGS_API size_t fsgs_lbs_blend_workspace_bytes(int M) { return align_up((size_t) (M > 0 ? M : 1) * 12 * 4, 256); }
+FSGS_API size_t fsgs_lbs_blend_workspace_bytes(int M) { return align_up((size_t) (M > 0 ? M : 1) * kXf * 4, 256); }
 
-FSGS_API int fsgs_lbs_blend(int N, int M, int K, int centred, double temperature, const float* points,
-    const float* sp_points, const float* sp_t, const float* sp_r, const float* sp_s, int S, const float* dist2,
-    const int64_t* index, float* weights_out, float* d_xyz, float* d_rot, float* d_scale, void* workspace,
+FSGS_API int fsgs_lbs_blend(int N, int M, int K, int warp_mode, int weight_mode, double temperature,
+    const float* points, const float* sp_points, const float* sp_t, const float* sp_rot, const float* sp_r,
+    const float* sp_s, int S, const float* pair_in, const int64_t* index, const float* sp_log_radius,
+    const float* sp_weight_logit, float* weights_out, float* d_xyz, float* d_rot, float* d_scale, void* workspace,
     size_t workspace_bytes, void* stream) {
-  FSGS_REQUIRE(N >= 0 && M > 0 && K > 0 && S >= 0 && S <= 4 && points && sp_points && sp_t && sp_r && dist2 && index &&
-                   d_xyz && d_rot && (S == 0 || (sp_s && d_scale)) && workspace,
-               "lbs_blend: bad arguments");
+  FSGS_REQUIRE(N >= 0 && M > 0 && K > 0 && K <= 16 && S >= 0 && S <= 4, "lbs_blend: bad sizes (K <= 16, S <= 4)");
+  FSGS_REQUIRE(warp_mode >= 0 && warp_mode <= 2 && weight_mode >= 0 && weight_mode <= 3, "lbs_blend: unknown mode");
+  FSGS_REQUIRE(points && sp_points && sp_t && sp_r && pair_in && index && d_xyz && d_rot &&
+                   (S == 0 || (sp_s && d_scale)) && workspace, "lbs_blend: null pointer");
+  FSGS_REQUIRE((warp_mode == 0) == (sp_rot == nullptr),
+               "lbs_blend: sp_rot goes with warp modes 1 and 2 and is absent in mode 0 (translation only)");
+  FSGS_REQUIRE(weight_mode != 1 || sp_log_radius, "lbs_blend: the kernel weights need sp_log_radius");
+  FSGS_REQUIRE(weight_mode != 0 || temperature > 0, "lbs_blend: temperature must be positive");
   if (workspace_bytes < fsgs_lbs_blend_workspace_bytes(M))
     return fail(kWorkspaceSmall, "lbs_blend: workspace %zu < %zu bytes", workspace_bytes,
                 fsgs_lbs_blend_workspace_bytes(M));
   if (N == 0) return kOk;
   hipStream_t s = (hipStream_t) stream;
   float* xf     = (float*) workspace;
-  hipLaunchKernelGGL(lbs_prepare_kernel, dim3(div_up(M, 256)), dim3(256), 0, s, M, centred, sp_points, sp_t, sp_r, xf);
-  hipLaunchKernelGGL(lbs_blend_kernel, dim3(div_up(N, 256)), dim3(256), 0, s, N, M, K, S, (float) temperature, points, xf,
-                     sp_r, sp_s, dist2, index, weights_out, d_xyz, d_rot, d_scale);
+  hipLaunchKernelGGL(lbs_prepare_kernel, dim3(div_up(M, 256)), dim3(256), 0, s, M, warp_mode, sp_points, sp_t, sp_rot,
+                     weight_mode == 1 ? sp_log_radius : nullptr, weight_mode == 1 ? sp_weight_logit : nullptr, xf);
+  auto kernel = K <= 4 ? lbs_blend_kernel<4> : lbs_blend_kernel<16>;
+  hipLaunchKernelGGL(kernel, dim3(div_up(N, 256)), dim3(256), 0, s, N, M, K, S, warp_mode, weight_mode,
+                     (float) temperature, points, xf, sp_r, sp_s, pair_in, index, weights_out, d_xyz, d_rot, d_scale);
   return check_launch("lbs_blend");
 }
 

@@ -239,27 +239,46 @@ int fsgs_cdist_top_backward(int B, int N, int M, int D, const float* p1, const f
 int fsgs_knn_topk(int N, int M, int D, int K, const float* x, const float* y, float* dist2, int64_t* index,
                   void* stream);
 
-/* LBS blend with weights softmax(-dist2 / temperature) -- fast_2d_gs/network.py:517 and :545-573 (warp with
- * apply_rotate == 'add'): q_k = normalize(sp_r_k + (0,0,0,1)); centred: t_k += c_k - R(q_k) c_k;
- * d_xyz = sum_k w_k (R(q_k) p + t_k) - p; d_rot = sum_k w_k sp_r_k; d_scale = sum_k w_k sp_s_k (S <= 4 columns). */
+/* The superpoint warp of fast_2d_gs/network.py:498-573 in one call: neighbour weights (calc_LBS_weight, :507-517) and
+ * the blend (warp, :545-573) over the K neighbours index[N,K] (int64, from fsgs_knn_topk; slots outside [0, M) get
+ * weight 0 and take no part in the normalisation).
+ * weight_mode selects what pair_in[N,K] is and how weights are formed:
+ *   0  LBS_method 'dist' (:517): pair_in = squared distances, w = softmax(-d2 / temperature);
+ *   1  'kernel' / 'weighted_kernel' (:507-513): pair_in = squared distances, u = exp(-d2 / (2 r_j^2)) [* sigmoid(omega_j)]
+ *      + 1e-7, w = u / sum u, with r_j = exp(sp_log_radius[j]) (the reference's raw _sp_radius, :255-256) and omega_j =
+ *      sp_weight_logit[j] (raw _sp_weight, :259-260; NULL for 'kernel');
+ *   2  'W' (:514-515): pair_in = the caller's gather sp_W[n, index[n, k]], w = softmax(pair_in);
+ *   3  pair_in = finished weights, used as they are (warp() called on weights the caller computed).
+ * warp_mode follows the branches of warp():
+ *   0  no local rotation (sp_rot == NULL; the default configuration, :563-564): d_xyz = sum_k w_k sp_t[j_k];
+ *   1  'LBS' with sp_rot[M,4] (:545-556): q_j = normalize(sp_rot_j + (0,0,0,1)), d_xyz = sum_k w_k (R(q_j) p + sp_t_j) - p;
+ *   2  'LBS_c': as 1 with sp_t_j replaced by sp_t_j + c_j - R(q_j) c_j, c = sp_points (:548-549).
+ * Always: d_rot[N,4] = sum_k w_k sp_r[j_k] (apply_rotate 'add', :565-566), d_scale[N,S] = sum_k w_k sp_s[j_k] (S <= 4; S = 0
+ * and NULL pointers when the net predicts no scale residual). weights_out[N,K] is optional. K <= 16. */
 size_t fsgs_lbs_blend_workspace_bytes(int M);
-int fsgs_lbs_blend(int N, int M, int K, int centred, double temperature, const float* points,
-    const float* sp_points, const float* sp_t, const float* sp_r, const float* sp_s, int S, const float* dist2,
-    const int64_t* index, float* weights_out, float* d_xyz, float* d_rot, float* d_scale, void* workspace,
-    size_t workspace_bytes, void* stream);
+int fsgs_lbs_blend(int N, int M, int K, int warp_mode, int weight_mode, double temperature, const float* points,
+    const float* sp_points, const float* sp_t, const float* sp_rot, const float* sp_r, const float* sp_s, int S,
+    const float* pair_in, const int64_t* index, const float* sp_log_radius, const float* sp_weight_logit,
+    float* weights_out, float* d_xyz, float* d_rot, float* d_scale, void* workspace, size_t workspace_bytes,
+    void* stream);
 
 /* Backward of fsgs_lbs_blend. The reference has no kernel for it: torch autograd differentiates
- * fast_2d_gs/network.py:517 and :545-573 op by op. Inputs as in the forward plus g_xyz[N,3], g_rot[N,4], g_scale[N,S].
- * Every output element is written: g_points[N,3] (optional), g_dist2[N,K], g_sp_points[M,3] (optional; zero unless
- * centred), g_sp_t[M,3], g_sp_r[M,4], g_sp_s[M,S]. Per-control-point sums use LDS float atomics inside a block and a
- * fixed order across blocks while M * (16 + S) <= 36864, device-scope float atomics beyond; either way the last bits
- * of the per-control-point outputs can differ between runs. */
+ * fast_2d_gs/network.py:507-517 and :545-573 op by op. Inputs as in the forward plus g_xyz[N,3], g_rot[N,4],
+ * g_scale[N,S]. Every output element is written: g_points[N,3] (optional; zeros in warp mode 0), g_pair[N,K] (the
+ * gradient of pair_in: of the squared distances in weight modes 0 and 1, of the logits in mode 2, of the weights in
+ * mode 3), g_sp_points[M,3] (optional; the pivot term of warp mode 2, zeros otherwise -- the dependence of the distances
+ * on sp_points goes through g_pair and fsgs_knn_topk_backward), g_sp_t[M,3], g_sp_rot[M,4] (warp modes 1, 2), g_sp_r[M,4],
+ * g_sp_s[M,S], and in weight mode 1 g_log_radius[M] and (optional, with sp_weight_logit) g_weight_logit[M].
+ * Per-control-point sums are taken without float atomics, in a fixed order, when M <= 1024, K <= 4 and M * columns <=
+ * 11264 (columns = 7 + S, + 9 with a rotation, + 2 in weight mode 1); larger cases use LDS float atomics inside a block
+ * (up to 36864 table cells) or device-scope float atomics, whose last bits can differ between runs. */
 size_t fsgs_lbs_blend_backward_workspace_bytes(int N, int M, int S);
-int fsgs_lbs_blend_backward(int N, int M, int K, int centred, double temperature, const float* points,
-    const float* sp_points, const float* sp_t, const float* sp_r, const float* sp_s, int S, const float* dist2,
-    const int64_t* index, const float* g_xyz, const float* g_rot, const float* g_scale, float* g_points,
-    float* g_dist2, float* g_sp_points, float* g_sp_t, float* g_sp_r, float* g_sp_s, void* workspace,
-    size_t workspace_bytes, void* stream);
+int fsgs_lbs_blend_backward(int N, int M, int K, int warp_mode, int weight_mode, double temperature,
+    const float* points, const float* sp_points, const float* sp_t, const float* sp_rot, const float* sp_r,
+    const float* sp_s, int S, const float* pair_in, const int64_t* index, const float* sp_log_radius,
+    const float* sp_weight_logit, const float* g_xyz, const float* g_rot, const float* g_scale, float* g_points,
+    float* g_pair, float* g_sp_points, float* g_sp_t, float* g_sp_rot, float* g_sp_r, float* g_sp_s,
+    float* g_log_radius, float* g_weight_logit, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Backward of fsgs_knn_topk's squared distances (what autograd through pytorch3d.ops.knn_points gives at
  * fast_2d_gs/network.py:504): g_x[N,D] (optional) = sum_k 2 g_dist2[n,k] (x_n - y_index), g_y[M,D] = minus the same

@@ -242,146 +242,7 @@ static inline void quat_R(const T* q, T* R) {
   R[6] = 2 * (x * z - y * w), R[7] = 2 * (x * w + y * z), R[8] = 1 - 2 * (x * x + y * y);
 }
 
-// LBS blend, network.py:517 (weights = softmax(-d2 / temperature)) and :545-573 (warp):
-// q_k = normalize(r_k + (0,0,0,1)); centred: t_k <- t_k + c_k + R(q_k)(-c_k);
-// d_xyz = sum_k w_k (R(q_k) p + t_k) - p ; d_rot = sum_k w_k r_k ; d_scale = sum_k w_k s_k.
-template <typename T>
-static void lbs_blend(int N, int M, int K, int centred, T temperature, const T* points, const T* sp_points,
-                      const T* sp_t, const T* sp_r, const T* sp_s, int S, const T* dist2, const int64_t* index,
-                      T* weights_out, T* d_xyz, T* d_rot, T* d_scale) {
-#pragma omp parallel for schedule(static)
-  for (int n = 0; n < N; ++n) {
-    std::vector<T> w(K, T(0));
-    // slots without a neighbour (index -1 when K > M) take no part in the softmax
-    auto valid = [&](int k) { const int64_t j = index[(size_t) n * K + k]; return j >= 0 && j < M; };
-    T mx = -std::numeric_limits<T>::infinity();
-    for (int k = 0; k < K; ++k)
-      if (valid(k)) mx = std::max(mx, -dist2[(size_t) n * K + k] / temperature);
-    T den = 0;
-    for (int k = 0; k < K; ++k)
-      if (valid(k)) w[k] = std::exp(-dist2[(size_t) n * K + k] / temperature - mx), den += w[k];
-    for (int k = 0; k < K; ++k)
-      if (valid(k)) w[k] = w[k] / den;
-    const T* p = points + 3 * (size_t) n;
-    T acc[3] = {0, 0, 0}, ar[4] = {0, 0, 0, 0};
-    std::vector<T> as(S, T(0));
-    for (int k = 0; k < K; ++k) {
-      const int64_t j = index[(size_t) n * K + k];
-      if (!valid(k)) {
-        if (weights_out) weights_out[(size_t) n * K + k] = 0;
-        continue;
-      }
-      T q[4] = {sp_r[4 * j], sp_r[4 * j + 1], sp_r[4 * j + 2], sp_r[4 * j + 3] + T(1)};
-      const T nq = T(1) / std::max(std::sqrt(q[0] * q[0] + q[1] * q[1] + q[2] * q[2] + q[3] * q[3]), T(1e-12));
-      for (int a = 0; a < 4; ++a) q[a] *= nq;
-      T R[9];
-      quat_R(q, R);
-      T t[3] = {sp_t[3 * j], sp_t[3 * j + 1], sp_t[3 * j + 2]};
-      if (centred) {
-        const T* c = sp_points + 3 * j;
-        for (int a = 0; a < 3; ++a) t[a] = t[a] + c[a] - (R[a * 3] * c[0] + R[a * 3 + 1] * c[1] + R[a * 3 + 2] * c[2]);
-      }
-      for (int a = 0; a < 3; ++a) acc[a] += w[k] * (R[a * 3] * p[0] + R[a * 3 + 1] * p[1] + R[a * 3 + 2] * p[2] + t[a]);
-      for (int a = 0; a < 4; ++a) ar[a] += w[k] * sp_r[4 * j + a];
-      for (int a = 0; a < S; ++a) as[a] += w[k] * sp_s[(size_t) S * j + a];
-      if (weights_out) weights_out[(size_t) n * K + k] = w[k];
-    }
-    for (int a = 0; a < 3; ++a) d_xyz[3 * (size_t) n + a] = acc[a] - p[a];
-    for (int a = 0; a < 4; ++a) d_rot[4 * (size_t) n + a] = ar[a];
-    for (int a = 0; a < S; ++a) d_scale[(size_t) S * n + a] = as[a];
-  }
-}
-
-// Backward of lbs_blend (there is no hand-written backward in the reference: network.py:517,545-573 is differentiated by
-// torch autograd / lietorch). Given g_xyz[N,3], g_rot[N,4], g_scale[N,S] it returns the gradients of every
-// differentiable input: g_points[N,3], g_dist2[N,K], and per control point g_sp_points[M,3] (non-zero only when
-// centred), g_sp_t[M,3], g_sp_r[M,4], g_sp_s[M,S]. Sums over Gaussians run in index order.
-template <typename T>
-static void lbs_blend_backward(int N, int M, int K, int centred, T temperature, const T* points, const T* sp_points,
-                               const T* sp_t, const T* sp_r, const T* sp_s, int S, const T* dist2,
-                               const int64_t* index, const T* g_xyz, const T* g_rot, const T* g_scale, T* g_points,
-                               T* g_dist2, T* g_sp_points, T* g_sp_t, T* g_sp_r, T* g_sp_s) {
-  std::vector<T> GR((size_t) M * 9, T(0)), Gt((size_t) M * 3, T(0)), Rm((size_t) M * 9), te((size_t) M * 3),
-      qh((size_t) M * 4), inv_norm(M);
-  std::vector<char> degenerate(M);
-  for (int j = 0; j < M; ++j) {
-    T q[4] = {sp_r[4 * j], sp_r[4 * j + 1], sp_r[4 * j + 2], sp_r[4 * j + 3] + T(1)};
-    const T nrm = std::sqrt(q[0] * q[0] + q[1] * q[1] + q[2] * q[2] + q[3] * q[3]);
-    degenerate[j] = nrm <= T(1e-12);
-    inv_norm[j]   = T(1) / std::max(nrm, T(1e-12));
-    for (int a = 0; a < 4; ++a) qh[4 * j + a] = q[a] * inv_norm[j];
-    quat_R(&qh[4 * j], &Rm[9 * (size_t) j]);
-    for (int a = 0; a < 3; ++a) {
-      te[3 * j + a] = sp_t[3 * j + a];
-      if (centred) {
-        const T* c = sp_points + 3 * j;
-        const T* R = &Rm[9 * (size_t) j];
-        te[3 * j + a] = te[3 * j + a] + c[a] - (R[a * 3] * c[0] + R[a * 3 + 1] * c[1] + R[a * 3 + 2] * c[2]);
-      }
-    }
-    for (int a = 0; a < 4; ++a) g_sp_r[4 * j + a] = 0;
-    for (int a = 0; a < S; ++a) g_sp_s[(size_t) S * j + a] = 0;
-  }
-  std::vector<T> w(K), gw(K);
-  for (int n = 0; n < N; ++n) {
-    auto valid = [&](int k) { const int64_t j = index[(size_t) n * K + k]; return j >= 0 && j < M; };
-    T mx = -std::numeric_limits<T>::infinity();
-    for (int k = 0; k < K; ++k)
-      if (valid(k)) mx = std::max(mx, -dist2[(size_t) n * K + k] / temperature);
-    T den = 0;
-    for (int k = 0; k < K; ++k) w[k] = 0, gw[k] = 0;
-    for (int k = 0; k < K; ++k)
-      if (valid(k)) w[k] = std::exp(-dist2[(size_t) n * K + k] / temperature - mx), den += w[k];
-    for (int k = 0; k < K; ++k)
-      if (valid(k)) w[k] = w[k] / den;
-    const T* p  = points + 3 * (size_t) n;
-    const T* g  = g_xyz + 3 * (size_t) n;
-    const T* gr = g_rot + 4 * (size_t) n;
-    const T* gs = S ? g_scale + (size_t) S * n : nullptr;
-    T gp[3] = {-g[0], -g[1], -g[2]}, dot = 0;
-    for (int k = 0; k < K; ++k) {
-      const int64_t j = index[(size_t) n * K + k];
-      if (!valid(k)) continue;
-      const T* R = &Rm[9 * (size_t) j];
-      T v = 0;
-      for (int a = 0; a < 3; ++a) {
-        v += g[a] * (R[a * 3] * p[0] + R[a * 3 + 1] * p[1] + R[a * 3 + 2] * p[2] + te[3 * j + a]);
-        for (int b = 0; b < 3; ++b) GR[9 * (size_t) j + a * 3 + b] += w[k] * g[a] * p[b];
-        Gt[3 * j + a] += w[k] * g[a];
-        gp[a] += w[k] * (R[a] * g[0] + R[3 + a] * g[1] + R[6 + a] * g[2]);
-      }
-      for (int a = 0; a < 4; ++a) v += gr[a] * sp_r[4 * j + a], g_sp_r[4 * j + a] += w[k] * gr[a];
-      for (int a = 0; a < S; ++a) v += gs[a] * sp_s[(size_t) S * j + a], g_sp_s[(size_t) S * j + a] += w[k] * gs[a];
-      gw[k] = v, dot += w[k] * v;
-    }
-    for (int k = 0; k < K; ++k) g_dist2[(size_t) n * K + k] = -(w[k] * (gw[k] - dot)) / temperature;
-    for (int a = 0; a < 3; ++a) g_points[3 * (size_t) n + a] = gp[a];
-  }
-  for (int j = 0; j < M; ++j) {
-    T* G = &GR[9 * (size_t) j];
-    const T* R = &Rm[9 * (size_t) j];
-    const T* t = &Gt[3 * j];
-    for (int a = 0; a < 3; ++a) {
-      g_sp_t[3 * j + a]      = t[a];
-      g_sp_points[3 * j + a] = 0;
-    }
-    if (centred) {
-      const T* c = sp_points + 3 * j;
-      for (int a = 0; a < 3; ++a) {
-        g_sp_points[3 * j + a] = t[a] - (R[a] * t[0] + R[3 + a] * t[1] + R[6 + a] * t[2]);
-        for (int b = 0; b < 3; ++b) G[a * 3 + b] -= t[a] * c[b];
-      }
-    }
-    const T x = qh[4 * j], y = qh[4 * j + 1], z = qh[4 * j + 2], ww = qh[4 * j + 3];
-    T dq[4];
-    dq[0] = 2 * (-2 * x * (G[4] + G[8]) + y * (G[1] + G[3]) + z * (G[2] + G[6]) + ww * (G[7] - G[5]));
-    dq[1] = 2 * (x * (G[1] + G[3]) - 2 * y * (G[0] + G[8]) + z * (G[5] + G[7]) + ww * (G[2] - G[6]));
-    dq[2] = 2 * (x * (G[2] + G[6]) + y * (G[5] + G[7]) - 2 * z * (G[0] + G[4]) + ww * (G[3] - G[1]));
-    dq[3] = 2 * (x * (G[7] - G[5]) + y * (G[2] - G[6]) + z * (G[3] - G[1]));
-    const T along = degenerate[j] ? T(0) : qh[4 * j] * dq[0] + qh[4 * j + 1] * dq[1] + qh[4 * j + 2] * dq[2] + ww * dq[3];
-    for (int a = 0; a < 4; ++a) g_sp_r[4 * j + a] += inv_norm[j] * (dq[a] - qh[4 * j + a] * along);
-  }
-}
+// (The LBS weights and warp are restated in oracle/lbs.py: the reference's own code for them is torch.)
 
 // Backward of knn_topk's squared distances: g_x[n] = sum_k 2 g_k (x_n - y_idx), g_y[j] = -sum over its users.
 template <typename T>
@@ -740,24 +601,9 @@ using namespace oracle;
     knn_topk<T>(N, M, D, K, x, y, dist2, index);                                                                     \
     return 0;                                                                                                        \
   }                                                                                                                  \
-  ORACLE_API int oracle_lbs_blend_backward_##SUF(int N, int M, int K, int centred, double temperature,               \
-      const T* points, const T* sp_points, const T* sp_t, const T* sp_r, const T* sp_s, int S, const T* dist2,       \
-      const int64_t* index, const T* g_xyz, const T* g_rot, const T* g_scale, T* g_points, T* g_dist2,               \
-      T* g_sp_points, T* g_sp_t, T* g_sp_r, T* g_sp_s) {                                                             \
-    lbs_blend_backward<T>(N, M, K, centred, (T) temperature, points, sp_points, sp_t, sp_r, sp_s, S, dist2, index,   \
-                          g_xyz, g_rot, g_scale, g_points, g_dist2, g_sp_points, g_sp_t, g_sp_r, g_sp_s);            \
-    return 0;                                                                                                        \
-  }                                                                                                                  \
   ORACLE_API int oracle_knn_topk_backward_##SUF(int N, int M, int D, int K, const T* x, const T* y,                  \
       const int64_t* index, const T* g_dist2, T* g_x, T* g_y) {                                                      \
     knn_topk_backward<T>(N, M, D, K, x, y, index, g_dist2, g_x, g_y);                                                \
-    return 0;                                                                                                        \
-  }                                                                                                                  \
-  ORACLE_API int oracle_lbs_blend_##SUF(int N, int M, int K, int centred, double temperature, const T* points,       \
-      const T* sp_points, const T* sp_t, const T* sp_r, const T* sp_s, int S, const T* dist2, const int64_t* index,  \
-      T* weights_out, T* d_xyz, T* d_rot, T* d_scale) {                                                              \
-    lbs_blend<T>(N, M, K, centred, (T) temperature, points, sp_points, sp_t, sp_r, sp_s, S, dist2, index,            \
-                 weights_out, d_xyz, d_rot, d_scale);                                                                \
     return 0;                                                                                                        \
   }
 

@@ -51,13 +51,6 @@ int oracle_cdist_top_backward_f32(int B, int N, int M, int D, const float* p1, c
 int oracle_adam_masked_update_f32(int64_t N, int64_t M, const uint8_t* mask, double lr, double b1, double b2,
     double eps, float* param, const float* grad, float* m, float* v);
 int oracle_knn_topk_f32(int N, int M, int D, int K, const float* x, const float* y, float* dist2, int64_t* index);
-int oracle_lbs_blend_f32(int N, int M, int K, int centred, double temperature, const float* points,
-    const float* sp_points, const float* sp_t, const float* sp_r, const float* sp_s, int S, const float* dist2,
-    const int64_t* index, float* weights_out, float* d_xyz, float* d_rot, float* d_scale);
-int oracle_lbs_blend_backward_f32(int N, int M, int K, int centred, double temperature, const float* points,
-    const float* sp_points, const float* sp_t, const float* sp_r, const float* sp_s, int S, const float* dist2,
-    const int64_t* index, const float* g_xyz, const float* g_rot, const float* g_scale, float* g_points,
-    float* g_dist2, float* g_sp_points, float* g_sp_t, float* g_sp_r, float* g_sp_s);
 int oracle_knn_topk_backward_f32(int N, int M, int D, int K, const float* x, const float* y, const int64_t* index,
     const float* g_dist2, float* g_x, float* g_y);
 int oracle_gs_2d_epilogue_forward_f32(int W, int H, double ratio, const float* Tw2v, const float* Tv2c,

@@ -120,91 +120,158 @@ def test_knn_and_lbs(device, oracle_mod, c1):
     O.call("knn_topk_f32", 3000, 100, 5, 4, npy(x5), npy(y5), rd, ri)
     assert np.array_equal(npy(idx), ri) and np.array_equal(npy(d2), rd)
 
-    K = 4
-    d2, idx = get_C_function('knn_topk')(pts.to(device), ctrl.to(device), K)
-    for centred in (False, True):
-        dx, dr, ds, w = get_C_function('lbs_blend')(pts.to(device), ctrl.to(device), c1['sp_t'].to(device),
-                                                    c1['sp_r'].to(device), c1['sp_s'].to(device), d2, idx, 0.01, centred)
-        rw, rx, rr, rs = (np.zeros((N, K), np.float32), np.zeros((N, 3), np.float32), np.zeros((N, 4), np.float32),
-                          np.zeros((N, 2), np.float32))
-        O.call("lbs_blend_f32", N, M, K, int(centred), 0.01, npy(pts), npy(ctrl), npy(c1['sp_t']), npy(c1['sp_r']),
-               npy(c1['sp_s']), 2, npy(d2), npy(idx), rw, rx, rr, rs)
-        assert abs_err(npy(w), rw) < 1e-5 and abs_err(npy(dx), rx) < 1e-5
-        assert abs_err(npy(dr), rr) < 1e-5 and abs_err(npy(ds), rs) < 1e-6
+    # 11 columns, K = 3: positions + 8 hyper features, the default configuration's search (exps/d_nerf.yaml:21-23)
+    x11, y11 = torch.randn(5000, 11, generator=g), torch.randn(512, 11, generator=g)
+    d2, idx = get_C_function('knn_topk')(x11.to(device), y11.to(device), 3)
+    rd, ri = np.zeros((5000, 3), np.float32), np.zeros((5000, 3), np.int64)
+    O.call("knn_topk_f32", 5000, 512, 11, 3, npy(x11), npy(y11), rd, ri)
+    assert np.array_equal(npy(idx), ri) and np.array_equal(npy(d2), rd)
 
 
-def _lbs_backward_case(O, device, pts, ctrl, sp_t, sp_r, sp_s, K, tau, centred, seed):
+LBS_CASES = [  # (warp method with a local rotation | None without one, weight method)
+    (None, 'weighted_kernel'),   # the reference's default configuration: translations only, kernel weights
+    (None, 'dist'), ('LBS', 'dist'), ('LBS_c', 'dist'), ('LBS_c', 'weighted_kernel'), ('LBS', 'kernel'),
+    ('LBS_c', 'W'), (None, 'given'), ('LBS', 'given'),
+]
+
+
+def _lbs_inputs(pts, ctrl, sp_t, sp_r, sp_s, K, warp_method, weight_method, seed, device):
+    """Device inputs of one LBS case + the same values in float64 for the oracle."""
     from fast_sp_gs_amd._C import get_C_function
+    g = torch.Generator().manual_seed(seed)
+    N, M = pts.shape[0], ctrl.shape[0]
+    d = lambda t: None if t is None else t.to(device).contiguous()
+    d2, idx = get_C_function('knn_topk')(d(pts), d(ctrl), K)
+    sp_rot = 0.3 * torch.randn(M, 4, generator=g) if warp_method is not None else None
+    # radii around the typical neighbour distance so that the kernel weights are neither uniform nor one-hot
+    typical = float(d2[d2 >= 0].median().sqrt()) if N else 0.1
+    rho = torch.log(torch.full((M,), max(typical, 1e-3))) + 0.3 * torch.randn(M, generator=g)
+    omega = torch.randn(M, generator=g)
+    if weight_method == 'W':
+        pair = torch.randn(N, K, generator=g).to(device)  # the caller's gather of sp_W rows
+    elif weight_method == 'given':
+        pair = torch.rand(N, K, generator=g).to(device)
+    else:
+        pair = d2
+    kw = dict(temperature=0.01 if typical < 0.3 else 0.05, warp_method=warp_method, sp_rot=d(sp_rot),
+              weight_method=weight_method,
+              sp_log_radius=d(rho) if 'kernel' in weight_method else None,
+              sp_weight_logit=d(omega) if weight_method == 'weighted_kernel' else None)
+    f64 = lambda t: None if t is None else t.detach().cpu().double()
+    okw = dict(weight_method=weight_method, temperature=kw['temperature'], warp_method=warp_method or 'LBS',
+               sp_radius=f64(rho) if 'kernel' in weight_method else None,
+               sp_weight=f64(omega) if weight_method == 'weighted_kernel' else None)
+    oargs = [f64(pts), f64(ctrl), f64(sp_t), f64(sp_r), f64(sp_s), f64(sp_rot), f64(pair), idx.cpu()]
+    return (d(pts), d(ctrl), d(sp_t), d(sp_r), d(sp_s), pair, idx), kw, oargs, okw
+
+
+@pytest.mark.parametrize("warp_method,weight_method", LBS_CASES)
+def test_lbs_forward(warp_method, weight_method, device, c1):
+    from fast_sp_gs_amd._C import get_C_function
+    from oracle import lbs as OL
+    args, kw, oargs, okw = _lbs_inputs(c1['points'], c1['ctrl'], c1['sp_t'], c1['sp_r'], c1['sp_s'], 3, warp_method,
+                                       weight_method, 40, device)
+    dx, dr, ds, w = get_C_function('lbs_blend')(*args, **kw)
+    rx, rr, rs, rw = OL.lbs_blend(*oargs, **okw)
+    assert abs_err(npy(w), rw.numpy()) < 1e-5 and abs_err(npy(dx), rx.numpy()) < 1e-5
+    assert abs_err(npy(dr), rr.numpy()) < 1e-5 and abs_err(npy(ds), rs.numpy()) < 1e-6
+    assert float(w.max(dim=1).values.mean()) < 0.98 or weight_method == 'given'  # the weights really mix neighbours
+
+
+def _lbs_backward_case(device, pts, ctrl, sp_t, sp_r, sp_s, K, warp_method, weight_method, seed):
+    from fast_sp_gs_amd._C import get_C_function
+    from oracle import lbs as OL
     N, M = pts.shape[0], ctrl.shape[0]
     S = 0 if sp_s is None else sp_s.shape[1]
-    g = torch.Generator().manual_seed(seed)
+    args, kw, oargs, okw = _lbs_inputs(pts, ctrl, sp_t, sp_r, sp_s, K, warp_method, weight_method, seed, device)
+    g = torch.Generator().manual_seed(seed + 1000)
     gx, gr = torch.randn(N, 3, generator=g), torch.randn(N, 4, generator=g)
     gs = torch.randn(N, S, generator=g) if S else None
     d = lambda t: None if t is None else t.to(device).contiguous()
-    d2, idx = get_C_function('knn_topk')(d(pts), d(ctrl), K)
-    print(f"[lbs backward] N={N} M={M} K={K} S={S} centred={centred}", flush=True)
-    out = get_C_function('lbs_blend_backward')(d(pts), d(ctrl), d(sp_t), d(sp_r), d(sp_s), d2, idx, d(gx), d(gr),
-                                               d(gs), tau, centred)
+    print(f"[lbs backward] N={N} M={M} K={K} S={S} warp={warp_method} weights={weight_method}", flush=True)
+    out = get_C_function('lbs_blend_backward')(*args, d(gx), d(gr), d(gs), **kw)
     torch.cuda.synchronize()
-    z = lambda *shape: np.zeros(shape, np.float32)
-    ref = [z(N, 3), z(N, K), z(M, 3), z(M, 3), z(M, 4), z(M, max(S, 1))]
-    O.call("lbs_blend_backward_f32", N, M, K, int(centred), tau, npy(pts), npy(ctrl), npy(sp_t), npy(sp_r),
-           None if sp_s is None else npy(sp_s), S, npy(d2), npy(idx), npy(gx), npy(gr), None if gs is None else npy(gs),
-           *ref)
-    names = ('points', 'dist2', 'sp_points', 'sp_t', 'sp_r', 'sp_s')
-    for name, a, b in zip(names, out, ref):
+    ref = OL.lbs_blend_backward(*oargs, gx.double(), gr.double(), None if gs is None else gs.double(), **okw)
+    pairs = [('g_points', 'points'), ('g_pair', 'pair_in'), ('g_sp_points', 'sp_points'), ('g_sp_t', 'sp_t'),
+             ('g_sp_rot', 'sp_rot'), ('g_sp_r', 'sp_r'), ('g_sp_s', 'sp_s'), ('g_log_radius', 'sp_radius'),
+             ('g_weight_logit', 'sp_weight')]
+    for mine, theirs in pairs:
+        a, b = out[mine], ref[theirs]
+        assert (a is None) == (b is None), mine
         if a is None:
             continue
-        # sums of thousands of fp32 terms in a different association than the oracle's running sum
-        assert rel_err(npy(a), b) < 2e-4, (name, rel_err(npy(a), b))
-    # the squared-distance gradient continues into both point sets
-    gd = out[1]
-    g_x, g_y = get_C_function('knn_topk_backward')(d(pts), d(ctrl), idx, gd)
-    torch.cuda.synchronize()
-    rx, ry = z(N, 3), z(M, 3)
-    O.call("knn_topk_backward_f32", N, M, 3, K, npy(pts), npy(ctrl), npy(idx), npy(gd), rx, ry)
-    assert rel_err(npy(g_x), rx) < 1e-5 and rel_err(npy(g_y), ry) < 2e-4
+        b = b.numpy()
+        if not np.abs(b).max() > 0:
+            assert not npy(a).any(), mine   # e.g. no pivot term outside LBS_c, no position gradient without a rotation
+            continue
+        # sums of thousands of fp32 terms in a different association than the oracle's float64 sum
+        assert rel_err(npy(a), b) < 2e-4, (mine, rel_err(npy(a), b))
+    if weight_method in ('dist', 'kernel', 'weighted_kernel'):
+        # the squared-distance gradient continues into both point sets
+        O = __import__('oracle')
+        gd = out['g_pair']
+        g_x, g_y = get_C_function('knn_topk_backward')(args[0], args[1], args[6], gd)
+        torch.cuda.synchronize()
+        rx, ry = np.zeros((N, 3), np.float32), np.zeros((M, 3), np.float32)
+        O.call("knn_topk_backward_f32", N, M, 3, K, npy(pts), npy(ctrl), npy(args[6]), npy(gd), rx, ry)
+        assert rel_err(npy(g_x), rx) < 1e-5 and rel_err(npy(g_y), ry) < 2e-4
 
 
-def test_lbs_and_knn_backward(device, oracle_mod, c1):
-    O = oracle_mod
+@pytest.mark.parametrize("warp_method,weight_method", LBS_CASES)
+def test_lbs_backward_modes(warp_method, weight_method, device, oracle_mod, c1):
+    """Every weight / warp combination at the default configuration's K = 3 (binned, atomic-free sums)."""
+    _lbs_backward_case(device, c1['points'][:30011], c1['ctrl'], c1['sp_t'], c1['sp_r'], c1['sp_s'], 3, warp_method,
+                       weight_method, seed=21)
+
+
+def test_lbs_and_knn_backward_shapes(device, oracle_mod, c1):
     pts, ctrl = c1['points'][:30011], c1['ctrl']
-    for centred in (False, True):
-        _lbs_backward_case(O, device, pts, ctrl, c1['sp_t'], c1['sp_r'], c1['sp_s'], 4, 0.01, centred, seed=21)
     g = torch.Generator().manual_seed(22)
-    # no scale residuals, K = 8, fewer points than one block
+    # three scale residuals (what the network predicts before the caller slices them), K = 4
+    s3 = 0.1 * torch.randn(512, 3, generator=g)
+    _lbs_backward_case(device, pts, ctrl, c1['sp_t'], c1['sp_r'], s3, 4, 'LBS_c', 'weighted_kernel', seed=28)
+    # no scale residuals, K = 8, fewer points than one block (LDS float atomics: not binned)
     small_ctrl = torch.rand(40, 3, generator=g) * 2 - 1
-    _lbs_backward_case(O, device, pts[:100], small_ctrl, 0.1 * torch.randn(40, 3, generator=g),
-                       0.2 * torch.randn(40, 4, generator=g), None, 8, 0.05, True, seed=23)
+    _lbs_backward_case(device, pts[:100], small_ctrl, 0.1 * torch.randn(40, 3, generator=g),
+                       0.2 * torch.randn(40, 4, generator=g), None, 8, 'LBS_c', 'weighted_kernel', seed=23)
     # more neighbours asked for than control points exist: the padded slots (index -1) carry nothing
     tiny_ctrl = torch.rand(3, 3, generator=g) * 2 - 1
-    _lbs_backward_case(O, device, pts[:500], tiny_ctrl, 0.1 * torch.randn(3, 3, generator=g),
-                       0.2 * torch.randn(3, 4, generator=g), 0.1 * torch.randn(3, 2, generator=g), 5, 0.05, False,
+    _lbs_backward_case(device, pts[:500], tiny_ctrl, 0.1 * torch.randn(3, 3, generator=g),
+                       0.2 * torch.randn(3, 4, generator=g), 0.1 * torch.randn(3, 2, generator=g), 5, 'LBS', 'dist',
                        seed=24)
     # K = 4 with a padded slot (3 control points), through the binned variant
-    _lbs_backward_case(O, device, pts[:700], tiny_ctrl, 0.1 * torch.randn(3, 3, generator=g),
-                       0.2 * torch.randn(3, 4, generator=g), 0.1 * torch.randn(3, 2, generator=g), 4, 0.05, True,
-                       seed=26)
+    for wm in ('dist', 'kernel'):
+        _lbs_backward_case(device, pts[:700], tiny_ctrl, 0.1 * torch.randn(3, 3, generator=g),
+                           0.2 * torch.randn(3, 4, generator=g), 0.1 * torch.randn(3, 2, generator=g), 4, 'LBS_c', wm,
+                           seed=26)
     # more points than one pass of the launch covers: every block bins several chunks into its table
     many = torch.rand(280_001, 3, generator=g) * 2 - 1
-    _lbs_backward_case(O, device, many, ctrl, c1['sp_t'], c1['sp_r'], c1['sp_s'], 4, 0.01, False, seed=27)
-    # a control set whose table exceeds LDS takes the atomic path
+    _lbs_backward_case(device, many, ctrl, c1['sp_t'], c1['sp_r'], c1['sp_s'], 3, None, 'weighted_kernel', seed=27)
+    # a control set whose table exceeds LDS takes the device-scope atomic path
     big_ctrl = torch.rand(2500, 3, generator=g) * 2 - 1
-    _lbs_backward_case(O, device, pts[:20000], big_ctrl, 0.1 * torch.randn(2500, 3, generator=g),
-                       0.2 * torch.randn(2500, 4, generator=g), 0.1 * torch.randn(2500, 2, generator=g), 4, 0.01, True,
-                       seed=25)
+    _lbs_backward_case(device, pts[:20000], big_ctrl, 0.1 * torch.randn(2500, 3, generator=g),
+                       0.2 * torch.randn(2500, 4, generator=g), 0.1 * torch.randn(2500, 2, generator=g), 4, 'LBS_c',
+                       'weighted_kernel', seed=25)
 
 
-def test_deform_branch_autograd(device):
+@pytest.mark.parametrize("local_frame,is_blender", [(True, True), (False, False)])
+def test_deform_branch_autograd(local_frame, is_blender, device):
     """superpoint_deform and the MLP are differentiable end to end: gradients through the HIP backward kernels equal
-    torch autograd of the same formulas written with torch ops on the device."""
+    torch autograd of the same formulas written with torch ops on the device. With a local-rotation head the warp is
+    the rigid blend about the control points (LBS_c), without one the translations are blended (the reference's default
+    configuration); with the D-NeRF time network in front, its parameters get their gradient through the MLP's input."""
     from fast_sp_gs_amd.deform import DeformNetwork, superpoint_deform
     g = torch.Generator().manual_seed(31)
-    N, M, K, tau = 5000, 64, 4, 0.02
+    N, M, K = 5000, 64, 3
     pts = (torch.rand(N, 3, generator=g) * 2 - 1).to(device)
     ctrl = (torch.rand(M, 3, generator=g) * 2 - 1).to(device).requires_grad_()
-    net = DeformNetwork().to(device)
-    for head in (net.gaussian_warp, net.gaussian_rotation, net.gaussian_scaling):
+    hyper = (0.1 * torch.randn(N, 8, generator=g)).to(device).requires_grad_()
+    sp_hyper = (0.1 * torch.randn(M, 8, generator=g)).to(device).requires_grad_()
+    rho = torch.full((M,), float(np.log(0.25)), device=device).requires_grad_()
+    omega = torch.randn(M, generator=g).to(device).requires_grad_()
+    torch.manual_seed(32)
+    net = DeformNetwork(t_degree=6 if is_blender else 10, is_blender=is_blender, local_frame=local_frame).to(device)
+    for head in net._heads():
         torch.nn.init.normal_(head.weight, std=0.05)  # the default 1e-5 would make every gradient vanish
     t = torch.full((1,), 0.3, device=device)
     gx, gr, gs = (torch.randn(N, c, generator=g).to(device) for c in (3, 4, 2))
@@ -212,35 +279,48 @@ def test_deform_branch_autograd(device):
     def loss_of(d_xyz, d_rot, d_scale):
         return (d_xyz * gx).sum() + (d_rot * gr).sum() + (d_scale * gs).sum()
 
-    c_xyz, c_rot, c_scale, _ = net(ctrl.detach(), t)
-    assert c_xyz.requires_grad
-    d_xyz, d_rot, d_scale, w, idx = superpoint_deform(pts, ctrl, c_xyz, c_rot, c_scale[:, :2], K=K, temperature=tau,
-                                                      centred=True)
+    c_xyz, c_rot, c_scale, c_local = net(ctrl.detach(), t)
+    assert c_xyz.requires_grad and (c_local is not None) == local_frame
+    d_xyz, d_rot, d_scale, w, idx = superpoint_deform(
+        pts, ctrl, c_xyz, c_rot, c_scale[:, :2], sp_rot=c_local, K=K, warp_method='LBS_c',
+        LBS_method='weighted_kernel', sp_radius=rho, sp_weight=omega, feature=hyper, sp_feature=sp_hyper)
+    leaves = [ctrl, hyper, sp_hyper, rho, omega]
+    leaf_names = ['sp_points', 'hyper', 'sp_hyper', 'sp_radius', 'sp_weight']
     params = list(net.parameters())
-    grads = torch.autograd.grad(loss_of(d_xyz, d_rot, d_scale), [ctrl] + params, allow_unused=True)
+    grads = torch.autograd.grad(loss_of(d_xyz, d_rot, d_scale), leaves + params, allow_unused=True)
 
-    # the same computation with torch ops (fp32 network, explicit softmax / rotation / blend)
-    r_xyz, r_rot, r_scale, _ = net.forward_fp32(ctrl.detach(), t)
-    diff = pts[:, None, :] - ctrl[idx]
-    wt = torch.softmax(-(diff * diff).sum(-1) / tau, -1)
-    q = r_rot + torch.tensor([0, 0, 0, 1.0], device=device)
-    q = q / q.norm(dim=-1, keepdim=True)
-    x, y, z, s = q.unbind(-1)
-    R = torch.stack([1 - 2 * (y * y + z * z), 2 * (x * y - z * s), 2 * (y * s + x * z),
-                     2 * (x * y + z * s), 1 - 2 * (x * x + z * z), 2 * (y * z - x * s),
-                     2 * (x * z - y * s), 2 * (x * s + y * z), 1 - 2 * (x * x + y * y)], -1).view(M, 3, 3)
-    tt = r_xyz + ctrl - torch.einsum('mab,mb->ma', R, ctrl)
-    moved = torch.einsum('nkab,nb->nka', R[idx], pts) + tt[idx]
-    e_xyz = (wt[..., None] * moved).sum(1) - pts
+    # the same computation with torch ops (fp32 network, the reference's expressions: network.py:498-573)
+    r_xyz, r_rot, r_scale, r_local = net.forward_fp32(ctrl.detach(), t)
+    x = torch.cat([pts, hyper], -1)
+    y = torch.cat([ctrl.detach(), sp_hyper], -1)
+    diff = x[:, None, :] - y[idx]
+    nn_dist = (diff * diff).sum(-1)
+    wt = torch.exp(-nn_dist / (2 * torch.exp(rho)[idx] ** 2)) * torch.sigmoid(omega)[idx] + 1e-7
+    wt = wt / wt.sum(-1, keepdim=True)
+    assert float((wt.detach() - w).abs().max()) < 1e-4
+    if local_frame:
+        q = r_local + torch.tensor([0, 0, 0, 1.0], device=device)
+        q = q / q.norm(dim=-1, keepdim=True)
+        qx, qy, qz, qs = q.unbind(-1)
+        R = torch.stack([1 - 2 * (qy * qy + qz * qz), 2 * (qx * qy - qz * qs), 2 * (qy * qs + qx * qz),
+                         2 * (qx * qy + qz * qs), 1 - 2 * (qx * qx + qz * qz), 2 * (qy * qz - qx * qs),
+                         2 * (qx * qz - qy * qs), 2 * (qx * qs + qy * qz), 1 - 2 * (qx * qx + qy * qy)], -1).view(M, 3, 3)
+        tt = r_xyz + ctrl - torch.einsum('mab,mb->ma', R, ctrl)
+        moved = torch.einsum('nkab,nb->nka', R[idx], pts) + tt[idx]
+        e_xyz = (wt[..., None] * moved).sum(1) - pts
+    else:
+        e_xyz = (wt[..., None] * r_xyz[idx]).sum(1)
     e_rot = (wt[..., None] * r_rot[idx]).sum(1)
     e_scale = (wt[..., None] * r_scale[:, :2][idx]).sum(1)
     assert float((e_xyz - d_xyz).detach().abs().max()) < 2e-2 * float(e_xyz.detach().abs().max())  # bf16 forward
-    ref = torch.autograd.grad(loss_of(e_xyz, e_rot, e_scale), [ctrl] + params, allow_unused=True)
-    for name, a, b in zip(['sp_points'] + [n for n, _ in net.named_parameters()], grads, ref):
-        assert (a is None) == (b is None), name
-        if a is None:
+    ref = torch.autograd.grad(loss_of(e_xyz, e_rot, e_scale), leaves + params, allow_unused=True)
+    seen_timenet = False
+    for name, a, b in zip(leaf_names + [n for n, _ in net.named_parameters()], grads, ref):
+        if b is None or not float(b.abs().max()) > 0:
+            assert a is None or not float(a.abs().max()) > 0, name  # e.g. sp_points without a pivot or a rotation
             continue
-        if name == 'sp_points':
+        assert a is not None, name
+        if name in leaf_names:
             # the HIP forward runs the layers in bf16, so the values the chain rule is evaluated at differ by ~1e-2 rel
             scale = float(b.abs().max())
             assert float((a - b).abs().max()) <= 5e-2 * scale + 1e-12, (name, float((a - b).abs().max()), scale)
@@ -249,6 +329,38 @@ def test_deform_branch_autograd(device):
             # sums of random-sign terms element-wise; the direction of the gradient is what has to agree
             cos = float((a * b).sum() / (a.norm() * b.norm()).clamp_min(1e-30))
             assert cos > 0.97, (name, cos)
+            seen_timenet |= name.startswith('timenet')
+    assert seen_timenet == is_blender
+
+
+def test_calc_LBS_weight_and_warp_mirror_the_fused_path(device):
+    """`calc_LBS_weight` (K-NN on the HIP kernel, the reference's torch weight expressions) followed by `warp` on those
+    weights gives what `superpoint_deform` computes in one kernel, values and gradients."""
+    from fast_sp_gs_amd.deform import calc_LBS_weight, superpoint_deform, warp
+    g = torch.Generator().manual_seed(33)
+    N, M, K = 3000, 40, 3
+    dev = lambda t: t.to(device)
+    pts = dev(torch.rand(N, 3, generator=g) * 2 - 1)
+    mk = lambda *shape, s=0.2: dev(s * torch.randn(*shape, generator=g)).requires_grad_()
+    ctrl, sp_t, sp_r, sp_s, sp_rot = mk(M, 3, s=0.6), mk(M, 3), mk(M, 4), mk(M, 3), mk(M, 4)
+    rho, omega = (dev(torch.full((M,), float(np.log(0.3))))).requires_grad_(), mk(M, s=1.0)
+    gx, gr, gs = (dev(torch.randn(N, c, generator=g)) for c in (3, 4, 3))
+    leaves = [ctrl, sp_t, sp_r, sp_s, sp_rot, rho, omega]
+    for rot, method in ((sp_rot, 'LBS_c'), (sp_rot, 'LBS'), (None, 'LBS')):
+        use = [l for l in leaves if not (l is sp_rot and rot is None)]
+        a = superpoint_deform(pts, ctrl, sp_t, sp_r, sp_s, sp_rot=rot, K=K, warp_method=method,
+                              LBS_method='weighted_kernel', sp_radius=rho, sp_weight=omega)
+        ga = torch.autograd.grad((a[0] * gx).sum() + (a[1] * gr).sum() + (a[2] * gs).sum(), use, allow_unused=True)
+        w, idx = calc_LBS_weight(pts, ctrl, K=K, LBS_method='weighted_kernel', sp_radius=rho, sp_weight=omega)
+        b = warp(pts, ctrl, sp_t, sp_r, sp_s, rot, w, idx, method)
+        gb = torch.autograd.grad((b[0] * gx).sum() + (b[1] * gr).sum() + (b[2] * gs).sum(), use, allow_unused=True)
+        assert torch.equal(idx, a[4]) and float((w - a[3]).abs().max()) < 1e-5
+        for x, y in zip(a[:3], b):
+            assert float((x - y).abs().max()) < 1e-5
+        for x, y in zip(ga, gb):
+            assert (x is None) == (y is None)
+            if x is not None:
+                assert float((x - y).abs().max()) <= 2e-4 * max(float(y.abs().max()), 1e-6)
 
 
 @pytest.mark.parametrize("B,D,p_degree,t_degree", [(512, 8, 10, 10), (500, 8, 10, 6), (70, 4, 4, 2), (1, 3, 2, 1)])

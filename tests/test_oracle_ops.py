@@ -64,96 +64,87 @@ def test_knn_matches_sorting(oracle_mod):
     assert (idx[:, 3:] == -1).all() and (d2[:, 3:] == -1).all()
 
 
-def _lbs(O, points, ctrl, sp_t, sp_r, sp_s, d2, idx, temperature, centred):
-    N, K = d2.shape
-    S = sp_s.shape[1]
-    w, dx, dr, ds = np.zeros((N, K)), np.zeros((N, 3)), np.zeros((N, 4)), np.zeros((N, S))
-    assert O.call("lbs_blend_f64", N, ctrl.shape[0], K, int(centred), float(temperature), points, ctrl, sp_t, sp_r,
-                  sp_s, S, d2, idx, w, dx, dr, ds) == 0
-    return w, dx, dr, ds
-
-
 def test_lbs_closed_forms(oracle_mod):
-    O = oracle_mod
-    rng = np.random.default_rng(3)
+    """oracle/lbs.py (weights and warp of network.py:507-517, 545-573) against closed forms that a dropped term, a
+    transposed rotation or a wrong branch would break."""
+    from oracle import lbs as OL
+    from scipy.spatial.transform import Rotation
+    g = torch.Generator().manual_seed(3)
     N, M, K = 50, 8, 4
-    pts, ctrl = rng.normal(size=(N, 3)), rng.normal(size=(M, 3))
-    idx = np.ascontiguousarray(np.stack([rng.permutation(M)[:K] for _ in range(N)]).astype(np.int64))
-    d2 = np.ascontiguousarray(np.sort(rng.uniform(0, 0.05, size=(N, K)), 1))
-    zero3, zero4, s0 = np.zeros((M, 3)), np.zeros((M, 4)), np.zeros((M, 2))
-    # identity transforms (residual rotation 0 -> q = (0,0,0,1), t = 0) move nothing; weights are a softmax
-    w, dx, dr, ds = _lbs(O, pts, ctrl, zero3, zero4, s0, d2, idx, 0.01, False)
-    assert np.abs(dx).max() < 1e-14 and np.abs(dr).max() == 0
-    assert np.allclose(w, torch.softmax(torch.from_numpy(-d2 / 0.01), -1).numpy(), atol=1e-14)
-    # one control point everywhere with weight 1: a rigid motion p -> R p + t
+    f64 = dict(dtype=torch.float64, generator=g)
+    pts, ctrl = torch.randn(N, 3, **f64), torch.randn(M, 3, **f64)
+    idx = torch.stack([torch.randperm(M, generator=g)[:K] for _ in range(N)])
+    d2 = torch.sort(torch.rand(N, K, **f64) * 0.05, 1).values
+    zero3, zero4, s0 = torch.zeros(M, 3, dtype=torch.float64), torch.zeros(M, 4, dtype=torch.float64), \
+        torch.zeros(M, 2, dtype=torch.float64)
+    # identity transforms (local rotation 0 -> q = (0,0,0,1), t = 0) move nothing; 'dist' weights are a softmax
+    dx, dr, ds, w = OL.lbs_blend(pts, ctrl, zero3, zero4, s0, zero4, d2, idx, 'dist', 0.01, 'LBS')
+    assert float(dx.abs().max()) < 1e-14 and float(dr.abs().max()) == 0
+    assert torch.allclose(w, torch.softmax(-d2 / 0.01, -1), atol=1e-14)
+    # one rigid motion everywhere: p -> R p + t, with R from scipy (x, y, z, w convention)
     ang, axis = 0.7, np.array([0.0, 0.6, 0.8])
     q = np.concatenate([axis * np.sin(ang / 2), [np.cos(ang / 2)]])
-    from scipy.spatial.transform import Rotation
-    Rm = Rotation.from_quat(q).as_matrix()
-    t = np.array([0.1, -0.2, 0.3])
-    sp_r = np.tile(2.5 * q - np.array([0, 0, 0, 1.0]), (M, 1))  # normalize(r + (0,0,0,1)) == q
-    sp_t = np.tile(t, (M, 1))
-    w, dx, dr, ds = _lbs(O, pts, ctrl, sp_t, sp_r, s0 + 0.5, d2, idx, 0.01, False)
-    assert np.abs(dx - (pts @ Rm.T + t - pts)).max() < 1e-12
-    assert np.allclose(dr, sp_r[0]) and np.allclose(ds, 0.5)
-    # centred: rotation about the control point c: p -> R (p - c) + c + t
-    same = np.zeros((N, K), np.int64) + 5
-    w, dx, dr, ds = _lbs(O, pts, ctrl, sp_t, sp_r, s0, d2, same, 0.01, True)
-    assert np.abs(dx - ((pts - ctrl[5]) @ Rm.T + ctrl[5] + t - pts)).max() < 1e-12
+    Rm = torch.from_numpy(Rotation.from_quat(q).as_matrix())
+    t = torch.tensor([0.1, -0.2, 0.3], dtype=torch.float64)
+    sp_rot = torch.from_numpy(2.5 * q - np.array([0, 0, 0, 1.0])).repeat(M, 1)  # normalize(rot + (0,0,0,1)) == q
+    sp_r = torch.randn(M, 4, **f64)
+    sp_t = t.repeat(M, 1)
+    dx, dr, ds, w = OL.lbs_blend(pts, ctrl, sp_t, sp_r, s0 + 0.5, sp_rot, d2, idx, 'dist', 0.01, 'LBS')
+    assert float((dx - (pts @ Rm.T + t - pts)).abs().max()) < 1e-12
+    # the rotation that moves the points is sp_rot; sp_r is only blended into d_rotation (network.py:546-547, 565-566)
+    assert float((dr - (w[..., None] * sp_r[idx]).sum(1)).abs().max()) < 1e-14 and torch.allclose(ds, ds * 0 + 0.5)
+    # LBS_c: rotation about the control point c: p -> R (p - c) + c + t
+    same = torch.full((N, K), 5)
+    dx = OL.lbs_blend(pts, ctrl, sp_t, sp_r, s0, sp_rot, d2, same, 'dist', 0.01, 'LBS_c')[0]
+    assert float((dx - ((pts - ctrl[5]) @ Rm.T + ctrl[5] + t - pts)).abs().max()) < 1e-12
+    # no local rotation (the default configuration): the translations are blended, nothing else, whatever the method
+    sp_t2 = torch.randn(M, 3, **f64)
+    for method in ('LBS', 'LBS_c'):
+        dx, dr, ds, w = OL.lbs_blend(pts, ctrl, sp_t2, sp_r, s0, None, d2, idx, 'dist', 0.01, method)
+        assert float((dx - (w[..., None] * sp_t2[idx]).sum(1)).abs().max()) < 1e-14
+    # kernel weights by an explicit loop on the raw parameters (radius = exp(.), weight = sigmoid(.))
+    rho, omega = 0.3 * torch.randn(M, **f64) - 2.0, torch.randn(M, **f64)
+    for method in ('kernel', 'weighted_kernel'):
+        w = OL.lbs_weights(d2, idx, M, method, 1.0, rho, omega)
+        for n in range(0, N, 7):
+            u = [np.exp(-float(d2[n, k]) / (2 * np.exp(float(rho[idx[n, k]])) ** 2)) *
+                 (1 / (1 + np.exp(-float(omega[idx[n, k]]))) if method == 'weighted_kernel' else 1.0) + 1e-7
+                 for k in range(K)]
+            assert np.allclose(w[n].numpy(), np.array(u) / sum(u), atol=1e-14)
+        assert torch.allclose(w.sum(-1), torch.ones(N, dtype=torch.float64))
+    # limiting cases: equal radii and weights -> softmax(-d2 / (2 r^2)) up to the 1e-7 floor; a huge radius -> uniform
+    w = OL.lbs_weights(d2, idx, M, 'kernel', 1.0, torch.full((M,), np.log(0.1), dtype=torch.float64), None)
+    assert float((w - torch.softmax(-d2 / (2 * 0.1 ** 2), -1)).abs().max()) < 1e-6
+    w = OL.lbs_weights(d2, idx, M, 'kernel', 1.0, torch.full((M,), 10.0, dtype=torch.float64), None)
+    assert float((w - 1.0 / K).abs().max()) < 1e-6
+    # 'W': softmax of the gathered rows; padded slots (index -1) get weight 0 and the rest still sums to 1
+    sp_W = torch.randn(N, M, **f64)
+    w = OL.lbs_weights(torch.gather(sp_W, 1, idx), idx, M, 'W')
+    assert torch.allclose(w, torch.gather(sp_W, 1, idx).softmax(-1))
+    padded = idx.clone()
+    padded[:, -1] = -1
+    w = OL.lbs_weights(d2, padded, M, 'dist', 0.01)
+    assert float(w[:, -1].abs().max()) == 0 and torch.allclose(w.sum(-1), torch.ones(N, dtype=torch.float64))
 
 
-def test_lbs_and_knn_backward_match_autograd(oracle_mod):
-    """The oracle's hand-derived LBS / K-NN gradients against torch autograd (fp64) of the forward written a different
-    way: rotation through Rodrigues' form R = (w^2 - v.v) I + 2 v v^T + 2 w [v]x of the normalised quaternion, weights
-    through torch.softmax, distances through explicit differences."""
+def test_knn_backward_matches_autograd(oracle_mod):
+    """K-NN squared distances: gradient of sum(g * d2) w.r.t. both point sets against torch autograd (fp64), with the 11
+    columns the default configuration searches in (positions + 8 hyper features, exps/d_nerf.yaml:21-23)."""
     O = oracle_mod
     g = torch.Generator().manual_seed(12)
-    N, M, K, S, tau = 70, 9, 4, 2, 0.05
-    for centred in (False, True):
-        pts = torch.randn(N, 3, generator=g, dtype=torch.float64, requires_grad=True)
-        ctrl = torch.randn(M, 3, generator=g, dtype=torch.float64, requires_grad=True)
-        sp_t = (0.2 * torch.randn(M, 3, generator=g, dtype=torch.float64)).requires_grad_()
-        sp_r = (0.4 * torch.randn(M, 4, generator=g, dtype=torch.float64)).requires_grad_()
-        sp_s = (0.1 * torch.randn(M, S, generator=g, dtype=torch.float64)).requires_grad_()
+    for D in (3, 11):
+        N, M, K = 70, 9, 3
+        pts = torch.randn(N, D, generator=g, dtype=torch.float64, requires_grad=True)
+        ctrl = torch.randn(M, D, generator=g, dtype=torch.float64, requires_grad=True)
         with torch.no_grad():
             idx = torch.cdist(pts, ctrl).topk(K, largest=False).indices.contiguous()
         diff = pts[:, None, :] - ctrl[idx]
         d2 = (diff * diff).sum(-1)
-        d2_leaf = d2.detach().clone().requires_grad_()
-        w = torch.softmax(-d2_leaf / tau, -1)
-        q = sp_r + torch.tensor([0, 0, 0, 1.0], dtype=torch.float64)
-        q = q / q.norm(dim=-1, keepdim=True)
-        v, s = q[:, :3], q[:, 3:]
-        zero = torch.zeros(M, dtype=torch.float64)
-        skew = torch.stack([zero, -v[:, 2], v[:, 1], v[:, 2], zero, -v[:, 0], -v[:, 1], v[:, 0], zero], -1).view(M, 3, 3)
-        eye = torch.eye(3, dtype=torch.float64)
-        R = (s * s - (v * v).sum(-1, keepdim=True))[..., None] * eye + 2 * v[:, :, None] * v[:, None, :] + \
-            2 * s[..., None] * skew
-        t = sp_t + ctrl - torch.einsum('mab,mb->ma', R, ctrl) if centred else sp_t
-        moved = torch.einsum('nkab,nb->nka', R[idx], pts) + t[idx]
-        d_xyz = (w[..., None] * moved).sum(1) - pts
-        d_rot = (w[..., None] * sp_r[idx]).sum(1)
-        d_scale = (w[..., None] * sp_s[idx]).sum(1)
-        gx, gr, gs = (torch.randn(*t_.shape, generator=g, dtype=torch.float64) for t_ in (d_xyz, d_rot, d_scale))
-        loss = (d_xyz * gx).sum() + (d_rot * gr).sum() + (d_scale * gs).sum()
-        a_pts, a_d2, a_ctrl, a_t, a_r, a_s = torch.autograd.grad(loss, [pts, d2_leaf, ctrl, sp_t, sp_r, sp_s],
-                                                                  allow_unused=True)
-        n = lambda x: np.ascontiguousarray(x.detach().numpy())
-        o_pts, o_d2, o_ctrl = np.zeros((N, 3)), np.zeros((N, K)), np.zeros((M, 3))
-        o_t, o_r, o_s = np.zeros((M, 3)), np.zeros((M, 4)), np.zeros((M, S))
-        assert O.call("lbs_blend_backward_f64", N, M, K, int(centred), tau, n(pts), n(ctrl), n(sp_t), n(sp_r), n(sp_s),
-                      S, n(d2), n(idx), n(gx), n(gr), n(gs), o_pts, o_d2, o_ctrl, o_t, o_r, o_s) == 0
-        a_ctrl = torch.zeros(M, 3, dtype=torch.float64) if a_ctrl is None else a_ctrl
-        for name, a, o in (("points", a_pts, o_pts), ("dist2", a_d2, o_d2), ("sp_points", a_ctrl, o_ctrl),
-                           ("sp_t", a_t, o_t), ("sp_r", a_r, o_r), ("sp_s", a_s, o_s)):
-            scale = max(float(a.abs().max()), 1e-30)
-            assert np.abs(n(a) - o).max() < 1e-11 * max(scale, 1.0), (centred, name)
-        assert centred or not o_ctrl.any()
-        # K-NN distances: gradient of sum(g * d2) w.r.t. both point sets
         gd = torch.randn(N, K, generator=g, dtype=torch.float64)
         k_x, k_y = torch.autograd.grad((d2 * gd).sum(), [pts, ctrl])
-        o_x, o_y = np.zeros((N, 3)), np.zeros((M, 3))
-        assert O.call("knn_topk_backward_f64", N, M, 3, K, n(pts), n(ctrl), n(idx), n(gd), o_x, o_y) == 0
+        n = lambda x: np.ascontiguousarray(x.detach().numpy())
+        o_x, o_y = np.zeros((N, D)), np.zeros((M, D))
+        assert O.call("knn_topk_backward_f64", N, M, D, K, n(pts), n(ctrl), n(idx), n(gd), o_x, o_y) == 0
         assert np.abs(n(k_x) - o_x).max() < 1e-12 and np.abs(n(k_y) - o_y).max() < 1e-12
 
 
