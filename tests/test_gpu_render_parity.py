@@ -3,15 +3,18 @@ CPU oracle, stage by stage, on the same seeded inputs. Every stage is fed the GP
 integer results (radii, keys, ranges, point lists) are compared on identical float inputs.
 
 Tolerances (stated by the task): images 1e-4 abs, gradients 1e-3 rel (max|d|/max|ref|), bit-exact keys / ranges /
-point lists. A (pixel, surfel) pair whose alpha sits within float rounding of the 1/255 or T<1e-4 thresholds may be
-accepted on one side and skipped on the other (exp and 1/x differ in the last ulp between libm and the GPU), which
-moves that pixel by up to ~4e-3; at most max(2, 1e-5 * H * W) such pixels are allowed per image.
+point lists. Float results of the blend are compared with the oracle evaluated in float64 on the GPU's float32 inputs
+(the exact value of the reference's formulas; the oracle in float32 without fused multiply-adds is itself up to 2e-3
+away from it on grazing surfels). A (pixel, surfel) pair whose alpha sits within float32 rounding of the 1/255 or
+T < 1e-4 thresholds may be accepted in float32 and skipped in float64 or the reverse, which shows as a different
+n_contrib for that pixel; at most max(2, 1e-5 * H * W) such pixels are allowed per image and every other pixel must
+hold the tolerance.
 """
 import numpy as np
 import pytest
 import torch
 
-from util import abs_err, frac_over, npy, rel_err
+from util import abs_err, f64, npy, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -68,33 +71,41 @@ def test_render_path_stage_by_stage(name, device, oracle_mod):
     assert np.array_equal(g['ranges'], ranges)
     assert np.array_equal(g['point_list'], pl)
 
-    # --- blend forward on the GPU's own inputs
-    oc, oo, oe, _, nc = O.render_forward(W, H, g['means2D'], g['colors'], g['normal_opacity'], g['trans_mat'],
+    # --- blend forward on the GPU's own inputs, against the oracle evaluated in float64 on those float32 values
+    d64 = {k: f64(g[k]) for k in ('means2D', 'colors', 'normal_opacity', 'trans_mat', 'opacity', 'extras')}
+    oc, oo, oe, _, nc = O.render_forward(W, H, d64['means2D'], d64['colors'], d64['normal_opacity'], d64['trans_mat'],
                                          g['point_list'], g['ranges'], cam.near, cam.far, False)
-    flips = max(int((np.abs(g['image'] - oc) > 1e-4).any(0).sum()), int((np.abs(g['opacity'] - oo) > 1e-4).sum()))
+    flip = (g['n_contrib'] != nc).any(0)  # pixels where a threshold decision (alpha < 1/255, T < 1e-4) fell the other way
     allowed = max(2, int(1e-5 * H * W))
-    print(f"[{name}] image abs err {abs_err(g['image'], oc):.3e}, opacity {abs_err(g['opacity'], oo):.3e}, "
-          f"extras {abs_err(g['extras'], oe):.3e}, threshold-flip pixels {flips} (allowed {allowed})")
-    assert flips <= allowed
-    if flips == 0:
-        assert abs_err(g['image'], oc) < 1e-4 and abs_err(g['opacity'], oo) < 1e-4
-    # Auxiliary maps: atol 1e-4 + rtol 1e-3. Grazing surfels make the plane-plane intersection p = k x l
-    # ill-conditioned (|p.z| << |k||l|), which amplifies the last-ulp difference between FMA-contracted GPU
-    # arithmetic and the oracle's uncontracted arithmetic; such pixels carry depths far from the scene (16..90 here).
+    keep = ~flip
+    print(f"[{name}] image abs err {abs_err(g['image'][:, keep], oc[:, keep]):.3e}, opacity "
+          f"{abs_err(g['opacity'][keep], oo[keep]):.3e}, extras {abs_err(g['extras'][:, keep], oe[:, keep]):.3e}, "
+          f"threshold-flip pixels {int(flip.sum())} (allowed {allowed})")
+    assert flip.sum() <= allowed
+    assert abs_err(g['image'][:, keep], oc[:, keep]) < 1e-4 and abs_err(g['opacity'][keep], oo[keep]) < 1e-4
+    # auxiliary maps: 1e-4 abs + 1e-3 rel (depths are unnormalised sums of z up to ~100)
     for ch in range(9):
         bad = np.abs(g['extras'][ch].astype(np.float64) - oe[ch]) > 1e-4 + 1e-3 * np.abs(oe[ch])
-        assert bad.sum() <= allowed, f"extras channel {ch}: {int(bad.sum())} pixels out of tolerance"
-    assert (g['n_contrib'] != nc).any(0).sum() <= allowed
+        assert not (bad & keep).any(), f"extras channel {ch}: {int((bad & keep).sum())} pixels out of tolerance"
 
-    # --- blend backward on the GPU's own forward outputs
-    gc, gm, gt, gn = O.render_backward(g['means2D'], g['normal_opacity'], g['colors'], g['trans_mat'], None,
-                                       g['opacity'], g['extras'], None, npy(gi), npy(go), npy(ge), None, g['ranges'],
-                                       g['point_list'], g['n_contrib'], cam.near, cam.far)
+    # --- blend backward on the GPU's own forward outputs, float64 oracle; the blend's own dL/dmeans2D included (the
+    # operator's output is overwritten in place by the preprocess backward, so the blend is called once more for it)
+    gc, gm, gt, gn = O.render_backward(d64['means2D'], d64['normal_opacity'], d64['colors'], d64['trans_mat'], None,
+                                       d64['opacity'], d64['extras'], None, f64(npy(gi)), f64(npy(go)), f64(npy(ge)),
+                                       None, g['ranges'], g['point_list'], g['n_contrib'], cam.near, cam.far)
+    from fast_sp_gs_amd._C import get_C_function
+    again = get_C_function('GS_2D_render_backward')(
+        out['means2D'], out['normal_opacity'], out['colors'], out['trans_mat'], None, out['opacity'], out['extras'],
+        None, gi.to(device), go.to(device), ge.to(device), None, out['ranges'], out['point_list'], out['n_contrib'],
+        cam.near, cam.far)
+    torch.cuda.synchronize()
     errs = dict(colors=rel_err(g['g_colors'], gc), trans=rel_err(g['g_trans'], gt),
-                normal_opacity=rel_err(g['g_normal_opacity'], gn))
+                normal_opacity=rel_err(g['g_normal_opacity'], gn), means2D=rel_err(npy(again[1]), gm),
+                trans_atomic=rel_err(npy(again[2]), gt))
     print(f"[{name}] blend backward rel errs {errs}")
     for k, v in errs.items():
         assert v < 1e-3, k
+    gm = gm.astype(np.float32)
 
     # --- preprocess backward on the GPU's own blend gradients. g_means2D was overwritten in place by the GPU pass, so
     # the oracle restarts from its own blend-backward means2D gradient (checked against the GPU's overwrite below).

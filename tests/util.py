@@ -7,6 +7,13 @@ def npy(t):
     return None if t is None else np.ascontiguousarray(t.detach().cpu().numpy())
 
 
+def f64(a):
+    """float arrays as float64 (same values) for the oracle's double instantiation; everything else unchanged."""
+    if a is None or not np.issubdtype(np.asarray(a).dtype, np.floating):
+        return a
+    return np.ascontiguousarray(np.asarray(a, np.float64))
+
+
 def rel_err(x, ref):
     """max|x - ref| / max|ref| -- the reference's own error measure (utils/test_utils.py:8-24)."""
     x, ref = np.asarray(x, np.float64), np.asarray(ref, np.float64)
