@@ -611,13 +611,12 @@ def GS_2D_fast_render_forward(width: int, height: int, near_n: float, far_n: flo
                               trans_mat_t2: Optional[Tensor] = None, accum_max_count: Optional[Tensor] = None,
                               accum_weights_p: Optional[Tensor] = None, accum_weights_count: Optional[Tensor] = None,
                               per_tile_bucket_offset: Optional[Tensor] = None):
-    """gs_2d_fast_redner.cu:839-953 -> [colors[3,H,W], opacity[H,W], extras[8,H,W]|None, flow (always None), n_contrib]
-    plus [max_contrib, bucket_to_tile, sampled_T, sampled_acc, sampled_aux] when per_tile_bucket_offset is given."""
+    """gs_2d_fast_redner.cu:839-953 -> [colors[3,H,W], opacity[H,W], extras[8,H,W]|None, flow[H,W,2]|None, n_contrib]
+    plus [max_contrib, bucket_to_tile, sampled_T, sampled_acc, sampled_aux[B, 8 | 10, 256]] when
+    per_tile_bucket_offset is given (10 channels with trans_mat_t2)."""
     what = 'GS_2D_fast_render_forward'
-    if trans_mat_t2 is not None:
-        raise RuntimeError(f'{what}: optical flow (trans_mat_t2) is not supported on the fast path')
     _f32(what, colors=colors, trans_mat=trans_mat, inverse_m=inverse_m, means2D=means2D,
-         normal_opacity=normal_opacity, accum_weights_p=accum_weights_p)
+         normal_opacity=normal_opacity, accum_weights_p=accum_weights_p, trans_mat_t2=trans_mat_t2)
     if colors.ndim != 2:
         raise RuntimeError(f'{what}: colors must have 2 dimensions')
     P = colors.shape[0]
@@ -634,13 +633,17 @@ def GS_2D_fast_render_forward(width: int, height: int, near_n: float, far_n: flo
             L.require_shape(what, name, t, P)
     if accum_weights_p is not None:
         L.require_shape(what, 'accum_weights_p', accum_weights_p, P)
+    flow = trans_mat_t2 is not None and not only_image
+    if flow:
+        L.require_shape(what, 'trans_mat_t2', trans_mat_t2, P, 3, 3)
     dev = colors.device
     opt = dict(dtype=torch.float32, device=dev)
     pixel_colors = torch.zeros((3, height, width), **opt)
     pixel_opacity = torch.zeros((height, width), **opt)
     n_contrib = torch.zeros((2, height, width), dtype=torch.int32, device=dev)
     pixel_extras = None if only_image else torch.zeros((8, height, width), **opt)
-    outputs = [pixel_colors, pixel_opacity, pixel_extras, None, n_contrib]
+    pixel_flow = torch.zeros((height, width, 2), **opt) if flow else None
+    outputs = [pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib]
     max_contrib = bucket_to_tile = sampled_T = sampled_acc = sampled_aux = None
     fast_bwd = per_tile_bucket_offset is not None
     if fast_bwd:
@@ -653,7 +656,7 @@ def GS_2D_fast_render_forward(width: int, height: int, near_n: float, far_n: flo
         bucket_to_tile = torch.empty((nb,), dtype=torch.int32, device=dev)
         sampled_T = torch.empty((nb, _TILE * _TILE), **opt)
         sampled_acc = torch.empty((nb, 3, _TILE * _TILE), **opt)
-        sampled_aux = torch.empty((nb, 8, _TILE * _TILE), **opt)
+        sampled_aux = torch.empty((nb, 10 if flow else 8, _TILE * _TILE), **opt)
         outputs += [max_contrib, bucket_to_tile[:B], sampled_T[:B], sampled_acc[:B], sampled_aux[:B]]
     if P == 0:
         return outputs
@@ -661,11 +664,11 @@ def GS_2D_fast_render_forward(width: int, height: int, near_n: float, far_n: flo
         rc = _lib().fsgs_gs_2d_fast_render_forward(
             P, width, height, float(near_n), float(far_n), int(bool(only_image)), L.ptr(means2D.contiguous()),
             L.ptr(colors.contiguous()), L.ptr(normal_opacity.contiguous()), L.ptr(trans_mat), L.ptr(inverse_m),
-            L.ptr(point_list.contiguous()), L.ptr(ranges.contiguous()), L.ptr(accum_max_count),
-            L.ptr(accum_weights_p), L.ptr(accum_weights_count),
+            L.ptr(point_list.contiguous()), L.ptr(ranges.contiguous()), L.ptr(trans_mat_t2) if flow else None,
+            L.ptr(accum_max_count), L.ptr(accum_weights_p), L.ptr(accum_weights_count),
             L.ptr(per_tile_bucket_offset) if (fast_bwd and not only_image) else None, L.ptr(pixel_colors),
-            L.ptr(pixel_opacity), L.ptr(pixel_extras), L.ptr(n_contrib), L.ptr(max_contrib), L.ptr(bucket_to_tile),
-            L.ptr(sampled_T), L.ptr(sampled_acc), L.ptr(sampled_aux), L.current_stream())
+            L.ptr(pixel_opacity), L.ptr(pixel_extras), L.ptr(pixel_flow), L.ptr(n_contrib), L.ptr(max_contrib),
+            L.ptr(bucket_to_tile), L.ptr(sampled_T), L.ptr(sampled_acc), L.ptr(sampled_aux), L.current_stream())
     L.check(rc, what)
     return outputs
 
@@ -677,10 +680,9 @@ def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inver
                                sampled_acc=None, sampled_aux=None):
     """gs_2d_fast_redner.cu:955-1074 -> [dL_dcolors[P,3], dL_dmeans2D[P,2], dL_dtrans_m[P,3,3], dL_dinverse_m[P,3,3],
     dL_dnorm_op[P,4]]. Passing per_tile_bucket_offset selects the per-splat channel set of the reference's second
-    kernel; the snapshot tensors themselves are not needed to evaluate it here."""
+    kernel; the snapshot tensors themselves are not needed to evaluate it here. With dL_dout_flow (and trans_mat2,
+    out_flows) the optical-flow gradient is added as the reference's kernels add it."""
     what = 'GS_2D_fast_render_backward'
-    if dL_dout_flow is not None:
-        raise RuntimeError(f'{what}: optical flow gradients are not supported on the fast path')
     L.require_cuda(what, dL_dout_color=dL_dout_color, dL_dout_opacity=dL_dout_opacity, dL_dothers=dL_dothers)
     P = means2D.shape[0]
     H, W = dL_dout_color.shape[1], dL_dout_color.shape[2]
@@ -698,13 +700,23 @@ def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inver
     ranges, point_list, n_contrib, out_others = c(ranges), c(point_list), c(n_contrib), c(out_others)
     use_aux = out_others is not None and dL_dothers is not None
     per_splat = per_tile_bucket_offset is not None
+    flow = dL_dout_flow is not None
+    if flow:
+        if not use_aux or trans_mat2 is None or out_flows is None:
+            raise RuntimeError(f'{what}: dL_dout_flow needs trans_mat2, out_flows, out_others and dL_dothers')
+        trans_mat2, out_flows, dL_dout_flow = c(trans_mat2), c(out_flows), c(dL_dout_flow)
+        _f32(what, trans_mat2=trans_mat2, out_flows=out_flows, dL_dout_flow=dL_dout_flow)
+        L.require_shape(what, 'trans_mat2', trans_mat2, P, 3, 3)
+        L.require_shape(what, 'out_flows', out_flows, H, W, 2)
+        L.require_shape(what, 'dL_dout_flow', dL_dout_flow, H, W, 2)
     with _timed('gs_2d_fast_render_backward'):
         rc = _lib().fsgs_gs_2d_fast_render_backward(
             P, W, H, float(near_n), float(far_n), int(per_splat), L.ptr(means2D), L.ptr(normal_opacity), L.ptr(colors),
-            L.ptr(trans_mat), L.ptr(inverse_m), L.ptr(out_opacity), L.ptr(out_others) if use_aux else None,
-            L.ptr(dL_dout_color), L.ptr(dL_dout_opacity), L.ptr(dL_dothers) if use_aux else None, L.ptr(ranges),
-            L.ptr(point_list), L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_inv),
-            L.ptr(g_norm_op), L.current_stream())
+            L.ptr(trans_mat), L.ptr(inverse_m), L.ptr(trans_mat2) if flow else None, L.ptr(out_opacity),
+            L.ptr(out_others) if use_aux else None, L.ptr(out_flows) if flow else None, L.ptr(dL_dout_color),
+            L.ptr(dL_dout_opacity), L.ptr(dL_dothers) if use_aux else None, L.ptr(dL_dout_flow) if flow else None,
+            L.ptr(ranges), L.ptr(point_list), L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans),
+            L.ptr(g_inv), L.ptr(g_norm_op), L.current_stream())
     L.check(rc, what)
     return [g_colors, g_means2D, g_trans, g_inv, g_norm_op]
 

@@ -9,7 +9,10 @@
 // its result is the same derivative with a different set of live channels (no distortion gradient, M1/M2 maps as
 // plain weighted sums with the M1 depth term overwritten, :751-757). Here both forms run the same tile-per-block
 // back-to-front kernel and differ only in that channel set; the snapshots are still produced by the forward for callers
-// that consume them. Optical flow is not supported on this path.
+// that consume them. Optical flow (a second set of transforms, :247-255): the forward divides the weighted sum of
+// displacements by the final opacity (:259-263); both backward forms take dL/dflow as the gradient of the UNDIVIDED sum
+// (:366, :704), and the per-splat form subtracts the DIVIDED final flow from its partial sums (:706), which amounts to
+// an opacity-map gradient lowered by (final flow . dL/dflow) -- reproduced here in that algebraic form.
 //
 // Layout as in the standard blend: one 256-lane block per tile, wavefront w owns an 8x8 quadrant, surfels staged 256 at
 // a time in LDS (64-byte hot record with the adjugate, 32-byte cold record), per-quadrant work lists from a
@@ -112,20 +115,23 @@ __device__ __forceinline__ float wave_sum8_transposed(const float (&v)[8]) {
   return cross_row_sum(z);
 }
 
-template <bool kAux, bool kSnap, bool kAccum>
+template <bool kAux, bool kSnap, bool kAccum, bool kFlow>
 __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
     int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const float2* __restrict__ means2D, const float* __restrict__ colors, const float* __restrict__ trans_mat,
     const float* __restrict__ inverse_m, const float4* __restrict__ normal_opacity,
-    const int64_t* __restrict__ bucket_offset, int32_t* __restrict__ n_contrib, float* __restrict__ out_color,
-    float* __restrict__ out_opacity, float* __restrict__ out_extras, int32_t* __restrict__ max_contrib,
+    const float* __restrict__ trans_mat_t2, const int64_t* __restrict__ bucket_offset, int32_t* __restrict__ n_contrib,
+    float* __restrict__ out_color, float* __restrict__ out_opacity, float* __restrict__ out_extras,
+    float2* __restrict__ out_flow, int32_t* __restrict__ max_contrib,
     int32_t* __restrict__ bucket_to_tile, float* __restrict__ sampled_T, float* __restrict__ sampled_acc,
     float* __restrict__ sampled_aux, int32_t* __restrict__ accum_max_count, float* __restrict__ accum_weights_p,
     int32_t* __restrict__ accum_weights_count) {
   __shared__ FastHot s_hot[kBatch];
   __shared__ SplatCold s_cold[kBatch];
+  __shared__ float s_t2[kFlow ? kBatch * 9 : 1];  // second-time-step transforms of the staged surfels
   __shared__ unsigned char s_mask[kBatch];
   __shared__ int s_max_contrib;
+  constexpr int kNum = kFlow ? 10 : 8;  // channels of a snapshot
 
   const int gx = (W + kTile - 1) / kTile;
   const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
@@ -153,14 +159,21 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
   bool done = !inside;
   const float far_scale = far_n / (far_n - near_n);
   float T = 1.0f, C0 = 0, C1 = 0, C2 = 0;
-  float N0 = 0, N1 = 0, N2 = 0, D = 0, M1 = 0, M2 = 0, dist = 0, median = 0;
+  float N0 = 0, N1 = 0, N2 = 0, D = 0, M1 = 0, M2 = 0, dist = 0, median = 0, f0 = 0, f1 = 0;
   int last = 0, median_c = -1, wmax_id = -1;
   float wmax = 0;
   bool flag  = false;
 
   FastSplat next;
-  if ((int) threadIdx.x < n_todo)
-    next = gather_fast(point_list[r0 + threadIdx.x], means2D, colors, normal_opacity, trans_mat, inverse_m);
+  float next_t2[9];
+  if ((int) threadIdx.x < n_todo) {
+    const int id = point_list[r0 + threadIdx.x];
+    next = gather_fast(id, means2D, colors, normal_opacity, trans_mat, inverse_m);
+    if (kFlow) {
+#pragma unroll
+      for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) id + k];
+    }
+  }
 
   for (int b = 0; b < rounds; ++b) {
     if (__syncthreads_count(done) == kBlendThreads) break;
@@ -169,11 +182,21 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
       s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
       s_mask[threadIdx.x] = (unsigned char) fast_quadrant_mask(next, tile_x * kTile, tile_y * kTile, ordered);
+      if (kFlow) {
+#pragma unroll
+        for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
+      }
     }
     __syncthreads();
     const int nxt = (b + 1) * kBatch + (int) threadIdx.x;
-    if (nxt < n_todo)
-      next = gather_fast(point_list[r0 + nxt], means2D, colors, normal_opacity, trans_mat, inverse_m);
+    if (nxt < n_todo) {
+      const int id = point_list[r0 + nxt];
+      next = gather_fast(id, means2D, colors, normal_opacity, trans_mat, inverse_m);
+      if (kFlow) {
+#pragma unroll
+        for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) id + k];
+      }
+    }
 
     for (int c = 0; c < kBatch / kWave; ++c) {
       const int jj = c * kWave + lane;
@@ -191,13 +214,17 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
             sampled_acc[(bk * 3 + 1) * 256 + rank] = C1;
             sampled_acc[(bk * 3 + 2) * 256 + rank] = C2;
             if (kAux) {
-              sampled_aux[(bk * 8 + 0) * 256 + rank] = D;
-              sampled_aux[(bk * 8 + 1) * 256 + rank] = N0;
-              sampled_aux[(bk * 8 + 2) * 256 + rank] = N1;
-              sampled_aux[(bk * 8 + 3) * 256 + rank] = N2;
-              sampled_aux[(bk * 8 + 5) * 256 + rank] = dist;
-              sampled_aux[(bk * 8 + 6) * 256 + rank] = M1;
-              sampled_aux[(bk * 8 + 7) * 256 + rank] = M2;
+              sampled_aux[(bk * kNum + 0) * 256 + rank] = D;
+              sampled_aux[(bk * kNum + 1) * 256 + rank] = N0;
+              sampled_aux[(bk * kNum + 2) * 256 + rank] = N1;
+              sampled_aux[(bk * kNum + 3) * 256 + rank] = N2;
+              sampled_aux[(bk * kNum + 5) * 256 + rank] = dist;
+              sampled_aux[(bk * kNum + 6) * 256 + rank] = M1;
+              sampled_aux[(bk * kNum + 7) * 256 + rank] = M2;
+              if (kFlow) {
+                sampled_aux[(bk * kNum + 8) * 256 + rank] = f0;
+                sampled_aux[(bk * kNum + 9) * 256 + rank] = f1;
+              }
             }
           }
           todo &= half ? 0xffffffff00000000ull : 0x00000000ffffffffull;
@@ -230,6 +257,15 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
               if (accum_weights_p) atomicAdd(&accum_weights_p[cold.id], w);
               if (accum_weights_count) atomicAdd(&accum_weights_count[cold.id], 1);
             }
+            if (kFlow) {
+              const float* Q = &s_t2[j * 9];
+              const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
+              const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
+              float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
+              w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
+              f0 += (u2 / w2 - pxf) * w;
+              f1 += (v2 / w2 - pyf) * w;
+            }
           }
           if (kAccum) {
             if (flag && accum_max_count) atomicAdd(&accum_max_count[wmax_id], 1);
@@ -258,6 +294,10 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
       out_extras[pix + 5 * HW] = dist;
       out_extras[pix + 6 * HW] = M1;
       out_extras[pix + 7 * HW] = M2;
+      if (kFlow) {
+        const float A = 1.0f - T;
+        out_flow[pix] = A > 0.0f ? make_float2(f0 / A, f1 / A) : make_float2(0.0f, 0.0f);
+      }
     }
   }
   if (kSnap) {
@@ -275,18 +315,21 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
 // 19-20 means2D.
 constexpr int kFastGradSlots = 21;
 
-template <bool kAux, bool kPerSplat>
+template <bool kAux, bool kPerSplat, bool kFlow>
 __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
     int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const int32_t* __restrict__ n_contrib, const float2* __restrict__ means2D,
     const float4* __restrict__ normal_opacity, const float* __restrict__ colors, const float* __restrict__ trans_mat,
-    const float* __restrict__ inverse_m, const float* __restrict__ out_opacity, const float* __restrict__ out_extras,
+    const float* __restrict__ inverse_m, const float* __restrict__ trans_mat_t2, const float* __restrict__ out_opacity,
+    const float* __restrict__ out_extras, const float2* __restrict__ out_flow,
     const float* __restrict__ dL_dpix, const float* __restrict__ dL_dextras, const float* __restrict__ dL_dopacity,
+    const float2* __restrict__ dL_dflow,
     float* __restrict__ g_means2D, float* __restrict__ g_normal_opacity, float* __restrict__ g_colors,
     float* __restrict__ g_trans, float* __restrict__ g_inv) {
   constexpr int kB = 64;  // surfels staged per round
   __shared__ FastHot s_hot[kB];
   __shared__ SplatCold s_cold[kB];
+  __shared__ float s_t2[kFlow ? kB * 9 : 1];
   // each wavefront's sums per staged surfel, written once per entry with a plain store and added in wavefront order at
   // the flush (LDS float atomics cost about three cycles per lane)
   __shared__ float s_part[4][kB][kFastGradSlots];
@@ -322,7 +365,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
   float T = T_final;
   float dLp0 = 0, dLp1 = 0, dLp2 = 0;
   float dL_dreg = 0, dL_ddepth = 0, dL_daccum = 0, dLn0 = 0, dLn1 = 0, dLn2 = 0, dL_dmedian = 0, dL_dM1 = 0, dL_dM2 = 0;
-  float final_D = 0, final_D2 = 0;
+  float final_D = 0, final_D2 = 0, dLf0 = 0, dLf1 = 0;
   if (inside) {
     dLp0 = dL_dpix[pix], dLp1 = dL_dpix[pix + HW], dLp2 = dL_dpix[pix + 2 * HW];
     if (kAux) {
@@ -339,6 +382,16 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
     } else if (kPerSplat) {
       dL_daccum = dL_dopacity[pix];
     }
+    if (kFlow) {
+      const float2 gf = dL_dflow[pix];
+      dLf0 = gf.x, dLf1 = gf.y;
+      if (kPerSplat) {
+        // partial sum - DIVIDED final flow  ==  -(sum over later entries) - final flow * T_final: the second part acts
+        // like the opacity map's gradient (both carry T_final / (1 - alpha) per entry)
+        const float2 ff = out_flow[pix];
+        dL_daccum -= ff.x * gf.x + ff.y * gf.y;
+      }
+    }
   }
   const float final_A   = 1.0f - T_final;
   const float far_scale = far_n / (far_n - near_n);
@@ -347,9 +400,15 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
   float last_dL_dT = 0, last_alpha = 0;
 
   FastSplat next;
-  if ((int) threadIdx.x < min(n_todo, kB))
-    next = gather_fast(point_list[r0 + (n_todo - 1 - (int) threadIdx.x)], means2D, colors, normal_opacity, trans_mat,
-                       inverse_m);
+  float next_t2[9];
+  if ((int) threadIdx.x < min(n_todo, kB)) {
+    const int id = point_list[r0 + (n_todo - 1 - (int) threadIdx.x)];
+    next = gather_fast(id, means2D, colors, normal_opacity, trans_mat, inverse_m);
+    if (kFlow) {
+#pragma unroll
+      for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) id + k];
+    }
+  }
 
   for (int b = 0; b < rounds; ++b) {
     const int n_here = min(kB, n_todo - b * kB);
@@ -357,11 +416,21 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
       s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
       s_mask[threadIdx.x] = (unsigned char) fast_quadrant_mask(next, tile_x * kTile, tile_y * kTile, ordered);
+      if (kFlow) {
+#pragma unroll
+        for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
+      }
     }
     __syncthreads();
     const int nxt = (b + 1) * kB + (int) threadIdx.x;
-    if ((int) threadIdx.x < kB && nxt < n_todo)
-      next = gather_fast(point_list[r0 + (n_todo - 1 - nxt)], means2D, colors, normal_opacity, trans_mat, inverse_m);
+    if ((int) threadIdx.x < kB && nxt < n_todo) {
+      const int id = point_list[r0 + (n_todo - 1 - nxt)];
+      next = gather_fast(id, means2D, colors, normal_opacity, trans_mat, inverse_m);
+      if (kFlow) {
+#pragma unroll
+        for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) id + k];
+      }
+    }
 
     for (int chunk = 0; chunk < kB / kWave; ++chunk) {
       const int jj = chunk * kWave + lane;
@@ -411,6 +480,20 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
             dL_dz += w * dL_ddepth;
           }
           if (kAux || kPerSplat) c_lin += dL_daccum;
+          float fsx = 0.0f, fsy = 0.0f;  // dL/d(intersection) through the second transform
+          if (kFlow) {
+            const float* Q = &s_t2[j * 9];
+            const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
+            const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
+            float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
+            w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
+            const float rw = 1.0f / w2;
+            c_lin += (u2 * rw - pxf) * dLf0 + (v2 * rw - pyf) * dLf1;
+            const float gu = w * rw * dLf0, gv = w * rw * dLf1;
+            const float gw = -w * rw * rw * (u2 * dLf0 + v2 * dLf1);
+            fsx = Q[0] * gu + Q[3] * gv + Q[6] * gw;
+            fsy = Q[1] * gu + Q[4] * gv + Q[7] * gw;
+          }
           acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
           last_lin = c_lin;
           dL_dalpha += c_lin - acc_lin;
@@ -419,8 +502,8 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
 
           const float dL_dG = hot.opacity * dL_dalpha;
           if (h.rho3d <= h.rho2d) {
-            const float dsx = dL_dG * -h.G * h.sx + dL_dz * hot.tw0;
-            const float dsy = dL_dG * -h.G * h.sy + dL_dz * hot.tw1;
+            const float dsx = fsx + dL_dG * -h.G * h.sx + dL_dz * hot.tw0;
+            const float dsy = fsy + dL_dG * -h.G * h.sy + dL_dz * hot.tw1;
             const float rz  = __builtin_amdgcn_rcpf(h.pz);
             const float da = dsx * rz, db = dsy * rz;
             const float dc = -(da * h.sx + db * h.sy);
@@ -483,10 +566,11 @@ using namespace fsgs;
 
 FSGS_API int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, double far_n, int only_image,
     const float* means2D, const float* colors, const float* normal_opacity, const float* trans_mat,
-    const float* inverse_m, const int32_t* point_list, const int64_t* ranges, int32_t* accum_max_count,
-    float* accum_weights_p, int32_t* accum_weights_count, const int64_t* bucket_offset, float* out_color,
-    float* out_opacity, float* out_extras, int32_t* n_contrib, int32_t* max_contrib, int32_t* bucket_to_tile,
-    float* sampled_T, float* sampled_acc, float* sampled_aux, void* stream) {
+    const float* inverse_m, const int32_t* point_list, const int64_t* ranges, const float* trans_mat_t2,
+    int32_t* accum_max_count, float* accum_weights_p, int32_t* accum_weights_count, const int64_t* bucket_offset,
+    float* out_color, float* out_opacity, float* out_extras, float* out_flow, int32_t* n_contrib,
+    int32_t* max_contrib, int32_t* bucket_to_tile, float* sampled_T, float* sampled_acc, float* sampled_aux,
+    void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_fast_render_forward: bad sizes");
   FSGS_REQUIRE(ranges && out_color && out_opacity && n_contrib, "GS_2D_fast_render_forward: null pointer");
   FSGS_REQUIRE(P == 0 || (means2D && colors && normal_opacity && trans_mat && inverse_m),
@@ -495,52 +579,63 @@ FSGS_API int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, 
   const bool aux   = !only_image;
   const bool snap  = aux && bucket_offset != nullptr;
   const bool accum = aux && (accum_max_count || accum_weights_p || accum_weights_count);
+  const bool flow  = aux && trans_mat_t2 != nullptr;
+  FSGS_REQUIRE(!flow || out_flow, "GS_2D_fast_render_forward: out_flow is required with trans_mat_t2");
   FSGS_REQUIRE(!snap || (max_contrib && bucket_to_tile && sampled_T && sampled_acc && sampled_aux),
                "GS_2D_fast_render_forward: snapshot outputs are required with per_tile_bucket_offset");
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
   const int ordered = launch_tile_order(gx, gy, ranges, s);
-#define FSGS_LAUNCH_FWD(AUX, SNAP, ACC)                                                                              \
-  hipLaunchKernelGGL((fast_blend_forward_kernel<AUX, SNAP, ACC>), grid, block, 0, s, ordered, W, H, (float) near_n,           \
-                     (float) far_n, ranges, point_list, (const float2*) means2D, colors, trans_mat, inverse_m,       \
-                     (const float4*) normal_opacity, bucket_offset, n_contrib, out_color, out_opacity, out_extras,   \
-                     max_contrib, bucket_to_tile, sampled_T, sampled_acc, sampled_aux, accum_max_count,              \
-                     accum_weights_p, accum_weights_count)
-  if (!aux) FSGS_LAUNCH_FWD(false, false, false);
-  else if (snap && accum) FSGS_LAUNCH_FWD(true, true, true);
-  else if (snap) FSGS_LAUNCH_FWD(true, true, false);
-  else if (accum) FSGS_LAUNCH_FWD(true, false, true);
-  else FSGS_LAUNCH_FWD(true, false, false);
+#define FSGS_LAUNCH_FWD(AUX, SNAP, ACC, FLOW)                                                                        \
+  hipLaunchKernelGGL((fast_blend_forward_kernel<AUX, SNAP, ACC, FLOW>), grid, block, 0, s, ordered, W, H,            \
+                     (float) near_n, (float) far_n, ranges, point_list, (const float2*) means2D, colors, trans_mat,  \
+                     inverse_m, (const float4*) normal_opacity, trans_mat_t2, bucket_offset, n_contrib, out_color,   \
+                     out_opacity, out_extras, (float2*) out_flow, max_contrib, bucket_to_tile, sampled_T,            \
+                     sampled_acc, sampled_aux, accum_max_count, accum_weights_p, accum_weights_count)
+#define FSGS_LAUNCH_FWD_F(AUX, SNAP, ACC) \
+  do { if (flow) FSGS_LAUNCH_FWD(AUX, SNAP, ACC, true); else FSGS_LAUNCH_FWD(AUX, SNAP, ACC, false); } while (0)
+  if (!aux) FSGS_LAUNCH_FWD(false, false, false, false);
+  else if (snap && accum) FSGS_LAUNCH_FWD_F(true, true, true);
+  else if (snap) FSGS_LAUNCH_FWD_F(true, true, false);
+  else if (accum) FSGS_LAUNCH_FWD_F(true, false, true);
+  else FSGS_LAUNCH_FWD_F(true, false, false);
+#undef FSGS_LAUNCH_FWD_F
 #undef FSGS_LAUNCH_FWD
   return check_launch("GS_2D_fast_render_forward");
 }
 
 FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n, double far_n, int per_splat_form,
     const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,
-    const float* inverse_m, const float* out_opacity, const float* out_extras, const float* dL_dpix,
-    const float* dL_dopacity, const float* dL_dextras, const int64_t* ranges, const int32_t* point_list,
-    const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans, float* g_inv,
-    float* g_normal_opacity, void* stream) {
+    const float* inverse_m, const float* trans_mat_t2, const float* out_opacity, const float* out_extras,
+    const float* out_flow, const float* dL_dpix, const float* dL_dopacity, const float* dL_dextras,
+    const float* dL_dflow, const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib,
+    float* g_colors, float* g_means2D, float* g_trans, float* g_inv, float* g_normal_opacity, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_fast_render_backward: bad sizes");
   if (P == 0) return kOk;
   FSGS_REQUIRE(means2D && normal_opacity && colors && trans_mat && inverse_m && out_opacity && dL_dpix && dL_dopacity &&
                    ranges && n_contrib && g_colors && g_means2D && g_trans && g_inv && g_normal_opacity,
                "GS_2D_fast_render_backward: null pointer");
-  const bool aux = out_extras && dL_dextras;
+  const bool aux  = out_extras && dL_dextras;
+  const bool flow = dL_dflow != nullptr;
+  FSGS_REQUIRE(!flow || (aux && trans_mat_t2 && out_flow),
+               "GS_2D_fast_render_backward: flow gradients need trans_mat2, out_flows and the auxiliary maps");
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
   const int ordered = launch_tile_order(gx, gy, ranges, s);
-#define FSGS_LAUNCH_BWD(AUX, SPLAT)                                                                                  \
-  hipLaunchKernelGGL((fast_blend_backward_kernel<AUX, SPLAT>), grid, block, 0, s, ordered, W, H, (float) near_n,              \
-                     (float) far_n, ranges, point_list, n_contrib, (const float2*) means2D,                          \
-                     (const float4*) normal_opacity, colors, trans_mat, inverse_m, out_opacity, out_extras, dL_dpix, \
-                     dL_dextras, dL_dopacity, g_means2D, g_normal_opacity, g_colors, g_trans, g_inv)
-  if (aux && per_splat_form) FSGS_LAUNCH_BWD(true, true);
-  else if (aux) FSGS_LAUNCH_BWD(true, false);
-  else if (per_splat_form) FSGS_LAUNCH_BWD(false, true);
-  else FSGS_LAUNCH_BWD(false, false);
+#define FSGS_LAUNCH_BWD(AUX, SPLAT, FLOW)                                                                            \
+  hipLaunchKernelGGL((fast_blend_backward_kernel<AUX, SPLAT, FLOW>), grid, block, 0, s, ordered, W, H,               \
+                     (float) near_n, (float) far_n, ranges, point_list, n_contrib, (const float2*) means2D,          \
+                     (const float4*) normal_opacity, colors, trans_mat, inverse_m, trans_mat_t2, out_opacity,        \
+                     out_extras, (const float2*) out_flow, dL_dpix, dL_dextras, dL_dopacity,                         \
+                     (const float2*) dL_dflow, g_means2D, g_normal_opacity, g_colors, g_trans, g_inv)
+  if (aux && per_splat_form && flow) FSGS_LAUNCH_BWD(true, true, true);
+  else if (aux && flow) FSGS_LAUNCH_BWD(true, false, true);
+  else if (aux && per_splat_form) FSGS_LAUNCH_BWD(true, true, false);
+  else if (aux) FSGS_LAUNCH_BWD(true, false, false);
+  else if (per_splat_form) FSGS_LAUNCH_BWD(false, true, false);
+  else FSGS_LAUNCH_BWD(false, false, false);
 #undef FSGS_LAUNCH_BWD
   return check_launch("GS_2D_fast_render_backward");
 }

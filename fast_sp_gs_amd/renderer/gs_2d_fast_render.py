@@ -94,15 +94,17 @@ class _fast_rasterize(torch.autograd.Function):
         ctx._info = (near_n, far_n)
         ctx._snap = (offset, *outs[5:]) if offset is not None and len(outs) > 5 else None
         ctx.save_for_backward(means2D, normal_opacity, trans_mat, inverse_m, colors, pixel_colors, pixel_extras,
-                              pixel_opacity, tile_range, point_list, n_contrib)
+                              pixel_opacity, tile_range, point_list, n_contrib, trans_mat_t2, pixel_flow)
         ctx.mark_non_differentiable(n_contrib)
         return pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib
 
     @classmethod
     def _backward(cls, ctx, grad_outputs):
         (means2D, normal_opacity, trans_mat, inverse_m, colors, pixel_colors, pixel_extras, pixel_opacity, tile_range,
-         point_list, n_contrib) = ctx.saved_tensors
+         point_list, n_contrib, trans_mat_t2, pixel_flow) = ctx.saved_tensors
         grad_images, grad_opacity, grad_others, grad_flow, _ = grad_outputs
+        if pixel_flow is None or grad_others is None:
+            grad_flow = None
         if grad_images is None:
             grad_images = torch.zeros_like(pixel_colors)
         if grad_opacity is None:
@@ -113,8 +115,9 @@ class _fast_rasterize(torch.autograd.Function):
         else:
             snap = (None,) * 6
         grad_colors, grad_means2D, grad_trans, grad_inv_m, grad_normal_opacity = cls._backward_func(
-            means2D, normal_opacity, colors, trans_mat, inverse_m, None, pixel_colors, pixel_opacity, pixel_extras,
-            None, grad_images, grad_opacity, grad_others, None, tile_range, point_list, n_contrib, *ctx._info, *snap)
+            means2D, normal_opacity, colors, trans_mat, inverse_m, trans_mat_t2, pixel_colors, pixel_opacity,
+            pixel_extras, pixel_flow, grad_images, grad_opacity, grad_others, grad_flow, tile_range, point_list,
+            n_contrib, *ctx._info, *snap)
         grad_inputs = [None] * 16
         grad_inputs[2] = grad_means2D
         grad_inputs[3] = grad_colors
@@ -186,7 +189,7 @@ class _Fast_Render(torch.autograd.Function):
         ctx._info = (W, H, sh_degree, is_opengl, near_n, far_n)
         ctx.save_for_backward(means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, Tv2s, campos,
                               means2D, trans_mat, inverse_m, radii, colors, normal_opacity, tile_range, point_list,
-                              pixel_colors, pixel_extras, pixel_opacity, n_contrib)
+                              pixel_colors, pixel_extras, pixel_opacity, n_contrib, trans_mat_t2, pixel_flow)
         ctx.mark_non_differentiable(n_contrib, radii)
         return pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib, radii
 
@@ -195,17 +198,19 @@ class _Fast_Render(torch.autograd.Function):
     def backward(ctx, *grad_outputs):
         (means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, Tv2s, campos, means2D, trans_mat,
          inverse_m, radii, colors, normal_opacity, tile_range, point_list, pixel_colors, pixel_extras, pixel_opacity,
-         n_contrib) = ctx.saved_tensors
+         n_contrib, trans_mat_t2, pixel_flow) = ctx.saved_tensors
         W, H, sh_degree, is_opengl, near_n, far_n = ctx._info
-        grad_images, grad_opacity, grad_others = grad_outputs[:3]
+        grad_images, grad_opacity, grad_others, grad_flow = grad_outputs[:4]
+        if pixel_flow is None or grad_others is None:
+            grad_flow = None
         if grad_images is None:
             grad_images = torch.zeros_like(pixel_colors)
         if grad_opacity is None:
             grad_opacity = torch.zeros_like(pixel_opacity)
         grad_colors, grad_means2D, grad_trans, grad_inv_m, grad_normal_opacity = _Fast_Render._render_backward(
-            means2D, normal_opacity, colors, trans_mat, inverse_m, None, pixel_colors, pixel_opacity, pixel_extras, None,
-            grad_images, grad_opacity, grad_others, None, tile_range, point_list, n_contrib, near_n, far_n,
-            None, None, None, None, None, None)
+            means2D, normal_opacity, colors, trans_mat, inverse_m, trans_mat_t2, pixel_colors, pixel_opacity,
+            pixel_extras, pixel_flow, grad_images, grad_opacity, grad_others, grad_flow, tile_range, point_list,
+            n_contrib, near_n, far_n, None, None, None, None, None, None)
         grad_inputs = [
             torch.zeros_like(means3D), torch.zeros_like(scales), torch.zeros_like(rotations),
             torch.zeros_like(opacities),

@@ -175,25 +175,32 @@ int fsgs_gs_2d_fast_compute_transmat_backward(int P, const float* means3D, const
     float* g_means3D, float* g_scales, float* g_rot, void* stream);
 
 /* GS_2D_fast_render_forward -- gs_2d_fast_redner.cu:839-953 (kernel :22-271). out_extras[8,H,W]. With
- * bucket_offset[T] (inclusive cumsum of ceil(len/32) per tile) the kernel also writes max_contrib[T],
- * bucket_to_tile[B], sampled_T[B,256], sampled_acc[B,3,256], sampled_aux[B,8,256] (state before every 32nd list
- * entry, for pixels still blending; channel 4 of sampled_aux is never written, as in the reference). */
+ * trans_mat_t2[P,3,3] (optional, not with only_image) out_flow[H,W,2] is the weighted displacement to the second time
+ * step divided by the final opacity, 0 where that is 0 (:247-263). With bucket_offset[T] (inclusive cumsum of
+ * ceil(len/32) per tile) the kernel also writes max_contrib[T], bucket_to_tile[B], sampled_T[B,256],
+ * sampled_acc[B,3,256], sampled_aux[B,C,256] with C = 10 when trans_mat_t2 is given (channels 8, 9: the undivided flow
+ * sums) and 8 otherwise (state before every 32nd list entry, for pixels still blending; channel 4 of sampled_aux is
+ * never written, as in the reference). */
 int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, double far_n, int only_image,
     const float* means2D, const float* colors, const float* normal_opacity, const float* trans_mat,
-    const float* inverse_m, const int32_t* point_list, const int64_t* ranges, int32_t* accum_max_count,
-    float* accum_weights_p, int32_t* accum_weights_count, const int64_t* bucket_offset, float* out_color,
-    float* out_opacity, float* out_extras, int32_t* n_contrib, int32_t* max_contrib, int32_t* bucket_to_tile,
-    float* sampled_T, float* sampled_acc, float* sampled_aux, void* stream);
+    const float* inverse_m, const int32_t* point_list, const int64_t* ranges, const float* trans_mat_t2,
+    int32_t* accum_max_count, float* accum_weights_p, int32_t* accum_weights_count, const int64_t* bucket_offset,
+    float* out_color, float* out_opacity, float* out_extras, float* out_flow, int32_t* n_contrib,
+    int32_t* max_contrib, int32_t* bucket_to_tile, float* sampled_T, float* sampled_acc, float* sampled_aux,
+    void* stream);
 
 /* GS_2D_fast_render_backward -- gs_2d_fast_redner.cu:955-1074. per_splat_form = 0: kernel :273-561 (image, opacity,
  * aux 0-5); per_splat_form = 1: the channel set of kernel :563-837 (image, opacity, aux 0-4 and 6-7, no distortion).
- * All five gradient outputs MUST be zero-filled by the caller. */
+ * dL_dflow[H,W,2] (optional, with trans_mat_t2 and out_flow) is taken as the gradient of the UNDIVIDED flow sum, as both
+ * reference kernels take it (:366, :704); the per-splat form additionally lowers the opacity map's gradient by
+ * (out_flow . dL_dflow), the effect of the reference subtracting the divided flow from its partial sums (:706). No
+ * gradient is produced for trans_mat_t2. All five gradient outputs MUST be zero-filled by the caller. */
 int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n, double far_n, int per_splat_form,
     const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,
-    const float* inverse_m, const float* out_opacity, const float* out_extras, const float* dL_dpix,
-    const float* dL_dopacity, const float* dL_dextras, const int64_t* ranges, const int32_t* point_list,
-    const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans, float* g_inv,
-    float* g_normal_opacity, void* stream);
+    const float* inverse_m, const float* trans_mat_t2, const float* out_opacity, const float* out_extras,
+    const float* out_flow, const float* dL_dpix, const float* dL_dopacity, const float* dL_dextras,
+    const float* dL_dflow, const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib,
+    float* g_colors, float* g_means2D, float* g_trans, float* g_inv, float* g_normal_opacity, void* stream);
 
 /* gs_2d_topk_weights -- fast_2d_gs/_C/src/gaussian_splatting/gaussian_topk.cu:230-250 (kernel :95-210).
  * top_indices[H,W,topk] int32 (-1 = empty), top_weights[H,W,topk] descending blend weights alpha*T; topk <= 16. */

@@ -210,33 +210,40 @@ def fast_preprocess_backward(W, H, sh_degree, means3D, scales, rotations, shs, s
 
 
 def fast_render_forward(W, H, near, far, only_image, means2D, colors, normal_opacity, trans_mat, inverse_m, point_list,
-                        ranges, bucket_offset=None):
+                        ranges, bucket_offset=None, trans_mat_t2=None, accum_max_count=None, accum_weights_p=None,
+                        accum_weights_count=None):
+    """-> (colors, opacity, extras[8], n_contrib, max_contrib, bucket_to_tile, sampled_T, sampled_acc, sampled_aux
+    [B, 8 | 10, 256]) and, when trans_mat_t2 is given, the flow [H,W,2] as a tenth element."""
     dt = means2D.dtype
     oc, oo = np.zeros((3, H, W), dt), np.zeros((H, W), dt)
     oe = None if only_image else np.zeros((8, H, W), dt)
+    flow = trans_mat_t2 is not None and not only_image
+    of = np.zeros((H, W, 2), dt) if flow else None
     nc = np.zeros((2, H, W), np.int32)
     snap = [None] * 5
     if bucket_offset is not None and not only_image:
         B = int(bucket_offset[-1])
         T = ranges.shape[0]
         snap = [np.zeros((T,), np.int32), np.zeros((B,), np.int32), np.zeros((B, 256), dt), np.zeros((B, 3, 256), dt),
-                np.zeros((B, 8, 256), dt)]
+                np.zeros((B, 10 if flow else 8, 256), dt)]
     rc = call(f"gs_2d_fast_render_forward_{_suffix(dt)}", W, H, float(near), float(far), int(only_image), means2D,
-              colors, normal_opacity, trans_mat, inverse_m, point_list, ranges, bucket_offset, oc, oo, oe, nc, *snap)
+              colors, normal_opacity, trans_mat, inverse_m, point_list, ranges, bucket_offset, trans_mat_t2,
+              accum_max_count, accum_weights_p, accum_weights_count, oc, oo, oe, of, nc, *snap)
     assert rc == 0
-    return (oc, oo, oe, nc) + tuple(snap)
+    return (oc, oo, oe, nc) + tuple(snap) + ((of,) if flow else ())
 
 
 def fast_render_backward(near, far, per_splat_form, means2D, normal_opacity, colors, trans_mat, inverse_m, out_opacity,
-                         out_extras, dL_dpix, dL_dopacity, dL_dextras, ranges, point_list, n_contrib):
+                         out_extras, dL_dpix, dL_dopacity, dL_dextras, ranges, point_list, n_contrib,
+                         trans_mat_t2=None, out_flow=None, dL_dflow=None):
     dt = means2D.dtype
     P = means2D.shape[0]
     H, W = dL_dpix.shape[1:]
     gc, gm, gt, gi, gn = (np.zeros((P, 3), dt), np.zeros((P, 2), dt), np.zeros((P, 3, 3), dt), np.zeros((P, 3, 3), dt),
                           np.zeros((P, 4), dt))
     rc = call(f"gs_2d_fast_render_backward_{_suffix(dt)}", P, W, H, float(near), float(far), int(per_splat_form),
-              means2D, normal_opacity, colors, trans_mat, inverse_m, out_opacity, out_extras, dL_dpix, dL_dopacity,
-              dL_dextras, ranges, point_list, n_contrib, gc, gm, gt, gi, gn)
+              means2D, normal_opacity, colors, trans_mat, inverse_m, trans_mat_t2, out_opacity, out_extras, out_flow,
+              dL_dpix, dL_dopacity, dL_dextras, dL_dflow, ranges, point_list, n_contrib, gc, gm, gt, gi, gn)
     assert rc == 0
     return gc, gm, gt, gi, gn
 

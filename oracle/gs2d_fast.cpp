@@ -295,18 +295,25 @@ static void fast_preprocess_backward(int P, int W, int H, int sh_degree, int n_s
 
 // gs_2d_fast_redner.cu:22-271. extras has 8 channels: depth, normal xyz, median depth, distortion, M1, M2.
 // Snapshot outputs (when bucket_offset != nullptr): state before every 32nd list entry, per pixel of the tile in
-// row-major (16 x 16) order, for pixels that are still blending.
+// row-major (16 x 16) order, for pixels that are still blending; sampled_aux has 8 channels, or 10 with optical flow
+// (channels 8, 9 = the unnormalised flow sums, :141-144). Optical flow (trans_mat_t2 given, :247-255) is normalised by
+// the final opacity, 0 where that is 0 (:259-263) -- the standard path divides by the sum of weights instead. The
+// accum_* side outputs are those of the standard path (:236-246, the arg-max flag is never reset).
 template <typename T>
 static void fast_render_forward(int W, int H, T near_n, T far_n, int only_image, const T* means2D, const T* colors,
                                 const T* normal_opacity, const T* trans_mat, const T* inverse_m,
                                 const int32_t* point_list, const int64_t* ranges, const int64_t* bucket_offset,
-                                T* out_color, T* out_opacity, T* out_extras, int32_t* n_contrib,
-                                int32_t* max_contrib, int32_t* bucket_to_tile, T* sampled_T, T* sampled_acc,
-                                T* sampled_aux) {
+                                const T* trans_mat_t2, int32_t* accum_max_count, T* accum_weights_p,
+                                int32_t* accum_weights_count, T* out_color, T* out_opacity, T* out_extras,
+                                T* out_flow, int32_t* n_contrib, int32_t* max_contrib, int32_t* bucket_to_tile,
+                                T* sampled_T, T* sampled_acc, T* sampled_aux) {
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const size_t HW = (size_t) H * W;
   const bool aux  = !only_image;
   const bool snap = aux && bucket_offset != nullptr;
+  const bool flow = aux && trans_mat_t2 != nullptr && out_flow != nullptr;
+  const int NUM   = flow ? 10 : 8;
+  const bool accum = accum_max_count || accum_weights_p || accum_weights_count;
   if (snap) {
     for (int t = 0; t < gx * gy; ++t) {
       const int64_t b0 = t == 0 ? 0 : bucket_offset[t - 1];
@@ -315,7 +322,8 @@ static void fast_render_forward(int W, int H, T near_n, T far_n, int only_image,
       max_contrib[t] = 0;
     }
   }
-#pragma omp parallel for schedule(dynamic, 1)
+  // the side outputs are sums over pixels of different tiles: serial when they are asked for
+#pragma omp parallel for schedule(dynamic, 1) if (!accum)
   for (int tile = 0; tile < gx * gy; ++tile) {
     const int tx = tile % gx, ty = tile / gx;
     const int64_t r0 = ranges[2 * tile], r1 = ranges[2 * tile + 1];
@@ -327,18 +335,22 @@ static void fast_render_forward(int W, int H, T near_n, T far_n, int only_image,
         const int rank   = ly * kTile + lx;
         const size_t pix = (size_t) W * py + px;
         const T pxf = (T) px, pyf = (T) py;
-        T t = 1, C[3] = {0}, N[3] = {0}, D = 0, M1 = 0, M2 = 0, dist = 0, med = 0;
+        T t = 1, C[3] = {0}, N[3] = {0}, D = 0, M1 = 0, M2 = 0, dist = 0, med = 0, fl[2] = {0, 0};
+        T wmax = 0;
+        int32_t wmax_id = -1;
+        bool flag = false;
         int32_t contributor = 0, last = 0, med_c = -1;
         int64_t bbm = snap ? (tile == 0 ? 0 : bucket_offset[tile - 1]) : 0;
         for (int64_t e = r0; e < r1; ++e) {
           if (snap && (e - r0) % 32 == 0) {
             sampled_T[bbm * 256 + rank] = t;
             for (int c = 0; c < 3; ++c) sampled_acc[(bbm * 3 + c) * 256 + rank] = C[c];
-            sampled_aux[(bbm * 8 + 0) * 256 + rank] = D;
-            for (int c = 0; c < 3; ++c) sampled_aux[(bbm * 8 + 1 + c) * 256 + rank] = N[c];
-            sampled_aux[(bbm * 8 + 5) * 256 + rank] = dist;
-            sampled_aux[(bbm * 8 + 6) * 256 + rank] = M1;
-            sampled_aux[(bbm * 8 + 7) * 256 + rank] = M2;
+            sampled_aux[(bbm * NUM + 0) * 256 + rank] = D;
+            for (int c = 0; c < 3; ++c) sampled_aux[(bbm * NUM + 1 + c) * 256 + rank] = N[c];
+            sampled_aux[(bbm * NUM + 5) * 256 + rank] = dist;
+            sampled_aux[(bbm * NUM + 6) * 256 + rank] = M1;
+            sampled_aux[(bbm * NUM + 7) * 256 + rank] = M2;
+            if (flow) sampled_aux[(bbm * NUM + 8) * 256 + rank] = fl[0], sampled_aux[(bbm * NUM + 9) * 256 + rank] = fl[1];
             ++bbm;
           }
           contributor++;
@@ -371,7 +383,20 @@ static void fast_render_forward(int W, int H, T near_n, T far_n, int only_image,
             M2 += m * m * w;
             if (t > 0.5) med = depth, med_c = contributor;
             for (int c = 0; c < 3; ++c) N[c] += no[c] * w;
+            if (wmax < w) wmax = w, wmax_id = id, flag = true;
+            if (accum_weights_p) accum_weights_p[id] += w;
+            if (accum_weights_count) accum_weights_count[id] += 1;
+            if (flow) {
+              const T* Q = trans_mat_t2 + 9 * (size_t) id;
+              const T u2 = Q[0] * s[0] + Q[1] * s[1] + Q[2];
+              const T v2 = Q[3] * s[0] + Q[4] * s[1] + Q[5];
+              T w2       = Q[6] * s[0] + Q[7] * s[1] + Q[8];
+              w2         = std::abs(w2) < 1e-5 ? T(1e-5) : w2;
+              fl[0] += (u2 / w2 - pxf) * w;
+              fl[1] += (v2 / w2 - pyf) * w;
+            }
           }
+          if (flag && accum_max_count) accum_max_count[wmax_id] += 1;
           for (int c = 0; c < 3; ++c) C[c] += colors[3 * (size_t) id + c] * w;
           t    = test_T;
           last = contributor;
@@ -387,6 +412,11 @@ static void fast_render_forward(int W, int H, T near_n, T far_n, int only_image,
           out_extras[pix + HW * 5] = dist;
           out_extras[pix + HW * 6] = M1;
           out_extras[pix + HW * 7] = M2;
+          if (flow) {
+            const T op = T(1) - t;
+            out_flow[2 * pix]     = op > 0 ? fl[0] / op : T(0);
+            out_flow[2 * pix + 1] = op > 0 ? fl[1] / op : T(0);
+          }
         }
         tile_max = std::max(tile_max, (int) last);
       }
@@ -396,17 +426,24 @@ static void fast_render_forward(int W, int H, T near_n, T far_n, int only_image,
 
 // gs_2d_fast_redner.cu:273-561 (per_splat_form == 0) and :563-837 (per_splat_form == 1, same derivative written as a
 // back-to-front recursion here; only the set of channels that carry gradient differs).
+// Optical flow (dL_dflow given): both kernels take dL_dflow as the gradient of the UNNORMALISED flow sum (no division by
+// the opacity the forward divided by, :366, :704) and send it to alpha and, through the second transform, to the
+// intersection (s.x, s.y) (:494-510, :765-782); no gradient goes to trans_mat_t2. The per-splat kernel forms "partial
+// sum up to and including this entry minus the total" with the NORMALISED out_flow as the total (:706); that is
+// restated literally here from a front-to-back pass over the pixel's contributors.
 template <typename T>
 static void fast_render_backward(int P, int W, int H, T near_n, T far_n, int per_splat_form, const T* means2D,
                                  const T* normal_opacity, const T* colors, const T* trans_mat, const T* inverse_m,
-                                 const T* out_opacity, const T* out_extras, const T* dL_dpix, const T* dL_dopacity,
-                                 const T* dL_dextras, const int64_t* ranges, const int32_t* point_list,
-                                 const int32_t* n_contrib, T* g_colors, T* g_means2D, T* g_trans, T* g_inv,
-                                 T* g_normal_opacity) {
+                                 const T* trans_mat_t2, const T* out_opacity, const T* out_extras, const T* out_flow,
+                                 const T* dL_dpix, const T* dL_dopacity, const T* dL_dextras, const T* dL_dflow,
+                                 const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib,
+                                 T* g_colors, T* g_means2D, T* g_trans, T* g_inv, T* g_normal_opacity) {
   const int gx = (W + kTile - 1) / kTile;
   const size_t HW = (size_t) H * W;
   const bool aux  = out_extras && dL_dextras;
+  const bool flow = dL_dflow != nullptr && trans_mat_t2 != nullptr;
   (void) P;
+  std::vector<T> pre_T, pre_P0, pre_P1;  // per list position of the current pixel (per-splat form with flow)
   for (int py = 0; py < H; ++py)
     for (int px = 0; px < W; ++px) {
       const size_t pix = (size_t) W * py + px;
@@ -437,6 +474,37 @@ static void fast_render_backward(int P, int W, int H, T near_n, T far_n, int per
       const T final_D2 = aux ? out_extras[pix + 7 * HW] : T(0);
       const T final_A  = 1 - t_final;
       T last_dL_dT = 0, last_alpha = 0;
+      T acc_f[2] = {0, 0}, last_f[2] = {0, 0}, gF[2] = {0, 0};
+      if (flow) gF[0] = dL_dflow[2 * pix], gF[1] = dL_dflow[2 * pix + 1];
+      if (flow && per_splat_form) {
+        // front-to-back: transmittance before each contributing entry and the flow sum up to and including it
+        pre_T.assign((size_t) (r1 - r0), T(0)), pre_P0.assign((size_t) (r1 - r0), T(0)),
+            pre_P1.assign((size_t) (r1 - r0), T(0));
+        T tt = 1, f0 = 0, f1 = 0;
+        for (int64_t e = r0; e < r0 + last_contributor; ++e) {
+          const int id = point_list[e];
+          const T* A   = inverse_m + 9 * (size_t) id;
+          const T* Mx  = trans_mat + 9 * (size_t) id;
+          const T p[3] = {A[0] * pxf + A[1] * pyf + A[2], A[3] * pxf + A[4] * pyf + A[5], A[6] * pxf + A[7] * pyf + A[8]};
+          if (p[2] == 0.0) continue;
+          const T s[2]  = {p[0] / p[2], p[1] / p[2]};
+          const T d[2]  = {means2D[2 * id] - pxf, means2D[2 * id + 1] - pyf};
+          const T rho   = std::min(s[0] * s[0] + s[1] * s[1], T(2.0) * (d[0] * d[0] + d[1] * d[1]));
+          if (s[0] * Mx[6] + s[1] * Mx[7] + Mx[8] < near_n) continue;
+          const T power = -T(0.5) * rho;
+          if (power > T(0.0)) continue;
+          const T alpha = std::min(T(0.99), normal_opacity[4 * (size_t) id + 3] * std::exp(power));
+          if (alpha < T(1.0 / 255.0)) continue;
+          const T* Q = trans_mat_t2 + 9 * (size_t) id;
+          T w2       = Q[6] * s[0] + Q[7] * s[1] + Q[8];
+          w2         = std::abs(w2) < 1e-5 ? T(1e-5) : w2;
+          pre_T[(size_t) (e - r0)] = tt;
+          f0 += alpha * tt * ((Q[0] * s[0] + Q[1] * s[1] + Q[2]) / w2 - pxf);
+          f1 += alpha * tt * ((Q[3] * s[0] + Q[4] * s[1] + Q[5]) / w2 - pyf);
+          pre_P0[(size_t) (e - r0)] = f0, pre_P1[(size_t) (e - r0)] = f1;
+          tt *= 1 - alpha;
+        }
+      }
       for (int64_t e = r1 - 1; e >= r0; --e) {
         contributor--;
         if (contributor >= (int64_t) last_contributor) continue;
@@ -499,7 +567,31 @@ static void fast_render_backward(int P, int W, int H, T near_n, T far_n, int per
           acc_alpha = last_alpha * T(1.0) + (T(1.) - last_alpha) * acc_alpha;
           dL_dalpha += (1 - acc_alpha) * g_acc;
         }
+        T flow_alpha = 0;  // the per-splat form's alpha term, already carrying its transmittance factors
+        if (flow) {
+          const T* Q = trans_mat_t2 + 9 * (size_t) id;
+          const T u2 = Q[0] * s[0] + Q[1] * s[1] + Q[2];
+          const T v2 = Q[3] * s[0] + Q[4] * s[1] + Q[5];
+          T w2       = Q[6] * s[0] + Q[7] * s[1] + Q[8];
+          w2         = std::abs(w2) < 1e-5 ? T(1e-5) : w2;
+          const T f[2] = {u2 / w2 - pxf, v2 / w2 - pyf};
+          if (!per_splat_form) {
+            for (int c = 0; c < 2; ++c) {
+              acc_f[c]  = last_alpha * last_f[c] + (T(1.) - last_alpha) * acc_f[c];
+              last_f[c] = f[c];
+              dL_dalpha += (f[c] - acc_f[c]) * gF[c];
+            }
+          } else {
+            const size_t k = (size_t) (e - r0);
+            flow_alpha = (f[0] * pre_T[k] + (pre_P0[k] - out_flow[2 * pix]) / (T(1.0) - alpha)) * gF[0] +
+                         (f[1] * pre_T[k] + (pre_P1[k] - out_flow[2 * pix + 1]) / (T(1.0) - alpha)) * gF[1];
+          }
+          const T gu = w / w2 * gF[0], gv = w / w2 * gF[1], gw = -w / (w2 * w2) * (u2 * gF[0] + v2 * gF[1]);
+          dL_dsx += Q[0] * gu + Q[3] * gv + Q[6] * gw;
+          dL_dsy += Q[1] * gu + Q[4] * gv + Q[7] * gw;
+        }
         dL_dalpha *= t;
+        dL_dalpha += flow_alpha;
         last_alpha    = alpha;
         const T dL_dG = no[3] * dL_dalpha;
         if (rho3d <= rho2d) {
@@ -570,22 +662,26 @@ using namespace oracle;
   }                                                                                                                  \
   ORACLE_API int oracle_gs_2d_fast_render_forward_##SUF(int W, int H, double near_n, double far_n, int only_image,   \
       const T* means2D, const T* colors, const T* normal_opacity, const T* trans_mat, const T* inverse_m,            \
-      const int32_t* point_list, const int64_t* ranges, const int64_t* bucket_offset, T* out_color, T* out_opacity,  \
-      T* out_extras, int32_t* n_contrib, int32_t* max_contrib, int32_t* bucket_to_tile, T* sampled_T,                \
+      const int32_t* point_list, const int64_t* ranges, const int64_t* bucket_offset, const T* trans_mat_t2,         \
+      int32_t* accum_max_count, T* accum_weights_p, int32_t* accum_weights_count, T* out_color, T* out_opacity,      \
+      T* out_extras, T* out_flow, int32_t* n_contrib, int32_t* max_contrib, int32_t* bucket_to_tile, T* sampled_T,   \
       T* sampled_acc, T* sampled_aux) {                                                                              \
     fast_render_forward<T>(W, H, (T) near_n, (T) far_n, only_image, means2D, colors, normal_opacity, trans_mat,      \
-                           inverse_m, point_list, ranges, bucket_offset, out_color, out_opacity, out_extras,         \
+                           inverse_m, point_list, ranges, bucket_offset, trans_mat_t2, accum_max_count,              \
+                           accum_weights_p, accum_weights_count, out_color, out_opacity, out_extras, out_flow,       \
                            n_contrib, max_contrib, bucket_to_tile, sampled_T, sampled_acc, sampled_aux);             \
     return 0;                                                                                                        \
   }                                                                                                                  \
   ORACLE_API int oracle_gs_2d_fast_render_backward_##SUF(int P, int W, int H, double near_n, double far_n,           \
       int per_splat_form, const T* means2D, const T* normal_opacity, const T* colors, const T* trans_mat,            \
-      const T* inverse_m, const T* out_opacity, const T* out_extras, const T* dL_dpix, const T* dL_dopacity,         \
-      const T* dL_dextras, const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib, T* g_colors,  \
-      T* g_means2D, T* g_trans, T* g_inv, T* g_normal_opacity) {                                                     \
+      const T* inverse_m, const T* trans_mat_t2, const T* out_opacity, const T* out_extras, const T* out_flow,       \
+      const T* dL_dpix, const T* dL_dopacity, const T* dL_dextras, const T* dL_dflow, const int64_t* ranges,         \
+      const int32_t* point_list, const int32_t* n_contrib, T* g_colors, T* g_means2D, T* g_trans, T* g_inv,          \
+      T* g_normal_opacity) {                                                                                         \
     fast_render_backward<T>(P, W, H, (T) near_n, (T) far_n, per_splat_form, means2D, normal_opacity, colors,         \
-                            trans_mat, inverse_m, out_opacity, out_extras, dL_dpix, dL_dopacity, dL_dextras, ranges, \
-                            point_list, n_contrib, g_colors, g_means2D, g_trans, g_inv, g_normal_opacity);           \
+                            trans_mat, inverse_m, trans_mat_t2, out_opacity, out_extras, out_flow, dL_dpix,          \
+                            dL_dopacity, dL_dextras, dL_dflow, ranges, point_list, n_contrib, g_colors, g_means2D,   \
+                            g_trans, g_inv, g_normal_opacity);                                                       \
     return 0;                                                                                                        \
   }
 

@@ -116,14 +116,15 @@ int oracle_gs_2d_fast_preprocess_backward_f32(int P, int W, int H, int sh_degree
 int oracle_gs_2d_fast_render_forward_f32(int W, int H, double near_n, double far_n, int only_image,
     const float* means2D, const float* colors, const float* normal_opacity, const float* trans_mat,
     const float* inverse_m, const int32_t* point_list, const int64_t* ranges, const int64_t* bucket_offset,
-    float* out_color, float* out_opacity, float* out_extras, int32_t* n_contrib, int32_t* max_contrib,
-    int32_t* bucket_to_tile, float* sampled_T, float* sampled_acc, float* sampled_aux);
+    const float* trans_mat_t2, int32_t* accum_max_count, float* accum_weights_p, int32_t* accum_weights_count,
+    float* out_color, float* out_opacity, float* out_extras, float* out_flow, int32_t* n_contrib,
+    int32_t* max_contrib, int32_t* bucket_to_tile, float* sampled_T, float* sampled_acc, float* sampled_aux);
 int oracle_gs_2d_fast_render_backward_f32(int P, int W, int H, double near_n, double far_n, int per_splat_form,
     const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,
-    const float* inverse_m, const float* out_opacity, const float* out_extras, const float* dL_dpix,
-    const float* dL_dopacity, const float* dL_dextras, const int64_t* ranges, const int32_t* point_list,
-    const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans, float* g_inv,
-    float* g_normal_opacity);
+    const float* inverse_m, const float* trans_mat_t2, const float* out_opacity, const float* out_extras,
+    const float* out_flow, const float* dL_dpix, const float* dL_dopacity, const float* dL_dextras,
+    const float* dL_dflow, const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib,
+    float* g_colors, float* g_means2D, float* g_trans, float* g_inv, float* g_normal_opacity);
 int oracle_gs_fast_prepare_fill(int P, int W, int H, const float* means2D, const float* inverse_m,
     const float* depths, const float* opacities, const int32_t* radii, const int64_t* offsets, int64_t R,
     int64_t* ranges, int32_t* point_list, int64_t* keys_sorted_out);

@@ -232,3 +232,129 @@ def test_per_splat_form_and_snapshots(oracle_mod):
         assert abs((lp - lm) / (2 * eps) - fgn[i, 3]) < 1e-5 * max(1.0, abs(fgn[i, 3]))
         checked += 1
     assert checked >= 6
+
+
+def _flow_case(O, seed=0, scale_mul=25.0, P=50, W=48, H=32):
+    s = _setup(O, P=P, W=W, H=H, seed=seed, scale_mul=scale_mul)
+    (m2, colors, tm, no), (fm2, fcolors, ftm, fim, fno), ranges, pl = _render_pair(O, s)
+    rng = np.random.default_rng(seed + 11)
+    t2 = np.ascontiguousarray(ftm + 0.05 * rng.normal(size=ftm.shape) * np.abs(ftm).mean())
+    std = dict(W=W, H=H, means2D=m2, colors=colors, trans_mat=tm, normal_opacity=no, ranges=ranges, point_list=pl,
+               near=0.2, far=100.0)
+    return s, std, (fm2, fcolors, ftm, fim, fno), ranges, pl, t2, rng
+
+
+def test_fast_flow_accum_and_snapshots_forward(oracle_mod):
+    """Fast-path optical flow (normalised by the final opacity, gs_2d_fast_redner.cu:259-263), the accum_* side outputs
+    and the 10-channel snapshots. With matched intrinsics the fast intersection equals the standard one, so the
+    independent per-pixel compositor of test_oracle_blend.py (closed forms on the whole list, pair sums, running
+    arg-max replay) applies with its flow divided by the opacity instead of the weight sum."""
+    from test_oracle_blend import _compose
+    O = oracle_mod
+    s, std, (fm2, fcolors, ftm, fim, fno), ranges, pl, t2, rng = _flow_case(O)
+    W, H, P = s['W'], s['H'], fno.shape[0]
+    lens = ranges[:, 1] - ranges[:, 0]
+    bucket_offset = np.ascontiguousarray(np.cumsum((lens + 31) // 32).astype(np.int64))
+    amc, awp, awc = np.zeros(P, np.int32), np.zeros(P), np.zeros(P, np.int32)
+    out = O.fast_render_forward(W, H, 0.2, 100.0, False, fm2, fcolors, fno, ftm, fim, pl, ranges, bucket_offset, t2,
+                                amc, awp, awc)
+    foc, foo, foe, fnc, max_contrib, b2t, sT, sacc, saux, flow = out
+    c = _compose(std, trans_mat_t2=t2, flow_by_opacity=True)
+    assert np.abs(flow - c['flow']).max() < 1e-7 * max(1.0, np.abs(c['flow']).max()) and np.abs(c['flow']).max() > 1e-2
+    assert (c['opacity'] < 0.7).sum() > 100  # the two normalisations really differ from "no normalisation"
+    assert np.abs(foo - c['opacity']).max() < 1e-9 and np.abs(foe[5] - c['distortion']).max() < 1e-9
+    assert np.array_equal(awc, c['accum_weights_count']) and np.abs(awp - c['accum_weights_p']).max() < 1e-9
+    assert np.array_equal(amc, c['accum_max_count']) and (amc != awc).any()
+    assert not flow[foo == 0].any()
+    # snapshots: 10 channels with flow; the first 8 are those of a run without flow, channels 8, 9 are the unnormalised
+    # flow sums over the list entries before the bucket = (flow * opacity) of a forward over the truncated lists
+    assert saux.shape[1] == 10 and (lens > 32).any()
+    plain = O.fast_render_forward(W, H, 0.2, 100.0, False, fm2, fcolors, fno, ftm, fim, pl, ranges, bucket_offset)
+    assert plain[8].shape[1] == 8 and np.array_equal(plain[8], saux[:, :8]) and np.array_equal(plain[6], sT)
+    gx = (W + 15) // 16
+    checked = 0
+    for t in np.flatnonzero(lens > 32):
+        b0 = 0 if t == 0 else int(bucket_offset[t - 1])
+        ty, tx = divmod(int(t), gx)
+        for k in range(1, int((lens[t] + 31) // 32)):
+            cut = ranges.copy()
+            cut[:, 1] = cut[:, 0]
+            cut[t, 1] = cut[t, 0] + 32 * k
+            o = O.fast_render_forward(W, H, 0.2, 100.0, False, fm2, fcolors, fno, ftm, fim, pl, cut, None, t2)
+            raw = o[-1] * o[1][..., None]
+            for ly in range(min(16, H - ty * 16)):
+                for lx in range(min(16, W - tx * 16)):
+                    rank = ly * 16 + lx
+                    if sT[b0 + k, rank] == 0:  # this pixel had stopped blending before the bucket: nothing written
+                        continue
+                    assert abs(saux[b0 + k, 8, rank] - raw[ty * 16 + ly, tx * 16 + lx, 0]) < 1e-9
+                    assert abs(saux[b0 + k, 9, rank] - raw[ty * 16 + ly, tx * 16 + lx, 1]) < 1e-9
+                    checked += 1
+    assert checked > 200
+
+
+def test_fast_flow_backward(oracle_mod):
+    """Per-pixel form: dL_dflow is taken as the gradient of the UNNORMALISED flow sum U = flow * opacity
+    (gs_2d_fast_redner.cu:366, :494-510), so the check is central differences of sum_pix g . U(theta) from the forward,
+    on surfels that never take the low-pass branch for the adjugate (the chain through the intersection is dropped
+    there, :524-548) and on all surfels for the opacity.
+    Per-splat form (:704-706, :765-782): its accumulator is (partial sum up to this entry) - (the NORMALISED final
+    flow); since total - final = -final * T_final, that equals the per-pixel form plus an opacity-map gradient of
+    -(final flow . g). The oracle restates the kernel literally (front-to-back partial sums); the identity is checked
+    here."""
+    from test_oracle_blend import _never_filtered
+    O = oracle_mod
+    s, std, (fm2, fcolors, ftm, fim, fno), ranges, pl, t2, rng = _flow_case(O, seed=4, scale_mul=40.0, P=30, W=32, H=32)
+    W, H = s['W'], s['H']
+    g_flow = np.ascontiguousarray(rng.normal(size=(H, W, 2)))
+    z3, z1, z8 = np.zeros((3, H, W)), np.zeros((H, W)), np.zeros((8, H, W))
+
+    def fwd(**over):
+        t = dict(means2D=fm2, normal_opacity=fno, trans_mat=ftm, inverse_m=fim)
+        t.update(over)
+        return O.fast_render_forward(W, H, 0.2, 100.0, False, t['means2D'], fcolors, t['normal_opacity'],
+                                     t['trans_mat'], t['inverse_m'], pl, ranges, None, t2)
+
+    base = fwd()
+    foo, foe, fnc, flow = base[1], base[2], base[3], base[-1]
+
+    def loss(**over):
+        o = fwd(**over)
+        return (g_flow * (o[-1] * o[1][..., None])).sum()
+
+    gc, gm, gt, gi, gn = O.fast_render_backward(0.2, 100.0, 0, fm2, fno, fcolors, ftm, fim, foo, foe, z3, z1, z8,
+                                                ranges, pl, fnc, t2, flow, g_flow)
+    assert not gc.any() and np.abs(gi).max() > 1e-3 and np.abs(gn[:, 3]).max() > 1e-3
+    used = list(np.unique(pl))
+    clean = [i for i in used if _never_filtered(std, i)]
+    assert len(clean) >= 4
+    eps, l0, checked = 1e-6, loss(), 0
+    for name, grad, which in (('normal_opacity', gn, used), ('inverse_m', gi, clean), ('means2D', gm, used)):
+        flat = grad.reshape(grad.shape[0], -1)
+        src = dict(normal_opacity=fno, inverse_m=fim, means2D=fm2)[name]
+        for i in which[:8]:
+            for a in ([3] if name == 'normal_opacity' else range(flat.shape[1])):
+                p, m = src.copy(), src.copy()
+                p.reshape(p.shape[0], -1)[i, a] += eps
+                m.reshape(m.shape[0], -1)[i, a] -= eps
+                lp, lm = loss(**{name: p}), loss(**{name: m})
+                if abs((lp - l0) - (l0 - lm)) > 1e-9 * max(1.0, abs(l0)):
+                    continue
+                fd = (lp - lm) / (2 * eps)
+                assert abs(fd - flat[i, a]) < 1e-5 * max(1.0, abs(fd)), (name, i, a, fd, flat[i, a])
+                checked += 1
+    assert checked > 60
+
+    # per-splat form = per-pixel flow terms + the other channels of the per-splat form with the opacity-map gradient
+    # lowered by (final flow . g)
+    g_img, g_opa = rng.normal(size=(3, H, W)), rng.normal(size=(H, W))
+    g_ext = np.zeros((8, H, W))
+    g_ext[[0, 1, 2, 3, 4, 6, 7]] = rng.normal(size=(7, H, W))
+    lit = O.fast_render_backward(0.2, 100.0, 1, fm2, fno, fcolors, ftm, fim, foo, foe, g_img, g_opa, g_ext, ranges, pl,
+                                 fnc, t2, flow, g_flow)
+    rest = O.fast_render_backward(0.2, 100.0, 1, fm2, fno, fcolors, ftm, fim, foo, foe, g_img,
+                                  np.ascontiguousarray(g_opa - (flow * g_flow).sum(-1)), g_ext, ranges, pl, fnc)
+    only_flow = (gc, gm, gt, gi, gn)
+    for a, b, c_ in zip(lit, rest, only_flow):
+        assert np.abs(a - (b + c_)).max() < 1e-9 * max(1.0, np.abs(a).max())
+    assert np.abs(lit[4][:, 3] - rest[4][:, 3] - 0).max() > 1e-3  # the flow terms are not negligible
