@@ -134,42 +134,20 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
     on the surfel parameters + Adam on the MLP weights and the control points (gradients reach them through the LBS and
     K-NN backward kernels and the MLP's fp32 GEMM backward)."""
     from fast_sp_gs_amd import scenes
-    from fast_sp_gs_amd.deform import DeformNetwork, deform_apply, superpoint_deform
-    from fast_sp_gs_amd.renderer import GS_2D_render
-    from fast_sp_gs_amd.sparse_gaussian_adam import SparseGaussianAdam
-    from fast_sp_gs_amd.ssim import l1_dssim_loss
+    from fast_sp_gs_amd.dynamic_step import DynamicStep
     scene_h, cam_h = scenes.config2(P=200_000, size=800, seed=2)
     scene, cam = scene_h.to(dev), cam_h.to(dev)
     g = torch.Generator().manual_seed(2)
-    ctrl = (torch.rand(512, 3, generator=g) * 2 - 1).to(dev).requires_grad_(True)
+    ctrl = (torch.rand(512, 3, generator=g) * 2 - 1).to(dev)
     target = torch.rand(3, cam.H, cam.W, generator=g).to(dev)
-    net = DeformNetwork(local_frame=True).to(dev)  # the fourth head gives each control point its rotation (6-DoF warp)
-    # a tiny rate keeps the random-target synthetic scene from drifting (Adam's steps are |lr| whatever the gradient, and
-    # the scale residuals are added after the activation, network.py:643), so every timed step sees the same workload
-    net_opt = torch.optim.Adam(list(net.parameters()) + [ctrl], lr=1e-7, fused=True)
-    names = ('means3D', 'scales', 'rotations', 'opacities', 'shs')
-    params = [getattr(scene, k).clone().requires_grad_(True) for k in names]
-    opt = SparseGaussianAdam([{'params': [p_], 'name': k} for p_, k in zip(params, names)], lr=1.6e-4, eps=1e-15)
-    bg = torch.ones(3, device=dev)
+    # the fourth head gives each control point its rotation (6-DoF warp). A tiny rate for the network and the control
+    # points keeps the random-target synthetic scene from drifting (Adam's steps are |lr| whatever the gradient, and the
+    # scale residuals are added after the activation, network.py:643), so every timed step sees the same workload
+    state = DynamicStep(scene, cam, ctrl, target, K=4, temperature=0.01, local_frame=True, warp_method='LBS',
+                        LBS_method='dist', lr=1.6e-4, net_lr=1e-7, lambda_dssim=0.2)
 
     def step(i):
-        t = torch.full((1,), (i % 17) / 17.0, device=dev)
-        c_xyz, c_rot, c_scale, c_local = net(ctrl.detach(), t)
-        d_xyz, d_rot, d_scale, _, _ = superpoint_deform(params[0].detach(), ctrl, c_xyz, c_rot, c_scale[:, :2],
-                                                        sp_rot=c_local, K=4, temperature=0.01, warp_method='LBS',
-                                                        LBS_method='dist')
-        xyz, scales, rot = deform_apply(params[0], d_xyz, params[1], d_scale, params[2], d_rot)
-        out = GS_2D_render(xyz, scales, rot, params[3], (cam.W, cam.H),
-                           cam.Tw2v, cam.Tv2c, campos=cam.campos, near=cam.near, far=cam.far, sh_degree=3,
-                           sh_features=params[4], background=bg)
-        image = out['images']
-        loss = l1_dssim_loss(image, target, 0.2)  # 0.8 * L1 + 0.2 * (1 - mean SSIM), fused
-        loss.backward()
-        opt.set_before_step(out['radii'] > 0, params[0].shape[0])
-        opt.step()
-        opt.zero_grad(set_to_none=True)
-        net_opt.step()
-        net_opt.zero_grad(set_to_none=True)
+        state.step(torch.full((1,), (i % 17) / 17.0, device=dev))
 
     for i in range(warmup):
         step(i)

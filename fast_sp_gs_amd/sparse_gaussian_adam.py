@@ -1,5 +1,6 @@
 """SparseGaussianAdam: same class and behaviour as the reference's `fast_2d_gs/sparse_gaussian_adam.py` (lines 10-49),
 driving the HIP masked-Adam kernel through the operator boundary."""
+import numpy as np
 import torch
 import torch.optim
 
@@ -23,6 +24,7 @@ class SparseGaussianAdam(torch.optim.Adam):
         """The reference's loop over parameter groups (sparse_gaussian_adam.py:20-45), with the groups' kernels folded
         into one launch per `_MAX` tensors; the arithmetic per element is the single-tensor kernel's."""
         params, grads, ms, vs, lrs, epss = [], [], [], [], [], []
+        corrections = {}  # step count -> the two bias corrections, shared by the groups that are at that count
         for group in self.param_groups:
             lr = group["lr"]
             eps = group["eps"]
@@ -36,10 +38,18 @@ class SparseGaussianAdam(torch.optim.Adam):
                 state['exp_avg'] = torch.zeros_like(param, memory_format=torch.preserve_format)
                 state['exp_avg_sq'] = torch.zeros_like(param, memory_format=torch.preserve_format)
             state['step'] += 1
-            step = float(state['step'])
+            step = state['step']
             params.append(param), grads.append(param.grad), ms.append(state["exp_avg"]), vs.append(state["exp_avg_sq"])
-            # bias corrections folded into the learning rate: lr * sqrt(1 - b2^t) / (1 - b1^t)
-            lrs.append(lr * (1 - 0.999 ** step) ** 0.5 / (1 - 0.9 ** step))
+            # Bias corrections folded into the learning rate: lr * sqrt(1 - b2^t) / (1 - b1^t). The reference evaluates
+            # this on `step`, a float32 tensor (sparse_gaussian_adam.py:42-46), so every operation rounds to float32
+            # and the product is widened to double at the call. The powers are taken by torch on the float32 tensor as
+            # there; the multiplication and division that follow are single correctly rounded float32 operations.
+            key = float(step)
+            if key not in corrections:
+                corrections[key] = (np.float32(((1 - 0.999 ** step) ** 0.5).item()),
+                                    np.float32((1 - 0.9 ** step).item()))
+            root_c2, c1 = corrections[key]
+            lrs.append(float(np.float32(lr) * root_c2 / c1))
             epss.append(eps)
         for i in range(0, len(params), self._MAX):
             j = slice(i, i + self._MAX)

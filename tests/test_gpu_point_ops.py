@@ -453,7 +453,11 @@ def test_sparse_adam(device, oracle_mod):
             p.grad = gr.to(device)
         opt.set_before_step(vis.to(device), N)
         opt.step()
-        lr = 1.6e-4 * (1 - 0.999 ** step) ** 0.5 / (1 - 0.9 ** step)
+        # the reference forms the rate on a float32 step TENSOR (sparse_gaussian_adam.py:42-46): float32 arithmetic,
+        # widened to double when it is handed to the kernel
+        step_t = torch.tensor(float(step), dtype=torch.float32)
+        lr = float(1.6e-4 * (1 - 0.999 ** step_t) ** 0.5 / (1 - 0.9 ** step_t))
+        assert lr != 1.6e-4 * (1 - 0.999 ** step) ** 0.5 / (1 - 0.9 ** step)  # ... which is not the double expression
         for k, s in enumerate(shapes):
             Mk = int(np.prod(s[1:]))
             O.call("adam_masked_update_f32", N, Mk, npy(vis.to(torch.uint8)), lr, 0.9, 0.999, 1e-15, ref_p[k],
