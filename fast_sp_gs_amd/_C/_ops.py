@@ -7,6 +7,7 @@ CHECK_INPUT / CHECK_SHAPE macros and raise RuntimeError like TORCH_CHECK does.
 from __future__ import annotations
 
 import ctypes
+import threading
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -94,16 +95,16 @@ def _f32(what, **tensors):
             L.require_dtype(what, k, t, torch.float32)
 
 
-_PINNED_COUNT = None
+_PINNED = threading.local()
 
 
 def _pinned_count() -> Tensor:
-    """One page-locked int64 the binning's instance count is copied into: a device-to-host copy into pinned memory is a
+    """A page-locked int64 the binning's instance count is copied into, one per host thread (a binning call waits for
+    its count before it returns, so a thread never has two in flight): a device-to-host copy into pinned memory is a
     direct transfer, into pageable memory it is staged by the runtime (about 25 us more per call)."""
-    global _PINNED_COUNT
-    if _PINNED_COUNT is None:
-        _PINNED_COUNT = torch.zeros(1, dtype=torch.int64, pin_memory=True)
-    return _PINNED_COUNT
+    if getattr(_PINNED, 'count', None) is None:
+        _PINNED.count = torch.zeros(1, dtype=torch.int64, pin_memory=True)
+    return _PINNED.count
 
 
 def _workspace(nbytes: int, device) -> Tensor:
@@ -188,8 +189,11 @@ def gs_2d_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotat
     P = means3D.shape[0]
     M = sh_rest.shape[1] if has_rest else (shs.shape[1] if shs.ndim == 3 else 0)
     L.require_shape(what, 'grad_means3D', grad_means3D, P, 3)
-    if grad_scales is None or grad_rotations is None:
-        raise RuntimeError(f'{what}: grad_scales and grad_rotations are required')
+    # optional in the reference (torch::optional, gs_2d_preprocess.cu:436, :447-448, :489-490): computed and dropped
+    if grad_scales is None:
+        grad_scales = torch.empty((P, 2), dtype=torch.float32, device=means3D.device)
+    if grad_rotations is None:
+        grad_rotations = torch.empty((P, 4), dtype=torch.float32, device=means3D.device)
     L.require_shape(what, 'grad_scales', grad_scales, P, 2)
     L.require_shape(what, 'grad_rotations', grad_rotations, P, 4)
     L.require_shape(what, 'grad_opacities', grad_opacities, P, 1)
@@ -548,8 +552,11 @@ def gs_2d_fast_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, 
     P = means3D.shape[0]
     M = sh_rest.shape[1] if has_rest else (shs.shape[1] if shs.ndim == 3 else 0)
     L.require_shape(what, 'grad_means3D', grad_means3D, P, 3)
-    if grad_scales is None or grad_rotations is None:
-        raise RuntimeError(f'{what}: grad_scales and grad_rotations are required')
+    # optional in the reference (torch::optional, gs_2d_preprocess.cu:436, :447-448, :489-490): computed and dropped
+    if grad_scales is None:
+        grad_scales = torch.empty((P, 2), dtype=torch.float32, device=means3D.device)
+    if grad_rotations is None:
+        grad_rotations = torch.empty((P, 4), dtype=torch.float32, device=means3D.device)
     L.require_shape(what, 'grad_scales', grad_scales, P, 2)
     L.require_shape(what, 'grad_rotations', grad_rotations, P, 4)
     L.require_shape(what, 'grad_opacities', grad_opacities, P, 1)

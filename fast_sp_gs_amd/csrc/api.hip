@@ -2,6 +2,9 @@
 #include "common.hpp"
 
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <utility>
 
 namespace fsgs {
 
@@ -16,6 +19,24 @@ int fail(int code, const char* fmt, ...) {
   vsnprintf(last_error_buffer(), 512, fmt, ap);
   va_end(ap);
   return code;
+}
+
+// One blockIdx -> tile table (65536 ints, see blend.hpp) per (device, stream) that a blend entry point was called on.
+int* tile_order_table(hipStream_t stream) {
+  static std::mutex mu;
+  static std::map<std::pair<int, hipStream_t>, int*> tables;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = tables.find({dev, stream});
+  if (it != tables.end()) return it->second;
+  int* p = nullptr;
+  if (hipMalloc((void**) &p, sizeof(int) * (1 << 16)) != hipSuccess) {
+    (void) hipGetLastError();
+    p = nullptr;
+  }
+  tables[{dev, stream}] = p;
+  return p;
 }
 
 static bool g_culling_enabled = true;

@@ -199,15 +199,17 @@ __device__ __forceinline__ unsigned quadrant_mask(const SplatHot& h, int tile_px
 // p % 8 == r (as long as it has tiles left), and inside a region tiles are listed by descending list length
 // (quarter-octave buckets, arbitrary order inside a bucket). Long lists start first and short ones fill the tail of the launch; a surfel
 // that overlaps several neighbouring tiles is gathered by blocks that share an L2.
-// The table lives in a file-scope device array (one copy per translation unit that includes this header): calls that
-// overlap on different streams would race on it, so the blend entry points must be issued on one stream at a time.
+// The table is a device buffer of kMaxOrderedTiles ints owned by the library, one per (device, stream) a blend entry
+// point has been called on (allocated on the first such call, kept until the process ends): calls on one stream are
+// ordered by the stream, calls on different streams use different tables.
 constexpr int kMaxOrderedTiles = 1 << 16;
 constexpr int kOrderBuckets    = 128;
 constexpr int kOrderRegions    = 8;
 
-namespace {
+// Defined in api.hip. nullptr if the table cannot be allocated (then blocks map to tiles directly).
+int* tile_order_table(hipStream_t stream);
 
-__device__ int g_tile_order[kMaxOrderedTiles];
+namespace {
 
 __device__ __forceinline__ int length_bucket(int64_t len64) {
   const unsigned len = len64 > 0x7fffffff ? 0x7fffffffu : (unsigned) (len64 < 0 ? 0 : len64);
@@ -229,7 +231,8 @@ __device__ __forceinline__ int tile_region(int t, int gx, int gy) {
   return ((tx / FSGS_TILE_GROUP) + 3 * (ty / FSGS_TILE_GROUP)) & (kOrderRegions - 1);
 }
 
-__global__ void __launch_bounds__(1024) tile_order_kernel(int gx, int gy, const int64_t* __restrict__ ranges) {
+__global__ void __launch_bounds__(1024) tile_order_kernel(int gx, int gy, const int64_t* __restrict__ ranges,
+                                                          int* __restrict__ tile_order) {
   __shared__ int s_count[kOrderRegions][kOrderBuckets];
   __shared__ int s_total[kOrderRegions];
   const int T = gx * gy;
@@ -255,21 +258,25 @@ __global__ void __launch_bounds__(1024) tile_order_kernel(int gx, int gy, const 
     int pos = 0;
 #pragma unroll
     for (int q = 0; q < kOrderRegions; ++q) pos += min(s_total[q], k) + ((q < r && s_total[q] > k) ? 1 : 0);
-    g_tile_order[pos] = t;
+    tile_order[pos] = t;
   }
 }
 
 // Launch flags of the blend kernels: bit 0 = the tile table was built for this launch (T small enough; otherwise blocks
 // map to tiles directly), bit 1 = per-quadrant culling switched off (verification aid, see fsgs_debug_set_culling).
-inline int launch_tile_order(int gx, int gy, const int64_t* ranges, hipStream_t s) {
+inline int launch_tile_order(int gx, int gy, const int64_t* ranges, hipStream_t s, const int** table) {
   int flags = culling_enabled() ? 0 : kFlagNoCull;
+  *table    = nullptr;
   if ((int64_t) gx * gy > kMaxOrderedTiles) return flags;
-  hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, s, gx, gy, ranges);
+  int* t = tile_order_table(s);
+  if (!t) return flags;
+  hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, s, gx, gy, ranges, t);
+  *table = t;
   return flags | kFlagOrdered;
 }
 
-__device__ __forceinline__ int scheduled_tile(int flags) {
-  return (flags & kFlagOrdered) ? g_tile_order[blockIdx.x] : (int) blockIdx.x;
+__device__ __forceinline__ int scheduled_tile(int flags, const int* __restrict__ tile_order) {
+  return (flags & kFlagOrdered) ? tile_order[blockIdx.x] : (int) blockIdx.x;
 }
 
 }  // namespace

@@ -34,7 +34,7 @@ static_assert(kBwdBatch <= kWave, "one wavefront stages a batch and another flus
 template <bool kAux, bool kFlow, bool kSlots>
 __global__ void __launch_bounds__(kBlendThreads) __attribute__((amdgpu_waves_per_eu(FSGS_BWD_WAVES, FSGS_BWD_WAVES)))
 blend_backward_kernel(
-    int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    int ordered, const int* __restrict__ tile_order, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const int32_t* __restrict__ n_contrib, const float2* __restrict__ means2D,
     const float4* __restrict__ normal_opacity, const float* __restrict__ colors, const float* __restrict__ trans_mat,
     const float* __restrict__ trans_mat_t2, const float* __restrict__ out_opacity, const float* __restrict__ out_extras,
@@ -57,7 +57,7 @@ blend_backward_kernel(
   __shared__ unsigned char s_mask[kBwdBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
 
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
-  const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(ordered, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -433,9 +433,10 @@ FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, doub
       hipLaunchKernelGGL(slot_fill_kernel, dim3((unsigned) std::min<size_t>((n4 + 255) / 256, 8192)), dim3(256), 0, s,
                          n4, (float4*) slot_grads);
   }
-  const int ordered = launch_tile_order(gx, gy, ranges, s);
+  const int* tile_order = nullptr;
+  const int ordered = launch_tile_order(gx, gy, ranges, s, &tile_order);
 #define FSGS_LAUNCH_BWD(AUX, FLOW, SLOTS)                                                                            \
-  hipLaunchKernelGGL((blend_backward_kernel<AUX, FLOW, SLOTS>), grid, block, 0, s, ordered, W, H, (float) near_n,    \
+  hipLaunchKernelGGL((blend_backward_kernel<AUX, FLOW, SLOTS>), grid, block, 0, s, ordered, tile_order, W, H, (float) near_n,    \
                      (float) far_n, ranges, point_list, n_contrib, (const float2*) means2D,                          \
                      (const float4*) normal_opacity, colors, trans_mat, trans_mat_t2, out_opacity, out_extras,       \
                      (const float2*) out_flow, dL_dpix, dL_dextras, dL_dopacity, (const float2*) dL_dflow,           \

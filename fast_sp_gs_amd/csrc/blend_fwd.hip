@@ -7,7 +7,7 @@
 // reset once set, :180-197).
 //
 // Layout: one 256-lane block per 16x16 tile; wavefront w owns an 8x8 pixel quadrant. Surfels of the tile's sorted
-// range are gathered 256 at a time (one per lane, colours included so the blend never goes back to HBM) into LDS as
+// range are gathered 128 at a time (one per lane of the first two wavefronts, colours included so the blend never goes back to HBM) into LDS as
 // 48-byte "hot" + 32-byte "cold" records; the next batch's gather is issued before the current batch is blended so its
 // HBM latency overlaps the arithmetic. All lanes of a wavefront read the same LDS record (broadcast, conflict free).
 #include "blend.hpp"
@@ -22,7 +22,7 @@ constexpr int kFwdBatch = FSGS_FWD_BATCH;  // surfels staged per round (<= block
 
 template <bool kAux, bool kFlow, bool kAccum>
 __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
-    int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    int ordered, const int* __restrict__ tile_order, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const float2* __restrict__ means2D, const float* __restrict__ colors, const float* __restrict__ trans_mat,
     const float4* __restrict__ normal_opacity, const float4* __restrict__ records,
     const float* __restrict__ trans_mat_t2, int32_t* __restrict__ n_contrib,
@@ -35,7 +35,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   __shared__ unsigned char s_mask[kFwdBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
 
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(ordered, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -249,9 +249,10 @@ FSGS_API int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, doubl
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
-  const int ordered = launch_tile_order(gx, gy, ranges, s);
+  const int* tile_order = nullptr;
+  const int ordered = launch_tile_order(gx, gy, ranges, s, &tile_order);
 #define FSGS_LAUNCH_FWD(AUX, FLOW, ACC)                                                                              \
-  hipLaunchKernelGGL((blend_forward_kernel<AUX, FLOW, ACC>), grid, block, 0, s, ordered, W, H, (float) near_n, (float) far_n, \
+  hipLaunchKernelGGL((blend_forward_kernel<AUX, FLOW, ACC>), grid, block, 0, s, ordered, tile_order, W, H, (float) near_n, (float) far_n, \
                      ranges, point_list, (const float2*) means2D, colors, trans_mat, (const float4*) normal_opacity, \
                      (const float4*) records, trans_mat_t2, n_contrib, out_color, out_opacity, out_extras, (float2*) out_flow,                \
                      accum_max_count, accum_weights_p, accum_weights_count)

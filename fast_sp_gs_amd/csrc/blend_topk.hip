@@ -33,7 +33,7 @@ __device__ __forceinline__ TopkEntry gather_topk(int id, const float2* __restric
 
 template <int kK>
 __global__ void __launch_bounds__(kBlendThreads) blend_topk_kernel(
-    int ordered, int W, int H, int topk, float near_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    int ordered, const int* __restrict__ tile_order, int W, int H, int topk, float near_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const float2* __restrict__ means2D, const float* __restrict__ trans_mat, const float4* __restrict__ normal_opacity,
     int32_t* __restrict__ top_indices, float* __restrict__ top_weights) {
   constexpr int kB = 128;  // surfels staged per round
@@ -42,7 +42,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_topk_kernel(
   __shared__ unsigned char s_mask[kB];
 
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(ordered, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -150,9 +150,10 @@ FSGS_API int fsgs_gs_2d_topk_weights(int topk, int P, int W, int H, double near_
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
-  const int ordered = launch_tile_order(gx, gy, ranges, s);
+  const int* tile_order = nullptr;
+  const int ordered = launch_tile_order(gx, gy, ranges, s, &tile_order);
 #define FSGS_TOPK(KK)                                                                                            \
-  hipLaunchKernelGGL((blend_topk_kernel<KK>), grid, block, 0, s, ordered, W, H, topk, (float) near_n, ranges, point_list, \
+  hipLaunchKernelGGL((blend_topk_kernel<KK>), grid, block, 0, s, ordered, tile_order, W, H, topk, (float) near_n, ranges, point_list, \
                      (const float2*) means2D, trans_mat, (const float4*) normal_opacity, top_indices, top_weights)
   if (topk <= 4) FSGS_TOPK(4);
   else if (topk <= 8) FSGS_TOPK(8);

@@ -117,7 +117,7 @@ __device__ __forceinline__ float wave_sum8_transposed(const float (&v)[8]) {
 
 template <bool kAux, bool kSnap, bool kAccum, bool kFlow>
 __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
-    int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    int ordered, const int* __restrict__ tile_order, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const float2* __restrict__ means2D, const float* __restrict__ colors, const float* __restrict__ trans_mat,
     const float* __restrict__ inverse_m, const float4* __restrict__ normal_opacity,
     const float* __restrict__ trans_mat_t2, const int64_t* __restrict__ bucket_offset, int32_t* __restrict__ n_contrib,
@@ -134,7 +134,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
   constexpr int kNum = kFlow ? 10 : 8;  // channels of a snapshot
 
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(ordered, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -317,7 +317,7 @@ constexpr int kFastGradSlots = 21;
 
 template <bool kAux, bool kPerSplat, bool kFlow>
 __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
-    int ordered, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
+    int ordered, const int* __restrict__ tile_order, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const int32_t* __restrict__ n_contrib, const float2* __restrict__ means2D,
     const float4* __restrict__ normal_opacity, const float* __restrict__ colors, const float* __restrict__ trans_mat,
     const float* __restrict__ inverse_m, const float* __restrict__ trans_mat_t2, const float* __restrict__ out_opacity,
@@ -337,7 +337,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
   __shared__ unsigned char s_mask[kB];
 
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = scheduled_tile(ordered), tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(ordered, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -586,9 +586,10 @@ FSGS_API int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, 
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
-  const int ordered = launch_tile_order(gx, gy, ranges, s);
+  const int* tile_order = nullptr;
+  const int ordered = launch_tile_order(gx, gy, ranges, s, &tile_order);
 #define FSGS_LAUNCH_FWD(AUX, SNAP, ACC, FLOW)                                                                        \
-  hipLaunchKernelGGL((fast_blend_forward_kernel<AUX, SNAP, ACC, FLOW>), grid, block, 0, s, ordered, W, H,            \
+  hipLaunchKernelGGL((fast_blend_forward_kernel<AUX, SNAP, ACC, FLOW>), grid, block, 0, s, ordered, tile_order, W, H,            \
                      (float) near_n, (float) far_n, ranges, point_list, (const float2*) means2D, colors, trans_mat,  \
                      inverse_m, (const float4*) normal_opacity, trans_mat_t2, bucket_offset, n_contrib, out_color,   \
                      out_opacity, out_extras, (float2*) out_flow, max_contrib, bucket_to_tile, sampled_T,            \
@@ -623,9 +624,10 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
-  const int ordered = launch_tile_order(gx, gy, ranges, s);
+  const int* tile_order = nullptr;
+  const int ordered = launch_tile_order(gx, gy, ranges, s, &tile_order);
 #define FSGS_LAUNCH_BWD(AUX, SPLAT, FLOW)                                                                            \
-  hipLaunchKernelGGL((fast_blend_backward_kernel<AUX, SPLAT, FLOW>), grid, block, 0, s, ordered, W, H,               \
+  hipLaunchKernelGGL((fast_blend_backward_kernel<AUX, SPLAT, FLOW>), grid, block, 0, s, ordered, tile_order, W, H,               \
                      (float) near_n, (float) far_n, ranges, point_list, n_contrib, (const float2*) means2D,          \
                      (const float4*) normal_opacity, colors, trans_mat, inverse_m, trans_mat_t2, out_opacity,        \
                      out_extras, (const float2*) out_flow, dL_dpix, dL_dextras, dL_dopacity,                         \

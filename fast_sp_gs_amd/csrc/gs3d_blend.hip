@@ -91,7 +91,7 @@ __device__ __forceinline__ bool conic_alpha_flat(const G3Hot& h, float pxf, floa
 }
 
 template <int E, bool kAccum>
-__global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, int W, int H,
+__global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, const int* __restrict__ tile_order, int W, int H,
     const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
     const float4* __restrict__ conic_opacity, const float* __restrict__ colors, const float* __restrict__ extras,
     float* __restrict__ out_color, float* __restrict__ out_opacity, float* __restrict__ out_extras,
@@ -100,7 +100,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
   __shared__ G3Hot s_hot[kG3Batch];
   __shared__ float s_feat[kG3Batch][3 + kMaxExtra + 1];  // odd stride
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(flags, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -204,12 +204,12 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
 // the reference's read-modify-write of global memory per contributing pair. `w >= slot` takes a slot (a later Gaussian
 // wins ties); indices start at -1, weights at 0.
 template <int kK>
-__global__ void __launch_bounds__(kBlendThreads) gs3d_topk_kernel(int flags, int W, int H, int topk,
+__global__ void __launch_bounds__(kBlendThreads) gs3d_topk_kernel(int flags, const int* __restrict__ tile_order, int W, int H, int topk,
     const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
     const float4* __restrict__ conic_opacity, int32_t* __restrict__ top_indices, float* __restrict__ top_weights) {
   __shared__ G3Hot s_hot[kG3Batch];
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(flags, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -285,7 +285,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_topk_kernel(int flags, int
 
 // gradient slots of one Gaussian: 0-2 colour | 3-6 extras | 7-8 mean2D | 9-11 conic | 12 opacity | 13-15 unused
 template <int E>
-__global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags, int W, int H,
+__global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags, const int* __restrict__ tile_order, int W, int H,
     const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
     const float4* __restrict__ conic_opacity, const float* __restrict__ colors, const float* __restrict__ extras,
     const float* __restrict__ out_opacity, const int32_t* __restrict__ n_contrib, const float* __restrict__ dL_dpix,
@@ -298,7 +298,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
   __shared__ float s_part[4][kB][17];  // each wavefront's sums per staged Gaussian: plain stores, added in wavefront order
   __shared__ int s_max_contrib;
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(flags, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -427,7 +427,7 @@ __device__ __forceinline__ int block_max_contrib(int last_contrib, int* s_max) {
 // of channels, so groups run side by side where the reference walks the list once per group in sequence. Output is
 // pixel-major [H, W, E].
 template <int kC>
-__global__ void __launch_bounds__(kBlendThreads) gs3d_extra_forward_kernel(int flags, int W, int H, int E,
+__global__ void __launch_bounds__(kBlendThreads) gs3d_extra_forward_kernel(int flags, const int* __restrict__ tile_order, int W, int H, int E,
     const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
     const float4* __restrict__ conic_opacity, const int32_t* __restrict__ n_contrib, const float* __restrict__ extras,
     float* __restrict__ out) {
@@ -436,7 +436,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_extra_forward_kernel(int f
   __shared__ float s_feat[kG3Batch][kC + 1];
   __shared__ int s_max_contrib;
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(flags, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -515,7 +515,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_extra_forward_kernel(int f
 // T_final = 1 - out_opacity without the background and opacity terms of the main backward. Each block adds its group's
 // share of the mean / conic / opacity gradients, as each of the reference's sequential groups does.
 // gradient slots of one Gaussian: 0-7 channels | 8-9 mean2D | 10-12 conic | 13 opacity | 14-15 unused
-__global__ void __launch_bounds__(kBlendThreads) gs3d_extra_backward_kernel(int flags, int W, int H, int E,
+__global__ void __launch_bounds__(kBlendThreads) gs3d_extra_backward_kernel(int flags, const int* __restrict__ tile_order, int W, int H, int E,
     const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
     const float4* __restrict__ conic_opacity, const float* __restrict__ out_opacity,
     const int32_t* __restrict__ n_contrib, const float* __restrict__ extras, const float* __restrict__ dL_dout,
@@ -526,7 +526,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_extra_backward_kernel(int 
   __shared__ float s_part[4][kB][17];  // each wavefront's sums per staged Gaussian: plain stores, added in wavefront order
   __shared__ int s_max_contrib;
   const int gx = (W + kTile - 1) / kTile;
-  const int tile = scheduled_tile(flags), tile_x = tile % gx, tile_y = tile / gx;
+  const int tile = scheduled_tile(flags, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
@@ -650,11 +650,12 @@ FSGS_API int fsgs_gaussian_rasterize_forward(int P, int W, int H, int E, const f
   FSGS_REQUIRE(P == 0 || (means2D && conic_opacity && colors), "gaussian_rasterize_forward: null pointer");
   hipStream_t s = (hipStream_t) stream;
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
-  const int flags = launch_tile_order(gx, gy, ranges, s);
+  const int* tile_order = nullptr;
+  const int flags = launch_tile_order(gx, gy, ranges, s, &tile_order);
   const dim3 grid(gx * gy), block(kBlendThreads);
   const bool accum = accum_max_count || accum_weights_p || accum_weights_count;
 #define FSGS_G3_FWD(EE, ACC)                                                                                        \
-  hipLaunchKernelGGL((gs3d_forward_kernel<EE, ACC>), grid, block, 0, s, flags, W, H, ranges, point_list,           \
+  hipLaunchKernelGGL((gs3d_forward_kernel<EE, ACC>), grid, block, 0, s, flags, tile_order, W, H, ranges, point_list,           \
                      (const float2*) means2D, (const float4*) conic_opacity, colors, extras, out_color,             \
                      out_opacity, out_extras, n_contrib, accum_max_count, accum_weights_p, accum_weights_count)
 #define FSGS_G3_FWD_E(EE) \
@@ -684,10 +685,11 @@ FSGS_API int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const 
                "gaussian_rasterize_backward: null pointer");
   hipStream_t s = (hipStream_t) stream;
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
-  const int flags = launch_tile_order(gx, gy, ranges, s);
+  const int* tile_order = nullptr;
+  const int flags = launch_tile_order(gx, gy, ranges, s, &tile_order);
   const dim3 grid(gx * gy), block(kBlendThreads);
 #define FSGS_G3_BWD(EE)                                                                                             \
-  hipLaunchKernelGGL((gs3d_backward_kernel<EE>), grid, block, 0, s, flags, W, H, ranges, point_list,               \
+  hipLaunchKernelGGL((gs3d_backward_kernel<EE>), grid, block, 0, s, flags, tile_order, W, H, ranges, point_list,               \
                      (const float2*) means2D, (const float4*) conic_opacity, colors, extras, out_opacity, n_contrib, \
                      dL_dpix, dL_dout_extras, dL_dout_opacity, g_means2D, g_conic_opacity, g_colors, g_extras)
   switch (E) {
@@ -711,9 +713,10 @@ FSGS_API int fsgs_gaussian_topk_weights(int topk, int P, int W, int H, const flo
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s   = (hipStream_t) stream;
-  const int flags = launch_tile_order(gx, gy, ranges, s);
+  const int* tile_order = nullptr;
+  const int flags = launch_tile_order(gx, gy, ranges, s, &tile_order);
 #define FSGS_TOPK3(KK)                                                                                          \
-  hipLaunchKernelGGL((gs3d_topk_kernel<KK>), grid, block, 0, s, flags, W, H, topk, ranges, point_list,          \
+  hipLaunchKernelGGL((gs3d_topk_kernel<KK>), grid, block, 0, s, flags, tile_order, W, H, topk, ranges, point_list,          \
                      (const float2*) means2D, (const float4*) conic_opacity, top_indices, top_weights)
   if (topk <= 4) FSGS_TOPK3(4);
   else if (topk <= 8) FSGS_TOPK3(8);
@@ -733,10 +736,11 @@ FSGS_API int fsgs_gaussian_rasterize_extra_forward(int P, int W, int H, int E, c
                "gaussian_rasterize_extra_forward: out_pixels must be 16-byte aligned");
   hipStream_t s = (hipStream_t) stream;
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
-  const int flags = launch_tile_order(gx, gy, ranges, s);
+  const int* tile_order = nullptr;
+  const int flags = launch_tile_order(gx, gy, ranges, s, &tile_order);
   const dim3 block(kBlendThreads);
 #define FSGS_G3_EXTRA(CC)                                                                                          \
-  hipLaunchKernelGGL((gs3d_extra_forward_kernel<CC>), dim3(gx * gy, (E + CC - 1) / CC), block, 0, s, flags, W, H,  \
+  hipLaunchKernelGGL((gs3d_extra_forward_kernel<CC>), dim3(gx * gy, (E + CC - 1) / CC), block, 0, s, flags, tile_order, W, H,  \
                      E, ranges, point_list, (const float2*) means2D, (const float4*) conic_opacity, n_contrib,     \
                      extras, out_pixels)
   if (E <= 8) FSGS_G3_EXTRA(8);
@@ -755,8 +759,9 @@ FSGS_API int fsgs_gaussian_rasterize_extra_backward(int P, int W, int H, int E, 
                "gaussian_rasterize_extra_backward: null pointer");
   hipStream_t s = (hipStream_t) stream;
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
-  const int flags = launch_tile_order(gx, gy, ranges, s);
-  hipLaunchKernelGGL(gs3d_extra_backward_kernel, dim3(gx * gy, (E + 7) / 8), dim3(kBlendThreads), 0, s, flags, W, H, E,
+  const int* tile_order = nullptr;
+  const int flags = launch_tile_order(gx, gy, ranges, s, &tile_order);
+  hipLaunchKernelGGL(gs3d_extra_backward_kernel, dim3(gx * gy, (E + 7) / 8), dim3(kBlendThreads), 0, s, flags, tile_order, W, H, E,
                      ranges, point_list, (const float2*) means2D, (const float4*) conic_opacity, out_opacity,
                      n_contrib, extras, grad_out, grad_means2D, grad_conic_opacity, grad_extras);
   return check_launch("gaussian_rasterize_extra_backward");

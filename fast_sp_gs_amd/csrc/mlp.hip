@@ -7,7 +7,7 @@
 //
 // One block owns 32 rows (control points) and keeps their activations in LDS for the whole network, so the only HBM/L2
 // traffic is the weights (about 1 MB in bf16, shared by all blocks through L2) and 40 bytes of output per row.
-// Each of the 4 wavefronts computes a 32 x 64 slab of a layer's output with v_mfma_f32_32x32x16_bf16: A fragments
+// Each of the 8 wavefronts computes a 32 x 32 slab of a layer's output with v_mfma_f32_32x32x16_bf16: A fragments
 // (activations) come from LDS as one 16-byte read per lane, B fragments (weights, packed in fragment order, see
 // frag_index) as one 16-byte global read per lane; both use the same (lane / 32, element) -> k mapping, so the product
 // is independent of how the hardware orders k inside a fragment.

@@ -104,3 +104,45 @@ def test_renderer_wrapper_is_importable_and_binds_by_name():
     from fast_sp_gs_amd._C import get_C_function
     assert m._GS_2D_Render._render_forward is get_C_function('GS_2D_render_forward')
     assert m.GS_prepare is get_C_function('GS_prepare')
+
+
+def test_operator_signatures_match_the_reference_prototypes():
+    """Positional arity of every exported operator against the reference's host-function prototypes
+    (tests/golden/op_signatures.json, written by tests/golden/make_op_signatures.py from the `m.def` bindings and the
+    C++ definitions): the reference's bindings are positional (no py::arg except cdist_top), so a drop-in must take the
+    same number of leading parameters in the same order; parameters added here must come after them and have defaults."""
+    import inspect
+    import json
+    from fast_sp_gs_amd._C import _ops
+    table = json.loads((ROOT / "tests" / "golden" / "op_signatures.json").read_text())
+    on_path = REFERENCE_NAMES + [
+        'gs_2d_fast_preprocess_forward', 'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward',
+        'gs_2d_fast_compute_trans_mat_backward', 'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward',
+        'gs_2d_topk_weights', 'fusedssim', 'fusedssim_backward', 'simple_knn', 'gs_preprocess_forward',
+        'gs_preprocess_backward', 'gaussian_rasterize_forward', 'gaussian_rasterize_backward', 'gaussian_topk_weights',
+        'gaussian_rasterize_extra_forward', 'gaussian_rasterize_extra_backward', 'gs_compute_cov3D_forward',
+        'gs_compute_cov3D_backward', 'gs_compute_cov2D_forward', 'gs_compute_cov2D_backward']
+    checked = 0
+    for name, entry in table.items():
+        fn = getattr(_ops, name, None)
+        if fn is None:
+            assert name not in on_path, f"{name} is on the path but not exported"
+            continue
+        ref = entry['params']
+        mine = [p for p in inspect.signature(fn).parameters.values()
+                if p.kind in (p.POSITIONAL_ONLY, p.POSITIONAL_OR_KEYWORD)]
+        assert len(mine) >= len(ref), (name, len(mine), len(ref))
+        for p in mine[len(ref):]:
+            assert p.default is not inspect.Parameter.empty, (name, p.name, "added parameter without a default")
+        for p, r in zip(mine, ref):
+            # what the reference lets a caller leave out (None for an optional tensor, a bound default) must be
+            # acceptable here too: a default here, if any, is None / the same kind of value
+            if r['optional'] and p.default is not inspect.Parameter.empty:
+                assert p.default is None, (name, p.name)
+        # same names where the reference spells them correctly (e.g. it has 'sh_featrues', 'tiles_touch')
+        same = sum(p.name == r['name'] for p, r in zip(mine, ref))
+        assert same >= len(ref) - 3, (name, [(p.name, r['name']) for p, r in zip(mine, ref) if p.name != r['name']])
+        checked += 1
+    assert checked >= 37
+    for name in on_path:
+        assert name in table and hasattr(_ops, name), name

@@ -95,6 +95,15 @@ def test_preprocess_variants(name, deg, n_rows, rest_rows, device, oracle_mod):
         assert rel_err(a, b) < 1e-5, (k, rel_err(a, b))
         if k != 'mean2D':
             assert not a[~vis].any(), f"{k}: non-zero gradient for a surfel that was not rendered"
+    # grad_scales / grad_rotations are optional in the reference (gs_2d_preprocess.cu:436, :447-448): the other outputs
+    # are what they are with them
+    g3b, gopb, gm2_b = nan(P, 3), nan(P, 1), d(gm2)
+    get_C_function('gs_2d_preprocess_backward')(
+        W, H, deg, False, d(scene.means3D), d(scene.scales), d(scene.rotations), d(scene.opacities), d(shs), d(rest),
+        d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), out[2], out[5], out[1], out[3], gm2_b, d(gt), None, d(gc), d(gno),
+        g3b, None, None, gopb, None if gsh is None else nan(*shs.shape), None if grest is None else nan(*rest.shape))
+    torch.cuda.synchronize()
+    assert torch.equal(g3b, g3) and torch.equal(gopb, gop) and torch.equal(gm2_b, gm2_d)
 
 
 def test_precomputed_transform(device, oracle_mod):
