@@ -25,7 +25,8 @@ __all__ = [
     'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward', 'gs_2d_fast_compute_trans_mat_backward',
     'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward', 'fusedssim', 'fusedssim_backward',
     'gs_2d_epilogue_forward', 'gs_2d_epilogue_backward', 'simple_knn', 'gs_preprocess_forward',
-    'gs_preprocess_backward', 'gaussian_rasterize_forward', 'gaussian_rasterize_backward', 'select_indices',
+    'gs_preprocess_backward', 'gaussian_rasterize_forward', 'gaussian_rasterize_backward', 'gaussian_rasterize_fast_backward',
+    'select_indices',
     'gather_rows', 'densify_masks', 'prune_mask', 'split_children', 'densification_stats',
     'gs_compute_cov3D_forward', 'gs_compute_cov3D_backward', 'gs_compute_cov2D_forward', 'gs_compute_cov2D_backward',
     'gaussian_topk_weights', 'gaussian_rasterize_extra_forward', 'gaussian_rasterize_extra_backward',
@@ -1719,21 +1720,21 @@ def gs_compute_cov2D_forward(cov3D: Tensor, mean: Tensor, viewmatrix: Tensor, fo
 def gs_compute_cov2D_backward(cov3D: Tensor, mean: Tensor, viewmatrix: Tensor, focal_x: float, focal_y: float,
                               tan_fovx: float, tan_fovy: float, grad_cov2D: Tensor,
                               grad_vm: Optional[Tensor] = None) -> List[Tensor]:
-    """gaussian_compute_cov2D.cu:229-248 -> [grad_cov3D, grad_mean]. The optional accumulation into a view-matrix
-    gradient is not supported."""
+    """gaussian_compute_cov2D.cu:229-248 -> [grad_cov3D, grad_mean]; with grad_vm[4,4] the view matrix's gradient is
+    added to its first three rows in place."""
     what = 'gs_compute_cov2D_backward'
-    if grad_vm is not None:
-        raise RuntimeError(f'{what}: the gradient to the view matrix is not supported')
     grad_cov2D = grad_cov2D.contiguous()
-    _f32(what, cov3D=cov3D, mean=mean, viewmatrix=viewmatrix, grad_cov2D=grad_cov2D)
+    _f32(what, cov3D=cov3D, mean=mean, viewmatrix=viewmatrix, grad_cov2D=grad_cov2D, grad_vm=grad_vm)
     N = mean.numel() // 3
     if cov3D.numel() != 6 * N or viewmatrix.numel() != 16 or grad_cov2D.numel() != 3 * N:
         raise RuntimeError(f'{what}: Error shape')
+    if grad_vm is not None and grad_vm.numel() != 16:
+        raise RuntimeError(f'{what}: grad_vm must have 16 elements')
     g_cov3D, g_mean = torch.empty_like(cov3D), torch.empty_like(mean)
     with _timed(what):
         rc = _lib().fsgs_gs_compute_cov2D_backward(N, L.ptr(cov3D), L.ptr(mean), L.ptr(viewmatrix), float(focal_x),
                                                    float(focal_y), float(tan_fovx), float(tan_fovy),
-                                                   L.ptr(grad_cov2D), L.ptr(g_cov3D), L.ptr(g_mean),
+                                                   L.ptr(grad_cov2D), L.ptr(g_cov3D), L.ptr(g_mean), L.ptr(grad_vm),
                                                    L.current_stream())
     L.check(rc, what)
     return [g_cov3D, g_mean]
@@ -1746,10 +1747,8 @@ def gs_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: bool, means
                           culling: Optional[Tensor] = None) -> List[Tensor]:
     """gaussian_preprocess.cu:372-466 -> [means2D, depths, colors, radii, tiles_touched, cov3Ds, conic_opacity]."""
     what = 'gs_preprocess_forward'
-    if cov3D_precomp is not None or cov2D_precomp is not None:
-        raise RuntimeError(f'{what}: pre-computed covariances are not supported by this library')
     _f32(what, means3D=means3D, scales=scales, rotations=rotations, opacities=opacities, shs=shs, Tw2v=Tw2v,
-         Tv2c=Tv2c, cam_pos=cam_pos)
+         Tv2c=Tv2c, cam_pos=cam_pos, cov3D_precomp=cov3D_precomp, cov2D_precomp=cov2D_precomp)
     if means3D.ndim != 2 or means3D.shape[-1] != 3:
         raise RuntimeError('Error shape for means3D')
     P = means3D.shape[0]
@@ -1780,21 +1779,28 @@ def gs_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: bool, means
     L.require_shape(what, 'cam_pos', cam_pos, 3)
     if sh_degree < 0:
         L.require_shape(what, 'shs', shs, P, 3)
+    if cov3D_precomp is not None:
+        L.require_shape(what, 'cov3D_precomp', cov3D_precomp, P, 6)
+    if cov2D_precomp is not None:
+        L.require_shape(what, 'cov2D_precomp', cov2D_precomp, P, 3)
     tx, ty = _tan_fov(tanFoV)
     opt = dict(dtype=torch.float32, device=means3D.device)
     colors = shs if sh_degree < 0 else torch.empty((P, 3), **opt)
     preserve = means2D is not None
     means2D_ = means2D if preserve else torch.empty((P, 2), **opt)
-    depths, cov3Ds, conic_opacity = torch.empty((P,), **opt), torch.empty((P, 6), **opt), torch.empty((P, 4), **opt)
+    depths, conic_opacity = torch.empty((P,), **opt), torch.empty((P, 4), **opt)
+    # the reference hands a pre-computed cov3D back as the cov3Ds output (gaussian_preprocess.cu:424)
+    cov3Ds = cov3D_precomp if cov3D_precomp is not None else torch.empty((P, 6), **opt)
     radii = torch.empty((P,), dtype=torch.int32, device=means3D.device)
     tiles_touched = torch.empty((P,), dtype=torch.int32, device=means3D.device)
     with _timed('gs_preprocess_forward'):
         rc = _lib().fsgs_gs_preprocess_forward(
             P, W, H, sh_degree, M, int(bool(is_opengl)), L.ptr(means3D), L.ptr(scales), L.ptr(rotations),
             L.ptr(opacities), L.ptr(shs), L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c),
-            L.ptr(cam_pos), tx, ty, L.ptr(culling), int(preserve), L.ptr(means2D_), L.ptr(depths),
-            None if sh_degree < 0 else L.ptr(colors), L.ptr(radii), L.ptr(tiles_touched), L.ptr(cov3Ds),
-            L.ptr(conic_opacity), L.current_stream())
+            L.ptr(cam_pos), tx, ty, L.ptr(culling), L.ptr(cov3D_precomp), L.ptr(cov2D_precomp), int(preserve),
+            L.ptr(means2D_), L.ptr(depths), None if sh_degree < 0 else L.ptr(colors), L.ptr(radii),
+            L.ptr(tiles_touched), None if cov3D_precomp is not None else L.ptr(cov3Ds), L.ptr(conic_opacity),
+            L.current_stream())
     L.check(rc, what)
     return [means2D_, depths, colors, radii, tiles_touched, cov3Ds, conic_opacity]
 
@@ -1804,21 +1810,29 @@ def gs_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotation
                            grad_conic, grad_means3D, grad_scales, grad_rotations, grad_opacities, grad_shs,
                            grad_sh_rest, grad_cov=None, grad_Tw2v=None, grad_campos=None) -> None:
     """gaussian_preprocess.cu:567-636: fills the caller's grad_* tensors in place (every row is assigned) and rewrites
-    grad_mean2D as the reference does. grad_depth is ignored there too."""
+    grad_mean2D as the reference does. grad_depth is ignored there too. With cov2Ds (pre-computed 2D covariances)
+    grad_cov is [P,3] and grad_scales / grad_rotations must be None; grad_Tw2v[4,4] and grad_campos[3] are added to."""
     what = 'gs_preprocess_backward'
-    if cov2Ds is not None:
-        raise RuntimeError(f'{what}: pre-computed 2D covariances are not supported by this library')
-    if grad_Tw2v is not None or grad_campos is not None:
-        raise RuntimeError(f'{what}: camera gradients are not supported by this library')
     _f32(what, grad_mean2D=grad_mean2D, grad_colors=grad_colors, grad_conic=grad_conic, grad_means3D=grad_means3D,
          grad_scales=grad_scales, grad_rotations=grad_rotations, grad_opacities=grad_opacities, grad_shs=grad_shs,
-         grad_sh_rest=grad_sh_rest, grad_cov=grad_cov, cov3Ds=cov3Ds)
+         grad_sh_rest=grad_sh_rest, grad_cov=grad_cov, cov3Ds=cov3Ds, cov2Ds=cov2Ds, grad_Tw2v=grad_Tw2v,
+         grad_campos=grad_campos)
+    if cov2Ds is not None and (grad_scales is not None or grad_rotations is not None):
+        raise RuntimeError(f'{what}: grad_scales / grad_rotations must be None with pre-computed 2D covariances')
+    if cov2Ds is None and cov3Ds is None:
+        raise RuntimeError(f"{what}: cov3Ds (the forward's output) or cov2Ds is required")
+    if grad_Tw2v is not None and grad_Tw2v.numel() != 16:
+        raise RuntimeError(f'{what}: grad_Tw2v must be [4,4]')
+    if grad_campos is not None and grad_campos.numel() != 3:
+        raise RuntimeError(f'{what}: grad_campos must be [3]')
     has_rest = sh_rest is not None and sh_rest.numel() > 0
     P = means3D.shape[0]
     M = sh_rest.shape[1] if has_rest else (shs.shape[1] if shs.ndim == 3 else 0)
     L.require_shape(what, 'grad_means3D', grad_means3D, P, 3)
     L.require_shape(what, 'grad_conic', grad_conic, P, 4)
     L.require_shape(what, 'grad_opacities', grad_opacities, P, 1)
+    if grad_cov is not None:
+        L.require_shape(what, 'grad_cov', grad_cov, P, 3 if cov2Ds is not None else 6)
     if sh_degree >= 0 and grad_colors is None:
         raise RuntimeError(f'{what}: grad_colors is required with SH colours')
     tx, ty = _tan_fov(tanFoV)
@@ -1826,9 +1840,10 @@ def gs_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotation
         rc = _lib().fsgs_gs_preprocess_backward(
             P, W, H, sh_degree, M, int(bool(is_opengl)), L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(shs),
             L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(cam_pos), tx, ty, L.ptr(radii),
-            L.ptr(colors), L.ptr(cov3Ds), L.ptr(grad_mean2D), L.ptr(grad_colors), L.ptr(grad_conic),
+            L.ptr(colors), L.ptr(cov3Ds), L.ptr(cov2Ds), L.ptr(grad_mean2D), L.ptr(grad_colors), L.ptr(grad_conic),
             L.ptr(grad_means3D), L.ptr(grad_scales), L.ptr(grad_rotations), L.ptr(grad_opacities), L.ptr(grad_shs),
-            L.ptr(grad_sh_rest) if has_rest else None, L.ptr(grad_cov), L.current_stream())
+            L.ptr(grad_sh_rest) if has_rest else None, L.ptr(grad_cov), L.ptr(grad_Tw2v), L.ptr(grad_campos),
+            L.current_stream())
     L.check(rc, what)
 
 
@@ -1838,10 +1853,9 @@ def gaussian_rasterize_forward(width: int, height: int, means2D: Tensor, conic_o
                                accum_weights_count: Optional[Tensor] = None,
                                per_tile_bucket_offset: Optional[Tensor] = None):
     """gaussian_render.cu:212-293 -> [pixel_colors[3,H,W], pixel_opacity[H,W], pixel_extras[E,H,W]|None,
-    n_contrib[H,W]]. The bucket snapshots for the per-Gaussian backward (per_tile_bucket_offset) are not built."""
+    n_contrib[H,W]] and, with per_tile_bucket_offset, [max_contrib[Ty,Tx], bucket_to_tile[B], sampled_T[B,256],
+    sampled_ar[B,3+E,256]] (the snapshots the per-Gaussian backward takes)."""
     what = 'gaussian_rasterize_forward'
-    if per_tile_bucket_offset is not None:
-        raise RuntimeError(f'{what}: the per-Gaussian (bucketed) backward is not supported by this library')
     _f32(what, means2D=means2D, conic_opacity=conic_opacity, colors=colors, extras=extras,
          accum_weights_p=accum_weights_p)
     L.require_cuda(what, point_list=point_list, ranges=ranges, accum_max_count=accum_max_count,
@@ -1870,14 +1884,28 @@ def gaussian_rasterize_forward(width: int, height: int, means2D: Tensor, conic_o
     pixel_colors, pixel_opacity = torch.empty((3, height, width), **opt), torch.empty((height, width), **opt)
     pixel_extras = torch.empty((E, height, width), **opt) if extras is not None else None
     n_contrib = torch.empty((height, width), dtype=torch.int32, device=colors.device)
+    snap = [None] * 4
+    if per_tile_bucket_offset is not None:
+        L.require_cuda(what, per_tile_bucket_offset=per_tile_bucket_offset)
+        L.require_dtype(what, 'per_tile_bucket_offset', per_tile_bucket_offset, torch.int64)
+        per_tile_bucket_offset = per_tile_bucket_offset.contiguous()
+        B = int(per_tile_bucket_offset.reshape(-1)[-1].item()) if per_tile_bucket_offset.numel() else 0
+        gy, gx = (height + _TILE - 1) // _TILE, (width + _TILE - 1) // _TILE
+        nb = max(B, 1)  # keep the base pointers valid when no tile has any entry
+        snap = [torch.zeros((gy, gx), dtype=torch.int32, device=colors.device),
+                torch.empty((nb,), dtype=torch.int32, device=colors.device),
+                torch.empty((nb, _TILE * _TILE), **opt), torch.empty((nb, 3 + E, _TILE * _TILE), **opt)]
     with _timed('gaussian_rasterize_forward'):
         rc = _lib().fsgs_gaussian_rasterize_forward(
             P, width, height, E, L.ptr(means2D), L.ptr(conic_opacity), L.ptr(colors), L.ptr(extras) if E else None,
             L.ptr(point_list), L.ptr(ranges), L.ptr(accum_max_count), L.ptr(accum_weights_p),
-            L.ptr(accum_weights_count), L.ptr(pixel_colors), L.ptr(pixel_opacity),
-            L.ptr(pixel_extras) if E else None, L.ptr(n_contrib), L.current_stream())
+            L.ptr(accum_weights_count), L.ptr(per_tile_bucket_offset), L.ptr(pixel_colors), L.ptr(pixel_opacity),
+            L.ptr(pixel_extras) if E else None, L.ptr(n_contrib), *[L.ptr(t) for t in snap], L.current_stream())
     L.check(rc, what)
-    return [pixel_colors, pixel_opacity, pixel_extras, n_contrib]
+    out = [pixel_colors, pixel_opacity, pixel_extras, n_contrib]
+    if per_tile_bucket_offset is not None:
+        out += [snap[0], snap[1][:B], snap[2][:B], snap[3][:B]]
+    return out
 
 
 def gaussian_rasterize_backward(means2D: Tensor, conic_opacity: Tensor, colors: Tensor, extras: Optional[Tensor],
@@ -1906,6 +1934,53 @@ def gaussian_rasterize_backward(means2D: Tensor, conic_opacity: Tensor, colors: 
             c(dL_dout_color), c(dL_dout_extra) if E else None, c(dL_dout_opacity), c(point_list), c(ranges)]
     with _timed('gaussian_rasterize_backward'):
         rc = _lib().fsgs_gaussian_rasterize_backward(
+            P, W, H, E, *[L.ptr(a) for a in args], L.ptr(dL_dmeans2D), L.ptr(dL_dconic_o), L.ptr(dL_dcolors),
+            L.ptr(dL_dextras), L.current_stream())
+    L.check(rc, what)
+    return dL_dcolors, dL_dextras, dL_dmeans2D, dL_dconic_o
+
+
+def gaussian_rasterize_fast_backward(means2D: Tensor, conic_opacity: Tensor, colors: Tensor, extras: Optional[Tensor],
+                                     images: Tensor, out_extras: Optional[Tensor], out_opacity: Tensor,
+                                     dL_dout_color: Tensor, dL_dout_opacity: Tensor, dL_dout_extra: Optional[Tensor],
+                                     ranges: Tensor, point_list: Tensor, n_contrib: Tensor, max_contrib: Tensor,
+                                     per_tile_bucket_offset: Tensor, bucket_to_tile: Tensor, sampled_T: Tensor,
+                                     sampled_ar: Tensor):
+    """gaussian_render.cu:760-812 -> (dL_dcolors[P,3], dL_dextras[P,E]|None, dL_dmeans2D[P,2], dL_dconic_opacity[P,4]):
+    the reference's per-Gaussian backward over the forward's bucket snapshots. The same derivative as
+    gaussian_rasterize_backward, evaluated by the same kernel; the snapshot tensors are checked and not read."""
+    what = 'gaussian_rasterize_fast_backward'
+    L.require_cuda(what, images=images, max_contrib=max_contrib, per_tile_bucket_offset=per_tile_bucket_offset,
+                   bucket_to_tile=bucket_to_tile, sampled_T=sampled_T, sampled_ar=sampled_ar)
+    L.require_dtype(what, 'per_tile_bucket_offset', per_tile_bucket_offset, torch.int64)
+    L.require_dtype(what, 'bucket_to_tile', bucket_to_tile, torch.int32)
+    L.require_dtype(what, 'max_contrib', max_contrib, torch.int32)
+    P = means2D.shape[0]
+    H, W = dL_dout_color.shape[1], dL_dout_color.shape[2]
+    E = extras.shape[-1] if (dL_dout_extra is not None and extras is not None) else 0
+    if E > 4:
+        raise RuntimeError('Only support NUM_EXTRA=0,1,2,3,4')
+    if E and out_extras is None:
+        raise RuntimeError(f'{what}: out_extras is required with extras')
+    B = int(bucket_to_tile.numel())
+    if tuple(sampled_T.shape) != (B, _TILE * _TILE) or tuple(sampled_ar.shape)[0] != B:
+        raise RuntimeError(f'{what}: the snapshot tensors do not match bucket_to_tile')
+    opt = dict(dtype=torch.float32, device=out_opacity.device)
+    grads = torch.zeros((P, 9 + E), **opt)  # one zero fill: means2D 2 | conic_opacity 4 | colours 3 | extras E
+    g_flat = grads.view(-1)
+    dL_dmeans2D = g_flat[:2 * P].view(P, 2)
+    dL_dconic_o = g_flat[2 * P:6 * P].view(P, 4)
+    dL_dcolors = g_flat[6 * P:9 * P].view(P, 3)
+    dL_dextras = g_flat[9 * P:].view(P, E) if E else None
+    if P == 0:
+        return dL_dcolors, dL_dextras, dL_dmeans2D, dL_dconic_o
+    c = lambda t: None if t is None else t.contiguous()
+    args = [c(means2D), c(conic_opacity), c(colors), c(extras) if E else None, c(images), c(out_extras) if E else None,
+            c(out_opacity), c(n_contrib), c(max_contrib), c(per_tile_bucket_offset), c(bucket_to_tile), c(sampled_T),
+            c(sampled_ar), c(dL_dout_color), c(dL_dout_extra) if E else None, c(dL_dout_opacity), c(point_list),
+            c(ranges)]
+    with _timed('gaussian_rasterize_backward'):
+        rc = _lib().fsgs_gaussian_rasterize_fast_backward(
             P, W, H, E, *[L.ptr(a) for a in args], L.ptr(dL_dmeans2D), L.ptr(dL_dconic_o), L.ptr(dL_dcolors),
             L.ptr(dL_dextras), L.current_stream())
     L.check(rc, what)

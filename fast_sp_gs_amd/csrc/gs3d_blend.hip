@@ -90,15 +90,21 @@ __device__ __forceinline__ bool conic_alpha_flat(const G3Hot& h, float pxf, floa
   return !(power > 0.0f) & !(o.alpha < (1.0f / 255.0f));
 }
 
-template <int E, bool kAccum>
+// kSnap (gaussian_render.cu:51-63, :100-106, :168-172): the state of every pixel still blending before each 32nd list
+// entry -- sampled_T[B,256], sampled_ar[B,3+E,256] by row-major position inside the tile -- plus bucket_to_tile[B] and
+// the tile's deepest contributor max_contrib[T], which the per-Gaussian backward of the reference consumes.
+template <int E, bool kAccum, bool kSnap>
 __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, const int* __restrict__ tile_order, int W, int H,
     const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
     const float4* __restrict__ conic_opacity, const float* __restrict__ colors, const float* __restrict__ extras,
     float* __restrict__ out_color, float* __restrict__ out_opacity, float* __restrict__ out_extras,
     int32_t* __restrict__ n_contrib, int32_t* __restrict__ accum_max_count, float* __restrict__ accum_weights_p,
-    int32_t* __restrict__ accum_weights_count) {
+    int32_t* __restrict__ accum_weights_count, const int64_t* __restrict__ bucket_offset,
+    int32_t* __restrict__ max_contrib, int32_t* __restrict__ bucket_to_tile, float* __restrict__ sampled_T,
+    float* __restrict__ sampled_ar) {
   __shared__ G3Hot s_hot[kG3Batch];
   __shared__ float s_feat[kG3Batch][3 + kMaxExtra + 1];  // odd stride
+  __shared__ int s_max_contrib;
   const int gx = (W + kTile - 1) / kTile;
   const int tile = scheduled_tile(flags, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
@@ -110,6 +116,14 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
   const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
   const int n_todo = (int) (r1 - r0);
   const int rounds = (n_todo + kG3Batch - 1) / kG3Batch;
+  const int rank = (py - tile_y * kTile) * kTile + (px - tile_x * kTile);  // row-major position inside the tile
+  int64_t bucket0 = 0;
+  if (kSnap) {
+    bucket0 = tile == 0 ? 0 : bucket_offset[tile - 1];
+    const int nb = (n_todo + 31) / 32;
+    for (int k = threadIdx.x; k < nb; k += kBlendThreads) bucket_to_tile[bucket0 + k] = tile;
+    if (threadIdx.x == 0) s_max_contrib = 0;
+  }
 
   bool done = !inside;
   float T = 1.0f, C[3 + (E > 0 ? E : 1)];
@@ -138,7 +152,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
     for (int c = 0; c < kG3Batch / kWave; ++c) {
       const int jj = c * kWave + lane;
       unsigned long long todo = __ballot(jj < n_here && ((s_hot[jj < kG3Batch ? jj : 0].mask >> wave) & 1u));
-      if (todo == 0ull) continue;
+      if (!kSnap && todo == 0ull) continue;  // with snapshots the state is stored even where nothing blends
       // One list entry. A wavefront walks its list alone and the launch lasts as long as its longest tile, so the next
       // entry's record is requested before the current one is evaluated (alternating registers) and the blend is one
       // divergent region behind one predicate.
@@ -164,6 +178,27 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
           last = b * kG3Batch + j + 1;
         }
       };
+      if (kSnap) {
+        // the chunk of 64 staged entries holds two buckets of 32: the state is stored in front of each
+        for (int half = 0; half < 2; ++half) {
+          const int base = c * kWave + half * 32;
+          if (base >= n_here) break;
+          if (!done) {
+            const size_t bk = (size_t) (bucket0 + (b * kG3Batch + base) / 32);
+            sampled_T[bk * 256 + rank] = T;
+#pragma unroll
+            for (int k = 0; k < 3 + E; ++k) sampled_ar[(bk * (3 + E) + k) * 256 + rank] = C[k];
+          }
+          unsigned long long part = todo & (half ? 0xffffffff00000000ull : 0x00000000ffffffffull);
+          while (part) {
+            if (__ballot(!done) == 0ull) break;
+            const int j = c * kWave + __builtin_ctzll(part);
+            part &= part - 1;
+            blend_entry(s_hot[j], j);
+          }
+        }
+        continue;
+      }
       auto pop = [&]() {
         const int j = c * kWave + __builtin_ctzll(todo);
         todo &= todo - 1;
@@ -197,6 +232,15 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
     for (int k = 0; k < 3; ++k) out_color[k * HW + pix] = C[k];
 #pragma unroll
     for (int k = 0; k < E; ++k) out_extras[k * HW + pix] = C[3 + k];
+  }
+  if (kSnap) {
+    int wave_max = last;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) wave_max = max(wave_max, __shfl_xor(wave_max, d, kWave));
+    __syncthreads();  // s_max_contrib was cleared before the first barrier of the loop only if the loop ran
+    if (lane == 0) atomicMax(&s_max_contrib, wave_max);
+    __syncthreads();
+    if (threadIdx.x == 0) max_contrib[tile] = s_max_contrib;
   }
 }
 
@@ -642,8 +686,12 @@ using namespace fsgs;
 FSGS_API int fsgs_gaussian_rasterize_forward(int P, int W, int H, int E, const float* means2D,
     const float* conic_opacity, const float* colors, const float* extras, const int32_t* point_list,
     const int64_t* ranges, int32_t* accum_max_count, float* accum_weights_p, int32_t* accum_weights_count,
-    float* out_color, float* out_opacity, float* out_extras, int32_t* n_contrib, void* stream) {
+    const int64_t* bucket_offset, float* out_color, float* out_opacity, float* out_extras, int32_t* n_contrib,
+    int32_t* max_contrib, int32_t* bucket_to_tile, float* sampled_T, float* sampled_ar, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "gaussian_rasterize_forward: bad sizes");
+  const bool snap = bucket_offset != nullptr;
+  FSGS_REQUIRE(!snap || (max_contrib && bucket_to_tile && sampled_T && sampled_ar),
+               "gaussian_rasterize_forward: snapshot outputs are required with per_tile_bucket_offset");
   FSGS_REQUIRE(E >= 0 && E <= kMaxExtra, "gaussian_rasterize_forward: only 0..%d extra channels are supported", kMaxExtra);
   FSGS_REQUIRE(ranges && out_color && out_opacity && n_contrib && (E == 0 || (extras && out_extras)),
                "gaussian_rasterize_forward: null pointer");
@@ -654,12 +702,18 @@ FSGS_API int fsgs_gaussian_rasterize_forward(int P, int W, int H, int E, const f
   const int flags = launch_tile_order(gx, gy, ranges, s, &tile_order);
   const dim3 grid(gx * gy), block(kBlendThreads);
   const bool accum = accum_max_count || accum_weights_p || accum_weights_count;
-#define FSGS_G3_FWD(EE, ACC)                                                                                        \
-  hipLaunchKernelGGL((gs3d_forward_kernel<EE, ACC>), grid, block, 0, s, flags, tile_order, W, H, ranges, point_list,           \
-                     (const float2*) means2D, (const float4*) conic_opacity, colors, extras, out_color,             \
-                     out_opacity, out_extras, n_contrib, accum_max_count, accum_weights_p, accum_weights_count)
-#define FSGS_G3_FWD_E(EE) \
-  if (accum) FSGS_G3_FWD(EE, true); else FSGS_G3_FWD(EE, false)
+#define FSGS_G3_FWD(EE, ACC, SNAP)                                                                                  \
+  hipLaunchKernelGGL((gs3d_forward_kernel<EE, ACC, SNAP>), grid, block, 0, s, flags, tile_order, W, H, ranges,      \
+                     point_list, (const float2*) means2D, (const float4*) conic_opacity, colors, extras, out_color, \
+                     out_opacity, out_extras, n_contrib, accum_max_count, accum_weights_p, accum_weights_count,     \
+                     bucket_offset, max_contrib, bucket_to_tile, sampled_T, sampled_ar)
+#define FSGS_G3_FWD_E(EE)                                     \
+  do {                                                        \
+    if (accum && snap) FSGS_G3_FWD(EE, true, true);           \
+    else if (accum) FSGS_G3_FWD(EE, true, false);             \
+    else if (snap) FSGS_G3_FWD(EE, false, true);              \
+    else FSGS_G3_FWD(EE, false, false);                       \
+  } while (0)
   switch (E) {
     case 0: FSGS_G3_FWD_E(0); break;
     case 1: FSGS_G3_FWD_E(1); break;
@@ -701,6 +755,24 @@ FSGS_API int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const 
   }
 #undef FSGS_G3_BWD
   return check_launch("gaussian_rasterize_backward");
+}
+
+// The reference's second backward walks 32-entry buckets from the forward's snapshots, one warp per bucket
+// (gaussian_render.cu:540-694). It evaluates the same derivative as the back-to-front kernel; here both names run
+// that kernel, and the snapshot arguments are accepted (and checked for presence) so that the binding is a drop-in.
+FSGS_API int fsgs_gaussian_rasterize_fast_backward(int P, int W, int H, int E, const float* means2D,
+    const float* conic_opacity, const float* colors, const float* extras, const float* images,
+    const float* out_extras, const float* out_opacity, const int32_t* n_contrib, const int32_t* max_contrib,
+    const int64_t* bucket_offset, const int32_t* bucket_to_tile, const float* sampled_T, const float* sampled_ar,
+    const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
+    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, void* stream) {
+  if (P == 0) return kOk;
+  FSGS_REQUIRE(images && max_contrib && bucket_offset && bucket_to_tile && sampled_T && sampled_ar &&
+                   (E == 0 || out_extras),
+               "gaussian_rasterize_fast_backward: null pointer");
+  return fsgs_gaussian_rasterize_backward(P, W, H, E, means2D, conic_opacity, colors, extras, out_opacity, n_contrib,
+                                          dL_dpix, dL_dout_extras, dL_dout_opacity, point_list, ranges, g_means2D,
+                                          g_conic_opacity, g_colors, g_extras, stream);
 }
 
 FSGS_API int fsgs_gaussian_topk_weights(int topk, int P, int W, int H, const float* means2D,

@@ -70,7 +70,7 @@ __device__ __forceinline__ void cov3d_backward(const float* s, const float4 q, c
 }
 
 struct Cov2DTerms {
-  float t[3], M[6], x_mul, y_mul;
+  float t[3], M[6], J[6], x_mul, y_mul;
 };
 
 // View-space mean with the 1.3 x FoV clamp, the projection Jacobian J and M = J W (W = rotation block of Tw2v).
@@ -87,6 +87,8 @@ __device__ __forceinline__ void cov2d_terms(const float* mean, float fx, float f
   o.t[1]  = fminf(fmaxf(o.t[1], -limy), limy);
   const float tz = o.t[2];
   const float J[6] = {fx / tz, 0.0f, -(fx * o.t[0]) / (tz * tz), 0.0f, fy / tz, -(fy * o.t[1]) / (tz * tz)};
+#pragma unroll
+  for (int k = 0; k < 6; ++k) o.J[k] = J[k];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -125,10 +127,12 @@ __device__ __forceinline__ void cov2d_product(const float* M, const float* c, fl
   out[0] = cov[0], out[1] = cov[1], out[2] = cov[3];
 }
 
-// dL/dcov2D = (da, db, dc) (b is the one stored off-diagonal entry) -> dL/dcov3D (6) and dL/dmean (3).
-__device__ __forceinline__ void cov2d_backward_cov(const Cov2DTerms& k, const float* c3, float fx, float fy,
-                                                   const float* V, float da, float db, float dc, float* g_cov3D,
-                                                   float* g_mean) {
+// dL/dcov2D = (da, db, dc) (b is the one stored off-diagonal entry) -> dL/dcov3D (6), dL/dmean (3) and, when g_vm is
+// given, this point's share of dL/d(view matrix rows 0-2) (12 values, row-major with the translation in column 3;
+// gaussian_compute_cov2D.cu:163-183), ADDED to g_vm.
+__device__ __forceinline__ void cov2d_backward_cov(const Cov2DTerms& k, const float* mean, const float* c3, float fx,
+                                                   float fy, const float* V, float da, float db, float dc,
+                                                   float* g_cov3D, float* g_mean, float* g_vm = nullptr) {
 #pragma clang fp contract(off)
   const float* M = k.M;
   g_cov3D[0] = (M[0] * M[0] * da + M[0] * M[3] * db + M[3] * M[3] * dc);
@@ -156,12 +160,21 @@ __device__ __forceinline__ void cov2d_backward_cov(const Cov2DTerms& k, const fl
       -fx * tz2 * dJ00 - fy * tz2 * dJ11 + (2 * fx * k.t[0]) * tz3 * dJ02 + (2 * fy * k.t[1]) * tz3 * dJ12;
 #pragma unroll
   for (int a2 = 0; a2 < 3; ++a2) g_mean[a2] = V[a2] * dtx + V[4 + a2] * dty + V[8 + a2] * dtz;
+  if (g_vm) {
+    const float dt[3] = {dtx, dty, dtz};
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+#pragma unroll
+      for (int j = 0; j < 3; ++j) g_vm[4 * i + j] += k.J[i] * dT[j] + k.J[3 + i] * dT[3 + j] + dt[i] * mean[j];
+      g_vm[4 * i + 3] += dt[i];
+    }
+  }
 }
 
 // dL/dconic -> dL/dcov3D (6) and dL/dmean (3); false when the covariance determinant is exactly zero.
 __device__ __forceinline__ bool cov2d_backward(const float* mean, const float* c3, float fx, float fy, float tanx,
                                                float tany, const float* V, const float* g_conic, float* g_cov3D,
-                                               float* g_mean) {
+                                               float* g_mean, float* g_vm = nullptr) {
 #pragma clang fp contract(off)
   Cov2DTerms k;
   cov2d_terms(mean, fx, fy, tanx, tany, V, k);
@@ -175,7 +188,7 @@ __device__ __forceinline__ bool cov2d_backward(const float* mean, const float* c
   const float da = denom2inv * (-c * tt + denom * g_conic[2]);
   const float dc = denom2inv * (-a * tt + denom * g_conic[0]);
   const float db = denom2inv * (2.0f * b * tt - denom * g_conic[1]);
-  cov2d_backward_cov(k, c3, fx, fy, V, da, db, dc, g_cov3D, g_mean);
+  cov2d_backward_cov(k, mean, c3, fx, fy, V, da, db, dc, g_cov3D, g_mean, g_vm);
   return true;
 }
 
@@ -201,15 +214,21 @@ struct Screen {
 };
 
 // Everything between the frustum test and the SH colour; false = rejected.
+// cov2D_given: a pre-computed 2D covariance, taken as it is (gaussian_preprocess.cu:76-78).
 __device__ __forceinline__ bool screen_geometry(int W, int H, int gx, int gy, bool is_opengl, const float* p,
-                                                const Projected& pr, const float* c3, float fx, float fy, float tanx,
-                                                float tany, const float* Tw2v, Screen& o) {
+                                                const Projected& pr, const float* c3, const float* cov2D_given,
+                                                float fx, float fy, float tanx, float tany, const float* Tw2v,
+                                                Screen& o) {
 #pragma clang fp contract(off)
-  Cov2DTerms k;
-  cov2d_terms(p, fx, fy, tanx, tany, Tw2v, k);
   float cov[3];
-  cov2d_product(k.M, c3, cov);
-  cov[0] += 0.3f, cov[2] += 0.3f;
+  if (cov2D_given) {
+    cov[0] = cov2D_given[0], cov[1] = cov2D_given[1], cov[2] = cov2D_given[2];
+  } else {
+    Cov2DTerms k;
+    cov2d_terms(p, fx, fy, tanx, tany, Tw2v, k);
+    cov2d_product(k.M, c3, cov);
+    cov[0] += 0.3f, cov[2] += 0.3f;
+  }
   const float det = cov[0] * cov[2] - cov[1] * cov[1];
   if (det == 0.0f) return false;
   const float mid = 0.5f * (cov[0] + cov[2]);
@@ -234,6 +253,7 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_forward_kernel(int P, int
     const float4* __restrict__ rotations, const float* __restrict__ opacities, const float* __restrict__ shs,
     const float* __restrict__ sh_rest, const float* __restrict__ Tw2v_g, const float* __restrict__ Tv2c_g,
     const float* __restrict__ campos, float tanx, float tany, const uint8_t* __restrict__ culling,
+    const float* __restrict__ cov3D_precomp, const float* __restrict__ cov2D_precomp,
     int means2D_preserve, float2* __restrict__ means2D, float* __restrict__ depths, float* __restrict__ colors,
     int32_t* __restrict__ radii, int32_t* __restrict__ tiles_touched, float* __restrict__ cov3Ds,
     float4* __restrict__ conic_opacity) {
@@ -268,9 +288,19 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_forward_kernel(int P, int
     Projected pr;
     project(p, Tw2v, Tv2c, pr);
     if (is_opengl ? (pr.proj[2] < -1.0f || pr.proj[2] > 1.0f) : pr.pv[2] <= 0.2f) break;
-    const float s[3] = {scales[3 * (size_t) i], scales[3 * (size_t) i + 1], scales[3 * (size_t) i + 2]};
-    cov3d_forward(s, rotations[i], c3);  // kept even when a later test rejects the Gaussian, as in the reference
-    ok = screen_geometry(W, H, gx, gy, is_opengl != 0, p, pr, c3, fx, fy, tanx, tany, Tw2v, sc);
+    float cov2[3] = {0, 0, 0};
+    if (cov2D_precomp) {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) cov2[k] = cov2D_precomp[3 * (size_t) i + k];
+    } else if (cov3D_precomp) {
+#pragma unroll
+      for (int k = 0; k < 6; ++k) c3[k] = cov3D_precomp[6 * (size_t) i + k];
+    } else {
+      const float s[3] = {scales[3 * (size_t) i], scales[3 * (size_t) i + 1], scales[3 * (size_t) i + 2]};
+      cov3d_forward(s, rotations[i], c3);  // kept even when a later test rejects the Gaussian, as in the reference
+    }
+    ok = screen_geometry(W, H, gx, gy, is_opengl != 0, p, pr, c3, cov2D_precomp ? cov2 : nullptr, fx, fy, tanx, tany,
+                         Tw2v, sc);
   } while (false);
 
   if (sh_degree >= 0) {
@@ -296,8 +326,9 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_forward_kernel(int P, int
     }
   }
   if (!valid) return;
+  if (cov3Ds)  // absent with a pre-computed 3D covariance: the caller hands that tensor on as the operator's output
 #pragma unroll
-  for (int k = 0; k < 6; ++k) cov3Ds[6 * (size_t) i + k] = c3[k];
+    for (int k = 0; k < 6; ++k) cov3Ds[6 * (size_t) i + k] = c3[k];
   if (sh_degree >= 0) {
     colors[3 * (size_t) i] = rgb[0], colors[3 * (size_t) i + 1] = rgb[1], colors[3 * (size_t) i + 2] = rgb[2];
   }
@@ -314,10 +345,11 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_backward_kernel(int P, in
     const float4* __restrict__ rotations, const float* __restrict__ shs, const float* __restrict__ sh_rest,
     const float* __restrict__ Tw2v_g, const float* __restrict__ Tv2c_g, const float* __restrict__ campos, float tanx,
     float tany, const int32_t* __restrict__ radii, const float* __restrict__ colors,
-    const float* __restrict__ cov3Ds, float2* __restrict__ grad_mean2D, const float* __restrict__ grad_colors,
+    const float* __restrict__ cov3Ds, const float* __restrict__ cov2Ds, float2* __restrict__ grad_mean2D,
+    const float* __restrict__ grad_colors,
     const float4* __restrict__ grad_conic, float* __restrict__ g_means3D, float* __restrict__ g_scales,
     float4* __restrict__ g_rot, float* __restrict__ g_opac, float* __restrict__ g_shs, float* __restrict__ g_sh_rest,
-    float* __restrict__ g_cov3D) {
+    float* __restrict__ g_cov3D, float* __restrict__ g_Tw2v, float* __restrict__ g_campos) {
   constexpr bool kStage = kSh == 16;
   __shared__ float s_Tw2v[16], s_Tv2c[16];
   __shared__ float s_rows[kStage ? kShStageRows * kShStageStride : 1];
@@ -347,6 +379,11 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_backward_kernel(int P, in
     stage_sh_rows(s_rows, s_flag, blockIdx.x * blockDim.x, P, n, n_sh, shs, sh_rest);
     __syncthreads();
   }
+  // this lane's share of the camera gradients: dL/dTw2v rows 0-2 (12 values) and dL/dcampos (3)
+  float cam[15];
+#pragma unroll
+  for (int k = 0; k < 15; ++k) cam[k] = 0.0f;
+  const int cov_w = cov2Ds ? 3 : 6;  // columns of g_cov3D
   if (vis) {
     float Tw2v[16], Tv2c[16];
 #pragma unroll
@@ -369,15 +406,36 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_backward_kernel(int P, in
       const float4 gc = grad_conic[i];
       g_opac[i] = gc.w;
       const float gcv[3] = {gc.x, gc.y, gc.z};
-      float c3[6], gmc[3];
+      if (cov2Ds) {
+        // a pre-computed 2D covariance: the conic's derivative, nothing reaches the mean (gaussian_preprocess.cu:293-301)
+        if (g_cov3D) {
+          const float a = cov2Ds[3 * (size_t) i], b = cov2Ds[3 * (size_t) i + 1], c = cov2Ds[3 * (size_t) i + 2];
+          const float denom = a * c - b * b;
+          const float denom2inv = 1.0f / ((denom * denom) + 0.0000001f);
+          const float tt = c * gcv[0] - b * gcv[1] + a * gcv[2];
+          g_cov3D[3 * (size_t) i + 0] = denom2inv * (-c * tt + denom * gcv[2]);
+          g_cov3D[3 * (size_t) i + 2] = denom2inv * (-a * tt + denom * gcv[0]);
+          g_cov3D[3 * (size_t) i + 1] = denom2inv * (2.0f * b * tt - denom * gcv[1]);
+        }
+      } else {
+        float c3[6], gmc[3];
 #pragma unroll
-      for (int k = 0; k < 6; ++k) c3[k] = cov3Ds[6 * (size_t) i + k];
-      if (cov2d_backward(p, c3, fx, fy, tanx, tany, Tw2v, gcv, gcov, gmc)) {
+        for (int k = 0; k < 6; ++k) c3[k] = cov3Ds[6 * (size_t) i + k];
+        if (cov2d_backward(p, c3, fx, fy, tanx, tany, Tw2v, gcv, gcov, gmc, g_Tw2v ? cam : nullptr)) {
 #pragma unroll
-        for (int a = 0; a < 3; ++a) gm[a] += gmc[a];
+          for (int a = 0; a < 3; ++a) gm[a] += gmc[a];
+        }
+      }
+      if (g_Tw2v) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+#pragma unroll
+          for (int b = 0; b < 3; ++b) cam[4 * a + b] += p[b] * dpv[a];
+          cam[4 * a + 3] += dpv[a];
+        }
       }
     }
-    if (g_cov3D)
+    if (g_cov3D && !cov2Ds)
 #pragma unroll
       for (int k = 0; k < 6; ++k) g_cov3D[6 * (size_t) i + k] = gcov[k];
     if (sh_degree >= 0) {
@@ -406,25 +464,28 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_backward_kernel(int P, in
       sh_grad_accumulate(sh_degree, x, y, z, tl, dx, dy, dz);
       const float vx = p[0] - campos[0], vy = p[1] - campos[1], vz = p[2] - campos[2];
       const float tt = -(vx * dx + vy * dy + vz * dz) * nn * nn * nn;
-      gm[0] = gm[0] + (dx * nn + tt * vx);
-      gm[1] = gm[1] + (dy * nn + tt * vy);
-      gm[2] = gm[2] + (dz * nn + tt * vz);
+      const float gd[3] = {dx * nn + tt * vx, dy * nn + tt * vy, dz * nn + tt * vz};
+      gm[0] = gm[0] + gd[0];
+      gm[1] = gm[1] + gd[1];
+      gm[2] = gm[2] + gd[2];
+      cam[12] = -gd[0], cam[13] = -gd[1], cam[14] = -gd[2];  // the view direction is normalize(p - campos)
     }
     g_means3D[3 * (size_t) i] = gm[0], g_means3D[3 * (size_t) i + 1] = gm[1], g_means3D[3 * (size_t) i + 2] = gm[2];
-    const float s[3] = {scales[3 * (size_t) i], scales[3 * (size_t) i + 1], scales[3 * (size_t) i + 2]};
-    float gs[3], gq[4];
-    cov3d_backward(s, rotations[i], gcov, gs, gq);
-    if (g_scales)
-      g_scales[3 * (size_t) i] = gs[0], g_scales[3 * (size_t) i + 1] = gs[1], g_scales[3 * (size_t) i + 2] = gs[2];
-    if (g_rot) g_rot[i] = make_float4(gq[0], gq[1], gq[2], gq[3]);
+    if (g_scales || g_rot) {
+      const float s[3] = {scales[3 * (size_t) i], scales[3 * (size_t) i + 1], scales[3 * (size_t) i + 2]};
+      float gs[3], gq[4];
+      cov3d_backward(s, rotations[i], gcov, gs, gq);
+      if (g_scales)
+        g_scales[3 * (size_t) i] = gs[0], g_scales[3 * (size_t) i + 1] = gs[1], g_scales[3 * (size_t) i + 2] = gs[2];
+      if (g_rot) g_rot[i] = make_float4(gq[0], gq[1], gq[2], gq[3]);
+    }
   } else if (valid) {
     g_opac[i] = 0.0f;
     g_means3D[3 * (size_t) i] = 0.0f, g_means3D[3 * (size_t) i + 1] = 0.0f, g_means3D[3 * (size_t) i + 2] = 0.0f;
     if (g_scales) g_scales[3 * (size_t) i] = 0.0f, g_scales[3 * (size_t) i + 1] = 0.0f, g_scales[3 * (size_t) i + 2] = 0.0f;
     if (g_rot) g_rot[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     if (g_cov3D)
-#pragma unroll
-      for (int k = 0; k < 6; ++k) g_cov3D[6 * (size_t) i + k] = 0.0f;
+      for (int k = 0; k < cov_w; ++k) g_cov3D[(size_t) cov_w * i + k] = 0.0f;
     if (sh_degree >= 0) {
       if (kStage) {
         for (int c = 0; c < n * 3; ++c) my_row[c] = 0.0f;
@@ -434,6 +495,27 @@ __global__ void __launch_bounds__(256) gs3d_preprocess_backward_kernel(int P, in
         if (g_sh_rest)
           for (int c = 0; c < n_sh * 3; ++c) g_sh_rest[(size_t) i * n_sh * 3 + c] = 0.0f;
       }
+    }
+  }
+  if (g_Tw2v || g_campos) {
+    // sums over the wavefront, then one atomic per value and wavefront (the reference: one per value and block,
+    // gaussian_preprocess.cu:340-355); rows of invisible points contribute zeros
+#pragma unroll
+    for (int k = 0; k < 15; ++k) {
+      float v = cam[k];
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+      cam[k] = v;
+    }
+    if ((threadIdx.x & 63) == 0) {
+      if (g_Tw2v)
+#pragma unroll
+        for (int k = 0; k < 12; ++k)
+          if (cam[k] != 0.0f) atomicAdd(&g_Tw2v[k], cam[k]);
+      if (g_campos)
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+          if (cam[12 + k] != 0.0f) atomicAdd(&g_campos[k], cam[12 + k]);
     }
   }
   if (kWave) {
@@ -490,22 +572,36 @@ __global__ void __launch_bounds__(256) cov2d_forward_kernel(int N, const float* 
 
 __global__ void __launch_bounds__(256) cov2d_backward_kernel(int N, const float* __restrict__ cov3D,
     const float* __restrict__ mean, const float* __restrict__ Tw2v, float fx, float fy, float tanx, float tany,
-    const float* __restrict__ g, float* __restrict__ g_cov3D, float* __restrict__ g_mean) {
+    const float* __restrict__ g, float* __restrict__ g_cov3D, float* __restrict__ g_mean, float* __restrict__ g_vm) {
   const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= N) return;
-  float V[16], c3[6], gc[6], gm[3];
+  float vm[12];
 #pragma unroll
-  for (int k = 0; k < 16; ++k) V[k] = Tw2v[k];
+  for (int k = 0; k < 12; ++k) vm[k] = 0.0f;
+  if (i < N) {
+    float V[16], c3[6], gc[6], gm[3];
 #pragma unroll
-  for (int k = 0; k < 6; ++k) c3[k] = cov3D[6 * (size_t) i + k];
-  const float p[3] = {mean[3 * (size_t) i], mean[3 * (size_t) i + 1], mean[3 * (size_t) i + 2]};
-  Cov2DTerms t;
-  cov2d_terms(p, fx, fy, tanx, tany, V, t);
-  cov2d_backward_cov(t, c3, fx, fy, V, g[3 * (size_t) i], g[3 * (size_t) i + 1], g[3 * (size_t) i + 2], gc, gm);
+    for (int k = 0; k < 16; ++k) V[k] = Tw2v[k];
 #pragma unroll
-  for (int k = 0; k < 6; ++k) g_cov3D[6 * (size_t) i + k] = gc[k];
+    for (int k = 0; k < 6; ++k) c3[k] = cov3D[6 * (size_t) i + k];
+    const float p[3] = {mean[3 * (size_t) i], mean[3 * (size_t) i + 1], mean[3 * (size_t) i + 2]};
+    Cov2DTerms t;
+    cov2d_terms(p, fx, fy, tanx, tany, V, t);
+    cov2d_backward_cov(t, p, c3, fx, fy, V, g[3 * (size_t) i], g[3 * (size_t) i + 1], g[3 * (size_t) i + 2], gc, gm,
+                       g_vm ? vm : nullptr);
 #pragma unroll
-  for (int k = 0; k < 3; ++k) g_mean[3 * (size_t) i + k] = gm[k];
+    for (int k = 0; k < 6; ++k) g_cov3D[6 * (size_t) i + k] = gc[k];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) g_mean[3 * (size_t) i + k] = gm[k];
+  }
+  if (g_vm) {  // gaussian_compute_cov2D.cu:223-227: added to the caller's buffer
+#pragma unroll
+    for (int k = 0; k < 12; ++k) {
+      float v = vm[k];
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+      if ((threadIdx.x & 63) == 0 && v != 0.0f) atomicAdd(&g_vm[k], v);
+    }
+  }
 }
 
 }  // namespace
@@ -544,21 +640,22 @@ FSGS_API int fsgs_gs_compute_cov2D_forward(int N, const float* cov3D, const floa
 
 FSGS_API int fsgs_gs_compute_cov2D_backward(int N, const float* cov3D, const float* mean, const float* Tw2v,
     double focal_x, double focal_y, double tan_fovx, double tan_fovy, const float* g_cov2D, float* g_cov3D,
-    float* g_mean, void* stream) {
+    float* g_mean, float* g_vm, void* stream) {
   FSGS_REQUIRE(N >= 0, "gs_compute_cov2D_backward: bad size");
   if (N == 0) return kOk;
   FSGS_REQUIRE(cov3D && mean && Tw2v && g_cov2D && g_cov3D && g_mean, "gs_compute_cov2D_backward: null pointer");
   hipLaunchKernelGGL(cov2d_backward_kernel, dim3(div_up(N, 256)), dim3(256), 0, (hipStream_t) stream, N, cov3D, mean,
                      Tw2v, (float) focal_x, (float) focal_y, (float) tan_fovx, (float) tan_fovy, g_cov2D, g_cov3D,
-                     g_mean);
+                     g_mean, g_vm);
   return check_launch("gs_compute_cov2D_backward");
 }
 
 FSGS_API int fsgs_gs_preprocess_forward(int P, int W, int H, int sh_degree, int n_sh, int is_opengl,
     const float* means3D, const float* scales, const float* rotations, const float* opacities, const float* shs,
     const float* sh_rest, const float* Tw2v, const float* Tv2c, const float* campos, double tan_fovx, double tan_fovy,
-    const uint8_t* culling, int means2D_preserve, float* means2D, float* depths, float* colors, int32_t* radii,
-    int32_t* tiles_touched, float* cov3Ds, float* conic_opacity, void* stream) {
+    const uint8_t* culling, const float* cov3D_precomp, const float* cov2D_precomp, int means2D_preserve,
+    float* means2D, float* depths, float* colors, int32_t* radii, int32_t* tiles_touched, float* cov3Ds,
+    float* conic_opacity, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && tan_fovx > 0 && tan_fovy > 0, "gs_preprocess_forward: bad sizes");
   FSGS_REQUIRE(sh_degree <= kMaxShDegree, "gs_preprocess_forward: sh_degree %d > %d not supported", sh_degree,
                kMaxShDegree);
@@ -567,7 +664,7 @@ FSGS_API int fsgs_gs_preprocess_forward(int P, int W, int H, int sh_degree, int 
                  "gs_preprocess_forward: %d SH coefficients are too few for degree %d", n_sh, sh_degree);
   if (P == 0) return kOk;
   FSGS_REQUIRE(means3D && scales && rotations && opacities && shs && Tw2v && Tv2c && campos && means2D && depths &&
-                   radii && tiles_touched && cov3Ds && conic_opacity && (colors || sh_degree < 0),
+                   radii && tiles_touched && (cov3Ds || cov3D_precomp) && conic_opacity && (colors || sh_degree < 0),
                "gs_preprocess_forward: null pointer");
   const bool wave_rows = sh_degree == 3 && n_sh == 16 && !sh_rest && (uintptr_t) shs % 16 == 0;
   auto kernel = sh_degree > 3 ? gs3d_preprocess_forward_kernel<64, false>
@@ -575,24 +672,27 @@ FSGS_API int fsgs_gs_preprocess_forward(int P, int W, int H, int sh_degree, int 
                                            : gs3d_preprocess_forward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh,
                      is_opengl, means3D, scales, (const float4*) rotations, opacities, shs, sh_rest, Tw2v, Tv2c,
-                     campos, (float) tan_fovx, (float) tan_fovy, culling, means2D_preserve, (float2*) means2D, depths,
-                     colors, radii, tiles_touched, cov3Ds, (float4*) conic_opacity);
+                     campos, (float) tan_fovx, (float) tan_fovy, culling, cov3D_precomp, cov2D_precomp, means2D_preserve,
+                     (float2*) means2D, depths, colors, radii, tiles_touched, cov3D_precomp ? nullptr : cov3Ds,
+                     (float4*) conic_opacity);
   return check_launch("gs_preprocess_forward");
 }
 
 FSGS_API int fsgs_gs_preprocess_backward(int P, int W, int H, int sh_degree, int n_sh, int is_opengl,
     const float* means3D, const float* scales, const float* rotations, const float* shs, const float* sh_rest,
     const float* Tw2v, const float* Tv2c, const float* campos, double tan_fovx, double tan_fovy, const int32_t* radii,
-    const float* colors, const float* cov3Ds, float* grad_mean2D, const float* grad_colors, const float* grad_conic,
-    float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs, float* g_sh_rest, float* g_cov3D,
-    void* stream) {
+    const float* colors, const float* cov3Ds, const float* cov2Ds, float* grad_mean2D, const float* grad_colors,
+    const float* grad_conic, float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs,
+    float* g_sh_rest, float* g_cov, float* g_Tw2v, float* g_campos, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && tan_fovx > 0 && tan_fovy > 0, "gs_preprocess_backward: bad sizes");
   FSGS_REQUIRE(sh_degree <= kMaxShDegree, "gs_preprocess_backward: sh_degree %d > %d not supported", sh_degree,
                kMaxShDegree);
   if (P == 0) return kOk;
-  FSGS_REQUIRE(means3D && scales && rotations && Tw2v && Tv2c && campos && radii && cov3Ds && grad_mean2D &&
-                   grad_conic && g_means3D && g_opac,
+  FSGS_REQUIRE(means3D && scales && rotations && Tw2v && Tv2c && campos && radii && (cov3Ds || cov2Ds) &&
+                   grad_mean2D && grad_conic && g_means3D && g_opac,
                "gs_preprocess_backward: null pointer");
+  FSGS_REQUIRE(!cov2Ds || (!g_scales && !g_rot),
+               "gs_preprocess_backward: no scale / rotation gradients with pre-computed 2D covariances");
   if (sh_degree >= 0)
     FSGS_REQUIRE(shs && colors && grad_colors, "gs_preprocess_backward: SH path needs shs, colors and grad_colors");
   const bool wave_rows = sh_degree == 3 && n_sh == 16 && !sh_rest && g_shs && (uintptr_t) shs % 16 == 0 &&
@@ -602,8 +702,8 @@ FSGS_API int fsgs_gs_preprocess_backward(int P, int W, int H, int sh_degree, int
                                            : gs3d_preprocess_backward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh,
                      is_opengl, means3D, scales, (const float4*) rotations, shs, sh_rest, Tw2v, Tv2c, campos,
-                     (float) tan_fovx, (float) tan_fovy, radii, colors, cov3Ds, (float2*) grad_mean2D, grad_colors,
-                     (const float4*) grad_conic, g_means3D, g_scales, (float4*) g_rot, g_opac, g_shs, g_sh_rest,
-                     g_cov3D);
+                     (float) tan_fovx, (float) tan_fovy, radii, colors, cov3Ds, cov2Ds, (float2*) grad_mean2D,
+                     grad_colors, (const float4*) grad_conic, g_means3D, g_scales, (float4*) g_rot, g_opac, g_shs,
+                     g_sh_rest, g_cov, g_Tw2v, g_campos);
   return check_launch("gs_preprocess_backward");
 }

@@ -1,8 +1,8 @@
 """Host side of the 3D-Gaussian (EWA) render path on the HIP operators: the autograd wiring and entry points of the
 reference's fast_2d_gs/renderer/gaussian_render.py (`_preprocess` :495-566, `preprocess` :569-, `GS_prepare` :742-772,
-`_GS_render` :775-800, `GS_render` :840-, `RasterizeGaussians` :226-274, `render` :277-359) for covariances computed
-from scales + rotations, and `_render_extra` / `render_extra` :925-962 for further feature tables of any width.
-Pre-computed covariances and camera gradients are not part of this build and raise."""
+`_GS_render` :775-800, `_GS_render_fast` :803-837, `GS_render` :840-, `RasterizeGaussians` :226-274, `render` :277-359),
+with covariances from scales + rotations or pre-computed (3D or 2D), gradients to the view matrix and the camera
+position, and `_render_extra` / `render_extra` :925-962 for further feature tables of any width."""
 from __future__ import annotations
 
 from typing import NamedTuple, Optional, Tuple
@@ -13,8 +13,8 @@ from torch import Tensor
 from fast_sp_gs_amd._C import get_C_function
 from fast_sp_gs_amd.renderer.gs_2d_render import GS_prepare
 
-__all__ = ['RasterizeBuffer3D', 'preprocess', 'GS_render', 'RasterizeGaussians', 'render', 'compute_cov3D',
-           'compute_cov2D', 'topk_weights', 'render_extra']
+__all__ = ['RasterizeBuffer3D', 'preprocess', 'GS_render', 'GS_render_fast', 'RasterizeGaussians', 'render',
+           'compute_cov3D', 'compute_cov2D', 'topk_weights', 'render_extra']
 
 
 class RasterizeBuffer3D(NamedTuple):
@@ -96,7 +96,7 @@ def compute_cov3D(scaling: Tensor, rotation: Tensor) -> Tensor:
 
 
 class _compute_cov2D(torch.autograd.Function):
-    """renderer/gaussian_render.py:427-447 of the reference; the view matrix gets no gradient here."""
+    """renderer/gaussian_render.py:427-447 of the reference."""
 
     @staticmethod
     def forward(ctx, means, cov3D, Tw2v, fx, fy, tx, ty):
@@ -109,11 +109,10 @@ class _compute_cov2D(torch.autograd.Function):
     @torch.autograd.function.once_differentiable
     def backward(ctx, grad_cov2D):
         cov3D, means, Tw2v = ctx.saved_tensors
-        if ctx.needs_input_grad[2]:
-            raise RuntimeError('compute_cov2D: the gradient to the view matrix is not supported')
+        grad_Tw2v = torch.zeros_like(Tw2v) if ctx.needs_input_grad[2] else None
         grad_cov3D, grad_mean = get_C_function('gs_compute_cov2D_backward')(cov3D, means, Tw2v, *ctx.focal_fov,
-                                                                           grad_cov2D)
-        return grad_mean, grad_cov3D, None, None, None, None, None
+                                                                           grad_cov2D, grad_Tw2v)
+        return grad_mean, grad_cov3D, grad_Tw2v, None, None, None, None
 
 
 def compute_cov2D(means: Tensor, cov3D: Tensor, Tw2v: Tensor, focal_x: float, focal_y: float, tan_fovx: float,
@@ -129,26 +128,23 @@ class _preprocess(torch.autograd.Function):
     @staticmethod
     def forward(ctx, means3D, scales, rotations, opacities, sh_or_colors, sh_rest, Tw2v, Tv2c, campos, tanFoV, W, H,
                 sh_degree, is_opengl, cov3D, cov2D, means2D, culling):
-        if cov3D is not None or cov2D is not None:
-            raise RuntimeError('pre-computed covariances are not supported by this library')
         tan = (float(tanFoV[0]), float(tanFoV[1]))
-        ctx._args = (W, H, sh_degree, is_opengl, tan)
+        ctx._args = (W, H, sh_degree, is_opengl, tan, cov3D is not None)
+        c = lambda t: None if t is None else t.contiguous()
         means2D, depths, colors, radii, tiles_touched, cov3D, conic_opacity = _preprocess._forward(
             W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, sh_or_colors, sh_rest, Tw2v, Tv2c,
-            campos, tan, None, None, means2D, culling)
+            campos, tan, c(cov3D), c(cov2D), means2D, culling)
         ctx.save_for_backward(means3D, scales, rotations, opacities, sh_or_colors, sh_rest, Tw2v, Tv2c, campos, cov3D,
-                              radii, colors)
+                              c(cov2D), radii, colors)
         ctx.mark_non_differentiable(radii, tiles_touched)
         return means2D, depths, colors, radii, tiles_touched, conic_opacity
 
     @staticmethod
     @torch.autograd.function.once_differentiable
     def backward(ctx, g_means2D, g_depths, g_colors, _g_radii, _g_tiles, g_conic):
-        means3D, scales, rotations, opacities, sh_or_colors, sh_rest, Tw2v, Tv2c, campos, cov3D, radii, colors = \
-            ctx.saved_tensors
-        W, H, sh_degree, is_opengl, tan = ctx._args
-        if ctx.needs_input_grad[6] or ctx.needs_input_grad[8]:
-            raise RuntimeError('camera gradients are not supported by this library')
+        (means3D, scales, rotations, opacities, sh_or_colors, sh_rest, Tw2v, Tv2c, campos, cov3D, cov2D, radii,
+         colors) = ctx.saved_tensors
+        W, H, sh_degree, is_opengl, tan, has_cov3D = ctx._args
         P = means3D.shape[0]
         zeros = lambda *shape: torch.zeros(shape, dtype=torch.float32, device=means3D.device)
         g_means2D = zeros(P, 2) if g_means2D is None else g_means2D.contiguous().clone()
@@ -156,16 +152,30 @@ class _preprocess(torch.autograd.Function):
         g_colors = zeros(P, 3) if g_colors is None else g_colors.contiguous()
         # every row of these is assigned by the kernel
         grad_means3D, grad_opacities = torch.empty_like(means3D), torch.empty_like(opacities)
-        grad_scales = torch.empty_like(scales) if ctx.needs_input_grad[1] else None
-        grad_rotations = torch.empty_like(rotations) if ctx.needs_input_grad[2] else None
+        grad_scales = grad_rotations = grad_cov = None
+        # which covariance was given decides where its gradient goes (gaussian_render.py:532-541 of the reference)
+        if cov2D is not None:
+            grad_cov = torch.empty_like(cov2D) if ctx.needs_input_grad[15] else None
+        elif has_cov3D:
+            grad_cov = torch.empty_like(cov3D) if ctx.needs_input_grad[14] else None
+        else:
+            grad_scales = torch.empty_like(scales) if ctx.needs_input_grad[1] else None
+            grad_rotations = torch.empty_like(rotations) if ctx.needs_input_grad[2] else None
         grad_shs = torch.empty_like(sh_or_colors) if sh_degree >= 0 and ctx.needs_input_grad[4] else None
         grad_sh_rest = torch.empty_like(sh_rest) if (sh_degree >= 0 and sh_rest is not None and
                                                      ctx.needs_input_grad[5]) else None
+        grad_Tw2v = torch.zeros_like(Tw2v) if ctx.needs_input_grad[6] else None  # these two are accumulated into
+        grad_campos = torch.zeros_like(campos) if ctx.needs_input_grad[8] else None
         _preprocess._backward(W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, sh_or_colors, sh_rest,
-                              Tw2v, Tv2c, campos, tan, cov3D, None, radii, colors, g_means2D, None, g_colors, g_conic,
-                              grad_means3D, grad_scales, grad_rotations, grad_opacities, grad_shs, grad_sh_rest, None,
-                              None, None)
-        grad_inputs = [grad_means3D, grad_scales, grad_rotations, grad_opacities, grad_shs, grad_sh_rest] + [None] * 12
+                              Tw2v, Tv2c, campos, tan, cov3D, cov2D, radii, colors, g_means2D, None, g_colors, g_conic,
+                              grad_means3D, grad_scales, grad_rotations, grad_opacities, grad_shs, grad_sh_rest,
+                              grad_cov, grad_Tw2v, grad_campos)
+        grad_inputs = [grad_means3D, grad_scales, grad_rotations, grad_opacities, grad_shs, grad_sh_rest,
+                       grad_Tw2v, None, grad_campos] + [None] * 9
+        if cov2D is not None:
+            grad_inputs[15] = grad_cov
+        elif has_cov3D:
+            grad_inputs[14] = grad_cov
         if sh_degree < 0:
             grad_inputs[4] = g_colors if ctx.needs_input_grad[4] else None  # pre-computed colours pass through
         # the dummy screen-space leaf receives the (rewritten) screen-space gradient: it is what densification reads
@@ -210,6 +220,51 @@ class _GS_render(torch.autograd.Function):
             mean2D, conic_opacity, colors, extras, out_opacity, grad_images.contiguous(), grad_alpha.contiguous(),
             None if grad_out_extra is None else grad_out_extra.contiguous(), tile_range, point_list, n_contrib)
         return None, None, grad_means2D, grad_colors, grad_conic_opacity, None, None, grad_extra, None, None, None
+
+
+class _GS_render_fast(torch.autograd.Function):
+    """The reference's bucketed variant (gaussian_render.py:803-837): the forward also stores the running state before
+    every 32nd list entry, the backward is `gaussian_rasterize_fast_backward` on those snapshots."""
+    _forward = get_C_function('gaussian_rasterize_forward')
+    _backward = get_C_function('gaussian_rasterize_fast_backward')
+
+    @staticmethod
+    def forward(ctx, W, H, mean2D, colors, conic_opacity, tile_range, point_list, extras, accum_max_count,
+                accum_weights_p, accum_weights_count):
+        per_tile_bucket_offset = (tile_range[..., 1] - tile_range[..., 0] + 31) // 32
+        per_tile_bucket_offset = torch.cumsum(per_tile_bucket_offset, dim=-1).contiguous()
+        (images, out_opacity, out_extras, n_contrib, max_contrib, bucket_to_tile, sampled_T,
+         sampled_ar) = _GS_render_fast._forward(W, H, mean2D, conic_opacity, colors, extras, point_list, tile_range,
+                                                accum_max_count, accum_weights_p, accum_weights_count,
+                                                per_tile_bucket_offset)
+        ctx.save_for_backward(mean2D, colors, conic_opacity, extras, tile_range, point_list, images, out_opacity,
+                              out_extras, n_contrib, per_tile_bucket_offset, max_contrib, bucket_to_tile, sampled_T,
+                              sampled_ar)
+        ctx.mark_non_differentiable(n_contrib)
+        return images, out_opacity, out_extras, n_contrib
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_images, grad_alpha, grad_out_extra, _):
+        (mean2D, colors, conic_opacity, extras, tile_range, point_list, images, out_opacity, out_extras, n_contrib,
+         per_tile_bucket_offset, max_contrib, bucket_to_tile, sampled_T, sampled_ar) = ctx.saved_tensors
+        grad_images = torch.zeros_like(images) if grad_images is None else grad_images
+        grad_alpha = torch.zeros_like(out_opacity) if grad_alpha is None else grad_alpha
+        if extras is not None and grad_out_extra is None:
+            grad_out_extra = torch.zeros_like(out_extras)
+        grad_colors, grad_extra, grad_means2D, grad_conic_opacity = _GS_render_fast._backward(
+            mean2D, conic_opacity, colors, extras, images, out_extras, out_opacity, grad_images.contiguous(),
+            grad_alpha.contiguous(), None if grad_out_extra is None else grad_out_extra.contiguous(), tile_range,
+            point_list, n_contrib, max_contrib, per_tile_bucket_offset, bucket_to_tile, sampled_T, sampled_ar)
+        return None, None, grad_means2D, grad_colors, grad_conic_opacity, None, None, grad_extra, None, None, None
+
+
+def GS_render_fast(W: int, H: int, mean2D: Tensor, colors: Tensor, conic_opacity: Tensor, tile_range: Tensor,
+                   point_list: Tensor, extra: Tensor = None, accum_max_count=None, accum_weights_p=None,
+                   accum_weights_count=None):
+    """`GS_render` through the bucketed forward / per-Gaussian backward pair (gaussian_render.py:803-837)."""
+    return _GS_render_fast.apply(W, H, mean2D, colors, conic_opacity, tile_range, point_list, extra, accum_max_count,
+                                 accum_weights_p, accum_weights_count)
 
 
 def GS_render(W: int, H: int, mean2D: Tensor, colors: Tensor, conic_opacity: Tensor, tile_range: Tensor,

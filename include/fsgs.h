@@ -300,25 +300,30 @@ int fsgs_knn_topk_backward(int N, int M, int D, int K, const float* x, const flo
  * scales[P,3], rotations[P,4] (x,y,z,w, used as given), opacities[P,1], shs[P,n_sh,3] (or shs[P,1,3] + sh_rest, or
  * colours[P,3] with sh_degree < 0), Tw2v, Tv2c [4,4], campos[3], tan(FoV/2) per axis -> means2D[P,2] (pixel - 0.5
  * convention unless is_opengl), depths[P], colors[P,3], radii[P], tiles_touched[P], cov3Ds[P,6], conic_opacity[P,4].
- * Covariances always come from scales + rotations (the reference's cov3D_precomp / cov2D_precomp inputs are not
- * implemented). Every row of every output is written; means2D_preserve keeps the caller's means2D rows of Gaussians
- * that are not rendered. culling: optional P bytes, non-zero = skip. */
+ * cov3D_precomp[P,6] (optional) replaces R S^2 R^T (cov3Ds is then not written and may be NULL: the reference's host
+ * returns the pre-computed tensor itself, :424); cov2D_precomp[P,3] (optional) is used as the 2D covariance as it is,
+ * without the 0.3 low-pass term (:76-78). Every row of every output is written; means2D_preserve keeps the caller's
+ * means2D rows of Gaussians that are not rendered. culling: optional P bytes, non-zero = skip. */
 int fsgs_gs_preprocess_forward(int P, int W, int H, int sh_degree, int n_sh, int is_opengl, const float* means3D,
     const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
     const float* Tw2v, const float* Tv2c, const float* campos, double tan_fovx, double tan_fovy,
-    const uint8_t* culling, int means2D_preserve, float* means2D, float* depths, float* colors, int32_t* radii,
-    int32_t* tiles_touched, float* cov3Ds, float* conic_opacity, void* stream);
+    const uint8_t* culling, const float* cov3D_precomp, const float* cov2D_precomp, int means2D_preserve,
+    float* means2D, float* depths, float* colors, int32_t* radii, int32_t* tiles_touched, float* cov3Ds,
+    float* conic_opacity, void* stream);
 
 /* gs_preprocess_backward -- gaussian_preprocess.cu:567-636 (kernel :246-372, with gaussian_compute_cov2D.cu:64-186 and
  * gaussian_compute_cov3D.cu:76-118). grad_mean2D[P,2] is rewritten in place as (0.5 W g.x, +-0.5 H g.y) as in the
  * reference; grad_conic[P,4] carries dL/dconic and dL/dopacity. All gradient rows are assigned (zeros for Gaussians
- * that were not rendered). g_scales, g_rot, g_shs, g_sh_rest, g_cov3D are optional. No camera gradients. */
+ * that were not rendered). g_scales, g_rot, g_shs, g_sh_rest, g_cov are optional. cov3Ds[P,6] is the forward's output
+ * (or the caller's pre-computed tensor) and g_cov is [P,6]; with cov2Ds[P,3] (the caller's pre-computed 2D covariances,
+ * :293-301) g_cov is [P,3], nothing reaches the means through the covariance and g_scales / g_rot must be NULL.
+ * g_Tw2v[4,4] (rows 0-2) and g_campos[3] (optional, :271, :318-355) are ADDED to, with float atomics. */
 int fsgs_gs_preprocess_backward(int P, int W, int H, int sh_degree, int n_sh, int is_opengl, const float* means3D,
     const float* scales, const float* rotations, const float* shs, const float* sh_rest, const float* Tw2v,
     const float* Tv2c, const float* campos, double tan_fovx, double tan_fovy, const int32_t* radii,
-    const float* colors, const float* cov3Ds, float* grad_mean2D, const float* grad_colors, const float* grad_conic,
-    float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs, float* g_sh_rest, float* g_cov3D,
-    void* stream);
+    const float* colors, const float* cov3Ds, const float* cov2Ds, float* grad_mean2D, const float* grad_colors,
+    const float* grad_conic, float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs,
+    float* g_sh_rest, float* g_cov, float* g_Tw2v, float* g_campos, void* stream);
 
 /* gaussian_topk_weights -- fast_2d_gs/_C/src/gaussian_splatting/gaussian_topk.cu:212-228 (kernel :12-93): per pixel
  * the topk (<= 16) largest blend weights of the 3D-Gaussian rasteriser and their Gaussian ids, descending;
@@ -350,25 +355,43 @@ int fsgs_gs_compute_cov3D_backward(int N, const float* q, const float* s, const 
 
 /* gs_compute_cov2D_forward / gs_compute_cov2D_backward -- gaussian_compute_cov2D.cu:186-248: cov2D[N,3] = (a, b, c) of
  * J W cov3D W^T J^T + 0.3 I with the view-space mean clamped to 1.3 x the field of view (W = rotation block of the
- * row-major Tw2v[4,4]); the backward takes dL/dcov2D[N,3] and writes g_cov3D[N,6] and g_mean[N,3] in full. The
- * reference's optional gradient to the view matrix is not produced. */
+ * row-major Tw2v[4,4]); the backward takes dL/dcov2D[N,3] and writes g_cov3D[N,6] and g_mean[N,3] in full; g_vm[4,4]
+ * (optional, :163-183, :223-227) gets the view matrix's gradient ADDED to its rows 0-2 with float atomics. */
 int fsgs_gs_compute_cov2D_forward(int N, const float* cov3D, const float* mean, const float* Tw2v, double focal_x,
     double focal_y, double tan_fovx, double tan_fovy, float* cov2D, void* stream);
 int fsgs_gs_compute_cov2D_backward(int N, const float* cov3D, const float* mean, const float* Tw2v, double focal_x,
-    double focal_y, double tan_fovx, double tan_fovy, const float* g_cov2D, float* g_cov3D, float* g_mean, void* stream);
+    double focal_y, double tan_fovx, double tan_fovy, const float* g_cov2D, float* g_cov3D, float* g_mean,
+    float* g_vm, void* stream);
 
-/* gaussian_rasterize_forward -- gaussian_render.cu:212-293 (kernel :20-173) without the bucket snapshots of the
- * per-Gaussian backward. colors[P,3], extras[P,E] (E <= 4, optional) -> out_color[3,H,W], out_opacity[H,W],
- * out_extras[E,H,W], n_contrib[H,W]; every output element is written. accum_* as in the surfel forward. */
+/* gaussian_rasterize_forward -- gaussian_render.cu:212-293 (kernel :20-173). colors[P,3], extras[P,E] (E <= 4,
+ * optional) -> out_color[3,H,W], out_opacity[H,W], out_extras[E,H,W], n_contrib[H,W]; every output element is written.
+ * accum_weights_* as in the surfel forward; accum_max_count gets one count per pixel, for the Gaussian with the
+ * largest weight (:166). With bucket_offset[T] (inclusive cumsum of ceil(len / 32) per tile) also max_contrib[T],
+ * bucket_to_tile[B], sampled_T[B,256], sampled_ar[B,3+E,256]: the state before every 32nd list entry for pixels still
+ * blending (the extra channels' running sums in channels 3.., where the reference indexes its colour array past its
+ * end, :103). */
 int fsgs_gaussian_rasterize_forward(int P, int W, int H, int E, const float* means2D, const float* conic_opacity,
     const float* colors, const float* extras, const int32_t* point_list, const int64_t* ranges,
-    int32_t* accum_max_count, float* accum_weights_p, int32_t* accum_weights_count, float* out_color,
-    float* out_opacity, float* out_extras, int32_t* n_contrib, void* stream);
+    int32_t* accum_max_count, float* accum_weights_p, int32_t* accum_weights_count, const int64_t* bucket_offset,
+    float* out_color, float* out_opacity, float* out_extras, int32_t* n_contrib, int32_t* max_contrib,
+    int32_t* bucket_to_tile, float* sampled_T, float* sampled_ar, void* stream);
 
 /* gaussian_rasterize_backward -- gaussian_render.cu:486-536 (kernel :296-444). Accumulates into caller-zeroed
  * g_means2D[P,2], g_conic_opacity[P,4], g_colors[P,3], g_extras[P,E]. */
 int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const float* means2D, const float* conic_opacity,
     const float* colors, const float* extras, const float* out_opacity, const int32_t* n_contrib,
+    const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
+    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, void* stream);
+
+/* gaussian_rasterize_fast_backward -- gaussian_render.cu:760-812 (kernel :540-694): the reference's per-Gaussian
+ * backward over the forward's bucket snapshots. It is the same derivative as gaussian_rasterize_backward and runs
+ * that kernel here; the snapshot arguments must be present but are not read. With E > 0 the reference reads the extra
+ * channels' upstream gradient into the wrong registers (:636); the gradient of what the forward computes is returned.
+ * Outputs caller-zeroed as above. */
+int fsgs_gaussian_rasterize_fast_backward(int P, int W, int H, int E, const float* means2D,
+    const float* conic_opacity, const float* colors, const float* extras, const float* images,
+    const float* out_extras, const float* out_opacity, const int32_t* n_contrib, const int32_t* max_contrib,
+    const int64_t* bucket_offset, const int32_t* bucket_to_tile, const float* sampled_T, const float* sampled_ar,
     const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
     const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, void* stream);
 

@@ -250,38 +250,47 @@ def fast_render_backward(near, far, per_splat_form, means2D, normal_opacity, col
 
 # ---- 3D-Gaussian (EWA) path ------------------------------------------------------------------------------------------
 def gs3d_preprocess_forward(W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs, sh_rest, Tw2v,
-                            Tv2c, campos, tan_fov, culling=None, means2D=None):
+                            Tv2c, campos, tan_fov, culling=None, means2D=None, cov3D_precomp=None,
+                            cov2D_precomp=None):
     dt = means3D.dtype
     P = means3D.shape[0]
     n_sh = 0 if sh_degree < 0 else (sh_rest.shape[1] if sh_rest is not None else shs.shape[1])
     m2 = np.zeros((P, 2), dt) if means2D is None else means2D
-    depths, cov3D, conic = np.zeros((P,), dt), np.zeros((P, 6), dt), np.zeros((P, 4), dt)
+    depths, conic = np.zeros((P,), dt), np.zeros((P, 4), dt)
+    cov3D = cov3D_precomp if cov3D_precomp is not None else np.zeros((P, 6), dt)  # the host returns the input itself
     colors = np.zeros((P, 3), dt) if sh_degree >= 0 else shs
     radii, tt = np.zeros((P,), np.int32), np.zeros((P,), np.int32)
     cull = None if culling is None else np.ascontiguousarray(culling.astype(np.uint8))
     rc = call(f"gs3d_preprocess_forward_{_suffix(dt)}", P, W, H, sh_degree, n_sh, int(is_opengl), means3D, scales,
-              rotations, opacities, shs, sh_rest, Tw2v, Tv2c, campos, float(tan_fov[0]), float(tan_fov[1]), cull, m2,
-              depths, colors, radii, tt, cov3D, conic)
+              rotations, opacities, shs, sh_rest, Tw2v, Tv2c, campos, float(tan_fov[0]), float(tan_fov[1]), cull,
+              cov3D_precomp, cov2D_precomp, m2, depths, colors, radii, tt, cov3D, conic)
     assert rc == 0
     return m2, depths, colors, radii, tt, cov3D, conic
 
 
 def gs3d_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotations, shs, sh_rest, Tw2v, Tv2c, campos,
-                             tan_fov, radii, colors, cov3D, grad_mean2D, grad_colors, grad_conic):
-    """-> (g_means3D, g_scales, g_rot, g_opac, g_shs, g_sh_rest, g_cov3D, grad_mean2D rewritten)"""
+                             tan_fov, radii, colors, cov3D, grad_mean2D, grad_colors, grad_conic, cov2D=None,
+                             precomputed=False, camera=False):
+    """-> (g_means3D, g_scales, g_rot, g_opac, g_shs, g_sh_rest, g_cov, grad_mean2D rewritten) and, with `camera`,
+    (g_Tw2v[4,4], g_campos[3]) appended. `cov2D` (pre-computed 2D covariances): g_cov is [P,3]; `precomputed` (cov3D or
+    cov2D given by the caller): no scale / rotation gradients, as the reference's wrapper passes None for them."""
     dt = means3D.dtype
     P = means3D.shape[0]
     n_sh = 0 if sh_degree < 0 else (sh_rest.shape[1] if sh_rest is not None else shs.shape[1])
-    g3, gs, gq, go = np.zeros((P, 3), dt), np.zeros((P, 3), dt), np.zeros((P, 4), dt), np.zeros((P, 1), dt)
+    g3, go = np.zeros((P, 3), dt), np.zeros((P, 1), dt)
+    no_sr = precomputed or cov2D is not None
+    gs, gq = (None, None) if no_sr else (np.zeros((P, 3), dt), np.zeros((P, 4), dt))
     gsh = np.zeros_like(shs) if sh_degree >= 0 else None
     grest = np.zeros_like(sh_rest) if (sh_degree >= 0 and sh_rest is not None) else None
-    gcov = np.zeros((P, 6), dt)
+    gcov = np.zeros((P, 3 if cov2D is not None else 6), dt)
     gm2 = np.ascontiguousarray(grad_mean2D.copy())
+    gv, gcam = (np.zeros((4, 4), dt), np.zeros((3,), dt)) if camera else (None, None)
     rc = call(f"gs3d_preprocess_backward_{_suffix(dt)}", P, W, H, sh_degree, n_sh, int(is_opengl), means3D, scales,
               rotations, shs, sh_rest, Tw2v, Tv2c, campos, float(tan_fov[0]), float(tan_fov[1]), radii, colors, cov3D,
-              gm2, grad_colors, grad_conic, g3, gs, gq, go, gsh, grest, gcov)
+              cov2D, gm2, grad_colors, grad_conic, g3, gs, gq, go, gsh, grest, gcov, gv, gcam)
     assert rc == 0
-    return g3, gs, gq, go, gsh, grest, gcov, gm2
+    out = (g3, gs, gq, go, gsh, grest, gcov, gm2)
+    return out + (gv, gcam) if camera else out
 
 
 def gs3d_extra_forward(W, H, extras, means2D, conic_opacity, ranges, point_list, n_contrib):
@@ -341,26 +350,51 @@ def gs3d_compute_cov2D(cov3D, mean, Tw2v, fx, fy, tanx, tany):
     return out
 
 
-def gs3d_compute_cov2D_backward(cov3D, mean, Tw2v, fx, fy, tanx, tany, g):
-    """gs_compute_cov2D_backward -> (grad_cov3D, grad_mean), no view-matrix gradient (gaussian_compute_cov2D.cu:229-248)."""
+def gs3d_compute_cov2D_backward(cov3D, mean, Tw2v, fx, fy, tanx, tany, g, grad_vm=None):
+    """gs_compute_cov2D_backward -> (grad_cov3D, grad_mean); with grad_vm[4,4] the view matrix's gradient is added to
+    its first three rows (gaussian_compute_cov2D.cu:229-248)."""
     N = mean.shape[0]
     gc, gm = np.zeros((N, 6), mean.dtype), np.zeros((N, 3), mean.dtype)
     assert call(f"gs3d_compute_cov2D_backward_{_suffix(mean.dtype)}", N, cov3D, mean, Tw2v, float(fx), float(fy),
-                float(tanx), float(tany), g, gc, gm) == 0
+                float(tanx), float(tany), g, gc, gm, grad_vm) == 0
     return gc, gm
 
 
 def gs3d_render_forward(W, H, means2D, conic_opacity, colors, extras, point_list, ranges, accum_max_count=None,
-                        accum_weights_p=None, accum_weights_count=None):
+                        accum_weights_p=None, accum_weights_count=None, bucket_offset=None):
+    """-> (colors, opacity, extras, n_contrib) and, with bucket_offset, (max_contrib[T], bucket_to_tile[B],
+    sampled_T[B,256], sampled_ar[B,3+E,256]) appended."""
     dt = means2D.dtype
     E = 0 if extras is None else extras.shape[1]
     oc, oo = np.zeros((3, H, W), dt), np.zeros((H, W), dt)
     oe = np.zeros((E, H, W), dt) if E else None
     nc = np.zeros((H, W), np.int32)
+    snap = [None] * 4
+    if bucket_offset is not None:
+        B = int(bucket_offset[-1]) if bucket_offset.size else 0
+        snap = [np.zeros((ranges.shape[0],), np.int32), np.zeros((B,), np.int32), np.zeros((B, 256), dt),
+                np.zeros((B, 3 + E, 256), dt)]
     rc = call(f"gs3d_render_forward_{_suffix(dt)}", W, H, E, means2D, conic_opacity, colors, extras, point_list, ranges,
-              oc, oo, oe, nc, accum_max_count, accum_weights_p, accum_weights_count)
+              oc, oo, oe, nc, accum_max_count, accum_weights_p, accum_weights_count, bucket_offset, *snap)
     assert rc == 0
-    return oc, oo, oe, nc
+    return (oc, oo, oe, nc) + (tuple(snap) if bucket_offset is not None else ())
+
+
+def gs3d_render_fast_backward(W, H, means2D, conic_opacity, colors, extras, images, out_extras, out_opacity, n_contrib,
+                              max_contrib, bucket_offset, bucket_to_tile, sampled_T, sampled_ar, dL_dpix, dL_dextras,
+                              dL_dopacity, point_list, ranges):
+    """gaussian_rasterize_fast_backward -> (g_colors, g_extras, g_means2D, g_conic_opacity)"""
+    dt = means2D.dtype
+    P = means2D.shape[0]
+    E = 0 if extras is None else extras.shape[1]
+    gm, gc, gcol = np.zeros((P, 2), dt), np.zeros((P, 4), dt), np.zeros((P, 3), dt)
+    gex = np.zeros((P, E), dt) if E else None
+    B = int(bucket_offset[-1]) if bucket_offset.size else 0
+    rc = call(f"gs3d_render_fast_backward_{_suffix(dt)}", W, H, E, means2D, conic_opacity, colors, extras, images,
+              out_extras, out_opacity, n_contrib, max_contrib, bucket_offset, bucket_to_tile, sampled_T, sampled_ar,
+              dL_dpix, dL_dextras, dL_dopacity, point_list, ranges, B, gm, gc, gcol, gex)
+    assert rc == 0
+    return gcol, gex, gm, gc
 
 
 def gs3d_render_backward(W, H, means2D, conic_opacity, colors, extras, out_opacity, n_contrib, dL_dpix, dL_dextras,

@@ -64,17 +64,25 @@ int oracle_simple_knn_f32(int P, const float* points, float* mean_dist2);
 int oracle_gs3d_preprocess_forward_f32(int P, int W, int H, int sh_degree, int n_sh, int is_opengl,
     const float* means3D, const float* scales, const float* rotations, const float* opacities, const float* shs,
     const float* sh_rest, const float* Tw2v, const float* Tv2c, const float* campos, double tanx, double tany,
-    const uint8_t* culling, float* means2D, float* depths, float* colors, int32_t* radii, int32_t* tiles_touched,
-    float* cov3Ds, float* conic_opacity);
+    const uint8_t* culling, const float* cov3D_precomp, const float* cov2D_precomp, float* means2D, float* depths,
+    float* colors, int32_t* radii, int32_t* tiles_touched, float* cov3Ds, float* conic_opacity);
 int oracle_gs3d_preprocess_backward_f32(int P, int W, int H, int sh_degree, int n_sh, int is_opengl,
     const float* means3D, const float* scales, const float* rotations, const float* shs, const float* sh_rest,
     const float* Tw2v, const float* Tv2c, const float* campos, double tanx, double tany, const int32_t* radii,
-    const float* colors, const float* cov3Ds, float* grad_mean2D, const float* grad_colors, const float* grad_conic,
-    float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs, float* g_sh_rest, float* g_cov3D);
+    const float* colors, const float* cov3Ds, const float* cov2Ds, float* grad_mean2D, const float* grad_colors,
+    const float* grad_conic, float* g_means3D, float* g_scales, float* g_rot, float* g_opac, float* g_shs,
+    float* g_sh_rest, float* g_cov3D, float* g_Tw2v, float* g_campos);
 int oracle_gs3d_render_forward_f32(int W, int H, int E, const float* means2D, const float* conic_opacity,
     const float* colors, const float* extras, const int32_t* point_list, const int64_t* ranges, float* out_color,
     float* out_opacity, float* out_extras, int32_t* n_contrib, int32_t* accum_max_count, float* accum_weights_p,
-    int32_t* accum_weights_count);
+    int32_t* accum_weights_count, const int64_t* bucket_offset, int32_t* max_contrib, int32_t* bucket_to_tile,
+    float* sampled_T, float* sampled_ar);
+int oracle_gs3d_render_fast_backward_f32(int W, int H, int E, const float* means2D, const float* conic_opacity,
+    const float* colors, const float* extras, const float* images, const float* out_extras, const float* out_opacity,
+    const int32_t* n_contrib, const int32_t* max_contrib, const int64_t* bucket_offset, const int32_t* bucket_to_tile,
+    const float* sampled_T, const float* sampled_ar, const float* dL_dpix, const float* dL_dout_extras,
+    const float* dL_dout_opacity, const int32_t* point_list, const int64_t* ranges, int64_t B, float* g_means2D,
+    float* g_conic_opacity, float* g_colors, float* g_extras);
 int oracle_gs3d_render_backward_f32(int W, int H, int E, const float* means2D, const float* conic_opacity,
     const float* colors, const float* extras, const float* out_opacity, const int32_t* n_contrib,
     const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
@@ -91,7 +99,7 @@ int oracle_gs3d_compute_cov3D_backward_f32(int N, const float* q, const float* s
 int oracle_gs3d_compute_cov2D_f32(int N, const float* cov3D, const float* mean, const float* Tw2v, double fx, double fy,
     double tanx, double tany, float* cov2D);
 int oracle_gs3d_compute_cov2D_backward_f32(int N, const float* cov3D, const float* mean, const float* Tw2v, double fx,
-    double fy, double tanx, double tany, const float* g, float* g_cov3D, float* g_mean);
+    double fy, double tanx, double tany, const float* g, float* g_cov3D, float* g_mean, float* g_vm);
 int64_t oracle_gs_prepare_count(int P, const int32_t* tiles_touched, int64_t* offsets);
 int oracle_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
     const int64_t* offsets, int64_t R, int64_t* ranges, int32_t* point_list, int64_t* keys_sorted_out);

@@ -309,8 +309,8 @@ def test_covariance_operators(device):
     g_cov3D, g_mean = f('gs_compute_cov2D_backward')(cov3D, d(means), d(Tw2v), fx, fy, tx, ty, d(g2))
     w3, wm = O.gs3d_compute_cov2D_backward(want, npy(means), npy(Tw2v), fx, fy, tx, ty, npy(g2))
     assert rel_err(npy(g_cov3D), w3) < 1e-5 and rel_err(npy(g_mean), wm) < 1e-5
-    with pytest.raises(RuntimeError):
-        f('gs_compute_cov2D_backward')(cov3D, d(means), d(Tw2v), fx, fy, tx, ty, d(g2), torch.zeros(4, 4, device=device))
+    with pytest.raises(RuntimeError):  # a view-matrix gradient buffer of the wrong size
+        f('gs_compute_cov2D_backward')(cov3D, d(means), d(Tw2v), fx, fy, tx, ty, d(g2), torch.zeros(3, 3, device=device))
 
     # autograd wrappers: scaling / rotation / means receive the chained gradients
     sa, qa, ma = d(s).requires_grad_(True), d(q).requires_grad_(True), d(means).requires_grad_(True)
@@ -319,3 +319,169 @@ def test_covariance_operators(device):
     c3g, wm2 = O.gs3d_compute_cov2D_backward(want, npy(means), npy(Tw2v), fx, fy, tx, ty, npy(g2))
     wq2, ws2 = O.gs3d_compute_cov3D_backward(npy(q), npy(s), c3g)
     assert rel_err(npy(ma.grad), wm2) < 1e-5 and rel_err(npy(qa.grad), wq2) < 1e-4 and rel_err(npy(sa.grad), ws2) < 1e-4
+
+
+def test_gs3d_precomputed_covariances_and_camera_gradients(device):
+    """gs_preprocess_forward / _backward with cov3D_precomp and cov2D_precomp (gaussian_preprocess.cu:76-92, :293-301),
+    and the gradients of the view matrix and the camera position (:271, :318-355), against the oracle; the autograd
+    entry `preprocess` hands the gradients to the right inputs."""
+    from fast_sp_gs_amd._C import get_C_function
+    from fast_sp_gs_amd.renderer.gaussian_render import compute_cov2D, compute_cov3D, preprocess
+    P, W, H = 4000, 160, 96
+    scene, scales, cam, tan_fov = _scene(P, W, H, 23, device)
+    d = lambda t: None if t is None else t.to(device).contiguous()
+    fwd = get_C_function('gs_preprocess_forward')
+    bwd = get_C_function('gs_preprocess_backward')
+    base_args = (W, H, 3, False, d(scene.means3D), d(scales), d(scene.rotations), d(scene.opacities), d(scene.shs),
+                 None, d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), tan_fov)
+    base = fwd(*base_args, None, None, None, None)
+    fx, fy = 0.5 * W / tan_fov[0], 0.5 * H / tan_fov[1]
+    cov3 = get_C_function('gs_compute_cov3D_forward')(d(scene.rotations), d(scales))
+    cov2 = get_C_function('gs_compute_cov2D_forward')(cov3, d(scene.means3D), d(cam.Tw2v), fx, fy, *tan_fov)
+    o3 = fwd(*base_args, cov3, None, None, None)
+    o2 = fwd(*base_args, None, cov2, None, None)
+    torch.cuda.synchronize()
+    assert o3[5].data_ptr() == cov3.data_ptr()  # the pre-computed tensor is handed back
+    n = lambda t: None if t is None else npy(t)
+    host = (W, H, 3, False, n(scene.means3D), n(scales), n(scene.rotations), n(scene.opacities), n(scene.shs), None,
+            n(cam.Tw2v), n(cam.Tv2c), n(cam.campos), tan_fov)
+    r3 = O.gs3d_preprocess_forward(*host, cov3D_precomp=n(cov3))
+    r2 = O.gs3d_preprocess_forward(*host, cov2D_precomp=n(cov2))
+    for got, ref, name in ((o3, r3, 'cov3D'), (o2, r2, 'cov2D')):
+        for k in (0, 1, 3, 4, 6):
+            assert np.array_equal(n(got[k]), ref[k]), (name, k)
+        assert abs_err(n(got[2]), ref[2]) < 2e-6
+        assert np.array_equal(n(got[3]), n(base[3]))  # same radii as from scales + rotations
+    assert not n(o2[5]).any()  # no 3D covariance is formed from a 2D one
+
+    # backward: the three covariance sources, camera gradients on the ordinary one
+    g = torch.Generator().manual_seed(7)
+    gm2, gcol, gco = torch.randn(P, 2, generator=g), torch.randn(P, 3, generator=g), torch.randn(P, 4, generator=g)
+    nan = lambda *shape: torch.full(shape, float('nan'), device=device)
+    rad, col = base[3], base[2]
+    bargs = (W, H, 3, False, d(scene.means3D), d(scales), d(scene.rotations), d(scene.opacities), d(scene.shs), None,
+             d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), tan_fov)
+    rargs = (W, H, 3, False, n(scene.means3D), n(scales), n(scene.rotations), n(scene.shs), None, n(cam.Tw2v),
+             n(cam.Tv2c), n(cam.campos), tan_fov, n(rad), n(col))
+    vis = n(rad) > 0
+    # (a) cov2D given: [P,3] gradient
+    g3, gop, gsh, gcov = nan(P, 3), nan(P, 1), nan(P, 16, 3), nan(P, 3)
+    bwd(*bargs, None, cov2, rad, col, d(gm2), None, d(gcol), d(gco), g3, None, None, gop, gsh, None, gcov)
+    ref = O.gs3d_preprocess_backward(*rargs, n(base[5]), n(gm2), n(gcol), n(gco), cov2D=n(cov2))
+    torch.cuda.synchronize()
+    for a, b, name in ((g3, ref[0], 'means3D'), (gcov, ref[6], 'cov2D'), (gsh, ref[4], 'shs')):
+        assert np.isfinite(n(a)).all() and rel_err(n(a), b) < 1e-5 and not n(a)[~vis].any(), name
+    with pytest.raises(RuntimeError):
+        bwd(*bargs, None, cov2, rad, col, d(gm2), None, d(gcol), d(gco), g3, nan(P, 3), None, gop, gsh, None, gcov)
+    # (b) cov3D given: [P,6] gradient, no scale / rotation outputs
+    g3b, gcov6 = nan(P, 3), nan(P, 6)
+    bwd(*bargs, cov3, None, rad, col, d(gm2), None, d(gcol), d(gco), g3b, None, None, gop, gsh, None, gcov6)
+    ref = O.gs3d_preprocess_backward(*rargs, n(cov3), n(gm2), n(gcol), n(gco), precomputed=True)
+    torch.cuda.synchronize()
+    assert rel_err(n(g3b), ref[0]) < 1e-5 and rel_err(n(gcov6), ref[6]) < 1e-5
+    # (c) camera gradients: added to the caller's buffers (start at 1 to show it)
+    g_vm, g_cam = torch.ones(4, 4, device=device), torch.ones(3, device=device)
+    g3c, gs, gq = nan(P, 3), nan(P, 3), nan(P, 4)
+    bwd(*bargs, base[5], None, rad, col, d(gm2), None, d(gcol), d(gco), g3c, gs, gq, gop, gsh, None, None, g_vm, g_cam)
+    ref = O.gs3d_preprocess_backward(*rargs, n(base[5]), n(gm2), n(gcol), n(gco), camera=True)
+    torch.cuda.synchronize()
+    r_vm, r_cam = ref[-2].astype(np.float64), ref[-1].astype(np.float64)
+    # sums over ~3000 points in float32, in a different order on each side
+    assert rel_err(n(g_vm) - 1.0, r_vm) < 1e-3 and np.all(n(g_vm)[3] == 1.0)
+    assert rel_err(n(g_cam) - 1.0, r_cam) < 1e-3 and np.abs(r_cam).max() > 0
+    assert rel_err(n(g3c), ref[0]) < 1e-5 and rel_err(n(gs), ref[1]) < 1e-5 and rel_err(n(gq), ref[2]) < 1e-5
+
+    # the stand-alone cov2D backward with the view-matrix gradient
+    g2 = torch.randn(P, 3, generator=g).to(device)
+    gvm = torch.zeros(4, 4, device=device)
+    gc3, gmean = get_C_function('gs_compute_cov2D_backward')(cov3, d(scene.means3D), d(cam.Tw2v), fx, fy, *tan_fov, g2,
+                                                             gvm)
+    torch.cuda.synchronize()
+    r_gvm = np.zeros((4, 4), np.float32)
+    r_gc3, r_gmean = O.gs3d_compute_cov2D_backward(n(cov3), n(scene.means3D), n(cam.Tw2v), fx, fy, *tan_fov, n(g2), r_gvm)
+    assert rel_err(n(gc3), r_gc3) < 1e-5 and rel_err(n(gmean), r_gmean) < 1e-5 and rel_err(n(gvm), r_gvm) < 1e-3
+
+    # autograd: the view matrix and the camera position as leaves; pre-computed covariances as leaves
+    Tw2v = d(cam.Tw2v).requires_grad_()
+    campos = d(cam.campos).requires_grad_()
+    means = d(scene.means3D).requires_grad_()
+    tan_t = torch.tensor(tan_fov)
+    out = preprocess(means, d(scales), d(scene.rotations), d(scene.opacities), d(scene.shs), None, Tw2v, d(cam.Tv2c),
+                     campos, tan_t, W, H, 3, False)
+    ((out[0] * d(gm2)).sum() + (out[2] * d(gcol)).sum() + (out[5] * d(gco)).sum()).backward()
+    assert rel_err(n(Tw2v.grad), r_vm) < 1e-3 and rel_err(n(campos.grad), r_cam) < 1e-3
+    assert rel_err(n(means.grad), ref[0]) < 1e-5
+    c2 = cov2.clone().requires_grad_()
+    out = preprocess(d(scene.means3D), d(scales), d(scene.rotations), d(scene.opacities), d(scene.shs), None,
+                     d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), tan_t, W, H, 3, False, None, c2)
+    (out[5] * d(gco)).sum().backward()
+    assert rel_err(n(c2.grad), n(gcov)) < 1e-6
+    # cov3D built by the differentiable operator: scales / rotations get their gradient through it
+    sc, rot = d(scales).requires_grad_(), d(scene.rotations).requires_grad_()
+    out = preprocess(d(scene.means3D), sc, rot, d(scene.opacities), d(scene.shs), None, d(cam.Tw2v), d(cam.Tv2c),
+                     d(cam.campos), tan_t, W, H, 3, False, compute_cov3D(sc, rot))
+    ((out[0] * d(gm2)).sum() + (out[2] * d(gcol)).sum() + (out[5] * d(gco)).sum()).backward()
+    assert rel_err(n(sc.grad), n(gs)) < 1e-5 and rel_err(n(rot.grad), n(gq)) < 1e-5
+    assert compute_cov2D is not None
+
+
+@pytest.mark.parametrize("P,W,H,E,mul", [(6000, 128, 96, 0, 2.5), (6000, 131, 77, 2, 2.5), (3, 40, 40, 1, 1.0)])
+def test_gs3d_bucket_snapshots_and_fast_backward(P, W, H, E, mul, device):
+    """gaussian_rasterize_forward with per_tile_bucket_offset (snapshots before every 32nd list entry) and
+    gaussian_rasterize_fast_backward against the oracle's bucket-by-bucket restatement of the reference's per-Gaussian
+    kernel (gaussian_render.cu:540-694); `GS_render_fast` end to end equals `GS_render`."""
+    from fast_sp_gs_amd._C import get_C_function
+    from fast_sp_gs_amd.renderer.gaussian_render import GS_render, GS_render_fast
+    scene, scales, cam, tan_fov = _scene(P, W, H, 41 + E, device)
+    d = lambda t: None if t is None else t.to(device).contiguous()
+    out = get_C_function('gs_preprocess_forward')(
+        W, H, 3, False, d(scene.means3D), d(scales * mul), d(scene.rotations), d(scene.opacities), d(scene.shs), None,
+        d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), tan_fov, None, None, None, None)
+    m2, dep, col, rad, tt, c3, co = out
+    ranges, pl = get_C_function('GS_prepare')(W, H, m2, dep, rad, tt, False)
+    g = torch.Generator().manual_seed(9)
+    ex = torch.randn(P, E, generator=g).to(device) if E else None
+    lens = ranges[:, 1] - ranges[:, 0]
+    offset = torch.cumsum((lens + 31) // 32, 0).contiguous()
+    print(f"[gs3d snapshots] P={P} {W}x{H} E={E} R={pl.numel()} longest list {int(lens.max())}", flush=True)
+    res = get_C_function('gaussian_rasterize_forward')(W, H, m2, co, col, ex, pl, ranges, None, None, None, offset)
+    oc, oo, oe, nc, max_c, b2t, sT, sar = res
+    plain = get_C_function('gaussian_rasterize_forward')(W, H, m2, co, col, ex, pl, ranges)
+    torch.cuda.synchronize()
+    assert torch.equal(oc, plain[0]) and torch.equal(nc, plain[3])
+    n = lambda t: None if t is None else npy(t)
+    n64 = lambda t: None if t is None else f64(npy(t))
+    from util import f64
+    ref = O.gs3d_render_forward(W, H, n64(m2), n64(co), n64(col), n64(ex), n(pl), n(ranges), bucket_offset=n(offset))
+    r_oc, r_oo, r_oe, r_nc, r_max, r_b2t, r_sT, r_sar = ref
+    flip = n(nc) != r_nc
+    assert flip.sum() <= max(2, int(1e-5 * W * H))
+    assert np.array_equal(n(b2t), r_b2t) and (n(max_c).reshape(-1) != r_max).sum() <= flip.sum()
+    wrote = r_sT > 0
+    tol = lambda a, b: np.abs(a.astype(np.float64) - b) > 1e-4 + 1e-3 * np.abs(b)
+    bad = int((tol(n(sT), r_sT) & wrote).sum()) + sum(int((tol(n(sar)[:, c], r_sar[:, c]) & wrote).sum())
+                                                      for c in range(3 + E))
+    assert bad <= 32 * (4 + E) * int(flip.sum()) and (P < 10 or (lens > 40).any())
+
+    gi, go = torch.randn(3, H, W, generator=g).to(device), torch.randn(H, W, generator=g).to(device)
+    ge = torch.randn(E, H, W, generator=g).to(device) if E else None
+    got = get_C_function('gaussian_rasterize_fast_backward')(m2, co, col, ex, oc, oe, oo, gi, go, ge, ranges, pl, nc,
+                                                             max_c, offset, b2t, sT, sar)
+    torch.cuda.synchronize()
+    # the oracle's per-Gaussian form from the GPU's own forward outputs and snapshots
+    want = O.gs3d_render_fast_backward(W, H, n64(m2), n64(co), n64(col), n64(ex), n64(oc), n64(oe), n64(oo), n(nc),
+                                       n(max_c).reshape(-1), n(offset), n(b2t), n64(sT), n64(sar), n64(gi), n64(ge),
+                                       n64(go), n(pl), n(ranges))
+    for a, b, name in zip(got, want, ('colors', 'extras', 'means2D', 'conic_opacity')):
+        assert (a is None) == (b is None), name
+        if a is not None:
+            assert rel_err(n(a), b) < 1e-3, (name, rel_err(n(a), b))
+    # end to end: the bucketed pair gives GS_render's gradients
+    leaves = [t.clone().requires_grad_() for t in (m2, col, co)]
+    leaves2 = [t.clone().requires_grad_() for t in (m2, col, co)]
+    a = GS_render_fast(W, H, leaves[0], leaves[1], leaves[2], ranges, pl, ex)
+    b = GS_render(W, H, leaves2[0], leaves2[1], leaves2[2], ranges, pl, ex)
+    ((a[0] * gi).sum() + (a[1] * go).sum()).backward()
+    ((b[0] * gi).sum() + (b[1] * go).sum()).backward()
+    for x, y in zip(leaves, leaves2):
+        assert rel_err(n(x.grad), n(y.grad)) < 1e-4

@@ -374,3 +374,142 @@ def test_extra_channels_forward_and_backward():
                 n += 1
                 ok += abs(fd - grad[i, c]) <= 2e-4 * max(abs(fd), np.abs(grad).max() * 1e-3, 1e-6)
     assert ok >= 0.97 * n  # a step that crosses the alpha = 1/255 threshold is the rare miss
+
+
+def test_precomputed_covariances_and_camera_gradients():
+    """Pre-computed cov3D / cov2D inputs (gaussian_preprocess.cu:76-92): feeding the covariances the stand-alone
+    operators give reproduces the ordinary forward; their gradients (the conic's derivative for cov2D, :293-301; the
+    [P,6] gradient for cov3D) against central differences. Camera gradients (:271, :318-355 and
+    gaussian_compute_cov2D.cu:163-183): dL/dTw2v rows 0-2 and dL/dcampos against central differences of the forward in
+    the view matrix and the camera position (points inside 1.3 x FoV, where the reference's formula is exact)."""
+    s, cam, tan_fov = _scene(P=60, size=64, seed=7)
+    W, H = cam.W, cam.H
+    base = _forward(s, cam, tan_fov)
+    m2, dep, col, rad, tt, c3, co = base
+    P = len(rad)
+    vis = np.flatnonzero(rad > 0)
+    fx, fy = 0.5 * W / tan_fov[0], 0.5 * H / tan_fov[1]
+    cov3 = O.gs3d_compute_cov3D(s['rotations'], s['scales'])
+    cov2 = O.gs3d_compute_cov2D(cov3, s['means3D'], s['Tw2v'], fx, fy, *tan_fov)
+
+    def fwd(**over):
+        a = {**s, **{k: v for k, v in over.items() if k in s}}
+        return O.gs3d_preprocess_forward(W, H, 3, False, a['means3D'], a['scales'], a['rotations'], a['opacities'],
+                                         a['shs'], None, a['Tw2v'], a['Tv2c'], a['campos'], tan_fov,
+                                         cov3D_precomp=over.get('cov3D'), cov2D_precomp=over.get('cov2D'))
+
+    o3 = fwd(cov3D=cov3.copy())
+    o2 = fwd(cov2D=cov2.copy())
+    for o in (o3, o2):
+        assert np.array_equal(o[3], rad) and np.array_equal(o[4], tt)
+        assert np.abs(o[6] - co).max() < 1e-12 * max(1, np.abs(co).max()) and np.abs(o[0] - m2).max() < 1e-12
+    assert o3[5] is not None and np.abs(o3[5] - cov3).max() == 0
+
+    rng = np.random.default_rng(4)
+    g_m2, g_col, g_co = rng.normal(size=(P, 2)), rng.normal(size=(P, 3)), rng.normal(size=(P, 4))
+    loss = lambda o: (o[0] * g_m2).sum() + (o[2] * g_col).sum() + (o[6] * g_co).sum()
+    args = (W, H, 3, False, s['means3D'], s['scales'], s['rotations'], s['shs'], None, s['Tw2v'], s['Tv2c'],
+            s['campos'], tan_fov, rad, col)
+    h = 1e-6
+    # cov2D pre-computed: [P,3] gradient, nothing reaches the means through the covariance, no scale / rotation outputs
+    r2 = O.gs3d_preprocess_backward(*args, c3, g_m2, g_col, g_co, cov2D=cov2)
+    assert r2[1] is None and r2[2] is None and r2[6].shape == (P, 3)
+    r3 = O.gs3d_preprocess_backward(*args, cov3, g_m2, g_col, g_co, precomputed=True)
+    assert r3[1] is None and r3[6].shape == (P, 6)
+    full = O.gs3d_preprocess_backward(*args, c3, g_m2, g_col, g_co)
+    assert np.abs(r3[0] - full[0]).max() < 1e-12 and np.abs(r3[6] - full[6]).max() < 1e-12
+    for name, arr, grad in (('cov2D', cov2, r2[6]), ('cov3D', cov3, r3[6])):
+        worst = 0.0
+        for i in vis[:10]:
+            for c in range(arr.shape[1]):
+                a, b = arr.copy(), arr.copy()
+                a[i, c] += h
+                b[i, c] -= h
+                fd = (loss(fwd(**{name: a})) - loss(fwd(**{name: b}))) / (2 * h)
+                worst = max(worst, abs(fd - grad[i, c]) / max(np.abs(grad[vis[:10]]).max(), 1e-9))
+        assert worst < 2e-5, (name, worst)
+    # the means' gradient with cov2D given is the projection's and the colours' alone
+    assert np.abs(r2[0] - full[0]).max() > 1e-3 * np.abs(full[0]).max()
+
+    # camera gradients: accumulate into the caller's buffers, rows 0-2 of the view matrix
+    out = O.gs3d_preprocess_backward(*args, c3, g_m2, g_col, g_co, camera=True)
+    g_vm, g_cam = out[-2], out[-1]
+    assert not g_vm[3].any() and np.abs(g_vm[:3]).max() > 0 and np.abs(g_cam).max() > 0
+    for a_ in range(3):
+        for b_ in range(4):
+            p, m = s['Tw2v'].copy(), s['Tw2v'].copy()
+            p[a_, b_] += h
+            m[a_, b_] -= h
+            fd = (loss(fwd(Tw2v=p)) - loss(fwd(Tw2v=m))) / (2 * h)
+            assert abs(fd - g_vm[a_, b_]) < 2e-5 * max(1.0, np.abs(g_vm).max()), (a_, b_, fd, g_vm[a_, b_])
+    for a_ in range(3):
+        p, m = s['campos'].copy(), s['campos'].copy()
+        p[a_] += h
+        m[a_] -= h
+        fd = (loss(fwd(campos=p)) - loss(fwd(campos=m))) / (2 * h)
+        assert abs(fd - g_cam[a_]) < 2e-5 * max(1.0, np.abs(g_cam).max())
+    # the stand-alone cov2D operator's view-matrix gradient (added to the caller's buffer)
+    g2 = rng.normal(size=(P, 3))
+    gvm = np.ones((4, 4))
+    O.gs3d_compute_cov2D_backward(cov3, s['means3D'], s['Tw2v'], fx, fy, *tan_fov, g2, gvm)
+    assert np.all(gvm[3] == 1.0)
+    for a_ in range(3):
+        for b_ in range(4):
+            p, m = s['Tw2v'].copy(), s['Tw2v'].copy()
+            p[a_, b_] += h
+            m[a_, b_] -= h
+            fd = ((O.gs3d_compute_cov2D(cov3, s['means3D'], p, fx, fy, *tan_fov) * g2).sum() -
+                  (O.gs3d_compute_cov2D(cov3, s['means3D'], m, fx, fy, *tan_fov) * g2).sum()) / (2 * h)
+            assert abs(fd - (gvm[a_, b_] - 1.0)) < 2e-5 * max(1.0, np.abs(gvm).max()), (a_, b_)
+
+
+def test_bucket_snapshots_and_per_gaussian_backward():
+    """gaussian_rasterize_forward's snapshots (state before every 32nd list entry) and gaussian_rasterize_fast_backward
+    (gaussian_render.cu:540-694), restated bucket by bucket from those snapshots: the same derivative as the
+    back-to-front backward (pinned by finite differences above), so the two must agree to rounding."""
+    s, cam, tan_fov = _scene(P=900, size=48, seed=5)
+    s['scales'] = s['scales'] * 2.5
+    W, H = cam.W, cam.H
+    m2, dep, col, rad, tt, c3, co = _forward(s, cam, tan_fov)
+    P = len(rad)
+    rng = np.random.default_rng(2)
+    ranges, pl = O.prepare(W, H, m2.astype(np.float32), dep.astype(np.float32), rad, tt)
+    lens = ranges[:, 1] - ranges[:, 0]
+    assert lens.max() > 70
+    offset = np.ascontiguousarray(np.cumsum((lens + 31) // 32).astype(np.int64))
+    for E in (0, 2):
+        ex = rng.normal(size=(P, E)) if E else None
+        oc, oo, oe, nc, max_c, b2t, sT, sar = O.gs3d_render_forward(W, H, m2, co, col, ex, pl, ranges,
+                                                                    bucket_offset=offset)
+        plain = O.gs3d_render_forward(W, H, m2, co, col, ex, pl, ranges)
+        assert np.array_equal(oc, plain[0]) and np.array_equal(nc, plain[3])
+        assert np.array_equal(b2t, np.repeat(np.arange(len(lens)), (lens + 31) // 32)) and sar.shape[1] == 3 + E
+        gx = (W + 15) // 16
+        for t in np.flatnonzero(lens > 0):
+            ty, tx = divmod(int(t), gx)
+            assert max_c[t] == nc[ty * 16:ty * 16 + 16, tx * 16:tx * 16 + 16].max()
+            b0 = 0 if t == 0 else int(offset[t - 1])
+            hh, ww = min(16, H - ty * 16), min(16, W - tx * 16)
+            assert np.all(sT[b0].reshape(16, 16)[:hh, :ww] == 1.0) and not sar[b0].any()
+            # a later bucket holds the image of the list cut in front of it, where the pixel was still blending
+            for k in range(1, int((lens[t] + 31) // 32)):
+                cut = ranges.copy()
+                cut[:, 1] = cut[:, 0]
+                cut[t, 1] = cut[t, 0] + 32 * k
+                pc, po, pe, _ = O.gs3d_render_forward(W, H, m2, co, col, ex, pl, cut)
+                live = sT[b0 + k].reshape(16, 16)[:hh, :ww] > 0
+                blk = lambda a: a[..., ty * 16:ty * 16 + hh, tx * 16:tx * 16 + ww]
+                assert np.abs((sT[b0 + k].reshape(16, 16)[:hh, :ww] - (1 - blk(po)))[live]).max(initial=0) < 1e-12
+                for c in range(3):
+                    assert np.abs((sar[b0 + k, c].reshape(16, 16)[:hh, :ww] - blk(pc)[c])[live]).max(initial=0) < 1e-12
+                for c in range(E):
+                    assert np.abs((sar[b0 + k, 3 + c].reshape(16, 16)[:hh, :ww] - blk(pe)[c])[live]).max(initial=0) < 1e-12
+        gi, go = rng.normal(size=(3, H, W)), rng.normal(size=(H, W))
+        ge = rng.normal(size=(E, H, W)) if E else None
+        slow = O.gs3d_render_backward(W, H, m2, co, col, ex, oo, nc, gi, ge, go, pl, ranges)
+        fast = O.gs3d_render_fast_backward(W, H, m2, co, col, ex, oc, oe, oo, nc, max_c, offset, b2t, sT, sar, gi, ge,
+                                           go, pl, ranges)
+        for a, b in zip(slow, fast):
+            assert (a is None) == (b is None)
+            if a is not None:
+                assert np.abs(a - b).max() < 1e-9 * max(1.0, np.abs(a).max()) and np.abs(a).max() > 0
