@@ -96,6 +96,25 @@ def _f32(what, **tensors):
             L.require_dtype(what, k, t, torch.float32)
 
 
+_DTYPE_CODES = {torch.float32: 0, torch.float64: 1, torch.float16: 2}  # FSGS_DTYPE_* of the `_typed` entry points
+
+
+def _same_float(what, allowed, **tensors):
+    """The selector of the tensors' common element type; all of them must be on the GPU, contiguous, of one of the
+    `allowed` floating types (the ones the reference dispatches this operator on) and agree with each other."""
+    L.require_cuda(what, **tensors)
+    first = next(iter(tensors.values()))
+    if first.dtype not in allowed:
+        raise RuntimeError(f'{what}: element type {first.dtype} is not supported (expected one of '
+                           f'{", ".join(str(d) for d in allowed)})')
+    for k, t in tensors.items():
+        L.require_dtype(what, k, t, first.dtype)
+    return _DTYPE_CODES[first.dtype]
+
+
+_FLOAT_DOUBLE = (torch.float32, torch.float64)
+_FLOAT_DOUBLE_HALF = (torch.float32, torch.float64, torch.float16)
+
 _PINNED = threading.local()
 
 
@@ -774,32 +793,33 @@ def SH_to_RGB_backward(degree: int, clamp: bool, dir_or_pos: Tensor, campos: Opt
 def sh_encode_forward(inputs: Tensor, outputs: Tensor, B: int, D: int, C: int) -> None:
     """nerf/shencoder.cu:657-673: outputs[B,(C+1)^2] <- basis values of inputs[B,D][:, :3]."""
     what = 'sh_encode_forward'
-    _f32(what, inputs=inputs, outputs=outputs)
+    dtype = _same_float(what, _FLOAT_DOUBLE_HALF, inputs=inputs, outputs=outputs)
     with _timed('sh_encode_forward'):
-        rc = _lib().fsgs_sh_encode_forward(B, D, C, L.ptr(inputs), L.ptr(outputs), L.current_stream())
+        rc = _lib().fsgs_sh_encode_forward_typed(dtype, B, D, C, L.ptr(inputs), L.ptr(outputs), L.current_stream())
     L.check(rc, what)
 
 
 def sh_encode_backward(grad: Tensor, inputs: Tensor, B: int, D: int, C: int, grad_inputs: Tensor) -> None:
     """nerf/shencoder.cu:675-691."""
     what = 'sh_encode_backward'
-    _f32(what, grad=grad, inputs=inputs, grad_inputs=grad_inputs)
+    dtype = _same_float(what, _FLOAT_DOUBLE_HALF, grad=grad, inputs=inputs, grad_inputs=grad_inputs)
     with _timed('sh_encode_backward'):
-        rc = _lib().fsgs_sh_encode_backward(B, D, C, L.ptr(grad), L.ptr(inputs), L.ptr(grad_inputs), L.current_stream())
+        rc = _lib().fsgs_sh_encode_backward_typed(dtype, B, D, C, L.ptr(grad), L.ptr(inputs), L.ptr(grad_inputs),
+                                                  L.current_stream())
     L.check(rc, what)
 
 
 def freq_encode_forward(inputs: Tensor, degree: int, include_inputs: bool, scale: float) -> Tensor:
     """nerf/freqencoder.cu:63-81 -> outputs[..., D * (2 * degree + include_inputs)]."""
     what = 'freq_encode_forward'
-    _f32(what, inputs=inputs)
+    dtype = _same_float(what, _FLOAT_DOUBLE, inputs=inputs)
     Din = inputs.shape[-1]
     Dout = Din * (degree * 2 + int(bool(include_inputs)))
     B = inputs.numel() // Din
-    out = torch.empty((*inputs.shape[:-1], Dout), dtype=torch.float32, device=inputs.device)
+    out = torch.empty((*inputs.shape[:-1], Dout), dtype=inputs.dtype, device=inputs.device)
     with _timed('freq_encode_forward'):
-        rc = _lib().fsgs_freq_encode_forward(B, Din, degree, int(bool(include_inputs)), float(scale), L.ptr(inputs),
-                                             L.ptr(out), L.current_stream())
+        rc = _lib().fsgs_freq_encode_forward_typed(dtype, B, Din, degree, int(bool(include_inputs)), float(scale),
+                                                   L.ptr(inputs), L.ptr(out), L.current_stream())
     L.check(rc, what)
     return out
 
@@ -807,38 +827,38 @@ def freq_encode_forward(inputs: Tensor, degree: int, include_inputs: bool, scale
 def freq_encode_backward(grad: Tensor, outputs: Tensor, degree: int, include_inputs: bool, scale: float) -> Tensor:
     """nerf/freqencoder.cu:83-104 -> grad_inputs."""
     what = 'freq_encode_backward'
-    _f32(what, grad=grad, outputs=outputs)
+    dtype = _same_float(what, _FLOAT_DOUBLE, grad=grad, outputs=outputs)
     if grad.shape != outputs.shape:
         raise RuntimeError(f'{what}: grad must have the shape of outputs')
     Dout = outputs.shape[-1]
     Din = Dout // (degree * 2 + int(bool(include_inputs)))
     B = outputs.numel() // Dout
-    gin = torch.empty((*outputs.shape[:-1], Din), dtype=torch.float32, device=outputs.device)
+    gin = torch.empty((*outputs.shape[:-1], Din), dtype=outputs.dtype, device=outputs.device)
     with _timed('freq_encode_backward'):
-        rc = _lib().fsgs_freq_encode_backward(B, Din, degree, int(bool(include_inputs)), float(scale), L.ptr(grad),
-                                              L.ptr(outputs), L.ptr(gin), L.current_stream())
+        rc = _lib().fsgs_freq_encode_backward_typed(dtype, B, Din, degree, int(bool(include_inputs)), float(scale),
+                                                    L.ptr(grad), L.ptr(outputs), L.ptr(gin), L.current_stream())
     L.check(rc, what)
     return gin
 
 
 # --------------------------------------------------------------------------------------------------------------------
 def cdist_top(x1: Tensor, x2: Tensor, largest: bool = False) -> List[Tensor]:
-    """other/cdist_top.cu:34-84 -> [distance[..., N] f32, index[..., N] int64]."""
+    """other/cdist_top.cu:34-84 -> [distance[..., N] (the points' element type), index[..., N] int64]."""
     what = 'cdist_top'
     if x1.device != x2.device:
         raise RuntimeError('x1 and x2 must be same device')
-    _f32(what, x1=x1, x2=x2)
+    dtype = _same_float(what, _FLOAT_DOUBLE, x1=x1, x2=x2)
     N, M, D = x1.shape[-2], x2.shape[-2], x1.shape[-1]
     B = x1.numel() // max(N * D, 1)
     if x2.shape[-1] != D:
         raise RuntimeError(f'The dimenstion of point must be {D}')
     if x2.numel() != B * M * D:
         raise RuntimeError('The shape[:-2] of x2 must be same with x1')
-    distance = torch.empty(x1.shape[:-1], dtype=torch.float32, device=x1.device)
+    distance = torch.empty(x1.shape[:-1], dtype=x1.dtype, device=x1.device)
     index = torch.empty(x1.shape[:-1], dtype=torch.int64, device=x1.device)
     with _timed('cdist_top_forward'):
-        rc = _lib().fsgs_cdist_top_forward(B, N, M, D, int(bool(largest)), L.ptr(x1), L.ptr(x2), L.ptr(distance),
-                                           L.ptr(index), L.current_stream())
+        rc = _lib().fsgs_cdist_top_forward_typed(dtype, B, N, M, D, int(bool(largest)), L.ptr(x1), L.ptr(x2),
+                                                 L.ptr(distance), L.ptr(index), L.current_stream())
     L.check(rc, what)
     return [distance, index]
 
@@ -846,15 +866,16 @@ def cdist_top(x1: Tensor, x2: Tensor, largest: bool = False) -> List[Tensor]:
 def cdist_top_backward(x1: Tensor, x2: Tensor, distance: Tensor, index: Tensor, grad_dist: Tensor) -> List[Tensor]:
     """other/cdist_top.cu:107-154 -> [grad_x1, grad_x2]."""
     what = 'cdist_top_backward'
-    _f32(what, x1=x1, x2=x2, distance=distance, grad_dist=grad_dist)
+    dtype = _same_float(what, _FLOAT_DOUBLE, x1=x1, x2=x2, distance=distance, grad_dist=grad_dist)
     L.require_cuda(what, index=index)
     N, D, M = x1.shape[-2], x1.shape[-1], x2.shape[-2]
     B = x1.numel() // max(N * D, 1)
     g1 = torch.zeros_like(x1)
     g2 = torch.zeros_like(x2)
     with _timed('cdist_top_backward'):
-        rc = _lib().fsgs_cdist_top_backward(B, N, M, D, L.ptr(x1), L.ptr(x2), L.ptr(distance), L.ptr(index),
-                                            L.ptr(grad_dist), L.ptr(g1), L.ptr(g2), L.current_stream())
+        rc = _lib().fsgs_cdist_top_backward_typed(dtype, B, N, M, D, L.ptr(x1), L.ptr(x2), L.ptr(distance),
+                                                  L.ptr(index), L.ptr(grad_dist), L.ptr(g1), L.ptr(g2),
+                                                  L.current_stream())
     L.check(rc, what)
     return [g1, g2]
 

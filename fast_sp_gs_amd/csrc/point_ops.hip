@@ -13,7 +13,9 @@
 // read as wave-wide broadcasts, distances accumulated in the reference's order with contraction off so that indices
 // are reproducible bit for bit.
 #include <algorithm>
+#include <type_traits>
 
+#include "../../include/fsgs.h"
 #include "common.hpp"
 #include "lbs.hpp"
 #include "sh.hpp"
@@ -100,71 +102,91 @@ __global__ void __launch_bounds__(256) sh_to_rgb_backward_kernel(int P, int F, i
   }
 }
 
+// ---- element types of the small operators -------------------------------------------------------------------------------
+// The encoders and the nearest / farthest search accept the floating types the reference dispatches on. Half precision
+// is a storage format only: values are widened on load, the arithmetic is single precision, the result is rounded once
+// on store.
+template <typename T> struct Arith { using type = T; };
+template <> struct Arith<_Float16> { using type = float; };
+
 // ---- bare SH encoder ------------------------------------------------------------------------------------------------
-template <int kSh>
-__global__ void __launch_bounds__(256) sh_encode_forward_kernel(int B, int D, int C, const float* __restrict__ in,
-                                                                float* __restrict__ out) {
+template <int kSh, typename T>
+__global__ void __launch_bounds__(256) sh_encode_forward_kernel(int B, int D, int C, const T* __restrict__ in,
+                                                                T* __restrict__ out) {
+  using A = typename Arith<T>::type;
   const int b = blockIdx.x * blockDim.x + threadIdx.x;
   if (b >= B) return;
-  float Y[kSh];
-  sh_eval(C, in[(size_t) b * D], in[(size_t) b * D + 1], in[(size_t) b * D + 2], Y);
+  A Y[kSh];
+  sh_eval(C, (A) in[(size_t) b * D], (A) in[(size_t) b * D + 1], (A) in[(size_t) b * D + 2], Y);
   const int n = sh_count(C);
-  float* o    = out + (size_t) b * n;
-  if ((n & 3) == 0) {
-    for (int l = 0; l < n; l += 4) *(float4*) (o + l) = make_float4(Y[l], Y[l + 1], Y[l + 2], Y[l + 3]);
-  } else {
-    for (int l = 0; l < n; ++l) o[l] = Y[l];
+  T* o        = out + (size_t) b * n;
+  if constexpr (std::is_same<T, float>::value) {
+    if ((n & 3) == 0) {
+      for (int l = 0; l < n; l += 4) *(float4*) (o + l) = make_float4(Y[l], Y[l + 1], Y[l + 2], Y[l + 3]);
+      return;
+    }
   }
+  for (int l = 0; l < n; ++l) o[l] = (T) Y[l];
 }
 
-template <int kSh>
-__global__ void __launch_bounds__(256) sh_encode_backward_kernel(int B, int D, int C, const float* __restrict__ grad,
-    const float* __restrict__ in, float* __restrict__ grad_in) {
+template <int kSh, typename T>
+__global__ void __launch_bounds__(256) sh_encode_backward_kernel(int B, int D, int C, const T* __restrict__ grad,
+    const T* __restrict__ in, T* __restrict__ grad_in) {
+  using A = typename Arith<T>::type;
   const int b = blockIdx.x * blockDim.x + threadIdx.x;
   if (b >= B) return;
   const int n = sh_count(C);
-  float t[kSh];
-  const float* g = grad + (size_t) b * n;
-  if ((n & 3) == 0) {
-    for (int l = 0; l < n; l += 4) {
-      const float4 v = *(const float4*) (g + l);
-      t[l] = v.x, t[l + 1] = v.y, t[l + 2] = v.z, t[l + 3] = v.w;
+  A t[kSh];
+  const T* g = grad + (size_t) b * n;
+  bool loaded = false;
+  if constexpr (std::is_same<T, float>::value) {
+    if ((n & 3) == 0) {
+      for (int l = 0; l < n; l += 4) {
+        const float4 v = *(const float4*) (g + l);
+        t[l] = v.x, t[l + 1] = v.y, t[l + 2] = v.z, t[l + 3] = v.w;
+      }
+      loaded = true;
     }
-  } else {
-    for (int l = 0; l < n; ++l) t[l] = g[l];
   }
-  float dx = 0, dy = 0, dz = 0;
-  sh_grad_accumulate(C, in[(size_t) b * D], in[(size_t) b * D + 1], in[(size_t) b * D + 2], t, dx, dy, dz);
-  grad_in[(size_t) b * D] = dx, grad_in[(size_t) b * D + 1] = dy, grad_in[(size_t) b * D + 2] = dz;
+  if (!loaded)
+    for (int l = 0; l < n; ++l) t[l] = (A) g[l];
+  A dx = 0, dy = 0, dz = 0;
+  sh_grad_accumulate(C, (A) in[(size_t) b * D], (A) in[(size_t) b * D + 1], (A) in[(size_t) b * D + 2], t, dx, dy, dz);
+  grad_in[(size_t) b * D] = (T) dx, grad_in[(size_t) b * D + 1] = (T) dy, grad_in[(size_t) b * D + 2] = (T) dz;
 }
 
 // ---- frequency encoder ------------------------------------------------------------------------------------------------
+// The angle is scaled and its sine / cosine taken in single precision for double tensors too: the reference goes through
+// scalbnf, whose argument and result are float (freqencoder.cu:27-28). The backward is in T throughout (:54).
+template <typename T>
 __global__ void __launch_bounds__(128) freq_encode_forward_kernel(int B, int Din, int degree, int include_input,
-    float scale, const float* __restrict__ in, float* __restrict__ out) {
+    T scale, const T* __restrict__ in, T* __restrict__ out) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= B * Din) return;
   const int b = t / Din, c = t - b * Din;
   const int Dout = Din * (2 * degree + (include_input ? 1 : 0));
-  float* o = out + (size_t) b * Dout + c;
-  float x  = in[t];
+  T* o = out + (size_t) b * Dout + c;
+  T x  = in[t];
   if (include_input) o[0] = x, o += Din;
   x = x * scale;
+  const float xf = (float) x;
   for (int d = 0; d < degree; ++d) {
-    const float v = ldexpf(x, d);
-    o[(2 * d + 0) * Din] = sinf(v);
-    o[(2 * d + 1) * Din] = cosf(v);
+    const float v = ldexpf(xf, d);
+    o[(2 * d + 0) * Din] = (T) sinf(v);
+    o[(2 * d + 1) * Din] = (T) cosf(v);
   }
 }
 
+template <typename T>
 __global__ void __launch_bounds__(128) freq_encode_backward_kernel(int B, int Din, int degree, int include_input,
-    float scale, const float* __restrict__ grad, const float* __restrict__ outv, float* __restrict__ gin) {
+    T scale, const T* __restrict__ grad, const T* __restrict__ outv, T* __restrict__ gin) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= B * Din) return;
   const int b = t / Din, c = t - b * Din;
   const int Dout = Din * (2 * degree + (include_input ? 1 : 0));
-  const float* g = grad + (size_t) b * Dout + c;
-  const float* o = outv + (size_t) b * Dout + c;
-  float gx = 0.0f;
+  const T* g = grad + (size_t) b * Dout + c;
+  const T* o = outv + (size_t) b * Dout + c;
+  T gx = 0;
   if (include_input) gx = g[0], g += Din, o += Din;
   for (int f = 0; f < degree; ++f) {
     gx += ldexpf(1.0f, f) * scale * (g[0] * o[Din] - g[Din] * o[0]);
@@ -174,23 +196,23 @@ __global__ void __launch_bounds__(128) freq_encode_backward_kernel(int B, int Di
 }
 
 // ---- nearest / farthest point -------------------------------------------------------------------------------------------
-constexpr int kCtrlChunk = 1024;  // control points staged per LDS round (x 3 floats for the D == 3 fast path)
+constexpr int kCtrlChunk = 1024;  // control points staged per LDS round (x 3 values for the D == 3 fast path)
 
-template <int kD>
-__global__ void __launch_bounds__(128) cdist_top_kernel(int N, int M, int D, int largest, const float* __restrict__ x,
-    const float* __restrict__ y, float* __restrict__ dist, int64_t* __restrict__ index) {
+template <int kD, typename T>
+__global__ void __launch_bounds__(128) cdist_top_kernel(int N, int M, int D, int largest, const T* __restrict__ x,
+    const T* __restrict__ y, T* __restrict__ dist, int64_t* __restrict__ index) {
 #pragma clang fp contract(off)
-  __shared__ float s_y[kD > 0 ? kCtrlChunk * kD : 1];
+  __shared__ T s_y[kD > 0 ? kCtrlChunk * kD : 1];
   const int b = blockIdx.y;
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
-  const float* yb = y + (size_t) b * M * D;
-  const float* xp = x + ((size_t) b * N + (n < N ? n : 0)) * D;
-  float xr[kD > 0 ? kD : 1];
+  const T* yb = y + (size_t) b * M * D;
+  const T* xp = x + ((size_t) b * N + (n < N ? n : 0)) * D;
+  T xr[kD > 0 ? kD : 1];
   if (kD > 0)
 #pragma unroll
     for (int d = 0; d < kD; ++d) xr[d] = xp[d];
-  float top = 0.0f;
-  int topi  = 0;
+  T top    = 0;
+  int topi = 0;
   if (kD > 0) {
     for (int m0 = 0; m0 < M; m0 += kCtrlChunk) {
       const int mc = min(kCtrlChunk, M - m0);
@@ -198,10 +220,10 @@ __global__ void __launch_bounds__(128) cdist_top_kernel(int N, int M, int D, int
       for (int k = threadIdx.x; k < mc * kD; k += blockDim.x) s_y[k] = yb[(size_t) m0 * kD + k];
       __syncthreads();
       for (int m = 0; m < mc; ++m) {
-        float sum = 0.0f;
+        T sum = 0;
 #pragma unroll
         for (int d = 0; d < kD; ++d) {
-          const float t = xr[d] - s_y[m * kD + d];
+          const T t = xr[d] - s_y[m * kD + d];
           sum += t * t;
         }
         if ((m0 + m) == 0 || (sum > top) == (bool) largest) top = sum, topi = m0 + m;
@@ -209,31 +231,31 @@ __global__ void __launch_bounds__(128) cdist_top_kernel(int N, int M, int D, int
     }
   } else {
     for (int m = 0; m < M; ++m) {
-      float sum = 0.0f;
+      T sum = 0;
       for (int d = 0; d < D; ++d) {
-        const float t = xp[d] - yb[(size_t) m * D + d];
+        const T t = xp[d] - yb[(size_t) m * D + d];
         sum += t * t;
       }
       if (m == 0 || (sum > top) == (bool) largest) top = sum, topi = m;
     }
   }
   if (n < N) {
-    dist[(size_t) b * N + n]  = sqrtf(top);
+    dist[(size_t) b * N + n]  = sqrt(top);
     index[(size_t) b * N + n] = topi;
   }
 }
 
-__global__ void __launch_bounds__(256) cdist_top_backward_kernel(int B, int N, int M, int D,
-    const float* __restrict__ p1, const float* __restrict__ p2, const float* __restrict__ gdist,
-    const float* __restrict__ dist, const int64_t* __restrict__ index, float* __restrict__ g1,
-    float* __restrict__ g2) {
+template <typename T>
+__global__ void __launch_bounds__(256) cdist_top_backward_kernel(int B, int N, int M, int D, const T* __restrict__ p1,
+    const T* __restrict__ p2, const T* __restrict__ gdist, const T* __restrict__ dist,
+    const int64_t* __restrict__ index, T* __restrict__ g1, T* __restrict__ g2) {
   const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= (int64_t) B * N) return;
   const int b  = (int) (i / N);
   const int j2 = (int) index[i];
-  const float g = gdist[i] / dist[i];
+  const T g    = gdist[i] / dist[i];
   for (int d = 0; d < D; ++d) {
-    const float t = g * (p1[(size_t) i * D + d] - p2[((size_t) b * M + j2) * D + d]);
+    const T t = g * (p1[(size_t) i * D + d] - p2[((size_t) b * M + j2) * D + d]);
     g1[(size_t) i * D + d] = t;
     atomicAdd(&g2[((size_t) b * M + j2) * D + d], -t);
   }
@@ -589,65 +611,151 @@ FSGS_API int fsgs_sh_to_rgb_backward(int P, int F, int degree, int clamp, const 
   return check_launch("SH_to_RGB_backward");
 }
 
-FSGS_API int fsgs_sh_encode_forward(int B, int D, int C, const float* in, float* out, void* stream) {
+// ---- encoders and nearest / farthest search: one typed entry each plus the single-precision shorthand -----------------
+namespace {
+template <typename T>
+int sh_encode_forward_t(int B, int D, int C, const void* in, void* out, hipStream_t s) {
+  auto kernel = C > 3 ? sh_encode_forward_kernel<64, T> : sh_encode_forward_kernel<16, T>;
+  hipLaunchKernelGGL(kernel, dim3(div_up(B, 256)), dim3(256), 0, s, B, D, C, (const T*) in, (T*) out);
+  return check_launch("sh_encode_forward");
+}
+template <typename T>
+int sh_encode_backward_t(int B, int D, int C, const void* grad, const void* in, void* grad_in, hipStream_t s) {
+  auto kernel = C > 3 ? sh_encode_backward_kernel<64, T> : sh_encode_backward_kernel<16, T>;
+  hipLaunchKernelGGL(kernel, dim3(div_up(B, 256)), dim3(256), 0, s, B, D, C, (const T*) grad, (const T*) in,
+                     (T*) grad_in);
+  return check_launch("sh_encode_backward");
+}
+template <typename T>
+int freq_encode_forward_t(int B, int Din, int degree, int include_input, double scale, const void* in, void* out,
+                          hipStream_t s) {
+  hipLaunchKernelGGL(freq_encode_forward_kernel<T>, dim3(div_up((int64_t) B * Din, 128)), dim3(128), 0, s, B, Din,
+                     degree, include_input, (T) scale, (const T*) in, (T*) out);
+  return check_launch("freq_encode_forward");
+}
+template <typename T>
+int freq_encode_backward_t(int B, int Din, int degree, int include_input, double scale, const void* grad,
+                           const void* outv, void* gin, hipStream_t s) {
+  hipLaunchKernelGGL(freq_encode_backward_kernel<T>, dim3(div_up((int64_t) B * Din, 128)), dim3(128), 0, s, B, Din,
+                     degree, include_input, (T) scale, (const T*) grad, (const T*) outv, (T*) gin);
+  return check_launch("freq_encode_backward");
+}
+template <typename T>
+int cdist_top_forward_t(int B, int N, int M, int D, int largest, const void* x, const void* y, void* dist,
+                        int64_t* index, hipStream_t s) {
+  const dim3 grid(div_up(N, 128), B), block(128);
+  if (D == 3)
+    hipLaunchKernelGGL((cdist_top_kernel<3, T>), grid, block, 0, s, N, M, D, largest, (const T*) x, (const T*) y,
+                       (T*) dist, index);
+  else
+    hipLaunchKernelGGL((cdist_top_kernel<0, T>), grid, block, 0, s, N, M, D, largest, (const T*) x, (const T*) y,
+                       (T*) dist, index);
+  return check_launch("cdist_top");
+}
+template <typename T>
+int cdist_top_backward_t(int B, int N, int M, int D, const void* p1, const void* p2, const void* dist,
+                         const int64_t* index, const void* gdist, void* g1, void* g2, hipStream_t s) {
+  hipLaunchKernelGGL(cdist_top_backward_kernel<T>, dim3(div_up((int64_t) B * N, 256)), dim3(256), 0, s, B, N, M, D,
+                     (const T*) p1, (const T*) p2, (const T*) gdist, (const T*) dist, index, (T*) g1, (T*) g2);
+  return check_launch("cdist_top_backward");
+}
+}  // namespace
+
+FSGS_API int fsgs_sh_encode_forward_typed(int dtype, int B, int D, int C, const void* in, void* out, void* stream) {
   FSGS_REQUIRE(B >= 0 && D >= 3 && in && out, "sh_encode_forward: bad arguments");
   FSGS_REQUIRE(0 <= C && C <= kMaxShDegree, "sh_encode_forward: degree %d not supported (max %d)", C, kMaxShDegree);
+  FSGS_REQUIRE(dtype == FSGS_DTYPE_F32 || dtype == FSGS_DTYPE_F64 || dtype == FSGS_DTYPE_F16,
+               "sh_encode_forward: element type %d not supported", dtype);
   if (B == 0) return kOk;
-  auto kernel = C > 3 ? sh_encode_forward_kernel<64> : sh_encode_forward_kernel<16>;
-  hipLaunchKernelGGL(kernel, dim3(div_up(B, 256)), dim3(256), 0, (hipStream_t) stream, B, D, C, in,
-                     out);
-  return check_launch("sh_encode_forward");
+  if (dtype == FSGS_DTYPE_F64) return sh_encode_forward_t<double>(B, D, C, in, out, (hipStream_t) stream);
+  if (dtype == FSGS_DTYPE_F16) return sh_encode_forward_t<_Float16>(B, D, C, in, out, (hipStream_t) stream);
+  return sh_encode_forward_t<float>(B, D, C, in, out, (hipStream_t) stream);
+}
+
+FSGS_API int fsgs_sh_encode_forward(int B, int D, int C, const float* in, float* out, void* stream) {
+  return fsgs_sh_encode_forward_typed(FSGS_DTYPE_F32, B, D, C, in, out, stream);
+}
+
+FSGS_API int fsgs_sh_encode_backward_typed(int dtype, int B, int D, int C, const void* grad, const void* in,
+                                           void* grad_in, void* stream) {
+  FSGS_REQUIRE(B >= 0 && D >= 3 && grad && in && grad_in, "sh_encode_backward: bad arguments");
+  FSGS_REQUIRE(0 <= C && C <= kMaxShDegree, "sh_encode_backward: degree %d not supported (max %d)", C, kMaxShDegree);
+  FSGS_REQUIRE(dtype == FSGS_DTYPE_F32 || dtype == FSGS_DTYPE_F64 || dtype == FSGS_DTYPE_F16,
+               "sh_encode_backward: element type %d not supported", dtype);
+  if (B == 0) return kOk;
+  if (dtype == FSGS_DTYPE_F64) return sh_encode_backward_t<double>(B, D, C, grad, in, grad_in, (hipStream_t) stream);
+  if (dtype == FSGS_DTYPE_F16) return sh_encode_backward_t<_Float16>(B, D, C, grad, in, grad_in, (hipStream_t) stream);
+  return sh_encode_backward_t<float>(B, D, C, grad, in, grad_in, (hipStream_t) stream);
 }
 
 FSGS_API int fsgs_sh_encode_backward(int B, int D, int C, const float* grad, const float* in, float* grad_in,
                                      void* stream) {
-  FSGS_REQUIRE(B >= 0 && D >= 3 && grad && in && grad_in, "sh_encode_backward: bad arguments");
-  FSGS_REQUIRE(0 <= C && C <= kMaxShDegree, "sh_encode_backward: degree %d not supported (max %d)", C, kMaxShDegree);
+  return fsgs_sh_encode_backward_typed(FSGS_DTYPE_F32, B, D, C, grad, in, grad_in, stream);
+}
+
+FSGS_API int fsgs_freq_encode_forward_typed(int dtype, int B, int Din, int degree, int include_input, double scale,
+                                            const void* in, void* out, void* stream) {
+  FSGS_REQUIRE(B >= 0 && Din > 0 && degree >= 0 && in && out, "freq_encode_forward: bad arguments");
+  FSGS_REQUIRE(dtype == FSGS_DTYPE_F32 || dtype == FSGS_DTYPE_F64, "freq_encode_forward: element type %d not supported",
+               dtype);
   if (B == 0) return kOk;
-  auto kernel = C > 3 ? sh_encode_backward_kernel<64> : sh_encode_backward_kernel<16>;
-  hipLaunchKernelGGL(kernel, dim3(div_up(B, 256)), dim3(256), 0, (hipStream_t) stream, B, D, C,
-                     grad, in, grad_in);
-  return check_launch("sh_encode_backward");
+  if (dtype == FSGS_DTYPE_F64)
+    return freq_encode_forward_t<double>(B, Din, degree, include_input, scale, in, out, (hipStream_t) stream);
+  return freq_encode_forward_t<float>(B, Din, degree, include_input, scale, in, out, (hipStream_t) stream);
 }
 
 FSGS_API int fsgs_freq_encode_forward(int B, int Din, int degree, int include_input, double scale, const float* in,
                                       float* out, void* stream) {
-  FSGS_REQUIRE(B >= 0 && Din > 0 && degree >= 0 && in && out, "freq_encode_forward: bad arguments");
+  return fsgs_freq_encode_forward_typed(FSGS_DTYPE_F32, B, Din, degree, include_input, scale, in, out, stream);
+}
+
+FSGS_API int fsgs_freq_encode_backward_typed(int dtype, int B, int Din, int degree, int include_input, double scale,
+                                             const void* grad, const void* outv, void* gin, void* stream) {
+  FSGS_REQUIRE(B >= 0 && Din > 0 && degree >= 0 && grad && outv && gin, "freq_encode_backward: bad arguments");
+  FSGS_REQUIRE(dtype == FSGS_DTYPE_F32 || dtype == FSGS_DTYPE_F64,
+               "freq_encode_backward: element type %d not supported", dtype);
   if (B == 0) return kOk;
-  hipLaunchKernelGGL(freq_encode_forward_kernel, dim3(div_up((int64_t) B * Din, 128)), dim3(128), 0,
-                     (hipStream_t) stream, B, Din, degree, include_input, (float) scale, in, out);
-  return check_launch("freq_encode_forward");
+  if (dtype == FSGS_DTYPE_F64)
+    return freq_encode_backward_t<double>(B, Din, degree, include_input, scale, grad, outv, gin, (hipStream_t) stream);
+  return freq_encode_backward_t<float>(B, Din, degree, include_input, scale, grad, outv, gin, (hipStream_t) stream);
 }
 
 FSGS_API int fsgs_freq_encode_backward(int B, int Din, int degree, int include_input, double scale, const float* grad,
                                        const float* outv, float* gin, void* stream) {
-  FSGS_REQUIRE(B >= 0 && Din > 0 && degree >= 0 && grad && outv && gin, "freq_encode_backward: bad arguments");
-  if (B == 0) return kOk;
-  hipLaunchKernelGGL(freq_encode_backward_kernel, dim3(div_up((int64_t) B * Din, 128)), dim3(128), 0,
-                     (hipStream_t) stream, B, Din, degree, include_input, (float) scale, grad, outv, gin);
-  return check_launch("freq_encode_backward");
+  return fsgs_freq_encode_backward_typed(FSGS_DTYPE_F32, B, Din, degree, include_input, scale, grad, outv, gin, stream);
+}
+
+FSGS_API int fsgs_cdist_top_forward_typed(int dtype, int B, int N, int M, int D, int largest, const void* x,
+                                          const void* y, void* dist, int64_t* index, void* stream) {
+  FSGS_REQUIRE(B >= 0 && N >= 0 && M > 0 && D > 0 && x && y && dist && index, "cdist_top: bad arguments");
+  FSGS_REQUIRE(dtype == FSGS_DTYPE_F32 || dtype == FSGS_DTYPE_F64, "cdist_top: element type %d not supported", dtype);
+  if (B == 0 || N == 0) return kOk;
+  if (dtype == FSGS_DTYPE_F64)
+    return cdist_top_forward_t<double>(B, N, M, D, largest, x, y, dist, index, (hipStream_t) stream);
+  return cdist_top_forward_t<float>(B, N, M, D, largest, x, y, dist, index, (hipStream_t) stream);
 }
 
 FSGS_API int fsgs_cdist_top_forward(int B, int N, int M, int D, int largest, const float* x, const float* y,
                                     float* dist, int64_t* index, void* stream) {
-  FSGS_REQUIRE(B >= 0 && N >= 0 && M > 0 && D > 0 && x && y && dist && index, "cdist_top: bad arguments");
+  return fsgs_cdist_top_forward_typed(FSGS_DTYPE_F32, B, N, M, D, largest, x, y, dist, index, stream);
+}
+
+FSGS_API int fsgs_cdist_top_backward_typed(int dtype, int B, int N, int M, int D, const void* p1, const void* p2,
+                                           const void* dist, const int64_t* index, const void* gdist, void* g1,
+                                           void* g2, void* stream) {
+  FSGS_REQUIRE(B >= 0 && N >= 0 && M > 0 && D > 0 && p1 && p2 && dist && index && gdist && g1 && g2,
+               "cdist_top_backward: bad arguments");
+  FSGS_REQUIRE(dtype == FSGS_DTYPE_F32 || dtype == FSGS_DTYPE_F64, "cdist_top_backward: element type %d not supported",
+               dtype);
   if (B == 0 || N == 0) return kOk;
-  const dim3 grid(div_up(N, 128), B), block(128);
-  if (D == 3)
-    hipLaunchKernelGGL((cdist_top_kernel<3>), grid, block, 0, (hipStream_t) stream, N, M, D, largest, x, y, dist, index);
-  else
-    hipLaunchKernelGGL((cdist_top_kernel<0>), grid, block, 0, (hipStream_t) stream, N, M, D, largest, x, y, dist, index);
-  return check_launch("cdist_top");
+  if (dtype == FSGS_DTYPE_F64)
+    return cdist_top_backward_t<double>(B, N, M, D, p1, p2, dist, index, gdist, g1, g2, (hipStream_t) stream);
+  return cdist_top_backward_t<float>(B, N, M, D, p1, p2, dist, index, gdist, g1, g2, (hipStream_t) stream);
 }
 
 FSGS_API int fsgs_cdist_top_backward(int B, int N, int M, int D, const float* p1, const float* p2, const float* dist,
                                      const int64_t* index, const float* gdist, float* g1, float* g2, void* stream) {
-  FSGS_REQUIRE(B >= 0 && N >= 0 && M > 0 && D > 0 && p1 && p2 && dist && index && gdist && g1 && g2,
-               "cdist_top_backward: bad arguments");
-  if (B == 0 || N == 0) return kOk;
-  hipLaunchKernelGGL(cdist_top_backward_kernel, dim3(div_up((int64_t) B * N, 256)), dim3(256), 0, (hipStream_t) stream,
-                     B, N, M, D, p1, p2, gdist, dist, index, g1, g2);
-  return check_launch("cdist_top_backward");
+  return fsgs_cdist_top_backward_typed(FSGS_DTYPE_F32, B, N, M, D, p1, p2, dist, index, gdist, g1, g2, stream);
 }
 
 FSGS_API int fsgs_knn_topk(int N, int M, int D, int K, const float* x, const float* y, float* dist2, int64_t* index,

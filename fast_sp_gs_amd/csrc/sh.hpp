@@ -15,16 +15,17 @@ constexpr int kMaxShDegree = 7;
 
 __device__ __forceinline__ int sh_count(int degree) { return (degree + 1) * (degree + 1); }
 
-// Entries beyond (degree+1)^2 are left untouched. kN = 16 serves degree <= 3, kN = 64 degree <= 7.
-template <int kN>
-__device__ __forceinline__ void sh_eval(int degree, float x, float y, float z, float (&Y)[kN]) {
+// Entries beyond (degree+1)^2 are left untouched. kN = 16 serves degree <= 3, kN = 64 degree <= 7. T is float or double;
+// the coefficients are single-precision literals for either (shencoder.cu:36-176 writes them so for every scalar_t).
+template <int kN, typename T>
+__device__ __forceinline__ void sh_eval(int degree, T x, T y, T z, T (&Y)[kN]) {
   Y[0] = 0.28209479177387814f;
   if (degree < 1) return;
   Y[1] = -0.48860251190291987f * y;
   Y[2] = 0.48860251190291987f * z;
   Y[3] = -0.48860251190291987f * x;
   if (degree < 2) return;
-  const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
+  const T xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
   Y[4] = 1.0925484305920792f * xy;
   Y[5] = -1.0925484305920792f * yz;
   Y[6] = 0.94617469575755997f * zz - 0.31539156525251999f;
@@ -43,15 +44,14 @@ __device__ __forceinline__ void sh_eval(int degree, float x, float y, float z, f
 
 // Accumulates t_l * grad(Y_l) for l >= 1 into (dx, dy, dz); t[l] is the caller's per-basis scalar
 // (dot(grad_rgb, coeff_l) for SH->RGB, the upstream gradient for the bare encoder).
-template <int kN>
-__device__ __forceinline__ void sh_grad_accumulate(int degree, float x, float y, float z, const float (&t)[kN],
-                                                   float& dx, float& dy, float& dz) {
+template <int kN, typename T>
+__device__ __forceinline__ void sh_grad_accumulate(int degree, T x, T y, T z, const T (&t)[kN], T& dx, T& dy, T& dz) {
   if (degree < 1) return;
   dy += t[1] * -0.48860251190291992f;
   dz += t[2] * 0.48860251190291992f;
   dx += t[3] * -0.48860251190291992f;
   if (degree < 2) return;
-  const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
+  const T xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
   dx += t[4] * (1.0925484305920792f * y);
   dy += t[4] * (1.0925484305920792f * x);
   dy += t[5] * (-1.0925484305920792f * z);

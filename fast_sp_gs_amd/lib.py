@@ -25,6 +25,7 @@ def parse_prototypes(header_text: str, prefix: str) -> Dict[str, Tuple[object, L
     """Returns {name: (restype, [argtypes])} for every `prefix*` function declared in a C header."""
     text = re.sub(r"/\*.*?\*/", " ", header_text, flags=re.S)
     text = re.sub(r"//[^\n]*", " ", text)
+    text = re.sub(r"^[ \t]*#[^\n]*", " ", text, flags=re.M)  # preprocessor lines
     protos = {}
     for m in re.finditer(r"([A-Za-z_][\w\s\*]*?)\b(" + prefix + r"\w+)\s*\(([^)]*)\)\s*;", text):
         ret, name, args = m.group(1).strip(), m.group(2), m.group(3).strip()

@@ -6,6 +6,7 @@ from __future__ import annotations
 import torch
 from torch import Tensor, nn
 from torch.autograd import Function
+from torch.amp import custom_bwd, custom_fwd
 from torch.autograd.function import once_differentiable
 
 from fast_sp_gs_amd._C import get_C_function
@@ -18,8 +19,9 @@ class _sh_encoder(Function):
     _backward = staticmethod(get_C_function('sh_encode_backward'))
 
     @staticmethod
+    @custom_fwd(cast_inputs=torch.float32, device_type='cuda')  # float32 under autocast; otherwise the caller's dtype
     def forward(ctx, inputs, degree):
-        inputs = inputs.float().contiguous()
+        inputs = inputs.contiguous()
         B, input_dim = inputs.shape
         outputs = torch.empty(B, (degree + 1) ** 2, dtype=inputs.dtype, device=inputs.device)
         _sh_encoder._forward(inputs, outputs, B, input_dim, degree)
@@ -29,6 +31,7 @@ class _sh_encoder(Function):
 
     @staticmethod
     @once_differentiable
+    @custom_bwd(device_type='cuda')
     def backward(ctx, grad):
         inputs, = ctx.saved_tensors
         B, input_dim, degree = ctx.dims
@@ -76,10 +79,11 @@ class _freq_encoder(Function):
     _backward = staticmethod(get_C_function('freq_encode_backward'))
 
     @staticmethod
+    @custom_fwd(cast_inputs=torch.float32, device_type='cuda')  # float32 under autocast; otherwise the caller's dtype
     def forward(ctx, inputs, degree, include_input, scale):
         if not inputs.is_cuda:
             inputs = inputs.cuda()
-        inputs = inputs.float().contiguous()
+        inputs = inputs.contiguous()
         outputs = _freq_encoder._forward(inputs, degree, include_input, scale)
         ctx._info = [degree, include_input, scale]
         ctx.save_for_backward(outputs)
@@ -87,6 +91,7 @@ class _freq_encoder(Function):
 
     @staticmethod
     @once_differentiable
+    @custom_bwd(device_type='cuda')
     def backward(ctx, grad):
         outputs, = ctx.saved_tensors
         degree, include_input, scale = ctx._info

@@ -218,17 +218,33 @@ int fsgs_sh_to_rgb_backward(int P, int F, int degree, int clamp, const float* po
     const float* sh, const float* rgb, const float* grad_rgb, float* grad_dir, float* grad_campos, float* grad_sh,
     void* stream);
 
-/* sh_encode_forward / sh_encode_backward -- fast_2d_gs/_C/src/nerf/shencoder.cu:657-691. in[B,D>=3], out[B,(C+1)^2];
- * the backward writes the first three components of every grad_in row. */
+/* Element types of the `_typed` entry points below. The reference dispatches these small operators on the tensor's
+ * scalar type (AT_DISPATCH_FLOATING_TYPES[_AND_HALF]); a `_typed` entry takes the same buffers as untyped addresses plus
+ * this selector. FSGS_DTYPE_F16 is IEEE binary16 storage with single-precision arithmetic. */
+#define FSGS_DTYPE_F32 0
+#define FSGS_DTYPE_F64 1
+#define FSGS_DTYPE_F16 2
+
+/* sh_encode_forward / sh_encode_backward -- fast_2d_gs/_C/src/nerf/shencoder.cu:657-691 (float, double and half, :667,
+ * :688). in[B,D>=3], out[B,(C+1)^2]; the backward writes the first three components of every grad_in row. The
+ * coefficients are single-precision literals for every element type, as at shencoder.cu:36-176. */
 int fsgs_sh_encode_forward(int B, int D, int C, const float* in, float* out, void* stream);
 int fsgs_sh_encode_backward(int B, int D, int C, const float* grad, const float* in, float* grad_in, void* stream);
+int fsgs_sh_encode_forward_typed(int dtype, int B, int D, int C, const void* in, void* out, void* stream);
+int fsgs_sh_encode_backward_typed(int dtype, int B, int D, int C, const void* grad, const void* in, void* grad_in,
+                                  void* stream);
 
-/* freq_encode_forward / freq_encode_backward -- fast_2d_gs/_C/src/nerf/freqencoder.cu:63-104.
- * out[B, Din * (2 * degree + include_input)] laid out [x | sin 2^0 s x | cos 2^0 s x | sin 2^1 s x | ...]. */
+/* freq_encode_forward / freq_encode_backward -- fast_2d_gs/_C/src/nerf/freqencoder.cu:63-104 (float and double, :76,
+ * :98). out[B, Din * (2 * degree + include_input)] laid out [x | sin 2^0 s x | cos 2^0 s x | sin 2^1 s x | ...]. For
+ * double tensors the scaled angle and its sine / cosine are single precision (scalbnf at freqencoder.cu:27-28). */
 int fsgs_freq_encode_forward(int B, int Din, int degree, int include_input, double scale, const float* in,
                              float* out, void* stream);
 int fsgs_freq_encode_backward(int B, int Din, int degree, int include_input, double scale, const float* grad,
                               const float* outv, float* gin, void* stream);
+int fsgs_freq_encode_forward_typed(int dtype, int B, int Din, int degree, int include_input, double scale,
+                                   const void* in, void* out, void* stream);
+int fsgs_freq_encode_backward_typed(int dtype, int B, int Din, int degree, int include_input, double scale,
+                                    const void* grad, const void* outv, void* gin, void* stream);
 
 /* ---- nearest points, K-NN, LBS, optimiser ---------------------------------------------------------------------- */
 
@@ -239,6 +255,12 @@ int fsgs_cdist_top_forward(int B, int N, int M, int D, int largest, const float*
                            int64_t* index, void* stream);
 int fsgs_cdist_top_backward(int B, int N, int M, int D, const float* p1, const float* p2, const float* dist,
                             const int64_t* index, const float* gdist, float* g1, float* g2, void* stream);
+/* The same for float or double points (cdist_top.cu:48, :116); dist, gdist, g1, g2 have the points' element type. */
+int fsgs_cdist_top_forward_typed(int dtype, int B, int N, int M, int D, int largest, const void* x, const void* y,
+                                 void* dist, int64_t* index, void* stream);
+int fsgs_cdist_top_backward_typed(int dtype, int B, int N, int M, int D, const void* p1, const void* p2,
+                                  const void* dist, const int64_t* index, const void* gdist, void* g1, void* g2,
+                                  void* stream);
 
 /* K nearest rows of y[M,D] for every row of x[N,D] (K <= 16): dist2[N,K] squared distances ascending, index[N,K]
  * int64, ties -> lower index first; slots beyond M hold (-1, -1). Replaces the reference's call

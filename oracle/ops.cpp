@@ -130,6 +130,25 @@ static void freq_fwd(int B, int Din, int degree, int include_input, T scale, con
     }
 }
 
+// The reference's kernel for double tensors (freqencoder.cu:7-30, dispatched at :76): the angle goes through scalbnf, so
+// it is narrowed to float, scaled and its sine / cosine taken in single precision; only the storage is double.
+static void freq_fwd_double_through_float(int B, int Din, int degree, int include_input, double scale, const double* in,
+                                          double* out) {
+  const int Dout = Din * (2 * degree + (include_input ? 1 : 0));
+  for (int b = 0; b < B; ++b)
+    for (int c = 0; c < Din; ++c) {
+      double* o = out + (size_t) b * Dout + c;
+      double x  = in[(size_t) b * Din + c];
+      if (include_input) o[0] = x, o += Din;
+      x = x * scale;
+      for (int d = 0; d < degree; ++d) {
+        const float v = scalbnf((float) x, d);
+        o[(2 * d + 0) * Din] = sinf(v);
+        o[(2 * d + 1) * Din] = cosf(v);
+      }
+    }
+}
+
 template <typename T>
 static void freq_bwd(int B, int Din, int degree, int include_input, T scale, const T* grad, const T* outv, T* gin) {
   const int Dout = Din * (2 * degree + (include_input ? 1 : 0));
@@ -651,6 +670,12 @@ ORACLE_API int oracle_deform_mlp_f32(int B, int Din, int Wd, int L, int skip, co
 
 INSTANTIATE_EPILOGUE(f32, float)
 INSTANTIATE_EPILOGUE(f64, double)
+
+ORACLE_API int oracle_freq_encode_forward_double_via_single(int B, int Din, int degree, int include_input, double scale,
+                                                          const double* in, double* out) {
+  freq_fwd_double_through_float(B, Din, degree, include_input, scale, in, out);
+  return 0;
+}
 
 ORACLE_API int oracle_simple_knn_f32(int P, const float* points, float* mean_dist2) {
   simple_knn<float>(P, points, mean_dist2);

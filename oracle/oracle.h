@@ -38,6 +38,9 @@ int oracle_sh_encode_forward_f32(int B, int D, int C, const float* in, float* ou
 int oracle_sh_encode_backward_f32(int B, int D, int C, const float* grad, const float* in, float* grad_in);
 int oracle_freq_encode_forward_f32(int B, int Din, int degree, int include_input, double scale, const float* in,
     float* out);
+/* The reference's forward for double tensors: angle, sine and cosine in single precision (freqencoder.cu:27-28). */
+int oracle_freq_encode_forward_double_via_single(int B, int Din, int degree, int include_input, double scale,
+    const double* in, double* out);
 int oracle_freq_encode_backward_f32(int B, int Din, int degree, int include_input, double scale, const float* grad,
     const float* outv, float* gin);
 int oracle_fusedssim_forward_f32(int B, int CH, int H, int W, double C1, double C2, const float* img1,

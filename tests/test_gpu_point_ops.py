@@ -102,6 +102,96 @@ def test_cdist_top(device, oracle_mod, c1):
             assert rel_err(npy(a.grad), g1) < 1e-5 and rel_err(npy(b.grad), g2) < 1e-4
 
 
+def test_small_operators_in_the_other_element_types(device, oracle_mod, c1):
+    """The element types the reference dispatches these operators on beside float32 (shencoder.cu:667,688 float / double /
+    half; freqencoder.cu:76,98 and cdist_top.cu:48,116 float / double). The outputs keep the inputs' type."""
+    O = oracle_mod
+    from fast_sp_gs_amd._C import get_C_function
+    from fast_sp_gs_amd.ops import FreqEncoder, cdist_top, sh_encode
+    g = torch.Generator().manual_seed(11)
+    dirs = c1['dirs'][:4000].double()
+    dirs = torch.nn.functional.normalize(dirs + 1e-3 * torch.randn(dirs.shape, generator=g, dtype=torch.float64), dim=-1)
+    P = dirs.shape[0]
+    # -- SH encoder, double: double arithmetic on single-precision coefficients. An axis direction shows the coefficient
+    # itself: Y_1 = -(double)(0.48860251190291987f) * y exactly.
+    axis = torch.tensor([[0.0, 1.0, 0.0]], dtype=torch.float64, device=device)
+    enc = sh_encode(axis, 1)
+    assert enc.dtype == torch.float64 and enc[0, 1].item() == -float(np.float32(0.48860251190291987))
+    for degree in (0, 3, 7):
+        n = (degree + 1) ** 2
+        d = dirs.to(device).requires_grad_()
+        enc = sh_encode(d, degree)
+        genc = torch.randn(P, n, generator=g, dtype=torch.float64)
+        enc.backward(genc.to(device))
+        ref, gref = np.zeros((P, n)), np.zeros((P, 3))
+        O.call("sh_encode_forward_f64", P, 3, degree, npy(dirs), ref)
+        O.call("sh_encode_backward_f64", P, 3, degree, npy(genc), npy(dirs), gref)
+        # the oracle's double coefficients are exact, the operator's are the reference's float literals: 6e-8 relative
+        # per coefficient, which the cancelling monomials of degree 4..7 (coefficients up to 1e2) turn into 1e-6
+        tol = 3e-7 if degree <= 3 else 3e-6
+        assert enc.dtype == torch.float64 and d.grad.dtype == torch.float64
+        assert abs_err(npy(enc), ref) < tol and rel_err(npy(d.grad), gref) < tol
+        if degree >= 2:  # two entries re-evaluated in double with the float literals: the arithmetic itself is double
+            x, y, z = (npy(dirs)[:, i] for i in range(3))
+            y4 = float(np.float32(1.0925484305920792)) * (x * y)
+            y6 = float(np.float32(0.94617469575755997)) * (z * z) - float(np.float32(0.31539156525251999))
+            assert np.abs(npy(enc)[:, 4] - y4).max() < 1e-15 and np.abs(npy(enc)[:, 6] - y6).max() < 1e-15
+        # -- half: storage only, one rounding of the single-precision result (2^-11 relative) on top of the rounding of
+        # the inputs, which the oracle receives as the same half values
+        dh = dirs.half()
+        d = dh.to(device).requires_grad_()
+        enc = sh_encode(d, degree)
+        gh = genc.half()
+        enc.backward(gh.to(device))
+        O.call("sh_encode_forward_f64", P, 3, degree, npy(dh.double()), ref)
+        O.call("sh_encode_backward_f64", P, 3, degree, npy(gh.double()), npy(dh.double()), gref)
+        assert enc.dtype == torch.float16 and d.grad.dtype == torch.float16
+        assert np.abs(npy(enc.double()) - ref).max() <= 2.0 ** -11 * max(np.abs(ref).max(), 1) * 1.01
+        assert np.abs(npy(d.grad.double()) - gref).max() <= 2.0 ** -11 * np.abs(gref).max() * 1.01
+    with pytest.raises(RuntimeError, match='element type'):
+        get_C_function('sh_encode_forward')(dirs.to(device).bfloat16(), torch.empty(P, 4, device=device).bfloat16(), P, 3, 1)
+    with pytest.raises(RuntimeError, match='dtype'):
+        get_C_function('sh_encode_forward')(dirs.to(device), torch.empty(P, 4, device=device), P, 3, 1)
+    # -- frequency encoder, double: the angle, its sine and cosine are single precision as in the reference's kernel, so
+    # the check is against the restatement of that, to the few ulp by which sinf of arguments up to 2^9 differs
+    for D, deg, inc in ((3, 10, True), (2, 6, False)):
+        x = torch.rand(777, D, generator=g, dtype=torch.float64) * 2 - 1
+        xd = x.to(device).requires_grad_()
+        out = FreqEncoder(D, deg, inc, scale=0.75)(xd)
+        gout = torch.randn(out.shape, generator=g, dtype=torch.float64)
+        out.backward(gout.to(device))
+        ref, exact = np.zeros(tuple(out.shape)), np.zeros(tuple(out.shape))
+        O.call("freq_encode_forward_double_via_single", 777, D, deg, int(inc), 0.75, npy(x), ref)
+        O.call("freq_encode_forward_f64", 777, D, deg, int(inc), 0.75, npy(x), exact)
+        assert out.dtype == torch.float64 and abs_err(npy(out), ref) < 5e-7
+        if deg == 10:  # ... which a double-precision evaluation would miss by the rounding of the angle times 2^9
+            assert abs_err(npy(out), exact) > 4e-6
+        gref = np.zeros((777, D))
+        O.call("freq_encode_backward_f64", 777, D, deg, int(inc), 0.75, npy(gout), npy(out), gref)
+        assert xd.grad.dtype == torch.float64 and rel_err(npy(xd.grad), gref) < 1e-12
+    with pytest.raises(RuntimeError, match='element type'):
+        get_C_function('freq_encode_forward')(x.to(device).half(), 4, True, 1.0)
+    # -- nearest / farthest point, double: same sequential sums, so bit for bit
+    for shape1, shape2 in (((2, 700, 3), (2, 129, 3)), ((900, 5), (33, 5))):
+        x1 = torch.randn(shape1, generator=g, dtype=torch.float64)
+        x2 = torch.randn(shape2, generator=g, dtype=torch.float64)
+        x2.view(-1, shape2[-1])[5] = x2.view(-1, shape2[-1])[2]
+        B = x1.numel() // (shape1[-2] * shape1[-1])
+        for largest in (False, True):
+            a, b = x1.to(device).requires_grad_(), x2.to(device).requires_grad_()
+            dist, idx = cdist_top(a, b, largest)
+            gd = torch.randn(dist.shape, generator=g, dtype=torch.float64)
+            dist.backward(gd.to(device))
+            rd, ri = np.zeros(dist.shape), np.zeros(dist.shape, np.int64)
+            O.call("cdist_top_forward_f64", B, shape1[-2], shape2[-2], shape1[-1], int(largest), npy(x1), npy(x2), rd, ri)
+            assert dist.dtype == torch.float64 and np.array_equal(npy(idx), ri) and np.array_equal(npy(dist), rd)
+            g1, g2 = np.zeros(shape1), np.zeros(shape2)
+            O.call("cdist_top_backward_f64", B, shape1[-2], shape2[-2], shape1[-1], npy(x1), npy(x2), rd, ri, npy(gd), g1, g2)
+            assert rel_err(npy(a.grad), g1) < 1e-14 and rel_err(npy(b.grad), g2) < 1e-13
+    with pytest.raises(RuntimeError, match='dtype'):
+        get_C_function('cdist_top')(x1.to(device), x2.to(device).float())
+
+
 def test_knn_and_lbs(device, oracle_mod, c1):
     O = oracle_mod
     from fast_sp_gs_amd._C import get_C_function

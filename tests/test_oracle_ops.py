@@ -354,3 +354,25 @@ def test_fusedssim_matches_conv2d_and_autograd(oracle_mod):
     same = np.zeros_like(a)
     assert O.call("fusedssim_forward_f64", B, CH, H, W, C1, C2, a, a, same, None, None, None) == 0
     assert np.abs(same - 1.0).max() < 1e-12
+
+
+def test_freq_encoder_double_tensor_goes_through_single_precision(oracle_mod):
+    """freqencoder.cu:27-28 scales the angle with scalbnf, which narrows a double to float: for double tensors the
+    forward is sinf / cosf of the float angle. Checked against numpy's float32 evaluation (one ulp of float), and shown
+    to be a different function from the double-precision evaluation."""
+    O = oracle_mod
+    rng = np.random.default_rng(6)
+    B, D, deg, scale = 41, 2, 10, 0.75
+    x = np.ascontiguousarray(rng.uniform(-1, 1, size=(B, D)))
+    out, exact = np.zeros((B, D * (2 * deg + 1))), np.zeros((B, D * (2 * deg + 1)))
+    assert O.call("freq_encode_forward_double_via_single", B, D, deg, 1, scale, x, out) == 0
+    assert O.call("freq_encode_forward_f64", B, D, deg, 1, scale, x, exact) == 0
+    xf = (x * scale).astype(np.float32)
+    parts = [x]
+    for d in range(deg):
+        v = np.ldexp(xf, d)
+        assert v.dtype == np.float32
+        parts += [np.sin(v).astype(np.float64), np.cos(v).astype(np.float64)]
+    assert np.abs(out - np.concatenate(parts, -1)).max() < 1.5e-7
+    assert np.array_equal(out[:, :D], x)  # the pass-through columns keep the double values
+    assert np.abs(out - exact).max() > 4e-6
