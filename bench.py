@@ -493,6 +493,35 @@ def topk_weights_ms(dev, scene, cam, reps: int = 20):
             "gs_2d_topk_weights_workload": f"k = 4 on the 300k-surfel 800x800 view, R = {int(point_list.numel())}"}
 
 
+def training_forward_ms(dev, scene, cam, reps: int = 30):
+    """The blend forward as the reference's training loop calls it (network.py:706-709): `accum_max_count` always, plus
+    `accum_weights_p` / `accum_weights_count` for its 'simp' render type, next to the plain forward of the headline."""
+    from fast_sp_gs_amd._C import get_C_function as f
+    W, H, P = cam.W, cam.H, scene.P
+    m2, colors, tm, no, depths, radii, tt = f('gs_2d_preprocess_forward')(
+        W, H, 3, False, scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs, None, cam.Tw2v,
+        cam.Tv2c, cam.campos, None, None, None)
+    ranges, point_list = f('GS_prepare')(W, H, m2, depths, radii, tt, False)
+    amc = torch.zeros(P, dtype=torch.int32, device=dev)
+    awp, awc = torch.zeros(P, device=dev), torch.zeros(P, dtype=torch.int32, device=dev)
+    fwd = f('GS_2D_render_forward')
+    out = {}
+    for name, side in (("plain", (None, None, None)), ("max_count", (amc, None, None)), ("all_three", (amc, awp, awc))):
+        run = lambda: fwd(W, H, m2, colors, no, tm, point_list, ranges, cam.near, cam.far, False, None, *side)
+        for _ in range(3):
+            run()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        out[f"blend_forward_{name}_ms"] = e0.elapsed_time(e1) / reps
+    out["blend_forward_accum_workload"] = ("GS_2D_render_forward on the benchmark view: no side outputs / accum_max_count "
+                                           "(every training step of the reference) / all three accum_* ('simp' render type)")
+    return out
+
+
 def fast_path_rate(dev, scene, cam, gi, steps: int = 20, warmup: int = 3):
     """The "fast" variant (adjugate intersection, fused corner-test binning) on the benchmark scene, forward + backward."""
     from fast_sp_gs_amd.renderer import fast_render_step
@@ -623,6 +652,7 @@ def main():
         extra.update(simple_knn_ms(dev, scene))
         extra.update(reference_note_blend_ms(dev))
         extra.update(topk_weights_ms(dev, scene, cam))
+        extra.update(training_forward_ms(dev, scene, cam))
         extra.update(gs3d_path_rate(dev, scene, cam, gi))
         extra.update(density_control_ms(dev, scene))
         extra.update(large_scene_ms(dev))

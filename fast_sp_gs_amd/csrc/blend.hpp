@@ -299,6 +299,42 @@ __device__ __forceinline__ float wave_sum_to_lane63(float v) {
   return v;
 }
 
+// ---- per-surfel side sums of the forward blends ---------------------------------------------------------------------
+// accum_weights_p / accum_weights_count: a wavefront blends one list entry at a time, so the up to 64 per-pixel adds of
+// an entry go to one address. They are summed in the wavefront first (one DPP reduction, one population count) and lane 63
+// issues one atomic per output. Must be reached by all 64 lanes; `id` and the two pointers are wave-uniform.
+__device__ __forceinline__ void wave_accumulate_weights(bool blended, float w, int id, float* __restrict__ weights_p,
+                                                        int32_t* __restrict__ weights_count) {
+  const unsigned long long who = __ballot(blended);
+  if (who == 0ull) return;
+  const float total = wave_sum_to_lane63(blended ? w : 0.0f);
+  if ((threadIdx.x & 63) == 63) {
+    if (weights_p) atomicAdd(&weights_p[id], total);
+    if (weights_count) atomicAdd(&weights_count[id], (int) __popcll(who));
+  }
+}
+
+// accum_max_count in the surfel paths: the reference adds 1 to the count of the pixel's current arg-max surfel at EVERY
+// blended entry from the first one on (its flag is never reset). A pixel's arg-max changes a few times at most, so the
+// adds are kept as a run length and issued when the arg-max moves and once after the last entry: the same integer
+// totals with a few atomics per pixel instead of one per blended entry.
+struct ArgmaxRun {
+  float wmax = 0.0f;
+  int id     = -1;
+  int run    = 0;
+};
+__device__ __forceinline__ void argmax_run_flush(ArgmaxRun& a, int32_t* __restrict__ max_count) {
+  if (a.run > 0 && max_count) atomicAdd(&max_count[a.id], a.run);
+  a.run = 0;
+}
+__device__ __forceinline__ void argmax_run_step(ArgmaxRun& a, float w, int id, int32_t* __restrict__ max_count) {
+  if (a.wmax < w) {
+    argmax_run_flush(a, max_count);
+    a.wmax = w, a.id = id;
+  }
+  ++a.run;
+}
+
 // Adds the values held by the same lane position of the four 16-lane rows; every lane gets the total.
 // gfx950's row/half swaps do it in the VALU (no LDS round trip as with a bpermute): after swapping the odd rows of one
 // copy with the even rows of another, copy A holds rows (0,0,2,2) and copy B rows (1,1,3,3); the 32-lane swap does the

@@ -4,7 +4,9 @@
 // (host entry GS_2D_render_forward): colour, opacity, the 9 auxiliary maps (depth, normal xyz, median depth,
 // distortion, M1, M2, weight sum), optional flow, n_contrib = (last contributor, median contributor), and the optional
 // accum_max_count / accum_weights_p / accum_weights_count side outputs with their quirks (the arg-max flag is never
-// reset once set, :180-197).
+// reset once set, :180-197). The side outputs are sums over (pixel, surfel) pairs; the kernel forms them per wavefront
+// or per pixel first and issues few atomics (see ArgmaxRun and the weight staging below) instead of up to three per
+// pair.
 //
 // Layout: one 256-lane block per 16x16 tile; wavefront w owns an 8x8 pixel quadrant. Surfels of the tile's sorted
 // range are gathered 128 at a time (one per lane of the first two wavefronts, colours included so the blend never goes back to HBM) into LDS as
@@ -20,7 +22,12 @@ namespace {
 #endif
 constexpr int kFwdBatch = FSGS_FWD_BATCH;  // surfels staged per round (<= block size)
 
-template <bool kAux, bool kFlow, bool kAccum>
+// kAccum: 0 = no side outputs, 1 = accum_max_count only (what the reference's training loop passes on every step),
+// 2 = accum_weights_p and / or accum_weights_count as well.
+constexpr int kAccSlots  = 16;  // entries whose per-pixel weights a wavefront stages before it sums them
+constexpr int kAccStride = 68;  // floats per staged entry: 64 lanes + 4, so that the 16 readers of a row hit 16 x 4 banks
+
+template <bool kAux, bool kFlow, int kAccum>
 __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
     int ordered, const int* __restrict__ tile_order, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const float2* __restrict__ means2D, const float* __restrict__ colors, const float* __restrict__ trans_mat,
@@ -33,6 +40,12 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   __shared__ SplatCold s_cold[kFwdBatch];
   __shared__ float s_t2[kFlow ? kFwdBatch * 9 : 1];
   __shared__ unsigned char s_mask[kFwdBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
+  // accum_weights_*: every lane of a wavefront blends the same entry, so an entry's per-pixel weights all go to one
+  // address. Each wavefront parks them in its own LDS rows (one plain store per entry), and after kAccSlots entries sums
+  // all rows at once -- lane l adds 16 lanes' worth of entry l & 15, two row / half swaps finish the sum -- and lanes
+  // 0..15 issue one atomic per entry and output.
+  __shared__ __attribute__((aligned(16))) float s_accw[kAccum == 2 ? 4 * kAccSlots * kAccStride : 4];
+  __shared__ int s_accid[kAccum == 2 ? 4 * kAccSlots : 1], s_accn[kAccum == 2 ? 4 * kAccSlots : 1];
 
   const int gx = (W + kTile - 1) / kTile;
   const int tile = scheduled_tile(ordered, tile_order), tile_x = tile % gx, tile_y = tile / gx;
@@ -52,9 +65,23 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   const float far_scale = far_n / (far_n - near_n);
   float T = 1.0f, C0 = 0, C1 = 0, C2 = 0;
   float N0 = 0, N1 = 0, N2 = 0, D = 0, M1 = 0, M2 = 0, dist = 0, median = 0, wsum = 0, f0 = 0, f1 = 0;
-  int last = 0, median_c = -1, wmax_id = -1;
-  float wmax = 0;
-  bool flag  = false;
+  int last = 0, median_c = -1;
+  ArgmaxRun argmax;
+  int acc_slot = 0;  // staged entries of this wavefront (wave-uniform)
+  auto flush_weights = [&]() {
+    if (acc_slot == 0) return;
+    const float4* src = (const float4*) &s_accw[(wave * kAccSlots + (lane & 15)) * kAccStride + (lane >> 4) * 16];
+    const float4 a = src[0], b = src[1], c = src[2], d = src[3];
+    float t = (((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w))) +
+              (((c.x + c.y) + (c.z + c.w)) + ((d.x + d.y) + (d.z + d.w)));
+    t = cross_row_sum(t);
+    if (lane < acc_slot) {
+      const int id = s_accid[wave * kAccSlots + lane];
+      if (accum_weights_p) atomicAdd(&accum_weights_p[id], t);
+      if (accum_weights_count) atomicAdd(&accum_weights_count[id], s_accn[wave * kAccSlots + lane]);
+    }
+    acc_slot = 0;
+  };
 
   Splat next;
   float next_t2[9];
@@ -105,8 +132,16 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
         const float test_T = T * (1.0f - h.alpha);
         const bool sat     = hit && test_T < 0.0001f;
         done               = done || sat;
+        const float w      = h.alpha * T;
+        if (kAccum == 2) {
+          const unsigned long long who = __ballot(hit && !sat);
+          if (who != 0ull) {
+            s_accw[(wave * kAccSlots + acc_slot) * kAccStride + lane] = hit && !sat ? w : 0.0f;
+            if (lane == 0) s_accid[wave * kAccSlots + acc_slot] = cold.id, s_accn[wave * kAccSlots + acc_slot] = (int) __popcll(who);
+            if (++acc_slot == kAccSlots) flush_weights();
+          }
+        }
         if (hit && !sat) {
-          const float w         = h.alpha * T;
           const int contributor = b * kFwdBatch + j + 1;
           if (kAux) {
             const float A  = 1.0f - T;
@@ -118,11 +153,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
             M2   = fmaf(mm, w, M2);
             if (T > 0.5f) median = h.depth, median_c = contributor;
             N0 = fmaf(cold.nx, w, N0), N1 = fmaf(cold.ny, w, N1), N2 = fmaf(cold.nz, w, N2);
-            if (kAccum) {
-              if (wmax < w) wmax = w, wmax_id = cold.id, flag = true;
-              if (accum_weights_p) atomicAdd(&accum_weights_p[cold.id], w);
-              if (accum_weights_count) atomicAdd(&accum_weights_count[cold.id], 1);
-            }
+            if (kAccum != 0) argmax_run_step(argmax, w, cold.id, accum_max_count);
             if (kFlow) {
               const float* Q = &s_t2[j * 9];
               const float u2 = fmaf(Q[0], h.sx, fmaf(Q[1], h.sy, Q[2]));
@@ -133,9 +164,6 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
               f1 = fmaf(v2 / w2 - pyf, w, f1);
             }
             wsum += w;
-          }
-          if (kAccum) {
-            if (flag && accum_max_count) atomicAdd(&accum_max_count[wmax_id], 1);
           }
           C0 = fmaf(cold.r, w, C0), C1 = fmaf(cold.g, w, C1), C2 = fmaf(cold.b, w, C2);
           T    = test_T;
@@ -170,6 +198,8 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
     }
   }
 
+  if (kAccum != 0) argmax_run_flush(argmax, accum_max_count);
+  if (kAccum == 2) flush_weights();
   if (inside) {
     out_opacity[pix]      = 1.0f - T;
     n_contrib[pix]        = last;
@@ -244,7 +274,7 @@ FSGS_API int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, doubl
   FSGS_REQUIRE(only_image || out_extras, "GS_2D_render_forward: out_extras is required unless only_image");
   const bool aux   = !only_image;
   const bool flow  = aux && trans_mat_t2 != nullptr;
-  const bool accum = aux && (accum_max_count || accum_weights_p || accum_weights_count);
+  const int accum = !aux ? 0 : (accum_weights_p || accum_weights_count) ? 2 : accum_max_count ? 1 : 0;
   FSGS_REQUIRE(!flow || out_flow, "GS_2D_render_forward: out_flow is required with trans_mat_t2");
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
@@ -256,11 +286,13 @@ FSGS_API int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, doubl
                      ranges, point_list, (const float2*) means2D, colors, trans_mat, (const float4*) normal_opacity, \
                      (const float4*) records, trans_mat_t2, n_contrib, out_color, out_opacity, out_extras, (float2*) out_flow,                \
                      accum_max_count, accum_weights_p, accum_weights_count)
-  if (!aux) FSGS_LAUNCH_FWD(false, false, false);
-  else if (flow && accum) FSGS_LAUNCH_FWD(true, true, true);
-  else if (flow) FSGS_LAUNCH_FWD(true, true, false);
-  else if (accum) FSGS_LAUNCH_FWD(true, false, true);
-  else FSGS_LAUNCH_FWD(true, false, false);
+  if (!aux) FSGS_LAUNCH_FWD(false, false, 0);
+  else if (flow && accum == 2) FSGS_LAUNCH_FWD(true, true, 2);
+  else if (flow && accum == 1) FSGS_LAUNCH_FWD(true, true, 1);
+  else if (flow) FSGS_LAUNCH_FWD(true, true, 0);
+  else if (accum == 2) FSGS_LAUNCH_FWD(true, false, 2);
+  else if (accum == 1) FSGS_LAUNCH_FWD(true, false, 1);
+  else FSGS_LAUNCH_FWD(true, false, 0);
 #undef FSGS_LAUNCH_FWD
   return check_launch("GS_2D_render_forward");
 }

@@ -160,9 +160,8 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
   const float far_scale = far_n / (far_n - near_n);
   float T = 1.0f, C0 = 0, C1 = 0, C2 = 0;
   float N0 = 0, N1 = 0, N2 = 0, D = 0, M1 = 0, M2 = 0, dist = 0, median = 0, f0 = 0, f1 = 0;
-  int last = 0, median_c = -1, wmax_id = -1;
-  float wmax = 0;
-  bool flag  = false;
+  int last = 0, median_c = -1;
+  ArgmaxRun argmax;
 
   FastSplat next;
   float next_t2[9];
@@ -239,9 +238,11 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
           const float test_T = T * (1.0f - h.alpha);
           const bool sat     = hit && test_T < 0.0001f;
           done               = done || sat;
-          if (!hit || sat) continue;
           const float w         = h.alpha * T;
           const SplatCold cold  = s_cold[j];
+          if (kAccum && (accum_weights_p || accum_weights_count))
+            wave_accumulate_weights(hit && !sat, w, cold.id, accum_weights_p, accum_weights_count);
+          if (!hit || sat) continue;
           const int contributor = b * kBatch + j + 1;
           if (kAux) {
             const float A = 1.0f - T;
@@ -252,11 +253,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
             M2 += m * m * w;
             if (T > 0.5f) median = h.depth, median_c = contributor;
             N0 += cold.nx * w, N1 += cold.ny * w, N2 += cold.nz * w;
-            if (kAccum) {
-              if (wmax < w) wmax = w, wmax_id = cold.id, flag = true;
-              if (accum_weights_p) atomicAdd(&accum_weights_p[cold.id], w);
-              if (accum_weights_count) atomicAdd(&accum_weights_count[cold.id], 1);
-            }
+            if (kAccum) argmax_run_step(argmax, w, cold.id, accum_max_count);
             if (kFlow) {
               const float* Q = &s_t2[j * 9];
               const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
@@ -267,9 +264,6 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
               f1 += (v2 / w2 - pyf) * w;
             }
           }
-          if (kAccum) {
-            if (flag && accum_max_count) atomicAdd(&accum_max_count[wmax_id], 1);
-          }
           C0 += cold.r * w, C1 += cold.g * w, C2 += cold.b * w;
           T    = test_T;
           last = contributor;
@@ -278,6 +272,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
     }
   }
 
+  if (kAccum) argmax_run_flush(argmax, accum_max_count);
   if (inside) {
     out_opacity[pix]        = 1.0f - T;
     n_contrib[pix]          = last;

@@ -164,15 +164,14 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
         const float test_T = T * (1.0f - h.alpha);
         const bool sat     = hit && test_T < 0.0001f;
         done               = done || sat;
+        const float w      = h.alpha * T;
+        if (kAccum && (accum_weights_p || accum_weights_count))
+          wave_accumulate_weights(hit && !sat, w, hot.id, accum_weights_p, accum_weights_count);
         if (hit && !sat) {
-          const float w = h.alpha * T;
 #pragma unroll
           for (int k = 0; k < 3 + E; ++k) C[k] = fmaf(s_feat[j][k], w, C[k]);
           if (kAccum) {
-            const int id = hot.id;
-            if (wmax < w) wmax = w, wmax_id = id, flag = true;
-            if (accum_weights_p) atomicAdd(&accum_weights_p[id], w);
-            if (accum_weights_count) atomicAdd(&accum_weights_count[id], 1);
+            if (wmax < w) wmax = w, wmax_id = hot.id, flag = true;
           }
           T    = test_T;
           last = b * kG3Batch + j + 1;
