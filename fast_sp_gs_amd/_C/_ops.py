@@ -135,8 +135,10 @@ def _workspace(nbytes: int, device) -> Tensor:
 def gs_2d_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: bool, means3D: Tensor, scales: Tensor,
                              rotations: Tensor, opacities: Tensor, shs: Tensor, sh_rest: Optional[Tensor],
                              Tw2v: Tensor, Tv2c: Tensor, cam_pos: Tensor, trans_precomp: Optional[Tensor] = None,
-                             means2D: Optional[Tensor] = None, culling: Optional[Tensor] = None) -> List[Tensor]:
-    """gs_2d_preprocess.cu:331-421 -> [means2D, colors, trans_mat, normal_opacity, depths, radii, tiles_touched]."""
+                             means2D: Optional[Tensor] = None, culling: Optional[Tensor] = None,
+                             return_records: bool = False) -> List[Tensor]:
+    """gs_2d_preprocess.cu:331-421 -> [means2D, colors, trans_mat, normal_opacity, depths, radii, tiles_touched]
+    (+ records[P,20], the packed per-surfel record of gs_2d_pack_records written by the same kernel, on request)."""
     what = 'gs_2d_preprocess_forward'
     _f32(what, means3D=means3D, scales=scales, rotations=rotations, opacities=opacities, shs=shs, Tw2v=Tw2v,
          Tv2c=Tv2c, cam_pos=cam_pos)
@@ -182,15 +184,17 @@ def gs_2d_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: bool, me
     radii = torch.empty((P,), dtype=torch.int32, device=means3D.device)
     tiles_touched = torch.empty((P,), dtype=torch.int32, device=means3D.device)
     normal_opacity = torch.empty((P, 4), **opt)
+    records = torch.empty((P, 20), **opt) if return_records else None
     with _timed('gs_2d_preprocess_forward'):
         rc = _lib().fsgs_gs_2d_preprocess_forward(
             P, W, H, sh_degree, M, L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(opacities), L.ptr(shs),
             L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(cam_pos), L.ptr(trans_precomp),
             L.ptr(culling), int(preserve), L.ptr(means2D_), None if sh_degree < 0 else L.ptr(colors),
             None if trans_precomp is not None else L.ptr(trans_mat), L.ptr(normal_opacity), L.ptr(depths), L.ptr(radii),
-            L.ptr(tiles_touched), L.current_stream())
+            L.ptr(tiles_touched), L.ptr(records), L.current_stream())
     L.check(rc, what)
-    return [means2D_, colors, trans_mat, normal_opacity, depths, radii, tiles_touched]
+    out = [means2D_, colors, trans_mat, normal_opacity, depths, radii, tiles_touched]
+    return out + [records] if return_records else out
 
 
 def gs_2d_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs, sh_rest,

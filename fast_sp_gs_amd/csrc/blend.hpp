@@ -39,7 +39,6 @@ constexpr int kRecordFloats = 20;
 
 struct SplatExtra {
   int radius;
-  int64_t offset;
 };
 
 __device__ __forceinline__ Splat gather_splat(int id, const float2* __restrict__ means2D,
@@ -57,7 +56,7 @@ __device__ __forceinline__ Splat gather_splat(int id, const float2* __restrict__
     s.cold.nx = q3.x, s.cold.ny = q3.y, s.cold.nz = q3.z, s.cold.r = q3.w;
     s.cold.g = q4.x, s.cold.b = q4.y;
     s.cold.id = id, s.cold.pad = 0;
-    if (extra) extra->radius = __float_as_int(q4.z), extra->offset = __float_as_int(q4.w);
+    if (extra) extra->radius = __float_as_int(q4.z);
     return s;
   }
   const float* M = trans_mat + 9 * (size_t) id;

@@ -89,7 +89,7 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
     const float* __restrict__ campos, const float* __restrict__ trans_precomp, const uint8_t* __restrict__ culling,
     int means2D_preserve, float2* __restrict__ means2D, float* __restrict__ colors, float* __restrict__ trans_mat,
     float4* __restrict__ normal_opacity, float* __restrict__ depths, int32_t* __restrict__ radii,
-    int32_t* __restrict__ tiles_touched) {
+    int32_t* __restrict__ tiles_touched, float4* __restrict__ records) {
   constexpr bool kStage = kSh == 16;  // degree <= 3: SH rows travel through LDS, read from HBM line by line
   __shared__ float s_Tw2v[16], s_Tw2c[16];
   __shared__ float s_rows[kStage ? kShStageRows * kShStageStride : 1];
@@ -184,6 +184,23 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
   tiles_touched[i] = ok ? area : 0;
   if (ok || !means2D_preserve) means2D[i] = ok ? make_float2(c2[0], c2[1]) : make_float2(0.0f, 0.0f);
   normal_opacity[i] = ok ? make_float4(nrm[0], nrm[1], nrm[2], opacities[i]) : make_float4(0, 0, 0, 0);
+  if (records) {
+    // The blend kernels' 80-byte record (layout of pack_records_kernel), written here while every field is in
+    // registers. Surfels that are not rendered never enter a tile list; their records are zeros.
+    const float* col = sh_degree >= 0 ? rgb : shs + 3 * (size_t) i;
+    const float op   = opacities[i];
+    float4* r        = records + 5 * (size_t) i;
+    if (ok) {
+      r[0] = make_float4(M[0], M[1], M[2], M[3]);
+      r[1] = make_float4(M[4], M[5], M[6], M[7]);
+      r[2] = make_float4(M[8], c2[0], c2[1], op);
+      r[3] = make_float4(nrm[0], nrm[1], nrm[2], col[0]);
+      r[4] = make_float4(col[1], col[2], __int_as_float(f2i_sat(radius)), 0.0f);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 5; ++k) r[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+  }
 }
 
 __device__ __forceinline__ void transmat_backward(int W, int H, float sx, float sy, const float4 q, const float* Tw2c,
@@ -418,8 +435,9 @@ FSGS_API int fsgs_gs_2d_preprocess_forward(int P, int W, int H, int sh_degree, i
     const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
     const float* Tw2v, const float* Tv2c, const float* campos, const float* trans_precomp, const uint8_t* culling,
     int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* normal_opacity, float* depths,
-    int32_t* radii, int32_t* tiles_touched, void* stream) {
+    int32_t* radii, int32_t* tiles_touched, float* records, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "gs_2d_preprocess_forward: bad sizes P=%d W=%d H=%d", P, W, H);
+  FSGS_REQUIRE(((uintptr_t) records & 15) == 0, "gs_2d_preprocess_forward: records must be 16-byte aligned");
   FSGS_REQUIRE(sh_degree <= kMaxShDegree, "gs_2d_preprocess_forward: sh_degree %d > %d not supported", sh_degree,
                kMaxShDegree);
   if (sh_degree >= 0)
@@ -435,7 +453,7 @@ FSGS_API int fsgs_gs_2d_preprocess_forward(int P, int W, int H, int sh_degree, i
                               : (wave_rows ? preprocess_forward_kernel<16, true> : preprocess_forward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh, means3D, (const float2*) scales, (const float4*) rotations, opacities, shs,
                      sh_rest, Tw2v, Tv2c, campos, trans_precomp, culling, means2D_preserve, (float2*) means2D, colors,
-                     trans_mat, (float4*) normal_opacity, depths, radii, tiles_touched);
+                     trans_mat, (float4*) normal_opacity, depths, radii, tiles_touched, (float4*) records);
   return check_launch("gs_2d_preprocess_forward");
 }
 

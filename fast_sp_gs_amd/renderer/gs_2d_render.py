@@ -60,20 +60,19 @@ class _GS_2D_Render(torch.autograd.Function):
     _preprocess_backward = get_C_function('gs_2d_preprocess_backward')
     _render_forward = get_C_function('GS_2D_render_forward')
     _render_backward = get_C_function('GS_2D_render_backward')
-    _pack_records = get_C_function('gs_2d_pack_records')
 
     @staticmethod
     def forward(ctx, means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, campos, size,
                 sh_degree, is_opengl, near_n, far_n, only_image, trans_precomp, means2D, transe_mat_t2, culling,
                 accum_max_count, accum_weights_p, accum_weights_count):
         W, H = size
-        means2D, colors, trans_mat, normal_opacity, depths, radii, tiles_touched = _GS_2D_Render._preprocess_forward(
+        # the preprocess kernel also writes the blend kernels' packed per-surfel record (no second pass, no launch)
+        (means2D, colors, trans_mat, normal_opacity, depths, radii, tiles_touched,
+         records) = _GS_2D_Render._preprocess_forward(
             W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c,
-            campos, trans_precomp, means2D, culling)
-        # the packed records need the scan but not the instance count: they are built while the host waits for it
-        tile_range, point_list, point_offsets, records = GS_prepare(
-            W, H, means2D, depths, radii, tiles_touched, False, return_offsets=True,
-            overlap=lambda off: _GS_2D_Render._pack_records(means2D, colors, normal_opacity, trans_mat, radii, off))
+            campos, trans_precomp, means2D, culling, return_records=True)
+        tile_range, point_list, point_offsets = GS_prepare(
+            W, H, means2D, depths, radii, tiles_touched, False, return_offsets=True)
         pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib = _GS_2D_Render._render_forward(
             W, H, means2D, colors, normal_opacity, trans_mat, point_list, tile_range, near_n, far_n, only_image,
             transe_mat_t2, accum_max_count, accum_weights_p, accum_weights_count, records)
@@ -217,13 +216,12 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
     f = get_C_function
     W, H = cam.W, cam.H
     dev = scene.means3D.device
-    m2, colors, tm, no, depths, radii, tt = f('gs_2d_preprocess_forward')(
+    # with `packed` the preprocess kernel also writes the blend kernels' packed per-surfel record
+    m2, colors, tm, no, depths, radii, tt, *rec = f('gs_2d_preprocess_forward')(
         W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs, None,
-        cam.Tw2v, cam.Tv2c, cam.campos, None, None, None)
-    # the packed records need the scan but not the instance count: they are built while the host waits for it
-    ranges, point_list, offsets, rec = f('GS_prepare')(
-        W, H, m2, depths, radii, tt, False, return_offsets=True,
-        overlap=lambda off: f('gs_2d_pack_records')(m2, colors, no, tm, radii, off) if packed else None)
+        cam.Tw2v, cam.Tv2c, cam.campos, None, None, None, return_records=packed)
+    rec = rec[0] if packed else None
+    ranges, point_list, offsets = f('GS_prepare')(W, H, m2, depths, radii, tt, False, return_offsets=True)
     oc, oo, oe, of, nc = f('GS_2D_render_forward')(W, H, m2, colors, no, tm, point_list, ranges, cam.near, cam.far,
                                                    False, None, None, None, None, rec)
     epilogue = {}

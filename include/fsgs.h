@@ -39,12 +39,14 @@ int fsgs_debug_set_culling(int enabled);
  * (or shs[P,1,3] + sh_rest[P,n_sh,3]); sh_degree < 0: colours are the caller's own tensor and `colors` is ignored.
  * trans_precomp[P,3,3] replaces the computed transform (then trans_mat is not written). culling[P] != 0 rejects.
  * Every output row is written (zeros for rejected surfels); rows of means2D belonging to rejected surfels are left
- * untouched when means2D_preserve != 0 (the reference's caller-supplied means2D buffer). */
+ * untouched when means2D_preserve != 0 (the reference's caller-supplied means2D buffer). records (optional, [P,20],
+ * 16-byte aligned, no counterpart in the reference) receives the packed per-surfel record of fsgs_gs_2d_pack_records
+ * without a second pass over the outputs. */
 int fsgs_gs_2d_preprocess_forward(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
     const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
     const float* Tw2v, const float* Tv2c, const float* campos, const float* trans_precomp, const uint8_t* culling,
     int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* normal_opacity, float* depths,
-    int32_t* radii, int32_t* tiles_touched, void* stream);
+    int32_t* radii, int32_t* tiles_touched, float* records, void* stream);
 
 /* gs_2d_preprocess_backward -- gs_2d_preprocess.cu:423-499 (kernel :268-329). Every row of g_* is ASSIGNED: the
  * gradient for surfels with radii > 0, zeros for the others and for SH coefficients above the active degree (the
@@ -103,8 +105,10 @@ int fsgs_gs_prepare_fill_counted(int P, int W, int H, const float* means2D, cons
 /* Optional accelerator without a counterpart in the reference: packs what the blend kernels gather per surfel
  * (trans_mat, means2D, opacity, normal, colour, and -- when given -- radius and prefix-scan offset) into one 80-byte
  * record, records[P,20] floats, 16-byte aligned. Passing `records` to fsgs_gs_2d_render_forward / _backward makes them
- * read one record per list entry instead of four tensors; results are identical. Pass radii and point_offsets here if
- * the backward is going to use its ordered-sum path. */
+ * read one record per list entry instead of four tensors; results are identical. Pass radii here if the backward is
+ * going to use its ordered-sum path (it takes the radius from the record; the offset field is stored but not read).
+ * fsgs_gs_2d_preprocess_forward writes the same record itself when given a records buffer; this entry serves callers
+ * whose per-surfel tensors come from elsewhere. */
 int fsgs_gs_2d_pack_records(int P, const float* means2D, const float* colors, const float* normal_opacity,
     const float* trans_mat, const int32_t* radii, const int64_t* point_offsets, float* records, void* stream);
 

@@ -55,6 +55,17 @@ def test_preprocess_variants(name, deg, n_rows, rest_rows, device, oracle_mod):
         W, H, deg, False, d(scene.means3D), d(scene.scales), d(scene.rotations), d(scene.opacities), d(shs), d(rest),
         d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), None, d(means2D_in), d(culling))
     torch.cuda.synchronize()
+    # the packed per-surfel record written by the same kernel == the one packed afterwards from the outputs, on every
+    # rendered surfel (radius field included; the last field is unused); rows of surfels that are not rendered are zeros
+    with_rec = get_C_function('gs_2d_preprocess_forward')(
+        W, H, deg, False, d(scene.means3D), d(scene.scales), d(scene.rotations), d(scene.opacities), d(shs), d(rest),
+        d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), None, d(means2D_in), d(culling), return_records=True)
+    for a, b in zip(out, with_rec[:7]):
+        assert torch.equal(a, b)
+    packed = get_C_function('gs_2d_pack_records')(out[0], out[1], out[3], out[2], out[5], None)
+    seen = out[5] > 0
+    assert torch.equal(with_rec[7][seen][:, :19].view(torch.int32), packed[seen][:, :19].view(torch.int32))
+    assert 0 < int(seen.sum()) < P and not with_rec[7][~seen].any()
     m2, colors, tm, no, dep, radii, tt = [npy(t) for t in out]
     s = dict(means3D=npy(scene.means3D), scales=npy(scene.scales), rotations=npy(scene.rotations),
              opacities=npy(scene.opacities), Tw2v=npy(cam.Tw2v), Tv2c=npy(cam.Tv2c), campos=npy(cam.campos))
