@@ -23,6 +23,9 @@ HIPCC_FLAGS = [
     # packed-FP32 instructions are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+# Build-time choices of the kernels (-DFSGS_BWD_ROWS=1, -DFSGS_FWD_BATCH=..., ...) can be handed in through the
+# environment; they select among variants that compute the same results.
+HIPCC_FLAGS += os.environ.get("FSGS_HIPCC_DEFINES", "").split()
 NOISE = "packed-fp32-ops"
 
 

@@ -78,6 +78,15 @@ __device__ __forceinline__ void lane_pixel(int tile_x, int tile_y, int& px, int&
   py = tile_y * kTile + (wave >> 1) * 8 + (lane >> 3);
 }
 
+// The same quadrant with every 16-lane DPP row on a 4x4 pixel block: row r = lane >> 4 is block (r & 1, r >> 1) of the
+// quadrant, lane & 15 runs row-major inside the block.
+__device__ __forceinline__ void lane_pixel_blocks(int tile_x, int tile_y, int& px, int& py) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int row = lane >> 4, in = lane & 15;
+  px = tile_x * kTile + (wave & 1) * 8 + (row & 1) * 4 + (in & 3);
+  py = tile_y * kTile + (wave >> 1) * 8 + (row >> 1) * 4 + (in >> 2);
+}
+
 struct Hit {
   float kx, ky, kz, lx, ly, lz;  // the two homogeneous planes through the pixel
   float pz;                      // z of their cross product
@@ -358,7 +367,8 @@ __device__ __forceinline__ float cross_row_sum(float z) {
 // registers while doubling the lanes a partial covers, so 16 wave-wide sums cost 15 merge steps (2 DPP adds + 1 select
 // each) plus two cross-row exchanges, instead of 16 x 6 dependent DPP adds. On return every lane holds the wave total of
 // v[lane & 15].
-__device__ __forceinline__ float wave_sum16_transposed(const float (&v)[16]) {
+// On return lane l of every 16-lane row holds that ROW's total of v[l & 15].
+__device__ __forceinline__ float row_sum16_transposed(const float (&v)[16]) {
   const int lane = __lane_id();
   const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4, b3 = lane & 8;
   float w[8], x[4], y[2];
@@ -382,8 +392,10 @@ __device__ __forceinline__ float wave_sum16_transposed(const float (&v)[16]) {
   }
   const float a = y[1] + dpp_shift_zero<0x118, 0xf, 0xf>(y[1]);  // row_shr:8
   const float b = y[0] + dpp_shift_zero<0x108, 0xf, 0xf>(y[0]);  // row_shl:8
-  float z = b3 ? a : b;                                          // lane l of every row: row total of v[l & 15]
-  return cross_row_sum(z);
+  return b3 ? a : b;
+}
+__device__ __forceinline__ float wave_sum16_transposed(const float (&v)[16]) {
+  return cross_row_sum(row_sum16_transposed(v));
 }
 
 }  // namespace fsgs

@@ -30,6 +30,17 @@ constexpr int kGradSlots = 18;
 #endif
 constexpr int kBwdBatch = FSGS_BWD_BATCH;  // surfels staged per round
 static_assert(kBwdBatch <= kWave, "one wavefront stages a batch and another flushes it");
+// Work unit of the gradient pass. 0 (default): one list entry per pass of a wavefront over its 8x8 quadrant. 1: each
+// 16-lane DPP row of a wavefront owns a 4x4 pixel block and walks its own list of the entries that blend into that block
+// (see "two phases" in the kernel). Measured at 300k surfels, 800x800: 6 % fewer vector instructions (213 M against
+// 227 M; the intersection has to be evaluated in both phases), 66 % more scalar ones, and the LDS adds that replace the
+// plain per-wavefront stores keep the LDS pipeline busy four times as long, so the launch takes 462 us against 449 us.
+// Same results either way; kept as a build-time choice.
+#ifndef FSGS_BWD_ROWS
+#define FSGS_BWD_ROWS 0
+#endif
+constexpr bool kBwdRows = FSGS_BWD_ROWS != 0;
+static_assert(!kBwdRows || kBwdBatch == kWave, "the per-row hit lists are 64-bit masks over one staged batch");
 
 template <bool kAux, bool kFlow, bool kSlots>
 __global__ void __launch_bounds__(kBlendThreads) __attribute__((amdgpu_waves_per_eu(FSGS_BWD_WAVES, FSGS_BWD_WAVES)))
@@ -59,7 +70,8 @@ blend_backward_kernel(
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int tile = scheduled_tile(ordered, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
-  lane_pixel(tile_x, tile_y, px, py);
+  if (kBwdRows) lane_pixel_blocks(tile_x, tile_y, px, py);
+  else lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
   const size_t HW   = (size_t) H * W;
   const size_t pix  = (size_t) W * py + px;
@@ -174,6 +186,81 @@ blend_backward_kernel(
      const int jj = chunk * kWave + lane;
      unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u) &&
                                         (n_todo - 1 - (b * kBwdBatch + jj)) < wave_max_contrib);
+     // Gradient of one (pixel, entry) pair that blends: advances the pixel's back-to-front state and fills the 16 + 2
+     // per-surfel components. `j` (staging slot) and `pos` (list position) may differ between the rows of a wavefront.
+     auto pair_gradients = [&](const SplatHot& hot, const SplatCold& cold, int j, int pos, const Hit& h, float (&g)[16],
+                               float& g2x, float& g2y, bool& filtered) {
+       T             = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+       const float w = h.alpha * T;
+       // All channels that enter the image linearly (colour, depth, opacity, normal) share one back-to-front
+       // recurrence: with c = <upstream gradient, channel values of this surfel>, the reference's per-channel
+       // accumulators acc_x = last_alpha * last_x + (1 - last_alpha) * acc_x contract to a single scalar.
+       float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
+       g[0] = w * dLp0, g[1] = w * dLp1, g[2] = w * dLp2;
+
+       float dL_dalpha = 0.0f, dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f;
+       if (kAux) {
+         const float rd     = __builtin_amdgcn_rcpf(h.depth);
+         const float m_d    = far_scale * (1.0f - near_n * rd);
+         const float dmd_dd = far_scale * near_n * rd * rd;
+         if (pos == median_contrib - 1) dL_dz += dL_dmedian;
+         const float dL_dweight = (final_D2 + m_d * m_d * final_A - 2.0f * m_d * final_D) * dL_dreg;
+         dL_dalpha += dL_dweight - last_dL_dT;
+         last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
+         const float dL_dmd = 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg;
+         dL_dz += dL_dmd * dmd_dd;
+         c_lin += h.depth * dL_ddepth + dL_daccum + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
+         g[12] = w * dLn0, g[13] = w * dLn1, g[14] = w * dLn2;
+         dL_dz += w * dL_ddepth;
+         dsx = dL_dz * hot.m[6], dsy = dL_dz * hot.m[7];
+       }
+       acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
+       last_lin = c_lin;
+       dL_dalpha += c_lin - acc_lin;
+       if (kFlow) {
+         const float* Q = &s_t2[j * 9];
+         const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
+         const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
+         float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
+         w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
+         acc_f0 = last_alpha * last_f0 + (1.0f - last_alpha) * acc_f0;
+         acc_f1 = last_alpha * last_f1 + (1.0f - last_alpha) * acc_f1;
+         last_f0 = u2 / w2 - pxf, last_f1 = v2 / w2 - pyf;
+         dL_dalpha += (last_f0 - acc_f0) * dLf0 + (last_f1 - acc_f1) * dLf1;
+         const float gu = w / w2 * dLf0, gv = w / w2 * dLf1;
+         const float gw = -w / (w2 * w2) * (u2 * dLf0 + v2 * dLf1);
+         dsx += Q[0] * gu + Q[3] * gv + Q[6] * gw;
+         dsy += Q[1] * gu + Q[4] * gv + Q[7] * gw;
+         acc_w = last_alpha + (1.0f - last_alpha) * acc_w;
+         dL_dalpha += (1.0f - acc_w) * dL_dsum_w;
+       }
+       dL_dalpha *= T;
+       last_alpha = h.alpha;
+
+       const float dL_dG = hot.opacity * dL_dalpha;
+       if (h.rho3d <= h.rho2d) {
+         dsx += dL_dG * -h.G * h.sx;
+         dsy += dL_dG * -h.G * h.sy;
+         const float rz  = __builtin_amdgcn_rcpf(h.pz);
+         const float dpx = dsx * rz, dpy = dsy * rz;
+         const float dpz = -(dpx * h.sx + dpy * h.sy);
+         const float dkx = h.ly * dpz - h.lz * dpy, dky = h.lz * dpx - h.lx * dpz, dkz = h.lx * dpy - h.ly * dpx;
+         const float dlx = dpy * h.kz - dpz * h.ky, dly = dpz * h.kx - dpx * h.kz, dlz = dpx * h.ky - dpy * h.kx;
+         g[3] = -dkx, g[4] = -dky, g[5] = -dkz;
+         g[6] = -dlx, g[7] = -dly, g[8] = -dlz;
+         g[9]  = pxf * dkx + pyf * dlx + dL_dz * h.sx;
+         g[10] = pxf * dky + pyf * dly + dL_dz * h.sy;
+         g[11] = pxf * dkz + pyf * dlz + dL_dz;
+       } else {
+         g2x   = dL_dG * (-h.G * 2.0f * h.dx);
+         g2y   = dL_dG * (-h.G * 2.0f * h.dy);
+         g[9]  = dL_dz * h.sx;
+         g[10] = dL_dz * h.sy;
+         g[11] = dL_dz;
+         filtered = true;
+       }
+       g[15] = h.G * dL_dalpha;
+           };
      auto backward_entry = [&](const SplatHot& hot, const SplatCold& cold, int j) {
       const int pos = n_todo - 1 - (b * kBwdBatch + j);  // 0-based position in the tile's list
       Hit h;
@@ -184,78 +271,7 @@ blend_backward_kernel(
       bool filtered = false;
 #pragma unroll
       for (int c = 0; c < 16; ++c) g[c] = 0.0f;
-      if (hit) {
-        T             = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
-        const float w = h.alpha * T;
-        // All channels that enter the image linearly (colour, depth, opacity, normal) share one back-to-front
-        // recurrence: with c = <upstream gradient, channel values of this surfel>, the reference's per-channel
-        // accumulators acc_x = last_alpha * last_x + (1 - last_alpha) * acc_x contract to a single scalar.
-        float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
-        g[0] = w * dLp0, g[1] = w * dLp1, g[2] = w * dLp2;
-
-        float dL_dalpha = 0.0f, dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f;
-        if (kAux) {
-          const float rd     = __builtin_amdgcn_rcpf(h.depth);
-          const float m_d    = far_scale * (1.0f - near_n * rd);
-          const float dmd_dd = far_scale * near_n * rd * rd;
-          if (pos == median_contrib - 1) dL_dz += dL_dmedian;
-          const float dL_dweight = (final_D2 + m_d * m_d * final_A - 2.0f * m_d * final_D) * dL_dreg;
-          dL_dalpha += dL_dweight - last_dL_dT;
-          last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
-          const float dL_dmd = 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg;
-          dL_dz += dL_dmd * dmd_dd;
-          c_lin += h.depth * dL_ddepth + dL_daccum + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
-          g[12] = w * dLn0, g[13] = w * dLn1, g[14] = w * dLn2;
-          dL_dz += w * dL_ddepth;
-          dsx = dL_dz * hot.m[6], dsy = dL_dz * hot.m[7];
-        }
-        acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
-        last_lin = c_lin;
-        dL_dalpha += c_lin - acc_lin;
-        if (kFlow) {
-          const float* Q = &s_t2[j * 9];
-          const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
-          const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
-          float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
-          w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
-          acc_f0 = last_alpha * last_f0 + (1.0f - last_alpha) * acc_f0;
-          acc_f1 = last_alpha * last_f1 + (1.0f - last_alpha) * acc_f1;
-          last_f0 = u2 / w2 - pxf, last_f1 = v2 / w2 - pyf;
-          dL_dalpha += (last_f0 - acc_f0) * dLf0 + (last_f1 - acc_f1) * dLf1;
-          const float gu = w / w2 * dLf0, gv = w / w2 * dLf1;
-          const float gw = -w / (w2 * w2) * (u2 * dLf0 + v2 * dLf1);
-          dsx += Q[0] * gu + Q[3] * gv + Q[6] * gw;
-          dsy += Q[1] * gu + Q[4] * gv + Q[7] * gw;
-          acc_w = last_alpha + (1.0f - last_alpha) * acc_w;
-          dL_dalpha += (1.0f - acc_w) * dL_dsum_w;
-        }
-        dL_dalpha *= T;
-        last_alpha = h.alpha;
-
-        const float dL_dG = hot.opacity * dL_dalpha;
-        if (h.rho3d <= h.rho2d) {
-          dsx += dL_dG * -h.G * h.sx;
-          dsy += dL_dG * -h.G * h.sy;
-          const float rz  = __builtin_amdgcn_rcpf(h.pz);
-          const float dpx = dsx * rz, dpy = dsy * rz;
-          const float dpz = -(dpx * h.sx + dpy * h.sy);
-          const float dkx = h.ly * dpz - h.lz * dpy, dky = h.lz * dpx - h.lx * dpz, dkz = h.lx * dpy - h.ly * dpx;
-          const float dlx = dpy * h.kz - dpz * h.ky, dly = dpz * h.kx - dpx * h.kz, dlz = dpx * h.ky - dpy * h.kx;
-          g[3] = -dkx, g[4] = -dky, g[5] = -dkz;
-          g[6] = -dlx, g[7] = -dly, g[8] = -dlz;
-          g[9]  = pxf * dkx + pyf * dlx + dL_dz * h.sx;
-          g[10] = pxf * dky + pyf * dly + dL_dz * h.sy;
-          g[11] = pxf * dkz + pyf * dlz + dL_dz;
-        } else {
-          g2x   = dL_dG * (-h.G * 2.0f * h.dx);
-          g2y   = dL_dG * (-h.G * 2.0f * h.dy);
-          g[9]  = dL_dz * h.sx;
-          g[10] = dL_dz * h.sy;
-          g[11] = dL_dz;
-          filtered = true;
-        }
-        g[15] = h.G * dL_dalpha;
-      }
+      if (hit) pair_gradients(hot, cold, j, pos, h, g, g2x, g2y, filtered);
       const float tot = wave_sum16_transposed(g);
       if (lane < 16) s_part[wave][j][lane] = tot;  // a wavefront meets an entry once per batch: a plain store
       if (__ballot(filtered) != 0ull) {
@@ -263,6 +279,99 @@ blend_backward_kernel(
         if (lane == 63) s_part[wave][j][16] = sx, s_part[wave][j][17] = sy;
       }
      };
+     if (kBwdRows) {
+      // ---- two phases per staged batch ----------------------------------------------------------------------------
+      // A surfel that reaches an 8x8 quadrant blends into a quarter of its pixels on average, so a pass of the whole
+      // wavefront over one entry leaves most lanes idle in the expensive part (gradients + reduction). Phase 1 walks
+      // the wavefront's list as before but only runs the intersection, and notes for each 4x4 block (= DPP row) which
+      // entries blend into it (four 64-bit masks, scalar registers). Phase 2 lets every row walk ITS list: in one pass
+      // the four rows evaluate four different entries, recompute the intersection (cheaper than parking it), form the
+      // gradients, sum them over the row's 16 pixels with the row part of the transposed butterfly, and add the 16
+      // totals to the entry's row of the batch accumulator in LDS (rows of one wavefront can meet the same entry, in
+      // the same or in different passes, hence an LDS add and not a store). A pixel still meets its entries back to
+      // front, so the recurrences are untouched.
+      if (todo == 0ull) continue;
+      unsigned long long rows_hit[4] = {0ull, 0ull, 0ull, 0ull};
+      auto test_entry = [&](const SplatHot& hot, int j) {
+        const int pos = n_todo - 1 - (b * kBwdBatch + j);
+        Hit h;
+        const bool hit = intersect_flat(hot, pxf, pyf, near_n, h) && (pos < last_contrib);
+        const unsigned long long who = __ballot(hit);
+        const unsigned long long bit = 1ull << j;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if ((who >> (16 * r)) & 0xffffull) rows_hit[r] |= bit;
+      };
+      {
+        auto pop = [&]() {
+          const int j = __builtin_ctzll(todo);
+          todo &= todo - 1;
+          return j;
+        };
+        auto peek = [&]() { return todo ? __builtin_ctzll(todo) : 0; };
+        SplatHot hot_a = s_hot[peek()], hot_b;
+        while (todo) {
+          {
+            const int j = pop();
+            hot_b       = s_hot[peek()];
+            __builtin_amdgcn_sched_barrier(0);
+            test_entry(hot_a, j);
+          }
+          if (todo == 0ull) break;
+          {
+            const int j = pop();
+            hot_a       = s_hot[peek()];
+            __builtin_amdgcn_sched_barrier(0);
+            test_entry(hot_b, j);
+          }
+        }
+      }
+      const int row = lane >> 4;
+      unsigned long long mine = row == 0 ? rows_hit[0] : row == 1 ? rows_hit[1] : row == 2 ? rows_hit[2] : rows_hit[3];
+      auto row_entry = [&](const SplatHot& hot, const SplatCold& cold, int j, bool active) {
+        const int pos = n_todo - 1 - (b * kBwdBatch + j);
+        Hit h;
+        const bool hit = intersect_flat(hot, pxf, pyf, near_n, h) && (pos < last_contrib) && active;
+        float g[16], g2x = 0.0f, g2y = 0.0f;
+        bool filtered = false;
+#pragma unroll
+        for (int c = 0; c < 16; ++c) g[c] = 0.0f;
+        if (hit) pair_gradients(hot, cold, j, pos, h, g, g2x, g2y, filtered);
+        const float tot = row_sum16_transposed(g);  // lane (row, c): the row's total of component c
+        if (active) atomicAdd(&s_part[wave][j][lane & 15], tot);
+        if (__ballot(filtered) != 0ull) {
+          float sx = g2x, sy = g2y;  // totals of the row end up in its lane 15
+          sx += dpp_shift_zero<0x111, 0xf, 0xf>(sx), sy += dpp_shift_zero<0x111, 0xf, 0xf>(sy);
+          sx += dpp_shift_zero<0x112, 0xf, 0xf>(sx), sy += dpp_shift_zero<0x112, 0xf, 0xf>(sy);
+          sx += dpp_shift_zero<0x114, 0xf, 0xf>(sx), sy += dpp_shift_zero<0x114, 0xf, 0xf>(sy);
+          sx += dpp_shift_zero<0x118, 0xf, 0xf>(sx), sy += dpp_shift_zero<0x118, 0xf, 0xf>(sy);
+          if (active && (lane & 15) == 15) atomicAdd(&s_part[wave][j][16], sx), atomicAdd(&s_part[wave][j][17], sy);
+        }
+      };
+      // the next entry's records are requested before the current one is evaluated (alternating registers)
+      auto front = [&]() { return mine ? (int) __builtin_ctzll(mine) : 0; };
+      int j_a = front(), j_b = 0;
+      SplatHot hot_a = s_hot[j_a], hot_b;
+      SplatCold cold_a = s_cold[j_a], cold_b;
+      while (__ballot(mine != 0ull) != 0ull) {
+        {
+          const bool active = mine != 0ull;
+          mine &= mine - 1;
+          j_b = front(), hot_b = s_hot[j_b], cold_b = s_cold[j_b];
+          __builtin_amdgcn_sched_barrier(0);
+          row_entry(hot_a, cold_a, j_a, active);
+        }
+        if (__ballot(mine != 0ull) == 0ull) break;
+        {
+          const bool active = mine != 0ull;
+          mine &= mine - 1;
+          j_a = front(), hot_a = s_hot[j_a], cold_a = s_cold[j_a];
+          __builtin_amdgcn_sched_barrier(0);
+          row_entry(hot_b, cold_b, j_b, active);
+        }
+      }
+      continue;
+     }
      // The record of the next entry is requested before the current one is evaluated (alternating registers): a
      // wavefront walks its list alone, so an exposed LDS round trip per entry sits on the tile's critical path.
      if (todo == 0ull) continue;
