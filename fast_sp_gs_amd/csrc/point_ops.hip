@@ -293,7 +293,7 @@ __global__ void __launch_bounds__(256) knn_topk_kernel(int N, int M, int D, int 
         bd[k] = __builtin_amdgcn_fmed3f(bd[k - 1], cd, bd[k]);
         bi[k] = lt[k - 1] ? bi[k - 1] : (lt[k] ? ci : bi[k]);
       }
-      bd[0] = fminf(bd[0], cd);
+      bd[0] = lt[0] ? cd : bd[0];  // a select on the comparison already made (fminf adds two canonicalising moves)
       bi[0] = lt[0] ? ci : bi[0];
     }
   };
