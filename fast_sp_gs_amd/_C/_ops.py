@@ -474,9 +474,11 @@ def gs_2d_fast_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: boo
                                   Tw2v: Tensor, Tv2c: Tensor, Tv2s: Tensor, cam_pos: Tensor,
                                   trans_precomp: Optional[Tensor] = None, means2D: Optional[Tensor] = None,
                                   culling: Optional[Tensor] = None, debug: bool = False,
-                                  return_keys: bool = False) -> List[Tensor]:
+                                  return_keys: bool = False, return_offsets: bool = False) -> List[Tensor]:
     """gs_2d_fast_preprocess.cu:611-782 -> [means2D, colors, trans_mat, inverse_m, normal_opacity, depths, radii,
-    ranges[T,2] int64, point_list[R] int32] (point_list keeps the -1 padding entries of culled tiles at its tail)."""
+    ranges[T,2] int64, point_list[R] int32] (point_list keeps the -1 padding entries of culled tiles at its tail)
+    (+ sorted keys and tiles_touched, + the prefix scan of tiles_touched, which GS_2D_fast_render_backward can use to sum
+    gradients without atomics)."""
     what = 'gs_2d_fast_preprocess_forward'
     _f32(what, means3D=means3D, scales=scales, rotations=rotations, opacities=opacities, shs=shs, Tw2v=Tw2v,
          Tv2c=Tv2c, Tv2s=Tv2s, cam_pos=cam_pos)
@@ -557,7 +559,11 @@ def gs_2d_fast_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: boo
     if debug:
         torch.cuda.synchronize()
     out = [means2D_, colors, trans_mat, inverse_m, normal_opacity, depths, radii, ranges, point_list]
-    return out + [keys, tiles_touched] if return_keys else out
+    if return_keys:
+        out += [keys, tiles_touched]
+    if return_offsets:
+        out.append(offsets)
+    return out
 
 
 def gs_2d_fast_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs, sh_rest,
@@ -708,21 +714,27 @@ def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inver
                                out_others, out_flows, dL_dout_color, dL_dout_opacity, dL_dothers, dL_dout_flow,
                                ranges, point_list, n_contrib, near_n: float, far_n: float,
                                per_tile_bucket_offset=None, bucket_to_tile=None, max_contrib=None, sampled_T=None,
-                               sampled_acc=None, sampled_aux=None):
+                               sampled_acc=None, sampled_aux=None, point_offsets: Optional[Tensor] = None,
+                               radii: Optional[Tensor] = None):
     """gs_2d_fast_redner.cu:955-1074 -> [dL_dcolors[P,3], dL_dmeans2D[P,2], dL_dtrans_m[P,3,3], dL_dinverse_m[P,3,3],
     dL_dnorm_op[P,4]]. Passing per_tile_bucket_offset selects the per-splat channel set of the reference's second
     kernel; the snapshot tensors themselves are not needed to evaluate it here. With dL_dout_flow (and trans_mat2,
-    out_flows) the optical-flow gradient is added as the reference's kernels add it."""
+    out_flows) the optical-flow gradient is added as the reference's kernels add it. With `point_offsets`
+    (gs_2d_fast_preprocess_forward(..., return_offsets=True)) and `radii` the per-surfel sums are taken in a fixed order
+    from per-instance records instead of with atomics."""
     what = 'GS_2D_fast_render_backward'
     L.require_cuda(what, dL_dout_color=dL_dout_color, dL_dout_opacity=dL_dout_opacity, dL_dothers=dL_dothers)
     P = means2D.shape[0]
     H, W = dL_dout_color.shape[1], dL_dout_color.shape[2]
     opt = dict(dtype=torch.float32, device=out_opacity.device)
-    g_means2D = torch.zeros((P, 2), **opt)
-    g_norm_op = torch.zeros((P, 4), **opt)
-    g_colors = torch.zeros((P, 3), **opt)
-    g_trans = torch.zeros((P, 3, 3), **opt)
-    g_inv = torch.zeros((P, 3, 3), **opt)
+    ordered, ws, R = _ordered_sum_inputs(what, P, point_list, point_offsets, radii,
+                                         'fsgs_gs_2d_fast_render_backward_workspace_bytes', out_opacity.device)
+    new = torch.empty if ordered else torch.zeros  # the ordered path assigns every row, the atomic path accumulates
+    g_means2D = new((P, 2), **opt)
+    g_norm_op = new((P, 4), **opt)
+    g_colors = new((P, 3), **opt)
+    g_trans = new((P, 3, 3), **opt)
+    g_inv = new((P, 3, 3), **opt)
     if P == 0:
         return [g_colors, g_means2D, g_trans, g_inv, g_norm_op]
     c = lambda t: None if t is None else t.contiguous()
@@ -747,7 +759,8 @@ def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inver
             L.ptr(out_others) if use_aux else None, L.ptr(out_flows) if flow else None, L.ptr(dL_dout_color),
             L.ptr(dL_dout_opacity), L.ptr(dL_dothers) if use_aux else None, L.ptr(dL_dout_flow) if flow else None,
             L.ptr(ranges), L.ptr(point_list), L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans),
-            L.ptr(g_inv), L.ptr(g_norm_op), L.current_stream())
+            L.ptr(g_inv), L.ptr(g_norm_op), R, L.ptr(point_offsets) if ordered else None,
+            L.ptr(radii) if ordered else None, L.ptr(ws), ws.numel() if ws is not None else 0, L.current_stream())
     L.check(rc, what)
     return [g_colors, g_means2D, g_trans, g_inv, g_norm_op]
 
@@ -1936,8 +1949,11 @@ def gaussian_rasterize_forward(width: int, height: int, means2D: Tensor, conic_o
 def gaussian_rasterize_backward(means2D: Tensor, conic_opacity: Tensor, colors: Tensor, extras: Optional[Tensor],
                                 out_opacity: Tensor, dL_dout_color: Tensor, dL_dout_opacity: Tensor,
                                 dL_dout_extra: Optional[Tensor], ranges: Tensor, point_list: Tensor,
-                                n_contrib: Tensor):
-    """gaussian_render.cu:486-536 -> (dL_dcolors[P,3], dL_dextras[P,E]|None, dL_dmeans2D[P,2], dL_dconic_opacity[P,4])."""
+                                n_contrib: Tensor, point_offsets: Optional[Tensor] = None,
+                                radii: Optional[Tensor] = None):
+    """gaussian_render.cu:486-536 -> (dL_dcolors[P,3], dL_dextras[P,E]|None, dL_dmeans2D[P,2], dL_dconic_opacity[P,4]).
+    With `point_offsets` (GS_prepare(..., return_offsets=True)) and `radii` the per-Gaussian sums are taken in a fixed
+    order from per-instance records instead of with atomics."""
     what = 'gaussian_rasterize_backward'
     L.require_cuda(what, dL_dout_color=dL_dout_color, dL_dout_opacity=dL_dout_opacity, dL_dout_extra=dL_dout_extra)
     P = means2D.shape[0]
@@ -1946,7 +1962,11 @@ def gaussian_rasterize_backward(means2D: Tensor, conic_opacity: Tensor, colors: 
     if E > 4:
         raise RuntimeError('Only support NUM_EXTRA=0,1,2,3,4')
     opt = dict(dtype=torch.float32, device=out_opacity.device)
-    grads = torch.zeros((P, 9 + E), **opt)  # one zero fill: means2D 2 | conic_opacity 4 | colours 3 | extras E
+    ordered, ws, R = _ordered_sum_inputs(what, P, point_list, point_offsets, radii,
+                                         'fsgs_gaussian_rasterize_backward_workspace_bytes', out_opacity.device)
+    # means2D 2 | conic_opacity 4 | colours 3 | extras E in one allocation: zero-filled for the atomic path, written row
+    # by row by the ordered path
+    grads = (torch.empty if ordered else torch.zeros)((P, 9 + E), **opt)
     g_flat = grads.view(-1)
     dL_dmeans2D = g_flat[:2 * P].view(P, 2)
     dL_dconic_o = g_flat[2 * P:6 * P].view(P, 4)
@@ -1960,9 +1980,25 @@ def gaussian_rasterize_backward(means2D: Tensor, conic_opacity: Tensor, colors: 
     with _timed('gaussian_rasterize_backward'):
         rc = _lib().fsgs_gaussian_rasterize_backward(
             P, W, H, E, *[L.ptr(a) for a in args], L.ptr(dL_dmeans2D), L.ptr(dL_dconic_o), L.ptr(dL_dcolors),
-            L.ptr(dL_dextras), L.current_stream())
+            L.ptr(dL_dextras), R, L.ptr(point_offsets) if ordered else None, L.ptr(radii) if ordered else None,
+            L.ptr(ws), ws.numel() if ws is not None else 0, L.current_stream())
     L.check(rc, what)
     return dL_dcolors, dL_dextras, dL_dmeans2D, dL_dconic_o
+
+
+def _ordered_sum_inputs(what, P, point_list, point_offsets, radii, workspace_bytes_fn, device):
+    """Checks the optional inputs of a backward's ordered-sum path and allocates its workspace:
+    -> (ordered, workspace | None, instance count R)."""
+    R = int(point_list.numel())
+    ordered = point_offsets is not None and P > 0
+    if not ordered:
+        return False, None, R
+    if radii is None:
+        raise RuntimeError(f'{what}: radii is required together with point_offsets')
+    L.require_cuda(what, point_offsets=point_offsets, radii=radii)
+    L.require_dtype(what, 'point_offsets', point_offsets, torch.int64)
+    L.require_dtype(what, 'radii', radii, torch.int32)
+    return True, _workspace(getattr(_lib(), workspace_bytes_fn)(R), device), R
 
 
 def gaussian_rasterize_fast_backward(means2D: Tensor, conic_opacity: Tensor, colors: Tensor, extras: Optional[Tensor],
@@ -1970,10 +2006,12 @@ def gaussian_rasterize_fast_backward(means2D: Tensor, conic_opacity: Tensor, col
                                      dL_dout_color: Tensor, dL_dout_opacity: Tensor, dL_dout_extra: Optional[Tensor],
                                      ranges: Tensor, point_list: Tensor, n_contrib: Tensor, max_contrib: Tensor,
                                      per_tile_bucket_offset: Tensor, bucket_to_tile: Tensor, sampled_T: Tensor,
-                                     sampled_ar: Tensor):
+                                     sampled_ar: Tensor, point_offsets: Optional[Tensor] = None,
+                                     radii: Optional[Tensor] = None):
     """gaussian_render.cu:760-812 -> (dL_dcolors[P,3], dL_dextras[P,E]|None, dL_dmeans2D[P,2], dL_dconic_opacity[P,4]):
     the reference's per-Gaussian backward over the forward's bucket snapshots. The same derivative as
-    gaussian_rasterize_backward, evaluated by the same kernel; the snapshot tensors are checked and not read."""
+    gaussian_rasterize_backward, evaluated by the same kernel; the snapshot tensors are checked and not read.
+    `point_offsets` / `radii` as for gaussian_rasterize_backward."""
     what = 'gaussian_rasterize_fast_backward'
     L.require_cuda(what, images=images, max_contrib=max_contrib, per_tile_bucket_offset=per_tile_bucket_offset,
                    bucket_to_tile=bucket_to_tile, sampled_T=sampled_T, sampled_ar=sampled_ar)
@@ -1991,7 +2029,9 @@ def gaussian_rasterize_fast_backward(means2D: Tensor, conic_opacity: Tensor, col
     if tuple(sampled_T.shape) != (B, _TILE * _TILE) or tuple(sampled_ar.shape)[0] != B:
         raise RuntimeError(f'{what}: the snapshot tensors do not match bucket_to_tile')
     opt = dict(dtype=torch.float32, device=out_opacity.device)
-    grads = torch.zeros((P, 9 + E), **opt)  # one zero fill: means2D 2 | conic_opacity 4 | colours 3 | extras E
+    ordered, ws, R = _ordered_sum_inputs(what, P, point_list, point_offsets, radii,
+                                         'fsgs_gaussian_rasterize_backward_workspace_bytes', out_opacity.device)
+    grads = (torch.empty if ordered else torch.zeros)((P, 9 + E), **opt)  # means2D 2 | conic_opacity 4 | colours 3 | extras E
     g_flat = grads.view(-1)
     dL_dmeans2D = g_flat[:2 * P].view(P, 2)
     dL_dconic_o = g_flat[2 * P:6 * P].view(P, 4)
@@ -2007,6 +2047,7 @@ def gaussian_rasterize_fast_backward(means2D: Tensor, conic_opacity: Tensor, col
     with _timed('gaussian_rasterize_backward'):
         rc = _lib().fsgs_gaussian_rasterize_fast_backward(
             P, W, H, E, *[L.ptr(a) for a in args], L.ptr(dL_dmeans2D), L.ptr(dL_dconic_o), L.ptr(dL_dcolors),
-            L.ptr(dL_dextras), L.current_stream())
+            L.ptr(dL_dextras), R, L.ptr(point_offsets) if ordered else None, L.ptr(radii) if ordered else None,
+            L.ptr(ws), ws.numel() if ws is not None else 0, L.current_stream())
     L.check(rc, what)
     return dL_dcolors, dL_dextras, dL_dmeans2D, dL_dconic_o

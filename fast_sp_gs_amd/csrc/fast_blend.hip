@@ -18,6 +18,7 @@
 // a time in LDS (64-byte hot record with the adjugate, 32-byte cold record), per-quadrant work lists from a
 // conservative bound, gradients reduced over the wavefront in registers before one LDS atomic per component.
 #include "blend.hpp"
+#include "ordered_sums.hpp"
 
 namespace fsgs {
 namespace {
@@ -308,9 +309,26 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
 
 // Per-surfel gradient slots: 0-2 colours | 3-11 adjugate | 12-14 normal | 15 opacity | 16-18 transform row 2 |
 // 19-20 means2D.
-constexpr int kFastGradSlots = 21;
+constexpr int kFastGradSlots  = 21;
+constexpr int kFastRecordSlots = 22;  // a record of the ordered-sum path: the 21 slots + one float of padding
 
-template <bool kAux, bool kPerSplat, bool kFlow>
+// Where slot_sum_kernel puts component c of surfel i: 0-2 colours | 3-11 inverse transform | 12-15 normal, opacity |
+// 16-18 third row of the transform (the other two rows get no gradient from the blend: zeros) | 19-20 means2D.
+struct FastScatter {
+  float *g_means2D, *g_normal_opacity, *g_colors, *g_trans, *g_inv;
+  __device__ __forceinline__ void operator()(int i, int c, float v) const {
+    if (c < 3) g_colors[3 * (size_t) i + c] = v;
+    else if (c < 12) g_inv[9 * (size_t) i + (c - 3)] = v;
+    else if (c < 16) g_normal_opacity[4 * (size_t) i + (c - 12)] = v;
+    else if (c < 19) {
+      g_trans[9 * (size_t) i + 6 + (c - 16)] = v;
+      g_trans[9 * (size_t) i + 2 * (c - 16)] = 0.0f, g_trans[9 * (size_t) i + 2 * (c - 16) + 1] = 0.0f;
+    } else if (c < 21) g_means2D[2 * (size_t) i + (c - 19)] = v;
+  }
+};
+
+// kSlots: the per-surfel sums go through per-instance records (ordered_sums.hpp) instead of device-scope atomics.
+template <bool kAux, bool kPerSplat, bool kFlow, bool kSlots>
 __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
     int ordered, const int* __restrict__ tile_order, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const int32_t* __restrict__ n_contrib, const float2* __restrict__ means2D,
@@ -320,7 +338,8 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
     const float* __restrict__ dL_dpix, const float* __restrict__ dL_dextras, const float* __restrict__ dL_dopacity,
     const float2* __restrict__ dL_dflow,
     float* __restrict__ g_means2D, float* __restrict__ g_normal_opacity, float* __restrict__ g_colors,
-    float* __restrict__ g_trans, float* __restrict__ g_inv) {
+    float* __restrict__ g_trans, float* __restrict__ g_inv, const int64_t* __restrict__ point_offsets,
+    const int32_t* __restrict__ radii, float* __restrict__ slot_records, unsigned char* __restrict__ slot_written) {
   constexpr int kB = 64;  // surfels staged per round
   __shared__ FastHot s_hot[kB];
   __shared__ SplatCold s_cold[kB];
@@ -331,7 +350,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
   __shared__ int s_max_contrib;
   __shared__ unsigned char s_mask[kB];
 
-  const int gx = (W + kTile - 1) / kTile;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int tile = scheduled_tile(ordered, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
@@ -396,14 +415,19 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
 
   FastSplat next;
   float next_t2[9];
-  if ((int) threadIdx.x < min(n_todo, kB)) {
-    const int id = point_list[r0 + (n_todo - 1 - (int) threadIdx.x)];
+  int next_radius = 0;
+  int64_t next_off = 0;
+  size_t slot = 0;  // record position of the entry this lane staged (the same lane flushes it)
+  auto gather = [&](int at) {
+    const int id = point_list[r0 + at];
     next = gather_fast(id, means2D, colors, normal_opacity, trans_mat, inverse_m);
     if (kFlow) {
 #pragma unroll
       for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) id + k];
     }
-  }
+    if (kSlots) next_radius = radii[id], next_off = id == 0 ? 0 : point_offsets[id - 1];
+  };
+  if ((int) threadIdx.x < min(n_todo, kB)) gather(n_todo - 1 - (int) threadIdx.x);
 
   for (int b = 0; b < rounds; ++b) {
     const int n_here = min(kB, n_todo - b * kB);
@@ -415,17 +439,17 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
 #pragma unroll
         for (int k = 0; k < 9; ++k) s_t2[threadIdx.x * 9 + k] = next_t2[k];
       }
+      if (kSlots) {
+        // The fused binning reserves one key position per tile of the surfel's rectangle, from its prefix-scan offset
+        // on (the tiles that pass its corner test are packed to the front of that span, the rest is padding). Any
+        // position of the span that no other tile of the surfel uses will do for the record: x-major over the rectangle.
+        const TileRect r = tile_rect(next.hot.cx, next.hot.cy, next_radius, gx, gy);
+        slot = (size_t) (next_off + (int64_t) (tile_x - r.x0) * (r.y1 - r.y0) + (tile_y - r.y0));
+      }
     }
     __syncthreads();
     const int nxt = (b + 1) * kB + (int) threadIdx.x;
-    if ((int) threadIdx.x < kB && nxt < n_todo) {
-      const int id = point_list[r0 + (n_todo - 1 - nxt)];
-      next = gather_fast(id, means2D, colors, normal_opacity, trans_mat, inverse_m);
-      if (kFlow) {
-#pragma unroll
-        for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) id + k];
-      }
-    }
+    if ((int) threadIdx.x < kB && nxt < n_todo) gather(n_todo - 1 - nxt);
 
     for (int chunk = 0; chunk < kB / kWave; ++chunk) {
       const int jj = chunk * kWave + lane;
@@ -535,21 +559,34 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
         for (int w = 0; w < 4; ++w) sum += s_part[w][threadIdx.x][c], s_part[w][threadIdx.x][c] = 0.0f;
         a[c] = sum;
       }
+      if (kSlots) {
+        bool any = false;
 #pragma unroll
-      for (int c = 0; c < 3; ++c)
-        if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
+        for (int c = 0; c < kFastGradSlots; ++c) any |= a[c] != 0.0f;
+        if (any) {
+          float2* dst = (float2*) (slot_records + slot * kFastRecordSlots);
 #pragma unroll
-      for (int c = 0; c < 9; ++c)
-        if (a[3 + c] != 0.0f) atomicAdd(&g_inv[9 * (size_t) id + c], a[3 + c]);
+          for (int c = 0; c < kFastRecordSlots / 2; ++c)
+            dst[c] = make_float2(a[2 * c], 2 * c + 1 < kFastGradSlots ? a[2 * c + 1] : 0.0f);
+          slot_written[slot] = 1;
+        }
+      } else {
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        if (a[12 + c] != 0.0f) atomicAdd(&g_normal_opacity[4 * (size_t) id + c], a[12 + c]);
+        for (int c = 0; c < 3; ++c)
+          if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
 #pragma unroll
-      for (int c = 0; c < 3; ++c)
-        if (a[16 + c] != 0.0f) atomicAdd(&g_trans[9 * (size_t) id + 6 + c], a[16 + c]);
+        for (int c = 0; c < 9; ++c)
+          if (a[3 + c] != 0.0f) atomicAdd(&g_inv[9 * (size_t) id + c], a[3 + c]);
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
-        if (a[19 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[19 + c]);
+        for (int c = 0; c < 4; ++c)
+          if (a[12 + c] != 0.0f) atomicAdd(&g_normal_opacity[4 * (size_t) id + c], a[12 + c]);
+#pragma unroll
+        for (int c = 0; c < 3; ++c)
+          if (a[16 + c] != 0.0f) atomicAdd(&g_trans[9 * (size_t) id + 6 + c], a[16 + c]);
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+          if (a[19 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[19 + c]);
+      }
     }
   }
 }
@@ -601,12 +638,17 @@ FSGS_API int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, 
   return check_launch("GS_2D_fast_render_forward");
 }
 
+FSGS_API size_t fsgs_gs_2d_fast_render_backward_workspace_bytes(int64_t R) {
+  return slot_workspace_bytes(R, kFastRecordSlots);
+}
+
 FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n, double far_n, int per_splat_form,
     const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,
     const float* inverse_m, const float* trans_mat_t2, const float* out_opacity, const float* out_extras,
     const float* out_flow, const float* dL_dpix, const float* dL_dopacity, const float* dL_dextras,
     const float* dL_dflow, const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib,
-    float* g_colors, float* g_means2D, float* g_trans, float* g_inv, float* g_normal_opacity, void* stream) {
+    float* g_colors, float* g_means2D, float* g_trans, float* g_inv, float* g_normal_opacity, int64_t R,
+    const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_fast_render_backward: bad sizes");
   if (P == 0) return kOk;
   FSGS_REQUIRE(means2D && normal_opacity && colors && trans_mat && inverse_m && out_opacity && dL_dpix && dL_dopacity &&
@@ -616,17 +658,32 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
   const bool flow = dL_dflow != nullptr;
   FSGS_REQUIRE(!flow || (aux && trans_mat_t2 && out_flow),
                "GS_2D_fast_render_backward: flow gradients need trans_mat2, out_flows and the auxiliary maps");
+  const bool slots = point_offsets != nullptr;
+  SlotWorkspace ws{nullptr, nullptr};
+  if (slots) {
+    FSGS_REQUIRE(radii && workspace && R >= 0 && R < (int64_t) 0x7fffffff,
+                 "GS_2D_fast_render_backward: the ordered-sum path needs radii, a workspace and the instance count R");
+    if (workspace_bytes < slot_workspace_bytes(R, kFastRecordSlots))
+      return fail(kWorkspaceSmall, "GS_2D_fast_render_backward: workspace %zu < %zu bytes", workspace_bytes,
+                  slot_workspace_bytes(R, kFastRecordSlots));
+    FSGS_REQUIRE(((uintptr_t) workspace & 15) == 0, "GS_2D_fast_render_backward: workspace must be 16-byte aligned");
+    ws = slot_workspace(workspace, R, kFastRecordSlots);
+  }
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
+  if (slots) launch_slot_clear(ws, R, s);
   const int* tile_order = nullptr;
   const int ordered = launch_tile_order(gx, gy, ranges, s, &tile_order);
-#define FSGS_LAUNCH_BWD(AUX, SPLAT, FLOW)                                                                            \
-  hipLaunchKernelGGL((fast_blend_backward_kernel<AUX, SPLAT, FLOW>), grid, block, 0, s, ordered, tile_order, W, H,               \
+#define FSGS_LAUNCH_BWD_S(AUX, SPLAT, FLOW, SL)                                                                      \
+  hipLaunchKernelGGL((fast_blend_backward_kernel<AUX, SPLAT, FLOW, SL>), grid, block, 0, s, ordered, tile_order, W, H, \
                      (float) near_n, (float) far_n, ranges, point_list, n_contrib, (const float2*) means2D,          \
                      (const float4*) normal_opacity, colors, trans_mat, inverse_m, trans_mat_t2, out_opacity,        \
                      out_extras, (const float2*) out_flow, dL_dpix, dL_dextras, dL_dopacity,                         \
-                     (const float2*) dL_dflow, g_means2D, g_normal_opacity, g_colors, g_trans, g_inv)
+                     (const float2*) dL_dflow, g_means2D, g_normal_opacity, g_colors, g_trans, g_inv, point_offsets, \
+                     radii, ws.records, ws.written)
+#define FSGS_LAUNCH_BWD(AUX, SPLAT, FLOW) \
+  do { if (slots) FSGS_LAUNCH_BWD_S(AUX, SPLAT, FLOW, true); else FSGS_LAUNCH_BWD_S(AUX, SPLAT, FLOW, false); } while (0)
   if (aux && per_splat_form && flow) FSGS_LAUNCH_BWD(true, true, true);
   else if (aux && flow) FSGS_LAUNCH_BWD(true, false, true);
   else if (aux && per_splat_form) FSGS_LAUNCH_BWD(true, true, false);
@@ -634,5 +691,9 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
   else if (per_splat_form) FSGS_LAUNCH_BWD(false, true, false);
   else FSGS_LAUNCH_BWD(false, false, false);
 #undef FSGS_LAUNCH_BWD
+#undef FSGS_LAUNCH_BWD_S
+  if (slots)
+    launch_slot_sum<kFastRecordSlots>(P, point_offsets, ws,
+                                      FastScatter{g_means2D, g_normal_opacity, g_colors, g_trans, g_inv}, s);
   return check_launch("GS_2D_fast_render_backward");
 }

@@ -16,6 +16,7 @@
 // its own LDS row (LDS float atomics cost about three cycles per lane here), adds the four rows in wavefront order and
 // flushes one global atomic per Gaussian, component and tile.
 #include "blend.hpp"
+#include "ordered_sums.hpp"
 
 namespace fsgs {
 namespace {
@@ -327,20 +328,37 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_topk_kernel(int flags, con
 }
 
 // gradient slots of one Gaussian: 0-2 colour | 3-6 extras | 7-8 mean2D | 9-11 conic | 12 opacity | 13-15 unused
+constexpr int kG3Slots = 16;
+
+// Where slot_sum_kernel puts component c of Gaussian i.
 template <int E>
+struct G3Scatter {
+  float *g_means2D, *g_conic_opacity, *g_colors, *g_extras;
+  __device__ __forceinline__ void operator()(int i, int c, float v) const {
+    if (c < 3) g_colors[3 * (size_t) i + c] = v;
+    else if (c < 7) {
+      if (c - 3 < E) g_extras[(size_t) E * i + (c - 3)] = v;
+    } else if (c < 9) g_means2D[2 * (size_t) i + (c - 7)] = v;
+    else if (c < 13) g_conic_opacity[4 * (size_t) i + (c - 9)] = v;
+  }
+};
+
+// kSlots: the per-Gaussian sums go through per-instance records (ordered_sums.hpp) instead of device-scope atomics.
+template <int E, bool kSlots>
 __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags, const int* __restrict__ tile_order, int W, int H,
     const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
     const float4* __restrict__ conic_opacity, const float* __restrict__ colors, const float* __restrict__ extras,
     const float* __restrict__ out_opacity, const int32_t* __restrict__ n_contrib, const float* __restrict__ dL_dpix,
     const float* __restrict__ dL_dout_extras, const float* __restrict__ dL_dout_opacity,
     float* __restrict__ g_means2D, float* __restrict__ g_conic_opacity, float* __restrict__ g_colors,
-    float* __restrict__ g_extras) {
+    float* __restrict__ g_extras, const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii,
+    float* __restrict__ slot_records, unsigned char* __restrict__ slot_written) {
   constexpr int kB = 64;
   __shared__ G3Hot s_hot[kB];
   __shared__ float s_feat[kB][3 + kMaxExtra + 1];
   __shared__ float s_part[4][kB][17];  // each wavefront's sums per staged Gaussian: plain stores, added in wavefront order
   __shared__ int s_max_contrib;
-  const int gx = (W + kTile - 1) / kTile;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int tile = scheduled_tile(flags, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
   lane_pixel(tile_x, tile_y, px, py);
@@ -373,8 +391,14 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
   }
 
   G3Entry next;
-  if ((int) threadIdx.x < min(n_todo, kB))
-    next = gather_gaussian<E>(point_list[r0 + (n_todo - 1 - (int) threadIdx.x)], means2D, conic_opacity, colors, extras);
+  int next_radius = 0;
+  int64_t next_off = 0;
+  size_t slot = 0;  // record position of the entry this lane staged (the same lane flushes it)
+  auto gather = [&](int at) {
+    next = gather_gaussian<E>(point_list[r0 + at], means2D, conic_opacity, colors, extras);
+    if (kSlots) next_radius = radii[next.hot.id], next_off = next.hot.id == 0 ? 0 : point_offsets[next.hot.id - 1];
+  };
+  if ((int) threadIdx.x < min(n_todo, kB)) gather(n_todo - 1 - (int) threadIdx.x);
   for (int b = 0; b < rounds; ++b) {
     const int n_here = min(kB, n_todo - b * kB);
     if ((int) threadIdx.x < n_here) {
@@ -382,11 +406,15 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
       s_hot[threadIdx.x] = next.hot;
 #pragma unroll
       for (int k = 0; k < 3 + E; ++k) s_feat[threadIdx.x][k] = next.feat[k];
+      if (kSlots) {
+        // the binning emits a Gaussian's tiles row-major over its rectangle, from its prefix-scan offset on
+        const TileRect r = tile_rect(next.hot.x, next.hot.y, next_radius, gx, gy);
+        slot = (size_t) (next_off + (int64_t) (tile_y - r.y0) * (r.x1 - r.x0) + (tile_x - r.x0));
+      }
     }
     __syncthreads();
     const int nxt = (b + 1) * kB + (int) threadIdx.x;
-    if ((int) threadIdx.x < kB && nxt < n_todo)
-      next = gather_gaussian<E>(point_list[r0 + (n_todo - 1 - nxt)], means2D, conic_opacity, colors, extras);
+    if ((int) threadIdx.x < kB && nxt < n_todo) gather(n_todo - 1 - nxt);
 
     unsigned long long todo = __ballot(lane < n_here && ((s_hot[lane].mask >> wave) & 1u) &&
                                        (n_todo - 1 - (b * kB + lane)) < wave_max);
@@ -434,19 +462,31 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
         for (int w = 0; w < 4; ++w) sum += s_part[w][threadIdx.x][c], s_part[w][threadIdx.x][c] = 0.0f;
         a[c] = sum;
       }
-      const int id = s_hot[threadIdx.x].id;
+      if (kSlots) {
+        bool any = false;
 #pragma unroll
-      for (int c = 0; c < 3; ++c)
-        if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
+        for (int c = 0; c < kG3Slots; ++c) any |= a[c] != 0.0f;
+        if (any) {
+          float4* dst = (float4*) (slot_records + slot * kG3Slots);
 #pragma unroll
-      for (int c = 0; c < E; ++c)
-        if (a[3 + c] != 0.0f) atomicAdd(&g_extras[(size_t) E * id + c], a[3 + c]);
+          for (int c = 0; c < kG3Slots / 4; ++c) dst[c] = make_float4(a[4 * c], a[4 * c + 1], a[4 * c + 2], a[4 * c + 3]);
+          slot_written[slot] = 1;
+        }
+      } else {
+        const int id = s_hot[threadIdx.x].id;
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
-        if (a[7 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[7 + c]);
+        for (int c = 0; c < 3; ++c)
+          if (a[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], a[c]);
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        if (a[9 + c] != 0.0f) atomicAdd(&g_conic_opacity[4 * (size_t) id + c], a[9 + c]);
+        for (int c = 0; c < E; ++c)
+          if (a[3 + c] != 0.0f) atomicAdd(&g_extras[(size_t) E * id + c], a[3 + c]);
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+          if (a[7 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], a[7 + c]);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (a[9 + c] != 0.0f) atomicAdd(&g_conic_opacity[4 * (size_t) id + c], a[9 + c]);
+      }
     }
     // a lane only touches its own rows of s_part and its staged entry between this flush and the barrier that follows
     // the next batch's LDS store
@@ -725,33 +765,61 @@ FSGS_API int fsgs_gaussian_rasterize_forward(int P, int W, int H, int E, const f
   return check_launch("gaussian_rasterize_forward");
 }
 
+FSGS_API size_t fsgs_gaussian_rasterize_backward_workspace_bytes(int64_t R) {
+  return slot_workspace_bytes(R, kG3Slots);
+}
+
 FSGS_API int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const float* means2D,
     const float* conic_opacity, const float* colors, const float* extras, const float* out_opacity,
     const int32_t* n_contrib, const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity,
     const int32_t* point_list, const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors,
-    float* g_extras, void* stream) {
+    float* g_extras, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
+    size_t workspace_bytes, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "gaussian_rasterize_backward: bad sizes");
   FSGS_REQUIRE(E >= 0 && E <= kMaxExtra, "gaussian_rasterize_backward: only 0..%d extra channels are supported", kMaxExtra);
   if (P == 0) return kOk;
   FSGS_REQUIRE(means2D && conic_opacity && colors && out_opacity && n_contrib && dL_dpix && dL_dout_opacity && ranges &&
                    g_means2D && g_conic_opacity && g_colors && (E == 0 || (extras && dL_dout_extras && g_extras)),
                "gaussian_rasterize_backward: null pointer");
+  const bool slots = point_offsets != nullptr;
+  SlotWorkspace ws{nullptr, nullptr};
+  if (slots) {
+    FSGS_REQUIRE(radii && workspace && R >= 0 && R < (int64_t) 0x7fffffff,
+                 "gaussian_rasterize_backward: the ordered-sum path needs radii, a workspace and the instance count R");
+    if (workspace_bytes < slot_workspace_bytes(R, kG3Slots))
+      return fail(kWorkspaceSmall, "gaussian_rasterize_backward: workspace %zu < %zu bytes", workspace_bytes,
+                  slot_workspace_bytes(R, kG3Slots));
+    FSGS_REQUIRE(((uintptr_t) workspace & 15) == 0, "gaussian_rasterize_backward: workspace must be 16-byte aligned");
+    ws = slot_workspace(workspace, R, kG3Slots);
+  }
   hipStream_t s = (hipStream_t) stream;
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  if (slots) launch_slot_clear(ws, R, s);
   const int* tile_order = nullptr;
   const int flags = launch_tile_order(gx, gy, ranges, s, &tile_order);
   const dim3 grid(gx * gy), block(kBlendThreads);
-#define FSGS_G3_BWD(EE)                                                                                             \
-  hipLaunchKernelGGL((gs3d_backward_kernel<EE>), grid, block, 0, s, flags, tile_order, W, H, ranges, point_list,               \
+#define FSGS_G3_BWD(EE, SL)                                                                                         \
+  hipLaunchKernelGGL((gs3d_backward_kernel<EE, SL>), grid, block, 0, s, flags, tile_order, W, H, ranges, point_list, \
                      (const float2*) means2D, (const float4*) conic_opacity, colors, extras, out_opacity, n_contrib, \
-                     dL_dpix, dL_dout_extras, dL_dout_opacity, g_means2D, g_conic_opacity, g_colors, g_extras)
+                     dL_dpix, dL_dout_extras, dL_dout_opacity, g_means2D, g_conic_opacity, g_colors, g_extras,      \
+                     point_offsets, radii, ws.records, ws.written)
+#define FSGS_G3_BWD_E(EE)                                                                                           \
+  do {                                                                                                              \
+    if (slots) {                                                                                                    \
+      FSGS_G3_BWD(EE, true);                                                                                        \
+      launch_slot_sum<kG3Slots>(P, point_offsets, ws, G3Scatter<EE>{g_means2D, g_conic_opacity, g_colors, g_extras}, s); \
+    } else {                                                                                                        \
+      FSGS_G3_BWD(EE, false);                                                                                       \
+    }                                                                                                               \
+  } while (0)
   switch (E) {
-    case 0: FSGS_G3_BWD(0); break;
-    case 1: FSGS_G3_BWD(1); break;
-    case 2: FSGS_G3_BWD(2); break;
-    case 3: FSGS_G3_BWD(3); break;
-    default: FSGS_G3_BWD(4); break;
+    case 0: FSGS_G3_BWD_E(0); break;
+    case 1: FSGS_G3_BWD_E(1); break;
+    case 2: FSGS_G3_BWD_E(2); break;
+    case 3: FSGS_G3_BWD_E(3); break;
+    default: FSGS_G3_BWD_E(4); break;
   }
+#undef FSGS_G3_BWD_E
 #undef FSGS_G3_BWD
   return check_launch("gaussian_rasterize_backward");
 }
@@ -764,14 +832,16 @@ FSGS_API int fsgs_gaussian_rasterize_fast_backward(int P, int W, int H, int E, c
     const float* out_extras, const float* out_opacity, const int32_t* n_contrib, const int32_t* max_contrib,
     const int64_t* bucket_offset, const int32_t* bucket_to_tile, const float* sampled_T, const float* sampled_ar,
     const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
-    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, void* stream) {
+    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, int64_t R,
+    const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes, void* stream) {
   if (P == 0) return kOk;
   FSGS_REQUIRE(images && max_contrib && bucket_offset && bucket_to_tile && sampled_T && sampled_ar &&
                    (E == 0 || out_extras),
                "gaussian_rasterize_fast_backward: null pointer");
   return fsgs_gaussian_rasterize_backward(P, W, H, E, means2D, conic_opacity, colors, extras, out_opacity, n_contrib,
                                           dL_dpix, dL_dout_extras, dL_dout_opacity, point_list, ranges, g_means2D,
-                                          g_conic_opacity, g_colors, g_extras, stream);
+                                          g_conic_opacity, g_colors, g_extras, R, point_offsets, radii, workspace,
+                                          workspace_bytes, stream);
 }
 
 FSGS_API int fsgs_gaussian_topk_weights(int topk, int P, int W, int H, const float* means2D,

@@ -1,0 +1,87 @@
+// Per-surfel sums of per-(surfel, tile) gradient records in a fixed order, without atomics and without a zero fill of
+// the outputs. The tile binning emits a surfel's instances at consecutive positions of the unsorted key list, starting at
+// the surfel's prefix-scan offset; a backward block that has summed one instance over its tile's pixels writes the sums
+// as one record at that position and sets the instance's "written" byte. slot_sum_kernel then adds a surfel's written
+// records in position order and hands every component of every surfel (zeros where nothing was written) to a scatter
+// functor that knows the output tensors. The reference flushes these sums with one device-scope atomic per component,
+// tile and surfel into caller-zeroed tensors (e.g. gaussian_render.cu:560-600, gs_2d_fast_redner.cu:520-560).
+#pragma once
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace fsgs {
+
+struct SlotWorkspace {
+  float* records;          // [R][kFloats]
+  unsigned char* written;  // [R], rounded up to whole float4s
+};
+
+inline size_t slot_written_offset(int64_t R, int floats) {
+  return align_up((size_t) (R > 0 ? R : 0) * floats * 4 + 16, 256);
+}
+inline size_t slot_workspace_bytes(int64_t R, int floats) {
+  return slot_written_offset(R, floats) + align_up((size_t) (R > 0 ? R : 0) + 16, 256);
+}
+inline SlotWorkspace slot_workspace(void* base, int64_t R, int floats) {
+  return SlotWorkspace{(float*) base, (unsigned char*) base + slot_written_offset(R, floats)};
+}
+
+namespace {
+
+__global__ void __launch_bounds__(256) slot_clear_kernel(size_t n4, float4* __restrict__ p) {
+  for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t) gridDim.x * blockDim.x)
+    p[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+}
+
+// kFloats / 2 lanes per surfel, each owning one float2 of the record, so the lanes of a surfel read consecutive bytes
+// and neighbouring surfels continue where the previous one ends. Eight records of a surfel are in flight together; a
+// record's load does not wait for its "written" byte (an unwritten record's bytes are read and dropped).
+template <int kFloats, typename Scatter>
+__global__ void __launch_bounds__(256) slot_sum_kernel(int P, const int64_t* __restrict__ point_offsets,
+    const float* __restrict__ records, const unsigned char* __restrict__ written, Scatter out) {
+  static_assert(kFloats % 2 == 0 && kFloats <= 64, "records are whole float2s");
+  constexpr int kLanes = kFloats / 2, kPerWave = 64 / kLanes, kDepth = 8;
+  const int lane = threadIdx.x & 63;
+  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int sub = lane / kLanes, k = lane - sub * kLanes;
+  const int i = wave * kPerWave + sub;
+  if (sub >= kPerWave || i >= P) return;
+  const int64_t e0 = i > 0 ? point_offsets[i - 1] : 0, e1 = point_offsets[i];
+  const float2* src = (const float2*) records + k;
+  float2 acc = make_float2(0.0f, 0.0f);
+  for (int64_t base = e0; base < e1; base += kDepth) {
+    float2 v[kDepth];
+    unsigned char ok[kDepth];
+#pragma unroll
+    for (int j = 0; j < kDepth; ++j) {
+      const size_t at = (size_t) (base + j < e1 ? base + j : e1 - 1);
+      v[j]  = src[at * kLanes];
+      ok[j] = written[at];
+    }
+#pragma unroll
+    for (int j = 0; j < kDepth; ++j) {
+      const bool on = base + j < e1 && ok[j] != 0;
+      acc.x += on ? v[j].x : 0.0f, acc.y += on ? v[j].y : 0.0f;
+    }
+  }
+  out(i, 2 * k, acc.x);
+  out(i, 2 * k + 1, acc.y);
+}
+
+inline void launch_slot_clear(const SlotWorkspace& ws, int64_t R, hipStream_t s) {
+  const size_t n4 = ((size_t) R + 15) / 16;
+  const unsigned blocks = (unsigned) std::min<size_t>((n4 + 255) / 256, 8192);
+  if (n4 > 0) hipLaunchKernelGGL(slot_clear_kernel, dim3(blocks), dim3(256), 0, s, n4, (float4*) ws.written);
+}
+
+template <int kFloats, typename Scatter>
+inline void launch_slot_sum(int P, const int64_t* point_offsets, const SlotWorkspace& ws, Scatter out, hipStream_t s) {
+  constexpr int kPerWave = 64 / (kFloats / 2);
+  const int64_t waves = div_up(P, kPerWave);
+  hipLaunchKernelGGL((slot_sum_kernel<kFloats, Scatter>), dim3((unsigned) div_up(waves * 64, 256)), dim3(256), 0, s, P,
+                     point_offsets, ws.records, ws.written, out);
+}
+
+}  // namespace
+}  // namespace fsgs

@@ -198,18 +198,20 @@ class _GS_render(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, W, H, mean2D, colors, conic_opacity, tile_range, point_list, extras, accum_max_count,
-                accum_weights_p, accum_weights_count):
+                accum_weights_p, accum_weights_count, point_offsets=None, radii=None):
         images, out_opacity, out_extras, n_contrib = _GS_render._forward(
             W, H, mean2D, conic_opacity, colors, extras, point_list, tile_range, accum_max_count, accum_weights_p,
             accum_weights_count, None)
-        ctx.save_for_backward(mean2D, colors, conic_opacity, extras, tile_range, point_list, out_opacity, n_contrib)
+        ctx.save_for_backward(mean2D, colors, conic_opacity, extras, tile_range, point_list, out_opacity, n_contrib,
+                              point_offsets, radii)
         ctx.mark_non_differentiable(n_contrib)
         return images, out_opacity, out_extras, n_contrib
 
     @staticmethod
     @torch.autograd.function.once_differentiable
     def backward(ctx, grad_images, grad_alpha, grad_out_extra, _):
-        mean2D, colors, conic_opacity, extras, tile_range, point_list, out_opacity, n_contrib = ctx.saved_tensors
+        (mean2D, colors, conic_opacity, extras, tile_range, point_list, out_opacity, n_contrib, point_offsets,
+         radii) = ctx.saved_tensors
         zeros_like = lambda t: torch.zeros_like(t)
         grad_images = zeros_like(out_opacity).expand(3, -1, -1).contiguous() if grad_images is None else grad_images
         grad_alpha = zeros_like(out_opacity) if grad_alpha is None else grad_alpha
@@ -218,8 +220,10 @@ class _GS_render(torch.autograd.Function):
                                          device=out_opacity.device)
         grad_colors, grad_extra, grad_means2D, grad_conic_opacity = _GS_render._backward(
             mean2D, conic_opacity, colors, extras, out_opacity, grad_images.contiguous(), grad_alpha.contiguous(),
-            None if grad_out_extra is None else grad_out_extra.contiguous(), tile_range, point_list, n_contrib)
-        return None, None, grad_means2D, grad_colors, grad_conic_opacity, None, None, grad_extra, None, None, None
+            None if grad_out_extra is None else grad_out_extra.contiguous(), tile_range, point_list, n_contrib,
+            point_offsets, radii)
+        return (None, None, grad_means2D, grad_colors, grad_conic_opacity, None, None, grad_extra, None, None, None,
+                None, None)
 
 
 class _GS_render_fast(torch.autograd.Function):
@@ -230,7 +234,7 @@ class _GS_render_fast(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, W, H, mean2D, colors, conic_opacity, tile_range, point_list, extras, accum_max_count,
-                accum_weights_p, accum_weights_count):
+                accum_weights_p, accum_weights_count, point_offsets=None, radii=None):
         per_tile_bucket_offset = (tile_range[..., 1] - tile_range[..., 0] + 31) // 32
         per_tile_bucket_offset = torch.cumsum(per_tile_bucket_offset, dim=-1).contiguous()
         (images, out_opacity, out_extras, n_contrib, max_contrib, bucket_to_tile, sampled_T,
@@ -239,7 +243,7 @@ class _GS_render_fast(torch.autograd.Function):
                                                 per_tile_bucket_offset)
         ctx.save_for_backward(mean2D, colors, conic_opacity, extras, tile_range, point_list, images, out_opacity,
                               out_extras, n_contrib, per_tile_bucket_offset, max_contrib, bucket_to_tile, sampled_T,
-                              sampled_ar)
+                              sampled_ar, point_offsets, radii)
         ctx.mark_non_differentiable(n_contrib)
         return images, out_opacity, out_extras, n_contrib
 
@@ -247,7 +251,8 @@ class _GS_render_fast(torch.autograd.Function):
     @torch.autograd.function.once_differentiable
     def backward(ctx, grad_images, grad_alpha, grad_out_extra, _):
         (mean2D, colors, conic_opacity, extras, tile_range, point_list, images, out_opacity, out_extras, n_contrib,
-         per_tile_bucket_offset, max_contrib, bucket_to_tile, sampled_T, sampled_ar) = ctx.saved_tensors
+         per_tile_bucket_offset, max_contrib, bucket_to_tile, sampled_T, sampled_ar, point_offsets,
+         radii) = ctx.saved_tensors
         grad_images = torch.zeros_like(images) if grad_images is None else grad_images
         grad_alpha = torch.zeros_like(out_opacity) if grad_alpha is None else grad_alpha
         if extras is not None and grad_out_extra is None:
@@ -255,24 +260,29 @@ class _GS_render_fast(torch.autograd.Function):
         grad_colors, grad_extra, grad_means2D, grad_conic_opacity = _GS_render_fast._backward(
             mean2D, conic_opacity, colors, extras, images, out_extras, out_opacity, grad_images.contiguous(),
             grad_alpha.contiguous(), None if grad_out_extra is None else grad_out_extra.contiguous(), tile_range,
-            point_list, n_contrib, max_contrib, per_tile_bucket_offset, bucket_to_tile, sampled_T, sampled_ar)
-        return None, None, grad_means2D, grad_colors, grad_conic_opacity, None, None, grad_extra, None, None, None
+            point_list, n_contrib, max_contrib, per_tile_bucket_offset, bucket_to_tile, sampled_T, sampled_ar,
+            point_offsets, radii)
+        return (None, None, grad_means2D, grad_colors, grad_conic_opacity, None, None, grad_extra, None, None, None,
+                None, None)
 
 
 def GS_render_fast(W: int, H: int, mean2D: Tensor, colors: Tensor, conic_opacity: Tensor, tile_range: Tensor,
                    point_list: Tensor, extra: Tensor = None, accum_max_count=None, accum_weights_p=None,
-                   accum_weights_count=None):
-    """`GS_render` through the bucketed forward / per-Gaussian backward pair (gaussian_render.py:803-837)."""
+                   accum_weights_count=None, point_offsets: Tensor = None, radii: Tensor = None):
+    """`GS_render` through the bucketed forward / per-Gaussian backward pair (gaussian_render.py:803-837).
+    `point_offsets` / `radii` as for `GS_render`."""
     return _GS_render_fast.apply(W, H, mean2D, colors, conic_opacity, tile_range, point_list, extra, accum_max_count,
-                                 accum_weights_p, accum_weights_count)
+                                 accum_weights_p, accum_weights_count, point_offsets, radii)
 
 
 def GS_render(W: int, H: int, mean2D: Tensor, colors: Tensor, conic_opacity: Tensor, tile_range: Tensor,
               point_list: Tensor, extra: Tensor = None, accum_max_count=None, accum_weights_p=None,
-              accum_weights_count=None):
-    """-> (images[3,H,W], opacity[H,W], extras[E,H,W]|None, n_contrib[H,W]); gaussian_render.py:839-845."""
+              accum_weights_count=None, point_offsets: Tensor = None, radii: Tensor = None):
+    """-> (images[3,H,W], opacity[H,W], extras[E,H,W]|None, n_contrib[H,W]); gaussian_render.py:839-845. With the
+    binning's scan offsets (`GS_prepare(..., return_offsets=True)`) and the radii the backward sums the per-Gaussian
+    gradients in a fixed order without atomics."""
     return _GS_render.apply(W, H, mean2D, colors, conic_opacity, tile_range, point_list, extra, accum_max_count,
-                            accum_weights_p, accum_weights_count)
+                            accum_weights_p, accum_weights_count, point_offsets, radii)
 
 
 def RasterizeGaussians(means3D: Tensor, means2D: Optional[Tensor], colors: Tensor, sh_rest: Optional[Tensor],
@@ -286,10 +296,11 @@ def RasterizeGaussians(means3D: Tensor, means2D: Optional[Tensor], colors: Tenso
     means2D, depths, colors, radii, tiles_touched, conic_opacity = preprocess(
         means3D, scales, rotations, opacities, colors, sh_rest, Tw2v, Tv2c, cam_pos, tanFoV, W, H, sh_degree,
         is_opengl, cov3Ds_precomp, cov2Ds_precomp, means2D, culling)
-    tile_ranges, point_list = GS_prepare(W, H, means2D.detach(), depths.detach(), radii, tiles_touched, False)
+    tile_ranges, point_list, point_offsets = GS_prepare(W, H, means2D.detach(), depths.detach(), radii, tiles_touched,
+                                                        False, return_offsets=True)
     out_pixels, out_opacities, out_extras, n_contrib = GS_render(
         W, H, means2D, colors, conic_opacity, tile_ranges, point_list, extras, accum_max_count, accum_weights_p,
-        accum_weights_count)
+        accum_weights_count, point_offsets, radii)
     buffer = RasterizeBuffer3D(W, H, len(opacities), point_list.shape[0], tile_ranges, point_list, n_contrib,
                                conic_opacity, means2D, out_opacities)
     out_other_extras = [_render_extra.apply(W, H, extras_, means2D, conic_opacity, tile_ranges, point_list, n_contrib,

@@ -179,17 +179,18 @@ class _Fast_Render(torch.autograd.Function):
                 sh_degree, is_opengl, near_n, far_n, only_image, trans_precomp, means2D, trans_mat_t2, culling,
                 accum_max_count, accum_weights_p, accum_weights_count):
         W, H = size
-        (means2D, colors, trans_mat, inverse_m, normal_opacity, depths, radii, tile_range,
-         point_list) = _Fast_Render._preprocess_forward(W, H, sh_degree, is_opengl, means3D, scales, rotations,
-                                                        opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, Tv2s, campos,
-                                                        trans_precomp, means2D, culling, False)
+        (means2D, colors, trans_mat, inverse_m, normal_opacity, depths, radii, tile_range, point_list,
+         point_offsets) = _Fast_Render._preprocess_forward(W, H, sh_degree, is_opengl, means3D, scales, rotations,
+                                                           opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, Tv2s, campos,
+                                                           trans_precomp, means2D, culling, False, return_offsets=True)
         pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib = _Fast_Render._render_forward(
             W, H, near_n, far_n, only_image, means2D, colors, normal_opacity, trans_mat, inverse_m, point_list,
             tile_range, trans_mat_t2, accum_max_count, accum_weights_p, accum_weights_count, None)
         ctx._info = (W, H, sh_degree, is_opengl, near_n, far_n)
         ctx.save_for_backward(means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, Tv2s, campos,
                               means2D, trans_mat, inverse_m, radii, colors, normal_opacity, tile_range, point_list,
-                              pixel_colors, pixel_extras, pixel_opacity, n_contrib, trans_mat_t2, pixel_flow)
+                              pixel_colors, pixel_extras, pixel_opacity, n_contrib, trans_mat_t2, pixel_flow,
+                              point_offsets)
         ctx.mark_non_differentiable(n_contrib, radii)
         return pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib, radii
 
@@ -198,7 +199,7 @@ class _Fast_Render(torch.autograd.Function):
     def backward(ctx, *grad_outputs):
         (means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, Tv2s, campos, means2D, trans_mat,
          inverse_m, radii, colors, normal_opacity, tile_range, point_list, pixel_colors, pixel_extras, pixel_opacity,
-         n_contrib, trans_mat_t2, pixel_flow) = ctx.saved_tensors
+         n_contrib, trans_mat_t2, pixel_flow, point_offsets) = ctx.saved_tensors
         W, H, sh_degree, is_opengl, near_n, far_n = ctx._info
         grad_images, grad_opacity, grad_others, grad_flow = grad_outputs[:4]
         if pixel_flow is None or grad_others is None:
@@ -210,7 +211,7 @@ class _Fast_Render(torch.autograd.Function):
         grad_colors, grad_means2D, grad_trans, grad_inv_m, grad_normal_opacity = _Fast_Render._render_backward(
             means2D, normal_opacity, colors, trans_mat, inverse_m, trans_mat_t2, pixel_colors, pixel_opacity,
             pixel_extras, pixel_flow, grad_images, grad_opacity, grad_others, grad_flow, tile_range, point_list,
-            n_contrib, near_n, far_n, None, None, None, None, None, None)
+            n_contrib, near_n, far_n, None, None, None, None, None, None, point_offsets, radii)
         grad_inputs = [
             torch.zeros_like(means3D), torch.zeros_like(scales), torch.zeros_like(rotations),
             torch.zeros_like(opacities),
@@ -285,17 +286,18 @@ def fast_compuate_transmat(means3D: Tensor, scales: Tensor, rotations: Tensor, T
 
 
 def fast_render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad_opacity: Tensor = None,
-                     per_splat: bool = False):
-    """One forward + backward pass of the fast path through the raw operators, returning every intermediate."""
+                     per_splat: bool = False, ordered_sums: bool = True):
+    """One forward + backward pass of the fast path through the raw operators, returning every intermediate. With
+    `ordered_sums` the blend backward adds per-instance records in a fixed order instead of using atomics."""
     pre_f = get_C_function('gs_2d_fast_preprocess_forward')
     pre_b = get_C_function('gs_2d_fast_preprocess_backward')
     ren_f = get_C_function('GS_2D_fast_render_forward')
     ren_b = get_C_function('GS_2D_fast_render_backward')
     W, H = cam.W, cam.H
     (means2D, colors, trans_mat, inverse_m, normal_opacity, depths, radii, ranges, point_list, keys,
-     tiles_touched) = pre_f(W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations,
-                            scene.opacities, scene.shs, None, cam.Tw2v, cam.Tv2c, cam.Tv2s, cam.campos, None, None,
-                            None, False, True)
+     tiles_touched, point_offsets) = pre_f(W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations,
+                                           scene.opacities, scene.shs, None, cam.Tw2v, cam.Tv2c, cam.Tv2s, cam.campos,
+                                           None, None, None, False, True, True)
     offset = None
     if per_splat:
         offset = torch.cumsum((ranges[:, 1] - ranges[:, 0] + 31) // 32, dim=0).contiguous()
@@ -307,7 +309,7 @@ def fast_render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None,
     g_colors, g_means2D, g_trans, g_inv, g_no = ren_b(
         means2D, normal_opacity, colors, trans_mat, inverse_m, None, image, opacity, extras, None, grad_image,
         grad_opacity, grad_extras, None, ranges, point_list, n_contrib, cam.near, cam.far, offset, None, None, None,
-        None, None)
+        None, None, point_offsets if ordered_sums else None, radii if ordered_sums else None)
     g_means2D_in = g_means2D.clone()
     g = dict(means3D=torch.zeros_like(scene.means3D), scales=torch.zeros_like(scene.scales),
              rotations=torch.zeros_like(scene.rotations), opacities=torch.zeros_like(scene.opacities),

@@ -198,13 +198,19 @@ int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, double fa
  * dL_dflow[H,W,2] (optional, with trans_mat_t2 and out_flow) is taken as the gradient of the UNDIVIDED flow sum, as both
  * reference kernels take it (:366, :704); the per-splat form additionally lowers the opacity map's gradient by
  * (out_flow . dL_dflow), the effect of the reference subtracting the divided flow from its partial sums (:706). No
- * gradient is produced for trans_mat_t2. All five gradient outputs MUST be zero-filled by the caller. */
+ * gradient is produced for trans_mat_t2. With point_offsets == NULL all five gradient outputs MUST be zero-filled by the
+ * caller (device-scope atomics, as in the reference). With point_offsets[P] (the inclusive prefix scan of tiles_touched
+ * that fsgs_gs_prepare_scan returns), radii[P], R = point_offsets[P-1] (the length of point_list, padding included) and
+ * a 16-byte aligned workspace of fsgs_gs_2d_fast_render_backward_workspace_bytes(R) bytes (no counterpart in the
+ * reference) every row of the outputs is ASSIGNED from per-(surfel, tile) records added in a fixed order. */
+size_t fsgs_gs_2d_fast_render_backward_workspace_bytes(int64_t R);
 int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n, double far_n, int per_splat_form,
     const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,
     const float* inverse_m, const float* trans_mat_t2, const float* out_opacity, const float* out_extras,
     const float* out_flow, const float* dL_dpix, const float* dL_dopacity, const float* dL_dextras,
     const float* dL_dflow, const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib,
-    float* g_colors, float* g_means2D, float* g_trans, float* g_inv, float* g_normal_opacity, void* stream);
+    float* g_colors, float* g_means2D, float* g_trans, float* g_inv, float* g_normal_opacity, int64_t R,
+    const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes, void* stream);
 
 /* gs_2d_topk_weights -- fast_2d_gs/_C/src/gaussian_splatting/gaussian_topk.cu:230-250 (kernel :95-210).
  * top_indices[H,W,topk] int32 (-1 = empty), top_weights[H,W,topk] descending blend weights alpha*T; topk <= 16. */
@@ -402,24 +408,32 @@ int fsgs_gaussian_rasterize_forward(int P, int W, int H, int E, const float* mea
     float* out_color, float* out_opacity, float* out_extras, int32_t* n_contrib, int32_t* max_contrib,
     int32_t* bucket_to_tile, float* sampled_T, float* sampled_ar, void* stream);
 
-/* gaussian_rasterize_backward -- gaussian_render.cu:486-536 (kernel :296-444). Accumulates into caller-zeroed
- * g_means2D[P,2], g_conic_opacity[P,4], g_colors[P,3], g_extras[P,E]. */
+/* gaussian_rasterize_backward -- gaussian_render.cu:486-536 (kernel :296-444). g_means2D[P,2], g_conic_opacity[P,4],
+ * g_colors[P,3], g_extras[P,E]. With point_offsets == NULL the per-Gaussian sums are accumulated with device-scope
+ * atomics into the caller-zeroed outputs, as in the reference. With point_offsets[P] (the inclusive prefix scan of
+ * tiles_touched that fsgs_gs_prepare_scan returns), radii[P], the instance count R and a 16-byte aligned workspace of
+ * fsgs_gaussian_rasterize_backward_workspace_bytes(R) bytes (no counterpart in the reference) every row of the outputs
+ * is ASSIGNED from per-(Gaussian, tile) records added in a fixed order: no zero fill, no atomics, and the sums do not
+ * vary from run to run. */
+size_t fsgs_gaussian_rasterize_backward_workspace_bytes(int64_t R);
 int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const float* means2D, const float* conic_opacity,
     const float* colors, const float* extras, const float* out_opacity, const int32_t* n_contrib,
     const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
-    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, void* stream);
+    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, int64_t R,
+    const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes, void* stream);
 
 /* gaussian_rasterize_fast_backward -- gaussian_render.cu:760-812 (kernel :540-694): the reference's per-Gaussian
  * backward over the forward's bucket snapshots. It is the same derivative as gaussian_rasterize_backward and runs
  * that kernel here; the snapshot arguments must be present but are not read. With E > 0 the reference reads the extra
  * channels' upstream gradient into the wrong registers (:636); the gradient of what the forward computes is returned.
- * Outputs caller-zeroed as above. */
+ * Outputs and the optional ordered-sum arguments as above. */
 int fsgs_gaussian_rasterize_fast_backward(int P, int W, int H, int E, const float* means2D,
     const float* conic_opacity, const float* colors, const float* extras, const float* images,
     const float* out_extras, const float* out_opacity, const int32_t* n_contrib, const int32_t* max_contrib,
     const int64_t* bucket_offset, const int32_t* bucket_to_tile, const float* sampled_T, const float* sampled_ar,
     const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
-    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, void* stream);
+    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, int64_t R,
+    const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- render epilogue -------------------------------------------------------------------------------------------- */
 

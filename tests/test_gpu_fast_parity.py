@@ -181,6 +181,32 @@ def test_fast_autograd_wrapper_and_accum(device):
     assert int(acc_n.sum()) >= int((raw['n_contrib'][0] > 0).sum())
 
 
+@pytest.mark.parametrize("per_splat", [False, True])
+@pytest.mark.parametrize("name", ["partial_tiles_511x127", "dense_6k_96"])
+def test_fast_ordered_sums_match_the_atomic_sums(name, per_splat, device):
+    """The blend backward's per-surfel sums through per-(surfel, tile) records added in a fixed order (what
+    fast_render_step does by default, and what the stage-by-stage test holds to the oracle) against the reference's way,
+    device-scope atomics into zero-filled outputs: equal up to the order of the additions, identical from run to run,
+    every row assigned (the record path's outputs are not zero-filled), rows 0 and 1 of dL/dtrans_mat zeros."""
+    from fast_sp_gs_amd.renderer import fast_render_step
+    scene, cam, gi, ge, go = _make(name)
+    args = (scene.to(device), cam.to(device), gi.to(device), ge.to(device), go.to(device))
+    a = fast_render_step(*args, per_splat=per_splat)
+    b = fast_render_step(*args, per_splat=per_splat)
+    c = fast_render_step(*args, per_splat=per_splat, ordered_sums=False)
+    torch.cuda.synchronize()
+    hidden = a['radii'] <= 0
+    assert int(hidden.sum()) < scene.P and (name != 'partial_tiles_511x127' or int(hidden.sum()) > 0)
+    for k in ('g_colors', 'g_means2D_blend', 'g_trans', 'g_inv', 'g_normal_opacity', 'g_means3D', 'g_scales',
+              'g_rotations', 'g_opacities', 'g_shs'):
+        assert torch.equal(a[k], b[k]) and bool(torch.isfinite(a[k]).all()), k
+        ref = float(c[k].abs().max())
+        assert ref > 0 and float((a[k] - c[k]).abs().max()) <= 2e-5 * ref, k
+        if k in ('g_colors', 'g_means2D_blend', 'g_trans', 'g_inv', 'g_normal_opacity'):
+            assert not a[k][hidden].any(), k
+    assert not a['g_trans'][:, :2].any() and a['g_trans'][:, 2].any()
+
+
 def test_fast_empty_scene(device):
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd.renderer import fast_render_step

@@ -82,7 +82,8 @@ def _binned(P, W, H, seed, device):
         W, H, 3, False, d(scene.means3D), d(scales), d(scene.rotations), d(scene.opacities), d(scene.shs), None,
         d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), tan_fov, None, None, None, None)
     m2, dep, col, rad, tt, c3, co = out
-    ranges, pl = get_C_function('GS_prepare')(W, H, m2, dep, rad, tt, False)
+    ranges, pl, offsets = get_C_function('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True)
+    _binned.offsets, _binned.radii = offsets, rad  # for the backward's ordered-sum path
     return m2, col, co, ranges, pl
 
 
@@ -125,6 +126,19 @@ def test_gs3d_rasterize(P, W, H, E, device):
         assert rel_err(n(g_ex), r_ex) < 1e-3
     else:
         assert g_ex is None
+    # the same sums through per-(Gaussian, tile) records added in a fixed order: equal to the atomic sums up to the
+    # order of the additions, identical from run to run, and every row assigned (the outputs are not zero-filled)
+    bwd = lambda: get_C_function('gaussian_rasterize_backward')(m2, co, col, ex, oo, gi, go, ge, ranges, pl, nc,
+                                                                _binned.offsets, _binned.radii)
+    first, second = bwd(), bwd()
+    torch.cuda.synchronize()
+    for a, b, c in zip(first, second, (g_col, g_ex, g_m2, g_co)):
+        if c is None:
+            assert a is None
+            continue
+        assert torch.equal(a, b) and bool(torch.isfinite(a).all())
+        assert float((a - c).abs().max()) <= 2e-5 * max(float(c.abs().max()), 1e-30)
+        assert not a[_binned.radii <= 0].any()
 
 
 @pytest.mark.parametrize("K", [1, 4, 7, 16])
