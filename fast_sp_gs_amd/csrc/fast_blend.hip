@@ -339,7 +339,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
     const float2* __restrict__ dL_dflow,
     float* __restrict__ g_means2D, float* __restrict__ g_normal_opacity, float* __restrict__ g_colors,
     float* __restrict__ g_trans, float* __restrict__ g_inv, const int64_t* __restrict__ point_offsets,
-    const int32_t* __restrict__ radii, float* __restrict__ slot_records, unsigned char* __restrict__ slot_written) {
+    const int32_t* __restrict__ radii, float* __restrict__ slot_records) {
   constexpr int kB = 64;  // surfels staged per round
   __shared__ FastHot s_hot[kB];
   __shared__ SplatCold s_cold[kB];
@@ -568,7 +568,6 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
 #pragma unroll
           for (int c = 0; c < kFastRecordSlots / 2; ++c)
             dst[c] = make_float2(a[2 * c], 2 * c + 1 < kFastGradSlots ? a[2 * c + 1] : 0.0f);
-          slot_written[slot] = 1;
         }
       } else {
 #pragma unroll
@@ -659,7 +658,7 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
   FSGS_REQUIRE(!flow || (aux && trans_mat_t2 && out_flow),
                "GS_2D_fast_render_backward: flow gradients need trans_mat2, out_flows and the auxiliary maps");
   const bool slots = point_offsets != nullptr;
-  SlotWorkspace ws{nullptr, nullptr};
+  SlotWorkspace ws{nullptr};
   if (slots) {
     FSGS_REQUIRE(radii && workspace && R >= 0 && R < (int64_t) 0x7fffffff,
                  "GS_2D_fast_render_backward: the ordered-sum path needs radii, a workspace and the instance count R");
@@ -672,7 +671,7 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
-  if (slots) launch_slot_clear(ws, R, s);
+  if (slots) launch_slot_clear<kFastRecordSlots>(ws, R, s);
   const int* tile_order = nullptr;
   const int ordered = launch_tile_order(gx, gy, ranges, s, &tile_order);
 #define FSGS_LAUNCH_BWD_S(AUX, SPLAT, FLOW, SL)                                                                      \
@@ -681,7 +680,7 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
                      (const float4*) normal_opacity, colors, trans_mat, inverse_m, trans_mat_t2, out_opacity,        \
                      out_extras, (const float2*) out_flow, dL_dpix, dL_dextras, dL_dopacity,                         \
                      (const float2*) dL_dflow, g_means2D, g_normal_opacity, g_colors, g_trans, g_inv, point_offsets, \
-                     radii, ws.records, ws.written)
+                     radii, ws.records)
 #define FSGS_LAUNCH_BWD(AUX, SPLAT, FLOW) \
   do { if (slots) FSGS_LAUNCH_BWD_S(AUX, SPLAT, FLOW, true); else FSGS_LAUNCH_BWD_S(AUX, SPLAT, FLOW, false); } while (0)
   if (aux && per_splat_form && flow) FSGS_LAUNCH_BWD(true, true, true);

@@ -352,7 +352,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
     const float* __restrict__ dL_dout_extras, const float* __restrict__ dL_dout_opacity,
     float* __restrict__ g_means2D, float* __restrict__ g_conic_opacity, float* __restrict__ g_colors,
     float* __restrict__ g_extras, const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii,
-    float* __restrict__ slot_records, unsigned char* __restrict__ slot_written) {
+    float* __restrict__ slot_records) {
   constexpr int kB = 64;
   __shared__ G3Hot s_hot[kB];
   __shared__ float s_feat[kB][3 + kMaxExtra + 1];
@@ -470,7 +470,6 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
           float4* dst = (float4*) (slot_records + slot * kG3Slots);
 #pragma unroll
           for (int c = 0; c < kG3Slots / 4; ++c) dst[c] = make_float4(a[4 * c], a[4 * c + 1], a[4 * c + 2], a[4 * c + 3]);
-          slot_written[slot] = 1;
         }
       } else {
         const int id = s_hot[threadIdx.x].id;
@@ -782,7 +781,7 @@ FSGS_API int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const 
                    g_means2D && g_conic_opacity && g_colors && (E == 0 || (extras && dL_dout_extras && g_extras)),
                "gaussian_rasterize_backward: null pointer");
   const bool slots = point_offsets != nullptr;
-  SlotWorkspace ws{nullptr, nullptr};
+  SlotWorkspace ws{nullptr};
   if (slots) {
     FSGS_REQUIRE(radii && workspace && R >= 0 && R < (int64_t) 0x7fffffff,
                  "gaussian_rasterize_backward: the ordered-sum path needs radii, a workspace and the instance count R");
@@ -794,7 +793,7 @@ FSGS_API int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const 
   }
   hipStream_t s = (hipStream_t) stream;
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
-  if (slots) launch_slot_clear(ws, R, s);
+  if (slots) launch_slot_clear<kG3Slots>(ws, R, s);
   const int* tile_order = nullptr;
   const int flags = launch_tile_order(gx, gy, ranges, s, &tile_order);
   const dim3 grid(gx * gy), block(kBlendThreads);
@@ -802,7 +801,7 @@ FSGS_API int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const 
   hipLaunchKernelGGL((gs3d_backward_kernel<EE, SL>), grid, block, 0, s, flags, tile_order, W, H, ranges, point_list, \
                      (const float2*) means2D, (const float4*) conic_opacity, colors, extras, out_opacity, n_contrib, \
                      dL_dpix, dL_dout_extras, dL_dout_opacity, g_means2D, g_conic_opacity, g_colors, g_extras,      \
-                     point_offsets, radii, ws.records, ws.written)
+                     point_offsets, radii, ws.records)
 #define FSGS_G3_BWD_E(EE)                                                                                           \
   do {                                                                                                              \
     if (slots) {                                                                                                    \

@@ -1,9 +1,9 @@
 // Per-surfel sums of per-(surfel, tile) gradient records in a fixed order, without atomics and without a zero fill of
 // the outputs. The tile binning emits a surfel's instances at consecutive positions of the unsorted key list, starting at
 // the surfel's prefix-scan offset; a backward block that has summed one instance over its tile's pixels writes the sums
-// as one record at that position and sets the instance's "written" byte. slot_sum_kernel then adds a surfel's written
-// records in position order and hands every component of every surfel (zeros where nothing was written) to a scatter
-// functor that knows the output tensors. The reference flushes these sums with one device-scope atomic per component,
+// as one record at that position (records nobody writes stay at the zero fill of the record buffer, a streaming write
+// that measured cheaper than per-instance "written" flags). slot_sum_kernel then adds a surfel's records in position
+// order and hands every component of every surfel to a scatter functor that knows the output tensors. The reference flushes these sums with one device-scope atomic per component,
 // tile and surfel into caller-zeroed tensors (e.g. gaussian_render.cu:560-600, gs_2d_fast_redner.cu:520-560).
 #pragma once
 #include <algorithm>
@@ -13,19 +13,13 @@
 namespace fsgs {
 
 struct SlotWorkspace {
-  float* records;          // [R][kFloats]
-  unsigned char* written;  // [R], rounded up to whole float4s
+  float* records;  // [R][kFloats]
 };
 
-inline size_t slot_written_offset(int64_t R, int floats) {
+inline size_t slot_workspace_bytes(int64_t R, int floats) {
   return align_up((size_t) (R > 0 ? R : 0) * floats * 4 + 16, 256);
 }
-inline size_t slot_workspace_bytes(int64_t R, int floats) {
-  return slot_written_offset(R, floats) + align_up((size_t) (R > 0 ? R : 0) + 16, 256);
-}
-inline SlotWorkspace slot_workspace(void* base, int64_t R, int floats) {
-  return SlotWorkspace{(float*) base, (unsigned char*) base + slot_written_offset(R, floats)};
-}
+inline SlotWorkspace slot_workspace(void* base, int64_t, int) { return SlotWorkspace{(float*) base}; }
 
 namespace {
 
@@ -35,11 +29,10 @@ __global__ void __launch_bounds__(256) slot_clear_kernel(size_t n4, float4* __re
 }
 
 // kFloats / 2 lanes per surfel, each owning one float2 of the record, so the lanes of a surfel read consecutive bytes
-// and neighbouring surfels continue where the previous one ends. Eight records of a surfel are in flight together; a
-// record's load does not wait for its "written" byte (an unwritten record's bytes are read and dropped).
+// and neighbouring surfels continue where the previous one ends. Eight records of a surfel are in flight together.
 template <int kFloats, typename Scatter>
 __global__ void __launch_bounds__(256) slot_sum_kernel(int P, const int64_t* __restrict__ point_offsets,
-    const float* __restrict__ records, const unsigned char* __restrict__ written, Scatter out) {
+    const float* __restrict__ records, Scatter out) {
   static_assert(kFloats % 2 == 0 && kFloats <= 64, "records are whole float2s");
   constexpr int kLanes = kFloats / 2, kPerWave = 64 / kLanes, kDepth = 8;
   const int lane = threadIdx.x & 63;
@@ -52,16 +45,11 @@ __global__ void __launch_bounds__(256) slot_sum_kernel(int P, const int64_t* __r
   float2 acc = make_float2(0.0f, 0.0f);
   for (int64_t base = e0; base < e1; base += kDepth) {
     float2 v[kDepth];
-    unsigned char ok[kDepth];
+#pragma unroll
+    for (int j = 0; j < kDepth; ++j) v[j] = src[(size_t) (base + j < e1 ? base + j : e1 - 1) * kLanes];
 #pragma unroll
     for (int j = 0; j < kDepth; ++j) {
-      const size_t at = (size_t) (base + j < e1 ? base + j : e1 - 1);
-      v[j]  = src[at * kLanes];
-      ok[j] = written[at];
-    }
-#pragma unroll
-    for (int j = 0; j < kDepth; ++j) {
-      const bool on = base + j < e1 && ok[j] != 0;
+      const bool on = base + j < e1;
       acc.x += on ? v[j].x : 0.0f, acc.y += on ? v[j].y : 0.0f;
     }
   }
@@ -69,10 +57,11 @@ __global__ void __launch_bounds__(256) slot_sum_kernel(int P, const int64_t* __r
   out(i, 2 * k + 1, acc.y);
 }
 
+template <int kFloats>
 inline void launch_slot_clear(const SlotWorkspace& ws, int64_t R, hipStream_t s) {
-  const size_t n4 = ((size_t) R + 15) / 16;
+  const size_t n4 = ((size_t) R * kFloats + 3) / 4;
   const unsigned blocks = (unsigned) std::min<size_t>((n4 + 255) / 256, 8192);
-  if (n4 > 0) hipLaunchKernelGGL(slot_clear_kernel, dim3(blocks), dim3(256), 0, s, n4, (float4*) ws.written);
+  if (n4 > 0) hipLaunchKernelGGL(slot_clear_kernel, dim3(blocks), dim3(256), 0, s, n4, (float4*) ws.records);
 }
 
 template <int kFloats, typename Scatter>
@@ -80,7 +69,7 @@ inline void launch_slot_sum(int P, const int64_t* point_offsets, const SlotWorks
   constexpr int kPerWave = 64 / (kFloats / 2);
   const int64_t waves = div_up(P, kPerWave);
   hipLaunchKernelGGL((slot_sum_kernel<kFloats, Scatter>), dim3((unsigned) div_up(waves * 64, 256)), dim3(256), 0, s, P,
-                     point_offsets, ws.records, ws.written, out);
+                     point_offsets, ws.records, out);
 }
 
 }  // namespace
