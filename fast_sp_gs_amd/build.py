@@ -48,7 +48,7 @@ def build(verbose: bool = False, incremental: bool = False, jobs: int = 0) -> Pa
     """Compile every HIP source into one shared object."""
     OBJ_DIR.mkdir(exist_ok=True)
     hipcc = hipcc_path()
-    headers_mtime = max(p.stat().st_mtime for p in list(CSRC.glob("*.hpp")) + [PKG_DIR.parent / "include" / "fsgs.h"])
+    headers_mtime = max(p.stat().st_mtime for p in list(CSRC.glob("*.hpp")) + list((PKG_DIR.parent / "include").glob("*.h")))
     todo = []
     for s in SOURCES:
         src, obj = CSRC / s, OBJ_DIR / (s + ".o")

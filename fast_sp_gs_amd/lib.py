@@ -13,6 +13,7 @@ import torch
 
 PKG_DIR = Path(__file__).resolve().parent
 HEADER = PKG_DIR.parent / "include" / "fsgs.h"
+DEBUG_HEADER = PKG_DIR.parent / "include" / "fsgs_debug.h"  # measurement / verification aids
 LIB_PATH = PKG_DIR / "libfsgs_hip.so"
 
 _SCALARS = {
@@ -49,7 +50,7 @@ _protos = None
 def prototypes():
     global _protos
     if _protos is None:
-        _protos = parse_prototypes(HEADER.read_text(), "fsgs_")
+        _protos = parse_prototypes(HEADER.read_text() + "\n" + DEBUG_HEADER.read_text(), "fsgs_")
     return _protos
 
 

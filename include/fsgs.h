@@ -24,14 +24,6 @@ extern "C" {
 const char* fsgs_last_error(void);
 int fsgs_version(void);
 int fsgs_check_device(void);
-/* Measurement aid without a counterpart in the reference: copies nbytes (multiple of 16, 16-byte aligned) from src to
- * dst with a plain streaming kernel; benchmarks use it as the achievable-bandwidth yardstick and counter calibration. */
-int fsgs_copy_probe(const void* src, void* dst, size_t nbytes, void* stream);
-/* Verification aid without a counterpart in the reference: the blend kernels skip, per 8x8 pixel quadrant, surfels whose
- * alpha >= 1/255 footprint cannot reach it. enabled = 0 turns that skip off process-wide (every staged surfel is then
- * evaluated at every pixel, as the reference does), so tests can show that results do not depend on it. Default: on. */
-int fsgs_debug_set_culling(int enabled);
-
 /* ---- 2DGS surfel preprocess ---------------------------------------------------------------------------------- */
 
 /* gs_2d_preprocess_forward -- fast_2d_gs/_C/src/gaussian_splatting/gs_2d_preprocess.cu:331-421 (kernel :158-246).

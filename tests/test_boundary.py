@@ -1,4 +1,4 @@
-"""CPU-side checks of the drop-in boundary: the shared library loads, exports every symbol include/fsgs.h declares,
+"""CPU-side checks of the drop-in boundary: the shared library loads, exports every symbol include/fsgs.h and include/fsgs_debug.h declare,
 the operator namespace mirrors the reference's `fast_2d_gs/_C/__init__.py` helpers, and argument errors surface as
 RuntimeError before any kernel is launched. No compute call is made here (no GPU)."""
 import ctypes
@@ -20,7 +20,7 @@ REFERENCE_NAMES = [  # the pybind m.def names on the hot path
 
 def test_library_exports_every_declared_symbol():
     from fast_sp_gs_amd import lib
-    text = (ROOT / "include" / "fsgs.h").read_text()
+    text = (ROOT / "include" / "fsgs.h").read_text() + (ROOT / "include" / "fsgs_debug.h").read_text()
     declared = set(re.findall(r"\b(fsgs_\w+)\s*\(", re.sub(r"/\*.*?\*/", " ", text, flags=re.S)))
     assert len(declared) >= 26
     L = lib.load()
