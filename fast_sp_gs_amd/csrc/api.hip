@@ -21,22 +21,28 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
-// One blockIdx -> tile table (65536 ints, see blend.hpp) per (device, stream) that a blend entry point was called on.
-int* tile_order_table(hipStream_t stream) {
+// One blockIdx -> tile table (65536 ints, see blend.hpp) per (device, stream) that a blend entry point was called on,
+// with the tile ranges it was built from.
+TileOrderState* tile_order_state(hipStream_t stream) {
   static std::mutex mu;
-  static std::map<std::pair<int, hipStream_t>, int*> tables;
+  static std::map<std::pair<int, hipStream_t>, TileOrderState> tables;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return nullptr;
   std::lock_guard<std::mutex> lock(mu);
   auto it = tables.find({dev, stream});
-  if (it != tables.end()) return it->second;
+  if (it != tables.end()) return it->second.table ? &it->second : nullptr;
   int* p = nullptr;
   if (hipMalloc((void**) &p, sizeof(int) * (1 << 16)) != hipSuccess) {
     (void) hipGetLastError();
     p = nullptr;
   }
-  tables[{dev, stream}] = p;
-  return p;
+  TileOrderState& st = tables[{dev, stream}];
+  st = TileOrderState{p, nullptr, 0, 0};
+  return p ? &st : nullptr;
+}
+
+void tile_order_invalidate(hipStream_t stream) {
+  if (TileOrderState* st = tile_order_state(stream)) st->ranges = nullptr;
 }
 
 static bool g_culling_enabled = true;

@@ -82,19 +82,6 @@ __global__ void __launch_bounds__(kScanThreads) scan_block_sums_kernel(int P, co
   if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
 }
 
-__global__ void __launch_bounds__(kScanThreads) scan_spine_kernel(int n, int64_t* __restrict__ block_sums) {
-  __shared__ int64_t s_wave[kScanThreads / kWave];
-  int64_t carry = 0;
-  for (int start = 0; start < n; start += kScanThreads) {
-    const int i = start + threadIdx.x;
-    const int64_t v = i < n ? block_sums[i] : 0;
-    int64_t total;
-    const int64_t ex = block_exclusive_scan<int64_t>(v, s_wave, total);
-    if (i < n) block_sums[i] = carry + ex;
-    carry += total;
-  }
-}
-
 __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(int P, const int32_t* __restrict__ in,
                                                                   const int64_t* __restrict__ block_sums,
                                                                   int64_t* __restrict__ out) {
@@ -107,8 +94,14 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(int P, const i
     v[k] = base + k < P ? in[base + k] : 0;
     sum += v[k];
   }
+  // The sum of the chunks in front of this one is formed here, by every block for itself (a few hundred values at most),
+  // instead of by a one-block kernel between the two passes: one launch less in front of the host's wait for the count.
+  int64_t before = 0;
+  for (int i = threadIdx.x; i < (int) blockIdx.x; i += kScanThreads) before += block_sums[i];
   int64_t total;
-  int64_t run = block_sums[blockIdx.x] + block_exclusive_scan<int64_t>(sum, s_wave, total);
+  block_exclusive_scan<int64_t>(before, s_wave, total);
+  const int64_t chunk_start = total;
+  int64_t run = chunk_start + block_exclusive_scan<int64_t>(sum, s_wave, total);
 #pragma unroll
   for (int k = 0; k < kScanItems; ++k) {
     run += v[k];
@@ -727,7 +720,6 @@ FSGS_API int fsgs_gs_prepare_scan_begin(int P, const int32_t* tiles_touched, int
     const int nb      = div_up(P, kScanChunk);
     int64_t* blk_sums = (int64_t*) workspace;
     hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(kScanThreads), 0, s, P, tiles_touched, blk_sums);
-    hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanThreads), 0, s, nb, blk_sums);
     hipLaunchKernelGGL(scan_apply_kernel, dim3(nb), dim3(kScanThreads), 0, s, P, tiles_touched, blk_sums,
                        point_offsets);
     if (int rc = check_launch("gs_prepare_scan")) return rc;
@@ -820,6 +812,7 @@ FSGS_API int fsgs_gs_prepare_count(int P, int W, int H, const float* means2D, co
                                    int32_t* large_count, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && ranges && large_count, "gs_prepare_count: bad arguments");
   FSGS_REQUIRE(P == 0 || (means2D && radii), "gs_prepare_count: null pointer");
+  tile_order_invalidate((hipStream_t) stream);  // the ranges are rewritten: the blend schedule of this stream is stale
   return fill_count(P, W, H, means2D, radii, ranges, large_count, (hipStream_t) stream);
 }
 
@@ -845,6 +838,7 @@ FSGS_API int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, con
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && R >= 0 && ranges, "gs_prepare_fill: bad arguments");
   FSGS_REQUIRE(R < (int64_t) 0x7fffffff, "gs_prepare_fill: %lld instances exceed the 2^31-1 limit", (long long) R);
   hipStream_t s = (hipStream_t) stream;
+  tile_order_invalidate(s);  // the ranges are rewritten: the blend schedule of this stream is stale
   if (R == 0 || P == 0) {
     const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
     hipLaunchKernelGGL(fill_zero_i64_kernel, dim3(div_up(2 * (int64_t) gx * gy, 256)), dim3(256), 0, s,

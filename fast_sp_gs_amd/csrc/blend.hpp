@@ -214,8 +214,7 @@ constexpr int kMaxOrderedTiles = 1 << 16;
 constexpr int kOrderBuckets    = 128;
 constexpr int kOrderRegions    = 8;
 
-// Defined in api.hip. nullptr if the table cannot be allocated (then blocks map to tiles directly).
-int* tile_order_table(hipStream_t stream);
+// (TileOrderState, tile_order_state and tile_order_invalidate are declared in common.hpp.)
 
 namespace {
 
@@ -276,10 +275,13 @@ inline int launch_tile_order(int gx, int gy, const int64_t* ranges, hipStream_t 
   int flags = culling_enabled() ? 0 : kFlagNoCull;
   *table    = nullptr;
   if ((int64_t) gx * gy > kMaxOrderedTiles) return flags;
-  int* t = tile_order_table(s);
-  if (!t) return flags;
-  hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, s, gx, gy, ranges, t);
-  *table = t;
+  TileOrderState* st = tile_order_state(s);
+  if (!st) return flags;
+  if (st->ranges != ranges || st->gx != gx || st->gy != gy) {
+    hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, s, gx, gy, ranges, st->table);
+    st->ranges = ranges, st->gx = gx, st->gy = gy;
+  }
+  *table = st->table;
   return flags | kFlagOrdered;
 }
 

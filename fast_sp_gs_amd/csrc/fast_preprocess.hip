@@ -502,6 +502,7 @@ FSGS_API int fsgs_gs_2d_fast_prepare_fill(int P, int W, int H, const float* mean
   hipStream_t s = (hipStream_t) stream;
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int T  = gx * gy;
+  tile_order_invalidate(s);  // the ranges are rewritten: the blend schedule of this stream is stale
   launch_zero_ranges(T, ranges, s);
   if (R == 0 || P == 0) return check_launch("gs_2d_fast_prepare_fill(zero)");
   FSGS_REQUIRE(means2D && inverse_m && depths && opacities && radii && point_offsets && point_list && workspace,
