@@ -243,13 +243,15 @@ def gs3d_path_rate(dev, scene, cam, gi, steps: int = 30, warmup: int = 5):
     go = -gi.sum(0)  # white-background composite
     R = [0]
 
-    def step():
+    def step(ordered=True):
         m2, dep, col, rad, tt, c3, co = f('gs_preprocess_forward')(
             W, H, 3, False, scene.means3D, scales, scene.rotations, scene.opacities, scene.shs, None, cam.Tw2v,
             cam.Tv2c, cam.campos, tan_fov, None, None, None, None)
-        ranges, pl = f('GS_prepare')(W, H, m2, dep, rad, tt, False)
+        ranges, pl, offsets = f('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True)
         oc, oo, _, nc = f('gaussian_rasterize_forward')(W, H, m2, co, col, None, pl, ranges)
-        g_col, _, g_m2, g_co = f('gaussian_rasterize_backward')(m2, co, col, None, oo, gi, go, None, ranges, pl, nc)
+        # per-Gaussian sums through ordered per-instance records (what RasterizeGaussians does), or the reference's atomics
+        g_col, _, g_m2, g_co = f('gaussian_rasterize_backward')(m2, co, col, None, oo, gi, go, None, ranges, pl, nc,
+                                                                offsets if ordered else None, rad if ordered else None)
         g3, gs, gq = torch.empty_like(scene.means3D), torch.empty_like(scales), torch.empty_like(scene.rotations)
         gop, gsh = torch.empty_like(scene.opacities), torch.empty_like(scene.shs)
         f('gs_preprocess_backward')(W, H, 3, False, scene.means3D, scales, scene.rotations, scene.opacities, scene.shs,
@@ -268,6 +270,14 @@ def gs3d_path_rate(dev, scene, cam, gi, steps: int = 30, warmup: int = 5):
         state = step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    for _ in range(warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(False)
+    torch.cuda.synchronize()
+    dt_atomic = time.perf_counter() - t0
     gc.enable()
 
     # a 16-channel feature table blended with the finished view's weights, and its backward
@@ -289,6 +299,7 @@ def gs3d_path_rate(dev, scene, cam, gi, steps: int = 30, warmup: int = 5):
     ev[2].record()
     torch.cuda.synchronize()
     return {"gs3d_path_frames_per_s": steps / dt,
+            "gs3d_path_atomic_sums_frames_per_s": steps / dt_atomic,
             "gs3d_path_workload": f"same 300k centres as 3D Gaussians (third scale added), 800x800, SH degree 3, "
                                   f"R = {R[0]}: gs_preprocess fwd/bwd + GS_prepare + gaussian_rasterize fwd/bwd",
             "gs3d_extra16_forward_ms": ev[0].elapsed_time(ev[1]) / 10,
@@ -523,22 +534,25 @@ def training_forward_ms(dev, scene, cam, reps: int = 30):
 
 
 def fast_path_rate(dev, scene, cam, gi, steps: int = 20, warmup: int = 3):
-    """The "fast" variant (adjugate intersection, fused corner-test binning) on the benchmark scene, forward + backward."""
+    """The "fast" variant (adjugate intersection, fused corner-test binning) on the benchmark scene, forward + backward,
+    with the blend backward's per-surfel sums through ordered per-instance records (default) and through atomics."""
     from fast_sp_gs_amd.renderer import fast_render_step
     ge = torch.zeros(8, cam.H, cam.W, device=dev)
     go = -gi.sum(0)
-    for _ in range(warmup):
-        fast_render_step(scene, cam, gi, ge, go)
-    torch.cuda.synchronize()
-    gc.collect()
-    gc.disable()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fast_render_step(scene, cam, gi, ge, go)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    gc.enable()
-    return steps / dt
+    rates = []
+    for ordered in (True, False):
+        for _ in range(warmup):
+            fast_render_step(scene, cam, gi, ge, go, ordered_sums=ordered)
+        torch.cuda.synchronize()
+        gc.collect()
+        gc.disable()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fast_render_step(scene, cam, gi, ge, go, ordered_sums=ordered)
+        torch.cuda.synchronize()
+        rates.append(steps / (time.perf_counter() - t0))
+        gc.enable()
+    return rates
 
 
 def main():
@@ -663,7 +677,7 @@ def main():
         extra.update(gs3d_path_rate(dev, scene, cam, gi))
         extra.update(density_control_ms(dev, scene))
         extra.update(large_scene_ms(dev))
-        extra["fast_path_frames_per_s"] = fast_path_rate(dev, scene, cam, gi)
+        extra["fast_path_frames_per_s"], extra["fast_path_atomic_sums_frames_per_s"] = fast_path_rate(dev, scene, cam, gi)
         extra["fast_path_workload"] = "same scene through GS_2D_fast_* (corner-test binning keeps fewer instances)"
         extra["dynamic_step_frames_per_s"] = dynamic_step_rate(dev)
         extra["dynamic_step_workload"] = ("200000 surfels, 512 control points, bf16 MFMA MLP + K-NN(4) + LBS -> render "

@@ -194,6 +194,23 @@ def test_gs3d_render_autograd_and_empty(device):
         assert rel_err(n(p_.grad), r) < 1e-3, (name, rel_err(n(p_.grad), r))
     assert rel_err(n(feat.grad), g_ex) < 1e-3
     assert rel_err(n(out['viewspace_points'].grad), rm2) < 1e-3  # what densification reads
+    # the same pass with the blend backward's sums taken in a fixed order (module switch): same gradients up to the
+    # order of the additions, and identical when repeated
+    atomic = [p_.grad.clone() for p_ in params] + [feat.grad.clone()]
+    runs = []
+    GR.DETERMINISTIC_SUMS = True
+    try:
+        for _ in range(2):
+            for p_ in params + [feat]:
+                p_.grad = None
+            o2 = GR.render(d(cam.Tw2v), d(cam.Tv2c), (W, H), params[0], params[3], scales=params[1], rotations=params[2],
+                           campos=d(cam.campos), focals=focals, sh_features=params[4], sh_degree=3, feat=feat)
+            ((o2['images'] * gi).sum() + (o2['opacity'] * go).sum() + (o2['feat'] * gf).sum()).backward()
+            runs.append([p_.grad.clone() for p_ in params] + [feat.grad.clone()])
+    finally:
+        GR.DETERMINISTIC_SUMS = False
+    for a, b, c in zip(runs[0], runs[1], atomic):
+        assert torch.equal(a, b) and float((a - c).abs().max()) <= 2e-5 * float(c.abs().max())
     # empty scene
     z = lambda *s: torch.zeros(s, device=device)
     out = GR.render(d(cam.Tw2v), d(cam.Tv2c), (W, H), z(0, 3), z(0, 1), scales=z(0, 3), rotations=z(0, 4),
