@@ -23,7 +23,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 ROOT = os.path.dirname(os.path.abspath(__file__))
 # Hardware-counter summary of the dominant kernel (two rocprofv3 --pmc passes, calibrated against the copy probe).
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gs_2d_render_backward_300k_800x800.pmc_traffic.txt")
-SQ_SUMMARY = os.path.join(ROOT, "profiles", "blend_kernels_300k_800x800_and_deform_mlp.pmc_sq.txt")
+SQ_SUMMARY = os.path.join(ROOT, "profiles", "blend_knn_mlp_kernels_default_bench.pmc_sq.txt")
 
 
 # The operator whose kernels take the largest share of a step; the run checks that this is still so.

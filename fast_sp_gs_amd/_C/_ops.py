@@ -275,10 +275,11 @@ def gs_2d_compute_trans_mat_backward(W, H, means3D, scales, rotations, Tw2v, Tw2
 # --------------------------------------------------------------------------------------------------------------------
 def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, tiles_touched: Tensor,
                debug: bool = False, return_keys: bool = False, return_offsets: bool = False,
-               overlap=None) -> List[Tensor]:
+               overlap=None, records: Optional[Tensor] = None) -> List[Tensor]:
     """gaussian_prepare.cu:282-308 -> [ranges[T,2] int64, point_list[R] int32] (+ sorted keys, + the prefix scan of
     tiles_touched, which GS_2D_render_backward can use to sum gradients without atomics). `overlap(offsets)`, if given,
-    is called once the scan is queued and before the host waits for the instance count; its result is appended."""
+    is called once the scan is queued and before the host waits for the instance count; its result is appended.
+    `records` (gs_2d_preprocess_forward(..., return_records=True)): the scan stores every surfel's offset into its record."""
     what = 'GS_prepare'
     _f32(what, means2D=means2D, depths=depths)
     L.require_cuda(what, radii=radii, tiles_touched=tiles_touched)
@@ -286,6 +287,9 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
     L.require_dtype(what, 'tiles_touched', tiles_touched, torch.int32)
     P = means2D.shape[0]
     dev = means2D.device
+    if records is not None:
+        _f32(what, records=records)
+        L.require_shape(what, 'records', records, P, 20)
     lib = _lib()
     stream = L.current_stream()
     T = ((W + _TILE - 1) // _TILE) * ((H + _TILE - 1) // _TILE)
@@ -299,7 +303,7 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
     # the device works while the host waits for the copy and allocates.
     with _timed('gs_prepare_scan'):
         rc = lib.fsgs_gs_prepare_scan_begin(P, L.ptr(tiles_touched), L.ptr(offsets), L.ptr(ws1), ws1.numel(),
-                                            count.data_ptr(), stream)
+                                            count.data_ptr(), L.ptr(records), stream)
     L.check(rc, what)
     with _timed('gs_prepare_fill'):  # first of the operator's two parts: callers that time stages add them up
         rc = lib.fsgs_gs_prepare_count(P, W, H, L.ptr(means2D), L.ptr(radii), L.ptr(ranges), L.ptr(large_count), stream)

@@ -82,9 +82,12 @@ __global__ void __launch_bounds__(kScanThreads) scan_block_sums_kernel(int P, co
   if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
 }
 
+// records (optional): the blend kernels' packed per-surfel records ([P][20] floats); the surfel's exclusive offset goes
+// into the last word of its record, so the blend backward finds it in the record it gathers anyway.
 __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(int P, const int32_t* __restrict__ in,
                                                                   const int64_t* __restrict__ block_sums,
-                                                                  int64_t* __restrict__ out) {
+                                                                  int64_t* __restrict__ out,
+                                                                  float* __restrict__ records) {
   __shared__ int64_t s_wave[kScanThreads / kWave];
   const int base = blockIdx.x * kScanChunk + threadIdx.x * kScanItems;
   int32_t v[kScanItems];
@@ -104,6 +107,7 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(int P, const i
   int64_t run = chunk_start + block_exclusive_scan<int64_t>(sum, s_wave, total);
 #pragma unroll
   for (int k = 0; k < kScanItems; ++k) {
+    if (records && base + k < P) records[20 * (size_t) (base + k) + 19] = __int_as_float((int) run);
     run += v[k];
     if (base + k < P) out[base + k] = run;
   }
@@ -704,7 +708,8 @@ thread_local bool t_count_pending = false;  // a scan_begin of this thread has q
 }  // namespace
 
 FSGS_API int fsgs_gs_prepare_scan_begin(int P, const int32_t* tiles_touched, int64_t* point_offsets, void* workspace,
-                                        size_t workspace_bytes, int64_t* num_rendered_host, void* stream) {
+                                        size_t workspace_bytes, int64_t* num_rendered_host, float* records,
+                                        void* stream) {
   FSGS_REQUIRE(P >= 0 && num_rendered_host, "gs_prepare_scan: bad arguments");
   *num_rendered_host = 0;
   t_count_pending    = false;
@@ -721,7 +726,7 @@ FSGS_API int fsgs_gs_prepare_scan_begin(int P, const int32_t* tiles_touched, int
     int64_t* blk_sums = (int64_t*) workspace;
     hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(kScanThreads), 0, s, P, tiles_touched, blk_sums);
     hipLaunchKernelGGL(scan_apply_kernel, dim3(nb), dim3(kScanThreads), 0, s, P, tiles_touched, blk_sums,
-                       point_offsets);
+                       point_offsets, records);
     if (int rc = check_launch("gs_prepare_scan")) return rc;
     // The number of (surfel, tile) instances sizes the caller's output, so it has to reach the host
     // (the reference blocks for it, gaussian_prepare.cu:238-239).
@@ -744,7 +749,7 @@ FSGS_API int fsgs_gs_prepare_scan_end(void) {
 FSGS_API int fsgs_gs_prepare_scan(int P, const int32_t* tiles_touched, int64_t* point_offsets, void* workspace,
                                   size_t workspace_bytes, int64_t* num_rendered_host, void* stream) {
   if (int rc = fsgs_gs_prepare_scan_begin(P, tiles_touched, point_offsets, workspace, workspace_bytes,
-                                          num_rendered_host, stream))
+                                          num_rendered_host, nullptr, stream))
     return rc;
   return fsgs_gs_prepare_scan_end();
 }

@@ -39,6 +39,7 @@ constexpr int kRecordFloats = 20;
 
 struct SplatExtra {
   int radius;
+  int64_t offset;  // exclusive prefix-scan offset of the surfel's instances; -1 until the binning's scan has stored it
 };
 
 __device__ __forceinline__ Splat gather_splat(int id, const float2* __restrict__ means2D,
@@ -56,7 +57,7 @@ __device__ __forceinline__ Splat gather_splat(int id, const float2* __restrict__
     s.cold.nx = q3.x, s.cold.ny = q3.y, s.cold.nz = q3.z, s.cold.r = q3.w;
     s.cold.g = q4.x, s.cold.b = q4.y;
     s.cold.id = id, s.cold.pad = 0;
-    if (extra) extra->radius = __float_as_int(q4.z);
+    if (extra) extra->radius = __float_as_int(q4.z), extra->offset = (int64_t) __float_as_int(q4.w);
     return s;
   }
   const float* M = trans_mat + 9 * (size_t) id;

@@ -142,8 +142,9 @@ blend_backward_kernel(
 #pragma unroll
       for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
     if (kSlots) {
+      // a record carries the surfel's radius and, once the binning's scan has stored it, its offset (-1 until then)
       next_radius = records ? ex.radius : radii[next.cold.id];
-      next_off    = next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1];
+      next_off    = records && ex.offset >= 0 ? ex.offset : (next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1]);
     }
   }
 
@@ -176,7 +177,7 @@ blend_backward_kernel(
         for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
       if (kSlots) {
         next_radius = records ? ex.radius : radii[next.cold.id];
-        next_off    = next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1];
+        next_off    = records && ex.offset >= 0 ? ex.offset : (next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1]);
       }
     }
 

@@ -195,7 +195,7 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
       r[1] = make_float4(M[4], M[5], M[6], M[7]);
       r[2] = make_float4(M[8], c2[0], c2[1], op);
       r[3] = make_float4(nrm[0], nrm[1], nrm[2], col[0]);
-      r[4] = make_float4(col[1], col[2], __int_as_float(f2i_sat(radius)), 0.0f);
+      r[4] = make_float4(col[1], col[2], __int_as_float(f2i_sat(radius)), __int_as_float(-1));  // offset: not known yet
     } else {
 #pragma unroll
       for (int k = 0; k < 5; ++k) r[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);

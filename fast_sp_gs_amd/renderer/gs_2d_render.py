@@ -72,7 +72,7 @@ class _GS_2D_Render(torch.autograd.Function):
             W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c,
             campos, trans_precomp, means2D, culling, return_records=True)
         tile_range, point_list, point_offsets = GS_prepare(
-            W, H, means2D, depths, radii, tiles_touched, False, return_offsets=True)
+            W, H, means2D, depths, radii, tiles_touched, False, return_offsets=True, records=records)
         pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib = _GS_2D_Render._render_forward(
             W, H, means2D, colors, normal_opacity, trans_mat, point_list, tile_range, near_n, far_n, only_image,
             transe_mat_t2, accum_max_count, accum_weights_p, accum_weights_count, records)
@@ -221,7 +221,7 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
         W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs, None,
         cam.Tw2v, cam.Tv2c, cam.campos, None, None, None, return_records=packed)
     rec = rec[0] if packed else None
-    ranges, point_list, offsets = f('GS_prepare')(W, H, m2, depths, radii, tt, False, return_offsets=True)
+    ranges, point_list, offsets = f('GS_prepare')(W, H, m2, depths, radii, tt, False, return_offsets=True, records=rec)
     oc, oo, oe, of, nc = f('GS_2D_render_forward')(W, H, m2, colors, no, tm, point_list, ranges, cam.near, cam.far,
                                                    False, None, None, None, None, rec)
     epilogue = {}

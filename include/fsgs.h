@@ -82,9 +82,11 @@ int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, const float*
  * host thread). Work queued on the stream in between runs while the host waits and allocates: fsgs_gs_prepare_count is
  * the part of the fill that does not need the count (zeroes ranges[T,2], counts the instances per tile, scans them,
  * resets *large_count, a device int32 the caller keeps until the fill has run); fsgs_gs_prepare_fill_counted is the rest
- * (scatter + per-tile sort). scan_begin + scan_end == fsgs_gs_prepare_scan, count + fill_counted == fsgs_gs_prepare_fill. */
+ * (scatter + per-tile sort). scan_begin + scan_end == fsgs_gs_prepare_scan, count + fill_counted == fsgs_gs_prepare_fill.
+ * records (optional): the packed per-surfel records fsgs_gs_2d_preprocess_forward wrote; the scan stores every surfel's
+ * exclusive offset into the last word of its record, where the blend backward's ordered-sum path looks for it. */
 int fsgs_gs_prepare_scan_begin(int P, const int32_t* tiles_touched, int64_t* point_offsets, void* workspace,
-                               size_t workspace_bytes, int64_t* num_rendered_host, void* stream);
+                               size_t workspace_bytes, int64_t* num_rendered_host, float* records, void* stream);
 int fsgs_gs_prepare_scan_end(void);
 int fsgs_gs_prepare_count(int P, int W, int H, const float* means2D, const int32_t* radii, int64_t* ranges,
                           int32_t* large_count, void* stream);
@@ -98,7 +100,9 @@ int fsgs_gs_prepare_fill_counted(int P, int W, int H, const float* means2D, cons
  * (trans_mat, means2D, opacity, normal, colour, and -- when given -- radius and prefix-scan offset) into one 80-byte
  * record, records[P,20] floats, 16-byte aligned. Passing `records` to fsgs_gs_2d_render_forward / _backward makes them
  * read one record per list entry instead of four tensors; results are identical. Pass radii here if the backward is
- * going to use its ordered-sum path (it takes the radius from the record; the offset field is stored but not read).
+ * going to use its ordered-sum path (it takes the radius from the record, and the offset too when point_offsets is
+ * given here or fsgs_gs_prepare_scan_begin has stored it; a record without an offset holds -1 there and the backward
+ * falls back to its point_offsets argument).
  * fsgs_gs_2d_preprocess_forward writes the same record itself when given a records buffer; this entry serves callers
  * whose per-surfel tensors come from elsewhere. */
 int fsgs_gs_2d_pack_records(int P, const float* means2D, const float* colors, const float* normal_opacity,

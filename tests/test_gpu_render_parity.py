@@ -156,3 +156,31 @@ def test_topk_weights(device, oracle_mod):
         # an index may differ only where two candidate weights are equal to rounding (then the two slots swap)
         assert mism.mean() < 1e-3
         assert (np.abs(gw - rw)[mism] < 1e-4).all()
+
+
+def test_packed_records_with_and_without_the_scan_offset(device):
+    """The blend backward's ordered-sum path finds a surfel's scan offset in its packed record once the binning's scan
+    has stored it there, and in point_offsets otherwise (a record straight from the preprocess holds -1): same records,
+    same sums, bit for bit -- also against the four-tensor gathers."""
+    from fast_sp_gs_amd._C import get_C_function as f
+    scene, cam = _make("partial_tiles_511x127", device)
+    s, c = scene.to(device), cam.to(device)
+    W, H = cam.W, cam.H
+    gi, ge, go = (scene.extra[k].to(device) for k in ('grad_image', 'grad_extras', 'grad_opacity'))
+    m2, colors, tm, no, depths, radii, tt, rec = f('gs_2d_preprocess_forward')(
+        W, H, 3, False, s.means3D, s.scales, s.rotations, s.opacities, s.shs, None, c.Tw2v, c.Tv2c, c.campos, None, None,
+        None, return_records=True)
+    plain = rec.clone()
+    assert bool((plain[:, 19].view(torch.int32) == -1)[radii > 0].all())
+    ranges, pl, offsets = f('GS_prepare')(W, H, m2, depths, radii, tt, False, return_offsets=True, records=rec)
+    seen = radii > 0
+    want = torch.cat([offsets.new_zeros(1), offsets[:-1]]).to(torch.int32)
+    assert torch.equal(rec[:, 19].view(torch.int32)[seen], want[seen]) and torch.equal(rec[:, :19], plain[:, :19])
+    oc, oo, oe, _, nc = f('GS_2D_render_forward')(W, H, m2, colors, no, tm, pl, ranges, cam.near, cam.far, False, None,
+                                                  None, None, None, rec)
+    bwd = lambda r: f('GS_2D_render_backward')(m2, no, colors, tm, None, oo, oe, None, gi, go, ge, None, ranges, pl, nc,
+                                               cam.near, cam.far, offsets, radii, r)
+    a, b, c0 = bwd(rec), bwd(plain), bwd(None)
+    torch.cuda.synchronize()
+    for x, y, z in zip(a, b, c0):
+        assert torch.equal(x, y) and torch.equal(x, z) and bool(x.any())
