@@ -18,6 +18,7 @@
 #include <algorithm>
 
 #include "binning.hpp"
+#include "blend.hpp"
 
 namespace fsgs {
 namespace {
@@ -436,11 +437,13 @@ constexpr int kLargeSegment = 16384;  // entries sorted by a 1024-lane block in 
 
 // One block per tile: segments up to kSmallSegment entries are sorted in LDS, longer ones are queued for
 // tile_sort_large_kernel; empty tiles get the (0, 0) range the reference's zero-initialised output has.
+// `order` (optional): the blend kernels' blockIdx -> tile table, longest lists first, so that the long segments start
+// sorting at once instead of wherever the image puts them in tile order (the launch ends with its slowest block).
 __global__ void __launch_bounds__(256) tile_sort_small_kernel(int64_t* __restrict__ ranges,
     const uint64_t* __restrict__ entries, int32_t* __restrict__ point_list, int64_t* __restrict__ keys_out,
-    int* __restrict__ large_count, int* __restrict__ large_list) {
+    int* __restrict__ large_count, int* __restrict__ large_list, const int* __restrict__ order) {
   __shared__ uint64_t s_e[kSmallSegment + kSmallSegment / 4];
-  const int tile = blockIdx.x;
+  const int tile = order ? order[blockIdx.x] : (int) blockIdx.x;
   const int64_t start = ranges[2 * (size_t) tile];
   const int64_t len   = ranges[2 * (size_t) tile + 1] - start;
   if (len == 0) {
@@ -805,8 +808,12 @@ int fill_sort(int P, int W, int H, const float* means2D, const float* depths, co
   else
     hipLaunchKernelGGL(tile_emit_kernel<true>, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
                        (const float2*) means2D, depths, radii, rng, entries);
+  // The ranges are final here: the schedule table the blend kernels of this frame are going to use is built now (they
+  // find it under this ranges buffer's key) and orders the per-tile sorts as well.
+  const int* order = nullptr;
+  (void) launch_tile_order(gx, gy, ranges, s, &order);
   hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
-                     large_count, large_list);
+                     large_count, large_list, order);
   hipLaunchKernelGGL(tile_sort_large_kernel, dim3(256), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,
                      large_count, large_list);
   return check_launch("gs_prepare_fill");
