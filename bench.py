@@ -562,6 +562,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the fast-path and dynamic-step side measurements")
+    ap.add_argument("--counter-run", action="store_true",
+                    help="the process runs under a counter collection: every dispatch then carries the profiler's "
+                         "serialisation, so the operator with the most launches looks largest; do not stop on that")
     ap.add_argument("--surfels", type=int, default=300_000)
     ap.add_argument("--size", type=int, default=800)
     args = ap.parse_args()
@@ -635,7 +638,7 @@ def main():
     # twice per step and its parts are added
     stage_avg = {k: float(np.sum(v)) / stage_steps for k, v in stage_ms.items()}
     dominant = max(stage_avg, key=stage_avg.get)
-    if dominant != DOMINANT:
+    if dominant != DOMINANT and not args.counter_run:
         raise RuntimeError(f"the dominant stage is {dominant}, not {DOMINANT}: bracket that one in the timed region")
     stage_avg[dominant] = dominant_ms  # the figure from the timed region itself
     bytes_dom = algorithmic_bytes(dominant, P, Pv, R, T, HW)
