@@ -372,6 +372,9 @@ __device__ __forceinline__ float cross_row_sum(float z) {
 // v[lane & 15].
 // On return lane l of every 16-lane row holds that ROW's total of v[l & 15].
 __device__ __forceinline__ float row_sum16_transposed(const float (&v)[16]) {
+  // no contraction: an input that is a product would otherwise be formed twice, as a multiply for the shifted operand
+  // and again inside a fused multiply-add for the lane's own, in place of one multiply and one DPP add
+#pragma clang fp contract(off)
   const int lane = __lane_id();
   const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4, b3 = lane & 8;
   float w[8], x[4], y[2];

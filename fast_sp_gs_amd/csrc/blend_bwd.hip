@@ -187,95 +187,99 @@ blend_backward_kernel(
      const int jj = chunk * kWave + lane;
      unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u) &&
                                         (n_todo - 1 - (b * kBwdBatch + jj)) < wave_max_contrib);
-     // Gradient of one (pixel, entry) pair that blends: advances the pixel's back-to-front state and fills the 16 + 2
-     // per-surfel components. `j` (staging slot) and `pos` (list position) may differ between the rows of a wavefront.
-     auto pair_gradients = [&](const SplatHot& hot, const SplatCold& cold, int j, int pos, const Hit& h, float (&g)[16],
-                               float& g2x, float& g2y, bool& filtered) {
-       T             = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
-       const float w = h.alpha * T;
-       // All channels that enter the image linearly (colour, depth, opacity, normal) share one back-to-front
-       // recurrence: with c = <upstream gradient, channel values of this surfel>, the reference's per-channel
-       // accumulators acc_x = last_alpha * last_x + (1 - last_alpha) * acc_x contract to a single scalar.
-       float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
-       g[0] = w * dLp0, g[1] = w * dLp1, g[2] = w * dLp2;
-
-       float dL_dalpha = 0.0f, dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f;
-       if (kAux) {
-         const float rd     = __builtin_amdgcn_rcpf(h.depth);
-         const float m_d    = far_scale * (1.0f - near_n * rd);
-         const float dmd_dd = far_scale * near_n * rd * rd;
-         if (pos == median_contrib - 1) dL_dz += dL_dmedian;
-         const float dL_dweight = (final_D2 + m_d * m_d * final_A - 2.0f * m_d * final_D) * dL_dreg;
-         dL_dalpha += dL_dweight - last_dL_dT;
-         last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
-         const float dL_dmd = 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg;
-         dL_dz += dL_dmd * dmd_dd;
-         c_lin += h.depth * dL_ddepth + dL_daccum + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
-         g[12] = w * dLn0, g[13] = w * dLn1, g[14] = w * dLn2;
-         dL_dz += w * dL_ddepth;
-         dsx = dL_dz * hot.m[6], dsy = dL_dz * hot.m[7];
-       }
-       acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
-       last_lin = c_lin;
-       dL_dalpha += c_lin - acc_lin;
-       if (kFlow) {
-         const float* Q = &s_t2[j * 9];
-         const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
-         const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
-         float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
-         w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
-         acc_f0 = last_alpha * last_f0 + (1.0f - last_alpha) * acc_f0;
-         acc_f1 = last_alpha * last_f1 + (1.0f - last_alpha) * acc_f1;
-         last_f0 = u2 / w2 - pxf, last_f1 = v2 / w2 - pyf;
-         dL_dalpha += (last_f0 - acc_f0) * dLf0 + (last_f1 - acc_f1) * dLf1;
-         const float gu = w / w2 * dLf0, gv = w / w2 * dLf1;
-         const float gw = -w / (w2 * w2) * (u2 * dLf0 + v2 * dLf1);
-         dsx += Q[0] * gu + Q[3] * gv + Q[6] * gw;
-         dsy += Q[1] * gu + Q[4] * gv + Q[7] * gw;
-         acc_w = last_alpha + (1.0f - last_alpha) * acc_w;
-         dL_dalpha += (1.0f - acc_w) * dL_dsum_w;
-       }
-       dL_dalpha *= T;
-       last_alpha = h.alpha;
-
-       const float dL_dG = hot.opacity * dL_dalpha;
-       if (h.rho3d <= h.rho2d) {
+     // Gradient terms of one (pixel, entry) pair. The part under `hit` advances the pixel's back-to-front state and
+     // leaves five factors (zero for a lane whose pixel does not blend the entry); the 16 + 2 per-surfel components
+     // are products of those factors with quantities that are finite in every lane, formed by all lanes alike, so no
+     // component needs a zero of its own and the two ways a surfel is met (ray-splat intersection / projected
+     // centre) share one instruction stream: the projected-centre case is the intersection case with a zero in place
+     // of 1 / p_z. `j` (staging slot) and `pos` (list position) may differ between the rows of a wavefront.
+     auto pair_gradients = [&](const SplatHot& hot, const SplatCold& cold, int j, int pos, const Hit& h, bool hit,
+                               float (&g)[16], float& g2x, float& g2y, bool& filtered) {
+       float w = 0.0f, dL_dalpha = 0.0f, dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f, s_ds = 0.0f, z_sx = 0.0f, z_sy = 0.0f;
+       if (hit) {
+         T = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+         w = h.alpha * T;
+         // All channels that enter the image linearly (colour, depth, opacity, normal) share one back-to-front
+         // recurrence: with c = <upstream gradient, channel values of this surfel>, the reference's per-channel
+         // accumulators acc_x = last_alpha * last_x + (1 - last_alpha) * acc_x contract to a single scalar.
+         float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
+         if (kAux) {
+           const float rd     = __builtin_amdgcn_rcpf(h.depth);
+           const float m_d    = far_scale * (1.0f - near_n * rd);
+           const float dmd_dd = far_scale * near_n * rd * rd;
+           if (pos == median_contrib - 1) dL_dz += dL_dmedian;
+           const float dL_dweight = (final_D2 + m_d * m_d * final_A - 2.0f * m_d * final_D) * dL_dreg;
+           dL_dalpha += dL_dweight - last_dL_dT;
+           last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
+           const float dL_dmd = 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg;
+           dL_dz += dL_dmd * dmd_dd;
+           c_lin += h.depth * dL_ddepth + dL_daccum + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
+           dL_dz += w * dL_ddepth;
+           dsx = dL_dz * hot.m[6], dsy = dL_dz * hot.m[7];
+         }
+         acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
+         last_lin = c_lin;
+         dL_dalpha += c_lin - acc_lin;
+         if (kFlow) {
+           const float* Q = &s_t2[j * 9];
+           const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
+           const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
+           float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
+           w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
+           acc_f0 = last_alpha * last_f0 + (1.0f - last_alpha) * acc_f0;
+           acc_f1 = last_alpha * last_f1 + (1.0f - last_alpha) * acc_f1;
+           last_f0 = u2 / w2 - pxf, last_f1 = v2 / w2 - pyf;
+           dL_dalpha += (last_f0 - acc_f0) * dLf0 + (last_f1 - acc_f1) * dLf1;
+           const float gu = w / w2 * dLf0, gv = w / w2 * dLf1;
+           const float gw = -w / (w2 * w2) * (u2 * dLf0 + v2 * dLf1);
+           dsx += Q[0] * gu + Q[3] * gv + Q[6] * gw;
+           dsy += Q[1] * gu + Q[4] * gv + Q[7] * gw;
+           acc_w = last_alpha + (1.0f - last_alpha) * acc_w;
+           dL_dalpha += (1.0f - acc_w) * dL_dsum_w;
+         }
+         dL_dalpha *= T;
+         last_alpha = h.alpha;
+         // the Gaussian's own part of d/ds: only the intersection case uses it (times 1 / p_z below)
+         const float dL_dG = hot.opacity * dL_dalpha;
          dsx += dL_dG * -h.G * h.sx;
          dsy += dL_dG * -h.G * h.sy;
-         const float rz  = __builtin_amdgcn_rcpf(h.pz);
-         const float dpx = dsx * rz, dpy = dsy * rz;
-         const float dpz = -(dpx * h.sx + dpy * h.sy);
-         const float dkx = h.ly * dpz - h.lz * dpy, dky = h.lz * dpx - h.lx * dpz, dkz = h.lx * dpy - h.ly * dpx;
-         const float dlx = dpy * h.kz - dpz * h.ky, dly = dpz * h.kx - dpx * h.kz, dlz = dpx * h.ky - dpy * h.kx;
-         g[3] = -dkx, g[4] = -dky, g[5] = -dkz;
-         g[6] = -dlx, g[7] = -dly, g[8] = -dlz;
-         g[9]  = pxf * dkx + pyf * dlx + dL_dz * h.sx;
-         g[10] = pxf * dky + pyf * dly + dL_dz * h.sy;
-         g[11] = pxf * dkz + pyf * dlz + dL_dz;
-       } else {
-         g2x   = dL_dG * (-h.G * 2.0f * h.dx);
-         g2y   = dL_dG * (-h.G * 2.0f * h.dy);
-         g[9]  = dL_dz * h.sx;
-         g[10] = dL_dz * h.sy;
-         g[11] = dL_dz;
-         filtered = true;
+         // s is not finite in a lane whose plane pair degenerates (p_z == 0), and such a lane never blends: every use
+         // of s sits on this side
+         s_ds = dsx * h.sx + dsy * h.sy;
+         z_sx = dL_dz * h.sx, z_sy = dL_dz * h.sy;
        }
+       const bool by_ray = h.rho3d <= h.rho2d;
+       filtered          = hit && !by_ray;
+       // d/dp of the homogeneous intersection point p = k x l, negated (the components below are minus the plane
+       // gradients): p_xy = s p_z, so dp_xy = ds / p_z and dp_z = -<ds, s> / p_z
+       const float rz  = (hit && by_ray) ? __builtin_amdgcn_rcpf(h.pz) : 0.0f;
+       const float npx = -(dsx * rz), npy = -(dsy * rz), npz = s_ds * rz;
+       const float nkx = h.ly * npz - h.lz * npy, nky = h.lz * npx - h.lx * npz, nkz = h.lx * npy - h.ly * npx;
+       const float nlx = npy * h.kz - npz * h.ky, nly = npz * h.kx - npx * h.kz, nlz = npx * h.ky - npy * h.kx;
+       g[0] = w * dLp0, g[1] = w * dLp1, g[2] = w * dLp2;
+       g[3] = nkx, g[4] = nky, g[5] = nkz;
+       g[6] = nlx, g[7] = nly, g[8] = nlz;
+       g[9]  = z_sx - (pxf * nkx + pyf * nlx);
+       g[10] = z_sy - (pxf * nky + pyf * nly);
+       g[11] = dL_dz - (pxf * nkz + pyf * nlz);
+       if (kAux) g[12] = w * dLn0, g[13] = w * dLn1, g[14] = w * dLn2;
+       else      g[12] = g[13] = g[14] = 0.0f;
        g[15] = h.G * dL_dalpha;
-           };
+       const float to_centre = filtered ? hot.opacity * dL_dalpha * (-2.0f * h.G) : 0.0f;
+       g2x = to_centre * h.dx, g2y = to_centre * h.dy;
+     };
      auto backward_entry = [&](const SplatHot& hot, const SplatCold& cold, int j) {
       const int pos = n_todo - 1 - (b * kBwdBatch + j);  // 0-based position in the tile's list
       Hit h;
       const bool hit = intersect_flat(hot, pxf, pyf, near_n, h) && (pos < last_contrib);
-      if (__ballot(hit) == 0ull) return;  // wave-uniform: nobody in this quadrant blends the surfel
+      if (wave_ballot(hit) == 0ull) return;  // wave-uniform: nobody in this quadrant blends the surfel
 
-      float g[16], g2x = 0.0f, g2y = 0.0f;
-      bool filtered = false;
-#pragma unroll
-      for (int c = 0; c < 16; ++c) g[c] = 0.0f;
-      if (hit) pair_gradients(hot, cold, j, pos, h, g, g2x, g2y, filtered);
+      float g[16], g2x, g2y;
+      bool filtered;
+      pair_gradients(hot, cold, j, pos, h, hit, g, g2x, g2y, filtered);
       const float tot = wave_sum16_transposed(g);
       if (lane < 16) s_part[wave][j][lane] = tot;  // a wavefront meets an entry once per batch: a plain store
-      if (__ballot(filtered) != 0ull) {
+      if (wave_ballot(filtered) != 0ull) {
         const float sx = wave_sum_to_lane63(g2x), sy = wave_sum_to_lane63(g2y);
         if (lane == 63) s_part[wave][j][16] = sx, s_part[wave][j][17] = sy;
       }
@@ -333,14 +337,12 @@ blend_backward_kernel(
         const int pos = n_todo - 1 - (b * kBwdBatch + j);
         Hit h;
         const bool hit = intersect_flat(hot, pxf, pyf, near_n, h) && (pos < last_contrib) && active;
-        float g[16], g2x = 0.0f, g2y = 0.0f;
-        bool filtered = false;
-#pragma unroll
-        for (int c = 0; c < 16; ++c) g[c] = 0.0f;
-        if (hit) pair_gradients(hot, cold, j, pos, h, g, g2x, g2y, filtered);
+        float g[16], g2x, g2y;
+        bool filtered;
+        pair_gradients(hot, cold, j, pos, h, hit, g, g2x, g2y, filtered);
         const float tot = row_sum16_transposed(g);  // lane (row, c): the row's total of component c
         if (active) atomicAdd(&s_part[wave][j][lane & 15], tot);
-        if (__ballot(filtered) != 0ull) {
+        if (wave_ballot(filtered) != 0ull) {
           float sx = g2x, sy = g2y;  // totals of the row end up in its lane 15
           sx += dpp_shift_zero<0x111, 0xf, 0xf>(sx), sy += dpp_shift_zero<0x111, 0xf, 0xf>(sy);
           sx += dpp_shift_zero<0x112, 0xf, 0xf>(sx), sy += dpp_shift_zero<0x112, 0xf, 0xf>(sy);

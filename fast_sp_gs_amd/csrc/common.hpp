@@ -53,6 +53,10 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Mask of the lanes where `b` holds, straight from the comparison's lane mask: HIP's __ballot takes an int, which makes
+// the compiler materialise the predicate in a register and compare it again.
+__device__ __forceinline__ unsigned long long wave_ballot(bool b) { return __builtin_amdgcn_ballot_w64(b); }
+
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 // float -> int with saturation and NaN -> 0 (what v_cvt_i32_f32 does; spelled out so the result does not depend on
