@@ -127,7 +127,11 @@ __device__ __forceinline__ bool intersect(const SplatHot& h, float pxf, float py
 // the caller gets one predicate instead of nested divergent regions. Contraction is switched off and every fused
 // multiply-add is written out, so that each inlined copy of this function rounds alike (a kernel that instantiates it
 // twice must not depend on which copy evaluated a surfel).
-__device__ __forceinline__ bool intersect_flat(const SplatHot& h, float pxf, float pyf, float near_n, Hit& o) {
+// `lanes`, if given, receives the mask of the lanes that pass, as the AND of the four comparisons' own lane masks: a
+// wave-uniform "does any lane pass" then stays in scalar registers (the ballot of a combined predicate is rebuilt by
+// the compiler from a 0 / 1 register, two vector instructions and their latency on the entry's critical path).
+__device__ __forceinline__ bool intersect_flat(const SplatHot& h, float pxf, float pyf, float near_n, Hit& o,
+                                               unsigned long long* lanes = nullptr) {
 #pragma clang fp contract(off)
   o.kx = fmaf(pxf, h.m[6], -h.m[0]), o.ky = fmaf(pxf, h.m[7], -h.m[1]), o.kz = fmaf(pxf, h.m[8], -h.m[2]);
   o.lx = fmaf(pyf, h.m[6], -h.m[3]), o.ly = fmaf(pyf, h.m[7], -h.m[4]), o.lz = fmaf(pyf, h.m[8], -h.m[5]);
@@ -144,7 +148,9 @@ __device__ __forceinline__ bool intersect_flat(const SplatHot& h, float pxf, flo
   const float power = -0.5f * rho;
   o.G     = __expf(power);
   o.alpha = fminf(0.99f, h.opacity * o.G);
-  return (o.pz != 0.0f) & !(o.depth < near_n) & !(power > 0.0f) & !(o.alpha < (1.0f / 255.0f));
+  const bool c0 = o.pz != 0.0f, c1 = !(o.depth < near_n), c2 = !(power > 0.0f), c3 = !(o.alpha < (1.0f / 255.0f));
+  if (lanes) *lanes = wave_ballot(c0) & wave_ballot(c1) & wave_ballot(c2) & wave_ballot(c3);
+  return c0 & c1 & c2 & c3;
 }
 
 // ---- conservative per-quadrant culling ------------------------------------------------------------------------------
@@ -301,6 +307,7 @@ __device__ __forceinline__ float dpp_shift_zero(float v) {
 
 // Sum over the 64 lanes; the total is valid in lane 63 only.
 __device__ __forceinline__ float wave_sum_to_lane63(float v) {
+#pragma clang fp contract(off)  // as in row_sum16_transposed: an input product must not be formed a second time
   v += dpp_shift_zero<0x111, 0xf, 0xf>(v);  // row_shr:1
   v += dpp_shift_zero<0x112, 0xf, 0xf>(v);  // row_shr:2
   v += dpp_shift_zero<0x114, 0xf, 0xf>(v);  // row_shr:4

@@ -194,7 +194,7 @@ blend_backward_kernel(
      // centre) share one instruction stream: the projected-centre case is the intersection case with a zero in place
      // of 1 / p_z. `j` (staging slot) and `pos` (list position) may differ between the rows of a wavefront.
      auto pair_gradients = [&](const SplatHot& hot, const SplatCold& cold, int j, int pos, const Hit& h, bool hit,
-                               float (&g)[16], float& g2x, float& g2y, bool& filtered) {
+                               float (&g)[16], float& g2x, float& g2y, unsigned long long& ray_lanes) {
        float w = 0.0f, dL_dalpha = 0.0f, dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f, s_ds = 0.0f, z_sx = 0.0f, z_sy = 0.0f;
        if (hit) {
          T = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
@@ -248,8 +248,9 @@ blend_backward_kernel(
          s_ds = dsx * h.sx + dsy * h.sy;
          z_sx = dL_dz * h.sx, z_sy = dL_dz * h.sy;
        }
-       const bool by_ray = h.rho3d <= h.rho2d;
-       filtered          = hit && !by_ray;
+       const bool by_ray   = h.rho3d <= h.rho2d;
+       const bool filtered = hit && !by_ray;
+       ray_lanes           = wave_ballot(by_ray);  // taken where the comparison is made: its own lane mask, no instruction
        // d/dp of the homogeneous intersection point p = k x l, negated (the components below are minus the plane
        // gradients): p_xy = s p_z, so dp_xy = ds / p_z and dp_z = -<ds, s> / p_z
        const float rz  = (hit && by_ray) ? __builtin_amdgcn_rcpf(h.pz) : 0.0f;
@@ -271,15 +272,17 @@ blend_backward_kernel(
      auto backward_entry = [&](const SplatHot& hot, const SplatCold& cold, int j) {
       const int pos = n_todo - 1 - (b * kBwdBatch + j);  // 0-based position in the tile's list
       Hit h;
-      const bool hit = intersect_flat(hot, pxf, pyf, near_n, h) && (pos < last_contrib);
-      if (wave_ballot(hit) == 0ull) return;  // wave-uniform: nobody in this quadrant blends the surfel
+      unsigned long long pass;
+      const bool hit = intersect_flat(hot, pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
+      pass &= wave_ballot(pos < last_contrib);
+      if (pass == 0ull) return;  // wave-uniform: nobody in this quadrant blends the surfel
 
       float g[16], g2x, g2y;
-      bool filtered;
-      pair_gradients(hot, cold, j, pos, h, hit, g, g2x, g2y, filtered);
+      unsigned long long ray_lanes;
+      pair_gradients(hot, cold, j, pos, h, hit, g, g2x, g2y, ray_lanes);
       const float tot = wave_sum16_transposed(g);
       if (lane < 16) s_part[wave][j][lane] = tot;  // a wavefront meets an entry once per batch: a plain store
-      if (wave_ballot(filtered) != 0ull) {
+      if ((pass & ~ray_lanes) != 0ull) {  // some lane met the surfel by its projected centre
         const float sx = wave_sum_to_lane63(g2x), sy = wave_sum_to_lane63(g2y);
         if (lane == 63) s_part[wave][j][16] = sx, s_part[wave][j][17] = sy;
       }
@@ -338,8 +341,9 @@ blend_backward_kernel(
         Hit h;
         const bool hit = intersect_flat(hot, pxf, pyf, near_n, h) && (pos < last_contrib) && active;
         float g[16], g2x, g2y;
-        bool filtered;
-        pair_gradients(hot, cold, j, pos, h, hit, g, g2x, g2y, filtered);
+        unsigned long long ray_lanes;
+        pair_gradients(hot, cold, j, pos, h, hit, g, g2x, g2y, ray_lanes);
+        const bool filtered = hit && !((ray_lanes >> lane) & 1ull);
         const float tot = row_sum16_transposed(g);  // lane (row, c): the row's total of component c
         if (active) atomicAdd(&s_part[wave][j][lane & 15], tot);
         if (wave_ballot(filtered) != 0ull) {

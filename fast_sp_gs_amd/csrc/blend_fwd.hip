@@ -61,7 +61,12 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   const int n_todo = (int) (r1 - r0);
   const int rounds = (n_todo + kFwdBatch - 1) / kFwdBatch;
 
-  bool done = !inside;
+  // A pixel stops blending once its transmittance would fall below 1e-4. The state is a float, not a bool: the test
+  // is then one comparison whose lane mask feeds the branches directly (a bool carried round the loop lives in a
+  // register as 0 / 1 and is turned into a mask again at every use).
+  float live = inside ? 1.0f : -1.0f;
+  // the same for the wavefront, as a lane mask in scalar registers: "is anybody still blending" costs no vector work
+  unsigned long long live_lanes = wave_ballot(inside);
   const float far_scale = far_n / (far_n - near_n);
   float T = 1.0f, C0 = 0, C1 = 0, C2 = 0;
   float N0 = 0, N1 = 0, N2 = 0, D = 0, M1 = 0, M2 = 0, dist = 0, median = 0, wsum = 0, f0 = 0, f1 = 0;
@@ -94,7 +99,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
 
   for (int b = 0; b < rounds; ++b) {
     // everyone has finished reading the previous batch; leave as soon as no pixel of the tile is still blending
-    if (__syncthreads_count(done) == kBlendThreads) break;
+    if (__syncthreads_count(live < 0.0f) == kBlendThreads) break;
     const int n_here = min(kFwdBatch, n_todo - b * kFwdBatch);
     if ((int) threadIdx.x < n_here) {
       s_hot[threadIdx.x]  = next.hot;
@@ -127,14 +132,17 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
       auto blend_entry = [&](const SplatHot& hot, const SplatCold& cold, int j) {
 #pragma clang fp contract(off)  // two copies of this body exist (alternating registers): both must round alike
         Hit h;
-        const bool hit = intersect_flat(hot, pxf, pyf, near_n, h) && !done;
-        if (__ballot(hit) == 0ull) return;
+        unsigned long long pass;
+        const bool hit = intersect_flat(hot, pxf, pyf, near_n, h, &pass) && live > 0.0f;
+        pass &= live_lanes;
+        if (pass == 0ull) return;
         const float test_T = T * (1.0f - h.alpha);
         const bool sat     = hit && test_T < 0.0001f;
-        done               = done || sat;
+        live               = sat ? -1.0f : live;
+        live_lanes &= ~(pass & wave_ballot(test_T < 0.0001f));
         const float w      = h.alpha * T;
         if (kAccum == 2) {
-          const unsigned long long who = __ballot(hit && !sat);
+          const unsigned long long who = wave_ballot(hit && !sat);
           if (who != 0ull) {
             s_accw[(wave * kAccSlots + acc_slot) * kAccStride + lane] = hit && !sat ? w : 0.0f;
             if (lane == 0) s_accid[wave * kAccSlots + acc_slot] = cold.id, s_accn[wave * kAccSlots + acc_slot] = (int) __popcll(who);
@@ -178,7 +186,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
       auto peek = [&]() { return c * kWave + (todo ? __builtin_ctzll(todo) : 0); };
       SplatHot hot_a = s_hot[peek()], hot_b;
       while (todo) {
-        if (__ballot(!done) == 0ull) break;  // every pixel of this quadrant is saturated
+        if (live_lanes == 0ull) break;  // every pixel of this quadrant is saturated
         {
           const int j = pop();
           hot_b       = s_hot[peek()];
@@ -186,7 +194,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
           __builtin_amdgcn_sched_barrier(0);
           blend_entry(hot_a, cold, j);
         }
-        if (todo == 0ull || __ballot(!done) == 0ull) break;
+        if (todo == 0ull || live_lanes == 0ull) break;
         {
           const int j = pop();
           hot_a       = s_hot[peek()];
