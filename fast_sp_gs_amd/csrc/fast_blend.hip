@@ -74,7 +74,9 @@ struct FastHit {
 // Written without early exits: every lane runs the whole sequence and the rejections (behind the camera plane, nearer
 // than `near`, positive exponent, alpha < 1/255) are combined into one predicate at the end, so the callers have one
 // divergent region instead of a nest of them on their per-entry critical path.
-__device__ __forceinline__ bool fast_intersect_flat(const FastHot& h, float pxf, float pyf, float near_n, FastHit& o) {
+// `lanes`, if given: mask of the lanes that pass, from the four comparisons' own lane masks (scalar registers).
+__device__ __forceinline__ bool fast_intersect_flat(const FastHot& h, float pxf, float pyf, float near_n, FastHit& o,
+                                                    unsigned long long* lanes = nullptr) {
   const float p0 = h.a[0] * pxf + h.a[1] * pyf + h.a[2];
   const float p1 = h.a[3] * pxf + h.a[4] * pyf + h.a[5];
   o.pz           = h.a[6] * pxf + h.a[7] * pyf + h.a[8];
@@ -88,7 +90,9 @@ __device__ __forceinline__ bool fast_intersect_flat(const FastHot& h, float pxf,
   const float power = -0.5f * rho;
   o.G     = __expf(power);
   o.alpha = fminf(0.99f, h.opacity * o.G);
-  return (o.pz != 0.0f) & !(o.depth < near_n) & !(power > 0.0f) & !(o.alpha < (1.0f / 255.0f));
+  const bool c0 = o.pz != 0.0f, c1 = !(o.depth < near_n), c2 = !(power > 0.0f), c3 = !(o.alpha < (1.0f / 255.0f));
+  if (lanes) *lanes = wave_ballot(c0) & wave_ballot(c1) & wave_ballot(c2) & wave_ballot(c3);
+  return c0 & c1 & c2 & c3;
 }
 
 // Sums 8 per-lane values over the 64 lanes at once: three merge steps inside aligned groups of 8 lanes, one rotate by 8
@@ -157,7 +161,10 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
     if (threadIdx.x == 0) s_max_contrib = 0;
   }
 
-  bool done = !inside;
+  // blending state of the pixel (float: its test is one comparison) and of the wavefront (a lane mask in scalar
+  // registers: "is anybody still blending" costs no vector instruction)
+  float live = inside ? 1.0f : -1.0f;
+  unsigned long long live_lanes = wave_ballot(inside);
   const float far_scale = far_n / (far_n - near_n);
   float T = 1.0f, C0 = 0, C1 = 0, C2 = 0;
   float N0 = 0, N1 = 0, N2 = 0, D = 0, M1 = 0, M2 = 0, dist = 0, median = 0, f0 = 0, f1 = 0;
@@ -176,7 +183,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
   }
 
   for (int b = 0; b < rounds; ++b) {
-    if (__syncthreads_count(done) == kBlendThreads) break;
+    if (__syncthreads_count(live < 0.0f) == kBlendThreads) break;
     const int n_here = min(kBatch, n_todo - b * kBatch);
     if ((int) threadIdx.x < n_here) {
       s_hot[threadIdx.x]  = next.hot;
@@ -206,7 +213,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
         if (kSnap) {
           const int base = c * kWave + half * 32;
           if (base >= n_here) break;
-          if (!done) {
+          if (live > 0.0f) {
             // state before list entry b * 256 + base, which starts a bucket of 32 (gs_2d_fast_redner.cu:126-147)
             const size_t bk = (size_t) (bucket0 + (b * kBatch + base) / 32);
             sampled_T[bk * 256 + rank]             = T;
@@ -230,15 +237,18 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
           todo &= half ? 0xffffffff00000000ull : 0x00000000ffffffffull;
         }
         while (todo) {
-          if (__ballot(!done) == 0ull) break;
+          if (live_lanes == 0ull) break;
           const int j = c * kWave + __builtin_ctzll(todo);
           todo &= todo - 1;
           FastHit h;
-          const bool hit = fast_intersect_flat(s_hot[j], pxf, pyf, near_n, h) && !done;
-          if (__ballot(hit) == 0ull) continue;
+          unsigned long long pass;
+          const bool hit = fast_intersect_flat(s_hot[j], pxf, pyf, near_n, h, &pass) && live > 0.0f;
+          pass &= live_lanes;
+          if (pass == 0ull) continue;
           const float test_T = T * (1.0f - h.alpha);
           const bool sat     = hit && test_T < 0.0001f;
-          done               = done || sat;
+          live               = sat ? -1.0f : live;
+          live_lanes &= ~(pass & wave_ballot(test_T < 0.0001f));
           const float w         = h.alpha * T;
           const SplatCold cold  = s_cold[j];
           if (kAccum && (accum_weights_p || accum_weights_count))
@@ -460,8 +470,9 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
         todo &= todo - 1;
         const int pos = n_todo - 1 - (b * kB + j);
         FastHit h;
-        const bool hit = fast_intersect_flat(s_hot[j], pxf, pyf, near_n, h) && (pos < last_contrib);
-        if (__ballot(hit) == 0ull) continue;
+        unsigned long long pass;
+        const bool hit = fast_intersect_flat(s_hot[j], pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
+        if ((pass & wave_ballot(pos < last_contrib)) == 0ull) continue;
 
         float g[16], g8[8];
         bool filtered = false;

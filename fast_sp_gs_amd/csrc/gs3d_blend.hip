@@ -82,13 +82,17 @@ struct G3Hit {
 // Alpha of one Gaussian at one pixel (gaussian_render.cu:118-130); false where the reference would `continue`. No early
 // exit, and every fused multiply-add is written out with contraction off: a kernel that inlines this twice gets the
 // same rounding from both copies.
-__device__ __forceinline__ bool conic_alpha_flat(const G3Hot& h, float pxf, float pyf, G3Hit& o) {
+// `lanes`, if given: mask of the lanes that pass, from the two comparisons' own lane masks (scalar registers).
+__device__ __forceinline__ bool conic_alpha_flat(const G3Hot& h, float pxf, float pyf, G3Hit& o,
+                                                 unsigned long long* lanes = nullptr) {
 #pragma clang fp contract(off)
   o.dx = h.x - pxf, o.dy = h.y - pyf;
   const float power = fmaf(-0.5f, fmaf(h.a * o.dx, o.dx, h.c * o.dy * o.dy), -(h.b * o.dx * o.dy));
   o.G     = __expf(power);
   o.alpha = fminf(0.99f, h.opacity * o.G);
-  return !(power > 0.0f) & !(o.alpha < (1.0f / 255.0f));
+  const bool c0 = !(power > 0.0f), c1 = !(o.alpha < (1.0f / 255.0f));
+  if (lanes) *lanes = wave_ballot(c0) & wave_ballot(c1);
+  return c0 & c1;
 }
 
 // kSnap (gaussian_render.cu:51-63, :100-106, :168-172): the state of every pixel still blending before each 32nd list
@@ -126,7 +130,10 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
     if (threadIdx.x == 0) s_max_contrib = 0;
   }
 
-  bool done = !inside;
+  // blending state of the pixel (float: its test is one comparison) and of the wavefront (a lane mask in scalar
+  // registers: "is anybody still blending" costs no vector instruction)
+  float live = inside ? 1.0f : -1.0f;
+  unsigned long long live_lanes = wave_ballot(inside);
   float T = 1.0f, C[3 + (E > 0 ? E : 1)];
 #pragma unroll
   for (int k = 0; k < 3 + E; ++k) C[k] = 0.0f;
@@ -138,7 +145,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
   if ((int) threadIdx.x < min(n_todo, kG3Batch))
     next = gather_gaussian<E>(point_list[r0 + threadIdx.x], means2D, conic_opacity, colors, extras);
   for (int b = 0; b < rounds; ++b) {
-    if (__syncthreads_count(done) == kBlendThreads) break;
+    if (__syncthreads_count(live < 0.0f) == kBlendThreads) break;
     const int n_here = min(kG3Batch, n_todo - b * kG3Batch);
     if ((int) threadIdx.x < n_here) {
       next.hot.mask = conic_quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile, flags);
@@ -160,11 +167,14 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
       auto blend_entry = [&](const G3Hot& hot, int j) {
 #pragma clang fp contract(off)  // two copies of this body exist: both must round alike
         G3Hit h;
-        const bool hit = conic_alpha_flat(hot, pxf, pyf, h) && !done;
-        if (__ballot(hit) == 0ull) return;
+        unsigned long long pass;
+        const bool hit = conic_alpha_flat(hot, pxf, pyf, h, &pass) && live > 0.0f;
+        pass &= live_lanes;
+        if (pass == 0ull) return;
         const float test_T = T * (1.0f - h.alpha);
         const bool sat     = hit && test_T < 0.0001f;
-        done               = done || sat;
+        live               = sat ? -1.0f : live;
+        live_lanes &= ~(pass & wave_ballot(test_T < 0.0001f));
         const float w      = h.alpha * T;
         if (kAccum && (accum_weights_p || accum_weights_count))
           wave_accumulate_weights(hit && !sat, w, hot.id, accum_weights_p, accum_weights_count);
@@ -183,7 +193,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
         for (int half = 0; half < 2; ++half) {
           const int base = c * kWave + half * 32;
           if (base >= n_here) break;
-          if (!done) {
+          if (live > 0.0f) {
             const size_t bk = (size_t) (bucket0 + (b * kG3Batch + base) / 32);
             sampled_T[bk * 256 + rank] = T;
 #pragma unroll
@@ -191,7 +201,7 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
           }
           unsigned long long part = todo & (half ? 0xffffffff00000000ull : 0x00000000ffffffffull);
           while (part) {
-            if (__ballot(!done) == 0ull) break;
+            if (live_lanes == 0ull) break;
             const int j = c * kWave + __builtin_ctzll(part);
             part &= part - 1;
             blend_entry(s_hot[j], j);
@@ -207,14 +217,14 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_forward_kernel(int flags, 
       auto peek = [&]() { return c * kWave + (todo ? __builtin_ctzll(todo) : 0); };
       G3Hot hot_a = s_hot[peek()], hot_b;
       while (todo) {
-        if (__ballot(!done) == 0ull) break;
+        if (live_lanes == 0ull) break;
         {
           const int j = pop();
           hot_b       = s_hot[peek()];
           __builtin_amdgcn_sched_barrier(0);
           blend_entry(hot_a, j);
         }
-        if (todo == 0ull || __ballot(!done) == 0ull) break;
+        if (todo == 0ull || live_lanes == 0ull) break;
         {
           const int j = pop();
           hot_a       = s_hot[peek()];
@@ -423,8 +433,9 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
       todo &= todo - 1;
       const int pos = n_todo - 1 - (b * kB + j);  // 0-based position in the tile's list
       G3Hit h;
-      const bool hit = conic_alpha_flat(s_hot[j], pxf, pyf, h) && (pos < last_contrib);
-      if (__ballot(hit) == 0ull) continue;
+      unsigned long long pass;
+      const bool hit = conic_alpha_flat(s_hot[j], pxf, pyf, h, &pass) && (pos < last_contrib);
+      if ((pass & wave_ballot(pos < last_contrib)) == 0ull) continue;
       float g[16];
 #pragma unroll
       for (int c = 0; c < 16; ++c) g[c] = 0.0f;
@@ -658,8 +669,9 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_extra_backward_kernel(int 
       todo &= todo - 1;
       const int pos = n_todo - 1 - (b * kB + j);  // 0-based position in the tile's list
       G3Hit h;
-      const bool hit = conic_alpha_flat(s_hot[j], pxf, pyf, h) && (pos < last_contrib);
-      if (__ballot(hit) == 0ull) continue;
+      unsigned long long pass;
+      const bool hit = conic_alpha_flat(s_hot[j], pxf, pyf, h, &pass) && (pos < last_contrib);
+      if ((pass & wave_ballot(pos < last_contrib)) == 0ull) continue;
       float g[16];
 #pragma unroll
       for (int c = 0; c < 16; ++c) g[c] = 0.0f;
