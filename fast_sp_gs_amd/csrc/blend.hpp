@@ -207,19 +207,37 @@ __device__ __forceinline__ unsigned quadrant_mask(const SplatHot& h, int tile_px
   return m;
 }
 
-// ---- tile schedule: longest lists first, neighbouring tiles on the same XCD -----------------------------------------
-// Blocks are handed out in blockIdx order, consecutive blocks go to consecutive XCDs (8 of them, each with its own L2),
-// and a tile's cost is proportional to the length of its list. The blend kernels therefore map blockIdx -> tile through
-// a table built per launch: small square groups of tiles are dealt to 8 regions, region r owns the table positions p with
-// p % 8 == r (as long as it has tiles left), and inside a region tiles are listed by descending list length
-// (quarter-octave buckets, arbitrary order inside a bucket). Long lists start first and short ones fill the tail of the launch; a surfel
-// that overlaps several neighbouring tiles is gathered by blocks that share an L2.
+// ---- tile schedule: longest lists first, neighbouring tiles on the same XCD, equal work per CU ------------------------
+// Blocks are handed out in blockIdx order, consecutive blocks go to consecutive XCDs (8 of them, each with its own L2,
+// 32 CUs behind each), and a tile's cost is proportional to the length of its list. The blend kernels therefore map
+// blockIdx -> tile through a table built once per frame: small square groups of tiles are dealt to 8 regions, region r
+// owns the table positions p with p % 8 == r (as long as it has tiles left), and inside a region tiles are listed by
+// descending list length (1/16-octave buckets, arbitrary order inside a bucket). Long lists start first and short ones
+// fill the tail of the launch; a surfel that overlaps several neighbouring tiles is gathered by blocks that share an L2.
+// An XCD places the first blocks it receives on its CUs in turn, and as many rounds of 32 as blocks fit on a CU stay
+// there together for most of the launch: CU c works on the region's tiles number c, 32 + c, 64 + c, ... In plain
+// descending order CU 0 would get the longest tile of every round and CU 31 the shortest (15 % above the mean for the
+// chord-length profile of a ball of surfels), and the launch lasts as long as its busiest CU. Inside each of the first
+// rounds the tiles are therefore dealt by load: the CU with the least work so far gets the round's longest tile.
+// Later rounds go wherever a slot frees up; for them descending order is what balances.
 // The table is a device buffer of kMaxOrderedTiles ints owned by the library, one per (device, stream) a blend entry
 // point has been called on (allocated on the first such call, kept until the process ends): calls on one stream are
 // ordered by the stream, calls on different streams use different tables.
+#ifndef FSGS_ORDER_FRAC_BITS
+#define FSGS_ORDER_FRAC_BITS 4
+#endif
+#ifndef FSGS_ORDER_BALANCE_ROUNDS
+#define FSGS_ORDER_BALANCE_ROUNDS 4
+#endif
 constexpr int kMaxOrderedTiles = 1 << 16;
-constexpr int kOrderBuckets    = 128;
+constexpr int kOrderFracBits   = FSGS_ORDER_FRAC_BITS;  // buckets per octave of list length = 2^this
+constexpr int kOrderFrac       = 1 << kOrderFracBits;
+constexpr int kOrderBuckets    = 32 * kOrderFrac;
 constexpr int kOrderRegions    = 8;
+constexpr int kCusPerXcd       = 32;  // compute units behind one region's table positions
+// rounds of a region's list whose tiles are dealt by CU load: the blocks of the blend backward that fit on a CU (4,
+// bounded by its 128 registers per lane); measured best among 3, 4, 5, 6, 8, 16
+constexpr int kBalanceRounds   = FSGS_ORDER_BALANCE_ROUNDS;
 
 // (TileOrderState, tile_order_state and tile_order_invalidate are declared in common.hpp.)
 
@@ -229,8 +247,9 @@ __device__ __forceinline__ int length_bucket(int64_t len64) {
   const unsigned len = len64 > 0x7fffffff ? 0x7fffffffu : (unsigned) (len64 < 0 ? 0 : len64);
   if (len == 0) return 0;
   const int m    = 31 - __clz(len);
-  const int frac = m >= 2 ? (int) ((len >> (m - 2)) & 3u) : (int) ((len << (2 - m)) & 3u);
-  return 1 + m * 4 + frac;  // <= 124
+  const int frac = m >= kOrderFracBits ? (int) ((len >> (m - kOrderFracBits)) & (kOrderFrac - 1))
+                                       : (int) ((len << (kOrderFracBits - m)) & (kOrderFrac - 1));
+  return 1 + m * kOrderFrac + frac;  // <= 31 * kOrderFrac
 }
 
 #ifndef FSGS_TILE_GROUP
@@ -249,30 +268,79 @@ __global__ void __launch_bounds__(1024) tile_order_kernel(int gx, int gy, const 
                                                           int* __restrict__ tile_order) {
   __shared__ int s_count[kOrderRegions][kOrderBuckets];
   __shared__ int s_total[kOrderRegions];
+  __shared__ int s_tile[kOrderRegions][kBalanceRounds * kCusPerXcd], s_len[kOrderRegions][kBalanceRounds * kCusPerXcd];
   const int T = gx * gy;
   for (int b = threadIdx.x; b < kOrderRegions * kOrderBuckets; b += blockDim.x) (&s_count[0][0])[b] = 0;
   __syncthreads();
   for (int t = threadIdx.x; t < T; t += blockDim.x)
     atomicAdd(&s_count[tile_region(t, gx, gy)][length_bucket(ranges[2 * (size_t) t + 1] - ranges[2 * (size_t) t])], 1);
   __syncthreads();
-  if (threadIdx.x < kOrderRegions) {  // exclusive prefix from the longest bucket down, per region
-    int run = 0;
-    for (int b = kOrderBuckets - 1; b >= 0; --b) {
-      const int c = s_count[threadIdx.x][b];
-      s_count[threadIdx.x][b] = run;
-      run += c;
+  {  // exclusive prefix from the longest bucket down, one wavefront per region
+    const int lane = threadIdx.x & 63, r = threadIdx.x >> 6;
+    constexpr int kPer = kOrderBuckets / 64;
+    if (r < kOrderRegions) {
+      int c[kPer], sum = 0;
+#pragma unroll
+      for (int i = 0; i < kPer; ++i) c[i] = s_count[r][kOrderBuckets - 1 - (lane * kPer + i)], sum += c[i];
+      int inc = sum;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(inc, d, 64);
+        if (lane >= d) inc += up;
+      }
+      int run = inc - sum;
+#pragma unroll
+      for (int i = 0; i < kPer; ++i) s_count[r][kOrderBuckets - 1 - (lane * kPer + i)] = run, run += c[i];
+      if (lane == 63) s_total[r] = inc;
     }
-    s_total[threadIdx.x] = run;
   }
   __syncthreads();
-  for (int t = threadIdx.x; t < T; t += blockDim.x) {
-    const int r = tile_region(t, gx, gy);
-    const int k = atomicAdd(&s_count[r][length_bucket(ranges[2 * (size_t) t + 1] - ranges[2 * (size_t) t])], 1);
-    // position of the k-th tile of region r when the regions are dealt round-robin, skipping exhausted ones
+  // position of the k-th tile of region r when the regions are dealt round-robin, skipping exhausted ones
+  auto position = [&](int r, int k) {
     int pos = 0;
 #pragma unroll
     for (int q = 0; q < kOrderRegions; ++q) pos += min(s_total[q], k) + ((q < r && s_total[q] > k) ? 1 : 0);
-    tile_order[pos] = t;
+    return pos;
+  };
+  for (int t = threadIdx.x; t < T; t += blockDim.x) {
+    const int r       = tile_region(t, gx, gy);
+    const int64_t len = ranges[2 * (size_t) t + 1] - ranges[2 * (size_t) t];
+    const int k       = atomicAdd(&s_count[r][length_bucket(len)], 1);
+    if (k < kBalanceRounds * kCusPerXcd) {
+      s_tile[r][k] = t;
+      s_len[r][k]  = (int) (len > 0x7fffffff ? 0x7fffffff : len);
+    } else {
+      tile_order[position(r, k)] = t;
+    }
+  }
+  __syncthreads();
+  // The first rounds of a region, one wavefront per region, lane c = the c-th longest tile of the round: the CUs are
+  // sorted by the work they hold so far (bitonic network over the lanes) and the c-th longest tile goes to the CU with
+  // the c-th smallest load. Round 0 keeps its order, round 1 comes out reversed, later rounds even out what is left.
+  {
+    const int lane = threadIdx.x & 63, r = threadIdx.x >> 6;
+    if (r < kOrderRegions && lane < kCusPerXcd) {
+      unsigned long long key = (unsigned long long) lane;  // (load << 8) | cu
+      const int n = s_total[r];
+      for (int j = 0; j < kBalanceRounds && j * kCusPerXcd < n; ++j) {
+        const int k = j * kCusPerXcd + lane;
+        if ((j + 1) * kCusPerXcd > n) {  // a partial last round keeps its order
+          if (k < n) tile_order[position(r, k)] = s_tile[r][k];
+          break;
+        }
+#pragma unroll
+        for (int size = 2; size <= kCusPerXcd; size <<= 1)
+#pragma unroll
+          for (int d = size >> 1; d > 0; d >>= 1) {
+            const unsigned long long other = __shfl_xor(key, d, kCusPerXcd);
+            const bool up = (lane & size) == 0, low = (lane & d) == 0;
+            key = (low == up) ? (key < other ? key : other) : (key < other ? other : key);
+          }
+        const int cu = (int) (key & 0xffull);
+        tile_order[position(r, j * kCusPerXcd + cu)] = s_tile[r][k];
+        key += (unsigned long long) (unsigned) s_len[r][k] << 8;
+      }
+    }
   }
 }
 
