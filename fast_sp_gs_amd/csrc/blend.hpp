@@ -212,7 +212,7 @@ __device__ __forceinline__ unsigned quadrant_mask(const SplatHot& h, int tile_px
 // 32 CUs behind each), and a tile's cost is proportional to the length of its list. The blend kernels therefore map
 // blockIdx -> tile through a table built once per frame: small square groups of tiles are dealt to 8 regions, region r
 // owns the table positions p with p % 8 == r (as long as it has tiles left), and inside a region tiles are listed by
-// descending list length (1/16-octave buckets, arbitrary order inside a bucket). Long lists start first and short ones
+// descending list length (sixteen buckets per octave, arbitrary order inside a bucket). Long lists start first and short ones
 // fill the tail of the launch; a surfel that overlaps several neighbouring tiles is gathered by blocks that share an L2.
 // An XCD places the first blocks it receives on its CUs in turn, and as many rounds of 32 as blocks fit on a CU stay
 // there together for most of the launch: CU c works on the region's tiles number c, 32 + c, 64 + c, ... In plain

@@ -304,3 +304,12 @@ FSGS_API int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, doubl
 #undef FSGS_LAUNCH_FWD
   return check_launch("GS_2D_render_forward");
 }
+
+FSGS_API int fsgs_debug_tile_order(int gx, int gy, const int64_t* ranges, int32_t* table, void* stream) {
+  using namespace fsgs;
+  FSGS_REQUIRE(gx > 0 && gy > 0 && (int64_t) gx * gy <= kMaxOrderedTiles && ranges && table,
+               "debug_tile_order: bad arguments (at most %d tiles)", kMaxOrderedTiles);
+  hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t) stream, gx, gy, ranges, table);
+  return check_launch("debug_tile_order");
+}
+

@@ -20,6 +20,11 @@ int fsgs_copy_probe(const void* src, void* dst, size_t nbytes, void* stream);
  * tests can show that results do not depend on it. Default: on. Process-global: not for use next to concurrent renders. */
 int fsgs_debug_set_culling(int enabled);
 
+/* Writes the blockIdx -> tile table the blend kernels would use for a gx x gy tile grid whose lists are ranges[t] =
+ * (start, end) into table[gx * gy] (device memory; gx * gy <= 65536): a permutation of the tile numbers, longest lists
+ * first inside each of the 8 interleaved position classes. For tests of the schedule itself. */
+int fsgs_debug_tile_order(int gx, int gy, const int64_t* ranges, int32_t* table, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

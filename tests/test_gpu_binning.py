@@ -94,3 +94,48 @@ def test_blocking_entry_points_match_the_operator(device):
                                      L.ptr(pl2), None, L.ptr(ws2), ws2.numel(), stream), 'fill')
     torch.cuda.synchronize()
     assert torch.equal(ranges2, ranges) and torch.equal(pl2, pl)
+
+
+@pytest.mark.parametrize("gx,gy,kind", [
+    (1, 1, "one"), (7, 5, "random"), (16, 16, "random"), (16, 16, "equal"), (50, 50, "ball"), (50, 50, "empty"),
+    (131, 97, "random"), (256, 256, "random"),
+])
+def test_blend_schedule_is_a_permutation_longest_first(device, gx, gy, kind):
+    """The blockIdx -> tile table of the blend kernels (fsgs_debug_tile_order): every tile exactly once, for grids from one
+    tile to the 65 536-tile limit, with empty and equal lists; inside each of the 8 interleaved position classes (one
+    XCD each) the list lengths fall from round to round of 32 positions (inside a round the tiles are dealt by the load of
+    the compute units, in any order), up to the resolution of the length buckets (sixteen per octave)."""
+    from fast_sp_gs_amd import lib as L
+    T = gx * gy
+    rng = np.random.default_rng(gx * 1000 + gy)
+    if kind == "random":
+        lens = rng.integers(0, 5000, T) * (rng.random(T) < 0.7)
+    elif kind == "equal":
+        lens = np.full(T, 777)
+    elif kind == "empty":
+        lens = np.zeros(T, np.int64)
+    elif kind == "one":
+        lens = np.array([12])
+    else:  # chord lengths of a ball centred on the grid, as in the benchmark scene
+        ty, tx = np.mgrid[0:gy, 0:gx]
+        r2 = ((tx - gx / 2 + 0.5) ** 2 + (ty - gy / 2 + 0.5) ** 2) / (0.36 * gx) ** 2
+        lens = (2000 * np.sqrt(np.clip(1 - r2, 0, None))).astype(np.int64).reshape(-1)
+    lens = lens.astype(np.int64)
+    start = np.concatenate([[0], np.cumsum(lens)[:-1]])
+    ranges = torch.from_numpy(np.stack([start, start + lens], 1)).to(device)
+    table = torch.full((T,), -1, dtype=torch.int32, device=device)
+    print(f"[schedule table] {gx}x{gy} {kind}", flush=True)
+    lib = L.load()
+    L.check(lib.fsgs_debug_tile_order(gx, gy, L.ptr(ranges), L.ptr(table), L.current_stream()), 'tile_order')
+    torch.cuda.synchronize()
+    t = npy(table)
+    assert np.array_equal(np.sort(t), np.arange(T)), "not a permutation of the tiles"
+    ll = lens[t]
+    for r in range(8):
+        cls = ll[r::8]                       # a region's tiles while it has any; exhausted regions are skipped, so the
+        if cls.size < 64: continue           # classes only line up with the regions at the start: check full rounds there
+        rounds = cls[:cls.size // 32 * 32].reshape(-1, 32)[:4]
+        lo, hi = rounds.min(1), rounds.max(1)
+        # a later round's longest tile is not above an earlier round's shortest by more than a bucket: sixteen equal
+        # steps per octave, so at most 1/16 of the length
+        assert (hi[1:] <= lo[:-1] * (1 + 1 / 16) + 1).all(), (r, lo, hi)
