@@ -98,6 +98,7 @@ __device__ __forceinline__ bool fast_intersect_flat(const FastHot& h, float pxf,
 // Sums 8 per-lane values over the 64 lanes at once: three merge steps inside aligned groups of 8 lanes, one rotate by 8
 // inside the row of 16, two cross-row exchanges. On return every lane holds the wave total of v[lane & 7].
 __device__ __forceinline__ float wave_sum8_transposed(const float (&v)[8]) {
+#pragma clang fp contract(off)  // an input that is a product must not be formed a second time inside a fused add
   const int lane = __lane_id();
   const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
   float w[4], x[2];
@@ -474,23 +475,20 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
         const bool hit = fast_intersect_flat(s_hot[j], pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
         if ((pass & wave_ballot(pos < last_contrib)) == 0ull) continue;
 
+        // The part under `hit` advances the pixel's back-to-front state and leaves a few factors (zero in a lane whose
+        // pixel does not blend the entry); the components are products of those factors with quantities that are
+        // finite in every lane, formed by all lanes alike: no component needs a zero of its own, and the
+        // projected-centre case is the intersection case with a zero in place of 1 / p_z.
         float g[16], g8[8];
-        bool filtered = false;
-#pragma unroll
-        for (int c = 0; c < 16; ++c) g[c] = 0.0f;
-#pragma unroll
-        for (int c = 0; c < 8; ++c) g8[c] = 0.0f;
+        float w = 0.0f, dL_dalpha = 0.0f, dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f, s_ds = 0.0f, z_sx = 0.0f, z_sy = 0.0f;
+        const FastHot& hot = s_hot[j];
         if (hit) {
-          const FastHot& hot   = s_hot[j];
           const SplatCold cold = s_cold[j];
-          T             = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
-          const float w = h.alpha * T;
+          T = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+          w = h.alpha * T;
           // one back-to-front recurrence for every channel that enters the image linearly: c = <upstream gradient,
           // channel values of this surfel> replaces the reference's per-channel accumulators
           float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
-          g[0] = w * dLp0, g[1] = w * dLp1, g[2] = w * dLp2;
-
-          float dL_dalpha = 0.0f, dL_dz = 0.0f;
           if (kAux) {
             const float rd     = __builtin_amdgcn_rcpf(h.depth);
             const float m_d    = far_scale * (1.0f - near_n * rd);
@@ -506,7 +504,6 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
               dL_dz += dmd_dd * (2.0f * m_d * w * dL_dM2);
             }
             c_lin += h.depth * dL_ddepth + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
-            g[12] = w * dLn0, g[13] = w * dLn1, g[14] = w * dLn2;
             dL_dz += w * dL_ddepth;
           }
           if (kAux || kPerSplat) c_lin += dL_daccum;
@@ -530,30 +527,35 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
           dL_dalpha *= T;
           last_alpha = h.alpha;
 
+          // d/ds of the intersection case (times 1 / p_z below); s is not finite in a lane whose p_z is 0, and such a
+          // lane never blends: every use of s sits on this side
           const float dL_dG = hot.opacity * dL_dalpha;
-          if (h.rho3d <= h.rho2d) {
-            const float dsx = fsx + dL_dG * -h.G * h.sx + dL_dz * hot.tw0;
-            const float dsy = fsy + dL_dG * -h.G * h.sy + dL_dz * hot.tw1;
-            const float rz  = __builtin_amdgcn_rcpf(h.pz);
-            const float da = dsx * rz, db = dsy * rz;
-            const float dc = -(da * h.sx + db * h.sy);
-            g[3] = da * pxf, g[4] = da * pyf, g[5] = da;
-            g[6] = db * pxf, g[7] = db * pyf, g[8] = db;
-            g[9] = dc * pxf, g[10] = dc * pyf, g[11] = dc;
-          } else {
-            g8[3]    = dL_dG * (-h.G * 2.0f * h.dx);
-            g8[4]    = dL_dG * (-h.G * 2.0f * h.dy);
-            filtered = true;
-          }
-          g8[0] = dL_dz * h.sx, g8[1] = dL_dz * h.sy, g8[2] = dL_dz;
-          g[15] = h.G * dL_dalpha;
+          dsx  = fsx + dL_dG * -h.G * h.sx + dL_dz * hot.tw0;
+          dsy  = fsy + dL_dG * -h.G * h.sy + dL_dz * hot.tw1;
+          s_ds = dsx * h.sx + dsy * h.sy;
+          z_sx = dL_dz * h.sx, z_sy = dL_dz * h.sy;
         }
+        const bool by_ray   = h.rho3d <= h.rho2d;
+        const bool filtered = hit && !by_ray;
+        const float rz = (hit && by_ray) ? __builtin_amdgcn_rcpf(h.pz) : 0.0f;
+        const float da = dsx * rz, db = dsy * rz, dc = -(s_ds * rz);
+        g[0] = w * dLp0, g[1] = w * dLp1, g[2] = w * dLp2;
+        g[3] = da * pxf, g[4] = da * pyf, g[5] = da;
+        g[6] = db * pxf, g[7] = db * pyf, g[8] = db;
+        g[9] = dc * pxf, g[10] = dc * pyf, g[11] = dc;
+        if (kAux) g[12] = w * dLn0, g[13] = w * dLn1, g[14] = w * dLn2;
+        else      g[12] = g[13] = g[14] = 0.0f;
+        g[15] = h.G * dL_dalpha;
+        const float to_centre = filtered ? hot.opacity * dL_dalpha * (-2.0f * h.G) : 0.0f;
+        g8[0] = z_sx, g8[1] = z_sy, g8[2] = dL_dz;
+        g8[3] = to_centre * h.dx, g8[4] = to_centre * h.dy;
+        g8[5] = g8[6] = g8[7] = 0.0f;
         const float tot = wave_sum16_transposed(g);
         if (lane < 16) s_part[wave][j][lane] = tot;
         if (kAux) {
           const float tot8 = wave_sum8_transposed(g8);
           if (lane < 5) s_part[wave][j][16 + lane] = tot8;
-        } else if (__ballot(filtered) != 0ull) {
+        } else if (wave_ballot(filtered) != 0ull) {
           const float sx = wave_sum_to_lane63(g8[3]), sy = wave_sum_to_lane63(g8[4]);
           if (lane == 63) s_part[wave][j][19] = sx, s_part[wave][j][20] = sy;
         }

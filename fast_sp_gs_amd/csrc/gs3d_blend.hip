@@ -436,30 +436,36 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
       unsigned long long pass;
       const bool hit = conic_alpha_flat(s_hot[j], pxf, pyf, h, &pass) && (pos < last_contrib);
       if ((pass & wave_ballot(pos < last_contrib)) == 0ull) continue;
+      // Under `hit`: the pixel's back-to-front state and two factors (zero in a lane that does not blend the entry). The
+      // components are their products with quantities that are finite in every lane, formed by all lanes alike, so none
+      // needs a zero of its own.
       float g[16];
-#pragma unroll
-      for (int c = 0; c < 16; ++c) g[c] = 0.0f;
+      const G3Hot& hot = s_hot[j];
+      float dch = 0.0f, dL_dalpha = 0.0f;
       if (hit) {
-        const G3Hot& hot = s_hot[j];
-        T = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
-        const float dch = h.alpha * T;
-        float dL_dalpha = 0.0f;
+        T   = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+        dch = h.alpha * T;
 #pragma unroll
         for (int k = 0; k < 3 + E; ++k) {
           const float v = s_feat[j][k];
           dL_dalpha += (v * T * (1.0f - h.alpha) - accum[k]) * g_out[k];
           accum[k] += v * dch;
-          g[k < 3 ? k : 3 + (k - 3)] = dch * g_out[k];
         }
         dL_dalpha = (dL_dalpha - T_final * dL_dT) * __builtin_amdgcn_rcpf(1.0f - h.alpha);
-        const float dL_dG = -hot.opacity * h.G * dL_dalpha;
-        g[7]  = dL_dG * (hot.a * h.dx + hot.b * h.dy);
-        g[8]  = dL_dG * (hot.c * h.dy + hot.b * h.dx);
-        g[9]  = 0.5f * h.dx * h.dx * dL_dG;
-        g[10] = h.dx * h.dy * dL_dG;
-        g[11] = 0.5f * h.dy * h.dy * dL_dG;
-        g[12] = h.G * dL_dalpha;
       }
+#pragma unroll
+      for (int c = 0; c < 16; ++c) g[c] = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 3 + E; ++k) g[k < 3 ? k : 3 + (k - 3)] = dch * g_out[k];
+      // G = exp(power) overflows in a lane whose conic gives a large positive power; such a lane never blends
+      const float G     = hit ? h.G : 0.0f;
+      const float dL_dG = -hot.opacity * G * dL_dalpha;
+      g[7]  = dL_dG * (hot.a * h.dx + hot.b * h.dy);
+      g[8]  = dL_dG * (hot.c * h.dy + hot.b * h.dx);
+      g[9]  = 0.5f * h.dx * h.dx * dL_dG;
+      g[10] = h.dx * h.dy * dL_dG;
+      g[11] = 0.5f * h.dy * h.dy * dL_dG;
+      g[12] = G * dL_dalpha;
       const float tot = wave_sum16_transposed(g);
       if (lane < 16) s_part[wave][j][lane] = tot;  // a wavefront meets an entry once per batch
     }
