@@ -93,6 +93,29 @@ blend_backward_kernel(
   __syncthreads();
   const int n_todo = min(s_max_contrib, (int) (r1 - r0));  // positions [0, n_todo) of the tile's list, walked from n_todo-1 down to 0
   const int rounds = (n_todo + kBwdBatch - 1) / kBwdBatch;
+  // No zero fill of the records: the instances behind the tile's deepest contributor are never staged, their records
+  // are cleared here; every staged instance writes its record at the flush, zeros included
+  if (kSlots) {
+    for (int e = n_todo + (int) threadIdx.x; e < (int) (r1 - r0); e += kBlendThreads) {
+      const int id = point_list[r0 + e];
+      float cx, cy;
+      int rad;
+      int64_t off;
+      if (records) {
+        const float4 q2 = records[5 * (size_t) id + 2], q4 = records[5 * (size_t) id + 4];
+        cx = q2.y, cy = q2.z, rad = __float_as_int(q4.z), off = (int64_t) __float_as_int(q4.w);
+        if (off < 0) off = id == 0 ? 0 : point_offsets[id - 1];
+      } else {
+        const float2 c = means2D[id];
+        cx = c.x, cy = c.y, rad = radii[id], off = id == 0 ? 0 : point_offsets[id - 1];
+      }
+      const TileRect r = tile_rect(cx, cy, rad, gx, gy);
+      const int64_t slot = off + (int64_t) (tile_y - r.y0) * (r.x1 - r.x0) + (tile_x - r.x0);
+      float2* dst = (float2*) (slot_grads + (size_t) slot * kGradSlots);
+#pragma unroll
+      for (int c = 0; c < kGradSlots / 2; ++c) dst[c] = make_float2(0.0f, 0.0f);
+    }
+  }
 
   const float T_final = inside ? 1.0f - out_opacity[pix] : 0.0f;
   float T = T_final;
@@ -419,15 +442,13 @@ blend_backward_kernel(
         a[c] = sum;
       }
       if (kSlots) {
-        // one 72-byte record per (surfel, tile) instance at the instance's position in surfel order; the per-surfel
-        // sums are taken afterwards by slot_reduce_kernel. Records nobody contributed to stay at their zero fill.
-        // (Measured alternative: a "written" byte per instance instead of the fill -- 1 byte cleared instead of 72, the
-        // sum skipping unwritten records. The scattered byte stores and loads cost more than the streaming fill saves:
-        // operator 0.505 ms against 0.488 ms.)
-        bool any = false;
-#pragma unroll
-        for (int c = 0; c < kGradSlots; ++c) any |= a[c] != 0.0f;
-        if (any) {
+        // One 72-byte record per (surfel, tile) instance at the instance's position in surfel order; the per-surfel
+        // sums are taken afterwards by slot_reduce_kernel. Every staged instance writes its record, zeros included (the
+        // instances that are never staged were cleared at the start), so nobody has to clear the buffer beforehand: a
+        // streaming zero fill of all records in front of this kernel cost 82 MB of writes and 13 us; the stores here
+        // ride on memory pipes this kernel leaves idle. (Also measured, and slower than the fill: a "written" byte per
+        // instance with the sum skipping unwritten records, 0.505 ms against 0.488 ms for the operator.)
+        {
           float2* dst = (float2*) (slot_grads + (size_t) s_slot[b & 1][threadIdx.x] * kGradSlots);
 #pragma unroll
           for (int c = 0; c < kGradSlots / 2; ++c) dst[c] = make_float2(a[2 * c], a[2 * c + 1]);
@@ -453,12 +474,6 @@ blend_backward_kernel(
     // touches its lanes' rows of s_part and this batch's copy of s_slot, wavefront 1 the staging arrays and the other
     // copy of s_slot.
   }
-}
-
-// Zero fill of the per-instance gradient records (float4 stores).
-__global__ void __launch_bounds__(256) slot_fill_kernel(size_t n4, float4* __restrict__ p) {
-  for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t) gridDim.x * blockDim.x)
-    p[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 }
 
 // Per-surfel sums of the instance records. Nine lanes per surfel, each owning one float2 of the 18-float record, so
@@ -540,12 +555,6 @@ FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, doub
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
   float* slot_grads = slots ? (float*) workspace : nullptr;
-  if (slots) {
-    const size_t n4 = ((size_t) R * kGradSlots + 3) / 4;
-    if (n4 > 0)
-      hipLaunchKernelGGL(slot_fill_kernel, dim3((unsigned) std::min<size_t>((n4 + 255) / 256, 8192)), dim3(256), 0, s,
-                         n4, (float4*) slot_grads);
-  }
   const int* tile_order = nullptr;
   const int ordered = launch_tile_order(gx, gy, ranges, s, &tile_order);
 #define FSGS_LAUNCH_BWD(AUX, FLOW, SLOTS)                                                                            \
