@@ -124,7 +124,8 @@ int fsgs_gs_2d_render_forward(int P, int W, int H, double near_n, double far_n, 
  *  - point_offsets[P] (the prefix scan fsgs_gs_prepare_scan produced for this point_list) with radii[P], R and a workspace
  *    of fsgs_gs_2d_render_backward_workspace_bytes(R): every (surfel, tile) instance writes one record at its position
  *    in surfel order and a second kernel sums each surfel's records in a fixed order. No atomics to HBM, the four outputs
- *    are fully written (no initialisation needed). Requires the point_list of fsgs_gs_prepare_fill for these means2D /
+ *    are fully written and the workspace needs no clearing (every instance's record is written, zeros included).
+ *    Requires the point_list of fsgs_gs_prepare_fill for these means2D /
  *    radii (the position of an instance is recomputed from the surfel's tile rectangle). */
 size_t fsgs_gs_2d_render_backward_workspace_bytes(int64_t R);
 int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n, const float* means2D,
