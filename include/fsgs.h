@@ -137,7 +137,7 @@ int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n,
     size_t workspace_bytes, const float* records, void* stream);
 
 /* ---- "fast" surfel path: transform through camera intrinsics Tv2s[3,3], adjugate-based intersection, fused
- * corner-test binning. Flow outputs are not supported on this path. ---- */
+ * corner-test binning. Optical flow (trans_mat_t2) is carried by the two blend entry points below. ---- */
 
 /* gs_2d_fast_preprocess_forward (per-surfel part) -- gs_2d_fast_preprocess.cu:160-262, host :611-709.
  * Same outputs as fsgs_gs_2d_preprocess_forward plus inverse_m[P,3,3] (adjugate of trans_mat). Only the z translation
