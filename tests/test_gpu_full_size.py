@@ -9,6 +9,8 @@
   * K-NN at 3M x 2048, k = 8: distances ascending, equal to the distance recomputed from the returned index, and no
     closer control point exists for a sample of queries (brute force with torch).
 Sizes: 300 000 surfels at 800x800, 3 000 000 surfels at 1352x1014 (one view), 400 000 surfels at 3840x2160.
+The fast path and the 3D-Gaussian path get the same kind of checks at 300 000 / 800x800 (culling, ordered against atomic
+sums, linearity, weight sums; for the fast path also its two backward algorithms against each other).
 """
 import numpy as np
 import pytest
@@ -129,3 +131,113 @@ def test_knn_3m_by_2048_k8(device):
     full = torch.cdist(x[sample], y) ** 2
     kth = full.topk(K, dim=1, largest=False).values
     assert float((kth - d2[sample]).abs().max()) < 1e-4 * float(kth.max())
+
+
+@pytest.mark.parametrize("per_splat", [False, True])
+def test_fast_path_properties_at_300k_800(per_splat, device):
+    """The fast path at the benchmark size: culling off == on (forward bit for bit, gradients to the rounding of
+    reordered sums), ordered per-instance sums == atomics, the backward linear in the upstream gradients, and the two
+    backward algorithms (per pixel / per 32-entry bucket from the forward's snapshots) agreeing with each other."""
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd.renderer import fast_render_step
+    scene_h, cam_h = scenes.config2()
+    W, H = cam_h.W, cam_h.H
+    g = torch.Generator().manual_seed(13)
+    gi, ge, go = torch.randn(3, H, W, generator=g).to(device), torch.randn(8, H, W, generator=g).to(device), \
+        torch.randn(H, W, generator=g).to(device)
+    scene, cam = scene_h.to(device), cam_h.to(device)
+    print(f"[full fast per_splat={per_splat}] P={scene.P} {W}x{H}", flush=True)
+    grads = ('g_colors', 'g_means2D_blend', 'g_trans', 'g_inv', 'g_normal_opacity', 'g_means3D', 'g_scales',
+             'g_rotations', 'g_opacities', 'g_shs')
+
+    def close(x, y, tol, what):
+        for k in grads:
+            ref = x[k].abs().max().clamp_min(1e-30)
+            assert float((x[k] - y[k]).abs().max() / ref) < tol, (what, k)
+
+    a = fast_render_step(scene, cam, gi, ge, go, per_splat=per_splat)
+    torch.cuda.synchronize()
+    print(f"[full fast] R={a['point_list'].numel()}", flush=True)
+    assert all(bool(torch.isfinite(a[k]).all()) for k in grads)
+    try:
+        _culling(False)
+        b = fast_render_step(scene, cam, gi, ge, go, per_splat=per_splat)
+        torch.cuda.synchronize()
+    finally:
+        _culling(True)
+    for k in ('image', 'opacity', 'extras', 'n_contrib', 'point_list', 'ranges'):
+        assert torch.equal(a[k], b[k]), f"{k} depends on the culling"
+    close(a, b, 2e-5, 'culling')
+    # (the atomics add in arrival order; the fast preprocess backward amplifies that rounding in dL/dscales)
+    close(a, fast_render_step(scene, cam, gi, ge, go, per_splat=per_splat, ordered_sums=False), 1e-4, 'atomic sums')
+    c = fast_render_step(scene, cam, 2.0 * gi, 2.0 * ge, 2.0 * go, per_splat=per_splat)
+    for k in grads:
+        ref = a[k].abs().max().clamp_min(1e-30)
+        assert float((c[k] - 2.0 * a[k]).abs().max() / ref) < 2e-5, ('linearity', k)
+    if per_splat:
+        # The bucketed backward restarts from the forward's snapshots: same gradients up to their rounding, for the
+        # upstream channels both algorithms define alike (the per-pixel one differentiates the distortion map, channel 5,
+        # the bucketed one takes channels 6 and 7, the two depth moments, as plain linear outputs).
+        ge_c = ge.clone()
+        ge_c[5:] = 0
+        close(fast_render_step(scene, cam, gi, ge_c, go, per_splat=True),
+              fast_render_step(scene, cam, gi, ge_c, go, per_splat=False), 2e-4, 'per-pixel backward')
+
+
+def test_gs3d_path_properties_at_300k_800(device):
+    """The 3D-Gaussian path at the benchmark size (the benchmark's centres with a third scale): culling off == on,
+    ordered per-instance sums == atomics, blend weights summing to the opacity image, linearity of the backward."""
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd._C import get_C_function as f
+    scene_h, cam_h = scenes.config2()
+    scene, cam = scene_h.to(device), cam_h.to(device)
+    W, H = cam.W, cam.H
+    g = torch.Generator().manual_seed(11)
+    scales = torch.cat([scene_h.scales, scene_h.scales[:, :1] * (0.5 + torch.rand(scene.P, 1, generator=g))],
+                       1).to(device).contiguous()
+    gi, go = torch.randn(3, H, W, generator=g).to(device), torch.randn(H, W, generator=g).to(device)
+    tan_fov = (W / 2 / float(cam.Tv2s[0, 0]), H / 2 / float(cam.Tv2s[1, 1]))
+    print(f"[full gs3d] P={scene.P} {W}x{H}", flush=True)
+
+    def step(gi, go, ordered):
+        m2, dep, col, rad, tt, c3, co = f('gs_preprocess_forward')(
+            W, H, 3, False, scene.means3D, scales, scene.rotations, scene.opacities, scene.shs, None, cam.Tw2v,
+            cam.Tv2c, cam.campos, tan_fov, None, None, None, None)
+        ranges, pl, offsets = f('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True)
+        oc, oo, _, nc = f('gaussian_rasterize_forward')(W, H, m2, co, col, None, pl, ranges)
+        g_col, _, g_m2, g_co = f('gaussian_rasterize_backward')(m2, co, col, None, oo, gi, go, None, ranges, pl, nc,
+                                                                offsets if ordered else None, rad if ordered else None)
+        g3, gs, gq = torch.empty_like(scene.means3D), torch.empty_like(scales), torch.empty_like(scene.rotations)
+        gop, gsh = torch.empty_like(scene.opacities), torch.empty_like(scene.shs)
+        f('gs_preprocess_backward')(W, H, 3, False, scene.means3D, scales, scene.rotations, scene.opacities, scene.shs,
+                                    None, cam.Tw2v, cam.Tv2c, cam.campos, tan_fov, c3, None, rad, col, g_m2.clone(), None,
+                                    g_col, g_co, g3, gs, gq, gop, gsh, None, None)
+        torch.cuda.synchronize()
+        return dict(image=oc, opacity=oo, n_contrib=nc, point_list=pl, ranges=ranges, m2=m2, co=co, col=col,
+                    g_col=g_col, g_m2=g_m2, g_co=g_co, g3=g3, gs=gs, gq=gq, gop=gop, gsh=gsh)
+
+    grads = ('g_col', 'g_m2', 'g_co', 'g3', 'gs', 'gq', 'gop', 'gsh')
+
+    def close(x, y, tol, what, scale=1.0):
+        for k in grads:
+            ref = x[k].abs().max().clamp_min(1e-30)
+            assert float((y[k] - scale * x[k]).abs().max() / ref) < tol, (what, k)
+
+    a = step(gi, go, True)
+    print(f"[full gs3d] R={a['point_list'].numel()}", flush=True)
+    assert all(bool(torch.isfinite(a[k]).all()) for k in grads)
+    try:
+        _culling(False)
+        b = step(gi, go, True)
+    finally:
+        _culling(True)
+    for k in ('image', 'opacity', 'n_contrib', 'point_list', 'ranges'):
+        assert torch.equal(a[k], b[k]), f"{k} depends on the culling"
+    close(a, b, 2e-5, 'culling')
+    close(a, step(gi, go, False), 1e-4, 'atomic sums')
+    close(a, step(2.0 * gi, 2.0 * go, True), 2e-5, 'linearity', 2.0)
+    acc = torch.zeros(scene.P, device=device)
+    f('gaussian_rasterize_forward')(W, H, a['m2'], a['co'], a['col'], None, a['point_list'], a['ranges'], None, acc, None)
+    torch.cuda.synchronize()
+    tot_w, tot_o = float(acc.double().sum()), float(a['opacity'].double().sum())
+    assert abs(tot_w - tot_o) < 1e-4 * tot_o
