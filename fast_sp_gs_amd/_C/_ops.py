@@ -430,6 +430,11 @@ def GS_2D_render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat2
         return g_colors, g_means2D, g_trans, g_norm_op
     c = lambda t: None if t is None else t.contiguous()
     means2D, normal_opacity, colors, out_opacity = c(means2D), c(normal_opacity), c(colors), c(out_opacity)
+    trans_mat, trans_mat2 = c(trans_mat), c(trans_mat2)
+    if records is not None:
+        L.require_cuda(what, records=records)
+        L.require_dtype(what, 'records', records, torch.float32)
+        L.require_shape(what, 'records', records, P, 20)
     dL_dout_color, dL_dout_opacity, dL_dothers, dL_dout_flows = (c(dL_dout_color), c(dL_dout_opacity),
                                                                 c(dL_dothers), c(dL_dout_flows))
     ranges, point_list, n_contrib = c(ranges), c(point_list), c(n_contrib)

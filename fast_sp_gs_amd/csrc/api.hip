@@ -2,9 +2,7 @@
 #include "common.hpp"
 
 #include <cstring>
-#include <map>
 #include <mutex>
-#include <utility>
 
 namespace fsgs {
 
@@ -21,28 +19,83 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
-// One blockIdx -> tile table (65536 ints, see blend.hpp) per (device, stream) that a blend entry point was called on,
-// with the tile ranges it was built from.
-TileOrderState* tile_order_state(hipStream_t stream) {
-  static std::mutex mu;
-  static std::map<std::pair<int, hipStream_t>, TileOrderState> tables;
+// blockIdx -> tile tables of the blend kernels (see blend.hpp): kTableSlots tables of kMaxOrderedTiles ints each in a
+// file-scope device array, so the library never calls hipMalloc. A (device, stream) pair takes a free slot on its first
+// binning or blend call and keeps it until fsgs_stream_release or the end of the process; when every slot of a device
+// is taken, further streams get no table and their blocks map to tiles directly (same results, no longest-first order).
+// Slots are never taken away from a stream behind its back: a kernel of that stream may still be reading the table.
+constexpr int kTableSlots   = 8;
+constexpr int kTableInts    = 1 << 16;  // == kMaxOrderedTiles
+constexpr int kMaxDevices   = 64;
+static __device__ __align__(256) int g_tile_order_tables[kTableSlots][kTableInts];
+
+namespace {
+struct TableSlot {
+  bool used = false;
+  hipStream_t stream = nullptr;
+  const int64_t* ranges = nullptr;  // what the table was built from (nullptr: nothing)
+  int gx = 0, gy = 0;
+};
+struct DeviceTables {
+  int* base = nullptr;  // device address of g_tile_order_tables on this device (each device holds its own copy)
+  bool resolved = false;
+  TableSlot slot[kTableSlots];
+};
+std::mutex g_table_mu;
+DeviceTables g_tables[kMaxDevices];
+
+// Caller holds g_table_mu. Returns the slot of (current device, stream), taking a free one if `take`; -1 if none.
+int find_slot(hipStream_t stream, bool take, DeviceTables** out) {
   int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
-  std::lock_guard<std::mutex> lock(mu);
-  auto it = tables.find({dev, stream});
-  if (it != tables.end()) return it->second.table ? &it->second : nullptr;
-  int* p = nullptr;
-  if (hipMalloc((void**) &p, sizeof(int) * (1 << 16)) != hipSuccess) {
-    (void) hipGetLastError();
-    p = nullptr;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -1;
+  DeviceTables& d = g_tables[dev];
+  *out = &d;
+  if (!d.resolved) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_tile_order_tables)) != hipSuccess) {
+      (void) hipGetLastError();
+      p = nullptr;
+    }
+    d.base = (int*) p, d.resolved = true;
   }
-  TileOrderState& st = tables[{dev, stream}];
-  st = TileOrderState{p, nullptr, 0, 0};
-  return p ? &st : nullptr;
+  if (!d.base) return -1;
+  int free_slot = -1;
+  for (int i = 0; i < kTableSlots; ++i) {
+    if (d.slot[i].used && d.slot[i].stream == stream) return i;
+    if (!d.slot[i].used && free_slot < 0) free_slot = i;
+  }
+  if (!take || free_slot < 0) return -1;
+  d.slot[free_slot] = TableSlot{true, stream, nullptr, 0, 0};
+  return free_slot;
+}
+}  // namespace
+
+int* tile_order_table(hipStream_t stream, const int64_t* ranges, int gx, int gy, bool* rebuild) {
+  std::lock_guard<std::mutex> lock(g_table_mu);
+  *rebuild = false;
+  DeviceTables* d = nullptr;
+  const int i = find_slot(stream, true, &d);
+  if (i < 0) return nullptr;
+  TableSlot& t = d->slot[i];
+  if (t.ranges != ranges || t.gx != gx || t.gy != gy) {
+    t.ranges = ranges, t.gx = gx, t.gy = gy;
+    *rebuild = true;
+  }
+  return d->base + (size_t) i * kTableInts;
 }
 
 void tile_order_invalidate(hipStream_t stream) {
-  if (TileOrderState* st = tile_order_state(stream)) st->ranges = nullptr;
+  std::lock_guard<std::mutex> lock(g_table_mu);
+  DeviceTables* d = nullptr;
+  const int i = find_slot(stream, false, &d);
+  if (i >= 0) d->slot[i].ranges = nullptr;
+}
+
+void tile_order_release(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_table_mu);
+  DeviceTables* d = nullptr;
+  const int i = find_slot(stream, false, &d);
+  if (i >= 0) d->slot[i] = TableSlot{};
 }
 
 static bool g_culling_enabled = true;
@@ -73,6 +126,11 @@ FSGS_API int fsgs_copy_probe(const void* src, void* dst, size_t nbytes, void* st
 
 FSGS_API int fsgs_debug_set_culling(int enabled) {
   fsgs::g_culling_enabled = enabled != 0;
+  return fsgs::kOk;
+}
+
+FSGS_API int fsgs_stream_release(void* stream) {
+  fsgs::tile_order_release((hipStream_t) stream);
   return fsgs::kOk;
 }
 

@@ -220,9 +220,9 @@ __device__ __forceinline__ unsigned quadrant_mask(const SplatHot& h, int tile_px
 // chord-length profile of a ball of surfels), and the launch lasts as long as its busiest CU. Inside each of the first
 // rounds the tiles are therefore dealt by load: the CU with the least work so far gets the round's longest tile.
 // Later rounds go wherever a slot frees up; for them descending order is what balances.
-// The table is a device buffer of kMaxOrderedTiles ints owned by the library, one per (device, stream) a blend entry
-// point has been called on (allocated on the first such call, kept until the process ends): calls on one stream are
-// ordered by the stream, calls on different streams use different tables.
+// The table is kMaxOrderedTiles ints in a file-scope device array of the library (no allocation), one slot per
+// (device, stream) that bins or blends: calls on one stream are ordered by the stream, calls on different streams use
+// different tables, and a stream that finds every slot taken runs without a table.
 #ifndef FSGS_ORDER_FRAC_BITS
 #define FSGS_ORDER_FRAC_BITS 4
 #endif
@@ -239,7 +239,7 @@ constexpr int kCusPerXcd       = 32;  // compute units behind one region's table
 // bounded by its 128 registers per lane); measured best among 3, 4, 5, 6, 8, 16
 constexpr int kBalanceRounds   = FSGS_ORDER_BALANCE_ROUNDS;
 
-// (TileOrderState, tile_order_state and tile_order_invalidate are declared in common.hpp.)
+// (tile_order_table, tile_order_invalidate and tile_order_release are declared in common.hpp.)
 
 namespace {
 
@@ -350,13 +350,11 @@ inline int launch_tile_order(int gx, int gy, const int64_t* ranges, hipStream_t 
   int flags = culling_enabled() ? 0 : kFlagNoCull;
   *table    = nullptr;
   if ((int64_t) gx * gy > kMaxOrderedTiles) return flags;
-  TileOrderState* st = tile_order_state(s);
-  if (!st) return flags;
-  if (st->ranges != ranges || st->gx != gx || st->gy != gy) {
-    hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, s, gx, gy, ranges, st->table);
-    st->ranges = ranges, st->gx = gx, st->gy = gy;
-  }
-  *table = st->table;
+  bool rebuild = false;
+  int* t = tile_order_table(s, ranges, gx, gy, &rebuild);
+  if (!t) return flags;
+  if (rebuild) hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, s, gx, gy, ranges, t);
+  *table = t;
   return flags | kFlagOrdered;
 }
 

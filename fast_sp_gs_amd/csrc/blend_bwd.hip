@@ -104,6 +104,7 @@ blend_backward_kernel(
       if (records) {
         const float4 q2 = records[5 * (size_t) id + 2], q4 = records[5 * (size_t) id + 4];
         cx = q2.y, cy = q2.z, rad = __float_as_int(q4.z), off = (int64_t) __float_as_int(q4.w);
+        if (rad < 0) rad = radii[id];  // a record packed without radii / offsets holds -1 there
         if (off < 0) off = id == 0 ? 0 : point_offsets[id - 1];
       } else {
         const float2 c = means2D[id];
@@ -165,8 +166,9 @@ blend_backward_kernel(
 #pragma unroll
       for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
     if (kSlots) {
-      // a record carries the surfel's radius and, once the binning's scan has stored it, its offset (-1 until then)
-      next_radius = records ? ex.radius : radii[next.cold.id];
+      // a record carries the surfel's radius (-1 if it was packed without radii) and, once the binning's scan has
+      // stored it, its offset (-1 until then)
+      next_radius = records && ex.radius >= 0 ? ex.radius : radii[next.cold.id];
       next_off    = records && ex.offset >= 0 ? ex.offset : (next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1]);
     }
   }
@@ -199,7 +201,7 @@ blend_backward_kernel(
 #pragma unroll
         for (int k = 0; k < 9; ++k) next_t2[k] = trans_mat_t2[9 * (size_t) next.cold.id + k];
       if (kSlots) {
-        next_radius = records ? ex.radius : radii[next.cold.id];
+        next_radius = records && ex.radius >= 0 ? ex.radius : radii[next.cold.id];
         next_off    = records && ex.offset >= 0 ? ex.offset : (next.cold.id == 0 ? 0 : point_offsets[next.cold.id - 1]);
       }
     }

@@ -242,7 +242,7 @@ __global__ void __launch_bounds__(256) pack_records_kernel(int P, const float2* 
   const float2 c  = means2D[i];
   const float4 no = normal_opacity[i];
   const float* rgb = colors + 3 * (size_t) i;
-  const int radius  = radii ? radii[i] : 0;
+  const int radius  = radii ? radii[i] : -1;  // -1: not known, the backward then reads its radii argument
   const int offset  = point_offsets ? (i == 0 ? 0 : (int) point_offsets[i - 1]) : -1;  // -1: not known
   float4* r = records + 5 * (size_t) i;
   r[0] = make_float4(M[0], M[1], M[2], M[3]);

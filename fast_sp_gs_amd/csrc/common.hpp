@@ -86,18 +86,16 @@ __device__ __forceinline__ TileRect tile_rect(float px, float py, int r, int gx,
 }
 
 // ---- blockIdx -> tile schedule of the blend kernels (built by tile_order_kernel in blend.hpp) ------------------------
-// The table is rebuilt when a launch sees other tile ranges (by address and grid size) than the ones it was built from;
-// the binning entry points forget the key of their stream when they rewrite a ranges buffer, so a frame builds the table
-// once, in its first blend launch, and the frame's other blend launches (backward, top-k, extra channels) reuse it. A
-// ranges buffer rewritten behind the library's back (or binned on another stream) keeps an older frame's order: still a
-// permutation of the same tile grid, so every tile is processed exactly once -- only the longest-first order is stale.
-struct TileOrderState {
-  int* table;
-  const int64_t* ranges;  // what the table was built from (nullptr: nothing)
-  int gx, gy;
-};
-// Defined in api.hip. nullptr if the table cannot be allocated (then blocks map to tiles directly).
-TileOrderState* tile_order_state(hipStream_t stream);
+// Each (device, stream) that bins or blends owns one of a few tables held in a file-scope device array (api.hip), keyed
+// on the tile ranges it was built from (address and grid size). tile_order_table returns the stream's table, or nullptr
+// when the device's tables are all taken (then blocks map to tiles directly), and sets *rebuild when the key changed: the
+// caller then launches tile_order_kernel on that stream. The binning entry points forget the key of their stream when
+// they rewrite a ranges buffer, so a frame builds the table once and the frame's blend launches (forward, backward,
+// top-k, extra channels) reuse it. A ranges buffer rewritten behind the library's back (or binned on another stream)
+// keeps an older frame's order: still a permutation of the same tile grid, so every tile is processed exactly once --
+// only the longest-first order is stale. All three functions take the same lock.
+int* tile_order_table(hipStream_t stream, const int64_t* ranges, int gx, int gy, bool* rebuild);
 void tile_order_invalidate(hipStream_t stream);
+void tile_order_release(hipStream_t stream);
 
 }  // namespace fsgs

@@ -4,37 +4,41 @@ import torch
 from torch import Tensor, nn
 
 from fast_sp_gs_amd._C import get_C_function
+from fast_sp_gs_amd.autograd import KernelPair
 
 __all__ = ['FusedSSIM', 'ssim', 'SSIM_Loss', 'l1_dssim_loss']
 
 
-class FusedSSIM(torch.autograd.Function):
-    _forward_func = get_C_function('fusedssim')
-    _backward_func = get_C_function('fusedssim_backward')
-    C1 = 0.01 ** 2
-    C2 = 0.03 ** 2
+C1, C2 = 0.01 ** 2, 0.03 ** 2  # the usual SSIM stabilisers for images in [0, 1]
 
-    @staticmethod
-    def forward(ctx, img1, img2, window=None):
-        ssim_map, d1, d2, d3 = FusedSSIM._forward_func(FusedSSIM.C1, FusedSSIM.C2, img1, img2, ctx.needs_input_grad[0])
-        assert not ctx.needs_input_grad[1]
-        ctx.save_for_backward(img1, img2, d1, d2, d3)
-        return ssim_map
 
-    @staticmethod
-    @torch.autograd.function.once_differentiable
-    def backward(ctx, *grad_outputs):
-        img1, img2, d1, d2, d3 = ctx.saved_tensors
-        grad_img1 = FusedSSIM._backward_func(FusedSSIM.C1, FusedSSIM.C2, img1, img2, grad_outputs[0].contiguous(), d1,
-                                             d2, d3)
-        return grad_img1, None, None
+def _ssim_launch(fwd, needs, img, target, _window=None):
+    if len(needs) > 1 and needs[1]:
+        raise RuntimeError('fused SSIM is differentiable in its first image only')
+    ssim_map, d_mu, d_var, d_cov = fwd(C1, C2, img, target, bool(needs[0]))
+    return ssim_map, (img, target, d_mu, d_var, d_cov), None
+
+
+def _ssim_grads(bwd, needs, keep, _, g_map):
+    img, target, d_mu, d_var, d_cov = keep
+    return (bwd(C1, C2, img, target, g_map, d_mu, d_var, d_cov), None, None)[:len(needs)]
+
+
+_ssim_pair = KernelPair('fusedssim', 'fusedssim_backward', _ssim_launch, _ssim_grads)
+
+
+class FusedSSIM:
+    """The reference's autograd function of this name (losses/ssim.py:24-47) as a call-compatible shim:
+    `FusedSSIM.apply(img1, img2, window)` -> SSIM map; the window argument is ignored (fixed 11 taps)."""
+    C1, C2 = C1, C2
+    apply = staticmethod(_ssim_pair)
 
 
 def ssim(img1: Tensor, img2: Tensor) -> Tensor:
     """SSIM map of [B,CH,H,W] (or [CH,H,W]) images; differentiable in img1."""
     if img1.ndim == 3:
-        return FusedSSIM.apply(img1[None], img2[None], None)[0]
-    return FusedSSIM.apply(img1, img2, None)
+        return _ssim_pair(img1[None], img2[None])[0]
+    return _ssim_pair(img1, img2)
 
 
 class _L1DssimLoss(torch.autograd.Function):
@@ -44,7 +48,7 @@ class _L1DssimLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, img, target, lambda_dssim):
         img, target = img.contiguous(), target.contiguous()
-        loss, d1, d2, d3 = get_C_function('image_loss_forward')(FusedSSIM.C1, FusedSSIM.C2, lambda_dssim, img, target,
+        loss, d1, d2, d3 = get_C_function('image_loss_forward')(C1, C2, lambda_dssim, img, target,
                                                                 ctx.needs_input_grad[0])
         assert not ctx.needs_input_grad[1]
         ctx.lambda_dssim = lambda_dssim
@@ -82,16 +86,12 @@ class SSIM_Loss(nn.Module):
             raise ValueError('the fused SSIM kernel has a fixed 11-tap window')
         self.reduction = reduction
 
+    @staticmethod
+    def _as_batch(img: Tensor) -> Tensor:
+        """[CH,H,W] / [H,W,3] / [B,H,W,3] / [B,CH,H,W] -> [B,CH,H,W] (a trailing dimension of 3 is taken as channels)."""
+        img = img if img.ndim == 4 else img[None]
+        return img.movedim(-1, 1) if img.shape[-1] == 3 else img
+
     def forward(self, img1: Tensor, img2: Tensor, mask: Tensor = None) -> Tensor:
-        if img1.ndim == 3:
-            img1 = img1.unsqueeze(0)
-        if img2.ndim == 3:
-            img2 = img2.unsqueeze(0)
-        if img1.shape[-1] == 3:
-            img1 = torch.permute(img1, (0, 3, 1, 2))  # -> [B, C, H, W]
-        if img2.shape[-1] == 3:
-            img2 = torch.permute(img2, (0, 3, 1, 2))
-        m = ssim(img1, img2)
-        if self.reduction == 'mean':
-            return 1.0 - m.mean()
-        return 1.0 - m.mean(dim=(1, 2, 3))
+        per_image = ssim(self._as_batch(img1), self._as_batch(img2)).flatten(1).mean(dim=1)
+        return 1.0 - (per_image.mean() if self.reduction == 'mean' else per_image)

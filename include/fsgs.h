@@ -6,8 +6,11 @@
  *    *_host. NULL stands for an absent optional tensor (Python `None` at the reference's pybind boundary).
  *  - `stream` is a hipStream_t (NULL = default stream). Calls enqueue work and return; the only blocking call is
  *    fsgs_gs_prepare_scan, which has to hand the instance count to the host (the reference blocks in the same place).
- *  - The library allocates nothing: outputs and workspaces come from the caller (the *_workspace_bytes functions size
- *    them). Outputs need not be zero-initialised unless stated.
+ *  - The library allocates nothing, neither device nor host memory, on any call: outputs and workspaces come from the
+ *    caller (the *_workspace_bytes functions size them). Outputs need not be zero-initialised unless stated. What the
+ *    library keeps of its own is in file-scope device arrays that exist once per GPU from the moment the library is
+ *    loaded: eight blockIdx -> tile schedule tables of 256 KiB (one per stream that bins or blends, see
+ *    fsgs_stream_release) and the 512 KiB of fsgs_image_loss_forward_static.
  *  - Return value 0 = success; otherwise fsgs_last_error() describes the failure (thread local).
  *  - `file:line` citations name the reference interface each entry point replaces (relative to the reference root).
  */
@@ -24,6 +27,11 @@ extern "C" {
 const char* fsgs_last_error(void);
 int fsgs_version(void);
 int fsgs_check_device(void);
+/* The binning and blend entry points map blockIdx -> tile through a per-stream schedule table (longest tile lists
+ * first). A stream takes one of eight table slots of its GPU on its first such call and keeps it; streams beyond the
+ * eighth run without a table (identical results, blocks map to tiles directly). A caller that creates and destroys
+ * streams hands a slot back with this call once the stream's work has completed. No counterpart in the reference. */
+int fsgs_stream_release(void* stream);
 /* ---- 2DGS surfel preprocess ---------------------------------------------------------------------------------- */
 
 /* gs_2d_preprocess_forward -- fast_2d_gs/_C/src/gaussian_splatting/gs_2d_preprocess.cu:331-421 (kernel :158-246).

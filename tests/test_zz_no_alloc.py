@@ -49,3 +49,26 @@ def test_image_loss_static_rejects_oversize(device):
     rc = lib.fsgs_image_loss_forward_static(1, 1, 32, 32 * (cap + 1), 1e-4, 9e-4, 0.2, L.ptr(tiny), L.ptr(tiny),
                                             L.ptr(loss), None, None, None, L.current_stream())
     assert rc != 0 and b'exceed' in lib.fsgs_last_error()
+
+
+def test_image_loss_static_leaves_device_memory_alone(device):
+    """Free device memory as the driver reports it (hipMemGetInfo) is the same before and after a call: the entry point
+    takes nothing from the device allocator. Every tensor the call touches exists beforehand, and one call has already
+    run on this device, so the lookup of the scratch array's address is not part of what is measured."""
+    from fast_sp_gs_amd import lib as L
+    lib = L.load()
+    g = torch.Generator().manual_seed(12)
+    shape = (1, 3, 96, 160)
+    img, target = torch.rand(*shape, generator=g).to(device), torch.rand(*shape, generator=g).to(device)
+    loss = torch.zeros(3, device=device)
+    d = [torch.empty_like(img) for _ in range(3)]
+    args = (*shape, 1e-4, 9e-4, 0.2, L.ptr(img), L.ptr(target), L.ptr(loss), L.ptr(d[0]), L.ptr(d[1]), L.ptr(d[2]))
+    stream = L.current_stream()
+    L.check(lib.fsgs_image_loss_forward_static(*args, stream), 'image_loss')
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        L.check(lib.fsgs_image_loss_forward_static(*args, stream), 'image_loss')
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
