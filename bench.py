@@ -163,6 +163,100 @@ def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
     return steps / dt
 
 
+def _timed_ms(fn, reps: int = 20, warm: int = 3) -> float:
+    """Average device time of `fn` (events on the current stream, the one the operators launch on)."""
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def standalone_ops(dev, copy_gbps: float):
+    """The stand-alone operators of BASELINE config 1 and the optimiser, each with its algorithmic bytes, the rate those
+    bytes give over the measured time, and that rate as a share of the 8 TB/s peak and of the copy probe:
+    SH encoder forward / backward at 1M directions (shencoder.cu:657-691), SH -> RGB forward / backward at 1M points
+    (ops_3d/spherical_harmonics.cu:15-16, 68-70), the LBS blend forward / backward at 200 000 x 512, K = 4
+    (network.py:545-573), the masked Adam at 300 000 x 58 floats (adam_masked_update.cu:9-38), one launch per parameter
+    tensor as the reference's optimiser loop does and all six in one launch. Output tensors are allocated outside the
+    timed calls wherever the operator takes them as arguments."""
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd._C import get_C_function as f
+    c1 = scenes.config1()
+    out = {}
+
+    def record(name, ms, nbytes, unit_count=None, unit=None):
+        gbps = nbytes / (ms * 1e-3) / 1e9
+        out[name] = {"ms": round(ms, 4), "algorithmic_bytes": int(nbytes), "GBps": round(gbps, 1),
+                     "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "frac_of_copy_probe": round(gbps / copy_gbps, 4)}
+        if unit_count:
+            out[name][unit] = unit_count / (ms * 1e-3)
+
+    # ---- SH encoder, degree 3: [B,3] -> [B,16]
+    dirs = c1['dirs'].to(dev)
+    B, deg = dirs.shape[0], 3
+    n_coef = (deg + 1) ** 2
+    enc = torch.empty(B, n_coef, device=dev)
+    g_enc, g_dirs = torch.randn(B, n_coef, device=dev), torch.zeros(B, 3, device=dev)
+    record("sh_encode_forward_1m", _timed_ms(lambda: f('sh_encode_forward')(dirs, enc, B, 3, deg)),
+           B * (12 + 4 * n_coef), B, "directions_per_s")
+    record("sh_encode_backward_1m", _timed_ms(lambda: f('sh_encode_backward')(g_enc, dirs, B, 3, deg, g_dirs)),
+           B * (4 * n_coef + 12 + 12), B, "directions_per_s")
+    # ---- SH -> RGB, degree 3: positions + camera centre + [B,16,3] coefficients -> rgb; backward writes dSH and d(pos)
+    shs = c1['shs'].to(dev)
+    campos = torch.tensor([0.0, 0.0, 4.0], device=dev)
+    rgb = f('SH_to_RGB_forward')(dirs, campos, shs, deg, True)
+    g_rgb, g_sh, g_pos, g_cam = torch.randn_like(rgb), torch.empty_like(shs), torch.empty_like(dirs), torch.zeros(3, device=dev)
+    record("sh_to_rgb_forward_1m", _timed_ms(lambda: f('SH_to_RGB_forward')(dirs, campos, shs, deg, True)),
+           B * (12 + 12 * n_coef + 12), B, "points_per_s")
+    record("sh_to_rgb_backward_1m",
+           _timed_ms(lambda: f('SH_to_RGB_backward')(deg, True, dirs, campos, shs, rgb, g_rgb, g_pos, g_cam, g_sh)),
+           B * (12 + 12 * n_coef + 12 + 12) + B * (12 * n_coef + 12), B, "points_per_s")
+    del enc, g_enc, g_dirs, shs, g_sh, g_pos, rgb, g_rgb
+    # ---- LBS blend, 200 000 points x 512 control points, K = 4, weights softmax(-d^2 / 0.01), rigid transforms
+    pts, ctrl = c1['points'].to(dev), c1['ctrl'].to(dev)
+    sp_t, sp_r, sp_s = c1['sp_t'].to(dev), c1['sp_r'].to(dev), c1['sp_s'].to(dev)
+    sp_rot = sp_r.clone()
+    N, M, K, S = pts.shape[0], ctrl.shape[0], 4, sp_s.shape[1]
+    d2, idx = f('knn_topk')(pts, ctrl, K)
+    fwd = lambda: f('lbs_blend')(pts, ctrl, sp_t, sp_r, sp_s, d2, idx, 0.01, 'LBS', sp_rot, 'dist')
+    g_xyz, g_rot, g_scale = torch.randn(N, 3, device=dev), torch.randn(N, 4, device=dev), torch.randn(N, S, device=dev)
+    bwd = lambda: f('lbs_blend_backward')(pts, ctrl, sp_t, sp_r, sp_s, d2, idx, g_xyz, g_rot, g_scale, 0.01, 'LBS',
+                                          sp_rot, 'dist')
+    record("lbs_blend_forward_200k_512_k4", _timed_ms(fwd), N * (12 + K * (8 + 4)) + M * 28 + N * 12, N, "points_per_s")
+    # backward: points, pair inputs, indices and the three upstream gradients in; g_points and g_pair out; per
+    # control point 3 + 3 + 4 + 4 + S floats in and out
+    record("lbs_blend_backward_200k_512_k4", _timed_ms(bwd),
+           N * (12 + K * 12 + 12 + 16 + 4 * S) + N * (12 + 4 * K) + 2 * M * 4 * (14 + S), N, "points_per_s")
+    # ---- masked Adam: the six parameter tensors of a 2DGS point set (3 + 3 + 45 + 1 + 2 + 4 = 58 floats per surfel)
+    P, widths = 300_000, (3, 3, 45, 1, 2, 4)
+    g = torch.Generator().manual_seed(4)
+    mask = (torch.rand(P, generator=g) < 0.9).to(dev)
+    params = [torch.randn(P, w, generator=g).to(dev) for w in widths]
+    grads = [torch.randn(P, w, generator=g).to(dev) for w in widths]
+    m1, m2 = [torch.zeros_like(t) for t in params], [torch.zeros_like(t) for t in params]
+    n_vis = int(mask.sum())
+    adam_bytes = len(widths) * P + n_vis * sum(widths) * 28  # the mask is read once per tensor
+    one = f('AdamMasksedUpdated')
+
+    def per_tensor():
+        for t, gr, a, b, w in zip(params, grads, m1, m2, widths):
+            one(t, gr, a, b, mask, 1.6e-4, 0.9, 0.999, 1e-15, P, w)
+
+    record("adam_masked_6_launches_300k_58", _timed_ms(per_tensor), adam_bytes)
+    multi = f('AdamMasksedUpdatedMulti')
+    record("adam_masked_1_launch_300k_58",
+           _timed_ms(lambda: multi(params, grads, m1, m2, mask, [1.6e-4] * 6, 0.9, 0.999, [1e-15] * 6, P)), adam_bytes)
+    out["workload"] = ("config 1: 1M unit directions / points at SH degree 3; 200000 x 512 control points, K = 4, rigid "
+                       "transforms, 'dist' weights; masked Adam on 300000 surfels x 58 floats, 90 % visible. Times are "
+                       "device time per call including the Python wrapper's output allocation where the operator allocates")
+    return out
+
+
 def simple_knn_ms(dev, scene):
     """simple_knn (mean squared 3-NN distance, used to initialise the surfel scales) on the benchmark scene's 300k
     centres and on 3M uniform points."""
@@ -671,6 +765,7 @@ def main():
 
     copy_gbps = copy_probe_gbps(dev)
     extra = {"knn_topk_queries_per_s": pts.shape[0] / (knn_ms * 1e-3), "knn_topk_workload": "200000 x 512, k=4, D=3"}
+    extra["standalone_ops"] = standalone_ops(dev, copy_gbps)
     if not args.no_extras:
         extra.update(ssim_rate(dev))
         extra.update(simple_knn_ms(dev, scene))

@@ -5,12 +5,21 @@
 // tile's list backwards, gradient channels consumed are image, opacity, aux 0-5 (depth, normal, median depth,
 // distortion) and optional flow; the 0.99 alpha clamp is not masked in the gradient, as in the reference.
 //
-// Where the reference issues 18-21 global float atomics per (pixel, surfel) pair, this kernel
-//   1. sums each of the 18 per-surfel gradient components over the 64 pixels of a wavefront with DPP row shifts and
-//      row broadcasts (no LDS traffic), skipping surfels no pixel of the wavefront blends,
-//   2. adds the 4 wavefront partials of a tile into an LDS accumulator of the staged batch, and
-//   3. flushes one global atomic per surfel, component and tile when the batch retires.
-// Surfels behind the deepest contributor of the whole tile are never gathered.
+// Where the reference issues 18-21 global float atomics per (pixel, surfel) pair, this kernel splits the work of a pair
+// into the part that depends on the order of the pixel's list and the part that does not:
+//   1. order-bound, one wavefront per 8x8 pixel quadrant, one list entry per pass: the ray-splat intersection and the
+//      pixel's back-to-front recurrences. A pixel that blends the entry leaves three numbers (blend weight,
+//      G * dL/dalpha, dL/ddepth) and its (pixel, entry) pair in the wavefront's queue in LDS. Few lanes of a pass blend
+//      (a quarter on the benchmark scene), so this part is kept as short as the recurrences allow.
+//   2. order-free, all 64 lanes busy: the wavefront takes 64 queued pairs at a time -- an entry's pairs padded to a
+//      16-lane row -- recomputes the two planes through the pixel from the staged record, forms the 16 + 2 gradient
+//      components and sums them over each row with DPP row shifts (no LDS traffic); each row adds its 16 totals to the
+//      entry's row of the wavefront's accumulator in LDS.
+//   3. per staged batch the four wavefronts' accumulators are added in wavefront order and every staged (surfel, tile)
+//      instance writes one record at its position in surfel order; slot_reduce_kernel sums a surfel's records in a
+//      fixed order. (Without scan offsets: one global atomic per surfel, component and tile, as the reference's sums.)
+// Surfels behind the deepest contributor of the whole tile are never gathered. The optical-flow instantiation keeps
+// parts 1 and 2 in one pass per entry (its extra per-pair terms would double the queue record).
 #include <algorithm>
 
 #include "blend.hpp"
@@ -19,7 +28,7 @@ namespace fsgs {
 namespace {
 
 // Per-surfel gradient slots: 0-2 colours | 3-11 trans_mat | 12-14 normal | 15 opacity | 16-17 means2D.
-// The first 16 go through one transposed wave reduction; the means2D pair is only non-zero for pixels where the
+// The first 16 go through one transposed row reduction; the means2D pair is only non-zero for pixels where the
 // screen-space low-pass filter wins (rho2d < rho3d) and is reduced separately when any lane took that branch.
 constexpr int kGradSlots = 18;
 #ifndef FSGS_BWD_BATCH
@@ -29,18 +38,18 @@ constexpr int kGradSlots = 18;
 #define FSGS_BWD_WAVES 4
 #endif
 constexpr int kBwdBatch = FSGS_BWD_BATCH;  // surfels staged per round
-static_assert(kBwdBatch <= kWave, "one wavefront stages a batch and another flushes it");
-// Work unit of the gradient pass. 0 (default): one list entry per pass of a wavefront over its 8x8 quadrant. 1: each
-// 16-lane DPP row of a wavefront owns a 4x4 pixel block and walks its own list of the entries that blend into that block
-// (see "two phases" in the kernel). Measured at 300k surfels, 800x800: 6 % fewer vector instructions (213 M against
-// 227 M; the intersection has to be evaluated in both phases), 66 % more scalar ones, and the LDS adds that replace the
-// plain per-wavefront stores keep the LDS pipeline busy four times as long, so the launch takes 462 us against 449 us.
-// Same results either way; kept as a build-time choice.
-#ifndef FSGS_BWD_ROWS
-#define FSGS_BWD_ROWS 0
+static_assert(kBwdBatch == kWave, "one wavefront stages a batch, another flushes it, and a queued pair names its entry in 6 bits");
+// Queue of blended (pixel, entry) pairs per wavefront, a ring of 16-byte items in two halves of 64. A pass over one
+// entry appends at most 64 items (its blending pixels padded to a multiple of 16) and a full half is drained as soon
+// as there is one, so the ring never holds more than 48 + 64 items and a drain always starts at a half.
+#ifndef FSGS_BWD_QUEUE
+#define FSGS_BWD_QUEUE 1
 #endif
-constexpr bool kBwdRows = FSGS_BWD_ROWS != 0;
-static_assert(!kBwdRows || kBwdBatch == kWave, "the per-row hit lists are 64-bit masks over one staged batch");
+constexpr bool kBwdQueue = FSGS_BWD_QUEUE != 0;
+constexpr int kQueueItems = 128;
+// item.w: pixel of the quadrant (6 bits) | blends (bit 12) | met by the ray-splat intersection rather than by its
+// projected centre (bit 13)
+constexpr int kItemHit = 1 << 12, kItemRay = 1 << 13;
 
 template <bool kAux, bool kFlow, bool kSlots>
 __global__ void __launch_bounds__(kBlendThreads) __attribute__((amdgpu_waves_per_eu(FSGS_BWD_WAVES, FSGS_BWD_WAVES)))
@@ -54,11 +63,11 @@ blend_backward_kernel(
     float* __restrict__ g_normal_opacity, float* __restrict__ g_colors, float* __restrict__ g_trans,
     const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii, float* __restrict__ slot_grads,
     const float4* __restrict__ records) {
+  constexpr bool kQueue = kBwdQueue && !kFlow;
   __shared__ SplatHot s_hot[kBwdBatch];
   __shared__ SplatCold s_cold[kBwdBatch];
-  // Each wavefront's sums over its 64 pixels, one row per staged surfel, written once per entry with a plain store (a
-  // wavefront meets an entry once per batch); the flush adds the four rows in wavefront order, so a tile's sums do not
-  // depend on timing. +1: the odd stride keeps the flush free of bank conflicts.
+  // Each wavefront's sums over its 64 pixels, one row per staged surfel; the flush adds the four rows in wavefront
+  // order, so a tile's sums do not depend on timing. +1: the odd stride keeps the flush free of bank conflicts.
   __shared__ float s_part[4][kBwdBatch][kGradSlots + 1];
   // Where a staged (surfel, tile) instance's sums go: its position in surfel order (kSlots) or the surfel's id. Two
   // copies by batch parity: wavefront 1 stages batch b + 1 while wavefront 0 still flushes batch b.
@@ -66,12 +75,16 @@ blend_backward_kernel(
   __shared__ float s_t2[kFlow ? kBwdBatch * 9 : 1];
   __shared__ int s_max_contrib;
   __shared__ unsigned char s_mask[kBwdBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
+  // queued pairs, and the upstream gradients of the tile's pixels (the lane that turns a queued pair into gradient
+  // components is not the lane that owns the pixel): image 3 + normal 3 per pixel
+  __shared__ float4 s_queue[kQueue ? 4 : 1][kQueue ? kQueueItems : 1];
+  __shared__ float4 s_up4[kQueue ? kBlendThreads : 1];
+  __shared__ float2 s_up2[kQueue && kAux ? kBlendThreads : 1];
 
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int tile = scheduled_tile(ordered, tile_order), tile_x = tile % gx, tile_y = tile / gx;
   int px, py;
-  if (kBwdRows) lane_pixel_blocks(tile_x, tile_y, px, py);
-  else lane_pixel(tile_x, tile_y, px, py);
+  lane_pixel(tile_x, tile_y, px, py);
   const bool inside = px < W && py < H;
   const size_t HW   = (size_t) H * W;
   const size_t pix  = (size_t) W * py + px;
@@ -138,6 +151,10 @@ blend_backward_kernel(
       sum_w      = out_extras[pix + 8 * HW];
     }
   }
+  if (kQueue) {  // read back by this wavefront only: no barrier needed
+    s_up4[threadIdx.x] = make_float4(dLp0, dLp1, dLp2, dLn0);
+    if (kAux) s_up2[threadIdx.x] = make_float2(dLn1, dLn2);
+  }
   const float final_A   = 1.0f - T_final;
   const float far_scale = far_n / (far_n - near_n);
   float dLf0 = 0, dLf1 = 0, dL_dsum_w = 0;
@@ -150,6 +167,11 @@ blend_backward_kernel(
   float acc_lin = 0, last_lin = 0;
   float last_dL_dT = 0, last_alpha = 0, acc_w = 0;
   float acc_f0 = 0, acc_f1 = 0, last_f0 = 0, last_f1 = 0;
+  // the wavefront's queue: items [q_head, q_head + q_count) of its ring (wave-uniform, multiples of 16)
+  int q_head = 0, q_count = 0;
+  unsigned long long q_rows = 0ull;            // entry (staging slot) of each of the ring's eight rows, a byte per row
+  const int row_shift = (lane >> 4) * 8;       // this lane's byte of the four rows of a pass
+  const float qx0 = (float) (tile_x * kTile + (wave & 1) * 8), qy0 = (float) (tile_y * kTile + (wave >> 1) * 8);
 
   Splat next;
   float next_t2[9];
@@ -206,45 +228,189 @@ blend_backward_kernel(
       }
     }
 
-    // Work list of this wavefront for 64 staged surfels at a time: those that can reach its quadrant and are not
-    // behind its deepest contributor; consumed bit by bit with scalar instructions.
-    for (int chunk = 0; chunk < kBwdBatch / kWave; ++chunk) {
-     const int jj = chunk * kWave + lane;
-     unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u) &&
-                                        (n_todo - 1 - (b * kBwdBatch + jj)) < wave_max_contrib);
-     // Gradient terms of one (pixel, entry) pair. The part under `hit` advances the pixel's back-to-front state and
-     // leaves five factors (zero for a lane whose pixel does not blend the entry); the 16 + 2 per-surfel components
-     // are products of those factors with quantities that are finite in every lane, formed by all lanes alike, so no
-     // component needs a zero of its own and the two ways a surfel is met (ray-splat intersection / projected
-     // centre) share one instruction stream: the projected-centre case is the intersection case with a zero in place
-     // of 1 / p_z. `j` (staging slot) and `pos` (list position) may differ between the rows of a wavefront.
+    // Work list of this wavefront for the staged surfels: those that can reach its quadrant and are not behind its
+    // deepest contributor; consumed bit by bit with scalar instructions.
+    unsigned long long todo = __ballot(lane < n_here && ((s_mask[lane] >> wave) & 1u) &&
+                                       (n_todo - 1 - (b * kBwdBatch + lane)) < wave_max_contrib);
+    // ---- order-bound part of one (pixel, entry) pair: advances the pixel's back-to-front state -------------------------
+    // All channels that enter the image linearly (colour, depth, opacity, normal) share one recurrence: with
+    // c = <upstream gradient, channel values of this surfel>, the reference's per-channel accumulators
+    // acc_x = last_alpha * last_x + (1 - last_alpha) * acc_x contract to a single scalar. Leaves the blend weight w,
+    // dL/dalpha and dL/ddepth of the pair; call under `hit` only.
+    auto advance_pixel = [&](const SplatCold& cold, int pos, const Hit& h, float& w, float& dL_dalpha, float& dL_dz) {
+      T = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+      w = h.alpha * T;
+      float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
+      if (kAux) {
+        const float rd     = __builtin_amdgcn_rcpf(h.depth);
+        const float m_d    = far_scale * (1.0f - near_n * rd);
+        const float dmd_dd = far_scale * near_n * rd * rd;
+        if (pos == median_contrib - 1) dL_dz += dL_dmedian;
+        const float dL_dweight = (final_D2 + m_d * m_d * final_A - 2.0f * m_d * final_D) * dL_dreg;
+        dL_dalpha += dL_dweight - last_dL_dT;
+        last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
+        const float dL_dmd = 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg;
+        dL_dz += dL_dmd * dmd_dd;
+        c_lin += h.depth * dL_ddepth + dL_daccum + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
+        dL_dz += w * dL_ddepth;
+      }
+      acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
+      last_lin = c_lin;
+      dL_dalpha += c_lin - acc_lin;
+    };
+    if (kQueue) {
+      // ---- order-free part: 64 queued pairs at a time, four 16-lane rows, every row one entry ---------------------------
+      // A lane rebuilds the two planes through its pair's pixel from the staged record and forms the 16 + 2 components
+      // as products of the three queued numbers with quantities that are finite in every lane (padding items carry
+      // zeros and no flags, and the reciprocal of p_z is only taken under the pair's flags), so no component needs a
+      // zero of its own; the projected-centre case is the intersection case with a zero in place of 1 / p_z.
+      auto drain = [&](int n_valid) {
+        // the entries of the four rows come from the wavefront's scalar bookkeeping, so the queued item, the staged
+        // record and the accumulator row are requested together (one LDS round trip instead of three in a chain)
+        const unsigned jrows = (unsigned) (q_rows >> (q_head >> 1));  // q_head is 0 or 64: byte r = entry of row r
+        const int j = (int) ((jrows >> row_shift) & 63u);
+        const float4 it = s_queue[wave][q_head + lane];
+        const SplatHot hot = s_hot[j];
+        float* const acc = &s_part[wave][j][lane & 15];
+        const float before = *acc;
+        const int bits = __float_as_int(it.w);
+        const int qp = bits & 63;
+        const bool blends = (bits & kItemHit) != 0, by_ray = (bits & kItemRay) != 0;
+        const float4 up = s_up4[wave * kWave + qp];
+        const float fx = qx0 + (float) (qp & 7), fy = qy0 + (float) (qp >> 3);
+        const float w = it.x, GdA = it.y, dL_dz = it.z;
+        const float kx = fx * hot.m[6] - hot.m[0], ky = fx * hot.m[7] - hot.m[1], kz = fx * hot.m[8] - hot.m[2];
+        const float lx = fy * hot.m[6] - hot.m[3], ly = fy * hot.m[7] - hot.m[4], lz = fy * hot.m[8] - hot.m[5];
+        const float p_x = ky * lz - kz * ly, p_y = kz * lx - kx * lz, p_z = kx * ly - ky * lx;
+        const float rz_s = blends ? __builtin_amdgcn_rcpf(p_z) : 0.0f;  // s is used by both cases of a blending pair
+        const float rz_p = by_ray ? rz_s : 0.0f;                         // d/dp only by the intersection case
+        const float sx = p_x * rz_s, sy = p_y * rz_s;
+        const float oG = hot.opacity * GdA;
+        float dsx = -(oG * sx), dsy = -(oG * sy);
+        if (kAux) dsx += dL_dz * hot.m[6], dsy += dL_dz * hot.m[7];
+        const float s_ds = dsx * sx + dsy * sy;
+        // d/dp of the homogeneous intersection point p = k x l, negated (the components below are minus the plane
+        // gradients): p_xy = s p_z, so dp_xy = ds / p_z and dp_z = -<ds, s> / p_z
+        const float npx = -(dsx * rz_p), npy = -(dsy * rz_p), npz = s_ds * rz_p;
+        float g[16];
+        g[0] = w * up.x, g[1] = w * up.y, g[2] = w * up.z;
+        g[3] = ly * npz - lz * npy, g[4] = lz * npx - lx * npz, g[5] = lx * npy - ly * npx;
+        g[6] = npy * kz - npz * ky, g[7] = npz * kx - npx * kz, g[8] = npx * ky - npy * kx;
+        g[9]  = dL_dz * sx - (fx * g[3] + fy * g[6]);
+        g[10] = dL_dz * sy - (fx * g[4] + fy * g[7]);
+        g[11] = dL_dz - (fx * g[5] + fy * g[8]);
+        if (kAux) {
+          const float2 un = s_up2[wave * kWave + qp];
+          g[12] = w * up.w, g[13] = w * un.x, g[14] = w * un.y;
+        } else {
+          g[12] = g[13] = g[14] = 0.0f;
+        }
+        g[15] = GdA;
+        const float own = row_sum16_transposed(g);  // lane (row, c): the row's total of component c
+        // An entry with more than 16 blending pixels fills neighbouring rows. The accumulator belongs to this wavefront
+        // alone, so a row adds with a plain read and write, provided no two rows of the pass write the same entry: rows
+        // 2k and 2k + 1 of one entry are added in registers first (one row swap) and row 2k writes for both; a run
+        // that continues from row 1 into row 2 makes row 2 wait for a second round. Rows past n_valid hold old items.
+        const int rows_valid = (n_valid + 15) >> 4;
+        const int j0 = (int) (jrows & 63u), j1 = rows_valid > 1 ? (int) ((jrows >> 8) & 63u) : -1;
+        const int j2 = rows_valid > 2 ? (int) ((jrows >> 16) & 63u) : -2, j3 = rows_valid > 3 ? (int) ((jrows >> 24) & 63u) : -3;
+        const bool s01 = j0 == j1, s12 = j1 == j2, s23 = j2 == j3;
+        float lo = own, hi = own;  // after the swap: lo = rows (0, 0, 2, 2), hi = rows (1, 1, 3, 3) of `own`
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32_e32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+        const float pair = lo + hi;
+        const int row = lane >> 4;
+        const bool joined = (row == 0 && s01) || (row == 2 && s23);          // this row writes for its odd neighbour too
+        const bool silent = (row == 1 && s01) || (row == 3 && s23) || row >= rows_valid;
+        const float mine = joined ? pair : own;
+        if (!silent && !(row == 2 && s12)) *acc = before + mine;
+        if (s12) {  // wave-uniform; the LDS serves a wavefront's accesses in order, so this read sees row 0 / 1's store
+          if (row == 2 && !silent) *acc = *(volatile float*) acc + mine;  // re-read: rows 0 / 1 may just have written it
+        }
+        const bool filtered = blends && !by_ray;
+        if (wave_ballot(filtered) != 0ull) {  // some pair met its surfel by the projected centre
+          const float to_centre = filtered ? -2.0f * oG : 0.0f;
+          float cx = to_centre * (hot.cx - fx), cy = to_centre * (hot.cy - fy);  // totals of a row end up in its lane 15
+          cx += dpp_shift_zero<0x111, 0xf, 0xf>(cx), cy += dpp_shift_zero<0x111, 0xf, 0xf>(cy);
+          cx += dpp_shift_zero<0x112, 0xf, 0xf>(cx), cy += dpp_shift_zero<0x112, 0xf, 0xf>(cy);
+          cx += dpp_shift_zero<0x114, 0xf, 0xf>(cx), cy += dpp_shift_zero<0x114, 0xf, 0xf>(cy);
+          cx += dpp_shift_zero<0x118, 0xf, 0xf>(cx), cy += dpp_shift_zero<0x118, 0xf, 0xf>(cy);
+          if (row < rows_valid && (lane & 15) == 15) atomicAdd(&s_part[wave][j][16], cx), atomicAdd(&s_part[wave][j][17], cy);
+        }
+        // a full pass leaves the other half of the ring in front; the last, partial pass of a batch empties the queue
+        if (n_valid >= kWave) q_head ^= kWave, q_count -= kWave;
+        else q_head = 0, q_count = 0;
+      };
+      // ---- order-bound part of one entry, and the append of its blending pixels to the queue -----------------------------
+      auto queue_entry = [&](const SplatHot& hot, const SplatCold& cold, int j) {
+        const int pos = n_todo - 1 - (b * kBwdBatch + j);  // 0-based position in the tile's list
+        Hit h;
+        unsigned long long pass;
+        const bool hit = intersect_flat(hot, pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
+        pass &= wave_ballot(pos < last_contrib);
+        if (pass == 0ull) return;  // wave-uniform: nobody in this quadrant blends the surfel
+        float w = 0.0f, dL_dalpha = 0.0f, dL_dz = 0.0f;
+        if (hit) {
+          advance_pixel(cold, pos, h, w, dL_dalpha, dL_dz);
+          dL_dalpha *= T * h.G;  // only G * dL/dalpha is ever used
+          last_alpha = h.alpha;
+        }
+        // blending lanes take the first popcount(pass) places in lane order; the next lanes that do not blend fill the
+        // row up with neutral items (zeros, no flags, their own pixel: every number formed from it is finite)
+        const int n_hit = (int) __popcll(pass), n_pad = (n_hit + 15) & ~15;
+        const int below = (int) __builtin_amdgcn_mbcnt_hi((unsigned) (pass >> 32), __builtin_amdgcn_mbcnt_lo((unsigned) pass, 0u));
+        const int place = hit ? below : n_hit + (lane - below);
+        const int flags = hit ? (h.rho3d <= h.rho2d ? (kItemHit | kItemRay) : kItemHit) : 0;
+        const int tail = q_head + q_count;  // first free place of the ring (mod its size), a multiple of 16
+        if (place < n_pad)
+          s_queue[wave][(tail + place) & (kQueueItems - 1)] =
+              make_float4(w, dL_dalpha, dL_dz, __int_as_float(lane | flags));
+        // which entry each 16-item row of the ring holds: one byte per row in a 64-bit scalar
+        for (int r = 0; r < n_pad; r += 16) {
+          const int sh = (((tail + r) & (kQueueItems - 1)) >> 4) * 8;
+          q_rows = (q_rows & ~(0xffull << sh)) | ((unsigned long long) j << sh);
+        }
+        q_count += n_pad;
+        if (q_count >= kWave) drain(kWave);
+      };
+      if (todo != 0ull) {
+        auto pop = [&]() {
+          const int j = __builtin_ctzll(todo);
+          todo &= todo - 1;
+          return j;
+        };
+        auto peek = [&]() { return todo ? (int) __builtin_ctzll(todo) : 0; };
+        SplatHot hot_a = s_hot[peek()], hot_b;
+        while (todo) {
+          {
+            const int j = pop();
+            hot_b       = s_hot[peek()];
+            const SplatCold cold = s_cold[j];
+            __builtin_amdgcn_sched_barrier(0);
+            queue_entry(hot_a, cold, j);
+          }
+          if (todo == 0ull) break;
+          {
+            const int j = pop();
+            hot_a       = s_hot[peek()];
+            const SplatCold cold = s_cold[j];
+            __builtin_amdgcn_sched_barrier(0);
+            queue_entry(hot_b, cold, j);
+          }
+        }
+        if (q_count > 0) drain(q_count);  // the staged records are replaced after the next barrier
+      }
+    } else {
+     // Gradient terms of one (pixel, entry) pair, formed in the pass that advances the pixel. The part under `hit` leaves
+     // a few factors (zero for a lane whose pixel does not blend the entry); the 16 + 2 per-surfel components are
+     // products of those factors with quantities that are finite in every lane, formed by all lanes alike, so no
+     // component needs a zero of its own and the two ways a surfel is met (ray-splat intersection / projected centre)
+     // share one instruction stream.
      auto pair_gradients = [&](const SplatHot& hot, const SplatCold& cold, int j, int pos, const Hit& h, bool hit,
                                float (&g)[16], float& g2x, float& g2y, unsigned long long& ray_lanes) {
        float w = 0.0f, dL_dalpha = 0.0f, dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f, s_ds = 0.0f, z_sx = 0.0f, z_sy = 0.0f;
        if (hit) {
-         T = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
-         w = h.alpha * T;
-         // All channels that enter the image linearly (colour, depth, opacity, normal) share one back-to-front
-         // recurrence: with c = <upstream gradient, channel values of this surfel>, the reference's per-channel
-         // accumulators acc_x = last_alpha * last_x + (1 - last_alpha) * acc_x contract to a single scalar.
-         float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
-         if (kAux) {
-           const float rd     = __builtin_amdgcn_rcpf(h.depth);
-           const float m_d    = far_scale * (1.0f - near_n * rd);
-           const float dmd_dd = far_scale * near_n * rd * rd;
-           if (pos == median_contrib - 1) dL_dz += dL_dmedian;
-           const float dL_dweight = (final_D2 + m_d * m_d * final_A - 2.0f * m_d * final_D) * dL_dreg;
-           dL_dalpha += dL_dweight - last_dL_dT;
-           last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
-           const float dL_dmd = 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg;
-           dL_dz += dL_dmd * dmd_dd;
-           c_lin += h.depth * dL_ddepth + dL_daccum + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
-           dL_dz += w * dL_ddepth;
-           dsx = dL_dz * hot.m[6], dsy = dL_dz * hot.m[7];
-         }
-         acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
-         last_lin = c_lin;
-         dL_dalpha += c_lin - acc_lin;
+         advance_pixel(cold, pos, h, w, dL_dalpha, dL_dz);
+         if (kAux) dsx = dL_dz * hot.m[6], dsy = dL_dz * hot.m[7];
          if (kFlow) {
            const float* Q = &s_t2[j * 9];
            const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
@@ -312,124 +478,33 @@ blend_backward_kernel(
         if (lane == 63) s_part[wave][j][16] = sx, s_part[wave][j][17] = sy;
       }
      };
-     if (kBwdRows) {
-      // ---- two phases per staged batch ----------------------------------------------------------------------------
-      // A surfel that reaches an 8x8 quadrant blends into a quarter of its pixels on average, so a pass of the whole
-      // wavefront over one entry leaves most lanes idle in the expensive part (gradients + reduction). Phase 1 walks
-      // the wavefront's list as before but only runs the intersection, and notes for each 4x4 block (= DPP row) which
-      // entries blend into it (four 64-bit masks, scalar registers). Phase 2 lets every row walk ITS list: in one pass
-      // the four rows evaluate four different entries, recompute the intersection (cheaper than parking it), form the
-      // gradients, sum them over the row's 16 pixels with the row part of the transposed butterfly, and add the 16
-      // totals to the entry's row of the batch accumulator in LDS (rows of one wavefront can meet the same entry, in
-      // the same or in different passes, hence an LDS add and not a store). A pixel still meets its entries back to
-      // front, so the recurrences are untouched.
-      if (todo == 0ull) continue;
-      unsigned long long rows_hit[4] = {0ull, 0ull, 0ull, 0ull};
-      auto test_entry = [&](const SplatHot& hot, int j) {
-        const int pos = n_todo - 1 - (b * kBwdBatch + j);
-        Hit h;
-        const bool hit = intersect_flat(hot, pxf, pyf, near_n, h) && (pos < last_contrib);
-        const unsigned long long who = __ballot(hit);
-        const unsigned long long bit = 1ull << j;
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if ((who >> (16 * r)) & 0xffffull) rows_hit[r] |= bit;
-      };
-      {
-        auto pop = [&]() {
-          const int j = __builtin_ctzll(todo);
-          todo &= todo - 1;
-          return j;
-        };
-        auto peek = [&]() { return todo ? __builtin_ctzll(todo) : 0; };
-        SplatHot hot_a = s_hot[peek()], hot_b;
-        while (todo) {
-          {
-            const int j = pop();
-            hot_b       = s_hot[peek()];
-            __builtin_amdgcn_sched_barrier(0);
-            test_entry(hot_a, j);
-          }
-          if (todo == 0ull) break;
-          {
-            const int j = pop();
-            hot_a       = s_hot[peek()];
-            __builtin_amdgcn_sched_barrier(0);
-            test_entry(hot_b, j);
-          }
-        }
-      }
-      const int row = lane >> 4;
-      unsigned long long mine = row == 0 ? rows_hit[0] : row == 1 ? rows_hit[1] : row == 2 ? rows_hit[2] : rows_hit[3];
-      auto row_entry = [&](const SplatHot& hot, const SplatCold& cold, int j, bool active) {
-        const int pos = n_todo - 1 - (b * kBwdBatch + j);
-        Hit h;
-        const bool hit = intersect_flat(hot, pxf, pyf, near_n, h) && (pos < last_contrib) && active;
-        float g[16], g2x, g2y;
-        unsigned long long ray_lanes;
-        pair_gradients(hot, cold, j, pos, h, hit, g, g2x, g2y, ray_lanes);
-        const bool filtered = hit && !((ray_lanes >> lane) & 1ull);
-        const float tot = row_sum16_transposed(g);  // lane (row, c): the row's total of component c
-        if (active) atomicAdd(&s_part[wave][j][lane & 15], tot);
-        if (wave_ballot(filtered) != 0ull) {
-          float sx = g2x, sy = g2y;  // totals of the row end up in its lane 15
-          sx += dpp_shift_zero<0x111, 0xf, 0xf>(sx), sy += dpp_shift_zero<0x111, 0xf, 0xf>(sy);
-          sx += dpp_shift_zero<0x112, 0xf, 0xf>(sx), sy += dpp_shift_zero<0x112, 0xf, 0xf>(sy);
-          sx += dpp_shift_zero<0x114, 0xf, 0xf>(sx), sy += dpp_shift_zero<0x114, 0xf, 0xf>(sy);
-          sx += dpp_shift_zero<0x118, 0xf, 0xf>(sx), sy += dpp_shift_zero<0x118, 0xf, 0xf>(sy);
-          if (active && (lane & 15) == 15) atomicAdd(&s_part[wave][j][16], sx), atomicAdd(&s_part[wave][j][17], sy);
-        }
-      };
-      // the next entry's records are requested before the current one is evaluated (alternating registers)
-      auto front = [&]() { return mine ? (int) __builtin_ctzll(mine) : 0; };
-      int j_a = front(), j_b = 0;
-      SplatHot hot_a = s_hot[j_a], hot_b;
-      SplatCold cold_a = s_cold[j_a], cold_b;
-      while (__ballot(mine != 0ull) != 0ull) {
-        {
-          const bool active = mine != 0ull;
-          mine &= mine - 1;
-          j_b = front(), hot_b = s_hot[j_b], cold_b = s_cold[j_b];
-          __builtin_amdgcn_sched_barrier(0);
-          row_entry(hot_a, cold_a, j_a, active);
-        }
-        if (__ballot(mine != 0ull) == 0ull) break;
-        {
-          const bool active = mine != 0ull;
-          mine &= mine - 1;
-          j_a = front(), hot_a = s_hot[j_a], cold_a = s_cold[j_a];
-          __builtin_amdgcn_sched_barrier(0);
-          row_entry(hot_b, cold_b, j_b, active);
-        }
-      }
-      continue;
-     }
      // The record of the next entry is requested before the current one is evaluated (alternating registers): a
      // wavefront walks its list alone, so an exposed LDS round trip per entry sits on the tile's critical path.
-     if (todo == 0ull) continue;
-     auto pop = [&]() {
-       const int j = chunk * kWave + __builtin_ctzll(todo);
-       todo &= todo - 1;
-       return j;
-     };
-     auto peek = [&]() { return chunk * kWave + (todo ? __builtin_ctzll(todo) : 0); };
-     SplatHot hot_a = s_hot[peek()], hot_b;
-     while (todo) {
-       {
-         const int j = pop();
-         hot_b       = s_hot[peek()];
-         const SplatCold cold = s_cold[j];
-         __builtin_amdgcn_sched_barrier(0);
-         backward_entry(hot_a, cold, j);
-       }
-       if (todo == 0ull) break;
-       {
-         const int j = pop();
-         hot_a       = s_hot[peek()];
-         const SplatCold cold = s_cold[j];
-         __builtin_amdgcn_sched_barrier(0);
-         backward_entry(hot_b, cold, j);
-       }
+     if (todo != 0ull) {
+      auto pop = [&]() {
+        const int j = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        return j;
+      };
+      auto peek = [&]() { return todo ? (int) __builtin_ctzll(todo) : 0; };
+      SplatHot hot_a = s_hot[peek()], hot_b;
+      while (todo) {
+        {
+          const int j = pop();
+          hot_b       = s_hot[peek()];
+          const SplatCold cold = s_cold[j];
+          __builtin_amdgcn_sched_barrier(0);
+          backward_entry(hot_a, cold, j);
+        }
+        if (todo == 0ull) break;
+        {
+          const int j = pop();
+          hot_a       = s_hot[peek()];
+          const SplatCold cold = s_cold[j];
+          __builtin_amdgcn_sched_barrier(0);
+          backward_entry(hot_b, cold, j);
+        }
+      }
      }
     }
     __syncthreads();
