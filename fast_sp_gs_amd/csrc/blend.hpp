@@ -197,12 +197,36 @@ __device__ __forceinline__ unsigned quadrant_mask(const SplatHot& h, int tile_px
   }
   if (!finite_box) return 0xfu;
   const float padx = kCullPad + 0.005f * (x1 - x0), pady = kCullPad + 0.005f * (y1 - y0);
-  x0 += ox - padx, x1 += ox + padx, y0 += oy - pady, y1 += oy + pady;
+  x0 -= padx, x1 += padx, y0 -= pady, y1 += pady;
+  // The same bound along the two diagonals (the extents of x + y and of x - y over the footprint, from the same
+  // homogeneous form with the rows added / subtracted) cuts the corners off the box: an 8x8 quadrant that only meets a
+  // corner of the box of a round or diagonally stretched footprint is not met by the footprint itself.
+  float a0 = -1e30f, a1 = 1e30f, b0 = -1e30f, b1 = 1e30f;
+  {
+    const float d  = tau * (M[6] * M[6] + M[7] * M[7]) - M[8] * M[8];
+    const float inv = 1.0f / d, f0 = tau * inv, f2 = -inv;
+    const float p0 = u0 + v0, p1 = u1 + v1, p2 = u2 + v2, q0 = u0 - v0, q1 = u1 - v1, q2 = u2 - v2;
+    const float ca = f0 * (p0 * M[6] + p1 * M[7]) + f2 * (p2 * M[8]);
+    const float cb = f0 * (q0 * M[6] + q1 * M[7]) + f2 * (q2 * M[8]);
+    const float ha = ca * ca - (f0 * (p0 * p0 + p1 * p1) + f2 * (p2 * p2));
+    const float hb = cb * cb - (f0 * (q0 * q0 + q1 * q1) + f2 * (q2 * q2));
+    const float ea = sqrtf(fmaxf(ha, 0.0f)), eb = sqrtf(fmaxf(hb, 0.0f));
+    if ((ea == ea) && (eb == eb) && (ca == ca) && (cb == cb)) {
+      const float rd = 1.41421357f * r2;  // the low-pass disc along a diagonal
+      const float la = fminf(ca - ea, -rd), ua = fmaxf(ca + ea, rd), lb = fminf(cb - eb, -rd), ub = fmaxf(cb + eb, rd);
+      const float pa = 1.5f * kCullPad + 0.005f * (ua - la), pb = 1.5f * kCullPad + 0.005f * (ub - lb);
+      a0 = la - pa, a1 = ua + pa, b0 = lb - pb, b1 = ub + pb;
+    }
+  }
   unsigned m = 0u;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
-    const float qx = (float) (tile_px + (q & 1) * 8), qy = (float) (tile_py + (q >> 1) * 8);
-    if (x1 >= qx && x0 <= qx + 7.0f && y1 >= qy && y0 <= qy + 7.0f) m |= 1u << q;
+    // the quadrant's pixel centres relative to the surfel's centre
+    const float qx0 = (float) (tile_px + (q & 1) * 8) - ox, qy0 = (float) (tile_py + (q >> 1) * 8) - oy;
+    const float qx1 = qx0 + 7.0f, qy1 = qy0 + 7.0f;
+    const bool box  = x1 >= qx0 && x0 <= qx1 && y1 >= qy0 && y0 <= qy1;
+    const bool diag = a1 >= qx0 + qy0 && a0 <= qx1 + qy1 && b1 >= qx0 - qy1 && b0 <= qx1 - qy0;
+    if (box && diag) m |= 1u << q;
   }
   return m;
 }
