@@ -296,7 +296,7 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
     ranges = torch.empty((T, 2), dtype=torch.int64, device=dev)
     offsets = torch.empty((max(P, 1),), dtype=torch.int64, device=dev)
     ws1 = _workspace(lib.fsgs_gs_prepare_scan_workspace_bytes(P), dev)
-    large_count = torch.empty((1,), dtype=torch.int32, device=dev)
+    bins = _workspace(lib.fsgs_gs_prepare_bins_bytes(P, W, H), dev)
     count = _pinned_count()
     # The host has to learn the instance count before it can size point_list. Everything that does not depend on it is
     # queued behind the count's copy first -- the per-tile counting, and whatever the caller hands in as `overlap` -- so
@@ -306,7 +306,8 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
                                             count.data_ptr(), L.ptr(records), stream)
     L.check(rc, what)
     with _timed('gs_prepare_fill'):  # first of the operator's two parts: callers that time stages add them up
-        rc = lib.fsgs_gs_prepare_count(P, W, H, L.ptr(means2D), L.ptr(radii), L.ptr(ranges), L.ptr(large_count), stream)
+        rc = lib.fsgs_gs_prepare_count(P, W, H, L.ptr(means2D), L.ptr(radii), L.ptr(ranges), L.ptr(bins), bins.numel(),
+                                       stream)
     L.check(rc, what)
     overlapped = overlap(offsets) if overlap is not None else None
     L.check(lib.fsgs_gs_prepare_scan_end(), what)
@@ -316,7 +317,7 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
     ws2 = _workspace(lib.fsgs_gs_prepare_fill_workspace_bytes(R), dev)
     with _timed('gs_prepare_fill'):
         rc = lib.fsgs_gs_prepare_fill_counted(P, W, H, L.ptr(means2D), L.ptr(depths), L.ptr(radii), R, L.ptr(ranges),
-                                              L.ptr(point_list), L.ptr(keys), L.ptr(large_count), L.ptr(ws2),
+                                              L.ptr(point_list), L.ptr(keys), L.ptr(bins), bins.numel(), L.ptr(ws2),
                                               ws2.numel(), stream)
     L.check(rc, what)
     if debug:

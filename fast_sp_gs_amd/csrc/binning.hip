@@ -121,13 +121,16 @@ constexpr int kCoopThreshold = 32;  // rectangles with more tiles are walked by 
 // tiles). The same final order -- tiles ascending, inside a tile depth bits ascending, equal depths by surfel index,
 // which is what the stable radix sort leaves from the emission order -- is produced here in four steps that touch the
 // instances twice instead of twelve times:
-//   1. count the instances of every tile (64-bit atomics straight into ranges[t].y),
-//   2. exclusive scan over the tiles: ranges[t] = (start, start),
-//   3. scatter (depth bits << 32 | surfel) into the tile's segment at a position drawn from ranges[t].y, which thereby
-//      ends at the segment's end,
-//   4. one block per tile sorts its segment (unique 64-bit keys, so the arbitrary order of step 3 does not matter):
-//      bitonic network in LDS for segments up to 16384 entries, in global memory beyond that.
-// Empty tiles get (0, 0) as the reference's zero-initialised ranges have.
+//   1. count the instances of every tile: blocks of 1024 lanes walk a slice of the surfels each and count in LDS; a
+//      block's counts become one row of a (block x tile) matrix,
+//   2. prefix of every matrix column over the blocks and exclusive scan of the column totals over the tiles:
+//      ranges[t] = (start, end), final from here on,
+//   3. the same walk again scatters (depth bits << 32 | surfel) into the tile's segment; a block's cursor of a tile
+//      starts at the tile's start plus its column prefix, so neither step 1 nor step 3 issues a global atomic,
+//   4. one block per tile sorts its segment (unique 64-bit keys, so the arbitrary order inside a block's run does not
+//      matter): bitonic network in LDS for segments up to 16384 entries, in global memory beyond that.
+// Empty tiles get (0, 0) as the reference's zero-initialised ranges have. Tile grids above kMaxLdsTiles tiles (no room
+// for one LDS counter per tile) count and scatter with 64-bit global atomics on ranges[t].y instead (tile_emit_kernel).
 
 // Visits every (surfel, tile) pair; kScatter = false counts, true scatters.
 template <bool kScatter>
@@ -172,15 +175,10 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(int P, int gx, int gy, i
   }
 }
 
-// Same traversal with the same-address traffic taken off the fabric: a block of 1024 lanes walks a few thousand
-// surfels, counts their instances per tile in LDS, and touches each global tile counter once. (Device-scope atomics on
-// one address are served one after the other at fabric latency; the busiest tile of a frame would otherwise receive a
-// thousand of them.) kScatter = true additionally reserves a contiguous run per (block, tile) and walks the surfels a
-// second time to place the entries. Needs T <= kMaxLdsTiles.
+// The same traversal with the counters in LDS, one per tile (tile grids up to kMaxLdsTiles tiles): blocks of 1024 lanes
+// walk a slice of the surfels each; what they do with an instance is up to the caller (tile_hist_kernel,
+// tile_scatter_kernel).
 constexpr int kMaxLdsTiles = 16384;
-#ifndef FSGS_EMIT_PER_BLOCK
-#define FSGS_EMIT_PER_BLOCK 2048
-#endif
 
 template <typename Visit>
 __device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, const float2* __restrict__ means2D,
@@ -210,11 +208,33 @@ __device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, 
   }
 }
 
-template <bool kScatter>
-__global__ void __launch_bounds__(1024) tile_emit_lds_kernel(int P, int per_block, int gx, int gy, int64_t R,
-    const float2* __restrict__ means2D, const float* __restrict__ depths, const int32_t* __restrict__ radii,
-    unsigned long long* __restrict__ ranges, uint64_t* __restrict__ entries) {
-  __shared__ unsigned s_count[kMaxLdsTiles];  // instances of this block per tile, then the block's cursor per tile
+// Layout of the `bins` buffer of the bucket binning: the queue length of the long segments in front of the B x T matrix
+// of per-(walk block, tile) instance counts.
+constexpr size_t kBinsHeader = 256;
+constexpr int kPrefixTiles = 64, kPrefixWaves = 16, kPrefixChunk = 32;  // walk blocks <= kPrefixWaves * kPrefixChunk
+struct BinsLayout {
+  int blocks;      // walk blocks B (0: the tile grid is too large for LDS counters, the global-atomic path is used)
+  int per_block;   // surfels per walk block
+  size_t bytes;
+};
+inline BinsLayout bins_layout(int P, int T) {
+  BinsLayout l{0, 0, kBinsHeader};
+  if (T > kMaxLdsTiles || P <= 0) return l;
+  // one 1024-lane block per 1024 surfels while that keeps every block resident at once (two fit on a compute unit),
+  // beyond that the blocks grow
+  l.per_block = 1024 * std::max(1, div_up(P, 1024 * kPrefixWaves * kPrefixChunk));
+  l.blocks    = div_up(P, l.per_block);
+  l.bytes     = kBinsHeader + align_up((size_t) l.blocks * T * sizeof(uint32_t), 256);
+  return l;
+}
+
+// Step 1: every block counts the instances of its surfels per tile in LDS and writes its row of the matrix with plain
+// stores (zeros included, so the matrix needs no clearing). No global atomics: device-scope atomics on one address are
+// served one after the other at fabric latency, and with surfels in no spatial order every block touches nearly
+// every tile.
+__global__ void __launch_bounds__(1024) tile_hist_kernel(int P, int per_block, int gx, int gy,
+    const float2* __restrict__ means2D, const int32_t* __restrict__ radii, uint32_t* __restrict__ hist) {
+  __shared__ unsigned s_count[kMaxLdsTiles];
   const int T = gx * gy;
   for (int t = threadIdx.x; t < T; t += blockDim.x) s_count[t] = 0u;
   __syncthreads();
@@ -226,26 +246,73 @@ __global__ void __launch_bounds__(1024) tile_emit_lds_kernel(int P, int per_bloc
     for_each_instance(i < last ? i : P, P, gx, gy, means2D, radii, [&](int tile, int) { atomicAdd(&s_count[tile], 1u); });
   }
   __syncthreads();
-  for (int t = threadIdx.x; t < T; t += blockDim.x) {
-    const unsigned c = s_count[t];
-    if (c == 0u) continue;
-    if (kScatter) s_count[t] = (unsigned) atomicAdd(ranges + 2 * (size_t) t + 1, (unsigned long long) c);
-    else atomicAdd(ranges + 2 * (size_t) t + 1, (unsigned long long) c);
+  uint32_t* row = hist + (size_t) blockIdx.x * T;
+  for (int t = threadIdx.x; t < T; t += blockDim.x) row[t] = s_count[t];
+}
+
+// Step 2: per tile, the exclusive prefix of its column over the walk blocks (in place) and the column total, which goes
+// to ranges[t].y for tile_scan_kernel. 64 tiles per block, lane = tile, the 16 wavefronts share the walk blocks in
+// contiguous chunks so that a wavefront's loads are all in flight at once.
+__global__ void __launch_bounds__(kPrefixTiles * kPrefixWaves) tile_prefix_kernel(int T, int B,
+    uint32_t* __restrict__ hist, unsigned long long* __restrict__ ranges) {
+  __shared__ uint32_t s_sum[kPrefixWaves][kPrefixTiles];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int t = blockIdx.x * kPrefixTiles + lane;
+  const int chunk = (B + kPrefixWaves - 1) / kPrefixWaves, b0 = wave * chunk;
+  // a wavefront's whole chunk of the column is loaded before anything is written back (B <= 512: at most 32 values per
+  // lane), so the loads are in flight together; a load placed behind a store to the same array would wait for it
+  uint32_t c[kPrefixChunk], sum = 0;
+#pragma unroll
+  for (int i = 0; i < kPrefixChunk; ++i) {
+    const int b = b0 + i;
+    c[i] = (t < T && i < chunk && b < B) ? hist[(size_t) b * T + t] : 0u;
+    sum += c[i];
   }
-  if (!kScatter) return;
+  s_sum[wave][lane] = sum;
   __syncthreads();
+  uint32_t run = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < kPrefixWaves; ++w) {
+    const uint32_t v = s_sum[w][lane];
+    if (w < wave) run += v;
+    total += v;
+  }
+  if (t < T) {
+#pragma unroll
+    for (int i = 0; i < kPrefixChunk; ++i) {
+      const int b = b0 + i;
+      if (i < chunk && b < B) hist[(size_t) b * T + t] = run;
+      run += c[i];
+    }
+    if (wave == 0) ranges[2 * (size_t) t + 1] = total;
+  }
+}
+
+// Step 3: the walk of step 1 again; a block's cursor of a tile starts at the tile's start plus the instances of the
+// blocks in front of it, so the placement needs no global atomics either.
+__global__ void __launch_bounds__(1024) tile_scatter_kernel(int P, int per_block, int gx, int gy, int64_t R,
+    const float2* __restrict__ means2D, const float* __restrict__ depths, const int32_t* __restrict__ radii,
+    const uint32_t* __restrict__ hist, const unsigned long long* __restrict__ ranges, uint64_t* __restrict__ entries) {
+  __shared__ unsigned s_cursor[kMaxLdsTiles];
+  const int T = gx * gy;
+  const uint32_t* row = hist + (size_t) blockIdx.x * T;
+  for (int t = threadIdx.x; t < T; t += blockDim.x) s_cursor[t] = (unsigned) ranges[2 * (size_t) t] + row[t];
+  __syncthreads();
+  const int first = blockIdx.x * per_block, last = min(P, first + per_block);
+  const int rounds = (last - first + (int) blockDim.x - 1) / (int) blockDim.x;
   for (int r = 0; r < rounds; ++r) {
     const int i = first + r * blockDim.x + threadIdx.x;
     for_each_instance(i < last ? i : P, P, gx, gy, means2D, radii, [&](int tile, int id) {
-      const unsigned pos = atomicAdd(&s_count[tile], 1u);
+      const unsigned pos = atomicAdd(&s_cursor[tile], 1u);
       if ((int64_t) pos < R) entries[pos] = ((uint64_t) __float_as_uint(depths[id]) << 32) | (uint32_t) id;
     });
   }
 }
 
 // One block: exclusive scan of the per-tile counts, 4 tiles per lane and step.
+// ends = false: ranges[t] = (start, start), for a scatter that advances ranges[t].y; ends = true: (start, end).
 __global__ void __launch_bounds__(1024) tile_scan_kernel(int T, unsigned long long* __restrict__ ranges,
-                                                         int* __restrict__ large_count) {
+                                                         int* __restrict__ large_count, bool ends) {
   __shared__ unsigned long long s_wave[16];
   const int lane = __lane_id(), wave = threadIdx.x / kWave;
   unsigned long long carry = 0;
@@ -268,7 +335,7 @@ __global__ void __launch_bounds__(1024) tile_scan_kernel(int T, unsigned long lo
     unsigned long long run = carry + base + inc - sum;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      if (t0 + k < T) ranges[2 * (size_t) (t0 + k)] = run, ranges[2 * (size_t) (t0 + k) + 1] = run;
+      if (t0 + k < T) ranges[2 * (size_t) (t0 + k)] = run, ranges[2 * (size_t) (t0 + k) + 1] = ends ? run + c[k] : run;
       run += c[k];
     }
     carry += total;
@@ -765,51 +832,60 @@ FSGS_API int fsgs_gs_prepare_sort_bits(int W, int H) {
 }
 
 namespace {
-// First part of the bucket binning, independent of the instance count: zero the ranges, count the instances of every
-// tile into ranges[t].y, scan them to ranges[t] = (start, start); *large_count is reset.
-int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, int64_t* ranges, int* large_count,
+// First part of the bucket binning, independent of the instance count: per-tile instance counts and the tile ranges
+// (start, end); the long-segment queue's counter (first word of `bins`) is reset.
+int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, int64_t* ranges, void* bins,
                hipStream_t s) {
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int T  = gx * gy;
-  hipLaunchKernelGGL(fill_zero_i64_kernel, dim3(div_up(2 * (int64_t) T, 256)), dim3(256), 0, s, 2 * (int64_t) T,
-                     ranges);
   unsigned long long* rng = (unsigned long long*) ranges;
-  if (P > 0) {
-    // the LDS-aggregated traversal needs one LDS counter per tile; larger tile grids count straight in global memory
-    const bool lds_path = T <= kMaxLdsTiles;
-    const int per_block = std::max(FSGS_EMIT_PER_BLOCK, div_up(P, 256));
-    if (lds_path)
-      hipLaunchKernelGGL(tile_emit_lds_kernel<false>, dim3(div_up(P, per_block)), dim3(1024), 0, s, P, per_block, gx, gy,
-                         (int64_t) 0, (const float2*) means2D, (const float*) nullptr, radii, rng, (uint64_t*) nullptr);
-    else
+  int* header = (int*) bins;
+  const BinsLayout bl = bins_layout(P, T);
+  if (bl.blocks > 0) {
+    uint32_t* hist = (uint32_t*) ((char*) bins + kBinsHeader);
+    hipLaunchKernelGGL(tile_hist_kernel, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
+                       (const float2*) means2D, radii, hist);
+    hipLaunchKernelGGL(tile_prefix_kernel, dim3(div_up(T, kPrefixTiles)), dim3(kPrefixTiles * kPrefixWaves), 0, s, T,
+                       bl.blocks, hist, rng);
+    hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, true);
+    // The ranges are final here, before the instance count has even reached the host: the schedule table the blend
+    // kernels of this frame are going to use (they find it under this ranges buffer's key) is built now, in the shadow of
+    // the host's wait; it orders the per-tile sorts as well.
+    const int* order = nullptr;
+    (void) launch_tile_order(gx, gy, ranges, s, &order);
+  } else {
+    // no room for one LDS counter per tile (or no surfels): count straight into ranges[t].y, then scan to (start, start)
+    hipLaunchKernelGGL(fill_zero_i64_kernel, dim3(div_up(2 * (int64_t) T, 256)), dim3(256), 0, s, 2 * (int64_t) T,
+                       ranges);
+    if (P > 0)
       hipLaunchKernelGGL(tile_emit_kernel<false>, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, (int64_t) 0,
                          (const float2*) means2D, (const float*) nullptr, radii, rng, (uint64_t*) nullptr);
+    hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, false);
   }
-  hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, large_count);
   return check_launch("gs_prepare_count");
 }
 
 // Second part: scatter (depth bits << 32 | surfel) into the tile segments and sort every segment.
 int fill_sort(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii, int64_t R,
-              int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out, void* workspace, int* large_count,
+              int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out, void* workspace, void* bins,
               hipStream_t s) {
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int T  = gx * gy;
   unsigned long long* rng = (unsigned long long*) ranges;
   uint64_t* entries       = sort_keys_in(R, workspace);
-  const bool lds_path = T <= kMaxLdsTiles;
-  const int per_block = std::max(FSGS_EMIT_PER_BLOCK, div_up(P, 256));
-  // queue of long segments: at most R / kSmallSegment tiles, kept behind the entries in the workspace (its first
-  // word is where fsgs_gs_prepare_fill keeps the queue's counter)
-  int* large_list = (int*) ((char*) workspace + sort_layout(R).keys1) + 1;
-  if (lds_path)
-    hipLaunchKernelGGL(tile_emit_lds_kernel<true>, dim3(div_up(P, per_block)), dim3(1024), 0, s, P, per_block, gx, gy, R,
-                       (const float2*) means2D, depths, radii, rng, entries);
+  int* large_count        = (int*) bins;
+  // queue of long segments: at most R / kSmallSegment tiles, kept behind the entries in the workspace
+  int* large_list = (int*) ((char*) workspace + sort_layout(R).keys1);
+  const BinsLayout bl = bins_layout(P, T);
+  if (bl.blocks > 0)
+    hipLaunchKernelGGL(tile_scatter_kernel, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
+                       (const float2*) means2D, depths, radii, (const uint32_t*) ((const char*) bins + kBinsHeader), rng,
+                       entries);
   else
     hipLaunchKernelGGL(tile_emit_kernel<true>, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
                        (const float2*) means2D, depths, radii, rng, entries);
-  // The ranges are final here: the schedule table the blend kernels of this frame are going to use is built now (they
-  // find it under this ranges buffer's key) and orders the per-tile sorts as well.
+  // the schedule table built by the counting part (or built now, on the global-atomic path, whose ranges only become
+  // final with the scatter)
   const int* order = nullptr;
   (void) launch_tile_order(gx, gy, ranges, s, &order);
   hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
@@ -820,33 +896,44 @@ int fill_sort(int P, int W, int H, const float* means2D, const float* depths, co
 }
 }  // namespace
 
+FSGS_API size_t fsgs_gs_prepare_bins_bytes(int P, int W, int H) {
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  return bins_layout(P, gx * gy).bytes;
+}
+
 FSGS_API int fsgs_gs_prepare_count(int P, int W, int H, const float* means2D, const int32_t* radii, int64_t* ranges,
-                                   int32_t* large_count, void* stream) {
-  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && ranges && large_count, "gs_prepare_count: bad arguments");
+                                   void* bins, size_t bins_bytes, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && ranges && bins, "gs_prepare_count: bad arguments");
   FSGS_REQUIRE(P == 0 || (means2D && radii), "gs_prepare_count: null pointer");
+  if (bins_bytes < fsgs_gs_prepare_bins_bytes(P, W, H))
+    return fail(kWorkspaceSmall, "gs_prepare_count: bins %zu < %zu bytes", bins_bytes,
+                fsgs_gs_prepare_bins_bytes(P, W, H));
   tile_order_invalidate((hipStream_t) stream);  // the ranges are rewritten: the blend schedule of this stream is stale
-  return fill_count(P, W, H, means2D, radii, ranges, large_count, (hipStream_t) stream);
+  return fill_count(P, W, H, means2D, radii, ranges, bins, (hipStream_t) stream);
 }
 
 FSGS_API int fsgs_gs_prepare_fill_counted(int P, int W, int H, const float* means2D, const float* depths,
                                           const int32_t* radii, int64_t R, int64_t* ranges, int32_t* point_list,
-                                          int64_t* sorted_keys_out, int32_t* large_count, void* workspace,
+                                          int64_t* sorted_keys_out, void* bins, size_t bins_bytes, void* workspace,
                                           size_t workspace_bytes, void* stream) {
-  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && R >= 0 && ranges && large_count, "gs_prepare_fill: bad arguments");
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && R >= 0 && ranges && bins, "gs_prepare_fill: bad arguments");
   FSGS_REQUIRE(R < (int64_t) 0x7fffffff, "gs_prepare_fill: %lld instances exceed the 2^31-1 limit", (long long) R);
-  if (R == 0 || P == 0) return kOk;  // the counting part left every range at (0, 0)
+  if (R == 0 || P == 0) return kOk;  // the counting part left every range empty
   FSGS_REQUIRE(means2D && depths && radii && point_list && workspace, "gs_prepare_fill: null pointer");
   if (workspace_bytes < sort_workspace_bytes(R))
     return fail(kWorkspaceSmall, "gs_prepare_fill: workspace %zu < %zu bytes", workspace_bytes,
                 sort_workspace_bytes(R));
-  return fill_sort(P, W, H, means2D, depths, radii, R, ranges, point_list, sorted_keys_out, workspace, large_count,
+  if (bins_bytes < fsgs_gs_prepare_bins_bytes(P, W, H))
+    return fail(kWorkspaceSmall, "gs_prepare_fill: bins %zu < %zu bytes", bins_bytes,
+                fsgs_gs_prepare_bins_bytes(P, W, H));
+  return fill_sort(P, W, H, means2D, depths, radii, R, ranges, point_list, sorted_keys_out, workspace, bins,
                    (hipStream_t) stream);
 }
 
 FSGS_API int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths,
                                   const int32_t* radii, const int64_t* point_offsets, int64_t R, int64_t* ranges,
-                                  int32_t* point_list, int64_t* sorted_keys_out, void* workspace,
-                                  size_t workspace_bytes, void* stream) {
+                                  int32_t* point_list, int64_t* sorted_keys_out, void* bins, size_t bins_bytes,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && R >= 0 && ranges, "gs_prepare_fill: bad arguments");
   FSGS_REQUIRE(R < (int64_t) 0x7fffffff, "gs_prepare_fill: %lld instances exceed the 2^31-1 limit", (long long) R);
   hipStream_t s = (hipStream_t) stream;
@@ -857,13 +944,14 @@ FSGS_API int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, con
                        2 * (int64_t) gx * gy, ranges);
     return check_launch("gs_prepare_fill(zero)");
   }
-  FSGS_REQUIRE(means2D && depths && radii && point_offsets && point_list && workspace,
+  FSGS_REQUIRE(means2D && depths && radii && point_offsets && point_list && workspace && bins,
                "gs_prepare_fill: null pointer");
   if (workspace_bytes < sort_workspace_bytes(R))
     return fail(kWorkspaceSmall, "gs_prepare_fill: workspace %zu < %zu bytes", workspace_bytes,
                 sort_workspace_bytes(R));
-  // the counter of long segments sits in front of their list, behind the entries in the workspace
-  int* large_count = (int*) ((char*) workspace + sort_layout(R).keys1);
-  if (int rc = fill_count(P, W, H, means2D, radii, ranges, large_count, s)) return rc;
-  return fill_sort(P, W, H, means2D, depths, radii, R, ranges, point_list, sorted_keys_out, workspace, large_count, s);
+  if (bins_bytes < fsgs_gs_prepare_bins_bytes(P, W, H))
+    return fail(kWorkspaceSmall, "gs_prepare_fill: bins %zu < %zu bytes", bins_bytes,
+                fsgs_gs_prepare_bins_bytes(P, W, H));
+  if (int rc = fill_count(P, W, H, means2D, radii, ranges, bins, s)) return rc;
+  return fill_sort(P, W, H, means2D, depths, radii, R, ranges, point_list, sorted_keys_out, workspace, bins, s);
 }

@@ -76,31 +76,35 @@ int fsgs_gs_prepare_scan(int P, const int32_t* tiles_touched, int64_t* point_off
 
 /* Phase 2: key duplication, stable sort on bits [0, 32 + msb(T)), tile ranges (gaussian_prepare.cu:47-83, 254-277,
  * 192-220). ranges[T,2] int64 (empty tile = (0,0)), point_list[R] int32. sorted_keys_out[R] (optional) receives the
- * sorted 64-bit keys (tile << 32 | depth bits). */
+ * sorted 64-bit keys (tile << 32 | depth bits). Two caller buffers, neither needs clearing: `workspace` of
+ * fsgs_gs_prepare_fill_workspace_bytes(R) bytes for the unsorted entries, and `bins` of
+ * fsgs_gs_prepare_bins_bytes(P, W, H) bytes for the per-tile instance counts of the surfel slices (known before R is). */
 size_t fsgs_gs_prepare_fill_workspace_bytes(int64_t R);
+size_t fsgs_gs_prepare_bins_bytes(int P, int W, int H);
 int fsgs_gs_prepare_sort_bits(int W, int H);
 int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
                          const int64_t* point_offsets, int64_t R, int64_t* ranges, int32_t* point_list,
-                         int64_t* sorted_keys_out, void* workspace, size_t workspace_bytes, void* stream);
+                         int64_t* sorted_keys_out, void* bins, size_t bins_bytes, void* workspace,
+                         size_t workspace_bytes, void* stream);
 
 /* The same two phases cut where the host has to wait, for callers that want the device to stay busy meanwhile (no
  * counterpart in the reference, which blocks inside GS_prepare). fsgs_gs_prepare_scan_begin queues the scan and the
  * copy of the instance count into *num_rendered_host (page-locked memory, or the copy is not asynchronous) and
  * returns; fsgs_gs_prepare_scan_end blocks the calling host thread until that copy has landed (one scan in flight per
  * host thread). Work queued on the stream in between runs while the host waits and allocates: fsgs_gs_prepare_count is
- * the part of the fill that does not need the count (zeroes ranges[T,2], counts the instances per tile, scans them,
- * resets *large_count, a device int32 the caller keeps until the fill has run); fsgs_gs_prepare_fill_counted is the rest
- * (scatter + per-tile sort). scan_begin + scan_end == fsgs_gs_prepare_scan, count + fill_counted == fsgs_gs_prepare_fill.
+ * the part of the fill that does not need the count (counts the instances per tile into `bins`, writes the final
+ * ranges[T,2]; the caller keeps `bins` until the fill has run); fsgs_gs_prepare_fill_counted is the rest (scatter +
+ * per-tile sort). scan_begin + scan_end == fsgs_gs_prepare_scan, count + fill_counted == fsgs_gs_prepare_fill.
  * records (optional): the packed per-surfel records fsgs_gs_2d_preprocess_forward wrote; the scan stores every surfel's
  * exclusive offset into the last word of its record, where the blend backward's ordered-sum path looks for it. */
 int fsgs_gs_prepare_scan_begin(int P, const int32_t* tiles_touched, int64_t* point_offsets, void* workspace,
                                size_t workspace_bytes, int64_t* num_rendered_host, float* records, void* stream);
 int fsgs_gs_prepare_scan_end(void);
 int fsgs_gs_prepare_count(int P, int W, int H, const float* means2D, const int32_t* radii, int64_t* ranges,
-                          int32_t* large_count, void* stream);
+                          void* bins, size_t bins_bytes, void* stream);
 int fsgs_gs_prepare_fill_counted(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
                                  int64_t R, int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out,
-                                 int32_t* large_count, void* workspace, size_t workspace_bytes, void* stream);
+                                 void* bins, size_t bins_bytes, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- per-tile alpha blend ------------------------------------------------------------------------------------- */
 

@@ -90,8 +90,10 @@ def test_blocking_entry_points_match_the_operator(device):
     ranges2 = torch.empty((T, 2), dtype=torch.int64, device=device)
     pl2 = torch.empty(R.value, dtype=torch.int32, device=device)
     ws2 = torch.empty(lib.fsgs_gs_prepare_fill_workspace_bytes(R.value), dtype=torch.uint8, device=device)
+    bins = torch.empty(lib.fsgs_gs_prepare_bins_bytes(P, W, H), dtype=torch.uint8, device=device)
+    bins.fill_(0xff)  # neither buffer needs clearing
     L.check(lib.fsgs_gs_prepare_fill(P, W, H, L.ptr(m2), L.ptr(dep), L.ptr(radii), L.ptr(off2), R.value, L.ptr(ranges2),
-                                     L.ptr(pl2), None, L.ptr(ws2), ws2.numel(), stream), 'fill')
+                                     L.ptr(pl2), None, L.ptr(bins), bins.numel(), L.ptr(ws2), ws2.numel(), stream), 'fill')
     torch.cuda.synchronize()
     assert torch.equal(ranges2, ranges) and torch.equal(pl2, pl)
 
