@@ -88,6 +88,12 @@ class AdaptiveControl:
     param_names_map = {'_xyz': 'xyz', '_features_dc': 'f_dc', '_features_rest': 'f_rest', '_scaling': 'scaling',
                        '_rotation': 'rotation', '_opacity': 'opacity'}
     is_surfel = True
+    # Per-point tensors of the host class that are not optimised but have to follow every structural change: a new point
+    # takes its parent's row, a pruned point's row goes. The superpoint model keeps three of them -- the per-frame culling
+    # flags, the visibility factor of the gradient statistics and the superpoint assignment (network.py:1195-1215) --
+    # which the reference carries along with `t[valid]` / `cat((t, t[mask]))` / `cat((t, t[mask].repeat(N, 1)))`. Here they
+    # go through the same row table as the parameters; attributes that are absent, None or empty are skipped.
+    per_point_buffers = ('_culling', 'factor_culling', 'p2sp')
 
     @property
     def get_scaling(self) -> Tensor:
@@ -130,15 +136,29 @@ class AdaptiveControl:
                 grad += p.grad
         # the kernel reads "radii > 0": hand it the filter as 0 / 1 radii and leave max_radii2D alone
         scratch = torch.zeros_like(self.max_radii2D)
+        # the superpoint model weighs a point's gradient norm by its visibility factor (network.py:1153)
+        factor = getattr(self, 'factor_culling', None)
+        if factor is not None and factor.numel() != self._xyz.shape[0]:
+            factor = None
         get_C_function('densification_stats')(update_filter.to(torch.int32), grad.contiguous(), scratch,
-                                              self.xyz_gradient_accum, self.denom, None)
+                                              self.xyz_gradient_accum, self.denom,
+                                              None if factor is None else factor.reshape(-1).contiguous())
 
     # ---- structural changes ------------------------------------------------------------------------------------------
     def _restructure(self, optimizer, source_row: Tensor, new_rows: int = 0, tail: Optional[Dict[str, Tensor]] = None,
                reset_statistics: bool = False):
+        P_old = self._xyz.shape[0]
         new = restructure_optimizer(optimizer, list(self.param_names_map.values()), source_row, new_rows, tail)
         for param_name, opt_name in self.param_names_map.items():
             setattr(self, param_name, new[opt_name])
+        carried = [n for n in self.per_point_buffers
+                   if isinstance(getattr(self, n, None), Tensor) and getattr(self, n).ndim >= 1 and
+                   getattr(self, n).shape[0] == P_old and P_old > 0]
+        if carried:
+            # densification_postfix marks its appended rows -1 (they come from `tail`); such rows have no parent to copy
+            # from, so they read zeros, as a model that appends foreign points has to fill them itself anyway
+            for n, t in zip(carried, get_C_function('gather_rows')([getattr(self, n) for n in carried], source_row)):
+                setattr(self, n, t)
         if reset_statistics:  # gaussian_splatting.py:575-578
             self.training_setup()
         else:  # gaussian_splatting.py:566-568

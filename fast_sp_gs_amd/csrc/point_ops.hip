@@ -104,8 +104,9 @@ __global__ void __launch_bounds__(256) sh_to_rgb_backward_kernel(int P, int F, i
 
 // ---- element types of the small operators -------------------------------------------------------------------------------
 // The encoders and the nearest / farthest search accept the floating types the reference dispatches on. Half precision
-// is a storage format only: values are widened on load, the arithmetic is single precision, the result is rounded once
-// on store.
+// is a storage format: values are widened on load, the arithmetic is single precision, the result is rounded once on
+// store -- except where the reference itself keeps intermediates in half (the SH encoder's monomials and backward sums,
+// restated for degree <= 3 in sh_eval_half / sh_grad_half).
 template <typename T> struct Arith { using type = T; };
 template <> struct Arith<_Float16> { using type = float; };
 
@@ -117,7 +118,10 @@ __global__ void __launch_bounds__(256) sh_encode_forward_kernel(int B, int D, in
   const int b = blockIdx.x * blockDim.x + threadIdx.x;
   if (b >= B) return;
   A Y[kSh];
-  sh_eval(C, (A) in[(size_t) b * D], (A) in[(size_t) b * D + 1], (A) in[(size_t) b * D + 2], Y);
+  if constexpr (std::is_same<T, _Float16>::value && kSh == 16)
+    sh_eval_half(C, (A) in[(size_t) b * D], (A) in[(size_t) b * D + 1], (A) in[(size_t) b * D + 2], Y);
+  else
+    sh_eval(C, (A) in[(size_t) b * D], (A) in[(size_t) b * D + 1], (A) in[(size_t) b * D + 2], Y);
   const int n = sh_count(C);
   T* o        = out + (size_t) b * n;
   if constexpr (std::is_same<T, float>::value) {
@@ -151,7 +155,10 @@ __global__ void __launch_bounds__(256) sh_encode_backward_kernel(int B, int D, i
   if (!loaded)
     for (int l = 0; l < n; ++l) t[l] = (A) g[l];
   A dx = 0, dy = 0, dz = 0;
-  sh_grad_accumulate(C, (A) in[(size_t) b * D], (A) in[(size_t) b * D + 1], (A) in[(size_t) b * D + 2], t, dx, dy, dz);
+  if constexpr (std::is_same<T, _Float16>::value && kSh == 16)
+    sh_grad_half(C, (A) in[(size_t) b * D], (A) in[(size_t) b * D + 1], (A) in[(size_t) b * D + 2], t, dx, dy, dz);
+  else
+    sh_grad_accumulate(C, (A) in[(size_t) b * D], (A) in[(size_t) b * D + 1], (A) in[(size_t) b * D + 2], t, dx, dy, dz);
   grad_in[(size_t) b * D] = (T) dx, grad_in[(size_t) b * D + 1] = (T) dy, grad_in[(size_t) b * D + 2] = (T) dz;
 }
 

@@ -248,26 +248,51 @@ def calc_LBS_weight(points: Tensor, sp_points: Tensor, feature: Tensor = None, s
     return weights, indices
 
 
+def assign_superpoints(weights: Tensor, indices: Tensor) -> Tensor:
+    """p2sp of the reference (network.py:594): for every Gaussian the neighbour that carries its largest weight."""
+    return torch.gather(indices, -1, weights.argmax(dim=-1, keepdim=True))[:, 0]
+
+
+def _rigid_by_assignment(points, sp_points, sp_t, sp_r, sp_rot, p2sp):
+    """warp_method 'largest' (network.py:555-561): every Gaussian is moved by the rigid transform of ONE control point,
+    `spT[p2sp].act(points) - points`, no blend. The blend kernel with K = 1 and a weight of one is exactly that gather
+    (and its backward the scatter of the gradients to the assigned control points)."""
+    one = points.new_ones(points.shape[0], 1)
+    d_xyz, _, _, _ = _LbsBlend.apply(points, sp_points, sp_t, sp_r, None, sp_rot, one, p2sp.long()[:, None].contiguous(),
+                                     None, None, 1.0, 'LBS', 'given')
+    return d_xyz
+
+
 def warp(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_s: Tensor, sp_rot: Tensor, weights: Tensor,
-         indices: Tensor, method: str = 'LBS'):
-    """The reference's `warp` (network.py:523-573) for apply_rotate == 'add' and methods 'LBS' / 'LBS_c' on finished
-    weights -> (d_points, d_rotation, d_scales). Without `sp_rot` (no local rotation, the default configuration) the
-    translations are blended; with it every Gaussian is moved by the blended rigid transforms
-    (normalize(sp_rot + (0,0,0,1)), sp_t), about the control point for 'LBS_c'. Differentiable in everything but the
-    indices."""
-    d_xyz, d_rot, d_scale, _ = _LbsBlend.apply(points, sp_points, sp_t, sp_r, sp_s, sp_rot, weights, indices, None,
-                                               None, 1.0, method if sp_rot is not None else None, 'given')
+         indices: Tensor, method: str = 'LBS', p2sp: Tensor = None):
+    """The reference's `warp` (network.py:523-573) for apply_rotate == 'add' on finished weights ->
+    (d_points, d_rotation, d_scales). Without `sp_rot` (no local rotation, the default configuration) the translations
+    are blended whatever the method; with it every Gaussian is moved by rigid transforms
+    (normalize(sp_rot + (0,0,0,1)), sp_t): blended over its neighbours for 'LBS', blended about the control points
+    for 'LBS_c', and for 'largest' the one transform of its assigned control point `p2sp` (default: the neighbour with
+    the largest weight, as sp_stage assigns it, :594). Rotation and scale residuals are blended in every case.
+    Differentiable in everything but the indices."""
+    if method not in ('LBS', 'LBS_c', 'largest'):
+        raise ValueError(f'unknown warp method {method!r}')  # the reference's assert, network.py:205
+    blended = method if (sp_rot is not None and method != 'largest') else None
+    d_xyz, d_rot, d_scale, _ = _LbsBlend.apply(points, sp_points, sp_t, sp_r, sp_s, sp_rot if blended else None, weights,
+                                               indices, None, None, 1.0, blended, 'given')
+    if method == 'largest' and sp_rot is not None:
+        if p2sp is None:
+            p2sp = assign_superpoints(weights.detach(), indices)
+        d_xyz = _rigid_by_assignment(points, sp_points, sp_t, sp_r, sp_rot, p2sp)
     return d_xyz, d_rot, d_scale
 
 
 def superpoint_deform(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Tensor, sp_s: Tensor,
                       sp_rot: Tensor = None, K: int = 3, temperature: float = 1.0, warp_method: str = 'LBS',
                       LBS_method: str = 'dist', sp_radius: Tensor = None, sp_weight: Tensor = None,
-                      sp_W: Tensor = None, feature: Tensor = None, sp_feature: Tensor = None):
+                      sp_W: Tensor = None, feature: Tensor = None, sp_feature: Tensor = None, p2sp: Tensor = None):
     """`calc_LBS_weight` + `warp` of the reference's `sp_stage` (network.py:576-599) with the weights formed inside the
     blend kernels: K-NN of the Gaussians to the control points (on positions, or on positions + hyper features when
     `feature` / `sp_feature` are given, :500-504), weights by `LBS_method` ('dist', 'kernel', 'weighted_kernel', 'W'),
-    then the warp. Returns (d_xyz, d_rot, d_scale, weights, indices). Differentiable with respect to sp_points and the
+    then the warp ('LBS', 'LBS_c', or 'largest' with the assignment `p2sp`, by default the neighbour of largest
+    weight). Returns (d_xyz, d_rot, d_scale, weights, indices). Differentiable with respect to sp_points and the
     hyper features (through the distances, and sp_points also through the pivot of 'LBS_c'), sp_t, sp_r, sp_s, sp_rot,
     sp_radius, sp_weight and sp_W; the returned weights are detached. As in the reference the Gaussians' positions are
     detached (:577, :501)."""
@@ -286,9 +311,14 @@ def superpoint_deform(points: Tensor, sp_points: Tensor, sp_t: Tensor, sp_r: Ten
         pair_in, radius, weight = d2, None, None
     else:
         raise ValueError(f'unknown LBS_method {LBS_method!r}')
-    d_xyz, d_rot, d_scale, w = _LbsBlend.apply(points, sp_points, sp_t, sp_r, sp_s, sp_rot, pair_in, idx, radius,
-                                               weight, temperature, warp_method if sp_rot is not None else None,
-                                               LBS_method)
+    if warp_method not in ('LBS', 'LBS_c', 'largest'):
+        raise ValueError(f'unknown warp method {warp_method!r}')
+    blended = warp_method if (sp_rot is not None and warp_method != 'largest') else None
+    d_xyz, d_rot, d_scale, w = _LbsBlend.apply(points, sp_points, sp_t, sp_r, sp_s, sp_rot if blended else None, pair_in,
+                                               idx, radius, weight, temperature, blended, LBS_method)
+    if warp_method == 'largest' and sp_rot is not None:
+        p2sp = assign_superpoints(w, idx) if p2sp is None else p2sp
+        d_xyz = _rigid_by_assignment(points, sp_points, sp_t, sp_r, sp_rot, p2sp)
     return d_xyz, d_rot, d_scale, w, idx
 
 

@@ -544,7 +544,10 @@ int fsgs_mlp_forward(int B, int Din, int width, int n_layers, int skip, int n_ou
  * of the weight transposed to [256 in][256 out] bf16 (fsgs_pack_bf16 of the transposed slice); heads_w[n_out][256] and
  * g_out[B][n_out] are fp32. Outputs, fully written: g_w = the layers' [256][K_l] gradients back to back (unpadded,
  * K_0 = Din, K_{skip+1} = Din + 256, else 256) followed by the heads' [n_out][256]; g_b[n_layers*256 + n_out].
- * Operands are bf16, accumulation fp32. No gradient is produced for `in`. */
+ * Operands are bf16, accumulation fp32. No gradient is produced for `in` directly; the workspace carries what a caller
+ * needs to form it: after the call its first n_layers * B * 256 * 2 bytes hold dZ[n_layers][B][256] in bf16, the
+ * gradient of every layer's pre-activation (masked by the stored state's zeros), so that
+ * dL/d in = dZ[0] W_0 + dZ[skip+1] W_{skip+1}[:, :Din]. The rest of the workspace is scratch. */
 size_t fsgs_mlp_backward_workspace_bytes(int B, int n_layers);
 int fsgs_mlp_backward(int B, int Din, int width, int n_layers, int skip, int n_out, const float* in,
     const uint16_t* packed_t, const float* heads_w, const uint16_t* saved, const float* g_out, float* g_w, float* g_b,

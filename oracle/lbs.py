@@ -52,8 +52,10 @@ def lbs_weights(pair_in: torch.Tensor, indices: torch.Tensor, M: int, method: st
     raise ValueError(method)
 
 
-def warp(points, sp_points, sp_t, sp_r, sp_s, sp_rot, weights, indices, method='LBS'):
-    """network.py:545-573 -> (d_points, d_rotation, d_scales). sp_rot None: translations only (:563-564)."""
+def warp(points, sp_points, sp_t, sp_r, sp_s, sp_rot, weights, indices, method='LBS', p2sp=None):
+    """network.py:545-573 -> (d_points, d_rotation, d_scales). sp_rot None: translations only (:563-564). Any method
+    other than 'LBS' / 'LBS_c' takes the reference's last branch (:555-561): every point is moved by the transform of its
+    assigned control point `p2sp` ([N] indices; sp_stage assigns the neighbour of largest weight, :594)."""
     M = sp_points.shape[0]
     safe = indices.clamp(0, M - 1)
     if sp_rot is not None:
@@ -62,8 +64,13 @@ def warp(points, sp_points, sp_t, sp_r, sp_s, sp_rot, weights, indices, method='
         R = quat_to_matrix(q)
         if method == 'LBS_c':
             sp_t = sp_t + sp_points + torch.einsum('mab,mb->ma', R, -sp_points)
-        moved = torch.einsum('nkab,nb->nka', R[safe], points) + sp_t[safe]
-        d_points = (moved * weights[..., None]).sum(dim=1) - points
+        if method in ('LBS', 'LBS_c'):
+            moved = torch.einsum('nkab,nb->nka', R[safe], points) + sp_t[safe]
+            d_points = (moved * weights[..., None]).sum(dim=1) - points
+        else:
+            if p2sp is None:
+                p2sp = torch.gather(indices, -1, weights.argmax(dim=-1, keepdim=True))[:, 0]
+            d_points = torch.einsum('nab,nb->na', R[p2sp], points) + sp_t[p2sp] - points
     else:
         d_points = (sp_t[safe] * weights[..., None]).sum(dim=1)
     d_rotation = (sp_r[safe] * weights[..., None]).sum(dim=1)

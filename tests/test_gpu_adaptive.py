@@ -220,3 +220,67 @@ def test_density_control_methods(S, device):
     model.reset_opacity(opt)
     assert float(torch.sigmoid(model._opacity).max()) <= 0.01 + 1e-6
     assert not opt.state[model._opacity]['exp_avg'].any()
+
+
+def test_superpoint_extras_follow_the_points(device):
+    """The superpoint model's per-point extras -- per-frame culling flags, the visibility factor, the superpoint
+    assignment -- through clone, split and prune, against the reference's own expressions for them
+    (network.py:1195-1215: `t[valid]`, `cat((t, t[mask]))`, `cat((t, t[mask].repeat(N, 1)))`, and the prune of the split
+    parents, :1190-1191), evaluated with torch indexing on the same masks; and the visibility factor inside the gradient
+    statistics (:1153)."""
+    P, N, F = 20011, 2, 7
+    thr, extent, pd = 1e-3, 5.0, 0.01
+    pts = _points(P, 2, 21)
+    model, opt, ps = _model(pts, device)
+    _statistics(model, ps, 5)
+    g = torch.Generator().manual_seed(9)
+    model._culling = (torch.rand(P, F, generator=g) < 0.3).to(device)
+    model.factor_culling = torch.rand(P, 1, generator=g).to(device)
+    model.p2sp = torch.randint(0, 512, (P,), generator=g, dtype=torch.int32).to(device)
+    ref = {k: getattr(model, k).clone() for k in ('_culling', 'factor_culling', 'p2sp')}
+
+    def carry(mask, n=None):  # densification_postfix of the superpoint model
+        for k, t in ref.items():
+            extra = t[mask] if n is None else t[mask].repeat(n, *[1] * (t.ndim - 1))
+            ref[k] = torch.cat((t, extra))
+
+    def drop(mask):  # prune_points of the superpoint model
+        for k, t in ref.items():
+            ref[k] = t[~mask]
+
+    def check():
+        for k, t in ref.items():
+            got = getattr(model, k)
+            assert got.dtype == t.dtype and got.shape == t.shape and torch.equal(got, t), k
+        assert model._culling.shape[0] == model._xyz.shape[0]
+
+    grads = torch.from_numpy(np.nan_to_num(ps.grad_accum / ps.denom, nan=0.0).astype(np.float32)).to(device)
+    scaling = model.get_scaling.detach()
+    clone_mask = (torch.norm(grads, dim=-1) >= thr) & (scaling.amax(1) <= pd * extent)
+    model.densify_and_clone(opt, grads, thr, pd * extent)
+    carry(clone_mask)
+    check()
+    P1 = model._xyz.shape[0]
+    padded = torch.zeros(P1, device=device)
+    padded[:P] = grads.squeeze(-1)
+    split_mask = (padded >= thr) & (model.get_scaling.detach().amax(1) > pd * extent)
+    assert int(clone_mask.sum()) > 0 and int(split_mask.sum()) > 0
+    model.densify_and_split(opt, grads, thr, pd * extent, N)
+    carry(split_mask, N)
+    drop(torch.cat((split_mask, split_mask.new_zeros(N * int(split_mask.sum())))))
+    check()
+    prune = torch.rand(model._xyz.shape[0], generator=g).to(device) < 0.25
+    model.prune_points(opt, prune)
+    drop(prune)
+    check()
+    # gradient statistics weighted by the visibility factor
+    Pn = model._xyz.shape[0]
+    vs = torch.zeros(Pn, 3, device=device, requires_grad=True)
+    vs.grad = torch.randn(Pn, 3, generator=g).to(device)
+    upd = torch.rand(Pn, generator=g).to(device) < 0.6
+    acc0, den0 = model.xyz_gradient_accum.clone(), model.denom.clone()
+    model.add_densification_stats(vs, upd)
+    want = acc0.clone()
+    want[upd] += torch.norm(vs.grad[upd, :2], dim=-1, keepdim=True) * model.factor_culling[upd]
+    assert float((model.xyz_gradient_accum - want).abs().max()) <= 1e-6 * float(want.abs().max())
+    assert torch.equal(model.denom, den0 + upd[:, None].float())

@@ -136,18 +136,32 @@ def test_small_operators_in_the_other_element_types(device, oracle_mod, c1):
             y4 = float(np.float32(1.0925484305920792)) * (x * y)
             y6 = float(np.float32(0.94617469575755997)) * (z * z) - float(np.float32(0.31539156525251999))
             assert np.abs(npy(enc)[:, 4] - y4).max() < 1e-15 and np.abs(npy(enc)[:, 6] - y6).max() < 1e-15
-        # -- half: storage only, one rounding of the single-precision result (2^-11 relative) on top of the rounding of
-        # the inputs, which the oracle receives as the same half values
+        # -- half. Degree <= 3 follows the reference's at::Half instantiation, which keeps its monomials and its backward
+        # sums in half (shencoder.cu:31-33, 188-193): checked against oracle/sh_half.py, the numpy restatement of exactly
+        # that, element for element up to the float expressions' contraction (one half ulp, rare). Degrees 4 - 7 are float
+        # arithmetic rounded once on store (2^-11 relative), checked against the float64 basis on the same half inputs.
         dh = dirs.half()
         d = dh.to(device).requires_grad_()
         enc = sh_encode(d, degree)
         gh = genc.half()
         enc.backward(gh.to(device))
-        O.call("sh_encode_forward_f64", P, 3, degree, npy(dh.double()), ref)
-        O.call("sh_encode_backward_f64", P, 3, degree, npy(gh.double()), npy(dh.double()), gref)
         assert enc.dtype == torch.float16 and d.grad.dtype == torch.float16
-        assert np.abs(npy(enc.double()) - ref).max() <= 2.0 ** -11 * max(np.abs(ref).max(), 1) * 1.01
-        assert np.abs(npy(d.grad.double()) - gref).max() <= 2.0 ** -11 * np.abs(gref).max() * 1.01
+        if degree <= 3:
+            from oracle import sh_half as H
+            want, gwant = H.sh_encode_half(npy(dh), degree), H.sh_encode_backward_half(npy(gh), npy(dh), degree)
+            # a contraction moves one term by a float ulp, which can cross a half rounding boundary: one half ulp of that
+            # TERM, whose size is bounded by 4 |upstream| for the sums of the backward and by the entry for the forward
+            term = 4.0 * np.abs(npy(gh).astype(np.float64)).max(axis=1, keepdims=True) if degree else 1.0
+            for got_, want_, size in ((npy(enc), want, None), (npy(d.grad), gwant, term)):
+                a, b = got_.astype(np.float64), want_.astype(np.float64)
+                ulp = np.maximum(np.abs(b) if size is None else np.maximum(np.abs(b), size), 2.0 ** -14) * 2.0 ** -10
+                assert (np.abs(a - b) <= ulp).all()
+                assert (got_ == want_).mean() > 0.98
+        else:
+            O.call("sh_encode_forward_f64", P, 3, degree, npy(dh.double()), ref)
+            O.call("sh_encode_backward_f64", P, 3, degree, npy(gh.double()), npy(dh.double()), gref)
+            assert np.abs(npy(enc.double()) - ref).max() <= 2.0 ** -11 * max(np.abs(ref).max(), 1) * 1.01
+            assert np.abs(npy(d.grad.double()) - gref).max() <= 2.0 ** -11 * np.abs(gref).max() * 1.01
     with pytest.raises(RuntimeError, match='element type'):
         get_C_function('sh_encode_forward')(dirs.to(device).bfloat16(), torch.empty(P, 4, device=device).bfloat16(), P, 3, 1)
     with pytest.raises(RuntimeError, match='dtype'):
@@ -453,12 +467,56 @@ def test_calc_LBS_weight_and_warp_mirror_the_fused_path(device):
                 assert float((x - y).abs().max()) <= 2e-4 * max(float(y.abs().max()), 1e-6)
 
 
+def test_warp_largest_matches_oracle(device):
+    """warp_method 'largest' (network.py:555-561, assignment :594): values and gradients of `warp` / `superpoint_deform`
+    against the float64 oracle and its autograd; the assignment defaults to the neighbour of largest weight and can be
+    handed in."""
+    from oracle import lbs as OL
+    from fast_sp_gs_amd.deform import assign_superpoints, superpoint_deform, warp
+    g = torch.Generator().manual_seed(71)
+    N, M, K = 4000, 48, 4
+    mk = lambda *shape, s=0.2: (s * torch.randn(*shape, generator=g))
+    pts = torch.rand(N, 3, generator=g) * 2 - 1
+    ctrl, sp_t, sp_r, sp_s, sp_rot = mk(M, 3, s=0.6), mk(M, 3), mk(M, 4), mk(M, 2), mk(M, 4, s=0.4)
+    gx, gr, gs = mk(N, 3, s=1.0), mk(N, 4, s=1.0), mk(N, 2, s=1.0)
+    names = ['ctrl', 'sp_t', 'sp_r', 'sp_s', 'sp_rot']
+    dev_leaves = [t.to(device).requires_grad_() for t in (ctrl, sp_t, sp_r, sp_s, sp_rot)]
+    d_xyz, d_rot, d_scale, w, idx = superpoint_deform(pts.to(device), *dev_leaves[:4], sp_rot=dev_leaves[4], K=K,
+                                                      temperature=0.05, warp_method='largest', LBS_method='dist')
+    got = torch.autograd.grad((d_xyz * gx.to(device)).sum() + (d_rot * gr.to(device)).sum() +
+                              (d_scale * gs.to(device)).sum(), dev_leaves, allow_unused=True)
+    p2sp = assign_superpoints(w, idx)
+    # oracle on the GPU's neighbour lists (float64), distances recomputed there
+    leaves = [t.double().requires_grad_() for t in (ctrl, sp_t, sp_r, sp_s, sp_rot)]
+    idx_c = idx.cpu()
+    d2 = ((pts.double()[:, None] - leaves[0][idx_c]) ** 2).sum(-1)
+    w_ref = OL.lbs_weights(d2, idx_c, M, 'dist', 0.05)
+    assert float((w.cpu().double() - w_ref.detach()).abs().max()) < 1e-5
+    assert torch.equal(p2sp.cpu(), torch.gather(idx_c, -1, w_ref.argmax(-1, keepdim=True))[:, 0])
+    r_xyz, r_rot, r_scale = OL.warp(pts.double(), *leaves[:4], leaves[4], w_ref, idx_c, 'largest')
+    for a, b in ((d_xyz, r_xyz), (d_rot, r_rot), (d_scale, r_scale)):
+        assert float((a.detach().cpu().double() - b.detach()).abs().max()) <= 2e-5 * max(float(b.abs().max()), 1.0)
+    want = torch.autograd.grad((r_xyz * gx.double()).sum() + (r_rot * gr.double()).sum() + (r_scale * gs.double()).sum(),
+                               leaves, allow_unused=True)
+    for name, a, b in zip(names, got, want):
+        assert a is not None and b is not None, name
+        assert float((a.cpu().double() - b).abs().max()) <= 1e-3 * float(b.abs().max()) + 1e-9, name
+    # an assignment handed in is used as it is: points follow control point 7 rigidly
+    fixed = torch.full((N,), 7, dtype=torch.int64, device=device)
+    d_fixed = warp(pts.to(device), *[t.detach() for t in dev_leaves[:4]], dev_leaves[4].detach(), w, idx, 'largest',
+                   p2sp=fixed)[0]
+    r_fixed = OL.warp(pts.double(), ctrl.double(), sp_t.double(), sp_r.double(), sp_s.double(), sp_rot.double(), w_ref,
+                      idx_c, 'largest', p2sp=fixed.cpu())[0]
+    assert float((d_fixed.cpu().double() - r_fixed).abs().max()) < 2e-5
+
+
 @pytest.mark.parametrize("B,D,p_degree,t_degree", [(512, 8, 10, 10), (500, 8, 10, 6), (70, 4, 4, 2), (1, 3, 2, 1)])
 def test_deform_mlp_backward_mfma(B, D, p_degree, t_degree, device):
-    """Weight / bias gradients from the MFMA backward kernels. The checkers for this floating-point kernel are torch:
-      * exactly the kernels' own arithmetic -- the chain rule evaluated at the stored bf16 hidden states (their zeros
-        are the ReLU mask) with bf16 operands where the matrix cores take them and every dZ rounded to bf16 -- restated
-        in float64: agreement to 1e-3 of each tensor's largest entry;
+    """Weight / bias / input gradients from the MFMA backward kernels. The checkers for this floating-point kernel:
+      * oracle/mlp.py with the kernels' roundings -- the chain rule evaluated at the stored bf16 hidden states (their
+        zeros are the ReLU mask) with bf16 operands where the matrix cores take them and every dZ rounded to bf16, in
+        float64; without the roundings that function equals torch.autograd (tests/test_oracle_mlp.py): agreement to
+        1e-3 of each tensor's largest entry;
       * torch autograd of the fp32 network: same direction (cosine > 0.98); element-wise it differs more because a
         hidden unit whose pre-activation is within bf16 rounding of zero is masked differently by the two forwards and
         each such unit moves a sum of B random-sign terms by a whole term.
@@ -483,35 +541,40 @@ def test_deform_mlp_backward_mfma(B, D, p_degree, t_degree, device):
     got = dict(zip(names, torch.autograd.grad(sum((o * g_).sum() for o, g_ in zip(outs, go)), params)))
     torch.cuda.synchronize()
 
-    # The kernels' arithmetic restated in float64 torch with their roundings: the chain starts from the fp32 product
-    # g_out . W_heads, every dZ is rounded to bf16 where it is stored (and masked by the stored state's zeros), the
-    # hidden weights, the encoded input and -- for the heads' gradients -- g_out enter the matrix cores as bf16; sums are
-    # fp32 on the GPU and float64 here. What is left is fp32 summation order plus the rare dZ element whose fp32 sum
-    # sits on a bf16 rounding boundary (one bf16 ulp of one term of a B-term sum): 1e-3 of each tensor's largest entry.
+    # The checker is oracle/mlp.py with its rounding switch on: the chain rule written out by hand in float64 (pinned on
+    # the CPU against torch.autograd, tests/test_oracle_mlp.py) with bf16 operands where the matrix cores take them,
+    # evaluated at the hidden states the forward kernel stored (their zeros are the ReLU mask). What is left is fp32
+    # summation order plus the rare dZ element whose fp32 sum sits on a bf16 rounding boundary (one bf16 ulp of one term
+    # of a B-term sum): 1e-3 of each tensor's largest entry.
+    from oracle import mlp as OM
+    from fast_sp_gs_amd.deform import _DeformMlp
+    cpu = lambda t_: t_.detach().cpu()
     with torch.no_grad():
-        bf = lambda t_: t_.to(torch.bfloat16).double()
         x_enc = net.encode(x, t)
         packed, bias = net._packed
         _, saved = get_C_function('mlp_forward')(x_enc, packed, bias, D, net.skip, 10, True)
-        H = saved.view(torch.bfloat16).double()  # [D, B, 256]
+        hidden = list(cpu(saved.view(torch.bfloat16)).double())  # D x [B, 256]
         Wh = torch.cat([net.gaussian_warp.weight, net.gaussian_rotation.weight, net.gaussian_scaling.weight], 0)
         g_out = torch.cat(go, -1)
+        ref = OM.mlp_backward(cpu(x_enc), [cpu(l.weight) for l in net.linear], cpu(Wh), net.skip, cpu(g_out), hidden,
+                              round_bf16=True)
         want = {}
         for name, lo, hi in (('gaussian_warp', 0, 3), ('gaussian_rotation', 3, 7), ('gaussian_scaling', 7, 10)):
-            want[name + '.weight'] = bf(g_out[:, lo:hi]).t() @ H[D - 1]
-            want[name + '.bias'] = bf(g_out[:, lo:hi]).sum(0)
-        dZ = bf(((g_out.double() @ Wh.double()) * (H[D - 1] != 0)).float())
-        for l in range(D - 1, -1, -1):
-            X = bf(x_enc) if l == 0 else (torch.cat([bf(x_enc), H[l - 1]], -1) if l == net.skip + 1 else H[l - 1])
-            want[f'linear.{l}.weight'] = dZ.t() @ X
-            want[f'linear.{l}.bias'] = dZ.sum(0)
-            if l > 0:
-                dZ = bf(((dZ @ bf(net.linear[l].weight[:, -256:])) * (H[l - 1] != 0)).float())
+            want[name + '.weight'], want[name + '.bias'] = ref['head_w'][lo:hi], ref['head_b'][lo:hi]
+        for l in range(D):
+            want[f'linear.{l}.weight'], want[f'linear.{l}.bias'] = ref['weights'][l], ref['biases'][l]
     for name in names:
-        a, b = got[name].double(), want[name]
+        a, b = cpu(got[name]).double(), want[name]
         assert a.shape == b.shape and bool(torch.isfinite(a).all()), name
         scale = float(b.abs().max())
         assert float((a - b).abs().max()) <= 1e-3 * scale + 1e-9, (name, float((a - b).abs().max()), scale)
+    # the gradient of the encoded input (what reaches the time network): dZ_0 W_0 + dZ_{skip+1} W_{skip+1}[:, :Din]
+    leaf = x_enc.detach().clone().requires_grad_()
+    out = _DeformMlp.apply(leaf, packed, bias, net._packed_t, net._heads_w, D, net.skip, 10, *net._mlp_parameters())
+    g_leaf, = torch.autograd.grad((out * g_out).sum(), [leaf])
+    # (a row of it is a sum over 2 x 256 hidden units of dZ, each of which may sit on a bf16 rounding boundary: 3e-3)
+    scale = float(ref['x'].abs().max())
+    assert float((cpu(g_leaf).double() - ref['x']).abs().max()) <= 3e-3 * scale + 1e-9
 
     refs = net.forward_fp32(x, t)[:3]
     auto = torch.autograd.grad(sum((o * g_).sum() for o, g_ in zip(refs, go)), params)

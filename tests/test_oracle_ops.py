@@ -97,9 +97,25 @@ def test_lbs_closed_forms(oracle_mod):
     same = torch.full((N, K), 5)
     dx = OL.lbs_blend(pts, ctrl, sp_t, sp_r, s0, sp_rot, d2, same, 'dist', 0.01, 'LBS_c')[0]
     assert float((dx - ((pts - ctrl[5]) @ Rm.T + ctrl[5] + t - pts)).abs().max()) < 1e-12
+    # 'largest' (network.py:555-561): ONE rigid transform per point, that of its assigned control point -- by default the
+    # neighbour of largest weight (:594) -- written out here point by point with scipy rotations; residuals stay blended
+    rots = torch.randn(M, 4, **f64) * 0.3
+    t_each = torch.randn(M, 3, **f64)
+    w_all = OL.lbs_weights(d2, idx, M, 'dist', 0.01)
+    dx, dr, ds = OL.warp(pts, ctrl, t_each, sp_r, s0 + 0.5, rots, w_all, idx, 'largest')
+    for n in range(N):
+        m = int(idx[n, int(w_all[n].argmax())])
+        qm = (rots[m] + torch.tensor([0, 0, 0, 1.0], dtype=torch.float64)).numpy()
+        Rn = torch.from_numpy(Rotation.from_quat(qm / np.linalg.norm(qm)).as_matrix())
+        assert float((dx[n] - (Rn @ pts[n] + t_each[m] - pts[n])).abs().max()) < 1e-12
+    assert float((dr - (w_all[..., None] * sp_r[idx]).sum(1)).abs().max()) < 1e-14
+    assigned = torch.randint(0, M, (N,), generator=g)
+    dx2 = OL.warp(pts, ctrl, t_each, sp_r, s0, rots, w_all, idx, 'largest', p2sp=assigned)[0]
+    one = OL.warp(pts, ctrl, t_each, sp_r, s0, rots, torch.ones(N, 1, dtype=torch.float64), assigned[:, None], 'LBS')[0]
+    assert float((dx2 - one).abs().max()) < 1e-14  # == the blend over a single neighbour of weight one
     # no local rotation (the default configuration): the translations are blended, nothing else, whatever the method
     sp_t2 = torch.randn(M, 3, **f64)
-    for method in ('LBS', 'LBS_c'):
+    for method in ('LBS', 'LBS_c', 'largest'):
         dx, dr, ds, w = OL.lbs_blend(pts, ctrl, sp_t2, sp_r, s0, None, d2, idx, 'dist', 0.01, method)
         assert float((dx - (w[..., None] * sp_t2[idx]).sum(1)).abs().max()) < 1e-14
     # kernel weights by an explicit loop on the raw parameters (radius = exp(.), weight = sigmoid(.))

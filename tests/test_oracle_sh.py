@@ -120,3 +120,43 @@ def test_sh_to_rgb_forward_backward(oracle_mod, use_campos, degree):
     if use_campos:
         assert np.abs(cam_fd - g_cam).max() < 1e-6
         assert np.abs(g_cam + g_dir.sum(0)).max() < 1e-9
+
+
+def test_half_encoder_restatement(oracle_mod):
+    """oracle/sh_half.py (the reference's at::Half instantiation of the SH encoder, degree <= 3): stays within the
+    accumulated half roundings of the float64 basis / gradient on the same half inputs, really rounds its monomials
+    (a value the unrounded evaluation would give differently), and agrees with a scalar evaluation whose half
+    conversions go through `struct` ('e' format) instead of numpy's float16."""
+    import struct
+    from oracle import sh_half as H
+    O = oracle_mod
+    rng = np.random.default_rng(5)
+    d = rng.normal(size=(3000, 3))
+    d16 = (d / np.linalg.norm(d, axis=1, keepdims=True)).astype(np.float16)
+    g16 = rng.normal(size=(3000, 16)).astype(np.float16)
+    for degree in (0, 1, 2, 3):
+        n = (degree + 1) ** 2
+        ref, gref = np.zeros((3000, n)), np.zeros((3000, 3))
+        O.call("sh_encode_forward_f64", 3000, 3, degree, np.ascontiguousarray(d16, np.float64), ref)
+        O.call("sh_encode_backward_f64", 3000, 3, degree, np.ascontiguousarray(g16[:, :n], np.float64),
+               np.ascontiguousarray(d16, np.float64), gref)
+        enc = H.sh_encode_half(d16, degree)
+        back = H.sh_encode_backward_half(np.ascontiguousarray(g16[:, :n]), d16, degree)
+        assert enc.dtype == np.float16 and back.dtype == np.float16
+        # forward: one rounding of a monomial + one on store; backward: up to 9 rounded terms and 9 rounded sums
+        assert np.abs(enc.astype(np.float64) - ref).max() <= 3 * 2.0 ** -11 * max(np.abs(ref).max(), 1.0)
+        if degree:
+            assert np.abs(back.astype(np.float64) - gref).max() <= 12 * 2.0 ** -11 * np.abs(gref).max()
+    # the monomials are rounded: recomputing entry 4 from the unrounded product differs somewhere
+    x, y = d16[:, 0].astype(np.float32), d16[:, 1].astype(np.float32)
+    unrounded = (np.float32(1.0925484305920792) * (x * y)).astype(np.float16)
+    assert (H.sh_encode_half(d16, 2)[:, 4] != unrounded).any()
+    # scalar evaluation with struct's half conversion
+    h = lambda v: struct.unpack('e', struct.pack('e', float(v)))[0]
+    f = lambda v: float(np.float32(v))
+    for i in range(0, 3000, 97):
+        xs, ys, zs = (float(v) for v in d16[i])
+        xy, zz = h(f(xs * ys)), h(f(zs * zs))
+        assert float(enc[i, 4]) == h(f(np.float32(1.0925484305920792) * np.float32(xy)))
+        want = h(f(np.float32(0.3731763325901154) * np.float32(zs)) * f(np.float32(5.0) * np.float32(zz) - np.float32(3.0)))
+        assert abs(float(enc[i, 12]) - want) <= abs(want) * 2.0 ** -10
