@@ -19,16 +19,32 @@
 #include "common.hpp"
 #include "lbs.hpp"
 #include "sh.hpp"
+#include "sh_stage.hpp"
 
 namespace fsgs {
 namespace {
 
 // ---- SH -> RGB ----------------------------------------------------------------------------------------------------
-template <int kSh>
+// kRows: all 16 coefficients of a point sit in one 16-byte-aligned 192-byte row (F == 16, degree 3). A lane that walks its
+// own row touches one 128-byte line per load instruction (920 GB/s measured at 1M points); each wavefront therefore moves
+// its 64 rows as twelve 16-byte pieces per lane, 1 KB of consecutive addresses per instruction, through its own slice of
+// LDS, and every lane then reads its row there (the scheme of the preprocess kernels, sh_stage.hpp).
+template <int kSh, bool kRows>
 __global__ void __launch_bounds__(256) sh_to_rgb_forward_kernel(int P, int F, int degree, int clamp,
     const float* __restrict__ pos, const float* __restrict__ campos, const float* __restrict__ sh,
     float* __restrict__ rgb) {
+  __shared__ float s_rows[kRows ? 4 * kWave * kShStageStride : 1];
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  float* my_rows = s_rows + (kRows ? (threadIdx.x >> 6) * kWave * kShStageStride : 0);
+  if (kRows) {
+    const unsigned long long live = __ballot(i < P);
+    if (live != 0ull) {
+      ShWaveRows regs;
+      wave_fetch_sh_rows(regs, live, (int) (blockIdx.x * blockDim.x + (threadIdx.x & ~63)), (const float4*) sh);
+      wave_rows_to_lds(regs, my_rows);
+      wave_lds_sync();
+    }
+  }
   if (i >= P) return;
   float x = pos[3 * (size_t) i], y = pos[3 * (size_t) i + 1], z = pos[3 * (size_t) i + 2];
   if (campos) {
@@ -38,7 +54,7 @@ __global__ void __launch_bounds__(256) sh_to_rgb_forward_kernel(int P, int F, in
   float Y[kSh];
   sh_eval(degree, x, y, z, Y);
   const int n    = sh_count(degree);
-  const float* c = sh + (size_t) i * F * 3;
+  const float* c = kRows ? my_rows + (threadIdx.x & 63) * kShStageStride : sh + (size_t) i * F * 3;
   float r = c[0] * Y[0], g = c[1] * Y[0], b = c[2] * Y[0];
   for (int l = 1; l < n; ++l) r += c[3 * l] * Y[l], g += c[3 * l + 1] * Y[l], b += c[3 * l + 2] * Y[l];
   r += 0.5f, g += 0.5f, b += 0.5f;
@@ -52,13 +68,25 @@ __device__ __forceinline__ float wave_sum_xor(float v) {
   return v;
 }
 
-template <int kSh>
+template <int kSh, bool kRows>
 __global__ void __launch_bounds__(256) sh_to_rgb_backward_kernel(int P, int F, int degree, int clamp,
     const float* __restrict__ pos, const float* __restrict__ campos, const float* __restrict__ sh,
     const float* __restrict__ rgb, const float* __restrict__ grad_rgb, float* __restrict__ grad_dir,
     float* __restrict__ grad_campos, float* __restrict__ grad_sh) {
   __shared__ float s_cam[4][3];
+  __shared__ float s_rows[kRows ? 4 * kWave * kShStageStride : 1];
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  const int wave_base = (int) (blockIdx.x * blockDim.x + (threadIdx.x & ~63));
+  float* my_rows = s_rows + (kRows ? (threadIdx.x >> 6) * kWave * kShStageStride : 0);
+  if (kRows) {  // coefficient rows in through LDS; the gradient rows leave the same way (a lane overwrites its own row)
+    const unsigned long long live = __ballot(i < P);
+    if (live != 0ull) {
+      ShWaveRows regs;
+      wave_fetch_sh_rows(regs, live, wave_base, (const float4*) sh);
+      wave_rows_to_lds(regs, my_rows);
+      wave_lds_sync();
+    }
+  }
   float dx = 0, dy = 0, dz = 0;
   if (i < P) {
     const float p[3] = {pos[3 * (size_t) i], pos[3 * (size_t) i + 1], pos[3 * (size_t) i + 2]};
@@ -73,12 +101,14 @@ __global__ void __launch_bounds__(256) sh_to_rgb_backward_kernel(int P, int F, i
     float Y[kSh], tl[kSh];
     sh_eval(degree, x, y, z, Y);
     const int n    = sh_count(degree);
-    const float* c = sh + (size_t) i * F * 3;
-    float* o       = grad_sh ? grad_sh + (size_t) i * F * 3 : nullptr;
+    float* row     = my_rows + (threadIdx.x & 63) * kShStageStride;
+    const float* c = kRows ? row : sh + (size_t) i * F * 3;
+    float* o       = kRows ? (grad_sh ? row : nullptr) : (grad_sh ? grad_sh + (size_t) i * F * 3 : nullptr);
     tl[0] = 0.0f;
-    for (int l = 0; l < n; ++l) {
+    for (int l = 0; l < n; ++l) {  // a coefficient is read before its slot takes the gradient
+      const float c0 = c[3 * l], c1 = c[3 * l + 1], c2 = c[3 * l + 2];
+      tl[l] = g[0] * c0 + g[1] * c1 + g[2] * c2;
       if (o) o[3 * l] = g[0] * Y[l], o[3 * l + 1] = g[1] * Y[l], o[3 * l + 2] = g[2] * Y[l];
-      tl[l] = g[0] * c[3 * l] + g[1] * c[3 * l + 1] + g[2] * c[3 * l + 2];
     }
     if (grad_dir || grad_campos) {
       sh_grad_accumulate(degree, x, y, z, tl, dx, dy, dz);
@@ -89,6 +119,10 @@ __global__ void __launch_bounds__(256) sh_to_rgb_backward_kernel(int P, int F, i
       }
       if (grad_dir) grad_dir[3 * (size_t) i] = dx, grad_dir[3 * (size_t) i + 1] = dy, grad_dir[3 * (size_t) i + 2] = dz;
     }
+  }
+  if (kRows && grad_sh) {
+    wave_lds_sync();
+    wave_rows_to_global(my_rows, wave_base, P, (float4*) grad_sh);
   }
   if (grad_campos) {  // block reduction, then 3 atomics per block (spherical_harmonics.cu:56-65)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -480,9 +514,12 @@ __global__ void __launch_bounds__(256) deform_apply_backward_kernel(int N, int l
   ((float4*) g_rot)[i] = o;
 }
 
-// The same update for every parameter tensor of a point set in one launch (blockIdx.y = tensor): the reference steps
-// its parameter groups one kernel at a time (sparse_gaussian_adam.py:20-45), each a few microseconds of work behind a
-// launch. Table passed by value; same arithmetic as adam_masked_kernel, element for element.
+// The same update for every parameter tensor of a point set in one launch: the reference steps its parameter groups one
+// kernel at a time (sparse_gaussian_adam.py:20-45), each a few microseconds of work behind a launch. Table passed by
+// value; the blocks of all tensors form one grid (a block finds its tensor in the table's block prefix), so no block
+// is launched for nothing, and every tensor whose element count and addresses allow it moves as 16-byte pieces whatever
+// its row length: the four elements of a piece look up their own rows in the mask. Same arithmetic as
+// adam_masked_kernel, element for element.
 constexpr int kMaxAdamTensors = 12;
 struct AdamTable {
   float* param[kMaxAdamTensors];
@@ -492,45 +529,58 @@ struct AdamTable {
   int64_t M[kMaxAdamTensors];
   float lr[kMaxAdamTensors], eps[kMaxAdamTensors];
   int vec4[kMaxAdamTensors];
+  unsigned first_block[kMaxAdamTensors + 1];
+  int n;
 };
-
-template <int kVec>
-__device__ __forceinline__ void adam_masked_body(int64_t e, float lr, float b1, float b2, float eps,
-    float* __restrict__ param, const float* __restrict__ grad, float* __restrict__ m, float* __restrict__ v) {
-#pragma clang fp contract(off)
-  float g[kVec], mm[kVec], vv[kVec], pp[kVec];
-  if (kVec == 4) {
-    *(float4*) g  = *(const float4*) (grad + e);
-    *(float4*) mm = *(const float4*) (m + e);
-    *(float4*) vv = *(const float4*) (v + e);
-    *(float4*) pp = *(const float4*) (param + e);
-  } else {
-    g[0] = grad[e], mm[0] = m[e], vv[0] = v[e], pp[0] = param[e];
-  }
-#pragma unroll
-  for (int k = 0; k < kVec; ++k) {
-    mm[k] = b1 * mm[k] + (1.0f - b1) * g[k];
-    vv[k] = b2 * vv[k] + (1.0f - b2) * g[k] * g[k];
-    pp[k] += -lr * mm[k] / (sqrtf(vv[k]) + eps);
-  }
-  if (kVec == 4) {
-    *(float4*) (param + e) = *(float4*) pp;
-    *(float4*) (m + e)     = *(float4*) mm;
-    *(float4*) (v + e)     = *(float4*) vv;
-  } else {
-    param[e] = pp[0], m[e] = mm[0], v[e] = vv[0];
-  }
-}
 
 __global__ void __launch_bounds__(256) adam_masked_multi_kernel(AdamTable t, int64_t N, float b1, float b2,
                                                                 const uint8_t* __restrict__ mask) {
-  const int q      = blockIdx.y;
-  const int64_t M  = t.M[q], total = N * M;
-  const int vec    = t.vec4[q] ? 4 : 1;
-  const int64_t e  = ((int64_t) blockIdx.x * blockDim.x + threadIdx.x) * vec;
-  if (e >= total || !mask[e / M]) return;
-  if (vec == 4) adam_masked_body<4>(e, t.lr[q], b1, b2, t.eps[q], t.param[q], t.grad[q], t.m[q], t.v[q]);
-  else adam_masked_body<1>(e, t.lr[q], b1, b2, t.eps[q], t.param[q], t.grad[q], t.m[q], t.v[q]);
+#pragma clang fp contract(off)
+  int q = 0;
+  while (q + 1 < t.n && blockIdx.x >= t.first_block[q + 1]) ++q;
+  const int64_t M = t.M[q], total = N * M;
+  const int vec   = t.vec4[q] ? 4 : 1;
+  const int64_t e = ((int64_t) (blockIdx.x - t.first_block[q]) * blockDim.x + threadIdx.x) * vec;
+  if (e >= total) return;
+  const float lr = t.lr[q], eps = t.eps[q];
+  float* __restrict__ param = t.param[q];
+  const float* __restrict__ grad = t.grad[q];
+  float* __restrict__ m = t.m[q];
+  float* __restrict__ v = t.v[q];
+  if (vec == 1) {
+    if (!mask[e / M]) return;
+    const float g = grad[e];
+    const float mm = b1 * m[e] + (1.0f - b1) * g;
+    const float vv = b2 * v[e] + (1.0f - b2) * g * g;
+    param[e] += -lr * mm / (sqrtf(vv) + eps);
+    m[e] = mm, v[e] = vv;
+    return;
+  }
+  // rows of the piece's four elements (a piece may straddle rows, several of them when rows are shorter than four)
+  int64_t row = e / M, rem = e - row * M;
+  bool on[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    on[k] = mask[row] != 0;
+    if (++rem == M) rem = 0, ++row;
+    if (row >= N) row = N - 1;  // only past the last element of the tensor, which e + k < total excludes
+  }
+  if (!(on[0] | on[1] | on[2] | on[3])) return;
+  float g[4], mm[4], vv[4], pp[4];
+  *(float4*) g  = *(const float4*) (grad + e);
+  *(float4*) mm = *(const float4*) (m + e);
+  *(float4*) vv = *(const float4*) (v + e);
+  *(float4*) pp = *(const float4*) (param + e);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float m1 = b1 * mm[k] + (1.0f - b1) * g[k];
+    const float v1 = b2 * vv[k] + (1.0f - b2) * g[k] * g[k];
+    const float p1 = pp[k] + -lr * m1 / (sqrtf(v1) + eps);
+    mm[k] = on[k] ? m1 : mm[k], vv[k] = on[k] ? v1 : vv[k], pp[k] = on[k] ? p1 : pp[k];
+  }
+  *(float4*) (param + e) = *(float4*) pp;  // elements of masked rows are written back as they were
+  *(float4*) (m + e)     = *(float4*) mm;
+  *(float4*) (v + e)     = *(float4*) vv;
 }
 
 }  // namespace
@@ -578,17 +628,23 @@ FSGS_API int fsgs_adam_masked_update_multi(int n_tensors, int64_t N, const int64
   if (n_tensors == 0 || N == 0) return kOk;
   FSGS_REQUIRE(M && mask && lr && eps && param && grad && m && v, "AdamMasksedUpdated (multi): null pointer");
   AdamTable t{};
-  int64_t most = 0;
+  t.n = n_tensors;
+  unsigned blocks = 0;
   for (int q = 0; q < n_tensors; ++q) {
     FSGS_REQUIRE(M[q] > 0 && param[q] && grad[q] && m[q] && v[q], "AdamMasksedUpdated (multi): bad tensor %d", q);
     t.param[q] = param[q], t.grad[q] = grad[q], t.m[q] = m[q], t.v[q] = v[q], t.M[q] = M[q];
     t.lr[q] = (float) lr[q], t.eps[q] = (float) eps[q];
-    t.vec4[q] = (M[q] % 4 == 0) &&
+    const int64_t total = N * M[q];
+    t.vec4[q] = (total % 4 == 0) &&
                 (((uintptr_t) param[q] | (uintptr_t) grad[q] | (uintptr_t) m[q] | (uintptr_t) v[q]) % 16 == 0);
-    most = std::max<int64_t>(most, t.vec4[q] ? N * M[q] / 4 : N * M[q]);
+    t.first_block[q] = blocks;
+    const int64_t nb = div_up(t.vec4[q] ? total / 4 : total, (int64_t) 256);
+    FSGS_REQUIRE((int64_t) blocks + nb < (int64_t) 0x7fffffff, "AdamMasksedUpdated (multi): too many elements");
+    blocks += (unsigned) nb;
   }
-  hipLaunchKernelGGL(adam_masked_multi_kernel, dim3((unsigned) div_up(most, (int64_t) 256), n_tensors), dim3(256), 0,
-                     (hipStream_t) stream, t, N, (float) b1, (float) b2, mask);
+  t.first_block[n_tensors] = blocks;
+  hipLaunchKernelGGL(adam_masked_multi_kernel, dim3(blocks), dim3(256), 0, (hipStream_t) stream, t, N, (float) b1,
+                     (float) b2, mask);
   return check_launch("AdamMasksedUpdated");
 }
 
@@ -598,7 +654,9 @@ FSGS_API int fsgs_sh_to_rgb_forward(int P, int F, int degree, int clamp, const f
   FSGS_REQUIRE(0 <= degree && degree <= kMaxShDegree && (degree + 1) * (degree + 1) <= F,
                "SH_to_RGB_forward: degree %d unsupported or > features %d", degree, F);
   if (P == 0) return kOk;
-  auto kernel = degree > 3 ? sh_to_rgb_forward_kernel<64> : sh_to_rgb_forward_kernel<16>;
+  const bool rows = degree == 3 && F == 16 && ((uintptr_t) sh & 15) == 0;
+  auto kernel = degree > 3 ? sh_to_rgb_forward_kernel<64, false>
+                           : (rows ? sh_to_rgb_forward_kernel<16, true> : sh_to_rgb_forward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, F, degree,
                      clamp, pos, campos, sh, rgb);
   return check_launch("SH_to_RGB_forward");
@@ -612,7 +670,9 @@ FSGS_API int fsgs_sh_to_rgb_backward(int P, int F, int degree, int clamp, const 
                "SH_to_RGB_backward: degree %d unsupported or > features %d", degree, F);
   FSGS_REQUIRE(!grad_campos || campos, "SH_to_RGB_backward: grad_campos without campos");
   if (P == 0) return kOk;
-  auto kernel = degree > 3 ? sh_to_rgb_backward_kernel<64> : sh_to_rgb_backward_kernel<16>;
+  const bool rows = degree == 3 && F == 16 && (((uintptr_t) sh | (uintptr_t) grad_sh) & 15) == 0;
+  auto kernel = degree > 3 ? sh_to_rgb_backward_kernel<64, false>
+                           : (rows ? sh_to_rgb_backward_kernel<16, true> : sh_to_rgb_backward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, F, degree,
                      clamp, pos, campos, sh, rgb, grad_rgb, grad_dir, grad_campos, grad_sh);
   return check_launch("SH_to_RGB_backward");
