@@ -128,11 +128,13 @@ def cpu_baseline(scene, cam, budget_s: float = 20.0):
                       f"host has {os.cpu_count()} logical cpus"}
 
 
-def dynamic_step_rate(dev, steps: int = 20, warmup: int = 3):
+def dynamic_step_rate(dev, steps: int = 50, warmup: int = 10):
     """Config 3 (dynamic scene, 200k surfels, 512 control points): bf16 MFMA deformation MLP on the control points ->
     K-NN (k = 4) -> LBS -> render forward -> 0.8 L1 + 0.2 (1 - SSIM) (fused SSIM kernel) -> render backward -> masked Adam
     on the surfel parameters + Adam on the MLP weights and the control points (gradients reach them through the LBS and
-    K-NN backward kernels and the MLP's fp32 GEMM backward)."""
+    K-NN backward kernels and the MLP's MFMA backward kernels). The render takes `accum_max_count` as the reference's
+    training render does (network.py:706). Ten warm-up steps: the caching allocator and the optimisers' state settle
+    over the first few."""
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd.dynamic_step import DynamicStep
     scene_h, cam_h = scenes.config2(P=200_000, size=800, seed=2)

@@ -40,6 +40,9 @@ class DynamicStep:
                                       eps=1e-15)
         self.net_opt = torch.optim.Adam(list(self.net.parameters()) + [self.ctrl], lr=net_lr, fused=True)
         self.sh_degree = scene.sh_degree
+        # the reference's training render passes `accum_max_count` on every step (network.py:706): per Gaussian, the
+        # number of (pixel, blended entry) events at which it was the pixel's strongest contributor so far
+        self.accum_max_count = torch.zeros(self.params[0].shape[0], dtype=torch.int32, device=dev)
 
     def forward_loss(self, t: Tensor):
         """-> (loss, render outputs). Differentiable in the Gaussians' parameters, the control points and the network."""
@@ -52,7 +55,7 @@ class DynamicStep:
         cam = self.cam
         out = GS_2D_render(xyz, sc, rot, opacities, (cam.W, cam.H), cam.Tw2v, cam.Tv2c, campos=cam.campos,
                            near=cam.near, far=cam.far, sh_degree=self.sh_degree, sh_features=shs,
-                           background=self.background)
+                           background=self.background, accum_max_count=self.accum_max_count)
         return l1_dssim_loss(out['images'], self.target, self.lambda_dssim), out
 
     def step(self, t: Tensor):

@@ -77,7 +77,10 @@ def ptr(t):
 
 
 def current_stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """Raw handle of torch's current stream on the current device. The operators ask for it on every call, so it is read
+    through torch's C accessor (a fraction of a microsecond) rather than through `torch.cuda.current_stream()`, which
+    builds a Python Stream object (about 10 us, a dozen times per training step)."""
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
 
 
 def check(rc: int, what: str) -> None:

@@ -57,6 +57,9 @@ def test_full_size_step_runs_and_respects_the_mask(device):
     assert any(not torch.equal(a.detach(), b) for a, b in zip(state.net.parameters(), net_before))
     assert not torch.equal(state.ctrl.detach(), ctrl_before)
     assert all(torch.isfinite(p).all() for p in state.net.parameters()) and torch.isfinite(state.ctrl).all()
+    # accum_max_count travelled with every render (network.py:706): only surfels that were rendered hold counts
+    amc = state.accum_max_count
+    assert int(amc.sum()) > 0 and not amc[never].any() and int((amc > 0).sum()) > 1000
 
 
 def _ssim_torch(img1, img2):
