@@ -661,6 +661,9 @@ def main():
     ap.add_argument("--counter-run", action="store_true",
                     help="the process runs under a counter collection: every dispatch then carries the profiler's "
                          "serialisation, so the operator with the most launches looks largest; do not stop on that")
+    ap.add_argument("--only", choices=["knn_large"], default=None,
+                    help="run one side workload alone (for counter collections that must see a single kernel): "
+                         "knn_large = K-NN of 3M points against 2048 control points, k = 8, three launches")
     ap.add_argument("--surfels", type=int, default=300_000)
     ap.add_argument("--size", type=int, default=800)
     args = ap.parse_args()
@@ -677,6 +680,17 @@ def main():
     from fast_sp_gs_amd.renderer import render_step
 
     dev = torch.device("cuda:0")
+    if args.only == "knn_large":
+        g = torch.Generator().manual_seed(9)
+        pts = (torch.randn(3_000_000, 3, generator=g) * 2).to(dev)
+        ctrl = (torch.randn(2048, 3, generator=g) * 2).to(dev)
+        knn = get_C_function('knn_topk')
+        knn(pts, ctrl, 8)
+        torch.cuda.synchronize()
+        ms = _timed_ms(lambda: knn(pts, ctrl, 8), reps=2, warm=0)
+        print(json.dumps({"knn_large_ms": ms, "queries_per_s": pts.shape[0] / (ms * 1e-3),
+                          "workload": "3000000 x 2048, k = 8, D = 3"}))
+        return
     scene_h, cam_h = scenes.config2(P=args.surfels, size=args.size)
     scene, cam = scene_h.to(dev), cam_h.to(dev)
     gi = scene_h.extra['grad_image'].to(dev)

@@ -389,6 +389,19 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
   __syncthreads();
   const int n_todo = min(s_max_contrib, (int) (r1 - r0));
   const int rounds = (n_todo + kB - 1) / kB;
+  // No zero fill of the record buffer: every staged instance writes its record at the flush, zeros included, and the
+  // instances behind the tile's deepest contributor, which are never staged, are cleared here.
+  if (kSlots) {
+    for (int e = n_todo + (int) threadIdx.x; e < (int) (r1 - r0); e += kBlendThreads) {
+      const int id = point_list[r0 + e];
+      const float2 c = means2D[id];
+      const TileRect r = tile_rect(c.x, c.y, radii[id], gx, gy);
+      const int64_t at = (id == 0 ? 0 : point_offsets[id - 1]) + (int64_t) (tile_y - r.y0) * (r.x1 - r.x0) + (tile_x - r.x0);
+      float4* dst = (float4*) (slot_records + (size_t) at * kG3Slots);
+#pragma unroll
+      for (int c4 = 0; c4 < kG3Slots / 4; ++c4) dst[c4] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+  }
 
   const float T_final = inside ? 1.0f - out_opacity[pix] : 0.0f;
   float T = T_final;
@@ -480,14 +493,9 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
         a[c] = sum;
       }
       if (kSlots) {
-        bool any = false;
+        float4* dst = (float4*) (slot_records + slot * kG3Slots);
 #pragma unroll
-        for (int c = 0; c < kG3Slots; ++c) any |= a[c] != 0.0f;
-        if (any) {
-          float4* dst = (float4*) (slot_records + slot * kG3Slots);
-#pragma unroll
-          for (int c = 0; c < kG3Slots / 4; ++c) dst[c] = make_float4(a[4 * c], a[4 * c + 1], a[4 * c + 2], a[4 * c + 3]);
-        }
+        for (int c = 0; c < kG3Slots / 4; ++c) dst[c] = make_float4(a[4 * c], a[4 * c + 1], a[4 * c + 2], a[4 * c + 3]);
       } else {
         const int id = s_hot[threadIdx.x].id;
 #pragma unroll
@@ -811,7 +819,6 @@ FSGS_API int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const 
   }
   hipStream_t s = (hipStream_t) stream;
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
-  if (slots) launch_slot_clear<kG3Slots>(ws, R, s);
   const int* tile_order = nullptr;
   const int flags = launch_tile_order(gx, gy, ranges, s, &tile_order);
   const dim3 grid(gx * gy), block(kBlendThreads);

@@ -1,8 +1,10 @@
 // Per-surfel sums of per-(surfel, tile) gradient records in a fixed order, without atomics and without a zero fill of
 // the outputs. The tile binning emits a surfel's instances at consecutive positions of the unsorted key list, starting at
 // the surfel's prefix-scan offset; a backward block that has summed one instance over its tile's pixels writes the sums
-// as one record at that position (records nobody writes stay at the zero fill of the record buffer, a streaming write
-// that measured cheaper than per-instance "written" flags). slot_sum_kernel then adds a surfel's records in position
+// as one record at that position. Either every instance's record is written by the blend kernel itself, zeros included
+// (the standard surfel and the 3D-Gaussian blends: each block also clears the records of its tile's never-staged tail),
+// or the record buffer is zero-filled first (launch_slot_clear; the fast path, whose key spans contain padding positions
+// that belong to no tile's list). slot_sum_kernel then adds a surfel's records in position
 // order and hands every component of every surfel to a scatter functor that knows the output tensors. The reference flushes these sums with one device-scope atomic per component,
 // tile and surfel into caller-zeroed tensors (e.g. gaussian_render.cu:560-600, gs_2d_fast_redner.cu:520-560).
 #pragma once
