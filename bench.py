@@ -394,8 +394,29 @@ def gs3d_path_rate(dev, scene, cam, gi, steps: int = 30, warmup: int = 5):
         x_b()
     ev[2].record()
     torch.cuda.synchronize()
+    # the two backward decompositions on that view: one block per tile walking its list back to front (both operator
+    # names by default) against the reference's second algorithm, one lane per list entry with the pixels passed from
+    # lane to lane from the forward's bucket snapshots (gaussian_render.cu:540-694)
+    col = f('gs_preprocess_forward')(W, H, 3, False, scene.means3D, scales, scene.rotations, scene.opacities,
+                                     scene.shs, None, cam.Tw2v, cam.Tv2c, cam.campos, tan_fov, None, None, None, None)[2]
+    lens = ranges[:, 1] - ranges[:, 0]
+    b_off = torch.cumsum((lens + 31) // 32, 0).contiguous()
+    oc, oo2, _, nc2, max_c, b2t, s_T, s_ar = f('gaussian_rasterize_forward')(W, H, m2, co, col, None, pl, ranges, None,
+                                                                           None, None, b_off)
+    fast_bwd = f('gaussian_rasterize_fast_backward')
+    bwd_ms = {}
+    for name, per_gaussian in (("tile", False), ("per_gaussian", True)):
+        call = lambda: fast_bwd(m2, co, col, None, oc, None, oo2, gi, go, None, ranges, pl, nc2, max_c, b_off, b2t, s_T,
+                                s_ar, per_gaussian=per_gaussian)
+        bwd_ms[name] = _timed_ms(call, reps=10)
+
     return {"gs3d_path_frames_per_s": steps / dt,
             "gs3d_path_atomic_sums_frames_per_s": steps / dt_atomic,
+            "gs3d_backward_tile_kernel_ms": bwd_ms["tile"],
+            "gs3d_backward_per_gaussian_kernel_ms": bwd_ms["per_gaussian"],
+            "gs3d_backward_workload": f"gaussian_rasterize_fast_backward on that view with atomic sums, {b2t.numel()} "
+                                      f"buckets of 32 entries: back-to-front tile kernel / the reference's "
+                                      f"per-Gaussian decomposition (wavefront = 64 entries)",
             "gs3d_path_workload": f"same 300k centres as 3D Gaussians (third scale added), 800x800, SH degree 3, "
                                   f"R = {R[0]}: gs_preprocess fwd/bwd + GS_prepare + gaussian_rasterize fwd/bwd",
             "gs3d_extra16_forward_ms": ev[0].elapsed_time(ev[1]) / 10,

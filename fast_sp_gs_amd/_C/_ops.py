@@ -2011,17 +2011,24 @@ def _ordered_sum_inputs(what, P, point_list, point_offsets, radii, workspace_byt
     return True, _workspace(getattr(_lib(), workspace_bytes_fn)(R), device), R
 
 
+# Which kernel gaussian_rasterize_fast_backward runs when the caller does not say: the reference's per-Gaussian
+# decomposition (True) or the back-to-front kernel that gives the same derivative faster on this chip (False).
+PER_GAUSSIAN_BACKWARD = False
+
+
 def gaussian_rasterize_fast_backward(means2D: Tensor, conic_opacity: Tensor, colors: Tensor, extras: Optional[Tensor],
                                      images: Tensor, out_extras: Optional[Tensor], out_opacity: Tensor,
                                      dL_dout_color: Tensor, dL_dout_opacity: Tensor, dL_dout_extra: Optional[Tensor],
                                      ranges: Tensor, point_list: Tensor, n_contrib: Tensor, max_contrib: Tensor,
                                      per_tile_bucket_offset: Tensor, bucket_to_tile: Tensor, sampled_T: Tensor,
                                      sampled_ar: Tensor, point_offsets: Optional[Tensor] = None,
-                                     radii: Optional[Tensor] = None):
+                                     radii: Optional[Tensor] = None, per_gaussian: Optional[bool] = None):
     """gaussian_render.cu:760-812 -> (dL_dcolors[P,3], dL_dextras[P,E]|None, dL_dmeans2D[P,2], dL_dconic_opacity[P,4]):
     the reference's per-Gaussian backward over the forward's bucket snapshots. The same derivative as
-    gaussian_rasterize_backward, evaluated by the same kernel; the snapshot tensors are checked and not read.
-    `point_offsets` / `radii` as for gaussian_rasterize_backward."""
+    gaussian_rasterize_backward; by default it is evaluated by that operator's back-to-front kernel (the faster one on
+    this chip; the snapshot tensors are checked and not read). `per_gaussian=True` (default: PER_GAUSSIAN_BACKWARD of
+    this module) runs the reference's decomposition instead: one lane per list entry, pixels passed from lane to lane,
+    started from the snapshots. `point_offsets` / `radii` as for gaussian_rasterize_backward."""
     what = 'gaussian_rasterize_fast_backward'
     L.require_cuda(what, images=images, max_contrib=max_contrib, per_tile_bucket_offset=per_tile_bucket_offset,
                    bucket_to_tile=bucket_to_tile, sampled_T=sampled_T, sampled_ar=sampled_ar)
@@ -2054,10 +2061,14 @@ def gaussian_rasterize_fast_backward(means2D: Tensor, conic_opacity: Tensor, col
             c(out_opacity), c(n_contrib), c(max_contrib), c(per_tile_bucket_offset), c(bucket_to_tile), c(sampled_T),
             c(sampled_ar), c(dL_dout_color), c(dL_dout_extra) if E else None, c(dL_dout_opacity), c(point_list),
             c(ranges)]
-    with _timed('gaussian_rasterize_backward'):
-        rc = _lib().fsgs_gaussian_rasterize_fast_backward(
-            P, W, H, E, *[L.ptr(a) for a in args], L.ptr(dL_dmeans2D), L.ptr(dL_dconic_o), L.ptr(dL_dcolors),
-            L.ptr(dL_dextras), R, L.ptr(point_offsets) if ordered else None, L.ptr(radii) if ordered else None,
-            L.ptr(ws), ws.numel() if ws is not None else 0, L.current_stream())
+    tail = (L.ptr(dL_dmeans2D), L.ptr(dL_dconic_o), L.ptr(dL_dcolors), L.ptr(dL_dextras), R,
+            L.ptr(point_offsets) if ordered else None, L.ptr(radii) if ordered else None, L.ptr(ws),
+            ws.numel() if ws is not None else 0, L.current_stream())
+    if PER_GAUSSIAN_BACKWARD if per_gaussian is None else per_gaussian:
+        with _timed('gaussian_rasterize_bucket_backward'):
+            rc = _lib().fsgs_gaussian_rasterize_bucket_backward(P, W, H, E, B, *[L.ptr(a) for a in args], *tail)
+    else:
+        with _timed('gaussian_rasterize_backward'):
+            rc = _lib().fsgs_gaussian_rasterize_fast_backward(P, W, H, E, *[L.ptr(a) for a in args], *tail)
     L.check(rc, what)
     return dL_dcolors, dL_dextras, dL_dmeans2D, dL_dconic_o

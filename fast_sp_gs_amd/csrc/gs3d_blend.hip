@@ -517,6 +517,168 @@ __global__ void __launch_bounds__(kBlendThreads) gs3d_backward_kernel(int flags,
   }
 }
 
+// The reference's second backward (gaussian_render.cu:540-694), the per-Gaussian decomposition: a lane owns ONE list
+// entry of a tile and keeps that Gaussian's gradient sums in registers, the tile's pixels pass through the lanes one
+// lane per step, each carrying its blending state (transmittance and accumulated colour, front to back, started from
+// the forward's snapshot in front of the bucket), so no sum ever crosses lanes and nothing is reduced.
+// Laid out for a 64-lane wavefront: one wavefront takes 64 consecutive entries = two of the forward's 32-entry buckets
+// (the wavefront of the odd bucket leaves at once), the state moves with one whole-wavefront DPP shift per value, the
+// per-pixel constants (upstream gradients, final transmittance, last contributor, coordinates) are staged in LDS once
+// and read by pixel number instead of travelling through the lanes, and only the pixels that still blend at the
+// group's first entry (n_contrib beyond it) are fed in, so a deep group takes `live + 63` steps instead of 256 + 63.
+// Per-Gaussian results: one record per lane (kSlots; entries the pipeline never reaches write zeros) or atomics.
+template <int E, bool kSlots>
+__global__ void __launch_bounds__(64) gs3d_bucket_backward_kernel(int W, int H, const int64_t* __restrict__ ranges,
+    const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
+    const float4* __restrict__ conic_opacity, const float* __restrict__ colors, const float* __restrict__ extras,
+    const float* __restrict__ images, const float* __restrict__ out_extras, const float* __restrict__ out_opacity,
+    const int32_t* __restrict__ n_contrib, const int32_t* __restrict__ max_contrib,
+    const int64_t* __restrict__ bucket_offset, const int32_t* __restrict__ bucket_to_tile,
+    const float* __restrict__ sampled_T, const float* __restrict__ sampled_ar, const float* __restrict__ dL_dpix,
+    const float* __restrict__ dL_dout_extras, const float* __restrict__ dL_dout_opacity,
+    float* __restrict__ g_means2D, float* __restrict__ g_conic_opacity, float* __restrict__ g_colors,
+    float* __restrict__ g_extras, const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii,
+    float* __restrict__ slot_records) {
+  constexpr int kC = 3 + E;
+  __shared__ float4 s_grad[256];   // dL/d(r, g, b) of the pixel | T_final * dL/dopacity
+  __shared__ float4 s_state[256];  // snapshot: T | accumulated colour minus the final colour
+  __shared__ float4 s_pixel[256];  // x | y | last contributor (int bits) | -
+  __shared__ float s_extra[E > 0 ? 256 : 1][2 * (E > 0 ? E : 1)];  // extras: upstream gradient | accumulated minus final
+  const int bucket = blockIdx.x, lane = threadIdx.x;
+  const int tile = bucket_to_tile[bucket];
+  const int in_tile = bucket - (int) (tile == 0 ? 0 : bucket_offset[tile - 1]);
+  if (in_tile & 1) return;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const int tile_x = tile % gx, tile_y = tile / gx;
+  const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
+  const int first = in_tile * 32, entry = first + lane;
+  const bool valid = entry < (int) (r1 - r0);
+  const size_t HW = (size_t) H * W;
+
+  G3Hot hot{};
+  float feat[kC];
+#pragma unroll
+  for (int k = 0; k < kC; ++k) feat[k] = 0.0f;
+  size_t slot = 0;
+  if (valid) {
+    const G3Entry g = gather_gaussian<E>(point_list[r0 + entry], means2D, conic_opacity, colors, extras);
+    hot = g.hot;
+#pragma unroll
+    for (int k = 0; k < kC; ++k) feat[k] = g.feat[k];
+    if (kSlots) {
+      const TileRect r = tile_rect(hot.x, hot.y, radii[hot.id], gx, gy);
+      slot = (size_t) ((hot.id == 0 ? 0 : point_offsets[hot.id - 1]) + (int64_t) (tile_y - r.y0) * (r.x1 - r.x0) +
+                       (tile_x - r.x0));
+    }
+  }
+
+  // the pixels that still blend at this group's first entry, in row-major order of the tile
+  int n_live = 0;
+  if (first < max_contrib[tile]) {
+#pragma unroll
+    for (int part = 0; part < 4; ++part) {
+      const int rank = part * 64 + lane;
+      const int px = tile_x * kTile + (rank & 15), py = tile_y * kTile + (rank >> 4);
+      const bool inside = px < W && py < H;
+      const size_t pix = (size_t) W * py + px;
+      const int last = inside ? n_contrib[pix] : 0;
+      const bool live = last > first;
+      const unsigned long long live_lanes = wave_ballot(live);
+      if (live) {
+        const int at = n_live + __builtin_amdgcn_mbcnt_hi((unsigned) (live_lanes >> 32),
+                                                          __builtin_amdgcn_mbcnt_lo((unsigned) live_lanes, 0u));
+        const float T_final = 1.0f - out_opacity[pix];
+        s_grad[at]  = make_float4(dL_dpix[pix], dL_dpix[HW + pix], dL_dpix[2 * HW + pix], T_final * dL_dout_opacity[pix]);
+        const size_t snap = (size_t) bucket * 256 + rank;
+        s_state[at] = make_float4(sampled_T[snap], sampled_ar[((size_t) bucket * kC + 0) * 256 + rank] - images[pix],
+                                  sampled_ar[((size_t) bucket * kC + 1) * 256 + rank] - images[HW + pix],
+                                  sampled_ar[((size_t) bucket * kC + 2) * 256 + rank] - images[2 * HW + pix]);
+        s_pixel[at] = make_float4((float) px, (float) py, __int_as_float(last), 0.0f);
+#pragma unroll
+        for (int k = 0; k < E; ++k) {
+          s_extra[at][k]     = dL_dout_extras[k * HW + pix];
+          s_extra[at][E + k] = sampled_ar[((size_t) bucket * kC + 3 + k) * 256 + rank] - out_extras[k * HW + pix];
+        }
+      }
+      n_live += __builtin_popcountll(live_lanes);
+    }
+  }
+  __syncthreads();
+
+  float g[16];
+#pragma unroll
+  for (int c = 0; c < 16; ++c) g[c] = 0.0f;
+  float T = 0.0f, ar[kC];
+#pragma unroll
+  for (int k = 0; k < kC; ++k) ar[k] = 0.0f;
+  // whole-wavefront shift by one lane (DPP wave_shr:1); lane 0 keeps `fresh`
+  auto pass_on = [](float fresh, float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, fresh),
+                                                                 __builtin_bit_cast(int, v), 0x138, 0xf, 0xf, false));
+  };
+  const int steps = n_live > 0 ? n_live + 63 : 0;
+  float4 next_state = s_state[0];
+  for (int i = 0; i < steps; ++i) {
+    const int head = min(i, n_live - 1);  // the pixel that enters at lane 0 (nothing new once all have entered)
+    const float4 fresh = next_state;
+    next_state = s_state[min(i + 1, n_live - 1)];  // requested a step ahead of its use
+    T     = pass_on(fresh.x, T);
+    ar[0] = pass_on(fresh.y, ar[0]);
+    ar[1] = pass_on(fresh.z, ar[1]);
+    ar[2] = pass_on(fresh.w, ar[2]);
+#pragma unroll
+    for (int k = 0; k < E; ++k) ar[3 + k] = pass_on(s_extra[head][E + k], ar[3 + k]);
+    const int q = i - lane;
+    if (q < 0 || q >= n_live) continue;
+    const float4 pixel = s_pixel[q];
+    G3Hit h;
+    const bool hit = conic_alpha_flat(hot, pixel.x, pixel.y, h) && valid && entry < __float_as_int(pixel.z);
+    if (!hit) continue;
+    const float4 up = s_grad[q];
+    float dL[kC];
+    dL[0] = up.x, dL[1] = up.y, dL[2] = up.z;
+#pragma unroll
+    for (int k = 0; k < E; ++k) dL[3 + k] = s_extra[q][k];
+    const float w = h.alpha * T, inv = __builtin_amdgcn_rcpf(1.0f - h.alpha);
+    float dL_dalpha = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kC; ++k) {
+      ar[k] += w * feat[k];  // accumulated colour up to and including this Gaussian, minus the final colour
+      g[k < 3 ? k : 3 + (k - 3)] += w * dL[k];
+      dL_dalpha += (feat[k] * T + inv * ar[k]) * dL[k];
+    }
+    dL_dalpha += inv * up.w;  // through the final transmittance: dL/dT_final = -dL/dopacity, dT_final/dalpha = -T_final / (1 - alpha)
+    T *= 1.0f - h.alpha;
+    const float dL_dG = -hot.opacity * h.G * dL_dalpha;
+    g[7]  += dL_dG * (hot.a * h.dx + hot.b * h.dy);
+    g[8]  += dL_dG * (hot.c * h.dy + hot.b * h.dx);
+    g[9]  += 0.5f * h.dx * h.dx * dL_dG;
+    g[10] += h.dx * h.dy * dL_dG;
+    g[11] += 0.5f * h.dy * h.dy * dL_dG;
+    g[12] += h.G * dL_dalpha;
+  }
+  if (!valid) return;
+  if (kSlots) {
+    float4* dst = (float4*) (slot_records + slot * kG3Slots);
+#pragma unroll
+    for (int c = 0; c < kG3Slots / 4; ++c) dst[c] = make_float4(g[4 * c], g[4 * c + 1], g[4 * c + 2], g[4 * c + 3]);
+  } else {
+    const int id = hot.id;
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+      if (g[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], g[c]);
+#pragma unroll
+    for (int c = 0; c < E; ++c)
+      if (g[3 + c] != 0.0f) atomicAdd(&g_extras[(size_t) E * id + c], g[3 + c]);
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+      if (g[7 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], g[7 + c]);
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      if (g[9 + c] != 0.0f) atomicAdd(&g_conic_opacity[4 * (size_t) id + c], g[9 + c]);
+  }
+}
+
 // Largest n_contrib of the tile's 256 pixels: no pixel looks past that list position.
 __device__ __forceinline__ int block_max_contrib(int last_contrib, int* s_max) {
   if (threadIdx.x == 0) *s_max = 0;
@@ -849,8 +1011,9 @@ FSGS_API int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const 
 }
 
 // The reference's second backward walks 32-entry buckets from the forward's snapshots, one warp per bucket
-// (gaussian_render.cu:540-694). It evaluates the same derivative as the back-to-front kernel; here both names run
-// that kernel, and the snapshot arguments are accepted (and checked for presence) so that the binding is a drop-in.
+// (gaussian_render.cu:540-694). It evaluates the same derivative as the back-to-front kernel, which is the faster of
+// the two on this chip; this name runs that kernel, and the snapshot arguments are accepted (and checked for presence)
+// so that the binding is a drop-in. fsgs_gaussian_rasterize_bucket_backward below runs the per-Gaussian decomposition.
 FSGS_API int fsgs_gaussian_rasterize_fast_backward(int P, int W, int H, int E, const float* means2D,
     const float* conic_opacity, const float* colors, const float* extras, const float* images,
     const float* out_extras, const float* out_opacity, const int32_t* n_contrib, const int32_t* max_contrib,
@@ -866,6 +1029,63 @@ FSGS_API int fsgs_gaussian_rasterize_fast_backward(int P, int W, int H, int E, c
                                           dL_dpix, dL_dout_extras, dL_dout_opacity, point_list, ranges, g_means2D,
                                           g_conic_opacity, g_colors, g_extras, R, point_offsets, radii, workspace,
                                           workspace_bytes, stream);
+}
+
+// The per-Gaussian decomposition itself (gs3d_bucket_backward_kernel), for callers that want the reference's second
+// algorithm rather than its result: B = the number of 32-entry buckets the forward announced (bucket_to_tile's length).
+FSGS_API int fsgs_gaussian_rasterize_bucket_backward(int P, int W, int H, int E, int B, const float* means2D,
+    const float* conic_opacity, const float* colors, const float* extras, const float* images,
+    const float* out_extras, const float* out_opacity, const int32_t* n_contrib, const int32_t* max_contrib,
+    const int64_t* bucket_offset, const int32_t* bucket_to_tile, const float* sampled_T, const float* sampled_ar,
+    const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
+    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, int64_t R,
+    const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && B >= 0, "gaussian_rasterize_bucket_backward: bad sizes");
+  FSGS_REQUIRE(E >= 0 && E <= kMaxExtra, "gaussian_rasterize_bucket_backward: only 0..%d extra channels are supported",
+               kMaxExtra);
+  if (P == 0) return kOk;
+  FSGS_REQUIRE(means2D && conic_opacity && colors && images && out_opacity && n_contrib && max_contrib &&
+                   bucket_offset && sampled_T && sampled_ar && dL_dpix && dL_dout_opacity && ranges && g_means2D &&
+                   g_conic_opacity && g_colors && (B == 0 || (bucket_to_tile && point_list)) &&
+                   (E == 0 || (extras && out_extras && dL_dout_extras && g_extras)),
+               "gaussian_rasterize_bucket_backward: null pointer");
+  const bool slots = point_offsets != nullptr;
+  SlotWorkspace ws{nullptr};
+  if (slots) {
+    FSGS_REQUIRE(radii && workspace && R >= 0 && R < (int64_t) 0x7fffffff,
+                 "gaussian_rasterize_bucket_backward: the ordered-sum path needs radii, a workspace and the instance count R");
+    if (workspace_bytes < slot_workspace_bytes(R, kG3Slots))
+      return fail(kWorkspaceSmall, "gaussian_rasterize_bucket_backward: workspace %zu < %zu bytes", workspace_bytes,
+                  slot_workspace_bytes(R, kG3Slots));
+    FSGS_REQUIRE(((uintptr_t) workspace & 15) == 0, "gaussian_rasterize_bucket_backward: workspace must be 16-byte aligned");
+    ws = slot_workspace(workspace, R, kG3Slots);
+  }
+  hipStream_t s = (hipStream_t) stream;
+#define FSGS_G3_BKT(EE, SL)                                                                                          \
+  hipLaunchKernelGGL((gs3d_bucket_backward_kernel<EE, SL>), dim3(B), dim3(64), 0, s, W, H, ranges, point_list,       \
+                     (const float2*) means2D, (const float4*) conic_opacity, colors, extras, images, out_extras,     \
+                     out_opacity, n_contrib, max_contrib, bucket_offset, bucket_to_tile, sampled_T, sampled_ar,      \
+                     dL_dpix, dL_dout_extras, dL_dout_opacity, g_means2D, g_conic_opacity, g_colors, g_extras,       \
+                     point_offsets, radii, ws.records)
+#define FSGS_G3_BKT_E(EE)                                                                                            \
+  do {                                                                                                               \
+    if (slots) {                                                                                                     \
+      if (B > 0) FSGS_G3_BKT(EE, true);                                                                              \
+      launch_slot_sum<kG3Slots>(P, point_offsets, ws, G3Scatter<EE>{g_means2D, g_conic_opacity, g_colors, g_extras}, s); \
+    } else if (B > 0) {                                                                                              \
+      FSGS_G3_BKT(EE, false);                                                                                        \
+    }                                                                                                                \
+  } while (0)
+  switch (E) {
+    case 0: FSGS_G3_BKT_E(0); break;
+    case 1: FSGS_G3_BKT_E(1); break;
+    case 2: FSGS_G3_BKT_E(2); break;
+    case 3: FSGS_G3_BKT_E(3); break;
+    default: FSGS_G3_BKT_E(4); break;
+  }
+#undef FSGS_G3_BKT_E
+#undef FSGS_G3_BKT
+  return check_launch("gaussian_rasterize_bucket_backward");
 }
 
 FSGS_API int fsgs_gaussian_topk_weights(int topk, int P, int W, int H, const float* means2D,

@@ -444,6 +444,21 @@ int fsgs_gaussian_rasterize_fast_backward(int P, int W, int H, int E, const floa
     const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, int64_t R,
     const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The per-Gaussian decomposition of gaussian_render.cu:540-694 itself (fsgs_gaussian_rasterize_fast_backward returns the
+ * same derivative through the back-to-front kernel, which is faster here): a lane owns one list entry and keeps its
+ * sums in registers, the tile's pixels pass through the lanes carrying their front-to-back blending state, started from
+ * the forward's snapshots. One wavefront takes two 32-entry buckets; B = number of buckets (length of bucket_to_tile).
+ * With point_offsets == NULL: one device-scope atomic per Gaussian, tile and component into caller-zeroed outputs (the
+ * reference's :679-694); with point_offsets / radii / workspace every lane writes its record and the outputs are
+ * assigned from the ordered sums, as above. */
+int fsgs_gaussian_rasterize_bucket_backward(int P, int W, int H, int E, int B, const float* means2D,
+    const float* conic_opacity, const float* colors, const float* extras, const float* images,
+    const float* out_extras, const float* out_opacity, const int32_t* n_contrib, const int32_t* max_contrib,
+    const int64_t* bucket_offset, const int32_t* bucket_to_tile, const float* sampled_T, const float* sampled_ar,
+    const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,
+    const int64_t* ranges, float* g_means2D, float* g_conic_opacity, float* g_colors, float* g_extras, int64_t R,
+    const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- render epilogue -------------------------------------------------------------------------------------------- */
 
 /* Everything fast_2d_gs/renderer/gs_2d_render.py:608-617 does per pixel after the blend, in one kernel: normals[3,H,W] =

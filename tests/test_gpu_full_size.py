@@ -8,7 +8,8 @@
     (per-instance records summed in order / device-scope atomics) agree;
   * K-NN at 3M x 2048, k = 8: distances ascending, equal to the distance recomputed from the returned index, and no
     closer control point exists for a sample of queries (brute force with torch).
-Sizes: 300 000 surfels at 800x800, 3 000 000 surfels at 1352x1014 (one view), 400 000 surfels at 3840x2160.
+Sizes: 300 000 surfels at 800x800, 3 000 000 surfels at 1352x1014 (each of the four views), 400 000 surfels at
+3840x2160.
 The fast path and the 3D-Gaussian path get the same kind of checks at 300 000 / 800x800 (culling, ordered against atomic
 sums, linearity, weight sums; for the fast path also its two backward algorithms against each other).
 """
@@ -54,7 +55,8 @@ def _check_binning(out, W, H):
     assert bool(((m2[:, 1] + rad + 16 > ty * 16) & (m2[:, 1] - rad < (ty + 1) * 16)).all())
 
 
-@pytest.mark.parametrize("config", ["c2_300k_800", "c4_3m_1352x1014", "uhd_400k_3840x2160"])
+@pytest.mark.parametrize("config", ["c2_300k_800", "c4_3m_1352x1014_view0", "c4_3m_1352x1014_view1",
+                                    "c4_3m_1352x1014_view2", "c4_3m_1352x1014_view3", "uhd_400k_3840x2160"])
 def test_render_path_properties(config, device):
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd._C import get_C_function
@@ -65,7 +67,7 @@ def test_render_path_properties(config, device):
         cam_h = scenes.pinhole(3840, 2160, 40.0, torch.tensor([0.5, 0.3, 4.0]))
     else:
         scene_h, cams = scenes.config4()
-        cam_h = cams[1]
+        cam_h = cams[int(config[-1])]
     W, H = cam_h.W, cam_h.H
     g = torch.Generator().manual_seed(9)
     gi = torch.randn(3, H, W, generator=g).to(device)

@@ -507,6 +507,25 @@ def test_gs3d_bucket_snapshots_and_fast_backward(P, W, H, E, mul, device):
         assert (a is None) == (b is None), name
         if a is not None:
             assert rel_err(n(a), b) < 1e-3, (name, rel_err(n(a), b))
+    # the reference's decomposition itself (one lane per list entry, pixels passed from lane to lane, started from the
+    # snapshots): against the same oracle, with atomic sums and with ordered records (which must not depend on what
+    # the workspace held, and must leave no row of the outputs unwritten)
+    _, _, offsets = get_C_function('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True)
+    fb = get_C_function('gaussian_rasterize_fast_backward')
+    per_g = fb(m2, co, col, ex, oc, oe, oo, gi, go, ge, ranges, pl, nc, max_c, offset, b2t, sT, sar, per_gaussian=True)
+    # the operator takes its record workspace from torch's caching allocator: leave a poisoned block of that size there
+    from fast_sp_gs_amd import lib as L
+    poison = torch.full((L.load().fsgs_gaussian_rasterize_backward_workspace_bytes(pl.numel()) // 4,), float('nan'),
+                        device=device)
+    del poison
+    per_g_ordered = fb(m2, co, col, ex, oc, oe, oo, gi, go, ge, ranges, pl, nc, max_c, offset, b2t, sT, sar, offsets,
+                       rad, per_gaussian=True)
+    torch.cuda.synchronize()
+    for a, o, b, name in zip(per_g, per_g_ordered, want, ('colors', 'extras', 'means2D', 'conic_opacity')):
+        assert (a is None) == (b is None) == (o is None), name
+        if a is not None:
+            assert rel_err(n(a), b) < 1e-3, (name, rel_err(n(a), b))
+            assert np.isfinite(n(o)).all() and rel_err(n(o), b) < 1e-3, (name, rel_err(n(o), b))
     # end to end: the bucketed pair gives GS_render's gradients
     leaves = [t.clone().requires_grad_() for t in (m2, col, co)]
     leaves2 = [t.clone().requires_grad_() for t in (m2, col, co)]

@@ -735,6 +735,33 @@ def test_full_size_properties(device):
     enc = torch.empty(dirs.shape[0], 16, device=device)
     get_C_function('sh_encode_forward')(dirs, enc, dirs.shape[0], 3, 3)
     assert float((enc.square().sum(-1) - 16 / (4 * np.pi)).abs().max()) < 1e-5
+    # SH encoder backward at 1M directions. |Y(d)|^2 is constant on the sphere, so with the encoding itself as upstream
+    # gradient (the gradient of |Y|^2 / 2) nothing may be left tangentially to the sphere, whatever polynomial extension
+    # off the sphere the basis is written in; and the backward is linear in the upstream gradient.
+    B = dirs.shape[0]
+    g1, g2 = torch.empty(B, 3, device=device), torch.empty(B, 3, device=device)
+    get_C_function('sh_encode_backward')(enc, dirs, B, 3, 3, g1)
+    tangential = g1 - (g1 * dirs).sum(-1, keepdim=True) * dirs
+    assert float(tangential.abs().max()) < 2e-5
+    up = torch.randn(B, 16, generator=torch.Generator().manual_seed(2)).to(device)
+    get_C_function('sh_encode_backward')(up, dirs, B, 3, 3, g1)
+    get_C_function('sh_encode_backward')(up * -3.0, dirs, B, 3, 3, g2)
+    assert float((g2 + 3.0 * g1).abs().max()) < 1e-5 * max(1.0, float(g1.abs().max()))
+    # SH -> RGB at 1M points through the other kernel family: positions on the unit sphere seen from the origin give
+    # the directions themselves, so the colours are the encoder's rows contracted with the coefficients, + 0.5, clamped;
+    # the backward's coefficient gradient is the outer product of the clamped upstream gradient and the same rows
+    shs = c['shs'].to(device)
+    origin = torch.zeros(3, device=device)
+    rgb = get_C_function('SH_to_RGB_forward')(dirs, origin, shs, 3, True)
+    want = torch.clamp_min(torch.einsum('pk,pkc->pc', enc.double(), shs.double()) + 0.5, 0.0)
+    assert float((rgb.double() - want).abs().max()) < 2e-6
+    g_rgb = torch.randn(B, 3, generator=torch.Generator().manual_seed(3)).to(device)
+    g_sh, g_pos, g_cam = torch.empty_like(shs), torch.empty_like(dirs), torch.zeros(3, device=device)
+    get_C_function('SH_to_RGB_backward')(3, True, dirs, origin, shs, rgb, g_rgb, g_pos, g_cam, g_sh)
+    masked = (g_rgb * (rgb > 0)).double()
+    assert float((g_sh.double() - enc.double()[:, :, None] * masked[:, None, :]).abs().max()) < 2e-6
+    assert float((g_pos * dirs).sum(-1).abs().max()) < 1e-4  # a direction's gradient has no radial part
+    assert float((g_cam.double() + g_pos.double().sum(0)).abs().max()) < 1e-3 * max(1.0, float(g_pos.abs().sum(0).max()))
 
 
 def test_deform_mlp_mfma(device, oracle_mod):
