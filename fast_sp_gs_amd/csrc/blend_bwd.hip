@@ -64,7 +64,8 @@ blend_backward_kernel(
     const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii, float* __restrict__ slot_grads,
     const float4* __restrict__ records) {
   constexpr bool kQueue = kBwdQueue && !kFlow;
-  __shared__ SplatHot s_hot[kBwdBatch];
+  __shared__ SplatHot s_hot[kBwdBatch];  // read by the order-free pass (the planes k, l themselves) and the flow variant
+  __shared__ SplatRay s_ray[kBwdBatch];  // read by the per-pixel test
   __shared__ SplatCold s_cold[kBwdBatch];
   // Each wavefront's sums over its 64 pixels, one row per staged surfel; the flush adds the four rows in wavefront
   // order, so a tile's sums do not depend on timing. +1: the odd stride keeps the flush free of bank conflicts.
@@ -75,11 +76,8 @@ blend_backward_kernel(
   __shared__ float s_t2[kFlow ? kBwdBatch * 9 : 1];
   __shared__ int s_max_contrib;
   __shared__ unsigned char s_mask[kBwdBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
-  // queued pairs, and the upstream gradients of the tile's pixels (the lane that turns a queued pair into gradient
-  // components is not the lane that owns the pixel): image 3 + normal 3 per pixel
+  // queued pairs
   __shared__ float4 s_queue[kQueue ? 4 : 1][kQueue ? kQueueItems : 1];
-  __shared__ float4 s_up4[kQueue ? kBlendThreads : 1];
-  __shared__ float2 s_up2[kQueue && kAux ? kBlendThreads : 1];
 
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int tile = scheduled_tile(ordered, tile_order), tile_x = tile % gx, tile_y = tile / gx;
@@ -151,10 +149,6 @@ blend_backward_kernel(
       sum_w      = out_extras[pix + 8 * HW];
     }
   }
-  if (kQueue) {  // read back by this wavefront only: no barrier needed
-    s_up4[threadIdx.x] = make_float4(dLp0, dLp1, dLp2, dLn0);
-    if (kAux) s_up2[threadIdx.x] = make_float2(dLn1, dLn2);
-  }
   const float final_A   = 1.0f - T_final;
   const float far_scale = far_n / (far_n - near_n);
   float dLf0 = 0, dLf1 = 0, dL_dsum_w = 0;
@@ -199,6 +193,7 @@ blend_backward_kernel(
     const int n_here = min(kBwdBatch, n_todo - b * kBwdBatch);
     if (st >= 0 && st < n_here) {
       s_hot[st]  = next.hot;
+      s_ray[st]  = make_ray(next.hot);
       s_cold[st] = next.cold;
       s_mask[st] = (unsigned char) quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile, ordered);
       if (kFlow)
@@ -276,7 +271,12 @@ blend_backward_kernel(
         const int bits = __float_as_int(it.w);
         const int qp = bits & 63;
         const bool blends = (bits & kItemHit) != 0, by_ray = (bits & kItemRay) != 0;
-        const float4 up = s_up4[wave * kWave + qp];
+        // the upstream gradients of the pair's pixel sit in the registers of the lane that owns it (lane qp of this
+        // wavefront): fetched with lane permutes, no LDS copy of them is kept
+        auto from_owner = [&](float v) {
+          return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(qp << 2, __builtin_bit_cast(int, v)));
+        };
+        const float up_x = from_owner(dLp0), up_y = from_owner(dLp1), up_z = from_owner(dLp2);
         const float fx = qx0 + (float) (qp & 7), fy = qy0 + (float) (qp >> 3);
         const float w = it.x, GdA = it.y, dL_dz = it.z;
         const float kx = fx * hot.m[6] - hot.m[0], ky = fx * hot.m[7] - hot.m[1], kz = fx * hot.m[8] - hot.m[2];
@@ -293,15 +293,14 @@ blend_backward_kernel(
         // gradients): p_xy = s p_z, so dp_xy = ds / p_z and dp_z = -<ds, s> / p_z
         const float npx = -(dsx * rz_p), npy = -(dsy * rz_p), npz = s_ds * rz_p;
         float g[16];
-        g[0] = w * up.x, g[1] = w * up.y, g[2] = w * up.z;
+        g[0] = w * up_x, g[1] = w * up_y, g[2] = w * up_z;
         g[3] = ly * npz - lz * npy, g[4] = lz * npx - lx * npz, g[5] = lx * npy - ly * npx;
         g[6] = npy * kz - npz * ky, g[7] = npz * kx - npx * kz, g[8] = npx * ky - npy * kx;
         g[9]  = dL_dz * sx - (fx * g[3] + fy * g[6]);
         g[10] = dL_dz * sy - (fx * g[4] + fy * g[7]);
         g[11] = dL_dz - (fx * g[5] + fy * g[8]);
         if (kAux) {
-          const float2 un = s_up2[wave * kWave + qp];
-          g[12] = w * up.w, g[13] = w * un.x, g[14] = w * un.y;
+          g[12] = w * from_owner(dLn0), g[13] = w * from_owner(dLn1), g[14] = w * from_owner(dLn2);
         } else {
           g[12] = g[13] = g[14] = 0.0f;
         }
@@ -341,11 +340,11 @@ blend_backward_kernel(
         else q_head = 0, q_count = 0;
       };
       // ---- order-bound part of one entry, and the append of its blending pixels to the queue -----------------------------
-      auto queue_entry = [&](const SplatHot& hot, const SplatCold& cold, int j) {
+      auto queue_entry = [&](const SplatRay& hot, const SplatCold& cold, int j) {
         const int pos = n_todo - 1 - (b * kBwdBatch + j);  // 0-based position in the tile's list
         Hit h;
         unsigned long long pass;
-        const bool hit = intersect_flat(hot, pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
+        const bool hit = intersect_ray(hot, pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
         pass &= wave_ballot(pos < last_contrib);
         if (pass == 0ull) return;  // wave-uniform: nobody in this quadrant blends the surfel
         float w = 0.0f, dL_dalpha = 0.0f, dL_dz = 0.0f;
@@ -379,11 +378,11 @@ blend_backward_kernel(
           return j;
         };
         auto peek = [&]() { return todo ? (int) __builtin_ctzll(todo) : 0; };
-        SplatHot hot_a = s_hot[peek()], hot_b;
+        SplatRay hot_a = s_ray[peek()], hot_b;
         while (todo) {
           {
             const int j = pop();
-            hot_b       = s_hot[peek()];
+            hot_b       = s_ray[peek()];
             const SplatCold cold = s_cold[j];
             __builtin_amdgcn_sched_barrier(0);
             queue_entry(hot_a, cold, j);
@@ -391,7 +390,7 @@ blend_backward_kernel(
           if (todo == 0ull) break;
           {
             const int j = pop();
-            hot_a       = s_hot[peek()];
+            hot_a       = s_ray[peek()];
             const SplatCold cold = s_cold[j];
             __builtin_amdgcn_sched_barrier(0);
             queue_entry(hot_b, cold, j);
@@ -464,9 +463,12 @@ blend_backward_kernel(
       const int pos = n_todo - 1 - (b * kBwdBatch + j);  // 0-based position in the tile's list
       Hit h;
       unsigned long long pass;
-      const bool hit = intersect_flat(hot, pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
+      const bool hit = intersect_ray(s_ray[j], pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
       pass &= wave_ballot(pos < last_contrib);
       if (pass == 0ull) return;  // wave-uniform: nobody in this quadrant blends the surfel
+      // the two planes through the pixel themselves: the gradients of the transform's rows are taken through them
+      h.kx = pxf * hot.m[6] - hot.m[0], h.ky = pxf * hot.m[7] - hot.m[1], h.kz = pxf * hot.m[8] - hot.m[2];
+      h.lx = pyf * hot.m[6] - hot.m[3], h.ly = pyf * hot.m[7] - hot.m[4], h.lz = pyf * hot.m[8] - hot.m[5];
 
       float g[16], g2x, g2y;
       unsigned long long ray_lanes;
