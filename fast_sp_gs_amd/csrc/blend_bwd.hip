@@ -149,8 +149,12 @@ blend_backward_kernel(
       sum_w      = out_extras[pix + 8 * HW];
     }
   }
-  const float final_A   = 1.0f - T_final;
-  const float far_scale = far_n / (far_n - near_n);
+  const float far_scale = far_n / (far_n - near_n), far_near = far_scale * near_n;
+  // The distortion term's per-pixel constants, folded once: with m the normalised depth of a pair,
+  //   dL/dweight = (D2 + m^2 A - 2 m D) dL/dreg = reg_D2 + m (m reg_A - reg_2D),
+  //   dL/dm      = 2 w (m A - D) dL/dreg        = w (m reg_2A - reg_2D).
+  const float reg_A = (1.0f - T_final) * dL_dreg, reg_2A = 2.0f * reg_A, reg_2D = 2.0f * final_D * dL_dreg,
+              reg_D2 = final_D2 * dL_dreg;
   float dLf0 = 0, dLf1 = 0, dL_dsum_w = 0;
   if (kFlow && inside) {
     const float2 g = dL_dflow[pix], o = out_flow[pix];
@@ -159,7 +163,7 @@ blend_backward_kernel(
   }
 
   float acc_lin = 0, last_lin = 0;
-  float last_dL_dT = 0, last_alpha = 0, acc_w = 0;
+  float last_alpha = 0, acc_w = 0;
   float acc_f0 = 0, acc_f1 = 0, last_f0 = 0, last_f1 = 0;
   // the wavefront's queue: items [q_head, q_head + q_count) of its ring (wave-uniform, multiples of 16)
   int q_head = 0, q_count = 0;
@@ -238,20 +242,20 @@ blend_backward_kernel(
       float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
       if (kAux) {
         const float rd     = __builtin_amdgcn_rcpf(h.depth);
-        const float m_d    = far_scale * (1.0f - near_n * rd);
-        const float dmd_dd = far_scale * near_n * rd * rd;
+        const float m_d    = far_scale - far_near * rd;
+        const float dmd_dd = far_near * rd * rd;
         if (pos == median_contrib - 1) dL_dz += dL_dmedian;
-        const float dL_dweight = (final_D2 + m_d * m_d * final_A - 2.0f * m_d * final_D) * dL_dreg;
-        dL_dalpha += dL_dweight - last_dL_dT;
-        last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
-        const float dL_dmd = 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg;
+        // the distortion's dL/dweight enters dL/dalpha exactly as a linear channel does (its own value minus what the
+        // pairs behind it accumulated, with the same weights), so it rides on the shared recurrence
+        c_lin += reg_D2 + m_d * (m_d * reg_A - reg_2D);
+        const float dL_dmd = w * (m_d * reg_2A - reg_2D);
         dL_dz += dL_dmd * dmd_dd;
         c_lin += h.depth * dL_ddepth + dL_daccum + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
         dL_dz += w * dL_ddepth;
       }
       acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
       last_lin = c_lin;
-      dL_dalpha += c_lin - acc_lin;
+      dL_dalpha = c_lin - acc_lin;
     };
     if (kQueue) {
       // ---- order-free part: 64 queued pairs at a time, four 16-lane rows, every row one entry ---------------------------

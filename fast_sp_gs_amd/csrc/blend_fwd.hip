@@ -67,7 +67,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
   float live = inside ? 1.0f : -1.0f;
   // the same for the wavefront, as a lane mask in scalar registers: "is anybody still blending" costs no vector work
   unsigned long long live_lanes = wave_ballot(inside);
-  const float far_scale = far_n / (far_n - near_n);
+  const float far_scale = far_n / (far_n - near_n), far_near = far_scale * near_n;
   float T = 1.0f, C0 = 0, C1 = 0, C2 = 0;
   float N0 = 0, N1 = 0, N2 = 0, D = 0, M1 = 0, M2 = 0, dist = 0, median = 0, wsum = 0, f0 = 0, f1 = 0;
   int last = 0, median_c = -1;
@@ -153,7 +153,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
           const int contributor = b * kFwdBatch + j + 1;
           if (kAux) {
             const float A  = 1.0f - T;
-            const float m  = far_scale * fmaf(-near_n, __builtin_amdgcn_rcpf(h.depth), 1.0f);
+            const float m  = fmaf(-far_near, __builtin_amdgcn_rcpf(h.depth), far_scale);
             const float mm = m * m;
             dist = fmaf(fmaf(-2.0f * m, M1, fmaf(mm, A, M2)), w, dist);
             D    = fmaf(h.depth, w, D);

@@ -418,11 +418,14 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
       }
     }
   }
-  const float final_A   = 1.0f - T_final;
-  const float far_scale = far_n / (far_n - near_n);
+  const float far_scale = far_n / (far_n - near_n), far_near = far_scale * near_n;
+  // the distortion term's per-pixel constants, folded once: with m the normalised depth of a pair,
+  //   dL/dweight = (D2 + m^2 A - 2 m D) dL/dreg = reg_D2 + m (m reg_A - reg_2D),  dL/dm = w (m reg_2A - reg_2D)
+  const float reg_A = (1.0f - T_final) * dL_dreg, reg_2A = 2.0f * reg_A, reg_2D = 2.0f * final_D * dL_dreg,
+              reg_D2 = final_D2 * dL_dreg;
 
   float acc_lin = 0, last_lin = 0;
-  float last_dL_dT = 0, last_alpha = 0;
+  float last_alpha = 0;
 
   FastSplat next;
   float next_t2[9];
@@ -491,14 +494,14 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
           float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
           if (kAux) {
             const float rd     = __builtin_amdgcn_rcpf(h.depth);
-            const float m_d    = far_scale * (1.0f - near_n * rd);
-            const float dmd_dd = far_scale * near_n * rd * rd;
+            const float m_d    = far_scale - far_near * rd;
+            const float dmd_dd = far_near * rd * rd;
             if (pos == median_contrib - 1) dL_dz += dL_dmedian;
             if (!kPerSplat) {
-              const float dL_dweight = (final_D2 + m_d * m_d * final_A - 2.0f * m_d * final_D) * dL_dreg;
-              dL_dalpha += dL_dweight - last_dL_dT;
-              last_dL_dT = dL_dweight * h.alpha + (1.0f - h.alpha) * last_dL_dT;
-              dL_dz += 2.0f * (T * h.alpha) * (m_d * final_A - final_D) * dL_dreg * dmd_dd;
+              // dL/dweight of the distortion enters dL/dalpha as a linear channel does (its value minus what the pairs
+              // behind it accumulated, with the same weights): it rides on the shared recurrence
+              c_lin += reg_D2 + m_d * (m_d * reg_A - reg_2D);
+              dL_dz += w * (m_d * reg_2A - reg_2D) * dmd_dd;
             } else {
               c_lin += m_d * dL_dM1 + (m_d * m_d) * dL_dM2;
               dL_dz += dmd_dd * (2.0f * m_d * w * dL_dM2);
