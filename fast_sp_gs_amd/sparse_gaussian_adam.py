@@ -19,41 +19,46 @@ class SparseGaussianAdam(torch.optim.Adam):
         self.N = None
         self.visibility = None
 
+    def _advance(self, param):
+        """The parameter's optimiser state with its step count advanced; created on first use with the keys torch's
+        Adam uses (sparse_gaussian_adam.py:28-33), so checkpoints of either optimiser load into the other."""
+        state = self.state[param]
+        if not state:
+            state.update(step=torch.zeros((), dtype=torch.float32),
+                         exp_avg=torch.zeros_like(param, memory_format=torch.preserve_format),
+                         exp_avg_sq=torch.zeros_like(param, memory_format=torch.preserve_format))
+        state['step'] += 1
+        return state
+
     @torch.no_grad()
     def step(self):
-        """The reference's loop over parameter groups (sparse_gaussian_adam.py:20-45), with the groups' kernels folded
-        into one launch per `_MAX` tensors; the arithmetic per element is the single-tensor kernel's."""
-        params, grads, ms, vs, lrs, epss = [], [], [], [], [], []
+        """One masked Adam update of every parameter group that has a gradient (sparse_gaussian_adam.py:20-45), the
+        groups' kernels folded into one launch per `_MAX` tensors; the arithmetic per element is the single-tensor
+        kernel's."""
+        jobs = []  # (param, grad, first moment, second moment, effective rate, eps)
         corrections = {}  # step count -> the two bias corrections, shared by the groups that are at that count
         for group in self.param_groups:
-            lr = group["lr"]
-            eps = group["eps"]
-            assert len(group["params"]) == 1, "more than one tensor in group"
+            if len(group["params"]) != 1:
+                raise AssertionError("more than one tensor in group")
             param = group["params"][0]
             if param.grad is None or param.grad.numel() == 0:
                 continue
-            state = self.state[param]
-            if len(state) == 0:  # lazy state initialisation
-                state['step'] = torch.tensor(0.0, dtype=torch.float32)
-                state['exp_avg'] = torch.zeros_like(param, memory_format=torch.preserve_format)
-                state['exp_avg_sq'] = torch.zeros_like(param, memory_format=torch.preserve_format)
-            state['step'] += 1
-            step = state['step']
-            params.append(param), grads.append(param.grad), ms.append(state["exp_avg"]), vs.append(state["exp_avg_sq"])
+            state = self._advance(param)
             # Bias corrections folded into the learning rate: lr * sqrt(1 - b2^t) / (1 - b1^t). The reference evaluates
-            # this on `step`, a float32 tensor (sparse_gaussian_adam.py:42-46), so every operation rounds to float32
-            # and the product is widened to double at the call. The powers are taken by torch on the float32 tensor as
-            # there; the multiplication and division that follow are single correctly rounded float32 operations.
-            key = float(step)
+            # this on the step count as a float32 tensor (sparse_gaussian_adam.py:42-46), so every operation rounds to
+            # float32 and the product is widened to double at the call. The powers are taken by torch on the float32
+            # tensor as there; the multiplication and division that follow are single correctly rounded float32
+            # operations.
+            t = state['step']
+            key = float(t)
             if key not in corrections:
-                corrections[key] = (np.float32(((1 - 0.999 ** step) ** 0.5).item()),
-                                    np.float32((1 - 0.9 ** step).item()))
+                corrections[key] = (np.float32(((1 - 0.999 ** t) ** 0.5).item()), np.float32((1 - 0.9 ** t).item()))
             root_c2, c1 = corrections[key]
-            lrs.append(float(np.float32(lr) * root_c2 / c1))
-            epss.append(eps)
-        for i in range(0, len(params), self._MAX):
-            j = slice(i, i + self._MAX)
-            self._update_multi_C(params[j], grads[j], ms[j], vs[j], self.visibility, lrs[j], 0.9, 0.999, epss[j], self.N)
+            jobs.append((param, param.grad, state["exp_avg"], state["exp_avg_sq"],
+                         float(np.float32(group["lr"]) * root_c2 / c1), group["eps"]))
+        for i in range(0, len(jobs), self._MAX):
+            p, g, m, v, rates, epss = map(list, zip(*jobs[i:i + self._MAX]))
+            self._update_multi_C(p, g, m, v, self.visibility, rates, 0.9, 0.999, epss, self.N)
 
     def set_before_step(self, visibility, N):
         self.visibility, self.N = visibility, N
