@@ -151,10 +151,10 @@ blend_backward_kernel(
   }
   const float far_scale = far_n / (far_n - near_n), far_near = far_scale * near_n;
   // The distortion term's per-pixel constants, folded once: with m the normalised depth of a pair,
-  //   dL/dweight = (D2 + m^2 A - 2 m D) dL/dreg = reg_D2 + m (m reg_A - reg_2D),
+  //   dL/dweight = (D2 + m^2 A - 2 m D) dL/dreg = D2 dL/dreg + m (m reg_A - reg_2D),
   //   dL/dm      = 2 w (m A - D) dL/dreg        = w (m reg_2A - reg_2D).
   const float reg_A = (1.0f - T_final) * dL_dreg, reg_2A = 2.0f * reg_A, reg_2D = 2.0f * final_D * dL_dreg,
-              reg_D2 = final_D2 * dL_dreg;
+              lin_const = final_D2 * dL_dreg + dL_daccum;  // dL/dweight's constant and the opacity map's gradient
   float dLf0 = 0, dLf1 = 0, dL_dsum_w = 0;
   if (kFlow && inside) {
     const float2 g = dL_dflow[pix], o = out_flow[pix];
@@ -162,7 +162,7 @@ blend_backward_kernel(
     dLf0 = g.x / sum_w, dLf1 = g.y / sum_w;
   }
 
-  float acc_lin = 0, last_lin = 0;
+  float acc_lin = 0;
   float last_alpha = 0, acc_w = 0;
   float acc_f0 = 0, acc_f1 = 0, last_f0 = 0, last_f1 = 0;
   // the wavefront's queue: items [q_head, q_head + q_count) of its ring (wave-uniform, multiples of 16)
@@ -234,28 +234,34 @@ blend_backward_kernel(
     // ---- order-bound part of one (pixel, entry) pair: advances the pixel's back-to-front state -------------------------
     // All channels that enter the image linearly (colour, depth, opacity, normal) share one recurrence: with
     // c = <upstream gradient, channel values of this surfel>, the reference's per-channel accumulators
-    // acc_x = last_alpha * last_x + (1 - last_alpha) * acc_x contract to a single scalar. Leaves the blend weight w,
-    // dL/dalpha and dL/ddepth of the pair; call under `hit` only.
+    // acc_x = last_alpha * last_x + (1 - last_alpha) * acc_x contract to a single scalar, updated at the end of the
+    // pair that supplies alpha and x. Leaves the blend weight w, dL/dalpha and dL/ddepth of the pair; call under `hit`
+    // only.
     auto advance_pixel = [&](const SplatCold& cold, int pos, const Hit& h, float& w, float& dL_dalpha, float& dL_dz) {
-      T = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+      const float keep = 1.0f - h.alpha;
+      T = T * __builtin_amdgcn_rcpf(keep);
       w = h.alpha * T;
-      float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
+      // one chain of fused multiply-adds; the per-pixel constant of the distortion term sits in lin_const
+      float c_lin;
       if (kAux) {
         const float rd     = __builtin_amdgcn_rcpf(h.depth);
-        const float m_d    = far_scale - far_near * rd;
+        const float m_d    = fmaf(-far_near, rd, far_scale);
         const float dmd_dd = far_near * rd * rd;
-        if (pos == median_contrib - 1) dL_dz += dL_dmedian;
-        // the distortion's dL/dweight enters dL/dalpha exactly as a linear channel does (its own value minus what the
+        // dL/dweight of the distortion enters dL/dalpha exactly as a linear channel does (its own value minus what the
         // pairs behind it accumulated, with the same weights), so it rides on the shared recurrence
-        c_lin += reg_D2 + m_d * (m_d * reg_A - reg_2D);
-        const float dL_dmd = w * (m_d * reg_2A - reg_2D);
-        dL_dz += dL_dmd * dmd_dd;
-        c_lin += h.depth * dL_ddepth + dL_daccum + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
-        dL_dz += w * dL_ddepth;
+        c_lin = fmaf(h.depth, dL_ddepth, lin_const);
+        c_lin = fmaf(m_d, fmaf(m_d, reg_A, -reg_2D), c_lin);
+        c_lin = fmaf(cold.nx, dLn0, fmaf(cold.ny, dLn1, fmaf(cold.nz, dLn2, c_lin)));
+        // dL/ddepth: through the distortion's normalised depth, the depth map, and the median depth
+        const float per_w = fmaf(fmaf(m_d, reg_2A, -reg_2D), dmd_dd, dL_ddepth);
+        dL_dz = fmaf(w, per_w, pos == median_contrib - 1 ? dL_dmedian : 0.0f);
+      } else {
+        c_lin = 0.0f;
       }
-      acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
-      last_lin = c_lin;
+      c_lin = fmaf(cold.r, dLp0, fmaf(cold.g, dLp1, fmaf(cold.b, dLp2, c_lin)));
+      // acc_lin: what the pairs behind this one accumulated, alpha_j c_j weighted by the transmittance between
       dL_dalpha = c_lin - acc_lin;
+      acc_lin   = fmaf(keep, acc_lin, h.alpha * c_lin);
     };
     if (kQueue) {
       // ---- order-free part: 64 queued pairs at a time, four 16-lane rows, every row one entry ---------------------------
@@ -355,7 +361,6 @@ blend_backward_kernel(
         if (hit) {
           advance_pixel(cold, pos, h, w, dL_dalpha, dL_dz);
           dL_dalpha *= T * h.G;  // only G * dL/dalpha is ever used
-          last_alpha = h.alpha;
         }
         // blending lanes take the first popcount(pass) places in lane order; the next lanes that do not blend fill the
         // row up with neutral items (zeros, no flags, their own pixel: every number formed from it is finite)

@@ -424,8 +424,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
   const float reg_A = (1.0f - T_final) * dL_dreg, reg_2A = 2.0f * reg_A, reg_2D = 2.0f * final_D * dL_dreg,
               reg_D2 = final_D2 * dL_dreg;
 
-  float acc_lin = 0, last_lin = 0;
-  float last_alpha = 0;
+  float acc_lin = 0;  // what the pairs behind the current one accumulated: alpha_j c_j weighted by the transmittance between
 
   FastSplat next;
   float next_t2[9];
@@ -524,11 +523,9 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
             fsx = Q[0] * gu + Q[3] * gv + Q[6] * gw;
             fsy = Q[1] * gu + Q[4] * gv + Q[7] * gw;
           }
-          acc_lin  = last_alpha * last_lin + (1.0f - last_alpha) * acc_lin;
-          last_lin = c_lin;
           dL_dalpha += c_lin - acc_lin;
+          acc_lin = fmaf(1.0f - h.alpha, acc_lin, h.alpha * c_lin);
           dL_dalpha *= T;
-          last_alpha = h.alpha;
 
           // d/ds of the intersection case (times 1 / p_z below); s is not finite in a lane whose p_z is 0, and such a
           // lane never blends: every use of s sits on this side
