@@ -131,6 +131,27 @@ __device__ __forceinline__ SplatRay make_ray(const SplatHot& h) {
   return r;
 }
 
+// A staged batch of SplatRays in LDS, stored as four planes of 16-byte quarters: the lanes that stage a batch write
+// consecutive 16-byte pieces (a 64-byte stride per lane would put every second lane on the same banks), and a
+// wavefront reads an entry's four quarters as four broadcasts.
+template <int kN>
+struct RayBatch {
+  float4 q[4][kN];
+  __device__ __forceinline__ void put(int i, const SplatRay& r) {
+    q[0][i] = make_float4(r.ax, r.ay, r.az, r.bx);
+    q[1][i] = make_float4(r.by, r.bz, r.px, r.py);
+    q[2][i] = make_float4(r.pz, r.wx, r.wy, r.wz);
+    q[3][i] = make_float4(r.cx, r.cy, r.opacity, 0.0f);
+  }
+  __device__ __forceinline__ SplatRay get(int j) const {
+    const float4 a = q[0][j], b = q[1][j], c = q[2][j], d = q[3][j];
+    SplatRay r;
+    r.ax = a.x, r.ay = a.y, r.az = a.z, r.bx = a.w, r.by = b.x, r.bz = b.y, r.px = b.z, r.py = b.w;
+    r.pz = c.x, r.wx = c.y, r.wy = c.z, r.wz = c.w, r.cx = d.x, r.cy = d.y, r.opacity = d.z, r.pad = 0.0f;
+    return r;
+  }
+};
+
 // Ray-splat intersection and alpha of one surfel at one pixel (gs_2d_redner.cu:122-155); false where the reference
 // would `continue`. No early exits: every lane runs the whole sequence and the rejections are combined at the end, so the
 // caller gets one predicate instead of nested divergent regions. Contraction is switched off and every fused
