@@ -99,59 +99,6 @@ struct Hit {
   float alpha;
 };
 
-// What the per-pixel test of a staged surfel reads, 64 bytes. The two planes through pixel (x, y) are k = x Tw - Tu and
-// l = y Tw - Tv, and their cross product is linear in the pixel because Tw x Tw = 0:
-//   p(x, y) = k x l = x (Tv x Tw) + y (Tw x Tu) + Tu x Tv = p(c) - (c_x - x) (Tv x Tw) - (c_y - y) (Tw x Tu)
-// for any point c. The lane that stages a surfel forms the two cross products and p at the surfel's screen-space centre
-// (there through k and l, the well-conditioned way) once per (surfel, tile), and every pixel gets p with six fused
-// multiply-adds on its offset from the centre -- which the low-pass filter needs anyway -- instead of six for k, l and
-// six more for the product. Expanding around the centre keeps the linear terms as small as the footprint; around the
-// image origin they would be hundreds of times larger than p itself and their rounding would show in the image.
-struct __attribute__((aligned(16))) SplatRay {
-  float ax, ay, az;  // Tv x Tw
-  float bx, by, bz;  // Tw x Tu
-  float px, py, pz;  // p at the centre
-  float wx, wy, wz;  // Tw: depth along the ray = <s, (wx, wy)> + wz
-  float cx, cy;      // screen-space centre (low-pass filter)
-  float opacity;
-  float pad;
-};
-
-__device__ __forceinline__ SplatRay make_ray(const SplatHot& h) {
-#pragma clang fp contract(off)
-  const float* m = h.m;
-  SplatRay r;
-  r.ax = fmaf(m[4], m[8], -(m[5] * m[7])), r.ay = fmaf(m[5], m[6], -(m[3] * m[8])), r.az = fmaf(m[3], m[7], -(m[4] * m[6]));
-  r.bx = fmaf(m[7], m[2], -(m[8] * m[1])), r.by = fmaf(m[8], m[0], -(m[6] * m[2])), r.bz = fmaf(m[6], m[1], -(m[7] * m[0]));
-  const float kx = fmaf(h.cx, m[6], -m[0]), ky = fmaf(h.cx, m[7], -m[1]), kz = fmaf(h.cx, m[8], -m[2]);
-  const float lx = fmaf(h.cy, m[6], -m[3]), ly = fmaf(h.cy, m[7], -m[4]), lz = fmaf(h.cy, m[8], -m[5]);
-  r.px = fmaf(ky, lz, -(kz * ly)), r.py = fmaf(kz, lx, -(kx * lz)), r.pz = fmaf(kx, ly, -(ky * lx));
-  r.wx = m[6], r.wy = m[7], r.wz = m[8];
-  r.cx = h.cx, r.cy = h.cy, r.opacity = h.opacity, r.pad = 0.0f;
-  return r;
-}
-
-// A staged batch of SplatRays in LDS, stored as four planes of 16-byte quarters: the lanes that stage a batch write
-// consecutive 16-byte pieces (a 64-byte stride per lane would put every second lane on the same banks), and a
-// wavefront reads an entry's four quarters as four broadcasts.
-template <int kN>
-struct RayBatch {
-  float4 q[4][kN];
-  __device__ __forceinline__ void put(int i, const SplatRay& r) {
-    q[0][i] = make_float4(r.ax, r.ay, r.az, r.bx);
-    q[1][i] = make_float4(r.by, r.bz, r.px, r.py);
-    q[2][i] = make_float4(r.pz, r.wx, r.wy, r.wz);
-    q[3][i] = make_float4(r.cx, r.cy, r.opacity, 0.0f);
-  }
-  __device__ __forceinline__ SplatRay get(int j) const {
-    const float4 a = q[0][j], b = q[1][j], c = q[2][j], d = q[3][j];
-    SplatRay r;
-    r.ax = a.x, r.ay = a.y, r.az = a.z, r.bx = a.w, r.by = b.x, r.bz = b.y, r.px = b.z, r.py = b.w;
-    r.pz = c.x, r.wx = c.y, r.wy = c.z, r.wz = c.w, r.cx = d.x, r.cy = d.y, r.opacity = d.z, r.pad = 0.0f;
-    return r;
-  }
-};
-
 // Ray-splat intersection and alpha of one surfel at one pixel (gs_2d_redner.cu:122-155); false where the reference
 // would `continue`. No early exits: every lane runs the whole sequence and the rejections are combined at the end, so the
 // caller gets one predicate instead of nested divergent regions. Contraction is switched off and every fused
@@ -159,26 +106,33 @@ struct RayBatch {
 // depend on which copy evaluated a surfel). The exponent is formed in base 2 (-rho / 2 * log2(e) =
 // max(-log2(e) / 2 * rho3d, -log2(e) * |d|^2), one v_exp_f32). rho is a sum of squares, so the reference's `power > 0`
 // rejection can only differ from `true` for a NaN, which passes it there as here.
+// The intersection point is formed the reference's way, as the cross product of the two planes k = x Tw - Tu and
+// l = y Tw - Tv. (It is also linear in the pixel, p = p(c) - (c_x - x) Tv x Tw - (c_y - y) Tw x Tu, which takes six
+// instructions less per test once the two cross products are staged per surfel; for surfels seen edge-on, where p_z
+// nearly vanishes over the footprint, that form lands three times farther from the exact value than this one does --
+// measured on the 300k-surfel scene against the float64 evaluation -- so it is not used.)
 // `lanes`, if given, receives the mask of the lanes that pass, as the AND of the comparisons' own lane masks: a
 // wave-uniform "does any lane pass" then stays in scalar registers (the ballot of a combined predicate is rebuilt by
 // the compiler from a 0 / 1 register, two vector instructions and their latency on the entry's critical path).
 // Forward and backward of the standard path decide a pair with this function, so they agree on every pair.
-__device__ __forceinline__ bool intersect_ray(const SplatRay& r, float pxf, float pyf, float near_n, Hit& o,
-                                              unsigned long long* lanes = nullptr) {
-#pragma clang fp contract(off)  // written out: every inlined copy rounds alike
-  o.dx = r.cx - pxf, o.dy = r.cy - pyf;
-  const float p_x = fmaf(-r.ax, o.dx, fmaf(-r.bx, o.dy, r.px));
-  const float p_y = fmaf(-r.ay, o.dx, fmaf(-r.by, o.dy, r.py));
-  o.pz            = fmaf(-r.az, o.dx, fmaf(-r.bz, o.dy, r.pz));
+__device__ __forceinline__ bool intersect_flat(const SplatHot& h, float pxf, float pyf, float near_n, Hit& o,
+                                               unsigned long long* lanes = nullptr) {
+#pragma clang fp contract(off)
+  o.kx = fmaf(pxf, h.m[6], -h.m[0]), o.ky = fmaf(pxf, h.m[7], -h.m[1]), o.kz = fmaf(pxf, h.m[8], -h.m[2]);
+  o.lx = fmaf(pyf, h.m[6], -h.m[3]), o.ly = fmaf(pyf, h.m[7], -h.m[4]), o.lz = fmaf(pyf, h.m[8], -h.m[5]);
+  const float p_x = fmaf(o.ky, o.lz, -(o.kz * o.ly));
+  const float p_y = fmaf(o.kz, o.lx, -(o.kx * o.lz));
+  o.pz            = fmaf(o.kx, o.ly, -(o.ky * o.lx));
   const float rz = __builtin_amdgcn_rcpf(o.pz);
   o.sx = p_x * rz, o.sy = p_y * rz;
   o.rho3d = fmaf(o.sx, o.sx, o.sy * o.sy);
+  o.dx = h.cx - pxf, o.dy = h.cy - pyf;
   const float d2 = fmaf(o.dx, o.dx, o.dy * o.dy);
   o.rho2d = 2.0f * d2;
-  o.depth = fmaf(o.sx, r.wx, fmaf(o.sy, r.wy, r.wz));
+  o.depth = fmaf(o.sx, h.m[6], fmaf(o.sy, h.m[7], h.m[8]));
   const float power2 = fmaxf(o.rho3d * -0.72134752044448170368f, d2 * -1.44269504088896340736f);
   o.G     = __builtin_amdgcn_exp2f(power2);
-  o.alpha = fminf(0.99f, r.opacity * o.G);
+  o.alpha = fminf(0.99f, h.opacity * o.G);
   const bool c0 = o.pz != 0.0f, c1 = !(o.depth < near_n), c3 = !(o.alpha < (1.0f / 255.0f));
   if (lanes) *lanes = wave_ballot(c0) & wave_ballot(c1) & wave_ballot(c3);
   return c0 & c1 & c3;

@@ -64,8 +64,7 @@ blend_backward_kernel(
     const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii, float* __restrict__ slot_grads,
     const float4* __restrict__ records) {
   constexpr bool kQueue = kBwdQueue && !kFlow;
-  __shared__ SplatHot s_hot[kBwdBatch];  // read by the order-free pass (the planes k, l themselves) and the flow variant
-  __shared__ RayBatch<kBwdBatch> s_ray;  // read by the per-pixel test
+  __shared__ SplatHot s_hot[kBwdBatch];
   __shared__ SplatCold s_cold[kBwdBatch];
   // Each wavefront's sums over its 64 pixels, one row per staged surfel; the flush adds the four rows in wavefront
   // order, so a tile's sums do not depend on timing. +1: the odd stride keeps the flush free of bank conflicts.
@@ -197,7 +196,6 @@ blend_backward_kernel(
     const int n_here = min(kBwdBatch, n_todo - b * kBwdBatch);
     if (st >= 0 && st < n_here) {
       s_hot[st]  = next.hot;
-      s_ray.put(st, make_ray(next.hot));
       s_cold[st] = next.cold;
       s_mask[st] = (unsigned char) quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile, ordered);
       if (kFlow)
@@ -350,11 +348,11 @@ blend_backward_kernel(
         else q_head = 0, q_count = 0;
       };
       // ---- order-bound part of one entry, and the append of its blending pixels to the queue -----------------------------
-      auto queue_entry = [&](const SplatRay& hot, const SplatCold& cold, int j) {
+      auto queue_entry = [&](const SplatHot& hot, const SplatCold& cold, int j) {
         const int pos = n_todo - 1 - (b * kBwdBatch + j);  // 0-based position in the tile's list
         Hit h;
         unsigned long long pass;
-        const bool hit = intersect_ray(hot, pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
+        const bool hit = intersect_flat(hot, pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
         pass &= wave_ballot(pos < last_contrib);
         if (pass == 0ull) return;  // wave-uniform: nobody in this quadrant blends the surfel
         float w = 0.0f, dL_dalpha = 0.0f, dL_dz = 0.0f;
@@ -387,11 +385,11 @@ blend_backward_kernel(
           return j;
         };
         auto peek = [&]() { return todo ? (int) __builtin_ctzll(todo) : 0; };
-        SplatRay hot_a = s_ray.get(peek()), hot_b;
+        SplatHot hot_a = s_hot[peek()], hot_b;
         while (todo) {
           {
             const int j = pop();
-            hot_b       = s_ray.get(peek());
+            hot_b       = s_hot[peek()];
             const SplatCold cold = s_cold[j];
             __builtin_amdgcn_sched_barrier(0);
             queue_entry(hot_a, cold, j);
@@ -399,7 +397,7 @@ blend_backward_kernel(
           if (todo == 0ull) break;
           {
             const int j = pop();
-            hot_a       = s_ray.get(peek());
+            hot_a       = s_hot[peek()];
             const SplatCold cold = s_cold[j];
             __builtin_amdgcn_sched_barrier(0);
             queue_entry(hot_b, cold, j);
@@ -472,12 +470,9 @@ blend_backward_kernel(
       const int pos = n_todo - 1 - (b * kBwdBatch + j);  // 0-based position in the tile's list
       Hit h;
       unsigned long long pass;
-      const bool hit = intersect_ray(s_ray.get(j), pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
+      const bool hit = intersect_flat(hot, pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
       pass &= wave_ballot(pos < last_contrib);
       if (pass == 0ull) return;  // wave-uniform: nobody in this quadrant blends the surfel
-      // the two planes through the pixel themselves: the gradients of the transform's rows are taken through them
-      h.kx = pxf * hot.m[6] - hot.m[0], h.ky = pxf * hot.m[7] - hot.m[1], h.kz = pxf * hot.m[8] - hot.m[2];
-      h.lx = pyf * hot.m[6] - hot.m[3], h.ly = pyf * hot.m[7] - hot.m[4], h.lz = pyf * hot.m[8] - hot.m[5];
 
       float g[16], g2x, g2y;
       unsigned long long ray_lanes;

@@ -36,7 +36,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
     float* __restrict__ out_color, float* __restrict__ out_opacity, float* __restrict__ out_extras,
     float2* __restrict__ out_flow, int32_t* __restrict__ accum_max_count, float* __restrict__ accum_weights_p,
     int32_t* __restrict__ accum_weights_count) {
-  __shared__ RayBatch<kFwdBatch> s_ray;
+  __shared__ SplatHot s_hot[kFwdBatch];
   __shared__ SplatCold s_cold[kFwdBatch];
   __shared__ float s_t2[kFlow ? kFwdBatch * 9 : 1];
   __shared__ unsigned char s_mask[kFwdBatch];  // which 8x8 quadrants of the tile each staged surfel can reach
@@ -102,7 +102,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
     if (__syncthreads_count(live < 0.0f) == kBlendThreads) break;
     const int n_here = min(kFwdBatch, n_todo - b * kFwdBatch);
     if ((int) threadIdx.x < n_here) {
-      s_ray.put(threadIdx.x, make_ray(next.hot));
+      s_hot[threadIdx.x]  = next.hot;
       s_cold[threadIdx.x] = next.cold;
       s_mask[threadIdx.x] = (unsigned char) quadrant_mask(next.hot, tile_x * kTile, tile_y * kTile, ordered);
       if (kFlow)
@@ -129,11 +129,11 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
       // entry on the tile's critical path (the launch lasts as long as its longest tile). Hence: the NEXT entry's record
       // is requested before the current one is evaluated, into alternating registers; the intersection runs without
       // early exits and yields one predicate; the blend is one divergent region.
-      auto blend_entry = [&](const SplatRay& hot, const SplatCold& cold, int j) {
+      auto blend_entry = [&](const SplatHot& hot, const SplatCold& cold, int j) {
 #pragma clang fp contract(off)  // two copies of this body exist (alternating registers): both must round alike
         Hit h;
         unsigned long long pass;
-        const bool hit = intersect_ray(hot, pxf, pyf, near_n, h, &pass) && live > 0.0f;
+        const bool hit = intersect_flat(hot, pxf, pyf, near_n, h, &pass) && live > 0.0f;
         pass &= live_lanes;
         if (pass == 0ull) return;
         const float test_T = T * (1.0f - h.alpha);
@@ -184,12 +184,12 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
         return j;
       };
       auto peek = [&]() { return c * kWave + (todo ? __builtin_ctzll(todo) : 0); };
-      SplatRay hot_a = s_ray.get(peek()), hot_b;
+      SplatHot hot_a = s_hot[peek()], hot_b;
       while (todo) {
         if (live_lanes == 0ull) break;  // every pixel of this quadrant is saturated
         {
           const int j = pop();
-          hot_b       = s_ray.get(peek());
+          hot_b       = s_hot[peek()];
           const SplatCold cold = s_cold[j];  // read only if a pixel blends the surfel, but then without waiting
           __builtin_amdgcn_sched_barrier(0);
           blend_entry(hot_a, cold, j);
@@ -197,7 +197,7 @@ __global__ void __launch_bounds__(kBlendThreads) blend_forward_kernel(
         if (todo == 0ull || live_lanes == 0ull) break;
         {
           const int j = pop();
-          hot_a       = s_ray.get(peek());
+          hot_a       = s_hot[peek()];
           const SplatCold cold = s_cold[j];
           __builtin_amdgcn_sched_barrier(0);
           blend_entry(hot_b, cold, j);
