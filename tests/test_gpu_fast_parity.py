@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from util import abs_err, f64, npy, rel_err
+from util import abs_err, check_blend_forward, check_blend_gradients, f64, npy, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -21,15 +21,19 @@ CASES = {
     "big_surfels_96x80": (300, 96, 80, 10.0),  # rectangles of more than 32 tiles: wave-cooperative emission
     "dense_6k_96": (6_000, 96, 96, 12.0),  # tile lists longer than one 256-entry batch, many 32-entry buckets
     "tiny_3_surfels": (3, 40, 24, 1.0),
+    "c2_300k_800": (300_000, 800, 800, 1.0),  # the benchmark's scene at full size
 }
 
 
 def _make(name):
     from fast_sp_gs_amd import scenes
     P, W, H, scale_mul = CASES[name]
-    scene, _ = scenes.config0(P=P, size=max(W, H), seed=0)
-    scene.scales = scene.scales * scale_mul
-    cam = scenes.pinhole(W, H, 50.0, torch.tensor([0.3, -0.2, 4.0]))  # off-axis: x/y translation in the view matrix
+    if name.startswith("c2_"):
+        scene, cam = scenes.config2(P=P, size=W, seed=0)
+    else:
+        scene, _ = scenes.config0(P=P, size=max(W, H), seed=0)
+        scene.scales = scene.scales * scale_mul
+        cam = scenes.pinhole(W, H, 50.0, torch.tensor([0.3, -0.2, 4.0]))  # off-axis: x/y translation in the view matrix
     g = torch.Generator().manual_seed(7)
     gi = torch.randn(3, H, W, generator=g)
     ge = torch.randn(8, H, W, generator=g)
@@ -78,17 +82,14 @@ def test_fast_path_stage_by_stage(name, per_splat, device, oracle_mod):
     ref_f = O.fast_render_forward(W, H, cam.near, cam.far, False, d64['means2D'], d64['colors'], d64['normal_opacity'],
                                   d64['trans_mat'], d64['inverse_m'], g['point_list'], g['ranges'], offset)
     oc, oo, oe, nc = ref_f[:4]
-    flip = (g['n_contrib'] != nc).any(0)
-    keep = ~flip
-    allowed = max(2, int(1e-5 * H * W))
-    print(f"[fast {name}] image abs err {abs_err(g['image'][:, keep], oc[:, keep]):.3e}, opacity "
-          f"{abs_err(g['opacity'][keep], oo[keep]):.3e}, threshold-flip pixels {int(flip.sum())} (allowed {allowed})",
-          flush=True)
-    assert flip.sum() <= allowed
-    assert abs_err(g['image'][:, keep], oc[:, keep]) < 1e-4 and abs_err(g['opacity'][keep], oo[keep]) < 1e-4
-    for ch in range(8):
-        bad = np.abs(g['extras'][ch].astype(np.float64) - oe[ch]) > 1e-4 + 1e-3 * np.abs(oe[ch])
-        assert not (bad & keep).any(), f"extras channel {ch}: {int((bad & keep).sum())} pixels out of tolerance"
+    def forward32():
+        f32 = lambda k: g[k].astype(np.float32)
+        r = O.fast_render_forward(W, H, cam.near, cam.far, False, f32('means2D'), f32('colors'), f32('normal_opacity'),
+                                  f32('trans_mat'), f32('inverse_m'), g['point_list'], g['ranges'], offset)
+        return r[0], r[1], r[2], r[3]
+
+    flip = check_blend_forward(f"fast {name}", (g['image'], g['opacity'], g['extras'][:8], g['n_contrib']),
+                               (oc, oo, oe[:8], nc), forward32, max(2, int(1e-5 * H * W)))
 
     if per_splat:
         # snapshots: compared where the oracle wrote them (a written transmittance is always >= 1e-4 > 0)
@@ -111,11 +112,18 @@ def test_fast_path_stage_by_stage(name, per_splat, device, oracle_mod):
         cam.near, cam.far, int(per_splat), d64['means2D'], d64['normal_opacity'], d64['colors'], d64['trans_mat'],
         d64['inverse_m'], d64['opacity'], d64['extras'], f64(npy(gi)), f64(npy(go)), f64(npy(ge)), g['ranges'],
         g['point_list'], g['n_contrib'])
-    errs = dict(colors=rel_err(g['g_colors'], gc), trans=rel_err(g['g_trans'], gt), inv=rel_err(g['g_inv'], ginv),
-                normal_opacity=rel_err(g['g_normal_opacity'], gn), means2D=rel_err(g['g_means2D_blend'], gm))
-    print(f"[fast {name}] blend backward rel errs {errs}", flush=True)
-    for k, v in errs.items():
-        assert v < 1e-3, k
+    def backward32():
+        f32 = lambda a: np.asarray(a, np.float32)
+        r = O.fast_render_backward(
+            cam.near, cam.far, int(per_splat), f32(d64['means2D']), f32(d64['normal_opacity']), f32(d64['colors']),
+            f32(d64['trans_mat']), f32(d64['inverse_m']), f32(d64['opacity']), f32(d64['extras']), npy(gi), npy(go),
+            npy(ge), g['ranges'], g['point_list'], g['n_contrib'])
+        return dict(colors=r[0], means2D=r[1], trans=r[2], inv=r[3], normal_opacity=r[4])
+
+    check_blend_gradients(f"fast {name} blend backward",
+                          dict(colors=g['g_colors'], trans=g['g_trans'], inv=g['g_inv'],
+                               normal_opacity=g['g_normal_opacity'], means2D=g['g_means2D_blend']),
+                          dict(colors=gc, trans=gt, inv=ginv, normal_opacity=gn, means2D=gm), backward32)
     assert np.abs(g['g_trans'][:, :2]).max() == 0  # only the depth row of the transform receives gradient here
 
     # --- preprocess backward on the GPU's own blend gradients

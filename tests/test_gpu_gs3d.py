@@ -87,7 +87,8 @@ def _binned(P, W, H, seed, device):
     return m2, col, co, ranges, pl
 
 
-@pytest.mark.parametrize("P,W,H,E", [(4000, 160, 96, 0), (4000, 131, 77, 2), (20000, 128, 128, 4), (3, 40, 40, 1)])
+@pytest.mark.parametrize("P,W,H,E", [(4000, 160, 96, 0), (4000, 131, 77, 2), (20000, 128, 128, 4), (3, 40, 40, 1),
+                                     (300_000, 800, 800, 0)])
 def test_gs3d_rasterize(P, W, H, E, device):
     from fast_sp_gs_amd._C import get_C_function
     m2, col, co, ranges, pl = _binned(P, W, H, 31 + E, device)
