@@ -1,4 +1,5 @@
-"""Full-size checks of the render path through size-independent properties (the oracle takes minutes at these sizes):
+"""Full-size checks of the render path through size-independent properties, beside the stage-by-stage comparisons with
+the oracle that test_gpu_render_parity.py and test_gpu_fast_parity.py also run at 300 000 / 3 000 000 surfels:
   * the per-quadrant culling of the blend kernels is exact: with it switched off (every staged surfel evaluated at every
     pixel, as the reference does) the forward outputs are identical bit for bit and the gradients agree to the rounding
     of the reordered atomic sums;

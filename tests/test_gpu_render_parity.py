@@ -27,6 +27,8 @@ CASES = {
     "tiny_3_surfels": (3, 40, 24),
     # the benchmark's own configuration, full size (the oracle takes a few seconds per stage on the host's cores)
     "c2_300k_800": (300_000, 800, 800),
+    # one view of the large-scene configuration (3M surfels, 5M instances)
+    "c4_3m_1352x1014": (3_000_000, 1352, 1014),
 }
 
 
@@ -35,6 +37,12 @@ def _make(name, device):
     P, W, H = CASES[name]
     if name.startswith("c2_"):
         return scenes.config2(P=P, size=W, seed=0)
+    if name.startswith("c4_"):
+        scene, cams = scenes.config4(P=P, W=W, H=H, seed=0)
+        g = torch.Generator().manual_seed(5)
+        scene.extra['grad_extras'] = torch.cat([torch.randn(5, H, W, generator=g), torch.zeros(4, H, W)])
+        scene.extra['grad_opacity'] = torch.randn(H, W, generator=g)
+        return scene, cams[1]
     scene, cam = scenes.config0(P=P, size=max(W, H), seed=0)
     if (W, H) != (cam.W, cam.H):
         cam = scenes.pinhole(W, H, 50.0, torch.tensor([0., 0., 4.]))
