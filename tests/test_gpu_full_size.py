@@ -7,8 +7,9 @@ the oracle that test_gpu_render_parity.py and test_gpu_fast_parity.py also run a
   * the blend weights accumulated per surfel sum to the opacity image;
   * the backward is linear in the upstream gradients, and its two ways of summing a surfel's gradient over tiles
     (per-instance records summed in order / device-scope atomics) agree;
-  * K-NN at 3M x 2048, k = 8: distances ascending, equal to the distance recomputed from the returned index, and no
-    closer control point exists for a sample of queries (brute force with torch).
+  * K-NN at 3M x 2048, k = 8: distances ascending, equal to the distance recomputed from the returned index, no
+    closer control point exists for a sample of queries (brute force with torch), and indices and distances bit for
+    bit against the oracle's all-pairs search.
 Sizes: 300 000 surfels at 800x800, 3 000 000 surfels at 1352x1014 (each of the four views), 400 000 surfels at
 3840x2160.
 The fast path and the 3D-Gaussian path get the same kind of checks at 300 000 / 800x800 (culling, ordered against atomic
@@ -134,6 +135,11 @@ def test_knn_3m_by_2048_k8(device):
     full = torch.cdist(x[sample], y) ** 2
     kth = full.topk(K, dim=1, largest=False).values
     assert float((kth - d2[sample]).abs().max()) < 1e-4 * float(kth.max())
+    # all 3M queries against the oracle's all-pairs search (6.1e9 distances): indices and distances bit for bit
+    import oracle as O
+    rd, ri = np.zeros((N, K), np.float32), np.zeros((N, K), np.int64)
+    O.call("knn_topk_f32", N, M, 3, K, x.cpu().numpy(), y.cpu().numpy(), rd, ri)
+    assert np.array_equal(idx.cpu().numpy(), ri) and np.array_equal(d2.cpu().numpy(), rd)
 
 
 @pytest.mark.parametrize("per_splat", [False, True])

@@ -764,6 +764,62 @@ def test_full_size_properties(device):
     assert float((g_cam.double() + g_pos.double().sum(0)).abs().max()) < 1e-3 * max(1.0, float(g_pos.abs().sum(0).max()))
 
 
+def test_full_size_against_the_oracle(device, oracle_mod):
+    """The stand-alone operators at the benchmark's sizes against the oracle itself: SH encoder forward / backward at
+    1M directions, K-NN at 200 000 x 512 (k = 4) bit for bit, its distances' backward, the LBS blend forward against the
+    float64 restatement, and the masked Adam at 300 000 x 58 floats bit for bit."""
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd._C import get_C_function as f
+    import oracle.lbs as OL
+    O = oracle_mod
+    c = scenes.config1(n_dirs=1_000_000, n_points=200_000, n_ctrl=512)
+    dirs = c['dirs']
+    B = dirs.shape[0]
+    g = torch.Generator().manual_seed(21)
+    enc, g_dirs = torch.empty(B, 16, device=device), torch.empty(B, 3, device=device)
+    up = torch.randn(B, 16, generator=g)
+    f('sh_encode_forward')(dirs.to(device), enc, B, 3, 3)
+    f('sh_encode_backward')(up.to(device), dirs.to(device), B, 3, 3, g_dirs)
+    ref, gref = np.zeros((B, 16), np.float32), np.zeros((B, 3), np.float32)
+    O.call("sh_encode_forward_f32", B, 3, 3, npy(dirs), ref)
+    O.call("sh_encode_backward_f32", B, 3, 3, npy(up), npy(dirs), gref)
+    print(f"[full config 1] sh_encode 1M: forward abs err {abs_err(npy(enc), ref):.2e}, backward rel err "
+          f"{rel_err(npy(g_dirs), gref):.2e}", flush=True)
+    assert abs_err(npy(enc), ref) < 6e-6 and rel_err(npy(g_dirs), gref) < 1e-5
+
+    pts, ctrl = c['points'], c['ctrl']
+    N, M, K = pts.shape[0], ctrl.shape[0], 4
+    d2, idx = f('knn_topk')(pts.to(device), ctrl.to(device), K)
+    rd, ri = np.zeros((N, K), np.float32), np.zeros((N, K), np.int64)
+    O.call("knn_topk_f32", N, M, 3, K, npy(pts), npy(ctrl), rd, ri)
+    assert np.array_equal(npy(idx), ri) and np.array_equal(npy(d2), rd)
+    gd = torch.randn(N, K, generator=g)
+    gx, gy = f('knn_topk_backward')(pts.to(device), ctrl.to(device), idx, gd.to(device))
+    rx, ry = np.zeros((N, 3), np.float32), np.zeros((M, 3), np.float32)
+    O.call("knn_topk_backward_f32", N, M, 3, K, npy(pts), npy(ctrl), ri, npy(gd), rx, ry)
+    assert rel_err(npy(gx), rx) < 1e-5 and rel_err(npy(gy), ry) < 2e-4
+    out = f('lbs_blend')(pts.to(device), ctrl.to(device), c['sp_t'].to(device), c['sp_r'].to(device),
+                         c['sp_s'].to(device), d2, idx, 0.01, 'LBS', c['sp_r'].to(device), 'dist')
+    want = OL.lbs_blend(pts.double(), ctrl.double(), c['sp_t'].double(), c['sp_r'].double(), c['sp_s'].double(),
+                        c['sp_r'].double(), d2.cpu().double(), idx.cpu(), 'dist', 0.01, 'LBS')
+    for a, b, name in zip(out[:3], want[:3], ('d_xyz', 'd_rot', 'd_scale')):
+        assert rel_err(npy(a), b.numpy()) < 2e-5, name
+    print(f"[full config 1] knn 200000 x 512 bit-exact, lbs_blend within 2e-5", flush=True)
+
+    P, widths = 300_000, (3, 3, 45, 1, 2, 4)
+    mask = torch.rand(P, generator=g) < 0.9
+    params = [torch.randn(P, w, generator=g) for w in widths]
+    grads = [torch.randn(P, w, generator=g) for w in widths]
+    dev = [[t.to(device) for t in group] for group in (params, grads)]
+    m1, m2 = [torch.zeros_like(t) for t in dev[0]], [torch.zeros_like(t) for t in dev[0]]
+    f('AdamMasksedUpdatedMulti')(dev[0], dev[1], m1, m2, mask.to(device), [1.6e-4] * 6, 0.9, 0.999, [1e-15] * 6, P)
+    for k, w in enumerate(widths):
+        rp, rm, rv = npy(params[k]).copy(), np.zeros((P, w), np.float32), np.zeros((P, w), np.float32)
+        O.call("adam_masked_update_f32", P, w, npy(mask.to(torch.uint8)), 1.6e-4, 0.9, 0.999, 1e-15, rp, npy(grads[k]),
+               rm, rv)
+        assert np.array_equal(npy(dev[0][k]), rp) and np.array_equal(npy(m1[k]), rm) and np.array_equal(npy(m2[k]), rv)
+
+
 def test_deform_mlp_mfma(device, oracle_mod):
     """Fused bf16 MFMA MLP against (a) the fp32 oracle on bf16-rounded weights and inputs -- isolates the kernel's own
     arithmetic up to the per-layer bf16 re-rounding of activations, tolerance 1e-2 relative -- and (b) the plain fp32 network, tolerance 2e-2 relative (bf16 rounding of
