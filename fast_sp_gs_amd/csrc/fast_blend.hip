@@ -19,6 +19,7 @@
 // conservative bound, gradients reduced over the wavefront in registers before one LDS atomic per component.
 #include "blend.hpp"
 #include "ordered_sums.hpp"
+#include "pair_queue.hpp"
 
 namespace fsgs {
 namespace {
@@ -95,9 +96,9 @@ __device__ __forceinline__ bool fast_intersect_flat(const FastHot& h, float pxf,
   return c0 & c1 & c2 & c3;
 }
 
-// Sums 8 per-lane values over the 64 lanes at once: three merge steps inside aligned groups of 8 lanes, one rotate by 8
-// inside the row of 16, two cross-row exchanges. On return every lane holds the wave total of v[lane & 7].
-__device__ __forceinline__ float wave_sum8_transposed(const float (&v)[8]) {
+// Sums 8 per-lane values over each 16-lane row at once: three merge steps inside aligned groups of 8 lanes, one rotate
+// by 8 inside the row. On return lane l of every row holds that row's total of v[l & 7].
+__device__ __forceinline__ float row_sum8_transposed(const float (&v)[8]) {
 #pragma clang fp contract(off)  // an input that is a product must not be formed a second time inside a fused add
   const int lane = __lane_id();
   const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
@@ -118,8 +119,10 @@ __device__ __forceinline__ float wave_sum8_transposed(const float (&v)[8]) {
   const float b = x[0] + dpp_shift_zero<0x104, 0xf, 0xf>(x[0]);  // row_shl:4
   float z = b2 ? a : b;
   z += dpp_shift_zero<0x128, 0xf, 0xf>(z);  // row_ror:8
-  return cross_row_sum(z);
+  return z;
 }
+// The same over the 64 lanes: every lane holds the wave total of v[lane & 7].
+__device__ __forceinline__ float wave_sum8_transposed(const float (&v)[8]) { return cross_row_sum(row_sum8_transposed(v)); }
 
 template <bool kAux, bool kSnap, bool kAccum, bool kFlow>
 __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
@@ -340,7 +343,11 @@ struct FastScatter {
 
 // kSlots: the per-surfel sums go through per-instance records (ordered_sums.hpp) instead of device-scope atomics.
 template <bool kAux, bool kPerSplat, bool kFlow, bool kSlots>
-__global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
+// Four blocks per compute unit where the per-surfel sums go through records (the flush of the other form keeps more
+// values live and would spill in the loop over the entries): the launch lasts little longer than the block with the
+// longest list, and the more wavefronts share a SIMD with that block's, the sooner the other blocks are out of the way.
+__global__ void __launch_bounds__(kBlendThreads)
+    __attribute__((amdgpu_waves_per_eu(kSlots && !kFlow ? 4 : 1, kSlots && !kFlow ? 4 : 8))) fast_blend_backward_kernel(
     int ordered, const int* __restrict__ tile_order, int W, int H, float near_n, float far_n, const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list,
     const int32_t* __restrict__ n_contrib, const float2* __restrict__ means2D,
     const float4* __restrict__ normal_opacity, const float* __restrict__ colors, const float* __restrict__ trans_mat,
@@ -352,6 +359,11 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
     float* __restrict__ g_trans, float* __restrict__ g_inv, const int64_t* __restrict__ point_offsets,
     const int32_t* __restrict__ radii, float* __restrict__ slot_records) {
   constexpr int kB = 64;  // surfels staged per round
+  static_assert(kB == kWave, "one ballot covers a round, and a queued pair names its entry in a byte");
+  // Two passes (pair_queue.hpp): the order-bound recurrence queues the blending pairs, the components are formed and
+  // summed 64 pairs at a time. Not with a second set of transforms, whose per-pair terms would double the item.
+  constexpr bool kQueue = !kFlow;
+  __shared__ float4 s_queue[kQueue ? 4 : 1][kQueue ? kQueueItems : 1];
   __shared__ FastHot s_hot[kB];
   __shared__ SplatCold s_cold[kB];
   __shared__ float s_t2[kFlow ? kB * 9 : 1];
@@ -370,6 +382,8 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
   const size_t pix  = (size_t) W * py + px;
   const float pxf = (float) px, pyf = (float) py;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float qx0 = pxf - (float) (lane & 7), qy0 = pyf - (float) (lane >> 3);  // first pixel of the wavefront's quadrant
+  PairQueue q;
 
   const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
   const int last_contrib   = inside ? n_contrib[pix] : 0;
@@ -464,69 +478,147 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
     const int nxt = (b + 1) * kB + (int) threadIdx.x;
     if ((int) threadIdx.x < kB && nxt < n_todo) gather(n_todo - 1 - nxt);
 
-    for (int chunk = 0; chunk < kB / kWave; ++chunk) {
-      const int jj = chunk * kWave + lane;
-      unsigned long long todo = __ballot(jj < n_here && ((s_mask[jj] >> wave) & 1u) &&
-                                         (n_todo - 1 - (b * kB + jj)) < wave_max_contrib);
-      while (todo) {
-        const int j = chunk * kWave + __builtin_ctzll(todo);
-        todo &= todo - 1;
+    // The part of a pair that is bound to the list's order: advances the pixel's back-to-front state and leaves the
+    // pair's weight, dL/dalpha (times the transmittance in front of the pair), dL/d(depth along the ray) and, with a
+    // second set of transforms, dL/d(intersection) through it. Only entered by lanes whose pixel blends the entry.
+    auto advance_pixel = [&](const SplatCold& cold, int j, int pos, const FastHit& h, float& w, float& dL_dalpha,
+                             float& dL_dz, float& fsx, float& fsy) {
+      T = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
+      w = h.alpha * T;
+      // one back-to-front recurrence for every channel that enters the image linearly: c = <upstream gradient,
+      // channel values of this surfel> replaces the reference's per-channel accumulators
+      float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
+      if (kAux) {
+        const float rd     = __builtin_amdgcn_rcpf(h.depth);
+        const float m_d    = far_scale - far_near * rd;
+        const float dmd_dd = far_near * rd * rd;
+        if (pos == median_contrib - 1) dL_dz += dL_dmedian;
+        if (!kPerSplat) {
+          // dL/dweight of the distortion enters dL/dalpha as a linear channel does (its value minus what the pairs
+          // behind it accumulated, with the same weights): it rides on the shared recurrence
+          c_lin += reg_D2 + m_d * (m_d * reg_A - reg_2D);
+          dL_dz += w * (m_d * reg_2A - reg_2D) * dmd_dd;
+        } else {
+          c_lin += m_d * dL_dM1 + (m_d * m_d) * dL_dM2;
+          dL_dz += dmd_dd * (2.0f * m_d * w * dL_dM2);
+        }
+        c_lin += h.depth * dL_ddepth + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
+        dL_dz += w * dL_ddepth;
+      }
+      if (kAux || kPerSplat) c_lin += dL_daccum;
+      if (kFlow) {
+        const float* Q = &s_t2[j * 9];
+        const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
+        const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
+        float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
+        w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
+        const float rw = 1.0f / w2;
+        c_lin += (u2 * rw - pxf) * dLf0 + (v2 * rw - pyf) * dLf1;
+        const float gu = w * rw * dLf0, gv = w * rw * dLf1;
+        const float gw = -w * rw * rw * (u2 * dLf0 + v2 * dLf1);
+        fsx = Q[0] * gu + Q[3] * gv + Q[6] * gw;
+        fsy = Q[1] * gu + Q[4] * gv + Q[7] * gw;
+      }
+      dL_dalpha = c_lin - acc_lin;
+      acc_lin   = fmaf(1.0f - h.alpha, acc_lin, h.alpha * c_lin);
+      dL_dalpha *= T;
+    };
+
+    // ---- order-free part: 64 queued pairs at a time, four 16-lane rows, every row one entry ---------------------------
+    // A lane rebuilds the intersection through its pair's pixel from the staged adjugate and forms the 16 + 5 components
+    // as products of the three queued numbers with quantities that are finite in every lane (padding items carry zeros
+    // and no flags, and the reciprocal of p_z is only taken under the pair's flags).
+    auto drain = [&](int n_valid) {
+      const unsigned jrows = queue_front_rows(q);
+      const int j = (int) ((jrows >> ((lane >> 4) * 8)) & 255u);
+      const float4 it = s_queue[wave][q.head + lane];
+      const FastHot hot = s_hot[j];
+      float* const acc  = &s_part[wave][j][lane & 15];
+      float* const acc2 = &s_part[wave][j][16 + (lane & 7)];  // used by lanes 0-4 of a row
+      const float before = *acc;
+      const bool second = (lane & 15) < 5;
+      const float before2 = (kAux && second) ? *acc2 : 0.0f;
+      const int bits = __float_as_int(it.w);
+      const int qp = bits & 63;
+      const bool blends = (bits & kItemHit) != 0, by_ray = (bits & kItemRay) != 0;
+      // the upstream gradients of the pair's pixel sit in the registers of the lane that owns it
+      auto from_owner = [&](float v) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(qp << 2, __builtin_bit_cast(int, v)));
+      };
+      const float up_x = from_owner(dLp0), up_y = from_owner(dLp1), up_z = from_owner(dLp2);
+      const float fx = qx0 + (float) (qp & 7), fy = qy0 + (float) (qp >> 3);
+      const float w = it.x, GdA = it.y, dL_dz = it.z;
+      const float p0 = hot.a[0] * fx + hot.a[1] * fy + hot.a[2];
+      const float p1 = hot.a[3] * fx + hot.a[4] * fy + hot.a[5];
+      const float pz = hot.a[6] * fx + hot.a[7] * fy + hot.a[8];
+      const float rz_s = blends ? __builtin_amdgcn_rcpf(pz) : 0.0f;  // s is used by both cases of a blending pair
+      const float rz_p = by_ray ? rz_s : 0.0f;                        // d/dp only by the intersection case
+      const float sx = p0 * rz_s, sy = p1 * rz_s;
+      const float oG = hot.opacity * GdA;
+      float dsx = -(oG * sx), dsy = -(oG * sy);
+      if (kAux) dsx += dL_dz * hot.tw0, dsy += dL_dz * hot.tw1;
+      const float s_ds = dsx * sx + dsy * sy;
+      const float da = dsx * rz_p, db = dsy * rz_p, dc = -(s_ds * rz_p);
+      float g[16];
+      g[0] = w * up_x, g[1] = w * up_y, g[2] = w * up_z;
+      g[3] = da * fx, g[4] = da * fy, g[5] = da;
+      g[6] = db * fx, g[7] = db * fy, g[8] = db;
+      g[9] = dc * fx, g[10] = dc * fy, g[11] = dc;
+      if (kAux) {
+        g[12] = w * from_owner(dLn0), g[13] = w * from_owner(dLn1), g[14] = w * from_owner(dLn2);
+      } else {
+        g[12] = g[13] = g[14] = 0.0f;
+      }
+      g[15] = GdA;
+      queue_accumulate(acc, before, row_sum16_transposed(g), jrows, n_valid, true);
+      const bool filtered = blends && !by_ray;
+      const float to_centre = filtered ? -2.0f * oG : 0.0f;
+      if (kAux) {
+        float g8[8];
+        g8[0] = dL_dz * sx, g8[1] = dL_dz * sy, g8[2] = dL_dz;
+        g8[3] = to_centre * (hot.cx - fx), g8[4] = to_centre * (hot.cy - fy);
+        g8[5] = g8[6] = g8[7] = 0.0f;
+        queue_accumulate(acc2, before2, row_sum8_transposed(g8), jrows, n_valid, second);
+      } else if (wave_ballot(filtered) != 0ull) {  // some pair met its surfel by the projected centre
+        float cx = to_centre * (hot.cx - fx), cy = to_centre * (hot.cy - fy);  // totals of a row end up in its lane 15
+        cx += dpp_shift_zero<0x111, 0xf, 0xf>(cx), cy += dpp_shift_zero<0x111, 0xf, 0xf>(cy);
+        cx += dpp_shift_zero<0x112, 0xf, 0xf>(cx), cy += dpp_shift_zero<0x112, 0xf, 0xf>(cy);
+        cx += dpp_shift_zero<0x114, 0xf, 0xf>(cx), cy += dpp_shift_zero<0x114, 0xf, 0xf>(cy);
+        cx += dpp_shift_zero<0x118, 0xf, 0xf>(cx), cy += dpp_shift_zero<0x118, 0xf, 0xf>(cy);
+        if ((lane >> 4) < ((n_valid + 15) >> 4) && (lane & 15) == 15)
+          atomicAdd(&s_part[wave][j][19], cx), atomicAdd(&s_part[wave][j][20], cy);
+      }
+      queue_pop(q, n_valid);
+    };
+
+    // one entry of the wavefront's work list; its records were requested from LDS while the entry before it ran
+    auto blend_entry = [&](const FastHot& hot, const SplatCold& cold, int j) {
         const int pos = n_todo - 1 - (b * kB + j);
         FastHit h;
         unsigned long long pass;
-        const bool hit = fast_intersect_flat(s_hot[j], pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
-        if ((pass & wave_ballot(pos < last_contrib)) == 0ull) continue;
+        const bool hit = fast_intersect_flat(hot, pxf, pyf, near_n, h, &pass) && (pos < last_contrib);
+        pass &= wave_ballot(pos < last_contrib);
+        if (pass == 0ull) return;
+        float w = 0.0f, dL_dalpha = 0.0f, dL_dz = 0.0f, fsx = 0.0f, fsy = 0.0f;
+        if (kQueue) {
+          if (hit) {
+            advance_pixel(cold, j, pos, h, w, dL_dalpha, dL_dz, fsx, fsy);
+            dL_dalpha *= h.G;  // only G * dL/dalpha is ever used
+          }
+          const int flags = h.rho3d <= h.rho2d ? (kItemHit | kItemRay) : kItemHit;
+          if (queue_append(s_queue[wave], q, j, hit, pass, w, dL_dalpha, dL_dz, flags)) drain(kWave);
+          return;
+        }
 
-        // The part under `hit` advances the pixel's back-to-front state and leaves a few factors (zero in a lane whose
-        // pixel does not blend the entry); the components are products of those factors with quantities that are
-        // finite in every lane, formed by all lanes alike: no component needs a zero of its own, and the
-        // projected-centre case is the intersection case with a zero in place of 1 / p_z.
+        // One pass per entry (second set of transforms: its per-pair terms would double the queue's item). The part
+        // under `hit` leaves a few factors (zero in a lane whose pixel does not blend the entry); the components are
+        // products of those factors with quantities that are finite in every lane, formed by all lanes alike: no
+        // component needs a zero of its own, and the projected-centre case is the intersection case with a zero in
+        // place of 1 / p_z.
         float g[16], g8[8];
-        float w = 0.0f, dL_dalpha = 0.0f, dL_dz = 0.0f, dsx = 0.0f, dsy = 0.0f, s_ds = 0.0f, z_sx = 0.0f, z_sy = 0.0f;
-        const FastHot& hot = s_hot[j];
+        float dsx = 0.0f, dsy = 0.0f, s_ds = 0.0f, z_sx = 0.0f, z_sy = 0.0f;
         if (hit) {
-          const SplatCold cold = s_cold[j];
-          T = T * __builtin_amdgcn_rcpf(1.0f - h.alpha);
-          w = h.alpha * T;
-          // one back-to-front recurrence for every channel that enters the image linearly: c = <upstream gradient,
-          // channel values of this surfel> replaces the reference's per-channel accumulators
-          float c_lin = cold.r * dLp0 + cold.g * dLp1 + cold.b * dLp2;
-          if (kAux) {
-            const float rd     = __builtin_amdgcn_rcpf(h.depth);
-            const float m_d    = far_scale - far_near * rd;
-            const float dmd_dd = far_near * rd * rd;
-            if (pos == median_contrib - 1) dL_dz += dL_dmedian;
-            if (!kPerSplat) {
-              // dL/dweight of the distortion enters dL/dalpha as a linear channel does (its value minus what the pairs
-              // behind it accumulated, with the same weights): it rides on the shared recurrence
-              c_lin += reg_D2 + m_d * (m_d * reg_A - reg_2D);
-              dL_dz += w * (m_d * reg_2A - reg_2D) * dmd_dd;
-            } else {
-              c_lin += m_d * dL_dM1 + (m_d * m_d) * dL_dM2;
-              dL_dz += dmd_dd * (2.0f * m_d * w * dL_dM2);
-            }
-            c_lin += h.depth * dL_ddepth + cold.nx * dLn0 + cold.ny * dLn1 + cold.nz * dLn2;
-            dL_dz += w * dL_ddepth;
-          }
-          if (kAux || kPerSplat) c_lin += dL_daccum;
-          float fsx = 0.0f, fsy = 0.0f;  // dL/d(intersection) through the second transform
-          if (kFlow) {
-            const float* Q = &s_t2[j * 9];
-            const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
-            const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
-            float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
-            w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
-            const float rw = 1.0f / w2;
-            c_lin += (u2 * rw - pxf) * dLf0 + (v2 * rw - pyf) * dLf1;
-            const float gu = w * rw * dLf0, gv = w * rw * dLf1;
-            const float gw = -w * rw * rw * (u2 * dLf0 + v2 * dLf1);
-            fsx = Q[0] * gu + Q[3] * gv + Q[6] * gw;
-            fsy = Q[1] * gu + Q[4] * gv + Q[7] * gw;
-          }
-          dL_dalpha += c_lin - acc_lin;
-          acc_lin = fmaf(1.0f - h.alpha, acc_lin, h.alpha * c_lin);
-          dL_dalpha *= T;
-
+          advance_pixel(cold, j, pos, h, w, dL_dalpha, dL_dz, fsx, fsy);
           // d/ds of the intersection case (times 1 / p_z below); s is not finite in a lane whose p_z is 0, and such a
           // lane never blends: every use of s sits on this side
           const float dL_dG = hot.opacity * dL_dalpha;
@@ -559,7 +651,35 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_backward_kernel(
           const float sx = wave_sum_to_lane63(g8[3]), sy = wave_sum_to_lane63(g8[4]);
           if (lane == 63) s_part[wave][j][19] = sx, s_part[wave][j][20] = sy;
         }
+    };
+    unsigned long long todo = __ballot(lane < n_here && ((s_mask[lane] >> wave) & 1u) &&
+                                       (n_todo - 1 - (b * kB + lane)) < wave_max_contrib);
+    if (todo != 0ull) {
+      auto pop = [&]() {
+        const int j = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        return j;
+      };
+      auto peek = [&]() { return todo ? (int) __builtin_ctzll(todo) : 0; };
+      FastHot hot_a = s_hot[peek()], hot_b;
+      while (todo) {
+        {
+          const int j = pop();
+          hot_b       = s_hot[peek()];
+          const SplatCold cold = s_cold[j];
+          __builtin_amdgcn_sched_barrier(0);
+          blend_entry(hot_a, cold, j);
+        }
+        if (todo == 0ull) break;
+        {
+          const int j = pop();
+          hot_a       = s_hot[peek()];
+          const SplatCold cold = s_cold[j];
+          __builtin_amdgcn_sched_barrier(0);
+          blend_entry(hot_b, cold, j);
+        }
       }
+      if (kQueue && q.count > 0) drain(q.count);  // the staged records are replaced after the next barrier
     }
     __syncthreads();
     if ((int) threadIdx.x < n_here) {
