@@ -23,6 +23,7 @@
 #include <algorithm>
 
 #include "blend.hpp"
+#include "pair_queue.hpp"
 
 namespace fsgs {
 namespace {
@@ -39,17 +40,11 @@ constexpr int kGradSlots = 18;
 #endif
 constexpr int kBwdBatch = FSGS_BWD_BATCH;  // surfels staged per round
 static_assert(kBwdBatch == kWave, "one wavefront stages a batch, another flushes it, and a queued pair names its entry in 6 bits");
-// Queue of blended (pixel, entry) pairs per wavefront, a ring of 16-byte items in two halves of 64. A pass over one
-// entry appends at most 64 items (its blending pixels padded to a multiple of 16) and a full half is drained as soon
-// as there is one, so the ring never holds more than 48 + 64 items and a drain always starts at a half.
+// the two-pass form (queue of blended pairs per wavefront, pair_queue.hpp) can be switched off at build time
 #ifndef FSGS_BWD_QUEUE
 #define FSGS_BWD_QUEUE 1
 #endif
 constexpr bool kBwdQueue = FSGS_BWD_QUEUE != 0;
-constexpr int kQueueItems = 128;
-// item.w: pixel of the quadrant (6 bits) | blends (bit 12) | met by the ray-splat intersection rather than by its
-// projected centre (bit 13)
-constexpr int kItemHit = 1 << 12, kItemRay = 1 << 13;
 
 template <bool kAux, bool kFlow, bool kSlots>
 __global__ void __launch_bounds__(kBlendThreads) __attribute__((amdgpu_waves_per_eu(FSGS_BWD_WAVES, FSGS_BWD_WAVES)))
@@ -164,9 +159,7 @@ blend_backward_kernel(
   float acc_lin = 0;
   float last_alpha = 0, acc_w = 0;
   float acc_f0 = 0, acc_f1 = 0, last_f0 = 0, last_f1 = 0;
-  // the wavefront's queue: items [q_head, q_head + q_count) of its ring (wave-uniform, multiples of 16)
-  int q_head = 0, q_count = 0;
-  unsigned long long q_rows = 0ull;            // entry (staging slot) of each of the ring's eight rows, a byte per row
+  PairQueue q;                                 // the wavefront's queue of blended pairs
   const int row_shift = (lane >> 4) * 8;       // this lane's byte of the four rows of a pass
   const float qx0 = (float) (tile_x * kTile + (wave & 1) * 8), qy0 = (float) (tile_y * kTile + (wave >> 1) * 8);
 
@@ -270,9 +263,9 @@ blend_backward_kernel(
       auto drain = [&](int n_valid) {
         // the entries of the four rows come from the wavefront's scalar bookkeeping, so the queued item, the staged
         // record and the accumulator row are requested together (one LDS round trip instead of three in a chain)
-        const unsigned jrows = (unsigned) (q_rows >> (q_head >> 1));  // q_head is 0 or 64: byte r = entry of row r
+        const unsigned jrows = queue_front_rows(q);  // byte r = entry of row r
         const int j = (int) ((jrows >> row_shift) & 63u);
-        const float4 it = s_queue[wave][q_head + lane];
+        const float4 it = s_queue[wave][q.head + lane];
         const SplatHot hot = s_hot[j];
         float* const acc = &s_part[wave][j][lane & 15];
         const float before = *acc;
@@ -313,26 +306,8 @@ blend_backward_kernel(
           g[12] = g[13] = g[14] = 0.0f;
         }
         g[15] = GdA;
-        const float own = row_sum16_transposed(g);  // lane (row, c): the row's total of component c
-        // An entry with more than 16 blending pixels fills neighbouring rows. The accumulator belongs to this wavefront
-        // alone, so a row adds with a plain read and write, provided no two rows of the pass write the same entry: rows
-        // 2k and 2k + 1 of one entry are added in registers first (one row swap) and row 2k writes for both; a run
-        // that continues from row 1 into row 2 makes row 2 wait for a second round. Rows past n_valid hold old items.
-        const int rows_valid = (n_valid + 15) >> 4;
-        const int j0 = (int) (jrows & 63u), j1 = rows_valid > 1 ? (int) ((jrows >> 8) & 63u) : -1;
-        const int j2 = rows_valid > 2 ? (int) ((jrows >> 16) & 63u) : -2, j3 = rows_valid > 3 ? (int) ((jrows >> 24) & 63u) : -3;
-        const bool s01 = j0 == j1, s12 = j1 == j2, s23 = j2 == j3;
-        float lo = own, hi = own;  // after the swap: lo = rows (0, 0, 2, 2), hi = rows (1, 1, 3, 3) of `own`
-        asm volatile("s_nop 1\n\tv_permlane16_swap_b32_e32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
-        const float pair = lo + hi;
-        const int row = lane >> 4;
-        const bool joined = (row == 0 && s01) || (row == 2 && s23);          // this row writes for its odd neighbour too
-        const bool silent = (row == 1 && s01) || (row == 3 && s23) || row >= rows_valid;
-        const float mine = joined ? pair : own;
-        if (!silent && !(row == 2 && s12)) *acc = before + mine;
-        if (s12) {  // wave-uniform; the LDS serves a wavefront's accesses in order, so this read sees row 0 / 1's store
-          if (row == 2 && !silent) *acc = *(volatile float*) acc + mine;  // re-read: rows 0 / 1 may just have written it
-        }
+        // lane (row, c) holds the row's total of component c
+        queue_accumulate(acc, before, row_sum16_transposed(g), jrows, n_valid, true);
         const bool filtered = blends && !by_ray;
         if (wave_ballot(filtered) != 0ull) {  // some pair met its surfel by the projected centre
           const float to_centre = filtered ? -2.0f * oG : 0.0f;
@@ -341,11 +316,10 @@ blend_backward_kernel(
           cx += dpp_shift_zero<0x112, 0xf, 0xf>(cx), cy += dpp_shift_zero<0x112, 0xf, 0xf>(cy);
           cx += dpp_shift_zero<0x114, 0xf, 0xf>(cx), cy += dpp_shift_zero<0x114, 0xf, 0xf>(cy);
           cx += dpp_shift_zero<0x118, 0xf, 0xf>(cx), cy += dpp_shift_zero<0x118, 0xf, 0xf>(cy);
-          if (row < rows_valid && (lane & 15) == 15) atomicAdd(&s_part[wave][j][16], cx), atomicAdd(&s_part[wave][j][17], cy);
+          if ((lane >> 4) < ((n_valid + 15) >> 4) && (lane & 15) == 15)
+            atomicAdd(&s_part[wave][j][16], cx), atomicAdd(&s_part[wave][j][17], cy);
         }
-        // a full pass leaves the other half of the ring in front; the last, partial pass of a batch empties the queue
-        if (n_valid >= kWave) q_head ^= kWave, q_count -= kWave;
-        else q_head = 0, q_count = 0;
+        queue_pop(q, n_valid);
       };
       // ---- order-bound part of one entry, and the append of its blending pixels to the queue -----------------------------
       auto queue_entry = [&](const SplatHot& hot, const SplatCold& cold, int j) {
@@ -360,23 +334,8 @@ blend_backward_kernel(
           advance_pixel(cold, pos, h, w, dL_dalpha, dL_dz);
           dL_dalpha *= T * h.G;  // only G * dL/dalpha is ever used
         }
-        // blending lanes take the first popcount(pass) places in lane order; the next lanes that do not blend fill the
-        // row up with neutral items (zeros, no flags, their own pixel: every number formed from it is finite)
-        const int n_hit = (int) __popcll(pass), n_pad = (n_hit + 15) & ~15;
-        const int below = (int) __builtin_amdgcn_mbcnt_hi((unsigned) (pass >> 32), __builtin_amdgcn_mbcnt_lo((unsigned) pass, 0u));
-        const int place = hit ? below : n_hit + (lane - below);
-        const int flags = hit ? (h.rho3d <= h.rho2d ? (kItemHit | kItemRay) : kItemHit) : 0;
-        const int tail = q_head + q_count;  // first free place of the ring (mod its size), a multiple of 16
-        if (place < n_pad)
-          s_queue[wave][(tail + place) & (kQueueItems - 1)] =
-              make_float4(w, dL_dalpha, dL_dz, __int_as_float(lane | flags));
-        // which entry each 16-item row of the ring holds: one byte per row in a 64-bit scalar
-        for (int r = 0; r < n_pad; r += 16) {
-          const int sh = (((tail + r) & (kQueueItems - 1)) >> 4) * 8;
-          q_rows = (q_rows & ~(0xffull << sh)) | ((unsigned long long) j << sh);
-        }
-        q_count += n_pad;
-        if (q_count >= kWave) drain(kWave);
+        const int flags = h.rho3d <= h.rho2d ? (kItemHit | kItemRay) : kItemHit;
+        if (queue_append(s_queue[wave], q, j, hit, pass, w, dL_dalpha, dL_dz, flags)) drain(kWave);
       };
       if (todo != 0ull) {
         auto pop = [&]() {
@@ -403,7 +362,7 @@ blend_backward_kernel(
             queue_entry(hot_b, cold, j);
           }
         }
-        if (q_count > 0) drain(q_count);  // the staged records are replaced after the next barrier
+        if (q.count > 0) drain(q.count);  // the staged records are replaced after the next barrier
       }
     } else {
      // Gradient terms of one (pixel, entry) pair, formed in the pass that advances the pixel. The part under `hit` leaves
