@@ -215,6 +215,29 @@ def test_fast_ordered_sums_match_the_atomic_sums(name, per_splat, device):
     assert not a['g_trans'][:, :2].any() and a['g_trans'][:, 2].any()
 
 
+@pytest.mark.parametrize("ordered", [True, False])
+@pytest.mark.parametrize("name", ["partial_tiles_511x127", "dense_6k_96", "big_surfels_96x80"])
+def test_fast_image_only_backward(name, ordered, device):
+    """Without gradients of the auxiliary maps the backward runs its image-only instantiation (no depth terms, the
+    projected-centre pairs' means2D sums on their own path). Its results against the full instantiation fed zeros for
+    those gradients, which the stage-by-stage test holds to the oracle: the same sums up to rounding."""
+    from fast_sp_gs_amd.renderer import fast_render_step
+    scene, cam, gi, _, _ = _make(name)
+    sc, cm, gi = scene.to(device), cam.to(device), gi.to(device)
+    lean = fast_render_step(sc, cm, gi, ordered_sums=ordered)
+    full = fast_render_step(sc, cm, gi, torch.zeros(8, cam.H, cam.W, device=device),
+                            torch.zeros(cam.H, cam.W, device=device), ordered_sums=ordered)
+    torch.cuda.synchronize()
+    assert float(full['g_means2D_blend'].abs().max()) > 0  # some pair is met by its projected centre
+    for k in ('g_colors', 'g_means2D_blend', 'g_inv', 'g_normal_opacity', 'g_means3D', 'g_scales', 'g_rotations',
+              'g_opacities', 'g_shs'):
+        ref = float(full[k].abs().max())
+        err = float((lean[k] - full[k]).abs().max())
+        print(f"[fast image-only {name} ordered={ordered}] {k}: max {ref:.3e} diff {err:.3e}", flush=True)
+        assert bool(torch.isfinite(lean[k]).all()) and err <= 2e-5 * max(ref, 1e-30), k
+    assert not lean['g_trans'].any()  # the third row only carries depth gradients
+
+
 def test_fast_empty_scene(device):
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd.renderer import fast_render_step
