@@ -653,6 +653,7 @@ def training_forward_ms(dev, scene, cam, reps: int = 30):
 def fast_path_rate(dev, scene, cam, gi, steps: int = 20, warmup: int = 3):
     """The "fast" variant (adjugate intersection, fused corner-test binning) on the benchmark scene, forward + backward,
     with the blend backward's per-surfel sums through ordered per-instance records (default) and through atomics."""
+    from fast_sp_gs_amd._C import _ops
     from fast_sp_gs_amd.renderer import fast_render_step
     ge = torch.zeros(8, cam.H, cam.W, device=dev)
     go = -gi.sum(0)
@@ -669,7 +670,22 @@ def fast_path_rate(dev, scene, cam, gi, steps: int = 20, warmup: int = 3):
         torch.cuda.synchronize()
         rates.append(steps / (time.perf_counter() - t0))
         gc.enable()
-    return rates
+    # the two backward decompositions on that view with the per-splat channel set: one block per tile walking its list
+    # back to front (the default behind both operator forms) against the reference's second algorithm, one lane per list
+    # entry with the pixels passed from lane to lane from the forward's bucket snapshots (gs_2d_fast_redner.cu:563-837)
+    bwd_ms = {}
+    for name, per_splat_kernel in (("tile", False), ("per_splat", True)):
+        call = lambda: fast_render_step(scene, cam, gi, ge, go, per_splat=True, per_splat_kernel=per_splat_kernel)
+        call()
+        _ops.STAGE_EVENTS, _ops.STAGE_FILTER = events, _ = [], {'gs_2d_fast_render_backward'}
+        try:
+            for _ in range(10):
+                call()
+            torch.cuda.synchronize()
+        finally:
+            _ops.STAGE_EVENTS, _ops.STAGE_FILTER = None, None
+        bwd_ms[name] = float(np.mean([a.elapsed_time(b) for _, a, b in events]))
+    return rates, bwd_ms
 
 
 def main():
@@ -812,8 +828,13 @@ def main():
         extra.update(gs3d_path_rate(dev, scene, cam, gi))
         extra.update(density_control_ms(dev, scene))
         extra.update(large_scene_ms(dev))
-        extra["fast_path_frames_per_s"], extra["fast_path_atomic_sums_frames_per_s"] = fast_path_rate(dev, scene, cam, gi)
+        (extra["fast_path_frames_per_s"], extra["fast_path_atomic_sums_frames_per_s"]), fast_bwd = fast_path_rate(dev, scene, cam, gi)
         extra["fast_path_workload"] = "same scene through GS_2D_fast_* (corner-test binning keeps fewer instances)"
+        extra["fast_backward_tile_kernel_ms"] = fast_bwd["tile"]
+        extra["fast_backward_per_splat_kernel_ms"] = fast_bwd["per_splat"]
+        extra["fast_backward_workload"] = ("GS_2D_fast_render_backward on that view, per-splat channel set, ordered sums "
+                                           "(record clear + kernel + record sum): back-to-front tile kernel / the "
+                                           "reference's per-splat decomposition (wavefront = 64 entries)")
         extra["dynamic_step_frames_per_s"] = dynamic_step_rate(dev)
         extra["dynamic_step_workload"] = ("200000 surfels, 512 control points, bf16 MFMA MLP + K-NN(4) + LBS -> render "
                                           "800x800 -> 0.8 L1 + 0.2 D-SSIM (fused kernel) -> backward through LBS / K-NN / MLP "

@@ -720,19 +720,27 @@ def GS_2D_fast_render_forward(width: int, height: int, near_n: float, far_n: flo
     return outputs
 
 
+# GS_2D_fast_render_backward with snapshots: the reference's per-splat kernel instead of the back-to-front one
+PER_SPLAT_BACKWARD = False
+
+
 def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inverse_m, trans_mat2, images, out_opacity,
                                out_others, out_flows, dL_dout_color, dL_dout_opacity, dL_dothers, dL_dout_flow,
                                ranges, point_list, n_contrib, near_n: float, far_n: float,
                                per_tile_bucket_offset=None, bucket_to_tile=None, max_contrib=None, sampled_T=None,
                                sampled_acc=None, sampled_aux=None, point_offsets: Optional[Tensor] = None,
-                               radii: Optional[Tensor] = None):
+                               radii: Optional[Tensor] = None, per_splat_kernel: Optional[bool] = None):
     """gs_2d_fast_redner.cu:955-1074 -> [dL_dcolors[P,3], dL_dmeans2D[P,2], dL_dtrans_m[P,3,3], dL_dinverse_m[P,3,3],
     dL_dnorm_op[P,4]]. Passing per_tile_bucket_offset selects the per-splat channel set of the reference's second
-    kernel; the snapshot tensors themselves are not needed to evaluate it here. With dL_dout_flow (and trans_mat2,
+    kernel; the snapshot tensors themselves are not needed to evaluate it with the back-to-front kernel, which is the
+    default (faster here). `per_splat_kernel=True` (default: PER_SPLAT_BACKWARD) runs the reference's per-splat
+    decomposition itself from the snapshots (no optical flow in that form). With dL_dout_flow (and trans_mat2,
     out_flows) the optical-flow gradient is added as the reference's kernels add it. With `point_offsets`
     (gs_2d_fast_preprocess_forward(..., return_offsets=True)) and `radii` the per-surfel sums are taken in a fixed order
     from per-instance records instead of with atomics."""
     what = 'GS_2D_fast_render_backward'
+    if per_splat_kernel is None:
+        per_splat_kernel = PER_SPLAT_BACKWARD
     L.require_cuda(what, dL_dout_color=dL_dout_color, dL_dout_opacity=dL_dout_opacity, dL_dothers=dL_dothers)
     P = means2D.shape[0]
     H, W = dL_dout_color.shape[1], dL_dout_color.shape[2]
@@ -762,6 +770,41 @@ def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inver
         L.require_shape(what, 'trans_mat2', trans_mat2, P, 3, 3)
         L.require_shape(what, 'out_flows', out_flows, H, W, 2)
         L.require_shape(what, 'dL_dout_flow', dL_dout_flow, H, W, 2)
+    if per_splat_kernel and per_splat and not flow:
+        snaps = dict(images=images, bucket_to_tile=bucket_to_tile, max_contrib=max_contrib, sampled_T=sampled_T,
+                     sampled_acc=sampled_acc)
+        if use_aux:
+            snaps['sampled_aux'] = sampled_aux
+        missing = [k for k, v in snaps.items() if v is None]
+        if missing:
+            raise RuntimeError(f'{what}: the per-splat kernel needs {", ".join(missing)}')
+        B = bucket_to_tile.shape[0]
+        T_tiles = ranges.shape[0]
+        images, sampled_T, sampled_acc, sampled_aux = c(images), c(sampled_T), c(sampled_acc), c(sampled_aux)
+        bucket_to_tile, max_contrib, offsets = c(bucket_to_tile), c(max_contrib), c(per_tile_bucket_offset)
+        _f32(what, images=images, sampled_T=sampled_T, sampled_acc=sampled_acc, sampled_aux=sampled_aux)
+        L.require_shape(what, 'images', images, 3, H, W)
+        L.require_shape(what, 'sampled_T', sampled_T, B, 256)
+        L.require_shape(what, 'sampled_acc', sampled_acc, B, 3, 256)
+        if use_aux:
+            L.require_shape(what, 'sampled_aux', sampled_aux, B, 8, 256)
+        for name, t, n, dt in (('bucket_to_tile', bucket_to_tile, B, torch.int32),
+                               ('max_contrib', max_contrib, T_tiles, torch.int32),
+                               ('per_tile_bucket_offset', offsets, T_tiles, torch.int64)):
+            if t.dtype != dt or t.numel() != n:
+                raise RuntimeError(f'{what}: {name} must be {dt} with {n} entries')
+        with _timed('gs_2d_fast_render_backward'):
+            rc = _lib().fsgs_gs_2d_fast_render_bucket_backward(
+                P, W, H, float(near_n), float(far_n), B, L.ptr(means2D), L.ptr(normal_opacity), L.ptr(colors),
+                L.ptr(trans_mat), L.ptr(inverse_m), L.ptr(images), L.ptr(out_opacity),
+                L.ptr(out_others) if use_aux else None, L.ptr(n_contrib), L.ptr(max_contrib), L.ptr(offsets),
+                L.ptr(bucket_to_tile), L.ptr(sampled_T), L.ptr(sampled_acc), L.ptr(sampled_aux) if use_aux else None,
+                L.ptr(dL_dout_color), L.ptr(dL_dout_opacity), L.ptr(dL_dothers) if use_aux else None, L.ptr(ranges),
+                L.ptr(point_list), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_inv), L.ptr(g_norm_op),
+                R, L.ptr(point_offsets) if ordered else None, L.ptr(radii) if ordered else None, L.ptr(ws),
+                ws.numel() if ws is not None else 0, L.current_stream())
+        L.check(rc, what)
+        return [g_colors, g_means2D, g_trans, g_inv, g_norm_op]
     with _timed('gs_2d_fast_render_backward'):
         rc = _lib().fsgs_gs_2d_fast_render_backward(
             P, W, H, float(near_n), float(far_n), int(per_splat), L.ptr(means2D), L.ptr(normal_opacity), L.ptr(colors),

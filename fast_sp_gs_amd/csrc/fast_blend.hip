@@ -8,15 +8,16 @@
 // The per-splat form of the reference re-walks 32-entry buckets from the forward snapshots with one warp per bucket;
 // its result is the same derivative with a different set of live channels (no distortion gradient, M1/M2 maps as
 // plain weighted sums with the M1 depth term overwritten, :751-757). Here both forms run the same tile-per-block
-// back-to-front kernel and differ only in that channel set; the snapshots are still produced by the forward for callers
-// that consume them. Optical flow (a second set of transforms, :247-255): the forward divides the weighted sum of
+// back-to-front kernel by default and differ only in that channel set; the per-splat decomposition itself is
+// fast_bucket_backward_kernel below, which consumes the forward's snapshots (slower on this chip). Optical flow (a second set of transforms, :247-255): the forward divides the weighted sum of
 // displacements by the final opacity (:259-263); both backward forms take dL/dflow as the gradient of the UNDIVIDED sum
 // (:366, :704), and the per-splat form subtracts the DIVIDED final flow from its partial sums (:706), which amounts to
 // an opacity-map gradient lowered by (final flow . dL/dflow) -- reproduced here in that algebraic form.
 //
-// Layout as in the standard blend: one 256-lane block per tile, wavefront w owns an 8x8 quadrant, surfels staged 256 at
-// a time in LDS (64-byte hot record with the adjugate, 32-byte cold record), per-quadrant work lists from a
-// conservative bound, gradients reduced over the wavefront in registers before one LDS atomic per component.
+// Layout as in the standard blend: one 256-lane block per tile, wavefront w owns an 8x8 quadrant, surfels staged in
+// LDS (64-byte hot record with the adjugate, 32-byte cold record), per-quadrant work lists from a conservative bound;
+// the backward queues its blended (pixel, entry) pairs and forms their gradient components 64 pairs at a time
+// (pair_queue.hpp).
 #include "blend.hpp"
 #include "ordered_sums.hpp"
 #include "pair_queue.hpp"
@@ -723,6 +724,187 @@ __global__ void __launch_bounds__(kBlendThreads)
   }
 }
 
+
+// The reference's second backward (gs_2d_fast_redner.cu:563-837), the per-splat decomposition itself: a lane owns ONE
+// list entry of a tile and keeps that surfel's 21 gradient sums in registers, the tile's pixels pass through the lanes
+// one lane per step, front to back, each carrying its blending state from the forward's snapshot in front of the
+// bucket on. Where the reference hands 27 values from lane to lane (transmittance, three colour and eight auxiliary
+// partial sums, the upstream gradients and counters of the pixel), here two travel: the transmittance T and
+//   S = <dL/d(outputs), partial sums - final outputs> + T_final dL/dopacity,
+// because dL/dalpha = T c + S / (1 - alpha) with c = <dL/d(outputs), this pair's channel values> only needs the partial
+// sums through that one product (S += w c per blended pair); the per-pixel constants are staged in LDS once and read
+// by pixel number. Laid out for a 64-lane wavefront as the 3D-Gaussian form of this decomposition: one wavefront takes
+// 64 consecutive entries = two of the forward's 32-entry buckets (the wavefront of the odd bucket leaves at once), the
+// state moves with one whole-wavefront DPP shift per value, and only the pixels that still blend at the group's first
+// entry are fed in. Channel set of the reference's kernel: image, opacity, depth, normal, median depth, M1, M2 (no
+// distortion; the depth gradient through M1 is dropped as there, :751-757).
+template <bool kAux, bool kSlots>
+__global__ void __launch_bounds__(64) fast_bucket_backward_kernel(int W, int H, float near_n, float far_n,
+    const int64_t* __restrict__ ranges, const int32_t* __restrict__ point_list, const float2* __restrict__ means2D,
+    const float4* __restrict__ normal_opacity, const float* __restrict__ colors, const float* __restrict__ trans_mat,
+    const float* __restrict__ inverse_m, const float* __restrict__ images, const float* __restrict__ out_opacity,
+    const float* __restrict__ out_extras, const int32_t* __restrict__ n_contrib,
+    const int32_t* __restrict__ max_contrib, const int64_t* __restrict__ bucket_offset,
+    const int32_t* __restrict__ bucket_to_tile, const float* __restrict__ sampled_T,
+    const float* __restrict__ sampled_acc, const float* __restrict__ sampled_aux, const float* __restrict__ dL_dpix,
+    const float* __restrict__ dL_dextras, const float* __restrict__ dL_dopacity, float* __restrict__ g_means2D,
+    float* __restrict__ g_normal_opacity, float* __restrict__ g_colors, float* __restrict__ g_trans,
+    float* __restrict__ g_inv, const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii,
+    float* __restrict__ slot_records) {
+  __shared__ float4 s_up[256];                // dL/d(r, g, b) | dL/ddepth
+  __shared__ float4 s_up2[kAux ? 256 : 1];    // dL/dnormal | dL/dM1
+  __shared__ float4 s_up3[kAux ? 256 : 1];    // dL/dM2 | dL/d(median depth) | median contributor (int bits) | -
+  __shared__ float4 s_pixel[256];             // x | y | last contributor (int bits) | -
+  __shared__ float2 s_state[256];             // snapshot: T | S
+  const int bucket = blockIdx.x, lane = threadIdx.x;
+  const int tile = bucket_to_tile[bucket];
+  const int in_tile = bucket - (int) (tile == 0 ? 0 : bucket_offset[tile - 1]);
+  if (in_tile & 1) return;
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const int tile_x = tile % gx, tile_y = tile / gx;
+  const int64_t r0 = ranges[2 * (size_t) tile], r1 = ranges[2 * (size_t) tile + 1];
+  const int first = in_tile * 32, entry = first + lane;
+  const bool valid = entry < (int) (r1 - r0);
+  const size_t HW = (size_t) H * W;
+  const float far_scale = far_n / (far_n - near_n), far_near = far_scale * near_n;
+
+  FastHot hot{};
+  SplatCold cold{};
+  size_t slot = 0;
+  if (valid) {
+    const FastSplat g = gather_fast(point_list[r0 + entry], means2D, colors, normal_opacity, trans_mat, inverse_m);
+    hot = g.hot, cold = g.cold;
+    if (kSlots) {
+      const TileRect r = tile_rect(hot.cx, hot.cy, radii[cold.id], gx, gy);
+      slot = (size_t) ((cold.id == 0 ? 0 : point_offsets[cold.id - 1]) + (int64_t) (tile_x - r.x0) * (r.y1 - r.y0) +
+                       (tile_y - r.y0));
+    }
+  }
+
+  // the pixels that still blend at this group's first entry, in row-major order of the tile
+  int n_live = 0;
+  if (first < max_contrib[tile]) {
+#pragma unroll
+    for (int part = 0; part < 4; ++part) {
+      const int rank = part * 64 + lane;
+      const int px = tile_x * kTile + (rank & 15), py = tile_y * kTile + (rank >> 4);
+      const bool inside = px < W && py < H;
+      const size_t pix = (size_t) W * py + px;
+      const int last = inside ? n_contrib[pix] : 0;
+      const bool live = last > first;
+      const unsigned long long live_lanes = wave_ballot(live);
+      if (live) {
+        const int at = n_live + __builtin_amdgcn_mbcnt_hi((unsigned) (live_lanes >> 32),
+                                                          __builtin_amdgcn_mbcnt_lo((unsigned) live_lanes, 0u));
+        const size_t snap = (size_t) bucket * 256 + rank;
+        const float up0 = dL_dpix[pix], up1 = dL_dpix[HW + pix], up2 = dL_dpix[2 * HW + pix];
+        float S = (1.0f - out_opacity[pix]) * dL_dopacity[pix];
+        S += up0 * (sampled_acc[((size_t) bucket * 3 + 0) * 256 + rank] - images[pix]);
+        S += up1 * (sampled_acc[((size_t) bucket * 3 + 1) * 256 + rank] - images[HW + pix]);
+        S += up2 * (sampled_acc[((size_t) bucket * 3 + 2) * 256 + rank] - images[2 * HW + pix]);
+        float up_depth = 0.0f;
+        if (kAux) {
+          auto behind = [&](int c) { return sampled_aux[((size_t) bucket * 8 + c) * 256 + rank] - out_extras[c * HW + pix]; };
+          up_depth = dL_dextras[pix];
+          const float n0 = dL_dextras[1 * HW + pix], n1 = dL_dextras[2 * HW + pix], n2 = dL_dextras[3 * HW + pix];
+          const float m1 = dL_dextras[6 * HW + pix], m2 = dL_dextras[7 * HW + pix];
+          S += up_depth * behind(0) + n0 * behind(1) + n1 * behind(2) + n2 * behind(3) + m1 * behind(6) + m2 * behind(7);
+          s_up2[at] = make_float4(n0, n1, n2, m1);
+          s_up3[at] = make_float4(m2, dL_dextras[4 * HW + pix], __int_as_float(n_contrib[HW + pix]), 0.0f);
+        }
+        s_up[at]    = make_float4(up0, up1, up2, up_depth);
+        s_state[at] = make_float2(sampled_T[snap], S);
+        s_pixel[at] = make_float4((float) px, (float) py, __int_as_float(last), 0.0f);
+      }
+      n_live += __builtin_popcountll(live_lanes);
+    }
+  }
+  __syncthreads();
+
+  float g[kFastGradSlots];
+#pragma unroll
+  for (int c = 0; c < kFastGradSlots; ++c) g[c] = 0.0f;
+  float T = 0.0f, S = 0.0f;
+  // whole-wavefront shift by one lane (DPP wave_shr:1); lane 0 keeps `fresh`
+  auto pass_on = [](float fresh, float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, fresh),
+                                                                 __builtin_bit_cast(int, v), 0x138, 0xf, 0xf, false));
+  };
+  const int steps = n_live > 0 ? n_live + 63 : 0;
+  float2 next_state = s_state[0];
+  for (int i = 0; i < steps; ++i) {
+    const float2 fresh = next_state;
+    next_state = s_state[min(i + 1, n_live - 1)];  // requested a step ahead of its use (nothing new once all have entered)
+    T = pass_on(fresh.x, T);
+    S = pass_on(fresh.y, S);
+    const int q = i - lane;
+    if (q < 0 || q >= n_live) continue;
+    const float4 pixel = s_pixel[q];
+    FastHit h;
+    const bool hit = fast_intersect_flat(hot, pixel.x, pixel.y, near_n, h) && valid && entry < __float_as_int(pixel.z);
+    if (!hit) continue;
+    const float4 up = s_up[q];
+    const float w = h.alpha * T, inv = __builtin_amdgcn_rcpf(1.0f - h.alpha);
+    float c_lin = cold.r * up.x + cold.g * up.y + cold.b * up.z;
+    float dL_dz = 0.0f;
+    if (kAux) {
+      const float4 upn = s_up2[q], upm = s_up3[q];
+      const float rd     = __builtin_amdgcn_rcpf(h.depth);
+      const float m_d    = far_scale - far_near * rd;
+      const float dmd_dd = far_near * rd * rd;
+      c_lin += h.depth * up.w + cold.nx * upn.x + cold.ny * upn.y + cold.nz * upn.z + m_d * upn.w + (m_d * m_d) * upm.x;
+      dL_dz = w * up.w + dmd_dd * (2.0f * m_d * w * upm.x);
+      if (entry == __float_as_int(upm.z) - 1) dL_dz += upm.y;
+      g[12] += w * upn.x, g[13] += w * upn.y, g[14] += w * upn.z;
+    }
+    S += w * c_lin;  // the partial sums up to and including this pair, minus the final outputs
+    const float dL_dalpha = T * c_lin + inv * S;
+    T *= 1.0f - h.alpha;
+    const float GdA = h.G * dL_dalpha, oG = hot.opacity * GdA;
+    const bool by_ray = h.rho3d <= h.rho2d;
+    const float rz = by_ray ? __builtin_amdgcn_rcpf(h.pz) : 0.0f;
+    const float dsx = dL_dz * hot.tw0 - oG * h.sx, dsy = dL_dz * hot.tw1 - oG * h.sy;
+    const float da = dsx * rz, db = dsy * rz, dc = -(da * h.sx + db * h.sy);
+    g[0] += w * up.x, g[1] += w * up.y, g[2] += w * up.z;
+    g[3] += da * pixel.x, g[4] += da * pixel.y, g[5] += da;
+    g[6] += db * pixel.x, g[7] += db * pixel.y, g[8] += db;
+    g[9] += dc * pixel.x, g[10] += dc * pixel.y, g[11] += dc;
+    g[15] += GdA;
+    g[16] += dL_dz * h.sx, g[17] += dL_dz * h.sy, g[18] += dL_dz;
+    const float to_centre = by_ray ? 0.0f : -2.0f * oG;
+    g[19] += to_centre * h.dx, g[20] += to_centre * h.dy;
+  }
+  if (!valid) return;
+  if (kSlots) {
+    bool any = false;
+#pragma unroll
+    for (int c = 0; c < kFastGradSlots; ++c) any |= g[c] != 0.0f;
+    if (any) {  // the record buffer is zero-filled
+      float2* dst = (float2*) (slot_records + slot * kFastRecordSlots);
+#pragma unroll
+      for (int c = 0; c < kFastRecordSlots / 2; ++c)
+        dst[c] = make_float2(g[2 * c], 2 * c + 1 < kFastGradSlots ? g[2 * c + 1] : 0.0f);
+    }
+  } else {
+    const int id = cold.id;
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+      if (g[c] != 0.0f) atomicAdd(&g_colors[3 * (size_t) id + c], g[c]);
+#pragma unroll
+    for (int c = 0; c < 9; ++c)
+      if (g[3 + c] != 0.0f) atomicAdd(&g_inv[9 * (size_t) id + c], g[3 + c]);
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      if (g[12 + c] != 0.0f) atomicAdd(&g_normal_opacity[4 * (size_t) id + c], g[12 + c]);
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+      if (g[16 + c] != 0.0f) atomicAdd(&g_trans[9 * (size_t) id + 6 + c], g[16 + c]);
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+      if (g[19 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], g[19 + c]);
+  }
+}
+
 }  // namespace
 }  // namespace fsgs
 
@@ -828,4 +1010,58 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
     launch_slot_sum<kFastRecordSlots>(P, point_offsets, ws,
                                       FastScatter{g_means2D, g_normal_opacity, g_colors, g_trans, g_inv}, s);
   return check_launch("GS_2D_fast_render_backward");
+}
+
+// The per-splat decomposition itself (fast_bucket_backward_kernel), for callers that want the reference's second
+// algorithm rather than its result: B = the number of 32-entry buckets the forward announced (bucket_to_tile's length).
+FSGS_API int fsgs_gs_2d_fast_render_bucket_backward(int P, int W, int H, double near_n, double far_n, int B,
+    const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,
+    const float* inverse_m, const float* images, const float* out_opacity, const float* out_extras,
+    const int32_t* n_contrib, const int32_t* max_contrib, const int64_t* bucket_offset,
+    const int32_t* bucket_to_tile, const float* sampled_T, const float* sampled_acc, const float* sampled_aux,
+    const float* dL_dpix, const float* dL_dopacity, const float* dL_dextras, const int64_t* ranges,
+    const int32_t* point_list, float* g_colors, float* g_means2D, float* g_trans, float* g_inv,
+    float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
+    size_t workspace_bytes, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && B >= 0, "GS_2D_fast_render_bucket_backward: bad sizes");
+  if (P == 0) return kOk;
+  FSGS_REQUIRE(means2D && normal_opacity && colors && trans_mat && inverse_m && images && out_opacity && n_contrib &&
+                   max_contrib && bucket_offset && dL_dpix && dL_dopacity && ranges && g_colors && g_means2D &&
+                   g_trans && g_inv && g_normal_opacity &&
+                   (B == 0 || (bucket_to_tile && point_list && sampled_T && sampled_acc)),
+               "GS_2D_fast_render_bucket_backward: null pointer");
+  const bool aux = out_extras && dL_dextras;
+  FSGS_REQUIRE(!aux || B == 0 || sampled_aux,
+               "GS_2D_fast_render_bucket_backward: the auxiliary maps need their snapshots");
+  const bool slots = point_offsets != nullptr;
+  SlotWorkspace ws{nullptr};
+  if (slots) {
+    FSGS_REQUIRE(radii && workspace && R >= 0 && R < (int64_t) 0x7fffffff,
+                 "GS_2D_fast_render_bucket_backward: the ordered-sum path needs radii, a workspace and the instance count R");
+    if (workspace_bytes < slot_workspace_bytes(R, kFastRecordSlots))
+      return fail(kWorkspaceSmall, "GS_2D_fast_render_bucket_backward: workspace %zu < %zu bytes", workspace_bytes,
+                  slot_workspace_bytes(R, kFastRecordSlots));
+    FSGS_REQUIRE(((uintptr_t) workspace & 15) == 0, "GS_2D_fast_render_bucket_backward: workspace must be 16-byte aligned");
+    ws = slot_workspace(workspace, R, kFastRecordSlots);
+  }
+  hipStream_t s = (hipStream_t) stream;
+  if (slots) launch_slot_clear<kFastRecordSlots>(ws, R, s);
+#define FSGS_FAST_BKT(AUX, SL)                                                                                        \
+  hipLaunchKernelGGL((fast_bucket_backward_kernel<AUX, SL>), dim3(B), dim3(64), 0, s, W, H, (float) near_n,           \
+                     (float) far_n, ranges, point_list, (const float2*) means2D, (const float4*) normal_opacity,      \
+                     colors, trans_mat, inverse_m, images, out_opacity, out_extras, n_contrib, max_contrib,           \
+                     bucket_offset, bucket_to_tile, sampled_T, sampled_acc, sampled_aux, dL_dpix, dL_dextras,         \
+                     dL_dopacity, g_means2D, g_normal_opacity, g_colors, g_trans, g_inv, point_offsets, radii,        \
+                     ws.records)
+  if (B > 0) {
+    if (aux && slots) FSGS_FAST_BKT(true, true);
+    else if (aux) FSGS_FAST_BKT(true, false);
+    else if (slots) FSGS_FAST_BKT(false, true);
+    else FSGS_FAST_BKT(false, false);
+  }
+#undef FSGS_FAST_BKT
+  if (slots)
+    launch_slot_sum<kFastRecordSlots>(P, point_offsets, ws,
+                                      FastScatter{g_means2D, g_normal_opacity, g_colors, g_trans, g_inv}, s);
+  return check_launch("GS_2D_fast_render_bucket_backward");
 }

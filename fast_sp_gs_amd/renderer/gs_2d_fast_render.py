@@ -286,9 +286,11 @@ def fast_compuate_transmat(means3D: Tensor, scales: Tensor, rotations: Tensor, T
 
 
 def fast_render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad_opacity: Tensor = None,
-                     per_splat: bool = False, ordered_sums: bool = True):
+                     per_splat: bool = False, ordered_sums: bool = True, per_splat_kernel: bool = False):
     """One forward + backward pass of the fast path through the raw operators, returning every intermediate. With
-    `ordered_sums` the blend backward adds per-instance records in a fixed order instead of using atomics."""
+    `ordered_sums` the blend backward adds per-instance records in a fixed order instead of using atomics. With
+    `per_splat_kernel` (needs `per_splat`) the backward is the reference's per-splat decomposition, started from the
+    forward's snapshots, instead of the back-to-front kernel with the per-splat channel set."""
     pre_f = get_C_function('gs_2d_fast_preprocess_forward')
     pre_b = get_C_function('gs_2d_fast_preprocess_backward')
     ren_f = get_C_function('GS_2D_fast_render_forward')
@@ -308,8 +310,10 @@ def fast_render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None,
         grad_opacity = torch.zeros_like(opacity)
     g_colors, g_means2D, g_trans, g_inv, g_no = ren_b(
         means2D, normal_opacity, colors, trans_mat, inverse_m, None, image, opacity, extras, None, grad_image,
-        grad_opacity, grad_extras, None, ranges, point_list, n_contrib, cam.near, cam.far, offset, None, None, None,
-        None, None, point_offsets if ordered_sums else None, radii if ordered_sums else None)
+        grad_opacity, grad_extras, None, ranges, point_list, n_contrib, cam.near, cam.far, offset,
+        *((outs[6], outs[5], outs[7], outs[8], outs[9]) if per_splat and per_splat_kernel else (None,) * 5),
+        point_offsets if ordered_sums else None, radii if ordered_sums else None,
+        per_splat_kernel=bool(per_splat and per_splat_kernel))
     g_means2D_in = g_means2D.clone()
     g = dict(means3D=torch.zeros_like(scene.means3D), scales=torch.zeros_like(scene.scales),
              rotations=torch.zeros_like(scene.rotations), opacities=torch.zeros_like(scene.opacities),

@@ -221,6 +221,23 @@ int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n, double f
     float* g_colors, float* g_means2D, float* g_trans, float* g_inv, float* g_normal_opacity, int64_t R,
     const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The per-splat decomposition of gs_2d_fast_redner.cu:563-837 itself (fsgs_gs_2d_fast_render_backward with
+ * per_splat_form = 1 returns the same derivative through the back-to-front kernel, which is faster here): a lane owns
+ * one list entry and keeps its 21 sums in registers, the tile's pixels pass through the lanes carrying their
+ * front-to-back blending state, started from the forward's snapshots (images[3,H,W], max_contrib[T], bucket_offset[T],
+ * bucket_to_tile[B], sampled_T[B,256], sampled_acc[B,3,256], sampled_aux[B,8,256], all as the forward wrote them). One
+ * wavefront takes two 32-entry buckets; B = number of buckets. No optical flow in this form. Outputs and the optional
+ * ordered-sum arguments as fsgs_gs_2d_fast_render_backward. */
+int fsgs_gs_2d_fast_render_bucket_backward(int P, int W, int H, double near_n, double far_n, int B,
+    const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,
+    const float* inverse_m, const float* images, const float* out_opacity, const float* out_extras,
+    const int32_t* n_contrib, const int32_t* max_contrib, const int64_t* bucket_offset,
+    const int32_t* bucket_to_tile, const float* sampled_T, const float* sampled_acc, const float* sampled_aux,
+    const float* dL_dpix, const float* dL_dopacity, const float* dL_dextras, const int64_t* ranges,
+    const int32_t* point_list, float* g_colors, float* g_means2D, float* g_trans, float* g_inv,
+    float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
+    size_t workspace_bytes, void* stream);
+
 /* gs_2d_topk_weights -- fast_2d_gs/_C/src/gaussian_splatting/gaussian_topk.cu:230-250 (kernel :95-210).
  * top_indices[H,W,topk] int32 (-1 = empty), top_weights[H,W,topk] descending blend weights alpha*T; topk <= 16. */
 int fsgs_gs_2d_topk_weights(int topk, int P, int W, int H, double near_n, double far_n, const float* means2D,

@@ -238,6 +238,34 @@ def test_fast_image_only_backward(name, ordered, device):
     assert not lean['g_trans'].any()  # the third row only carries depth gradients
 
 
+@pytest.mark.parametrize("ordered", [True, False])
+@pytest.mark.parametrize("name", ["c0_10k_256", "partial_tiles_511x127", "big_surfels_96x80", "dense_6k_96",
+                                  "tiny_3_surfels"])
+def test_fast_per_splat_kernel(name, ordered, device):
+    """The reference's per-splat decomposition (one lane per list entry, pixels handed from lane to lane, restart from
+    the forward's snapshots) against the back-to-front kernel with the same channel set, which the stage-by-stage test
+    holds to the oracle: the same derivative summed in another order (front to back instead of back to front)."""
+    from fast_sp_gs_amd.renderer import fast_render_step
+    scene, cam, gi, ge, go = _make(name)
+    args = (scene.to(device), cam.to(device), gi.to(device), ge.to(device), go.to(device))
+    tile = fast_render_step(*args, per_splat=True, ordered_sums=ordered)
+    splat = fast_render_step(*args, per_splat=True, ordered_sums=ordered, per_splat_kernel=True)
+    torch.cuda.synchronize()
+    errs = {}
+    for k in ('g_colors', 'g_means2D_blend', 'g_trans', 'g_inv', 'g_normal_opacity', 'g_means3D', 'g_scales',
+              'g_rotations', 'g_opacities', 'g_shs'):
+        assert bool(torch.isfinite(splat[k]).all()), k
+        errs[k] = rel_err(npy(splat[k]), npy(tile[k]))
+    print(f"[fast per-splat kernel {name} ordered={ordered}] rel errs {errs}", flush=True)
+    assert name.startswith('tiny') or (float(tile['g_inv'].abs().max()) > 0 and float(tile['g_trans'].abs().max()) > 0)
+    for k, v in errs.items():
+        assert v < 1e-3, k
+    if ordered:  # fixed order of the additions: identical from run to run
+        again = fast_render_step(*args, per_splat=True, per_splat_kernel=True)
+        for k in ('g_colors', 'g_means2D_blend', 'g_trans', 'g_inv', 'g_normal_opacity'):
+            assert torch.equal(again[k], splat[k]), k
+
+
 def test_fast_empty_scene(device):
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd.renderer import fast_render_step
