@@ -240,7 +240,7 @@ def test_fast_image_only_backward(name, ordered, device):
 
 @pytest.mark.parametrize("ordered", [True, False])
 @pytest.mark.parametrize("name", ["c0_10k_256", "partial_tiles_511x127", "big_surfels_96x80", "dense_6k_96",
-                                  "tiny_3_surfels"])
+                                  "tiny_3_surfels", "c2_300k_800"])
 def test_fast_per_splat_kernel(name, ordered, device):
     """The reference's per-splat decomposition (one lane per list entry, pixels handed from lane to lane, restart from
     the forward's snapshots) against the back-to-front kernel with the same channel set, which the stage-by-stage test
