@@ -535,9 +535,9 @@ __global__ void __launch_bounds__(kBlendThreads)
       const float4 it = s_queue[wave][q.head + lane];
       const FastHot hot = s_hot[j];
       float* const acc  = &s_part[wave][j][lane & 15];
-      float* const acc2 = &s_part[wave][j][16 + (lane & 7)];  // used by lanes 0-4 of a row
+      const bool second = (lane & 15) < 5;  // lanes 0-4 of a row add the five other components
+      float* const acc2 = &s_part[wave][j][16 + (second ? (lane & 15) : 0)];
       const float before = *acc;
-      const bool second = (lane & 15) < 5;
       const float before2 = (kAux && second) ? *acc2 : 0.0f;
       const int bits = __float_as_int(it.w);
       const int qp = bits & 63;
