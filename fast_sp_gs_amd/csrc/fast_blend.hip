@@ -241,24 +241,21 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
           }
           todo &= half ? 0xffffffff00000000ull : 0x00000000ffffffffull;
         }
-        while (todo) {
-          if (live_lanes == 0ull) break;
-          const int j = c * kWave + __builtin_ctzll(todo);
-          todo &= todo - 1;
+        // one entry of the wavefront's work list; its records were requested from LDS while the entry before it ran
+        auto blend_entry = [&](const FastHot& hot, const SplatCold& cold, int j) {
           FastHit h;
           unsigned long long pass;
-          const bool hit = fast_intersect_flat(s_hot[j], pxf, pyf, near_n, h, &pass) && live > 0.0f;
+          const bool hit = fast_intersect_flat(hot, pxf, pyf, near_n, h, &pass) && live > 0.0f;
           pass &= live_lanes;
-          if (pass == 0ull) continue;
+          if (pass == 0ull) return;
           const float test_T = T * (1.0f - h.alpha);
           const bool sat     = hit && test_T < 0.0001f;
           live               = sat ? -1.0f : live;
           live_lanes &= ~(pass & wave_ballot(test_T < 0.0001f));
           const float w         = h.alpha * T;
-          const SplatCold cold  = s_cold[j];
           if (kAccum && (accum_weights_p || accum_weights_count))
             wave_accumulate_weights(hit && !sat, w, cold.id, accum_weights_p, accum_weights_count);
-          if (!hit || sat) continue;
+          if (!hit || sat) return;
           const int contributor = b * kBatch + j + 1;
           if (kAux) {
             const float A = 1.0f - T;
@@ -283,6 +280,32 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
           C0 += cold.r * w, C1 += cold.g * w, C2 += cold.b * w;
           T    = test_T;
           last = contributor;
+        };
+        if (todo == 0ull) continue;
+        auto pop = [&]() {
+          const int j = c * kWave + __builtin_ctzll(todo);
+          todo &= todo - 1;
+          return j;
+        };
+        auto peek = [&]() { return c * kWave + (todo ? __builtin_ctzll(todo) : 0); };
+        FastHot hot_a = s_hot[peek()], hot_b;
+        while (todo) {
+          if (live_lanes == 0ull) break;  // every pixel of this quadrant is saturated
+          {
+            const int j = pop();
+            hot_b       = s_hot[peek()];
+            const SplatCold cold = s_cold[j];  // used only if a pixel blends the surfel, but then without waiting
+            __builtin_amdgcn_sched_barrier(0);
+            blend_entry(hot_a, cold, j);
+          }
+          if (todo == 0ull || live_lanes == 0ull) break;
+          {
+            const int j = pop();
+            hot_a       = s_hot[peek()];
+            const SplatCold cold = s_cold[j];
+            __builtin_amdgcn_sched_barrier(0);
+            blend_entry(hot_b, cold, j);
+          }
         }
       }
     }

@@ -209,7 +209,7 @@ def test_fast_ordered_sums_match_the_atomic_sums(name, per_splat, device):
               'g_rotations', 'g_opacities', 'g_shs'):
         assert torch.equal(a[k], b[k]) and bool(torch.isfinite(a[k]).all()), k
         ref = float(c[k].abs().max())
-        assert ref > 0 and float((a[k] - c[k]).abs().max()) <= 2e-5 * ref, k
+        assert ref > 0 and float((a[k] - c[k]).abs().max()) <= 5e-5 * ref, k  # the atomics add in any order
         if k in ('g_colors', 'g_means2D_blend', 'g_trans', 'g_inv', 'g_normal_opacity'):
             assert not a[k][hidden].any(), k
     assert not a['g_trans'][:, :2].any() and a['g_trans'][:, 2].any()
