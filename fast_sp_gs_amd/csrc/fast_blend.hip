@@ -79,22 +79,27 @@ struct FastHit {
 // `lanes`, if given: mask of the lanes that pass, from the four comparisons' own lane masks (scalar registers).
 __device__ __forceinline__ bool fast_intersect_flat(const FastHot& h, float pxf, float pyf, float near_n, FastHit& o,
                                                     unsigned long long* lanes = nullptr) {
-  const float p0 = h.a[0] * pxf + h.a[1] * pyf + h.a[2];
-  const float p1 = h.a[3] * pxf + h.a[4] * pyf + h.a[5];
-  o.pz           = h.a[6] * pxf + h.a[7] * pyf + h.a[8];
+  // Every fused multiply-add is written out and contraction is off: the kernels inline this more than once (two copies
+  // of a loop body that alternate their registers), and which copy evaluates an entry depends on the work list, so the
+  // copies must round alike. Exponent in base 2 (one v_exp_f32, the factor folded into the scale of rho); the
+  // reference's `power > 0` rejection cannot fire for a sum of squares and is not evaluated.
+#pragma clang fp contract(off)
+  const float p0 = fmaf(h.a[0], pxf, fmaf(h.a[1], pyf, h.a[2]));
+  const float p1 = fmaf(h.a[3], pxf, fmaf(h.a[4], pyf, h.a[5]));
+  o.pz           = fmaf(h.a[6], pxf, fmaf(h.a[7], pyf, h.a[8]));
   const float rz = __builtin_amdgcn_rcpf(o.pz);
   o.sx = p0 * rz, o.sy = p1 * rz;
-  o.rho3d = o.sx * o.sx + o.sy * o.sy;
+  o.rho3d = fmaf(o.sx, o.sx, o.sy * o.sy);
   o.dx = h.cx - pxf, o.dy = h.cy - pyf;
-  o.rho2d = 2.0f * (o.dx * o.dx + o.dy * o.dy);
-  const float rho = fminf(o.rho3d, o.rho2d);
-  o.depth = (o.sx * h.tw0 + o.sy * h.tw1) + h.tw2;
-  const float power = -0.5f * rho;
-  o.G     = __expf(power);
+  const float d2 = fmaf(o.dx, o.dx, o.dy * o.dy);
+  o.rho2d = 2.0f * d2;
+  o.depth = fmaf(o.sx, h.tw0, fmaf(o.sy, h.tw1, h.tw2));
+  const float power2 = fmaxf(o.rho3d * -0.72134752044448170368f, d2 * -1.44269504088896340736f);
+  o.G     = __builtin_amdgcn_exp2f(power2);
   o.alpha = fminf(0.99f, h.opacity * o.G);
-  const bool c0 = o.pz != 0.0f, c1 = !(o.depth < near_n), c2 = !(power > 0.0f), c3 = !(o.alpha < (1.0f / 255.0f));
-  if (lanes) *lanes = wave_ballot(c0) & wave_ballot(c1) & wave_ballot(c2) & wave_ballot(c3);
-  return c0 & c1 & c2 & c3;
+  const bool c0 = o.pz != 0.0f, c1 = !(o.depth < near_n), c3 = !(o.alpha < (1.0f / 255.0f));
+  if (lanes) *lanes = wave_ballot(c0) & wave_ballot(c1) & wave_ballot(c3);
+  return c0 & c1 & c3;
 }
 
 // Sums 8 per-lane values over each 16-lane row at once: three merge steps inside aligned groups of 8 lanes, one rotate
@@ -243,6 +248,7 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
         }
         // one entry of the wavefront's work list; its records were requested from LDS while the entry before it ran
         auto blend_entry = [&](const FastHot& hot, const SplatCold& cold, int j) {
+#pragma clang fp contract(off)  // two copies of this body exist (alternating registers): both must round alike
           FastHit h;
           unsigned long long pass;
           const bool hit = fast_intersect_flat(hot, pxf, pyf, near_n, h, &pass) && live > 0.0f;
@@ -260,24 +266,25 @@ __global__ void __launch_bounds__(kBlendThreads) fast_blend_forward_kernel(
           if (kAux) {
             const float A = 1.0f - T;
             const float m = far_scale * (1.0f - near_n * __builtin_amdgcn_rcpf(h.depth));
-            dist += (m * m * A + M2 - 2.0f * m * M1) * w;
-            D += h.depth * w;
-            M1 += m * w;
-            M2 += m * m * w;
+            const float mm = m * m;
+            dist = fmaf(fmaf(mm, A, fmaf(-2.0f * m, M1, M2)), w, dist);
+            D    = fmaf(h.depth, w, D);
+            M1   = fmaf(m, w, M1);
+            M2   = fmaf(mm, w, M2);
             if (T > 0.5f) median = h.depth, median_c = contributor;
-            N0 += cold.nx * w, N1 += cold.ny * w, N2 += cold.nz * w;
+            N0 = fmaf(cold.nx, w, N0), N1 = fmaf(cold.ny, w, N1), N2 = fmaf(cold.nz, w, N2);
             if (kAccum) argmax_run_step(argmax, w, cold.id, accum_max_count);
             if (kFlow) {
               const float* Q = &s_t2[j * 9];
-              const float u2 = Q[0] * h.sx + Q[1] * h.sy + Q[2];
-              const float v2 = Q[3] * h.sx + Q[4] * h.sy + Q[5];
-              float w2       = Q[6] * h.sx + Q[7] * h.sy + Q[8];
+              const float u2 = fmaf(Q[0], h.sx, fmaf(Q[1], h.sy, Q[2]));
+              const float v2 = fmaf(Q[3], h.sx, fmaf(Q[4], h.sy, Q[5]));
+              float w2       = fmaf(Q[6], h.sx, fmaf(Q[7], h.sy, Q[8]));
               w2             = fabsf(w2) < 1e-5f ? 1e-5f : w2;
-              f0 += (u2 / w2 - pxf) * w;
-              f1 += (v2 / w2 - pyf) * w;
+              f0 = fmaf(u2 / w2 - pxf, w, f0);
+              f1 = fmaf(v2 / w2 - pyf, w, f1);
             }
           }
-          C0 += cold.r * w, C1 += cold.g * w, C2 += cold.b * w;
+          C0 = fmaf(cold.r, w, C0), C1 = fmaf(cold.g, w, C1), C2 = fmaf(cold.b, w, C2);
           T    = test_T;
           last = contributor;
         };
@@ -572,9 +579,10 @@ __global__ void __launch_bounds__(kBlendThreads)
       const float up_x = from_owner(dLp0), up_y = from_owner(dLp1), up_z = from_owner(dLp2);
       const float fx = qx0 + (float) (qp & 7), fy = qy0 + (float) (qp >> 3);
       const float w = it.x, GdA = it.y, dL_dz = it.z;
-      const float p0 = hot.a[0] * fx + hot.a[1] * fy + hot.a[2];
-      const float p1 = hot.a[3] * fx + hot.a[4] * fy + hot.a[5];
-      const float pz = hot.a[6] * fx + hot.a[7] * fy + hot.a[8];
+      // the same fused forms as the per-pixel test: for a surfel seen edge-on p_z is a small difference of large terms
+      const float p0 = fmaf(hot.a[0], fx, fmaf(hot.a[1], fy, hot.a[2]));
+      const float p1 = fmaf(hot.a[3], fx, fmaf(hot.a[4], fy, hot.a[5]));
+      const float pz = fmaf(hot.a[6], fx, fmaf(hot.a[7], fy, hot.a[8]));
       const float rz_s = blends ? __builtin_amdgcn_rcpf(pz) : 0.0f;  // s is used by both cases of a blending pair
       const float rz_p = by_ray ? rz_s : 0.0f;                        // d/dp only by the intersection case
       const float sx = p0 * rz_s, sy = p1 * rz_s;
