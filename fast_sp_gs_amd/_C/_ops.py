@@ -560,7 +560,7 @@ def gs_2d_fast_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: boo
     R = ctypes.c_int64.from_address(count.data_ptr()).value
     point_list = torch.empty((R,), dtype=torch.int32, device=dev)
     keys = torch.empty((R,), dtype=torch.int64, device=dev) if return_keys else None
-    ws2 = _workspace(lib.fsgs_gs_prepare_fill_workspace_bytes(R), dev)
+    ws2 = _workspace(lib.fsgs_gs_2d_fast_prepare_fill_workspace_bytes(P, W, H, R), dev)
     with _timed('gs_2d_fast_prepare_fill'):
         rc = lib.fsgs_gs_2d_fast_prepare_fill(P, W, H, L.ptr(means2D_), L.ptr(inverse_m), L.ptr(depths),
                                               L.ptr(opacities), L.ptr(radii), L.ptr(offsets), R, L.ptr(ranges),

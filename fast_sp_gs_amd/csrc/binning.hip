@@ -180,20 +180,34 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(int P, int gx, int gy, i
 // tile_scatter_kernel).
 constexpr int kMaxLdsTiles = 16384;
 
-template <typename Visit>
+// kCorner: only the tiles that pass the fast path's corner test (CornerTest, from the surfel's adjugate and opacity) are
+// visited.
+template <bool kCorner, typename Visit>
 __device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, const float2* __restrict__ means2D,
-                                                  const int32_t* __restrict__ radii, Visit visit) {
+                                                  const int32_t* __restrict__ radii,
+                                                  const float* __restrict__ inverse_m,
+                                                  const float* __restrict__ opacities, Visit visit) {
   const int lane = __lane_id();
   int x0 = 0, y0 = 0, w = 0, h = 0;
+  float IM[kCorner ? 9 : 1], opacity = 1.0f;
+#pragma unroll
+  for (int k = 0; k < (kCorner ? 9 : 1); ++k) IM[k] = 0.0f;
   if (i < P && radii[i] > 0) {
     const float2 c   = means2D[i];
     const TileRect r = tile_rect(c.x, c.y, radii[i], gx, gy);
     x0 = r.x0, y0 = r.y0, w = max(r.x1 - r.x0, 0), h = max(r.y1 - r.y0, 0);
+    if (kCorner) {
+      opacity = opacities[i];
+#pragma unroll
+      for (int k = 0; k < 9; ++k) IM[k] = inverse_m[9 * (size_t) i + k];
+    }
   }
   const int count = w * h;
   if (count > 0 && count <= kCoopThreshold) {
+    const CornerTest ct(IM, opacity);  // unused (and removed) without kCorner
     for (int y = 0; y < h; ++y)
-      for (int x = 0; x < w; ++x) visit((y0 + y) * gx + (x0 + x), i);
+      for (int x = 0; x < w; ++x)
+        if (!kCorner || ct.tile(x0 + x, y0 + y)) visit((y0 + y) * gx + (x0 + x), i);
   }
   unsigned long long big = __ballot(count > kCoopThreshold);
   while (big) {
@@ -201,9 +215,13 @@ __device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, 
     big &= big - 1;
     const int sx0 = __shfl(x0, src, kWave), sy0 = __shfl(y0, src, kWave), sw = __shfl(w, src, kWave);
     const int scount = __shfl(count, src, kWave), sid = __shfl(i, src, kWave);
+    float sIM[kCorner ? 9 : 1];
+#pragma unroll
+    for (int k = 0; k < (kCorner ? 9 : 1); ++k) sIM[k] = kCorner ? __shfl(IM[k], src, kWave) : 0.0f;
+    const CornerTest ct(sIM, kCorner ? __shfl(opacity, src, kWave) : 1.0f);
     for (int e = lane; e < scount; e += kWave) {
       const int y = e / sw, x = e - y * sw;
-      visit((sy0 + y) * gx + (sx0 + x), sid);
+      if (!kCorner || ct.tile(sx0 + x, sy0 + y)) visit((sy0 + y) * gx + (sx0 + x), sid);
     }
   }
 }
@@ -232,8 +250,10 @@ inline BinsLayout bins_layout(int P, int T) {
 // stores (zeros included, so the matrix needs no clearing). No global atomics: device-scope atomics on one address are
 // served one after the other at fabric latency, and with surfels in no spatial order every block touches nearly
 // every tile.
+template <bool kCorner>
 __global__ void __launch_bounds__(1024) tile_hist_kernel(int P, int per_block, int gx, int gy,
-    const float2* __restrict__ means2D, const int32_t* __restrict__ radii, uint32_t* __restrict__ hist) {
+    const float2* __restrict__ means2D, const int32_t* __restrict__ radii, const float* __restrict__ inverse_m,
+    const float* __restrict__ opacities, uint32_t* __restrict__ hist) {
   __shared__ unsigned s_count[kMaxLdsTiles];
   const int T = gx * gy;
   for (int t = threadIdx.x; t < T; t += blockDim.x) s_count[t] = 0u;
@@ -243,7 +263,8 @@ __global__ void __launch_bounds__(1024) tile_hist_kernel(int P, int per_block, i
   const int rounds = (last - first + (int) blockDim.x - 1) / (int) blockDim.x;
   for (int r = 0; r < rounds; ++r) {
     const int i = first + r * blockDim.x + threadIdx.x;
-    for_each_instance(i < last ? i : P, P, gx, gy, means2D, radii, [&](int tile, int) { atomicAdd(&s_count[tile], 1u); });
+    for_each_instance<kCorner>(i < last ? i : P, P, gx, gy, means2D, radii, inverse_m, opacities,
+                               [&](int tile, int) { atomicAdd(&s_count[tile], 1u); });
   }
   __syncthreads();
   uint32_t* row = hist + (size_t) blockIdx.x * T;
@@ -290,9 +311,11 @@ __global__ void __launch_bounds__(kPrefixTiles * kPrefixWaves) tile_prefix_kerne
 
 // Step 3: the walk of step 1 again; a block's cursor of a tile starts at the tile's start plus the instances of the
 // blocks in front of it, so the placement needs no global atomics either.
+template <bool kCorner>
 __global__ void __launch_bounds__(1024) tile_scatter_kernel(int P, int per_block, int gx, int gy, int64_t R,
     const float2* __restrict__ means2D, const float* __restrict__ depths, const int32_t* __restrict__ radii,
-    const uint32_t* __restrict__ hist, const unsigned long long* __restrict__ ranges, uint64_t* __restrict__ entries) {
+    const float* __restrict__ inverse_m, const float* __restrict__ opacities, const uint32_t* __restrict__ hist,
+    const unsigned long long* __restrict__ ranges, uint64_t* __restrict__ entries) {
   __shared__ unsigned s_cursor[kMaxLdsTiles];
   const int T = gx * gy;
   const uint32_t* row = hist + (size_t) blockIdx.x * T;
@@ -302,7 +325,7 @@ __global__ void __launch_bounds__(1024) tile_scatter_kernel(int P, int per_block
   const int rounds = (last - first + (int) blockDim.x - 1) / (int) blockDim.x;
   for (int r = 0; r < rounds; ++r) {
     const int i = first + r * blockDim.x + threadIdx.x;
-    for_each_instance(i < last ? i : P, P, gx, gy, means2D, radii, [&](int tile, int id) {
+    for_each_instance<kCorner>(i < last ? i : P, P, gx, gy, means2D, radii, inverse_m, opacities, [&](int tile, int id) {
       const unsigned pos = atomicAdd(&s_cursor[tile], 1u);
       if ((int64_t) pos < R) entries[pos] = ((uint64_t) __float_as_uint(depths[id]) << 32) | (uint32_t) id;
     });
@@ -340,7 +363,7 @@ __global__ void __launch_bounds__(1024) tile_scan_kernel(int T, unsigned long lo
     }
     carry += total;
   }
-  if (threadIdx.x == 0) *large_count = 0;
+  if (threadIdx.x == 0) large_count[0] = 0, large_count[1] = (int) carry;  // queue length | instances in all tiles
 }
 
 // Where element i of a segment sits in LDS. With kPad one slot in five stays empty: the rounds of the sorting network
@@ -683,6 +706,18 @@ __global__ void __launch_bounds__(256) tile_ranges_kernel(int64_t R, int num_til
   if (i == R - 1 && cur_ok) ranges[2 * (size_t) cur + 1] = R;
 }
 
+// The fast path reserves one list position per tile of a surfel's rectangle; the positions behind the instances that
+// pass the corner test hold the reference's padding entries (key = T << 32, value = -1), which its sort leaves at the
+// tail of the list.
+__global__ void __launch_bounds__(256) pad_tail_kernel(int64_t R, const int* __restrict__ kept, uint64_t pad_key,
+                                                       int32_t* __restrict__ point_list, int64_t* __restrict__ keys_out) {
+  const int64_t o = (int64_t) *kept + (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+  if (o < R) {
+    point_list[o] = -1;
+    if (keys_out) keys_out[o] = (int64_t) pad_key;
+  }
+}
+
 }  // namespace
 
 uint32_t higher_msb(uint32_t n) {  // number of bits needed for the tile id, as gaussian_prepare.cu:32-44 computes it
@@ -756,6 +791,42 @@ void launch_zero_ranges(int num_tiles, int64_t* ranges, hipStream_t s) {
 }
 void launch_tile_ranges(int64_t R, int num_tiles, const uint64_t* sorted_keys, int64_t* ranges, hipStream_t s) {
   hipLaunchKernelGGL(tile_ranges_kernel, dim3(div_up(R, 256)), dim3(256), 0, s, R, num_tiles, sorted_keys, ranges);
+}
+
+size_t fast_bucket_bins_bytes(int P, int W, int H) {
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const BinsLayout bl = bins_layout(P, gx * gy);
+  return bl.blocks > 0 ? bl.bytes : 0;
+}
+
+int fast_bucket_fill(int P, int W, int H, const float* means2D, const float* inverse_m, const float* depths,
+                     const float* opacities, const int32_t* radii, int64_t R, int64_t* ranges, int32_t* point_list,
+                     int64_t* sorted_keys_out, void* workspace, void* bins, hipStream_t s) {
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  const int T  = gx * gy;
+  const BinsLayout bl = bins_layout(P, T);
+  unsigned long long* rng = (unsigned long long*) ranges;
+  int* header      = (int*) bins;  // [0] length of the long-segment queue, [1] instances kept by the corner test
+  uint32_t* hist   = (uint32_t*) ((char*) bins + kBinsHeader);
+  uint64_t* entries = sort_keys_in(R, workspace);
+  int* large_list   = (int*) ((char*) workspace + sort_layout(R).keys1);
+  hipLaunchKernelGGL(tile_hist_kernel<true>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
+                     (const float2*) means2D, radii, inverse_m, opacities, hist);
+  hipLaunchKernelGGL(tile_prefix_kernel, dim3(div_up(T, kPrefixTiles)), dim3(kPrefixTiles * kPrefixWaves), 0, s, T,
+                     bl.blocks, hist, rng);
+  hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, true);
+  const int* order = nullptr;
+  (void) launch_tile_order(gx, gy, ranges, s, &order);  // the blend kernels of this view find it under `ranges`
+  hipLaunchKernelGGL(tile_scatter_kernel<true>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
+                     (const float2*) means2D, depths, radii, inverse_m, opacities, (const uint32_t*) hist, rng, entries);
+  hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
+                     header, large_list, order);
+  hipLaunchKernelGGL(tile_sort_large_kernel, dim3(256), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,
+                     header, large_list);
+  // at most R positions are padding; blocks beyond the tail leave at once
+  hipLaunchKernelGGL(pad_tail_kernel, dim3(div_up(R, 256)), dim3(256), 0, s, R, header + 1, (uint64_t) (uint32_t) T << 32,
+                     point_list, sorted_keys_out);
+  return check_launch("gs_2d_fast_prepare_fill");
 }
 
 }  // namespace fsgs
@@ -843,8 +914,8 @@ int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, 
   const BinsLayout bl = bins_layout(P, T);
   if (bl.blocks > 0) {
     uint32_t* hist = (uint32_t*) ((char*) bins + kBinsHeader);
-    hipLaunchKernelGGL(tile_hist_kernel, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
-                       (const float2*) means2D, radii, hist);
+    hipLaunchKernelGGL(tile_hist_kernel<false>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
+                       (const float2*) means2D, radii, (const float*) nullptr, (const float*) nullptr, hist);
     hipLaunchKernelGGL(tile_prefix_kernel, dim3(div_up(T, kPrefixTiles)), dim3(kPrefixTiles * kPrefixWaves), 0, s, T,
                        bl.blocks, hist, rng);
     hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, true);
@@ -878,9 +949,9 @@ int fill_sort(int P, int W, int H, const float* means2D, const float* depths, co
   int* large_list = (int*) ((char*) workspace + sort_layout(R).keys1);
   const BinsLayout bl = bins_layout(P, T);
   if (bl.blocks > 0)
-    hipLaunchKernelGGL(tile_scatter_kernel, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
-                       (const float2*) means2D, depths, radii, (const uint32_t*) ((const char*) bins + kBinsHeader), rng,
-                       entries);
+    hipLaunchKernelGGL(tile_scatter_kernel<false>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
+                       (const float2*) means2D, depths, radii, (const float*) nullptr, (const float*) nullptr,
+                       (const uint32_t*) ((const char*) bins + kBinsHeader), rng, entries);
   else
     hipLaunchKernelGGL(tile_emit_kernel<true>, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
                        (const float2*) means2D, depths, radii, rng, entries);

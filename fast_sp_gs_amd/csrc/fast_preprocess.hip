@@ -208,28 +208,6 @@ __global__ void __launch_bounds__(256) fast_preprocess_forward_kernel(
   normal_opacity[i] = ok ? make_float4(nrm[0], nrm[1], nrm[2], opacities[i]) : make_float4(0, 0, 0, 0);
 }
 
-// Implicit conic of the alpha >= 1/255 region, evaluated at tile corners in tile units (gs_2d_fast_preprocess.cu:277-304).
-struct CornerTest {
-  float Wxx, Wyy, Wxy, Wx_, Wy_, W__;
-  __device__ __forceinline__ CornerTest(const float* IM, float opacity) {
-    const float d = -2.0f * 0.69314718055f * (7.9886846867721655f + (float) log2((double) opacity));
-    Wxx = IM[0] * IM[0] + IM[3] * IM[3] + d * IM[6] * IM[6];
-    Wyy = IM[1] * IM[1] + IM[4] * IM[4] + d * IM[7] * IM[7];
-    W__ = IM[2] * IM[2] + IM[5] * IM[5] + d * IM[8] * IM[8];
-    Wxy = 2 * (IM[0] * IM[1] + IM[3] * IM[4] + d * IM[6] * IM[7]);
-    Wx_ = 2 * (IM[0] * IM[2] + IM[3] * IM[5] + d * IM[6] * IM[8]);
-    Wy_ = 2 * (IM[1] * IM[2] + IM[4] * IM[5] + d * IM[7] * IM[8]);
-    Wxx = Wxx * 16 * 16, Wyy = Wyy * 16 * 16, Wxy = Wxy * 16 * 16, Wx_ = Wx_ * 16, Wy_ = Wy_ * 16;
-  }
-  __device__ __forceinline__ bool at(float u, float v) const {
-    return Wxx * u * u + Wyy * v * v + Wxy * u * v + Wx_ * u + Wy_ * v + W__ <= 0;
-  }
-  __device__ __forceinline__ bool tile(int x, int y) const {
-    return at((float) x, (float) y) || at((float) (x + 1), (float) y) || at((float) x, (float) (y + 1)) ||
-           at((float) (x + 1), (float) (y + 1));
-  }
-};
-
 constexpr int kCoopThreshold = 32;
 
 __global__ void __launch_bounds__(256) fast_duplicate_keys_kernel(int P, int gx, int gy, int64_t R,
@@ -492,6 +470,10 @@ FSGS_API int fsgs_gs_2d_fast_prepare_sort_bits(int W, int H) {
   return 32 + (int) higher_msb((uint32_t) (gx * gy) + 1u);
 }
 
+FSGS_API size_t fsgs_gs_2d_fast_prepare_fill_workspace_bytes(int P, int W, int H, int64_t R) {
+  return align_up(sort_workspace_bytes(R), 256) + fast_bucket_bins_bytes(P, W, H);
+}
+
 FSGS_API int fsgs_gs_2d_fast_prepare_fill(int P, int W, int H, const float* means2D, const float* inverse_m,
     const float* depths, const float* opacities, const int32_t* radii, const int64_t* point_offsets, int64_t R,
     int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out, void* workspace, size_t workspace_bytes,
@@ -510,6 +492,14 @@ FSGS_API int fsgs_gs_2d_fast_prepare_fill(int P, int W, int H, const float* mean
   if (workspace_bytes < sort_workspace_bytes(R))
     return fail(kWorkspaceSmall, "gs_2d_fast_prepare_fill: workspace %zu < %zu bytes", workspace_bytes,
                 sort_workspace_bytes(R));
+  // With room for the per-tile counters behind the sort buffers (fsgs_gs_2d_fast_prepare_fill_workspace_bytes) the kept
+  // instances are counted, scattered and sorted per tile, as on the standard path; the same lists, keys and ranges come
+  // out of the device-wide sort of the padded key array below, which serves tile grids too large for that scheme and
+  // callers that size the workspace for the sort alone.
+  const size_t bins_at = align_up(sort_workspace_bytes(R), 256), bins_bytes = fast_bucket_bins_bytes(P, W, H);
+  if (bins_bytes > 0 && workspace_bytes >= bins_at + bins_bytes)
+    return fast_bucket_fill(P, W, H, means2D, inverse_m, depths, opacities, radii, R, ranges, point_list,
+                            sorted_keys_out, workspace, (char*) workspace + bins_at, s);
   const int bits = fsgs_gs_2d_fast_prepare_sort_bits(W, H);
   hipLaunchKernelGGL(fast_duplicate_keys_kernel, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
                      (const float2*) means2D, inverse_m, depths, opacities, radii, point_offsets,

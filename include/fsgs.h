@@ -162,9 +162,13 @@ int fsgs_gs_2d_fast_preprocess_forward(int P, int W, int H, int sh_degree, int n
 
 /* Binning half of gs_2d_fast_preprocess_forward -- gs_2d_fast_preprocess.cu:264-327 (duplicateWithKeys with the
  * per-tile corner test, x-major, unused slots padded with key = T << 32 / value = -1), :711-778 (sort on
- * 32 + msb(T + 1) bits, ranges). The prefix scan is fsgs_gs_prepare_scan; workspace size is
- * fsgs_gs_prepare_fill_workspace_bytes(R). point_list[R] keeps the -1 padding entries at its tail. */
+ * 32 + msb(T + 1) bits, ranges). The prefix scan is fsgs_gs_prepare_scan. point_list[R] keeps the -1 padding entries
+ * at its tail. Workspace: fsgs_gs_2d_fast_prepare_fill_workspace_bytes(P, W, H, R) (no counterpart in the reference);
+ * with it the kept instances are counted, scattered and sorted per tile and the padding entries are written behind
+ * them -- the same lists, keys and ranges as the reference's device-wide sort of the padded key array, which is what a
+ * workspace of only fsgs_gs_prepare_fill_workspace_bytes(R) bytes (and any grid above 16 384 tiles) still gets. */
 int fsgs_gs_2d_fast_prepare_sort_bits(int W, int H);
+size_t fsgs_gs_2d_fast_prepare_fill_workspace_bytes(int P, int W, int H, int64_t R);
 int fsgs_gs_2d_fast_prepare_fill(int P, int W, int H, const float* means2D, const float* inverse_m,
     const float* depths, const float* opacities, const int32_t* radii, const int64_t* point_offsets, int64_t R,
     int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out, void* workspace, size_t workspace_bytes,
