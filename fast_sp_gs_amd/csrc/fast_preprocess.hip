@@ -291,14 +291,35 @@ __global__ void __launch_bounds__(256) fast_preprocess_backward_kernel(
     float* __restrict__ g_means3D, float2* __restrict__ g_scales, float4* __restrict__ g_rot,
     float* __restrict__ g_opac, float* __restrict__ g_shs, float* __restrict__ g_sh_rest) {
   __shared__ float s_rows[kWave ? kShStageRows * kShStageStride : 1];
-  const int i    = blockIdx.x * blockDim.x + threadIdx.x;
-  const bool vis = i < P && radii[i] > 0;
+  const int i      = blockIdx.x * blockDim.x + threadIdx.x;
+  const bool valid = i < P;
+  const bool vis   = valid && radii[i] > 0;
   const int wave_base = blockIdx.x * blockDim.x + (threadIdx.x & ~63);
   float* s_wave_rows  = &s_rows[kWave ? (threadIdx.x & ~63) * kShStageStride : 0];
   float* my_row       = &s_rows[kWave ? threadIdx.x * kShStageStride : 0];
+  // Rows of surfels that were not rendered get explicit zeros, so the outputs need no initialisation (the reference
+  // leaves them to the caller's zero fill; a caller that zero-fills gets the same result).
+  auto zero_geometry = [&]() {
+    g_opac[i] = 0.0f;
+    g_means3D[3 * (size_t) i] = 0.0f, g_means3D[3 * (size_t) i + 1] = 0.0f, g_means3D[3 * (size_t) i + 2] = 0.0f;
+    g_scales[i] = make_float2(0.0f, 0.0f);
+    g_rot[i]    = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  };
   if (kWave) {
     const unsigned long long wanted = __ballot(vis);
-    if (wanted == 0ull) return;  // rows nobody rendered keep the caller's zeros
+    if (wanted == 0ull) {  // nothing of this wavefront was rendered: its gradient rows are zeros
+      if (wave_base < P) {
+#pragma unroll
+        for (int k = 0; k < kShWavePieces; ++k) {
+          int r, c4;
+          wave_piece(k, r, c4);
+          if (wave_base + r < P)
+            ((float4*) g_shs)[(size_t) (wave_base + r) * kShWavePieces + c4] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+      }
+      if (valid) zero_geometry();
+      return;
+    }
     ShWaveRows sh_regs;
     wave_fetch_sh_rows(sh_regs, wanted, wave_base, (const float4*) shs);
     wave_rows_to_lds(sh_regs, s_wave_rows);
@@ -306,8 +327,19 @@ __global__ void __launch_bounds__(256) fast_preprocess_backward_kernel(
     if (!vis) {
 #pragma unroll
       for (int c = 0; c < kShStageFloats; ++c) my_row[c] = 0.0f;
+      if (valid) zero_geometry();
     }
   } else if (!vis) {
+    if (valid) {
+      zero_geometry();
+      if (sh_degree >= 0) {
+        const int m1 = sh_rest ? 1 : n_sh;
+        if (g_shs)
+          for (int c = 0; c < m1 * 3; ++c) g_shs[(size_t) i * m1 * 3 + c] = 0.0f;
+        if (g_sh_rest)
+          for (int c = 0; c < n_sh * 3; ++c) g_sh_rest[(size_t) i * n_sh * 3 + c] = 0.0f;
+      }
+    }
     return;
   }
   if (vis) {

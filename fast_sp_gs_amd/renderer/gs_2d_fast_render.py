@@ -15,6 +15,20 @@ __all__ = ['GS_2D_fast_render', 'GS_2D_fast_preprocess', 'GS_2D_fast_rasterize',
            'fast_compuate_transmat', 'fast_render_step']
 
 
+def _grad_buffers(means3D, scales, rotations, opacities, shs_or_colors, shs_rest, sh_degree, want_shs, want_rest):
+    """Outputs of gs_2d_fast_preprocess_backward. The kernel writes every row of the geometry gradients (zeros for
+    surfels that were not rendered) and, when every stored coefficient is active, of the SH gradient, so those are
+    allocated uninitialised; anything else starts from zeros, as the reference's wrapper has it."""
+    full_sh = (sh_degree >= 0 and shs_rest is None and shs_or_colors is not None
+               and shs_or_colors.shape[1] == (sh_degree + 1) ** 2)
+    g_shs = None
+    if want_shs and shs_or_colors is not None:
+        g_shs = torch.empty_like(shs_or_colors) if full_sh else torch.zeros_like(shs_or_colors)
+    g_rest = torch.zeros_like(shs_rest) if shs_rest is not None and want_rest else None
+    return (torch.empty_like(means3D), torch.empty_like(scales), torch.empty_like(rotations),
+            torch.empty_like(opacities), g_shs, g_rest)
+
+
 class _fast_preprocess(torch.autograd.Function):
     _forward_func = get_C_function('gs_2d_fast_preprocess_forward')
     _backward_func = get_C_function('gs_2d_fast_preprocess_backward')
@@ -45,10 +59,8 @@ class _fast_preprocess(torch.autograd.Function):
         grad_normal_opacity = z(grad_normal_opacity, normal_opacity)
         grad_inputs = [
             None, None, None, None,
-            torch.zeros_like(means3D), torch.zeros_like(scales), torch.zeros_like(rotations),
-            torch.zeros_like(opacities),
-            torch.zeros_like(shs_or_colors) if shs_or_colors is not None and ctx.needs_input_grad[8] else None,
-            torch.zeros_like(shs_rest) if shs_rest is not None and ctx.needs_input_grad[9] else None,
+            *_grad_buffers(means3D, scales, rotations, opacities, shs_or_colors, shs_rest, sh_degree,
+                           ctx.needs_input_grad[8], ctx.needs_input_grad[9]),
             None, None, None, None, None, None, None,
         ]
         _fast_preprocess._backward_func(
@@ -213,10 +225,8 @@ class _Fast_Render(torch.autograd.Function):
             pixel_extras, pixel_flow, grad_images, grad_opacity, grad_others, grad_flow, tile_range, point_list,
             n_contrib, near_n, far_n, None, None, None, None, None, None, point_offsets, radii)
         grad_inputs = [
-            torch.zeros_like(means3D), torch.zeros_like(scales), torch.zeros_like(rotations),
-            torch.zeros_like(opacities),
-            torch.zeros_like(shs_or_colors) if ctx.needs_input_grad[4] else None,
-            torch.zeros_like(shs_rest) if shs_rest is not None and ctx.needs_input_grad[5] else None,
+            *_grad_buffers(means3D, scales, rotations, opacities, shs_or_colors, shs_rest, sh_degree,
+                           ctx.needs_input_grad[4], ctx.needs_input_grad[5]),
             None, None, None, None,
             None, None, None, None, None, None,
             None, grad_means2D, None,
@@ -315,9 +325,10 @@ def fast_render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None,
         point_offsets if ordered_sums else None, radii if ordered_sums else None,
         per_splat_kernel=bool(per_splat and per_splat_kernel))
     g_means2D_in = g_means2D.clone()
-    g = dict(means3D=torch.zeros_like(scene.means3D), scales=torch.zeros_like(scene.scales),
-             rotations=torch.zeros_like(scene.rotations), opacities=torch.zeros_like(scene.opacities),
-             shs=torch.zeros_like(scene.shs))
+    # the preprocess backward writes every row of its outputs (zeros for surfels that were not rendered)
+    g = dict(means3D=torch.empty_like(scene.means3D), scales=torch.empty_like(scene.scales),
+             rotations=torch.empty_like(scene.rotations), opacities=torch.empty_like(scene.opacities),
+             shs=torch.empty_like(scene.shs))
     pre_b(W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs, None,
           cam.Tw2v, cam.Tv2s, cam.campos, trans_mat, radii, colors, normal_opacity, g_means2D, g_trans, g_inv, None,
           g_colors, g_no, g['means3D'], g['scales'], g['rotations'], g['opacities'], g['shs'], None)

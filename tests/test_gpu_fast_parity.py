@@ -266,6 +266,53 @@ def test_fast_per_splat_kernel(name, ordered, device):
             assert torch.equal(again[k], splat[k]), k
 
 
+@pytest.mark.parametrize("layout", ["full", "split", "wide"])
+def test_fast_preprocess_backward_assigns_every_row(layout, device):
+    """gs_2d_fast_preprocess_backward writes every row of its geometry gradients and of a fully active SH gradient
+    (zeros for surfels that were not rendered): outputs poisoned with NaN come out equal to outputs that started from
+    zeros. With unused higher coefficients ("wide") or a split DC / rest layout the wrapper still starts from zeros."""
+    from fast_sp_gs_amd._C import get_C_function as f
+    from fast_sp_gs_amd.renderer import fast_render_step
+    from fast_sp_gs_amd.renderer.gs_2d_fast_render import _grad_buffers
+    scene, cam, gi, ge, go = _make("partial_tiles_511x127")
+    sc, cm = scene.to(device), cam.to(device)
+    out = fast_render_step(sc, cm, gi.to(device), ge.to(device), go.to(device))
+    hidden = out['radii'] <= 0
+    assert 0 < int(hidden.sum()) < scene.P
+    shs, rest, degree = sc.shs, None, 3
+    if layout == "split":
+        shs, rest = sc.shs[:, :1].contiguous(), sc.shs[:, 1:].contiguous()
+    elif layout == "wide":
+        degree = 2
+    W, H = cam.W, cam.H
+
+    def run(poison):
+        bufs = list(_grad_buffers(sc.means3D, sc.scales, sc.rotations, sc.opacities, shs, rest, degree, True, True))
+        expect_assigned = [True, True, True, True, layout == "full", False]
+        for b, assigned in zip(bufs, expect_assigned):
+            if b is None:
+                continue
+            if poison and assigned:
+                b.fill_(float('nan'))
+            elif not assigned:
+                assert not b.any()  # the wrapper's own zeros
+        gm2 = out['g_means2D_blend'].clone()
+        f('gs_2d_fast_preprocess_backward')(
+            W, H, degree, False, sc.means3D, sc.scales, sc.rotations, sc.opacities, shs, rest, cm.Tw2v, cm.Tv2s,
+            cm.campos, out['trans_mat'], out['radii'], out['colors'], out['normal_opacity'], gm2, out['g_trans'],
+            out['g_inv'], None, out['g_colors'], out['g_normal_opacity'], *bufs)
+        return bufs
+
+    a, b = run(False), run(True)
+    torch.cuda.synchronize()
+    for x, y in zip(a, b):
+        if x is None:
+            continue
+        assert bool(torch.isfinite(y).all())
+        assert torch.equal(x, y)
+        assert not y[hidden].any()
+
+
 def test_fast_empty_scene(device):
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd.renderer import fast_render_step
