@@ -685,11 +685,12 @@ def GS_2D_fast_render_forward(width: int, height: int, near_n: float, far_n: flo
         L.require_shape(what, 'trans_mat_t2', trans_mat_t2, P, 3, 3)
     dev = colors.device
     opt = dict(dtype=torch.float32, device=dev)
-    pixel_colors = torch.zeros((3, height, width), **opt)
-    pixel_opacity = torch.zeros((height, width), **opt)
-    n_contrib = torch.zeros((2, height, width), dtype=torch.int32, device=dev)
-    pixel_extras = None if only_image else torch.zeros((8, height, width), **opt)
-    pixel_flow = torch.zeros((height, width, 2), **opt) if flow else None
+    # one block per tile writes every pixel of every output, empty tiles included
+    pixel_colors = torch.empty((3, height, width), **opt)
+    pixel_opacity = torch.empty((height, width), **opt)
+    n_contrib = torch.empty((2, height, width), dtype=torch.int32, device=dev)
+    pixel_extras = None if only_image else torch.empty((8, height, width), **opt)
+    pixel_flow = torch.empty((height, width, 2), **opt) if flow else None
     outputs = [pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib]
     max_contrib = bucket_to_tile = sampled_T = sampled_acc = sampled_aux = None
     fast_bwd = per_tile_bucket_offset is not None

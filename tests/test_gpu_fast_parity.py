@@ -313,6 +313,31 @@ def test_fast_preprocess_backward_assigns_every_row(layout, device):
         assert not y[hidden].any()
 
 
+@pytest.mark.parametrize("name", ["partial_tiles_511x127", "tiny_3_surfels"])
+def test_fast_forward_writes_every_pixel(name, device):
+    """The forward's outputs are allocated uninitialised: every pixel of every map is written by the tile's block, empty
+    tiles and partial tiles included. The allocator's free blocks are poisoned with NaN / a large count first; the
+    second call must reproduce the first bit for bit and hold no NaN."""
+    from fast_sp_gs_amd.renderer import fast_render_step
+    scene, cam, gi, ge, go = _make(name)
+    args = (scene.to(device), cam.to(device), gi.to(device), ge.to(device), go.to(device))
+    first = fast_render_step(*args, per_splat=True)
+    keep = {k: first[k].clone() for k in ('image', 'opacity', 'extras', 'n_contrib')}
+    del first
+    H, W = cam.H, cam.W
+    poison = [torch.full((3, H, W), float('nan'), device=device), torch.full((H, W), float('nan'), device=device),
+              torch.full((8, H, W), float('nan'), device=device),
+              torch.full((2, H, W), 1 << 30, dtype=torch.int32, device=device)]
+    torch.cuda.synchronize()
+    del poison
+    again = fast_render_step(*args, per_splat=True)
+    torch.cuda.synchronize()
+    for k, v in keep.items():
+        assert bool(torch.isfinite(again[k].float()).all()), k
+        assert torch.equal(again[k], v), k
+    assert int(again['n_contrib'].max()) < 1 << 30
+
+
 def test_fast_empty_scene(device):
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd.renderer import fast_render_step
