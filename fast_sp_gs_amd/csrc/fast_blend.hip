@@ -18,6 +18,7 @@
 // LDS (64-byte hot record with the adjugate, 32-byte cold record), per-quadrant work lists from a conservative bound;
 // the backward queues its blended (pixel, entry) pairs and forms their gradient components 64 pairs at a time
 // (pair_queue.hpp).
+#include "binning.hpp"
 #include "blend.hpp"
 #include "ordered_sums.hpp"
 #include "pair_queue.hpp"
@@ -372,6 +373,60 @@ struct FastScatter {
   }
 };
 
+// Sum of a surfel's records on the fast path. Its key span holds one position per tile of its rectangle, x-major, but
+// only the tiles that pass the binning's corner test are in a tile list, and only those positions were written by the
+// blend (a list entry's record by the flush of its batch, or zeros by its tile's block if the entry lies behind the
+// deepest contributor). The test is repeated here, with the binning's own arithmetic, so the other positions are
+// neither cleared nor read. 11 lanes per surfel, each owning one float2 of the 88-byte record: a step covers 11
+// positions of the span -- lane k tests position base + k, the 11 verdicts are shared through a ballot, and the
+// records of the positions that passed are requested together.
+__global__ void __launch_bounds__(256) fast_slot_sum_kernel(int P, int gx, int gy,
+    const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii, const float2* __restrict__ means2D,
+    const float* __restrict__ inverse_m, const float4* __restrict__ normal_opacity,
+    const float* __restrict__ records, FastScatter out) {
+  constexpr int kLanes = kFastRecordSlots / 2, kPerWave = 64 / kLanes;
+  const int lane = threadIdx.x & 63;
+  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int sub = lane / kLanes, k = lane - sub * kLanes;
+  const int i = wave * kPerWave + sub;
+  const bool active = sub < kPerWave && i < P;
+  const int radius = active ? radii[i] : 0;
+  int count = 0, h = 1, x0 = 0, y0 = 0;
+  float IM[9], opacity = 1.0f;
+#pragma unroll
+  for (int q = 0; q < 9; ++q) IM[q] = 0.0f;
+  const float2* src = (const float2*) records;
+  if (radius > 0) {
+    const float2 c   = means2D[i];
+    const TileRect r = tile_rect(c.x, c.y, radius, gx, gy);
+    h = max(r.y1 - r.y0, 1), count = max(r.x1 - r.x0, 0) * max(r.y1 - r.y0, 0), x0 = r.x0, y0 = r.y0;
+#pragma unroll
+    for (int q = 0; q < 9; ++q) IM[q] = inverse_m[9 * (size_t) i + q];
+    opacity = normal_opacity[i].w;
+    src += (size_t) (i > 0 ? point_offsets[i - 1] : 0) * kLanes + k;
+  }
+  const CornerTest ct(IM, opacity);
+  float2 acc = make_float2(0.0f, 0.0f);
+  // the wavefront's surfels step together (the ballot needs every lane): as many steps as its largest rectangle asks
+  int steps = (count + kLanes - 1) / kLanes;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) steps = max(steps, __shfl_xor(steps, d, kWave));
+  for (int st = 0; st < steps; ++st) {
+    const int base = st * kLanes, p = base + k, x = p / h, y = p - x * h;  // x-major over the rectangle
+    const bool on = p < count && ct.tile(x0 + x, y0 + y);
+    const unsigned bits = (unsigned) (wave_ballot(on) >> (sub * kLanes)) & ((1u << kLanes) - 1u);
+    float2 v[kLanes];
+#pragma unroll
+    for (int j = 0; j < kLanes; ++j)
+      v[j] = ((bits >> j) & 1u) ? src[(size_t) (base + j) * kLanes] : make_float2(0.0f, 0.0f);
+#pragma unroll
+    for (int j = 0; j < kLanes; ++j) acc.x += v[j].x, acc.y += v[j].y;
+  }
+  if (!active) return;
+  out(i, 2 * k, acc.x);
+  out(i, 2 * k + 1, acc.y);
+}
+
 // kSlots: the per-surfel sums go through per-instance records (ordered_sums.hpp) instead of device-scope atomics.
 template <bool kAux, bool kPerSplat, bool kFlow, bool kSlots>
 // Four blocks per compute unit where the per-surfel sums go through records (the flush of the other form keeps more
@@ -430,6 +485,19 @@ __global__ void __launch_bounds__(kBlendThreads)
   __syncthreads();
   const int n_todo = min(s_max_contrib, (int) (r1 - r0));
   const int rounds = (n_todo + kB - 1) / kB;
+  // No zero fill of the record buffer: every staged instance writes its record at the flush, zeros included, and the
+  // instances behind the tile's deepest contributor, which are never staged, are cleared here.
+  if (kSlots) {
+    for (int e = n_todo + (int) threadIdx.x; e < (int) (r1 - r0); e += kBlendThreads) {
+      const int id = point_list[r0 + e];
+      const float2 c = means2D[id];
+      const TileRect r = tile_rect(c.x, c.y, radii[id], gx, gy);
+      const int64_t at = (id == 0 ? 0 : point_offsets[id - 1]) + (int64_t) (tile_x - r.x0) * (r.y1 - r.y0) + (tile_y - r.y0);
+      float2* dst = (float2*) (slot_records + (size_t) at * kFastRecordSlots);
+#pragma unroll
+      for (int c2 = 0; c2 < kFastRecordSlots / 2; ++c2) dst[c2] = make_float2(0.0f, 0.0f);
+    }
+  }
 
   const float T_final = inside ? 1.0f - out_opacity[pix] : 0.0f;
   float T = T_final;
@@ -725,15 +793,10 @@ __global__ void __launch_bounds__(kBlendThreads)
         a[c] = sum;
       }
       if (kSlots) {
-        bool any = false;
+        float2* dst = (float2*) (slot_records + slot * kFastRecordSlots);
 #pragma unroll
-        for (int c = 0; c < kFastGradSlots; ++c) any |= a[c] != 0.0f;
-        if (any) {
-          float2* dst = (float2*) (slot_records + slot * kFastRecordSlots);
-#pragma unroll
-          for (int c = 0; c < kFastRecordSlots / 2; ++c)
-            dst[c] = make_float2(a[2 * c], 2 * c + 1 < kFastGradSlots ? a[2 * c + 1] : 0.0f);
-        }
+        for (int c = 0; c < kFastRecordSlots / 2; ++c)
+          dst[c] = make_float2(a[2 * c], 2 * c + 1 < kFastGradSlots ? a[2 * c + 1] : 0.0f);
       } else {
 #pragma unroll
         for (int c = 0; c < 3; ++c)
@@ -906,16 +969,11 @@ __global__ void __launch_bounds__(64) fast_bucket_backward_kernel(int W, int H, 
     g[19] += to_centre * h.dx, g[20] += to_centre * h.dy;
   }
   if (!valid) return;
-  if (kSlots) {
-    bool any = false;
+  if (kSlots) {  // every list entry has a lane in some wavefront of this launch: all records are written, zeros included
+    float2* dst = (float2*) (slot_records + slot * kFastRecordSlots);
 #pragma unroll
-    for (int c = 0; c < kFastGradSlots; ++c) any |= g[c] != 0.0f;
-    if (any) {  // the record buffer is zero-filled
-      float2* dst = (float2*) (slot_records + slot * kFastRecordSlots);
-#pragma unroll
-      for (int c = 0; c < kFastRecordSlots / 2; ++c)
-        dst[c] = make_float2(g[2 * c], 2 * c + 1 < kFastGradSlots ? g[2 * c + 1] : 0.0f);
-    }
+    for (int c = 0; c < kFastRecordSlots / 2; ++c)
+      dst[c] = make_float2(g[2 * c], 2 * c + 1 < kFastGradSlots ? g[2 * c + 1] : 0.0f);
   } else {
     const int id = cold.id;
 #pragma unroll
@@ -934,6 +992,16 @@ __global__ void __launch_bounds__(64) fast_bucket_backward_kernel(int W, int H, 
     for (int c = 0; c < 2; ++c)
       if (g[19 + c] != 0.0f) atomicAdd(&g_means2D[2 * (size_t) id + c], g[19 + c]);
   }
+}
+
+void launch_fast_slot_sum(int P, int gx, int gy, const int64_t* point_offsets, const int32_t* radii,
+                          const float* means2D, const float* inverse_m, const float* normal_opacity,
+                          const SlotWorkspace& ws, FastScatter out, hipStream_t s) {
+  constexpr int kPerWave = 64 / (kFastRecordSlots / 2);
+  const int64_t waves = div_up(P, kPerWave);
+  hipLaunchKernelGGL(fast_slot_sum_kernel, dim3((unsigned) div_up(waves * 64, 256)), dim3(256), 0, s, P, gx, gy,
+                     point_offsets, radii, (const float2*) means2D, inverse_m, (const float4*) normal_opacity,
+                     ws.records, out);
 }
 
 }  // namespace
@@ -1017,7 +1085,6 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const dim3 grid(gx * gy), block(kBlendThreads);
   hipStream_t s = (hipStream_t) stream;
-  if (slots) launch_slot_clear<kFastRecordSlots>(ws, R, s);
   const int* tile_order = nullptr;
   const int ordered = launch_tile_order(gx, gy, ranges, s, &tile_order);
 #define FSGS_LAUNCH_BWD_S(AUX, SPLAT, FLOW, SL)                                                                      \
@@ -1038,8 +1105,8 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
 #undef FSGS_LAUNCH_BWD
 #undef FSGS_LAUNCH_BWD_S
   if (slots)
-    launch_slot_sum<kFastRecordSlots>(P, point_offsets, ws,
-                                      FastScatter{g_means2D, g_normal_opacity, g_colors, g_trans, g_inv}, s);
+    launch_fast_slot_sum(P, gx, gy, point_offsets, radii, means2D, inverse_m, normal_opacity, ws,
+                         FastScatter{g_means2D, g_normal_opacity, g_colors, g_trans, g_inv}, s);
   return check_launch("GS_2D_fast_render_backward");
 }
 
@@ -1076,7 +1143,6 @@ FSGS_API int fsgs_gs_2d_fast_render_bucket_backward(int P, int W, int H, double 
     ws = slot_workspace(workspace, R, kFastRecordSlots);
   }
   hipStream_t s = (hipStream_t) stream;
-  if (slots) launch_slot_clear<kFastRecordSlots>(ws, R, s);
 #define FSGS_FAST_BKT(AUX, SL)                                                                                        \
   hipLaunchKernelGGL((fast_bucket_backward_kernel<AUX, SL>), dim3(B), dim3(64), 0, s, W, H, (float) near_n,           \
                      (float) far_n, ranges, point_list, (const float2*) means2D, (const float4*) normal_opacity,      \
@@ -1092,7 +1158,7 @@ FSGS_API int fsgs_gs_2d_fast_render_bucket_backward(int P, int W, int H, double 
   }
 #undef FSGS_FAST_BKT
   if (slots)
-    launch_slot_sum<kFastRecordSlots>(P, point_offsets, ws,
-                                      FastScatter{g_means2D, g_normal_opacity, g_colors, g_trans, g_inv}, s);
+    launch_fast_slot_sum(P, (W + kTile - 1) / kTile, (H + kTile - 1) / kTile, point_offsets, radii, means2D, inverse_m,
+                         normal_opacity, ws, FastScatter{g_means2D, g_normal_opacity, g_colors, g_trans, g_inv}, s);
   return check_launch("GS_2D_fast_render_bucket_backward");
 }

@@ -1,12 +1,13 @@
 // Per-surfel sums of per-(surfel, tile) gradient records in a fixed order, without atomics and without a zero fill of
 // the outputs. The tile binning emits a surfel's instances at consecutive positions of the unsorted key list, starting at
 // the surfel's prefix-scan offset; a backward block that has summed one instance over its tile's pixels writes the sums
-// as one record at that position. Either every instance's record is written by the blend kernel itself, zeros included
-// (the standard surfel and the 3D-Gaussian blends: each block also clears the records of its tile's never-staged tail),
-// or the record buffer is zero-filled first (launch_slot_clear; the fast path, whose key spans contain padding positions
-// that belong to no tile's list). slot_sum_kernel then adds a surfel's records in position
-// order and hands every component of every surfel to a scatter functor that knows the output tensors. The reference flushes these sums with one device-scope atomic per component,
-// tile and surfel into caller-zeroed tensors (e.g. gaussian_render.cu:560-600, gs_2d_fast_redner.cu:520-560).
+// as one record at that position. Every instance's record is written by the blend kernel itself, zeros included (each
+// block also clears the records of its tile's never-staged tail), so the buffer is never zero-filled. slot_sum_kernel
+// then adds a surfel's records in position order and hands every component of every surfel to a scatter functor that
+// knows the output tensors. (The fast path's key spans also hold positions that belong to no tile's list; its own sum
+// kernel, in fast_blend.hip, repeats the binning's corner test and skips them.) The reference flushes these sums with
+// one device-scope atomic per component, tile and surfel into caller-zeroed tensors (e.g. gaussian_render.cu:560-600,
+// gs_2d_fast_redner.cu:520-560).
 #pragma once
 #include <algorithm>
 
@@ -24,11 +25,6 @@ inline size_t slot_workspace_bytes(int64_t R, int floats) {
 inline SlotWorkspace slot_workspace(void* base, int64_t, int) { return SlotWorkspace{(float*) base}; }
 
 namespace {
-
-__global__ void __launch_bounds__(256) slot_clear_kernel(size_t n4, float4* __restrict__ p) {
-  for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t) gridDim.x * blockDim.x)
-    p[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-}
 
 // kFloats / 2 lanes per surfel, each owning one float2 of the record, so the lanes of a surfel read consecutive bytes
 // and neighbouring surfels continue where the previous one ends. Eight records of a surfel are in flight together.
@@ -57,13 +53,6 @@ __global__ void __launch_bounds__(256) slot_sum_kernel(int P, const int64_t* __r
   }
   out(i, 2 * k, acc.x);
   out(i, 2 * k + 1, acc.y);
-}
-
-template <int kFloats>
-inline void launch_slot_clear(const SlotWorkspace& ws, int64_t R, hipStream_t s) {
-  const size_t n4 = ((size_t) R * kFloats + 3) / 4;
-  const unsigned blocks = (unsigned) std::min<size_t>((n4 + 255) / 256, 8192);
-  if (n4 > 0) hipLaunchKernelGGL(slot_clear_kernel, dim3(blocks), dim3(256), 0, s, n4, (float4*) ws.records);
 }
 
 template <int kFloats, typename Scatter>

@@ -215,7 +215,9 @@ int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, double fa
  * caller (device-scope atomics, as in the reference). With point_offsets[P] (the inclusive prefix scan of tiles_touched
  * that fsgs_gs_prepare_scan returns), radii[P], R = point_offsets[P-1] (the length of point_list, padding included) and
  * a 16-byte aligned workspace of fsgs_gs_2d_fast_render_backward_workspace_bytes(R) bytes (no counterpart in the
- * reference) every row of the outputs is ASSIGNED from per-(surfel, tile) records added in a fixed order. */
+ * reference) every row of the outputs is ASSIGNED from per-(surfel, tile) records added in a fixed order. The
+ * workspace needs no clearing: every list entry's record is written on every call, and the sum repeats the binning's
+ * corner test so that it reads no other position of a surfel's key span. */
 size_t fsgs_gs_2d_fast_render_backward_workspace_bytes(int64_t R);
 int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n, double far_n, int per_splat_form,
     const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,

@@ -120,3 +120,79 @@ def test_backward_workspace_needs_no_clearing(variant, source, device):
     for name, a, b in zip(('colors', 'means2D', 'trans', 'normal_opacity'), zeroed, atomic):
         if np.abs(b).max() > 0:
             assert rel_err(a, b) < 1e-3, name
+
+
+@pytest.mark.parametrize("kernel", ["tile", "per_splat"])
+@pytest.mark.parametrize("variant", ["aux", "image_only"])
+def test_fast_backward_workspace_needs_no_clearing(variant, kernel, device):
+    """The same promise on the fast path, whose key spans hold positions that belong to no tile's list (tiles of the
+    rectangle that fail the corner test): the record sum repeats the binning's test and reads only the positions the
+    blend wrote, so nothing is cleared there either. Both backward kernels (back to front per tile / the per-splat
+    decomposition over 32-entry buckets), with and without the auxiliary maps."""
+    from fast_sp_gs_amd import lib as L, scenes
+    from fast_sp_gs_amd._C import get_C_function as f
+    lib = L.load()
+    W, H, P = 320, 208, 6000
+    g = torch.Generator().manual_seed(3)
+    scene = scenes._surfels(g, P, 'cube', -3.2, 0.4, 3.0, 1.0)
+    scene.means3D[:, 0] = scene.means3D[:, 0] * 0.6 - 0.5
+    cam = scenes.pinhole(W, H, 50.0, torch.tensor([0., 0., 4.]))
+    sc, cm = scene.to(device), cam.to(device)
+    (m2, colors, tm, im, no, depths, radii, ranges, point_list, keys, tt, offsets) = f('gs_2d_fast_preprocess_forward')(
+        W, H, 3, False, sc.means3D, sc.scales, sc.rotations, sc.opacities, sc.shs, None, cm.Tw2v, cm.Tv2c, cm.Tv2s,
+        cm.campos, None, None, None, False, True, True)
+    b_off = torch.cumsum((ranges[:, 1] - ranges[:, 0] + 31) // 32, 0).contiguous()
+    image, oo, oe, _, nc, max_c, b2t, s_T, s_acc, s_aux = f('GS_2D_fast_render_forward')(
+        W, H, cam.near, cam.far, False, m2, colors, no, tm, im, point_list, ranges, None, None, None, None, b_off)[:10]
+    d = dict(W=W, H=H, ranges=ranges)
+    empty, long_, cut = _tile_classes(d, nc)
+    n_pad = int((point_list == -1).sum())
+    print(f"[fast {variant}/{kernel}] tiles: {empty} empty, {long_} longer than 64 entries, {cut} cut before their "
+          f"end; {n_pad} of {point_list.numel()} key positions are padding")
+    assert empty > 0 and long_ > 0 and cut > 0 and n_pad > 0
+    g2 = torch.Generator().manual_seed(9)
+    gi = torch.randn(3, H, W, generator=g2).to(device)
+    ge = torch.randn(8, H, W, generator=g2).to(device)
+    go = torch.randn(H, W, generator=g2).to(device)
+    aux = variant == "aux"
+    R = int(point_list.numel())
+    nbytes = lib.fsgs_gs_2d_fast_render_backward_workspace_bytes(R)
+    B = int(b2t.numel())
+
+    def run(fill, ordered=True):
+        ws = torch.empty(nbytes // 4, device=device)
+        ws.fill_(fill)
+        out = [torch.full((P, n), float('nan'), device=device) if ordered else torch.zeros(P, n, device=device)
+               for n in (3, 2, 9, 9, 4)]  # colours, means2D, transform, adjugate, normal + opacity
+        tail = (R, L.ptr(offsets) if ordered else None, L.ptr(radii) if ordered else None,
+                L.ptr(ws) if ordered else None, nbytes if ordered else 0, L.current_stream())
+        if kernel == "tile":
+            rc = lib.fsgs_gs_2d_fast_render_backward(
+                P, W, H, float(cam.near), float(cam.far), 1, L.ptr(m2), L.ptr(no), L.ptr(colors), L.ptr(tm), L.ptr(im),
+                None, L.ptr(oo), L.ptr(oe) if aux else None, None, L.ptr(gi), L.ptr(go), L.ptr(ge) if aux else None,
+                None, L.ptr(ranges), L.ptr(point_list), L.ptr(nc), L.ptr(out[0]), L.ptr(out[1]), L.ptr(out[2]),
+                L.ptr(out[3]), L.ptr(out[4]), *tail)
+        else:
+            rc = lib.fsgs_gs_2d_fast_render_bucket_backward(
+                P, W, H, float(cam.near), float(cam.far), B, L.ptr(m2), L.ptr(no), L.ptr(colors), L.ptr(tm), L.ptr(im),
+                L.ptr(image), L.ptr(oo), L.ptr(oe) if aux else None, L.ptr(nc), L.ptr(max_c), L.ptr(b_off), L.ptr(b2t),
+                L.ptr(s_T), L.ptr(s_acc), L.ptr(s_aux), L.ptr(gi), L.ptr(go), L.ptr(ge) if aux else None,
+                L.ptr(ranges), L.ptr(point_list), L.ptr(out[0]), L.ptr(out[1]), L.ptr(out[2]), L.ptr(out[3]),
+                L.ptr(out[4]), *tail)
+        L.check(rc, 'fast backward')
+        torch.cuda.synchronize()
+        return [npy(o) for o in out]
+
+    zeroed = run(0.0)
+    for o in zeroed:
+        assert np.isfinite(o).all()
+    for fill in (float('nan'), 3.0e30):
+        poisoned = run(fill)
+        for a, b in zip(poisoned, zeroed):
+            assert np.isfinite(a).all(), fill
+            assert np.array_equal(a, b), fill
+    atomic = run(0.0, ordered=False)
+    for name, a, b in zip(('colors', 'means2D', 'trans', 'inv', 'normal_opacity'), zeroed, atomic):
+        if np.abs(b).max() > 0:
+            assert rel_err(a, b) < 1e-3, name
+    assert np.abs(zeroed[0]).max() > 0 and np.abs(zeroed[3]).max() > 0
