@@ -544,7 +544,7 @@ def large_scene_ms(dev, views: int = 4, reps: int = 3):
 
     def batch():
         for cam in cams:
-            out = render_step(scene, cam, gi, ge, None, background=bg)
+            out = render_step(scene, cam, gi, ge, None, background=bg, cull=True)
         return out
 
     out = batch()
@@ -738,7 +738,7 @@ def main():
         # the fused per-pixel epilogue runs between the two blend passes, as in training: composite on the background,
         # normals to world space, surf_depth, pseudo surface normal; its backward supplies dL/dextras and the
         # composite's dL/dopacity = -sum_c dL/dimage_c * bg_c to the blend backward
-        return render_step(scene, cam, gi, ge, None, background=bg)
+        return render_step(scene, cam, gi, ge, None, background=bg, cull=True)
 
     # The per-stage events of the timed steps are created and recorded once here, outside the timed region: the runtime
     # grows its event pool in bursts that stall the host for tens of milliseconds.

@@ -136,9 +136,10 @@ def gs_2d_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: bool, me
                              rotations: Tensor, opacities: Tensor, shs: Tensor, sh_rest: Optional[Tensor],
                              Tw2v: Tensor, Tv2c: Tensor, cam_pos: Tensor, trans_precomp: Optional[Tensor] = None,
                              means2D: Optional[Tensor] = None, culling: Optional[Tensor] = None,
-                             return_records: bool = False) -> List[Tensor]:
+                             return_records: bool = False, return_masks: bool = False) -> List[Tensor]:
     """gs_2d_preprocess.cu:331-421 -> [means2D, colors, trans_mat, normal_opacity, depths, radii, tiles_touched]
-    (+ records[P,20], the packed per-surfel record of gs_2d_pack_records written by the same kernel, on request)."""
+    (+ records[P,20], the packed per-surfel record of gs_2d_pack_records written by the same kernel, on request;
+    + keep_masks[P] int32, the per-surfel tile masks of the culled binning, GS_prepare(..., cull=True), on request)."""
     what = 'gs_2d_preprocess_forward'
     _f32(what, means3D=means3D, scales=scales, rotations=rotations, opacities=opacities, shs=shs, Tw2v=Tw2v,
          Tv2c=Tv2c, cam_pos=cam_pos)
@@ -185,16 +186,21 @@ def gs_2d_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: bool, me
     tiles_touched = torch.empty((P,), dtype=torch.int32, device=means3D.device)
     normal_opacity = torch.empty((P, 4), **opt)
     records = torch.empty((P, 20), **opt) if return_records else None
+    masks = torch.empty((max(P, 1),), dtype=torch.int32, device=means3D.device) if return_masks else None
     with _timed('gs_2d_preprocess_forward'):
         rc = _lib().fsgs_gs_2d_preprocess_forward(
             P, W, H, sh_degree, M, L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(opacities), L.ptr(shs),
             L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2c), L.ptr(cam_pos), L.ptr(trans_precomp),
             L.ptr(culling), int(preserve), L.ptr(means2D_), None if sh_degree < 0 else L.ptr(colors),
             None if trans_precomp is not None else L.ptr(trans_mat), L.ptr(normal_opacity), L.ptr(depths), L.ptr(radii),
-            L.ptr(tiles_touched), L.ptr(records), L.current_stream())
+            L.ptr(tiles_touched), L.ptr(records), L.ptr(masks), L.current_stream())
     L.check(rc, what)
     out = [means2D_, colors, trans_mat, normal_opacity, depths, radii, tiles_touched]
-    return out + [records] if return_records else out
+    if return_records:
+        out.append(records)
+    if return_masks:
+        out.append(masks)
+    return out
 
 
 def gs_2d_preprocess_backward(W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs, sh_rest,
@@ -275,11 +281,16 @@ def gs_2d_compute_trans_mat_backward(W, H, means3D, scales, rotations, Tw2v, Tw2
 # --------------------------------------------------------------------------------------------------------------------
 def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, tiles_touched: Tensor,
                debug: bool = False, return_keys: bool = False, return_offsets: bool = False,
-               overlap=None, records: Optional[Tensor] = None) -> List[Tensor]:
+               overlap=None, records: Optional[Tensor] = None, cull: bool = False,
+               keep_masks: Optional[Tensor] = None) -> List[Tensor]:
     """gaussian_prepare.cu:282-308 -> [ranges[T,2] int64, point_list[R] int32] (+ sorted keys, + the prefix scan of
     tiles_touched, which GS_2D_render_backward can use to sum gradients without atomics). `overlap(offsets)`, if given,
     is called once the scan is queued and before the host waits for the instance count; its result is appended.
-    `records` (gs_2d_preprocess_forward(..., return_records=True)): the scan stores every surfel's offset into its record."""
+    `records` (gs_2d_preprocess_forward(..., return_records=True)): the scan stores every surfel's offset into its record.
+    `cull` (needs `records`, or the `keep_masks` the preprocess wrote; no counterpart in the reference): instances that no pixel of their tile can blend are left
+    out of the lists -- same images and gradients from shorter lists; point_list keeps its length R, the entries behind
+    the last tile's end are unused, n_contrib counts positions of the shorter lists. The per-surfel keep masks [P] int32
+    are appended to the result; GS_2D_render_backward must get them (`culled=masks`) when it sums ordered records."""
     what = 'GS_prepare'
     _f32(what, means2D=means2D, depths=depths)
     L.require_cuda(what, radii=radii, tiles_touched=tiles_touched)
@@ -290,8 +301,20 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
     if records is not None:
         _f32(what, records=records)
         L.require_shape(what, 'records', records, P, 20)
+    if cull and records is None and keep_masks is None:
+        raise RuntimeError(f'{what}: cull needs the packed records or the keep masks')
     lib = _lib()
     stream = L.current_stream()
+    masks = keep_masks
+    if masks is not None:
+        L.require_cuda(what, keep_masks=masks)
+        L.require_dtype(what, 'keep_masks', masks, torch.int32)
+        L.require_shape(what, 'keep_masks', masks, max(P, 1))
+    if cull and masks is None:
+        masks = torch.empty((max(P, 1),), dtype=torch.int32, device=dev)
+        with _timed('gs_prepare_fill'):
+            rc = lib.fsgs_gs_2d_cull_masks(P, W, H, L.ptr(records), L.ptr(radii), L.ptr(masks), stream)
+        L.check(rc, what)
     T = ((W + _TILE - 1) // _TILE) * ((H + _TILE - 1) // _TILE)
     ranges = torch.empty((T, 2), dtype=torch.int64, device=dev)
     offsets = torch.empty((max(P, 1),), dtype=torch.int64, device=dev)
@@ -306,8 +329,12 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
                                             count.data_ptr(), L.ptr(records), stream)
     L.check(rc, what)
     with _timed('gs_prepare_fill'):  # first of the operator's two parts: callers that time stages add them up
-        rc = lib.fsgs_gs_prepare_count(P, W, H, L.ptr(means2D), L.ptr(radii), L.ptr(ranges), L.ptr(bins), bins.numel(),
-                                       stream)
+        if cull:
+            rc = lib.fsgs_gs_prepare_count_culled(P, W, H, L.ptr(means2D), L.ptr(radii), L.ptr(masks), L.ptr(ranges),
+                                                  L.ptr(bins), bins.numel(), stream)
+        else:
+            rc = lib.fsgs_gs_prepare_count(P, W, H, L.ptr(means2D), L.ptr(radii), L.ptr(ranges), L.ptr(bins),
+                                           bins.numel(), stream)
     L.check(rc, what)
     overlapped = overlap(offsets) if overlap is not None else None
     L.check(lib.fsgs_gs_prepare_scan_end(), what)
@@ -316,9 +343,15 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
     keys = torch.empty((R,), dtype=torch.int64, device=dev) if return_keys else None
     ws2 = _workspace(lib.fsgs_gs_prepare_fill_workspace_bytes(R), dev)
     with _timed('gs_prepare_fill'):
-        rc = lib.fsgs_gs_prepare_fill_counted(P, W, H, L.ptr(means2D), L.ptr(depths), L.ptr(radii), R, L.ptr(ranges),
-                                              L.ptr(point_list), L.ptr(keys), L.ptr(bins), bins.numel(), L.ptr(ws2),
-                                              ws2.numel(), stream)
+        if cull:
+            rc = lib.fsgs_gs_prepare_fill_counted_culled(P, W, H, L.ptr(means2D), L.ptr(depths), L.ptr(radii),
+                                                         L.ptr(masks), R, L.ptr(ranges), L.ptr(point_list),
+                                                         L.ptr(keys), L.ptr(bins), bins.numel(), L.ptr(ws2),
+                                                         ws2.numel(), stream)
+        else:
+            rc = lib.fsgs_gs_prepare_fill_counted(P, W, H, L.ptr(means2D), L.ptr(depths), L.ptr(radii), R,
+                                                  L.ptr(ranges), L.ptr(point_list), L.ptr(keys), L.ptr(bins),
+                                                  bins.numel(), L.ptr(ws2), ws2.numel(), stream)
     L.check(rc, what)
     if debug:
         torch.cuda.synchronize()
@@ -329,6 +362,8 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
         out.append(offsets)
     if overlap is not None:
         out.append(overlapped)
+    if cull:
+        out.append(masks)
     return out
 
 
@@ -404,10 +439,12 @@ def gs_2d_pack_records(means2D: Tensor, colors: Tensor, normal_opacity: Tensor, 
 def GS_2D_render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat2, out_opacity, out_others, out_flows,
                           dL_dout_color, dL_dout_opacity, dL_dothers, dL_dout_flows, ranges, point_list, n_contrib,
                           near_n: float, far_n: float, point_offsets: Optional[Tensor] = None,
-                          radii: Optional[Tensor] = None, records: Optional[Tensor] = None):
+                          radii: Optional[Tensor] = None, records: Optional[Tensor] = None,
+                          culled: Optional[Tensor] = None):
     """gs_2d_redner.cu:631-717 -> (dL_dcolors[P,3], dL_dmeans2D[P,2], dL_dtrans_m[P,3,3], dL_dnorm_op[P,4]).
     With `point_offsets` (GS_prepare(..., return_offsets=True)) and `radii` the per-surfel sums are taken in a fixed
-    order from per-instance records instead of with atomics."""
+    order from per-instance records instead of with atomics. `culled`: the keep masks GS_prepare(..., cull=True) returned
+    with these lists."""
     what = 'GS_2D_render_backward'
     L.require_cuda(what, dL_dout_color=dL_dout_color, dL_dout_opacity=dL_dout_opacity, dL_dothers=dL_dothers,
                    dL_dout_flows=dL_dout_flows, point_offsets=point_offsets, radii=radii)
@@ -446,15 +483,20 @@ def GS_2D_render_backward(means2D, normal_opacity, colors, trans_mat, trans_mat2
         L.require_dtype(what, 'point_offsets', point_offsets, torch.int64)
         L.require_dtype(what, 'radii', radii, torch.int32)
         ws = _workspace(lib.fsgs_gs_2d_render_backward_workspace_bytes(R), out_opacity.device)
+    if culled is not None:
+        L.require_cuda(what, culled=culled)
+        L.require_dtype(what, 'culled', culled, torch.int32)
+        L.require_shape(what, 'culled', culled, max(P, 1))
+    tail = (L.ptr(records), L.current_stream()) if culled is None else (L.ptr(records), L.ptr(culled), L.current_stream())
     with _timed('gs_2d_render_backward'):
-        rc = lib.fsgs_gs_2d_render_backward(
+        rc = (lib.fsgs_gs_2d_render_backward if culled is None else lib.fsgs_gs_2d_render_backward_culled)(
             P, W, H, float(near_n), float(far_n), L.ptr(means2D), L.ptr(normal_opacity), L.ptr(colors), L.ptr(trans_mat),
             L.ptr(trans_mat2), L.ptr(out_opacity), L.ptr(out_others) if use_aux else None,
             L.ptr(out_flows) if dL_dout_flows is not None else None, L.ptr(dL_dout_color), L.ptr(dL_dout_opacity),
             L.ptr(dL_dothers) if use_aux else None, L.ptr(dL_dout_flows), L.ptr(ranges), L.ptr(point_list),
             L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_norm_op), R,
             L.ptr(point_offsets) if ordered else None, L.ptr(radii) if ordered else None, L.ptr(ws),
-            ws.numel() if ws is not None else 0, L.ptr(records), L.current_stream())
+            ws.numel() if ws is not None else 0, *tail)
     L.check(rc, what)
     return g_colors, g_means2D, g_trans, g_norm_op
 

@@ -115,6 +115,7 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(int P, const i
 }
 
 constexpr int kCoopThreshold = 32;  // rectangles with more tiles are walked by the whole wavefront
+static_assert(kCoopThreshold == kCullMaskTiles, "a lane's serial walk covers exactly the rectangles that have a keep mask");
 
 // ---- binning by tile buckets -----------------------------------------------------------------------------------------
 // The reference sorts all (tile << 32 | depth bits) keys with one device-wide radix sort (6 passes of 8 bits for 2500
@@ -180,34 +181,42 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(int P, int gx, int gy, i
 // tile_scatter_kernel).
 constexpr int kMaxLdsTiles = 16384;
 
-// kCorner: only the tiles that pass the fast path's corner test (CornerTest, from the surfel's adjugate and opacity) are
-// visited.
-template <bool kCorner, typename Visit>
+// Which tiles of a surfel's rectangle are visited: all of them (the reference's lists), those that pass the fast path's
+// corner test (CornerTest, from the surfel's adjugate and opacity), or those whose bit is set in the surfel's keep mask
+// (cull_mask_kernel: the tiles some pixel of which can blend the surfel; rectangles above 32 tiles are kept whole).
+enum WalkMode { kWalkAll = 0, kWalkCorner = 1, kWalkMask = 2 };
+
+template <int kMode, typename Visit>
 __device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, const float2* __restrict__ means2D,
                                                   const int32_t* __restrict__ radii,
-                                                  const float* __restrict__ inverse_m,
+                                                  const float* __restrict__ inverse_m,   // kWalkMask: keep masks
                                                   const float* __restrict__ opacities, Visit visit) {
   const int lane = __lane_id();
   int x0 = 0, y0 = 0, w = 0, h = 0;
-  float IM[kCorner ? 9 : 1], opacity = 1.0f;
+  float IM[kMode == kWalkCorner ? 9 : 1], opacity = 1.0f;
 #pragma unroll
-  for (int k = 0; k < (kCorner ? 9 : 1); ++k) IM[k] = 0.0f;
+  for (int k = 0; k < (kMode == kWalkCorner ? 9 : 1); ++k) IM[k] = 0.0f;
+  uint32_t keep_mask = 0xffffffffu;
   if (i < P && radii[i] > 0) {
     const float2 c   = means2D[i];
     const TileRect r = tile_rect(c.x, c.y, radii[i], gx, gy);
     x0 = r.x0, y0 = r.y0, w = max(r.x1 - r.x0, 0), h = max(r.y1 - r.y0, 0);
-    if (kCorner) {
+    if (kMode == kWalkCorner) {
       opacity = opacities[i];
 #pragma unroll
       for (int k = 0; k < 9; ++k) IM[k] = inverse_m[9 * (size_t) i + k];
     }
+    if (kMode == kWalkMask) keep_mask = ((const uint32_t*) inverse_m)[i];
   }
   const int count = w * h;
   if (count > 0 && count <= kCoopThreshold) {
-    const CornerTest ct(IM, opacity);  // unused (and removed) without kCorner
+    const CornerTest ct(IM, opacity);  // unused (and removed) in the other modes
+    int e = 0;
     for (int y = 0; y < h; ++y)
-      for (int x = 0; x < w; ++x)
-        if (!kCorner || ct.tile(x0 + x, y0 + y)) visit((y0 + y) * gx + (x0 + x), i);
+      for (int x = 0; x < w; ++x, ++e) {
+        const bool keep = kMode == kWalkCorner ? ct.tile(x0 + x, y0 + y) : kMode == kWalkMask ? ((keep_mask >> e) & 1u) != 0u : true;
+        if (keep) visit((y0 + y) * gx + (x0 + x), i);
+      }
   }
   unsigned long long big = __ballot(count > kCoopThreshold);
   while (big) {
@@ -215,15 +224,41 @@ __device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, 
     big &= big - 1;
     const int sx0 = __shfl(x0, src, kWave), sy0 = __shfl(y0, src, kWave), sw = __shfl(w, src, kWave);
     const int scount = __shfl(count, src, kWave), sid = __shfl(i, src, kWave);
-    float sIM[kCorner ? 9 : 1];
+    float sIM[kMode == kWalkCorner ? 9 : 1];
 #pragma unroll
-    for (int k = 0; k < (kCorner ? 9 : 1); ++k) sIM[k] = kCorner ? __shfl(IM[k], src, kWave) : 0.0f;
-    const CornerTest ct(sIM, kCorner ? __shfl(opacity, src, kWave) : 1.0f);
+    for (int k = 0; k < (kMode == kWalkCorner ? 9 : 1); ++k) sIM[k] = kMode == kWalkCorner ? __shfl(IM[k], src, kWave) : 0.0f;
+    const CornerTest ct(sIM, kMode == kWalkCorner ? __shfl(opacity, src, kWave) : 1.0f);
     for (int e = lane; e < scount; e += kWave) {
       const int y = e / sw, x = e - y * sw;
-      if (!kCorner || ct.tile(sx0 + x, sy0 + y)) visit((sy0 + y) * gx + (sx0 + x), sid);
+      if (kMode != kWalkCorner || ct.tile(sx0 + x, sy0 + y)) visit((sy0 + y) * gx + (sx0 + x), sid);
     }
   }
+}
+
+// One lane per surfel: the keep mask of its rectangle (see kCullMaskTiles) from its packed record.
+__global__ void __launch_bounds__(256) cull_mask_kernel(int P, int gx, int gy, const float4* __restrict__ records,
+                                                        const int32_t* __restrict__ radii, uint32_t* __restrict__ masks) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= P) return;
+  uint32_t m = 0xffffffffu;
+  const int radius = radii[i];
+  if (radius > 0) {
+    const float4* rec = records + 5 * (size_t) i;
+    const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
+    const float M[9] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w, q2.x};
+    const float ox = q2.y, oy = q2.z;
+    const TileRect r = tile_rect(ox, oy, radius, gx, gy);
+    const int w = max(r.x1 - r.x0, 0), h = max(r.y1 - r.y0, 0);
+    if (w * h <= kCullMaskTiles) {
+      const CullBounds cb = cull_bounds(M, ox, oy, q2.w);
+      m = 0u;
+      int e = 0;
+      for (int y = 0; y < h; ++y)
+        for (int x = 0; x < w; ++x, ++e)
+          if (cull_keeps_tile(cb, ox, oy, r.x0 + x, r.y0 + y)) m |= 1u << e;
+    }
+  }
+  masks[i] = m;
 }
 
 // Layout of the `bins` buffer of the bucket binning: the queue length of the long segments in front of the B x T matrix
@@ -250,7 +285,7 @@ inline BinsLayout bins_layout(int P, int T) {
 // stores (zeros included, so the matrix needs no clearing). No global atomics: device-scope atomics on one address are
 // served one after the other at fabric latency, and with surfels in no spatial order every block touches nearly
 // every tile.
-template <bool kCorner>
+template <int kMode>
 __global__ void __launch_bounds__(1024) tile_hist_kernel(int P, int per_block, int gx, int gy,
     const float2* __restrict__ means2D, const int32_t* __restrict__ radii, const float* __restrict__ inverse_m,
     const float* __restrict__ opacities, uint32_t* __restrict__ hist) {
@@ -263,7 +298,7 @@ __global__ void __launch_bounds__(1024) tile_hist_kernel(int P, int per_block, i
   const int rounds = (last - first + (int) blockDim.x - 1) / (int) blockDim.x;
   for (int r = 0; r < rounds; ++r) {
     const int i = first + r * blockDim.x + threadIdx.x;
-    for_each_instance<kCorner>(i < last ? i : P, P, gx, gy, means2D, radii, inverse_m, opacities,
+    for_each_instance<kMode>(i < last ? i : P, P, gx, gy, means2D, radii, inverse_m, opacities,
                                [&](int tile, int) { atomicAdd(&s_count[tile], 1u); });
   }
   __syncthreads();
@@ -311,7 +346,7 @@ __global__ void __launch_bounds__(kPrefixTiles * kPrefixWaves) tile_prefix_kerne
 
 // Step 3: the walk of step 1 again; a block's cursor of a tile starts at the tile's start plus the instances of the
 // blocks in front of it, so the placement needs no global atomics either.
-template <bool kCorner>
+template <int kMode>
 __global__ void __launch_bounds__(1024) tile_scatter_kernel(int P, int per_block, int gx, int gy, int64_t R,
     const float2* __restrict__ means2D, const float* __restrict__ depths, const int32_t* __restrict__ radii,
     const float* __restrict__ inverse_m, const float* __restrict__ opacities, const uint32_t* __restrict__ hist,
@@ -325,7 +360,7 @@ __global__ void __launch_bounds__(1024) tile_scatter_kernel(int P, int per_block
   const int rounds = (last - first + (int) blockDim.x - 1) / (int) blockDim.x;
   for (int r = 0; r < rounds; ++r) {
     const int i = first + r * blockDim.x + threadIdx.x;
-    for_each_instance<kCorner>(i < last ? i : P, P, gx, gy, means2D, radii, inverse_m, opacities, [&](int tile, int id) {
+    for_each_instance<kMode>(i < last ? i : P, P, gx, gy, means2D, radii, inverse_m, opacities, [&](int tile, int id) {
       const unsigned pos = atomicAdd(&s_cursor[tile], 1u);
       if ((int64_t) pos < R) entries[pos] = ((uint64_t) __float_as_uint(depths[id]) << 32) | (uint32_t) id;
     });
@@ -810,14 +845,14 @@ int fast_bucket_fill(int P, int W, int H, const float* means2D, const float* inv
   uint32_t* hist   = (uint32_t*) ((char*) bins + kBinsHeader);
   uint64_t* entries = sort_keys_in(R, workspace);
   int* large_list   = (int*) ((char*) workspace + sort_layout(R).keys1);
-  hipLaunchKernelGGL(tile_hist_kernel<true>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
+  hipLaunchKernelGGL(tile_hist_kernel<kWalkCorner>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
                      (const float2*) means2D, radii, inverse_m, opacities, hist);
   hipLaunchKernelGGL(tile_prefix_kernel, dim3(div_up(T, kPrefixTiles)), dim3(kPrefixTiles * kPrefixWaves), 0, s, T,
                      bl.blocks, hist, rng);
   hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, true);
   const int* order = nullptr;
   (void) launch_tile_order(gx, gy, ranges, s, &order);  // the blend kernels of this view find it under `ranges`
-  hipLaunchKernelGGL(tile_scatter_kernel<true>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
+  hipLaunchKernelGGL(tile_scatter_kernel<kWalkCorner>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
                      (const float2*) means2D, depths, radii, inverse_m, opacities, (const uint32_t*) hist, rng, entries);
   hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
                      header, large_list, order);
@@ -905,8 +940,10 @@ FSGS_API int fsgs_gs_prepare_sort_bits(int W, int H) {
 namespace {
 // First part of the bucket binning, independent of the instance count: per-tile instance counts and the tile ranges
 // (start, end); the long-segment queue's counter (first word of `bins`) is reset.
-int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, int64_t* ranges, void* bins,
-               hipStream_t s) {
+// cull_records (optional): the per-surfel keep masks of cull_mask_kernel; with them an instance is only counted (and
+// later scattered) when its bit is set.
+int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, const float* cull_records,
+               int64_t* ranges, void* bins, hipStream_t s) {
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int T  = gx * gy;
   unsigned long long* rng = (unsigned long long*) ranges;
@@ -914,8 +951,12 @@ int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, 
   const BinsLayout bl = bins_layout(P, T);
   if (bl.blocks > 0) {
     uint32_t* hist = (uint32_t*) ((char*) bins + kBinsHeader);
-    hipLaunchKernelGGL(tile_hist_kernel<false>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
-                       (const float2*) means2D, radii, (const float*) nullptr, (const float*) nullptr, hist);
+    if (cull_records)
+      hipLaunchKernelGGL(tile_hist_kernel<kWalkMask>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
+                         (const float2*) means2D, radii, cull_records, (const float*) nullptr, hist);
+    else
+      hipLaunchKernelGGL(tile_hist_kernel<kWalkAll>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
+                         (const float2*) means2D, radii, (const float*) nullptr, (const float*) nullptr, hist);
     hipLaunchKernelGGL(tile_prefix_kernel, dim3(div_up(T, kPrefixTiles)), dim3(kPrefixTiles * kPrefixWaves), 0, s, T,
                        bl.blocks, hist, rng);
     hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, true);
@@ -937,9 +978,9 @@ int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, 
 }
 
 // Second part: scatter (depth bits << 32 | surfel) into the tile segments and sort every segment.
-int fill_sort(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii, int64_t R,
-              int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out, void* workspace, void* bins,
-              hipStream_t s) {
+int fill_sort(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
+              const float* cull_records, int64_t R, int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out,
+              void* workspace, void* bins, hipStream_t s) {
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int T  = gx * gy;
   unsigned long long* rng = (unsigned long long*) ranges;
@@ -948,8 +989,12 @@ int fill_sort(int P, int W, int H, const float* means2D, const float* depths, co
   // queue of long segments: at most R / kSmallSegment tiles, kept behind the entries in the workspace
   int* large_list = (int*) ((char*) workspace + sort_layout(R).keys1);
   const BinsLayout bl = bins_layout(P, T);
-  if (bl.blocks > 0)
-    hipLaunchKernelGGL(tile_scatter_kernel<false>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
+  if (bl.blocks > 0 && cull_records)
+    hipLaunchKernelGGL(tile_scatter_kernel<kWalkMask>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
+                       (const float2*) means2D, depths, radii, cull_records, (const float*) nullptr,
+                       (const uint32_t*) ((const char*) bins + kBinsHeader), rng, entries);
+  else if (bl.blocks > 0)
+    hipLaunchKernelGGL(tile_scatter_kernel<kWalkAll>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
                        (const float2*) means2D, depths, radii, (const float*) nullptr, (const float*) nullptr,
                        (const uint32_t*) ((const char*) bins + kBinsHeader), rng, entries);
   else
@@ -980,7 +1025,7 @@ FSGS_API int fsgs_gs_prepare_count(int P, int W, int H, const float* means2D, co
     return fail(kWorkspaceSmall, "gs_prepare_count: bins %zu < %zu bytes", bins_bytes,
                 fsgs_gs_prepare_bins_bytes(P, W, H));
   tile_order_invalidate((hipStream_t) stream);  // the ranges are rewritten: the blend schedule of this stream is stale
-  return fill_count(P, W, H, means2D, radii, ranges, bins, (hipStream_t) stream);
+  return fill_count(P, W, H, means2D, radii, nullptr, ranges, bins, (hipStream_t) stream);
 }
 
 FSGS_API int fsgs_gs_prepare_fill_counted(int P, int W, int H, const float* means2D, const float* depths,
@@ -997,8 +1042,56 @@ FSGS_API int fsgs_gs_prepare_fill_counted(int P, int W, int H, const float* mean
   if (bins_bytes < fsgs_gs_prepare_bins_bytes(P, W, H))
     return fail(kWorkspaceSmall, "gs_prepare_fill: bins %zu < %zu bytes", bins_bytes,
                 fsgs_gs_prepare_bins_bytes(P, W, H));
-  return fill_sort(P, W, H, means2D, depths, radii, R, ranges, point_list, sorted_keys_out, workspace, bins,
+  return fill_sort(P, W, H, means2D, depths, radii, nullptr, R, ranges, point_list, sorted_keys_out, workspace, bins,
                    (hipStream_t) stream);
+}
+
+// Keep masks for the culled binning: a bit per tile of a surfel's rectangle (row-major, rectangles of at most 32 tiles;
+// larger ones are kept whole), set when some pixel of the tile can blend the surfel by the blend kernels' own bound.
+FSGS_API int fsgs_gs_2d_cull_masks(int P, int W, int H, const float* records, const int32_t* radii, uint32_t* masks,
+                                   void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "gs_2d_cull_masks: bad sizes");
+  if (P == 0) return kOk;
+  FSGS_REQUIRE(records && radii && masks, "gs_2d_cull_masks: null pointer");
+  FSGS_REQUIRE(((uintptr_t) records & 15) == 0, "gs_2d_cull_masks: records must be 16-byte aligned");
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  hipLaunchKernelGGL(cull_mask_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, gx, gy,
+                     (const float4*) records, radii, masks);
+  return check_launch("gs_2d_cull_masks");
+}
+
+// The two phases of the binning over the kept tiles only (masks: fsgs_gs_2d_cull_masks). Tile grids too large for the
+// per-tile counters, and a process with the culling switched off for debugging, get the full lists.
+FSGS_API int fsgs_gs_prepare_count_culled(int P, int W, int H, const float* means2D, const int32_t* radii,
+                                          const uint32_t* masks, int64_t* ranges, void* bins, size_t bins_bytes,
+                                          void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && ranges && bins, "gs_prepare_count_culled: bad arguments");
+  FSGS_REQUIRE(P == 0 || (means2D && radii && masks), "gs_prepare_count_culled: null pointer");
+  if (bins_bytes < fsgs_gs_prepare_bins_bytes(P, W, H))
+    return fail(kWorkspaceSmall, "gs_prepare_count_culled: bins %zu < %zu bytes", bins_bytes,
+                fsgs_gs_prepare_bins_bytes(P, W, H));
+  tile_order_invalidate((hipStream_t) stream);
+  return fill_count(P, W, H, means2D, radii, culling_enabled() ? (const float*) masks : nullptr, ranges, bins,
+                    (hipStream_t) stream);
+}
+
+FSGS_API int fsgs_gs_prepare_fill_counted_culled(int P, int W, int H, const float* means2D, const float* depths,
+                                                 const int32_t* radii, const uint32_t* masks, int64_t R,
+                                                 int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out,
+                                                 void* bins, size_t bins_bytes, void* workspace,
+                                                 size_t workspace_bytes, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && R >= 0 && ranges && bins, "gs_prepare_fill_culled: bad arguments");
+  FSGS_REQUIRE(R < (int64_t) 0x7fffffff, "gs_prepare_fill_culled: %lld instances exceed the 2^31-1 limit", (long long) R);
+  if (R == 0 || P == 0) return kOk;
+  FSGS_REQUIRE(means2D && depths && radii && masks && point_list && workspace, "gs_prepare_fill_culled: null pointer");
+  if (workspace_bytes < sort_workspace_bytes(R))
+    return fail(kWorkspaceSmall, "gs_prepare_fill_culled: workspace %zu < %zu bytes", workspace_bytes,
+                sort_workspace_bytes(R));
+  if (bins_bytes < fsgs_gs_prepare_bins_bytes(P, W, H))
+    return fail(kWorkspaceSmall, "gs_prepare_fill_culled: bins %zu < %zu bytes", bins_bytes,
+                fsgs_gs_prepare_bins_bytes(P, W, H));
+  return fill_sort(P, W, H, means2D, depths, radii, culling_enabled() ? (const float*) masks : nullptr, R, ranges,
+                   point_list, sorted_keys_out, workspace, bins, (hipStream_t) stream);
 }
 
 FSGS_API int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, const float* depths,
@@ -1023,6 +1116,6 @@ FSGS_API int fsgs_gs_prepare_fill(int P, int W, int H, const float* means2D, con
   if (bins_bytes < fsgs_gs_prepare_bins_bytes(P, W, H))
     return fail(kWorkspaceSmall, "gs_prepare_fill: bins %zu < %zu bytes", bins_bytes,
                 fsgs_gs_prepare_bins_bytes(P, W, H));
-  if (int rc = fill_count(P, W, H, means2D, radii, ranges, bins, s)) return rc;
-  return fill_sort(P, W, H, means2D, depths, radii, R, ranges, point_list, sorted_keys_out, workspace, bins, s);
+  if (int rc = fill_count(P, W, H, means2D, radii, nullptr, ranges, bins, s)) return rc;
+  return fill_sort(P, W, H, means2D, depths, radii, nullptr, R, ranges, point_list, sorted_keys_out, workspace, bins, s);
 }

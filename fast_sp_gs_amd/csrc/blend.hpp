@@ -2,6 +2,7 @@
 // surfels, the ray-splat intersection, and wave64 cross-lane reductions.
 #pragma once
 #include "common.hpp"
+#include "cull_bound.hpp"
 
 namespace fsgs {
 
@@ -147,10 +148,6 @@ __device__ __forceinline__ bool intersect_flat(const SplatHot& h, float pxf, flo
 // padded by 1/8 pixel + 0.5 % of its extent against rounding, is tested against the four 8x8 quadrants of the tile; a
 // clear bit means no pixel of that quadrant can pass the reference's alpha test, so skipping it changes nothing.
 // Surfels whose tau-ellipse reaches the camera plane (no finite box) keep all bits set.
-#ifndef FSGS_CULL_PAD
-#define FSGS_CULL_PAD 0.125f
-#endif
-constexpr float kCullPad = FSGS_CULL_PAD;  // pixels added around the footprint box against rounding
 
 __device__ __forceinline__ unsigned quadrant_mask(const SplatHot& h, int tile_px, int tile_py, int flags) {
   if (flags & kFlagNoCull) return 0xfu;

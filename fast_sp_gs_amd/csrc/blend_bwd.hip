@@ -560,6 +560,44 @@ __global__ void __launch_bounds__(256) slot_reduce_kernel(int P, const int64_t* 
   }
 }
 
+// The same sum over lists built by the culled binning (fsgs_gs_prepare_*_culled): the positions of a surfel's span
+// whose bit is clear in its keep mask belong to no list, were never written and are not read. Nine positions of the
+// span per step, row-major over the surfel's rectangle, the records of the kept ones requested together.
+__global__ void __launch_bounds__(256) slot_reduce_culled_kernel(int P, const int64_t* __restrict__ point_offsets,
+    const uint32_t* __restrict__ masks, const float* __restrict__ slot_grads, float* __restrict__ g_colors,
+    float* __restrict__ g_means2D, float* __restrict__ g_trans, float* __restrict__ g_normal_opacity) {
+  constexpr int kPerWave = 7, kLanes = 9;
+  const int lane = threadIdx.x & 63;
+  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int sub = lane / kLanes, k = lane - sub * kLanes;
+  const int i = wave * kPerWave + sub;
+  if (sub >= kPerWave || i >= P) return;
+  const int64_t e0 = i > 0 ? point_offsets[i - 1] : 0, e1 = point_offsets[i];
+  const int count = (int) (e1 - e0);
+  // rectangles above kCullMaskTiles tiles are kept whole
+  const uint32_t mask = count > kCullMaskTiles ? 0xffffffffu : masks[i];
+  const float2* src = (const float2*) slot_grads + (size_t) e0 * kLanes + k;
+  float2 acc = make_float2(0.0f, 0.0f);
+  for (int base = 0; base < count; base += kLanes) {
+    const uint32_t bits = count > kCullMaskTiles ? 0xffffffffu : (mask >> base);
+    float2 v[kLanes];
+#pragma unroll
+    for (int j = 0; j < kLanes; ++j)
+      v[j] = (base + j < count && ((bits >> j) & 1u)) ? src[(size_t) (base + j) * kLanes] : make_float2(0.0f, 0.0f);
+#pragma unroll
+    for (int j = 0; j < kLanes; ++j) acc.x += v[j].x, acc.y += v[j].y;
+  }
+  const float vals[2] = {acc.x, acc.y};
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int c = 2 * k + h;
+    if (c < 3) g_colors[3 * (size_t) i + c] = vals[h];
+    else if (c < 12) g_trans[9 * (size_t) i + (c - 3)] = vals[h];
+    else if (c < 16) g_normal_opacity[4 * (size_t) i + (c - 12)] = vals[h];
+    else g_means2D[2 * (size_t) i + (c - 16)] = vals[h];
+  }
+}
+
 }  // namespace
 }  // namespace fsgs
 
@@ -569,13 +607,15 @@ FSGS_API size_t fsgs_gs_2d_render_backward_workspace_bytes(int64_t R) {
   return align_up((size_t) (R > 0 ? R : 0) * kGradSlots * 4 + 16, 256);
 }
 
-FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n, const float* means2D,
+namespace {
+// keep_masks: the lists come from fsgs_gs_prepare_*_culled, so the record sum has to skip the positions the binning left out
+int render_backward(int P, int W, int H, double near_n, double far_n, const float* means2D,
     const float* normal_opacity, const float* colors, const float* trans_mat, const float* trans_mat_t2,
     const float* out_opacity, const float* out_extras, const float* out_flow, const float* dL_dpix,
     const float* dL_dopacity, const float* dL_dextras, const float* dL_dflow, const int64_t* ranges,
     const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
     float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
-    size_t workspace_bytes, const float* records, void* stream) {
+    size_t workspace_bytes, const float* records, const uint32_t* keep_masks, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_render_backward: bad sizes");
   if (P == 0) return kOk;
   FSGS_REQUIRE(means2D && normal_opacity && colors && trans_mat && out_opacity && dL_dpix && dL_dopacity && ranges &&
@@ -612,8 +652,12 @@ FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, doub
     else if (aux) FSGS_LAUNCH_BWD(true, false, true);
     else FSGS_LAUNCH_BWD(false, false, true);
     const int waves = div_up(P, 7);  // kPerWave surfels per wavefront
-    hipLaunchKernelGGL(slot_reduce_kernel, dim3(div_up((int64_t) waves * 64, 256)), dim3(256), 0, s, P, point_offsets,
-                       slot_grads, g_colors, g_means2D, g_trans, g_normal_opacity);
+    if (keep_masks && culling_enabled())
+      hipLaunchKernelGGL(slot_reduce_culled_kernel, dim3(div_up((int64_t) waves * 64, 256)), dim3(256), 0, s, P,
+                         point_offsets, keep_masks, slot_grads, g_colors, g_means2D, g_trans, g_normal_opacity);
+    else
+      hipLaunchKernelGGL(slot_reduce_kernel, dim3(div_up((int64_t) waves * 64, 256)), dim3(256), 0, s, P, point_offsets,
+                         slot_grads, g_colors, g_means2D, g_trans, g_normal_opacity);
   } else {
     if (aux && flow) FSGS_LAUNCH_BWD(true, true, false);
     else if (aux) FSGS_LAUNCH_BWD(true, false, false);
@@ -621,4 +665,33 @@ FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, doub
   }
 #undef FSGS_LAUNCH_BWD
   return check_launch("GS_2D_render_backward");
+}
+}  // namespace
+
+FSGS_API int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n, const float* means2D,
+    const float* normal_opacity, const float* colors, const float* trans_mat, const float* trans_mat_t2,
+    const float* out_opacity, const float* out_extras, const float* out_flow, const float* dL_dpix,
+    const float* dL_dopacity, const float* dL_dextras, const float* dL_dflow, const int64_t* ranges,
+    const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
+    float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
+    size_t workspace_bytes, const float* records, void* stream) {
+  return render_backward(P, W, H, near_n, far_n, means2D, normal_opacity, colors, trans_mat, trans_mat_t2, out_opacity,
+                         out_extras, out_flow, dL_dpix, dL_dopacity, dL_dextras, dL_dflow, ranges, point_list, n_contrib,
+                         g_colors, g_means2D, g_trans, g_normal_opacity, R, point_offsets, radii, workspace,
+                         workspace_bytes, records, nullptr, stream);
+}
+
+FSGS_API int fsgs_gs_2d_render_backward_culled(int P, int W, int H, double near_n, double far_n, const float* means2D,
+    const float* normal_opacity, const float* colors, const float* trans_mat, const float* trans_mat_t2,
+    const float* out_opacity, const float* out_extras, const float* out_flow, const float* dL_dpix,
+    const float* dL_dopacity, const float* dL_dextras, const float* dL_dflow, const int64_t* ranges,
+    const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
+    float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
+    size_t workspace_bytes, const float* records, const uint32_t* keep_masks, void* stream) {
+  FSGS_REQUIRE(P == 0 || !point_offsets || keep_masks,
+               "GS_2D_render_backward_culled: the ordered-sum path over culled lists needs the keep masks");
+  return render_backward(P, W, H, near_n, far_n, means2D, normal_opacity, colors, trans_mat, trans_mat_t2, out_opacity,
+                         out_extras, out_flow, dL_dpix, dL_dopacity, dL_dextras, dL_dflow, ranges, point_list, n_contrib,
+                         g_colors, g_means2D, g_trans, g_normal_opacity, R, point_offsets, radii, workspace,
+                         workspace_bytes, records, keep_masks, stream);
 }

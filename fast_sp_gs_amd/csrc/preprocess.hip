@@ -6,6 +6,7 @@
 // reference's operation order, so radii / tiles_touched / means2D / trans_mat / depths are reproducible bit for bit
 // against a plain IEEE evaluation of the same expressions.
 #include "common.hpp"
+#include "cull_bound.hpp"
 #include "sh.hpp"
 #include "sh_stage.hpp"
 #include "surfel_geom.hpp"
@@ -89,7 +90,7 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
     const float* __restrict__ campos, const float* __restrict__ trans_precomp, const uint8_t* __restrict__ culling,
     int means2D_preserve, float2* __restrict__ means2D, float* __restrict__ colors, float* __restrict__ trans_mat,
     float4* __restrict__ normal_opacity, float* __restrict__ depths, int32_t* __restrict__ radii,
-    int32_t* __restrict__ tiles_touched, float4* __restrict__ records) {
+    int32_t* __restrict__ tiles_touched, float4* __restrict__ records, uint32_t* __restrict__ keep_masks) {
   constexpr bool kStage = kSh == 16;  // degree <= 3: SH rows travel through LDS, read from HBM line by line
   __shared__ float s_Tw2v[16], s_Tw2c[16];
   __shared__ float s_rows[kStage ? kShStageRows * kShStageStride : 1];
@@ -200,6 +201,26 @@ __global__ void __launch_bounds__(256) preprocess_forward_kernel(
 #pragma unroll
       for (int k = 0; k < 5; ++k) r[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
+  }
+  if (keep_masks) {
+    // Which tiles of the surfel's rectangle some pixel of which can blend it (the culled binning's input): a bit per
+    // tile, row-major; rectangles above kCullMaskTiles tiles keep every bit. Evaluated here, where transform, centre
+    // and radius are in registers and the vector units wait for memory anyway.
+    uint32_t m = 0xffffffffu;
+    if (ok) {
+      const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+      const TileRect r = tile_rect(c2[0], c2[1], f2i_sat(radius), gx, gy);
+      const int w = max(r.x1 - r.x0, 0), h = max(r.y1 - r.y0, 0);
+      if (w * h <= kCullMaskTiles) {
+        const CullBounds cb = cull_bounds(M, c2[0], c2[1], opacities[i]);
+        m = 0u;
+        int e = 0;
+        for (int y = 0; y < h; ++y)
+          for (int x = 0; x < w; ++x, ++e)
+            if (cull_keeps_tile(cb, c2[0], c2[1], r.x0 + x, r.y0 + y)) m |= 1u << e;
+      }
+    }
+    keep_masks[i] = m;
   }
 }
 
@@ -435,7 +456,7 @@ FSGS_API int fsgs_gs_2d_preprocess_forward(int P, int W, int H, int sh_degree, i
     const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
     const float* Tw2v, const float* Tv2c, const float* campos, const float* trans_precomp, const uint8_t* culling,
     int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* normal_opacity, float* depths,
-    int32_t* radii, int32_t* tiles_touched, float* records, void* stream) {
+    int32_t* radii, int32_t* tiles_touched, float* records, uint32_t* keep_masks, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "gs_2d_preprocess_forward: bad sizes P=%d W=%d H=%d", P, W, H);
   FSGS_REQUIRE(((uintptr_t) records & 15) == 0, "gs_2d_preprocess_forward: records must be 16-byte aligned");
   FSGS_REQUIRE(sh_degree <= kMaxShDegree, "gs_2d_preprocess_forward: sh_degree %d > %d not supported", sh_degree,
@@ -453,7 +474,7 @@ FSGS_API int fsgs_gs_2d_preprocess_forward(int P, int W, int H, int sh_degree, i
                               : (wave_rows ? preprocess_forward_kernel<16, true> : preprocess_forward_kernel<16, false>);
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh, means3D, (const float2*) scales, (const float4*) rotations, opacities, shs,
                      sh_rest, Tw2v, Tv2c, campos, trans_precomp, culling, means2D_preserve, (float2*) means2D, colors,
-                     trans_mat, (float4*) normal_opacity, depths, radii, tiles_touched, (float4*) records);
+                     trans_mat, (float4*) normal_opacity, depths, radii, tiles_touched, (float4*) records, keep_masks);
   return check_launch("gs_2d_preprocess_forward");
 }
 

@@ -14,6 +14,10 @@ from fast_sp_gs_amd._C import get_C_function
 __all__ = ['GS_2D_render', 'RasterizeBuffer', 'GS_2D_topk_weights', 'GS_prepare', 'render_step']
 
 GS_prepare = get_C_function('GS_prepare')
+# `_GS_2D_Render` bins with the blend kernels' own bound applied per (surfel, tile) instance: instances that no pixel of
+# their tile can blend are left out of the lists (same images and gradients from shorter lists; the lists and n_contrib
+# handed back in RasterizeBuffer are the shorter ones). False: the reference's lists, every tile of a surfel's rectangle.
+CULL_LISTS = True
 
 
 class RasterizeBuffer(NamedTuple):
@@ -67,16 +71,20 @@ class _GS_2D_Render(torch.autograd.Function):
                 accum_max_count, accum_weights_p, accum_weights_count):
         W, H = size
         # the preprocess kernel also writes the blend kernels' packed per-surfel record (no second pass, no launch)
-        (means2D, colors, trans_mat, normal_opacity, depths, radii, tiles_touched,
-         records) = _GS_2D_Render._preprocess_forward(
+        cull = bool(CULL_LISTS)
+        (means2D, colors, trans_mat, normal_opacity, depths, radii, tiles_touched, records,
+         *keep) = _GS_2D_Render._preprocess_forward(
             W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c,
-            campos, trans_precomp, means2D, culling, return_records=True)
+            campos, trans_precomp, means2D, culling, return_records=True, return_masks=cull)
+        keep = keep[0] if cull else None
         tile_range, point_list, point_offsets = GS_prepare(
-            W, H, means2D, depths, radii, tiles_touched, False, return_offsets=True, records=records)
+            W, H, means2D, depths, radii, tiles_touched, False, return_offsets=True, records=records, cull=cull,
+            keep_masks=keep)[:3]
         pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib = _GS_2D_Render._render_forward(
             W, H, means2D, colors, normal_opacity, trans_mat, point_list, tile_range, near_n, far_n, only_image,
             transe_mat_t2, accum_max_count, accum_weights_p, accum_weights_count, records)
         ctx._info = (W, H, sh_degree, is_opengl, near_n, far_n)
+        ctx._keep_masks = keep
         ctx.save_for_backward(means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, campos,
                               means2D, trans_mat, transe_mat_t2, radii, colors, normal_opacity, tile_range,
                               point_list, pixel_extras, pixel_opacity, pixel_flow, n_contrib, point_offsets, records)
@@ -100,7 +108,7 @@ class _GS_2D_Render(torch.autograd.Function):
         grad_colors, grad_means2D, grad_trans, grad_normal_opacity = _GS_2D_Render._render_backward(
             means2D, normal_opacity, colors, trans_mat, transe_mat_t2, pixel_opacity, pixel_extras, pixel_flow,
             grad_images, grad_opacity, grad_others, grad_flows, tile_range, point_list, n_contrib, near_n, far_n,
-            point_offsets, radii, records)
+            point_offsets, radii, records, culled=ctx._keep_masks)
         # the preprocess backward writes every row of its outputs (zeros for surfels that were not rendered), so they
         # are allocated uninitialised; pre-computed colours (sh_degree < 0) receive no gradient, as in the reference
         new = torch.empty_like
@@ -203,7 +211,8 @@ def GS_2D_topk_weights(topk: int, buffer: RasterizeBuffer) -> Tuple[Tensor, Tens
 
 
 def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad_opacity: Tensor = None,
-                ordered_sums: bool = True, packed: bool = True, background: Tensor = None, depth_ratio: float = 1.0):
+                ordered_sums: bool = True, packed: bool = True, background: Tensor = None, depth_ratio: float = 1.0,
+                cull: bool = False):
     """One forward + backward pass of the hot path on raw operators (no autograd graph): preprocess -> binning ->
     blend -> blend backward -> preprocess backward, in the order `_GS_2D_Render` runs them. Returns a dict with every
     intermediate so callers (benchmark, parity tests) can inspect or time the stages.
@@ -212,16 +221,24 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
     training: forward -> normals / depths / surf_depth / surf_normal / composited image; then `grad_image` is the
     gradient of the COMPOSITED image and the first six channels of `grad_extras` are read as the gradients of
     (surf_depth, normals x 3, depths, distortion); the epilogue backward turns them into the blend's dL/dextras and
-    the composite's dL/dopacity (added to `grad_opacity`)."""
+    the composite's dL/dopacity (added to `grad_opacity`).
+
+    `cull` (needs `packed`): bin as `_GS_2D_Render` does by default, leaving out the (surfel, tile) instances that no
+    pixel of their tile can blend; every image and gradient is the same, `ranges` / `point_list` / `n_contrib` are those
+    of the shorter lists."""
     f = get_C_function
+    if cull and not packed:
+        raise ValueError('cull needs the packed records')
     W, H = cam.W, cam.H
     dev = scene.means3D.device
     # with `packed` the preprocess kernel also writes the blend kernels' packed per-surfel record
     m2, colors, tm, no, depths, radii, tt, *rec = f('gs_2d_preprocess_forward')(
         W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs, None,
-        cam.Tw2v, cam.Tv2c, cam.campos, None, None, None, return_records=packed)
+        cam.Tw2v, cam.Tv2c, cam.campos, None, None, None, return_records=packed, return_masks=cull)
+    keep = rec[-1] if cull else None
     rec = rec[0] if packed else None
-    ranges, point_list, offsets = f('GS_prepare')(W, H, m2, depths, radii, tt, False, return_offsets=True, records=rec)
+    ranges, point_list, offsets = f('GS_prepare')(W, H, m2, depths, radii, tt, False, return_offsets=True,
+                                                  records=rec, cull=cull, keep_masks=keep)[:3]
     oc, oo, oe, of, nc = f('GS_2D_render_forward')(W, H, m2, colors, no, tm, point_list, ranges, cam.near, cam.far,
                                                    False, None, None, None, None, rec)
     epilogue = {}
@@ -243,7 +260,7 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
         grad_opacity = torch.zeros((H, W), dtype=torch.float32, device=dev)
     gc, gm2, gt, gno = f('GS_2D_render_backward')(m2, no, colors, tm, None, oo, oe, None, grad_image, grad_opacity,
                                                   grad_extras, None, ranges, point_list, nc, cam.near, cam.far,
-                                                  offsets if ordered_sums else None, radii, rec)
+                                                  offsets if ordered_sums else None, radii, rec, culled=keep)
     g_means3D, g_scales = torch.empty_like(scene.means3D), torch.empty_like(scene.scales)
     g_rot, g_opac, g_shs = torch.empty_like(scene.rotations), torch.empty_like(scene.opacities), torch.empty_like(scene.shs)
     f('gs_2d_preprocess_backward')(W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations,

@@ -41,12 +41,13 @@ int fsgs_stream_release(void* stream);
  * Every output row is written (zeros for rejected surfels); rows of means2D belonging to rejected surfels are left
  * untouched when means2D_preserve != 0 (the reference's caller-supplied means2D buffer). records (optional, [P,20],
  * 16-byte aligned, no counterpart in the reference) receives the packed per-surfel record of fsgs_gs_2d_pack_records
- * without a second pass over the outputs. */
+ * without a second pass over the outputs; keep_masks (optional, [P], no counterpart in the reference) the masks of
+ * fsgs_gs_2d_cull_masks, likewise. */
 int fsgs_gs_2d_preprocess_forward(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
     const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
     const float* Tw2v, const float* Tv2c, const float* campos, const float* trans_precomp, const uint8_t* culling,
     int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* normal_opacity, float* depths,
-    int32_t* radii, int32_t* tiles_touched, float* records, void* stream);
+    int32_t* radii, int32_t* tiles_touched, float* records, uint32_t* keep_masks, void* stream);
 
 /* gs_2d_preprocess_backward -- gs_2d_preprocess.cu:423-499 (kernel :268-329). Every row of g_* is ASSIGNED: the
  * gradient for surfels with radii > 0, zeros for the others and for SH coefficients above the active degree (the
@@ -106,6 +107,24 @@ int fsgs_gs_prepare_fill_counted(int P, int W, int H, const float* means2D, cons
                                  int64_t R, int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out,
                                  void* bins, size_t bins_bytes, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same two phases over the tiles a surfel can actually reach (no counterpart in the reference, whose lists hold
+ * every tile of a surfel's rectangle). fsgs_gs_2d_cull_masks evaluates the blend kernels' own bound -- the padded
+ * footprint box and diagonal slabs of the alpha >= 1/255 region -- once per surfel from its packed record
+ * (records[P,20]: transform, centre, opacity) and leaves masks[P]: a bit per tile of the surfel's rectangle, row-major,
+ * set when some pixel of the tile may blend the surfel (rectangles above 32 tiles: all bits set, kept whole). The
+ * culled phases leave the other instances out of the tile lists. Images, maps and gradients are the same as with the
+ * full lists; the lists are shorter (point_list keeps its length R, the entries behind the last tile's end are unused),
+ * n_contrib counts positions of the shorter lists, and the ordered-sum path of the backward must be entered through
+ * fsgs_gs_2d_render_backward_culled with the same masks. Tile grids above 16 384 tiles get the full lists. */
+int fsgs_gs_2d_cull_masks(int P, int W, int H, const float* records, const int32_t* radii, uint32_t* masks,
+                          void* stream);
+int fsgs_gs_prepare_count_culled(int P, int W, int H, const float* means2D, const int32_t* radii,
+                                 const uint32_t* masks, int64_t* ranges, void* bins, size_t bins_bytes, void* stream);
+int fsgs_gs_prepare_fill_counted_culled(int P, int W, int H, const float* means2D, const float* depths,
+                                        const int32_t* radii, const uint32_t* masks, int64_t R, int64_t* ranges,
+                                        int32_t* point_list, int64_t* sorted_keys_out, void* bins, size_t bins_bytes,
+                                        void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- per-tile alpha blend ------------------------------------------------------------------------------------- */
 
 /* Optional accelerator without a counterpart in the reference: packs what the blend kernels gather per surfel
@@ -147,6 +166,16 @@ int fsgs_gs_2d_render_backward(int P, int W, int H, double near_n, double far_n,
     const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
     float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
     size_t workspace_bytes, const float* records, void* stream);
+/* The same over lists built by fsgs_gs_prepare_*_culled (no counterpart in the reference): the sum of the ordered
+ * records reads the binning's keep masks (required with point_offsets) and skips the positions of a surfel's span that
+ * were left out of every list, which nobody wrote. R stays the scan's instance count. */
+int fsgs_gs_2d_render_backward_culled(int P, int W, int H, double near_n, double far_n, const float* means2D,
+    const float* normal_opacity, const float* colors, const float* trans_mat, const float* trans_mat_t2,
+    const float* out_opacity, const float* out_extras, const float* out_flow, const float* dL_dpix,
+    const float* dL_dopacity, const float* dL_dextras, const float* dL_dflow, const int64_t* ranges,
+    const int32_t* point_list, const int32_t* n_contrib, float* g_colors, float* g_means2D, float* g_trans,
+    float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
+    size_t workspace_bytes, const float* records, const uint32_t* keep_masks, void* stream);
 
 /* ---- "fast" surfel path: transform through camera intrinsics Tv2s[3,3], adjugate-based intersection, fused
  * corner-test binning. Optical flow (trans_mat_t2) is carried by the two blend entry points below. ---- */
