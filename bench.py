@@ -775,7 +775,8 @@ def main():
 
     P = scene.P
     Pv = int((out['radii'] > 0).sum())
-    R = int(out['point_list'].numel())
+    R = int(out['point_list'].numel())  # the reference's instance count: every tile of every surfel's rectangle
+    R_lists = int((out['ranges'][:, 1] - out['ranges'][:, 0]).sum())  # what the culled binning left in the tile lists
     HW = cam.W * cam.H
     T = ((cam.W + 15) // 16) * ((cam.H + 15) // 16)
     stage_ms = {}
@@ -855,10 +856,11 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": f"static 2DGS fwd+bwd: {P} surfels in the unit ball, {cam.W}x{cam.H}, FoV 40, radius 4, "
-                               "SH degree 3, white background, 16x16 tiles, per-tile binning of (tile, depth) keys, "
-                               "depth/normal outputs, fused per-pixel epilogue (composite, world normals, surf depth / "
-                               "normal) and its backward between the two blend passes",
-                   "P": P, "P_visible": Pv, "R": R, "tiles": T},
+                               "SH degree 3, white background, 16x16 tiles, per-tile binning of (tile, depth) keys "
+                               "(instances that no pixel of their tile can blend are left out of the lists: same images "
+                               "and gradients), depth/normal outputs, fused per-pixel epilogue (composite, world normals, "
+                               "surf depth / normal) and its backward between the two blend passes",
+                   "P": P, "P_visible": Pv, "R": R, "R_in_tile_lists": R_lists, "tiles": T},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(dominant),
                      "algorithmic_bytes_per_launch": bytes_dom, "valu_issue_frac": measured_valu_issue(dominant), "avg_launch_ms": stage_avg[dominant],

@@ -35,17 +35,18 @@ __device__ __forceinline__ CullBounds cull_bounds(const float* M, float ox, floa
   }
   c.state = 1;
   const float tau = 2.0f * __logf(oa) * 1.0001f + 1e-3f;
-  const float r2  = sqrtf(0.5f * tau);
+  // v_sqrt_f32 / v_rcp_f32 (1 ulp): the bound is padded by 1/8 pixel + 0.5 % of its extent
+  const float r2  = __builtin_amdgcn_sqrtf(0.5f * tau);
   const float u0 = M[0] - ox * M[6], u1 = M[1] - ox * M[7], u2 = M[2] - ox * M[8];
   const float v0 = M[3] - oy * M[6], v1 = M[4] - oy * M[7], v2 = M[5] - oy * M[8];
   const float d  = tau * (M[6] * M[6] + M[7] * M[7]) - M[8] * M[8];
   if (!((M[8] > 0.0f) && (d < -1e-6f * M[8] * M[8]))) return c;
-  const float inv = 1.0f / d, f0 = tau * inv, f2 = -inv;
+  const float inv = __builtin_amdgcn_rcpf(d), f0 = tau * inv, f2 = -inv;
   // centre and half extent of the footprint along direction (p0, p1, p2) = a combination of the two rows
   auto extent = [&](float p0, float p1, float p2, float& centre, float& half) {
     centre        = f0 * (p0 * M[6] + p1 * M[7]) + f2 * (p2 * M[8]);
     const float h = centre * centre - (f0 * (p0 * p0 + p1 * p1) + f2 * (p2 * p2));
-    half          = sqrtf(fmaxf(h, 0.0f));
+    half          = __builtin_amdgcn_sqrtf(fmaxf(h, 0.0f));
   };
   float cx, ex, cy, ey, ca, ea, cb, eb;
   extent(u0, u1, u2, cx, ex);
