@@ -133,11 +133,12 @@ static_assert(kCoopThreshold == kCullMaskTiles, "a lane's serial walk covers exa
 // Empty tiles get (0, 0) as the reference's zero-initialised ranges have. Tile grids above kMaxLdsTiles tiles (no room
 // for one LDS counter per tile) count and scatter with 64-bit global atomics on ranges[t].y instead (tile_emit_kernel).
 
-// Visits every (surfel, tile) pair; kScatter = false counts, true scatters.
+// Visits every (surfel, tile) pair; kScatter = false counts, true scatters. `masks` (optional): a surfel's keep mask,
+// the cleared bits of a rectangle of at most kCoopThreshold tiles are passed over.
 template <bool kScatter>
 __global__ void __launch_bounds__(256) tile_emit_kernel(int P, int gx, int gy, int64_t R,
     const float2* __restrict__ means2D, const float* __restrict__ depths, const int32_t* __restrict__ radii,
-    unsigned long long* __restrict__ ranges, uint64_t* __restrict__ entries) {
+    const uint32_t* __restrict__ masks, unsigned long long* __restrict__ ranges, uint64_t* __restrict__ entries) {
   const int i    = blockIdx.x * blockDim.x + threadIdx.x;
   const int lane = __lane_id();
   int x0 = 0, y0 = 0, w = 0, h = 0;
@@ -159,8 +160,10 @@ __global__ void __launch_bounds__(256) tile_emit_kernel(int P, int gx, int gy, i
   };
   const int count = w * h;
   if (count > 0 && count <= kCoopThreshold) {
+    uint32_t keep = masks ? masks[i] : 0xffffffffu;
     for (int y = 0; y < h; ++y)
-      for (int x = 0; x < w; ++x) visit((y0 + y) * gx + (x0 + x), dbits, i);
+      for (int x = 0; x < w; ++x, keep >>= 1)
+        if (keep & 1u) visit((y0 + y) * gx + (x0 + x), dbits, i);
   }
   unsigned long long big = __ballot(count > kCoopThreshold);
   while (big) {
@@ -971,7 +974,8 @@ int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, 
                        ranges);
     if (P > 0)
       hipLaunchKernelGGL(tile_emit_kernel<false>, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, (int64_t) 0,
-                         (const float2*) means2D, (const float*) nullptr, radii, rng, (uint64_t*) nullptr);
+                         (const float2*) means2D, (const float*) nullptr, radii, (const uint32_t*) cull_records, rng,
+                         (uint64_t*) nullptr);
     hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, false);
   }
   return check_launch("gs_prepare_count");
@@ -999,7 +1003,7 @@ int fill_sort(int P, int W, int H, const float* means2D, const float* depths, co
                        (const uint32_t*) ((const char*) bins + kBinsHeader), rng, entries);
   else
     hipLaunchKernelGGL(tile_emit_kernel<true>, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
-                       (const float2*) means2D, depths, radii, rng, entries);
+                       (const float2*) means2D, depths, radii, (const uint32_t*) cull_records, rng, entries);
   // the schedule table built by the counting part (or built now, on the global-atomic path, whose ranges only become
   // final with the scatter)
   const int* order = nullptr;
@@ -1060,8 +1064,8 @@ FSGS_API int fsgs_gs_2d_cull_masks(int P, int W, int H, const float* records, co
   return check_launch("gs_2d_cull_masks");
 }
 
-// The two phases of the binning over the kept tiles only (masks: fsgs_gs_2d_cull_masks). Tile grids too large for the
-// per-tile counters, and a process with the culling switched off for debugging, get the full lists.
+// The two phases of the binning over the kept tiles only (masks: fsgs_gs_2d_cull_masks). A process with the culling
+// switched off for debugging gets the full lists.
 FSGS_API int fsgs_gs_prepare_count_culled(int P, int W, int H, const float* means2D, const int32_t* radii,
                                           const uint32_t* masks, int64_t* ranges, void* bins, size_t bins_bytes,
                                           void* stream) {

@@ -115,7 +115,7 @@ int fsgs_gs_prepare_fill_counted(int P, int W, int H, const float* means2D, cons
  * culled phases leave the other instances out of the tile lists. Images, maps and gradients are the same as with the
  * full lists; the lists are shorter (point_list keeps its length R, the entries behind the last tile's end are unused),
  * n_contrib counts positions of the shorter lists, and the ordered-sum path of the backward must be entered through
- * fsgs_gs_2d_render_backward_culled with the same masks. Tile grids above 16 384 tiles get the full lists. */
+ * fsgs_gs_2d_render_backward_culled with the same masks. */
 int fsgs_gs_2d_cull_masks(int P, int W, int H, const float* records, const int32_t* radii, uint32_t* masks,
                           void* stream);
 int fsgs_gs_prepare_count_culled(int P, int W, int H, const float* means2D, const int32_t* radii,

@@ -3,6 +3,8 @@ the oracle that test_gpu_render_parity.py and test_gpu_fast_parity.py also run a
   * the per-quadrant culling of the blend kernels is exact: with it switched off (every staged surfel evaluated at every
     pixel, as the reference does) the forward outputs are identical bit for bit and the gradients agree to the rounding
     of the reordered atomic sums;
+  * the tile lists without the instances that no pixel of their tile can blend (the benchmark step's lists) give the
+    same maps bit for bit and the same gradients to rounding as the reference's full lists;
   * binning invariants: sorted masked keys, ranges partition [0, R) in tile order, every entry carries its tile's id;
   * the blend weights accumulated per surfel sum to the opacity image;
   * the backward is linear in the upstream gradients, and its two ways of summing a surfel's gradient over tiles
@@ -27,9 +29,9 @@ def _culling(enabled):
     lib.check(lib.load().fsgs_debug_set_culling(int(enabled)), 'debug_set_culling')
 
 
-def _render(scene, cam, gi, ge, go, ordered_sums=True, packed=True):
+def _render(scene, cam, gi, ge, go, ordered_sums=True, packed=True, cull=False):
     from fast_sp_gs_amd.renderer import render_step
-    out = render_step(scene, cam, gi, ge, go, ordered_sums=ordered_sums, packed=packed)
+    out = render_step(scene, cam, gi, ge, go, ordered_sums=ordered_sums, packed=packed, cull=cull)
     torch.cuda.synchronize()
     return out
 
@@ -101,6 +103,19 @@ def test_render_path_properties(config, device):
     for k in ('g_colors', 'g_trans', 'g_normal_opacity', 'g_means2D', 'g_means3D', 'g_scales', 'g_rot', 'g_opac', 'g_shs'):
         ref = a[k].abs().max().clamp_min(1e-30)
         assert float((a[k] - d[k]).abs().max() / ref) < 2e-5, k
+
+    # lists without the instances that no pixel of their tile can blend (what the benchmark step and _GS_2D_Render use)
+    # == the reference's full lists: maps bit for bit, gradients to the rounding of a different grouping of the sums
+    e = _render(scene, cam, gi, ge, go, cull=True)
+    n_full, n_cull = int((a['ranges'][:, 1] - a['ranges'][:, 0]).sum()), int((e['ranges'][:, 1] - e['ranges'][:, 0]).sum())
+    print(f"[full {config}] instances in the tile lists {n_full} -> {n_cull}", flush=True)
+    assert n_cull < n_full
+    for k in ('image', 'opacity', 'extras'):
+        assert torch.equal(a[k], e[k]), f"{k} depends on the culled lists"
+    for k in ('g_colors', 'g_trans', 'g_normal_opacity', 'g_means2D', 'g_means3D', 'g_scales', 'g_rot', 'g_opac', 'g_shs'):
+        ref = a[k].abs().max().clamp_min(1e-30)
+        assert float((a[k] - e[k]).abs().max() / ref) < 2e-5, k
+    del e
 
     # accumulated blend weights == opacity image (both are the sum of alpha * T over blended pairs)
     acc = torch.zeros(scene.P, device=device)
