@@ -528,7 +528,7 @@ def density_control_ms(dev, scene, reps: int = 5):
     return out
 
 
-def large_scene_ms(dev, views: int = 4, reps: int = 3):
+def large_scene_ms(dev, views: int = 4, reps: int = 3, cull: bool = False):
     """BASELINE config 4: 3M surfels, a batch of 4 views at 1352x1014 rendered forward + backward one after the other,
     and the K-NN of the 3M centres against 2048 control points with k = 8."""
     from fast_sp_gs_amd import scenes
@@ -544,7 +544,7 @@ def large_scene_ms(dev, views: int = 4, reps: int = 3):
 
     def batch():
         for cam in cams:
-            out = render_step(scene, cam, gi, ge, None, background=bg, cull=True)
+            out = render_step(scene, cam, gi, ge, None, background=bg, cull=cull)
         return out
 
     out = batch()
@@ -701,6 +701,10 @@ def main():
     ap.add_argument("--only", choices=["knn_large"], default=None,
                     help="run one side workload alone (for counter collections that must see a single kernel): "
                          "knn_large = K-NN of 3M points against 2048 control points, k = 8, three launches")
+    ap.add_argument("--culled-lists", action="store_true",
+                    help="time the step on tile lists without the (surfel, tile) instances that no pixel of their tile "
+                         "can blend (same images and gradients, shorter lists) instead of the reference's full lists; "
+                         "the default run reports that rate as extra_metrics.culled_lists_frames_per_s")
     ap.add_argument("--surfels", type=int, default=300_000)
     ap.add_argument("--size", type=int, default=800)
     args = ap.parse_args()
@@ -738,7 +742,7 @@ def main():
         # the fused per-pixel epilogue runs between the two blend passes, as in training: composite on the background,
         # normals to world space, surf_depth, pseudo surface normal; its backward supplies dL/dextras and the
         # composite's dL/dopacity = -sum_c dL/dimage_c * bg_c to the blend backward
-        return render_step(scene, cam, gi, ge, None, background=bg, cull=True)
+        return render_step(scene, cam, gi, ge, None, background=bg, cull=args.culled_lists)
 
     # The per-stage events of the timed steps are created and recorded once here, outside the timed region: the runtime
     # grows its event pool in bursts that stall the host for tens of milliseconds.
@@ -776,7 +780,7 @@ def main():
     P = scene.P
     Pv = int((out['radii'] > 0).sum())
     R = int(out['point_list'].numel())  # the reference's instance count: every tile of every surfel's rectangle
-    R_lists = int((out['ranges'][:, 1] - out['ranges'][:, 0]).sum())  # what the culled binning left in the tile lists
+    R_lists = int((out['ranges'][:, 1] - out['ranges'][:, 0]).sum())  # R, or what the culled binning left in the lists
     HW = cam.W * cam.H
     T = ((cam.W + 15) // 16) * ((cam.H + 15) // 16)
     stage_ms = {}
@@ -820,6 +824,24 @@ def main():
     copy_gbps = copy_probe_gbps(dev)
     extra = {"knn_topk_queries_per_s": pts.shape[0] / (knn_ms * 1e-3), "knn_topk_workload": "200000 x 512, k=4, D=3"}
     extra["standalone_ops"] = standalone_ops(dev, copy_gbps)
+    if not args.no_extras and not args.counter_run and not args.culled_lists:
+        # the same step on culled tile lists: identical images and gradients from shorter lists (what _GS_2D_Render uses)
+        for _ in range(max(args.warmup, 2)):
+            culled = render_step(scene, cam, gi, ge, None, background=bg, cull=True)
+        torch.cuda.synchronize()
+        gc.collect()
+        gc.disable()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            culled = render_step(scene, cam, gi, ge, None, background=bg, cull=True)
+        torch.cuda.synchronize()
+        extra["culled_lists_frames_per_s"] = args.steps / (time.perf_counter() - t0)
+        gc.enable()
+        extra["culled_lists_instances"] = int((culled['ranges'][:, 1] - culled['ranges'][:, 0]).sum())
+        extra["culled_lists_workload"] = ("the benchmark step with GS_prepare(cull=True): instances that no pixel of "
+                                          "their tile can blend are left out of the tile lists; images bit-identical, "
+                                          "gradients equal to rounding")
+        del culled
     if not args.no_extras:
         extra.update(ssim_rate(dev))
         extra.update(simple_knn_ms(dev, scene))
@@ -829,6 +851,7 @@ def main():
         extra.update(gs3d_path_rate(dev, scene, cam, gi))
         extra.update(density_control_ms(dev, scene))
         extra.update(large_scene_ms(dev))
+        extra["large_scene_culled_lists_views_per_s"] = large_scene_ms(dev, cull=True)["large_scene_views_per_s"]
         (extra["fast_path_frames_per_s"], extra["fast_path_atomic_sums_frames_per_s"]), fast_bwd = fast_path_rate(dev, scene, cam, gi)
         extra["fast_path_workload"] = "same scene through GS_2D_fast_* (corner-test binning keeps fewer instances)"
         extra["fast_backward_tile_kernel_ms"] = fast_bwd["tile"]
@@ -857,8 +880,10 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"static 2DGS fwd+bwd: {P} surfels in the unit ball, {cam.W}x{cam.H}, FoV 40, radius 4, "
                                "SH degree 3, white background, 16x16 tiles, per-tile binning of (tile, depth) keys "
-                               "(instances that no pixel of their tile can blend are left out of the lists: same images "
-                               "and gradients), depth/normal outputs, fused per-pixel epilogue (composite, world normals, "
+                               + ("(instances that no pixel of their tile can blend are left out of the lists: same "
+                                  "images and gradients)" if args.culled_lists else
+                                  "(every tile of every surfel's rectangle: the reference's lists, bit for bit)")
+                               + ", depth/normal outputs, fused per-pixel epilogue (composite, world normals, "
                                "surf depth / normal) and its backward between the two blend passes",
                    "P": P, "P_visible": Pv, "R": R, "R_in_tile_lists": R_lists, "tiles": T},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",

@@ -1,4 +1,4 @@
-"""The culled binning of the standard path (GS_prepare(..., cull=True), what `_GS_2D_Render` and the benchmark use):
+"""The culled binning of the standard path (GS_prepare(..., cull=True), what `_GS_2D_Render` uses and what the benchmark reports beside its headline):
 (surfel, tile) instances that no pixel of their tile can blend are left out of the tile lists. The reference's lists hold
 every tile of a surfel's rectangle, so the lists differ by construction; what must not change is everything computed
 from them. Checked here: every tile's culled list is the full list with entries removed (order kept), the forward's

@@ -3,7 +3,7 @@ the oracle that test_gpu_render_parity.py and test_gpu_fast_parity.py also run a
   * the per-quadrant culling of the blend kernels is exact: with it switched off (every staged surfel evaluated at every
     pixel, as the reference does) the forward outputs are identical bit for bit and the gradients agree to the rounding
     of the reordered atomic sums;
-  * the tile lists without the instances that no pixel of their tile can blend (the benchmark step's lists) give the
+  * the tile lists without the instances that no pixel of their tile can blend (what _GS_2D_Render bins) give the
     same maps bit for bit and the same gradients to rounding as the reference's full lists;
   * binning invariants: sorted masked keys, ranges partition [0, R) in tile order, every entry carries its tile's id;
   * the blend weights accumulated per surfel sum to the opacity image;
@@ -104,7 +104,7 @@ def test_render_path_properties(config, device):
         ref = a[k].abs().max().clamp_min(1e-30)
         assert float((a[k] - d[k]).abs().max() / ref) < 2e-5, k
 
-    # lists without the instances that no pixel of their tile can blend (what the benchmark step and _GS_2D_Render use)
+    # lists without the instances that no pixel of their tile can blend (what _GS_2D_Render uses)
     # == the reference's full lists: maps bit for bit, gradients to the rounding of a different grouping of the sums
     e = _render(scene, cam, gi, ge, go, cull=True)
     n_full, n_cull = int((a['ranges'][:, 1] - a['ranges'][:, 0]).sum()), int((e['ranges'][:, 1] - e['ranges'][:, 0]).sum())
