@@ -282,11 +282,13 @@ def gs_2d_compute_trans_mat_backward(W, H, means3D, scales, rotations, Tw2v, Tw2
 def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, tiles_touched: Tensor,
                debug: bool = False, return_keys: bool = False, return_offsets: bool = False,
                overlap=None, records: Optional[Tensor] = None, cull: bool = False,
-               keep_masks: Optional[Tensor] = None) -> List[Tensor]:
+               keep_masks: Optional[Tensor] = None, store_offsets: bool = True) -> List[Tensor]:
     """gaussian_prepare.cu:282-308 -> [ranges[T,2] int64, point_list[R] int32] (+ sorted keys, + the prefix scan of
     tiles_touched, which GS_2D_render_backward can use to sum gradients without atomics). `overlap(offsets)`, if given,
     is called once the scan is queued and before the host waits for the instance count; its result is appended.
-    `records` (gs_2d_preprocess_forward(..., return_records=True)): the scan stores every surfel's offset into its record.
+    `records` (gs_2d_preprocess_forward(..., return_records=True)): the scan stores every surfel's offset into its record
+    unless `store_offsets` is False (the blend backward then takes the offsets from the scan's own output, which it is
+    given anyway; the 4-byte stores into 80-byte records cost the scan more than the backward's extra read).
     `cull` (needs `records`, or the `keep_masks` the preprocess wrote; no counterpart in the reference): instances that no pixel of their tile can blend are left
     out of the lists -- same images and gradients from shorter lists; point_list keeps its length R, the entries behind
     the last tile's end are unused, n_contrib counts positions of the shorter lists. The per-surfel keep masks [P] int32
@@ -326,7 +328,7 @@ def GS_prepare(W: int, H: int, means2D: Tensor, depths: Tensor, radii: Tensor, t
     # the device works while the host waits for the copy and allocates.
     with _timed('gs_prepare_scan'):
         rc = lib.fsgs_gs_prepare_scan_begin(P, L.ptr(tiles_touched), L.ptr(offsets), L.ptr(ws1), ws1.numel(),
-                                            count.data_ptr(), L.ptr(records), stream)
+                                            count.data_ptr(), L.ptr(records) if store_offsets else None, stream)
     L.check(rc, what)
     with _timed('gs_prepare_fill'):  # first of the operator's two parts: callers that time stages add them up
         if cull:
