@@ -339,21 +339,27 @@ def gs3d_path_rate(dev, scene, cam, gi, steps: int = 30, warmup: int = 5):
     go = -gi.sum(0)  # white-background composite
     R = [0]
 
-    def step(ordered=True):
+    def step(ordered=True, cull=False):
         m2, dep, col, rad, tt, c3, co = f('gs_preprocess_forward')(
             W, H, 3, False, scene.means3D, scales, scene.rotations, scene.opacities, scene.shs, None, cam.Tw2v,
             cam.Tv2c, cam.campos, tan_fov, None, None, None, None)
-        ranges, pl, offsets = f('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True)
+        # cull: lists without the (Gaussian, tile) instances that no pixel of their tile can blend (what
+        # RasterizeGaussians bins by default); otherwise the reference's lists
+        keep = f('gs_cull_masks')(W, H, m2, co, rad) if cull else None
+        ranges, pl, offsets = f('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True, cull=cull,
+                                              keep_masks=keep)[:3]
         oc, oo, _, nc = f('gaussian_rasterize_forward')(W, H, m2, co, col, None, pl, ranges)
-        # per-Gaussian sums through ordered per-instance records (what RasterizeGaussians does), or the reference's atomics
+        # per-Gaussian sums through ordered per-instance records, or the reference's atomics (RasterizeGaussians' default)
         g_col, _, g_m2, g_co = f('gaussian_rasterize_backward')(m2, co, col, None, oo, gi, go, None, ranges, pl, nc,
-                                                                offsets if ordered else None, rad if ordered else None)
+                                                                offsets if ordered else None, rad if ordered else None,
+                                                                culled=keep if ordered else None)
         g3, gs, gq = torch.empty_like(scene.means3D), torch.empty_like(scales), torch.empty_like(scene.rotations)
         gop, gsh = torch.empty_like(scene.opacities), torch.empty_like(scene.shs)
         f('gs_preprocess_backward')(W, H, 3, False, scene.means3D, scales, scene.rotations, scene.opacities, scene.shs,
                                     None, cam.Tw2v, cam.Tv2c, cam.campos, tan_fov, c3, None, rad, col, g_m2, None, g_col,
                                     g_co, g3, gs, gq, gop, gsh, None, None)
-        R[0] = pl.numel()
+        if not cull:
+            R[0] = pl.numel()
         return m2, co, ranges, pl, nc, oo
 
     for _ in range(warmup):
@@ -374,7 +380,17 @@ def gs3d_path_rate(dev, scene, cam, gi, steps: int = 30, warmup: int = 5):
         step(False)
     torch.cuda.synchronize()
     dt_atomic = time.perf_counter() - t0
+    for _ in range(warmup):
+        culled_state = step(False, True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(False, True)
+    torch.cuda.synchronize()
+    dt_culled = time.perf_counter() - t0
     gc.enable()
+    R_culled = int((culled_state[2][:, 1] - culled_state[2][:, 0]).sum())
+    del culled_state
 
     # a 16-channel feature table blended with the finished view's weights, and its backward
     m2, co, ranges, pl, nc, oo = state
@@ -412,6 +428,8 @@ def gs3d_path_rate(dev, scene, cam, gi, steps: int = 30, warmup: int = 5):
 
     return {"gs3d_path_frames_per_s": steps / dt,
             "gs3d_path_atomic_sums_frames_per_s": steps / dt_atomic,
+            "gs3d_path_culled_lists_atomic_sums_frames_per_s": steps / dt_culled,
+            "gs3d_path_culled_lists_instances": R_culled,
             "gs3d_backward_tile_kernel_ms": bwd_ms["tile"],
             "gs3d_backward_per_gaussian_kernel_ms": bwd_ms["per_gaussian"],
             "gs3d_backward_workload": f"gaussian_rasterize_fast_backward on that view with atomic sums, {b2t.numel()} "

@@ -21,7 +21,7 @@ __all__ = [
     'SH_to_RGB_forward', 'SH_to_RGB_backward', 'sh_encode_forward', 'sh_encode_backward', 'freq_encode_forward',
     'freq_encode_backward', 'cdist_top', 'cdist_top_backward', 'AdamMasksedUpdated', 'knn_topk', 'lbs_blend',
     'knn_topk_backward', 'lbs_blend_backward',
-    'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'mlp_pack_transposed', 'mlp_backward', 'gs_2d_pack_records', 'gs_2d_fast_preprocess_forward',
+    'gs_2d_topk_weights', 'mlp_pack_weights', 'mlp_forward', 'mlp_pack_transposed', 'mlp_backward', 'gs_2d_pack_records', 'gs_cull_masks', 'gs_2d_fast_preprocess_forward',
     'gs_2d_fast_preprocess_backward', 'gs_2d_fast_compute_transmat_forward', 'gs_2d_fast_compute_trans_mat_backward',
     'GS_2D_fast_render_forward', 'GS_2D_fast_render_backward', 'fusedssim', 'fusedssim_backward',
     'gs_2d_epilogue_forward', 'gs_2d_epilogue_backward', 'simple_knn', 'gs_preprocess_forward',
@@ -412,6 +412,27 @@ def GS_2D_render_forward(width: int, height: int, means2D: Tensor, colors: Tenso
             L.current_stream())
     L.check(rc, what)
     return pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib
+
+
+def gs_cull_masks(W: int, H: int, means2D: Tensor, conic_opacity: Tensor, radii: Tensor) -> Tensor:
+    """-> keep_masks[P] int32 for 3D Gaussians (no reference counterpart): a bit per tile of a Gaussian's rectangle, set
+    when some pixel of the tile can reach alpha >= 1/255; `GS_prepare(..., cull=True, keep_masks=...)` leaves the other
+    (Gaussian, tile) instances out of the tile lists, and `gaussian_rasterize_backward(..., culled=...)` must get the
+    masks when it sums ordered records."""
+    what = 'gs_cull_masks'
+    _f32(what, means2D=means2D, conic_opacity=conic_opacity)
+    L.require_cuda(what, radii=radii)
+    L.require_dtype(what, 'radii', radii, torch.int32)
+    P = means2D.shape[0]
+    L.require_shape(what, 'means2D', means2D, P, 2)
+    L.require_shape(what, 'conic_opacity', conic_opacity, P, 4)
+    L.require_shape(what, 'radii', radii, P)
+    masks = torch.empty((max(P, 1),), dtype=torch.int32, device=means2D.device)
+    with _timed(what):
+        rc = _lib().fsgs_gs_cull_masks(P, W, H, L.ptr(means2D.contiguous()), L.ptr(conic_opacity.contiguous()),
+                                       L.ptr(radii.contiguous()), L.ptr(masks), L.current_stream())
+    L.check(rc, what)
+    return masks
 
 
 def gs_2d_pack_records(means2D: Tensor, colors: Tensor, normal_opacity: Tensor, trans_mat: Tensor,
@@ -2048,10 +2069,11 @@ def gaussian_rasterize_backward(means2D: Tensor, conic_opacity: Tensor, colors: 
                                 out_opacity: Tensor, dL_dout_color: Tensor, dL_dout_opacity: Tensor,
                                 dL_dout_extra: Optional[Tensor], ranges: Tensor, point_list: Tensor,
                                 n_contrib: Tensor, point_offsets: Optional[Tensor] = None,
-                                radii: Optional[Tensor] = None):
+                                radii: Optional[Tensor] = None, culled: Optional[Tensor] = None):
     """gaussian_render.cu:486-536 -> (dL_dcolors[P,3], dL_dextras[P,E]|None, dL_dmeans2D[P,2], dL_dconic_opacity[P,4]).
     With `point_offsets` (GS_prepare(..., return_offsets=True)) and `radii` the per-Gaussian sums are taken in a fixed
-    order from per-instance records instead of with atomics."""
+    order from per-instance records instead of with atomics; `culled`: the keep masks, when the lists were built by
+    GS_prepare(..., cull=True) (the records of the instances left out are zeroed first)."""
     what = 'gaussian_rasterize_backward'
     L.require_cuda(what, dL_dout_color=dL_dout_color, dL_dout_opacity=dL_dout_opacity, dL_dout_extra=dL_dout_extra)
     P = means2D.shape[0]
@@ -2076,12 +2098,22 @@ def gaussian_rasterize_backward(means2D: Tensor, conic_opacity: Tensor, colors: 
     args = [c(means2D), c(conic_opacity), c(colors), c(extras) if E else None, c(out_opacity), c(n_contrib),
             c(dL_dout_color), c(dL_dout_extra) if E else None, c(dL_dout_opacity), c(point_list), c(ranges)]
     with _timed('gaussian_rasterize_backward'):
+        if ordered and culled is not None:
+            _clear_culled_records(what, P, R, point_offsets, culled, ws)
         rc = _lib().fsgs_gaussian_rasterize_backward(
             P, W, H, E, *[L.ptr(a) for a in args], L.ptr(dL_dmeans2D), L.ptr(dL_dconic_o), L.ptr(dL_dcolors),
             L.ptr(dL_dextras), R, L.ptr(point_offsets) if ordered else None, L.ptr(radii) if ordered else None,
             L.ptr(ws), ws.numel() if ws is not None else 0, L.current_stream())
     L.check(rc, what)
     return dL_dcolors, dL_dextras, dL_dmeans2D, dL_dconic_o
+
+
+def _clear_culled_records(what, P, R, point_offsets, keep_masks, ws):
+    L.require_cuda(what, culled=keep_masks)
+    L.require_dtype(what, 'culled', keep_masks, torch.int32)
+    L.require_shape(what, 'culled', keep_masks, max(P, 1))
+    L.check(_lib().fsgs_gaussian_rasterize_clear_culled(P, R, L.ptr(point_offsets), L.ptr(keep_masks), L.ptr(ws),
+                                                        ws.numel(), L.current_stream()), what)
 
 
 def _ordered_sum_inputs(what, P, point_list, point_offsets, radii, workspace_bytes_fn, device):
@@ -2110,7 +2142,8 @@ def gaussian_rasterize_fast_backward(means2D: Tensor, conic_opacity: Tensor, col
                                      ranges: Tensor, point_list: Tensor, n_contrib: Tensor, max_contrib: Tensor,
                                      per_tile_bucket_offset: Tensor, bucket_to_tile: Tensor, sampled_T: Tensor,
                                      sampled_ar: Tensor, point_offsets: Optional[Tensor] = None,
-                                     radii: Optional[Tensor] = None, per_gaussian: Optional[bool] = None):
+                                     radii: Optional[Tensor] = None, per_gaussian: Optional[bool] = None,
+                                     culled: Optional[Tensor] = None):
     """gaussian_render.cu:760-812 -> (dL_dcolors[P,3], dL_dextras[P,E]|None, dL_dmeans2D[P,2], dL_dconic_opacity[P,4]):
     the reference's per-Gaussian backward over the forward's bucket snapshots. The same derivative as
     gaussian_rasterize_backward; by default it is evaluated by that operator's back-to-front kernel (the faster one on
@@ -2152,6 +2185,8 @@ def gaussian_rasterize_fast_backward(means2D: Tensor, conic_opacity: Tensor, col
     tail = (L.ptr(dL_dmeans2D), L.ptr(dL_dconic_o), L.ptr(dL_dcolors), L.ptr(dL_dextras), R,
             L.ptr(point_offsets) if ordered else None, L.ptr(radii) if ordered else None, L.ptr(ws),
             ws.numel() if ws is not None else 0, L.current_stream())
+    if ordered and culled is not None:  # lists from GS_prepare(..., cull=True): see gaussian_rasterize_backward
+        _clear_culled_records(what, P, R, point_offsets, culled, ws)
     if PER_GAUSSIAN_BACKWARD if per_gaussian is None else per_gaussian:
         with _timed('gaussian_rasterize_bucket_backward'):
             rc = _lib().fsgs_gaussian_rasterize_bucket_backward(P, W, H, E, B, *[L.ptr(a) for a in args], *tail)

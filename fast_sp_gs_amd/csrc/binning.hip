@@ -238,6 +238,30 @@ __device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, 
   }
 }
 
+// One lane per 3D Gaussian: the keep mask of its rectangle from its projected mean, conic and opacity.
+__global__ void __launch_bounds__(256) conic_cull_mask_kernel(int P, int gx, int gy, const float2* __restrict__ means2D,
+    const float4* __restrict__ conic_opacity, const int32_t* __restrict__ radii, uint32_t* __restrict__ masks) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= P) return;
+  uint32_t m = 0xffffffffu;
+  const int radius = radii[i];
+  if (radius > 0) {
+    const float2 c    = means2D[i];
+    const TileRect r  = tile_rect(c.x, c.y, radius, gx, gy);
+    const int w = max(r.x1 - r.x0, 0), h = max(r.y1 - r.y0, 0);
+    if (w * h <= kCullMaskTiles) {
+      const float4 co     = conic_opacity[i];
+      const CullBounds cb = conic_cull_bounds(co.x, co.y, co.z, co.w);
+      m = 0u;
+      int e = 0;
+      for (int y = 0; y < h; ++y)
+        for (int x = 0; x < w; ++x, ++e)
+          if (cull_keeps_tile(cb, c.x, c.y, r.x0 + x, r.y0 + y)) m |= 1u << e;
+    }
+  }
+  masks[i] = m;
+}
+
 // One lane per surfel: the keep mask of its rectangle (see kCullMaskTiles) from its packed record.
 __global__ void __launch_bounds__(256) cull_mask_kernel(int P, int gx, int gy, const float4* __restrict__ records,
                                                         const int32_t* __restrict__ radii, uint32_t* __restrict__ masks) {
@@ -1063,6 +1087,21 @@ FSGS_API int fsgs_gs_2d_cull_masks(int P, int W, int H, const float* records, co
   hipLaunchKernelGGL(cull_mask_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, gx, gy,
                      (const float4*) records, radii, masks);
   return check_launch("gs_2d_cull_masks");
+}
+
+// The same for 3D Gaussians, from the tensors their preprocess leaves (gaussian_rasterize's alpha test in place of the
+// surfel's).
+FSGS_API int fsgs_gs_cull_masks(int P, int W, int H, const float* means2D, const float* conic_opacity,
+                                const int32_t* radii, uint32_t* masks, void* stream) {
+  FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "gs_cull_masks: bad sizes");
+  if (P == 0) return kOk;
+  FSGS_REQUIRE(means2D && conic_opacity && radii && masks, "gs_cull_masks: null pointer");
+  FSGS_REQUIRE(((uintptr_t) conic_opacity & 15) == 0 && ((uintptr_t) means2D & 7) == 0,
+               "gs_cull_masks: means2D / conic_opacity must be 8 / 16-byte aligned");
+  const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+  hipLaunchKernelGGL(conic_cull_mask_kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, gx, gy,
+                     (const float2*) means2D, (const float4*) conic_opacity, radii, masks);
+  return check_launch("gs_cull_masks");
 }
 
 // The two phases of the binning over the kept tiles only (masks: fsgs_gs_2d_cull_masks). A process with the culling

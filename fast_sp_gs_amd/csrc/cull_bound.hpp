@@ -67,6 +67,37 @@ __device__ __forceinline__ CullBounds cull_bounds(const float* M, float ox, floa
   return c;
 }
 
+// The same for a 3D Gaussian's screen-space conic Q = [[a, b], [b, c]] (offsets relative to its projected mean): alpha =
+// min(0.99, o exp(-d^T Q d / 2)) >= 1/255 inside the ellipse d^T Q d <= tau = 2 ln(255 o), whose half extent along a
+// direction n is sqrt(tau n^T Q^-1 n): sqrt(tau c / det), sqrt(tau a / det) along the axes, sqrt(tau (a + c -+ 2 b) /
+// det) along x + y and x - y. A conic that is not positive definite has no finite bound (state 1).
+__device__ __forceinline__ CullBounds conic_cull_bounds(float a, float b, float c, float opacity) {
+#pragma clang fp contract(off)
+  CullBounds r;
+  r.x0 = r.y0 = r.a0 = r.b0 = -1e30f, r.x1 = r.y1 = r.a1 = r.b1 = 1e30f;
+  const float oa = 255.0f * opacity;
+  if (!(oa >= 1.0f)) {
+    r.state = 0;
+    return r;
+  }
+  r.state = 1;
+  const float det = a * c - b * b;
+  if (!(det > 0.0f) || !(a > 0.0f)) return r;
+  const float tau = 2.0f * (__logf(oa) * 1.0001f + 1e-3f);
+  const float s   = tau / det;
+  const float ex = sqrtf(s * c), ey = sqrtf(s * a);
+  if (!(ex == ex) || !(ey == ey)) return r;
+  const float padx = kCullPad + 0.01f * ex, pady = kCullPad + 0.01f * ey;
+  r.x0 = -(ex + padx), r.x1 = ex + padx, r.y0 = -(ey + pady), r.y1 = ey + pady;
+  r.state = 2;
+  const float ea = sqrtf(s * fmaxf(a + c - 2.0f * b, 0.0f)), eb = sqrtf(s * fmaxf(a + c + 2.0f * b, 0.0f));
+  if ((ea == ea) && (eb == eb)) {
+    const float pa = 1.5f * kCullPad + 0.01f * ea, pb = 1.5f * kCullPad + 0.01f * eb;
+    r.a0 = -(ea + pa), r.a1 = ea + pa, r.b0 = -(eb + pb), r.b1 = eb + pb;
+  }
+  return r;
+}
+
 // true: some pixel of tile (tile_x, tile_y) may blend the surfel. The four quadrant tests of quadrant_mask folded into
 // one over the tile's 16x16 pixel centres (it only lets through, in addition, footprints that fit between two
 // quadrants' pixel centres).

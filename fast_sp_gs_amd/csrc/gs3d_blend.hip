@@ -956,6 +956,39 @@ FSGS_API size_t fsgs_gaussian_rasterize_backward_workspace_bytes(int64_t R) {
   return slot_workspace_bytes(R, kG3Slots);
 }
 
+// Tile lists built by the culled binning leave out the instances whose keep bit is clear; no block stages them, so no
+// block writes (or clears) their records, and the ordered sum reads every position of a Gaussian's span. Four lanes
+// per Gaussian zero those records, 16 bytes each.
+__global__ void __launch_bounds__(256) clear_culled_records_kernel(int P, const int64_t* __restrict__ point_offsets,
+    const uint32_t* __restrict__ keep_masks, float* __restrict__ records) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x, i = t >> 2, part = t & 3;
+  if (i >= P) return;
+  const int64_t e0 = i > 0 ? point_offsets[i - 1] : 0, e1 = point_offsets[i];
+  const int64_t count = e1 - e0;
+  if (count <= 0 || count > 32) return;  // rectangles above 32 tiles are kept whole
+  uint32_t dropped = ~keep_masks[i] & (count == 32 ? 0xffffffffu : (1u << (int) count) - 1u);
+  while (dropped) {
+    const int j = __builtin_ctz(dropped);
+    dropped &= dropped - 1u;
+    ((float4*) (records + (size_t) (e0 + j) * kG3Slots))[part] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  }
+}
+
+FSGS_API int fsgs_gaussian_rasterize_clear_culled(int P, int64_t R, const int64_t* point_offsets,
+    const uint32_t* keep_masks, void* workspace, size_t workspace_bytes, void* stream) {
+  static_assert(kG3Slots == 16, "four lanes of 16 bytes per record");
+  FSGS_REQUIRE(P >= 0 && R >= 0, "gaussian_rasterize_clear_culled: bad sizes");
+  if (P == 0 || R == 0) return kOk;
+  FSGS_REQUIRE(point_offsets && keep_masks && workspace, "gaussian_rasterize_clear_culled: null pointer");
+  FSGS_REQUIRE(((uintptr_t) workspace & 15) == 0, "gaussian_rasterize_clear_culled: workspace must be 16-byte aligned");
+  if (workspace_bytes < slot_workspace_bytes(R, kG3Slots))
+    return fail(kWorkspaceSmall, "gaussian_rasterize_clear_culled: workspace %zu < %zu bytes", workspace_bytes,
+                slot_workspace_bytes(R, kG3Slots));
+  hipLaunchKernelGGL(clear_culled_records_kernel, dim3((unsigned) div_up(4 * (int64_t) P, 256)), dim3(256), 0,
+                     (hipStream_t) stream, P, point_offsets, keep_masks, (float*) workspace);
+  return check_launch("gaussian_rasterize_clear_culled");
+}
+
 FSGS_API int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const float* means2D,
     const float* conic_opacity, const float* colors, const float* extras, const float* out_opacity,
     const int32_t* n_contrib, const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity,

@@ -13,6 +13,8 @@ from torch import Tensor
 from fast_sp_gs_amd._C import get_C_function
 from fast_sp_gs_amd.renderer.gs_2d_render import GS_prepare
 
+_cull_masks = get_C_function('gs_cull_masks')
+
 __all__ = ['RasterizeBuffer3D', 'preprocess', 'GS_render', 'GS_render_fast', 'RasterizeGaussians', 'render',
            'compute_cov3D', 'compute_cov2D', 'topk_weights', 'render_extra']
 
@@ -197,6 +199,10 @@ def preprocess(means3D: Tensor, scales: Tensor, rotations: Tensor, opacities: Te
 # Gaussians, 800x800, because a Gaussian's record is small and the records' fill and second pass cost more than its few
 # atomics); True = per-instance records added in a fixed order, so that the sums do not vary from run to run.
 DETERMINISTIC_SUMS = False
+# `RasterizeGaussians` bins without the (Gaussian, tile) instances that no pixel of their tile can blend (the ellipse on
+# which alpha reaches 1/255 against each tile of the 3-sigma rectangle): same images and gradients from shorter lists;
+# the lists and n_contrib in RasterizeBuffer3D are the shorter ones. False: the reference's lists.
+CULL_LISTS = True
 
 
 class _GS_render(torch.autograd.Function):
@@ -205,12 +211,12 @@ class _GS_render(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, W, H, mean2D, colors, conic_opacity, tile_range, point_list, extras, accum_max_count,
-                accum_weights_p, accum_weights_count, point_offsets=None, radii=None):
+                accum_weights_p, accum_weights_count, point_offsets=None, radii=None, keep_masks=None):
         images, out_opacity, out_extras, n_contrib = _GS_render._forward(
             W, H, mean2D, conic_opacity, colors, extras, point_list, tile_range, accum_max_count, accum_weights_p,
             accum_weights_count, None)
         ctx.save_for_backward(mean2D, colors, conic_opacity, extras, tile_range, point_list, out_opacity, n_contrib,
-                              point_offsets, radii)
+                              point_offsets, radii, keep_masks)
         ctx.mark_non_differentiable(n_contrib)
         return images, out_opacity, out_extras, n_contrib
 
@@ -218,7 +224,7 @@ class _GS_render(torch.autograd.Function):
     @torch.autograd.function.once_differentiable
     def backward(ctx, grad_images, grad_alpha, grad_out_extra, _):
         (mean2D, colors, conic_opacity, extras, tile_range, point_list, out_opacity, n_contrib, point_offsets,
-         radii) = ctx.saved_tensors
+         radii, keep_masks) = ctx.saved_tensors
         zeros_like = lambda t: torch.zeros_like(t)
         grad_images = zeros_like(out_opacity).expand(3, -1, -1).contiguous() if grad_images is None else grad_images
         grad_alpha = zeros_like(out_opacity) if grad_alpha is None else grad_alpha
@@ -228,9 +234,9 @@ class _GS_render(torch.autograd.Function):
         grad_colors, grad_extra, grad_means2D, grad_conic_opacity = _GS_render._backward(
             mean2D, conic_opacity, colors, extras, out_opacity, grad_images.contiguous(), grad_alpha.contiguous(),
             None if grad_out_extra is None else grad_out_extra.contiguous(), tile_range, point_list, n_contrib,
-            point_offsets, radii)
+            point_offsets, radii, culled=keep_masks)
         return (None, None, grad_means2D, grad_colors, grad_conic_opacity, None, None, grad_extra, None, None, None,
-                None, None)
+                None, None, None)
 
 
 class _GS_render_fast(torch.autograd.Function):
@@ -241,7 +247,7 @@ class _GS_render_fast(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, W, H, mean2D, colors, conic_opacity, tile_range, point_list, extras, accum_max_count,
-                accum_weights_p, accum_weights_count, point_offsets=None, radii=None):
+                accum_weights_p, accum_weights_count, point_offsets=None, radii=None, keep_masks=None):
         per_tile_bucket_offset = (tile_range[..., 1] - tile_range[..., 0] + 31) // 32
         per_tile_bucket_offset = torch.cumsum(per_tile_bucket_offset, dim=-1).contiguous()
         (images, out_opacity, out_extras, n_contrib, max_contrib, bucket_to_tile, sampled_T,
@@ -250,7 +256,7 @@ class _GS_render_fast(torch.autograd.Function):
                                                 per_tile_bucket_offset)
         ctx.save_for_backward(mean2D, colors, conic_opacity, extras, tile_range, point_list, images, out_opacity,
                               out_extras, n_contrib, per_tile_bucket_offset, max_contrib, bucket_to_tile, sampled_T,
-                              sampled_ar, point_offsets, radii)
+                              sampled_ar, point_offsets, radii, keep_masks)
         ctx.mark_non_differentiable(n_contrib)
         return images, out_opacity, out_extras, n_contrib
 
@@ -259,7 +265,7 @@ class _GS_render_fast(torch.autograd.Function):
     def backward(ctx, grad_images, grad_alpha, grad_out_extra, _):
         (mean2D, colors, conic_opacity, extras, tile_range, point_list, images, out_opacity, out_extras, n_contrib,
          per_tile_bucket_offset, max_contrib, bucket_to_tile, sampled_T, sampled_ar, point_offsets,
-         radii) = ctx.saved_tensors
+         radii, keep_masks) = ctx.saved_tensors
         grad_images = torch.zeros_like(images) if grad_images is None else grad_images
         grad_alpha = torch.zeros_like(out_opacity) if grad_alpha is None else grad_alpha
         if extras is not None and grad_out_extra is None:
@@ -268,28 +274,31 @@ class _GS_render_fast(torch.autograd.Function):
             mean2D, conic_opacity, colors, extras, images, out_extras, out_opacity, grad_images.contiguous(),
             grad_alpha.contiguous(), None if grad_out_extra is None else grad_out_extra.contiguous(), tile_range,
             point_list, n_contrib, max_contrib, per_tile_bucket_offset, bucket_to_tile, sampled_T, sampled_ar,
-            point_offsets, radii)
+            point_offsets, radii, culled=keep_masks)
         return (None, None, grad_means2D, grad_colors, grad_conic_opacity, None, None, grad_extra, None, None, None,
-                None, None)
+                None, None, None)
 
 
 def GS_render_fast(W: int, H: int, mean2D: Tensor, colors: Tensor, conic_opacity: Tensor, tile_range: Tensor,
                    point_list: Tensor, extra: Tensor = None, accum_max_count=None, accum_weights_p=None,
-                   accum_weights_count=None, point_offsets: Tensor = None, radii: Tensor = None):
+                   accum_weights_count=None, point_offsets: Tensor = None, radii: Tensor = None,
+                   keep_masks: Tensor = None):
     """`GS_render` through the bucketed forward / per-Gaussian backward pair (gaussian_render.py:803-837).
-    `point_offsets` / `radii` as for `GS_render`."""
+    `point_offsets` / `radii` / `keep_masks` as for `GS_render`."""
     return _GS_render_fast.apply(W, H, mean2D, colors, conic_opacity, tile_range, point_list, extra, accum_max_count,
-                                 accum_weights_p, accum_weights_count, point_offsets, radii)
+                                 accum_weights_p, accum_weights_count, point_offsets, radii, keep_masks)
 
 
 def GS_render(W: int, H: int, mean2D: Tensor, colors: Tensor, conic_opacity: Tensor, tile_range: Tensor,
               point_list: Tensor, extra: Tensor = None, accum_max_count=None, accum_weights_p=None,
-              accum_weights_count=None, point_offsets: Tensor = None, radii: Tensor = None):
+              accum_weights_count=None, point_offsets: Tensor = None, radii: Tensor = None,
+              keep_masks: Tensor = None):
     """-> (images[3,H,W], opacity[H,W], extras[E,H,W]|None, n_contrib[H,W]); gaussian_render.py:839-845. With the
     binning's scan offsets (`GS_prepare(..., return_offsets=True)`) and the radii the backward sums the per-Gaussian
-    gradients in a fixed order without atomics."""
+    gradients in a fixed order without atomics; `keep_masks` must come along when the lists were built by
+    `GS_prepare(..., cull=True)`."""
     return _GS_render.apply(W, H, mean2D, colors, conic_opacity, tile_range, point_list, extra, accum_max_count,
-                            accum_weights_p, accum_weights_count, point_offsets, radii)
+                            accum_weights_p, accum_weights_count, point_offsets, radii, keep_masks)
 
 
 def RasterizeGaussians(means3D: Tensor, means2D: Optional[Tensor], colors: Tensor, sh_rest: Optional[Tensor],
@@ -303,12 +312,15 @@ def RasterizeGaussians(means3D: Tensor, means2D: Optional[Tensor], colors: Tenso
     means2D, depths, colors, radii, tiles_touched, conic_opacity = preprocess(
         means3D, scales, rotations, opacities, colors, sh_rest, Tw2v, Tv2c, cam_pos, tanFoV, W, H, sh_degree,
         is_opengl, cov3Ds_precomp, cov2Ds_precomp, means2D, culling)
+    keep = _cull_masks(W, H, means2D.detach(), conic_opacity.detach(), radii) if CULL_LISTS else None
     tile_ranges, point_list, point_offsets = GS_prepare(W, H, means2D.detach(), depths.detach(), radii, tiles_touched,
-                                                        False, return_offsets=True)
+                                                        False, return_offsets=True, cull=keep is not None,
+                                                        keep_masks=keep)[:3]
     ordered = DETERMINISTIC_SUMS
     out_pixels, out_opacities, out_extras, n_contrib = GS_render(
         W, H, means2D, colors, conic_opacity, tile_ranges, point_list, extras, accum_max_count, accum_weights_p,
-        accum_weights_count, point_offsets if ordered else None, radii if ordered else None)
+        accum_weights_count, point_offsets if ordered else None, radii if ordered else None,
+        keep if ordered else None)
     buffer = RasterizeBuffer3D(W, H, len(opacities), point_list.shape[0], tile_ranges, point_list, n_contrib,
                                conic_opacity, means2D, out_opacities)
     out_other_extras = [_render_extra.apply(W, H, extras_, means2D, conic_opacity, tile_ranges, point_list, n_contrib,

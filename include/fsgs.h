@@ -118,6 +118,11 @@ int fsgs_gs_prepare_fill_counted(int P, int W, int H, const float* means2D, cons
  * fsgs_gs_2d_render_backward_culled with the same masks. */
 int fsgs_gs_2d_cull_masks(int P, int W, int H, const float* records, const int32_t* radii, uint32_t* masks,
                           void* stream);
+/* The masks of 3D Gaussians, from what fsgs_gs_preprocess_forward leaves (means2D[P,2], conic_opacity[P,4], radii[P]):
+ * the ellipse on which gaussian_rasterize's alpha reaches 1/255, tested against each tile of the rectangle. The culled
+ * binning phases and the culled backwards take them as they take the surfels' masks. */
+int fsgs_gs_cull_masks(int P, int W, int H, const float* means2D, const float* conic_opacity, const int32_t* radii,
+                       uint32_t* masks, void* stream);
 int fsgs_gs_prepare_count_culled(int P, int W, int H, const float* means2D, const int32_t* radii,
                                  const uint32_t* masks, int64_t* ranges, void* bins, size_t bins_bytes, void* stream);
 int fsgs_gs_prepare_fill_counted_culled(int P, int W, int H, const float* means2D, const float* depths,
@@ -477,6 +482,12 @@ int fsgs_gaussian_rasterize_forward(int P, int W, int H, int E, const float* mea
  * is ASSIGNED from per-(Gaussian, tile) records added in a fixed order: no zero fill, no atomics, and the sums do not
  * vary from run to run. */
 size_t fsgs_gaussian_rasterize_backward_workspace_bytes(int64_t R);
+/* For tile lists built by fsgs_gs_prepare_*_culled (masks: fsgs_gs_cull_masks; no counterpart in the reference): the
+ * instances left out of the lists are staged by no block, so nobody writes their records. Call this on the workspace
+ * before an ordered-sum backward (fsgs_gaussian_rasterize_backward / _fast_backward / _bucket_backward with
+ * point_offsets); it zeroes exactly those records. The atomic path needs nothing. */
+int fsgs_gaussian_rasterize_clear_culled(int P, int64_t R, const int64_t* point_offsets, const uint32_t* keep_masks,
+                                         void* workspace, size_t workspace_bytes, void* stream);
 int fsgs_gaussian_rasterize_backward(int P, int W, int H, int E, const float* means2D, const float* conic_opacity,
     const float* colors, const float* extras, const float* out_opacity, const int32_t* n_contrib,
     const float* dL_dpix, const float* dL_dout_extras, const float* dL_dout_opacity, const int32_t* point_list,

@@ -161,3 +161,109 @@ def test_culled_backward_workspace_needs_no_clearing(variant, device):
     for name, a, b in zip(('colors', 'means2D', 'trans', 'normal_opacity'), zeroed, atomic):
         if np.abs(b).max() > 0:
             assert rel_err(a, b) < 1e-3, name
+
+
+# ---- 3D Gaussians: the same culling with the conic's alpha >= 1/255 ellipse ---------------------------------------------
+def _gs3d_stages(device, P, W, H, scale_mul, seed=3):
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd._C import get_C_function as f
+    scene, _ = scenes.config0(P=P, size=max(W, H), seed=seed)
+    cam = scenes.pinhole(W, H, 50.0, torch.tensor([0.3, -0.2, 4.0]))
+    g = torch.Generator().manual_seed(seed + 100)
+    scales = torch.cat([scene.scales * scale_mul,
+                        scene.scales[:, :1] * scale_mul * (0.3 + 3.0 * torch.rand(P, 1, generator=g))], 1).contiguous()
+    tan_fov = (W / 2 / float(cam.Tv2s[0, 0]), H / 2 / float(cam.Tv2s[1, 1]))
+    d = lambda t: t.to(device).contiguous()
+    m2, dep, col, rad, tt, c3, co = f('gs_preprocess_forward')(
+        W, H, 3, False, d(scene.means3D), d(scales), d(scene.rotations), d(scene.opacities), d(scene.shs), None,
+        d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), tan_fov, None, None, None, None)
+    gi = torch.randn(3, H, W, generator=g).to(device)
+    go = torch.randn(H, W, generator=g).to(device)
+    return f, m2, dep, col, rad, tt, co, gi, go
+
+
+@pytest.mark.parametrize("name,P,W,H,mul", [("small_4k_200x120", 4_000, 200, 120, 3.0),
+                                            ("big_300_96x80", 300, 96, 80, 30.0),
+                                            ("c2_300k_800", 300_000, 800, 800, 1.0)])
+@pytest.mark.parametrize("sums", ["atomic", "ordered", "ordered_bucket"])
+def test_gs3d_culled_lists_change_no_result(name, P, W, H, mul, sums, device):
+    f, m2, dep, col, rad, tt, co, gi, go = _gs3d_stages(device, P, W, H, mul)
+    masks = f('gs_cull_masks')(W, H, m2, co, rad)
+    full = f('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True)
+    cull = f('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True, cull=True, keep_masks=masks)
+    ra, rb = npy(full[0]), npy(cull[0])
+    la, lb = ra[:, 1] - ra[:, 0], rb[:, 1] - rb[:, 0]
+    print(f"[gs3d culled {name} {sums}] instances {int(la.sum())} -> {int(lb.sum())}, longest list {int(la.max())} -> "
+          f"{int(lb.max())}", flush=True)
+    assert (lb <= la).all() and (name.startswith("big_") or lb.sum() < la.sum())
+    assert torch.equal(full[2], cull[2])  # the scan is over the full rectangles either way
+    if P <= 10_000:
+        pa, pb = npy(full[1]), npy(cull[1])
+        for t in range(ra.shape[0]):
+            a, b = pa[ra[t, 0]:ra[t, 1]], pb[rb[t, 0]:rb[t, 1]]
+            assert np.array_equal(a[np.isin(a, b)], b), t
+    outs = []
+    for (ranges, pl, offsets), keep in ((full[:3], None), (cull[:3], masks)):
+        if sums == "ordered_bucket":
+            boff = torch.cumsum((ranges[:, 1] - ranges[:, 0] + 31) // 32, 0).contiguous()
+            oc, oo, _, nc, mc, b2t, sT, sar = f('gaussian_rasterize_forward')(W, H, m2, co, col, None, pl, ranges, None,
+                                                                              None, None, boff)
+            # poison what the caching allocator is going to hand out as the record workspace
+            junk = torch.full((int(pl.numel()) * 16 + 64,), float('nan'), device=device)
+            del junk
+            g = f('gaussian_rasterize_fast_backward')(m2, co, col, None, oc, None, oo, gi, go, None, ranges, pl, nc, mc,
+                                                      boff, b2t, sT, sar, offsets, rad, per_gaussian=True, culled=keep)
+        else:
+            oc, oo, _, nc = f('gaussian_rasterize_forward')(W, H, m2, co, col, None, pl, ranges)
+            junk = torch.full((int(pl.numel()) * 16 + 64,), float('nan'), device=device)
+            del junk
+            g = f('gaussian_rasterize_backward')(m2, co, col, None, oo, gi, go, None, ranges, pl, nc,
+                                                 offsets if sums == "ordered" else None,
+                                                 rad if sums == "ordered" else None, culled=keep)
+        outs.append((oc, oo, g))
+    torch.cuda.synchronize()
+    (oc_a, oo_a, g_a), (oc_b, oo_b, g_b) = outs
+    assert torch.equal(oc_a, oc_b) and torch.equal(oo_a, oo_b)
+    for k, (a, b) in zip(('g_colors', 'g_extras', 'g_means2D', 'g_conic_opacity'), zip(g_a, g_b)):
+        if a is None:
+            continue
+        assert bool(torch.isfinite(b).all()), k
+        assert rel_err(npy(b), npy(a)) < (1e-5 if sums != "atomic" else 1e-4), k
+
+
+def test_gs3d_renderer_culls_by_default(device):
+    """`RasterizeGaussians` (CULL_LISTS) against the same call on the reference's lists: images bit for bit, parameter
+    gradients to rounding, for the atomic and the ordered sums."""
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd.renderer import gaussian_render as GR
+    P, W, H = 5_000, 160, 112
+    scene, _ = scenes.config0(P=P, size=W, seed=5)
+    cam = scenes.pinhole(W, H, 50.0, torch.tensor([0.3, -0.2, 4.0]))
+    g = torch.Generator().manual_seed(9)
+    scales = torch.cat([scene.scales * 3, scene.scales[:, :1] * (0.5 + 3.5 * torch.rand(P, 1, generator=g))], 1)
+    gi = torch.randn(3, H, W, generator=g).to(device)
+    d = lambda t: t.to(device).contiguous()
+    focals = torch.tensor([float(cam.Tv2s[0, 0]), float(cam.Tv2s[1, 1])], device=device)
+    results = {}
+    try:
+        for ordered in (False, True):
+            for cull in (False, True):
+                GR.CULL_LISTS, GR.DETERMINISTIC_SUMS = cull, ordered
+                params = [d(t).requires_grad_(True) for t in (scene.means3D, scene.opacities, scales, scene.rotations,
+                                                              scene.shs)]
+                out = GR.render(d(cam.Tw2v), d(cam.Tv2c), (W, H), params[0], params[1], scales=params[2],
+                                rotations=params[3], campos=d(cam.campos), focals=focals, sh_features=params[4],
+                                sh_degree=3)
+                (out['images'] * gi).sum().backward()
+                results[(ordered, cull)] = (out['images'].detach(), [p.grad for p in params],
+                                            int(out['buffer'].point_list.numel()),
+                                            int((out['buffer'].tile_ranges[:, 1] - out['buffer'].tile_ranges[:, 0]).sum()))
+    finally:
+        GR.CULL_LISTS, GR.DETERMINISTIC_SUMS = True, False
+    torch.cuda.synchronize()
+    for ordered in (False, True):
+        (im_a, g_a, _, n_a), (im_b, g_b, _, n_b) = results[(ordered, False)], results[(ordered, True)]
+        assert n_b < n_a
+        assert torch.equal(im_a, im_b)
+        for a, b in zip(g_a, g_b):
+            assert rel_err(npy(b), npy(a)) < 1e-4

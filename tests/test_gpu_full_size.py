@@ -210,7 +210,7 @@ def test_fast_path_properties_at_300k_800(per_splat, device):
 
 def test_gs3d_path_properties_at_300k_800(device):
     """The 3D-Gaussian path at the benchmark size (the benchmark's centres with a third scale): culling off == on,
-    ordered per-instance sums == atomics, blend weights summing to the opacity image, linearity of the backward."""
+    culled tile lists == the reference's lists, ordered per-instance sums == atomics, blend weights summing to the opacity image, linearity of the backward."""
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd._C import get_C_function as f
     scene_h, cam_h = scenes.config2()
@@ -223,14 +223,17 @@ def test_gs3d_path_properties_at_300k_800(device):
     tan_fov = (W / 2 / float(cam.Tv2s[0, 0]), H / 2 / float(cam.Tv2s[1, 1]))
     print(f"[full gs3d] P={scene.P} {W}x{H}", flush=True)
 
-    def step(gi, go, ordered):
+    def step(gi, go, ordered, cull=False):
         m2, dep, col, rad, tt, c3, co = f('gs_preprocess_forward')(
             W, H, 3, False, scene.means3D, scales, scene.rotations, scene.opacities, scene.shs, None, cam.Tw2v,
             cam.Tv2c, cam.campos, tan_fov, None, None, None, None)
-        ranges, pl, offsets = f('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True)
+        keep = f('gs_cull_masks')(W, H, m2, co, rad) if cull else None
+        ranges, pl, offsets = f('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True, cull=cull,
+                                              keep_masks=keep)[:3]
         oc, oo, _, nc = f('gaussian_rasterize_forward')(W, H, m2, co, col, None, pl, ranges)
         g_col, _, g_m2, g_co = f('gaussian_rasterize_backward')(m2, co, col, None, oo, gi, go, None, ranges, pl, nc,
-                                                                offsets if ordered else None, rad if ordered else None)
+                                                                offsets if ordered else None, rad if ordered else None,
+                                                                culled=keep if ordered else None)
         g3, gs, gq = torch.empty_like(scene.means3D), torch.empty_like(scales), torch.empty_like(scene.rotations)
         gop, gsh = torch.empty_like(scene.opacities), torch.empty_like(scene.shs)
         f('gs_preprocess_backward')(W, H, 3, False, scene.means3D, scales, scene.rotations, scene.opacities, scene.shs,
@@ -260,6 +263,15 @@ def test_gs3d_path_properties_at_300k_800(device):
     close(a, b, 2e-5, 'culling')
     close(a, step(gi, go, False), 1e-4, 'atomic sums')
     close(a, step(2.0 * gi, 2.0 * go, True), 2e-5, 'linearity', 2.0)
+    # lists without the instances that no pixel of their tile can blend (what RasterizeGaussians bins)
+    for ordered in (True, False):
+        e = step(gi, go, ordered, cull=True)
+        n_full, n_cull = int((a['ranges'][:, 1] - a['ranges'][:, 0]).sum()), int((e['ranges'][:, 1] - e['ranges'][:, 0]).sum())
+        print(f"[full gs3d] instances in the tile lists {n_full} -> {n_cull}", flush=True)
+        assert n_cull < n_full
+        for k in ('image', 'opacity'):
+            assert torch.equal(a[k], e[k]), f"{k} depends on the culled lists"
+        close(a, e, 2e-5 if ordered else 1e-4, 'culled lists')
     acc = torch.zeros(scene.P, device=device)
     f('gaussian_rasterize_forward')(W, H, a['m2'], a['co'], a['col'], None, a['point_list'], a['ranges'], None, acc, None)
     torch.cuda.synchronize()

@@ -196,3 +196,69 @@ def test_fast_backward_workspace_needs_no_clearing(variant, kernel, device):
         if np.abs(b).max() > 0:
             assert rel_err(a, b) < 1e-3, name
     assert np.abs(zeroed[0]).max() > 0 and np.abs(zeroed[3]).max() > 0
+
+
+@pytest.mark.parametrize("lists", ["full", "culled"])
+def test_gs3d_backward_workspace_needs_no_clearing(lists, device):
+    """The same promise on the 3D-Gaussian path: every staged instance writes its record, a tile's block clears the
+    records of its never-staged tail, and with culled lists fsgs_gaussian_rasterize_clear_culled zeroes exactly the
+    records of the instances that are in no list. A workspace full of NaN or 3e30 gives the zeroed workspace's result
+    bit for bit."""
+    from fast_sp_gs_amd import lib as L, scenes
+    from fast_sp_gs_amd._C import get_C_function as f
+    lib = L.load()
+    W, H, P = 320, 208, 6000
+    scene, _ = scenes.config0(P=P, size=W, seed=3)
+    cam = scenes.pinhole(W, H, 50.0, torch.tensor([0.3, -0.2, 4.0]))
+    g = torch.Generator().manual_seed(103)
+    scales = torch.cat([scene.scales * 3, scene.scales[:, :1] * (0.5 + 3.5 * torch.rand(P, 1, generator=g))], 1)
+    scene.opacities[::3] = 0.999  # opaque Gaussians in front: tiles whose lists are cut before their end
+    tan_fov = (W / 2 / float(cam.Tv2s[0, 0]), H / 2 / float(cam.Tv2s[1, 1]))
+    d = lambda t: t.to(device).contiguous()
+    m2, dep, col, rad, tt, c3, co = f('gs_preprocess_forward')(
+        W, H, 3, False, d(scene.means3D), d(scales), d(scene.rotations), d(scene.opacities), d(scene.shs), None,
+        d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), tan_fov, None, None, None, None)
+    masks = f('gs_cull_masks')(W, H, m2, co, rad)
+    culled = lists == "culled"
+    ranges, pl, offsets = f('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True, cull=culled,
+                                          keep_masks=masks if culled else None)[:3]
+    oc, oo, _, nc = f('gaussian_rasterize_forward')(W, H, m2, co, col, None, pl, ranges)
+    lens = npy(ranges[:, 1] - ranges[:, 0]).reshape((H + 15) // 16, (W + 15) // 16)
+    deepest = torch.nn.functional.max_pool2d(nc[None, None].float(), 16, ceil_mode=True)[0, 0].cpu().numpy()
+    empty, long_, cut = int((lens == 0).sum()), int((lens > 64).sum()), int(((deepest < lens) & (lens > 0)).sum())
+    print(f"[gs3d {lists}] tiles: {empty} empty, {long_} longer than 64 entries, {cut} cut before their end; "
+          f"{int(lens.sum())} of {pl.numel()} instances listed")
+    assert empty > 0 and long_ > 0 and cut > 0
+    gi = torch.randn(3, H, W, generator=g).to(device)
+    go = torch.randn(H, W, generator=g).to(device)
+    R = int(pl.numel())
+    nbytes = lib.fsgs_gaussian_rasterize_backward_workspace_bytes(R)
+
+    def run(fill, ordered=True):
+        ws = torch.empty(nbytes // 4, device=device)
+        ws.fill_(fill)
+        out = [torch.full((P, n), float('nan'), device=device) if ordered else torch.zeros(P, n, device=device)
+               for n in (2, 4, 3)]  # means2D, conic + opacity, colours
+        if ordered and culled:
+            L.check(lib.fsgs_gaussian_rasterize_clear_culled(P, R, L.ptr(offsets), L.ptr(masks), L.ptr(ws), nbytes,
+                                                             L.current_stream()), 'clear_culled')
+        rc = lib.fsgs_gaussian_rasterize_backward(
+            P, W, H, 0, L.ptr(m2), L.ptr(co), L.ptr(col), None, L.ptr(oo), L.ptr(nc), L.ptr(gi), None, L.ptr(go),
+            L.ptr(pl), L.ptr(ranges), L.ptr(out[0]), L.ptr(out[1]), L.ptr(out[2]), None, R,
+            L.ptr(offsets) if ordered else None, L.ptr(rad) if ordered else None, L.ptr(ws) if ordered else None,
+            nbytes if ordered else 0, L.current_stream())
+        L.check(rc, 'fsgs_gaussian_rasterize_backward')
+        torch.cuda.synchronize()
+        return [npy(o) for o in out]
+
+    zeroed = run(0.0)
+    for o in zeroed:
+        assert np.isfinite(o).all()
+    for fill in (float('nan'), 3.0e30):
+        poisoned = run(fill)
+        for a, b in zip(poisoned, zeroed):
+            assert np.isfinite(a).all(), fill
+            assert np.array_equal(a, b), fill
+    atomic = run(0.0, ordered=False)
+    for name, a, b in zip(('means2D', 'conic_opacity', 'colors'), zeroed, atomic):
+        assert np.abs(b).max() > 0 and rel_err(a, b) < 1e-3, name
