@@ -179,7 +179,7 @@ def _timed_ms(fn, reps: int = 20, warm: int = 3) -> float:
 
 
 def standalone_ops(dev, copy_gbps: float):
-    """The stand-alone operators of BASELINE config 1 and the optimiser, each with its algorithmic bytes, the rate those
+    """The operators of the stand-alone benchmark configuration (1M directions, 200 000 x 512 points) and the optimiser, each with its algorithmic bytes, the rate those
     bytes give over the measured time, and that rate as a share of the 8 TB/s peak and of the copy probe:
     SH encoder forward / backward at 1M directions (shencoder.cu:657-691), SH -> RGB forward / backward at 1M points
     (ops_3d/spherical_harmonics.cu:15-16, 68-70), the LBS blend forward / backward at 200 000 x 512, K = 4
@@ -547,7 +547,7 @@ def density_control_ms(dev, scene, reps: int = 5):
 
 
 def large_scene_ms(dev, views: int = 4, reps: int = 3, cull: bool = False):
-    """BASELINE config 4: 3M surfels, a batch of 4 views at 1352x1014 rendered forward + backward one after the other,
+    """The large-scene configuration: 3M surfels, a batch of 4 views at 1352x1014 rendered forward + backward one after the other,
     and the K-NN of the 3M centres against 2048 control points with k = 8."""
     from fast_sp_gs_amd import scenes
     from fast_sp_gs_amd._C import get_C_function
