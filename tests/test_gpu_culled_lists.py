@@ -267,3 +267,42 @@ def test_gs3d_renderer_culls_by_default(device):
         assert torch.equal(im_a, im_b)
         for a, b in zip(g_a, g_b):
             assert rel_err(npy(b), npy(a)) < 1e-4
+
+
+def test_culled_paths_with_nothing_to_do(device):
+    """A scene entirely behind the camera through the culled paths (R == 0: every mask is all-ones by convention and no
+    kernel of the binning or the backward has anything to visit), surfels and 3D Gaussians."""
+    from fast_sp_gs_amd import scenes
+    from fast_sp_gs_amd._C import get_C_function as f
+    from fast_sp_gs_amd.renderer import render_step
+    scene, cam = scenes.config0(P=64, size=64, seed=3)
+    scene.means3D[:, 2] += 10.0
+    for ordered in (True, False):
+        out = render_step(scene.to(device), cam.to(device), torch.zeros(3, 64, 64, device=device), cull=True,
+                          ordered_sums=ordered)
+        torch.cuda.synchronize()
+        assert out['point_list'].numel() == 0 and int(out['ranges'].abs().sum()) == 0
+        assert float(out['image'].abs().sum()) == 0 and float(out['g_means3D'].abs().sum()) == 0
+    W = H = 64
+    tan_fov = (W / 2 / float(cam.Tv2s[0, 0]), H / 2 / float(cam.Tv2s[1, 1]))
+    d = lambda t: t.to(device).contiguous()
+    scales = torch.cat([scene.scales, scene.scales[:, :1]], 1)
+    m2, dep, col, rad, tt, c3, co = f('gs_preprocess_forward')(
+        W, H, 3, False, d(scene.means3D), d(scales), d(scene.rotations), d(scene.opacities), d(scene.shs), None,
+        d(cam.Tw2v), d(cam.Tv2c), d(cam.campos), tan_fov, None, None, None, None)
+    masks = f('gs_cull_masks')(W, H, m2, co, rad)
+    ranges, pl, offsets = f('GS_prepare')(W, H, m2, dep, rad, tt, False, return_offsets=True, cull=True,
+                                          keep_masks=masks)[:3]
+    oc, oo, _, nc = f('gaussian_rasterize_forward')(W, H, m2, co, col, None, pl, ranges)
+    z = torch.zeros(3, H, W, device=device)
+    for ordered in (True, False):
+        g = f('gaussian_rasterize_backward')(m2, co, col, None, oo, z, z[0], None, ranges, pl, nc,
+                                             offsets if ordered else None, rad if ordered else None,
+                                             culled=masks if ordered else None)
+        torch.cuda.synchronize()
+        assert pl.numel() == 0 and int((masks != -1).sum()) == 0
+        assert all(float(t.abs().sum()) == 0 for t in g if t is not None)
+    # no points at all
+    e = lambda *s: torch.zeros(*s, device=device)
+    masks0 = f('gs_cull_masks')(W, H, e(0, 2), e(0, 4), torch.zeros(0, dtype=torch.int32, device=device))
+    assert masks0.numel() == 1
