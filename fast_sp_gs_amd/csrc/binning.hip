@@ -189,11 +189,17 @@ constexpr int kMaxLdsTiles = 16384;
 // (cull_mask_kernel: the tiles some pixel of which can blend the surfel; rectangles above 32 tiles are kept whole).
 enum WalkMode { kWalkAll = 0, kWalkCorner = 1, kWalkMask = 2 };
 
+// What a mode reads beside centres and radii: kWalkCorner the adjugates and opacities, kWalkMask the keep masks.
+struct WalkInputs {
+  const float* inverse_m;
+  const float* opacities;
+  const uint32_t* keep_masks;
+};
+
 template <int kMode, typename Visit>
 __device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, const float2* __restrict__ means2D,
-                                                  const int32_t* __restrict__ radii,
-                                                  const float* __restrict__ inverse_m,   // kWalkMask: keep masks
-                                                  const float* __restrict__ opacities, Visit visit) {
+                                                  const int32_t* __restrict__ radii, const WalkInputs& in,
+                                                  Visit visit) {
   const int lane = __lane_id();
   int x0 = 0, y0 = 0, w = 0, h = 0;
   float IM[kMode == kWalkCorner ? 9 : 1], opacity = 1.0f;
@@ -205,11 +211,11 @@ __device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, 
     const TileRect r = tile_rect(c.x, c.y, radii[i], gx, gy);
     x0 = r.x0, y0 = r.y0, w = max(r.x1 - r.x0, 0), h = max(r.y1 - r.y0, 0);
     if (kMode == kWalkCorner) {
-      opacity = opacities[i];
+      opacity = in.opacities[i];
 #pragma unroll
-      for (int k = 0; k < 9; ++k) IM[k] = inverse_m[9 * (size_t) i + k];
+      for (int k = 0; k < 9; ++k) IM[k] = in.inverse_m[9 * (size_t) i + k];
     }
-    if (kMode == kWalkMask) keep_mask = ((const uint32_t*) inverse_m)[i];
+    if (kMode == kWalkMask) keep_mask = in.keep_masks[i];
   }
   const int count = w * h;
   if (count > 0 && count <= kCoopThreshold) {
@@ -314,8 +320,8 @@ inline BinsLayout bins_layout(int P, int T) {
 // every tile.
 template <int kMode>
 __global__ void __launch_bounds__(1024) tile_hist_kernel(int P, int per_block, int gx, int gy,
-    const float2* __restrict__ means2D, const int32_t* __restrict__ radii, const float* __restrict__ inverse_m,
-    const float* __restrict__ opacities, uint32_t* __restrict__ hist) {
+    const float2* __restrict__ means2D, const int32_t* __restrict__ radii, WalkInputs in,
+    uint32_t* __restrict__ hist) {
   __shared__ unsigned s_count[kMaxLdsTiles];
   const int T = gx * gy;
   for (int t = threadIdx.x; t < T; t += blockDim.x) s_count[t] = 0u;
@@ -325,8 +331,8 @@ __global__ void __launch_bounds__(1024) tile_hist_kernel(int P, int per_block, i
   const int rounds = (last - first + (int) blockDim.x - 1) / (int) blockDim.x;
   for (int r = 0; r < rounds; ++r) {
     const int i = first + r * blockDim.x + threadIdx.x;
-    for_each_instance<kMode>(i < last ? i : P, P, gx, gy, means2D, radii, inverse_m, opacities,
-                               [&](int tile, int) { atomicAdd(&s_count[tile], 1u); });
+    for_each_instance<kMode>(i < last ? i : P, P, gx, gy, means2D, radii, in,
+                             [&](int tile, int) { atomicAdd(&s_count[tile], 1u); });
   }
   __syncthreads();
   uint32_t* row = hist + (size_t) blockIdx.x * T;
@@ -376,8 +382,8 @@ __global__ void __launch_bounds__(kPrefixTiles * kPrefixWaves) tile_prefix_kerne
 template <int kMode>
 __global__ void __launch_bounds__(1024) tile_scatter_kernel(int P, int per_block, int gx, int gy, int64_t R,
     const float2* __restrict__ means2D, const float* __restrict__ depths, const int32_t* __restrict__ radii,
-    const float* __restrict__ inverse_m, const float* __restrict__ opacities, const uint32_t* __restrict__ hist,
-    const unsigned long long* __restrict__ ranges, uint64_t* __restrict__ entries) {
+    WalkInputs in, const uint32_t* __restrict__ hist, const unsigned long long* __restrict__ ranges,
+    uint64_t* __restrict__ entries) {
   __shared__ unsigned s_cursor[kMaxLdsTiles];
   const int T = gx * gy;
   const uint32_t* row = hist + (size_t) blockIdx.x * T;
@@ -387,7 +393,7 @@ __global__ void __launch_bounds__(1024) tile_scatter_kernel(int P, int per_block
   const int rounds = (last - first + (int) blockDim.x - 1) / (int) blockDim.x;
   for (int r = 0; r < rounds; ++r) {
     const int i = first + r * blockDim.x + threadIdx.x;
-    for_each_instance<kMode>(i < last ? i : P, P, gx, gy, means2D, radii, inverse_m, opacities, [&](int tile, int id) {
+    for_each_instance<kMode>(i < last ? i : P, P, gx, gy, means2D, radii, in, [&](int tile, int id) {
       const unsigned pos = atomicAdd(&s_cursor[tile], 1u);
       if ((int64_t) pos < R) entries[pos] = ((uint64_t) __float_as_uint(depths[id]) << 32) | (uint32_t) id;
     });
@@ -875,14 +881,15 @@ int fast_bucket_fill(int P, int W, int H, const float* means2D, const float* inv
   uint64_t* entries = sort_keys_in(R, workspace);
   int* large_list   = (int*) ((char*) workspace + sort_layout(R).keys1);
   hipLaunchKernelGGL(tile_hist_kernel<kWalkCorner>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
-                     (const float2*) means2D, radii, inverse_m, opacities, hist);
+                     (const float2*) means2D, radii, WalkInputs{inverse_m, opacities, nullptr}, hist);
   hipLaunchKernelGGL(tile_prefix_kernel, dim3(div_up(T, kPrefixTiles)), dim3(kPrefixTiles * kPrefixWaves), 0, s, T,
                      bl.blocks, hist, rng);
   hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, true);
   const int* order = nullptr;
   (void) launch_tile_order(gx, gy, ranges, s, &order);  // the blend kernels of this view find it under `ranges`
   hipLaunchKernelGGL(tile_scatter_kernel<kWalkCorner>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
-                     (const float2*) means2D, depths, radii, inverse_m, opacities, (const uint32_t*) hist, rng, entries);
+                     (const float2*) means2D, depths, radii, WalkInputs{inverse_m, opacities, nullptr},
+                     (const uint32_t*) hist, rng, entries);
   hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
                      header, large_list, order);
   hipLaunchKernelGGL(tile_sort_large_kernel, dim3(256), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,
@@ -969,9 +976,9 @@ FSGS_API int fsgs_gs_prepare_sort_bits(int W, int H) {
 namespace {
 // First part of the bucket binning, independent of the instance count: per-tile instance counts and the tile ranges
 // (start, end); the long-segment queue's counter (first word of `bins`) is reset.
-// cull_records (optional): the per-surfel keep masks of cull_mask_kernel; with them an instance is only counted (and
+// keep_masks (optional): the per-surfel keep masks of cull_mask_kernel; with them an instance is only counted (and
 // later scattered) when its bit is set.
-int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, const float* cull_records,
+int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, const uint32_t* keep_masks,
                int64_t* ranges, void* bins, hipStream_t s) {
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int T  = gx * gy;
@@ -980,12 +987,12 @@ int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, 
   const BinsLayout bl = bins_layout(P, T);
   if (bl.blocks > 0) {
     uint32_t* hist = (uint32_t*) ((char*) bins + kBinsHeader);
-    if (cull_records)
+    if (keep_masks)
       hipLaunchKernelGGL(tile_hist_kernel<kWalkMask>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
-                         (const float2*) means2D, radii, cull_records, (const float*) nullptr, hist);
+                         (const float2*) means2D, radii, WalkInputs{nullptr, nullptr, keep_masks}, hist);
     else
       hipLaunchKernelGGL(tile_hist_kernel<kWalkAll>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
-                         (const float2*) means2D, radii, (const float*) nullptr, (const float*) nullptr, hist);
+                         (const float2*) means2D, radii, WalkInputs{nullptr, nullptr, nullptr}, hist);
     hipLaunchKernelGGL(tile_prefix_kernel, dim3(div_up(T, kPrefixTiles)), dim3(kPrefixTiles * kPrefixWaves), 0, s, T,
                        bl.blocks, hist, rng);
     hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, true);
@@ -1000,8 +1007,7 @@ int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, 
                        ranges);
     if (P > 0)
       hipLaunchKernelGGL(tile_emit_kernel<false>, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, (int64_t) 0,
-                         (const float2*) means2D, (const float*) nullptr, radii, (const uint32_t*) cull_records, rng,
-                         (uint64_t*) nullptr);
+                         (const float2*) means2D, (const float*) nullptr, radii, keep_masks, rng, (uint64_t*) nullptr);
     hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, false);
   }
   return check_launch("gs_prepare_count");
@@ -1009,7 +1015,7 @@ int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, 
 
 // Second part: scatter (depth bits << 32 | surfel) into the tile segments and sort every segment.
 int fill_sort(int P, int W, int H, const float* means2D, const float* depths, const int32_t* radii,
-              const float* cull_records, int64_t R, int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out,
+              const uint32_t* keep_masks, int64_t R, int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out,
               void* workspace, void* bins, hipStream_t s) {
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int T  = gx * gy;
@@ -1019,17 +1025,17 @@ int fill_sort(int P, int W, int H, const float* means2D, const float* depths, co
   // queue of long segments: at most R / kSmallSegment tiles, kept behind the entries in the workspace
   int* large_list = (int*) ((char*) workspace + sort_layout(R).keys1);
   const BinsLayout bl = bins_layout(P, T);
-  if (bl.blocks > 0 && cull_records)
+  if (bl.blocks > 0 && keep_masks)
     hipLaunchKernelGGL(tile_scatter_kernel<kWalkMask>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
-                       (const float2*) means2D, depths, radii, cull_records, (const float*) nullptr,
+                       (const float2*) means2D, depths, radii, WalkInputs{nullptr, nullptr, keep_masks},
                        (const uint32_t*) ((const char*) bins + kBinsHeader), rng, entries);
   else if (bl.blocks > 0)
     hipLaunchKernelGGL(tile_scatter_kernel<kWalkAll>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
-                       (const float2*) means2D, depths, radii, (const float*) nullptr, (const float*) nullptr,
+                       (const float2*) means2D, depths, radii, WalkInputs{nullptr, nullptr, nullptr},
                        (const uint32_t*) ((const char*) bins + kBinsHeader), rng, entries);
   else
     hipLaunchKernelGGL(tile_emit_kernel<true>, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
-                       (const float2*) means2D, depths, radii, (const uint32_t*) cull_records, rng, entries);
+                       (const float2*) means2D, depths, radii, keep_masks, rng, entries);
   // the schedule table built by the counting part (or built now, on the global-atomic path, whose ranges only become
   // final with the scatter)
   const int* order = nullptr;
@@ -1116,7 +1122,7 @@ FSGS_API int fsgs_gs_prepare_count_culled(int P, int W, int H, const float* mean
     return fail(kWorkspaceSmall, "gs_prepare_count_culled: bins %zu < %zu bytes", bins_bytes,
                 fsgs_gs_prepare_bins_bytes(P, W, H));
   tile_order_invalidate((hipStream_t) stream);
-  return fill_count(P, W, H, means2D, radii, culling_enabled() ? (const float*) masks : nullptr, ranges, bins,
+  return fill_count(P, W, H, means2D, radii, culling_enabled() ? masks : nullptr, ranges, bins,
                     (hipStream_t) stream);
 }
 
@@ -1135,7 +1141,7 @@ FSGS_API int fsgs_gs_prepare_fill_counted_culled(int P, int W, int H, const floa
   if (bins_bytes < fsgs_gs_prepare_bins_bytes(P, W, H))
     return fail(kWorkspaceSmall, "gs_prepare_fill_culled: bins %zu < %zu bytes", bins_bytes,
                 fsgs_gs_prepare_bins_bytes(P, W, H));
-  return fill_sort(P, W, H, means2D, depths, radii, culling_enabled() ? (const float*) masks : nullptr, R, ranges,
+  return fill_sort(P, W, H, means2D, depths, radii, culling_enabled() ? masks : nullptr, R, ranges,
                    point_list, sorted_keys_out, workspace, bins, (hipStream_t) stream);
 }
 
