@@ -79,7 +79,7 @@ class _GS_2D_Render(torch.autograd.Function):
         keep = keep[0] if cull else None
         tile_range, point_list, point_offsets = GS_prepare(
             W, H, means2D, depths, radii, tiles_touched, False, return_offsets=True, records=records, cull=cull,
-            keep_masks=keep, store_offsets=False)[:3]
+            keep_masks=keep)[:3]
         pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib = _GS_2D_Render._render_forward(
             W, H, means2D, colors, normal_opacity, trans_mat, point_list, tile_range, near_n, far_n, only_image,
             transe_mat_t2, accum_max_count, accum_weights_p, accum_weights_count, records)
@@ -238,8 +238,7 @@ def render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad
     keep = rec[-1] if cull else None
     rec = rec[0] if packed else None
     ranges, point_list, offsets = f('GS_prepare')(W, H, m2, depths, radii, tt, False, return_offsets=True,
-                                                  records=rec, cull=cull, keep_masks=keep,
-                                                  store_offsets=False)[:3]
+                                                  records=rec, cull=cull, keep_masks=keep)[:3]
     oc, oo, oe, of, nc = f('GS_2D_render_forward')(W, H, m2, colors, no, tm, point_list, ranges, cam.near, cam.far,
                                                    False, None, None, None, None, rec)
     epilogue = {}
