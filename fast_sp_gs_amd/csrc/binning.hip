@@ -383,8 +383,15 @@ template <int kMode>
 __global__ void __launch_bounds__(1024) tile_scatter_kernel(int P, int per_block, int gx, int gy, int64_t R,
     const float2* __restrict__ means2D, const float* __restrict__ depths, const int32_t* __restrict__ radii,
     WalkInputs in, const uint32_t* __restrict__ hist, const unsigned long long* __restrict__ ranges,
-    uint64_t* __restrict__ entries) {
+    uint64_t* __restrict__ entries, int* __restrict__ order_table) {
   __shared__ unsigned s_cursor[kMaxLdsTiles];
+  // One block more than the walk needs, when the frame's blockIdx -> tile schedule is still to be built: the ranges are
+  // final, nothing in this kernel reads the table, and the per-tile sorts and the blend kernels that follow do.
+  if (order_table && blockIdx.x == gridDim.x - 1) {
+    static_assert(sizeof(TileOrderLds) <= sizeof(s_cursor), "the schedule's LDS fits the cursor array");
+    build_tile_order(gx, gy, (const int64_t*) ranges, order_table, *reinterpret_cast<TileOrderLds*>(s_cursor));
+    return;
+  }
   const int T = gx * gy;
   const uint32_t* row = hist + (size_t) blockIdx.x * T;
   for (int t = threadIdx.x; t < T; t += blockDim.x) s_cursor[t] = (unsigned) ranges[2 * (size_t) t] + row[t];
@@ -885,11 +892,13 @@ int fast_bucket_fill(int P, int W, int H, const float* means2D, const float* inv
   hipLaunchKernelGGL(tile_prefix_kernel, dim3(div_up(T, kPrefixTiles)), dim3(kPrefixTiles * kPrefixWaves), 0, s, T,
                      bl.blocks, hist, rng);
   hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, true);
+  // the schedule the blend kernels of this view find under `ranges`, built by an extra block of the scatter
   const int* order = nullptr;
-  (void) launch_tile_order(gx, gy, ranges, s, &order);  // the blend kernels of this view find it under `ranges`
-  hipLaunchKernelGGL(tile_scatter_kernel<kWalkCorner>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
-                     (const float2*) means2D, depths, radii, WalkInputs{inverse_m, opacities, nullptr},
-                     (const uint32_t*) hist, rng, entries);
+  int* build       = nullptr;
+  (void) defer_tile_order(gx, gy, ranges, s, &order, &build);
+  hipLaunchKernelGGL(tile_scatter_kernel<kWalkCorner>, dim3(bl.blocks + (build ? 1 : 0)), dim3(1024), 0, s, P,
+                     bl.per_block, gx, gy, R, (const float2*) means2D, depths, radii,
+                     WalkInputs{inverse_m, opacities, nullptr}, (const uint32_t*) hist, rng, entries, build);
   hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
                      header, large_list, order);
   hipLaunchKernelGGL(tile_sort_large_kernel, dim3(256), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,
@@ -996,11 +1005,8 @@ int fill_count(int P, int W, int H, const float* means2D, const int32_t* radii, 
     hipLaunchKernelGGL(tile_prefix_kernel, dim3(div_up(T, kPrefixTiles)), dim3(kPrefixTiles * kPrefixWaves), 0, s, T,
                        bl.blocks, hist, rng);
     hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, true);
-    // The ranges are final here, before the instance count has even reached the host: the schedule table the blend
-    // kernels of this frame are going to use (they find it under this ranges buffer's key) is built now, in the shadow of
-    // the host's wait; it orders the per-tile sorts as well.
-    const int* order = nullptr;
-    (void) launch_tile_order(gx, gy, ranges, s, &order);
+    // The ranges are final here; the schedule table the blend kernels of this frame are going to use (and the per-tile
+    // sorts) is built from them by an extra block of the scatter, in the second part.
   } else {
     // no room for one LDS counter per tile (or no surfels): count straight into ranges[t].y, then scan to (start, start)
     hipLaunchKernelGGL(fill_zero_i64_kernel, dim3(div_up(2 * (int64_t) T, 256)), dim3(256), 0, s, 2 * (int64_t) T,
@@ -1025,21 +1031,25 @@ int fill_sort(int P, int W, int H, const float* means2D, const float* depths, co
   // queue of long segments: at most R / kSmallSegment tiles, kept behind the entries in the workspace
   int* large_list = (int*) ((char*) workspace + sort_layout(R).keys1);
   const BinsLayout bl = bins_layout(P, T);
+  // The schedule table: built by one extra block of the scatter (the ranges are final since the counting part), or by a
+  // launch of its own on the global-atomic path, whose ranges only become final with the scatter.
+  const int* order = nullptr;
+  int* build       = nullptr;
+  if (bl.blocks > 0) (void) defer_tile_order(gx, gy, ranges, s, &order, &build);
+  const dim3 scatter_grid(bl.blocks + (build ? 1 : 0));
   if (bl.blocks > 0 && keep_masks)
-    hipLaunchKernelGGL(tile_scatter_kernel<kWalkMask>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
+    hipLaunchKernelGGL(tile_scatter_kernel<kWalkMask>, scatter_grid, dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
                        (const float2*) means2D, depths, radii, WalkInputs{nullptr, nullptr, keep_masks},
-                       (const uint32_t*) ((const char*) bins + kBinsHeader), rng, entries);
+                       (const uint32_t*) ((const char*) bins + kBinsHeader), rng, entries, build);
   else if (bl.blocks > 0)
-    hipLaunchKernelGGL(tile_scatter_kernel<kWalkAll>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
+    hipLaunchKernelGGL(tile_scatter_kernel<kWalkAll>, scatter_grid, dim3(1024), 0, s, P, bl.per_block, gx, gy, R,
                        (const float2*) means2D, depths, radii, WalkInputs{nullptr, nullptr, nullptr},
-                       (const uint32_t*) ((const char*) bins + kBinsHeader), rng, entries);
-  else
+                       (const uint32_t*) ((const char*) bins + kBinsHeader), rng, entries, build);
+  else {
     hipLaunchKernelGGL(tile_emit_kernel<true>, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
                        (const float2*) means2D, depths, radii, keep_masks, rng, entries);
-  // the schedule table built by the counting part (or built now, on the global-atomic path, whose ranges only become
-  // final with the scatter)
-  const int* order = nullptr;
-  (void) launch_tile_order(gx, gy, ranges, s, &order);
+    (void) launch_tile_order(gx, gy, ranges, s, &order);
+  }
   hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
                      large_count, large_list, order);
   hipLaunchKernelGGL(tile_sort_large_kernel, dim3(256), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,

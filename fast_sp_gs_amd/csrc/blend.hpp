@@ -270,11 +270,23 @@ __device__ __forceinline__ int tile_region(int t, int gx, int gy) {
   return ((tx / FSGS_TILE_GROUP) + 3 * (ty / FSGS_TILE_GROUP)) & (kOrderRegions - 1);
 }
 
-__global__ void __launch_bounds__(1024) tile_order_kernel(int gx, int gy, const int64_t* __restrict__ ranges,
-                                                          int* __restrict__ tile_order) {
-  __shared__ int s_count[kOrderRegions][kOrderBuckets];
-  __shared__ int s_total[kOrderRegions];
-  __shared__ int s_tile[kOrderRegions][kBalanceRounds * kCusPerXcd], s_len[kOrderRegions][kBalanceRounds * kCusPerXcd];
+// LDS of one block that builds a table (24.6 KB)
+struct TileOrderLds {
+  int count[kOrderRegions][kOrderBuckets];
+  int total[kOrderRegions];
+  int tile[kOrderRegions][kBalanceRounds * kCusPerXcd], len[kOrderRegions][kBalanceRounds * kCusPerXcd];
+};
+
+// The work of one whole block (any size that is a multiple of 64 with at least 8 wavefronts): either a launch of its
+// own (tile_order_kernel) or one extra block of a kernel that has nothing to do with it but runs at the right time --
+// the binning's scatter, whose other blocks keep the chip busy while this one orders 2 500 numbers (a single-block
+// launch of its own holds up the stream for 10 us).
+__device__ __forceinline__ void build_tile_order(int gx, int gy, const int64_t* __restrict__ ranges,
+                                                 int* __restrict__ tile_order, TileOrderLds& lds) {
+  auto& s_count = lds.count;
+  auto& s_total = lds.total;
+  auto& s_tile  = lds.tile;
+  auto& s_len   = lds.len;
   const int T = gx * gy;
   for (int b = threadIdx.x; b < kOrderRegions * kOrderBuckets; b += blockDim.x) (&s_count[0][0])[b] = 0;
   __syncthreads();
@@ -350,6 +362,12 @@ __global__ void __launch_bounds__(1024) tile_order_kernel(int gx, int gy, const 
   }
 }
 
+__global__ void __launch_bounds__(1024) tile_order_kernel(int gx, int gy, const int64_t* __restrict__ ranges,
+                                                          int* __restrict__ tile_order) {
+  __shared__ TileOrderLds lds;
+  build_tile_order(gx, gy, ranges, tile_order, lds);
+}
+
 // Launch flags of the blend kernels: bit 0 = the tile table was built for this launch (T small enough; otherwise blocks
 // map to tiles directly), bit 1 = per-quadrant culling switched off (verification aid, see fsgs_debug_set_culling).
 inline int launch_tile_order(int gx, int gy, const int64_t* ranges, hipStream_t s, const int** table) {
@@ -360,6 +378,20 @@ inline int launch_tile_order(int gx, int gy, const int64_t* ranges, hipStream_t 
   int* t = tile_order_table(s, ranges, gx, gy, &rebuild);
   if (!t) return flags;
   if (rebuild) hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, s, gx, gy, ranges, t);
+  *table = t;
+  return flags | kFlagOrdered;
+}
+
+// The same, with the build left to a kernel the caller is about to launch on the stream anyway: *build receives the
+// table to fill (build_tile_order in one extra block), or stays nullptr when the table is up to date or there is none.
+inline int defer_tile_order(int gx, int gy, const int64_t* ranges, hipStream_t s, const int** table, int** build) {
+  int flags = culling_enabled() ? 0 : kFlagNoCull;
+  *table = nullptr, *build = nullptr;
+  if ((int64_t) gx * gy > kMaxOrderedTiles) return flags;
+  bool rebuild = false;
+  int* t = tile_order_table(s, ranges, gx, gy, &rebuild);
+  if (!t) return flags;
+  if (rebuild) *build = t;
   *table = t;
   return flags | kFlagOrdered;
 }
