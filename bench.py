@@ -709,8 +709,8 @@ def fast_path_rate(dev, scene, cam, gi, steps: int = 20, warmup: int = 3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the fast-path and dynamic-step side measurements")
     ap.add_argument("--counter-run", action="store_true",
