@@ -549,11 +549,13 @@ def gs_2d_fast_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: boo
                                   Tw2v: Tensor, Tv2c: Tensor, Tv2s: Tensor, cam_pos: Tensor,
                                   trans_precomp: Optional[Tensor] = None, means2D: Optional[Tensor] = None,
                                   culling: Optional[Tensor] = None, debug: bool = False,
-                                  return_keys: bool = False, return_offsets: bool = False) -> List[Tensor]:
+                                  return_keys: bool = False, return_offsets: bool = False,
+                                  return_masks: bool = False) -> List[Tensor]:
     """gs_2d_fast_preprocess.cu:611-782 -> [means2D, colors, trans_mat, inverse_m, normal_opacity, depths, radii,
     ranges[T,2] int64, point_list[R] int32] (point_list keeps the -1 padding entries of culled tiles at its tail)
     (+ sorted keys and tiles_touched, + the prefix scan of tiles_touched, which GS_2D_fast_render_backward can use to sum
-    gradients without atomics)."""
+    gradients without atomics, + keep_masks[P] int32, the corner test's verdicts per surfel that the preprocess kernel
+    leaves for the binning, which the ordered sum of GS_2D_fast_render_backward can reuse)."""
     what = 'gs_2d_fast_preprocess_forward'
     _f32(what, means3D=means3D, scales=scales, rotations=rotations, opacities=opacities, shs=shs, Tw2v=Tw2v,
          Tv2c=Tv2c, Tv2s=Tv2s, cam_pos=cam_pos)
@@ -604,13 +606,14 @@ def gs_2d_fast_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: boo
     radii = torch.empty((P,), dtype=torch.int32, device=dev)
     tiles_touched = torch.empty((P,), dtype=torch.int32, device=dev)
     normal_opacity = torch.empty((P, 4), **opt)
+    keep_masks = torch.empty((max(P, 1),), dtype=torch.int32, device=dev)
     with _timed('gs_2d_fast_preprocess_forward'):
         rc = lib.fsgs_gs_2d_fast_preprocess_forward(
             P, W, H, sh_degree, M, L.ptr(means3D), L.ptr(scales), L.ptr(rotations), L.ptr(opacities), L.ptr(shs),
             L.ptr(sh_rest) if has_rest else None, L.ptr(Tw2v), L.ptr(Tv2s), L.ptr(cam_pos), L.ptr(trans_precomp),
             L.ptr(culling), int(preserve), L.ptr(means2D_), None if sh_degree < 0 else L.ptr(colors),
             None if trans_precomp is not None else L.ptr(trans_mat), L.ptr(inverse_m), L.ptr(normal_opacity),
-            L.ptr(depths), L.ptr(radii), L.ptr(tiles_touched), stream)
+            L.ptr(depths), L.ptr(radii), L.ptr(tiles_touched), L.ptr(keep_masks), stream)
     L.check(rc, what)
 
     T = ((W + _TILE - 1) // _TILE) * ((H + _TILE - 1) // _TILE)
@@ -629,7 +632,8 @@ def gs_2d_fast_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: boo
     with _timed('gs_2d_fast_prepare_fill'):
         rc = lib.fsgs_gs_2d_fast_prepare_fill(P, W, H, L.ptr(means2D_), L.ptr(inverse_m), L.ptr(depths),
                                               L.ptr(opacities), L.ptr(radii), L.ptr(offsets), R, L.ptr(ranges),
-                                              L.ptr(point_list), L.ptr(keys), L.ptr(ws2), ws2.numel(), stream)
+                                              L.ptr(point_list), L.ptr(keys), L.ptr(ws2), ws2.numel(),
+                                              L.ptr(keep_masks), stream)
     L.check(rc, what)
     if debug:
         torch.cuda.synchronize()
@@ -638,6 +642,8 @@ def gs_2d_fast_preprocess_forward(W: int, H: int, sh_degree: int, is_opengl: boo
         out += [keys, tiles_touched]
     if return_offsets:
         out.append(offsets)
+    if return_masks:
+        out.append(keep_masks)
     return out
 
 
@@ -795,7 +801,8 @@ def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inver
                                ranges, point_list, n_contrib, near_n: float, far_n: float,
                                per_tile_bucket_offset=None, bucket_to_tile=None, max_contrib=None, sampled_T=None,
                                sampled_acc=None, sampled_aux=None, point_offsets: Optional[Tensor] = None,
-                               radii: Optional[Tensor] = None, per_splat_kernel: Optional[bool] = None):
+                               radii: Optional[Tensor] = None, per_splat_kernel: Optional[bool] = None,
+                               keep_masks: Optional[Tensor] = None):
     """gs_2d_fast_redner.cu:955-1074 -> [dL_dcolors[P,3], dL_dmeans2D[P,2], dL_dtrans_m[P,3,3], dL_dinverse_m[P,3,3],
     dL_dnorm_op[P,4]]. Passing per_tile_bucket_offset selects the per-splat channel set of the reference's second
     kernel; the snapshot tensors themselves are not needed to evaluate it with the back-to-front kernel, which is the
@@ -803,7 +810,8 @@ def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inver
     decomposition itself from the snapshots (no optical flow in that form). With dL_dout_flow (and trans_mat2,
     out_flows) the optical-flow gradient is added as the reference's kernels add it. With `point_offsets`
     (gs_2d_fast_preprocess_forward(..., return_offsets=True)) and `radii` the per-surfel sums are taken in a fixed order
-    from per-instance records instead of with atomics."""
+    from per-instance records instead of with atomics; `keep_masks` (gs_2d_fast_preprocess_forward(...,
+    return_masks=True)) spares that sum the corner test it otherwise repeats."""
     what = 'GS_2D_fast_render_backward'
     if per_splat_kernel is None:
         per_splat_kernel = PER_SPLAT_BACKWARD
@@ -813,6 +821,11 @@ def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inver
     opt = dict(dtype=torch.float32, device=out_opacity.device)
     ordered, ws, R = _ordered_sum_inputs(what, P, point_list, point_offsets, radii,
                                          'fsgs_gs_2d_fast_render_backward_workspace_bytes', out_opacity.device)
+    if keep_masks is not None:
+        L.require_cuda(what, keep_masks=keep_masks)
+        L.require_dtype(what, 'keep_masks', keep_masks, torch.int32)
+        L.require_shape(what, 'keep_masks', keep_masks, max(P, 1))
+    masks_ptr = L.ptr(keep_masks) if ordered else None
     new = torch.empty if ordered else torch.zeros  # the ordered path assigns every row, the atomic path accumulates
     g_means2D = new((P, 2), **opt)
     g_norm_op = new((P, 4), **opt)
@@ -868,7 +881,7 @@ def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inver
                 L.ptr(dL_dout_color), L.ptr(dL_dout_opacity), L.ptr(dL_dothers) if use_aux else None, L.ptr(ranges),
                 L.ptr(point_list), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans), L.ptr(g_inv), L.ptr(g_norm_op),
                 R, L.ptr(point_offsets) if ordered else None, L.ptr(radii) if ordered else None, L.ptr(ws),
-                ws.numel() if ws is not None else 0, L.current_stream())
+                ws.numel() if ws is not None else 0, masks_ptr, L.current_stream())
         L.check(rc, what)
         return [g_colors, g_means2D, g_trans, g_inv, g_norm_op]
     with _timed('gs_2d_fast_render_backward'):
@@ -879,7 +892,8 @@ def GS_2D_fast_render_backward(means2D, normal_opacity, colors, trans_mat, inver
             L.ptr(dL_dout_opacity), L.ptr(dL_dothers) if use_aux else None, L.ptr(dL_dout_flow) if flow else None,
             L.ptr(ranges), L.ptr(point_list), L.ptr(n_contrib), L.ptr(g_colors), L.ptr(g_means2D), L.ptr(g_trans),
             L.ptr(g_inv), L.ptr(g_norm_op), R, L.ptr(point_offsets) if ordered else None,
-            L.ptr(radii) if ordered else None, L.ptr(ws), ws.numel() if ws is not None else 0, L.current_stream())
+            L.ptr(radii) if ordered else None, L.ptr(ws), ws.numel() if ws is not None else 0, masks_ptr,
+            L.current_stream())
     L.check(rc, what)
     return [g_colors, g_means2D, g_trans, g_inv, g_norm_op]
 

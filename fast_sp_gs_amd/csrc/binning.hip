@@ -187,9 +187,14 @@ constexpr int kMaxLdsTiles = 16384;
 // Which tiles of a surfel's rectangle are visited: all of them (the reference's lists), those that pass the fast path's
 // corner test (CornerTest, from the surfel's adjugate and opacity), or those whose bit is set in the surfel's keep mask
 // (cull_mask_kernel: the tiles some pixel of which can blend the surfel; rectangles above 32 tiles are kept whole).
-enum WalkMode { kWalkAll = 0, kWalkCorner = 1, kWalkMask = 2 };
+// kWalkCornerMask is the corner test with its verdicts for rectangles of at most 32 tiles taken from a mask the
+// preprocess kernel left (bit x * h + y: x-major, the order of the fast path's key span), so that the test's set-up (a
+// double-precision logarithm among it) runs once per surfel and view instead of once per walk; larger rectangles are
+// tested here.
+enum WalkMode { kWalkAll = 0, kWalkCorner = 1, kWalkMask = 2, kWalkCornerMask = 3 };
 
-// What a mode reads beside centres and radii: kWalkCorner the adjugates and opacities, kWalkMask the keep masks.
+// What a mode reads beside centres and radii: kWalkCorner the adjugates and opacities, kWalkMask the keep masks,
+// kWalkCornerMask all three.
 struct WalkInputs {
   const float* inverse_m;
   const float* opacities;
@@ -200,32 +205,40 @@ template <int kMode, typename Visit>
 __device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, const float2* __restrict__ means2D,
                                                   const int32_t* __restrict__ radii, const WalkInputs& in,
                                                   Visit visit) {
+  constexpr bool kCorner = kMode == kWalkCorner || kMode == kWalkCornerMask;  // large rectangles are corner-tested
   const int lane = __lane_id();
   int x0 = 0, y0 = 0, w = 0, h = 0;
-  float IM[kMode == kWalkCorner ? 9 : 1], opacity = 1.0f;
+  float IM[kCorner ? 9 : 1], opacity = 1.0f;
 #pragma unroll
-  for (int k = 0; k < (kMode == kWalkCorner ? 9 : 1); ++k) IM[k] = 0.0f;
+  for (int k = 0; k < (kCorner ? 9 : 1); ++k) IM[k] = 0.0f;
   uint32_t keep_mask = 0xffffffffu;
   if (i < P && radii[i] > 0) {
     const float2 c   = means2D[i];
     const TileRect r = tile_rect(c.x, c.y, radii[i], gx, gy);
     x0 = r.x0, y0 = r.y0, w = max(r.x1 - r.x0, 0), h = max(r.y1 - r.y0, 0);
-    if (kMode == kWalkCorner) {
+    if (kMode == kWalkCorner || (kMode == kWalkCornerMask && w * h > kCoopThreshold)) {
       opacity = in.opacities[i];
 #pragma unroll
       for (int k = 0; k < 9; ++k) IM[k] = in.inverse_m[9 * (size_t) i + k];
     }
-    if (kMode == kWalkMask) keep_mask = in.keep_masks[i];
+    if (kMode == kWalkMask || kMode == kWalkCornerMask) keep_mask = in.keep_masks[i];
   }
   const int count = w * h;
   if (count > 0 && count <= kCoopThreshold) {
-    const CornerTest ct(IM, opacity);  // unused (and removed) in the other modes
-    int e = 0;
-    for (int y = 0; y < h; ++y)
-      for (int x = 0; x < w; ++x, ++e) {
-        const bool keep = kMode == kWalkCorner ? ct.tile(x0 + x, y0 + y) : kMode == kWalkMask ? ((keep_mask >> e) & 1u) != 0u : true;
-        if (keep) visit((y0 + y) * gx + (x0 + x), i);
-      }
+    if (kMode == kWalkCorner) {
+      const CornerTest ct(IM, opacity);
+      for (int y = 0; y < h; ++y)
+        for (int x = 0; x < w; ++x)
+          if (ct.tile(x0 + x, y0 + y)) visit((y0 + y) * gx + (x0 + x), i);
+    } else {
+      int e = 0;
+      for (int y = 0; y < h; ++y)
+        for (int x = 0; x < w; ++x, ++e) {
+          const int bit   = kMode == kWalkCornerMask ? x * h + y : e;
+          const bool keep = kMode == kWalkAll || ((keep_mask >> bit) & 1u) != 0u;
+          if (keep) visit((y0 + y) * gx + (x0 + x), i);
+        }
+    }
   }
   unsigned long long big = __ballot(count > kCoopThreshold);
   while (big) {
@@ -233,13 +246,13 @@ __device__ __forceinline__ void for_each_instance(int i, int P, int gx, int gy, 
     big &= big - 1;
     const int sx0 = __shfl(x0, src, kWave), sy0 = __shfl(y0, src, kWave), sw = __shfl(w, src, kWave);
     const int scount = __shfl(count, src, kWave), sid = __shfl(i, src, kWave);
-    float sIM[kMode == kWalkCorner ? 9 : 1];
+    float sIM[kCorner ? 9 : 1];
 #pragma unroll
-    for (int k = 0; k < (kMode == kWalkCorner ? 9 : 1); ++k) sIM[k] = kMode == kWalkCorner ? __shfl(IM[k], src, kWave) : 0.0f;
-    const CornerTest ct(sIM, kMode == kWalkCorner ? __shfl(opacity, src, kWave) : 1.0f);
+    for (int k = 0; k < (kCorner ? 9 : 1); ++k) sIM[k] = kCorner ? __shfl(IM[k], src, kWave) : 0.0f;
+    const CornerTest ct(sIM, kCorner ? __shfl(opacity, src, kWave) : 1.0f);
     for (int e = lane; e < scount; e += kWave) {
       const int y = e / sw, x = e - y * sw;
-      if (kMode != kWalkCorner || ct.tile(sx0 + x, sy0 + y)) visit((sy0 + y) * gx + (sx0 + x), sid);
+      if (!kCorner || ct.tile(sx0 + x, sy0 + y)) visit((sy0 + y) * gx + (sx0 + x), sid);
     }
   }
 }
@@ -877,8 +890,9 @@ size_t fast_bucket_bins_bytes(int P, int W, int H) {
 }
 
 int fast_bucket_fill(int P, int W, int H, const float* means2D, const float* inverse_m, const float* depths,
-                     const float* opacities, const int32_t* radii, int64_t R, int64_t* ranges, int32_t* point_list,
-                     int64_t* sorted_keys_out, void* workspace, void* bins, hipStream_t s) {
+                     const float* opacities, const int32_t* radii, const uint32_t* keep_masks, int64_t R,
+                     int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out, void* workspace, void* bins,
+                     hipStream_t s) {
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int T  = gx * gy;
   const BinsLayout bl = bins_layout(P, T);
@@ -887,8 +901,13 @@ int fast_bucket_fill(int P, int W, int H, const float* means2D, const float* inv
   uint32_t* hist   = (uint32_t*) ((char*) bins + kBinsHeader);
   uint64_t* entries = sort_keys_in(R, workspace);
   int* large_list   = (int*) ((char*) workspace + sort_layout(R).keys1);
-  hipLaunchKernelGGL(tile_hist_kernel<kWalkCorner>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
-                     (const float2*) means2D, radii, WalkInputs{inverse_m, opacities, nullptr}, hist);
+  const WalkInputs in{inverse_m, opacities, keep_masks};
+  if (keep_masks)
+    hipLaunchKernelGGL(tile_hist_kernel<kWalkCornerMask>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
+                       (const float2*) means2D, radii, in, hist);
+  else
+    hipLaunchKernelGGL(tile_hist_kernel<kWalkCorner>, dim3(bl.blocks), dim3(1024), 0, s, P, bl.per_block, gx, gy,
+                       (const float2*) means2D, radii, in, hist);
   hipLaunchKernelGGL(tile_prefix_kernel, dim3(div_up(T, kPrefixTiles)), dim3(kPrefixTiles * kPrefixWaves), 0, s, T,
                      bl.blocks, hist, rng);
   hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, s, T, rng, header, true);
@@ -896,9 +915,14 @@ int fast_bucket_fill(int P, int W, int H, const float* means2D, const float* inv
   const int* order = nullptr;
   int* build       = nullptr;
   (void) defer_tile_order(gx, gy, ranges, s, &order, &build);
-  hipLaunchKernelGGL(tile_scatter_kernel<kWalkCorner>, dim3(bl.blocks + (build ? 1 : 0)), dim3(1024), 0, s, P,
-                     bl.per_block, gx, gy, R, (const float2*) means2D, depths, radii,
-                     WalkInputs{inverse_m, opacities, nullptr}, (const uint32_t*) hist, rng, entries, build);
+  if (keep_masks)
+    hipLaunchKernelGGL(tile_scatter_kernel<kWalkCornerMask>, dim3(bl.blocks + (build ? 1 : 0)), dim3(1024), 0, s, P,
+                       bl.per_block, gx, gy, R, (const float2*) means2D, depths, radii, in, (const uint32_t*) hist, rng,
+                       entries, build);
+  else
+    hipLaunchKernelGGL(tile_scatter_kernel<kWalkCorner>, dim3(bl.blocks + (build ? 1 : 0)), dim3(1024), 0, s, P,
+                       bl.per_block, gx, gy, R, (const float2*) means2D, depths, radii, in, (const uint32_t*) hist, rng,
+                       entries, build);
   hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
                      header, large_list, order);
   hipLaunchKernelGGL(tile_sort_large_kernel, dim3(256), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,

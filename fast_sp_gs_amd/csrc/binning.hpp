@@ -19,15 +19,19 @@ void launch_tile_ranges(int64_t R, int num_tiles, const uint64_t* sorted_keys, i
 // the reference's padding entries (-1 / T << 32) up to R. `bins`: fast_bucket_bins_bytes(P, W, H) bytes (0: the tile
 // grid is too large for this scheme and the caller sorts device-wide instead); `workspace`: sort_workspace_bytes(R).
 size_t fast_bucket_bins_bytes(int P, int W, int H);
+// `keep_masks` (optional): the verdicts of the test for rectangles of at most 32 tiles, bit x * h + y of a surfel's word
+// (fast_preprocess_forward_kernel writes them); the walks then test only the larger rectangles themselves.
 int fast_bucket_fill(int P, int W, int H, const float* means2D, const float* inverse_m, const float* depths,
-                     const float* opacities, const int32_t* radii, int64_t R, int64_t* ranges, int32_t* point_list,
-                     int64_t* sorted_keys_out, void* workspace, void* bins, hipStream_t s);
+                     const float* opacities, const int32_t* radii, const uint32_t* keep_masks, int64_t R,
+                     int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out, void* workspace, void* bins,
+                     hipStream_t s);
 
 // Implicit conic of the alpha >= 1/255 region, evaluated at tile corners in tile units (gs_2d_fast_preprocess.cu:277-304).
 // Contraction off, the reference's operation order: which tiles a surfel keeps must not depend on the compiler's choice
 // of fused multiply-adds (the lists are compared bit for bit with a plain IEEE evaluation).
 struct CornerTest {
   float Wxx, Wyy, Wxy, Wx_, Wy_, W__;
+  __device__ __forceinline__ CornerTest() : Wxx(0), Wyy(0), Wxy(0), Wx_(0), Wy_(0), W__(1) {}  // passes nowhere
   __device__ __forceinline__ CornerTest(const float* IM, float opacity) {
 #pragma clang fp contract(off)
     const float d = -2.0f * 0.69314718055f * (7.9886846867721655f + (float) log2((double) opacity));

@@ -380,10 +380,13 @@ struct FastScatter {
 // neither cleared nor read. 11 lanes per surfel, each owning one float2 of the 88-byte record: a step covers 11
 // positions of the span -- lane k tests position base + k, the 11 verdicts are shared through a ballot, and the
 // records of the positions that passed are requested together.
+// `keep_masks` (optional, what the preprocess kernel left): the verdicts for rectangles of at most 32 tiles, bit = position
+// in the span; a wavefront none of whose surfels has a larger rectangle then reads neither the adjugates nor the opacity
+// and does not set the test up.
 __global__ void __launch_bounds__(256) fast_slot_sum_kernel(int P, int gx, int gy,
     const int64_t* __restrict__ point_offsets, const int32_t* __restrict__ radii, const float2* __restrict__ means2D,
     const float* __restrict__ inverse_m, const float4* __restrict__ normal_opacity,
-    const float* __restrict__ records, FastScatter out) {
+    const uint32_t* __restrict__ keep_masks, const float* __restrict__ records, FastScatter out) {
   constexpr int kLanes = kFastRecordSlots / 2, kPerWave = 64 / kLanes;
   const int lane = threadIdx.x & 63;
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
@@ -396,16 +399,25 @@ __global__ void __launch_bounds__(256) fast_slot_sum_kernel(int P, int gx, int g
 #pragma unroll
   for (int q = 0; q < 9; ++q) IM[q] = 0.0f;
   const float2* src = (const float2*) records;
+  uint32_t mask = 0u;
+  bool masked = false;  // this surfel's verdicts come from its mask
   if (radius > 0) {
     const float2 c   = means2D[i];
     const TileRect r = tile_rect(c.x, c.y, radius, gx, gy);
     h = max(r.y1 - r.y0, 1), count = max(r.x1 - r.x0, 0) * max(r.y1 - r.y0, 0), x0 = r.x0, y0 = r.y0;
+    masked = keep_masks != nullptr && count <= 32;
+    if (masked) mask = keep_masks[i];
+    src += (size_t) (i > 0 ? point_offsets[i - 1] : 0) * kLanes + k;
+  }
+  const bool tested     = radius > 0 && !masked;
+  const bool any_tested = wave_ballot(tested) != 0ull;  // wave-uniform
+  if (tested) {
 #pragma unroll
     for (int q = 0; q < 9; ++q) IM[q] = inverse_m[9 * (size_t) i + q];
     opacity = normal_opacity[i].w;
-    src += (size_t) (i > 0 ? point_offsets[i - 1] : 0) * kLanes + k;
   }
-  const CornerTest ct(IM, opacity);
+  CornerTest ct;
+  if (any_tested) ct = CornerTest(IM, opacity);
   float2 acc = make_float2(0.0f, 0.0f);
   // the wavefront's surfels step together (the ballot needs every lane): as many steps as its largest rectangle asks
   int steps = (count + kLanes - 1) / kLanes;
@@ -413,7 +425,8 @@ __global__ void __launch_bounds__(256) fast_slot_sum_kernel(int P, int gx, int g
   for (int d = 32; d >= 1; d >>= 1) steps = max(steps, __shfl_xor(steps, d, kWave));
   for (int st = 0; st < steps; ++st) {
     const int base = st * kLanes, p = base + k, x = p / h, y = p - x * h;  // x-major over the rectangle
-    const bool on = p < count && ct.tile(x0 + x, y0 + y);
+    bool on = masked && p < count && ((mask >> (p & 31)) & 1u) != 0u;
+    if (any_tested) on = on || (tested && p < count && ct.tile(x0 + x, y0 + y));
     const unsigned bits = (unsigned) (wave_ballot(on) >> (sub * kLanes)) & ((1u << kLanes) - 1u);
     float2 v[kLanes];
 #pragma unroll
@@ -996,12 +1009,12 @@ __global__ void __launch_bounds__(64) fast_bucket_backward_kernel(int W, int H, 
 
 void launch_fast_slot_sum(int P, int gx, int gy, const int64_t* point_offsets, const int32_t* radii,
                           const float* means2D, const float* inverse_m, const float* normal_opacity,
-                          const SlotWorkspace& ws, FastScatter out, hipStream_t s) {
+                          const uint32_t* keep_masks, const SlotWorkspace& ws, FastScatter out, hipStream_t s) {
   constexpr int kPerWave = 64 / (kFastRecordSlots / 2);
   const int64_t waves = div_up(P, kPerWave);
   hipLaunchKernelGGL(fast_slot_sum_kernel, dim3((unsigned) div_up(waves * 64, 256)), dim3(256), 0, s, P, gx, gy,
                      point_offsets, radii, (const float2*) means2D, inverse_m, (const float4*) normal_opacity,
-                     ws.records, out);
+                     keep_masks, ws.records, out);
 }
 
 }  // namespace
@@ -1061,7 +1074,8 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
     const float* out_flow, const float* dL_dpix, const float* dL_dopacity, const float* dL_dextras,
     const float* dL_dflow, const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib,
     float* g_colors, float* g_means2D, float* g_trans, float* g_inv, float* g_normal_opacity, int64_t R,
-    const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes, void* stream) {
+    const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes,
+    const uint32_t* keep_masks, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "GS_2D_fast_render_backward: bad sizes");
   if (P == 0) return kOk;
   FSGS_REQUIRE(means2D && normal_opacity && colors && trans_mat && inverse_m && out_opacity && dL_dpix && dL_dopacity &&
@@ -1105,7 +1119,7 @@ FSGS_API int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n,
 #undef FSGS_LAUNCH_BWD
 #undef FSGS_LAUNCH_BWD_S
   if (slots)
-    launch_fast_slot_sum(P, gx, gy, point_offsets, radii, means2D, inverse_m, normal_opacity, ws,
+    launch_fast_slot_sum(P, gx, gy, point_offsets, radii, means2D, inverse_m, normal_opacity, keep_masks, ws,
                          FastScatter{g_means2D, g_normal_opacity, g_colors, g_trans, g_inv}, s);
   return check_launch("GS_2D_fast_render_backward");
 }
@@ -1120,7 +1134,7 @@ FSGS_API int fsgs_gs_2d_fast_render_bucket_backward(int P, int W, int H, double 
     const float* dL_dpix, const float* dL_dopacity, const float* dL_dextras, const int64_t* ranges,
     const int32_t* point_list, float* g_colors, float* g_means2D, float* g_trans, float* g_inv,
     float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
-    size_t workspace_bytes, void* stream) {
+    size_t workspace_bytes, const uint32_t* keep_masks, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && B >= 0, "GS_2D_fast_render_bucket_backward: bad sizes");
   if (P == 0) return kOk;
   FSGS_REQUIRE(means2D && normal_opacity && colors && trans_mat && inverse_m && images && out_opacity && n_contrib &&
@@ -1159,6 +1173,7 @@ FSGS_API int fsgs_gs_2d_fast_render_bucket_backward(int P, int W, int H, double 
 #undef FSGS_FAST_BKT
   if (slots)
     launch_fast_slot_sum(P, (W + kTile - 1) / kTile, (H + kTile - 1) / kTile, point_offsets, radii, means2D, inverse_m,
-                         normal_opacity, ws, FastScatter{g_means2D, g_normal_opacity, g_colors, g_trans, g_inv}, s);
+                         normal_opacity, keep_masks, ws,
+                         FastScatter{g_means2D, g_normal_opacity, g_colors, g_trans, g_inv}, s);
   return check_launch("GS_2D_fast_render_bucket_backward");
 }

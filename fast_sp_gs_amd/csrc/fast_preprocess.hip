@@ -97,6 +97,8 @@ __device__ __forceinline__ void fast_transmat_backward(float sx, float sy, const
 }
 
 // kWave: complete degree-3 rows in one 16-byte aligned [P,16,3] tensor, moved by each wavefront on its own (sh_stage.hpp).
+constexpr int kCoopThreshold = 32;  // rectangles with more tiles are walked (and corner-tested) by a whole wavefront
+
 template <int kSh, bool kWave>
 __global__ void __launch_bounds__(256) fast_preprocess_forward_kernel(
     int P, int W, int H, int sh_degree, int n_sh, const float* __restrict__ means3D, const float2* __restrict__ scales,
@@ -105,7 +107,7 @@ __global__ void __launch_bounds__(256) fast_preprocess_forward_kernel(
     const float* __restrict__ campos, const float* __restrict__ trans_precomp, const uint8_t* __restrict__ culling,
     int means2D_preserve, float2* __restrict__ means2D, float* __restrict__ colors, float* __restrict__ trans_mat,
     float* __restrict__ inverse_m, float4* __restrict__ normal_opacity, float* __restrict__ depths,
-    int32_t* __restrict__ radii, int32_t* __restrict__ tiles_touched) {
+    int32_t* __restrict__ radii, int32_t* __restrict__ tiles_touched, uint32_t* __restrict__ keep_masks) {
   __shared__ float s_rows[kWave ? kShStageRows * kShStageStride : 1];
   const int i0     = blockIdx.x * blockDim.x + threadIdx.x;
   const bool valid = i0 < P;
@@ -206,9 +208,36 @@ __global__ void __launch_bounds__(256) fast_preprocess_forward_kernel(
   tiles_touched[i] = ok ? area : 0;
   if (ok || !means2D_preserve) means2D[i] = ok ? make_float2(c2[0], c2[1]) : make_float2(0.0f, 0.0f);
   normal_opacity[i] = ok ? make_float4(nrm[0], nrm[1], nrm[2], opacities[i]) : make_float4(0, 0, 0, 0);
+  if (keep_masks) {
+    // The binning's corner test for every tile of a rectangle of at most 32 tiles, here where adjugate, opacity and
+    // rectangle are in registers: bit x * h + y (x-major, the order of the surfel's key span). The two walks of the
+    // binning and the backward's record sum read the word instead of repeating the test and its set-up; larger
+    // rectangles (all bits set here) are tested where they are walked.
+    uint32_t m = 0xffffffffu;
+    if (ok && area <= kCoopThreshold) {
+      const TileRect r = tile_rect(c2[0], c2[1], f2i_sat(radius), gx, gy);
+      const int w = r.x1 - r.x0, h = r.y1 - r.y0;
+      const CornerTest ct(adj, opacities[i]);
+      // a tile passes if one of its four corners does: every corner of the rectangle is evaluated once, a column of
+      // corners at a time (h + 1 <= 33 bits), and a column of tiles is the OR of its two corner columns and their
+      // shifts
+      auto corner_column = [&](int X) {
+        unsigned long long c = 0ull;
+        for (int y = 0; y <= h; ++y)
+          if (ct.at((float) X, (float) (r.y0 + y))) c |= 1ull << y;
+        return c;
+      };
+      m = 0u;
+      unsigned long long left = corner_column(r.x0);
+      for (int x = 0; x < w; ++x) {
+        const unsigned long long right = corner_column(r.x0 + x + 1), any = left | right;
+        m |= (uint32_t) ((any | (any >> 1)) & ((1ull << h) - 1ull)) << (x * h);
+        left = right;
+      }
+    }
+    keep_masks[i] = m;
+  }
 }
-
-constexpr int kCoopThreshold = 32;
 
 __global__ void __launch_bounds__(256) fast_duplicate_keys_kernel(int P, int gx, int gy, int64_t R,
     const float2* __restrict__ means2D, const float* __restrict__ inverse_m, const float* __restrict__ depths,
@@ -475,7 +504,7 @@ FSGS_API int fsgs_gs_2d_fast_preprocess_forward(int P, int W, int H, int sh_degr
     const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
     const float* Tw2v, const float* Tv2s, const float* campos, const float* trans_precomp, const uint8_t* culling,
     int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* inverse_m, float* normal_opacity,
-    float* depths, int32_t* radii, int32_t* tiles_touched, void* stream) {
+    float* depths, int32_t* radii, int32_t* tiles_touched, uint32_t* keep_masks, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0, "gs_2d_fast_preprocess_forward: bad sizes");
   FSGS_REQUIRE(sh_degree <= kMaxShDegree, "gs_2d_fast_preprocess_forward: sh_degree %d not supported", sh_degree);
   if (sh_degree >= 0)
@@ -493,7 +522,7 @@ FSGS_API int fsgs_gs_2d_fast_preprocess_forward(int P, int W, int H, int sh_degr
   hipLaunchKernelGGL(kernel, dim3(div_up(P, 256)), dim3(256), 0, (hipStream_t) stream, P, W, H, sh_degree, n_sh,
                      means3D, (const float2*) scales, (const float4*) rotations, opacities, shs, sh_rest, Tw2v, Tv2s,
                      campos, trans_precomp, culling, means2D_preserve, (float2*) means2D, colors, trans_mat, inverse_m,
-                     (float4*) normal_opacity, depths, radii, tiles_touched);
+                     (float4*) normal_opacity, depths, radii, tiles_touched, keep_masks);
   return check_launch("gs_2d_fast_preprocess_forward");
 }
 
@@ -509,7 +538,7 @@ FSGS_API size_t fsgs_gs_2d_fast_prepare_fill_workspace_bytes(int P, int W, int H
 FSGS_API int fsgs_gs_2d_fast_prepare_fill(int P, int W, int H, const float* means2D, const float* inverse_m,
     const float* depths, const float* opacities, const int32_t* radii, const int64_t* point_offsets, int64_t R,
     int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out, void* workspace, size_t workspace_bytes,
-    void* stream) {
+    const uint32_t* keep_masks, void* stream) {
   FSGS_REQUIRE(P >= 0 && W > 0 && H > 0 && R >= 0 && ranges, "gs_2d_fast_prepare_fill: bad arguments");
   FSGS_REQUIRE(R < (int64_t) 0x7fffffff, "gs_2d_fast_prepare_fill: %lld instances exceed the 2^31-1 limit",
                (long long) R);
@@ -530,7 +559,7 @@ FSGS_API int fsgs_gs_2d_fast_prepare_fill(int P, int W, int H, const float* mean
   // callers that size the workspace for the sort alone.
   const size_t bins_at = align_up(sort_workspace_bytes(R), 256), bins_bytes = fast_bucket_bins_bytes(P, W, H);
   if (bins_bytes > 0 && workspace_bytes >= bins_at + bins_bytes)
-    return fast_bucket_fill(P, W, H, means2D, inverse_m, depths, opacities, radii, R, ranges, point_list,
+    return fast_bucket_fill(P, W, H, means2D, inverse_m, depths, opacities, radii, keep_masks, R, ranges, point_list,
                             sorted_keys_out, workspace, (char*) workspace + bins_at, s);
   const int bits = fsgs_gs_2d_fast_prepare_sort_bits(W, H);
   hipLaunchKernelGGL(fast_duplicate_keys_kernel, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,

@@ -192,9 +192,9 @@ class _Fast_Render(torch.autograd.Function):
                 accum_max_count, accum_weights_p, accum_weights_count):
         W, H = size
         (means2D, colors, trans_mat, inverse_m, normal_opacity, depths, radii, tile_range, point_list,
-         point_offsets) = _Fast_Render._preprocess_forward(W, H, sh_degree, is_opengl, means3D, scales, rotations,
-                                                           opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, Tv2s, campos,
-                                                           trans_precomp, means2D, culling, False, return_offsets=True)
+         point_offsets, keep_masks) = _Fast_Render._preprocess_forward(
+            W, H, sh_degree, is_opengl, means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, Tv2s,
+            campos, trans_precomp, means2D, culling, False, return_offsets=True, return_masks=True)
         pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib = _Fast_Render._render_forward(
             W, H, near_n, far_n, only_image, means2D, colors, normal_opacity, trans_mat, inverse_m, point_list,
             tile_range, trans_mat_t2, accum_max_count, accum_weights_p, accum_weights_count, None)
@@ -202,7 +202,7 @@ class _Fast_Render(torch.autograd.Function):
         ctx.save_for_backward(means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, Tv2s, campos,
                               means2D, trans_mat, inverse_m, radii, colors, normal_opacity, tile_range, point_list,
                               pixel_colors, pixel_extras, pixel_opacity, n_contrib, trans_mat_t2, pixel_flow,
-                              point_offsets)
+                              point_offsets, keep_masks)
         ctx.mark_non_differentiable(n_contrib, radii)
         return pixel_colors, pixel_opacity, pixel_extras, pixel_flow, n_contrib, radii
 
@@ -211,7 +211,7 @@ class _Fast_Render(torch.autograd.Function):
     def backward(ctx, *grad_outputs):
         (means3D, scales, rotations, opacities, shs_or_colors, shs_rest, Tw2v, Tv2c, Tv2s, campos, means2D, trans_mat,
          inverse_m, radii, colors, normal_opacity, tile_range, point_list, pixel_colors, pixel_extras, pixel_opacity,
-         n_contrib, trans_mat_t2, pixel_flow, point_offsets) = ctx.saved_tensors
+         n_contrib, trans_mat_t2, pixel_flow, point_offsets, keep_masks) = ctx.saved_tensors
         W, H, sh_degree, is_opengl, near_n, far_n = ctx._info
         grad_images, grad_opacity, grad_others, grad_flow = grad_outputs[:4]
         if pixel_flow is None or grad_others is None:
@@ -223,7 +223,8 @@ class _Fast_Render(torch.autograd.Function):
         grad_colors, grad_means2D, grad_trans, grad_inv_m, grad_normal_opacity = _Fast_Render._render_backward(
             means2D, normal_opacity, colors, trans_mat, inverse_m, trans_mat_t2, pixel_colors, pixel_opacity,
             pixel_extras, pixel_flow, grad_images, grad_opacity, grad_others, grad_flow, tile_range, point_list,
-            n_contrib, near_n, far_n, None, None, None, None, None, None, point_offsets, radii)
+            n_contrib, near_n, far_n, None, None, None, None, None, None, point_offsets, radii,
+            keep_masks=keep_masks)
         grad_inputs = [
             *_grad_buffers(means3D, scales, rotations, opacities, shs_or_colors, shs_rest, sh_degree,
                            ctx.needs_input_grad[4], ctx.needs_input_grad[5]),
@@ -296,20 +297,23 @@ def fast_compuate_transmat(means3D: Tensor, scales: Tensor, rotations: Tensor, T
 
 
 def fast_render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None, grad_opacity: Tensor = None,
-                     per_splat: bool = False, ordered_sums: bool = True, per_splat_kernel: bool = False):
+                     per_splat: bool = False, ordered_sums: bool = True, per_splat_kernel: bool = False,
+                     reuse_masks: bool = True):
     """One forward + backward pass of the fast path through the raw operators, returning every intermediate. With
     `ordered_sums` the blend backward adds per-instance records in a fixed order instead of using atomics. With
     `per_splat_kernel` (needs `per_splat`) the backward is the reference's per-splat decomposition, started from the
-    forward's snapshots, instead of the back-to-front kernel with the per-splat channel set."""
+    forward's snapshots, instead of the back-to-front kernel with the per-splat channel set. `reuse_masks`: the ordered
+    sum reads the corner test's verdicts the preprocess left instead of repeating the test (same sums)."""
     pre_f = get_C_function('gs_2d_fast_preprocess_forward')
     pre_b = get_C_function('gs_2d_fast_preprocess_backward')
     ren_f = get_C_function('GS_2D_fast_render_forward')
     ren_b = get_C_function('GS_2D_fast_render_backward')
     W, H = cam.W, cam.H
     (means2D, colors, trans_mat, inverse_m, normal_opacity, depths, radii, ranges, point_list, keys,
-     tiles_touched, point_offsets) = pre_f(W, H, scene.sh_degree, False, scene.means3D, scene.scales, scene.rotations,
-                                           scene.opacities, scene.shs, None, cam.Tw2v, cam.Tv2c, cam.Tv2s, cam.campos,
-                                           None, None, None, False, True, True)
+     tiles_touched, point_offsets, keep_masks) = pre_f(W, H, scene.sh_degree, False, scene.means3D, scene.scales,
+                                                       scene.rotations, scene.opacities, scene.shs, None, cam.Tw2v,
+                                                       cam.Tv2c, cam.Tv2s, cam.campos, None, None, None, False, True,
+                                                       True, True)
     offset = None
     if per_splat:
         offset = torch.cumsum((ranges[:, 1] - ranges[:, 0] + 31) // 32, dim=0).contiguous()
@@ -323,7 +327,7 @@ def fast_render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None,
         grad_opacity, grad_extras, None, ranges, point_list, n_contrib, cam.near, cam.far, offset,
         *((outs[6], outs[5], outs[7], outs[8], outs[9]) if per_splat and per_splat_kernel else (None,) * 5),
         point_offsets if ordered_sums else None, radii if ordered_sums else None,
-        per_splat_kernel=bool(per_splat and per_splat_kernel))
+        per_splat_kernel=bool(per_splat and per_splat_kernel), keep_masks=keep_masks if reuse_masks else None)
     g_means2D_in = g_means2D.clone()
     # the preprocess backward writes every row of its outputs (zeros for surfels that were not rendered)
     g = dict(means3D=torch.empty_like(scene.means3D), scales=torch.empty_like(scene.scales),
@@ -334,7 +338,7 @@ def fast_render_step(scene, cam, grad_image: Tensor, grad_extras: Tensor = None,
           g_colors, g_no, g['means3D'], g['scales'], g['rotations'], g['opacities'], g['shs'], None)
     out = dict(means2D=means2D, colors=colors, trans_mat=trans_mat, inverse_m=inverse_m,
                normal_opacity=normal_opacity, depths=depths, radii=radii, tiles_touched=tiles_touched, ranges=ranges,
-               point_list=point_list, keys=keys, image=image, opacity=opacity, extras=extras, n_contrib=n_contrib,
+               point_list=point_list, keys=keys, keep_masks=keep_masks, image=image, opacity=opacity, extras=extras, n_contrib=n_contrib,
                g_colors=g_colors, g_means2D_blend=g_means2D_in, g_trans=g_trans, g_inv=g_inv, g_normal_opacity=g_no,
                g_means2D_proxy=g_means2D, g_means3D=g['means3D'], g_scales=g['scales'], g_rotations=g['rotations'],
                g_opacities=g['opacities'], g_shs=g['shs'])

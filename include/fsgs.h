@@ -187,12 +187,16 @@ int fsgs_gs_2d_render_backward_culled(int P, int W, int H, double near_n, double
 
 /* gs_2d_fast_preprocess_forward (per-surfel part) -- gs_2d_fast_preprocess.cu:160-262, host :611-709.
  * Same outputs as fsgs_gs_2d_preprocess_forward plus inverse_m[P,3,3] (adjugate of trans_mat). Only the z translation
- * of Tw2v enters the transform, as in the reference (:95). */
+ * of Tw2v enters the transform, as in the reference (:95). keep_masks[P] (optional, no counterpart in the reference)
+ * receives the binning's corner test for every tile of a rectangle of at most 32 tiles, bit x * h + y of the surfel's
+ * word (x-major over the w x h rectangle, the order of its key span; larger rectangles: all bits set). The binning and
+ * the ordered-sum backwards take the masks back and then repeat the test, and its set-up, only for larger rectangles:
+ * same lists, keys, ranges and sums. */
 int fsgs_gs_2d_fast_preprocess_forward(int P, int W, int H, int sh_degree, int n_sh, const float* means3D,
     const float* scales, const float* rotations, const float* opacities, const float* shs, const float* sh_rest,
     const float* Tw2v, const float* Tv2s, const float* campos, const float* trans_precomp, const uint8_t* culling,
     int means2D_preserve, float* means2D, float* colors, float* trans_mat, float* inverse_m, float* normal_opacity,
-    float* depths, int32_t* radii, int32_t* tiles_touched, void* stream);
+    float* depths, int32_t* radii, int32_t* tiles_touched, uint32_t* keep_masks, void* stream);
 
 /* Binning half of gs_2d_fast_preprocess_forward -- gs_2d_fast_preprocess.cu:264-327 (duplicateWithKeys with the
  * per-tile corner test, x-major, unused slots padded with key = T << 32 / value = -1), :711-778 (sort on
@@ -200,13 +204,14 @@ int fsgs_gs_2d_fast_preprocess_forward(int P, int W, int H, int sh_degree, int n
  * at its tail. Workspace: fsgs_gs_2d_fast_prepare_fill_workspace_bytes(P, W, H, R) (no counterpart in the reference);
  * with it the kept instances are counted, scattered and sorted per tile and the padding entries are written behind
  * them -- the same lists, keys and ranges as the reference's device-wide sort of the padded key array, which is what a
- * workspace of only fsgs_gs_prepare_fill_workspace_bytes(R) bytes (and any grid above 16 384 tiles) still gets. */
+ * workspace of only fsgs_gs_prepare_fill_workspace_bytes(R) bytes (and any grid above 16 384 tiles) still gets.
+ * keep_masks (optional): what fsgs_gs_2d_fast_preprocess_forward left for these surfels. */
 int fsgs_gs_2d_fast_prepare_sort_bits(int W, int H);
 size_t fsgs_gs_2d_fast_prepare_fill_workspace_bytes(int P, int W, int H, int64_t R);
 int fsgs_gs_2d_fast_prepare_fill(int P, int W, int H, const float* means2D, const float* inverse_m,
     const float* depths, const float* opacities, const int32_t* radii, const int64_t* point_offsets, int64_t R,
     int64_t* ranges, int32_t* point_list, int64_t* sorted_keys_out, void* workspace, size_t workspace_bytes,
-    void* stream);
+    const uint32_t* keep_masks, void* stream);
 
 /* gs_2d_fast_preprocess_backward -- gs_2d_fast_preprocess.cu:536-609, host :784-852. grad_mean2D is read, then
  * overwritten with the densification proxy computed from the ACCUMULATED transform gradient (:606-608). */
@@ -251,7 +256,8 @@ int fsgs_gs_2d_fast_render_forward(int P, int W, int H, double near_n, double fa
  * a 16-byte aligned workspace of fsgs_gs_2d_fast_render_backward_workspace_bytes(R) bytes (no counterpart in the
  * reference) every row of the outputs is ASSIGNED from per-(surfel, tile) records added in a fixed order. The
  * workspace needs no clearing: every list entry's record is written on every call, and the sum repeats the binning's
- * corner test so that it reads no other position of a surfel's key span. */
+ * corner test (or reads its verdicts from keep_masks, optional, as fsgs_gs_2d_fast_preprocess_forward left them) so
+ * that it reads no other position of a surfel's key span. */
 size_t fsgs_gs_2d_fast_render_backward_workspace_bytes(int64_t R);
 int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n, double far_n, int per_splat_form,
     const float* means2D, const float* normal_opacity, const float* colors, const float* trans_mat,
@@ -259,7 +265,8 @@ int fsgs_gs_2d_fast_render_backward(int P, int W, int H, double near_n, double f
     const float* out_flow, const float* dL_dpix, const float* dL_dopacity, const float* dL_dextras,
     const float* dL_dflow, const int64_t* ranges, const int32_t* point_list, const int32_t* n_contrib,
     float* g_colors, float* g_means2D, float* g_trans, float* g_inv, float* g_normal_opacity, int64_t R,
-    const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes, void* stream);
+    const int64_t* point_offsets, const int32_t* radii, void* workspace, size_t workspace_bytes,
+    const uint32_t* keep_masks, void* stream);
 
 /* The per-splat decomposition of gs_2d_fast_redner.cu:563-837 itself (fsgs_gs_2d_fast_render_backward with
  * per_splat_form = 1 returns the same derivative through the back-to-front kernel, which is faster here): a lane owns
@@ -276,7 +283,7 @@ int fsgs_gs_2d_fast_render_bucket_backward(int P, int W, int H, double near_n, d
     const float* dL_dpix, const float* dL_dopacity, const float* dL_dextras, const int64_t* ranges,
     const int32_t* point_list, float* g_colors, float* g_means2D, float* g_trans, float* g_inv,
     float* g_normal_opacity, int64_t R, const int64_t* point_offsets, const int32_t* radii, void* workspace,
-    size_t workspace_bytes, void* stream);
+    size_t workspace_bytes, const uint32_t* keep_masks, void* stream);
 
 /* gs_2d_topk_weights -- fast_2d_gs/_C/src/gaussian_splatting/gaussian_topk.cu:230-250 (kernel :95-210).
  * top_indices[H,W,topk] int32 (-1 = empty), top_weights[H,W,topk] descending blend weights alpha*T; topk <= 16. */

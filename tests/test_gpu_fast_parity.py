@@ -342,32 +342,39 @@ def test_fast_forward_writes_every_pixel(name, device):
 def test_fast_binning_per_tile_equals_device_wide_sort(name, device):
     """fsgs_gs_2d_fast_prepare_fill builds the lists per tile when its workspace has room for the per-tile counters and
     by the reference's device-wide sort of the padded key array otherwise: ranges, lists (padding tail included) and
-    sorted keys are the same bit for bit (the stage-by-stage test holds the per-tile result to the oracle)."""
+    sorted keys are the same bit for bit (the stage-by-stage test holds the per-tile result to the oracle). The per-tile
+    scheme with the corner test's verdicts read from the preprocess kernel's keep masks (what the operator does) and
+    with the test repeated in both walks (no masks) give the same as well."""
     from fast_sp_gs_amd import lib as L
     from fast_sp_gs_amd._C import get_C_function as f
     lib = L.load()
     scene, cam, *_ = _make(name)
     sc, cm = scene.to(device), cam.to(device)
     W, H, P = cam.W, cam.H, scene.P
-    (m2, colors, tm, im, no, depths, radii, ranges, point_list, keys, tt, offsets) = f('gs_2d_fast_preprocess_forward')(
+    (m2, colors, tm, im, no, depths, radii, ranges, point_list, keys, tt, offsets,
+     masks) = f('gs_2d_fast_preprocess_forward')(
         W, H, 3, False, sc.means3D, sc.scales, sc.rotations, sc.opacities, sc.shs, None, cm.Tw2v, cm.Tv2c, cm.Tv2s,
-        cm.campos, None, None, None, False, True, True)
+        cm.campos, None, None, None, False, True, True, True)
     R = int(point_list.numel())
     small, large = lib.fsgs_gs_prepare_fill_workspace_bytes(R), lib.fsgs_gs_2d_fast_prepare_fill_workspace_bytes(P, W, H, R)
     assert large > small
+    small_rects = (tt > 0) & (tt <= 32)
+    assert int(small_rects.sum()) > 0 and int((masks[small_rects] != -1).sum()) > 0  # some tile of some rectangle fails
     results = []
-    for nbytes in (small, large):
+    for nbytes, use_masks in ((small, False), (large, False), (large, True)):
         ws = torch.full((nbytes,), 0xA5, dtype=torch.uint8, device=device)
         rng = torch.full_like(ranges, -7)
         pl = torch.full((R,), -9, dtype=torch.int32, device=device)
         ks = torch.full((R,), -11, dtype=torch.int64, device=device)
         L.check(lib.fsgs_gs_2d_fast_prepare_fill(P, W, H, L.ptr(m2), L.ptr(im), L.ptr(depths), L.ptr(sc.opacities),
                                                  L.ptr(radii), L.ptr(offsets), R, L.ptr(rng), L.ptr(pl), L.ptr(ks),
-                                                 L.ptr(ws), nbytes, L.current_stream()), 'fast_prepare_fill')
+                                                 L.ptr(ws), nbytes, L.ptr(masks) if use_masks else None,
+                                                 L.current_stream()), 'fast_prepare_fill')
         torch.cuda.synchronize()
         results.append((rng, pl, ks))
-    for a, b, what in zip(results[0], results[1], ('ranges', 'point_list', 'keys')):
-        assert torch.equal(a, b), what
+    for other in (1, 2):
+        for a, b, what in zip(results[0], results[other], ('ranges', 'point_list', 'keys')):
+            assert torch.equal(a, b), (what, other)
     assert torch.equal(results[1][0], ranges) and torch.equal(results[1][1], point_list)
     assert int((point_list == -1).sum()) > 0
 

@@ -192,6 +192,12 @@ def test_fast_path_properties_at_300k_800(per_splat, device):
     for k in ('image', 'opacity', 'extras', 'n_contrib', 'point_list', 'ranges'):
         assert torch.equal(a[k], b[k]), f"{k} depends on the culling"
     close(a, b, 2e-5, 'culling')
+    # the ordered sum with the corner test repeated instead of read from the preprocess kernel's keep masks: the same
+    # records in the same order, bit for bit
+    m = fast_render_step(scene, cam, gi, ge, go, per_splat=per_splat, reuse_masks=False)
+    for k in grads:
+        assert torch.equal(a[k], m[k]), ('keep masks', k)
+    del m
     # (the atomics add in arrival order; the fast preprocess backward amplifies that rounding in dL/dscales)
     close(a, fast_render_step(scene, cam, gi, ge, go, per_splat=per_splat, ordered_sums=False), 1e-4, 'atomic sums')
     c = fast_render_step(scene, cam, 2.0 * gi, 2.0 * ge, 2.0 * go, per_splat=per_splat)

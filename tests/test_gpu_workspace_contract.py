@@ -122,13 +122,15 @@ def test_backward_workspace_needs_no_clearing(variant, source, device):
             assert rel_err(a, b) < 1e-3, name
 
 
+@pytest.mark.parametrize("masks", ["test_repeated", "keep_masks"])
 @pytest.mark.parametrize("kernel", ["tile", "per_splat"])
 @pytest.mark.parametrize("variant", ["aux", "image_only"])
-def test_fast_backward_workspace_needs_no_clearing(variant, kernel, device):
+def test_fast_backward_workspace_needs_no_clearing(variant, kernel, masks, device):
     """The same promise on the fast path, whose key spans hold positions that belong to no tile's list (tiles of the
     rectangle that fail the corner test): the record sum repeats the binning's test and reads only the positions the
     blend wrote, so nothing is cleared there either. Both backward kernels (back to front per tile / the per-splat
-    decomposition over 32-entry buckets), with and without the auxiliary maps."""
+    decomposition over 32-entry buckets), with and without the auxiliary maps, the sum repeating the test or reading its
+    verdicts from the preprocess kernel's keep masks."""
     from fast_sp_gs_amd import lib as L, scenes
     from fast_sp_gs_amd._C import get_C_function as f
     lib = L.load()
@@ -138,9 +140,10 @@ def test_fast_backward_workspace_needs_no_clearing(variant, kernel, device):
     scene.means3D[:, 0] = scene.means3D[:, 0] * 0.6 - 0.5
     cam = scenes.pinhole(W, H, 50.0, torch.tensor([0., 0., 4.]))
     sc, cm = scene.to(device), cam.to(device)
-    (m2, colors, tm, im, no, depths, radii, ranges, point_list, keys, tt, offsets) = f('gs_2d_fast_preprocess_forward')(
+    (m2, colors, tm, im, no, depths, radii, ranges, point_list, keys, tt, offsets,
+     keep) = f('gs_2d_fast_preprocess_forward')(
         W, H, 3, False, sc.means3D, sc.scales, sc.rotations, sc.opacities, sc.shs, None, cm.Tw2v, cm.Tv2c, cm.Tv2s,
-        cm.campos, None, None, None, False, True, True)
+        cm.campos, None, None, None, False, True, True, True)
     b_off = torch.cumsum((ranges[:, 1] - ranges[:, 0] + 31) // 32, 0).contiguous()
     image, oo, oe, _, nc, max_c, b2t, s_T, s_acc, s_aux = f('GS_2D_fast_render_forward')(
         W, H, cam.near, cam.far, False, m2, colors, no, tm, im, point_list, ranges, None, None, None, None, b_off)[:10]
@@ -165,7 +168,8 @@ def test_fast_backward_workspace_needs_no_clearing(variant, kernel, device):
         out = [torch.full((P, n), float('nan'), device=device) if ordered else torch.zeros(P, n, device=device)
                for n in (3, 2, 9, 9, 4)]  # colours, means2D, transform, adjugate, normal + opacity
         tail = (R, L.ptr(offsets) if ordered else None, L.ptr(radii) if ordered else None,
-                L.ptr(ws) if ordered else None, nbytes if ordered else 0, L.current_stream())
+                L.ptr(ws) if ordered else None, nbytes if ordered else 0,
+                L.ptr(keep) if ordered and masks == "keep_masks" else None, L.current_stream())
         if kernel == "tile":
             rc = lib.fsgs_gs_2d_fast_render_backward(
                 P, W, H, float(cam.near), float(cam.far), 1, L.ptr(m2), L.ptr(no), L.ptr(colors), L.ptr(tm), L.ptr(im),
