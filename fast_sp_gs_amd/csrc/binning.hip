@@ -621,8 +621,21 @@ constexpr int kLargeSegment = 16384;  // entries sorted by a 1024-lane block in 
 // sorting at once instead of wherever the image puts them in tile order (the launch ends with its slowest block).
 __global__ void __launch_bounds__(256) tile_sort_small_kernel(int64_t* __restrict__ ranges,
     const uint64_t* __restrict__ entries, int32_t* __restrict__ point_list, int64_t* __restrict__ keys_out,
-    int* __restrict__ large_count, int* __restrict__ large_list, const int* __restrict__ order) {
+    int* __restrict__ large_count, int* __restrict__ large_list, const int* __restrict__ order, int n_tiles,
+    int64_t R, const int* __restrict__ kept, uint64_t pad_key) {
   __shared__ uint64_t s_e[kSmallSegment + kSmallSegment / 4];
+  // Blocks past the tile grid (the fast path launches some): that path reserves one list position per tile of a
+  // surfel's rectangle, and the positions behind the instances that passed the corner test hold the reference's padding
+  // entries (key = T << 32, value = -1), which its sort leaves at the tail of the list. Written here, beside the sorts,
+  // rather than by a launch of its own behind them.
+  if ((int) blockIdx.x >= n_tiles) {
+    const int64_t stride = (int64_t) (gridDim.x - n_tiles) * blockDim.x;
+    for (int64_t o = (int64_t) *kept + (int64_t) (blockIdx.x - n_tiles) * blockDim.x + threadIdx.x; o < R; o += stride) {
+      point_list[o] = -1;
+      if (keys_out) keys_out[o] = (int64_t) pad_key;
+    }
+    return;
+  }
   const int tile = order ? order[blockIdx.x] : (int) blockIdx.x;
   const int64_t start = ranges[2 * (size_t) tile];
   const int64_t len   = ranges[2 * (size_t) tile + 1] - start;
@@ -796,18 +809,6 @@ __global__ void __launch_bounds__(256) tile_ranges_kernel(int64_t R, int num_til
   if (i == R - 1 && cur_ok) ranges[2 * (size_t) cur + 1] = R;
 }
 
-// The fast path reserves one list position per tile of a surfel's rectangle; the positions behind the instances that
-// pass the corner test hold the reference's padding entries (key = T << 32, value = -1), which its sort leaves at the
-// tail of the list.
-__global__ void __launch_bounds__(256) pad_tail_kernel(int64_t R, const int* __restrict__ kept, uint64_t pad_key,
-                                                       int32_t* __restrict__ point_list, int64_t* __restrict__ keys_out) {
-  const int64_t o = (int64_t) *kept + (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
-  if (o < R) {
-    point_list[o] = -1;
-    if (keys_out) keys_out[o] = (int64_t) pad_key;
-  }
-}
-
 }  // namespace
 
 uint32_t higher_msb(uint32_t n) {  // number of bits needed for the tile id, as gaussian_prepare.cu:32-44 computes it
@@ -923,13 +924,12 @@ int fast_bucket_fill(int P, int W, int H, const float* means2D, const float* inv
     hipLaunchKernelGGL(tile_scatter_kernel<kWalkCorner>, dim3(bl.blocks + (build ? 1 : 0)), dim3(1024), 0, s, P,
                        bl.per_block, gx, gy, R, (const float2*) means2D, depths, radii, in, (const uint32_t*) hist, rng,
                        entries, build);
-  hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
-                     header, large_list, order);
+  // 256 blocks more than tiles: they write the padding entries behind the kept instances
+  hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T + 256), dim3(256), 0, s, ranges, entries, point_list,
+                     sorted_keys_out, header, large_list, order, T, R, (const int*) (header + 1),
+                     (uint64_t) (uint32_t) T << 32);
   hipLaunchKernelGGL(tile_sort_large_kernel, dim3(256), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,
                      header, large_list);
-  // at most R positions are padding; blocks beyond the tail leave at once
-  hipLaunchKernelGGL(pad_tail_kernel, dim3(div_up(R, 256)), dim3(256), 0, s, R, header + 1, (uint64_t) (uint32_t) T << 32,
-                     point_list, sorted_keys_out);
   return check_launch("gs_2d_fast_prepare_fill");
 }
 
@@ -1075,7 +1075,7 @@ int fill_sort(int P, int W, int H, const float* means2D, const float* depths, co
     (void) launch_tile_order(gx, gy, ranges, s, &order);
   }
   hipLaunchKernelGGL(tile_sort_small_kernel, dim3(T), dim3(256), 0, s, ranges, entries, point_list, sorted_keys_out,
-                     large_count, large_list, order);
+                     large_count, large_list, order, T, (int64_t) 0, (const int*) nullptr, (uint64_t) 0);
   hipLaunchKernelGGL(tile_sort_large_kernel, dim3(256), dim3(1024), 0, s, ranges, entries, point_list, sorted_keys_out,
                      large_count, large_list);
   return check_launch("gs_prepare_fill");

@@ -546,8 +546,10 @@ FSGS_API int fsgs_gs_2d_fast_prepare_fill(int P, int W, int H, const float* mean
   const int gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
   const int T  = gx * gy;
   tile_order_invalidate(s);  // the ranges are rewritten: the blend schedule of this stream is stale
-  launch_zero_ranges(T, ranges, s);
-  if (R == 0 || P == 0) return check_launch("gs_2d_fast_prepare_fill(zero)");
+  if (R == 0 || P == 0) {
+    launch_zero_ranges(T, ranges, s);
+    return check_launch("gs_2d_fast_prepare_fill(zero)");
+  }
   FSGS_REQUIRE(means2D && inverse_m && depths && opacities && radii && point_offsets && point_list && workspace,
                "gs_2d_fast_prepare_fill: null pointer");
   if (workspace_bytes < sort_workspace_bytes(R))
@@ -561,6 +563,8 @@ FSGS_API int fsgs_gs_2d_fast_prepare_fill(int P, int W, int H, const float* mean
   if (bins_bytes > 0 && workspace_bytes >= bins_at + bins_bytes)
     return fast_bucket_fill(P, W, H, means2D, inverse_m, depths, opacities, radii, keep_masks, R, ranges, point_list,
                             sorted_keys_out, workspace, (char*) workspace + bins_at, s);
+  // the range kernel below writes the tiles that have entries (the per-tile scheme above writes every range itself)
+  launch_zero_ranges(T, ranges, s);
   const int bits = fsgs_gs_2d_fast_prepare_sort_bits(W, H);
   hipLaunchKernelGGL(fast_duplicate_keys_kernel, dim3(div_up(P, 256)), dim3(256), 0, s, P, gx, gy, R,
                      (const float2*) means2D, inverse_m, depths, opacities, radii, point_offsets,
